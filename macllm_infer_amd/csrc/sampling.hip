@@ -1,0 +1,285 @@
+// Sampling over rows of float32 logits [B, V]: penalties, greedy argmax, and
+// temperature / top-k / top-p with one uniform draw per token.
+//
+// Order of operations (reference: src/sampling.rs:95-161):
+//   repetition penalty over prompt+generated (x<0 ? x*p : x/p, :407-423), presence and
+//   frequency penalties over generated tokens (:392-405), then either argmax with the
+//   lowest index on ties (:425-433) or: divide by temperature, keep the k largest
+//   (value descending, index ascending), softmax with the maximum subtracted, keep the
+//   shortest descending prefix whose mass reaches top_p (:337-375), draw u * (kept mass)
+//   and walk the kept tokens in index order (:165-169, :378-390).
+// The uniform u comes from a counter-based generator: splitmix64 of
+// seed + (draw_index + 1) * 0x9E3779B97F4A7C15, top 24 bits / 2^24.
+#include "common.h"
+
+#define SAMPLE_THREADS 1024
+
+__device__ __forceinline__ unsigned int orderable(float v) {
+  const unsigned int bits = __float_as_uint(v);
+  return (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);   // ascending in v
+}
+
+__device__ __forceinline__ float from_orderable(unsigned int key) {
+  const unsigned int bits = (key & 0x80000000u) ? (key & 0x7fffffffu) : ~key;
+  return __uint_as_float(bits);
+}
+
+// ---------------------------------------------------------------- penalties
+// tokens[offsets[b] .. offsets[b+1]) is row b's history (prompt then generated);
+// the first prompt_lens[b] of them are the prompt.  count_all / count_gen are [B, V]
+// int32 work areas that hold zeros on entry and on exit.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+penalties_kernel(float* __restrict__ logits, int V, const int* __restrict__ tokens,
+                 const int* __restrict__ offsets, const int* __restrict__ prompt_lens,
+                 const float* __restrict__ repetition, const float* __restrict__ presence,
+                 const float* __restrict__ frequency, int* __restrict__ count_all, int* __restrict__ count_gen) {
+  const int row = blockIdx.x;
+  float* values = logits + (long)row * V;
+  int* all = count_all + (long)row * V;
+  int* gen = count_gen + (long)row * V;
+  const int begin = offsets[row];
+  const int end = offsets[row + 1];
+  const int prompt = prompt_lens[row];
+  for (int i = begin + threadIdx.x; i < end; i += blockDim.x) {
+    const int token = tokens[i];
+    if (token < 0 || token >= V) continue;
+    atomicAdd(&all[token], 1);
+    if (i - begin >= prompt) atomicAdd(&gen[token], 1);
+  }
+  __threadfence();
+  __syncthreads();
+  const float rep = repetition[row];
+  const bool use_rep = rep > 0.f && fabsf(rep - 1.0f) >= 1.1920929e-07f;
+  const float pres = presence[row];
+  const float freq = frequency[row];
+  const bool use_openai = pres != 0.f || freq != 0.f;
+  for (int v = threadIdx.x; v < V; v += blockDim.x) {
+    const int seen = all[v];
+    if (seen == 0) continue;
+    float x = values[v];
+    if (use_rep) x = x < 0.f ? x * rep : x / rep;
+    const int generated = gen[v];
+    if (use_openai && generated > 0) x -= freq * (float)generated + pres;
+    values[v] = x;
+    all[v] = 0;
+    gen[v] = 0;
+  }
+}
+
+extern "C" int mi_apply_penalties(float* logits, int B, int V, const int* tokens, const int* offsets,
+                                  const int* prompt_lens, const float* repetition, const float* presence,
+                                  const float* frequency, int* count_all, int* count_gen, hipStream_t stream) {
+  if (B <= 0 || V <= 0) return ERR_BAD_ARGUMENT;
+  penalties_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, V, tokens, offsets, prompt_lens, repetition,
+                                                     presence, frequency, count_all, count_gen);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- argmax
+// (value descending, index ascending) packed so that the smallest 64-bit key wins.
+__device__ __forceinline__ unsigned long long rank_key(float value, int index) {
+  return ((unsigned long long)(~orderable(value)) << 32) | (unsigned int)index;
+}
+
+__device__ unsigned long long block_min_key(unsigned long long key, unsigned long long* scratch) {
+#pragma unroll
+  for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+    const unsigned long long other = __shfl_xor(key, offset, WAVE);
+    key = other < key ? other : key;
+  }
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wave = threadIdx.x / WAVE;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = key;
+  __syncthreads();
+  unsigned long long best = scratch[0];
+  for (int i = 1; i < (int)(blockDim.x / WAVE); ++i) best = scratch[i] < best ? scratch[i] : best;
+  return best;
+}
+
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+argmax_kernel(const float* __restrict__ logits, int V, int* __restrict__ out) {
+  __shared__ unsigned long long scratch[SAMPLE_THREADS / WAVE];
+  const float* values = logits + (long)blockIdx.x * V;
+  unsigned long long best = ~0ull;
+  for (int v = threadIdx.x; v < V; v += blockDim.x) {
+    const unsigned long long key = rank_key(values[v], v);
+    best = key < best ? key : best;
+  }
+  best = block_min_key(best, scratch);
+  if (threadIdx.x == 0) out[blockIdx.x] = (int)(best & 0xffffffffu);
+}
+
+extern "C" int mi_argmax(const float* logits, int B, int V, int* out, hipStream_t stream) {
+  if (B <= 0 || V <= 0) return ERR_BAD_ARGUMENT;
+  argmax_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, V, out);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- stochastic sampling
+__device__ __forceinline__ float draw_uniform(unsigned long long seed, unsigned long long draw_index) {
+  unsigned long long z = seed + (draw_index + 1ull) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  z = z ^ (z >> 31);
+  return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+
+// Exclusive prefix of per-thread sums over the block (thread order), plus the block total.
+__device__ float block_exclusive_scan(float value, float* scratch /* blockDim.x floats */, float* total) {
+  __syncthreads();
+  scratch[threadIdx.x] = value;
+  __syncthreads();
+  // Hillis-Steele inclusive scan
+  for (int offset = 1; offset < (int)blockDim.x; offset <<= 1) {
+    float add = 0.f;
+    if ((int)threadIdx.x >= offset) add = scratch[threadIdx.x - offset];
+    __syncthreads();
+    scratch[threadIdx.x] += add;
+    __syncthreads();
+  }
+  const float inclusive = scratch[threadIdx.x];
+  *total = scratch[blockDim.x - 1];
+  return inclusive - value;
+}
+
+// One block per row.  `keys` is a [B, padded] 64-bit work area, padded = power of two >= V.
+// Rows with temperature <= 0 take the argmax.  The row of logits is overwritten.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_kernel(float* __restrict__ logits, int V, int padded, const float* __restrict__ temperature,
+              const int* __restrict__ top_k, const float* __restrict__ top_p,
+              const unsigned long long* __restrict__ seeds, const int* __restrict__ draw_index,
+              unsigned long long* __restrict__ keys, int* __restrict__ out) {
+  __shared__ float scan_scratch[SAMPLE_THREADS];
+  __shared__ unsigned long long key_scratch[SAMPLE_THREADS / WAVE];
+  __shared__ int found;
+  const int row = blockIdx.x;
+  float* values = logits + (long)row * V;
+  unsigned long long* sorted = keys + (long)row * padded;
+  const float temp = temperature[row];
+
+  if (temp <= 0.f) {
+    unsigned long long best = ~0ull;
+    for (int v = threadIdx.x; v < V; v += blockDim.x) {
+      const unsigned long long key = rank_key(values[v], v);
+      best = key < best ? key : best;
+    }
+    best = block_min_key(best, key_scratch);
+    if (threadIdx.x == 0) out[row] = (int)(best & 0xffffffffu);
+    return;
+  }
+
+  // scale and build sort keys
+  for (int v = threadIdx.x; v < padded; v += blockDim.x) {
+    if (v < V) {
+      const float scaled = values[v] / temp;
+      values[v] = scaled;
+      sorted[v] = rank_key(scaled, v);
+    } else {
+      sorted[v] = ~0ull;
+    }
+  }
+  __threadfence_block();
+  __syncthreads();
+
+  // bitonic sort, ascending keys = descending values, ties by ascending index
+  for (int size = 2; size <= padded; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int i = threadIdx.x; i < padded / 2; i += blockDim.x) {
+        const int low = ((i / stride) * stride * 2) + (i % stride);
+        const int high = low + stride;
+        const bool ascending = ((low & size) == 0);
+        const unsigned long long a = sorted[low];
+        const unsigned long long b = sorted[high];
+        if ((a > b) == ascending) {
+          sorted[low] = b;
+          sorted[high] = a;
+        }
+      }
+      __threadfence_block();
+      __syncthreads();
+    }
+  }
+
+  int kept = V;
+  const int k = top_k[row];
+  if (k > 0 && k < V) kept = k;
+  const float maximum = from_orderable(~(unsigned int)(sorted[0] >> 32));
+
+  // softmax normalizer over the kept prefix
+  const int chunk = (kept + blockDim.x - 1) / blockDim.x;
+  const int chunk_begin = min(kept, (int)threadIdx.x * chunk);
+  const int chunk_end = min(kept, chunk_begin + chunk);
+  float local = 0.f;
+  for (int i = chunk_begin; i < chunk_end; ++i)
+    local += expf(from_orderable(~(unsigned int)(sorted[i] >> 32)) - maximum);
+  float normalizer;
+  float before = block_exclusive_scan(local, scan_scratch, &normalizer);
+
+  // top-p: first sorted position whose cumulative probability reaches top_p
+  const float p_limit = top_p[row];
+  if (threadIdx.x == 0) found = kept;
+  __syncthreads();
+  if (p_limit >= 0.f && p_limit < 1.f) {
+    // this thread's chunk starts at the scanned mass of its predecessors
+    float cumulative = before / normalizer;
+    for (int i = chunk_begin; i < chunk_end; ++i) {
+      cumulative += expf(from_orderable(~(unsigned int)(sorted[i] >> 32)) - maximum) / normalizer;
+      if (cumulative >= p_limit) {
+        atomicMin(&found, i + 1);
+        break;
+      }
+    }
+  }
+  __syncthreads();
+  const int nucleus = found;
+  __syncthreads();
+
+  // probabilities of the kept tokens, scattered back in index order; zero elsewhere
+  for (int v = threadIdx.x; v < V; v += blockDim.x) values[v] = 0.f;
+  __threadfence_block();
+  __syncthreads();
+  for (int i = threadIdx.x; i < nucleus; i += blockDim.x) {
+    const unsigned long long key = sorted[i];
+    const int index = (int)(key & 0xffffffffu);
+    values[index] = expf(from_orderable(~(unsigned int)(key >> 32)) - maximum) / normalizer;
+  }
+  __threadfence_block();
+  __syncthreads();
+
+  // walk in index order
+  const int vchunk = (V + blockDim.x - 1) / blockDim.x;
+  const int vbegin = min(V, (int)threadIdx.x * vchunk);
+  const int vend = min(V, vbegin + vchunk);
+  float mass = 0.f;
+  for (int v = vbegin; v < vend; ++v) mass += values[v];
+  float total;
+  const float start = block_exclusive_scan(mass, scan_scratch, &total);
+  const float target = draw_uniform(seeds[row], (unsigned long long)draw_index[row]) * total;
+  if (threadIdx.x == 0) found = V;
+  __syncthreads();
+  float cumulative = start;
+  for (int v = vbegin; v < vend; ++v) {
+    const float p = values[v];
+    if (p <= 0.f) continue;
+    cumulative += p;
+    if (target < cumulative) {
+      atomicMin(&found, v);
+      break;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) out[row] = found < V ? found : (int)(sorted[0] & 0xffffffffu);
+}
+
+extern "C" int mi_sample(float* logits, int B, int V, int padded, const float* temperature, const int* top_k,
+                         const float* top_p, const unsigned long long* seeds, const int* draw_index,
+                         unsigned long long* keys, int* out, hipStream_t stream) {
+  if (B <= 0 || V <= 0 || padded < V || (padded & (padded - 1)) != 0) return ERR_BAD_ARGUMENT;
+  sample_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, V, padded, temperature, top_k, top_p, seeds,
+                                                  draw_index, keys, out);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}

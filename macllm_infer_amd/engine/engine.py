@@ -1,0 +1,126 @@
+"""The engine: a loaded model, its cache manager and the one step function.
+
+``step`` takes a batch of lanes (request, its next tokens, the places whose logits are
+wanted): portions of prompts beside single decoded tokens, cut anywhere.  It runs only
+the tokens it is given, as one batch, from the cache earlier steps left, and returns the
+logits at the wanted places.  Everything is validated and all pages are reserved before
+anything is launched, so a refused step changes nothing
+(reference: src/architecture.rs:1187-1227 contract, src/decoder.rs:3878-3968 checks,
+:4125-4201 transactional execute).
+"""
+from __future__ import annotations
+
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.pages import CacheExhausted
+from ..config.registry import config_from_dict, load_config
+from ..kernels import build as kernel_build
+from ..kernels import ops
+from ..parts.base import BuildContext
+from ..weights.loader import WeightSource, bind
+from .context import Lane, build_step_context
+from .model import DecoderModel
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           "f32": torch.float32}
+
+
+class StepError(ValueError):
+    """A step was refused before anything ran; the engine's state is unchanged."""
+
+
+def resolve_dtype(dtype) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"dtype must be bfloat16 or float32, got {dtype}")
+        return dtype
+    if dtype not in _DTYPES:
+        raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, got {dtype!r}")
+    return _DTYPES[dtype]
+
+
+class Engine:
+    def __init__(self, model_dir: Optional[str] = None, *, config=None, tensors=None, dtype="bfloat16",
+                 device="cuda:0", kv_cache_block_tokens: int = 16,
+                 kv_cache_capacity_tokens: Optional[int] = None, max_active_sequences: int = 8,
+                 check_device: bool = True):
+        """Load from ``model_dir`` (config.json + safetensors), or from a config object (or raw
+        dict) plus a name -> tensor mapping.  ``kv_cache_capacity_tokens`` defaults to one
+        model context shared by all requests (reference: src/runtime.rs:175-201)."""
+        self.dtype = resolve_dtype(dtype)
+        self.device = ops.require_gpu(device) if check_device else torch.device(device)
+        if model_dir is not None:
+            self.config = load_config(model_dir)
+            source = WeightSource.from_dir(model_dir)
+        else:
+            self.config = config_from_dict(config) if isinstance(config, dict) else config
+            source = WeightSource.from_tensors(tensors)
+        self.spec = self.config.to_model_spec()
+        self.spec.validate()
+        if check_device:
+            kernel_build.ensure_modules(DecoderModel.kernel_modules(self.spec))
+        bound = bind(source, DecoderModel.expected_tensors(self.spec))
+        source.close()
+        build = BuildContext(hidden_size=self.spec.hidden_size, dtype=self.dtype, device=self.device,
+                             max_context=self.spec.max_context)
+        self.model = DecoderModel(self.spec, bound, build)
+        needs, shared = DecoderModel.cache_layout(self.spec)
+        capacity = kv_cache_capacity_tokens or self.spec.max_context
+        self.cache = CacheManager(needs, shared, kv_cache_block_tokens, capacity, max_active_sequences,
+                                  self.dtype, self.device)
+        self.vocab_size = self.spec.vocab_size
+        self.max_context = self.spec.max_context
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, request: Hashable) -> None:
+        """Make ``request`` live: a zeroed state slot and empty block tables."""
+        self.cache.add_request(request)
+
+    def finish(self, request: Hashable) -> None:
+        """Give back everything ``request`` holds."""
+        self.cache.finish(request)
+
+    def has_request(self, request: Hashable) -> bool:
+        return request in self.cache.requests
+
+    def length(self, request: Hashable) -> int:
+        return self.cache.requests[request].length
+
+    # ------------------------------------------------------------------ the step function
+    def validate(self, lanes: Sequence[Lane]) -> None:
+        if not lanes:
+            raise StepError("a step needs at least one lane")
+        seen = set()
+        for lane in lanes:
+            if lane.request not in self.cache.requests:
+                raise StepError(f"request {lane.request!r} is not live")
+            if lane.request in seen:
+                raise StepError(f"request {lane.request!r} appears twice in one step")
+            seen.add(lane.request)
+            count = len(lane.tokens)
+            if count == 0:
+                raise StepError(f"request {lane.request!r}: a lane cannot be empty")
+            for token in lane.tokens:
+                if not (0 <= int(token) < self.vocab_size):
+                    raise StepError(f"request {lane.request!r}: token {token} is outside the vocabulary "
+                                    f"of {self.vocab_size}")
+            if self.cache.requests[lane.request].length + count > self.max_context:
+                raise StepError(f"request {lane.request!r}: {self.cache.requests[lane.request].length} + {count} "
+                                f"tokens exceed the context limit {self.max_context}")
+            for place in lane.want:
+                if not (0 <= int(place) < count):
+                    raise StepError(f"request {lane.request!r}: wanted place {place} is outside its {count} tokens")
+
+    def step(self, lanes: Sequence[Lane]) -> torch.Tensor:
+        """Run one batch; returns float32 logits [wanted, vocab] in the order of the lanes and
+        of each lane's ``want``.  Raises StepError or CacheExhausted with nothing changed."""
+        self.validate(lanes)
+        self.cache.reserve([(lane.request, len(lane.tokens)) for lane in lanes])
+        context = build_step_context(lanes, self.cache, self.device)
+        logits = self.model.forward(context, self.cache)
+        for lane in lanes:
+            self.cache.commit(lane.request, len(lane.tokens))
+        return logits

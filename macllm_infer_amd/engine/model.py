@@ -1,0 +1,89 @@
+"""The decoder model: embedding, the layers in the order the schedule gives, final norm
+and output projection, put together from registered parts according to a ``ModelSpec``.
+(reference: src/decoder.rs:2980-3105 load, :3146-3358 packed forward.)
+"""
+from __future__ import annotations
+
+from typing import Dict, Hashable, List, Tuple
+
+import torch
+
+from ..config.spec import ModelSpec
+from ..kernels import ops
+from ..parts.base import BuildContext, Residual, part_class
+from ..parts.block import arrangement_class
+from ..weights.loader import Expect
+
+
+class DecoderModel:
+    @staticmethod
+    def expected_tensors(spec: ModelSpec) -> List[Expect]:
+        """Every tensor the model binds, by exact name with its shape
+        (name tables: src/architecture.rs:1595-1647)."""
+        out = [Expect(f"{spec.embedding_name}.weight", ((spec.vocab_size, spec.hidden_size),), init="embedding")]
+        for layer in spec.layers:
+            out += arrangement_class(layer.arrangement).expected_tensors(layer, spec.hidden_size)
+        out += part_class(spec.final_norm).expected_tensors(spec.final_norm, spec.final_norm_name, spec.hidden_size)
+        if not spec.tied_embeddings:
+            out.append(Expect(f"{spec.lm_head_name}.weight", ((spec.vocab_size, spec.hidden_size),)))
+        return out
+
+    @staticmethod
+    def kernel_modules(spec: ModelSpec) -> List[str]:
+        modules = ["common", "gemm"]
+        for layer in spec.layers:
+            modules += arrangement_class(layer.arrangement).kernel_modules(layer)
+        return list(dict.fromkeys(modules))
+
+    @staticmethod
+    def cache_layout(spec: ModelSpec):
+        """(needs, shared): (entry, mixer name) -> that mixer's cache needs, and which
+        (entry, mixer) reads the K/V of which earlier one."""
+        needs: Dict[Hashable, list] = {}
+        shared: Dict[Hashable, Hashable] = {}
+        for index, entry in enumerate(spec.schedule):
+            layer = spec.layers[entry.layer]
+            for slot in layer.mixers:
+                key = (index, slot.name)
+                needs[key] = list(part_class(slot.spec).cache_needs(slot.spec))
+                if entry.kv_from is not None and any(type(need).__name__ == "KVNeed" for need in needs[key]):
+                    shared[key] = (entry.kv_from, slot.name)
+        return needs, shared
+
+    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], build: BuildContext):
+        spec.validate()
+        self.spec = spec
+        self.build = build
+        table = tensors[f"{spec.embedding_name}.weight"]
+        if build.dtype == torch.float32:
+            table = table.to(torch.float32)
+        self.embedding = table.contiguous().to(build.device)
+        self.blocks = [arrangement_class(layer.arrangement)(layer, tensors, build) for layer in spec.layers]
+        self.final_norm = part_class(spec.final_norm)(spec.final_norm, spec.final_norm_name, tensors, build)
+        if spec.tied_embeddings:
+            self.lm_head = self.embedding
+        else:
+            head = tensors[f"{spec.lm_head_name}.weight"]
+            if build.dtype == torch.float32:
+                head = head.to(torch.float32)
+            self.lm_head = head.contiguous().to(build.device)
+
+    def forward(self, step, cache) -> torch.Tensor:
+        """Run the step's tokens through every scheduled layer and return float32 logits
+        [wanted, vocab] at ``step.want_rows`` (empty tensor when nothing is wanted)."""
+        spec = self.spec
+        h = torch.empty((step.num_tokens, spec.hidden_size), dtype=torch.float32, device=self.build.device)
+        ops.embed(step.token_ids, self.embedding, spec.embedding_multiplier, h)
+        residual = Residual(h)
+        for index, entry in enumerate(spec.schedule):
+            block = self.blocks[entry.layer]
+            caches = {name: cache.entry((index, name)) for name, _ in block.mixers}
+            block.forward(residual, step, caches)
+        wanted = step.want_rows.numel()
+        if wanted == 0:
+            return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.build.device)
+        normed = self.final_norm.forward(residual, rows=step.want_rows)
+        raw = ops.linear(normed, self.lm_head, None)
+        logits = torch.empty((wanted, spec.vocab_size), dtype=torch.float32, device=self.build.device)
+        ops.scale_to_f32(raw, spec.logit_multiplier, logits)
+        return logits

@@ -1,0 +1,396 @@
+"""The operations the parts are made of, each a hand-written HIP kernel for gfx950
+(matrix products of the bfloat16 path go to the BLAS library, as the reference's do:
+src/model_weights.rs:307-415 hands them to its tensor library).
+
+Every wrapper checks operand shapes, dtypes and devices on the host before the launch,
+and raises ``KernelError`` when a kernel refuses a size.  There is no other code path:
+without a GPU and the built modules these functions fail.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Sequence
+
+import torch
+
+from . import build
+
+_c_int = ctypes.c_int
+_c_long = ctypes.c_long
+_c_float = ctypes.c_float
+_c_ptr = ctypes.c_void_p
+
+DT_F32, DT_BF16 = 0, 1
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_SIGNATURES = {
+    "common": {
+        "mi_embed": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_int, _c_ptr],
+        "mi_add_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int,
+                           _c_int, _c_ptr],
+        "mi_swiglu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_ptr],
+        "mi_scale_to_f32": [_c_ptr, _c_int, _c_float, _c_ptr, _c_long, _c_ptr],
+    },
+    "attention": {
+        "mi_rope_kv_store": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int,
+                             _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr],
+        "mi_paged_attention": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
+                               _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_long, _c_ptr],
+    },
+    "mamba2": {
+        "mi_conv1d_silu": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+        "mi_conv_state_update": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                                 _c_ptr],
+        "mi_ssm_scan": [_c_ptr, _c_int, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_ptr],
+        "mi_gate_norm": [_c_ptr, _c_long, _c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_float, _c_ptr, _c_long,
+                         _c_int, _c_int, _c_ptr],
+    },
+    "gemm": {
+        "mi_gemm_f32": [_c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr],
+    },
+    "sampling": {
+        "mi_apply_penalties": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                               _c_ptr, _c_ptr],
+        "mi_argmax": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
+        "mi_sample": [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                      _c_ptr],
+    },
+}
+
+_functions = {}
+
+
+def _fn(module: str, name: str):
+    key = (module, name)
+    if key not in _functions:
+        library = build.load_module(module)
+        function = getattr(library, name)
+        function.argtypes = _SIGNATURES[module][name]
+        function.restype = _c_int
+        _functions[key] = function
+    return _functions[key]
+
+
+def require_gpu(device) -> torch.device:
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise KernelError("the HIP kernels need a GPU (device 'cuda:N'); there is no CPU path")
+    return device
+
+
+def _dt(tensor: torch.Tensor) -> int:
+    if tensor.dtype == torch.float32:
+        return DT_F32
+    if tensor.dtype == torch.bfloat16:
+        return DT_BF16
+    raise KernelError(f"unsupported dtype {tensor.dtype}; kernels take float32 or bfloat16")
+
+
+def _p(tensor: Optional[torch.Tensor]):
+    return None if tensor is None else tensor.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(code: int, name: str, detail: str = "") -> None:
+    if code == 0:
+        return
+    if code == -1:
+        raise KernelError(f"{name}: bad argument {detail}")
+    if code == -2:
+        raise KernelError(f"{name}: size not supported by this kernel {detail}")
+    raise KernelError(f"{name}: HIP launch failed with error {code} {detail}")
+
+
+def _need(condition: bool, message: str) -> None:
+    if not condition:
+        raise KernelError(message)
+
+
+def _i32(tensor: torch.Tensor, name: str) -> None:
+    _need(tensor.dtype == torch.int32 and tensor.is_contiguous() and tensor.is_cuda,
+          f"{name} must be a contiguous int32 GPU tensor")
+
+
+def _row_major(tensor: torch.Tensor, name: str) -> int:
+    """A 2-D tensor whose rows are contiguous; returns the row stride in elements."""
+    _need(tensor.dim() == 2 and tensor.stride(1) == 1 and tensor.is_cuda,
+          f"{name} must be a 2-D GPU tensor with contiguous rows")
+    return tensor.stride(0) if tensor.shape[0] > 1 else max(tensor.stride(0), tensor.shape[1])
+
+
+# --------------------------------------------------------------------------- common
+def embed(token_ids: torch.Tensor, table: torch.Tensor, multiplier: float, out: torch.Tensor) -> None:
+    """out[t] = table[token_ids[t]] * multiplier, out float32 [T, d]."""
+    _i32(token_ids, "token_ids")
+    T, d = out.shape
+    _need(token_ids.numel() == T and table.dim() == 2 and table.shape[1] == d and table.is_contiguous(),
+          "embed: shapes do not match")
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous float32")
+    _check(_fn("common", "mi_embed")(_p(token_ids), _p(table), _dt(table), float(multiplier), _p(out), T, d,
+                                     _stream()), "embed")
+
+
+def add_rmsnorm(h: torch.Tensor, deltas: Sequence[torch.Tensor], weight: torch.Tensor, eps: float,
+                out: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> None:
+    """h += sum(deltas) (float32, in place); out = h / sqrt(mean(h^2) + eps) * weight.
+
+    With ``rows`` (int32 indices) only those rows are read, ``out[i]`` gets row ``rows[i]``
+    and ``h`` is left as it is.  ``out`` may be None when only the sum is wanted."""
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous() and h.is_cuda,
+          "add_rmsnorm: h must be contiguous float32 [T, d]")
+    T, d = h.shape
+    _need(len(deltas) <= 2, "add_rmsnorm: at most two deltas")
+    for delta in deltas:
+        _need(delta.shape == h.shape and delta.is_contiguous() and delta.dtype == deltas[0].dtype,
+              "add_rmsnorm: deltas must be contiguous [T, d] of one dtype")
+    _need(weight.dtype == torch.float32 and weight.numel() == d and weight.is_contiguous(),
+          "add_rmsnorm: weight must be float32 [d]")
+    n_rows = T
+    if rows is not None:
+        _i32(rows, "rows")
+        n_rows = rows.numel()
+    if out is not None:
+        _need(out.shape == (n_rows, d) and out.is_contiguous(), "add_rmsnorm: out must be contiguous [rows, d]")
+    delta_dtype = _dt(deltas[0]) if deltas else DT_F32
+    out_dtype = _dt(out) if out is not None else DT_F32
+    _check(_fn("common", "mi_add_rmsnorm")(
+        _p(h), _p(deltas[0]) if len(deltas) > 0 else None, _p(deltas[1]) if len(deltas) > 1 else None,
+        delta_dtype, _p(weight), float(eps), _p(out), out_dtype, _p(rows), n_rows, d, _stream()),
+        "add_rmsnorm", f"(d={d})")
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, i] = SiLU(gate_up[t, i]) * gate_up[t, I + i]."""
+    ld = _row_major(gate_up, "gate_up")
+    T, two_i = gate_up.shape
+    _need(two_i % 2 == 0 and out.shape == (T, two_i // 2) and out.is_contiguous() and out.dtype == gate_up.dtype,
+          "swiglu: out must be contiguous [T, I] of the input's dtype")
+    _check(_fn("common", "mi_swiglu")(_p(gate_up), _dt(gate_up), ld, _p(out), T, two_i // 2, _stream()), "swiglu")
+
+
+def scale_to_f32(values: torch.Tensor, multiplier: float, out: torch.Tensor) -> None:
+    _need(values.is_contiguous() and out.is_contiguous() and out.dtype == torch.float32
+          and out.numel() == values.numel() and values.is_cuda, "scale_to_f32: shapes do not match")
+    _check(_fn("common", "mi_scale_to_f32")(_p(values), _dt(values), float(multiplier), _p(out), values.numel(),
+                                            _stream()), "scale_to_f32")
+
+
+# --------------------------------------------------------------------------- matrix products
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """x [M, K] . weight[N, K]^T (+ bias float32 [N]) -> [M, N] in x's dtype.
+
+    float32 operands: the hand-written float32 FMA kernel (true 32-bit).  bfloat16 operands:
+    the BLAS library with float32 accumulation.  A float32 weight with bfloat16 activations
+    (a tensor that was stored in 32-bit) runs in float32 and the result is rounded once."""
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "linear: shapes do not match")
+    if weight.dtype == torch.float32:
+        xf = x if x.dtype == torch.float32 else x.float()
+        ldx = _row_major(xf, "x")
+        ldw = _row_major(weight, "weight")
+        M, K = xf.shape
+        N = weight.shape[0]
+        out = torch.empty((M, N), dtype=torch.float32, device=x.device)
+        if bias is not None:
+            _need(bias.dtype == torch.float32 and bias.numel() == N, "linear: bias must be float32 [N]")
+        _check(_fn("gemm", "mi_gemm_f32")(_p(xf), ldx, _p(weight), ldw, _p(bias), _p(out), N, M, N, K, _stream()),
+               "gemm_f32", f"(M={M}, N={N}, K={K})")
+        return out if x.dtype == torch.float32 else out.to(x.dtype)
+    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear: operands must share a dtype")
+    if bias is None:
+        return torch.matmul(x, weight.t())
+    return torch.addmm(bias.to(torch.bfloat16), x, weight.t())
+
+
+# --------------------------------------------------------------------------- attention
+def rope_kv_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                  positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rotary_dim: int,
+                  slot_mapping: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                  v_cache: Optional[torch.Tensor]) -> None:
+    """Rotate q (in place) and k of every token; store rotated k and raw v into the cache.
+
+    ``qkv`` [T, >= (Hq+2Hkv)*dh] holds q heads, k heads, v heads.  ``k_cache``/``v_cache``
+    are one layer's views [pages, Hkv, page_size, dh] of the paged pool;
+    ``slot_mapping[t] = page*page_size + offset``.  Without ``slot_mapping`` nothing is stored."""
+    ld = _row_major(qkv, "qkv")
+    T = qkv.shape[0]
+    _need(qkv.shape[1] >= (num_heads + 2 * num_kv_heads) * head_dim, "rope_kv_store: qkv is too narrow")
+    _i32(positions, "positions")
+    _need(positions.numel() == T, "rope_kv_store: one position per token")
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == rotary_dim // 2 and inv_freq.is_cuda,
+              "rope_kv_store: inv_freq must be float32 [rotary_dim/2]")
+    page_stride, page_size = 0, 0
+    if slot_mapping is not None:
+        _i32(slot_mapping, "slot_mapping")
+        _need(slot_mapping.numel() == T, "rope_kv_store: one cache cell per token")
+        page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype)
+    _check(_fn("attention", "mi_rope_kv_store")(
+        _p(qkv), _dt(qkv), ld, T, num_heads, num_kv_heads, head_dim, _p(positions), _p(inv_freq),
+        rotary_dim if inv_freq is not None else 0, _p(slot_mapping),
+        _p(k_cache) if slot_mapping is not None else None, _p(v_cache) if slot_mapping is not None else None,
+        page_stride, page_size, _stream()), "rope_kv_store")
+
+
+def _cache_view(k_cache, v_cache, num_kv_heads, head_dim, dtype):
+    for name, cache in (("k_cache", k_cache), ("v_cache", v_cache)):
+        _need(cache is not None and cache.dim() == 4 and cache.shape[1] == num_kv_heads
+              and cache.shape[3] == head_dim and cache.dtype == dtype and cache.is_cuda,
+              f"{name} must be [pages, Hkv, page_size, dh] of the activation dtype")
+        _need(cache.stride(3) == 1 and cache.stride(2) == head_dim
+              and cache.stride(1) == cache.shape[2] * head_dim, f"{name}: a page's [Hkv, page_size, dh] must be dense")
+    _need(k_cache.stride(0) == v_cache.stride(0) and k_cache.shape == v_cache.shape,
+          "k_cache and v_cache must share a geometry")
+    return k_cache.stride(0), k_cache.shape[2]
+
+
+def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                    k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                    lane_of_token: torch.Tensor, positions: torch.Tensor, scale: float,
+                    window: Optional[int], out: torch.Tensor) -> None:
+    """Causal attention of every token over its request's cached keys (its own included).
+
+    ``q`` [T, >= Hq*dh] (rotated); ``block_tables`` [lanes, max_pages] page ids by logical
+    page; a key at position p is visible to a query at position s when p <= s and, with a
+    window w, s - p < w.  ``out`` [T, Hq*dh]."""
+    q_ld = _row_major(q, "q")
+    out_ld = _row_major(out, "out")
+    T = q.shape[0]
+    _need(q.shape[1] >= num_heads * head_dim and out.shape == (T, num_heads * head_dim)
+          and out.dtype == q.dtype, "paged_attention: q/out shapes do not match")
+    page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, q.dtype)
+    _i32(block_tables, "block_tables")
+    _i32(lane_of_token, "lane_of_token")
+    _i32(positions, "positions")
+    _need(block_tables.dim() == 2 and lane_of_token.numel() == T and positions.numel() == T,
+          "paged_attention: metadata shapes do not match")
+    _check(_fn("attention", "mi_paged_attention")(
+        _p(q), _dt(q), q_ld, T, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride,
+        page_size, _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale),
+        int(window or 0), _p(out), out_ld, _stream()), "paged_attention", f"(head_dim={head_dim})")
+
+
+# --------------------------------------------------------------------------- mamba2
+def conv1d_silu(u: torch.Tensor, col_offset: int, width: int, weight: torch.Tensor,
+                bias: Optional[torch.Tensor], conv_state: torch.Tensor, lane_of_token: torch.Tensor,
+                cu_seqlens: torch.Tensor, slot_ids: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t] = SiLU(causal depthwise conv of u[:, col_offset:col_offset+width]) per lane,
+    the K-1 rows before a lane's first token coming from ``conv_state[slot]`` [K-1, width]."""
+    ld = _row_major(u, "u")
+    T = u.shape[0]
+    K = weight.shape[1]
+    _need(weight.shape == (width, K) and weight.dtype == torch.float32 and weight.is_contiguous(),
+          "conv1d_silu: weight must be float32 [C, K]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == width), "conv1d_silu: bad bias")
+    _need(conv_state.dim() == 3 and conv_state.shape[1:] == (max(K - 1, 0), width)
+          and conv_state.dtype == u.dtype and conv_state.is_contiguous(), "conv1d_silu: bad conv_state")
+    _need(out.shape == (T, width) and out.is_contiguous() and out.dtype == u.dtype, "conv1d_silu: bad out")
+    _need(u.shape[1] >= col_offset + width, "conv1d_silu: u is too narrow")
+    for name, tensor in (("lane_of_token", lane_of_token), ("cu_seqlens", cu_seqlens), ("slot_ids", slot_ids)):
+        _i32(tensor, name)
+    _check(_fn("mamba2", "mi_conv1d_silu")(
+        _p(u), _dt(u), ld, col_offset, T, width, K, _p(weight), _p(bias), _p(conv_state), _p(lane_of_token),
+        _p(cu_seqlens), _p(slot_ids), _p(out), _stream()), "conv1d_silu", f"(K={K})")
+
+
+def conv_state_update(u: torch.Tensor, col_offset: int, width: int, kernel: int, conv_state: torch.Tensor,
+                      cu_seqlens: torch.Tensor, slot_ids: torch.Tensor) -> None:
+    """conv_state[slot] = last K-1 rows of [conv_state[slot] ; the lane's rows of u]."""
+    ld = _row_major(u, "u")
+    num_lanes = slot_ids.numel()
+    _need(conv_state.dim() == 3 and conv_state.shape[1:] == (max(kernel - 1, 0), width)
+          and conv_state.dtype == u.dtype and conv_state.is_contiguous(), "conv_state_update: bad conv_state")
+    _need(cu_seqlens.numel() == num_lanes + 1, "conv_state_update: cu_seqlens must have lanes+1 entries")
+    _i32(cu_seqlens, "cu_seqlens")
+    _i32(slot_ids, "slot_ids")
+    _check(_fn("mamba2", "mi_conv_state_update")(
+        _p(u), _dt(u), ld, col_offset, width, kernel, _p(conv_state), _p(cu_seqlens), _p(slot_ids), num_lanes,
+        _stream()), "conv_state_update", f"(K={kernel})")
+
+
+def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
+             ssm_state: torch.Tensor, cu_seqlens: torch.Tensor, slot_ids: torch.Tensor, num_groups: int,
+             y: torch.Tensor) -> None:
+    """Selective scan of every lane from and into ``ssm_state[slot]`` [H, P, N] (float32).
+
+    ``xbc`` [T, E + 2*G*N] = post-conv x | B | C; ``dt`` [T, H] raw (a column view is fine);
+    ``y`` float32 [T, E] gets s.C + D*x."""
+    xbc_ld = _row_major(xbc, "xbc")
+    dt_ld = _row_major(dt, "dt")
+    y_ld = _row_major(y, "y")
+    _need(ssm_state.dim() == 4 and ssm_state.dtype == torch.float32 and ssm_state.is_contiguous(),
+          "ssm_scan: state must be contiguous float32 [slots, H, P, N]")
+    _, H, P, N = ssm_state.shape
+    T = xbc.shape[0]
+    _need(xbc.shape[1] == H * P + 2 * num_groups * N and dt.shape == (T, H) and dt.dtype == xbc.dtype
+          and y.shape == (T, H * P) and y.dtype == torch.float32, "ssm_scan: shapes do not match")
+    for name, vector in (("dt_bias", dt_bias), ("A", A), ("D", D)):
+        _need(vector.dtype == torch.float32 and vector.numel() == H and vector.is_contiguous() and vector.is_cuda,
+              f"ssm_scan: {name} must be float32 [H]")
+    _i32(cu_seqlens, "cu_seqlens")
+    _i32(slot_ids, "slot_ids")
+    num_lanes = slot_ids.numel()
+    _need(cu_seqlens.numel() == num_lanes + 1, "ssm_scan: cu_seqlens must have lanes+1 entries")
+    _check(_fn("mamba2", "mi_ssm_scan")(
+        _p(xbc), _dt(xbc), xbc_ld, _p(dt), dt_ld, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(cu_seqlens),
+        _p(slot_ids), num_lanes, H, P, N, num_groups, _p(y), y_ld, _stream()), "ssm_scan", f"(N={N})")
+
+
+def gate_norm(y: torch.Tensor, z: torch.Tensor, weight: Optional[torch.Tensor], num_groups: int, eps: float,
+              out: torch.Tensor) -> None:
+    """out = y * SiLU(z), then (with a weight) RMSNorm over each group of E/G channels."""
+    y_ld = _row_major(y, "y")
+    z_ld = _row_major(z, "z")
+    out_ld = _row_major(out, "out")
+    T, E = y.shape
+    _need(y.dtype == torch.float32 and z.shape == (T, E) and out.shape == (T, E) and out.dtype == z.dtype,
+          "gate_norm: shapes do not match")
+    _need(weight is None or (weight.dtype == torch.float32 and weight.numel() == E and weight.is_contiguous()),
+          "gate_norm: weight must be float32 [E]")
+    _check(_fn("mamba2", "mi_gate_norm")(_p(y), y_ld, _p(z), _dt(z), z_ld, _p(weight), num_groups, float(eps),
+                                         _p(out), out_ld, T, E, _stream()), "gate_norm")
+
+
+# --------------------------------------------------------------------------- sampling
+def apply_penalties(logits, tokens, offsets, prompt_lens, repetition, presence, frequency, count_all, count_gen):
+    B, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.is_contiguous() and logits.is_cuda, "penalties: bad logits")
+    for name, tensor in (("tokens", tokens), ("offsets", offsets), ("prompt_lens", prompt_lens),
+                         ("count_all", count_all), ("count_gen", count_gen)):
+        _i32(tensor, name)
+    _need(count_all.numel() >= B * V and count_gen.numel() >= B * V, "penalties: work areas are too small")
+    _need(offsets.numel() == B + 1 and prompt_lens.numel() == B, "penalties: bad history layout")
+    _check(_fn("sampling", "mi_apply_penalties")(
+        _p(logits), B, V, _p(tokens), _p(offsets), _p(prompt_lens), _p(repetition), _p(presence), _p(frequency),
+        _p(count_all), _p(count_gen), _stream()), "apply_penalties")
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    B, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.is_contiguous() and logits.is_cuda, "argmax: bad logits")
+    _i32(out, "out")
+    _need(out.numel() == B, "argmax: one output per row")
+    _check(_fn("sampling", "mi_argmax")(_p(logits), B, V, _p(out), _stream()), "argmax")
+
+
+def sample(logits, temperature, top_k, top_p, seeds, draw_index, keys, out) -> None:
+    """One token per row; overwrites ``logits``.  ``keys`` int64 [B, padded] work area."""
+    B, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.is_contiguous() and logits.is_cuda, "sample: bad logits")
+    padded = keys.shape[1]
+    _need(keys.dtype == torch.int64 and keys.shape[0] >= B and keys.is_contiguous(), "sample: bad work area")
+    _need(temperature.dtype == torch.float32 and top_p.dtype == torch.float32 and seeds.dtype == torch.int64,
+          "sample: bad parameter dtypes")
+    _i32(top_k, "top_k")
+    _i32(draw_index, "draw_index")
+    _i32(out, "out")
+    _check(_fn("sampling", "mi_sample")(_p(logits), B, V, padded, _p(temperature), _p(top_k), _p(top_p),
+                                        _p(seeds), _p(draw_index), _p(keys), _p(out), _stream()), "sample")

@@ -1,0 +1,81 @@
+"""What every part of a layer looks like from outside, and the registry of part kinds.
+
+A part is built from its spec (sizes and constants as fields), the path of its
+tensors, the tensors themselves and a ``BuildContext``; it never learns which model it
+is in.  ``register_part(kind)`` maps the ``kind`` string of a spec dataclass to the class
+that runs it, so a new mixer, feed-forward, norm or position encoding is added by
+registering a class, without a change to this package.
+
+Interfaces
+----------
+every part      ``expected_tensors(spec, prefix, hidden_size) -> [Expect]`` (classmethod),
+                ``kernel_modules`` (names of the HIP modules it launches),
+                ``__init__(spec, prefix, tensors, build)``
+mixer           ``cache_needs(spec) -> [KVNeed | StateNeed]`` (classmethod);
+                ``forward(x [T, d], step, cache: EntryCache) -> [T, d]``
+feed-forward    ``forward(x [T, d]) -> [T, d]``
+norm            ``forward(residual, rows=None) -> normed activations``
+position        ``rotate_and_store(qkv, heads, kv_heads, head_dim, step, cache)``
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import torch
+
+_PARTS: Dict[str, type] = {}
+
+
+def register_part(kind: str):
+    def decorate(cls):
+        _PARTS[kind] = cls
+        cls.kind = kind
+        return cls
+    return decorate
+
+
+def part_class(spec) -> type:
+    kind = getattr(spec, "kind", None)
+    if kind not in _PARTS:
+        raise KeyError(f"no part is registered for kind {kind!r}; registered: {sorted(_PARTS)}")
+    return _PARTS[kind]
+
+
+@dataclass
+class BuildContext:
+    hidden_size: int
+    dtype: torch.dtype            # activation dtype: torch.float32 or torch.bfloat16
+    device: torch.device
+    max_context: int
+
+
+class Residual:
+    """The float32 residual stream [T, d] plus the branch outputs not yet added to it.
+    The next norm adds them and normalizes in one kernel."""
+
+    def __init__(self, h: torch.Tensor):
+        self.h = h
+        self.pending: List[torch.Tensor] = []
+
+
+class Part:
+    kernel_modules = ()
+
+    @classmethod
+    def expected_tensors(cls, spec, prefix: str, hidden_size: int):
+        return []
+
+
+class Mixer(Part):
+    @classmethod
+    def cache_needs(cls, spec):
+        return []
+
+    def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError

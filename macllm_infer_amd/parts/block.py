@@ -1,0 +1,65 @@
+"""Arrangements of parts in a layer."""
+from __future__ import annotations
+
+from typing import Dict
+
+from .base import BuildContext, Residual, part_class
+
+_ARRANGEMENTS: Dict[str, type] = {}
+
+
+def register_arrangement(name: str):
+    def decorate(cls):
+        _ARRANGEMENTS[name] = cls
+        return cls
+    return decorate
+
+
+def arrangement_class(name: str) -> type:
+    if name not in _ARRANGEMENTS:
+        raise KeyError(f"no arrangement named {name!r}; registered: {sorted(_ARRANGEMENTS)}")
+    return _ARRANGEMENTS[name]
+
+
+@register_arrangement("parallel_prenorm")
+class ParallelPreNormBlock:
+    """n = norm(h); h += sum over mixers of mixer(n); h += ffn(norm(h)).
+    All mixers read the same normed input and their outputs are summed into the residual
+    (reference: src/decoder.rs:2658-2682, 2684-2699).  With one mixer this is the ordinary
+    sequential pre-norm layer."""
+
+    @classmethod
+    def expected_tensors(cls, layer, hidden_size: int):
+        out = []
+        out += part_class(layer.mixer_norm).expected_tensors(
+            layer.mixer_norm, f"{layer.prefix}.{layer.mixer_norm_name}", hidden_size)
+        for slot in layer.mixers:
+            out += part_class(slot.spec).expected_tensors(slot.spec, f"{layer.prefix}.{slot.name}", hidden_size)
+        out += part_class(layer.ffn_norm).expected_tensors(
+            layer.ffn_norm, f"{layer.prefix}.{layer.ffn_norm_name}", hidden_size)
+        out += part_class(layer.ffn).expected_tensors(layer.ffn, f"{layer.prefix}.{layer.ffn_name}", hidden_size)
+        return out
+
+    @classmethod
+    def kernel_modules(cls, layer):
+        modules = []
+        for spec in [layer.mixer_norm, layer.ffn_norm, layer.ffn] + [slot.spec for slot in layer.mixers]:
+            modules += list(part_class(spec).kernel_modules)
+        return modules
+
+    def __init__(self, layer, tensors, build: BuildContext):
+        self.layer = layer
+        self.mixer_norm = part_class(layer.mixer_norm)(
+            layer.mixer_norm, f"{layer.prefix}.{layer.mixer_norm_name}", tensors, build)
+        self.mixers = [(slot.name, part_class(slot.spec)(slot.spec, f"{layer.prefix}.{slot.name}", tensors, build))
+                       for slot in layer.mixers]
+        self.ffn_norm = part_class(layer.ffn_norm)(
+            layer.ffn_norm, f"{layer.prefix}.{layer.ffn_norm_name}", tensors, build)
+        self.ffn = part_class(layer.ffn)(layer.ffn, f"{layer.prefix}.{layer.ffn_name}", tensors, build)
+
+    def forward(self, residual: Residual, step, caches) -> None:
+        """``caches``: mixer name -> EntryCache of this run of the layer."""
+        normed = self.mixer_norm.forward(residual)
+        residual.pending = [mixer.forward(normed, step, caches[name]) for name, mixer in self.mixers]
+        normed = self.ffn_norm.forward(residual)
+        residual.pending = [self.ffn.forward(normed)]

@@ -1,0 +1,40 @@
+"""RMSNorm fused with the residual add that precedes it."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from ..weights.loader import Expect
+from .base import BuildContext, Part, Residual, register_part
+
+
+@register_part("rmsnorm")
+class RmsNorm(Part):
+    """y = x / sqrt(mean(x^2) + eps) * w, statistics in float32
+    (reference: src/model_weights.rs:563-565, golden src/decoder.rs:10331-10334)."""
+    kernel_modules = ("common",)
+
+    @classmethod
+    def expected_tensors(cls, spec, prefix: str, hidden_size: int):
+        return [Expect(f"{prefix}.weight", ((hidden_size,),), init="norm")]
+
+    def __init__(self, spec, prefix: str, tensors, build: BuildContext):
+        self.eps = spec.eps
+        self.build = build
+        self.weight = tensors[f"{prefix}.weight"].to(torch.float32).contiguous().to(build.device)
+
+    def forward(self, residual: Residual, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Add the pending branch outputs to the residual stream and return its normed rows
+        (all of them, or only ``rows``; with ``rows`` the stream itself is left unchanged)."""
+        pending = residual.pending
+        while len(pending) > 2:                    # more than two branches: add the extra ones first
+            ops.add_rmsnorm(residual.h, pending[:2], self.weight, self.eps, None)
+            pending = pending[2:]
+        count = residual.h.shape[0] if rows is None else rows.numel()
+        out = torch.empty((count, residual.h.shape[1]), dtype=self.build.dtype, device=residual.h.device)
+        ops.add_rmsnorm(residual.h, pending, self.weight, self.eps, out, rows)
+        if rows is None:
+            residual.pending = []
+        return out

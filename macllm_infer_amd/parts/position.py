@@ -1,0 +1,49 @@
+"""Position encodings applied to q and k before the cache write."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import BuildContext, Part, register_part
+
+
+class PositionEncoding(Part):
+    """Interface: ``rotate_and_store`` encodes the absolute positions ``step.positions`` into
+    the q and k heads of ``qkv`` (q in place) and, if ``cache.owns_kv``, writes the encoded
+    k and the raw v of every token into the cache cell ``step.slot_mappings[cache.group]``.
+    A subclass may implement only ``rotate`` (in place on ``qkv``); the store is then done
+    by the cache-write kernel without rotation."""
+    kernel_modules = ("attention",)
+
+    def rotate(self, qkv, num_heads, num_kv_heads, head_dim, step) -> None:
+        return None
+
+    def rotate_and_store(self, qkv, num_heads, num_kv_heads, head_dim, step, cache) -> None:
+        self.rotate(qkv, num_heads, num_kv_heads, head_dim, step)
+        if cache.owns_kv:
+            ops.rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, step.positions, None, 0,
+                              step.slot_mappings[cache.group], cache.k_cache, cache.v_cache)
+
+
+@register_part("none")
+class NoPosition(PositionEncoding):
+    def __init__(self, spec, head_dim: int, build: BuildContext):
+        pass
+
+
+@register_part("rope")
+class Rope(PositionEncoding):
+    """Half-split rotary encoding: f_j = theta^(-2j/rotary_dim) formed in float64 and rounded
+    to float32; angle = position * f_j, cos and sin in float32
+    (reference: src/decoder.rs:136-144, 186-195, 226-229)."""
+
+    def __init__(self, spec, head_dim: int, build: BuildContext):
+        self.rotary_dim = spec.rotary_dim
+        frequencies = [1.0 / (spec.theta ** (index / spec.rotary_dim)) for index in range(0, spec.rotary_dim, 2)]
+        self.inv_freq = torch.tensor(frequencies, dtype=torch.float64).to(torch.float32).to(build.device)
+
+    def rotate_and_store(self, qkv, num_heads, num_kv_heads, head_dim, step, cache) -> None:
+        owns = cache.owns_kv
+        ops.rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, step.positions, self.inv_freq,
+                          self.rotary_dim, step.slot_mappings[cache.group] if owns else None,
+                          cache.k_cache if owns else None, cache.v_cache if owns else None)

@@ -1,0 +1,171 @@
+"""Plain PyTorch float32 versions of the HIP operations, with the same signatures and the
+same effects on the same (paged, slotted) buffers.
+
+Two uses: GPU tests run a kernel and its reference here on copies of the same inputs and
+compare; CPU tests install these in place of the kernels (``install``) to exercise the
+cache manager, the step function and the scheduler where there is no GPU.  They are test
+doubles only: the package itself has no CPU path.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def _f(t):
+    return t.float()
+
+
+def embed(token_ids, table, multiplier, out):
+    out.copy_(_f(table)[token_ids.long()] * multiplier)
+
+
+def add_rmsnorm(h, deltas, weight, eps, out, rows=None):
+    total = h.clone()
+    for delta in deltas:
+        total += _f(delta)
+    if rows is None:
+        if deltas:
+            h.copy_(total)
+        picked = total
+    else:
+        picked = total[rows.long()]
+    if out is not None:
+        normed = picked / torch.sqrt(picked.pow(2).mean(-1, keepdim=True) + eps) * weight
+        out.copy_(normed.to(out.dtype))
+
+
+def swiglu(gate_up, out):
+    inner = gate_up.shape[1] // 2
+    out.copy_((F.silu(_f(gate_up[:, :inner])) * _f(gate_up[:, inner:])).to(out.dtype))
+
+
+def scale_to_f32(values, multiplier, out):
+    out.copy_(_f(values).reshape(out.shape) * multiplier)
+
+
+def linear(x, weight, bias):
+    y = _f(x) @ _f(weight).T
+    if bias is not None:
+        y = y + bias
+    return y.to(x.dtype)
+
+
+def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, rotary_dim, slot_mapping,
+                  k_cache, v_cache):
+    T = qkv.shape[0]
+    q_cols = num_heads * head_dim
+    k_cols = num_kv_heads * head_dim
+    q = _f(qkv[:, :q_cols]).reshape(T, num_heads, head_dim)
+    k = _f(qkv[:, q_cols:q_cols + k_cols]).reshape(T, num_kv_heads, head_dim)
+    v = qkv[:, q_cols + k_cols:q_cols + 2 * k_cols].reshape(T, num_kv_heads, head_dim)
+    if inv_freq is not None and rotary_dim > 0:
+        half = rotary_dim // 2
+        angle = positions.to(torch.float32)[:, None] * inv_freq[None, :]
+        cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+
+        def rotate(x):
+            a, b = x[..., :half], x[..., half:rotary_dim]
+            return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., rotary_dim:]], dim=-1)
+        q, k = rotate(q), rotate(k)
+    qkv[:, :q_cols] = q.reshape(T, q_cols).to(qkv.dtype)
+    if slot_mapping is not None:
+        page_size = k_cache.shape[2]
+        pages = (slot_mapping // page_size).long()
+        offsets = (slot_mapping % page_size).long()
+        k_cache[pages, :, offsets, :] = k.to(k_cache.dtype)
+        v_cache[pages, :, offsets, :] = v.to(v_cache.dtype)
+
+
+def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token,
+                    positions, scale, window, out):
+    T = q.shape[0]
+    page_size = k_cache.shape[2]
+    group = num_heads // num_kv_heads
+    for token in range(T):
+        lane = int(lane_of_token[token])
+        position = int(positions[token])
+        first = 0 if not window else max(0, position - window + 1)
+        keys = torch.arange(first, position + 1)
+        pages = block_tables[lane][(keys // page_size).long()].long()
+        offsets = (keys % page_size).long()
+        k = _f(k_cache[pages, :, offsets, :])        # [keys, Hkv, dh]
+        v = _f(v_cache[pages, :, offsets, :])
+        for head in range(num_heads):
+            query = _f(q[token, head * head_dim:(head + 1) * head_dim])
+            scores = (k[:, head // group, :] @ query) * scale
+            weights = torch.softmax(scores, dim=0)
+            out[token, head * head_dim:(head + 1) * head_dim] = (weights @ v[:, head // group, :]).to(out.dtype)
+
+
+def conv1d_silu(u, col_offset, width, weight, bias, conv_state, lane_of_token, cu_seqlens, slot_ids, out):
+    K = weight.shape[1]
+    for lane in range(slot_ids.numel()):
+        begin, end = int(cu_seqlens[lane]), int(cu_seqlens[lane + 1])
+        rows = _f(u[begin:end, col_offset:col_offset + width])
+        window = torch.cat([_f(conv_state[int(slot_ids[lane])]), rows], dim=0)
+        total = torch.zeros(end - begin, width)
+        for tap in range(K):
+            total += window[tap:tap + end - begin] * weight[:, tap][None, :]
+        if bias is not None:
+            total += bias[None, :]
+        out[begin:end] = F.silu(total).to(out.dtype)
+
+
+def conv_state_update(u, col_offset, width, kernel, conv_state, cu_seqlens, slot_ids):
+    if kernel <= 1:
+        return
+    for lane in range(slot_ids.numel()):
+        begin, end = int(cu_seqlens[lane]), int(cu_seqlens[lane + 1])
+        slot = int(slot_ids[lane])
+        window = torch.cat([conv_state[slot], u[begin:end, col_offset:col_offset + width]], dim=0)
+        conv_state[slot] = window[-(kernel - 1):]
+
+
+def ssm_scan(xbc, dt, dt_bias, A, D, ssm_state, cu_seqlens, slot_ids, num_groups, y):
+    _, H, P, N = ssm_state.shape
+    E = H * P
+    GN = num_groups * N
+    group_of_head = torch.arange(H) // (H // num_groups)
+    for lane in range(slot_ids.numel()):
+        begin, end = int(cu_seqlens[lane]), int(cu_seqlens[lane + 1])
+        slot = int(slot_ids[lane])
+        state = ssm_state[slot].clone()
+        for t in range(begin, end):
+            row = _f(xbc[t])
+            x = row[:E].reshape(H, P)
+            B = row[E:E + GN].reshape(num_groups, N)[group_of_head]
+            C = row[E + GN:].reshape(num_groups, N)[group_of_head]
+            raw = _f(dt[t]) + dt_bias
+            delta = torch.clamp(raw, min=0) + torch.log1p(torch.exp(-raw.abs()))
+            decay = torch.exp(delta * A)
+            state = state * decay[:, None, None] + (delta[:, None] * x)[:, :, None] * B[:, None, :]
+            y[t] = ((state * C[:, None, :]).sum(-1) + D[:, None] * x).reshape(E)
+        ssm_state[slot] = state
+
+
+def gate_norm(y, z, weight, num_groups, eps, out):
+    T, E = y.shape
+    v = y * F.silu(_f(z))
+    if weight is not None:
+        grouped = v.reshape(T, num_groups, E // num_groups)
+        grouped = grouped / torch.sqrt(grouped.pow(2).mean(-1, keepdim=True) + eps)
+        v = grouped.reshape(T, E) * weight[None, :]
+    out.copy_(v.to(out.dtype))
+
+
+def argmax(logits, out):
+    out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
+
+
+NAMES = ["embed", "add_rmsnorm", "swiglu", "scale_to_f32", "linear", "rope_kv_store", "paged_attention",
+         "conv1d_silu", "conv_state_update", "ssm_scan", "gate_norm", "argmax"]
+
+
+def install(monkeypatch):
+    """Replace the package's kernels with the functions above for one test."""
+    from macllm_infer_amd.kernels import ops
+    for name in NAMES:
+        monkeypatch.setattr(ops, name, globals()[name])

@@ -1,0 +1,38 @@
+"""The two tiny Falcon-H1 configurations of the test-suite.  They differ in every size
+and option: layers, width, heads and groups, head size, feed-forward width, SSM heads,
+head size, state size, groups, conv taps, chunk, biases, gated norm, tied embeddings,
+multipliers, rope base, norm eps and vocabulary."""
+import torch
+
+from macllm_infer_amd.config import FalconH1Config
+from macllm_infer_amd.weights.random_init import random_tensors, write_random_model
+
+TINY_A = dict(
+    architectures=["FalconH1ForCausalLM"], model_type="falcon_h1",
+    hidden_size=64, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+    intermediate_size=128, vocab_size=256, max_position_embeddings=1024, rms_norm_eps=1e-5, rope_theta=1e4,
+    mamba_n_heads=8, mamba_d_head=8, mamba_d_ssm=64, mamba_d_state=16, mamba_n_groups=1, mamba_d_conv=4,
+    mamba_chunk_size=16, mamba_conv_bias=False, mamba_proj_bias=False, mamba_rms_norm=False,
+    attention_bias=False, mlp_bias=False, tie_word_embeddings=True)
+
+TINY_B = dict(
+    architectures=["FalconH1ForCausalLM"], model_type="falcon_h1",
+    hidden_size=96, num_hidden_layers=3, num_attention_heads=6, num_key_value_heads=3, head_dim=32,
+    intermediate_size=160, vocab_size=320, max_position_embeddings=768, rms_norm_eps=3e-6, rope_theta=1e11,
+    mamba_n_heads=6, mamba_d_head=16, mamba_d_ssm=96, mamba_d_state=32, mamba_n_groups=2, mamba_d_conv=3,
+    mamba_chunk_size=8, mamba_conv_bias=True, mamba_proj_bias=True, mamba_rms_norm=True,
+    attention_bias=True, mlp_bias=True, tie_word_embeddings=False,
+    embedding_multiplier=1.7, lm_head_multiplier=0.6, attention_in_multiplier=1.3,
+    attention_out_multiplier=0.8, key_multiplier=0.7, ssm_in_multiplier=1.2, ssm_out_multiplier=0.9,
+    ssm_multipliers=[0.8, 1.4, 0.6, 1.5, 1.1], mlp_multipliers=[1.25, 0.75])
+
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1)}
+
+
+def config(name):
+    return FalconH1Config.from_dict(CONFIGS[name][0])
+
+
+def make_model_dir(name, folder, dtype=torch.float32, preset="unit"):
+    raw, seed = CONFIGS[name]
+    return write_random_model(FalconH1Config.from_dict(raw), seed, str(folder), dtype, preset)
