@@ -1,0 +1,202 @@
+"""Continuous batching above the step function.
+
+Each round (reference: ``ServingScheduler::drive_once``, src/engine.rs:1938-1988):
+  1. admit queued requests while fewer than ``max_active_sequences`` are live
+     (FIFO; a request that could never fit is rejected up front, :2839-2863);
+  2. visit the live requests in queue order under a token budget: a decoding request
+     costs one token, a prefilling one gets ``min(prefill_token_quantum, rest of the
+     prompt, budget left)`` (:2005-2095); requests not reached keep their place;
+  3. run all chosen lanes as one step.  If the pages do not suffice the last lane is
+     dropped and the step retried (:2145-2149); if a single lane cannot fit, that request
+     alone fails with ``resource_exhausted`` and gives back what it holds (:2150-2153,
+     :2205-2231).  There is no preemption or swap;
+  4. sample for the lanes whose last prompt token or decoded token ran; a stop token ends
+     the request without being emitted, ``max_new_tokens`` ends it with the token emitted
+     (src/generation.rs:1221-1263);
+  5. finished requests give back pages and slot; visited ones go to the back of the line.
+"""
+from __future__ import annotations
+
+import time
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Callable, Deque, Dict, Hashable, List, Optional, Sequence
+
+from ..cache.pages import CacheExhausted
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import SamplerRow
+from .context import Lane
+
+
+@dataclass
+class EngineConfig:
+    """Scheduler knobs, with the reference's names (src/engine.rs:309-385).  The reference's
+    defaults (2 / 256 / 128 / 8) are sized for a laptop; these are sized for one MI355X."""
+    max_active_sequences: int = 64
+    scheduler_token_budget: int = 4096
+    prefill_token_quantum: int = 2048
+    queue_capacity: int = 4096
+
+    def __post_init__(self):
+        if min(self.max_active_sequences, self.scheduler_token_budget, self.prefill_token_quantum,
+               self.queue_capacity) <= 0:
+            raise ValueError("scheduler settings must be positive")
+        if self.prefill_token_quantum > self.scheduler_token_budget:
+            raise ValueError("prefill_token_quantum cannot exceed scheduler_token_budget")
+
+
+@dataclass
+class Request:
+    request_id: Hashable
+    prompt: List[int]
+    params: SamplingParams
+    generated: List[int] = field(default_factory=list)
+    cursor: int = 0                        # prompt tokens already in the cache
+    finish_reason: Optional[str] = None    # "stop", "length", "resource_exhausted", "rejected: ..."
+    submitted_at: float = 0.0
+    first_token_at: Optional[float] = None
+    finished_at: Optional[float] = None
+
+    @property
+    def finished(self) -> bool:
+        return self.finish_reason is not None
+
+    @property
+    def prefilling(self) -> bool:
+        return self.cursor < len(self.prompt)
+
+
+class QueueFull(RuntimeError):
+    pass
+
+
+class Scheduler:
+    def __init__(self, engine, sampler, config: Optional[EngineConfig] = None,
+                 stop_token_ids: Sequence[int] = (), on_token: Optional[Callable] = None):
+        """``engine``: add_request / finish / step(lanes) / cache.can_ever_fit / vocab_size /
+        max_context.  ``sampler``: sample(logits, rows) -> tokens."""
+        self.engine = engine
+        self.sampler = sampler
+        self.config = config or EngineConfig()
+        self.stop_token_ids = set(int(token) for token in stop_token_ids)
+        self.on_token = on_token
+        self.queue: Deque[Request] = deque()
+        self.active: Deque[Request] = deque()
+        self.finished: Dict[Hashable, Request] = {}
+        self.rounds = 0
+        self.last_lanes: List[Lane] = []        # what the last round ran (for tests and metrics)
+
+    # ------------------------------------------------------------------ submission
+    def submit(self, request_id: Hashable, prompt: Sequence[int], params: SamplingParams) -> Request:
+        if len(self.queue) >= self.config.queue_capacity:
+            raise QueueFull(f"the queue holds {len(self.queue)} requests, its capacity")
+        request = Request(request_id, [int(token) for token in prompt], params, submitted_at=time.perf_counter())
+        self.queue.append(request)
+        return request
+
+    def has_work(self) -> bool:
+        return bool(self.queue or self.active)
+
+    # ------------------------------------------------------------------ one round
+    def _reject(self, request: Request, why: str) -> None:
+        request.finish_reason = f"rejected: {why}"
+        request.finished_at = time.perf_counter()
+        self.finished[request.request_id] = request
+
+    def _admit(self) -> None:
+        while self.queue and len(self.active) < self.config.max_active_sequences:
+            request = self.queue.popleft()
+            needed = len(request.prompt) + request.params.max_new_tokens - 1
+            if not request.prompt:
+                self._reject(request, "prompt must contain at least one token")
+            elif any(not (0 <= token < self.engine.vocab_size) for token in request.prompt):
+                self._reject(request, "input contains a token ID outside the model vocabulary")
+            elif needed > self.engine.max_context:
+                self._reject(request, "prompt plus requested output exceeds model context limit")
+            elif not self.engine.cache.can_ever_fit(needed):
+                self._reject(request, "prompt plus requested output exceeds the cache capacity")
+            else:
+                self.engine.add_request(request.request_id)
+                self.active.append(request)
+
+    def _collect(self) -> List[tuple]:
+        """(request, tokens, samples?) for this round, in queue order under the budget."""
+        budget = self.config.scheduler_token_budget
+        visits = []
+        for request in self.active:
+            if budget <= 0:
+                break
+            if request.prefilling:
+                count = min(self.config.prefill_token_quantum, len(request.prompt) - request.cursor, budget)
+                tokens = request.prompt[request.cursor:request.cursor + count]
+                samples = request.cursor + count == len(request.prompt)
+            else:
+                tokens = [request.generated[-1]]
+                samples = True
+            budget -= len(tokens)
+            visits.append((request, tokens, samples))
+        return visits
+
+    def _finish(self, request: Request, reason: str) -> None:
+        request.finish_reason = reason
+        request.finished_at = time.perf_counter()
+        self.engine.finish(request.request_id)
+        self.active.remove(request)
+        self.finished[request.request_id] = request
+
+    def step(self) -> List[Request]:
+        """One round; returns the requests that finished in it."""
+        self.rounds += 1
+        done_before = set(self.finished)
+        self._admit()
+        visits = self._collect()
+        logits = None
+        while visits:
+            lanes = [Lane(request.request_id, tokens, [len(tokens) - 1] if samples else [])
+                     for request, tokens, samples in visits]
+            try:
+                logits = self.engine.step(lanes)
+                self.last_lanes = lanes
+                break
+            except CacheExhausted:
+                if len(visits) > 1:
+                    visits.pop()                 # the last lane waits for a later round
+                else:
+                    self._finish(visits[0][0], "resource_exhausted")
+                    visits = self._collect()
+        if visits:
+            sampled = [(request, tokens) for request, tokens, samples in visits if samples]
+            for request, tokens, samples in visits:
+                if request.prefilling:
+                    request.cursor += len(tokens)
+            if sampled:
+                rows = [SamplerRow(request.params, request.prompt, request.generated) for request, _ in sampled]
+                tokens_out = self.sampler.sample(logits, rows)
+                now = time.perf_counter()
+                for (request, _), token in zip(sampled, tokens_out):
+                    self._complete(request, int(token), now)
+            for request, _, _ in visits:         # visited requests go to the back of the line
+                if not request.finished:
+                    self.active.remove(request)
+                    self.active.append(request)
+        return [request for key, request in self.finished.items() if key not in done_before]
+
+    def _complete(self, request: Request, token: int, now: float) -> None:
+        params = request.params
+        stops = self.stop_token_ids | set(params.stop_token_ids)
+        if not params.ignore_eos and token in stops:
+            self._finish(request, "stop")            # the stop token is not emitted
+            return
+        if request.first_token_at is None:
+            request.first_token_at = now
+        request.generated.append(token)
+        if self.on_token is not None:
+            self.on_token(request, token)
+        if len(request.generated) >= params.max_new_tokens:
+            self._finish(request, "length")
+
+    def run(self) -> Dict[Hashable, Request]:
+        """Rounds until every submitted request has finished."""
+        while self.has_work():
+            self.step()
+        return self.finished

@@ -1,0 +1,94 @@
+"""Sampling on the GPU over rows of float32 logits.
+
+Order of operations, as the reference's sampler (src/sampling.rs:95-161): repetition
+penalty over prompt and generated tokens, presence and frequency penalties over generated
+tokens, then argmax (lowest index on ties) or temperature -> top-k -> softmax -> top-p ->
+one uniform draw, walked in index order.  One draw per stochastic token; the uniform
+comes from a counter-based generator keyed by (seed, number of tokens drawn so far), so a
+request's tokens do not depend on what else is in the batch.
+"""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+
+from ..kernels import build as kernel_build
+from ..kernels import ops
+from .params import SamplingParams
+
+
+class SamplerRow:
+    """What the sampler needs to know of one request."""
+    __slots__ = ("params", "prompt", "generated")
+
+    def __init__(self, params: SamplingParams, prompt: Sequence[int], generated: Sequence[int]):
+        self.params, self.prompt, self.generated = params, prompt, generated
+
+
+class Sampler:
+    kernel_modules = ("sampling",)
+
+    def __init__(self, vocab_size: int, device, check_device: bool = True):
+        self.vocab_size = vocab_size
+        self.device = torch.device(device)
+        self.padded = 1
+        while self.padded < vocab_size:
+            self.padded <<= 1
+        if check_device:
+            ops.require_gpu(device)
+            kernel_build.ensure_modules(self.kernel_modules)
+        self._keys = None
+        self._counts = None
+
+    def _work(self, rows: int):
+        if self._keys is None or self._keys.shape[0] < rows:
+            self._keys = torch.empty((rows, self.padded), dtype=torch.int64, device=self.device)
+        return self._keys
+
+    def _count_areas(self, rows: int):
+        if self._counts is None or self._counts[0].numel() < rows * self.vocab_size:
+            self._counts = (torch.zeros(rows * self.vocab_size, dtype=torch.int32, device=self.device),
+                            torch.zeros(rows * self.vocab_size, dtype=torch.int32, device=self.device))
+        return self._counts
+
+    def sample(self, logits: torch.Tensor, rows: Sequence[SamplerRow]) -> List[int]:
+        """One token for each row of ``logits`` [B, V] (float32; overwritten)."""
+        B = len(rows)
+        if logits.shape != (B, self.vocab_size):
+            raise ValueError(f"logits have shape {tuple(logits.shape)}, expected {(B, self.vocab_size)}")
+        device = self.device
+
+        def upload(values, dtype):
+            return torch.tensor(values, dtype=dtype).to(device, non_blocking=True)
+
+        if any(row.params.uses_penalties for row in rows):
+            tokens: List[int] = []
+            offsets = [0]
+            for row in rows:
+                if row.params.uses_penalties:
+                    tokens.extend(row.prompt)
+                    tokens.extend(row.generated)
+                offsets.append(len(tokens))
+            count_all, count_gen = self._count_areas(B)
+            ops.apply_penalties(
+                logits, upload(tokens or [0], torch.int32), upload(offsets, torch.int32),
+                upload([len(row.prompt) for row in rows], torch.int32),
+                upload([row.params.repetition_penalty for row in rows], torch.float32),
+                upload([row.params.presence_penalty for row in rows], torch.float32),
+                upload([row.params.frequency_penalty for row in rows], torch.float32), count_all, count_gen)
+        out = torch.empty(B, dtype=torch.int32, device=device)
+        if all(row.params.greedy for row in rows):
+            ops.argmax(logits, out)
+        else:
+            def as_signed(seed: int) -> int:
+                seed &= (1 << 64) - 1
+                return seed - (1 << 64) if seed >= (1 << 63) else seed
+            ops.sample(logits,
+                       upload([row.params.temperature for row in rows], torch.float32),
+                       upload([row.params.top_k for row in rows], torch.int32),
+                       upload([row.params.top_p for row in rows], torch.float32),
+                       upload([as_signed(row.params.seed) for row in rows], torch.int64),
+                       upload([len(row.generated) for row in rows], torch.int32),
+                       self._work(B), out)
+        return out.cpu().tolist()
