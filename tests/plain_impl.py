@@ -86,7 +86,7 @@ def gqa_causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scal
     T, Hq, dh = q.shape
     Hkv = k.shape[1]
     group = Hq // Hkv
-    out = torch.empty_like(q)
+    out = torch.empty(T, Hq, v.shape[-1])
     position = torch.arange(T)
     masked = position[None, :] > position[:, None]
     if window is not None:

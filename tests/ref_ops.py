@@ -169,3 +169,28 @@ def install(monkeypatch):
     from macllm_infer_amd.kernels import ops
     for name in NAMES:
         monkeypatch.setattr(ops, name, globals()[name])
+
+
+def apply_penalties(logits, tokens, offsets, prompt_lens, repetition, presence, frequency, count_all, count_gen):
+    for row in range(logits.shape[0]):
+        history = tokens[int(offsets[row]):int(offsets[row + 1])].tolist()
+        generated = history[int(prompt_lens[row]):]
+        rep, pres, freq = float(repetition[row]), float(presence[row]), float(frequency[row])
+        if rep > 0 and abs(rep - 1.0) >= 1.1920929e-07:
+            for token in set(history):
+                value = logits[row, token]
+                logits[row, token] = value * rep if value < 0 else value / rep
+        if pres != 0.0 or freq != 0.0:
+            for token in set(generated):
+                logits[row, token] -= freq * generated.count(token) + pres
+
+
+def sample(logits, temperature, top_k, top_p, seeds, draw_index, keys, out):
+    import plain_impl
+    for row in range(logits.shape[0]):
+        out[row] = plain_impl.sample_token(
+            logits[row], temperature=float(temperature[row]), top_k=int(top_k[row]), top_p=float(top_p[row]),
+            seed=int(seeds[row]) & ((1 << 64) - 1), draw_index=int(draw_index[row]))
+
+
+NAMES += ["apply_penalties", "sample"]

@@ -1,0 +1,176 @@
+"""The cache manager on the CPU: no page lost, held twice or freed twice under random
+orders of requests; exhaustion is typed and changes nothing; windows give pages back;
+slots are zeroed when they are handed out again."""
+import random
+
+import pytest
+import torch
+
+from macllm_infer_amd.cache import CacheExhausted, CacheManager, KVNeed, PagePool, SlotPool, StateNeed
+
+
+def make(capacity=64, page=8, requests=3, window=None):
+    needs = {(0, "attn"): [KVNeed(2, 4, None)], (1, "attn"): [KVNeed(2, 4, None)],
+             (1, "rec"): [StateNeed("s", (3, 2), "float32"), StateNeed("c", (2, 5), "activation")]}
+    if window:
+        needs[(2, "attn")] = [KVNeed(2, 4, window)]
+    return CacheManager(needs, {}, page, capacity, requests, torch.float32, "cpu")
+
+
+def test_page_pool_invariants():
+    pool = PagePool(5)
+    first = pool.alloc(3)
+    assert len(set(first)) == 3 and pool.free_count == 2
+    with pytest.raises(CacheExhausted) as caught:
+        pool.alloc(3)
+    assert (caught.value.requested, caught.value.free, caught.value.total) == (3, 2, 5)
+    assert pool.free_count == 2                                   # nothing changed
+    pool.free(first[:1])
+    with pytest.raises(RuntimeError, match="not held"):
+        pool.free(first[:1])                                      # freed twice
+    assert pool.alloc(1) == first[:1]                             # most recently freed page comes back first
+    pool.check(first + [])
+    with pytest.raises(AssertionError):
+        pool.check(first[:2])                                     # a page lost
+
+
+def test_groups_share_a_table_per_geometry_and_windows_get_their_own():
+    cache = make(window=10)
+    assert len(cache.groups) == 2
+    assert cache.groups[0].storage.shape == (8, 2, 2, 2, 8, 4)    # [page, layer, K|V, kv head, token, dim]
+    assert cache.groups[1].need.window == 10 and len(cache.groups[1].members) == 1
+    first, second = cache.entry((0, "attn")), cache.entry((1, "attn"))
+    assert first.group == second.group == 0 and first.k_cache.data_ptr() != second.k_cache.data_ptr()
+    assert cache.entry((1, "rec")).states["s"].shape == (3, 3, 2)
+    assert cache.entry((1, "rec")).states["c"].dtype == torch.float32
+
+
+def test_reservation_is_all_or_nothing():
+    cache = make(capacity=32, page=8)                             # 4 pages
+    cache.add_request("a")
+    cache.add_request("b")
+    cache.reserve([("a", 9)])                                     # 2 pages
+    cache.commit("a", 9)
+    before = cache.stats()
+    with pytest.raises(CacheExhausted) as caught:
+        cache.reserve([("a", 8), ("b", 9)])                       # a: +1 page, b: +2 pages > 2 free
+    assert caught.value.requested == 3 and caught.value.free == 2
+    assert cache.stats() == before and cache.table(0, "b").pages == []
+    cache.reserve([("a", 7), ("b", 8)])                           # a stays within page 2; b takes 1
+    assert cache.stats()["groups"][0]["free_pages"] == 1
+    cache.check()
+
+
+def test_pages_per_request_and_reuse_after_finish():
+    cache = make(capacity=32, page=8)
+    cache.add_request("a")
+    for length, pages in ((1, 1), (8, 1), (9, 2), (17, 3)):
+        cache.reserve([("a", length - cache.requests["a"].length)])
+        cache.commit("a", length - cache.requests["a"].length)
+        assert len(cache.table(0, "a").pages) == pages == -(-length // 8)
+    held = list(cache.table(0, "a").pages)
+    cache.finish("a")
+    assert cache.stats()["groups"][0]["free_pages"] == 4 and cache.stats()["free_slots"] == 3
+    cache.add_request("b")
+    cache.reserve([("b", 24)])
+    assert sorted(cache.table(0, "b").pages) == sorted(held)      # the same pages are used again
+    with pytest.raises(KeyError):
+        cache.finish("a")
+
+
+def test_window_group_gives_back_passed_pages():
+    cache = make(capacity=64, page=4, window=6)
+    cache.add_request("a")
+    freed_total = 0
+    for step in range(30):
+        cache.reserve([("a", 1)])
+        cache.commit("a", 1)
+        length = cache.requests["a"].length
+        table = cache.table(1, "a")
+        live = [index for index, page in enumerate(table.pages) if page >= 0]
+        # the next query (position = length) sees keys >= length - 5: every such key's page is live
+        for key in range(max(0, length - 5), length):
+            assert table.pages[key // 4] >= 0
+        assert len(live) <= 3                                      # a window of 6 spans at most 3 pages of 4
+        assert len(cache.table(0, "a").live_pages()) == -(-length // 4)   # the full group keeps all
+        cache.check()
+    assert cache.groups[1].pool.used_count <= 3
+    # a long portion at once: pages for the whole portion are needed during the step, then released
+    cache.add_request("b")
+    cache.reserve([("b", 22)])
+    assert len(cache.table(1, "b").live_pages()) == 6
+    cache.commit("b", 22)
+    assert len(cache.table(1, "b").live_pages()) == 2
+
+
+def test_slots_are_zeroed_when_reused():
+    cache = make(requests=2)
+    cache.add_request("a")
+    slot = cache.requests["a"].slot
+    state = cache.entry((1, "rec")).states["s"]
+    state[slot] = 7.0
+    cache.finish("a")
+    cache.add_request("b")
+    assert cache.requests["b"].slot == slot and (state[slot] == 0).all()
+    cache.add_request("c")
+    with pytest.raises(CacheExhausted, match="state slots"):
+        cache.add_request("d")
+    with pytest.raises(KeyError):
+        cache.add_request("b")
+
+
+def test_can_ever_fit():
+    cache = make(capacity=32, page=8)
+    assert cache.can_ever_fit(32) and not cache.can_ever_fit(33)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_never_lose_or_double_a_page(seed):
+    rng = random.Random(seed)
+    cache = make(capacity=96, page=4, requests=4, window=9)
+    live = {}
+    next_id = 0
+    for _ in range(400):
+        action = rng.random()
+        if action < 0.15 and len(live) < 4:
+            cache.add_request(next_id)
+            live[next_id] = 0
+            next_id += 1
+        elif action < 0.25 and live:
+            victim = rng.choice(list(live))
+            cache.finish(victim)
+            del live[victim]
+        elif live:
+            chosen = rng.sample(list(live), rng.randint(1, len(live)))
+            growth = [(request, rng.choice([1, 1, 1, 2, 5, 11])) for request in chosen]
+            before = cache.stats()
+            try:
+                cache.reserve(growth)
+            except CacheExhausted:
+                assert cache.stats() == before
+                continue
+            for request, tokens in growth:
+                cache.commit(request, tokens)
+                live[request] += tokens
+        cache.check()
+        for request, length in live.items():
+            assert cache.requests[request].length == length
+            assert len(cache.table(0, request).live_pages()) == -(-length // 4)
+        slots = [cache.requests[request].slot for request in live]
+        assert len(set(slots)) == len(slots)
+    for request in list(live):
+        cache.finish(request)
+    stats = cache.stats()
+    assert all(group["free_pages"] == group["total_pages"] for group in stats["groups"])
+    assert stats["free_slots"] == stats["total_slots"]
+
+
+def test_shared_kv_entries_read_the_owner():
+    needs = {(0, "attn"): [KVNeed(2, 4, None)], (1, "attn"): [KVNeed(2, 4, None)]}
+    cache = CacheManager(needs, {(1, "attn"): (0, "attn")}, 8, 32, 2, torch.float32, "cpu")
+    assert len(cache.groups[0].members) == 1
+    reader, owner = cache.entry((1, "attn")), cache.entry((0, "attn"))
+    assert reader.k_cache.data_ptr() == owner.k_cache.data_ptr() and not reader.owns_kv and owner.owns_kv
+    with pytest.raises(ValueError, match="differ"):
+        CacheManager({(0, "attn"): [KVNeed(2, 4, None)], (1, "attn"): [KVNeed(1, 4, None)]},
+                     {(1, "attn"): (0, "attn")}, 8, 32, 2, torch.float32, "cpu")

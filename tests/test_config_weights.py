@@ -1,0 +1,168 @@
+"""Configuration, registry, safetensors reading, weight errors and the random-weights mode."""
+import json
+import os
+
+import pytest
+import torch
+
+import tiny_configs
+from macllm_infer_amd.config import (ConfigError, FalconH1Config, config_from_dict, load_config,
+                                     registered_architectures)
+from macllm_infer_amd.engine.model import DecoderModel
+from macllm_infer_amd.weights import WeightError, WeightSource, bind, write_safetensors
+from macllm_infer_amd.weights.random_init import random_tensors, write_random_model
+
+
+def test_config_reads_its_own_keys_and_defaults():
+    config = FalconH1Config.from_dict(tiny_configs.TINY_B)
+    assert (config.hidden_size, config.num_hidden_layers, config.head_dim) == (96, 3, 32)
+    assert config.num_attention_heads * config.head_dim != config.hidden_size      # heads*dim need not be the width
+    assert config.ssm_multipliers == (0.8, 1.4, 0.6, 1.5, 1.1) and config.mlp_multipliers == (1.25, 0.75)
+    minimal = FalconH1Config.from_dict(dict(
+        model_type="falcon_h1", hidden_size=32, num_hidden_layers=1, num_attention_heads=4,
+        intermediate_size=48, vocab_size=50, max_position_embeddings=64, mamba_n_heads=2, mamba_d_ssm=16,
+        mamba_d_state=8))
+    assert minimal.head_dim == 8 and minimal.num_key_value_heads == 4 and minimal.mamba_d_head == 8
+    assert minimal.mamba_d_conv == 4 and minimal.mamba_n_groups == 1 and minimal.rope_theta == 1e11
+    assert minimal.rms_norm_eps == 1e-5 and minimal.mamba_conv_bias and not minimal.tie_word_embeddings
+    spec = minimal.to_model_spec()
+    assert [slot.name for slot in spec.layers[0].mixers] == ["self_attn", "mamba"]
+    assert spec.layers[0].mixers[0].spec.scale == pytest.approx(8 ** -0.5)
+    assert [entry.layer for entry in spec.schedule] == [0]
+
+
+def test_state_and_cache_sizes_match_the_reference_gate():
+    """Sizes asserted by the reference for Falcon-H1-Tiny-90M (tests/falcon_h1_gguf_reference.rs:50-114):
+    kv bytes/token 12288 at 16-bit, fixed state 4 976 640 B with a float32 conv tail."""
+    config = FalconH1Config.from_dict(dict(
+        model_type="falcon_h1", hidden_size=512, num_hidden_layers=24, num_attention_heads=8,
+        num_key_value_heads=2, head_dim=64, intermediate_size=1024, vocab_size=32768,
+        max_position_embeddings=2048, mamba_n_heads=24, mamba_d_head=32, mamba_d_state=64, mamba_n_groups=1,
+        mamba_d_conv=4))
+    assert config.kv_bytes_per_token(2) == 12288
+    assert config.fixed_state_bytes(4) == 4976640
+
+
+@pytest.mark.parametrize("change, word", [
+    ({"hidden_size": None}, "hidden_size"),
+    ({"num_key_value_heads": 4}, "num_key_value_heads"),
+    ({"mamba_n_groups": 4}, "mamba_n_groups"),
+    ({"mamba_d_ssm": 100}, "mamba_d_ssm"),
+    ({"ssm_multipliers": [1.0, 2.0]}, "ssm_multipliers"),
+    ({"rms_norm_eps": 0.0}, "eps"),
+    ({"head_dim": 31}, "head_dim"),
+    ({"rope_scaling": {"type": "linear", "factor": 2}}, "rope_scaling"),
+    ({"sliding_window": 128}, "sliding_window"),
+    ({"hidden_act": "gelu"}, "hidden_act"),
+    ({"mamba_norm_before_gate": True}, "mamba_norm_before_gate"),
+    ({"vocab_size": "many"}, "vocab_size"),
+    ({"max_position_embeddings": 1 << 21}, "max_position_embeddings"),
+])
+def test_config_errors_name_the_field(change, word):
+    raw = dict(tiny_configs.TINY_B)
+    raw.update(change)
+    if change.get("hidden_size", 0) is None:
+        del raw["hidden_size"]
+    with pytest.raises(ConfigError, match=word):
+        FalconH1Config.from_dict(raw)
+
+
+def test_registry_maps_names_and_lists_them_for_an_unknown_one(tmp_path):
+    assert "FalconH1ForCausalLM" in registered_architectures() and "falcon_h1" in registered_architectures()
+    assert isinstance(config_from_dict(tiny_configs.TINY_A), FalconH1Config)
+    only_type = {k: v for k, v in tiny_configs.TINY_A.items() if k != "architectures"}
+    assert isinstance(config_from_dict(only_type), FalconH1Config)
+    with pytest.raises(ConfigError, match="FalconH1ForCausalLM"):
+        config_from_dict({"architectures": ["SomethingElse"], "hidden_size": 8})
+    with pytest.raises(ConfigError, match="names no architecture"):
+        config_from_dict({"hidden_size": 8})
+    with pytest.raises(ConfigError, match="does not exist"):
+        load_config(str(tmp_path))
+
+
+def test_unknown_keys_are_ignored():
+    raw = dict(tiny_configs.TINY_A, some_future_key=3, torch_dtype="bfloat16")
+    assert FalconH1Config.from_dict(raw) == FalconH1Config.from_dict(tiny_configs.TINY_A)
+
+
+def test_random_model_folder_round_trips_and_keeps_dtypes(tmp_path):
+    folder = tiny_configs.make_model_dir("B", tmp_path / "b", torch.bfloat16)
+    assert sorted(os.listdir(folder)) == ["config.json", "model.safetensors"]
+    config = load_config(folder)
+    assert config == tiny_configs.config("B")
+    source = WeightSource.from_dir(folder)
+    bound = bind(source, DecoderModel.expected_tensors(config.to_model_spec()))
+    assert bound["model.layers.0.mamba.in_proj.weight"].dtype == torch.bfloat16
+    assert bound["model.layers.0.mamba.A_log"].dtype == torch.float32          # stored in 32-bit, stays so
+    assert bound["model.layers.2.mamba.norm.weight"].shape == (2, 48)
+    # the library reads the same bytes
+    from safetensors.torch import load_file
+    theirs = load_file(os.path.join(folder, "model.safetensors"))
+    assert set(theirs) == set(bound)
+    for name, tensor in theirs.items():
+        assert torch.equal(tensor.reshape(bound[name].shape), bound[name]) and tensor.dtype == bound[name].dtype
+    # same seed, same bits; another seed, other bits
+    again = random_tensors(config, 1, torch.bfloat16, "unit")
+    assert all(torch.equal(again[name], bound[name]) for name in bound)
+    other = random_tensors(config, 2, torch.bfloat16, "unit")
+    assert not torch.equal(other["lm_head.weight"], bound["lm_head.weight"])
+
+
+def test_baseline_preset_distributions():
+    tensors = random_tensors(tiny_configs.config("B"), 3, torch.float32, "baseline")
+    assert abs(tensors["lm_head.weight"].std().item() - 0.02) < 0.002
+    assert abs(tensors["model.norm.weight"].mean().item() - 1.0) < 0.05
+    a = torch.exp(tensors["model.layers.0.mamba.A_log"])
+    assert (a >= 1).all() and (a <= 16).all()
+    step = torch.nn.functional.softplus(tensors["model.layers.1.mamba.dt_bias"])
+    assert (step >= 1e-3 * 0.999).all() and (step <= 0.1 * 1.001).all()
+
+
+def test_weight_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    config = tiny_configs.config("A")
+    expectations = DecoderModel.expected_tensors(config.to_model_spec())
+    tensors = random_tensors(config, 0, torch.float32)
+    del tensors["model.layers.1.mamba.D"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.mlp.extra.weight"] = torch.zeros(2)
+    tensors["lm_head.weight"] = torch.zeros(256, 64)                       # tied model: not expected
+    tensors["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(16, 64)
+    tensors["model.layers.0.mamba.dt_bias"] = torch.zeros(8, dtype=torch.int32)
+    path = tmp_path / "model.safetensors"
+    write_safetensors(str(path), tensors)
+    with pytest.raises(WeightError) as caught:
+        bind(WeightSource.from_dir(str(tmp_path)), expectations)
+    error = caught.value
+    assert error.missing == ["model.layers.1.mamba.D", "model.norm.weight"]
+    assert error.unexpected == ["lm_head.weight", "model.layers.0.mlp.extra.weight"]
+    assert [(name, got) for name, _, got in error.wrong_shape] == [("model.layers.0.self_attn.k_proj.weight", (16, 64))]
+    assert error.wrong_dtype[0][0] == "model.layers.0.mamba.dt_bias"
+    text = str(error)
+    for word in ("model.layers.1.mamba.D", "lm_head.weight", "expected [32, 64], got [16, 64]"):
+        assert word in text
+
+
+def test_alternative_shapes_and_widening(tmp_path):
+    config = tiny_configs.config("A")
+    tensors = random_tensors(config, 0, torch.float32)
+    tensors["model.layers.0.mamba.conv1d.weight"] = tensors["model.layers.0.mamba.conv1d.weight"].reshape(96, 1, 4)
+    tensors["model.layers.0.mamba.A_log"] = tensors["model.layers.0.mamba.A_log"].reshape(8, 1).double()
+    tensors["model.layers.0.mamba.D"] = tensors["model.layers.0.mamba.D"].half()
+    bound = bind(WeightSource.from_tensors(tensors), DecoderModel.expected_tensors(config.to_model_spec()))
+    assert bound["model.layers.0.mamba.conv1d.weight"].shape == (96, 4)
+    assert bound["model.layers.0.mamba.A_log"].shape == (8,) and bound["model.layers.0.mamba.A_log"].dtype == torch.float32
+    assert bound["model.layers.0.mamba.D"].dtype == torch.bfloat16
+
+
+def test_sharded_checkpoint(tmp_path):
+    config = tiny_configs.config("A")
+    tensors = random_tensors(config, 0, torch.float32)
+    names = sorted(tensors)
+    half = len(names) // 2
+    write_safetensors(str(tmp_path / "model-00001-of-00002.safetensors"), {n: tensors[n] for n in names[:half]})
+    write_safetensors(str(tmp_path / "model-00002-of-00002.safetensors"), {n: tensors[n] for n in names[half:]})
+    weight_map = {n: ("model-00001-of-00002.safetensors" if i < half else "model-00002-of-00002.safetensors")
+                  for i, n in enumerate(names)}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": weight_map}))
+    bound = bind(WeightSource.from_dir(str(tmp_path)), DecoderModel.expected_tensors(config.to_model_spec()))
+    assert all(torch.equal(bound[n], tensors[n]) for n in names)

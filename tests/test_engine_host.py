@@ -1,0 +1,138 @@
+"""The step function, cache manager and scheduler with the kernels replaced by their plain
+PyTorch references (tests/ref_ops.py), on the CPU: what the host code does with pages,
+slots, lanes and rows, compared with the plain whole-sequence implementation."""
+import pytest
+import torch
+
+import plain_impl
+import ref_ops
+import tiny_configs
+from macllm_infer_amd.cache import CacheExhausted
+from macllm_infer_amd.engine import Engine, EngineConfig, Lane, Scheduler, StepError
+from macllm_infer_amd.sampling import Sampler, SamplingParams
+
+
+@pytest.fixture
+def host_ops(monkeypatch):
+    ref_ops.install(monkeypatch)
+
+
+def engine_for(name, folder, capacity=256, page=8, requests=4):
+    tiny_configs.make_model_dir(name, folder)
+    cfg, tensors = plain_impl.load_model_dir(str(folder))
+    engine = Engine(str(folder), dtype="float32", device="cpu", kv_cache_block_tokens=page,
+                    kv_cache_capacity_tokens=capacity, max_active_sequences=requests, check_device=False)
+    return engine, cfg, tensors
+
+
+def tokens_for(cfg, count, seed):
+    return torch.randint(0, cfg["vocab_size"], (count,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_whole_chunked_and_mixed_match_the_plain_model(host_ops, tmp_path, name):
+    engine, cfg, tensors = engine_for(name, tmp_path, capacity=96, page=8)
+    first, second = tokens_for(cfg, 45, 1), tokens_for(cfg, 30, 2)
+    want_first = plain_impl.falcon_h1_logits(cfg, tensors, first)
+    want_second = plain_impl.falcon_h1_logits(cfg, tensors, second)
+    engine.add_request("whole")
+    got = engine.step([Lane("whole", first, list(range(45)))])
+    assert (got - want_first).abs().max() < 1e-4
+    engine.finish("whole")
+    engine.add_request("cut")
+    outputs, cursor = [], 0
+    for size in [7, 2, 5, 3, 11, 2, 1, 1, 13]:
+        outputs.append(engine.step([Lane("cut", first[cursor:cursor + size], list(range(size)))]))
+        cursor += size
+    assert (torch.cat(outputs) - want_first).abs().max() < 1e-4
+    engine.finish("cut")
+    engine.add_request("c")
+    engine.add_request("d")
+    one = engine.step([Lane("c", first[:20], [19]), Lane("d", second[:3], [0, 1, 2])])
+    two = engine.step([Lane("d", second[3:30], list(range(27))), Lane("c", first[20:21], [0])])
+    assert (one[0] - want_first[19]).abs().max() < 1e-4 and (one[1:] - want_second[:3]).abs().max() < 1e-4
+    assert (two[:27] - want_second[3:30]).abs().max() < 1e-4 and (two[27] - want_first[20]).abs().max() < 1e-4
+    engine.cache.check()
+
+
+def test_refused_steps_change_nothing(host_ops, tmp_path):
+    engine, cfg, tensors = engine_for("A", tmp_path, capacity=32, page=8, requests=2)
+    engine.add_request("a")
+    tokens = tokens_for(cfg, 40, 3)
+    engine.step([Lane("a", tokens[:10], [9])])
+    before = engine.cache.stats()
+    for lanes, error in [
+            ([Lane("a", [], [])], StepError), ([Lane("ghost", [1], [])], StepError),
+            ([Lane("a", [1], []), Lane("a", [2], [])], StepError), ([Lane("a", [256], [])], StepError),
+            ([Lane("a", [-1], [])], StepError), ([Lane("a", [1, 2], [2])], StepError), ([], StepError),
+            ([Lane("a", tokens[10:40], [])], CacheExhausted)]:          # 40 tokens > 32 of capacity
+        with pytest.raises(error):
+            engine.step(lanes)
+        assert engine.cache.stats() == before and engine.length("a") == 10
+    # and the request goes on as if nothing had happened
+    want = plain_impl.falcon_h1_logits(cfg, tensors, tokens[:12])
+    got = engine.step([Lane("a", tokens[10:12], [0, 1])])
+    assert (got - want[10:12]).abs().max() < 1e-4
+    with pytest.raises(StepError, match="context limit"):
+        engine.max_context = 12
+        engine.step([Lane("a", [1], [])])
+
+
+def test_pages_and_slots_are_used_again_without_leaking_state(host_ops, tmp_path):
+    """A pool for one request at a time: each new request gets the pages and the slot the last
+    one gave back, and its logits are those of a fresh sequence."""
+    engine, cfg, tensors = engine_for("B", tmp_path, capacity=40, page=8, requests=1)
+    for seed in range(3):
+        tokens = tokens_for(cfg, 33 + seed, 10 + seed)
+        engine.add_request(seed)
+        got = engine.step([Lane(seed, tokens[:20], [19])])
+        got = torch.cat([got, engine.step([Lane(seed, tokens[20:], [len(tokens) - 21])])])
+        want = plain_impl.falcon_h1_logits(cfg, tensors, tokens)
+        assert (got - want[[19, len(tokens) - 1]]).abs().max() < 1e-4
+        engine.finish(seed)
+    assert engine.cache.stats()["groups"][0]["free_pages"] == 5
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_scheduler_greedy_generation_equals_the_plain_model(host_ops, tmp_path, name):
+    engine, cfg, tensors = engine_for(name, tmp_path, capacity=160, page=8, requests=3)
+    sampler = Sampler(engine.vocab_size, "cpu", check_device=False)
+    scheduler = Scheduler(engine, sampler, EngineConfig(max_active_sequences=3, scheduler_token_budget=16,
+                                                        prefill_token_quantum=11))
+    prompts = [tokens_for(cfg, length, 20 + length) for length in (5, 17, 33)]
+    params = SamplingParams(max_new_tokens=6, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0)
+    for index, prompt in enumerate(prompts):
+        scheduler.submit(index, prompt, params)
+    finished = scheduler.run()
+    for index, prompt in enumerate(prompts):
+        assert finished[index].generated == plain_impl.greedy_generate(cfg, tensors, prompt, 6)
+    stats = engine.cache.stats()
+    assert stats["live_requests"] == 0 and stats["free_slots"] == 3
+
+
+def test_scheduler_seeded_sampling_equals_the_plain_sampler(host_ops, tmp_path):
+    engine, cfg, tensors = engine_for("B", tmp_path, capacity=256, page=8, requests=4)
+    sampler = Sampler(engine.vocab_size, "cpu", check_device=False)
+    scheduler = Scheduler(engine, sampler, EngineConfig(max_active_sequences=4, scheduler_token_budget=24,
+                                                        prefill_token_quantum=11))
+    prompts = [tokens_for(cfg, length, 40 + length) for length in (1, 7, 24)]
+    params = [SamplingParams(max_new_tokens=5, temperature=0.8, top_k=0, top_p=1.0, repetition_penalty=1.0, seed=3),
+              SamplingParams(max_new_tokens=5, temperature=0.9, top_k=12, top_p=0.7, repetition_penalty=1.3, seed=4),
+              SamplingParams(max_new_tokens=5, temperature=1.1, top_k=0, top_p=0.9, presence_penalty=0.4,
+                             frequency_penalty=0.2, repetition_penalty=1.0, seed=5)]
+    for index, prompt in enumerate(prompts):
+        scheduler.submit(index, prompt, params[index])
+    finished = scheduler.run()
+    for index, prompt in enumerate(prompts):
+        p = params[index]
+        tokens, generated = list(prompt), []
+        for draw in range(5):
+            logits = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-1]
+            token = plain_impl.sample_token(
+                logits, temperature=p.temperature, top_k=p.top_k, top_p=p.top_p,
+                repetition_penalty=p.repetition_penalty, presence_penalty=p.presence_penalty,
+                frequency_penalty=p.frequency_penalty, history=tokens, generated=generated, seed=p.seed,
+                draw_index=draw)
+            tokens.append(token)
+            generated.append(token)
+        assert finished[index].generated == generated

@@ -1,0 +1,367 @@
+"""Pins the plain implementation by what fixes it beside the reference's text: vectors the
+reference's own tests hold, special cases that reduce to a library routine, and invariants.
+Each check is chosen so that a plausible mistake (a wrong sign or pairing, a reversed
+convolution, a norm in the wrong place) fails it."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_impl as P
+
+
+def rand(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+# ------------------------------------------------------------------ vectors from the reference's tests
+def test_mamba2_scalar_golden_from_reference():
+    """Fixture and golden of src/decoder.rs:5940-5976 and :7192-7216 (H=P=N=G=1, K=2):
+    catches projection order, convolution orientation, discretization, recurrence order,
+    skip, gate and output.  The reference stores the decay itself (-0.7); here A_log."""
+    w = {"conv1d.weight": torch.tensor([[0.25, 1.0], [-0.5, 0.75], [0.6, -1.2]]),
+         "conv1d.bias": torch.tensor([0.1, -0.2, 0.05]),
+         "dt_bias": torch.tensor([0.15]), "A_log": torch.tensor([math.log(0.7)]), "D": torch.tensor([0.3]),
+         "out_proj.weight": torch.tensor([[1.1]])}
+    projected = torch.tensor([[0.5, 1.0, 0.5, -0.25, 0.2], [-0.4, -0.5, 0.75, 0.4, -0.1],
+                              [0.8, 0.25, -0.6, 0.9, 0.35]])
+    out, state, tail = P.mamba2_mixer(None, w, num_heads=1, head_dim=1, state_size=1, num_groups=1,
+                                      conv_kernel=2, eps=1e-5, projected=projected, return_state=True)
+    golden = torch.tensor([[0.08963693], [0.005108623], [0.024774795]])
+    assert (out - golden).abs().max() < 2e-6
+    assert abs(state.item() - (-0.013268862)) < 2e-6
+    assert (tail - torch.tensor([[0.25, -0.6, 0.9]])).abs().max() < 1e-7
+
+
+def test_attention_mlp_norm_golden_from_reference():
+    """The closed form of src/decoder.rs:10293-10339 with the tensors of :7612-7667: zero
+    embeddings and q/k/v/gate/up matrices, biases only; one token.  Pins bias placement,
+    the head concatenation into o_proj, SiLU(gate)*up, and eps inside the root."""
+    n = torch.zeros(1, 2)
+    attention = {"q_proj.weight": torch.zeros(4, 2), "k_proj.weight": torch.zeros(2, 2),
+                 "v_proj.weight": torch.zeros(2, 2), "q_proj.bias": torch.tensor([0.1, 0.2, 0.3, 0.4]),
+                 "k_proj.bias": torch.tensor([0.2, -0.3]), "v_proj.bias": torch.tensor([1.0, -1.0]),
+                 "o_proj.weight": torch.tensor([[1.0, 0, 0, 0], [0, 1.0, 0, 0]]),
+                 "o_proj.bias": torch.tensor([0.5, 0.25])}
+    h = n + P.attention_mixer(P.rms_norm(n, torch.ones(2), 1e-5), attention, num_heads=2, num_kv_heads=1,
+                              head_dim=2, theta=1e4)
+    assert torch.allclose(h, torch.tensor([[1.5, -0.75]]))
+    mlp = {"gate_proj.weight": torch.zeros(2, 2), "up_proj.weight": torch.zeros(2, 2),
+           "down_proj.weight": torch.eye(2), "gate_proj.bias": torch.tensor([0.5, -0.5]),
+           "up_proj.bias": torch.tensor([2.0, 3.0]), "down_proj.bias": torch.tensor([0.25, 0.5])}
+    h = h + P.swiglu_mlp(P.rms_norm(h, torch.ones(2), 1e-5), mlp)
+    logits = P.rms_norm(h, torch.ones(2), 1e-5) @ torch.eye(2)
+    silu = lambda v: v / (1.0 + math.exp(-v))
+    hidden = [1.5 + silu(0.5) * 2.0 + 0.25, -0.75 + silu(-0.5) * 3.0 + 0.5]
+    rms = math.sqrt((hidden[0] ** 2 + hidden[1] ** 2) / 2 + 1e-5)
+    assert (logits - torch.tensor([[hidden[0] / rms, hidden[1] / rms]])).abs().max() < 1e-5
+
+
+def test_selective_scan_matches_reference_kernel_fixture():
+    """Fixture of crates/macllm-kernels/src/mamba2.rs:544-573 (dt = +-100 locks the stable
+    softplus; non-zero initial state; 2 groups) against an independent scalar loop written
+    from :633-670, and split 2+1 with the carried state."""
+    T, H, P_, N, G = 3, 4, 2, 3, 2
+    E, GN = H * P_, G * N
+    xbc = []
+    for t in range(T):
+        xbc += [((t * 11 + i * 7) % 19) * 0.07 - 0.5 for i in range(E)]
+        xbc += [((t * 5 + i * 3) % 13) * 0.04 - 0.2 for i in range(GN)]
+        xbc += [((t * 7 + i * 5) % 17) * 0.03 - 0.18 for i in range(GN)]
+    xbc = np.array(xbc, dtype=np.float32).reshape(T, E + 2 * GN)
+    raw_dt = np.array([100.0, -100.0, 0.2, -0.7, -1.3, 0.9, 1.4, -0.2, 0.0, 0.4, -0.8, 1.1], np.float32).reshape(T, H)
+    dt_bias = np.array([-0.15, 0.25, -0.4, 0.05], np.float32)
+    a = np.array([-0.03, -0.2, -0.45, -0.1], np.float32)
+    d = np.array([0.2, -0.3, 0.5, 0.1], np.float32)
+    state0 = ((np.arange(E * N) - 11.0) * 0.015).astype(np.float32)
+    state = state0.astype(np.float64).copy()
+    expected = np.zeros((T, E))
+    for t in range(T):
+        for h in range(H):
+            shifted = float(raw_dt[t, h]) + float(dt_bias[h])
+            delta = max(shifted, 0.0) + math.log1p(math.exp(-abs(shifted)))
+            decay = math.exp(delta * float(a[h]))
+            g = h // (H // G)
+            for p in range(P_):
+                lane = h * P_ + p
+                value = float(xbc[t, lane])
+                projected = 0.0
+                for n in range(N):
+                    index = lane * N + n
+                    state[index] = decay * state[index] + delta * value * float(xbc[t, E + g * N + n])
+                    projected += state[index] * float(xbc[t, E + GN + g * N + n])
+                expected[t, lane] = projected + float(d[h]) * value
+    x = torch.from_numpy(xbc)
+    args = dict(dt_bias=torch.from_numpy(dt_bias), A=torch.from_numpy(a), D=torch.from_numpy(d))
+    split = lambda rows: (rows[:, :E].reshape(-1, H, P_), rows[:, E:E + GN].reshape(-1, G, N),
+                          rows[:, E + GN:].reshape(-1, G, N))
+    initial = torch.from_numpy(state0).reshape(H, P_, N)
+    y, final = P.selective_scan(*split(x), torch.from_numpy(raw_dt), initial_state=initial, **args)
+    assert torch.isfinite(y).all()
+    assert np.abs(y.reshape(T, E).numpy() - expected).max() < 1e-6
+    assert np.abs(final.reshape(-1).numpy() - state).max() < 1e-6
+    assert torch.equal(initial, torch.from_numpy(state0).reshape(H, P_, N))      # input state not mutated
+    y1, mid = P.selective_scan(*split(x[:2]), torch.from_numpy(raw_dt[:2]), initial_state=initial, **args)
+    y2, last = P.selective_scan(*split(x[2:]), torch.from_numpy(raw_dt[2:]), initial_state=mid, **args)
+    assert (torch.cat([y1, y2]) - y).abs().max() < 1e-6 and (last - final).abs().max() < 1e-6
+
+
+def test_sampler_vectors_from_reference():
+    """src/sampling.rs:467-511: greedy picks the largest, ties pick the first, the
+    repetition penalty divides positive and multiplies negative logits, a zero target never
+    selects a masked token."""
+    assert P.sample_token(torch.tensor([0.0, 3.0, 2.0])) == 1
+    assert P.sample_token(torch.tensor([3.0, 3.0, 2.0])) == 0
+    # [2, -2, 1] with history [0, 1, 0] and penalty 2 -> [1, -4, 1]: the tie then picks index 0
+    assert P.sample_token(torch.tensor([2.0, -2.0, 1.0]), repetition_penalty=2.0, history=[0, 1, 0]) == 0
+    assert P.sample_token(torch.tensor([2.0, -2.0, 1.5]), repetition_penalty=2.0, history=[0, 1, 0]) == 2
+    for seed in range(20):     # top_k = 1 leaves one token, whatever is drawn
+        assert P.sample_token(torch.tensor([0.1, 5.0, 0.2]), temperature=1.0, top_k=1, seed=seed) == 1
+        assert P.sample_token(torch.tensor([0.0, 9.0, 0.0, 8.0]), temperature=1.0, top_p=0.5, seed=seed) == 1
+
+
+def test_sampler_distribution_and_presence_penalty():
+    logits = torch.tensor([1.0, 2.0, 0.5, -1.0])
+    counts = np.zeros(4)
+    for draw in range(4000):
+        counts[P.sample_token(logits, temperature=0.8, seed=7, draw_index=draw)] += 1
+    expected = torch.softmax(logits / 0.8, 0).numpy()
+    assert np.abs(counts / 4000 - expected).max() < 0.03
+    # presence/frequency act on generated tokens only
+    assert P.sample_token(torch.tensor([1.0, 1.2]), presence_penalty=0.5, history=[1], generated=[]) == 1
+    assert P.sample_token(torch.tensor([1.0, 1.2]), presence_penalty=0.5, history=[1], generated=[1]) == 0
+    assert P.sample_token(torch.tensor([1.0, 1.4]), frequency_penalty=0.25, history=[1, 1], generated=[1, 1]) == 0
+
+
+# ------------------------------------------------------------------ reductions to library routines
+def test_rms_norm_is_the_library_routine():
+    x, w = rand(5, 24, seed=1), rand(24, seed=2)
+    assert torch.allclose(P.rms_norm(x, w, 3e-6), F.rms_norm(x, (24,), w, 3e-6), atol=1e-6)
+    unit = P.rms_norm(x, torch.ones(24), 1e-12)
+    assert torch.allclose(unit.pow(2).mean(-1), torch.ones(5), atol=1e-5)
+
+
+def test_attention_is_library_sdpa_for_a_whole_prompt():
+    T, Hq, Hkv, dh = 19, 6, 3, 8
+    q, k, v = rand(T, Hq, dh, seed=3), rand(T, Hkv, dh, seed=4), rand(T, Hkv, dh, seed=5)
+    ours = P.gqa_causal_attention(q, k, v, 1 / math.sqrt(dh))
+    lib = F.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], k.transpose(0, 1).repeat_interleave(Hq // Hkv, 0)[None],
+        v.transpose(0, 1).repeat_interleave(Hq // Hkv, 0)[None], is_causal=True)[0].transpose(0, 1)
+    assert torch.allclose(ours, lib, atol=1e-5)
+    # one head, no mask effect on the last row: plain softmax(q k^T / sqrt(d)) v
+    last = torch.softmax(q[-1, 0] @ k[:, 0].T / math.sqrt(dh), 0) @ v[:, 0]
+    assert torch.allclose(ours[-1, 0], last, atol=1e-5)
+
+
+def test_gqa_head_pairing():
+    """Query head h reads kv head h // group (src/decoder.rs:7753-7780): with one-hot values
+    per kv head the output names the head that was read."""
+    T, Hq, Hkv, dh = 3, 4, 2, 2
+    q, k = rand(T, Hq, dh, seed=6), rand(T, Hkv, dh, seed=7)
+    v = torch.zeros(T, Hkv, dh)
+    v[:, 0, 0] = 1.0
+    v[:, 1, 1] = 1.0
+    out = P.gqa_causal_attention(q, k, v, 1.0)
+    assert torch.allclose(out[:, :2, 0], torch.ones(T, 2)) and torch.allclose(out[:, 2:, 1], torch.ones(T, 2))
+    assert torch.allclose(out[:, :2, 1], torch.zeros(T, 2)) and torch.allclose(out[:, 2:, 0], torch.zeros(T, 2))
+
+
+def test_window_masks_exactly_the_keys_at_distance_window_or_more():
+    T, dh, window = 12, 4, 5
+    q, k = rand(T, 1, dh, seed=8), rand(T, 1, dh, seed=9)
+    v = torch.eye(T)[:, None, :]                       # output row = attention weights
+    weights = P.gqa_causal_attention(q, k, v, 0.5, window=window)[:, 0, :]
+    for s in range(T):
+        for p in range(T):
+            visible = p <= s and s - p < window
+            assert (weights[s, p] > 0) == visible
+    assert torch.allclose(weights.sum(-1), torch.ones(T), atol=1e-6)
+
+
+def test_conv_is_library_conv1d_and_splits_with_a_tail():
+    T, C, K = 11, 6, 4
+    x, w, b = rand(T, C, seed=10), rand(C, K, seed=11), rand(C, seed=12)
+    ours = P.causal_depthwise_conv(x, w, b)
+    lib = F.conv1d(F.pad(x.T[None], (K - 1, 0)), w[:, None, :], b, groups=C)[0].T
+    assert torch.allclose(ours, lib, atol=1e-6)
+    # the last output only sees the last K rows, oldest first
+    assert torch.allclose(ours[-1], (x[-K:] * w.T).sum(0) + b, atol=1e-6)
+
+
+def test_softplus_is_the_library_routine_and_stable():
+    x = torch.tensor([-100.0, -3.0, 0.0, 0.5, 30.0, 100.0])
+    assert torch.allclose(P.softplus(x), F.softplus(x), atol=1e-6)
+    assert torch.isfinite(P.softplus(x)).all() and P.softplus(x)[-1] == 100.0
+
+
+def test_scan_reduces_to_a_cumulative_sum_and_a_scalar_recurrence():
+    T, H, P_, N = 9, 2, 3, 4
+    x, B, C = rand(T, H, P_, seed=13), rand(T, 1, N, seed=14), rand(T, 1, N, seed=15)
+    dt = rand(T, H, seed=16)
+    # A -> 0, D = 0: y_t = C_t . cumsum_s(delta_s x_s (outer) B_s)
+    y, _ = P.selective_scan(x, B, C, dt, torch.zeros(H), torch.zeros(H), torch.zeros(H))
+    delta = F.softplus(dt)
+    summed = torch.cumsum(delta[:, :, None, None] * x[:, :, :, None] * B[:, :, None, :], dim=0)
+    assert torch.allclose(y, (summed * C[:, :, None, :]).sum(-1), atol=1e-5)
+    # H = P = N = G = 1: s = exp(delta a) s + delta x b; y = s c + d x
+    x1, b1, c1, dt1 = rand(T, 1, 1, seed=17), rand(T, 1, 1, seed=18), rand(T, 1, 1, seed=19), rand(T, 1, seed=20)
+    y1, s1 = P.selective_scan(x1, b1, c1, dt1, torch.tensor([0.1]), torch.tensor([-0.8]), torch.tensor([0.4]))
+    s = 0.0
+    for t in range(T):
+        step = F.softplus(dt1[t, 0] + 0.1).item()
+        s = math.exp(step * -0.8) * s + step * x1[t, 0, 0].item() * b1[t, 0, 0].item()
+        assert abs(y1[t, 0, 0].item() - (s * c1[t, 0, 0].item() + 0.4 * x1[t, 0, 0].item())) < 1e-5
+    assert abs(s1.item() - s) < 1e-5
+
+
+def test_group_of_a_head():
+    """Head h uses B and C of group h // (H/G) (src/decoder.rs:2423-2435)."""
+    T, H, P_, N, G = 4, 4, 1, 2, 2
+    x, dt = torch.ones(T, H, P_), torch.zeros(T, H)
+    B = torch.zeros(T, G, N)
+    B[:, 1] = 1.0                                        # only group 1 feeds the state
+    C = torch.ones(T, G, N)
+    y, _ = P.selective_scan(x, B, C, dt, torch.zeros(H), -torch.ones(H), torch.zeros(H))
+    assert (y[:, :2] == 0).all() and (y[:, 2:] > 0).all()
+
+
+def test_gate_then_norm_and_single_group():
+    y, z, w = rand(5, 12, seed=21), rand(5, 12, seed=22), rand(12, seed=23)
+    gated = y * F.silu(z)
+    assert torch.allclose(P.gate_and_group_norm(y, z, None, 1, 1e-5), gated, atol=1e-6)
+    assert torch.allclose(P.gate_and_group_norm(y, z, w, 1, 1e-5), F.rms_norm(gated, (12,), w, 1e-5), atol=1e-6)
+    two = P.gate_and_group_norm(y, z, w, 2, 1e-5)
+    assert torch.allclose(two[:, 6:], F.rms_norm(gated[:, 6:], (6,), w[6:], 1e-5), atol=1e-6)
+    # norm before the gate would differ
+    assert not torch.allclose(two, F.rms_norm(y.view(5, 2, 6), (6,), None, 1e-5).reshape(5, 12) * w * F.silu(z), atol=1e-3)
+
+
+def test_swiglu_and_linear():
+    g, u = rand(3, 5, seed=24), rand(3, 5, seed=25)
+    assert torch.allclose(P.swiglu(g, u), F.silu(g) * u)
+    x, w, b = rand(3, 5, seed=26), rand(4, 5, seed=27), rand(4, seed=28)
+    assert torch.allclose(P.linear(x, w, b), F.linear(x, w, b), atol=1e-6)
+
+
+# ------------------------------------------------------------------ invariants
+def test_rope_identity_norm_pairing_and_relative_positions():
+    T, H, dh, theta = 6, 2, 8, 1e4
+    x = rand(T, H, dh, seed=29)
+    assert torch.allclose(P.rope_half_split(x, torch.zeros(T, dtype=torch.long), theta), x)
+    rotated = P.rope_half_split(x, torch.arange(T) + 17, theta)
+    assert torch.allclose(rotated.norm(dim=-1), x.norm(dim=-1), atol=1e-5)
+    # half-split pairing (j, j + dh/2) as a complex multiplication
+    position = torch.tensor([5])
+    z = torch.complex(x[:1, :, :dh // 2], x[:1, :, dh // 2:])
+    turn = torch.polar(torch.ones(dh // 2), 5.0 * P.rope_inverse_frequencies(theta, dh))
+    expected = z * turn
+    got = P.rope_half_split(x[:1], position, theta)
+    assert torch.allclose(got[..., :dh // 2], expected.real, atol=1e-5)
+    assert torch.allclose(got[..., dh // 2:], expected.imag, atol=1e-5)
+    # <R_m q, R_n k> depends on m - n only
+    q, k = rand(1, 1, dh, seed=30), rand(1, 1, dh, seed=31)
+    dot = lambda m, n: (P.rope_half_split(q, torch.tensor([m]), theta) * P.rope_half_split(k, torch.tensor([n]), theta)).sum()
+    assert abs(dot(9, 4) - dot(105, 100)) < 1e-4 and abs(dot(9, 4) - dot(4, 9)) > 1e-3
+    # partial rotation leaves the tail untouched (src/decoder.rs:8465-8499)
+    partial = P.rope_half_split(x, torch.arange(T) + 3, theta, rotary_dim=4)
+    assert torch.equal(partial[..., 4:], x[..., 4:]) and not torch.allclose(partial[..., :4], x[..., :4])
+    assert P.rope_inverse_frequencies(1e11, 64).dtype == torch.float32
+
+
+def test_attention_depends_on_distances_only():
+    """A shift of all positions leaves the attention mixer's output unchanged."""
+    d, Hq, Hkv, dh, T = 16, 4, 2, 4, 10
+    w = {"q_proj.weight": rand(Hq * dh, d, seed=32, scale=0.3), "k_proj.weight": rand(Hkv * dh, d, seed=33, scale=0.3),
+         "v_proj.weight": rand(Hkv * dh, d, seed=34, scale=0.3), "o_proj.weight": rand(d, Hq * dh, seed=35, scale=0.3)}
+    n = rand(T, d, seed=36)
+    base = P.attention_mixer(n, w, num_heads=Hq, num_kv_heads=Hkv, head_dim=dh, theta=100.0)
+    shifted = P.attention_mixer(n, w, num_heads=Hq, num_kv_heads=Hkv, head_dim=dh, theta=100.0,
+                                positions=torch.arange(T) + 37)
+    assert torch.allclose(base, shifted, atol=1e-4)
+    without = P.attention_mixer(n, w, num_heads=Hq, num_kv_heads=Hkv, head_dim=dh, theta=100.0, use_rope=False)
+    assert not torch.allclose(base, without, atol=1e-3)
+
+
+def _tiny_model(seed=0, **overrides):
+    import tiny_configs
+    raw = dict(tiny_configs.TINY_B)
+    raw.update(overrides)
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.weights.random_init import random_tensors
+    tensors = random_tensors(FalconH1Config.from_dict(raw), seed, torch.float32, "unit")
+    return raw, tensors
+
+
+def test_layer_is_identity_when_output_projections_are_zero_and_branches_add_up():
+    cfg, tensors = _tiny_model()
+    tokens = [3, 9, 200, 41, 7, 7, 100]
+    h = rand(len(tokens), cfg["hidden_size"], seed=40)
+    full = P.falcon_h1_layer(h, tensors, 0, cfg)
+    only_attention = P.falcon_h1_layer(h, tensors, 0, cfg, ablate=("mamba", "mlp"))
+    only_mamba = P.falcon_h1_layer(h, tensors, 0, cfg, ablate=("attention", "mlp"))
+    both = P.falcon_h1_layer(h, tensors, 0, cfg, ablate=("mlp",))
+    assert torch.allclose((only_attention - h) + (only_mamba - h), both - h, atol=1e-5)   # parallel sum
+    assert not torch.allclose(full, both, atol=1e-3)
+    zeroed = dict(tensors)
+    for name in ("self_attn.o_proj", "mamba.out_proj", "mlp.down_proj"):
+        zeroed[f"model.layers.0.{name}.weight"] = torch.zeros_like(tensors[f"model.layers.0.{name}.weight"])
+        zeroed[f"model.layers.0.{name}.bias"] = torch.zeros_like(tensors[f"model.layers.0.{name}.bias"])
+    assert torch.allclose(P.falcon_h1_layer(h, zeroed, 0, cfg), h)
+
+
+def test_tied_equals_untied_with_the_copied_matrix_and_multipliers_fold():
+    cfg, tensors = _tiny_model()
+    tokens = [1, 2, 3, 4, 5, 6, 7, 8, 9]
+    untied = P.falcon_h1_logits(cfg, tensors, tokens)
+    copied = dict(tensors)
+    copied["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    tied_cfg = dict(cfg, tie_word_embeddings=True)
+    assert torch.allclose(P.falcon_h1_logits(tied_cfg, tensors, tokens), P.falcon_h1_logits(cfg, copied, tokens))
+    # folding every multiplier into the weights gives the same logits as applying them at run time
+    folded = {name: value.clone().float() for name, value in tensors.items()}
+    unit = dict(cfg)
+    E, GN, H = cfg["mamba_d_ssm"], cfg["mamba_n_groups"] * cfg["mamba_d_state"], cfg["mamba_n_heads"]
+    m = cfg["ssm_multipliers"]
+    segment = torch.cat([torch.full((E,), m[0]), torch.full((E,), m[1]), torch.full((GN,), m[2]),
+                         torch.full((GN,), m[3]), torch.full((H,), m[4])])
+    for layer in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{layer}."
+        for proj, weight_scale, bias_scale in (
+                ("self_attn.q_proj", cfg["attention_in_multiplier"], 1.0),
+                ("self_attn.k_proj", cfg["attention_in_multiplier"] * cfg["key_multiplier"], cfg["key_multiplier"]),
+                ("self_attn.v_proj", cfg["attention_in_multiplier"], 1.0),
+                ("self_attn.o_proj", cfg["attention_out_multiplier"], cfg["attention_out_multiplier"]),
+                ("mamba.out_proj", cfg["ssm_out_multiplier"], cfg["ssm_out_multiplier"]),
+                ("mlp.gate_proj", cfg["mlp_multipliers"][0], cfg["mlp_multipliers"][0]),
+                ("mlp.down_proj", cfg["mlp_multipliers"][1], cfg["mlp_multipliers"][1])):
+            folded[p + proj + ".weight"] *= weight_scale
+            folded[p + proj + ".bias"] *= bias_scale
+        folded[p + "mamba.in_proj.weight"] *= (segment * cfg["ssm_in_multiplier"])[:, None]
+        folded[p + "mamba.in_proj.bias"] *= segment
+    for key in ("attention_in_multiplier", "attention_out_multiplier", "key_multiplier", "ssm_in_multiplier",
+                "ssm_out_multiplier"):
+        unit[key] = 1.0
+    unit["ssm_multipliers"] = [1.0] * 5
+    unit["mlp_multipliers"] = [1.0, 1.0]
+    assert torch.allclose(P.falcon_h1_logits(unit, folded, tokens), untied, atol=2e-5)
+    assert not torch.allclose(P.falcon_h1_logits(unit, tensors, tokens), untied, atol=1e-2)
+
+
+def test_every_branch_matters_in_the_tiny_models():
+    """With the "unit" init each branch moves the logits, so a fault in one shows."""
+    for name in ("A", "B"):
+        import tiny_configs
+        raw, seed = tiny_configs.CONFIGS[name]
+        from macllm_infer_amd.config import FalconH1Config
+        from macllm_infer_amd.weights.random_init import random_tensors
+        tensors = random_tensors(FalconH1Config.from_dict(raw), seed, torch.float32, "unit")
+        tokens = list(range(3, 40))
+        full = P.falcon_h1_logits(raw, tensors, tokens)
+        for branch in ("attention", "mamba", "mlp"):
+            assert (P.falcon_h1_logits(raw, tensors, tokens, ablate=(branch,)) - full).abs().max() > 0.05
+        # and the past matters: changing the first token changes the last logits
+        other = [tokens[0] + 1] + tokens[1:]
+        assert (P.falcon_h1_logits(raw, tensors, other)[-1] - full[-1]).abs().max() > 1e-3

@@ -1,0 +1,178 @@
+"""The scheduler's decisions, with a fake engine that scripts logits and records what ran
+(the reference tests its scheduler the same way: src/engine.rs:3158-3599)."""
+import pytest
+import torch
+
+from macllm_infer_amd.cache import CacheExhausted
+from macllm_infer_amd.engine.scheduler import EngineConfig, QueueFull, Scheduler
+from macllm_infer_amd.sampling import GREEDY, SamplingParams
+
+
+class FakeCache:
+    def __init__(self, engine):
+        self.engine = engine
+
+    def can_ever_fit(self, tokens):
+        return tokens <= self.engine.capacity
+
+
+class FakeEngine:
+    """Next token = (last token of the lane + 1) % vocab; counts pages of ``page`` tokens."""
+    vocab_size = 50
+    max_context = 200
+
+    def __init__(self, capacity=10_000, page=4):
+        self.capacity, self.page = capacity, page
+        self.lengths = {}
+        self.calls = []
+        self.cache = FakeCache(self)
+
+    def add_request(self, request):
+        assert request not in self.lengths
+        self.lengths[request] = 0
+
+    def finish(self, request):
+        del self.lengths[request]
+
+    def pages(self, lengths):
+        return sum(-(-length // self.page) for length in lengths)
+
+    def step(self, lanes):
+        grown = dict(self.lengths)
+        for lane in lanes:
+            grown[lane.request] += len(lane.tokens)
+        if self.pages(grown.values()) * self.page > self.capacity:
+            raise CacheExhausted("pages", 1, 0, self.capacity // self.page)
+        self.calls.append([(lane.request, list(lane.tokens), self.lengths[lane.request], list(lane.want))
+                           for lane in lanes])
+        self.lengths = grown
+        rows = []
+        for lane in lanes:
+            for place in lane.want:
+                row = torch.zeros(self.vocab_size)
+                row[(lane.tokens[place] + 1) % self.vocab_size] = 5.0
+                rows.append(row)
+        return torch.stack(rows) if rows else torch.zeros(0, self.vocab_size)
+
+
+class ArgmaxSampler:
+    def sample(self, logits, rows):
+        assert logits.shape[0] == len(rows)
+        return torch.argmax(logits, dim=-1).tolist()
+
+
+def run(prompts, params=GREEDY, config=None, engine=None, stop=()):
+    engine = engine or FakeEngine()
+    scheduler = Scheduler(engine, ArgmaxSampler(), config or EngineConfig(), stop)
+    for index, prompt in enumerate(prompts):
+        scheduler.submit(index, prompt, params if isinstance(params, SamplingParams) else params[index])
+    finished = scheduler.run()
+    return engine, scheduler, finished
+
+
+def test_prompt_is_cut_into_portions_and_only_the_last_is_sampled():
+    params = SamplingParams(max_new_tokens=3, temperature=0.0)
+    engine, _, finished = run([[1, 2, 3, 4, 5, 6, 7]], params,
+                              EngineConfig(scheduler_token_budget=3, prefill_token_quantum=3))
+    portions = [call[0] for call in engine.calls]
+    assert [(p[1], p[2], p[3]) for p in portions[:3]] == [([1, 2, 3], 0, []), ([4, 5, 6], 3, []), ([7], 6, [0])]
+    assert [(p[1], p[2]) for p in portions[3:]] == [([8], 7), ([9], 8)]          # decoded tokens, one each
+    assert finished[0].generated == [8, 9, 10] and finished[0].finish_reason == "length"
+    assert engine.lengths == {}                                                    # everything given back
+
+
+def test_token_budget_and_round_robin():
+    """Budget 4, quantum 3: requests not reached keep their place and go first next round
+    (src/engine.rs:4968)."""
+    params = SamplingParams(max_new_tokens=2, temperature=0.0)
+    engine, _, finished = run([[1, 2, 3, 4, 5], [10, 11, 12, 13, 14], [20]], params,
+                              EngineConfig(scheduler_token_budget=4, prefill_token_quantum=3))
+    for call in engine.calls:
+        assert sum(len(tokens) for _, tokens, _, _ in call) <= 4
+    first = [(request, tokens) for request, tokens, _, _ in engine.calls[0]]
+    assert first == [(0, [1, 2, 3]), (1, [10])]
+    second = [(request, tokens) for request, tokens, _, _ in engine.calls[1]]
+    assert second[0] == (2, [20])                       # the unvisited request is first in line
+    assert {k: v.generated for k, v in finished.items()} == {0: [6, 7], 1: [15, 16], 2: [21, 22]}
+
+
+def test_mixed_rows_stay_aligned():
+    """Portions of prompts beside decoded tokens: logits row i belongs to the i-th sampled lane
+    (src/engine.rs:4701)."""
+    params = [SamplingParams(max_new_tokens=4, temperature=0.0), SamplingParams(max_new_tokens=2, temperature=0.0)]
+    engine, _, finished = run([[5], [30, 31, 32, 33, 34, 35]], params,
+                              EngineConfig(scheduler_token_budget=4, prefill_token_quantum=3))
+    assert finished[0].generated == [6, 7, 8, 9] and finished[1].generated == [36, 37]
+    mixed = [call for call in engine.calls if len(call) == 2 and {len(call[0][1]), len(call[1][1])} == {1, 3}]
+    assert mixed, "a decode token ran beside a prompt portion"
+
+
+def test_admission_limits_and_rejections():
+    engine = FakeEngine(capacity=40)
+    params = SamplingParams(max_new_tokens=4, temperature=0.0)
+    scheduler = Scheduler(engine, ArgmaxSampler(), EngineConfig(max_active_sequences=2, queue_capacity=5))
+    scheduler.submit("empty", [], params)
+    scheduler.submit("vocab", [1, 50], params)
+    scheduler.submit("context", list(range(10)) * 20, params)
+    scheduler.submit("capacity", list(range(40)), params)
+    scheduler.submit("ok1", [1, 2], params)
+    with pytest.raises(QueueFull):
+        scheduler.submit("late", [1], params)
+    scheduler.step()
+    scheduler.submit("ok2", [3], params)
+    scheduler.submit("ok3", [4], params)
+    finished = scheduler.run()
+    assert finished["empty"].finish_reason == "rejected: prompt must contain at least one token"
+    assert "vocabulary" in finished["vocab"].finish_reason and "context" in finished["context"].finish_reason
+    assert "cache capacity" in finished["capacity"].finish_reason
+    assert all(len(call) <= 2 for call in engine.calls)            # never more than two live
+    assert finished["ok3"].generated == [5, 6, 7, 8]
+
+
+def test_stop_token_is_not_emitted_and_ignore_eos():
+    _, _, finished = run([[1]], SamplingParams(max_new_tokens=8, temperature=0.0), stop=(4,))
+    assert finished[0].generated == [2, 3] and finished[0].finish_reason == "stop"
+    _, _, finished = run([[1]], SamplingParams(max_new_tokens=5, temperature=0.0, ignore_eos=True), stop=(4,))
+    assert finished[0].generated == [2, 3, 4, 5, 6] and finished[0].finish_reason == "length"
+    _, _, finished = run([[1]], SamplingParams(max_new_tokens=5, temperature=0.0, stop_token_ids=(3,)))
+    assert finished[0].generated == [2] and finished[0].finish_reason == "stop"
+
+
+def test_page_pressure_drops_the_last_lane_for_a_round():
+    """Pages for 6 tokens (3 pages of 2): three 2-token prompts fill them; decoding then needs
+    a fourth page... the round shrinks until it fits (src/engine.rs:4845)."""
+    engine = FakeEngine(capacity=12, page=4)
+    params = SamplingParams(max_new_tokens=1, temperature=0.0)
+    _, scheduler, finished = run([[1, 2, 3, 4], [5, 6, 7, 8], [9, 10, 11, 12], [13, 14, 15, 16]], params,
+                                 engine=engine)
+    assert all(request.finish_reason == "length" for request in finished.values())
+    assert len(engine.calls[0]) == 3                                  # the fourth lane waited
+    assert [request for request, _, _, _ in engine.calls[1]] == [3]
+
+
+def test_irreducible_pressure_fails_only_that_request():
+    """Two requests whose growth cannot both fit: the one whose single lane cannot be reserved
+    fails with resource_exhausted and frees its pages; the other completes
+    (src/engine.rs:4898)."""
+    engine = FakeEngine(capacity=16, page=4)
+    params = SamplingParams(max_new_tokens=6, temperature=0.0)
+    _, _, finished = run([[1, 2, 3, 4, 5, 6, 7], [20, 21, 22, 23, 24, 25, 26]], params, engine=engine)
+    reasons = sorted(request.finish_reason for request in finished.values())
+    assert reasons == ["length", "resource_exhausted"]
+    done = [request for request in finished.values() if request.finish_reason == "length"][0]
+    assert len(done.generated) == 6
+    assert engine.lengths == {}
+
+
+def test_scheduler_settings_are_checked():
+    with pytest.raises(ValueError):
+        EngineConfig(prefill_token_quantum=10, scheduler_token_budget=5)
+    with pytest.raises(ValueError):
+        SamplingParams(top_p=0.0)
+    with pytest.raises(ValueError):
+        SamplingParams(temperature=-1.0)
+    with pytest.raises(ValueError):
+        SamplingParams(repetition_penalty=0.0)
+    defaults = SamplingParams()                # the reference's defaults, src/sampling.rs:23-33
+    assert (defaults.temperature, defaults.top_k, defaults.top_p, defaults.repetition_penalty, defaults.seed,
+            defaults.max_new_tokens) == (0.7, 20, 0.8, 1.1, 42, 128)
