@@ -58,8 +58,8 @@ def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, r
     T = qkv.shape[0]
     q_cols = num_heads * head_dim
     k_cols = num_kv_heads * head_dim
-    q = _f(qkv[:, :q_cols]).reshape(T, num_heads, head_dim)
-    k = _f(qkv[:, q_cols:q_cols + k_cols]).reshape(T, num_kv_heads, head_dim)
+    q = _f(qkv[:, :q_cols]).reshape(T, num_heads, head_dim).clone()
+    k = _f(qkv[:, q_cols:q_cols + k_cols]).reshape(T, num_kv_heads, head_dim).clone()
     v = qkv[:, q_cols + k_cols:q_cols + 2 * k_cols].reshape(T, num_kv_heads, head_dim)
     if inv_freq is not None and rotary_dim > 0:
         half = rotary_dim // 2

@@ -136,3 +136,12 @@ def test_scheduler_seeded_sampling_equals_the_plain_sampler(host_ops, tmp_path):
             tokens.append(token)
             generated.append(token)
         assert finished[index].generated == generated
+
+
+@pytest.mark.parametrize("schedule", __import__("toy_parts").SCHEDULES, ids=__import__("toy_parts").SCHEDULE_IDS)
+def test_toy_parts_register_build_and_step_on_the_host(host_ops, schedule):
+    """The framework's generality without a GPU: a mixer with state of its own, another
+    position encoding, a window, a layer that runs twice and a run that reads another run's
+    cache, registered from the tests and stepped through the engine."""
+    import toy_parts
+    toy_parts.exercise(schedule, "cpu", check_device=False)

@@ -1,0 +1,230 @@
+"""In-process GPU tests: each part alone against the plain implementation, greedy and seeded
+generation through the entry points, and the framework's generality: a toy mixer with state
+of its own, another position encoding, a window, a layer that runs twice and a layer that
+reads another layer's cache, all registered from here without a change to the package."""
+import math
+import subprocess
+import sys
+import pytest
+import torch
+
+import plain_impl
+import tiny_configs
+import toy_parts
+from traces import ROOT
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def tolerance(dtype):
+    return 1e-4 if dtype == torch.float32 else 6e-2
+
+
+def rand(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def tokens_for(vocab, count, seed):
+    return torch.randint(0, vocab, (count,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+# ------------------------------------------------------------------ a harness for single parts
+class PartHarness:
+    """Builds one mixer with a cache of its own and feeds it lanes of normed inputs."""
+
+    def __init__(self, spec, tensors, hidden, dtype, page_size=8, capacity=512, requests=4):
+        from macllm_infer_amd.cache import CacheManager
+        from macllm_infer_amd.kernels import build
+        from macllm_infer_amd.parts import BuildContext, part_class
+        cls = part_class(spec)
+        build.ensure_modules(cls.kernel_modules)
+        self.build = BuildContext(hidden_size=hidden, dtype=dtype, device=torch.device(DEV), max_context=4096)
+        self.part = cls(spec, "p", {f"p.{name}": value for name, value in tensors.items()}, self.build)
+        self.cache = CacheManager({(0, "p"): cls.cache_needs(spec)}, {}, page_size, capacity, requests, dtype, DEV)
+
+    def run(self, lanes):
+        """lanes: [(request, x [t, hidden])] -> outputs per lane."""
+        from macllm_infer_amd.engine import Lane, build_step_context
+        for request, x in lanes:
+            if request not in self.cache.requests:
+                self.cache.add_request(request)
+        self.cache.reserve([(request, x.shape[0]) for request, x in lanes])
+        step = build_step_context([Lane(request, [0] * x.shape[0]) for request, x in lanes], self.cache, DEV)
+        x = torch.cat([x for _, x in lanes]).to(self.build.dtype).to(DEV)
+        out = self.part.forward(x, step, self.cache.entry((0, "p"))).float().cpu()
+        pieces, cursor = [], 0
+        for request, lane_x in lanes:
+            self.cache.commit(request, lane_x.shape[0])
+            pieces.append(out[cursor:cursor + lane_x.shape[0]])
+            cursor += lane_x.shape[0]
+        return pieces
+
+
+def rounded(tensors, dtype):
+    """What the part sees: matrices in ``dtype``; the plain model gets the same values."""
+    return {name: value.to(dtype) if value.dim() >= 2 else value for name, value in tensors.items()}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window, use_rope", [(None, True), (11, True), (None, False)])
+def test_attention_part_alone(dtype, window, use_rope):
+    """Hq*dh != hidden, 3 query heads per kv head, biases, all three multipliers; fed whole,
+    in portions and token by token, beside another request."""
+    from macllm_infer_amd.config import AttentionSpec, NoPositionSpec, RopeSpec
+    hidden, Hq, Hkv, dh = 40, 6, 2, 16
+    spec = AttentionSpec(num_heads=Hq, num_kv_heads=Hkv, head_dim=dh, scale=1 / math.sqrt(dh),
+                         position=RopeSpec(theta=1e4, rotary_dim=dh) if use_rope else NoPositionSpec(),
+                         window=window, qkv_bias=True, out_bias=True, in_multiplier=1.3, key_multiplier=0.7,
+                         out_multiplier=0.8)
+    tensors = {"q_proj.weight": rand(Hq * dh, hidden, seed=1, scale=0.3), "k_proj.weight": rand(Hkv * dh, hidden, seed=2, scale=0.3),
+               "v_proj.weight": rand(Hkv * dh, hidden, seed=3, scale=0.3), "o_proj.weight": rand(hidden, Hq * dh, seed=4, scale=0.2),
+               "q_proj.bias": rand(Hq * dh, seed=5, scale=0.1), "k_proj.bias": rand(Hkv * dh, seed=6, scale=0.1),
+               "v_proj.bias": rand(Hkv * dh, seed=7, scale=0.1), "o_proj.bias": rand(hidden, seed=8, scale=0.1)}
+    tensors = rounded(tensors, dtype)
+    x = rand(50, hidden, seed=9).to(dtype).float()
+    other = rand(23, hidden, seed=10).to(dtype).float()
+    plain = lambda rows: plain_impl.attention_mixer(
+        rows, tensors, num_heads=Hq, num_kv_heads=Hkv, head_dim=dh, theta=1e4, in_multiplier=1.3,
+        key_multiplier=0.7, out_multiplier=0.8, window=window, use_rope=use_rope)
+    want, want_other = plain(x), plain(other)
+    harness = PartHarness(spec, tensors, hidden, dtype)
+    assert (harness.run([("whole", x)])[0] - want).abs().max() < tolerance(dtype)
+    got, got_other = [], []
+    got.append(harness.run([("cut", x[:19])])[0])
+    a, b = harness.run([("cut", x[19:21]), ("other", other[:20])])
+    got.append(a), got_other.append(b)
+    for position in range(21, 24):
+        a, b = harness.run([("other", other[position - 1:position]), ("cut", x[position:position + 1])])
+        got.append(b), got_other.append(a)
+    got.append(harness.run([("cut", x[24:])])[0])
+    assert (torch.cat(got) - want).abs().max() < tolerance(dtype)
+    assert (torch.cat(got_other) - want_other[:23]).abs().max() < tolerance(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("gated_norm, bias, K", [(False, False, 4), (True, True, 3), (True, False, 2)])
+def test_mamba2_part_alone(dtype, gated_norm, bias, K):
+    from macllm_infer_amd.config import Mamba2Spec
+    hidden, H, P, N, G = 40, 6, 8, 24, 2
+    multipliers = (0.8, 1.4, 0.6, 1.5, 1.1)
+    spec = Mamba2Spec(num_heads=H, head_dim=P, state_size=N, num_groups=G, conv_kernel=K, chunk_size=8,
+                      norm_eps=2e-5, conv_bias=bias, proj_bias=bias, gated_norm=gated_norm, in_multiplier=1.2,
+                      out_multiplier=0.9, multipliers=multipliers)
+    E, C = H * P, H * P + 2 * G * N
+    tensors = {"in_proj.weight": rand(E + C + H, hidden, seed=1, scale=0.25), "conv1d.weight": rand(C, K, seed=2, scale=0.5),
+               "dt_bias": rand(H, seed=3) - 2.0, "A_log": torch.log(torch.rand(H, generator=torch.Generator().manual_seed(4)) * 3 + 0.2),
+               "D": rand(H, seed=5), "out_proj.weight": rand(hidden, E, seed=6, scale=0.2)}
+    if bias:
+        tensors.update({"conv1d.bias": rand(C, seed=7, scale=0.1), "in_proj.bias": rand(E + C + H, seed=8, scale=0.1),
+                        "out_proj.bias": rand(hidden, seed=9, scale=0.1)})
+    if gated_norm:
+        tensors["norm.weight"] = (rand(G, E // G, seed=10, scale=0.1) + 1.0)
+    tensors = rounded(tensors, dtype)
+    x = rand(60, hidden, seed=11).to(dtype).float()
+    other = rand(9, hidden, seed=12).to(dtype).float()
+    plain = lambda rows: plain_impl.mamba2_mixer(
+        rows, tensors, num_heads=H, head_dim=P, state_size=N, num_groups=G, conv_kernel=K, eps=2e-5,
+        in_multiplier=1.2, out_multiplier=0.9, multipliers=multipliers)
+    want, want_other = plain(x), plain(other)
+    harness = PartHarness(spec, tensors, hidden, dtype)
+    scale = max(1.0, want.abs().max().item())
+    assert (harness.run([("whole", x)])[0] - want).abs().max() < tolerance(dtype) * scale
+    got = [harness.run([("cut", x[:1])])[0]]                    # one token: shorter than the conv tail
+    a, b = harness.run([("other", other), ("cut", x[1:3])])
+    got.append(b)
+    assert (a - want_other).abs().max() < tolerance(dtype) * scale
+    got.append(harness.run([("cut", x[3:40])])[0])
+    for position in range(40, 60):
+        got.append(harness.run([("cut", x[position:position + 1])])[0])
+    assert (torch.cat(got) - want).abs().max() < tolerance(dtype) * scale
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_and_norm_parts_alone(dtype):
+    from macllm_infer_amd.config import RmsNormSpec, SwiGLUSpec
+    from macllm_infer_amd.kernels import build
+    from macllm_infer_amd.parts import BuildContext, Residual, RmsNorm, SwiGLU
+    build.ensure_modules(("common", "gemm"))
+    hidden, inner = 72, 100
+    context = BuildContext(hidden_size=hidden, dtype=dtype, device=torch.device(DEV), max_context=64)
+    tensors = rounded({"f.gate_proj.weight": rand(inner, hidden, seed=1, scale=0.2), "f.up_proj.weight": rand(inner, hidden, seed=2, scale=0.2),
+                       "f.down_proj.weight": rand(hidden, inner, seed=3, scale=0.2), "f.gate_proj.bias": rand(inner, seed=4, scale=0.1),
+                       "f.up_proj.bias": rand(inner, seed=5, scale=0.1), "f.down_proj.bias": rand(hidden, seed=6, scale=0.1)}, dtype)
+    ffn = SwiGLU(SwiGLUSpec(intermediate_size=inner, bias=True, gate_multiplier=1.25, down_multiplier=0.75), "f", tensors, context)
+    x = rand(13, hidden, seed=7).to(dtype)
+    want = plain_impl.swiglu_mlp(x.float(), {name[2:]: value for name, value in tensors.items()}, 1.25, 0.75)
+    assert (ffn.forward(x.to(DEV)).float().cpu() - want).abs().max() < tolerance(dtype)
+    weight = rand(hidden, seed=8, scale=0.1) + 1.0
+    norm = RmsNorm(RmsNormSpec(eps=3e-6), "n", {"n.weight": weight}, context)
+    h, delta = rand(13, hidden, seed=9), rand(13, hidden, seed=10).to(dtype)
+    residual = Residual(h.clone().to(DEV))
+    residual.pending = [delta.to(DEV)]
+    got = norm.forward(residual)
+    assert (residual.h.cpu() - (h + delta.float())).abs().max() < 1e-6 and residual.pending == []
+    assert (got.float().cpu() - plain_impl.rms_norm(h + delta.float(), weight, 3e-6)).abs().max() < tolerance(dtype)
+
+
+# ------------------------------------------------------------------ generation through the entry points
+@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16")])
+def test_greedy_generation_through_the_entry_point(tmp_path, name, dtype):
+    """The workload of the tiny configurations: prompts of 5/17/33 tokens, 12 greedy steps."""
+    from macllm_infer_amd import LLM, EngineConfig, SamplingParams, generate
+    folder = tiny_configs.make_model_dir(name, tmp_path, torch.float32 if dtype == "float32" else torch.bfloat16)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    prompts = [tokens_for(cfg["vocab_size"], length, 60 + length) for length in (5, 17, 33)]
+    llm = LLM(folder, dtype=dtype, kv_cache_block_tokens=16 if name == "A" else 8, kv_cache_capacity_tokens=256,
+              engine_config=EngineConfig(max_active_sequences=3, scheduler_token_budget=24, prefill_token_quantum=11))
+    params = SamplingParams(max_new_tokens=12, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0)
+    got = generate(llm, prompts, params)
+    for prompt, tokens in zip(prompts, got):
+        want = plain_impl.greedy_generate(cfg, tensors, prompt, 12)
+        if dtype == "float32":
+            assert tokens == want
+        else:       # bfloat16 may part ways where two logits are close; the first tokens agree
+            assert tokens[:2] == want[:2]
+    assert llm.engine.cache.stats()["live_requests"] == 0
+
+
+def test_seeded_sampling_through_the_entry_point(tmp_path):
+    """Config B's workload: five requests of 1/7/24/40/63 tokens, prompts cut into portions of
+    11, temperature 0.8 with seeded draws, 20 decode steps, pages of 8."""
+    from macllm_infer_amd import LLM, EngineConfig, SamplingParams
+    folder = tiny_configs.make_model_dir("B", tmp_path)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    prompts = [tokens_for(cfg["vocab_size"], length, 80 + length) for length in (1, 7, 24, 40, 63)]
+    llm = LLM(folder, dtype="float32", kv_cache_block_tokens=8, kv_cache_capacity_tokens=512,
+              engine_config=EngineConfig(max_active_sequences=5, scheduler_token_budget=64, prefill_token_quantum=11))
+    params = SamplingParams(max_new_tokens=20, temperature=0.8, top_k=0, top_p=1.0, repetition_penalty=1.0, seed=5)
+    results = llm.generate(prompts, params)
+    for index, (prompt, result) in enumerate(zip(prompts, results)):
+        tokens = list(prompt)
+        for draw in range(20):
+            logits = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-1]
+            tokens.append(plain_impl.sample_token(logits, temperature=0.8, seed=5 + index, draw_index=draw))
+        assert result.token_ids == tokens[len(prompt):] and result.finish_reason == "length"
+        assert result.time_to_first_token is not None and result.total_time > 0
+
+
+def test_command_line_run(tmp_path):
+    folder = tiny_configs.make_model_dir("A", tmp_path)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    prompt = tokens_for(cfg["vocab_size"], 9, 70)
+    done = subprocess.run([sys.executable, "-m", "macllm_infer_amd", "run", "-m", folder, "--dtype", "f32",
+                           "--tokens", ",".join(map(str, prompt)), "--max-new-tokens", "5", "--temperature", "0",
+                           "--repetition-penalty", "1.0", "--prefill-token-quantum", "4"],
+                          cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr
+    assert [int(t) for t in done.stdout.split()] == plain_impl.greedy_generate(cfg, tensors, prompt, 5)
+    assert "finish=length" in done.stderr and "decode_tok_s" in done.stderr
+
+
+# ------------------------------------------------------------------ generality, shown with toy parts
+@pytest.mark.parametrize("schedule", toy_parts.SCHEDULES, ids=toy_parts.SCHEDULE_IDS)
+def test_toy_parts_register_build_and_step(schedule):
+    """A mixer with state of its own, another position encoding, a windowed layer whose pages
+    are given back, a layer that runs twice with two caches and a run that reads another
+    run's cache: registered in the tests, built by the engine, stepped whole, in portions
+    and mixed, on the GPU with the package's kernels."""
+    toy_parts.exercise(schedule, DEV, check_device=True)

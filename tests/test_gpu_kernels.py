@@ -1,0 +1,377 @@
+"""Each HIP kernel alone against its plain PyTorch reference (tests/ref_ops.py), at sizes
+other than the tiny models': head sizes in steps of 16, odd head and group counts, widths
+and vocabularies that are no power of two, several page sizes; and inputs built so that a
+fault that random data would hide (a far key, a window's edge, a page's edge) shows."""
+import math
+
+import pytest
+import torch
+
+import ref_ops
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from macllm_infer_amd.kernels import build, ops as module
+    module.require_gpu(DEV)
+    build.ensure_modules(build.MODULES)
+    return module
+
+
+def rand(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    return (torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale).to(dtype)
+
+
+def tol(dtype, scale=1.0):
+    return (3e-5 if dtype == torch.float32 else 2.5e-2) * scale
+
+
+def gpu(*tensors):
+    return [None if t is None else t.to(DEV) for t in tensors]
+
+
+def i32(values):
+    return torch.tensor(values, dtype=torch.int32)
+
+
+def close(got, want, dtype, scale=1.0):
+    got, want = got.float().cpu(), want.float()
+    assert torch.isfinite(got).all()
+    error = (got - want).abs().max().item()
+    assert error <= tol(dtype, scale), f"max error {error}"
+
+
+# ------------------------------------------------------------------ common
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("d", [40, 1000, 4100])
+def test_embed_and_add_rmsnorm(ops, dtype, d):
+    T, V = 7, 203
+    table = rand(V, d, seed=1, dtype=dtype)
+    ids = i32([0, 202, 5, 5, 17, 100, 1])
+    want_h = torch.empty(T, d)
+    ref_ops.embed(ids, table, 1.7, want_h)
+    h = torch.empty(T, d, device=DEV)
+    ops.embed(ids.to(DEV), table.to(DEV), 1.7, h)
+    close(h, want_h, torch.float32)
+    deltas = [rand(T, d, seed=2, dtype=dtype), rand(T, d, seed=3, dtype=dtype)]
+    weight = rand(d, seed=4) + 1.0
+    for count in (0, 1, 2):
+        want_h2, want_out = want_h.clone(), torch.empty(T, d, dtype=dtype)
+        ref_ops.add_rmsnorm(want_h2, deltas[:count], weight, 3e-6, want_out)
+        h2, out = h.clone(), torch.empty(T, d, dtype=dtype, device=DEV)
+        ops.add_rmsnorm(h2, gpu(*deltas[:count]), weight.to(DEV), 3e-6, out)
+        close(h2, want_h2, torch.float32)
+        close(out, want_out, dtype, 4.0)
+    rows = i32([6, 0, 3])
+    want_out = torch.empty(3, d, dtype=dtype)
+    keep = want_h.clone()
+    ref_ops.add_rmsnorm(keep, deltas[:1], weight, 1e-5, want_out, rows)
+    h3, out = h.clone(), torch.empty(3, d, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(h3, gpu(deltas[0]), weight.to(DEV), 1e-5, out, rows.to(DEV))
+    close(out, want_out, dtype, 4.0)
+    assert torch.equal(h3, h)                                   # with rows the stream is left alone
+
+
+def test_rmsnorm_refuses_a_width_beyond_its_limit(ops):
+    h = torch.zeros(1, 20000, device=DEV)
+    with pytest.raises(ops.KernelError, match="size not supported"):
+        ops.add_rmsnorm(h, [], torch.ones(20000, device=DEV), 1e-5, torch.empty(1, 20000, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu_and_scale(ops, dtype):
+    gu = rand(9, 2 * 77, seed=5, scale=2.0, dtype=dtype)
+    want = torch.empty(9, 77, dtype=dtype)
+    ref_ops.swiglu(gu, want)
+    out = torch.empty(9, 77, dtype=dtype, device=DEV)
+    ops.swiglu(gu.to(DEV), out)
+    close(out, want, dtype, 4.0)
+    logits = torch.empty(9, 154, device=DEV)
+    ops.scale_to_f32(gu.to(DEV), 0.6, logits)
+    close(logits, gu.float() * 0.6, torch.float32)
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 32), (5, 130, 97), (67, 100, 260), (130, 33, 1000)])
+def test_float32_product_is_true_float32(ops, shape):
+    M, N, K = shape
+    x, w, b = rand(M, K, seed=6), rand(N, K, seed=7), rand(N, seed=8)
+    want = (x.double() @ w.double().T + b.double()).float()
+    got = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV))
+    assert (got.cpu() - want).abs().max() < 2e-5 * math.sqrt(K)       # float32 rounding only
+    # a row's result does not depend on the rows beside it
+    alone = ops.linear(x[:1].to(DEV), w.to(DEV), b.to(DEV))
+    assert torch.equal(alone[0], got[0])
+    # a strided input (a column block of a wider matrix)
+    wide = rand(M, K + 24, seed=9)
+    got = ops.linear(wide.to(DEV)[:, 8:8 + K], w.to(DEV), None)
+    assert (got.cpu() - (wide[:, 8:8 + K].double() @ w.double().T).float()).abs().max() < 2e-5 * math.sqrt(K)
+
+
+def test_mixed_product_keeps_a_32bit_weight(ops):
+    x, w = rand(4, 96, seed=10, dtype=torch.bfloat16), rand(50, 96, seed=11)
+    got = ops.linear(x.to(DEV), w.to(DEV), None)
+    assert got.dtype == torch.bfloat16
+    close(got, (x.float() @ w.T).to(torch.bfloat16), torch.bfloat16, 10.0)
+    both = ops.linear(x.to(DEV), w.to(torch.bfloat16).to(DEV), rand(50, seed=12).to(DEV))
+    close(both, x.float() @ w.to(torch.bfloat16).float().T + rand(50, seed=12), torch.bfloat16, 10.0)
+
+
+# ------------------------------------------------------------------ attention
+def paged_setup(lengths, page_size, Hkv, dh, dtype, layers=2, seed=0):
+    """A pool of shuffled pages [page, layer, K|V, Hkv, page_size, dh] and a block table per lane."""
+    generator = torch.Generator().manual_seed(seed)
+    pages_per_lane = [-(-length // page_size) for length in lengths]
+    total = sum(pages_per_lane) + 3
+    order = torch.randperm(total, generator=generator).tolist()
+    table = torch.zeros(len(lengths), max(pages_per_lane), dtype=torch.int32)
+    cursor = 0
+    for lane, count in enumerate(pages_per_lane):
+        table[lane, :count] = torch.tensor(order[cursor:cursor + count], dtype=torch.int32)
+        cursor += count
+    pool = torch.full((total, layers, 2, Hkv, page_size, dh), float("nan"), dtype=dtype)
+    return pool, table
+
+
+def fill_cache(pool, table, lane, keys, values, page_size, layer=1):
+    for position in range(keys.shape[0]):
+        page = int(table[lane, position // page_size])
+        pool[page, layer, 0, :, position % page_size, :] = keys[position]
+        pool[page, layer, 1, :, position % page_size, :] = values[position]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq, Hkv, dh, page_size, rotary", [
+    (4, 2, 16, 8, 16), (5, 5, 48, 16, 48), (6, 2, 80, 4, 32), (8, 2, 64, 64, 64), (3, 1, 128, 16, 128),
+    (2, 1, 256, 32, 256)])
+def test_rope_store_and_attention_over_pages(ops, dtype, Hq, Hkv, dh, page_size, rotary):
+    """Three lanes: a prompt portion that continues a cached prefix, a single decoded token,
+    and a fresh prompt.  Every unwritten cache cell holds NaN, so reading a cell that is
+    not the request's shows."""
+    starts, counts = [21, 70, 0], [13, 1, 37]
+    lengths = [s + c for s, c in zip(starts, counts)]
+    pool, table = paged_setup(lengths, page_size, Hkv, dh, dtype)
+    for lane, start in enumerate(starts):       # prefixes already in the cache (post-rotation keys)
+        fill_cache(pool, table, lane, rand(start, Hkv, dh, seed=20 + lane, dtype=dtype),
+                   rand(start, Hkv, dh, seed=30 + lane, dtype=dtype), page_size)
+    T = sum(counts)
+    width = (Hq + 2 * Hkv) * dh
+    qkv = rand(T, width + 8, seed=40, dtype=dtype)            # wider than needed: a row stride
+    positions = torch.cat([torch.arange(s, s + c) for s, c in zip(starts, counts)]).to(torch.int32)
+    lane_of_token = torch.repeat_interleave(torch.arange(3), torch.tensor(counts)).to(torch.int32)
+    slot_mapping = torch.tensor([int(table[l, p // page_size]) * page_size + p % page_size
+                                 for l, p in zip(lane_of_token.tolist(), positions.tolist())], dtype=torch.int32)
+    inv_freq = torch.tensor([1.0 / (1e4 ** (i / rotary)) for i in range(0, rotary, 2)], dtype=torch.float64).float()
+    want_qkv, want_pool = qkv.clone(), pool.clone()
+    ref_ops.rope_kv_store(want_qkv, Hq, Hkv, dh, positions, inv_freq, rotary, slot_mapping,
+                          want_pool[:, 1, 0], want_pool[:, 1, 1])
+    got_qkv, got_pool = qkv.to(DEV), pool.to(DEV)
+    ops.rope_kv_store(got_qkv, Hq, Hkv, dh, positions.to(DEV), inv_freq.to(DEV), rotary, slot_mapping.to(DEV),
+                      got_pool[:, 1, 0], got_pool[:, 1, 1])
+    close(got_qkv[:, :Hq * dh], want_qkv[:, :Hq * dh], dtype, 4.0)
+    assert torch.equal(got_qkv[:, Hq * dh:].cpu(), qkv[:, Hq * dh:])         # k, v columns untouched
+    written = ~torch.isnan(want_pool.float())
+    assert torch.equal(torch.isnan(got_pool.float().cpu()), ~written)          # exactly the same cells
+    close(torch.nan_to_num(got_pool.float()), torch.nan_to_num(want_pool.float()), dtype, 4.0)
+    assert torch.isnan(got_pool[:, 0].float()).all()                           # the other layer is untouched
+    for window in (None, 9):
+        want = torch.empty(T, Hq * dh, dtype=dtype)
+        ref_ops.paged_attention(want_qkv, Hq, Hkv, dh, want_pool[:, 1, 0], want_pool[:, 1, 1], table,
+                                lane_of_token, positions, 0.37, window, want)
+        got = torch.empty(T, Hq * dh, dtype=dtype, device=DEV)
+        ops.paged_attention(got_qkv, Hq, Hkv, dh, got_pool[:, 1, 0], got_pool[:, 1, 1], table.to(DEV),
+                            lane_of_token.to(DEV), positions.to(DEV), 0.37, window, got)
+        close(got, want, dtype, 3.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_one_far_key_among_hundreds_is_found(ops, dtype, page_size):
+    """One decoded token over 700 cached keys.  The query and one chosen key are scaled so that
+    this key takes all the weight: the output must be that key's value, for keys at the
+    start, at both sides of page edges, and at the end."""
+    Hq, Hkv, dh, length = 4, 2, 64, 700
+    pool, table = paged_setup([length], page_size, Hkv, dh, dtype, seed=3)
+    values = rand(length, Hkv, dh, seed=50, dtype=dtype)
+    base_keys = rand(length, Hkv, dh, seed=51, scale=0.1, dtype=dtype)
+    direction = torch.zeros(dh)
+    direction[5] = 1.0
+    for chosen in (0, 1, page_size - 1, page_size, 63, 64, 65, 511, 512, length - 2, length - 1):
+        keys = base_keys.clone()
+        keys[chosen] = (direction * 30.0).to(dtype)
+        fill_cache(pool, table, 0, keys, values, page_size)
+        q = (direction * 30.0).repeat(Hq)[None].to(dtype)
+        out = torch.empty(1, Hq * dh, dtype=dtype, device=DEV)
+        dev_pool = pool.to(DEV)
+        ops.paged_attention(q.to(DEV), Hq, Hkv, dh, dev_pool[:, 1, 0], dev_pool[:, 1, 1], table.to(DEV),
+                            i32([0]).to(DEV), i32([length - 1]).to(DEV), 1.0 / math.sqrt(dh), None, out)
+        expected = values[chosen].float()[[0, 0, 1, 1]].reshape(-1)
+        assert (out.float().cpu()[0] - expected).abs().max() < 1e-2, f"key {chosen} was missed"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_window_edge(ops, dtype):
+    """Window 37 at query position 299: key 263 is the last one inside, key 262 the first one
+    outside.  Whichever is made to stand out, the output tells whether it was seen."""
+    Hq, Hkv, dh, length, window, page_size = 2, 1, 32, 300, 37, 16
+    pool, table = paged_setup([length], page_size, Hkv, dh, dtype, seed=4)
+    values = rand(length, Hkv, dh, seed=52, dtype=dtype)
+    direction = torch.zeros(dh)
+    direction[0] = 1.0
+    q = (direction * 30.0).repeat(Hq)[None].to(dtype).to(DEV)
+    for chosen, visible in ((263, True), (262, False), (299, True), (0, False)):
+        keys = rand(length, Hkv, dh, seed=53, scale=0.1, dtype=dtype)
+        keys[chosen] = (direction * 30.0).to(dtype)
+        fill_cache(pool, table, 0, keys, values, page_size)
+        dev_pool = pool.to(DEV)
+        out = torch.empty(1, Hq * dh, dtype=dtype, device=DEV)
+        ops.paged_attention(q, Hq, Hkv, dh, dev_pool[:, 1, 0], dev_pool[:, 1, 1], table.to(DEV), i32([0]).to(DEV),
+                            i32([length - 1]).to(DEV), 1.0 / math.sqrt(dh), window, out)
+        hit = (out.float().cpu()[0, :dh] - values[chosen, 0].float()).abs().max() < 1e-2
+        assert hit == visible, f"key {chosen} should be {'visible' if visible else 'masked'}"
+        want = torch.empty(1, Hq * dh, dtype=dtype)
+        ref_ops.paged_attention(q.cpu(), Hq, Hkv, dh, pool[:, 1, 0], pool[:, 1, 1], table, i32([0]),
+                                i32([length - 1]), 1.0 / math.sqrt(dh), window, want)
+        close(out, want, dtype, 3.0)
+
+
+def test_attention_refuses_a_head_size_beyond_its_limit(ops):
+    pool = torch.zeros(2, 1, 2, 1, 16, 320, device=DEV)
+    q = torch.zeros(1, 320, device=DEV)
+    with pytest.raises(ops.KernelError, match="size not supported"):
+        ops.paged_attention(q, 1, 1, 320, pool[:, 0, 0], pool[:, 0, 1], i32([[0]]).to(DEV), i32([0]).to(DEV),
+                            i32([0]).to(DEV), 1.0, None, torch.empty(1, 320, device=DEV))
+
+
+# ------------------------------------------------------------------ mamba2
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H, P, N, G, K", [(8, 8, 16, 1, 4), (6, 16, 32, 2, 3), (3, 24, 40, 3, 2), (4, 64, 128, 1, 4),
+                                             (2, 40, 256, 2, 4), (5, 7, 9, 1, 1)])
+def test_mamba2_kernels_over_ragged_lanes(ops, dtype, H, P, N, G, K):
+    """Lanes of 1, 2 (shorter than the conv tail), 19 and 45 tokens with non-zero conv tails
+    and states in shuffled slots; the slot no lane uses must stay as it was."""
+    E, GN = H * P, G * N
+    C, W = E + 2 * GN, 2 * E + 2 * GN + H
+    counts = [1, 2, 19, 45]
+    T = sum(counts)
+    slots = 6
+    slot_ids = i32([4, 0, 5, 2])
+    cu = i32([0, 1, 3, 22, 67])
+    lane_of_token = torch.repeat_interleave(torch.arange(4), torch.tensor(counts)).to(torch.int32)
+    u = rand(T, W, seed=60, dtype=dtype)
+    conv_w, conv_b = rand(C, K, seed=61, scale=0.5), rand(C, seed=62, scale=0.1)
+    conv_state = rand(slots, max(K - 1, 0), C, seed=63, dtype=dtype)
+    ssm_state = rand(slots, H, P, N, seed=64, scale=0.5)
+    dt_bias, A, D = rand(H, seed=65) - 2.0, -(rand(H, seed=66).abs() + 0.1), rand(H, seed=67)
+    norm_w = rand(E, seed=68) + 1.0
+
+    def run(module, device):
+        mv = lambda t: None if t is None else t.to(device)
+        uu, cs, ss = mv(u), mv(conv_state.clone()), mv(ssm_state.clone())
+        xbc = torch.empty(T, C, dtype=dtype, device=device)
+        module.conv1d_silu(uu, E, C, mv(conv_w), mv(conv_b), cs, mv(lane_of_token), mv(cu), mv(slot_ids), xbc)
+        module.conv_state_update(uu, E, C, K, cs, mv(cu), mv(slot_ids))
+        y = torch.empty(T, E, dtype=torch.float32, device=device)
+        module.ssm_scan(xbc, uu[:, E + C:], mv(dt_bias), mv(A), mv(D), ss, mv(cu), mv(slot_ids), G, y)
+        outs = []
+        for weight in (None, norm_w):
+            out = torch.empty(T, E, dtype=dtype, device=device)
+            module.gate_norm(y, uu[:, :E], mv(weight), G, 1e-5, out)
+            outs.append(out)
+        return xbc, cs, ss, y, outs
+
+    want = run(ref_ops, "cpu")
+    got = run(ops, DEV)
+    close(got[0], want[0], dtype, 4.0)
+    close(got[1], want[1], dtype)
+    scale = max(1.0, want[3].abs().max().item())
+    # the scan's inputs are the GPU conv outputs; in bfloat16 they may differ from the reference's by one rounding
+    close(got[2], want[2], dtype, scale)
+    close(got[3], want[3], dtype, scale)
+    close(got[4][0], want[4][0], dtype, scale)
+    close(got[4][1], want[4][1], dtype, 8.0)
+    for untouched in (1, 3):
+        assert torch.equal(got[1][untouched].cpu(), conv_state[untouched])
+        assert torch.equal(got[2][untouched].cpu(), ssm_state[untouched])
+
+
+def test_scan_refuses_a_state_size_beyond_its_limit(ops):
+    with pytest.raises(ops.KernelError, match="size not supported"):
+        ops.ssm_scan(torch.zeros(1, 1 + 2 * 600, device=DEV), torch.zeros(1, 1, device=DEV), torch.zeros(1, device=DEV),
+                     torch.zeros(1, device=DEV), torch.zeros(1, device=DEV), torch.zeros(1, 1, 1, 600, device=DEV),
+                     i32([0, 1]).to(DEV), i32([0]).to(DEV), 1, torch.zeros(1, 1, device=DEV))
+
+
+def test_softplus_is_stable_in_the_scan(ops):
+    """dt = +-100 (the fixture of crates/macllm-kernels/src/mamba2.rs:561-565)."""
+    H, P, N = 2, 4, 8
+    xbc = rand(3, H * P + 2 * N, seed=70)
+    dt = torch.tensor([[100.0, -100.0], [0.2, -0.7], [-100.0, 100.0]])
+    args = [torch.zeros(H), -torch.ones(H) * 0.03, torch.ones(H)]
+    state = rand(1, H, P, N, seed=71)
+    want_y, want_state = torch.empty(3, H * P), state.clone()
+    ref_ops.ssm_scan(xbc, dt, *args, want_state, i32([0, 3]), i32([0]), 1, want_y)
+    y, dev_state = torch.empty(3, H * P, device=DEV), state.to(DEV)
+    ops.ssm_scan(xbc.to(DEV), dt.to(DEV), *gpu(*args), dev_state, i32([0, 3]).to(DEV), i32([0]).to(DEV), 1, y)
+    close(y, want_y, torch.float32, 30.0)
+    close(dev_state, want_state, torch.float32, 30.0)
+
+
+# ------------------------------------------------------------------ sampling
+def test_argmax_and_ties(ops):
+    logits = rand(5, 1003, seed=80)
+    logits[1, 17] = logits[1, 900] = 9.0                         # a tie: the lower index wins
+    logits[2, 1002] = 11.0
+    out = torch.empty(5, dtype=torch.int32, device=DEV)
+    ops.argmax(logits.to(DEV), out)
+    assert out.cpu().tolist() == torch.argmax(logits, -1).tolist()
+    assert out.cpu()[1] == 17 and out.cpu()[2] == 1002
+
+
+@pytest.mark.parametrize("V", [320, 1003, 32784])
+def test_sampling_matches_the_plain_sampler(ops, V):
+    import plain_impl
+    settings = [(0.8, 0, 1.0), (1.0, 7, 1.0), (0.9, 0, 0.7), (1.2, 40, 0.85), (0.0, 0, 1.0), (0.7, 20, 0.8),
+                (1.0, V + 5, 0.999), (0.5, 1, 0.1)]
+    B = len(settings)
+    logits = rand(B, V, seed=81, scale=2.5)
+    seeds = [3, 99, 2 ** 63 + 5, 42, 0, 7, 11, 13]
+    draws = [0, 5, 17, 3, 0, 100, 1, 2]
+    padded = 1
+    while padded < V:
+        padded <<= 1
+    for repeat in range(3):
+        work = logits.clone().to(DEV)
+        out = torch.empty(B, dtype=torch.int32, device=DEV)
+        signed = [s - (1 << 64) if s >= (1 << 63) else s for s in seeds]
+        ops.sample(work, torch.tensor([s[0] for s in settings]).to(DEV), i32([s[1] for s in settings]).to(DEV),
+                   torch.tensor([s[2] for s in settings]).to(DEV), torch.tensor(signed, dtype=torch.int64).to(DEV),
+                   i32([d + repeat for d in draws]).to(DEV),
+                   torch.empty(B, padded, dtype=torch.int64, device=DEV), out)
+        want = [plain_impl.sample_token(logits[row], temperature=settings[row][0], top_k=settings[row][1],
+                                        top_p=settings[row][2], seed=seeds[row], draw_index=draws[row] + repeat)
+                for row in range(B)]
+        assert out.cpu().tolist() == want
+
+
+def test_penalties_match_the_plain_rule(ops):
+    V = 500
+    logits = rand(3, V, seed=82)
+    histories = [[5, 9, 5, 400, 9, 9], [], [1, 2, 3, 499]]
+    prompt_lens = [2, 0, 4]
+    flat = [token for history in histories for token in history]
+    offsets = [0, 6, 6, 10]
+    rep, pres, freq = [1.3, 1.0, 2.0], [0.5, 0.0, 0.0], [0.25, 0.0, 0.3]
+    want = logits.clone()
+    ref_ops.apply_penalties(want, i32(flat), i32(offsets), i32(prompt_lens), torch.tensor(rep), torch.tensor(pres),
+                            torch.tensor(freq), None, None)
+    got = logits.clone().to(DEV)
+    counts = [torch.zeros(3 * V, dtype=torch.int32, device=DEV) for _ in range(2)]
+    ops.apply_penalties(got, i32(flat).to(DEV), i32(offsets).to(DEV), i32(prompt_lens).to(DEV),
+                        torch.tensor(rep).to(DEV), torch.tensor(pres).to(DEV), torch.tensor(freq).to(DEV), *counts)
+    close(got, want, torch.float32)
+    assert not torch.equal(want, logits) and int(counts[0].sum()) == 0 and int(counts[1].sum()) == 0

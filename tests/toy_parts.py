@@ -1,0 +1,212 @@
+"""Toy parts for the tests of the framework's generality: a mixer with state of its own, a
+position encoding that is no rotation, and a toy architecture that uses them together with a
+windowed attention layer, a layer that runs twice and a run that reads another run's cache.
+They are registered from here, without a change to the package, and never become a model."""
+from dataclasses import dataclass
+
+import torch
+
+import plain_impl
+
+@dataclass(frozen=True)
+class DecayMixerSpec:
+    """A toy mixer with state of its own: s_t = a * s_{t-1} + x_t W; y_t = s_t."""
+    width: int
+    decay: float
+    kind: str = "toy_decay"
+
+    def validate(self):
+        assert 0 < self.decay < 1
+
+
+@dataclass(frozen=True)
+class AlibiLikeSpec:
+    """A toy position encoding: scales q and k of head h by (1 + position * slope_h)."""
+    slope: float
+    kind: str = "toy_scale_position"
+
+    def validate(self, head_dim):
+        pass
+
+
+@dataclass
+class ToyConfig:
+    """A toy architecture: layer 0 = attention (toy position encoding) and the decay mixer in
+    parallel, layer 1 = windowed attention with partial RoPE.  ``raw["schedule"]`` lists
+    (layer, entry whose cache is read or None) in running order."""
+    raw: dict
+    architecture_names = ("ToyForTests",)
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw)
+
+    def to_dict(self):
+        return dict(self.raw)
+
+    def to_model_spec(self):
+        from macllm_infer_amd.config import (AttentionSpec, LayerSpec, MixerSlot, ModelSpec, RmsNormSpec, RopeSpec,
+                                             ScheduleEntry, SwiGLUSpec)
+        raw = self.raw
+        hidden = raw["hidden"]
+        norm = RmsNormSpec(eps=1e-5)
+        full = AttentionSpec(num_heads=4, num_kv_heads=2, head_dim=16, scale=0.25,
+                             position=AlibiLikeSpec(slope=raw["slope"]))
+        windowed = AttentionSpec(num_heads=4, num_kv_heads=2, head_dim=16, scale=0.25,
+                                 position=RopeSpec(theta=100.0, rotary_dim=8), window=raw["window"])
+        ffn = SwiGLUSpec(intermediate_size=48)
+        layers = (LayerSpec(prefix="model.layers.0", ffn=ffn, mixer_norm=norm, ffn_norm=norm,
+                            mixers=(MixerSlot("self_attn", full), MixerSlot("decay", DecayMixerSpec(hidden, raw["decay"])))),
+                  LayerSpec(prefix="model.layers.1", ffn=ffn, mixer_norm=norm, ffn_norm=norm,
+                            mixers=(MixerSlot("self_attn", windowed),)))
+        schedule = tuple(ScheduleEntry(layer=layer, kv_from=source) for layer, source in raw["schedule"])
+        return ModelSpec(architecture="ToyForTests", hidden_size=hidden, vocab_size=raw["vocab"], max_context=512,
+                         layers=layers, schedule=schedule, final_norm=norm, tied_embeddings=True)
+
+
+def register_toys():
+    from macllm_infer_amd.cache import StateNeed
+    from macllm_infer_amd.config import register_architecture
+    from macllm_infer_amd.parts import Mixer, PositionEncoding, register_part
+    from macllm_infer_amd.weights import Expect
+
+    @register_part("toy_decay")
+    class DecayMixer(Mixer):
+        kernel_modules = ()
+
+        @classmethod
+        def expected_tensors(cls, spec, prefix, hidden_size):
+            return [Expect(f"{prefix}.w.weight", ((spec.width, hidden_size),))]
+
+        @classmethod
+        def cache_needs(cls, spec):
+            return [StateNeed("s", (spec.width,), "float32")]
+
+        def __init__(self, spec, prefix, tensors, build):
+            self.spec = spec
+            self.weight = tensors[f"{prefix}.w.weight"].float().to(build.device)
+
+        def forward(self, x, step, cache):
+            state = cache.states["s"]
+            projected = x.float() @ self.weight.T
+            out = torch.empty_like(projected)
+            cursor = 0
+            for lane, length in enumerate(step.lane_lengths):          # a toy: token-serial on the host
+                slot = int(step.slot_ids[lane])
+                s = state[slot].clone()
+                for t in range(cursor, cursor + length):
+                    s = self.spec.decay * s + projected[t]
+                    out[t] = s
+                state[slot] = s
+                cursor += length
+            return out.to(x.dtype)
+
+    @register_part("toy_scale_position")
+    class ScalePosition(PositionEncoding):
+        def __init__(self, spec, head_dim, build):
+            self.slope = spec.slope
+
+        def rotate(self, qkv, num_heads, num_kv_heads, head_dim, step):
+            factor = (1.0 + step.positions.float() * self.slope)[:, None]
+            width = (num_heads + num_kv_heads) * head_dim
+            qkv[:, :width] = (qkv[:, :width].float() * factor).to(qkv.dtype)
+
+    register_architecture(ToyConfig)
+
+
+def toy_plain_logits(raw, tensors, tokens):
+    """The toy model, whole sequence, from the plain parts."""
+    T = len(tokens)
+    positions = torch.arange(T)
+    h = tensors["model.embed_tokens.weight"].float()[torch.tensor(tokens)]
+    caches = {}
+    for index, (layer, source) in enumerate(raw["schedule"]):
+        p = f"model.layers.{layer}."
+        n = plain_impl.rms_norm(h, tensors[p + "attn_norm.weight"], 1e-5)
+        w = {name[len(p + "self_attn."):]: value for name, value in tensors.items() if name.startswith(p + "self_attn.")}
+        q = plain_impl.linear(n, w["q_proj.weight"], None).view(T, 4, 16)
+        k = plain_impl.linear(n, w["k_proj.weight"], None).view(T, 2, 16)
+        v = plain_impl.linear(n, w["v_proj.weight"], None).view(T, 2, 16)
+        if layer == 0:
+            factor = (1.0 + positions.float() * raw["slope"])[:, None, None]
+            q, k = q * factor, k * factor
+            window = None
+        else:
+            q = plain_impl.rope_half_split(q, positions, 100.0, rotary_dim=8)
+            k = plain_impl.rope_half_split(k, positions, 100.0, rotary_dim=8)
+            window = raw["window"]
+        if source is None:
+            caches[index] = (k, v)
+        else:
+            k, v = caches[source]                       # reads the other run's keys and values
+        mixed = plain_impl.linear(plain_impl.gqa_causal_attention(q, k, v, 0.25, window).reshape(T, 64),
+                                  w["o_proj.weight"], None)
+        if layer == 0:
+            projected = n @ tensors[p + "decay.w.weight"].float().T
+            s = torch.zeros(raw["hidden"])
+            rows = []
+            for t in range(T):
+                s = raw["decay"] * s + projected[t]
+                rows.append(s)
+            mixed = mixed + torch.stack(rows)
+        h = h + mixed
+        f = plain_impl.rms_norm(h, tensors[p + "ffn_norm.weight"], 1e-5)
+        h = h + plain_impl.swiglu_mlp(f, {name[len(p + "mlp."):]: value for name, value in tensors.items()
+                                          if name.startswith(p + "mlp.")})
+    h = plain_impl.rms_norm(h, tensors["model.norm.weight"], 1e-5)
+    return h @ tensors["model.embed_tokens.weight"].float().T
+
+
+
+
+SCHEDULES = [[(0, None), (1, None)], [(0, None), (0, None), (1, None), (1, 2)]]
+SCHEDULE_IDS = ["plain-order", "layer-twice-and-shared-cache"]
+
+
+def tokens_for(vocab, count, seed):
+    return torch.randint(0, vocab, (count,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def exercise(schedule, device, check_device):
+    """Register the toys, build the toy model through the engine and compare whole, cut and
+    mixed steps with ``toy_plain_logits``."""
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.engine.model import DecoderModel
+    from macllm_infer_amd.weights.random_init import random_tensors
+    register_toys()
+    raw = {"architectures": ["ToyForTests"], "hidden": 32, "vocab": 90, "slope": 0.01, "decay": 0.9, "window": 13,
+           "schedule": schedule}
+    config = ToyConfig(raw)
+    tensors = random_tensors(config, 5, torch.float32, "unit")
+    assert "model.layers.0.decay.w.weight" in tensors
+    engine = Engine(config=config, tensors=tensors, dtype="float32", device=device, kv_cache_block_tokens=4,
+                    kv_cache_capacity_tokens=160, max_active_sequences=3, check_device=check_device)
+    windows = sorted(str(group.need.window) for group in engine.cache.groups)
+    assert windows == ["13", "None"]                                           # two groups, pages of their own
+    if len(schedule) == 4:
+        assert len(engine.cache.groups[0].members) == 2 and not engine.cache.entry((3, "self_attn")).owns_kv
+    first, second = tokens_for(90, 70, 1), tokens_for(90, 41, 2)
+    want_first, want_second = toy_plain_logits(raw, tensors, first), toy_plain_logits(raw, tensors, second)
+    engine.add_request("whole")
+    got = engine.step([Lane("whole", first, list(range(70)))]).cpu()
+    assert (got - want_first).abs().max() < 1e-4
+    engine.finish("whole")
+    engine.add_request("a")
+    engine.add_request("b")
+    rows_a, rows_b = [], []
+    rows_a.append(engine.step([Lane("a", first[:30], list(range(30)))]).cpu())
+    out = engine.step([Lane("a", first[30:32], [0, 1]), Lane("b", second[:25], list(range(25)))]).cpu()
+    rows_a.append(out[:2]), rows_b.append(out[2:])
+    for position in range(32, 70):
+        lanes = [Lane("a", first[position:position + 1], [0])]
+        if position - 7 < 41:
+            lanes.insert(0, Lane("b", second[position - 7:position - 6], [0]))
+        out = engine.step(lanes).cpu()
+        rows_a.append(out[-1:])
+        if len(lanes) == 2:
+            rows_b.append(out[:1])
+    assert (torch.cat(rows_a) - want_first).abs().max() < 1e-4
+    assert (torch.cat(rows_b) - want_second[:len(torch.cat(rows_b))]).abs().max() < 1e-4
+    window_group = [group for group in engine.cache.groups if group.need.window][0]
+    assert len(window_group.tables["a"].live_pages()) <= 5 < len(window_group.tables["a"].pages)   # passed pages went back
+    engine.cache.check()
