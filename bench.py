@@ -1,0 +1,162 @@
+"""Decode and prefill throughput of a Falcon-H1 0.5B-shaped model with random weights on one
+MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|f32] [--layers L]
+
+One JSON line: ``value`` = decoded tokens a second at batch 8 with every request at a
+2,048-token context (a step = one decode step of the whole batch: model, greedy sampling,
+tokens fed back); ``prefill`` = one 2,048-token prompt in one step; ``roofline`` = the bytes
+the decode step has to read (every weight it uses once, and the cache and state of the live
+requests) over its time, against 8 TB/s; ``points`` = decode at batch 1 and 64.
+"""
+import argparse
+import json
+import sys
+import time
+
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "f32": 157.3e12}
+
+# Falcon-H1-0.5B-shaped: the layer sizes of the benchmark configuration
+SHAPE = dict(
+    architectures=["FalconH1ForCausalLM"], model_type="falcon_h1", hidden_size=1024, num_hidden_layers=36,
+    num_attention_heads=8, num_key_value_heads=2, head_dim=64, intermediate_size=2048, vocab_size=32784,
+    max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=1e11, mamba_n_heads=24, mamba_d_head=64,
+    mamba_d_ssm=1536, mamba_d_state=128, mamba_n_groups=1, mamba_d_conv=4, mamba_chunk_size=128,
+    mamba_conv_bias=True, mamba_proj_bias=False, mamba_rms_norm=False, attention_bias=False, mlp_bias=False,
+    tie_word_embeddings=True)
+CONTEXT = 2048
+PREFILL_TOKENS = 2048
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
+    parser.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"],
+                        help="fewer layers than the configuration's 36 (both numbers are reported)")
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--page-tokens", type=int, default=16)
+    parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
+        return 2
+
+    import torch
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.sampling import GREEDY, Sampler, SamplerRow
+    from macllm_infer_amd.weights.random_init import random_tensors
+
+    raw = dict(SHAPE, num_hidden_layers=args.layers)
+    config = FalconH1Config.from_dict(raw)
+    storage = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    element = 2 if args.dtype == "bf16" else 4
+    tensors = random_tensors(config, 0, storage, "baseline")
+    batches = [args.batch] if args.skip_points else sorted({1, args.batch, 64})
+    largest = max(batches)
+    total_steps = args.steps + args.warmup
+    per_request = -(-(CONTEXT + total_steps + 1) // 64) * 64
+    engine = Engine(config=config, tensors=tensors, dtype="bfloat16" if args.dtype == "bf16" else "float32",
+                    kv_cache_block_tokens=args.page_tokens,
+                    kv_cache_capacity_tokens=per_request * largest + PREFILL_TOKENS + 64,
+                    max_active_sequences=largest + 1)
+    del tensors
+    sampler = Sampler(engine.vocab_size, engine.device)
+    generator = torch.Generator().manual_seed(0)
+    vocab = config.vocab_size
+
+    def synchronize():
+        torch.cuda.synchronize()
+
+    # ---------------------------------------------------------------- prefill: one 2,048-token prompt
+    prefill_times = []
+    for repeat in range(3):
+        prompt = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=generator).tolist()
+        engine.add_request("prefill")
+        synchronize()
+        started = time.perf_counter()
+        engine.step([Lane("prefill", prompt, [PREFILL_TOKENS - 1])])
+        synchronize()
+        prefill_times.append(time.perf_counter() - started)
+        engine.finish("prefill")
+    prefill_seconds = min(prefill_times[1:])
+
+    d, L = config.hidden_size, config.num_hidden_layers
+    E = config.mamba_d_ssm
+    conv_width = E + 2 * config.mamba_n_groups * config.mamba_d_state
+    q_width = config.num_attention_heads * config.head_dim
+    kv_width = config.num_key_value_heads * config.head_dim
+    layer_matrix = (d * (q_width + 2 * kv_width) + q_width * d + d * (E + conv_width + config.mamba_n_heads)
+                    + E * d + 3 * d * config.intermediate_size)
+    T = PREFILL_TOKENS
+    prefill_flops = (2.0 * T * layer_matrix * L + 2.0 * vocab * d
+                     + L * 2.0 * config.num_attention_heads * config.head_dim * T * T
+                     + L * 6.0 * config.mamba_n_heads * config.mamba_d_head * config.mamba_d_state * T)
+
+    # ---------------------------------------------------------------- decode at each batch size
+    weight_bytes = (layer_matrix * L + vocab * d) * element
+    state_bytes_per_request = L * (2 * config.mamba_n_heads * config.mamba_d_head * config.mamba_d_state * 4
+                                   + 2 * (config.mamba_d_conv - 1) * conv_width * element)
+    kv_bytes_per_token = config.kv_bytes_per_token(element)
+    results = {}
+    for batch in batches:
+        names = [f"b{batch}_{index}" for index in range(batch)]
+        for name in names:
+            engine.add_request(name)
+            prompt = torch.randint(0, vocab, (CONTEXT,), generator=generator).tolist()
+            engine.step([Lane(name, prompt, [])])
+        tokens = torch.randint(0, vocab, (batch,), generator=generator).tolist()
+        rows = [SamplerRow(GREEDY, (), ()) for _ in names]
+
+        def decode_step(tokens):
+            logits = engine.step([Lane(name, [token], [0]) for name, token in zip(names, tokens)])
+            return sampler.sample(logits, rows)
+
+        for _ in range(args.warmup):
+            tokens = decode_step(tokens)
+        synchronize()
+        started = time.perf_counter()
+        for _ in range(args.steps):
+            tokens = decode_step(tokens)
+        synchronize()
+        seconds = time.perf_counter() - started
+        for name in names:
+            engine.finish(name)
+        step_seconds = seconds / args.steps
+        context = CONTEXT + args.warmup + args.steps / 2.0
+        bytes_moved = weight_bytes + batch * (state_bytes_per_request + kv_bytes_per_token * context)
+        results[batch] = dict(tokens_per_second=batch / step_seconds, ms=step_seconds * 1e3,
+                              gbs=bytes_moved / step_seconds / 1e9)
+
+    headline = results[args.batch]
+    record = {
+        "metric": "decode tok/s at batch 8 (2,048-token context); prefill tok/s at 2,048 tokens",
+        "value": round(headline["tokens_per_second"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(headline["ms"], 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+        "config": {"model": "falcon-h1-0.5b-shaped, random weights", "layers": L,
+                   "layers_of_configuration": SHAPE["num_hidden_layers"], "hidden": d,
+                   "heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
+                   "head_dim": config.head_dim, "intermediate": config.intermediate_size,
+                   "mamba_heads": config.mamba_n_heads, "mamba_head_dim": config.mamba_d_head,
+                   "mamba_state": config.mamba_d_state, "mamba_conv": config.mamba_d_conv, "vocab": vocab,
+                   "tied_embeddings": True, "global_batch": args.batch, "seq_len": CONTEXT,
+                   "page_tokens": args.page_tokens, "parallelism": "single GPU"},
+        "prefill": {"value": round(PREFILL_TOKENS / prefill_seconds, 1), "tokens": PREFILL_TOKENS,
+                    "ms": round(prefill_seconds * 1e3, 3),
+                    "frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS[args.dtype], 5)},
+        "roofline": {"bound": "hbm", "achieved": round(headline["gbs"], 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(headline["gbs"] / PEAK_HBM_GBS, 5)},
+        "points": {f"decode_b{batch}": round(result["tokens_per_second"], 1) for batch, result in results.items()
+                   if batch != args.batch},
+    }
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
