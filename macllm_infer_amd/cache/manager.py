@@ -4,7 +4,7 @@ per group of layers with the same needs, and slots for per-request state of fixe
 What a mixer needs is declared by the mixer (``KVNeed`` / ``StateNeed``); the manager
 groups equal ``KVNeed``s (same heads, head size and window) into one ``PagedGroup`` whose
 pages hold every member layer, so one block table per request serves all of them
-(layout [page, layer, K|V, kv_head, token, dim]; crates/macllm-kv/src/cache.rs:558-566,
+(layout [page, layer, K|V, kv_head, token x dim], V transposed inside its block; crates/macllm-kv/src/cache.rs:558-566,
 one pool per geometry :165-169).  Layers that keep all keys and layers that keep a
 window are different groups: a window group gives a page back as soon as every query
 still to come is past it.
@@ -55,11 +55,15 @@ class PagedGroup:
 
     def allocate(self, dtype: torch.dtype, device) -> None:
         need = self.need
-        self.storage = torch.zeros((self.pool.total, len(self.members), 2, need.num_kv_heads, self.page_size,
-                                    need.head_dim), dtype=dtype, device=device)
+        self.storage = torch.zeros((self.pool.total, len(self.members), 2, need.num_kv_heads,
+                                    self.page_size * need.head_dim), dtype=dtype, device=device)
 
     def layer_views(self, layer: int):
-        return self.storage[:, layer, 0], self.storage[:, layer, 1]
+        """One layer's K pages [pages, Hkv, page_size, dh] and V pages [pages, Hkv, dh, page_size]
+        (V is kept transposed: its product contracts over tokens)."""
+        need = self.need
+        return (self.storage[:, layer, 0].unflatten(-1, (self.page_size, need.head_dim)),
+                self.storage[:, layer, 1].unflatten(-1, (need.head_dim, self.page_size)))
 
     def bytes_per_page(self, element_size: int) -> int:
         need = self.need

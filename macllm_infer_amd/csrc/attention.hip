@@ -1,11 +1,15 @@
 // Rotary position encoding fused with the write of K and V into cache pages, and
 // attention over the paged cache.
 //
-// Cache layout of one paged group: [page, layer, 2 (K,V), kv_head, token_in_page, head_dim].
-// Entry points get the base pointers of one layer's K and V inside page 0 and the
-// stride between pages, so  K(page, kvh, off) = k_base + page*page_stride + (kvh*page_size + off)*dh.
-// (The reference addresses its pages the same way: crates/macllm-kv/src/cache.rs:558-566,
-// crates/macllm-kernels/src/metal/paged_decode.metal:109-113.)
+// Cache layout of one paged group: [page, layer, 2 (K,V), kv_head, page_size*head_dim].
+// Inside a page, K of one kv head is [token, dim] and V is transposed, [dim, token]: the
+// value product contracts over tokens, and a matrix-core operand wants its contraction index
+// contiguous.  Entry points get the base pointers of one layer's K and V inside page 0 and
+// the stride between pages:
+//   K(page, kvh, off, i) = k_base + page*page_stride + (kvh*page_size + off)*dh + i
+//   V(page, kvh, off, i) = v_base + page*page_stride + (kvh*dh + i)*page_size + off
+// (The reference pages its cache the same way, K and V both token-major:
+// crates/macllm-kv/src/cache.rs:558-566, crates/macllm-kernels/src/metal/paged_decode.metal:109-113.)
 #include "common.h"
 
 // ---------------------------------------------------------------- rope + cache write
@@ -80,7 +84,7 @@ __global__ void rope_kv_store_kernel(T* __restrict__ qkv, long ld, int Hq, int H
     for (int item = threadIdx.x; item < Hkv * dh; item += blockDim.x) {
       const int kvh = item / dh;
       const int i = item - kvh * dh;
-      v_base[page * page_stride + ((long)kvh * page_size + offset) * dh + i] = v[item];
+      v_base[page * page_stride + ((long)kvh * dh + i) * page_size + offset] = v[item];
     }
   }
 }
@@ -127,7 +131,8 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
                        int window, T* __restrict__ out, long out_ld) {
   __shared__ float q_shared[ATT_MAX_DH];
   __shared__ float p_shared[WAVE];
-  __shared__ long row_shared[WAVE];
+  __shared__ long row_shared[WAVE];      // base of the key's (page, kv head) block
+  __shared__ int offset_shared[WAVE];    // the key's place inside its page
   const long token = blockIdx.x;
   const int head = blockIdx.y;
   const int kvh = head / (Hq / Hkv);
@@ -153,11 +158,12 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
     const int key = base + lane;
     float score = -INFINITY;
     long row_offset = 0;
+    int offset = 0;
     if (key <= last_key) {
       const int page = table[key / page_size];
-      const int offset = key % page_size;
-      row_offset = (long)page * page_stride + ((long)kvh * page_size + offset) * dh;
-      const T* k_row = k_base + row_offset;
+      offset = key % page_size;
+      row_offset = (long)page * page_stride + (long)kvh * page_size * dh;
+      const T* k_row = k_base + row_offset + (long)offset * dh;
       float dot = 0.f;
       for (int i = 0; i < dh; ++i) dot += q_shared[i] * to_float(k_row[i]);
       score = dot * scale;
@@ -171,6 +177,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
     __syncthreads();
     p_shared[lane] = p;
     row_shared[lane] = row_offset;
+    offset_shared[lane] = offset;
     __syncthreads();
     const int valid = min(WAVE, last_key - base + 1);
 #pragma unroll
@@ -178,7 +185,8 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
       const int dim = lane + i * WAVE;
       if (dim < dh) {
         float sum = acc[i] * correction;
-        for (int j = 0; j < valid; ++j) sum += p_shared[j] * to_float(v_base[row_shared[j] + dim]);
+        for (int j = 0; j < valid; ++j)
+          sum += p_shared[j] * to_float(v_base[row_shared[j] + (long)dim * page_size + offset_shared[j]]);
         acc[i] = sum;
       }
     }
@@ -211,6 +219,252 @@ extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, in
         page_size, block_tables, max_pages, lane_of_token, positions, scale, window, (bf16_t*)out, out_ld);
   else
     return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- decode attention, split over the context
+// For batches of single-token queries in bfloat16.  grid = (splits, kv heads, tokens); a block
+// takes one page-aligned range of `split_keys` keys of one request and one kv head and serves
+// all G query heads of that kv head from the same K and V loads:
+//   scores : LPR = DH/8 lanes share a key row (16 B each), partial dots are summed across them;
+//   softmax: over the block's range in float32 (scores staged in LDS), giving (max, sum);
+//   values : V pages are [dim, token]; lane d owns output dim d and reads 8 tokens per load.
+// Every block writes an unnormalized partial output with its (max, sum); the merge kernel
+// combines the splits (the same (maximum, normalizer, accumulator) merge the reference does
+// across simdgroups, crates/macllm-kernels/src/metal/paged_decode.metal:145-183).
+#define DEC_THREADS 256
+#define DEC_WAVES (DEC_THREADS / WAVE)
+#define DEC_MAX_SPLIT 512
+
+struct alignas(16) bf16x8 {
+  bf16_t v[8];
+};
+
+template <int DH, int G>
+__global__ void __launch_bounds__(DEC_THREADS)
+decode_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, const bf16_t* __restrict__ k_base,
+                        const bf16_t* __restrict__ v_base, long page_stride, int page_size,
+                        const int* __restrict__ block_tables, int max_pages,
+                        const int* __restrict__ lane_of_token, const int* __restrict__ positions, float scale,
+                        int window, int split_keys, int splits, float* __restrict__ partial_o,
+                        float* __restrict__ partial_ml) {
+  constexpr int LPR = DH / 8;
+  constexpr int KPW = WAVE / LPR;
+  constexpr int KPB = KPW * DEC_WAVES;
+  constexpr int DPL = DH / WAVE;
+  __shared__ float s_lds[G][DEC_MAX_SPLIT];
+  __shared__ float red[DEC_WAVES][G];
+  __shared__ float acc_lds[DEC_WAVES][G][DH];
+
+  const int split = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const long token = blockIdx.z;
+  const int pos = positions[token];
+  int first_key = 0;
+  if (window > 0 && pos - window + 1 > 0) first_key = pos - window + 1;
+  const int range_lo = (first_key / page_size) * page_size + split * split_keys;
+  if (range_lo > pos) return;
+  const int range_hi = min(range_lo + split_keys, pos + 1);
+  const int count = range_hi - range_lo;
+  const int* table = block_tables + (long)lane_of_token[token] * max_pages;
+  const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  const int r = lane / LPR;
+  const int c = lane % LPR;
+
+  float qf[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const bf16x8 packed = *reinterpret_cast<const bf16x8*>(q + token * q_ld + (long)(kvh * G + g) * DH + c * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) qf[g][j] = (float)packed.v[j] * scale;
+  }
+
+  // scores
+  for (int base = 0; base < count; base += KPB) {
+    const int local = base + wave * KPW + r;
+    const int key = range_lo + local;
+    const bool valid = local < count;
+    float s[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) s[g] = 0.f;
+    if (valid) {
+      const int page = table[key / page_size];
+      const int offset = key % page_size;
+      const bf16x8 packed = *reinterpret_cast<const bf16x8*>(
+          k_base + (long)page * page_stride + ((long)kvh * page_size + offset) * DH + c * 8);
+      float kf[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) kf[j] = (float)packed.v[j];
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[g] = fmaf(qf[g][j], kf[j], s[g]);
+    }
+#pragma unroll
+    for (int offset = LPR / 2; offset > 0; offset >>= 1)
+#pragma unroll
+      for (int g = 0; g < G; ++g) s[g] += __shfl_xor(s[g], offset, WAVE);
+    if (valid && c == 0) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) s_lds[g][local] = key >= first_key ? s[g] : -INFINITY;
+    }
+  }
+  __syncthreads();
+
+  // softmax over the range: maximum, then exp and sum
+  float m[G], l[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float v = -INFINITY;
+    for (int i = tid; i < count; i += DEC_THREADS) v = fmaxf(v, s_lds[g][i]);
+    v = wave_max(v);
+    if (lane == 0) red[wave][g] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float v = red[0][g];
+#pragma unroll
+    for (int w = 1; w < DEC_WAVES; ++w) v = fmaxf(v, red[w][g]);
+    m[g] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float sum = 0.f;
+    for (int i = tid; i < count; i += DEC_THREADS) {
+      const float p = __expf(s_lds[g][i] - m[g]);
+      s_lds[g][i] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) red[wave][g] = sum;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) v += red[w][g];
+    l[g] = v;
+  }
+
+  // values: each wave takes every fourth page of the range
+  float acc[G][DPL];
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) acc[g][i] = 0.f;
+  const int range_pages = (count + page_size - 1) / page_size;
+  for (int pg = wave; pg < range_pages; pg += DEC_WAVES) {
+    const int local0 = pg * page_size;
+    const int page = table[(range_lo + local0) / page_size];
+    const int keys_here = min(page_size, count - local0);
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      const int dim = lane + i * WAVE;
+      const bf16_t* v_row = v_base + (long)page * page_stride + ((long)kvh * DH + dim) * page_size;
+      for (int j0 = 0; j0 < keys_here; j0 += 8) {
+        const bf16x8 packed = *reinterpret_cast<const bf16x8*>(v_row + j0);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (j0 + j < keys_here) {
+            const float value = (float)packed.v[j];
+#pragma unroll
+            for (int g = 0; g < G; ++g) acc[g][i] = fmaf(s_lds[g][local0 + j0 + j], value, acc[g][i]);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) acc_lds[wave][g][lane + i * WAVE] = acc[g][i];
+  __syncthreads();
+  for (int index = tid; index < G * DH; index += DEC_THREADS) {
+    const int g = index / DH;
+    const int dim = index - g * DH;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) sum += acc_lds[w][g][dim];
+    partial_o[((token * Hq + kvh * G + g) * splits + split) * DH + dim] = sum;
+  }
+  if (tid < G) {
+    float* ml = partial_ml + ((token * Hq + kvh * G + tid) * splits + split) * 2;
+    ml[0] = m[tid];
+    ml[1] = l[tid];
+  }
+}
+
+// out[token, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s over the splits that hold keys.
+__global__ void decode_merge_kernel(const float* __restrict__ partial_o, const float* __restrict__ partial_ml,
+                                    const int* __restrict__ positions, int window, int page_size,
+                                    int split_keys, int splits, int Hq, int dh, bf16_t* __restrict__ out,
+                                    long out_ld) {
+  const long token = blockIdx.x;
+  const int head = blockIdx.y;
+  const int pos = positions[token];
+  int first_key = 0;
+  if (window > 0 && pos - window + 1 > 0) first_key = pos - window + 1;
+  const int first_page_key = (first_key / page_size) * page_size;
+  const int used = min(splits, (pos - first_page_key) / split_keys + 1);
+  const float* ml = partial_ml + (token * Hq + head) * splits * 2;
+  const float* o = partial_o + (token * Hq + head) * (long)splits * dh;
+  float maximum = -INFINITY;
+  for (int s = 0; s < used; ++s) maximum = fmaxf(maximum, ml[2 * s]);
+  float denominator = 0.f;
+  for (int s = 0; s < used; ++s) denominator += __expf(ml[2 * s] - maximum) * ml[2 * s + 1];
+  for (int dim = threadIdx.x; dim < dh; dim += blockDim.x) {
+    float sum = 0.f;
+    for (int s = 0; s < used; ++s) sum += __expf(ml[2 * s] - maximum) * o[(long)s * dh + dim];
+    out[token * out_ld + (long)head * dh + dim] = (bf16_t)(sum / denominator);
+  }
+}
+
+template <int DH, int G>
+static int launch_decode(const bf16_t* q, long q_ld, int T, int Hq, int Hkv, const bf16_t* k_base,
+                         const bf16_t* v_base, long page_stride, int page_size, const int* block_tables,
+                         int max_pages, const int* lane_of_token, const int* positions, float scale, int window,
+                         int split_keys, int splits, float* partial_o, float* partial_ml, hipStream_t stream) {
+  const dim3 grid(splits, Hkv, T);
+  decode_attention_kernel<DH, G><<<grid, DEC_THREADS, 0, stream>>>(
+      q, q_ld, Hq, k_base, v_base, page_stride, page_size, block_tables, max_pages, lane_of_token, positions,
+      scale, window, split_keys, splits, partial_o, partial_ml);
+  return 0;
+}
+
+// Returns ERR_UNSUPPORTED_SIZE for shapes this kernel does not cover (the caller then uses
+// mi_paged_attention): head_dim 64 or 128, 1..8 query heads per kv head, page_size a multiple of 8,
+// split_keys a multiple of page_size and at most DEC_MAX_SPLIT.
+extern "C" int mi_decode_attention(const void* q, long q_ld, int T, int Hq, int Hkv, int dh, const void* k_base,
+                                   const void* v_base, long page_stride, int page_size, const int* block_tables,
+                                   int max_pages, const int* lane_of_token, const int* positions, float scale,
+                                   int window, int split_keys, int splits, float* partial_o, float* partial_ml,
+                                   void* out, long out_ld, hipStream_t stream) {
+  if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || page_size <= 0 || splits <= 0 || max_pages <= 0)
+    return ERR_BAD_ARGUMENT;
+  const int G = Hq / Hkv;
+  if ((dh != 64 && dh != 128) || G > 8 || page_size % 8 != 0 || split_keys % page_size != 0 ||
+      split_keys <= 0 || split_keys > DEC_MAX_SPLIT || T > 65535 || Hkv > 65535)
+    return ERR_UNSUPPORTED_SIZE;
+#define DECODE_CASE(DH_, G_)                                                                                     \
+  if (dh == DH_ && G == G_)                                                                                      \
+    launch_decode<DH_, G_>((const bf16_t*)q, q_ld, T, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base,     \
+                           page_stride, page_size, block_tables, max_pages, lane_of_token, positions, scale,     \
+                           window, split_keys, splits, partial_o, partial_ml, stream);
+  DECODE_CASE(64, 1) DECODE_CASE(64, 2) DECODE_CASE(64, 3) DECODE_CASE(64, 4) DECODE_CASE(64, 5)
+  DECODE_CASE(64, 6) DECODE_CASE(64, 7) DECODE_CASE(64, 8)
+  DECODE_CASE(128, 1) DECODE_CASE(128, 2) DECODE_CASE(128, 3) DECODE_CASE(128, 4) DECODE_CASE(128, 5)
+  DECODE_CASE(128, 6) DECODE_CASE(128, 7) DECODE_CASE(128, 8)
+#undef DECODE_CASE
+  RETURN_IF_LAUNCH_FAILED();
+  const dim3 merge_grid(T, Hq);
+  decode_merge_kernel<<<merge_grid, dh, 0, stream>>>(partial_o, partial_ml, positions, window, page_size,
+                                                     split_keys, splits, Hq, dh, (bf16_t*)out, out_ld);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

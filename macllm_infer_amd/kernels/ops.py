@@ -40,6 +40,9 @@ _SIGNATURES = {
                              _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr],
         "mi_paged_attention": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
                                _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_long, _c_ptr],
+        "mi_decode_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int,
+                                _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
+                                _c_ptr, _c_long, _c_ptr],
     },
     "mamba2": {
         "mi_conv1d_silu": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
@@ -217,8 +220,8 @@ def rope_kv_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
                   v_cache: Optional[torch.Tensor]) -> None:
     """Rotate q (in place) and k of every token; store rotated k and raw v into the cache.
 
-    ``qkv`` [T, >= (Hq+2Hkv)*dh] holds q heads, k heads, v heads.  ``k_cache``/``v_cache``
-    are one layer's views [pages, Hkv, page_size, dh] of the paged pool;
+    ``qkv`` [T, >= (Hq+2Hkv)*dh] holds q heads, k heads, v heads.  ``k_cache`` [pages, Hkv,
+    page_size, dh] and ``v_cache`` [pages, Hkv, dh, page_size] are one layer's views of the pool;
     ``slot_mapping[t] = page*page_size + offset``.  Without ``slot_mapping`` nothing is stored."""
     ld = _row_major(qkv, "qkv")
     T = qkv.shape[0]
@@ -241,15 +244,19 @@ def rope_kv_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
 
 
 def _cache_view(k_cache, v_cache, num_kv_heads, head_dim, dtype):
+    """K pages are [pages, Hkv, page_size, dh]; V pages are transposed, [pages, Hkv, dh, page_size]."""
+    _need(k_cache is not None and v_cache is not None and k_cache.dim() == 4 and v_cache.dim() == 4,
+          "k_cache must be [pages, Hkv, page_size, dh] and v_cache [pages, Hkv, dh, page_size]")
+    page_size = k_cache.shape[2]
+    _need(k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == head_dim
+          and v_cache.shape == (k_cache.shape[0], num_kv_heads, head_dim, page_size),
+          "k_cache must be [pages, Hkv, page_size, dh] and v_cache [pages, Hkv, dh, page_size]")
     for name, cache in (("k_cache", k_cache), ("v_cache", v_cache)):
-        _need(cache is not None and cache.dim() == 4 and cache.shape[1] == num_kv_heads
-              and cache.shape[3] == head_dim and cache.dtype == dtype and cache.is_cuda,
-              f"{name} must be [pages, Hkv, page_size, dh] of the activation dtype")
-        _need(cache.stride(3) == 1 and cache.stride(2) == head_dim
-              and cache.stride(1) == cache.shape[2] * head_dim, f"{name}: a page's [Hkv, page_size, dh] must be dense")
-    _need(k_cache.stride(0) == v_cache.stride(0) and k_cache.shape == v_cache.shape,
-          "k_cache and v_cache must share a geometry")
-    return k_cache.stride(0), k_cache.shape[2]
+        _need(cache.dtype == dtype and cache.is_cuda, f"{name} must be a GPU tensor of the activation dtype")
+        _need(cache.stride(3) == 1 and cache.stride(2) == cache.shape[3]
+              and cache.stride(1) == page_size * head_dim, f"{name}: a page's block per kv head must be dense")
+    _need(k_cache.stride(0) == v_cache.stride(0), "k_cache and v_cache must share a page stride")
+    return k_cache.stride(0), page_size
 
 
 def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -276,6 +283,47 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
         _p(q), _dt(q), q_ld, T, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride,
         page_size, _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale),
         int(window or 0), _p(out), out_ld, _stream()), "paged_attention", f"(head_dim={head_dim})")
+
+
+def decode_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> bool:
+    """Whether the split-context kernel for single-token queries covers this geometry."""
+    return (dtype == torch.bfloat16 and head_dim in (64, 128) and num_heads // num_kv_heads <= 8
+            and page_size % 8 == 0 and page_size <= 512)
+
+
+def decode_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_cache: torch.Tensor,
+                     v_cache: torch.Tensor, block_tables: torch.Tensor, lane_of_token: torch.Tensor,
+                     positions: torch.Tensor, scale: float, window: Optional[int], max_seq_len: int,
+                     out: torch.Tensor) -> None:
+    """``paged_attention`` for batches of single decoded tokens in bfloat16: the context of each
+    request is split over many workgroups and the G query heads of a kv head share its K/V
+    loads.  ``max_seq_len``: an upper bound of the longest context in the batch."""
+    q_ld = _row_major(q, "q")
+    out_ld = _row_major(out, "out")
+    T = q.shape[0]
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "decode_attention: bfloat16 only")
+    _need(q.shape[1] >= num_heads * head_dim and out.shape == (T, num_heads * head_dim) and q_ld % 8 == 0
+          and q.data_ptr() % 16 == 0, "decode_attention: q/out shapes or alignment do not fit")
+    page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, q.dtype)
+    _need(decode_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim, page_size),
+          "decode_attention: geometry not covered; use paged_attention")
+    _i32(block_tables, "block_tables")
+    _i32(lane_of_token, "lane_of_token")
+    _i32(positions, "positions")
+    _need(block_tables.dim() == 2 and lane_of_token.numel() == T and positions.numel() == T,
+          "decode_attention: metadata shapes do not match")
+    span = max_seq_len if not window else min(max_seq_len, window + page_size)
+    split_keys = 64
+    while split_keys < 512 and span * T * num_kv_heads > 1024 * split_keys:
+        split_keys *= 2
+    split_keys = max(split_keys, page_size)
+    splits = max(1, -(-span // split_keys))
+    partial_o = torch.empty((T, num_heads, splits, head_dim), dtype=torch.float32, device=q.device)
+    partial_ml = torch.empty((T, num_heads, splits, 2), dtype=torch.float32, device=q.device)
+    _check(_fn("attention", "mi_decode_attention")(
+        _p(q), q_ld, T, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride, page_size,
+        _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale), int(window or 0),
+        split_keys, splits, _p(partial_o), _p(partial_ml), _p(out), out_ld, _stream()), "decode_attention")
 
 
 # --------------------------------------------------------------------------- mamba2

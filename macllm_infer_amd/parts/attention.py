@@ -66,7 +66,12 @@ class Attention(Mixer):
         qkv = self.qkv(x)
         self.position.rotate_and_store(qkv, spec.num_heads, spec.num_kv_heads, spec.head_dim, step, cache)
         attended = torch.empty((x.shape[0], spec.num_heads * spec.head_dim), dtype=qkv.dtype, device=x.device)
-        ops.paged_attention(qkv, spec.num_heads, spec.num_kv_heads, spec.head_dim, cache.k_cache, cache.v_cache,
-                            step.block_tables[cache.group], step.lane_of_token, step.positions, spec.scale,
-                            spec.window, attended)
+        geometry = (spec.num_heads, spec.num_kv_heads, spec.head_dim)
+        if step.max_query_len == 1 and ops.decode_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2]):
+            ops.decode_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                 step.lane_of_token, step.positions, spec.scale, spec.window, step.max_seq_len,
+                                 attended)
+        else:
+            ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                step.lane_of_token, step.positions, spec.scale, spec.window, attended)
         return self.out(attended)

@@ -76,7 +76,7 @@ def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, r
         pages = (slot_mapping // page_size).long()
         offsets = (slot_mapping % page_size).long()
         k_cache[pages, :, offsets, :] = k.to(k_cache.dtype)
-        v_cache[pages, :, offsets, :] = v.to(v_cache.dtype)
+        v_cache[pages, :, :, offsets] = v.to(v_cache.dtype)        # V pages are [Hkv, dh, token]
 
 
 def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token,
@@ -92,12 +92,22 @@ def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, bloc
         pages = block_tables[lane][(keys // page_size).long()].long()
         offsets = (keys % page_size).long()
         k = _f(k_cache[pages, :, offsets, :])        # [keys, Hkv, dh]
-        v = _f(v_cache[pages, :, offsets, :])
+        v = _f(v_cache[pages, :, :, offsets])
         for head in range(num_heads):
             query = _f(q[token, head * head_dim:(head + 1) * head_dim])
             scores = (k[:, head // group, :] @ query) * scale
             weights = torch.softmax(scores, dim=0)
             out[token, head * head_dim:(head + 1) * head_dim] = (weights @ v[:, head // group, :]).to(out.dtype)
+
+
+def decode_attention_supported(dtype, num_heads, num_kv_heads, head_dim, page_size):
+    return False
+
+
+def decode_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token, positions,
+                     scale, window, max_seq_len, out):
+    paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token, positions,
+                    scale, window, out)
 
 
 def conv1d_silu(u, col_offset, width, weight, bias, conv_state, lane_of_token, cu_seqlens, slot_ids, out):
@@ -160,7 +170,7 @@ def argmax(logits, out):
     out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
 
 
-NAMES = ["embed", "add_rmsnorm", "swiglu", "scale_to_f32", "linear", "rope_kv_store", "paged_attention",
+NAMES = ["decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "linear", "rope_kv_store", "paged_attention",
          "conv1d_silu", "conv_state_update", "ssm_scan", "gate_norm", "argmax"]
 
 

@@ -17,6 +17,11 @@ def make(capacity=64, page=8, requests=3, window=None):
     return CacheManager(needs, {}, page, capacity, requests, torch.float32, "cpu")
 
 
+def first_views(cache):
+    entry = cache.entry((0, "attn"))
+    return tuple(entry.k_cache.shape), tuple(entry.v_cache.shape)
+
+
 def test_page_pool_invariants():
     pool = PagePool(5)
     first = pool.alloc(3)
@@ -37,7 +42,8 @@ def test_page_pool_invariants():
 def test_groups_share_a_table_per_geometry_and_windows_get_their_own():
     cache = make(window=10)
     assert len(cache.groups) == 2
-    assert cache.groups[0].storage.shape == (8, 2, 2, 2, 8, 4)    # [page, layer, K|V, kv head, token, dim]
+    assert cache.groups[0].storage.shape == (8, 2, 2, 2, 32)      # [page, layer, K|V, kv head, token x dim]
+    assert first_views(cache) == ((8, 2, 8, 4), (8, 2, 4, 8))     # V pages are transposed
     assert cache.groups[1].need.window == 10 and len(cache.groups[1].members) == 1
     first, second = cache.entry((0, "attn")), cache.entry((1, "attn"))
     assert first.group == second.group == 0 and first.k_cache.data_ptr() != second.k_cache.data_ptr()

@@ -126,7 +126,7 @@ def test_mixed_product_keeps_a_32bit_weight(ops):
 
 # ------------------------------------------------------------------ attention
 def paged_setup(lengths, page_size, Hkv, dh, dtype, layers=2, seed=0):
-    """A pool of shuffled pages [page, layer, K|V, Hkv, page_size, dh] and a block table per lane."""
+    """A pool of shuffled pages [page, layer, K|V, Hkv, page_size*dh] and a block table per lane."""
     generator = torch.Generator().manual_seed(seed)
     pages_per_lane = [-(-length // page_size) for length in lengths]
     total = sum(pages_per_lane) + 3
@@ -136,15 +136,22 @@ def paged_setup(lengths, page_size, Hkv, dh, dtype, layers=2, seed=0):
     for lane, count in enumerate(pages_per_lane):
         table[lane, :count] = torch.tensor(order[cursor:cursor + count], dtype=torch.int32)
         cursor += count
-    pool = torch.full((total, layers, 2, Hkv, page_size, dh), float("nan"), dtype=dtype)
+    pool = torch.full((total, layers, 2, Hkv, page_size * dh), float("nan"), dtype=dtype)
     return pool, table
 
 
+def views(pool, page_size, layer=1):
+    """One layer's K pages [pages, Hkv, page_size, dh] and transposed V pages [pages, Hkv, dh, page_size]."""
+    dh = pool.shape[-1] // page_size
+    return (pool[:, layer, 0].unflatten(-1, (page_size, dh)), pool[:, layer, 1].unflatten(-1, (dh, page_size)))
+
+
 def fill_cache(pool, table, lane, keys, values, page_size, layer=1):
+    k_pages, v_pages = views(pool, page_size, layer)
     for position in range(keys.shape[0]):
         page = int(table[lane, position // page_size])
-        pool[page, layer, 0, :, position % page_size, :] = keys[position]
-        pool[page, layer, 1, :, position % page_size, :] = values[position]
+        k_pages[page, :, position % page_size, :] = keys[position]
+        v_pages[page, :, :, position % page_size] = values[position]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -171,10 +178,10 @@ def test_rope_store_and_attention_over_pages(ops, dtype, Hq, Hkv, dh, page_size,
     inv_freq = torch.tensor([1.0 / (1e4 ** (i / rotary)) for i in range(0, rotary, 2)], dtype=torch.float64).float()
     want_qkv, want_pool = qkv.clone(), pool.clone()
     ref_ops.rope_kv_store(want_qkv, Hq, Hkv, dh, positions, inv_freq, rotary, slot_mapping,
-                          want_pool[:, 1, 0], want_pool[:, 1, 1])
+                          *views(want_pool, page_size))
     got_qkv, got_pool = qkv.to(DEV), pool.to(DEV)
     ops.rope_kv_store(got_qkv, Hq, Hkv, dh, positions.to(DEV), inv_freq.to(DEV), rotary, slot_mapping.to(DEV),
-                      got_pool[:, 1, 0], got_pool[:, 1, 1])
+                      *views(got_pool, page_size))
     close(got_qkv[:, :Hq * dh], want_qkv[:, :Hq * dh], dtype, 4.0)
     assert torch.equal(got_qkv[:, Hq * dh:].cpu(), qkv[:, Hq * dh:])         # k, v columns untouched
     written = ~torch.isnan(want_pool.float())
@@ -183,10 +190,10 @@ def test_rope_store_and_attention_over_pages(ops, dtype, Hq, Hkv, dh, page_size,
     assert torch.isnan(got_pool[:, 0].float()).all()                           # the other layer is untouched
     for window in (None, 9):
         want = torch.empty(T, Hq * dh, dtype=dtype)
-        ref_ops.paged_attention(want_qkv, Hq, Hkv, dh, want_pool[:, 1, 0], want_pool[:, 1, 1], table,
+        ref_ops.paged_attention(want_qkv, Hq, Hkv, dh, *views(want_pool, page_size), table,
                                 lane_of_token, positions, 0.37, window, want)
         got = torch.empty(T, Hq * dh, dtype=dtype, device=DEV)
-        ops.paged_attention(got_qkv, Hq, Hkv, dh, got_pool[:, 1, 0], got_pool[:, 1, 1], table.to(DEV),
+        ops.paged_attention(got_qkv, Hq, Hkv, dh, *views(got_pool, page_size), table.to(DEV),
                             lane_of_token.to(DEV), positions.to(DEV), 0.37, window, got)
         close(got, want, dtype, 3.0)
 
@@ -210,7 +217,7 @@ def test_one_far_key_among_hundreds_is_found(ops, dtype, page_size):
         q = (direction * 30.0).repeat(Hq)[None].to(dtype)
         out = torch.empty(1, Hq * dh, dtype=dtype, device=DEV)
         dev_pool = pool.to(DEV)
-        ops.paged_attention(q.to(DEV), Hq, Hkv, dh, dev_pool[:, 1, 0], dev_pool[:, 1, 1], table.to(DEV),
+        ops.paged_attention(q.to(DEV), Hq, Hkv, dh, *views(dev_pool, page_size), table.to(DEV),
                             i32([0]).to(DEV), i32([length - 1]).to(DEV), 1.0 / math.sqrt(dh), None, out)
         expected = values[chosen].float()[[0, 0, 1, 1]].reshape(-1)
         assert (out.float().cpu()[0] - expected).abs().max() < 1e-2, f"key {chosen} was missed"
@@ -232,21 +239,21 @@ def test_window_edge(ops, dtype):
         fill_cache(pool, table, 0, keys, values, page_size)
         dev_pool = pool.to(DEV)
         out = torch.empty(1, Hq * dh, dtype=dtype, device=DEV)
-        ops.paged_attention(q, Hq, Hkv, dh, dev_pool[:, 1, 0], dev_pool[:, 1, 1], table.to(DEV), i32([0]).to(DEV),
+        ops.paged_attention(q, Hq, Hkv, dh, *views(dev_pool, page_size), table.to(DEV), i32([0]).to(DEV),
                             i32([length - 1]).to(DEV), 1.0 / math.sqrt(dh), window, out)
         hit = (out.float().cpu()[0, :dh] - values[chosen, 0].float()).abs().max() < 1e-2
         assert hit == visible, f"key {chosen} should be {'visible' if visible else 'masked'}"
         want = torch.empty(1, Hq * dh, dtype=dtype)
-        ref_ops.paged_attention(q.cpu(), Hq, Hkv, dh, pool[:, 1, 0], pool[:, 1, 1], table, i32([0]),
+        ref_ops.paged_attention(q.cpu(), Hq, Hkv, dh, *views(pool, page_size), table, i32([0]),
                                 i32([length - 1]), 1.0 / math.sqrt(dh), window, want)
         close(out, want, dtype, 3.0)
 
 
 def test_attention_refuses_a_head_size_beyond_its_limit(ops):
-    pool = torch.zeros(2, 1, 2, 1, 16, 320, device=DEV)
+    pool = torch.zeros(2, 1, 2, 1, 16 * 320, device=DEV)
     q = torch.zeros(1, 320, device=DEV)
     with pytest.raises(ops.KernelError, match="size not supported"):
-        ops.paged_attention(q, 1, 1, 320, pool[:, 0, 0], pool[:, 0, 1], i32([[0]]).to(DEV), i32([0]).to(DEV),
+        ops.paged_attention(q, 1, 1, 320, *views(pool, 16, 0), i32([[0]]).to(DEV), i32([0]).to(DEV),
                             i32([0]).to(DEV), 1.0, None, torch.empty(1, 320, device=DEV))
 
 
@@ -378,3 +385,51 @@ def test_penalties_match_the_plain_rule(ops):
                         torch.tensor(rep).to(DEV), torch.tensor(pres).to(DEV), torch.tensor(freq).to(DEV), *counts)
     close(got, want, torch.float32)
     assert not torch.equal(want, logits) and int(counts[0].sum()) == 0 and int(counts[1].sum()) == 0
+
+
+# ------------------------------------------------------------------ decode attention (split over the context)
+@pytest.mark.parametrize("Hq, Hkv, dh, page_size, window", [(8, 2, 64, 16, None), (12, 2, 128, 16, None),
+                                                              (5, 5, 64, 8, None), (8, 1, 128, 64, None),
+                                                              (8, 2, 64, 16, 300), (4, 2, 64, 32, 40)])
+def test_decode_attention_over_ragged_contexts(ops, Hq, Hkv, dh, page_size, window):
+    """Single decoded tokens of requests with contexts of 1 to 2 500 keys, cut into splits of
+    different sizes; NaN in every cell that is not a request's; against the plain reference."""
+    dtype = torch.bfloat16
+    lengths = [1, 2, 15, 16, 17, 63, 64, 65, 129, 777, 2500, 1024]
+    pool, table = paged_setup(lengths, page_size, Hkv, dh, dtype, seed=9)
+    for lane, length in enumerate(lengths):
+        fill_cache(pool, table, lane, rand(length, Hkv, dh, seed=100 + lane, dtype=dtype),
+                   rand(length, Hkv, dh, seed=200 + lane, dtype=dtype), page_size)
+    T = len(lengths)
+    q = rand(T, Hq * dh, seed=90, dtype=dtype)
+    positions = i32([length - 1 for length in lengths])
+    lane_of_token = torch.arange(T, dtype=torch.int32)
+    want = torch.empty(T, Hq * dh, dtype=dtype)
+    ref_ops.paged_attention(q, Hq, Hkv, dh, *views(pool, page_size), table, lane_of_token, positions, 0.11, window, want)
+    dev_pool = pool.to(DEV)
+    assert ops.decode_attention_supported(dtype, Hq, Hkv, dh, page_size)
+    for subset in (list(range(T)), [10], [0, 10, 3]):            # different batch sizes pick different splits
+        got = torch.empty(len(subset), Hq * dh, dtype=dtype, device=DEV)
+        ops.decode_attention(q[subset].to(DEV), Hq, Hkv, dh, *views(dev_pool, page_size), table.to(DEV),
+                             i32(subset).to(DEV), positions[subset].to(DEV), 0.11, window,
+                             max(lengths[index] for index in subset), got)
+        close(got, want[subset], dtype, 2.0)
+
+
+def test_decode_attention_finds_one_far_key(ops):
+    Hq, Hkv, dh, length, page_size = 8, 2, 64, 2048, 16
+    dtype = torch.bfloat16
+    pool, table = paged_setup([length], page_size, Hkv, dh, dtype, seed=5)
+    values = rand(length, Hkv, dh, seed=54, dtype=dtype)
+    direction = torch.zeros(dh)
+    direction[9] = 1.0
+    q = (direction * 30.0).repeat(Hq)[None].to(dtype).to(DEV)
+    for chosen in (0, 15, 16, 255, 256, 257, 1023, 1024, 2046, 2047):
+        keys = rand(length, Hkv, dh, seed=55, scale=0.1, dtype=dtype)
+        keys[chosen] = (direction * 30.0).to(dtype)
+        fill_cache(pool, table, 0, keys, values, page_size)
+        out = torch.empty(1, Hq * dh, dtype=dtype, device=DEV)
+        ops.decode_attention(q, Hq, Hkv, dh, *views(pool.to(DEV), page_size), table.to(DEV), i32([0]).to(DEV),
+                             i32([length - 1]).to(DEV), 1.0 / math.sqrt(dh), None, length, out)
+        expected = values[chosen].float()[[0] * 4 + [1] * 4].reshape(-1)
+        assert (out.float().cpu()[0] - expected).abs().max() < 1e-2, f"key {chosen} was missed"
