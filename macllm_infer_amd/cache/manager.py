@@ -55,8 +55,13 @@ class PagedGroup:
 
     def allocate(self, dtype: torch.dtype, device) -> None:
         need = self.need
-        self.storage = torch.zeros((self.pool.total, len(self.members), 2, need.num_kv_heads,
+        # one page more than the pool hands out: the scratch page padding lanes of a captured step write to
+        self.storage = torch.zeros((self.pool.total + 1, len(self.members), 2, need.num_kv_heads,
                                     self.page_size * need.head_dim), dtype=dtype, device=device)
+
+    @property
+    def scratch_page(self) -> int:
+        return self.pool.total
 
     def layer_views(self, layer: int):
         """One layer's K pages [pages, Hkv, page_size, dh] and V pages [pages, Hkv, dh, page_size]
@@ -155,7 +160,9 @@ class CacheManager:
                     layer_of[key] = (group, self.groups[group].add_member(key))
                 elif isinstance(need, StateNeed):
                     state_dtype = dtype if need.dtype == "activation" else torch.float32
-                    tensor = torch.zeros((max_requests,) + tuple(need.shape), dtype=state_dtype, device=self.device)
+                    # one slot more than the pool hands out: the scratch slot of padding lanes
+                    tensor = torch.zeros((max_requests + 1,) + tuple(need.shape), dtype=state_dtype,
+                                         device=self.device)
                     entry.states[need.name] = tensor
                     self._state_tensors.append(tensor)
                 else:
@@ -177,6 +184,10 @@ class CacheManager:
                 entry.owns_kv = key not in shared_kv
             elif key in shared_kv:
                 raise ValueError(f"{key} reads the cache of {source}, which keeps none")
+
+    @property
+    def scratch_slot(self) -> int:
+        return self.slots.total
 
     # ------------------------------------------------------------------ requests
     def add_request(self, request: Hashable) -> RequestCache:

@@ -5,11 +5,15 @@ starting at that request's current length: a portion of a prompt or one decoded
 token.  Lanes are packed without padding in submission order
 (reference: src/decoder.rs:4248-4260, lane struct paged_decode.metal:51-58).
 All index arrays are built on the host and uploaded in one copy.
+
+``StaticStep`` keeps the arrays of a batch of single-token lanes at fixed addresses and
+fixed shapes, so that a captured HIP graph can be replayed on them; lanes beyond the
+batch's real ones are padding that reads and writes the cache's scratch page and slot.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Hashable, List, Sequence
+from typing import Hashable, List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -39,16 +43,18 @@ class StepContext:
     lane_lengths: List[int] = field(default_factory=list)            # host copies
     lane_starts: List[int] = field(default_factory=list)
     max_query_len: int = 0
-    max_seq_len: int = 0
+    max_seq_len: int = 0             # an upper bound of the longest context in the batch
 
 
-def build_step_context(lanes: Sequence[Lane], cache, device) -> StepContext:
-    """``cache``: the CacheManager, after the step's pages were reserved."""
-    lengths = [len(lane.tokens) for lane in lanes]
-    starts = [cache.requests[lane.request].length for lane in lanes]
+def _pack(lanes: Sequence[Lane], cache, pad_lanes: int = 0, max_pages: Optional[int] = None):
+    """Numpy sections of the step (in the order of ``_assemble``) and the block-table shapes.
+    ``pad_lanes`` single-token lanes on the scratch page and slot are appended."""
+    lengths = [len(lane.tokens) for lane in lanes] + [1] * pad_lanes
+    starts = [cache.requests[lane.request].length for lane in lanes] + [0] * pad_lanes
+    Ln = len(lengths)
     T = sum(lengths)
-    Ln = len(lanes)
-    token_ids = np.concatenate([np.asarray(lane.tokens, dtype=np.int32) for lane in lanes])
+    token_ids = np.concatenate([np.asarray(lane.tokens, dtype=np.int32) for lane in lanes]
+                               + [np.zeros(pad_lanes, dtype=np.int32)])
     positions = np.concatenate([np.arange(start, start + length, dtype=np.int32)
                                 for start, length in zip(starts, lengths)])
     lane_of_token = np.repeat(np.arange(Ln, dtype=np.int32), lengths)
@@ -56,16 +62,17 @@ def build_step_context(lanes: Sequence[Lane], cache, device) -> StepContext:
     cu[1:] = np.cumsum(lengths)
     start_pos = np.asarray(starts, dtype=np.int32)
     seq_lens = start_pos + np.asarray(lengths, dtype=np.int32)
-    slot_ids = np.asarray([cache.requests[lane.request].slot for lane in lanes], dtype=np.int32)
+    slot_ids = np.asarray([cache.requests[lane.request].slot for lane in lanes]
+                          + [cache.scratch_slot] * pad_lanes, dtype=np.int32)
     want_rows = np.asarray([cu[index] + place for index, lane in enumerate(lanes) for place in lane.want],
                            dtype=np.int32)
     sections = [token_ids, positions, lane_of_token, cu, start_pos, seq_lens, slot_ids, want_rows]
     group_shapes = []
-    for index, group in enumerate(cache.groups):
+    for group in cache.groups:
         page_size = group.page_size
-        tables = [group.tables[lane.request].pages for lane in lanes]
-        max_pages = max(1, max(len(pages) for pages in tables))
-        table = np.zeros((Ln, max_pages), dtype=np.int32)
+        tables = [group.tables[lane.request].pages for lane in lanes] + [[group.scratch_page]] * pad_lanes
+        width = max_pages if max_pages is not None else max(1, max(len(pages) for pages in tables))
+        table = np.zeros((Ln, width), dtype=np.int32)
         mapping = np.empty(T, dtype=np.int32)
         for row, pages in enumerate(tables):
             pages = np.asarray(pages, dtype=np.int32)
@@ -73,24 +80,62 @@ def build_step_context(lanes: Sequence[Lane], cache, device) -> StepContext:
             lane_positions = positions[cu[row]:cu[row + 1]]
             mapping[cu[row]:cu[row + 1]] = pages[lane_positions // page_size] * page_size + lane_positions % page_size
         sections += [mapping, table.reshape(-1)]
-        group_shapes.append((Ln, max_pages))
-    packed = np.concatenate(sections) if sections else np.zeros(0, dtype=np.int32)
-    host = torch.from_numpy(packed)
-    if torch.device(device).type == "cuda":
-        host = host.pin_memory()
-    packed_device = host.to(device, non_blocking=True)
-    views = []
-    offset = 0
-    for section in sections:
-        views.append(packed_device[offset:offset + section.size])
-        offset += section.size
+        group_shapes.append((Ln, width))
+    return sections, group_shapes, lengths, starts
+
+
+def _assemble(views, group_shapes, lengths, starts, max_seq_len) -> StepContext:
     context = StepContext(
-        num_tokens=T, num_lanes=Ln, token_ids=views[0], positions=views[1], lane_of_token=views[2],
-        cu_seqlens=views[3], start_pos=views[4], seq_lens=views[5], slot_ids=views[6], want_rows=views[7],
-        lane_lengths=lengths, lane_starts=starts, max_query_len=max(lengths),
-        max_seq_len=int(seq_lens.max()))
+        num_tokens=sum(lengths), num_lanes=len(lengths), token_ids=views[0], positions=views[1],
+        lane_of_token=views[2], cu_seqlens=views[3], start_pos=views[4], seq_lens=views[5], slot_ids=views[6],
+        want_rows=views[7], lane_lengths=list(lengths), lane_starts=list(starts), max_query_len=max(lengths),
+        max_seq_len=max_seq_len)
     for index, shape in enumerate(group_shapes):
         context.slot_mappings.append(views[8 + 2 * index])
         context.block_tables.append(views[9 + 2 * index].view(shape))
+    return context
+
+
+def _split(buffer: torch.Tensor, sections):
+    views, offset = [], 0
+    for section in sections:
+        views.append(buffer[offset:offset + section.size])
+        offset += section.size
+    return views
+
+
+def build_step_context(lanes: Sequence[Lane], cache, device) -> StepContext:
+    """``cache``: the CacheManager, after the step's pages were reserved."""
+    sections, group_shapes, lengths, starts = _pack(lanes, cache)
+    host = torch.from_numpy(np.concatenate(sections))
+    if torch.device(device).type == "cuda":
+        host = host.pin_memory()
+    packed = host.to(device, non_blocking=True)
+    context = _assemble(_split(packed, sections), group_shapes, lengths, starts,
+                        max(start + length for start, length in zip(starts, lengths)))
     context._keepalive = host
     return context
+
+
+class StaticStep:
+    """The arrays of a batch of ``lanes`` single-token lanes (every lane's logits wanted) at
+    fixed device addresses.  ``fill`` rewrites them for the real lanes of a step."""
+
+    def __init__(self, cache, lanes: int, max_seq_len: int, device):
+        self.cache = cache
+        self.lanes = lanes
+        self.max_pages = max(-(-max_seq_len // group.page_size) for group in cache.groups) if cache.groups else 1
+        sections, group_shapes, lengths, starts = _pack([], cache, pad_lanes=lanes, max_pages=self.max_pages)
+        sections[7] = np.arange(lanes, dtype=np.int32)             # every lane's row is wanted
+        total = sum(section.size for section in sections)
+        self.host = torch.empty(total, dtype=torch.int32).pin_memory()
+        self.device_buffer = torch.empty(total, dtype=torch.int32, device=device)
+        self.host.copy_(torch.from_numpy(np.concatenate(sections)))
+        self.device_buffer.copy_(self.host)
+        self.context = _assemble(_split(self.device_buffer, sections), group_shapes, lengths, starts, max_seq_len)
+
+    def fill(self, lanes: Sequence[Lane]) -> None:
+        sections, _, _, _ = _pack(lanes, self.cache, pad_lanes=self.lanes - len(lanes), max_pages=self.max_pages)
+        sections[7] = np.arange(self.lanes, dtype=np.int32)
+        self.host.copy_(torch.from_numpy(np.concatenate(sections)))
+        self.device_buffer.copy_(self.host, non_blocking=True)

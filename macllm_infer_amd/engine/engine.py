@@ -46,10 +46,11 @@ class Engine:
     def __init__(self, model_dir: Optional[str] = None, *, config=None, tensors=None, dtype="bfloat16",
                  device="cuda:0", kv_cache_block_tokens: int = 16,
                  kv_cache_capacity_tokens: Optional[int] = None, max_active_sequences: int = 8,
-                 check_device: bool = True):
+                 check_device: bool = True, decode_graphs: bool = True):
         """Load from ``model_dir`` (config.json + safetensors), or from a config object (or raw
         dict) plus a name -> tensor mapping.  ``kv_cache_capacity_tokens`` defaults to one
-        model context shared by all requests (reference: src/runtime.rs:175-201)."""
+        model context shared by all requests (reference: src/runtime.rs:175-201).  With
+        ``decode_graphs`` steps made of single tokens run as captured HIP graphs."""
         self.dtype = resolve_dtype(dtype)
         self.device = ops.require_gpu(device) if check_device else torch.device(device)
         if model_dir is not None:
@@ -73,6 +74,10 @@ class Engine:
                                   self.dtype, self.device)
         self.vocab_size = self.spec.vocab_size
         self.max_context = self.spec.max_context
+        self.graphs = None
+        if decode_graphs and check_device and self.model.graph_safe:
+            from .graphs import DecodeGraphs
+            self.graphs = DecodeGraphs(self.model, self.cache, self.device, min(self.max_context, capacity))
 
     # ------------------------------------------------------------------ requests
     def add_request(self, request: Hashable) -> None:
@@ -119,8 +124,11 @@ class Engine:
         of each lane's ``want``.  Raises StepError or CacheExhausted with nothing changed."""
         self.validate(lanes)
         self.cache.reserve([(lane.request, len(lane.tokens)) for lane in lanes])
-        context = build_step_context(lanes, self.cache, self.device)
-        logits = self.model.forward(context, self.cache)
+        if self.graphs is not None and all(len(lane.tokens) == 1 for lane in lanes):
+            logits = self.graphs.run(lanes)                  # decode-only batch: a captured graph
+        else:
+            context = build_step_context(lanes, self.cache, self.device)
+            logits = self.model.forward(context, self.cache)
         for lane in lanes:
             self.cache.commit(lane.request, len(lane.tokens))
         return logits

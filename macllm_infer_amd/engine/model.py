@@ -68,6 +68,10 @@ class DecoderModel:
                 head = head.to(torch.float32)
             self.lm_head = head.contiguous().to(build.device)
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(block.graph_safe for block in self.blocks) and getattr(self.final_norm, "graph_safe", False)
+
     def forward(self, step, cache) -> torch.Tensor:
         """Run the step's tokens through every scheduled layer and return float32 logits
         [wanted, vocab] at ``step.want_rows`` (empty tensor when nothing is wanted)."""

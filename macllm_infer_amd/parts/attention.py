@@ -21,6 +21,7 @@ class Attention(Mixer):
     Multipliers: ``in_multiplier`` scales the input of q/k/v (folded into their weights),
     ``key_multiplier`` the k projection's output (weights and bias), ``out_multiplier``
     the output projection's output."""
+    graph_safe = True
     kernel_modules = ("common", "attention", "gemm")
 
     @classmethod
@@ -60,6 +61,7 @@ class Attention(Mixer):
         self.out = Linear([get("o_proj.weight")], [get("o_proj.bias")], build,
                           weight_scale=spec.out_multiplier, bias_scale=spec.out_multiplier)
         self.position = part_class(spec.position)(spec.position, spec.head_dim, build)
+        self.graph_safe = bool(getattr(self.position, "graph_safe", False))
 
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         spec = self.spec

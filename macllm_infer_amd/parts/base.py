@@ -16,6 +16,7 @@ mixer           ``cache_needs(spec) -> [KVNeed | StateNeed]`` (classmethod);
 feed-forward    ``forward(x [T, d]) -> [T, d]``
 norm            ``forward(residual, rows=None) -> normed activations``
 position        ``rotate_and_store(qkv, heads, kv_heads, head_dim, step, cache)``
+every part      ``graph_safe = True`` if its forward may be captured in a HIP graph
 """
 from __future__ import annotations
 
@@ -61,6 +62,10 @@ class Residual:
 
 class Part:
     kernel_modules = ()
+    # True when ``forward`` only enqueues work on the current stream (no host read-back, no
+    # data-dependent launch shapes), so that a decode step containing the part can be captured
+    # as a HIP graph.  Parts that do not say so run eagerly.
+    graph_safe = False
 
     @classmethod
     def expected_tensors(cls, spec, prefix: str, hidden_size: int):

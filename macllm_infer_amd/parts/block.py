@@ -57,6 +57,11 @@ class ParallelPreNormBlock:
             layer.ffn_norm, f"{layer.prefix}.{layer.ffn_norm_name}", tensors, build)
         self.ffn = part_class(layer.ffn)(layer.ffn, f"{layer.prefix}.{layer.ffn_name}", tensors, build)
 
+    @property
+    def graph_safe(self) -> bool:
+        parts = [self.mixer_norm, self.ffn_norm, self.ffn] + [mixer for _, mixer in self.mixers]
+        return all(getattr(part, "graph_safe", False) for part in parts)
+
     def forward(self, residual: Residual, step, caches) -> None:
         """``caches``: mixer name -> EntryCache of this run of the layer."""
         normed = self.mixer_norm.forward(residual)

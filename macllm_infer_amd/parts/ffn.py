@@ -14,6 +14,7 @@ class SwiGLU(FeedForward):
     """down(SiLU(gate(x)) * up(x)); gate and up are one fused product
     (reference: src/decoder.rs:261-306).  ``gate_multiplier`` scales gate's output,
     ``down_multiplier`` down's output; both are folded into the weights."""
+    graph_safe = True
     kernel_modules = ("common", "gemm")
 
     @classmethod

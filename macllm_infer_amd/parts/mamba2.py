@@ -21,6 +21,7 @@ class Mamba2(Mixer):
     The decay is stored as ``A_log`` and used as A = -exp(A_log).  ``multipliers`` scale the
     five segments of in_proj's output (after its bias), ``in_multiplier`` its input,
     ``out_multiplier`` out_proj's output; all are folded into the weights."""
+    graph_safe = True
     kernel_modules = ("common", "mamba2", "gemm")
 
     @classmethod

@@ -14,6 +14,7 @@ from .base import BuildContext, Part, Residual, register_part
 class RmsNorm(Part):
     """y = x / sqrt(mean(x^2) + eps) * w, statistics in float32
     (reference: src/model_weights.rs:563-565, golden src/decoder.rs:10331-10334)."""
+    graph_safe = True
     kernel_modules = ("common",)
 
     @classmethod

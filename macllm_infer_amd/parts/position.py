@@ -27,6 +27,8 @@ class PositionEncoding(Part):
 
 @register_part("none")
 class NoPosition(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, spec, head_dim: int, build: BuildContext):
         pass
 
@@ -36,6 +38,7 @@ class Rope(PositionEncoding):
     """Half-split rotary encoding: f_j = theta^(-2j/rotary_dim) formed in float64 and rounded
     to float32; angle = position * f_j, cos and sin in float32
     (reference: src/decoder.rs:136-144, 186-195, 226-229)."""
+    graph_safe = True
 
     def __init__(self, spec, head_dim: int, build: BuildContext):
         self.rotary_dim = spec.rotary_dim

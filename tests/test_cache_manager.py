@@ -42,12 +42,12 @@ def test_page_pool_invariants():
 def test_groups_share_a_table_per_geometry_and_windows_get_their_own():
     cache = make(window=10)
     assert len(cache.groups) == 2
-    assert cache.groups[0].storage.shape == (8, 2, 2, 2, 32)      # [page, layer, K|V, kv head, token x dim]
-    assert first_views(cache) == ((8, 2, 8, 4), (8, 2, 4, 8))     # V pages are transposed
+    assert cache.groups[0].storage.shape == (9, 2, 2, 2, 32)      # [page (+1 scratch), layer, K|V, kv head, token x dim]
+    assert first_views(cache) == ((9, 2, 8, 4), (9, 2, 4, 8))     # V pages are transposed
     assert cache.groups[1].need.window == 10 and len(cache.groups[1].members) == 1
     first, second = cache.entry((0, "attn")), cache.entry((1, "attn"))
     assert first.group == second.group == 0 and first.k_cache.data_ptr() != second.k_cache.data_ptr()
-    assert cache.entry((1, "rec")).states["s"].shape == (3, 3, 2)
+    assert cache.entry((1, "rec")).states["s"].shape == (4, 3, 2)      # 3 slots + the scratch slot
     assert cache.entry((1, "rec")).states["c"].dtype == torch.float32
 
 

@@ -230,3 +230,46 @@ def test_toy_parts_register_build_and_step(schedule):
     run's cache: registered in the tests, built by the engine, stepped whole, in portions
     and mixed, on the GPU with the package's kernels."""
     toy_parts.exercise(schedule, DEV, check_device=True)
+
+
+@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16")])
+def test_decode_graphs_match_eager_steps(tmp_path, name, dtype):
+    """Decode steps replayed from captured graphs, with eager prompt portions of other requests
+    and synchronizations between the replays; every replay is compared with the same step of an
+    engine without graphs, for changing batch sizes (buckets 1, 2, 4 with padding lanes)."""
+    from macllm_infer_amd import Engine, Lane
+    folder = tiny_configs.make_model_dir(name, tmp_path, torch.float32 if dtype == "float32" else torch.bfloat16)
+    cfg, _ = plain_impl.load_model_dir(folder)
+    make = lambda graphs: Engine(folder, dtype=dtype, kv_cache_block_tokens=8, kv_cache_capacity_tokens=512,
+                                 max_active_sequences=4, decode_graphs=graphs)
+    with_graphs, eager = make(True), make(False)
+    assert with_graphs.graphs is not None and eager.graphs is None
+    sequences = {key: tokens_for(cfg["vocab_size"], 90, 30 + index) for index, key in enumerate("abcd")}
+    cursor = {key: 0 for key in sequences}
+
+    def both(lanes_spec):
+        lanes = [Lane(key, sequences[key][cursor[key]:cursor[key] + count], list(range(count)))
+                 for key, count in lanes_spec]
+        got, want = with_graphs.step(lanes).float().cpu(), eager.step(lanes).float().cpu()
+        for key, count in lanes_spec:
+            cursor[key] += count
+        scale = max(1.0, want.abs().max().item())
+        assert (got - want).abs().max() <= (1e-5 if dtype == "float32" else 3e-2) * scale
+
+    for engine in (with_graphs, eager):
+        for key in sequences:
+            engine.add_request(key)
+    both([("a", 9)])
+    for turn in range(40):
+        if turn == 3:
+            both([("b", 17)])                                   # an eager prompt between replays
+        if turn == 10:
+            both([("c", 5), ("d", 12)])
+        if turn == 20:
+            torch.cuda.synchronize()
+        live = [key for key in "abcd" if cursor[key] > 0]
+        if turn % 7 == 6:
+            live = live[:1]                                     # bucket 1
+        both([(key, 1) for key in live])
+    assert set(with_graphs.graphs._graphs) == {1, 2, 4}
+    assert with_graphs.cache.stats() == eager.cache.stats()
