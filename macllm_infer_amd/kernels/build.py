@@ -25,8 +25,8 @@ CSRC = os.path.normpath(CSRC)
 ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-shared", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
-MODULES = ("common", "attention", "mamba2", "gemm", "sampling")
+         "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", "-Wno-pass-failed"]
+MODULES = ("common", "attention", "mamba2", "gemm", "decode", "sampling")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

@@ -57,6 +57,16 @@ _SIGNATURES = {
     "gemm": {
         "mi_gemm_f32": [_c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr],
     },
+    "decode": {
+        "mi_fused_gemm": [_c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_long, _c_ptr,
+                          _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_int, _c_float, _c_int, _c_int, _c_int,
+                          _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+        "mi_fused_gemm_supported": [_c_int, _c_int, _c_int],
+        "mi_mixer_decode": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int,
+                            _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int,
+                            _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                            _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr],
+    },
     "sampling": {
         "mi_apply_penalties": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                _c_ptr, _c_ptr],
@@ -405,6 +415,134 @@ def gate_norm(y: torch.Tensor, z: torch.Tensor, weight: Optional[torch.Tensor], 
           "gate_norm: weight must be float32 [E]")
     _check(_fn("mamba2", "mi_gate_norm")(_p(y), y_ld, _p(z), _dt(z), z_ld, _p(weight), num_groups, float(eps),
                                          _p(out), out_ld, T, E, _stream()), "gate_norm")
+
+
+# --------------------------------------------------------------------------- fused decode kernels
+PRO_NORM, PRO_PLAIN = 0, 1
+EPI_PLAIN, EPI_SWIGLU, EPI_CONV = 0, 1, 2
+
+
+def fused_gemm_supported(normed: bool, rows: int, in_features: int) -> bool:
+    """Whether ``fused_gemm`` covers a batch of ``rows`` rows of ``in_features`` inputs."""
+    return bool(_fn("decode", "mi_fused_gemm_supported")(PRO_NORM if normed else PRO_PLAIN, rows, in_features))
+
+
+def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, *, out_scale: float = 1.0,
+               x: Optional[torch.Tensor] = None, h_in: Optional[torch.Tensor] = None,
+               deltas: Sequence[torch.Tensor] = (), h_out: Optional[torch.Tensor] = None,
+               norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, epilogue: int = EPI_PLAIN,
+               conv: Optional[dict] = None) -> None:
+    """out[M, N'] = epilogue(prologue . weight[N, K]^T + bias) for a small batch in bfloat16.
+
+    Prologue: ``x`` [M, K] bfloat16, or ``h_in`` float32 [M, K] with up to two bfloat16 ``deltas``:
+    the rows are summed (the sum goes to ``h_out``, a different tensor, if given), RMS-normed
+    with ``norm_weight`` and ``eps``.  Epilogue PLAIN: bfloat16 or float32 ``out`` [M, N] times
+    ``out_scale``.  SWIGLU: weight rows in tiles of 8 gate + 8 up rows, ``out`` [M, N/2].
+    CONV: ``conv`` = {lo, hi, taps, weight [C, taps], bias, state [slots, taps-1, C], slot_ids}:
+    rows lo..hi-1 go through the causal depthwise conv step of their channel with the request's
+    tail (which is rolled) and SiLU."""
+    _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
+          "fused_gemm: weight must be contiguous bfloat16 [N, K]")
+    N, K = weight.shape
+    M = out.shape[0]
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()),
+          "fused_gemm: bias must be float32 [N]")
+    out_ld = _row_major(out, "out")
+    _need(out.dtype in (torch.bfloat16, torch.float32), "fused_gemm: out must be bfloat16 or float32")
+    _need(out.shape[1] == (N // 2 if epilogue == EPI_SWIGLU else N), "fused_gemm: out has the wrong width")
+    if x is not None:
+        pro = PRO_PLAIN
+        x_ld = _row_major(x, "x")
+        _need(x.dtype == torch.bfloat16 and x.shape == (M, K) and x.data_ptr() % 16 == 0, "fused_gemm: bad x")
+    else:
+        pro = PRO_NORM
+        x_ld = 0
+        _need(h_in is not None and h_in.dtype == torch.float32 and h_in.shape == (M, K) and h_in.is_contiguous(),
+              "fused_gemm: h_in must be contiguous float32 [M, K]")
+        _need(len(deltas) <= 2 and all(d.dtype == torch.bfloat16 and d.shape == (M, K) and d.is_contiguous()
+                                       for d in deltas), "fused_gemm: deltas must be contiguous bfloat16 [M, K]")
+        _need(h_out is None or (h_out.shape == (M, K) and h_out.dtype == torch.float32 and h_out.is_contiguous()
+                                and h_out.data_ptr() != h_in.data_ptr()), "fused_gemm: bad h_out")
+        _need(norm_weight is not None and norm_weight.dtype == torch.float32 and norm_weight.numel() == K,
+              "fused_gemm: norm_weight must be float32 [K]")
+    lo = hi = taps = 0
+    conv_w = conv_b = conv_state = slot_ids = None
+    if epilogue == EPI_CONV:
+        lo, hi, taps = conv["lo"], conv["hi"], conv["taps"]
+        conv_w, conv_b, conv_state, slot_ids = conv["weight"], conv.get("bias"), conv["state"], conv["slot_ids"]
+        channels = hi - lo
+        _need(conv_w.dtype == torch.float32 and conv_w.shape == (channels, taps) and conv_w.is_contiguous(),
+              "fused_gemm: conv weight must be float32 [C, taps]")
+        _need(conv_b is None or (conv_b.dtype == torch.float32 and conv_b.numel() == channels), "fused_gemm: bad conv bias")
+        _need(conv_state.dtype == torch.bfloat16 and conv_state.shape[1:] == (max(taps - 1, 0), channels)
+              and conv_state.is_contiguous(), "fused_gemm: bad conv state")
+        _i32(slot_ids, "slot_ids")
+        _need(slot_ids.numel() >= M, "fused_gemm: one slot per row")
+    _check(_fn("decode", "mi_fused_gemm")(
+        pro, epilogue, _p(h_in), _p(deltas[0]) if len(deltas) > 0 else None, _p(deltas[1]) if len(deltas) > 1 else None,
+        _p(h_out), _p(norm_weight), float(eps), _p(x), x_ld, _p(weight), _p(bias), M, N, K, _p(out), out_ld,
+        1 if out.dtype == torch.float32 else 0, float(out_scale), lo, hi, taps, _p(conv_w), _p(conv_b), _p(conv_state),
+        _p(slot_ids), _stream()), "fused_gemm", f"(M={M}, N={N}, K={K})")
+
+
+def mixer_decode_supported(num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, state_size: int) -> bool:
+    return (head_dim in (64, 128) and num_heads // num_kv_heads <= 8 and page_size % 8 == 0 and page_size <= 512
+            and state_size <= 512)
+
+
+def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int, q_col: int, k_col: int,
+                 v_col: int, inv_freq: Optional[torch.Tensor], rotary_dim: int, k_cache: torch.Tensor,
+                 v_cache: torch.Tensor, block_tables: torch.Tensor, positions: torch.Tensor,
+                 slot_mapping: torch.Tensor, scale: float, window: Optional[int], max_seq_len: int,
+                 counters: torch.Tensor, ssm_heads: int, ssm_head_dim: int, state_size: int, num_groups: int,
+                 z_col: int, x_col: int, dt_col: int, dt_bias: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
+                 ssm_state: torch.Tensor, slot_ids: torch.Tensor, out: torch.Tensor,
+                 ssm_y: Optional[torch.Tensor]) -> None:
+    """Both mixers of a decode step in one launch.  ``u`` [M, >=cols] holds each token's projected
+    row (q, k, v unrotated; x, B, C after the conv).  Attention: rotates q and the new key, writes
+    the new K/V into the cache cell ``slot_mapping``, attends over the request's pages, writes
+    ``out[:, :Hq*dh]``.  State space: one scan step from and into ``ssm_state[slot_ids]``, writes
+    ``y * SiLU(z)`` to ``out[:, Hq*dh:]``, or float32 ``y`` to ``ssm_y`` when a grouped norm
+    follows.  ``counters``: int32 zeros [>= M*Hkv], left at zero."""
+    u_ld = _row_major(u, "u")
+    out_ld = _row_major(out, "out")
+    M = u.shape[0]
+    E = ssm_heads * ssm_head_dim
+    _need(u.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and out.shape == (M, num_heads * head_dim + E),
+          "mixer_decode: u/out shapes do not match")
+    page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, u.dtype)
+    _need(mixer_decode_supported(num_heads, num_kv_heads, head_dim, page_size, state_size),
+          "mixer_decode: geometry not covered")
+    for name, tensor in (("block_tables", block_tables), ("positions", positions), ("slot_mapping", slot_mapping),
+                         ("slot_ids", slot_ids), ("counters", counters)):
+        _i32(tensor, name)
+    _need(block_tables.dim() == 2 and block_tables.shape[0] >= M and positions.numel() == M
+          and slot_mapping.numel() == M and slot_ids.numel() == M and counters.numel() >= M * num_kv_heads,
+          "mixer_decode: metadata shapes do not match")
+    _need(ssm_state.dtype == torch.float32 and ssm_state.shape[1:] == (ssm_heads, ssm_head_dim, state_size)
+          and ssm_state.is_contiguous(), "mixer_decode: bad state")
+    for name, vector in (("dt_bias", dt_bias), ("A", A), ("D", D)):
+        _need(vector.dtype == torch.float32 and vector.numel() == ssm_heads, f"mixer_decode: {name} must be float32 [H]")
+    _need(ssm_y is None or (ssm_y.dtype == torch.float32 and ssm_y.shape == (M, E) and ssm_y.is_contiguous()),
+          "mixer_decode: bad ssm_y")
+    widest = max(q_col + num_heads * head_dim, k_col + num_kv_heads * head_dim, v_col + num_kv_heads * head_dim,
+                 z_col + E, x_col + E + 2 * num_groups * state_size, dt_col + ssm_heads)
+    _need(u.shape[1] >= widest, "mixer_decode: u is too narrow")
+    span = max_seq_len if not window else min(max_seq_len, window + page_size)
+    split_keys = 64
+    while split_keys < 512 and span * M * num_kv_heads > 1024 * split_keys:
+        split_keys *= 2
+    split_keys = max(split_keys, page_size)
+    splits = max(1, -(-span // split_keys))
+    partial_o = torch.empty((M, num_heads, splits, head_dim), dtype=torch.float32, device=u.device)
+    partial_ml = torch.empty((M, num_heads, splits, 2), dtype=torch.float32, device=u.device)
+    _check(_fn("decode", "mi_mixer_decode")(
+        _p(u), u_ld, M, num_heads, num_kv_heads, head_dim, q_col, k_col, v_col, _p(inv_freq), rotary_dim,
+        _p(k_cache), _p(v_cache), page_stride, page_size, _p(block_tables), block_tables.shape[1], _p(positions),
+        _p(slot_mapping), float(scale), int(window or 0), split_keys, splits, _p(partial_o), _p(partial_ml),
+        _p(counters), ssm_heads, ssm_head_dim, state_size, num_groups, z_col, x_col, dt_col, _p(dt_bias), _p(A),
+        _p(D), _p(ssm_state), _p(slot_ids), _p(out), out.data_ptr() + 2 * num_heads * head_dim,
+        _p(ssm_y), out_ld, _stream()), "mixer_decode")
 
 
 # --------------------------------------------------------------------------- sampling

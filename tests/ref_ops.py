@@ -204,3 +204,78 @@ def sample(logits, temperature, top_k, top_p, seeds, draw_index, keys, out):
 
 
 NAMES += ["apply_penalties", "sample"]
+
+
+# ---------------------------------------------------------------- fused decode kernels, as compositions
+PRO_NORM, PRO_PLAIN = 0, 1
+EPI_PLAIN, EPI_SWIGLU, EPI_CONV = 0, 1, 2
+
+
+def fused_gemm_supported(normed, rows, in_features):
+    return False
+
+
+def mixer_decode_supported(num_heads, num_kv_heads, head_dim, page_size, state_size):
+    return False
+
+
+def fused_gemm(weight, bias, out, *, out_scale=1.0, x=None, h_in=None, deltas=(), h_out=None, norm_weight=None,
+               eps=0.0, epilogue=EPI_PLAIN, conv=None):
+    if x is None:
+        total = h_in.clone()
+        for delta in deltas:
+            total += _f(delta)
+        if h_out is not None:
+            h_out.copy_(total)
+        normed = total / torch.sqrt(total.pow(2).mean(-1, keepdim=True) + eps) * norm_weight
+        rows = _f(normed.to(torch.bfloat16))
+    else:
+        rows = _f(x)
+    y = rows @ _f(weight).T
+    if bias is not None:
+        y = y + bias
+    M, N = y.shape
+    if epilogue == EPI_PLAIN:
+        out.copy_((y * out_scale).to(out.dtype))
+    elif epilogue == EPI_SWIGLU:
+        tiles = _f(y.to(torch.bfloat16)).reshape(M, N // 16, 16)
+        out.copy_((F.silu(tiles[..., :8]) * tiles[..., 8:]).reshape(M, N // 2).to(out.dtype))
+    else:
+        lo, hi, taps = conv["lo"], conv["hi"], conv["taps"]
+        result = y.to(torch.bfloat16)
+        sample = result[:, lo:hi].clone()
+        for m in range(M):
+            slot = int(conv["slot_ids"][m])
+            window = torch.cat([conv["state"][slot], sample[m:m + 1]], dim=0)        # [taps, C]
+            total = (_f(window) * conv["weight"].T).sum(0)
+            if conv.get("bias") is not None:
+                total = total + conv["bias"]
+            result[m, lo:hi] = F.silu(total).to(torch.bfloat16)
+            if taps > 1:
+                conv["state"][slot] = window[1:]
+        out.copy_(result)
+
+
+def mixer_decode(u, *, num_heads, num_kv_heads, head_dim, q_col, k_col, v_col, inv_freq, rotary_dim, k_cache, v_cache,
+                 block_tables, positions, slot_mapping, scale, window, max_seq_len, counters, ssm_heads, ssm_head_dim,
+                 state_size, num_groups, z_col, x_col, dt_col, dt_bias, A, D, ssm_state, slot_ids, out, ssm_y):
+    M = u.shape[0]
+    q_width, kv_width = num_heads * head_dim, num_kv_heads * head_dim
+    qkv = torch.cat([u[:, q_col:q_col + q_width], u[:, k_col:k_col + kv_width], u[:, v_col:v_col + kv_width]], dim=1).clone()
+    rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, rotary_dim, slot_mapping, k_cache, v_cache)
+    lanes = torch.arange(M, dtype=torch.int32)
+    paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lanes, positions, scale,
+                    window, out[:, :q_width])
+    E = ssm_heads * ssm_head_dim
+    width = E + 2 * num_groups * state_size
+    y = torch.empty(M, E)
+    cu = torch.arange(M + 1, dtype=torch.int32)
+    ssm_scan(u[:, x_col:x_col + width], u[:, dt_col:dt_col + ssm_heads], dt_bias, A, D, ssm_state, cu, slot_ids,
+             num_groups, y)
+    if ssm_y is not None:
+        ssm_y.copy_(y)
+    else:
+        gate_norm(y, u[:, z_col:z_col + E], None, num_groups, 0.0, out[:, q_width:])
+
+
+NAMES += ["fused_gemm_supported", "mixer_decode_supported", "fused_gemm", "mixer_decode"]

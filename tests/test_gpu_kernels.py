@@ -433,3 +433,125 @@ def test_decode_attention_finds_one_far_key(ops):
                              i32([length - 1]).to(DEV), 1.0 / math.sqrt(dh), None, length, out)
         expected = values[chosen].float()[[0] * 4 + [1] * 4].reshape(-1)
         assert (out.float().cpu()[0] - expected).abs().max() < 1e-2, f"key {chosen} was missed"
+
+
+# ------------------------------------------------------------------ fused decode kernels
+@pytest.mark.parametrize("M, N, K", [(1, 48, 64), (8, 4120, 1024), (5, 100, 96), (16, 250, 1024), (33, 64, 256),
+                                     (64, 130, 2048)])
+def test_fused_gemm_plain_prologue(ops, M, N, K):
+    x = rand(M, K + 8, seed=300, dtype=torch.bfloat16)[:, :K]            # a row stride
+    W, b = rand(N, K, seed=301, scale=0.1, dtype=torch.bfloat16), rand(N, seed=302)
+    for out_dtype, scale, bias in ((torch.bfloat16, 1.0, b), (torch.float32, 0.6, None)):
+        want = torch.empty(M, N, dtype=out_dtype)
+        ref_ops.fused_gemm(W, bias, want, x=x, out_scale=scale)
+        got = torch.empty(M, N, dtype=out_dtype, device=DEV)
+        ops.fused_gemm(W.to(DEV), None if bias is None else bias.to(DEV), got, x=x.to(DEV), out_scale=scale)
+        close(got, want, out_dtype, 6.0 if out_dtype == torch.bfloat16 else 200.0)
+    assert ops.fused_gemm_supported(False, M, K) and not ops.fused_gemm_supported(False, 65, K)
+    assert not ops.fused_gemm_supported(False, M, K + 8)
+
+
+@pytest.mark.parametrize("M, N, K, deltas", [(1, 64, 64, 0), (8, 160, 1024, 2), (13, 48, 96, 1), (16, 4120, 1024, 2)])
+def test_fused_gemm_norm_prologue_and_epilogues(ops, M, N, K, deltas):
+    h = rand(M, K, seed=310)
+    ds = [rand(M, K, seed=311 + i, dtype=torch.bfloat16) for i in range(deltas)]
+    norm_w = rand(K, seed=314, scale=0.1) + 1.0
+    W, b = rand(N, K, seed=315, scale=0.1, dtype=torch.bfloat16), rand(N, seed=316)
+    assert ops.fused_gemm_supported(True, M, K)
+    # plain
+    want, want_h = torch.empty(M, N, dtype=torch.bfloat16), torch.empty(M, K)
+    ref_ops.fused_gemm(W, b, want, h_in=h, deltas=ds, h_out=want_h, norm_weight=norm_w, eps=3e-6)
+    got, got_h = torch.empty(M, N, dtype=torch.bfloat16, device=DEV), torch.full((M, K), float("nan"), device=DEV)
+    ops.fused_gemm(W.to(DEV), b.to(DEV), got, h_in=h.to(DEV), deltas=gpu(*ds), h_out=got_h, norm_weight=norm_w.to(DEV),
+                   eps=3e-6)
+    close(got, want, torch.bfloat16, 8.0)
+    close(got_h, want_h, torch.float32)
+    # swiglu (tiles of 8 gate rows + 8 up rows)
+    if N % 16 == 0:
+        want = torch.empty(M, N // 2, dtype=torch.bfloat16)
+        ref_ops.fused_gemm(W, b, want, h_in=h, deltas=ds, norm_weight=norm_w, eps=3e-6, epilogue=ref_ops.EPI_SWIGLU)
+        got = torch.empty(M, N // 2, dtype=torch.bfloat16, device=DEV)
+        ops.fused_gemm(W.to(DEV), b.to(DEV), got, h_in=h.to(DEV), deltas=gpu(*ds), norm_weight=norm_w.to(DEV),
+                       eps=3e-6, epilogue=ops.EPI_SWIGLU)
+        close(got, want, torch.bfloat16, 16.0)
+    # conv rows in the middle, taps 1..4, shuffled slots (one slot untouched)
+    lo, hi = 16, N - 8
+    for taps in (4, 3, 1):
+        C = hi - lo
+        state = rand(M + 2, max(taps - 1, 0), C, seed=320, dtype=torch.bfloat16)
+        slot_ids = torch.randperm(M + 2, generator=torch.Generator().manual_seed(taps))[:M].to(torch.int32)
+        conv = dict(lo=lo, hi=hi, taps=taps, weight=rand(C, taps, seed=321, scale=0.5), bias=rand(C, seed=322, scale=0.1))
+        want_state, got_state = state.clone(), state.clone().to(DEV)
+        want = torch.empty(M, N, dtype=torch.bfloat16)
+        ref_ops.fused_gemm(W, b, want, h_in=h, deltas=ds, norm_weight=norm_w, eps=3e-6, epilogue=ref_ops.EPI_CONV,
+                           conv=dict(conv, state=want_state, slot_ids=slot_ids))
+        got = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        ops.fused_gemm(W.to(DEV), b.to(DEV), got, h_in=h.to(DEV), deltas=gpu(*ds), norm_weight=norm_w.to(DEV), eps=3e-6,
+                       epilogue=ops.EPI_CONV,
+                       conv=dict(lo=lo, hi=hi, taps=taps, weight=conv["weight"].to(DEV), bias=conv["bias"].to(DEV),
+                                 state=got_state, slot_ids=slot_ids.to(DEV)))
+        close(got, want, torch.bfloat16, 8.0)
+        close(got_state, want_state, torch.bfloat16, 8.0)
+        unused = [slot for slot in range(M + 2) if slot not in slot_ids.tolist()]
+        assert torch.equal(got_state[unused].cpu(), state[unused])
+
+
+@pytest.mark.parametrize("Hq, Hkv, dh, H, P, N, G, page_size, window, rotary, gated", [
+    (8, 2, 64, 24, 64, 128, 1, 16, None, 64, False), (12, 2, 128, 6, 40, 256, 2, 16, None, 128, True),
+    (4, 4, 64, 3, 24, 40, 3, 8, 100, 32, False), (8, 1, 64, 5, 7, 9, 1, 32, None, 0, False)])
+def test_mixer_decode_against_the_separate_kernels(ops, Hq, Hkv, dh, H, P, N, G, page_size, window, rotary, gated):
+    """Both mixers of a decode step in one launch, for requests with contexts of 1 to 1 500
+    tokens; compared with the composition of the plain references, cache and state included.
+    Twice in a row: the split counters must be back at zero."""
+    dtype = torch.bfloat16
+    lengths = [1, 17, 64, 65, 300, 1500, 2]
+    M = len(lengths)
+    pool, table = paged_setup(lengths, page_size, Hkv, dh, dtype, seed=11)
+    for lane, length in enumerate(lengths):          # everything before the new token is cached already
+        fill_cache(pool, table, lane, rand(length, Hkv, dh, seed=400 + lane, dtype=dtype),
+                   rand(length, Hkv, dh, seed=500 + lane, dtype=dtype), page_size)
+    E, GN = H * P, G * N
+    q_col, k_col, v_col = 0, Hq * dh, (Hq + Hkv) * dh
+    z_col = (Hq + 2 * Hkv) * dh
+    x_col, dt_col = z_col + E, z_col + 2 * E + 2 * GN
+    u = rand(M, -(-(dt_col + H) // 8) * 8, seed=410, dtype=dtype)      # rows 16-byte aligned
+    positions = i32([length - 1 for length in lengths])
+    slot_mapping = i32([int(table[lane, (length - 1) // page_size]) * page_size + (length - 1) % page_size
+                        for lane, length in enumerate(lengths)])
+    inv_freq = None if rotary == 0 else torch.tensor([1.0 / (1e4 ** (i / rotary)) for i in range(0, rotary, 2)],
+                                                      dtype=torch.float64).float()
+    slots = M + 1
+    slot_ids = torch.randperm(slots, generator=torch.Generator().manual_seed(5))[:M].to(torch.int32)
+    state = rand(slots, H, P, N, seed=411, scale=0.5)
+    dt_bias, A, D = rand(H, seed=412) - 2.0, -(rand(H, seed=413).abs() + 0.1), rand(H, seed=414)
+    common = dict(num_heads=Hq, num_kv_heads=Hkv, head_dim=dh, q_col=q_col, k_col=k_col, v_col=v_col,
+                  rotary_dim=rotary, scale=0.11, window=window, max_seq_len=2048, ssm_heads=H, ssm_head_dim=P,
+                  state_size=N, num_groups=G, z_col=z_col, x_col=x_col, dt_col=dt_col)
+    want_pool, want_state = pool.clone(), state.clone()
+    want_out = torch.zeros(M, Hq * dh + E, dtype=dtype)
+    want_y = torch.empty(M, E) if gated else None
+    ref_ops.mixer_decode(u, inv_freq=inv_freq, k_cache=views(want_pool, page_size)[0], v_cache=views(want_pool, page_size)[1],
+                         block_tables=table, positions=positions, slot_mapping=slot_mapping, counters=None,
+                         dt_bias=dt_bias, A=A, D=D, ssm_state=want_state, slot_ids=slot_ids, out=want_out, ssm_y=want_y,
+                         **common)
+    assert ops.mixer_decode_supported(Hq, Hkv, dh, page_size, N)
+    counters = torch.zeros(M * Hkv, dtype=torch.int32, device=DEV)
+    for repeat in range(2):
+        got_pool, got_state = pool.clone().to(DEV), state.clone().to(DEV)
+        got_out = torch.zeros(M, Hq * dh + E, dtype=dtype, device=DEV)
+        got_y = torch.empty(M, E, device=DEV) if gated else None
+        ops.mixer_decode(u.to(DEV), inv_freq=None if inv_freq is None else inv_freq.to(DEV),
+                         k_cache=views(got_pool, page_size)[0], v_cache=views(got_pool, page_size)[1],
+                         block_tables=table.to(DEV), positions=positions.to(DEV), slot_mapping=slot_mapping.to(DEV),
+                         counters=counters, dt_bias=dt_bias.to(DEV), A=A.to(DEV), D=D.to(DEV), ssm_state=got_state,
+                         slot_ids=slot_ids.to(DEV), out=got_out, ssm_y=got_y, **common)
+        close(got_out[:, :Hq * dh], want_out[:, :Hq * dh], dtype, 2.0)
+        scale = max(1.0, want_state.abs().max().item())
+        close(got_state, want_state, torch.float32, scale)
+        if gated:
+            close(got_y, want_y, torch.float32, max(1.0, want_y.abs().max().item()))
+        else:
+            close(got_out[:, Hq * dh:], want_out[:, Hq * dh:], dtype, max(1.0, want_out.float().abs().max().item()))
+        assert torch.equal(torch.isnan(got_pool.float().cpu()), torch.isnan(want_pool.float()))
+        close(torch.nan_to_num(got_pool.float()), torch.nan_to_num(want_pool.float()), dtype, 4.0)
+        assert int(counters.abs().sum()) == 0
