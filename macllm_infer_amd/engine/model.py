@@ -86,8 +86,21 @@ class DecoderModel:
         wanted = step.want_rows.numel()
         if wanted == 0:
             return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.build.device)
+        logits = torch.empty((wanted, spec.vocab_size), dtype=torch.float32, device=self.build.device)
+        if self._fused_head(step, wanted):
+            # a decode step whose every row is wanted: residual add, norm, projection and scaling in one launch
+            ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, h_in=residual.h,
+                           deltas=residual.pending, norm_weight=self.final_norm.weight, eps=self.final_norm.eps)
+            return logits
         normed = self.final_norm.forward(residual, rows=step.want_rows)
         raw = ops.linear(normed, self.lm_head, None)
-        logits = torch.empty((wanted, spec.vocab_size), dtype=torch.float32, device=self.build.device)
         ops.scale_to_f32(raw, spec.logit_multiplier, logits)
         return logits
+
+    def _fused_head(self, step, wanted: int) -> bool:
+        from ..parts.norm import RmsNorm
+        return (step.max_query_len == 1 and wanted == step.num_tokens and wanted <= 16
+                and self.build.dtype == torch.bfloat16 and self.lm_head.dtype == torch.bfloat16
+                and type(self.final_norm) is RmsNorm and len(step.lane_lengths) == wanted
+                and self.build.device.type == "cuda" and self.spec.hidden_size % 32 == 0
+                and ops.fused_gemm_supported(True, wanted, self.spec.hidden_size))

@@ -56,6 +56,8 @@ class ParallelPreNormBlock:
         self.ffn_norm = part_class(layer.ffn_norm)(
             layer.ffn_norm, f"{layer.prefix}.{layer.ffn_norm_name}", tensors, build)
         self.ffn = part_class(layer.ffn)(layer.ffn, f"{layer.prefix}.{layer.ffn_name}", tensors, build)
+        from .fused_decode import ParallelDecodeFusion
+        self.decode_fusion = ParallelDecodeFusion.build(self, build)      # None when the parts or sizes do not fit
 
     @property
     def graph_safe(self) -> bool:
@@ -64,6 +66,10 @@ class ParallelPreNormBlock:
 
     def forward(self, residual: Residual, step, caches) -> None:
         """``caches``: mixer name -> EntryCache of this run of the layer."""
+        fusion = self.decode_fusion
+        if fusion is not None and fusion.supports(step, caches[fusion.attention_name]):
+            fusion.forward(residual, step, caches)
+            return
         normed = self.mixer_norm.forward(residual)
         residual.pending = [mixer.forward(normed, step, caches[name]) for name, mixer in self.mixers]
         normed = self.ffn_norm.forward(residual)

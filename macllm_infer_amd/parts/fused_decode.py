@@ -1,0 +1,163 @@
+"""The decode fast path of a layer: when every lane of a step holds one token, a block made
+of RMSNorm, attention, Mamba2 and SwiGLU runs as five launches instead of fifteen.
+
+    1. residual add + norm + [q|k|v|z|x B C|dt] projection + conv step        (fused_gemm)
+    2. attention (rotation, cache write, split context, merge) and SSM step    (mixer_decode)
+    3. [attention | ssm] . [Wo | W_out]^T                                       (fused_gemm)
+    4. residual add + norm + gate/up projection + SiLU(g)*u                     (fused_gemm)
+    5. down projection                                                          (fused_gemm)
+
+The fusion belongs to the arrangement, which knows its parts; the parts stay as they are and
+serve every other kind of step.  It is built only for bfloat16 weights and sizes the kernels
+cover; otherwise the block runs part by part.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from .attention import Attention
+from .base import Residual
+from .ffn import SwiGLU
+from .mamba2 import Mamba2
+from .norm import RmsNorm
+from .position import NoPosition, Rope
+
+MAX_ROWS = 16          # the norm prologue recomputes the normed rows in every workgroup: small batches only
+
+
+class ParallelDecodeFusion:
+    @staticmethod
+    def build(block, build) -> Optional["ParallelDecodeFusion"]:
+        if build.dtype != torch.bfloat16 or build.device.type != "cuda":
+            return None
+        mixers = dict(block.mixers)
+        if len(mixers) != 2:
+            return None
+        attention = next((m for m in mixers.values() if type(m) is Attention), None)
+        mamba = next((m for m in mixers.values() if type(m) is Mamba2), None)
+        if attention is None or mamba is None or type(block.ffn) is not SwiGLU:
+            return None
+        if type(block.mixer_norm) is not RmsNorm or type(block.ffn_norm) is not RmsNorm:
+            return None
+        if type(attention.position) not in (Rope, NoPosition):
+            return None
+        linears = [attention.qkv, attention.out, mamba.in_proj, mamba.out_proj, block.ffn.gate_up, block.ffn.down]
+        if any(linear.weight.dtype != torch.bfloat16 for linear in linears):
+            return None
+        a, s = attention.spec, mamba.spec
+        hidden = build.hidden_size
+        inner = block.ffn.spec.intermediate_size
+        mixed_width = a.num_heads * a.head_dim + s.inner_size
+        if a.head_dim not in (64, 128) or a.num_heads // a.num_kv_heads > 8 or s.state_size > 512:
+            return None
+        if inner % 8 != 0 or hidden % 32 != 0 or mixed_width % 32 != 0 or inner % 32 != 0:
+            return None
+        if not ops.fused_gemm_supported(True, 1, hidden):
+            return None
+        return ParallelDecodeFusion(block, attention, mamba, build)
+
+    def __init__(self, block, attention: Attention, mamba: Mamba2, build):
+        self.block = block
+        self.attention = attention
+        self.mamba = mamba
+        self.attention_name = next(name for name, mixer in block.mixers if mixer is attention)
+        self.mamba_name = next(name for name, mixer in block.mixers if mixer is mamba)
+        device = build.device
+        a, s = attention.spec, mamba.spec
+        self.hidden = build.hidden_size
+        q_width, kv_width = a.num_heads * a.head_dim, a.num_kv_heads * a.head_dim
+        E, C = s.inner_size, s.conv_width
+        # 1: [q | k | v | z | x B C | dt]
+        self.w_in = torch.cat([attention.qkv.weight, mamba.in_proj.weight], dim=0).contiguous()
+        self.b_in = _cat_bias([attention.qkv, mamba.in_proj], device)
+        self.q_col, self.k_col, self.v_col = 0, q_width, q_width + kv_width
+        self.z_col = q_width + 2 * kv_width
+        self.x_col = self.z_col + E
+        self.dt_col = self.x_col + C
+        self.in_width = self.w_in.shape[0]
+        self.in_ld = -(-self.in_width // 8) * 8
+        # 3: [attention | ssm] . [Wo | W_out]^T
+        self.w_out = torch.cat([attention.out.weight, mamba.out_proj.weight], dim=1).contiguous()
+        biases = [linear.bias for linear in (attention.out, mamba.out_proj) if linear.bias is not None]
+        self.b_out = sum(biases[1:], biases[0]).contiguous() if biases else None
+        self.mixed_width = q_width + E
+        # 4: gate and up rows interleaved in tiles of 8
+        ffn = block.ffn
+        inner = ffn.spec.intermediate_size
+        order = torch.arange(2 * inner, device=device).view(2, inner // 8, 8).permute(1, 0, 2).reshape(-1)
+        self.w_gate_up = ffn.gate_up.weight[order].contiguous()
+        self.b_gate_up = None if ffn.gate_up.bias is None else ffn.gate_up.bias[order].contiguous()
+        self.inner = inner
+        self.position = attention.position
+        self.counters = torch.zeros(64 * a.num_kv_heads, dtype=torch.int32, device=device)
+
+    def supports(self, step, cache) -> bool:
+        a = self.attention.spec
+        return (step.max_query_len == 1 and step.num_tokens <= MAX_ROWS and cache.owns_kv
+                and ops.mixer_decode_supported(a.num_heads, a.num_kv_heads, a.head_dim, cache.k_cache.shape[2],
+                                               self.mamba.spec.state_size))
+
+    def forward(self, residual: Residual, step, caches) -> None:
+        block, a, s = self.block, self.attention.spec, self.mamba.spec
+        kv, state = caches[self.attention_name], caches[self.mamba_name]
+        M = step.num_tokens
+        device = residual.h.device
+        bf16 = torch.bfloat16
+
+        def norm_prologue(norm):
+            pending = residual.pending
+            h_out = torch.empty_like(residual.h) if pending else None
+            arguments = dict(h_in=residual.h, deltas=pending, h_out=h_out, norm_weight=norm.weight, eps=norm.eps)
+            return arguments, h_out
+
+        # 1
+        u = torch.empty((M, self.in_ld), dtype=bf16, device=device)
+        arguments, h_out = norm_prologue(block.mixer_norm)
+        ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=ops.EPI_CONV,
+                       conv=dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=self.mamba.conv_weight,
+                                 bias=self.mamba.conv_bias, state=state.states["conv"], slot_ids=step.slot_ids),
+                       **arguments)
+        if h_out is not None:
+            residual.h, residual.pending = h_out, []
+        # 2
+        mixed = torch.empty((M, self.mixed_width), dtype=bf16, device=device)
+        gated_norm = self.mamba.norm_weight is not None
+        y = torch.empty((M, s.inner_size), dtype=torch.float32, device=device) if gated_norm else None
+        rope = isinstance(self.position, Rope)
+        ops.mixer_decode(
+            u, num_heads=a.num_heads, num_kv_heads=a.num_kv_heads, head_dim=a.head_dim, q_col=self.q_col,
+            k_col=self.k_col, v_col=self.v_col, inv_freq=self.position.inv_freq if rope else None,
+            rotary_dim=self.position.rotary_dim if rope else 0, k_cache=kv.k_cache, v_cache=kv.v_cache,
+            block_tables=step.block_tables[kv.group], positions=step.positions,
+            slot_mapping=step.slot_mappings[kv.group], scale=a.scale, window=a.window, max_seq_len=step.max_seq_len,
+            counters=self.counters, ssm_heads=s.num_heads, ssm_head_dim=s.head_dim, state_size=s.state_size,
+            num_groups=s.num_groups, z_col=self.z_col, x_col=self.x_col, dt_col=self.dt_col,
+            dt_bias=self.mamba.dt_bias, A=self.mamba.A, D=self.mamba.D, ssm_state=state.states["ssm"],
+            slot_ids=step.slot_ids, out=mixed, ssm_y=y)
+        if gated_norm:
+            ops.gate_norm(y, u[:, self.z_col:self.z_col + s.inner_size], self.mamba.norm_weight, s.num_groups,
+                          s.norm_eps, mixed[:, a.num_heads * a.head_dim:])
+        # 3
+        delta = torch.empty((M, self.hidden), dtype=bf16, device=device)
+        ops.fused_gemm(self.w_out, self.b_out, delta, x=mixed)
+        residual.pending = [delta]
+        # 4
+        activated = torch.empty((M, self.inner), dtype=bf16, device=device)
+        arguments, h_out = norm_prologue(block.ffn_norm)
+        ops.fused_gemm(self.w_gate_up, self.b_gate_up, activated, epilogue=ops.EPI_SWIGLU, **arguments)
+        residual.h, residual.pending = h_out, []
+        # 5
+        down = block.ffn.down
+        delta = torch.empty((M, self.hidden), dtype=bf16, device=device)
+        ops.fused_gemm(down.weight, down.bias, delta, x=activated)
+        residual.pending = [delta]
+
+
+def _cat_bias(linears, device):
+    if all(linear.bias is None for linear in linears):
+        return None
+    return torch.cat([torch.zeros(linear.out_features, dtype=torch.float32, device=device)
+                      if linear.bias is None else linear.bias for linear in linears]).contiguous()

@@ -169,7 +169,7 @@ def test_feed_forward_and_norm_parts_alone(dtype):
 
 
 # ------------------------------------------------------------------ generation through the entry points
-@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16")])
+@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
 def test_greedy_generation_through_the_entry_point(tmp_path, name, dtype):
     """The workload of the tiny configurations: prompts of 5/17/33 tokens, 12 greedy steps."""
     from macllm_infer_amd import LLM, EngineConfig, SamplingParams, generate
@@ -232,7 +232,7 @@ def test_toy_parts_register_build_and_step(schedule):
     toy_parts.exercise(schedule, DEV, check_device=True)
 
 
-@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16")])
+@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
 def test_decode_graphs_match_eager_steps(tmp_path, name, dtype):
     """Decode steps replayed from captured graphs, with eager prompt portions of other requests
     and synchronizations between the replays; every replay is compared with the same step of an

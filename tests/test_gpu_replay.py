@@ -46,7 +46,8 @@ def check(steps, out_dir, cfg, tensors, requests, dtype):
                 f"{name}: max error {np.abs(got[name] - want).max():.3e} of scale {np.abs(want).max():.2f}"
 
 
-@pytest.fixture(scope="module", params=[("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16")],
+@pytest.fixture(scope="module", params=[("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16"),
+                                        ("C", "float32"), ("C", "bfloat16")],
                 ids=lambda p: f"{p[0]}-{p[1]}")
 def model(request, tmp_path_factory):
     name, dtype = request.param

@@ -26,7 +26,18 @@ TINY_B = dict(
     attention_out_multiplier=0.8, key_multiplier=0.7, ssm_in_multiplier=1.2, ssm_out_multiplier=0.9,
     ssm_multipliers=[0.8, 1.4, 0.6, 1.5, 1.1], mlp_multipliers=[1.25, 0.75])
 
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1)}
+# Small, but with the head size, state size and widths that the matrix-core and fused decode
+# kernels cover (head_dim 64, widths that are multiples of 32), so that replay runs through them.
+TINY_C = dict(
+    architectures=["FalconH1ForCausalLM"], model_type="falcon_h1",
+    hidden_size=128, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
+    intermediate_size=96, vocab_size=200, max_position_embeddings=640, rms_norm_eps=1e-5, rope_theta=1e6,
+    mamba_n_heads=4, mamba_d_head=16, mamba_d_ssm=64, mamba_d_state=24, mamba_n_groups=1, mamba_d_conv=4,
+    mamba_chunk_size=32, mamba_conv_bias=True, mamba_proj_bias=False, mamba_rms_norm=False,
+    attention_bias=False, mlp_bias=False, tie_word_embeddings=True,
+    embedding_multiplier=1.2, lm_head_multiplier=0.8, key_multiplier=0.9, ssm_multipliers=[1.0, 1.2, 0.9, 1.1, 1.0])
+
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
 
 
 def config(name):
