@@ -468,3 +468,110 @@ extern "C" int mi_decode_attention(const void* q, long q_ld, int T, int Hq, int 
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
+
+// ---------------------------------------------------------------- prefill attention on the matrix cores
+// bfloat16, head_dim 64 or 128.  grid = (query tiles, kv heads, head passes): a tile is up to 64
+// consecutive tokens of one lane; each of the block's four waves takes 16 of them and all the
+// query heads of the kv head (NSET column sets that share every K and V fragment).  Keys run
+// from the first visible one to the tile's last position, read straight from the cache pages
+// (the chunk's own keys were written by rope_kv_store before).
+#include "attn_mfma.h"
+
+template <int DH, int NSET>
+__global__ void __launch_bounds__(256)
+prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hkv, const bf16_t* __restrict__ k_base,
+                         const bf16_t* __restrict__ v_base, long page_stride, int page_size,
+                         const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
+                         const int* __restrict__ cu_seqlens, const int* __restrict__ start_pos, float scale,
+                         int window, bf16_t* __restrict__ out, long out_ld) {
+  const int tile = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const int G = Hq / Hkv;
+  const int head0 = kvh * G + blockIdx.z * NSET;             // first head of this pass
+  const int request = tiles[2 * tile];
+  const int tile_token = tiles[2 * tile + 1];
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wave = threadIdx.x / WAVE;
+  const int qd = lane / 16;
+  const int n = lane % 16;
+  const int lane_end = cu_seqlens[request + 1];
+  const int first_token = tile_token + 16 * wave;
+  if (first_token >= lane_end) return;
+  const int token = first_token + n;
+  const bool has_query = token < lane_end;
+  const int base_position = start_pos[request] - cu_seqlens[request];
+  const int position = base_position + token;
+  const int last_position = base_position + min(first_token + 15, lane_end - 1);
+  const int first_position = base_position + first_token;
+
+  mfma_bf16x8 q_frag[NSET][DH / 32];
+  int col_pos[NSET];
+#pragma unroll
+  for (int s = 0; s < NSET; ++s) {
+    const bool valid = has_query && blockIdx.z * NSET + s < G;
+    col_pos[s] = valid ? position : -1;
+#pragma unroll
+    for (int kk = 0; kk < DH / 32; ++kk) {
+      if (valid) {
+        q_frag[s][kk] = *reinterpret_cast<const mfma_bf16x8*>(q + (long)token * q_ld + (long)(head0 + s) * DH +
+                                                               32 * kk + 8 * qd);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) q_frag[s][kk][j] = (bf16_t)0.f;
+      }
+    }
+  }
+  AttnAccumulator<DH, NSET> acc;
+  acc.clear();
+  AttnCache cache;
+  cache.k_base = k_base;
+  cache.v_base = v_base;
+  cache.page_stride = page_stride;
+  cache.page_size = page_size;
+  cache.kvh = kvh;
+  cache.pages = block_tables + (long)request * max_pages;
+  cache.base_page = 0;
+  int key_lo = 0;
+  if (window > 0 && first_position - window + 1 > 0) key_lo = ((first_position - window + 1) / 32) * 32;
+  attend_keys<DH, NSET, 1>(acc, q_frag, col_pos, window, scale, key_lo, last_position + 1, cache);
+#pragma unroll
+  for (int s = 0; s < NSET; ++s) {
+    const float l = attn_normalizer<DH, NSET>(acc, s);
+    if (col_pos[s] < 0) continue;
+    bf16_t* o = out + (long)token * out_ld + (long)(head0 + s) * DH;
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt) {
+      mfma_bf16x4 packed;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(acc.o[s][dt][i] / l);
+      *reinterpret_cast<mfma_bf16x4*>(o + 16 * dt + 4 * qd) = packed;
+    }
+  }
+}
+
+// tiles: int32 [n_tiles, 2] = (lane, first token row of the tile); a tile never crosses a lane.
+// Returns ERR_UNSUPPORTED_SIZE for shapes it does not cover (the caller uses mi_paged_attention).
+extern "C" int mi_prefill_attention(const void* q, long q_ld, int Hq, int Hkv, int dh, const void* k_base,
+                                    const void* v_base, long page_stride, int page_size, const int* block_tables,
+                                    int max_pages, const int* tiles, int n_tiles, const int* cu_seqlens,
+                                    const int* start_pos, float scale, int window, void* out, long out_ld,
+                                    hipStream_t stream) {
+  if (n_tiles <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || page_size <= 0 || max_pages <= 0)
+    return ERR_BAD_ARGUMENT;
+  const int G = Hq / Hkv;
+  if ((dh != 64 && dh != 128) || page_size % 4 != 0 || q_ld % 8 != 0 || out_ld % 4 != 0 || Hkv > 65535 || G > 64)
+    return ERR_UNSUPPORTED_SIZE;
+  const int passes = (G + 3) / 4;
+  const int nset = (G + passes - 1) / passes;
+  const dim3 grid(n_tiles, Hkv, passes);
+#define PREFILL_CASE(DH_, NSET_)                                                                              \
+  if (dh == DH_ && nset == NSET_)                                                                             \
+    prefill_attention_kernel<DH_, NSET_><<<grid, 256, 0, stream>>>(                                           \
+        (const bf16_t*)q, q_ld, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride, page_size, \
+        block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld);
+  PREFILL_CASE(64, 1) PREFILL_CASE(64, 2) PREFILL_CASE(64, 3) PREFILL_CASE(64, 4)
+  PREFILL_CASE(128, 1) PREFILL_CASE(128, 2) PREFILL_CASE(128, 3) PREFILL_CASE(128, 4)
+#undef PREFILL_CASE
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}

@@ -16,22 +16,21 @@
 //     contiguous in k), then sum their partial tiles through LDS.
 //
 //   mixer_decode : one launch with two kinds of blocks
-//       attention blocks: split-context attention as in attention.hip, with the rotation of q
-//         and of the new key, the write of the new K and V into their cache cell, and the merge
-//         of the splits (by the last block of each (token, kv head) to finish) folded in;
+//       attention blocks: one per (token, kv head): rotation of q and of the new key, the write
+//         of the new K and V into their cache cell, and attention over the request's pages with
+//         an online softmax per wave, merged through LDS;
 //       state-space blocks: one step of the selective scan from and into the slot state, D skip
 //         and the SiLU(z) gate.
 //
 // Formulas and their reference lines are the ones cited in common.hip, attention.hip and
 // mamba2.hip; these kernels only change what runs together.
 #include "common.h"
+#include "attn_mfma.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-#define FG_THREADS 256
-#define FG_WAVES 4
 #define FG_PAD 8
 
 enum { PRO_NORM = 0, PRO_PLAIN = 1 };
@@ -62,8 +61,9 @@ struct FusedGemmParams {
 
 __device__ __forceinline__ float round_bf16(float v) { return (float)(bf16_t)v; }
 
-template <int MT, int PRO, int EPI>
-__global__ void __launch_bounds__(FG_THREADS) fused_gemm_kernel(FusedGemmParams p) {
+template <int MT, int PRO, int EPI, int FG_WAVES>
+__global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmParams p) {
+  constexpr int FG_THREADS = FG_WAVES * WAVE;
   extern __shared__ __align__(16) unsigned char smem[];
   const int K = p.K;
   const int ldx = K + FG_PAD;
@@ -74,91 +74,178 @@ __global__ void __launch_bounds__(FG_THREADS) fused_gemm_kernel(FusedGemmParams 
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
 
+  // the first weight fragments do not depend on anything: request them before the prologue
+  const int n0 = blockIdx.x * 16;
+  const int q = lane / 16;
+  const int r = lane % 16;
+  const int n_row = min(n0 + r, p.N - 1);
+  const bf16_t* w_row = p.W + (long)n_row * K + 8 * q;
+  // wave w takes a contiguous run of k-chunks (of 32), so that its loads cover whole cache lines
+  const int chunks = K / 32;
+  const int per_wave = (chunks + FG_WAVES - 1) / FG_WAVES;
+  const int first_chunk = wave * per_wave;
+  const int iterations = max(0, min(per_wave, chunks - first_chunk));
+  constexpr int BATCH = 8;
+  bf16x8_t a[BATCH];
+  if (iterations > 0) {
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) {
+      const int c = first_chunk + min(j, iterations - 1);
+      a[j] = *reinterpret_cast<const bf16x8_t*>(w_row + c * 32);
+    }
+  }
+  // so does the conv tail of the element this thread finishes in the epilogue (one element per
+  // thread when the block has 16 x 16 outputs)
+  bf16_t tail_values[8];
+  bool tail_ready = false;
+  if (EPI == EPI_CONV && MT == 1 && FG_THREADS == 256 && p.conv_k <= 9) {
+    const int n = n0 + 4 * ((tid % 64) / 16) + (tid / 64);
+    const int m = tid % 16;
+    if (n >= p.conv_lo && n < p.conv_hi && m < p.M) {
+      const int channels = p.conv_hi - p.conv_lo;
+      const bf16_t* tail = p.conv_state + (long)p.slot_ids[m] * (p.conv_k - 1) * channels + (n - p.conv_lo);
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (k < p.conv_k - 1) tail_values[k] = tail[(long)k * channels];
+      tail_ready = true;
+    }
+  }
+
   if (PRO == PRO_NORM) {
-    // one wave per row: sum of squares in float32, then the normalized row in bfloat16
-    for (int m = wave; m < MT * 16; m += FG_WAVES) {
-      bf16_t* x_row = xs + (long)m * ldx;
-      if (m < p.M) {
+    // one wave per row, four rows at a time: the rows are read once into registers (K <= 2048),
+    // their sums of squares reduced in float32, and the normalized rows written in bfloat16
+    constexpr int MAXV = 8;
+    const bool in_registers = K <= MAXV * WAVE * 4;
+    for (int m0 = 0; m0 < MT * 16; m0 += FG_WAVES * 4) {
+      floatx4 v[4][MAXV];
+      if (in_registers) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int m = m0 + wave + t * FG_WAVES;
+          if (m < p.M) {
+            const float* h_row = p.h_in + (long)m * K;
+#pragma unroll
+            for (int i = 0; i < MAXV; ++i) {
+              const int k = lane * 4 + i * WAVE * 4;
+              if (k < K) {
+                v[t][i] = *reinterpret_cast<const floatx4*>(h_row + k);
+                if (p.delta0) {
+                  const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(p.delta0 + (long)m * K + k);
+#pragma unroll
+                  for (int j = 0; j < 4; ++j) v[t][i][j] += (float)d[j];
+                }
+                if (p.delta1) {
+                  const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(p.delta1 + (long)m * K + k);
+#pragma unroll
+                  for (int j = 0; j < 4; ++j) v[t][i][j] += (float)d[j];
+                }
+              }
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int m = m0 + wave + t * FG_WAVES;
+        if (m >= MT * 16) continue;
+        bf16_t* x_row = xs + (long)m * ldx;
+        if (m >= p.M) {
+          for (int k = lane * 4; k < K; k += WAVE * 4) {
+            const bf16x4_t zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+            *reinterpret_cast<bf16x4_t*>(x_row + k) = zero;
+          }
+          continue;
+        }
         const float* h_row = p.h_in + (long)m * K;
-        const bf16_t* d0 = p.delta0 ? p.delta0 + (long)m * K : nullptr;
-        const bf16_t* d1 = p.delta1 ? p.delta1 + (long)m * K : nullptr;
+        auto row_value = [&](int k) {
+          floatx4 value = *reinterpret_cast<const floatx4*>(h_row + k);
+          if (p.delta0) {
+            const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(p.delta0 + (long)m * K + k);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) value[j] += (float)d[j];
+          }
+          if (p.delta1) {
+            const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(p.delta1 + (long)m * K + k);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) value[j] += (float)d[j];
+          }
+          return value;
+        };
         float sum_squares = 0.f;
-        for (int k = lane * 4; k < K; k += WAVE * 4) {
-          floatx4 v = *reinterpret_cast<const floatx4*>(h_row + k);
-          if (d0) {
-            const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(d0 + k);
+        if (in_registers) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] += (float)d[j];
+          for (int i = 0; i < MAXV; ++i)
+            if (lane * 4 + i * WAVE * 4 < K)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) sum_squares += v[t][i][j] * v[t][i][j];
+        } else {
+          for (int k = lane * 4; k < K; k += WAVE * 4) {
+            const floatx4 value = row_value(k);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sum_squares += value[j] * value[j];
           }
-          if (d1) {
-            const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(d1 + k);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] += (float)d[j];
-          }
-#pragma unroll
-          for (int j = 0; j < 4; ++j) sum_squares += v[j] * v[j];
         }
         sum_squares = wave_sum(sum_squares);
-        const float denominator = sqrtf(sum_squares / (float)K + p.eps);
-        for (int k = lane * 4; k < K; k += WAVE * 4) {
-          floatx4 v = *reinterpret_cast<const floatx4*>(h_row + k);
-          if (d0) {
-            const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(d0 + k);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] += (float)d[j];
-          }
-          if (d1) {
-            const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(d1 + k);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] += (float)d[j];
-          }
-          if (blockIdx.x == 0 && p.h_out) *reinterpret_cast<floatx4*>(p.h_out + (long)m * K + k) = v;
+        const float inverse = 1.0f / sqrtf(sum_squares / (float)K + p.eps);
+        auto finish = [&](int k, const floatx4& value) {
+          if (blockIdx.x == 0 && p.h_out) *reinterpret_cast<floatx4*>(p.h_out + (long)m * K + k) = value;
           const floatx4 w = *reinterpret_cast<const floatx4*>(p.norm_w + k);
           bf16x4_t packed;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) packed[j] = (bf16_t)(v[j] / denominator * w[j]);
+          for (int j = 0; j < 4; ++j) packed[j] = (bf16_t)(value[j] * inverse * w[j]);
           *reinterpret_cast<bf16x4_t*>(x_row + k) = packed;
-        }
-      } else {
-        for (int k = lane * 4; k < K; k += WAVE * 4) {
-          bf16x4_t zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
-          *reinterpret_cast<bf16x4_t*>(x_row + k) = zero;
+        };
+        if (in_registers) {
+#pragma unroll
+          for (int i = 0; i < MAXV; ++i) {
+            const int k = lane * 4 + i * WAVE * 4;
+            if (k < K) finish(k, v[t][i]);
+          }
+        } else {
+          for (int k = lane * 4; k < K; k += WAVE * 4) finish(k, row_value(k));
         }
       }
     }
     __syncthreads();
   }
 
-  // the product: wave w takes k-chunks w, w+4, ... of 32
-  const int n0 = blockIdx.x * 16;
-  const int q = lane / 16;
-  const int r = lane % 16;
-  const int n_row = min(n0 + r, p.N - 1);
-  const bf16_t* w_row = p.W + (long)n_row * K + 8 * q;
+  // the product: eight weight fragments are requested before the first is used, so that a
+  // wave keeps eight 1 KiB loads in flight
   floatx4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const int chunks = K / 32;
-  const int iterations = (chunks - wave + FG_WAVES - 1) / FG_WAVES;
-#pragma unroll 4
-  for (int iteration = 0; iteration < iterations; ++iteration) {
-    const int c = wave + iteration * FG_WAVES;
-    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(w_row + c * 32);
+  for (int first = 0; first < iterations; first += BATCH) {
+    if (first > 0) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      bf16x8_t b;
-      if (PRO == PRO_NORM) {
-        b = *reinterpret_cast<const bf16x8_t*>(xs + (long)(mt * 16 + r) * ldx + c * 32 + 8 * q);
-      } else {
-        const int m = mt * 16 + r;
-        if (m < p.M) {
-          b = *reinterpret_cast<const bf16x8_t*>(p.x + (long)m * p.x_ld + c * 32 + 8 * q);
-        } else {
+      for (int j = 0; j < BATCH; ++j) {
+        const int c = first_chunk + min(first + j, iterations - 1);
+        a[j] = *reinterpret_cast<const bf16x8_t*>(w_row + c * 32);
+      }
+    }
+    bf16x8_t b[BATCH][MT];
+    if (PRO == PRO_PLAIN) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) b[j] = (bf16_t)0.f;
+      for (int j = 0; j < BATCH; ++j) {
+        const int c = first_chunk + min(first + j, iterations - 1);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const int m = min(mt * 16 + r, p.M - 1);
+          b[j][mt] = *reinterpret_cast<const bf16x8_t*>(p.x + (long)m * p.x_ld + c * 32 + 8 * q);
         }
       }
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) {
+      if (first + j < iterations) {
+        const int c = first_chunk + first + j;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          bf16x8_t operand;
+          if (PRO == PRO_NORM) operand = *reinterpret_cast<const bf16x8_t*>(xs + (long)(mt * 16 + r) * ldx + c * 32 + 8 * q);
+          else operand = b[j][mt];
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], operand, acc[mt], 0, 0, 0);
+        }
+      }
     }
   }
 #pragma unroll
@@ -191,7 +278,7 @@ __global__ void __launch_bounds__(FG_THREADS) fused_gemm_kernel(FusedGemmParams 
       const bf16_t sample = (bf16_t)v;
       float sum = p.conv_b ? p.conv_b[channel] : 0.f;
       for (int k = 0; k < taps - 1; ++k) {
-        const bf16_t old = tail[(long)k * channels];
+        const bf16_t old = tail_ready ? tail_values[k] : tail[(long)k * channels];
         sum += p.conv_w[channel * taps + k] * (float)old;
         if (k > 0) tail[(long)(k - 1) * channels] = old;       // roll the tail by one
       }
@@ -219,8 +306,10 @@ __global__ void __launch_bounds__(FG_THREADS) fused_gemm_kernel(FusedGemmParams 
   }
 }
 
+static int fused_gemm_waves(int K) { return K / 32 > 32 ? 8 : 4; }   // 8 waves split a long K
+
 static size_t fused_gemm_lds(int MT, int pro, int K) {
-  size_t bytes = (size_t)FG_WAVES * MT * 256 * sizeof(float) + (size_t)16 * MT * 16 * sizeof(float);
+  size_t bytes = (size_t)fused_gemm_waves(K) * MT * 256 * sizeof(float) + (size_t)16 * MT * 16 * sizeof(float);
   if (pro == PRO_NORM) bytes += (size_t)MT * 16 * (K + FG_PAD) * sizeof(bf16_t);
   return bytes;
 }
@@ -229,8 +318,12 @@ template <int MT>
 static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStream_t stream) {
   const int blocks = (p.N + 15) / 16;
   const size_t lds = fused_gemm_lds(MT, pro, p.K);
-#define FG_LAUNCH(PRO_, EPI_) \
-  fused_gemm_kernel<MT, PRO_, EPI_><<<blocks, FG_THREADS, lds, stream>>>(p)
+  const int waves = fused_gemm_waves(p.K);
+#define FG_LAUNCH(PRO_, EPI_)                                                                   \
+  do {                                                                                          \
+    if (waves == 8) fused_gemm_kernel<MT, PRO_, EPI_, 8><<<blocks, 8 * WAVE, lds, stream>>>(p); \
+    else fused_gemm_kernel<MT, PRO_, EPI_, 4><<<blocks, 4 * WAVE, lds, stream>>>(p);            \
+  } while (0)
   if (pro == PRO_NORM && epi == EPI_PLAIN) FG_LAUNCH(PRO_NORM, EPI_PLAIN);
   else if (pro == PRO_NORM && epi == EPI_SWIGLU) FG_LAUNCH(PRO_NORM, EPI_SWIGLU);
   else if (pro == PRO_NORM && epi == EPI_CONV) FG_LAUNCH(PRO_NORM, EPI_CONV);
@@ -302,9 +395,9 @@ extern "C" int mi_fused_gemm_supported(int pro, int M, int K) {
 }
 
 // ---------------------------------------------------------------- mixer decode
-#define MX_THREADS 256
-#define MX_WAVES 4
-#define MX_MAX_SPLIT 512
+#define MX_THREADS 512
+#define MX_WAVES 8
+#define MX_MAX_PAGES 4096
 #define MX_SCAN_PER_THREAD 8
 
 struct MixerParams {
@@ -325,12 +418,9 @@ struct MixerParams {
   const int* positions;
   const int* slot_mapping;
   float scale;
-  int window, split_keys, splits;
-  float* partial_o;
-  float* partial_ml;
-  int* counters;
+  int window;
   // state space
-  int H, P, N, G, R, p_tiles, z_col, x_col, dt_col;
+  int H, P, N, G, R, p_tiles, vector_scan, z_col, x_col, dt_col;
   const float* dt_bias;
   const float* A;
   const float* D;
@@ -344,215 +434,170 @@ struct MixerParams {
   int attention_blocks;
 };
 
-// one dim of a rotated head: pairs (j, j + rotary_dim/2) of the first rotary_dim dims
-__device__ __forceinline__ float rotated_dim(const bf16_t* head, int dim, int rotary_dim, float position,
-                                             const float* inv_freq) {
+// one dim of a rotated head: pairs (j, j + rotary_dim/2) of the first rotary_dim dims;
+// cs holds cos (first half) and sin (second half) of the token's angles, rotary_dim/2 each
+__device__ __forceinline__ float rotated_dim(const bf16_t* head, int dim, int rotary_dim, const float* cs) {
   const float x = (float)head[dim];
   if (dim >= rotary_dim) return x;
   const int half = rotary_dim / 2;
   const int j = dim < half ? dim : dim - half;
-  const float angle = position * inv_freq[j];
-  const float s = sinf(angle), c = cosf(angle);
+  const float c = cs[j], s = cs[half + j];
   return dim < half ? x * c - (float)head[dim + half] * s : x * c + (float)head[dim - half] * s;
 }
 
-template <int DH, int G>
-__device__ void mixer_attention_block(const MixerParams& p, int block, float (*s_lds)[MX_MAX_SPLIT],
-                                      float (*red)[8], float* acc_lds, int* flag) {
-  constexpr int LPR = DH / 8;
-  constexpr int KPW = WAVE / LPR;
-  constexpr int KPB = KPW * MX_WAVES;
-  constexpr int DPL = DH / WAVE;
-  const int split = block % p.splits;
-  const int kvh = (block / p.splits) % p.Hkv;
-  const long token = block / (p.splits * p.Hkv);
-  const int pos = p.positions[token];
-  int first_key = 0;
-  if (p.window > 0 && pos - p.window + 1 > 0) first_key = pos - p.window + 1;
-  const int first_page_key = (first_key / p.page_size) * p.page_size;
-  const int range_lo = first_page_key + split * p.split_keys;
-  if (range_lo > pos) return;
-  const int range_hi = min(range_lo + p.split_keys, pos + 1);
-  const int count = range_hi - range_lo;
-  const int used = min(p.splits, (pos - first_page_key) / p.split_keys + 1);
-  const int* table = p.block_tables + token * p.max_pages;
+// Latency matters more than bandwidth here (a request's K and V for one layer are about a
+// megabyte), and a synchronization between workgroups costs more than the whole read, so one
+// workgroup serves one (token, kv head) alone.  Its waves take contiguous runs of keys and work
+// through them on the matrix cores without talking to each other (attn_mfma.h, with the query
+// heads of the kv head as the columns), and merge once through LDS at the end.  The new
+// token's rotated key and its value are written to their cache cell first, so the run reads
+// them like any other key.
+template <int DH>
+__device__ void mixer_attention_block(const MixerParams& p, int block, int* pages_lds, float* cs,
+                                      float* merge_lds) {
+  const int G = p.Hq / p.Hkv;
+  const int kvh = block % p.Hkv;
+  const long token = block / p.Hkv;
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
-  const int r = lane / LPR;
-  const int c = lane % LPR;
+  const int qd = lane / 16;
+  const int n = lane % 16;
   const bf16_t* row = p.u + token * p.u_ld;
-  const float position = (float)pos;
+  const int* table = p.block_tables + token * p.max_pages;
+  const int half = p.rotary_dim / 2;
 
-  // the block whose range ends at the new token writes its rotated key and its value first
-  if (range_hi == pos + 1) {
+  // ---- round 1: the position, and what does not depend on it
+  const int pos = p.positions[token];
+  mfma_bf16x8 q_own[DH / 32], q_pair[DH / 32];
+  const bool has_head = n < G;
+#pragma unroll
+  for (int kk = 0; kk < DH / 32; ++kk) {
+    const int own_dim = 32 * kk + 8 * qd;
+    const bf16_t* head = row + p.q_col + (kvh * G + (has_head ? n : 0)) * DH;
+    q_own[kk] = *reinterpret_cast<const mfma_bf16x8*>(head + own_dim);
+    if (p.inv_freq && own_dim < p.rotary_dim)
+      q_pair[kk] = *reinterpret_cast<const mfma_bf16x8*>(head + (own_dim < half ? own_dim + half : own_dim - half));
+  }
+  float k_raw = 0.f, k_raw_pair = 0.f, v_raw = 0.f;
+  if (tid < DH) {
+    const bf16_t* k_head = row + p.k_col + kvh * DH;
+    k_raw = (float)k_head[tid];
+    if (p.inv_freq && tid < p.rotary_dim) k_raw_pair = (float)k_head[tid < half ? tid + half : tid - half];
+    v_raw = (float)row[p.v_col + kvh * DH + tid];
+  }
+  if (p.window == 0) {                      // the range starts at key 0: its pages are known already
+    for (int t = tid; t < p.max_pages && t < MX_MAX_PAGES; t += MX_THREADS) pages_lds[t] = table[t];
+  }
+
+  int first_key = 0;
+  if (p.window > 0 && pos - p.window + 1 > 0) first_key = pos - p.window + 1;
+  const int base_key = (first_key / p.page_size) * p.page_size;       // a page edge
+  const int base_page = base_key / p.page_size;
+  if (p.window != 0) {
+    const int last_page = pos / p.page_size;
+    for (int t = tid; t <= last_page - base_page; t += MX_THREADS) pages_lds[t] = table[base_page + t];
+  }
+  if (p.inv_freq) {
+    const float position = (float)pos;
+    for (int j = tid; j < half; j += MX_THREADS) {
+      const float angle = position * p.inv_freq[j];
+      cs[j] = cosf(angle);
+      cs[half + j] = sinf(angle);
+    }
+  }
+  __syncthreads();
+
+  // the new token's key (rotated) and value go to their cache cell
+  if (tid < DH) {
+    float k = k_raw;
+    if (p.inv_freq && tid < p.rotary_dim) {
+      const int j = tid < half ? tid : tid - half;
+      k = tid < half ? k_raw * cs[j] - k_raw_pair * cs[half + j] : k_raw * cs[j] + k_raw_pair * cs[half + j];
+    }
     const long cell = p.slot_mapping[token];
     const long page = cell / p.page_size;
     const int offset = (int)(cell - page * p.page_size);
-    for (int dim = tid; dim < DH; dim += MX_THREADS) {
-      const float k = p.inv_freq ? rotated_dim(row + p.k_col + kvh * DH, dim, p.rotary_dim, position, p.inv_freq)
-                                 : (float)row[p.k_col + kvh * DH + dim];
-      p.k_base[page * p.page_stride + ((long)kvh * p.page_size + offset) * DH + dim] = (bf16_t)k;
-      p.v_base[page * p.page_stride + ((long)kvh * DH + dim) * p.page_size + offset] = row[p.v_col + kvh * DH + dim];
-    }
-    __threadfence_block();
-    __syncthreads();
+    p.k_base[page * p.page_stride + ((long)kvh * p.page_size + offset) * DH + tid] = (bf16_t)k;
+    p.v_base[page * p.page_stride + ((long)kvh * DH + tid) * p.page_size + offset] = (bf16_t)v_raw;
   }
-
-  float qf[G][8];
+  // q: rotated in float32, rounded to bfloat16 as when it is stored
+  mfma_bf16x8 q_frag[1][DH / 32];
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const bf16_t* head = row + p.q_col + (kvh * G + g) * DH;
+  for (int kk = 0; kk < DH / 32; ++kk) {
+    const int own_dim = 32 * kk + 8 * qd;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int dim = c * 8 + j;
-      const float value = p.inv_freq ? rotated_dim(head, dim, p.rotary_dim, position, p.inv_freq) : (float)head[dim];
-      qf[g][j] = round_bf16(value) * p.scale;      // q is rounded to bfloat16 after rotation, as when it is stored
-    }
-  }
-
-  for (int base = 0; base < count; base += KPB) {
-    const int local = base + wave * KPW + r;
-    const int key = range_lo + local;
-    const bool valid = local < count;
-    float s[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) s[g] = 0.f;
-    if (valid) {
-      const int page = table[key / p.page_size];
-      const int offset = key % p.page_size;
-      const bf16x8_t packed = *reinterpret_cast<const bf16x8_t*>(
-          p.k_base + (long)page * p.page_stride + ((long)kvh * p.page_size + offset) * DH + c * 8);
-#pragma unroll
-      for (int g = 0; g < G; ++g)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) s[g] = fmaf(qf[g][j], (float)packed[j], s[g]);
-    }
-#pragma unroll
-    for (int offset = LPR / 2; offset > 0; offset >>= 1)
-#pragma unroll
-      for (int g = 0; g < G; ++g) s[g] += __shfl_xor(s[g], offset, WAVE);
-    if (valid && c == 0) {
-#pragma unroll
-      for (int g = 0; g < G; ++g) s_lds[g][local] = key >= first_key ? s[g] : -INFINITY;
-    }
-  }
-  __syncthreads();
-
-  float m[G], l[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float v = -INFINITY;
-    for (int i = tid; i < count; i += MX_THREADS) v = fmaxf(v, s_lds[g][i]);
-    v = wave_max(v);
-    if (lane == 0) red[wave][g] = v;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float v = red[0][g];
-#pragma unroll
-    for (int w = 1; w < MX_WAVES; ++w) v = fmaxf(v, red[w][g]);
-    m[g] = v;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float sum = 0.f;
-    for (int i = tid; i < count; i += MX_THREADS) {
-      const float e = __expf(s_lds[g][i] - m[g]);
-      s_lds[g][i] = e;
-      sum += e;
-    }
-    sum = wave_sum(sum);
-    if (lane == 0) red[wave][g] = sum;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float v = 0.f;
-#pragma unroll
-    for (int w = 0; w < MX_WAVES; ++w) v += red[w][g];
-    l[g] = v;
-  }
-
-  float acc[G][DPL];
-#pragma unroll
-  for (int g = 0; g < G; ++g)
-#pragma unroll
-    for (int i = 0; i < DPL; ++i) acc[g][i] = 0.f;
-  const int range_pages = (count + p.page_size - 1) / p.page_size;
-  for (int pg = wave; pg < range_pages; pg += MX_WAVES) {
-    const int local0 = pg * p.page_size;
-    const int page = table[(range_lo + local0) / p.page_size];
-    const int keys_here = min(p.page_size, count - local0);
-#pragma unroll
-    for (int i = 0; i < DPL; ++i) {
-      const int dim = lane + i * WAVE;
-      const bf16_t* v_row = p.v_base + (long)page * p.page_stride + ((long)kvh * DH + dim) * p.page_size;
-      for (int j0 = 0; j0 < keys_here; j0 += 8) {
-        const bf16x8_t packed = *reinterpret_cast<const bf16x8_t*>(v_row + j0);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          if (j0 + j < keys_here) {
-            const float value = (float)packed[j];
-#pragma unroll
-            for (int g = 0; g < G; ++g) acc[g][i] = fmaf(s_lds[g][local0 + j0 + j], value, acc[g][i]);
-          }
-        }
+      float value = (float)q_own[kk][j];
+      if (p.inv_freq && own_dim < p.rotary_dim) {
+        const int dim = own_dim + j;
+        const int f = dim < half ? dim : dim - half;
+        value = dim < half ? value * cs[f] - (float)q_pair[kk][j] * cs[half + f]
+                           : value * cs[f] + (float)q_pair[kk][j] * cs[half + f];
       }
+      q_frag[0][kk][j] = has_head ? (bf16_t)value : (bf16_t)0.f;
     }
   }
-#pragma unroll
-  for (int g = 0; g < G; ++g)
-#pragma unroll
-    for (int i = 0; i < DPL; ++i) acc_lds[(wave * G + g) * DH + lane + i * WAVE] = acc[g][i];
+  __threadfence_block();
   __syncthreads();
-  const long head0 = token * p.Hq + kvh * G;
-  for (int index = tid; index < G * DH; index += MX_THREADS) {
-    const int g = index / DH;
-    const int dim = index - g * DH;
-    float sum = 0.f;
-#pragma unroll
-    for (int w = 0; w < MX_WAVES; ++w) sum += acc_lds[(w * G + g) * DH + dim];
-    p.partial_o[((head0 + g) * p.splits + split) * DH + dim] = sum;
-  }
-  if (tid < G) {
-    float* ml = p.partial_ml + ((head0 + tid) * p.splits + split) * 2;
-    ml[0] = m[tid];
-    ml[1] = l[tid];
+
+  // ---- this wave's run of keys
+  const int total = pos + 1 - base_key;
+  int span = (total + MX_WAVES - 1) / MX_WAVES;
+  span = ((span + 63) / 64) * 64;
+  const int wave_lo = base_key + wave * span;
+  const int wave_hi = min(wave_lo + span, pos + 1);
+  AttnAccumulator<DH, 1> acc;
+  acc.clear();
+  if (wave_lo <= pos) {
+    AttnCache cache;
+    cache.k_base = p.k_base;
+    cache.v_base = p.v_base;
+    cache.page_stride = p.page_stride;
+    cache.page_size = p.page_size;
+    cache.kvh = kvh;
+    cache.pages = pages_lds;
+    cache.base_page = base_page;
+    const int col_pos[1] = {has_head ? pos : -1};
+    attend_keys<DH, 1, 2>(acc, q_frag, col_pos, p.window, p.scale, wave_lo, wave_hi, cache);
   }
 
-  // the last block of this (token, kv head) to get here merges the splits
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) {
-    int* counter = p.counters + token * p.Hkv + kvh;
-    const int arrived = atomicAdd(counter, 1);
-    *flag = (arrived == used - 1) ? 1 : 0;
-    if (arrived == used - 1) *counter = 0;          // left at zero for the next step
+  // ---- merge the waves: merge_lds[wave][head] = {m, l, o[DH]}
+  const float l = attn_normalizer<DH, 1>(acc, 0);
+  if (has_head) {
+    float* mine = merge_lds + (long)(wave * G + n) * (DH + 2);
+    if (qd == 0) {
+      mine[0] = acc.m[0];
+      mine[1] = l;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mine[2 + 16 * dt + 4 * qd + i] = acc.o[0][dt][i];
   }
   __syncthreads();
-  if (*flag == 0) return;
-  __threadfence();
   for (int index = tid; index < G * DH; index += MX_THREADS) {
     const int g = index / DH;
     const int dim = index - g * DH;
-    const float* ml = p.partial_ml + (head0 + g) * p.splits * 2;
-    const float* o = p.partial_o + (head0 + g) * (long)p.splits * DH;
     float maximum = -INFINITY;
-    for (int s = 0; s < used; ++s) maximum = fmaxf(maximum, ml[2 * s]);
+#pragma unroll
+    for (int w = 0; w < MX_WAVES; ++w) maximum = fmaxf(maximum, merge_lds[(long)(w * G + g) * (DH + 2)]);
     float denominator = 0.f, sum = 0.f;
-    for (int s = 0; s < used; ++s) {
-      const float weight = __expf(ml[2 * s] - maximum);
-      denominator += weight * ml[2 * s + 1];
-      sum += weight * o[(long)s * DH + dim];
+#pragma unroll
+    for (int w = 0; w < MX_WAVES; ++w) {
+      const float* theirs = merge_lds + (long)(w * G + g) * (DH + 2);
+      const float weight = __expf(theirs[0] - maximum);      // 0 for a wave without keys (m = -inf)
+      denominator += weight * theirs[1];
+      sum += weight * theirs[2 + dim];
     }
     p.attn_out[token * p.out_ld + (long)(kvh * G + g) * DH + dim] = (bf16_t)(sum / denominator);
   }
 }
 
 // One step of the selective scan for (token, head, tile of state rows); see ssm_scan_kernel.
+// A state row of N floats is shared by R lanes.  When N is 8*R (VECTOR) each lane owns 8
+// consecutive elements: two 16-byte state loads and one 16-byte load each of B and C.
+template <bool VECTOR>
 __device__ void mixer_ssm_block(const MixerParams& p, int block) {
   const int tile = block % p.p_tiles;
   const int head = (block / p.p_tiles) % p.H;
@@ -574,13 +619,32 @@ __device__ void mixer_ssm_block(const MixerParams& p, int block) {
   const bf16_t* c_row = b_row + p.G * N;
   const float dx = delta * x;
   float partial = 0.f;
+  if (VECTOR) {
+    if (active) {
+      floatx4 s0 = *reinterpret_cast<const floatx4*>(s_row + r * 8);
+      floatx4 s1 = *reinterpret_cast<const floatx4*>(s_row + r * 8 + 4);
+      const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(b_row + r * 8);
+      const bf16x8_t c = *reinterpret_cast<const bf16x8_t*>(c_row + r * 8);
 #pragma unroll
-  for (int i = 0; i < MX_SCAN_PER_THREAD; ++i) {
-    const int n = r + i * R;
-    if (active && n < N) {
-      const float next = decay * s_row[n] + dx * (float)b_row[n];
-      s_row[n] = next;
-      partial += next * (float)c_row[n];
+      for (int i = 0; i < 4; ++i) {
+        s0[i] = decay * s0[i] + dx * (float)b[i];
+        s1[i] = decay * s1[i] + dx * (float)b[4 + i];
+        partial += s0[i] * (float)c[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) partial += s1[i] * (float)c[4 + i];
+      *reinterpret_cast<floatx4*>(s_row + r * 8) = s0;
+      *reinterpret_cast<floatx4*>(s_row + r * 8 + 4) = s1;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < MX_SCAN_PER_THREAD; ++i) {
+      const int n = r + i * R;
+      if (active && n < N) {
+        const float next = decay * s_row[n] + dx * (float)b_row[n];
+        s_row[n] = next;
+        partial += next * (float)c_row[n];
+      }
     }
   }
   for (int offset = R / 2; offset > 0; offset >>= 1) partial += __shfl_xor(partial, offset, WAVE);
@@ -592,32 +656,34 @@ __device__ void mixer_ssm_block(const MixerParams& p, int block) {
   }
 }
 
-template <int DH, int G>
+template <int DH>
 __global__ void __launch_bounds__(MX_THREADS) mixer_decode_kernel(MixerParams p) {
-  __shared__ float s_lds[G][MX_MAX_SPLIT];
-  __shared__ float red[MX_WAVES][8];
-  __shared__ float acc_lds[MX_WAVES * G * DH];
-  __shared__ int flag;
+  __shared__ int pages_lds[MX_MAX_PAGES];
+  __shared__ float cs[DH];
+  __shared__ float merge_lds[MX_WAVES * 8 * (DH + 2)];
   if ((int)blockIdx.x < p.attention_blocks)
-    mixer_attention_block<DH, G>(p, blockIdx.x, s_lds, red, acc_lds, &flag);
+    mixer_attention_block<DH>(p, blockIdx.x, pages_lds, cs, merge_lds);
+  else if (p.vector_scan)
+    mixer_ssm_block<true>(p, blockIdx.x - p.attention_blocks);
   else
-    mixer_ssm_block(p, blockIdx.x - p.attention_blocks);
+    mixer_ssm_block<false>(p, blockIdx.x - p.attention_blocks);
 }
 
 extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv, int dh, int q_col, int k_col,
                                int v_col, const float* inv_freq, int rotary_dim, void* k_base, void* v_base,
                                long page_stride, int page_size, const int* block_tables, int max_pages,
                                const int* positions, const int* slot_mapping, float scale, int window,
-                               int split_keys, int splits, float* partial_o, float* partial_ml, int* counters,
-                               int H, int P, int N, int G, int z_col, int x_col, int dt_col, const float* dt_bias,
+                               int max_seq_len, int H, int P, int N, int G, int z_col, int x_col, int dt_col, const float* dt_bias,
                                const float* A, const float* D, float* ssm_state, const int* slot_ids,
                                void* attn_out, void* ssm_out, float* ssm_y, long out_ld, hipStream_t stream) {
   if (M <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || H <= 0 || P <= 0 || N <= 0 || G <= 0 || H % G != 0)
     return ERR_BAD_ARGUMENT;
   const int group = Hq / Hkv;
-  if ((dh != 64 && dh != 128) || group > 8 || page_size % 8 != 0 || split_keys % page_size != 0 ||
-      split_keys <= 0 || split_keys > MX_MAX_SPLIT || splits <= 0 || N > WAVE * MX_SCAN_PER_THREAD ||
-      u_ld % 8 != 0 || q_col % 8 != 0 || rotary_dim > dh || (rotary_dim & 1))
+  // the page ids of a request's whole visible range are staged in LDS
+  const long span = window > 0 ? (long)window + page_size : (long)max_seq_len;
+  if ((dh != 64 && dh != 128) || group > 8 || page_size % 8 != 0 || max_seq_len <= 0 ||
+      span / page_size + 2 > MX_MAX_PAGES || N > WAVE * MX_SCAN_PER_THREAD ||
+      u_ld % 8 != 0 || q_col % 8 != 0 || rotary_dim > dh || rotary_dim % 16 != 0)
     return ERR_UNSUPPORTED_SIZE;
   MixerParams p;
   p.u = (const bf16_t*)u;
@@ -640,18 +706,23 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
   p.slot_mapping = slot_mapping;
   p.scale = scale;
   p.window = window;
-  p.split_keys = split_keys;
-  p.splits = splits;
-  p.partial_o = partial_o;
-  p.partial_ml = partial_ml;
-  p.counters = counters;
   p.H = H;
   p.P = P;
   p.N = N;
   p.G = G;
+  // a state row is shared by R lanes: N/8 of them with 8 consecutive elements each when N is
+  // 8 times a power of two (and the rows of B and C are 16-byte aligned), else up to 64 with
+  // strided elements
   int R = 1;
-  while (R < N && R < WAVE) R <<= 1;
+  const bool vector_scan = N % 8 == 0 && ((N / 8) & (N / 8 - 1)) == 0 && N / 8 <= WAVE &&
+                           (x_col + H * P) % 8 == 0;
+  if (vector_scan) {
+    R = N / 8;
+  } else {
+    while (R < N && R < WAVE) R <<= 1;
+  }
   p.R = R;
+  p.vector_scan = vector_scan ? 1 : 0;
   const int rows_per_block = MX_THREADS / R;
   p.p_tiles = (P + rows_per_block - 1) / rows_per_block;
   p.z_col = z_col;
@@ -666,15 +737,11 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
   p.ssm_out = (bf16_t*)ssm_out;
   p.ssm_y = ssm_y;
   p.out_ld = out_ld;
-  p.attention_blocks = splits * Hkv * M;
+  p.attention_blocks = Hkv * M;
   const long total = (long)p.attention_blocks + (long)p.p_tiles * H * M;
   if (total > 0x7fffffffL) return ERR_UNSUPPORTED_SIZE;
-#define MX_CASE(DH_, G_) \
-  if (dh == DH_ && group == G_) mixer_decode_kernel<DH_, G_><<<(unsigned)total, MX_THREADS, 0, stream>>>(p);
-  MX_CASE(64, 1) MX_CASE(64, 2) MX_CASE(64, 3) MX_CASE(64, 4) MX_CASE(64, 5) MX_CASE(64, 6) MX_CASE(64, 7)
-  MX_CASE(64, 8) MX_CASE(128, 1) MX_CASE(128, 2) MX_CASE(128, 3) MX_CASE(128, 4) MX_CASE(128, 5)
-  MX_CASE(128, 6) MX_CASE(128, 7) MX_CASE(128, 8)
-#undef MX_CASE
+  if (dh == 64) mixer_decode_kernel<64><<<(unsigned)total, MX_THREADS, 0, stream>>>(p);
+  else mixer_decode_kernel<128><<<(unsigned)total, MX_THREADS, 0, stream>>>(p);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

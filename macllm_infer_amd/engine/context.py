@@ -19,6 +19,9 @@ import numpy as np
 import torch
 
 
+QUERY_TILE = 64        # tokens of one lane that one workgroup of the prefill attention kernel takes
+
+
 @dataclass
 class Lane:
     request: Hashable
@@ -38,6 +41,7 @@ class StepContext:
     seq_lens: torch.Tensor           # [lanes] request length after the step
     slot_ids: torch.Tensor           # [lanes] state slot of each lane's request
     want_rows: torch.Tensor          # [wanted] token rows whose logits are returned
+    query_tiles: torch.Tensor        # [tiles, 2] (lane, first token row) of runs of up to 64 tokens of one lane
     block_tables: List[torch.Tensor] = field(default_factory=list)   # per group [lanes, max_pages]
     slot_mappings: List[torch.Tensor] = field(default_factory=list)  # per group [T] page*page_size+offset
     lane_lengths: List[int] = field(default_factory=list)            # host copies
@@ -66,7 +70,9 @@ def _pack(lanes: Sequence[Lane], cache, pad_lanes: int = 0, max_pages: Optional[
                           + [cache.scratch_slot] * pad_lanes, dtype=np.int32)
     want_rows = np.asarray([cu[index] + place for index, lane in enumerate(lanes) for place in lane.want],
                            dtype=np.int32)
-    sections = [token_ids, positions, lane_of_token, cu, start_pos, seq_lens, slot_ids, want_rows]
+    tiles = np.asarray([(index, row) for index in range(Ln) for row in range(cu[index], cu[index + 1], QUERY_TILE)],
+                       dtype=np.int32).reshape(-1)
+    sections = [token_ids, positions, lane_of_token, cu, start_pos, seq_lens, slot_ids, want_rows, tiles]
     group_shapes = []
     for group in cache.groups:
         page_size = group.page_size
@@ -88,11 +94,11 @@ def _assemble(views, group_shapes, lengths, starts, max_seq_len) -> StepContext:
     context = StepContext(
         num_tokens=sum(lengths), num_lanes=len(lengths), token_ids=views[0], positions=views[1],
         lane_of_token=views[2], cu_seqlens=views[3], start_pos=views[4], seq_lens=views[5], slot_ids=views[6],
-        want_rows=views[7], lane_lengths=list(lengths), lane_starts=list(starts), max_query_len=max(lengths),
+        want_rows=views[7], query_tiles=views[8].view(-1, 2), lane_lengths=list(lengths), lane_starts=list(starts), max_query_len=max(lengths),
         max_seq_len=max_seq_len)
     for index, shape in enumerate(group_shapes):
-        context.slot_mappings.append(views[8 + 2 * index])
-        context.block_tables.append(views[9 + 2 * index].view(shape))
+        context.slot_mappings.append(views[9 + 2 * index])
+        context.block_tables.append(views[10 + 2 * index].view(shape))
     return context
 
 

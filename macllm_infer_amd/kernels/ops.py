@@ -40,6 +40,8 @@ _SIGNATURES = {
                              _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr],
         "mi_paged_attention": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
                                _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_long, _c_ptr],
+        "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
+                                 _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_long, _c_ptr],
         "mi_decode_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int,
                                 _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
                                 _c_ptr, _c_long, _c_ptr],
@@ -64,8 +66,8 @@ _SIGNATURES = {
         "mi_fused_gemm_supported": [_c_int, _c_int, _c_int],
         "mi_mixer_decode": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int,
                             _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int,
-                            _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                            _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr],
+                            _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                            _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr],
     },
     "sampling": {
         "mi_apply_penalties": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
@@ -295,6 +297,40 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
         int(window or 0), _p(out), out_ld, _stream()), "paged_attention", f"(head_dim={head_dim})")
 
 
+def prefill_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> bool:
+    """Whether the matrix-core attention kernel covers this geometry."""
+    return (dtype == torch.bfloat16 and head_dim in (64, 128) and page_size % 4 == 0
+            and num_heads // num_kv_heads <= 64)
+
+
+def prefill_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_cache: torch.Tensor,
+                      v_cache: torch.Tensor, block_tables: torch.Tensor, query_tiles: torch.Tensor,
+                      cu_seqlens: torch.Tensor, start_pos: torch.Tensor, scale: float, window: Optional[int],
+                      out: torch.Tensor) -> None:
+    """``paged_attention`` on the matrix cores for bfloat16 (flash-style, online softmax in
+    float32).  ``query_tiles`` [tiles, 2]: (lane, first token row) of runs of up to 64 tokens of
+    one lane; the keys and values of the step's own tokens must be in the cache already."""
+    q_ld = _row_major(q, "q")
+    out_ld = _row_major(out, "out")
+    T = q.shape[0]
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "prefill_attention: bfloat16 only")
+    _need(q.shape[1] >= num_heads * head_dim and out.shape == (T, num_heads * head_dim) and q_ld % 8 == 0
+          and q.data_ptr() % 16 == 0 and out_ld % 4 == 0 and out.data_ptr() % 8 == 0,
+          "prefill_attention: q/out shapes or alignment do not fit")
+    page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, q.dtype)
+    _need(prefill_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim, page_size),
+          "prefill_attention: geometry not covered; use paged_attention")
+    for name, tensor in (("block_tables", block_tables), ("query_tiles", query_tiles), ("cu_seqlens", cu_seqlens),
+                         ("start_pos", start_pos)):
+        _i32(tensor, name)
+    _need(block_tables.dim() == 2 and query_tiles.dim() == 2 and query_tiles.shape[1] == 2
+          and cu_seqlens.numel() == start_pos.numel() + 1, "prefill_attention: metadata shapes do not match")
+    _check(_fn("attention", "mi_prefill_attention")(
+        _p(q), q_ld, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride, page_size,
+        _p(block_tables), block_tables.shape[1], _p(query_tiles), query_tiles.shape[0], _p(cu_seqlens),
+        _p(start_pos), float(scale), int(window or 0), _p(out), out_ld, _stream()), "prefill_attention")
+
+
 def decode_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> bool:
     """Whether the split-context kernel for single-token queries covers this geometry."""
     return (dtype == torch.bfloat16 and head_dim in (64, 128) and num_heads // num_kv_heads <= 8
@@ -485,16 +521,18 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
         _p(slot_ids), _stream()), "fused_gemm", f"(M={M}, N={N}, K={K})")
 
 
-def mixer_decode_supported(num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, state_size: int) -> bool:
-    return (head_dim in (64, 128) and num_heads // num_kv_heads <= 8 and page_size % 8 == 0 and page_size <= 512
-            and state_size <= 512)
+def mixer_decode_supported(num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, state_size: int,
+                           max_seq_len: int = 1, window: Optional[int] = None, rotary_dim: int = 0) -> bool:
+    span = max_seq_len if not window else window + page_size
+    return (head_dim in (64, 128) and num_heads // num_kv_heads <= 8 and page_size % 8 == 0 and state_size <= 512
+            and span // page_size + 2 <= 4096 and rotary_dim % 16 == 0)
 
 
 def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int, q_col: int, k_col: int,
                  v_col: int, inv_freq: Optional[torch.Tensor], rotary_dim: int, k_cache: torch.Tensor,
                  v_cache: torch.Tensor, block_tables: torch.Tensor, positions: torch.Tensor,
                  slot_mapping: torch.Tensor, scale: float, window: Optional[int], max_seq_len: int,
-                 counters: torch.Tensor, ssm_heads: int, ssm_head_dim: int, state_size: int, num_groups: int,
+                 ssm_heads: int, ssm_head_dim: int, state_size: int, num_groups: int,
                  z_col: int, x_col: int, dt_col: int, dt_bias: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
                  ssm_state: torch.Tensor, slot_ids: torch.Tensor, out: torch.Tensor,
                  ssm_y: Optional[torch.Tensor]) -> None:
@@ -503,7 +541,7 @@ def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim
     the new K/V into the cache cell ``slot_mapping``, attends over the request's pages, writes
     ``out[:, :Hq*dh]``.  State space: one scan step from and into ``ssm_state[slot_ids]``, writes
     ``y * SiLU(z)`` to ``out[:, Hq*dh:]``, or float32 ``y`` to ``ssm_y`` when a grouped norm
-    follows.  ``counters``: int32 zeros [>= M*Hkv], left at zero."""
+    follows.  ``max_seq_len``: an upper bound of the longest context in the batch."""
     u_ld = _row_major(u, "u")
     out_ld = _row_major(out, "out")
     M = u.shape[0]
@@ -511,14 +549,13 @@ def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim
     _need(u.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and out.shape == (M, num_heads * head_dim + E),
           "mixer_decode: u/out shapes do not match")
     page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, u.dtype)
-    _need(mixer_decode_supported(num_heads, num_kv_heads, head_dim, page_size, state_size),
-          "mixer_decode: geometry not covered")
+    _need(mixer_decode_supported(num_heads, num_kv_heads, head_dim, page_size, state_size, max_seq_len, window,
+                                 rotary_dim if inv_freq is not None else 0), "mixer_decode: geometry not covered")
     for name, tensor in (("block_tables", block_tables), ("positions", positions), ("slot_mapping", slot_mapping),
-                         ("slot_ids", slot_ids), ("counters", counters)):
+                         ("slot_ids", slot_ids)):
         _i32(tensor, name)
     _need(block_tables.dim() == 2 and block_tables.shape[0] >= M and positions.numel() == M
-          and slot_mapping.numel() == M and slot_ids.numel() == M and counters.numel() >= M * num_kv_heads,
-          "mixer_decode: metadata shapes do not match")
+          and slot_mapping.numel() == M and slot_ids.numel() == M, "mixer_decode: metadata shapes do not match")
     _need(ssm_state.dtype == torch.float32 and ssm_state.shape[1:] == (ssm_heads, ssm_head_dim, state_size)
           and ssm_state.is_contiguous(), "mixer_decode: bad state")
     for name, vector in (("dt_bias", dt_bias), ("A", A), ("D", D)):
@@ -528,20 +565,12 @@ def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim
     widest = max(q_col + num_heads * head_dim, k_col + num_kv_heads * head_dim, v_col + num_kv_heads * head_dim,
                  z_col + E, x_col + E + 2 * num_groups * state_size, dt_col + ssm_heads)
     _need(u.shape[1] >= widest, "mixer_decode: u is too narrow")
-    span = max_seq_len if not window else min(max_seq_len, window + page_size)
-    split_keys = 64
-    while split_keys < 512 and span * M * num_kv_heads > 1024 * split_keys:
-        split_keys *= 2
-    split_keys = max(split_keys, page_size)
-    splits = max(1, -(-span // split_keys))
-    partial_o = torch.empty((M, num_heads, splits, head_dim), dtype=torch.float32, device=u.device)
-    partial_ml = torch.empty((M, num_heads, splits, 2), dtype=torch.float32, device=u.device)
     _check(_fn("decode", "mi_mixer_decode")(
         _p(u), u_ld, M, num_heads, num_kv_heads, head_dim, q_col, k_col, v_col, _p(inv_freq), rotary_dim,
         _p(k_cache), _p(v_cache), page_stride, page_size, _p(block_tables), block_tables.shape[1], _p(positions),
-        _p(slot_mapping), float(scale), int(window or 0), split_keys, splits, _p(partial_o), _p(partial_ml),
-        _p(counters), ssm_heads, ssm_head_dim, state_size, num_groups, z_col, x_col, dt_col, _p(dt_bias), _p(A),
-        _p(D), _p(ssm_state), _p(slot_ids), _p(out), out.data_ptr() + 2 * num_heads * head_dim,
+        _p(slot_mapping), float(scale), int(window or 0), int(max_seq_len), ssm_heads, ssm_head_dim, state_size,
+        num_groups, z_col, x_col, dt_col, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(slot_ids), _p(out),
+        out.data_ptr() + 2 * num_heads * head_dim,
         _p(ssm_y), out_ld, _stream()), "mixer_decode")
 
 

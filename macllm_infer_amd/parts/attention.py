@@ -73,6 +73,10 @@ class Attention(Mixer):
             ops.decode_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                  step.lane_of_token, step.positions, spec.scale, spec.window, step.max_seq_len,
                                  attended)
+        elif ops.prefill_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2]):
+            ops.prefill_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                  step.query_tiles, step.cu_seqlens, step.start_pos, spec.scale, spec.window,
+                                  attended)
         else:
             ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                 step.lane_of_token, step.positions, spec.scale, spec.window, attended)

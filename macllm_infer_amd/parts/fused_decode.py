@@ -92,13 +92,13 @@ class ParallelDecodeFusion:
         self.b_gate_up = None if ffn.gate_up.bias is None else ffn.gate_up.bias[order].contiguous()
         self.inner = inner
         self.position = attention.position
-        self.counters = torch.zeros(64 * a.num_kv_heads, dtype=torch.int32, device=device)
 
     def supports(self, step, cache) -> bool:
         a = self.attention.spec
+        rotary = self.position.rotary_dim if isinstance(self.position, Rope) else 0
         return (step.max_query_len == 1 and step.num_tokens <= MAX_ROWS and cache.owns_kv
                 and ops.mixer_decode_supported(a.num_heads, a.num_kv_heads, a.head_dim, cache.k_cache.shape[2],
-                                               self.mamba.spec.state_size))
+                                               self.mamba.spec.state_size, step.max_seq_len, a.window, rotary))
 
     def forward(self, residual: Residual, step, caches) -> None:
         block, a, s = self.block, self.attention.spec, self.mamba.spec
@@ -133,7 +133,7 @@ class ParallelDecodeFusion:
             rotary_dim=self.position.rotary_dim if rope else 0, k_cache=kv.k_cache, v_cache=kv.v_cache,
             block_tables=step.block_tables[kv.group], positions=step.positions,
             slot_mapping=step.slot_mappings[kv.group], scale=a.scale, window=a.window, max_seq_len=step.max_seq_len,
-            counters=self.counters, ssm_heads=s.num_heads, ssm_head_dim=s.head_dim, state_size=s.state_size,
+            ssm_heads=s.num_heads, ssm_head_dim=s.head_dim, state_size=s.state_size,
             num_groups=s.num_groups, z_col=self.z_col, x_col=self.x_col, dt_col=self.dt_col,
             dt_bias=self.mamba.dt_bias, A=self.mamba.A, D=self.mamba.D, ssm_state=state.states["ssm"],
             slot_ids=step.slot_ids, out=mixed, ssm_y=y)

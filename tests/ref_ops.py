@@ -104,6 +104,10 @@ def decode_attention_supported(dtype, num_heads, num_kv_heads, head_dim, page_si
     return False
 
 
+def prefill_attention_supported(dtype, num_heads, num_kv_heads, head_dim, page_size):
+    return False
+
+
 def decode_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token, positions,
                      scale, window, max_seq_len, out):
     paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token, positions,
@@ -170,7 +174,7 @@ def argmax(logits, out):
     out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
 
 
-NAMES = ["decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "linear", "rope_kv_store", "paged_attention",
+NAMES = ["prefill_attention_supported", "decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "linear", "rope_kv_store", "paged_attention",
          "conv1d_silu", "conv_state_update", "ssm_scan", "gate_norm", "argmax"]
 
 
@@ -215,7 +219,8 @@ def fused_gemm_supported(normed, rows, in_features):
     return False
 
 
-def mixer_decode_supported(num_heads, num_kv_heads, head_dim, page_size, state_size):
+def mixer_decode_supported(num_heads, num_kv_heads, head_dim, page_size, state_size, max_seq_len=1, window=None,
+                           rotary_dim=0):
     return False
 
 
@@ -257,7 +262,7 @@ def fused_gemm(weight, bias, out, *, out_scale=1.0, x=None, h_in=None, deltas=()
 
 
 def mixer_decode(u, *, num_heads, num_kv_heads, head_dim, q_col, k_col, v_col, inv_freq, rotary_dim, k_cache, v_cache,
-                 block_tables, positions, slot_mapping, scale, window, max_seq_len, counters, ssm_heads, ssm_head_dim,
+                 block_tables, positions, slot_mapping, scale, window, max_seq_len, ssm_heads, ssm_head_dim,
                  state_size, num_groups, z_col, x_col, dt_col, dt_bias, A, D, ssm_state, slot_ids, out, ssm_y):
     M = u.shape[0]
     q_width, kv_width = num_heads * head_dim, num_kv_heads * head_dim

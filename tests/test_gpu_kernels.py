@@ -502,7 +502,7 @@ def test_fused_gemm_norm_prologue_and_epilogues(ops, M, N, K, deltas):
 def test_mixer_decode_against_the_separate_kernels(ops, Hq, Hkv, dh, H, P, N, G, page_size, window, rotary, gated):
     """Both mixers of a decode step in one launch, for requests with contexts of 1 to 1 500
     tokens; compared with the composition of the plain references, cache and state included.
-    Twice in a row: the split counters must be back at zero."""
+    Twice in a row on fresh copies of the cache and state."""
     dtype = torch.bfloat16
     lengths = [1, 17, 64, 65, 300, 1500, 2]
     M = len(lengths)
@@ -531,11 +531,10 @@ def test_mixer_decode_against_the_separate_kernels(ops, Hq, Hkv, dh, H, P, N, G,
     want_out = torch.zeros(M, Hq * dh + E, dtype=dtype)
     want_y = torch.empty(M, E) if gated else None
     ref_ops.mixer_decode(u, inv_freq=inv_freq, k_cache=views(want_pool, page_size)[0], v_cache=views(want_pool, page_size)[1],
-                         block_tables=table, positions=positions, slot_mapping=slot_mapping, counters=None,
+                         block_tables=table, positions=positions, slot_mapping=slot_mapping,
                          dt_bias=dt_bias, A=A, D=D, ssm_state=want_state, slot_ids=slot_ids, out=want_out, ssm_y=want_y,
                          **common)
-    assert ops.mixer_decode_supported(Hq, Hkv, dh, page_size, N)
-    counters = torch.zeros(M * Hkv, dtype=torch.int32, device=DEV)
+    assert ops.mixer_decode_supported(Hq, Hkv, dh, page_size, N, 2048, window, rotary)
     for repeat in range(2):
         got_pool, got_state = pool.clone().to(DEV), state.clone().to(DEV)
         got_out = torch.zeros(M, Hq * dh + E, dtype=dtype, device=DEV)
@@ -543,7 +542,7 @@ def test_mixer_decode_against_the_separate_kernels(ops, Hq, Hkv, dh, H, P, N, G,
         ops.mixer_decode(u.to(DEV), inv_freq=None if inv_freq is None else inv_freq.to(DEV),
                          k_cache=views(got_pool, page_size)[0], v_cache=views(got_pool, page_size)[1],
                          block_tables=table.to(DEV), positions=positions.to(DEV), slot_mapping=slot_mapping.to(DEV),
-                         counters=counters, dt_bias=dt_bias.to(DEV), A=A.to(DEV), D=D.to(DEV), ssm_state=got_state,
+                         dt_bias=dt_bias.to(DEV), A=A.to(DEV), D=D.to(DEV), ssm_state=got_state,
                          slot_ids=slot_ids.to(DEV), out=got_out, ssm_y=got_y, **common)
         close(got_out[:, :Hq * dh], want_out[:, :Hq * dh], dtype, 2.0)
         scale = max(1.0, want_state.abs().max().item())
@@ -554,4 +553,60 @@ def test_mixer_decode_against_the_separate_kernels(ops, Hq, Hkv, dh, H, P, N, G,
             close(got_out[:, Hq * dh:], want_out[:, Hq * dh:], dtype, max(1.0, want_out.float().abs().max().item()))
         assert torch.equal(torch.isnan(got_pool.float().cpu()), torch.isnan(want_pool.float()))
         close(torch.nan_to_num(got_pool.float()), torch.nan_to_num(want_pool.float()), dtype, 4.0)
-        assert int(counters.abs().sum()) == 0
+
+
+# ------------------------------------------------------------------ prefill attention on the matrix cores
+@pytest.mark.parametrize("Hq, Hkv, dh, page_size, window", [(8, 2, 64, 16, None), (4, 4, 128, 16, None),
+                                                              (12, 2, 64, 4, None), (5, 1, 64, 64, None),
+                                                              (8, 2, 64, 16, 100), (6, 2, 128, 8, 33)])
+def test_prefill_attention_on_the_matrix_cores(ops, Hq, Hkv, dh, page_size, window):
+    """A prompt portion that continues a cached prefix, a fresh prompt longer than one tile, a
+    two-token portion and single tokens, in one batch; every unwritten cache cell holds NaN."""
+    dtype = torch.bfloat16
+    starts, counts = [37, 0, 500, 129, 0], [83, 150, 2, 1, 1]
+    lengths = [s + c for s, c in zip(starts, counts)]
+    pool, table = paged_setup(lengths, page_size, Hkv, dh, dtype, seed=21)
+    T = sum(counts)
+    keys, values = {}, {}
+    for lane, length in enumerate(lengths):          # the whole context, the step's own tokens included
+        keys[lane] = rand(length, Hkv, dh, seed=600 + lane, dtype=dtype)
+        values[lane] = rand(length, Hkv, dh, seed=700 + lane, dtype=dtype)
+        fill_cache(pool, table, lane, keys[lane], values[lane], page_size)
+    q = rand(T, Hq * dh + 16, seed=610, dtype=dtype)
+    positions = torch.cat([torch.arange(s, s + c) for s, c in zip(starts, counts)]).to(torch.int32)
+    lane_of_token = torch.repeat_interleave(torch.arange(len(counts)), torch.tensor(counts)).to(torch.int32)
+    cu = torch.zeros(len(counts) + 1, dtype=torch.int32)
+    cu[1:] = torch.cumsum(torch.tensor(counts), 0)
+    tiles = i32([(lane, row) for lane in range(len(counts)) for row in range(int(cu[lane]), int(cu[lane + 1]), 64)])
+    want = torch.empty(T, Hq * dh, dtype=dtype)
+    ref_ops.paged_attention(q, Hq, Hkv, dh, *views(pool, page_size), table, lane_of_token, positions, 0.21, window, want)
+    assert ops.prefill_attention_supported(dtype, Hq, Hkv, dh, page_size)
+    got = torch.full((T, Hq * dh), float("nan"), dtype=dtype, device=DEV)
+    ops.prefill_attention(q.to(DEV), Hq, Hkv, dh, *views(pool.to(DEV), page_size), table.to(DEV), tiles.to(DEV),
+                          cu.to(DEV), i32(starts).to(DEV), 0.21, window, got)
+    close(got, want, dtype, 2.0)
+
+
+def test_prefill_attention_finds_far_keys_and_edges(ops):
+    """Queries at the end of a 700-token prompt; one chosen key takes all the weight."""
+    Hq, Hkv, dh, length, page_size = 4, 2, 64, 700, 16
+    dtype = torch.bfloat16
+    pool, table = paged_setup([length], page_size, Hkv, dh, dtype, seed=6)
+    values = rand(length, Hkv, dh, seed=56, dtype=dtype)
+    direction = torch.zeros(dh)
+    direction[3] = 1.0
+    T = 20
+    q = (direction * 30.0).repeat(Hq)[None].repeat(T, 1).to(dtype).to(DEV)
+    tiles = i32([(0, 0)])
+    for chosen in (0, 1, 15, 16, 31, 32, 33, 511, 512, 679, 680, 698):
+        keys = rand(length, Hkv, dh, seed=57, scale=0.1, dtype=dtype)
+        keys[chosen] = (direction * 30.0).to(dtype)
+        fill_cache(pool, table, 0, keys, values, page_size)
+        out = torch.empty(T, Hq * dh, dtype=dtype, device=DEV)
+        ops.prefill_attention(q, Hq, Hkv, dh, *views(pool.to(DEV), page_size), table.to(DEV), tiles.to(DEV),
+                              i32([0, T]).to(DEV), i32([length - T]).to(DEV), 1.0 / math.sqrt(dh), None, out)
+        expected = values[chosen].float()[[0, 0, 1, 1]].reshape(-1)
+        for row in range(T):
+            position = length - T + row
+            hit = (out.float().cpu()[row] - expected).abs().max() < 1e-2
+            assert hit == (chosen <= position), f"key {chosen}, query at {position}"
