@@ -1,0 +1,359 @@
+// The Mamba2 selective scan for prompt portions in bfloat16, in chunks on the matrix cores
+// (the "state space duality" form).  Per lane (consecutive tokens of one request), head h,
+// group g of the head, with delta_t = softplus(dt_t + dt_bias), a_t = delta_t * A_h and the
+// recurrence of mamba2.hip
+//     S_t = exp(a_t) S_{t-1} + delta_t x_t (outer) B_t,   y_t = S_t . C_t + D_h x_t,
+// cut the lane into chunks of Q tokens and let L_t be the running sum of a inside a chunk:
+//     y_t   = exp(L_t) (S_in . C_t) + sum_{s<=t} exp(L_t - L_s) delta_s (C_t . B_s) x_s + D_h x_t
+//     S_out = exp(L_end) S_in + sum_s exp(L_end - L_s) delta_s x_s (outer) B_s
+// Every exponent is a difference of a non-increasing sequence taken forwards, so it is <= 0 and
+// nothing overflows.  The result does not depend on Q beyond rounding.  Five kernels:
+//     prepare     delta, L                                    (one workgroup per chunk and head)
+//     transpose   x and B of each chunk, token-contiguous and zero-padded to Q
+//     chunk_state sum_s exp(L_end - L_s) delta_s x_s (outer) B_s  per chunk and head (matrix cores)
+//     state_pass  S_in of every chunk from the slot's state, serially over a lane's chunks; the
+//                 lane's final state goes back to the slot (float32 throughout)
+//     chunk_scan  y: the two sums above on the matrix cores, (C . B^T) shared by the heads of a group
+// Operand layouts follow attn_mfma.h: a matrix-core operand wants its contraction index
+// contiguous, which is the state index n for C . B^T and S_in . C, and the token for the other
+// two products, hence the transposed copies.
+// (reference recurrence: crates/macllm-kernels/src/mamba2.rs:259-288; the reference scans token by token.)
+#include "common.h"
+
+typedef __bf16 s_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 s_bf16x4 __attribute__((ext_vector_type(4)));
+typedef float s_floatx4 __attribute__((ext_vector_type(4)));
+
+#define SSD_MAX_Q 256
+#define SSD_HEADS_PER_BLOCK 4
+
+// chunk table: int32 [n_chunks, 4] = (lane, first token row, length, index of the chunk within its lane)
+
+// ---------------------------------------------------------------- prepare
+// delta[t, h] = softplus(dt + bias); cum[t, h] = sum of delta*A over the chunk up to t (inclusive).
+__global__ void ssd_prepare_kernel(const bf16_t* __restrict__ dt, long dt_ld, const float* __restrict__ dt_bias,
+                                   const float* __restrict__ A, const int* __restrict__ chunks, int H,
+                                   float* __restrict__ delta, float* __restrict__ cum) {
+  __shared__ float wave_total[SSD_MAX_Q / WAVE];
+  const int chunk = blockIdx.x;
+  const int head = blockIdx.y;
+  const int t0 = chunks[4 * chunk + 1];
+  const int length = chunks[4 * chunk + 2];
+  const int s = threadIdx.x;
+  const int lane = s & (WAVE - 1);
+  const int wave = s / WAVE;
+  float step = 0.f, a = 0.f;
+  if (s < length) {
+    step = softplus_f((float)dt[(long)(t0 + s) * dt_ld + head] + dt_bias[head]);
+    a = step * A[head];
+  }
+  float running = a;                       // inclusive scan inside the wave
+#pragma unroll
+  for (int offset = 1; offset < WAVE; offset <<= 1) {
+    const float other = __shfl_up(running, offset, WAVE);
+    if (lane >= offset) running += other;
+  }
+  if (lane == WAVE - 1) wave_total[wave] = running;
+  __syncthreads();
+  float before = 0.f;
+  for (int w = 0; w < wave; ++w) before += wave_total[w];
+  if (s < length) {
+    delta[(long)(t0 + s) * H + head] = step;
+    cum[(long)(t0 + s) * H + head] = running + before;
+  }
+}
+
+// ---------------------------------------------------------------- transpose
+// out[chunk, channel, s] = xbc[t0 + s, channel] for s < length, 0 for the padding up to Q.
+__global__ void __launch_bounds__(256)
+ssd_transpose_kernel(const bf16_t* __restrict__ xbc, long ld, int channels, const int* __restrict__ chunks, int Q,
+                     bf16_t* __restrict__ out) {
+  __shared__ bf16_t tile[SSD_MAX_Q][66];
+  const int chunk = blockIdx.x;
+  const int c0 = blockIdx.y * 64;
+  const int t0 = chunks[4 * chunk + 1];
+  const int length = chunks[4 * chunk + 2];
+  for (int index = threadIdx.x; index < Q * 64; index += 256) {
+    const int s = index / 64;
+    const int c = index % 64;
+    tile[s][c] = (s < length && c0 + c < channels) ? xbc[(long)(t0 + s) * ld + c0 + c] : (bf16_t)0.f;
+  }
+  __syncthreads();
+  for (int index = threadIdx.x; index < Q * 64; index += 256) {
+    const int c = index / Q;
+    const int s = index % Q;
+    if (c0 + c < channels) out[((long)chunk * channels + c0 + c) * Q + s] = tile[s][c];
+  }
+}
+
+// ---------------------------------------------------------------- chunk state
+// chunk_state[chunk, h, p, n] = sum_s xT[h*P + p, s] * (BT[g*N + n, s] * exp(L_end - L_s) * delta_s)
+// computed as its transpose on the matrix cores: A = weighted BT rows (n), B = xT rows (p),
+// contraction over the Q tokens; a lane ends up with 4 consecutive n of one p.
+// chunk_decay[chunk, h] = exp(L_end).
+__global__ void __launch_bounds__(256)
+ssd_chunk_state_kernel(const bf16_t* __restrict__ xT, int E, const bf16_t* __restrict__ BT, int GN,
+                       const float* __restrict__ delta, const float* __restrict__ cum,
+                       const int* __restrict__ chunks, int Q, int H, int P, int N, int G,
+                       float* __restrict__ chunk_state, float* __restrict__ chunk_decay) {
+  __shared__ float weight[SSD_MAX_Q];
+  const int chunk = blockIdx.x;
+  const int head = blockIdx.y;
+  const int group = head / (H / G);
+  const int t0 = chunks[4 * chunk + 1];
+  const int length = chunks[4 * chunk + 2];
+  const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  const int q = lane / 16;
+  const int r = lane % 16;
+  const float total = cum[(long)(t0 + length - 1) * H + head];
+  for (int s = tid; s < Q; s += 256)
+    weight[s] = s < length ? __expf(total - cum[(long)(t0 + s) * H + head]) * delta[(long)(t0 + s) * H + head] : 0.f;
+  if (tid == 0) chunk_decay[(long)chunk * H + head] = __expf(total);
+  __syncthreads();
+  const bf16_t* x_rows = xT + ((long)chunk * E + (long)head * P) * Q;
+  const bf16_t* b_rows = BT + ((long)chunk * GN + (long)group * N) * Q;
+  float* out = chunk_state + ((long)chunk * H + head) * P * N;
+  for (int nt = wave; nt < N / 16; nt += 4) {
+    for (int pt0 = 0; pt0 < P / 16; pt0 += 4) {            // up to four p-tiles share the weighted B fragments
+      s_floatx4 acc[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = s_floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int ks = 0; ks < Q / 32; ++ks) {
+        const s_bf16x8 b_raw = *reinterpret_cast<const s_bf16x8*>(b_rows + (long)(nt * 16 + r) * Q + 32 * ks + 8 * q);
+        s_bf16x8 a;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a[j] = (bf16_t)((float)b_raw[j] * weight[32 * ks + 8 * q + j]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (pt0 + i < P / 16) {
+            const s_bf16x8 x = *reinterpret_cast<const s_bf16x8*>(x_rows + (long)((pt0 + i) * 16 + r) * Q + 32 * ks + 8 * q);
+            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, x, acc[i], 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (pt0 + i < P / 16)
+          *reinterpret_cast<s_floatx4*>(out + (long)((pt0 + i) * 16 + r) * N + nt * 16 + 4 * q) = acc[i];
+    }
+  }
+}
+
+// ---------------------------------------------------------------- state pass
+// Per lane, serially over its chunks: state_in[chunk] = running (rounded to bfloat16: it is a
+// matrix-core operand); running = decay[chunk] * running + chunk_state[chunk].  The running state
+// starts from the request's slot and goes back to it, in float32.
+__global__ void ssd_state_pass_kernel(const float* __restrict__ chunk_state, const float* __restrict__ chunk_decay,
+                                      const int* __restrict__ lane_chunks, const int* __restrict__ slot_ids, int H,
+                                      long per_head, float* __restrict__ ssm_state, bf16_t* __restrict__ state_in) {
+  const int lane = blockIdx.z;
+  const int head = blockIdx.y;
+  const long element = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (element >= per_head) return;
+  const int first = lane_chunks[2 * lane];
+  const int count = lane_chunks[2 * lane + 1];
+  float* slot = ssm_state + ((long)slot_ids[lane] * H + head) * per_head + element;
+  float running = *slot;
+  for (int c = first; c < first + count; ++c) {
+    const long at = ((long)c * H + head) * per_head + element;
+    state_in[at] = (bf16_t)running;
+    running = chunk_decay[(long)c * H + head] * running + chunk_state[at];
+  }
+  *slot = running;
+}
+
+// ---------------------------------------------------------------- chunk scan
+// One workgroup per (chunk, group, up to 4 heads of the group); each of its waves takes tiles of
+// 16 tokens t.  For a tile, with lane (q, n) holding column t = tile*16 + n:
+//   inter:  O^T[p, t] = S_in[p, :] . C[t, :]         A = S_in rows (bfloat16), B = C rows; then * exp(L_t)
+//   intra:  for 32 tokens s at a time, W^T[s, t] = B[s, :] . C[t, :] (shared by the heads), then per
+//           head  P^T[s, t] = W^T exp(L_t - L_s) delta_s [s <= t]  and  O^T += xT[p, s] . P^T[s, t]
+//   y[t, p] = O^T[p, t] + D x[t, p]
+template <int HB>
+__global__ void __launch_bounds__(256)
+ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t* __restrict__ xT, int E,
+                      const bf16_t* __restrict__ state_in, const float* __restrict__ delta,
+                      const float* __restrict__ cum, const float* __restrict__ D, const int* __restrict__ chunks,
+                      int Q, int H, int P, int N, int G, float* __restrict__ y, long y_ld) {
+  __shared__ float L[HB][SSD_MAX_Q];
+  __shared__ float step[HB][SSD_MAX_Q];
+  const int chunk = blockIdx.x;
+  const int heads_per_group = H / G;
+  const int subsets = (heads_per_group + HB - 1) / HB;
+  const int group = blockIdx.y / subsets;
+  const int head0 = group * heads_per_group + (blockIdx.y % subsets) * HB;
+  const int heads = min(HB, group * heads_per_group + heads_per_group - head0);
+  const int t0 = chunks[4 * chunk + 1];
+  const int length = chunks[4 * chunk + 2];
+  const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  const int q = lane / 16;
+  const int n = lane % 16;
+  for (int index = tid; index < HB * Q; index += 256) {
+    const int hb = index / Q;
+    const int s = index % Q;
+    const bool valid = hb < heads && s < length;
+    L[hb][s] = valid ? cum[(long)(t0 + s) * H + head0 + hb] : 0.f;
+    step[hb][s] = valid ? delta[(long)(t0 + s) * H + head0 + hb] : 0.f;
+  }
+  __syncthreads();
+  const int b_col = E + group * N;                 // columns of B and C in a row of xbc
+  const int c_col = E + G * N + group * N;
+  const int last_row = t0 + length - 1;
+  for (int tile = wave; tile * 16 < length; tile += 4) {
+    const int t = tile * 16 + n;                   // this lane's column
+    const bool has_t = t < length;
+    const long t_row = min(t0 + t, last_row);
+    // C of the column, all of N: the B operand of both score products (N <= 256: 8 fragments)
+    s_bf16x8 c_frag[8];
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+      if (32 * kk < N) {
+        c_frag[kk] = *reinterpret_cast<const s_bf16x8*>(xbc + t_row * xbc_ld + c_col + 32 * kk + 8 * q);
+        if (!has_t) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) c_frag[kk][j] = (bf16_t)0.f;
+        }
+      }
+    }
+    for (int pt = 0; pt < P / 16; ++pt) {          // 16 state rows p at a time keeps the accumulators small
+      s_floatx4 acc[HB];
+#pragma unroll
+      for (int hb = 0; hb < HB; ++hb) acc[hb] = s_floatx4{0.f, 0.f, 0.f, 0.f};
+      // inter-chunk term
+#pragma unroll
+      for (int hb = 0; hb < HB; ++hb) {
+        if (hb < heads) {
+          const bf16_t* s_rows = state_in + (((long)chunk * H + head0 + hb) * P + pt * 16 + n) * N + 8 * q;
+#pragma unroll
+          for (int kk = 0; kk < 8; ++kk) {
+            if (32 * kk < N) {
+              const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(s_rows + 32 * kk);
+              acc[hb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], acc[hb], 0, 0, 0);
+            }
+          }
+          const float carry = __expf(L[hb][min(t, length - 1)]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[hb][i] *= carry;
+        }
+      }
+      // intra-chunk term
+      for (int s0 = 0; s0 <= tile * 16 + 15 && s0 < length; s0 += 32) {
+        s_floatx4 w[2];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          w[half] = s_floatx4{0.f, 0.f, 0.f, 0.f};
+          const long s_row = min((long)t0 + s0 + 16 * half + n, (long)last_row);
+#pragma unroll
+          for (int kk = 0; kk < 8; ++kk) {
+            if (32 * kk < N) {
+              const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(xbc + s_row * xbc_ld + b_col + 32 * kk + 8 * q);
+              w[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], w[half], 0, 0, 0);
+            }
+          }
+        }
+#pragma unroll
+        for (int hb = 0; hb < HB; ++hb) {
+          if (hb < heads) {
+            s_bf16x8 p_frag;
+            const float l_t = L[hb][min(t, length - 1)];
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                const int s = s0 + 16 * half + 4 * q + i;
+                const bool visible = has_t && s <= t && s < length;
+                const float value = visible ? w[half][i] * __expf(l_t - L[hb][min(s, length - 1)]) * step[hb][min(s, length - 1)] : 0.f;
+                p_frag[4 * half + i] = (bf16_t)value;
+              }
+            const bf16_t* x_row = xT + ((long)chunk * E + (long)(head0 + hb) * P + pt * 16 + n) * Q + s0 + 4 * q;
+            const s_bf16x4 lo = *reinterpret_cast<const s_bf16x4*>(x_row);
+            const s_bf16x4 hi = *reinterpret_cast<const s_bf16x4*>(x_row + 16);
+            s_bf16x8 a;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              a[j] = lo[j];
+              a[4 + j] = hi[j];
+            }
+            acc[hb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p_frag, acc[hb], 0, 0, 0);
+          }
+        }
+      }
+      // y[t, h*P + 16 pt + 4q + i] = acc + D x
+      if (has_t) {
+#pragma unroll
+        for (int hb = 0; hb < HB; ++hb) {
+          if (hb < heads) {
+            const long column = (long)(head0 + hb) * P + pt * 16 + 4 * q;
+            const s_bf16x4 x = *reinterpret_cast<const s_bf16x4*>(xbc + t_row * xbc_ld + column);
+            const float skip = D[head0 + hb];
+            s_floatx4 out;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[i] = acc[hb][i] + skip * (float)x[i];
+            *reinterpret_cast<s_floatx4*>(y + t_row * y_ld + column) = out;
+          }
+        }
+      }
+    }
+  }
+}
+
+// Sizes: bfloat16; Q a multiple of 32 and at most 256; head_dim P a multiple of 16; state size N a
+// multiple of 32 and at most 256; row strides multiples of 8 elements.  Otherwise
+// ERR_UNSUPPORTED_SIZE (the caller uses mi_ssm_scan).
+extern "C" int mi_ssd_supported(int Q, int P, int N, int G, int E) {
+  return (Q % 32 == 0 && Q > 0 && Q <= SSD_MAX_Q && P % 16 == 0 && N % 32 == 0 && N <= 256 &&
+          (E % 8) == 0 && ((long)G * N) % 8 == 0) ? 1 : 0;
+}
+
+extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long dt_ld, const float* dt_bias,
+                              const float* A, const float* D, float* ssm_state, const int* chunks, int n_chunks,
+                              const int* lane_chunks, const int* slot_ids, int n_lanes, int Q, int H, int P, int N,
+                              int G, float* delta, float* cum, void* xT, void* BT, float* chunk_state,
+                              float* chunk_decay, void* state_in, float* y, long y_ld, hipStream_t stream) {
+  if (n_chunks <= 0 || n_lanes <= 0 || H <= 0 || G <= 0 || H % G != 0) return ERR_BAD_ARGUMENT;
+  const int E = H * P;
+  const int GN = G * N;
+  if (!mi_ssd_supported(Q, P, N, G, E) || xbc_ld % 8 != 0 || y_ld % 4 != 0 || n_chunks > 65535 * 32 ||
+      H > 65535 || n_lanes > 65535)
+    return ERR_UNSUPPORTED_SIZE;
+  {
+    const dim3 grid(n_chunks, H);
+    const int threads = ((Q + WAVE - 1) / WAVE) * WAVE;
+    ssd_prepare_kernel<<<grid, threads, 0, stream>>>((const bf16_t*)dt, dt_ld, dt_bias, A, chunks, H, delta, cum);
+    RETURN_IF_LAUNCH_FAILED();
+  }
+  {
+    const dim3 grid_x(n_chunks, (E + 63) / 64);
+    ssd_transpose_kernel<<<grid_x, 256, 0, stream>>>((const bf16_t*)xbc, xbc_ld, E, chunks, Q, (bf16_t*)xT);
+    RETURN_IF_LAUNCH_FAILED();
+    const dim3 grid_b(n_chunks, (GN + 63) / 64);
+    ssd_transpose_kernel<<<grid_b, 256, 0, stream>>>((const bf16_t*)xbc + E, xbc_ld, GN, chunks, Q, (bf16_t*)BT);
+    RETURN_IF_LAUNCH_FAILED();
+  }
+  {
+    const dim3 grid(n_chunks, H);
+    ssd_chunk_state_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)xT, E, (const bf16_t*)BT, GN, delta, cum, chunks,
+                                                     Q, H, P, N, G, chunk_state, chunk_decay);
+    RETURN_IF_LAUNCH_FAILED();
+  }
+  {
+    const long per_head = (long)P * N;
+    const dim3 grid((unsigned)((per_head + 255) / 256), H, n_lanes);
+    ssd_state_pass_kernel<<<grid, 256, 0, stream>>>(chunk_state, chunk_decay, lane_chunks, slot_ids, H, per_head,
+                                                    ssm_state, (bf16_t*)state_in);
+    RETURN_IF_LAUNCH_FAILED();
+  }
+  {
+    const int subsets = (H / G + SSD_HEADS_PER_BLOCK - 1) / SSD_HEADS_PER_BLOCK;
+    const dim3 grid(n_chunks, G * subsets);
+    ssd_chunk_scan_kernel<SSD_HEADS_PER_BLOCK><<<grid, 256, 0, stream>>>(
+        (const bf16_t*)xbc, xbc_ld, (const bf16_t*)xT, E, (const bf16_t*)state_in, delta, cum, D, chunks, Q, H, P, N,
+        G, y, y_ld);
+    RETURN_IF_LAUNCH_FAILED();
+  }
+  return 0;
+}

@@ -48,6 +48,7 @@ class StepContext:
     lane_starts: List[int] = field(default_factory=list)
     max_query_len: int = 0
     max_seq_len: int = 0             # an upper bound of the longest context in the batch
+    derived: dict = field(default_factory=dict)   # tables parts derive from the step, shared by the layers
 
 
 def _pack(lanes: Sequence[Lane], cache, pad_lanes: int = 0, max_pages: Optional[int] = None):

@@ -26,7 +26,7 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-shared", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", "-Wno-pass-failed"]
-MODULES = ("common", "attention", "mamba2", "gemm", "decode", "sampling")
+MODULES = ("common", "attention", "mamba2", "ssd", "gemm", "decode", "sampling")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

@@ -56,6 +56,12 @@ _SIGNATURES = {
         "mi_gate_norm": [_c_ptr, _c_long, _c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_float, _c_ptr, _c_long,
                          _c_int, _c_int, _c_ptr],
     },
+    "ssd": {
+        "mi_ssd_supported": [_c_int, _c_int, _c_int, _c_int, _c_int],
+        "mi_ssd_prefill": [_c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr,
+                           _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr],
+    },
     "gemm": {
         "mi_gemm_f32": [_c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr],
     },
@@ -436,6 +442,76 @@ def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: torc
     _check(_fn("mamba2", "mi_ssm_scan")(
         _p(xbc), _dt(xbc), xbc_ld, _p(dt), dt_ld, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(cu_seqlens),
         _p(slot_ids), num_lanes, H, P, N, num_groups, _p(y), y_ld, _stream()), "ssm_scan", f"(N={N})")
+
+
+class SsdChunks:
+    """The chunk table of one step for chunks of ``chunk_size`` tokens: every lane is cut from its
+    first token into chunks (the last one may be short).  ``chunks`` int32 [n, 4] = (lane, first
+    token row, length, index within the lane); ``lane_chunks`` int32 [lanes, 2] = (first chunk,
+    number of chunks)."""
+
+    def __init__(self, lane_lengths: Sequence[int], chunk_size: int, device):
+        _need(chunk_size > 0 and len(lane_lengths) > 0 and all(length > 0 for length in lane_lengths),
+              "ssd: lanes and the chunk size must be positive")
+        rows, lanes, first = [], [], 0
+        for lane, length in enumerate(lane_lengths):
+            count = -(-length // chunk_size)
+            lanes.append((len(rows), count))
+            for index in range(count):
+                rows.append((lane, first + index * chunk_size, min(chunk_size, length - index * chunk_size), index))
+            first += length
+        self.chunk_size = chunk_size
+        self.num_tokens = first
+        self.num_lanes = len(lane_lengths)
+        self.num_chunks = len(rows)
+        flat = [value for row in rows for value in row] + [value for row in lanes for value in row]
+        packed = torch.tensor(flat, dtype=torch.int32)
+        packed = packed.to(device, non_blocking=True)
+        self.chunks = packed[:4 * len(rows)]
+        self.lane_chunks = packed[4 * len(rows):]
+
+
+def ssd_supported(chunk_size: int, head_dim: int, state_size: int, num_groups: int, inner_size: int) -> bool:
+    """Whether ``ssd_prefill`` covers these sizes (otherwise ``ssm_scan`` does)."""
+    return bool(_fn("ssd", "mi_ssd_supported")(chunk_size, head_dim, state_size, num_groups, inner_size))
+
+
+def ssd_prefill(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
+                ssm_state: torch.Tensor, table: SsdChunks, slot_ids: torch.Tensor, num_groups: int,
+                y: torch.Tensor) -> None:
+    """The selective scan of ``ssm_scan`` (same arguments and results beyond rounding) for bfloat16,
+    in chunks on the matrix cores.  ``table`` cuts this step's lanes into chunks."""
+    xbc_ld = _row_major(xbc, "xbc")
+    dt_ld = _row_major(dt, "dt")
+    y_ld = _row_major(y, "y")
+    _need(ssm_state.dim() == 4 and ssm_state.dtype == torch.float32 and ssm_state.is_contiguous(),
+          "ssd_prefill: state must be contiguous float32 [slots, H, P, N]")
+    _, H, P, N = ssm_state.shape
+    T = xbc.shape[0]
+    E, GN = H * P, num_groups * N
+    _need(xbc.dtype == torch.bfloat16 and xbc.shape[1] == E + 2 * GN and dt.shape == (T, H)
+          and dt.dtype == xbc.dtype and y.shape == (T, E) and y.dtype == torch.float32,
+          "ssd_prefill: shapes do not match (bfloat16 only)")
+    _need(table.num_tokens == T and table.num_lanes == slot_ids.numel(),
+          "ssd_prefill: the chunk table was made for another step")
+    for name, vector in (("dt_bias", dt_bias), ("A", A), ("D", D)):
+        _need(vector.dtype == torch.float32 and vector.numel() == H and vector.is_contiguous() and vector.is_cuda,
+              f"ssd_prefill: {name} must be float32 [H]")
+    _i32(slot_ids, "slot_ids")
+    _need(xbc.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0, "ssd_prefill: xbc and y must be 16-byte aligned")
+    Q, chunks = table.chunk_size, table.num_chunks
+    device = xbc.device
+    delta = torch.empty((2, T, H), dtype=torch.float32, device=device)
+    transposed = torch.empty((chunks * (E + GN) * Q,), dtype=torch.bfloat16, device=device)
+    chunk_state = torch.empty((chunks * H * P * N + chunks * H,), dtype=torch.float32, device=device)
+    state_in = torch.empty((chunks * H * P * N,), dtype=torch.bfloat16, device=device)
+    xT, BT = transposed[:chunks * E * Q], transposed[chunks * E * Q:]
+    decay = chunk_state[chunks * H * P * N:]
+    _check(_fn("ssd", "mi_ssd_prefill")(
+        _p(xbc), xbc_ld, _p(dt), dt_ld, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(table.chunks), chunks,
+        _p(table.lane_chunks), _p(slot_ids), table.num_lanes, Q, H, P, N, num_groups, _p(delta[0]), _p(delta[1]),
+        _p(xT), _p(BT), _p(chunk_state), _p(decay), _p(state_in), _p(y), y_ld, _stream()),
+        "ssd_prefill", f"(Q={Q}, P={P}, N={N})")
 
 
 def gate_norm(y: torch.Tensor, z: torch.Tensor, weight: Optional[torch.Tensor], num_groups: int, eps: float,

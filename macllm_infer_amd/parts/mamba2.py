@@ -22,7 +22,8 @@ class Mamba2(Mixer):
     five segments of in_proj's output (after its bias), ``in_multiplier`` its input,
     ``out_multiplier`` out_proj's output; all are folded into the weights."""
     graph_safe = True
-    kernel_modules = ("common", "mamba2", "gemm")
+    CHUNKED_FROM = 8        # the longest lane of a step has at least this many tokens
+    kernel_modules = ("common", "mamba2", "ssd", "gemm")
 
     @classmethod
     def expected_tensors(cls, spec, prefix: str, hidden_size: int):
@@ -69,6 +70,24 @@ class Mamba2(Mixer):
         self.A = f32(-torch.exp(get("A_log").to(torch.float32).reshape(H)))
         self.D = f32(get("D").reshape(H))
         self.norm_weight = f32(get("norm.weight").reshape(E)) if spec.gated_norm else None
+        self._chunks_supported = None
+
+    def _chunked(self, u: torch.Tensor, step) -> bool:
+        """Prompt portions in bfloat16 scan in chunks on the matrix cores; single tokens, float32
+        and sizes the chunked kernels do not take scan token by token."""
+        spec = self.spec
+        if u.dtype != torch.bfloat16 or step.max_query_len < self.CHUNKED_FROM:
+            return False
+        if self._chunks_supported is None:
+            self._chunks_supported = ops.ssd_supported(spec.chunk_size, spec.head_dim, spec.state_size,
+                                                       spec.num_groups, spec.inner_size)
+        return self._chunks_supported
+
+    def _chunk_table(self, step):
+        key = ("ssd_chunks", self.spec.chunk_size)
+        if key not in step.derived:
+            step.derived[key] = ops.SsdChunks(step.lane_lengths, self.spec.chunk_size, step.token_ids.device)
+        return step.derived[key]
 
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         spec = self.spec
@@ -81,8 +100,12 @@ class Mamba2(Mixer):
                         step.cu_seqlens, step.slot_ids, xbc)
         ops.conv_state_update(u, E, C, spec.conv_kernel, conv_state, step.cu_seqlens, step.slot_ids)
         y = torch.empty((T, E), dtype=torch.float32, device=u.device)
-        ops.ssm_scan(xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, step.cu_seqlens,
-                     step.slot_ids, spec.num_groups, y)
+        if self._chunked(u, step):
+            ops.ssd_prefill(xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, self._chunk_table(step),
+                            step.slot_ids, spec.num_groups, y)
+        else:
+            ops.ssm_scan(xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, step.cu_seqlens,
+                         step.slot_ids, spec.num_groups, y)
         gated = torch.empty((T, E), dtype=u.dtype, device=u.device)
         ops.gate_norm(y, u[:, :E], self.norm_weight, spec.num_groups, spec.norm_eps, gated)
         return self.out_proj(gated)

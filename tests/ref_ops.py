@@ -284,3 +284,10 @@ def mixer_decode(u, *, num_heads, num_kv_heads, head_dim, q_col, k_col, v_col, i
 
 
 NAMES += ["fused_gemm_supported", "mixer_decode_supported", "fused_gemm", "mixer_decode"]
+
+
+def ssd_supported(chunk_size, head_dim, state_size, num_groups, inner_size):
+    return False          # the host engine scans token by token
+
+
+NAMES += ["ssd_supported"]

@@ -309,6 +309,68 @@ def test_mamba2_kernels_over_ragged_lanes(ops, dtype, H, P, N, G, K):
         assert torch.equal(got[2][untouched].cpu(), ssm_state[untouched])
 
 
+@pytest.mark.parametrize("Q", [32, 64, 128, 256])
+@pytest.mark.parametrize("H, P, N, G", [(4, 16, 32, 1), (6, 32, 64, 2), (5, 64, 128, 1), (9, 16, 96, 3), (2, 48, 256, 2)])
+def test_chunked_scan_matches_the_token_by_token_scan(ops, Q, H, P, N, G):
+    """Lanes of 1, 2, 37, 128 and 301 tokens from non-zero states in shuffled slots, whatever the
+    chunk size; the decay is strong enough in some heads to forget a chunk and weak in others."""
+    E, GN = H * P, G * N
+    counts = [1, 2, 37, 128, 301]
+    T = sum(counts)
+    slot_ids = i32([4, 0, 5, 2, 1])
+    cu = i32([0] + torch.tensor(counts).cumsum(0).tolist())
+    xbc = rand(T, E + 2 * GN, seed=80, dtype=torch.bfloat16)
+    dt = rand(T, H, seed=81, dtype=torch.bfloat16)
+    dt_bias = rand(H, seed=82) - 1.0
+    A = -torch.exp(torch.linspace(-4.0, 1.5, H))
+    D = rand(H, seed=83)
+    state = rand(7, H, P, N, seed=84, scale=0.5)
+    want_y, want_state = torch.empty(T, E), state.clone()
+    ref_ops.ssm_scan(xbc, dt, dt_bias, A, D, want_state, cu, slot_ids, G, want_y)
+    assert ops.ssd_supported(Q, P, N, G, E)
+    y, got_state = torch.full((T, E), float("nan"), device=DEV), state.to(DEV)
+    table = ops.SsdChunks(counts, Q, DEV)
+    ops.ssd_prefill(xbc.to(DEV), dt.to(DEV), *gpu(dt_bias, A, D), got_state, table, slot_ids.to(DEV), G, y)
+    scale = max(1.0, want_y.abs().max().item())
+    close(y, want_y, torch.bfloat16, scale)
+    close(got_state, want_state, torch.bfloat16, max(1.0, want_state.abs().max().item()))
+    for untouched in (3, 6):
+        assert torch.equal(got_state[untouched].cpu(), state[untouched])
+
+
+def test_chunked_scan_carries_a_far_token_through_many_chunks(ops):
+    """One token with a large x and a head that barely decays: 600 tokens later its state is what
+    the output consists of; every chunk boundary between must pass it on."""
+    H, P, N, G, Q = 4, 16, 32, 1, 32
+    E, T = H * P, 640
+    xbc = rand(T, E + 2 * N, seed=90, dtype=torch.bfloat16) * 0.05
+    xbc[3, :E] = 8.0
+    xbc[3, E:E + N] = 1.0
+    xbc[T - 1, E + N:] = 1.0
+    dt = torch.zeros(T, H, dtype=torch.bfloat16)
+    dt_bias, A, D = torch.zeros(H), -torch.tensor([1e-4, 1e-3, 1e-2, 1.0]), torch.zeros(H)
+    want_y, want_state = torch.empty(T, E), torch.zeros(1, H, P, N)
+    ref_ops.ssm_scan(xbc, dt, dt_bias, A, D, want_state, i32([0, T]), i32([0]), G, want_y)
+    assert want_y[T - 1, 0].item() > 50.0          # head 0 still holds the token
+    y, state = torch.empty(T, E, device=DEV), torch.zeros(1, H, P, N, device=DEV)
+    ops.ssd_prefill(xbc.to(DEV), dt.to(DEV), *gpu(dt_bias, A, D), state, ops.SsdChunks([T], Q, DEV), i32([0]).to(DEV),
+                    G, y)
+    close(y[T - 1:], want_y[T - 1:], torch.bfloat16, want_y[T - 1].abs().max().item())
+    close(state, want_state, torch.bfloat16, want_state.abs().max().item())
+
+
+def test_chunked_scan_refuses_sizes_it_does_not_take(ops):
+    assert not ops.ssd_supported(48, 16, 32, 1, 64)       # chunk not a multiple of 32
+    assert not ops.ssd_supported(32, 8, 32, 1, 64)        # head size not a multiple of 16
+    assert not ops.ssd_supported(32, 16, 24, 1, 64)       # state size not a multiple of 32
+    assert not ops.ssd_supported(512, 16, 32, 1, 64)
+    with pytest.raises(ops.KernelError, match="size not supported"):
+        ops.ssd_prefill(torch.zeros(4, 16 + 48, device=DEV, dtype=torch.bfloat16),
+                        torch.zeros(4, 1, device=DEV, dtype=torch.bfloat16), torch.zeros(1, device=DEV),
+                        torch.zeros(1, device=DEV), torch.zeros(1, device=DEV), torch.zeros(1, 1, 16, 24, device=DEV),
+                        ops.SsdChunks([4], 32, DEV), i32([0]).to(DEV), 1, torch.zeros(4, 16, device=DEV))
+
+
 def test_scan_refuses_a_state_size_beyond_its_limit(ops):
     with pytest.raises(ops.KernelError, match="size not supported"):
         ops.ssm_scan(torch.zeros(1, 1 + 2 * 600, device=DEV), torch.zeros(1, 1, device=DEV), torch.zeros(1, device=DEV),

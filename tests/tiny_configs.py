@@ -32,7 +32,7 @@ TINY_C = dict(
     architectures=["FalconH1ForCausalLM"], model_type="falcon_h1",
     hidden_size=128, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
     intermediate_size=96, vocab_size=200, max_position_embeddings=640, rms_norm_eps=1e-5, rope_theta=1e6,
-    mamba_n_heads=4, mamba_d_head=16, mamba_d_ssm=64, mamba_d_state=24, mamba_n_groups=1, mamba_d_conv=4,
+    mamba_n_heads=4, mamba_d_head=16, mamba_d_ssm=64, mamba_d_state=32, mamba_n_groups=1, mamba_d_conv=4,
     mamba_chunk_size=32, mamba_conv_bias=True, mamba_proj_bias=False, mamba_rms_norm=False,
     attention_bias=False, mlp_bias=False, tie_word_embeddings=True,
     embedding_multiplier=1.2, lm_head_multiplier=0.8, key_multiplier=0.9, ssm_multipliers=[1.0, 1.2, 0.9, 1.1, 1.0])
