@@ -40,6 +40,8 @@ def main() -> int:
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--page-tokens", type=int, default=16)
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
+    parser.add_argument("--prefill-only", action="store_true",
+                        help="only the 2,048-token prefill (for profiles; the line then reports prefill tokens/s)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -57,7 +59,9 @@ def main() -> int:
     element = 2 if args.dtype == "bf16" else 4
     tensors = random_tensors(config, 0, storage, "baseline")
     batches = [args.batch] if args.skip_points else sorted({1, args.batch, 64})
-    largest = max(batches)
+    if args.prefill_only:
+        batches = []
+    largest = max(batches, default=1)
     total_steps = args.steps + args.warmup
     per_request = -(-(CONTEXT + total_steps + 1) // 64) * 64
     engine = Engine(config=config, tensors=tensors, dtype="bfloat16" if args.dtype == "bf16" else "float32",
@@ -132,6 +136,12 @@ def main() -> int:
         results[batch] = dict(tokens_per_second=batch / step_seconds, ms=step_seconds * 1e3,
                               gbs=bytes_moved / step_seconds / 1e9)
 
+    if args.prefill_only:
+        print(json.dumps({"metric": "prefill tok/s at 2,048 tokens", "value": round(PREFILL_TOKENS / prefill_seconds, 1),
+                          "unit": "tokens/s", "n_gpus": 1, "ms": round(prefill_seconds * 1e3, 3), "dtype": args.dtype,
+                          "frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS[args.dtype], 5),
+                          "higher_is_better": True, "data": "synthetic", "config": {"layers": L}}))
+        return 0
     headline = results[args.batch]
     record = {
         "metric": "decode tok/s at batch 8 (2,048-token context); prefill tok/s at 2,048 tokens",

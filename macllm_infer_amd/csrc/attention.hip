@@ -470,11 +470,13 @@ extern "C" int mi_decode_attention(const void* q, long q_ld, int T, int Hq, int 
 }
 
 // ---------------------------------------------------------------- prefill attention on the matrix cores
-// bfloat16, head_dim 64 or 128.  grid = (query tiles, kv heads, head passes): a tile is up to 64
-// consecutive tokens of one lane; each of the block's four waves takes 16 of them and all the
-// query heads of the kv head (NSET column sets that share every K and V fragment).  Keys run
-// from the first visible one to the tile's last position, read straight from the cache pages
-// (the chunk's own keys were written by rope_kv_store before).
+// bfloat16, head_dim 64 or 128.  grid = (4 x query tiles, kv heads, head passes): a tile is up to 64
+// consecutive tokens of one lane and a workgroup takes 16 of them with the query heads of one kv
+// head (NSET column sets that share every K and V fragment).  The keys, from the first visible
+// one to the workgroup's last position, are split in four runs of whole 32-key steps, one per
+// wave, read straight from the cache pages (the portion's own keys were written by rope_kv_store
+// before); the four partial results are merged through LDS, set by set.  Workgroups with the
+// longest contexts (the last tiles) are launched first.
 #include "attn_mfma.h"
 
 template <int DH, int NSET>
@@ -484,19 +486,21 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
                          const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
                          const int* __restrict__ cu_seqlens, const int* __restrict__ start_pos, float scale,
                          int window, bf16_t* __restrict__ out, long out_ld) {
-  const int tile = blockIdx.x;
+  constexpr int ITEMS = 2 + 4 * (DH / 16);                    // m, l and the accumulator of one set
+  __shared__ float part[4][ITEMS][WAVE];
+  const int block = gridDim.x - 1 - blockIdx.x;               // heavy ones first
+  const int tile = block / 4;
   const int kvh = blockIdx.y;
   const int G = Hq / Hkv;
   const int head0 = kvh * G + blockIdx.z * NSET;             // first head of this pass
   const int request = tiles[2 * tile];
-  const int tile_token = tiles[2 * tile + 1];
   const int lane = threadIdx.x & (WAVE - 1);
   const int wave = threadIdx.x / WAVE;
   const int qd = lane / 16;
   const int n = lane % 16;
   const int lane_end = cu_seqlens[request + 1];
-  const int first_token = tile_token + 16 * wave;
-  if (first_token >= lane_end) return;
+  const int first_token = tiles[2 * tile + 1] + 16 * (block % 4);
+  if (first_token >= lane_end) return;                        // the whole workgroup
   const int token = first_token + n;
   const bool has_query = token < lane_end;
   const int base_position = start_pos[request] - cu_seqlens[request];
@@ -533,17 +537,51 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
   cache.base_page = 0;
   int key_lo = 0;
   if (window > 0 && first_position - window + 1 > 0) key_lo = ((first_position - window + 1) / 32) * 32;
-  attend_keys<DH, NSET, 1>(acc, q_frag, col_pos, window, scale, key_lo, last_position + 1, cache);
+  const int key_hi = last_position + 1;
+  const int steps = (key_hi - key_lo + 31) / 32;
+  const int steps_per_wave = (steps + 3) / 4;
+  const int my_lo = key_lo + 32 * steps_per_wave * wave;
+  const int my_hi = min(key_hi, my_lo + 32 * steps_per_wave);
+  if (my_lo < my_hi) attend_keys<DH, NSET, 2>(acc, q_frag, col_pos, window, scale, my_lo, my_hi, cache);
+
+  // merge: set s is finished by wave s % 4
 #pragma unroll
   for (int s = 0; s < NSET; ++s) {
-    const float l = attn_normalizer<DH, NSET>(acc, s);
+    __syncthreads();
+    part[wave][0][lane] = acc.m[s];
+    part[wave][1][lane] = acc.l[s];
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[wave][2 + 4 * dt + i][lane] = acc.o[s][dt][i];
+    __syncthreads();
+    if (wave != (s & 3)) continue;
+    float m = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) m = fmaxf(m, part[w][0][lane]);
+    float factor[4];
+    float l = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float m_w = part[w][0][lane];
+      factor[w] = m_w == -INFINITY ? 0.f : __expf(m_w - m);
+      l += part[w][1][lane] * factor[w];
+    }
+    l += __shfl_xor(l, 16, WAVE);
+    l += __shfl_xor(l, 32, WAVE);
     if (col_pos[s] < 0) continue;
+    const float inverse = 1.f / l;
     bf16_t* o = out + (long)token * out_ld + (long)(head0 + s) * DH;
 #pragma unroll
     for (int dt = 0; dt < DH / 16; ++dt) {
       mfma_bf16x4 packed;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(acc.o[s][dt][i] / l);
+      for (int i = 0; i < 4; ++i) {
+        float value = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) value += part[w][2 + 4 * dt + i][lane] * factor[w];
+        packed[i] = (bf16_t)(value * inverse);
+      }
       *reinterpret_cast<mfma_bf16x4*>(o + 16 * dt + 4 * qd) = packed;
     }
   }
@@ -563,7 +601,8 @@ extern "C" int mi_prefill_attention(const void* q, long q_ld, int Hq, int Hkv, i
     return ERR_UNSUPPORTED_SIZE;
   const int passes = (G + 3) / 4;
   const int nset = (G + passes - 1) / passes;
-  const dim3 grid(n_tiles, Hkv, passes);
+  if (n_tiles > (1 << 28)) return ERR_UNSUPPORTED_SIZE;
+  const dim3 grid(4 * n_tiles, Hkv, passes);
 #define PREFILL_CASE(DH_, NSET_)                                                                              \
   if (dh == DH_ && nset == NSET_)                                                                             \
     prefill_attention_kernel<DH_, NSET_><<<grid, 256, 0, stream>>>(                                           \

@@ -41,6 +41,65 @@ __global__ void conv1d_silu_kernel(const T* __restrict__ u, long ld, int col_off
   out[index] = from_float<T>(silu_f(sum));
 }
 
+// The same for bfloat16 with 8 channels and 4 consecutive token rows per thread: the rows the four
+// windows share are loaded once, 16 bytes at a time.  A row that lies before its token's lane
+// comes from the lane's conv tail instead.
+typedef __bf16 conv_bf16x8 __attribute__((ext_vector_type(8)));
+
+template <int K>
+__global__ void __launch_bounds__(256)
+conv1d_silu_vec_kernel(const bf16_t* __restrict__ u, long ld, int col_offset, int C, int T,
+                       const float* __restrict__ weight, const float* __restrict__ bias,
+                       const bf16_t* __restrict__ conv_state, const int* __restrict__ lane_of_token,
+                       const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids,
+                       bf16_t* __restrict__ out) {
+  constexpr int ROWS = 4;
+  const int vectors = C / 8;
+  const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long group = index / vectors;
+  const int channel = (int)(index - group * vectors) * 8;
+  const long t0 = group * ROWS;
+  if (t0 >= T) return;
+  conv_bf16x8 window[ROWS + K - 1];                 // rows t0-(K-1) .. t0+ROWS-1 of u
+#pragma unroll
+  for (int j = 0; j < ROWS + K - 1; ++j) {
+    const long row = t0 - (K - 1) + j;
+    if (row >= 0 && row < T) window[j] = *reinterpret_cast<const conv_bf16x8*>(u + row * ld + col_offset + channel);
+  }
+  float w[8][K];
+  float b[8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    b[c] = bias ? bias[channel + c] : 0.f;
+#pragma unroll
+    for (int k = 0; k < K; ++k) w[c][k] = weight[(long)(channel + c) * K + k];
+  }
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) {
+    const long token = t0 + i;
+    if (token >= T) break;
+    const int lane = lane_of_token[token];
+    const long lane_start = cu_seqlens[lane];
+    float sum[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) sum[c] = b[c];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const long source = token - (K - 1) + k;
+      conv_bf16x8 sample = window[i + k];
+      if (source < lane_start)
+        sample = *reinterpret_cast<const conv_bf16x8*>(conv_state + ((long)slot_ids[lane] * (K - 1) + (K - 1) +
+                                                                     (source - lane_start)) * C + channel);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) sum[c] += w[c][k] * (float)sample[c];
+    }
+    conv_bf16x8 result;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) result[c] = (bf16_t)silu_f(sum[c]);
+    *reinterpret_cast<conv_bf16x8*>(out + token * C + channel) = result;
+  }
+}
+
 extern "C" int mi_conv1d_silu(const void* u, int dtype, long ld, int col_offset, int T, int C, int K,
                               const float* weight, const float* bias, const void* conv_state,
                               const int* lane_of_token, const int* cu_seqlens, const int* slot_ids, void* out,
@@ -48,6 +107,22 @@ extern "C" int mi_conv1d_silu(const void* u, int dtype, long ld, int col_offset,
   if (T <= 0 || C <= 0 || K <= 0 || K > CONV_MAX_K || ld < col_offset + C) return ERR_BAD_ARGUMENT;
   const long total = (long)T * C;
   const int blocks = (int)((total + 255) / 256);
+  const bool aligned = C % 8 == 0 && ld % 8 == 0 && col_offset % 8 == 0 && ((uintptr_t)u % 16) == 0 &&
+                       ((uintptr_t)out % 16) == 0 && ((uintptr_t)conv_state % 16) == 0;
+  if (dtype == DT_BF16 && aligned && K >= 2 && K <= 4) {
+    const long threads = (long)((T + 3) / 4) * (C / 8);
+    const int vec_blocks = (int)((threads + 255) / 256);
+#define CONV_CASE(K_)                                                                                          \
+  conv1d_silu_vec_kernel<K_><<<vec_blocks, 256, 0, stream>>>((const bf16_t*)u, ld, col_offset, C, T, weight,   \
+                                                             bias, (const bf16_t*)conv_state, lane_of_token,   \
+                                                             cu_seqlens, slot_ids, (bf16_t*)out)
+    if (K == 2) CONV_CASE(2);
+    else if (K == 3) CONV_CASE(3);
+    else CONV_CASE(4);
+#undef CONV_CASE
+    RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
   if (dtype == DT_F32)
     conv1d_silu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)u, ld, col_offset, C, K, weight, bias,
                                                            (const float*)conv_state, lane_of_token, cu_seqlens,

@@ -13,7 +13,8 @@
 //     chunk_state sum_s exp(L_end - L_s) delta_s x_s (outer) B_s  per chunk and head (matrix cores)
 //     state_pass  S_in of every chunk from the slot's state, serially over a lane's chunks; the
 //                 lane's final state goes back to the slot (float32 throughout)
-//     chunk_scan  y: the two sums above on the matrix cores, (C . B^T) shared by the heads of a group
+//     chunk_scan  y: the two sums above on the matrix cores, (C . B^T) shared by the heads of a group;
+//                 optionally the gate y * SiLU(z) on the way out
 // Operand layouts follow attn_mfma.h: a matrix-core operand wants its contraction index
 // contiguous, which is the state index n for C . B^T and S_in . C, and the token for the other
 // two products, hence the transposed copies.
@@ -65,24 +66,41 @@ __global__ void ssd_prepare_kernel(const bf16_t* __restrict__ dt, long dt_ld, co
 
 // ---------------------------------------------------------------- transpose
 // out[chunk, channel, s] = xbc[t0 + s, channel] for s < length, 0 for the padding up to Q.
+// 64 channels of a chunk per workgroup: 16-byte loads along the channels, 2-byte stores into a
+// transposed LDS tile whose row stride (Q + 2 elements = an odd number of banks) keeps them
+// apart, 4-byte LDS reads and 16-byte stores along the tokens.
 __global__ void __launch_bounds__(256)
 ssd_transpose_kernel(const bf16_t* __restrict__ xbc, long ld, int channels, const int* __restrict__ chunks, int Q,
                      bf16_t* __restrict__ out) {
-  __shared__ bf16_t tile[SSD_MAX_Q][66];
+  __shared__ __align__(4) bf16_t tile[64 * (SSD_MAX_Q + 2)];
+  const int stride = Q + 2;
   const int chunk = blockIdx.x;
   const int c0 = blockIdx.y * 64;
   const int t0 = chunks[4 * chunk + 1];
   const int length = chunks[4 * chunk + 2];
-  for (int index = threadIdx.x; index < Q * 64; index += 256) {
-    const int s = index / 64;
-    const int c = index % 64;
-    tile[s][c] = (s < length && c0 + c < channels) ? xbc[(long)(t0 + s) * ld + c0 + c] : (bf16_t)0.f;
+  for (int index = threadIdx.x; index < Q * 8; index += 256) {
+    const int s = index / 8;
+    const int c = (index % 8) * 8;
+    s_bf16x8 v;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (bf16_t)0.f;
+    if (s < length && c0 + c < channels) v = *reinterpret_cast<const s_bf16x8*>(xbc + (long)(t0 + s) * ld + c0 + c);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) tile[(c + j) * stride + s] = v[j];
   }
   __syncthreads();
-  for (int index = threadIdx.x; index < Q * 64; index += 256) {
-    const int c = index / Q;
-    const int s = index % Q;
-    if (c0 + c < channels) out[((long)chunk * channels + c0 + c) * Q + s] = tile[s][c];
+  const int vectors = Q / 8;
+  for (int index = threadIdx.x; index < 64 * vectors; index += 256) {
+    const int c = index / vectors;
+    const int s = (index % vectors) * 8;
+    if (c0 + c >= channels) continue;
+    const unsigned* words = reinterpret_cast<const unsigned*>(tile + c * stride + s);
+    uint4 v;
+    v.x = words[0];
+    v.y = words[1];
+    v.z = words[2];
+    v.w = words[3];
+    *reinterpret_cast<uint4*>(out + ((long)chunk * channels + c0 + c) * Q + s) = v;
   }
 }
 
@@ -165,18 +183,20 @@ __global__ void ssd_state_pass_kernel(const float* __restrict__ chunk_state, con
 }
 
 // ---------------------------------------------------------------- chunk scan
-// One workgroup per (chunk, group, up to 4 heads of the group); each of its waves takes tiles of
-// 16 tokens t.  For a tile, with lane (q, n) holding column t = tile*16 + n:
+// One workgroup per (chunk, group, up to HB heads of the group, 64 tokens); each of its waves
+// takes a tile of 16 tokens t.  For a tile, with lane (q, n) holding column t = tile*16 + n:
 //   inter:  O^T[p, t] = S_in[p, :] . C[t, :]         A = S_in rows (bfloat16), B = C rows; then * exp(L_t)
 //   intra:  for 32 tokens s at a time, W^T[s, t] = B[s, :] . C[t, :] (shared by the heads), then per
 //           head  P^T[s, t] = W^T exp(L_t - L_s) delta_s [s <= t]  and  O^T += xT[p, s] . P^T[s, t]
-//   y[t, p] = O^T[p, t] + D x[t, p]
-template <int HB>
+//   y[t, p] = O^T[p, t] + D x[t, p];  with z given, gated[t, p] = y * SiLU(z[t, p]) is written instead.
+// Up to 64 state rows p are held at a time (PT tiles of 16); a larger head repeats the pass.
+template <int HB, int PT>
 __global__ void __launch_bounds__(256)
 ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t* __restrict__ xT, int E,
                       const bf16_t* __restrict__ state_in, const float* __restrict__ delta,
                       const float* __restrict__ cum, const float* __restrict__ D, const int* __restrict__ chunks,
-                      int Q, int H, int P, int N, int G, float* __restrict__ y, long y_ld) {
+                      int Q, int H, int P, int N, int G, float* __restrict__ y, long y_ld,
+                      const bf16_t* __restrict__ z, long z_ld, bf16_t* __restrict__ gated, long gated_ld) {
   __shared__ float L[HB][SSD_MAX_Q];
   __shared__ float step[HB][SSD_MAX_Q];
   const int chunk = blockIdx.x;
@@ -190,110 +210,138 @@ ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t*
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
+  const int tile = (gridDim.z - 1 - blockIdx.z) * 4 + wave;    // the tiles with the most tokens before them first
+  if ((tile - wave) * 16 >= length) return;                      // the whole workgroup
   const int q = lane / 16;
   const int n = lane % 16;
-  for (int index = tid; index < HB * Q; index += 256) {
-    const int hb = index / Q;
-    const int s = index % Q;
-    const bool valid = hb < heads && s < length;
+  const int first_s = 0;
+  const int end_s = min(length, (tile - wave) * 16 + 64);        // tokens any wave of the workgroup looks at
+  for (int index = tid; index < HB * (end_s - first_s); index += 256) {
+    const int hb = index / (end_s - first_s);
+    const int s = first_s + index % (end_s - first_s);
+    const bool valid = hb < heads;
     L[hb][s] = valid ? cum[(long)(t0 + s) * H + head0 + hb] : 0.f;
     step[hb][s] = valid ? delta[(long)(t0 + s) * H + head0 + hb] : 0.f;
   }
   __syncthreads();
+  if (tile * 16 >= length) return;
   const int b_col = E + group * N;                 // columns of B and C in a row of xbc
   const int c_col = E + G * N + group * N;
   const int last_row = t0 + length - 1;
-  for (int tile = wave; tile * 16 < length; tile += 4) {
-    const int t = tile * 16 + n;                   // this lane's column
-    const bool has_t = t < length;
-    const long t_row = min(t0 + t, last_row);
-    // C of the column, all of N: the B operand of both score products (N <= 256: 8 fragments)
-    s_bf16x8 c_frag[8];
+  const int t = tile * 16 + n;                     // this lane's column
+  const bool has_t = t < length;
+  const int t_safe = min(t, length - 1);
+  const long t_row = t0 + t_safe;
+  // C of the column, all of N: the B operand of both score products (N <= 256: 8 fragments)
+  s_bf16x8 c_frag[8];
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-      if (32 * kk < N) {
-        c_frag[kk] = *reinterpret_cast<const s_bf16x8*>(xbc + t_row * xbc_ld + c_col + 32 * kk + 8 * q);
-        if (!has_t) {
+  for (int kk = 0; kk < 8; ++kk) {
+    if (32 * kk < N) {
+      c_frag[kk] = *reinterpret_cast<const s_bf16x8*>(xbc + t_row * xbc_ld + c_col + 32 * kk + 8 * q);
+      if (!has_t) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) c_frag[kk][j] = (bf16_t)0.f;
+        for (int j = 0; j < 8; ++j) c_frag[kk][j] = (bf16_t)0.f;
+      }
+    }
+  }
+  for (int pt0 = 0; pt0 < P / 16; pt0 += PT) {
+    s_floatx4 acc[HB][PT];
+    // inter-chunk term
+#pragma unroll
+    for (int hb = 0; hb < HB; ++hb) {
+#pragma unroll
+      for (int pi = 0; pi < PT; ++pi) acc[hb][pi] = s_floatx4{0.f, 0.f, 0.f, 0.f};
+      if (hb < heads) {
+        const float carry = __expf(L[hb][t_safe]);
+#pragma unroll
+        for (int pi = 0; pi < PT; ++pi) {
+          if (pt0 + pi < P / 16) {
+            const bf16_t* s_rows = state_in + (((long)chunk * H + head0 + hb) * P + (pt0 + pi) * 16 + n) * N + 8 * q;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+              if (32 * kk < N) {
+                const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(s_rows + 32 * kk);
+                acc[hb][pi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], acc[hb][pi], 0, 0, 0);
+              }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[hb][pi][i] *= carry;
+          }
         }
       }
     }
-    for (int pt = 0; pt < P / 16; ++pt) {          // 16 state rows p at a time keeps the accumulators small
-      s_floatx4 acc[HB];
+    // intra-chunk term
+    for (int s0 = 0; s0 <= tile * 16 + 15 && s0 < length; s0 += 32) {
+      s_floatx4 w[2];
 #pragma unroll
-      for (int hb = 0; hb < HB; ++hb) acc[hb] = s_floatx4{0.f, 0.f, 0.f, 0.f};
-      // inter-chunk term
+      for (int half = 0; half < 2; ++half) {
+        w[half] = s_floatx4{0.f, 0.f, 0.f, 0.f};
+        const long s_row = min((long)t0 + s0 + 16 * half + n, (long)last_row);
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+          if (32 * kk < N) {
+            const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(xbc + s_row * xbc_ld + b_col + 32 * kk + 8 * q);
+            w[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], w[half], 0, 0, 0);
+          }
+        }
+      }
 #pragma unroll
       for (int hb = 0; hb < HB; ++hb) {
         if (hb < heads) {
-          const bf16_t* s_rows = state_in + (((long)chunk * H + head0 + hb) * P + pt * 16 + n) * N + 8 * q;
+          s_bf16x8 p_frag;
+          const float l_t = L[hb][t_safe];
 #pragma unroll
-          for (int kk = 0; kk < 8; ++kk) {
-            if (32 * kk < N) {
-              const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(s_rows + 32 * kk);
-              acc[hb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], acc[hb], 0, 0, 0);
+          for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int s = s0 + 16 * half + 4 * q + i;
+              const int s_safe = min(s, length - 1);
+              const bool visible = has_t && s <= t && s < length;
+              const float value = visible ? w[half][i] * __expf(l_t - L[hb][s_safe]) * step[hb][s_safe] : 0.f;
+              p_frag[4 * half + i] = (bf16_t)value;
             }
-          }
-          const float carry = __expf(L[hb][min(t, length - 1)]);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[hb][i] *= carry;
-        }
-      }
-      // intra-chunk term
-      for (int s0 = 0; s0 <= tile * 16 + 15 && s0 < length; s0 += 32) {
-        s_floatx4 w[2];
+          for (int pi = 0; pi < PT; ++pi) {
+            if (pt0 + pi < P / 16) {
+              const bf16_t* x_row = xT + ((long)chunk * E + (long)(head0 + hb) * P + (pt0 + pi) * 16 + n) * Q + s0 + 4 * q;
+              const s_bf16x4 lo = *reinterpret_cast<const s_bf16x4*>(x_row);
+              const s_bf16x4 hi = *reinterpret_cast<const s_bf16x4*>(x_row + 16);
+              s_bf16x8 a;
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          w[half] = s_floatx4{0.f, 0.f, 0.f, 0.f};
-          const long s_row = min((long)t0 + s0 + 16 * half + n, (long)last_row);
-#pragma unroll
-          for (int kk = 0; kk < 8; ++kk) {
-            if (32 * kk < N) {
-              const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(xbc + s_row * xbc_ld + b_col + 32 * kk + 8 * q);
-              w[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], w[half], 0, 0, 0);
-            }
-          }
-        }
-#pragma unroll
-        for (int hb = 0; hb < HB; ++hb) {
-          if (hb < heads) {
-            s_bf16x8 p_frag;
-            const float l_t = L[hb][min(t, length - 1)];
-#pragma unroll
-            for (int half = 0; half < 2; ++half)
-#pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                const int s = s0 + 16 * half + 4 * q + i;
-                const bool visible = has_t && s <= t && s < length;
-                const float value = visible ? w[half][i] * __expf(l_t - L[hb][min(s, length - 1)]) * step[hb][min(s, length - 1)] : 0.f;
-                p_frag[4 * half + i] = (bf16_t)value;
+              for (int j = 0; j < 4; ++j) {
+                a[j] = lo[j];
+                a[4 + j] = hi[j];
               }
-            const bf16_t* x_row = xT + ((long)chunk * E + (long)(head0 + hb) * P + pt * 16 + n) * Q + s0 + 4 * q;
-            const s_bf16x4 lo = *reinterpret_cast<const s_bf16x4*>(x_row);
-            const s_bf16x4 hi = *reinterpret_cast<const s_bf16x4*>(x_row + 16);
-            s_bf16x8 a;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              a[j] = lo[j];
-              a[4 + j] = hi[j];
+              acc[hb][pi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p_frag, acc[hb][pi], 0, 0, 0);
             }
-            acc[hb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p_frag, acc[hb], 0, 0, 0);
           }
         }
       }
-      // y[t, h*P + 16 pt + 4q + i] = acc + D x
-      if (has_t) {
+    }
+    // y[t, h*P + 16 pt + 4q + i] = acc + D x
+    if (has_t) {
 #pragma unroll
-        for (int hb = 0; hb < HB; ++hb) {
-          if (hb < heads) {
-            const long column = (long)(head0 + hb) * P + pt * 16 + 4 * q;
-            const s_bf16x4 x = *reinterpret_cast<const s_bf16x4*>(xbc + t_row * xbc_ld + column);
-            const float skip = D[head0 + hb];
-            s_floatx4 out;
+      for (int hb = 0; hb < HB; ++hb) {
+        if (hb < heads) {
+          const float skip = D[head0 + hb];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) out[i] = acc[hb][i] + skip * (float)x[i];
-            *reinterpret_cast<s_floatx4*>(y + t_row * y_ld + column) = out;
+          for (int pi = 0; pi < PT; ++pi) {
+            if (pt0 + pi < P / 16) {
+              const long column = (long)(head0 + hb) * P + (pt0 + pi) * 16 + 4 * q;
+              const s_bf16x4 x = *reinterpret_cast<const s_bf16x4*>(xbc + t_row * xbc_ld + column);
+              s_floatx4 out;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) out[i] = acc[hb][pi][i] + skip * (float)x[i];
+              if (z != nullptr) {
+                const s_bf16x4 gate = *reinterpret_cast<const s_bf16x4*>(z + t_row * z_ld + column);
+                s_bf16x4 packed;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(out[i] * silu_f((float)gate[i]));
+                *reinterpret_cast<s_bf16x4*>(gated + t_row * gated_ld + column) = packed;
+              } else {
+                *reinterpret_cast<s_floatx4*>(y + t_row * y_ld + column) = out;
+              }
+            }
           }
         }
       }
@@ -313,11 +361,14 @@ extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long
                               const float* A, const float* D, float* ssm_state, const int* chunks, int n_chunks,
                               const int* lane_chunks, const int* slot_ids, int n_lanes, int Q, int H, int P, int N,
                               int G, float* delta, float* cum, void* xT, void* BT, float* chunk_state,
-                              float* chunk_decay, void* state_in, float* y, long y_ld, hipStream_t stream) {
+                              float* chunk_decay, void* state_in, float* y, long y_ld, const void* z, long z_ld,
+                              void* gated, long gated_ld, hipStream_t stream) {
   if (n_chunks <= 0 || n_lanes <= 0 || H <= 0 || G <= 0 || H % G != 0) return ERR_BAD_ARGUMENT;
   const int E = H * P;
   const int GN = G * N;
-  if (!mi_ssd_supported(Q, P, N, G, E) || xbc_ld % 8 != 0 || y_ld % 4 != 0 || n_chunks > 65535 * 32 ||
+  if ((z == nullptr) != (gated == nullptr) || (z == nullptr && y == nullptr)) return ERR_BAD_ARGUMENT;
+  if (!mi_ssd_supported(Q, P, N, G, E) || xbc_ld % 8 != 0 || y_ld % 4 != 0 || z_ld % 4 != 0 || gated_ld % 4 != 0 ||
+      n_chunks > 65535 * 32 ||
       H > 65535 || n_lanes > 65535)
     return ERR_UNSUPPORTED_SIZE;
   {
@@ -349,10 +400,16 @@ extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long
   }
   {
     const int subsets = (H / G + SSD_HEADS_PER_BLOCK - 1) / SSD_HEADS_PER_BLOCK;
-    const dim3 grid(n_chunks, G * subsets);
-    ssd_chunk_scan_kernel<SSD_HEADS_PER_BLOCK><<<grid, 256, 0, stream>>>(
-        (const bf16_t*)xbc, xbc_ld, (const bf16_t*)xT, E, (const bf16_t*)state_in, delta, cum, D, chunks, Q, H, P, N,
-        G, y, y_ld);
+    const dim3 grid(n_chunks, G * subsets, (Q + 63) / 64);
+#define SCAN_CASE(PT_)                                                                                            \
+  ssd_chunk_scan_kernel<SSD_HEADS_PER_BLOCK, PT_><<<grid, 256, 0, stream>>>(                                      \
+      (const bf16_t*)xbc, xbc_ld, (const bf16_t*)xT, E, (const bf16_t*)state_in, delta, cum, D, chunks, Q, H, P, \
+      N, G, y, y_ld, (const bf16_t*)z, z_ld, (bf16_t*)gated, gated_ld)
+    if (P / 16 == 1) SCAN_CASE(1);
+    else if (P / 16 == 2) SCAN_CASE(2);
+    else if (P / 16 == 3) SCAN_CASE(3);
+    else SCAN_CASE(4);
+#undef SCAN_CASE
     RETURN_IF_LAUNCH_FAILED();
   }
   return 0;

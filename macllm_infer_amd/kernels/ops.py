@@ -60,7 +60,7 @@ _SIGNATURES = {
         "mi_ssd_supported": [_c_int, _c_int, _c_int, _c_int, _c_int],
         "mi_ssd_prefill": [_c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr,
                            _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr],
+                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr],
     },
     "gemm": {
         "mi_gemm_f32": [_c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr],
@@ -478,27 +478,40 @@ def ssd_supported(chunk_size: int, head_dim: int, state_size: int, num_groups: i
 
 def ssd_prefill(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
                 ssm_state: torch.Tensor, table: SsdChunks, slot_ids: torch.Tensor, num_groups: int,
-                y: torch.Tensor) -> None:
+                y: Optional[torch.Tensor], z: Optional[torch.Tensor] = None,
+                gated: Optional[torch.Tensor] = None) -> None:
     """The selective scan of ``ssm_scan`` (same arguments and results beyond rounding) for bfloat16,
-    in chunks on the matrix cores.  ``table`` cuts this step's lanes into chunks."""
+    in chunks on the matrix cores.  ``table`` cuts this step's lanes into chunks.  With ``z`` and
+    ``gated`` (bfloat16 [T, E], column views are fine) it writes gated = y * SiLU(z) and no y."""
     xbc_ld = _row_major(xbc, "xbc")
     dt_ld = _row_major(dt, "dt")
-    y_ld = _row_major(y, "y")
+    fused_gate = z is not None
+    _need((gated is not None) == fused_gate and (y is None) == fused_gate,
+          "ssd_prefill: give either y, or z and gated")
+    if fused_gate:
+        z_ld, gated_ld, y_ld = _row_major(z, "z"), _row_major(gated, "gated"), 0
+        _need(z.dtype == torch.bfloat16 and gated.dtype == torch.bfloat16 and z.shape == gated.shape
+              and z.data_ptr() % 8 == 0 and gated.data_ptr() % 8 == 0, "ssd_prefill: z/gated do not fit")
+    else:
+        z_ld = gated_ld = 0
+        y_ld = _row_major(y, "y")
     _need(ssm_state.dim() == 4 and ssm_state.dtype == torch.float32 and ssm_state.is_contiguous(),
           "ssd_prefill: state must be contiguous float32 [slots, H, P, N]")
     _, H, P, N = ssm_state.shape
     T = xbc.shape[0]
     E, GN = H * P, num_groups * N
     _need(xbc.dtype == torch.bfloat16 and xbc.shape[1] == E + 2 * GN and dt.shape == (T, H)
-          and dt.dtype == xbc.dtype and y.shape == (T, E) and y.dtype == torch.float32,
-          "ssd_prefill: shapes do not match (bfloat16 only)")
+          and dt.dtype == xbc.dtype, "ssd_prefill: shapes do not match (bfloat16 only)")
+    result = gated if fused_gate else y
+    _need(result.shape == (T, E) and (fused_gate or y.dtype == torch.float32), "ssd_prefill: output shape")
     _need(table.num_tokens == T and table.num_lanes == slot_ids.numel(),
           "ssd_prefill: the chunk table was made for another step")
     for name, vector in (("dt_bias", dt_bias), ("A", A), ("D", D)):
         _need(vector.dtype == torch.float32 and vector.numel() == H and vector.is_contiguous() and vector.is_cuda,
               f"ssd_prefill: {name} must be float32 [H]")
     _i32(slot_ids, "slot_ids")
-    _need(xbc.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0, "ssd_prefill: xbc and y must be 16-byte aligned")
+    _need(xbc.data_ptr() % 16 == 0 and (fused_gate or y.data_ptr() % 16 == 0),
+          "ssd_prefill: xbc and y must be 16-byte aligned")
     Q, chunks = table.chunk_size, table.num_chunks
     device = xbc.device
     delta = torch.empty((2, T, H), dtype=torch.float32, device=device)
@@ -510,7 +523,8 @@ def ssd_prefill(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: t
     _check(_fn("ssd", "mi_ssd_prefill")(
         _p(xbc), xbc_ld, _p(dt), dt_ld, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(table.chunks), chunks,
         _p(table.lane_chunks), _p(slot_ids), table.num_lanes, Q, H, P, N, num_groups, _p(delta[0]), _p(delta[1]),
-        _p(xT), _p(BT), _p(chunk_state), _p(decay), _p(state_in), _p(y), y_ld, _stream()),
+        _p(xT), _p(BT), _p(chunk_state), _p(decay), _p(state_in), _p(y), y_ld, _p(z), z_ld, _p(gated), gated_ld,
+        _stream()),
         "ssd_prefill", f"(Q={Q}, P={P}, N={N})")
 
 

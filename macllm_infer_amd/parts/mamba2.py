@@ -99,13 +99,18 @@ class Mamba2(Mixer):
         ops.conv1d_silu(u, E, C, self.conv_weight, self.conv_bias, conv_state, step.lane_of_token,
                         step.cu_seqlens, step.slot_ids, xbc)
         ops.conv_state_update(u, E, C, spec.conv_kernel, conv_state, step.cu_seqlens, step.slot_ids)
-        y = torch.empty((T, E), dtype=torch.float32, device=u.device)
+        gated = torch.empty((T, E), dtype=u.dtype, device=u.device)
         if self._chunked(u, step):
-            ops.ssd_prefill(xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, self._chunk_table(step),
-                            step.slot_ids, spec.num_groups, y)
+            arguments = (xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, self._chunk_table(step),
+                         step.slot_ids, spec.num_groups)
+            if self.norm_weight is None and u.stride(0) % 4 == 0:
+                ops.ssd_prefill(*arguments, None, z=u[:, :E], gated=gated)      # the gate on the scan's way out
+                return self.out_proj(gated)
+            y = torch.empty((T, E), dtype=torch.float32, device=u.device)
+            ops.ssd_prefill(*arguments, y)
         else:
+            y = torch.empty((T, E), dtype=torch.float32, device=u.device)
             ops.ssm_scan(xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, step.cu_seqlens,
                          step.slot_ids, spec.num_groups, y)
-        gated = torch.empty((T, E), dtype=u.dtype, device=u.device)
         ops.gate_norm(y, u[:, :E], self.norm_weight, spec.num_groups, spec.norm_eps, gated)
         return self.out_proj(gated)

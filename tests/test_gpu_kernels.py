@@ -336,6 +336,15 @@ def test_chunked_scan_matches_the_token_by_token_scan(ops, Q, H, P, N, G):
     close(got_state, want_state, torch.bfloat16, max(1.0, want_state.abs().max().item()))
     for untouched in (3, 6):
         assert torch.equal(got_state[untouched].cpu(), state[untouched])
+    # the gate on the way out: y * SiLU(z), z a column view of a wider matrix
+    wide = rand(T, E + 8, seed=85, dtype=torch.bfloat16)
+    want_gated = torch.empty(T, E, dtype=torch.bfloat16)
+    ref_ops.gate_norm(want_y, wide[:, 8:], None, G, 1e-5, want_gated)
+    gated, again = torch.empty(T, E, dtype=torch.bfloat16, device=DEV), state.to(DEV)
+    ops.ssd_prefill(xbc.to(DEV), dt.to(DEV), *gpu(dt_bias, A, D), again, table, slot_ids.to(DEV), G, None,
+                    z=wide.to(DEV)[:, 8:], gated=gated)
+    close(gated, want_gated, torch.bfloat16, max(1.0, want_gated.float().abs().max().item()))
+    assert torch.equal(again, got_state)
 
 
 def test_chunked_scan_carries_a_far_token_through_many_chunks(ops):
