@@ -1,5 +1,6 @@
 """The decode fast path of a layer: when every lane of a step holds one token, a block made
-of RMSNorm, attention, Mamba2 and SwiGLU runs as five launches instead of fifteen.
+of RMSNorm, attention, Mamba2 and SwiGLU runs as five launches instead of fifteen (seven for
+batches of more than 16 rows, whose two norms run as kernels of their own).
 
     1. residual add + norm + [q|k|v|z|x B C|dt] projection + conv step        (fused_gemm)
     2. attention (rotation, cache write, split context, merge) and SSM step    (mixer_decode)
@@ -25,7 +26,8 @@ from .mamba2 import Mamba2
 from .norm import RmsNorm
 from .position import NoPosition, Rope
 
-MAX_ROWS = 16          # the norm prologue recomputes the normed rows in every workgroup: small batches only
+MAX_ROWS = 64          # rows of a step the skinny kernels take
+MAX_NORM_ROWS = 16     # the norm prologue recomputes the normed rows in every workgroup: small batches only
 
 
 class ParallelDecodeFusion:
@@ -108,6 +110,9 @@ class ParallelDecodeFusion:
         bf16 = torch.bfloat16
 
         def norm_prologue(norm):
+            """The input of a projection: the norm in the kernel's prologue, or its own kernel before."""
+            if M > MAX_NORM_ROWS:
+                return dict(x=norm.forward(residual)), None          # adds the pending deltas in place
             pending = residual.pending
             h_out = torch.empty_like(residual.h) if pending else None
             arguments = dict(h_in=residual.h, deltas=pending, h_out=h_out, norm_weight=norm.weight, eps=norm.eps)
@@ -148,7 +153,8 @@ class ParallelDecodeFusion:
         activated = torch.empty((M, self.inner), dtype=bf16, device=device)
         arguments, h_out = norm_prologue(block.ffn_norm)
         ops.fused_gemm(self.w_gate_up, self.b_gate_up, activated, epilogue=ops.EPI_SWIGLU, **arguments)
-        residual.h, residual.pending = h_out, []
+        if h_out is not None:
+            residual.h, residual.pending = h_out, []
         # 5
         down = block.ffn.down
         delta = torch.empty((M, self.hidden), dtype=bf16, device=device)

@@ -273,3 +273,30 @@ def test_decode_graphs_match_eager_steps(tmp_path, name, dtype):
         both([(key, 1) for key in live])
     assert set(with_graphs.graphs._graphs) == {1, 2, 4}
     assert with_graphs.cache.stats() == eager.cache.stats()
+
+
+@pytest.mark.parametrize("requests", [24, 40])
+def test_wide_decode_batches_match_the_plain_model(tmp_path, requests):
+    """More single-token lanes than the norm-fused kernels take (16): the block's fast path with
+    norms of their own, through graphs of buckets 32 and 64, against the plain model."""
+    from macllm_infer_amd import Engine, Lane
+    folder = tiny_configs.make_model_dir("C", tmp_path, torch.bfloat16)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * requests,
+                    max_active_sequences=requests)
+    prompts = {index: tokens_for(cfg["vocab_size"], 3 + index % 7 + 6, 500 + index) for index in range(requests)}
+    for index, tokens in prompts.items():
+        engine.add_request(index)
+    engine.step([Lane(index, tokens[:-6], []) for index, tokens in prompts.items()])
+    got = {index: [] for index in prompts}
+    for turn in range(6):
+        logits = engine.step([Lane(index, [tokens[len(tokens) - 6 + turn]], [0]) for index, tokens in prompts.items()])
+        for row, index in enumerate(prompts):
+            got[index].append(logits[row].float().cpu())
+    assert set(engine.graphs._graphs) == {32 if requests <= 32 else 64}
+    for index, tokens in prompts.items():
+        want = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-6:]
+        have = torch.stack(got[index])
+        scale = want.abs().max().item()
+        assert (have - want).abs().max().item() <= 6e-2 * scale
+        assert ((have - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()).item() <= 3e-2
