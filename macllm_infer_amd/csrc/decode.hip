@@ -397,7 +397,8 @@ extern "C" int mi_fused_gemm_supported(int pro, int M, int K) {
 // ---------------------------------------------------------------- mixer decode
 #define MX_THREADS 512
 #define MX_WAVES 8
-#define MX_MAX_PAGES 4096
+#define MX_MAX_PAGES 80        // page ids of one run of keys (at most MX_SPLIT_KEYS / 8 + 2)
+#define MX_SPLIT_KEYS 512
 #define MX_SCAN_PER_THREAD 8
 
 struct MixerParams {
@@ -432,6 +433,11 @@ struct MixerParams {
   float* ssm_y;           // or float32 y before the gate (when a grouped norm follows)
   long out_ld;
   int attention_blocks;
+  // the context of a request is cut into runs of split_keys keys, one workgroup each; their
+  // partial results [M, Hq, splits, DH + 2] = (maximum, normalizer, sums) are merged by mixer_merge_kernel
+  int splits;
+  int split_keys;
+  float* partial;
 };
 
 // one dim of a rotated head: pairs (j, j + rotary_dim/2) of the first rotary_dim dims;
@@ -446,18 +452,21 @@ __device__ __forceinline__ float rotated_dim(const bf16_t* head, int dim, int ro
 }
 
 // Latency matters more than bandwidth here (a request's K and V for one layer are about a
-// megabyte), and a synchronization between workgroups costs more than the whole read, so one
-// workgroup serves one (token, kv head) alone.  Its waves take contiguous runs of keys and work
-// through them on the matrix cores without talking to each other (attn_mfma.h, with the query
-// heads of the kv head as the columns), and merge once through LDS at the end.  The new
-// token's rotated key and its value are written to their cache cell first, so the run reads
-// them like any other key.
+// megabyte): what a workgroup does is a chain of dependent memory round trips, so the context is
+// cut into runs of split_keys keys, one workgroup per (token, kv head, run), each wave of which
+// asks for all its keys at once (64 keys: two steps of attn_mfma.h in flight, the query heads of
+// the kv head as the columns).  The waves merge through LDS and the workgroup leaves (maximum,
+// normalizer, sums) per head; a small kernel merges the runs (a merge inside this kernel would
+// need a device-wide fence, which costs more than the whole read).  The new token's rotated key
+// and its value are written to their cache cell by the workgroup whose run holds it, before it
+// reads, so the run reads them like any other key.
 template <int DH>
 __device__ void mixer_attention_block(const MixerParams& p, int block, int* pages_lds, float* cs,
                                       float* merge_lds) {
   const int G = p.Hq / p.Hkv;
-  const int kvh = block % p.Hkv;
-  const long token = block / p.Hkv;
+  const int split = block % p.splits;
+  const int kvh = (block / p.splits) % p.Hkv;
+  const long token = block / (p.splits * p.Hkv);
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
@@ -467,8 +476,7 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
   const int* table = p.block_tables + token * p.max_pages;
   const int half = p.rotary_dim / 2;
 
-  // ---- round 1: the position, and what does not depend on it
-  const int pos = p.positions[token];
+  // ---- what does not depend on the position: the query heads
   mfma_bf16x8 q_own[DH / 32], q_pair[DH / 32];
   const bool has_head = n < G;
 #pragma unroll
@@ -479,23 +487,26 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
     if (p.inv_freq && own_dim < p.rotary_dim)
       q_pair[kk] = *reinterpret_cast<const mfma_bf16x8*>(head + (own_dim < half ? own_dim + half : own_dim - half));
   }
+
+  // ---- this workgroup's run of keys
+  const int pos = p.positions[token];
+  int first_key = 0;
+  if (p.window > 0 && pos - p.window + 1 > 0) first_key = pos - p.window + 1;
+  const int base_key = (first_key / p.page_size) * p.page_size;       // a page edge
+  const int run_lo = base_key + split * p.split_keys;
+  if (run_lo > pos) return;                                            // nothing of this request here
+  const int run_hi = min(run_lo + p.split_keys, pos + 1);
+  const bool writer = run_hi == pos + 1;                               // the run that holds the new token
+  const int base_page = run_lo / p.page_size;
   float k_raw = 0.f, k_raw_pair = 0.f, v_raw = 0.f;
-  if (tid < DH) {
+  if (writer && tid < DH) {
     const bf16_t* k_head = row + p.k_col + kvh * DH;
     k_raw = (float)k_head[tid];
     if (p.inv_freq && tid < p.rotary_dim) k_raw_pair = (float)k_head[tid < half ? tid + half : tid - half];
     v_raw = (float)row[p.v_col + kvh * DH + tid];
   }
-  if (p.window == 0) {                      // the range starts at key 0: its pages are known already
-    for (int t = tid; t < p.max_pages && t < MX_MAX_PAGES; t += MX_THREADS) pages_lds[t] = table[t];
-  }
-
-  int first_key = 0;
-  if (p.window > 0 && pos - p.window + 1 > 0) first_key = pos - p.window + 1;
-  const int base_key = (first_key / p.page_size) * p.page_size;       // a page edge
-  const int base_page = base_key / p.page_size;
-  if (p.window != 0) {
-    const int last_page = pos / p.page_size;
+  {
+    const int last_page = (run_hi - 1) / p.page_size;
     for (int t = tid; t <= last_page - base_page; t += MX_THREADS) pages_lds[t] = table[base_page + t];
   }
   if (p.inv_freq) {
@@ -509,7 +520,7 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
   __syncthreads();
 
   // the new token's key (rotated) and value go to their cache cell
-  if (tid < DH) {
+  if (writer && tid < DH) {
     float k = k_raw;
     if (p.inv_freq && tid < p.rotary_dim) {
       const int j = tid < half ? tid : tid - half;
@@ -541,15 +552,14 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
   __threadfence_block();
   __syncthreads();
 
-  // ---- this wave's run of keys
-  const int total = pos + 1 - base_key;
-  int span = (total + MX_WAVES - 1) / MX_WAVES;
+  // ---- this wave's share of the run
+  int span = (p.split_keys + MX_WAVES - 1) / MX_WAVES;
   span = ((span + 63) / 64) * 64;
-  const int wave_lo = base_key + wave * span;
-  const int wave_hi = min(wave_lo + span, pos + 1);
+  const int wave_lo = run_lo + wave * span;
+  const int wave_hi = min(wave_lo + span, run_hi);
   AttnAccumulator<DH, 1> acc;
   acc.clear();
-  if (wave_lo <= pos) {
+  if (wave_lo < run_hi) {
     AttnCache cache;
     cache.k_base = p.k_base;
     cache.v_base = p.v_base;
@@ -590,7 +600,34 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
       denominator += weight * theirs[1];
       sum += weight * theirs[2 + dim];
     }
-    p.attn_out[token * p.out_ld + (long)(kvh * G + g) * DH + dim] = (bf16_t)(sum / denominator);
+    float* mine = p.partial + ((token * p.Hq + kvh * G + g) * p.splits + split) * (long)(DH + 2);
+    if (dim == 0) {
+      mine[0] = maximum;
+      mine[1] = denominator;
+    }
+    mine[2 + dim] = sum;
+  }
+}
+
+// out[token, head, :] = sum_s exp(m_s - m) o_s / sum_s exp(m_s - m) l_s over the runs that hold keys.
+__global__ void mixer_merge_kernel(MixerParams p, int dh) {
+  const long token = blockIdx.x;
+  const int head = blockIdx.y;
+  const int pos = p.positions[token];
+  int first_key = 0;
+  if (p.window > 0 && pos - p.window + 1 > 0) first_key = pos - p.window + 1;
+  const int base_key = (first_key / p.page_size) * p.page_size;
+  const int used = min(p.splits, (pos - base_key) / p.split_keys + 1);
+  const float* runs = p.partial + (token * p.Hq + head) * p.splits * (long)(dh + 2);
+  float maximum = -INFINITY;
+  for (int s = 0; s < used; ++s) maximum = fmaxf(maximum, runs[(long)s * (dh + 2)]);
+  float denominator = 0.f;
+  for (int s = 0; s < used; ++s) denominator += __expf(runs[(long)s * (dh + 2)] - maximum) * runs[(long)s * (dh + 2) + 1];
+  const float inverse = 1.f / denominator;
+  for (int dim = threadIdx.x; dim < dh; dim += blockDim.x) {
+    float sum = 0.f;
+    for (int s = 0; s < used; ++s) sum += __expf(runs[(long)s * (dh + 2)] - maximum) * runs[(long)s * (dh + 2) + 2 + dim];
+    p.attn_out[token * p.out_ld + (long)head * dh + dim] = (bf16_t)(sum * inverse);
   }
 }
 
@@ -675,14 +712,14 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
                                const int* positions, const int* slot_mapping, float scale, int window,
                                int max_seq_len, int H, int P, int N, int G, int z_col, int x_col, int dt_col, const float* dt_bias,
                                const float* A, const float* D, float* ssm_state, const int* slot_ids,
-                               void* attn_out, void* ssm_out, float* ssm_y, long out_ld, hipStream_t stream) {
+                               void* attn_out, void* ssm_out, float* ssm_y, long out_ld, float* partial,
+                               long partial_floats, hipStream_t stream) {
   if (M <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || H <= 0 || P <= 0 || N <= 0 || G <= 0 || H % G != 0)
     return ERR_BAD_ARGUMENT;
   const int group = Hq / Hkv;
-  // the page ids of a request's whole visible range are staged in LDS
   const long span = window > 0 ? (long)window + page_size : (long)max_seq_len;
-  if ((dh != 64 && dh != 128) || group > 8 || page_size % 8 != 0 || max_seq_len <= 0 ||
-      span / page_size + 2 > MX_MAX_PAGES || N > WAVE * MX_SCAN_PER_THREAD ||
+  if ((dh != 64 && dh != 128) || group > 8 || page_size % 8 != 0 || page_size > MX_SPLIT_KEYS || max_seq_len <= 0 ||
+      N > WAVE * MX_SCAN_PER_THREAD ||
       u_ld % 8 != 0 || q_col % 8 != 0 || rotary_dim > dh || rotary_dim % 16 != 0)
     return ERR_UNSUPPORTED_SIZE;
   MixerParams p;
@@ -737,11 +774,19 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
   p.ssm_out = (bf16_t*)ssm_out;
   p.ssm_y = ssm_y;
   p.out_ld = out_ld;
-  p.attention_blocks = Hkv * M;
+  p.split_keys = (MX_SPLIT_KEYS / page_size) * page_size;          // whole pages
+  p.splits = (int)((span + p.split_keys - 1) / p.split_keys);
+  if ((long)Hkv * M * p.splits > 0x3fffffffL || M > 65535 || Hq > 65535) return ERR_UNSUPPORTED_SIZE;
+  if (!partial || partial_floats < (long)M * Hq * p.splits * (dh + 2)) return ERR_BAD_ARGUMENT;
+  p.partial = partial;
+  p.attention_blocks = Hkv * M * p.splits;
   const long total = (long)p.attention_blocks + (long)p.p_tiles * H * M;
   if (total > 0x7fffffffL) return ERR_UNSUPPORTED_SIZE;
   if (dh == 64) mixer_decode_kernel<64><<<(unsigned)total, MX_THREADS, 0, stream>>>(p);
   else mixer_decode_kernel<128><<<(unsigned)total, MX_THREADS, 0, stream>>>(p);
+  RETURN_IF_LAUNCH_FAILED();
+  const dim3 merge_grid(M, Hq);
+  mixer_merge_kernel<<<merge_grid, dh, 0, stream>>>(p, dh);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

@@ -73,7 +73,8 @@ _SIGNATURES = {
         "mi_mixer_decode": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int,
                             _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int,
                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                            _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr],
+                            _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr, _c_long,
+                            _c_ptr],
     },
     "sampling": {
         "mi_apply_penalties": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
@@ -613,9 +614,8 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
 
 def mixer_decode_supported(num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, state_size: int,
                            max_seq_len: int = 1, window: Optional[int] = None, rotary_dim: int = 0) -> bool:
-    span = max_seq_len if not window else window + page_size
-    return (head_dim in (64, 128) and num_heads // num_kv_heads <= 8 and page_size % 8 == 0 and state_size <= 512
-            and span // page_size + 2 <= 4096 and rotary_dim % 16 == 0)
+    return (head_dim in (64, 128) and num_heads // num_kv_heads <= 8 and page_size % 8 == 0 and page_size <= 512
+            and state_size <= 512 and rotary_dim % 16 == 0)
 
 
 def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int, q_col: int, k_col: int,
@@ -655,13 +655,17 @@ def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim
     widest = max(q_col + num_heads * head_dim, k_col + num_kv_heads * head_dim, v_col + num_kv_heads * head_dim,
                  z_col + E, x_col + E + 2 * num_groups * state_size, dt_col + ssm_heads)
     _need(u.shape[1] >= widest, "mixer_decode: u is too narrow")
+    span = max(1, int(max_seq_len)) if not window else window + page_size
+    split_keys = (512 // page_size) * page_size
+    partial = torch.empty((M * num_heads * (-(-span // split_keys)) * (head_dim + 2),), dtype=torch.float32,
+                          device=u.device)
     _check(_fn("decode", "mi_mixer_decode")(
         _p(u), u_ld, M, num_heads, num_kv_heads, head_dim, q_col, k_col, v_col, _p(inv_freq), rotary_dim,
         _p(k_cache), _p(v_cache), page_stride, page_size, _p(block_tables), block_tables.shape[1], _p(positions),
         _p(slot_mapping), float(scale), int(window or 0), int(max_seq_len), ssm_heads, ssm_head_dim, state_size,
         num_groups, z_col, x_col, dt_col, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(slot_ids), _p(out),
         out.data_ptr() + 2 * num_heads * head_dim,
-        _p(ssm_y), out_ld, _stream()), "mixer_decode")
+        _p(ssm_y), out_ld, _p(partial), partial.numel(), _stream()), "mixer_decode")
 
 
 # --------------------------------------------------------------------------- sampling
