@@ -74,7 +74,6 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
 
-  // the first weight fragments do not depend on anything: request them before the prologue
   const int n0 = blockIdx.x * 16;
   const int q = lane / 16;
   const int r = lane % 16;
@@ -87,126 +86,152 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   const int iterations = max(0, min(per_wave, chunks - first_chunk));
   constexpr int BATCH = 8;
   bf16x8_t a[BATCH];
-  if (iterations > 0) {
-#pragma unroll
-    for (int j = 0; j < BATCH; ++j) {
-      const int c = first_chunk + min(j, iterations - 1);
-      a[j] = *reinterpret_cast<const bf16x8_t*>(w_row + c * 32);
-    }
-  }
-  // so does the conv tail of the element this thread finishes in the epilogue (one element per
-  // thread when the block has 16 x 16 outputs)
-  bf16_t tail_values[8];
-  bool tail_ready = false;
-  if (EPI == EPI_CONV && MT == 1 && FG_THREADS == 256 && p.conv_k <= 9) {
-    const int n = n0 + 4 * ((tid % 64) / 16) + (tid / 64);
-    const int m = tid % 16;
-    if (n >= p.conv_lo && n < p.conv_hi && m < p.M) {
-      const int channels = p.conv_hi - p.conv_lo;
-      const bf16_t* tail = p.conv_state + (long)p.slot_ids[m] * (p.conv_k - 1) * channels + (n - p.conv_lo);
-#pragma unroll
-      for (int k = 0; k < 8; ++k)
-        if (k < p.conv_k - 1) tail_values[k] = tail[(long)k * channels];
-      tail_ready = true;
-    }
+
+  // the slot of the row whose conv tail this thread will need: asked for before everything else,
+  // because the tail's address waits for it
+  int tail_slot = 0, tail_n = 0;
+  bool tail_wanted = false;
+  if (EPI == EPI_CONV && MT == 1 && FG_THREADS == 256 && p.conv_k >= 2 && p.conv_k <= 9) {
+    tail_n = n0 + 4 * ((tid % 64) / 16) + (tid / 64);
+    tail_slot = p.slot_ids[min(tid % 16, p.M - 1)];
+    tail_wanted = tail_n >= p.conv_lo && tail_n < p.conv_hi && tid % 16 < p.M;
   }
 
-  if (PRO == PRO_NORM) {
-    // one wave per row, four rows at a time: the rows are read once into registers (K <= 2048),
-    // their sums of squares reduced in float32, and the normalized rows written in bfloat16
-    constexpr int MAXV = 8;
-    const bool in_registers = K <= MAXV * WAVE * 4;
-    for (int m0 = 0; m0 < MT * 16; m0 += FG_WAVES * 4) {
-      floatx4 v[4][MAXV];
-      if (in_registers) {
+  // Loads come back in the order they were asked for, and a wait counts all of them.  The rows
+  // to normalize (written by the kernels before, so close by) are asked for first, two rows a
+  // wave and without a branch between the loads (a row past M or an absent delta reads a valid
+  // address and is not used); the weights, which stream from memory, right after: the norm is
+  // computed while the weights are on their way.
+  constexpr int MAXV = FG_WAVES == 8 ? 8 : 4;       // 8 waves are launched for K > 1024 only
+  const bool in_registers = PRO == PRO_NORM && K <= MAXV * WAVE * 4;
+  floatx4 hv[2][MAXV];
+  bf16x4_t d0v[2][MAXV], d1v[2][MAXV];
+  floatx4 norm_weight[MAXV];
+  const bool has0 = p.delta0 != nullptr, has1 = p.delta1 != nullptr;
+  auto load_pair = [&](int m0, int pair) {
+    long at[2][MAXV];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int m = m0 + wave + t * FG_WAVES;
-          if (m < p.M) {
-            const float* h_row = p.h_in + (long)m * K;
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int i = 0; i < MAXV; ++i)
+        at[tt][i] = (long)min(m0 + wave + (2 * pair + tt) * FG_WAVES, p.M - 1) * K + min(lane * 4 + i * WAVE * 4, K - 4);
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int i = 0; i < MAXV; ++i) hv[tt][i] = *reinterpret_cast<const floatx4*>(p.h_in + at[tt][i]);
+    if (has0) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int i = 0; i < MAXV; ++i) d0v[tt][i] = *reinterpret_cast<const bf16x4_t*>(p.delta0 + at[tt][i]);
+    }
+    if (has1) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int i = 0; i < MAXV; ++i) d1v[tt][i] = *reinterpret_cast<const bf16x4_t*>(p.delta1 + at[tt][i]);
+    }
+  };
+  if (in_registers) {
+    load_pair(0, 0);
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i)
+      norm_weight[i] = *reinterpret_cast<const floatx4*>(p.norm_w + min(lane * 4 + i * WAVE * 4, K - 4));
+  }
+#pragma unroll
+  for (int j = 0; j < BATCH; ++j)      // no condition around these loads: a wave without chunks reads the last one
+    a[j] = *reinterpret_cast<const bf16x8_t*>(w_row + min(first_chunk + min(j, max(iterations, 1) - 1), chunks - 1) * 32);
+  if (PRO == PRO_NORM) {
+    // one wave per row, two rows at a time: the rows are read once into registers (K <= 2048),
+    // their sums of squares reduced in float32, and the normalized rows written in bfloat16
+    for (int m0 = 0; m0 < MT * 16; m0 += FG_WAVES * 4) {
+#pragma unroll
+      for (int pair = 0; pair < 2; ++pair) {
+        if (in_registers && (m0 > 0 || pair > 0) && m0 + wave + 2 * pair * FG_WAVES < p.M) load_pair(m0, pair);
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+          const int m = m0 + wave + (2 * pair + tt) * FG_WAVES;
+          if (m >= MT * 16) continue;
+          bf16_t* x_row = xs + (long)m * ldx;
+          if (m >= p.M) {
+            for (int k = lane * 4; k < K; k += WAVE * 4) {
+              const bf16x4_t zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+              *reinterpret_cast<bf16x4_t*>(x_row + k) = zero;
+            }
+            continue;
+          }
+          const float* h_row = p.h_in + (long)m * K;
+          auto row_value = [&](int k) {
+            floatx4 value = *reinterpret_cast<const floatx4*>(h_row + k);
+            if (has0) {
+              const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(p.delta0 + (long)m * K + k);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) value[j] += (float)d[j];
+            }
+            if (has1) {
+              const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(p.delta1 + (long)m * K + k);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) value[j] += (float)d[j];
+            }
+            return value;
+          };
+          float sum_squares = 0.f;
+          if (in_registers) {
+#pragma unroll
+            for (int i = 0; i < MAXV; ++i) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                float value = hv[tt][i][j];
+                if (has0) value += (float)d0v[tt][i][j];
+                if (has1) value += (float)d1v[tt][i][j];
+                hv[tt][i][j] = value;
+                if (lane * 4 + i * WAVE * 4 < K) sum_squares += value * value;
+              }
+            }
+          } else {
+            for (int k = lane * 4; k < K; k += WAVE * 4) {
+              const floatx4 value = row_value(k);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) sum_squares += value[j] * value[j];
+            }
+          }
+          sum_squares = wave_sum(sum_squares);
+          const float inverse = 1.0f / sqrtf(sum_squares / (float)K + p.eps);
+          auto finish = [&](int k, const floatx4& value, const floatx4& w) {
+            if (blockIdx.x == 0 && p.h_out) *reinterpret_cast<floatx4*>(p.h_out + (long)m * K + k) = value;
+            bf16x4_t packed;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) packed[j] = (bf16_t)(value[j] * inverse * w[j]);
+            *reinterpret_cast<bf16x4_t*>(x_row + k) = packed;
+          };
+          if (in_registers) {
 #pragma unroll
             for (int i = 0; i < MAXV; ++i) {
               const int k = lane * 4 + i * WAVE * 4;
-              if (k < K) {
-                v[t][i] = *reinterpret_cast<const floatx4*>(h_row + k);
-                if (p.delta0) {
-                  const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(p.delta0 + (long)m * K + k);
-#pragma unroll
-                  for (int j = 0; j < 4; ++j) v[t][i][j] += (float)d[j];
-                }
-                if (p.delta1) {
-                  const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(p.delta1 + (long)m * K + k);
-#pragma unroll
-                  for (int j = 0; j < 4; ++j) v[t][i][j] += (float)d[j];
-                }
-              }
+              if (k < K) finish(k, hv[tt][i], norm_weight[i]);
             }
+          } else {
+            for (int k = lane * 4; k < K; k += WAVE * 4)
+              finish(k, row_value(k), *reinterpret_cast<const floatx4*>(p.norm_w + k));
           }
-        }
-      }
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int m = m0 + wave + t * FG_WAVES;
-        if (m >= MT * 16) continue;
-        bf16_t* x_row = xs + (long)m * ldx;
-        if (m >= p.M) {
-          for (int k = lane * 4; k < K; k += WAVE * 4) {
-            const bf16x4_t zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
-            *reinterpret_cast<bf16x4_t*>(x_row + k) = zero;
-          }
-          continue;
-        }
-        const float* h_row = p.h_in + (long)m * K;
-        auto row_value = [&](int k) {
-          floatx4 value = *reinterpret_cast<const floatx4*>(h_row + k);
-          if (p.delta0) {
-            const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(p.delta0 + (long)m * K + k);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) value[j] += (float)d[j];
-          }
-          if (p.delta1) {
-            const bf16x4_t d = *reinterpret_cast<const bf16x4_t*>(p.delta1 + (long)m * K + k);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) value[j] += (float)d[j];
-          }
-          return value;
-        };
-        float sum_squares = 0.f;
-        if (in_registers) {
-#pragma unroll
-          for (int i = 0; i < MAXV; ++i)
-            if (lane * 4 + i * WAVE * 4 < K)
-#pragma unroll
-              for (int j = 0; j < 4; ++j) sum_squares += v[t][i][j] * v[t][i][j];
-        } else {
-          for (int k = lane * 4; k < K; k += WAVE * 4) {
-            const floatx4 value = row_value(k);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) sum_squares += value[j] * value[j];
-          }
-        }
-        sum_squares = wave_sum(sum_squares);
-        const float inverse = 1.0f / sqrtf(sum_squares / (float)K + p.eps);
-        auto finish = [&](int k, const floatx4& value) {
-          if (blockIdx.x == 0 && p.h_out) *reinterpret_cast<floatx4*>(p.h_out + (long)m * K + k) = value;
-          const floatx4 w = *reinterpret_cast<const floatx4*>(p.norm_w + k);
-          bf16x4_t packed;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) packed[j] = (bf16_t)(value[j] * inverse * w[j]);
-          *reinterpret_cast<bf16x4_t*>(x_row + k) = packed;
-        };
-        if (in_registers) {
-#pragma unroll
-          for (int i = 0; i < MAXV; ++i) {
-            const int k = lane * 4 + i * WAVE * 4;
-            if (k < K) finish(k, v[t][i]);
-          }
-        } else {
-          for (int k = lane * 4; k < K; k += WAVE * 4) finish(k, row_value(k));
         }
       }
     }
     __syncthreads();
+  }
+
+  // the conv tail of the element this thread finishes in the epilogue (one element per thread
+  // when the block has 16 x 16 outputs) is asked for now, behind the weights; no branch between
+  // its loads either
+  bf16_t tail_values[8];
+  bool tail_ready = false;
+  if (EPI == EPI_CONV) asm volatile("" : "+v"(tail_slot));      // keeps every use of the slot (and its wait) down here
+  if (tail_wanted) {
+    const int channels = p.conv_hi - p.conv_lo;
+    const bf16_t* tail = p.conv_state + (long)tail_slot * (p.conv_k - 1) * channels + (tail_n - p.conv_lo);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) tail_values[k] = tail[(long)min(k, p.conv_k - 2) * channels];
+    tail_ready = true;
   }
 
   // the product: eight weight fragments are requested before the first is used, so that a
