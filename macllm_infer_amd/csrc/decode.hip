@@ -501,20 +501,31 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
   const int* table = p.block_tables + token * p.max_pages;
   const int half = p.rotary_dim / 2;
 
-  // ---- what does not depend on the position: the query heads
+  // ---- everything that does not depend on the position is asked for at once, with no branch
+  // between the loads (an index that is not needed is clamped to one that is valid): the query
+  // heads, the new key and value, the cache cell, the rotation frequencies
+  const bool rotate = p.inv_freq != nullptr;
   mfma_bf16x8 q_own[DH / 32], q_pair[DH / 32];
   const bool has_head = n < G;
+  const bf16_t* q_head = row + p.q_col + (kvh * G + (has_head ? n : 0)) * DH;
 #pragma unroll
   for (int kk = 0; kk < DH / 32; ++kk) {
     const int own_dim = 32 * kk + 8 * qd;
-    const bf16_t* head = row + p.q_col + (kvh * G + (has_head ? n : 0)) * DH;
-    q_own[kk] = *reinterpret_cast<const mfma_bf16x8*>(head + own_dim);
-    if (p.inv_freq && own_dim < p.rotary_dim)
-      q_pair[kk] = *reinterpret_cast<const mfma_bf16x8*>(head + (own_dim < half ? own_dim + half : own_dim - half));
+    const int pair_dim = own_dim < p.rotary_dim ? (own_dim < half ? own_dim + half : own_dim - half) : own_dim;
+    q_own[kk] = *reinterpret_cast<const mfma_bf16x8*>(q_head + own_dim);
+    q_pair[kk] = *reinterpret_cast<const mfma_bf16x8*>(q_head + pair_dim);
   }
+  const int pos = p.positions[token];
+  const long cell = p.slot_mapping[token];
+  const int k_dim = min(tid, DH - 1);
+  const int k_pair_dim = k_dim < p.rotary_dim ? (k_dim < half ? k_dim + half : k_dim - half) : k_dim;
+  const bf16_t* k_head = row + p.k_col + kvh * DH;
+  const bf16_t k_raw_bits = k_head[k_dim];
+  const bf16_t k_pair_bits = k_head[k_pair_dim];
+  const bf16_t v_raw_bits = row[p.v_col + kvh * DH + k_dim];
+  const float frequency = rotate ? p.inv_freq[min(tid, max(half, 1) - 1)] : 0.f;
 
   // ---- this workgroup's run of keys
-  const int pos = p.positions[token];
   int first_key = 0;
   if (p.window > 0 && pos - p.window + 1 > 0) first_key = pos - p.window + 1;
   const int base_key = (first_key / p.page_size) * p.page_size;       // a page edge
@@ -523,20 +534,19 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
   const int run_hi = min(run_lo + p.split_keys, pos + 1);
   const bool writer = run_hi == pos + 1;                               // the run that holds the new token
   const int base_page = run_lo / p.page_size;
-  float k_raw = 0.f, k_raw_pair = 0.f, v_raw = 0.f;
-  if (writer && tid < DH) {
-    const bf16_t* k_head = row + p.k_col + kvh * DH;
-    k_raw = (float)k_head[tid];
-    if (p.inv_freq && tid < p.rotary_dim) k_raw_pair = (float)k_head[tid < half ? tid + half : tid - half];
-    v_raw = (float)row[p.v_col + kvh * DH + tid];
-  }
   {
     const int last_page = (run_hi - 1) / p.page_size;
     for (int t = tid; t <= last_page - base_page; t += MX_THREADS) pages_lds[t] = table[base_page + t];
   }
-  if (p.inv_freq) {
+  const float k_raw = (float)k_raw_bits, k_raw_pair = (float)k_pair_bits, v_raw = (float)v_raw_bits;
+  if (rotate) {
     const float position = (float)pos;
-    for (int j = tid; j < half; j += MX_THREADS) {
+    if (tid < half) {
+      const float angle = position * frequency;
+      cs[tid] = cosf(angle);
+      cs[half + tid] = sinf(angle);
+    }
+    for (int j = tid + MX_THREADS; j < half; j += MX_THREADS) {      // head sizes beyond the workgroup: none today
       const float angle = position * p.inv_freq[j];
       cs[j] = cosf(angle);
       cs[half + j] = sinf(angle);
@@ -547,11 +557,10 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
   // the new token's key (rotated) and value go to their cache cell
   if (writer && tid < DH) {
     float k = k_raw;
-    if (p.inv_freq && tid < p.rotary_dim) {
+    if (rotate && tid < p.rotary_dim) {
       const int j = tid < half ? tid : tid - half;
       k = tid < half ? k_raw * cs[j] - k_raw_pair * cs[half + j] : k_raw * cs[j] + k_raw_pair * cs[half + j];
     }
-    const long cell = p.slot_mapping[token];
     const long page = cell / p.page_size;
     const int offset = (int)(cell - page * p.page_size);
     p.k_base[page * p.page_stride + ((long)kvh * p.page_size + offset) * DH + tid] = (bf16_t)k;
@@ -565,7 +574,7 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       float value = (float)q_own[kk][j];
-      if (p.inv_freq && own_dim < p.rotary_dim) {
+      if (rotate && own_dim < p.rotary_dim) {
         const int dim = own_dim + j;
         const int f = dim < half ? dim : dim - half;
         value = dim < half ? value * cs[f] - (float)q_pair[kk][j] * cs[half + f]
@@ -635,25 +644,44 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
 }
 
 // out[token, head, :] = sum_s exp(m_s - m) o_s / sum_s exp(m_s - m) l_s over the runs that hold keys.
+// Eight runs are asked for at once, before it is known how many hold keys (the position is on
+// its way too); what a run without keys left in its place is read and not used.
 __global__ void mixer_merge_kernel(MixerParams p, int dh) {
   const long token = blockIdx.x;
   const int head = blockIdx.y;
-  const int pos = p.positions[token];
-  int first_key = 0;
-  if (p.window > 0 && pos - p.window + 1 > 0) first_key = pos - p.window + 1;
-  const int base_key = (first_key / p.page_size) * p.page_size;
-  const int used = min(p.splits, (pos - base_key) / p.split_keys + 1);
+  const int dim = min((int)threadIdx.x, dh - 1);
   const float* runs = p.partial + (token * p.Hq + head) * p.splits * (long)(dh + 2);
-  float maximum = -INFINITY;
-  for (int s = 0; s < used; ++s) maximum = fmaxf(maximum, runs[(long)s * (dh + 2)]);
-  float denominator = 0.f;
-  for (int s = 0; s < used; ++s) denominator += __expf(runs[(long)s * (dh + 2)] - maximum) * runs[(long)s * (dh + 2) + 1];
-  const float inverse = 1.f / denominator;
-  for (int dim = threadIdx.x; dim < dh; dim += blockDim.x) {
-    float sum = 0.f;
-    for (int s = 0; s < used; ++s) sum += __expf(runs[(long)s * (dh + 2)] - maximum) * runs[(long)s * (dh + 2) + 2 + dim];
-    p.attn_out[token * p.out_ld + (long)head * dh + dim] = (bf16_t)(sum * inverse);
+  const int pos = p.positions[token];
+  float maximum = -INFINITY, denominator = 0.f, sum = 0.f;
+  int used = p.splits;
+  for (int s0 = 0; s0 < used; s0 += 8) {
+    float m_s[8], l_s[8], o_s[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float* run = runs + (long)min(s0 + j, p.splits - 1) * (dh + 2);
+      m_s[j] = run[0];
+      l_s[j] = run[1];
+      o_s[j] = run[2 + dim];
+    }
+    if (s0 == 0) {
+      int first_key = 0;
+      if (p.window > 0 && pos - p.window + 1 > 0) first_key = pos - p.window + 1;
+      const int base_key = (first_key / p.page_size) * p.page_size;
+      used = min(p.splits, (pos - base_key) / p.split_keys + 1);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (s0 + j < used) {
+        const float larger = fmaxf(maximum, m_s[j]);
+        const float keep = __expf(maximum - larger);        // 0 the first time (maximum = -inf)
+        const float weight = __expf(m_s[j] - larger);
+        denominator = denominator * keep + weight * l_s[j];
+        sum = sum * keep + weight * o_s[j];
+        maximum = larger;
+      }
+    }
   }
+  if ((int)threadIdx.x < dh) p.attn_out[token * p.out_ld + (long)head * dh + dim] = (bf16_t)(sum / denominator);
 }
 
 // One step of the selective scan for (token, head, tile of state rows); see ssm_scan_kernel.
@@ -674,19 +702,29 @@ __device__ void mixer_ssm_block(const MixerParams& p, int block) {
   const int N = p.N;
   const bf16_t* row = p.u + token * p.u_ld;
   float* s_row = p.ssm_state + (((long)p.slot_ids[token] * p.H + head) * p.P + (active ? pi : 0)) * N;
-  const float delta = softplus_f((float)row[p.dt_col + head] + p.dt_bias[head]);
-  const float decay = expf(delta * p.A[head]);
-  const float x = active ? (float)row[p.x_col + head * p.P + pi] : 0.f;
   const bf16_t* b_row = row + p.x_col + p.H * p.P + group * N;
   const bf16_t* c_row = b_row + p.G * N;
+  const long column = (long)head * p.P + (active ? pi : 0);
+  // every load of the step is asked for before the first is used (the state first: it comes from
+  // furthest away), with no branch between them
+  floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+  bf16x8_t b, c;
+  if (VECTOR) {
+    s0 = *reinterpret_cast<const floatx4*>(s_row + r * 8);
+    s1 = *reinterpret_cast<const floatx4*>(s_row + r * 8 + 4);
+    b = *reinterpret_cast<const bf16x8_t*>(b_row + r * 8);
+    c = *reinterpret_cast<const bf16x8_t*>(c_row + r * 8);
+  }
+  const bf16_t dt_bits = row[p.dt_col + head];
+  const bf16_t x_bits = row[p.x_col + column];
+  const bf16_t z_bits = row[p.z_col + column];
+  const float delta = softplus_f((float)dt_bits + p.dt_bias[head]);
+  const float decay = expf(delta * p.A[head]);
+  const float x = active ? (float)x_bits : 0.f;
   const float dx = delta * x;
   float partial = 0.f;
   if (VECTOR) {
     if (active) {
-      floatx4 s0 = *reinterpret_cast<const floatx4*>(s_row + r * 8);
-      floatx4 s1 = *reinterpret_cast<const floatx4*>(s_row + r * 8 + 4);
-      const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(b_row + r * 8);
-      const bf16x8_t c = *reinterpret_cast<const bf16x8_t*>(c_row + r * 8);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         s0[i] = decay * s0[i] + dx * (float)b[i];
@@ -712,9 +750,8 @@ __device__ void mixer_ssm_block(const MixerParams& p, int block) {
   for (int offset = R / 2; offset > 0; offset >>= 1) partial += __shfl_xor(partial, offset, WAVE);
   if (active && r == 0) {
     const float y = partial + p.D[head] * x;
-    const long column = (long)head * p.P + pi;
     if (p.ssm_y) p.ssm_y[token * (long)(p.H * p.P) + column] = y;
-    else p.ssm_out[token * p.out_ld + column] = (bf16_t)(y * silu_f((float)row[p.z_col + column]));
+    else p.ssm_out[token * p.out_ld + column] = (bf16_t)(y * silu_f((float)z_bits));
   }
 }
 
