@@ -473,21 +473,25 @@ extern "C" int mi_decode_attention(const void* q, long q_ld, int T, int Hq, int 
 // bfloat16, head_dim 64 or 128.  grid = (4 x query tiles, kv heads, head passes): a tile is up to 64
 // consecutive tokens of one lane and a workgroup takes 16 of them with the query heads of one kv
 // head (NSET column sets that share every K and V fragment).  The keys, from the first visible
-// one to the workgroup's last position, are split in four runs of whole 32-key steps, one per
+// one to the workgroup's last position, are split in eight runs of whole 32-key steps, one per
 // wave, read straight from the cache pages (the portion's own keys were written by rope_kv_store
-// before); the four partial results are merged through LDS, set by set.  Workgroups with the
-// longest contexts (the last tiles) are launched first.
+// before), four steps in flight at a time; the eight partial results are merged through LDS,
+// set by set.  Workgroups with the longest contexts (the last tiles) are launched first.
 #include "attn_mfma.h"
 
+#define PREFILL_STEPS 4
+#define PREFILL_WAVES 8
+
 template <int DH, int NSET>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(PREFILL_WAVES * WAVE)
 prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hkv, const bf16_t* __restrict__ k_base,
                          const bf16_t* __restrict__ v_base, long page_stride, int page_size,
                          const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
                          const int* __restrict__ cu_seqlens, const int* __restrict__ start_pos, float scale,
                          int window, bf16_t* __restrict__ out, long out_ld) {
   constexpr int ITEMS = 2 + 4 * (DH / 16);                    // m, l and the accumulator of one set
-  __shared__ float part[4][ITEMS][WAVE];
+  __shared__ float part[PREFILL_WAVES][ITEMS][WAVE];
+  __shared__ int wave_pages[PREFILL_WAVES][WAVE];
   const int block = gridDim.x - 1 - blockIdx.x;               // heavy ones first
   const int tile = block / 4;
   const int kvh = blockIdx.y;
@@ -533,18 +537,27 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
   cache.page_stride = page_stride;
   cache.page_size = page_size;
   cache.kvh = kvh;
-  cache.pages = block_tables + (long)request * max_pages;
-  cache.base_page = 0;
+  const int* cache_pages = block_tables + (long)request * max_pages;
   int key_lo = 0;
   if (window > 0 && first_position - window + 1 > 0) key_lo = ((first_position - window + 1) / 32) * 32;
   const int key_hi = last_position + 1;
   const int steps = (key_hi - key_lo + 31) / 32;
-  const int steps_per_wave = (steps + 3) / 4;
+  const int steps_per_wave = (steps + PREFILL_WAVES - 1) / PREFILL_WAVES;
   const int my_lo = key_lo + 32 * steps_per_wave * wave;
   const int my_hi = min(key_hi, my_lo + 32 * steps_per_wave);
-  if (my_lo < my_hi) attend_keys<DH, NSET, 2>(acc, q_frag, col_pos, window, scale, my_lo, my_hi, cache);
+  // the page ids of the run go through LDS, 64 pages at a time (a wave's own corner of it: no
+  // barrier), so that a K or V load does not wait for a load of its page id
+  for (int part_lo = my_lo; part_lo < my_hi;) {
+    const int first_page = part_lo / page_size;
+    const int part_hi = min(my_hi, (first_page + WAVE) * page_size);
+    wave_pages[wave][lane] = cache_pages[min(first_page + lane, max_pages - 1)];
+    cache.pages = wave_pages[wave];
+    cache.base_page = first_page;
+    attend_keys<DH, NSET, PREFILL_STEPS>(acc, q_frag, col_pos, window, scale, part_lo, part_hi, cache);
+    part_lo = part_hi;
+  }
 
-  // merge: set s is finished by wave s % 4
+  // merge: set s is finished by wave s
 #pragma unroll
   for (int s = 0; s < NSET; ++s) {
     __syncthreads();
@@ -555,16 +568,16 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
 #pragma unroll
       for (int i = 0; i < 4; ++i) part[wave][2 + 4 * dt + i][lane] = acc.o[s][dt][i];
     __syncthreads();
-    if (wave != (s & 3)) continue;
+    if (wave != s % PREFILL_WAVES) continue;
     float m = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) m = fmaxf(m, part[w][0][lane]);
-    float factor[4];
+    for (int w = 0; w < PREFILL_WAVES; ++w) m = fmaxf(m, part[w][0][lane]);
+    float factor[PREFILL_WAVES];
     float l = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < PREFILL_WAVES; ++w) {
       const float m_w = part[w][0][lane];
-      factor[w] = m_w == -INFINITY ? 0.f : __expf(m_w - m);
+      factor[w] = m_w == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_w - m);
       l += part[w][1][lane] * factor[w];
     }
     l += __shfl_xor(l, 16, WAVE);
@@ -579,7 +592,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
       for (int i = 0; i < 4; ++i) {
         float value = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) value += part[w][2 + 4 * dt + i][lane] * factor[w];
+        for (int w = 0; w < PREFILL_WAVES; ++w) value += part[w][2 + 4 * dt + i][lane] * factor[w];
         packed[i] = (bf16_t)(value * inverse);
       }
       *reinterpret_cast<mfma_bf16x4*>(o + 16 * dt + 4 * qd) = packed;
@@ -605,7 +618,7 @@ extern "C" int mi_prefill_attention(const void* q, long q_ld, int Hq, int Hkv, i
   const dim3 grid(4 * n_tiles, Hkv, passes);
 #define PREFILL_CASE(DH_, NSET_)                                                                              \
   if (dh == DH_ && nset == NSET_)                                                                             \
-    prefill_attention_kernel<DH_, NSET_><<<grid, 256, 0, stream>>>(                                           \
+    prefill_attention_kernel<DH_, NSET_><<<grid, PREFILL_WAVES * WAVE, 0, stream>>>(                                           \
         (const bf16_t*)q, q_ld, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride, page_size, \
         block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld);
   PREFILL_CASE(64, 1) PREFILL_CASE(64, 2) PREFILL_CASE(64, 3) PREFILL_CASE(64, 4)

@@ -630,7 +630,7 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
 #pragma unroll
     for (int w = 0; w < MX_WAVES; ++w) {
       const float* theirs = merge_lds + (long)(w * G + g) * (DH + 2);
-      const float weight = __expf(theirs[0] - maximum);      // 0 for a wave without keys (m = -inf)
+      const float weight = __builtin_amdgcn_exp2f(theirs[0] - maximum);      // 0 for a wave without keys (m = -inf); maxima are in units of log2
       denominator += weight * theirs[1];
       sum += weight * theirs[2 + dim];
     }
@@ -673,8 +673,8 @@ __global__ void mixer_merge_kernel(MixerParams p, int dh) {
     for (int j = 0; j < 8; ++j) {
       if (s0 + j < used) {
         const float larger = fmaxf(maximum, m_s[j]);
-        const float keep = __expf(maximum - larger);        // 0 the first time (maximum = -inf)
-        const float weight = __expf(m_s[j] - larger);
+        const float keep = __builtin_amdgcn_exp2f(maximum - larger);        // 0 the first time (maximum = -inf); units of log2
+        const float weight = __builtin_amdgcn_exp2f(m_s[j] - larger);
         denominator = denominator * keep + weight * l_s[j];
         sum = sum * keep + weight * o_s[j];
         maximum = larger;
