@@ -189,14 +189,19 @@ __global__ void ssd_state_pass_kernel(const float* __restrict__ chunk_state, con
 //   intra:  for 32 tokens s at a time, W^T[s, t] = B[s, :] . C[t, :] (shared by the heads), then per
 //           head  P^T[s, t] = W^T exp(L_t - L_s) delta_s [s <= t]  and  O^T += xT[p, s] . P^T[s, t]
 //   y[t, p] = O^T[p, t] + D x[t, p];  with z given, gated[t, p] = y * SiLU(z[t, p]) is written instead.
-// Up to 64 state rows p are held at a time (PT tiles of 16); a larger head repeats the pass.
-template <int HB, int PT>
+// 64 state rows p (4 tiles of 16) are held at a time; a larger head repeats the pass.  NK = N / 32
+// is a template parameter and no load stands under a condition (a head or a tile of rows that
+// does not exist is clamped to the last that does, computed and not stored): loads come back in
+// order and a condition between them would make each wait for the one before.
+template <int HB, int NK>
 __global__ void __launch_bounds__(256)
 ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t* __restrict__ xT, int E,
                       const bf16_t* __restrict__ state_in, const float* __restrict__ delta,
                       const float* __restrict__ cum, const float* __restrict__ D, const int* __restrict__ chunks,
-                      int Q, int H, int P, int N, int G, float* __restrict__ y, long y_ld,
+                      int Q, int H, int P, int G, float* __restrict__ y, long y_ld,
                       const bf16_t* __restrict__ z, long z_ld, bf16_t* __restrict__ gated, long gated_ld) {
+  constexpr int PT = 4;
+  constexpr int N = 32 * NK;
   __shared__ float L[HB][SSD_MAX_Q];
   __shared__ float step[HB][SSD_MAX_Q];
   const int chunk = blockIdx.x;
@@ -214,14 +219,13 @@ ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t*
   if ((tile - wave) * 16 >= length) return;                      // the whole workgroup
   const int q = lane / 16;
   const int n = lane % 16;
-  const int first_s = 0;
   const int end_s = min(length, (tile - wave) * 16 + 64);        // tokens any wave of the workgroup looks at
-  for (int index = tid; index < HB * (end_s - first_s); index += 256) {
-    const int hb = index / (end_s - first_s);
-    const int s = first_s + index % (end_s - first_s);
-    const bool valid = hb < heads;
-    L[hb][s] = valid ? cum[(long)(t0 + s) * H + head0 + hb] : 0.f;
-    step[hb][s] = valid ? delta[(long)(t0 + s) * H + head0 + hb] : 0.f;
+  for (int index = tid; index < HB * end_s; index += 256) {
+    const int hb = index / end_s;
+    const int s = index % end_s;
+    const int head = head0 + min(hb, heads - 1);
+    L[hb][s] = cum[(long)(t0 + s) * H + head];
+    step[hb][s] = delta[(long)(t0 + s) * H + head];
   }
   __syncthreads();
   if (tile * 16 >= length) return;
@@ -232,42 +236,37 @@ ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t*
   const bool has_t = t < length;
   const int t_safe = min(t, length - 1);
   const long t_row = t0 + t_safe;
-  // C of the column, all of N: the B operand of both score products (N <= 256: 8 fragments)
-  s_bf16x8 c_frag[8];
+  const int p_tiles = P / 16;
+  // C of the column, all of N: the B operand of both score products
+  s_bf16x8 c_frag[NK];
 #pragma unroll
-  for (int kk = 0; kk < 8; ++kk) {
-    if (32 * kk < N) {
-      c_frag[kk] = *reinterpret_cast<const s_bf16x8*>(xbc + t_row * xbc_ld + c_col + 32 * kk + 8 * q);
-      if (!has_t) {
+  for (int kk = 0; kk < NK; ++kk)
+    c_frag[kk] = *reinterpret_cast<const s_bf16x8*>(xbc + t_row * xbc_ld + c_col + 32 * kk + 8 * q);
+  if (!has_t) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) c_frag[kk][j] = (bf16_t)0.f;
-      }
-    }
+    for (int kk = 0; kk < NK; ++kk)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) c_frag[kk][j] = (bf16_t)0.f;
   }
-  for (int pt0 = 0; pt0 < P / 16; pt0 += PT) {
+  for (int pt0 = 0; pt0 < p_tiles; pt0 += PT) {
     s_floatx4 acc[HB][PT];
     // inter-chunk term
 #pragma unroll
     for (int hb = 0; hb < HB; ++hb) {
+      const int head = head0 + min(hb, heads - 1);
+      const float carry = __expf(L[hb][t_safe]);
 #pragma unroll
-      for (int pi = 0; pi < PT; ++pi) acc[hb][pi] = s_floatx4{0.f, 0.f, 0.f, 0.f};
-      if (hb < heads) {
-        const float carry = __expf(L[hb][t_safe]);
+      for (int pi = 0; pi < PT; ++pi) {
+        const int pt = min(pt0 + pi, p_tiles - 1);
+        const bf16_t* s_rows = state_in + (((long)chunk * H + head) * P + pt * 16 + n) * N + 8 * q;
+        s_floatx4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int pi = 0; pi < PT; ++pi) {
-          if (pt0 + pi < P / 16) {
-            const bf16_t* s_rows = state_in + (((long)chunk * H + head0 + hb) * P + (pt0 + pi) * 16 + n) * N + 8 * q;
-#pragma unroll
-            for (int kk = 0; kk < 8; ++kk) {
-              if (32 * kk < N) {
-                const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(s_rows + 32 * kk);
-                acc[hb][pi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], acc[hb][pi], 0, 0, 0);
-              }
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[hb][pi][i] *= carry;
-          }
+        for (int kk = 0; kk < NK; ++kk) {
+          const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(s_rows + 32 * kk);
+          sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], sum, 0, 0, 0);
         }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[hb][pi][i] = sum[i] * carry;
       }
     }
     // intra-chunk term
@@ -278,71 +277,77 @@ ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t*
         w[half] = s_floatx4{0.f, 0.f, 0.f, 0.f};
         const long s_row = min((long)t0 + s0 + 16 * half + n, (long)last_row);
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
-          if (32 * kk < N) {
-            const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(xbc + s_row * xbc_ld + b_col + 32 * kk + 8 * q);
-            w[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], w[half], 0, 0, 0);
-          }
+        for (int kk = 0; kk < NK; ++kk) {
+          const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(xbc + s_row * xbc_ld + b_col + 32 * kk + 8 * q);
+          w[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], w[half], 0, 0, 0);
+        }
+      }
+      // the A operands of all heads and row tiles of this step: asked for before the exponentials
+      s_bf16x4 x_lo[HB][PT], x_hi[HB][PT];
+#pragma unroll
+      for (int hb = 0; hb < HB; ++hb) {
+        const int head = head0 + min(hb, heads - 1);
+#pragma unroll
+        for (int pi = 0; pi < PT; ++pi) {
+          const int pt = min(pt0 + pi, p_tiles - 1);
+          const bf16_t* x_row = xT + ((long)chunk * E + (long)head * P + pt * 16 + n) * Q + s0 + 4 * q;
+          x_lo[hb][pi] = *reinterpret_cast<const s_bf16x4*>(x_row);
+          x_hi[hb][pi] = *reinterpret_cast<const s_bf16x4*>(x_row + 16);
         }
       }
 #pragma unroll
       for (int hb = 0; hb < HB; ++hb) {
-        if (hb < heads) {
-          s_bf16x8 p_frag;
-          const float l_t = L[hb][t_safe];
+        s_bf16x8 p_frag;
+        const float l_t = L[hb][t_safe];
 #pragma unroll
-          for (int half = 0; half < 2; ++half)
+        for (int half = 0; half < 2; ++half)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int s = s0 + 16 * half + 4 * q + i;
-              const int s_safe = min(s, length - 1);
-              const bool visible = has_t && s <= t && s < length;
-              const float value = visible ? w[half][i] * __expf(l_t - L[hb][s_safe]) * step[hb][s_safe] : 0.f;
-              p_frag[4 * half + i] = (bf16_t)value;
-            }
-#pragma unroll
-          for (int pi = 0; pi < PT; ++pi) {
-            if (pt0 + pi < P / 16) {
-              const bf16_t* x_row = xT + ((long)chunk * E + (long)(head0 + hb) * P + (pt0 + pi) * 16 + n) * Q + s0 + 4 * q;
-              const s_bf16x4 lo = *reinterpret_cast<const s_bf16x4*>(x_row);
-              const s_bf16x4 hi = *reinterpret_cast<const s_bf16x4*>(x_row + 16);
-              s_bf16x8 a;
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                a[j] = lo[j];
-                a[4 + j] = hi[j];
-              }
-              acc[hb][pi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p_frag, acc[hb][pi], 0, 0, 0);
-            }
+          for (int i = 0; i < 4; ++i) {
+            const int s = s0 + 16 * half + 4 * q + i;
+            const int s_safe = min(s, length - 1);
+            const bool visible = has_t && s <= t && s < length;
+            const float value = visible ? w[half][i] * __expf(l_t - L[hb][s_safe]) * step[hb][s_safe] : 0.f;
+            p_frag[4 * half + i] = (bf16_t)value;
           }
+#pragma unroll
+        for (int pi = 0; pi < PT; ++pi) {
+          s_bf16x8 a;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            a[j] = x_lo[hb][pi][j];
+            a[4 + j] = x_hi[hb][pi][j];
+          }
+          acc[hb][pi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p_frag, acc[hb][pi], 0, 0, 0);
         }
       }
     }
-    // y[t, h*P + 16 pt + 4q + i] = acc + D x
-    if (has_t) {
+    // y[t, h*P + 16 pt + 4q + i] = acc + D x: the skip and gate operands first, then the stores
+    s_bf16x4 x_skip[HB][PT], gate[HB][PT];
 #pragma unroll
-      for (int hb = 0; hb < HB; ++hb) {
-        if (hb < heads) {
-          const float skip = D[head0 + hb];
+    for (int hb = 0; hb < HB; ++hb)
 #pragma unroll
-          for (int pi = 0; pi < PT; ++pi) {
-            if (pt0 + pi < P / 16) {
-              const long column = (long)(head0 + hb) * P + (pt0 + pi) * 16 + 4 * q;
-              const s_bf16x4 x = *reinterpret_cast<const s_bf16x4*>(xbc + t_row * xbc_ld + column);
-              s_floatx4 out;
+      for (int pi = 0; pi < PT; ++pi) {
+        const long column = (long)(head0 + min(hb, heads - 1)) * P + min(pt0 + pi, p_tiles - 1) * 16 + 4 * q;
+        x_skip[hb][pi] = *reinterpret_cast<const s_bf16x4*>(xbc + t_row * xbc_ld + column);
+        gate[hb][pi] = *reinterpret_cast<const s_bf16x4*>((z != nullptr ? z + t_row * z_ld : xbc + t_row * xbc_ld) + column);
+      }
 #pragma unroll
-              for (int i = 0; i < 4; ++i) out[i] = acc[hb][pi][i] + skip * (float)x[i];
-              if (z != nullptr) {
-                const s_bf16x4 gate = *reinterpret_cast<const s_bf16x4*>(z + t_row * z_ld + column);
-                s_bf16x4 packed;
+    for (int hb = 0; hb < HB; ++hb) {
+      const float skip = D[head0 + min(hb, heads - 1)];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(out[i] * silu_f((float)gate[i]));
-                *reinterpret_cast<s_bf16x4*>(gated + t_row * gated_ld + column) = packed;
-              } else {
-                *reinterpret_cast<s_floatx4*>(y + t_row * y_ld + column) = out;
-              }
-            }
-          }
+      for (int pi = 0; pi < PT; ++pi) {
+        if (!has_t || hb >= heads || pt0 + pi >= p_tiles) continue;
+        const long column = (long)(head0 + hb) * P + (pt0 + pi) * 16 + 4 * q;
+        s_floatx4 out;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out[i] = acc[hb][pi][i] + skip * (float)x_skip[hb][pi][i];
+        if (z != nullptr) {
+          s_bf16x4 packed;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(out[i] * silu_f((float)gate[hb][pi][i]));
+          *reinterpret_cast<s_bf16x4*>(gated + t_row * gated_ld + column) = packed;
+        } else {
+          *reinterpret_cast<s_floatx4*>(y + t_row * y_ld + column) = out;
         }
       }
     }
@@ -401,14 +406,16 @@ extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long
   {
     const int subsets = (H / G + SSD_HEADS_PER_BLOCK - 1) / SSD_HEADS_PER_BLOCK;
     const dim3 grid(n_chunks, G * subsets, (Q + 63) / 64);
-#define SCAN_CASE(PT_)                                                                                            \
-  ssd_chunk_scan_kernel<SSD_HEADS_PER_BLOCK, PT_><<<grid, 256, 0, stream>>>(                                      \
-      (const bf16_t*)xbc, xbc_ld, (const bf16_t*)xT, E, (const bf16_t*)state_in, delta, cum, D, chunks, Q, H, P, \
-      N, G, y, y_ld, (const bf16_t*)z, z_ld, (bf16_t*)gated, gated_ld)
-    if (P / 16 == 1) SCAN_CASE(1);
-    else if (P / 16 == 2) SCAN_CASE(2);
-    else if (P / 16 == 3) SCAN_CASE(3);
-    else SCAN_CASE(4);
+#define SCAN_CASE(NK_)                                                                                            \
+  case NK_:                                                                                                       \
+    ssd_chunk_scan_kernel<SSD_HEADS_PER_BLOCK, NK_><<<grid, 256, 0, stream>>>(                                    \
+        (const bf16_t*)xbc, xbc_ld, (const bf16_t*)xT, E, (const bf16_t*)state_in, delta, cum, D, chunks, Q, H, P, \
+        G, y, y_ld, (const bf16_t*)z, z_ld, (bf16_t*)gated, gated_ld);                                          \
+    break;
+    switch (N / 32) {
+      SCAN_CASE(1) SCAN_CASE(2) SCAN_CASE(3) SCAN_CASE(4) SCAN_CASE(5) SCAN_CASE(6) SCAN_CASE(7) SCAN_CASE(8)
+      default: return ERR_UNSUPPORTED_SIZE;
+    }
 #undef SCAN_CASE
     RETURN_IF_LAUNCH_FAILED();
   }
