@@ -51,15 +51,19 @@ class StepContext:
     derived: dict = field(default_factory=dict)   # tables parts derive from the step, shared by the layers
 
 
-def _pack(lanes: Sequence[Lane], cache, pad_lanes: int = 0, max_pages: Optional[int] = None):
+def _pack(lanes: Sequence[Lane], cache, pad_lanes: int = 0, max_pages: Optional[int] = None,
+          pad_lengths: Sequence[int] = ()):
     """Numpy sections of the step (in the order of ``_assemble``) and the block-table shapes.
-    ``pad_lanes`` single-token lanes on the scratch page and slot are appended."""
-    lengths = [len(lane.tokens) for lane in lanes] + [1] * pad_lanes
+    ``pad_lanes`` single-token lanes on the scratch page and slot are appended (or lanes of
+    ``pad_lengths`` tokens, all of them on the scratch page)."""
+    pad_lengths = list(pad_lengths) if pad_lengths else [1] * pad_lanes
+    pad_lanes = len(pad_lengths)
+    lengths = [len(lane.tokens) for lane in lanes] + pad_lengths
     starts = [cache.requests[lane.request].length for lane in lanes] + [0] * pad_lanes
     Ln = len(lengths)
     T = sum(lengths)
     token_ids = np.concatenate([np.asarray(lane.tokens, dtype=np.int32) for lane in lanes]
-                               + [np.zeros(pad_lanes, dtype=np.int32)])
+                               + [np.zeros(sum(pad_lengths), dtype=np.int32)])
     positions = np.concatenate([np.arange(start, start + length, dtype=np.int32)
                                 for start, length in zip(starts, lengths)])
     lane_of_token = np.repeat(np.arange(Ln, dtype=np.int32), lengths)
@@ -77,7 +81,8 @@ def _pack(lanes: Sequence[Lane], cache, pad_lanes: int = 0, max_pages: Optional[
     group_shapes = []
     for group in cache.groups:
         page_size = group.page_size
-        tables = [group.tables[lane.request].pages for lane in lanes] + [[group.scratch_page]] * pad_lanes
+        tables = ([group.tables[lane.request].pages for lane in lanes]
+                  + [[group.scratch_page] * -(-length // page_size) for length in pad_lengths])
         width = max_pages if max_pages is not None else max(1, max(len(pages) for pages in tables))
         table = np.zeros((Ln, width), dtype=np.int32)
         mapping = np.empty(T, dtype=np.int32)
@@ -125,15 +130,21 @@ def build_step_context(lanes: Sequence[Lane], cache, device) -> StepContext:
 
 
 class StaticStep:
-    """The arrays of a batch of ``lanes`` single-token lanes (every lane's logits wanted) at
-    fixed device addresses.  ``fill`` rewrites them for the real lanes of a step."""
+    """The arrays of a step of fixed shape at fixed device addresses: ``lanes`` single-token lanes
+    whose logits are all wanted, or lanes of ``lengths`` tokens with the wanted rows ``want_rows``.
+    ``fill`` rewrites them for the real lanes of a step of that shape."""
 
-    def __init__(self, cache, lanes: int, max_seq_len: int, device):
+    def __init__(self, cache, lanes: int, max_seq_len: int, device, lengths: Sequence[int] = (),
+                 want_rows: Sequence[int] = ()):
         self.cache = cache
         self.lanes = lanes
+        self.lengths = list(lengths)
         self.max_pages = max(-(-max_seq_len // group.page_size) for group in cache.groups) if cache.groups else 1
-        sections, group_shapes, lengths, starts = _pack([], cache, pad_lanes=lanes, max_pages=self.max_pages)
-        sections[7] = np.arange(lanes, dtype=np.int32)             # every lane's row is wanted
+        self.want_rows = (np.asarray(want_rows, dtype=np.int32) if self.lengths
+                          else np.arange(lanes, dtype=np.int32))             # every lane's row is wanted
+        sections, group_shapes, lengths, starts = _pack([], cache, pad_lanes=lanes, max_pages=self.max_pages,
+                                                        pad_lengths=self.lengths)
+        sections[7] = self.want_rows
         total = sum(section.size for section in sections)
         self.host = torch.empty(total, dtype=torch.int32).pin_memory()
         self.device_buffer = torch.empty(total, dtype=torch.int32, device=device)
@@ -143,6 +154,6 @@ class StaticStep:
 
     def fill(self, lanes: Sequence[Lane]) -> None:
         sections, _, _, _ = _pack(lanes, self.cache, pad_lanes=self.lanes - len(lanes), max_pages=self.max_pages)
-        sections[7] = np.arange(self.lanes, dtype=np.int32)
+        sections[7] = self.want_rows
         self.host.copy_(torch.from_numpy(np.concatenate(sections)))
         self.device_buffer.copy_(self.host, non_blocking=True)

@@ -124,9 +124,13 @@ class Engine:
         of each lane's ``want``.  Raises StepError or CacheExhausted with nothing changed."""
         self.validate(lanes)
         self.cache.reserve([(lane.request, len(lane.tokens)) for lane in lanes])
-        if self.graphs is not None and all(len(lane.tokens) == 1 for lane in lanes):
-            logits = self.graphs.run(lanes)                  # decode-only batch: a captured graph
-        else:
+        logits = None
+        if self.graphs is not None:
+            if all(len(lane.tokens) == 1 for lane in lanes):
+                logits = self.graphs.run(lanes)              # decode-only batch: a captured graph
+            else:
+                logits = self.graphs.run_portion(lanes)      # a shape of prompt portions seen before
+        if logits is None:
             context = build_step_context(lanes, self.cache, self.device)
             logits = self.model.forward(context, self.cache)
         for lane in lanes:

@@ -300,3 +300,39 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, requests):
         scale = want.abs().max().item()
         assert (have - want).abs().max().item() <= 6e-2 * scale
         assert ((have - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()).item() <= 3e-2
+
+
+@pytest.mark.parametrize("name, dtype", [("B", "float32"), ("C", "bfloat16")])
+def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
+    """Steps of one shape (two prompt portions of 70 and 40 tokens, some places wanted) come back:
+    from the second time on they are replayed from a captured graph.  Every step, through pages
+    that are given back and used again and with a decode replay between, is compared with an
+    engine without graphs."""
+    from macllm_infer_amd import Engine, Lane
+    folder = tiny_configs.make_model_dir(name, tmp_path, torch.float32 if dtype == "float32" else torch.bfloat16)
+    cfg, _ = plain_impl.load_model_dir(folder)
+    make = lambda graphs: Engine(folder, dtype=dtype, kv_cache_block_tokens=16, kv_cache_capacity_tokens=640,
+                                 max_active_sequences=4, decode_graphs=graphs)
+    with_graphs, eager = make(True), make(False)
+
+    def both(lanes):
+        got, want = with_graphs.step(lanes).float().cpu(), eager.step(lanes).float().cpu()
+        scale = max(1.0, want.abs().max().item())
+        assert got.shape == want.shape
+        assert (got - want).abs().max() <= (1e-5 if dtype == "float32" else 3e-2) * scale
+
+    for round_index in range(4):
+        a, b = f"a{round_index}", f"b{round_index}"
+        tokens_a = tokens_for(cfg["vocab_size"], 141, 700 + round_index)
+        tokens_b = tokens_for(cfg["vocab_size"], 81, 800 + round_index)
+        for engine in (with_graphs, eager):
+            engine.add_request(a)
+            engine.add_request(b)
+        both([Lane(a, tokens_a[:70], [3, 69]), Lane(b, tokens_b[:40], [39])])
+        both([Lane(a, tokens_a[70:140], [3, 69]), Lane(b, tokens_b[40:80], [39])])      # same shape, later positions
+        both([Lane(a, tokens_a[140:], [0]), Lane(b, tokens_b[80:], [0])])                 # a decode replay between
+        for engine in (with_graphs, eager):
+            engine.finish(a)
+            engine.finish(b)
+    assert len(with_graphs.graphs._portion_graphs) == 1
+    assert with_graphs.cache.stats() == eager.cache.stats()
