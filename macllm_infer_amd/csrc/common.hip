@@ -59,15 +59,100 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   }
 }
 
+// The same with four consecutive elements a thread and every load of a row asked for before the
+// first is used (d a multiple of 4, at most 256 * 4 * NORM_MAX_ROUNDS).  The order of the sum is
+// again fixed by d alone.
+#define NORM_MAX_ROUNDS 8
+template <typename T> struct Vec4;
+template <> struct Vec4<float> { typedef float type __attribute__((ext_vector_type(4))); };
+template <> struct Vec4<bf16_t> { typedef __bf16 type __attribute__((ext_vector_type(4))); };
+
+template <typename TD, typename TO>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta0, const TD* __restrict__ delta1,
+                       const float* __restrict__ weight, float eps, TO* __restrict__ out,
+                       const int* __restrict__ rows, int d) {
+  typedef typename Vec4<float>::type f4;
+  typedef typename Vec4<TD>::type d4;
+  typedef typename Vec4<TO>::type o4;
+  __shared__ float scratch[16];
+  const long out_row = blockIdx.x;
+  const long row = rows ? (long)rows[out_row] : out_row;
+  float* hr = h + row * d;
+  const int rounds = (d / 4 + 255) / 256;
+  f4 v[NORM_MAX_ROUNDS], w[NORM_MAX_ROUNDS];
+  d4 a[NORM_MAX_ROUNDS], b[NORM_MAX_ROUNDS];
+  int at[NORM_MAX_ROUNDS];
+#pragma unroll
+  for (int r = 0; r < NORM_MAX_ROUNDS; ++r) at[r] = min(((int)threadIdx.x + r * 256) * 4, d - 4);
+#pragma unroll
+  for (int r = 0; r < NORM_MAX_ROUNDS; ++r)
+    if (r < rounds) v[r] = *reinterpret_cast<const f4*>(hr + at[r]);
+  if (delta0) {
+#pragma unroll
+    for (int r = 0; r < NORM_MAX_ROUNDS; ++r)
+      if (r < rounds) a[r] = *reinterpret_cast<const d4*>(delta0 + row * d + at[r]);
+  }
+  if (delta1) {
+#pragma unroll
+    for (int r = 0; r < NORM_MAX_ROUNDS; ++r)
+      if (r < rounds) b[r] = *reinterpret_cast<const d4*>(delta1 + row * d + at[r]);
+  }
+  if (out) {
+#pragma unroll
+    for (int r = 0; r < NORM_MAX_ROUNDS; ++r)
+      if (r < rounds) w[r] = *reinterpret_cast<const f4*>(weight + at[r]);
+  }
+  float sum_squares = 0.f;
+#pragma unroll
+  for (int r = 0; r < NORM_MAX_ROUNDS; ++r) {
+    if (r < rounds) {
+      const bool mine = ((int)threadIdx.x + r * 256) * 4 < d;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float value = v[r][j];
+        if (delta0) value += (float)a[r][j];
+        if (delta1) value += (float)b[r][j];
+        v[r][j] = value;
+        if (mine) sum_squares += value * value;
+      }
+      if (mine && !rows && (delta0 || delta1)) *reinterpret_cast<f4*>(hr + at[r]) = v[r];
+    }
+  }
+  const float total = block_sum(sum_squares, scratch);
+  const float denominator = sqrtf(total / (float)d + eps);
+  if (out) {
+    TO* o = out + out_row * d;
+#pragma unroll
+    for (int r = 0; r < NORM_MAX_ROUNDS; ++r) {
+      if (r < rounds && ((int)threadIdx.x + r * 256) * 4 < d) {
+        o4 packed;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) packed[j] = from_float<TO>(v[r][j] / denominator * w[r][j]);
+        *reinterpret_cast<o4*>(o + at[r]) = packed;
+      }
+    }
+  }
+}
+
 extern "C" int mi_add_rmsnorm(float* h, const void* delta0, const void* delta1, int delta_dtype,
                               const float* weight, float eps, void* out, int out_dtype, const int* rows,
                               int n_rows, int d, hipStream_t stream) {
   if (n_rows <= 0 || d <= 0) return ERR_BAD_ARGUMENT;
-  if ((size_t)d * sizeof(float) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  const bool vectors = d % 4 == 0 && d <= 256 * 4 * NORM_MAX_ROUNDS && ((uintptr_t)h % 16) == 0 &&
+                       ((uintptr_t)delta0 % 16) == 0 && ((uintptr_t)delta1 % 16) == 0 &&
+                       ((uintptr_t)out % 16) == 0 && ((uintptr_t)weight % 16) == 0;
+  if (!vectors && (size_t)d * sizeof(float) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   const size_t lds = (size_t)d * sizeof(float);
-#define LAUNCH(TD, TO)                                                                               \
-  add_rmsnorm_kernel<TD, TO><<<n_rows, 256, lds, stream>>>(h, (const TD*)delta0, (const TD*)delta1, \
-                                                            weight, eps, (TO*)out, rows, d)
+#define LAUNCH(TD, TO)                                                                                      \
+  do {                                                                                                      \
+    if (vectors)                                                                                            \
+      add_rmsnorm_vec_kernel<TD, TO><<<n_rows, 256, 0, stream>>>(h, (const TD*)delta0, (const TD*)delta1,   \
+                                                                 weight, eps, (TO*)out, rows, d);           \
+    else                                                                                                    \
+      add_rmsnorm_kernel<TD, TO><<<n_rows, 256, lds, stream>>>(h, (const TD*)delta0, (const TD*)delta1,     \
+                                                               weight, eps, (TO*)out, rows, d);             \
+  } while (0)
   if (delta_dtype == DT_F32 && out_dtype == DT_F32) LAUNCH(float, float);
   else if (delta_dtype == DT_BF16 && out_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
   else if (delta_dtype == DT_F32 && out_dtype == DT_BF16) LAUNCH(float, bf16_t);
@@ -91,11 +176,30 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, long ld, T* __restrict__
   out[index] = from_float<T>(silu_f(gate) * up);
 }
 
+// bfloat16, eight elements a thread (I, ld and the addresses multiples of 8 elements)
+typedef __bf16 common_bf16x8 __attribute__((ext_vector_type(8)));
+__global__ void __launch_bounds__(256)
+swiglu_vec_kernel(const bf16_t* __restrict__ gu, long ld, bf16_t* __restrict__ out, int I, long total) {
+  const long index = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (index >= total) return;
+  const long t = index / I;
+  const int i = (int)(index - t * I);
+  const common_bf16x8 gate = *reinterpret_cast<const common_bf16x8*>(gu + t * ld + i);
+  const common_bf16x8 up = *reinterpret_cast<const common_bf16x8*>(gu + t * ld + I + i);
+  common_bf16x8 result;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) result[j] = (bf16_t)(silu_f((float)gate[j]) * (float)up[j]);
+  *reinterpret_cast<common_bf16x8*>(out + index) = result;
+}
+
 extern "C" int mi_swiglu(const void* gu, int dtype, long ld, void* out, int T, int I, hipStream_t stream) {
   if (T <= 0 || I <= 0 || ld < 2L * I) return ERR_BAD_ARGUMENT;
   const long total = (long)T * I;
   const int blocks = (int)((total + 255) / 256);
-  if (dtype == DT_F32)
+  if (dtype == DT_BF16 && I % 8 == 0 && ld % 8 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+    const int vec_blocks = (int)((total / 8 + 255) / 256);
+    swiglu_vec_kernel<<<vec_blocks, 256, 0, stream>>>((const bf16_t*)gu, ld, (bf16_t*)out, I, total);
+  } else if (dtype == DT_F32)
     swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, ld, (float*)out, I, total);
   else if (dtype == DT_BF16)
     swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, ld, (bf16_t*)out, I, total);

@@ -42,9 +42,12 @@ __global__ void conv1d_silu_kernel(const T* __restrict__ u, long ld, int col_off
 }
 
 // The same for bfloat16 with 8 channels and 4 consecutive token rows per thread: the rows the four
-// windows share are loaded once, 16 bytes at a time.  A row that lies before its token's lane
-// comes from the lane's conv tail instead.
+// windows share are loaded once, 16 bytes at a time, together with the taps (contiguous for 8
+// channels) and the lanes of the four tokens; no load stands under a condition.  The common case
+// (every row of a window belongs to the token's lane) is computed from these; a token among the
+// first K-1 of its lane is redone with the rows of the lane's conv tail.
 typedef __bf16 conv_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float conv_floatx4 __attribute__((ext_vector_type(4)));
 
 template <int K>
 __global__ void __launch_bounds__(256)
@@ -60,38 +63,50 @@ conv1d_silu_vec_kernel(const bf16_t* __restrict__ u, long ld, int col_offset, in
   const int channel = (int)(index - group * vectors) * 8;
   const long t0 = group * ROWS;
   if (t0 >= T) return;
-  conv_bf16x8 window[ROWS + K - 1];                 // rows t0-(K-1) .. t0+ROWS-1 of u
+  conv_bf16x8 window[ROWS + K - 1];                 // rows t0-(K-1) .. t0+ROWS-1 of u, clamped into [0, T)
 #pragma unroll
   for (int j = 0; j < ROWS + K - 1; ++j) {
-    const long row = t0 - (K - 1) + j;
-    if (row >= 0 && row < T) window[j] = *reinterpret_cast<const conv_bf16x8*>(u + row * ld + col_offset + channel);
+    const long row = min(max(t0 - (K - 1) + j, 0L), (long)T - 1);
+    window[j] = *reinterpret_cast<const conv_bf16x8*>(u + row * ld + col_offset + channel);
   }
-  float w[8][K];
-  float b[8];
+  conv_floatx4 taps[2 * K];                          // weight[channel .. channel+8, 0 .. K): 8K contiguous floats
 #pragma unroll
-  for (int c = 0; c < 8; ++c) {
-    b[c] = bias ? bias[channel + c] : 0.f;
-#pragma unroll
-    for (int k = 0; k < K; ++k) w[c][k] = weight[(long)(channel + c) * K + k];
+  for (int j = 0; j < 2 * K; ++j) taps[j] = *reinterpret_cast<const conv_floatx4*>(weight + (long)channel * K + 4 * j);
+  conv_floatx4 b_lo = {0.f, 0.f, 0.f, 0.f}, b_hi = {0.f, 0.f, 0.f, 0.f};
+  if (bias) {
+    b_lo = *reinterpret_cast<const conv_floatx4*>(bias + channel);
+    b_hi = *reinterpret_cast<const conv_floatx4*>(bias + channel + 4);
   }
+  int lane[ROWS];
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) lane[i] = lane_of_token[min(t0 + i, (long)T - 1)];
+  int lane_start[ROWS];
+#pragma unroll
+  for (int i = 0; i < ROWS; ++i) lane_start[i] = cu_seqlens[lane[i]];
+  auto tap = [&](int c, int k) { return taps[(c * K + k) / 4][(c * K + k) % 4]; };
 #pragma unroll
   for (int i = 0; i < ROWS; ++i) {
     const long token = t0 + i;
     if (token >= T) break;
-    const int lane = lane_of_token[token];
-    const long lane_start = cu_seqlens[lane];
     float sum[8];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) sum[c] = b[c];
+    for (int c = 0; c < 8; ++c) sum[c] = c < 4 ? b_lo[c] : b_hi[c - 4];
+    if (token - (K - 1) >= lane_start[i]) {
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-      const long source = token - (K - 1) + k;
-      conv_bf16x8 sample = window[i + k];
-      if (source < lane_start)
-        sample = *reinterpret_cast<const conv_bf16x8*>(conv_state + ((long)slot_ids[lane] * (K - 1) + (K - 1) +
-                                                                     (source - lane_start)) * C + channel);
+      for (int k = 0; k < K; ++k)
 #pragma unroll
-      for (int c = 0; c < 8; ++c) sum[c] += w[c][k] * (float)sample[c];
+        for (int c = 0; c < 8; ++c) sum[c] += tap(c, k) * (float)window[i + k][c];
+    } else {
+      const bf16_t* tail = conv_state + (long)slot_ids[lane[i]] * (K - 1) * C + channel;
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const long source = token - (K - 1) + k;
+        conv_bf16x8 sample = window[i + k];
+        if (source < lane_start[i])
+          sample = *reinterpret_cast<const conv_bf16x8*>(tail + ((K - 1) + (source - lane_start[i])) * C);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) sum[c] += tap(c, k) * (float)sample[c];
+      }
     }
     conv_bf16x8 result;
 #pragma unroll
@@ -108,7 +123,8 @@ extern "C" int mi_conv1d_silu(const void* u, int dtype, long ld, int col_offset,
   const long total = (long)T * C;
   const int blocks = (int)((total + 255) / 256);
   const bool aligned = C % 8 == 0 && ld % 8 == 0 && col_offset % 8 == 0 && ((uintptr_t)u % 16) == 0 &&
-                       ((uintptr_t)out % 16) == 0 && ((uintptr_t)conv_state % 16) == 0;
+                       ((uintptr_t)out % 16) == 0 && ((uintptr_t)conv_state % 16) == 0 &&
+                       ((uintptr_t)weight % 16) == 0 && ((uintptr_t)bias % 16) == 0;
   if (dtype == DT_BF16 && aligned && K >= 2 && K <= 4) {
     const long threads = (long)((T + 3) / 4) * (C / 8);
     const int vec_blocks = (int)((threads + 255) / 256);
