@@ -65,9 +65,15 @@ class Attention(Mixer):
 
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         spec = self.spec
-        qkv = self.qkv(x)
+        attended = torch.empty((x.shape[0], spec.num_heads * spec.head_dim), dtype=x.dtype, device=x.device)
+        self.mix(self.qkv(x), step, cache, attended)
+        return self.out(attended)
+
+    def mix(self, qkv: torch.Tensor, step, cache, attended: torch.Tensor) -> None:
+        """From the projected rows [q | k | v] (rotated and stored in place) to the attended rows
+        ``attended`` [T, Hq * dh]; both may be column views of wider matrices."""
+        spec = self.spec
         self.position.rotate_and_store(qkv, spec.num_heads, spec.num_kv_heads, spec.head_dim, step, cache)
-        attended = torch.empty((x.shape[0], spec.num_heads * spec.head_dim), dtype=qkv.dtype, device=x.device)
         geometry = (spec.num_heads, spec.num_kv_heads, spec.head_dim)
         if step.max_query_len == 1 and ops.decode_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2]):
             ops.decode_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
@@ -80,4 +86,3 @@ class Attention(Mixer):
         else:
             ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                 step.lane_of_token, step.positions, spec.scale, spec.window, attended)
-        return self.out(attended)

@@ -56,8 +56,8 @@ class ParallelPreNormBlock:
         self.ffn_norm = part_class(layer.ffn_norm)(
             layer.ffn_norm, f"{layer.prefix}.{layer.ffn_norm_name}", tensors, build)
         self.ffn = part_class(layer.ffn)(layer.ffn, f"{layer.prefix}.{layer.ffn_name}", tensors, build)
-        from .fused_decode import ParallelDecodeFusion
-        self.decode_fusion = ParallelDecodeFusion.build(self, build)      # None when the parts or sizes do not fit
+        from .fused import ParallelFusion
+        self.fusion = ParallelFusion.build(self, build)      # None when the parts or sizes do not fit
 
     @property
     def graph_safe(self) -> bool:
@@ -66,9 +66,8 @@ class ParallelPreNormBlock:
 
     def forward(self, residual: Residual, step, caches) -> None:
         """``caches``: mixer name -> EntryCache of this run of the layer."""
-        fusion = self.decode_fusion
-        if fusion is not None and fusion.supports(step, caches[fusion.attention_name]):
-            fusion.forward(residual, step, caches)
+        fusion = self.fusion
+        if fusion is not None and fusion.forward(residual, step, caches):
             return
         normed = self.mixer_norm.forward(residual)
         residual.pending = [mixer.forward(normed, step, caches[name]) for name, mixer in self.mixers]

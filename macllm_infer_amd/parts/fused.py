@@ -1,16 +1,24 @@
-"""The decode fast path of a layer: when every lane of a step holds one token, a block made
-of RMSNorm, attention, Mamba2 and SwiGLU runs as five launches instead of fifteen (seven for
-batches of more than 16 rows, whose two norms run as kernels of their own).
+"""The fast paths of a layer made of RMSNorm, attention, Mamba2 and SwiGLU.  The two mixers read
+the same normed rows and their outputs are added, so their input projections are one matrix
+[q|k|v|z|x B C|dt] and their output projections one matrix [Wo | W_out] along the inputs; the
+parts' own matrices are views of these.
+
+Any step in bfloat16 (prompt portions, mixed batches): norm, one input GEMM, the two mixers on
+column views of its output, one output GEMM, norm, feed-forward: two library GEMMs fewer than
+part by part.
+
+Decode steps (every lane holds one token, at most 64 rows): five launches instead of fifteen
+(seven for batches of more than 16 rows, whose two norms run as kernels of their own)
 
     1. residual add + norm + [q|k|v|z|x B C|dt] projection + conv step        (fused_gemm)
-    2. attention (rotation, cache write, split context, merge) and SSM step    (mixer_decode)
+    2. attention (rotation, cache write, split context) and SSM step           (mixer_decode)
     3. [attention | ssm] . [Wo | W_out]^T                                       (fused_gemm)
     4. residual add + norm + gate/up projection + SiLU(g)*u                     (fused_gemm)
     5. down projection                                                          (fused_gemm)
 
-The fusion belongs to the arrangement, which knows its parts; the parts stay as they are and
-serve every other kind of step.  It is built only for bfloat16 weights and sizes the kernels
-cover; otherwise the block runs part by part.
+The fusion belongs to the arrangement, which knows its parts; the parts stay as they are.  It
+is built only for bfloat16 weights and sizes the kernels cover; otherwise the block runs part
+by part.
 """
 from __future__ import annotations
 
@@ -30,9 +38,9 @@ MAX_ROWS = 64          # rows of a step the skinny kernels take
 MAX_NORM_ROWS = 16     # the norm prologue recomputes the normed rows in every workgroup: small batches only
 
 
-class ParallelDecodeFusion:
+class ParallelFusion:
     @staticmethod
-    def build(block, build) -> Optional["ParallelDecodeFusion"]:
+    def build(block, build) -> Optional["ParallelFusion"]:
         if build.dtype != torch.bfloat16 or build.device.type != "cuda":
             return None
         mixers = dict(block.mixers)
@@ -59,7 +67,7 @@ class ParallelDecodeFusion:
             return None
         if not ops.fused_gemm_supported(True, 1, hidden):
             return None
-        return ParallelDecodeFusion(block, attention, mamba, build)
+        return ParallelFusion(block, attention, mamba, build)
 
     def __init__(self, block, attention: Attention, mamba: Mamba2, build):
         self.block = block
@@ -81,11 +89,20 @@ class ParallelDecodeFusion:
         self.dt_col = self.x_col + C
         self.in_width = self.w_in.shape[0]
         self.in_ld = -(-self.in_width // 8) * 8
+        self.qkv_width = q_width + 2 * kv_width
+        attention.qkv.weight = self.w_in[:self.qkv_width]             # the parts' matrices: views of the fused ones
+        mamba.in_proj.weight = self.w_in[self.qkv_width:]
         # 3: [attention | ssm] . [Wo | W_out]^T
         self.w_out = torch.cat([attention.out.weight, mamba.out_proj.weight], dim=1).contiguous()
         biases = [linear.bias for linear in (attention.out, mamba.out_proj) if linear.bias is not None]
         self.b_out = sum(biases[1:], biases[0]).contiguous() if biases else None
         self.mixed_width = q_width + E
+        self.q_width = q_width
+        attention.out.weight = self.w_out[:, :q_width]
+        mamba.out_proj.weight = self.w_out[:, q_width:]
+        # the column views the mixers get must start at 16 bytes and rows must be multiples of 8 elements
+        self.general = (self.in_width % 8 == 0 and self.qkv_width % 8 == 0 and q_width % 8 == 0
+                        and self.mixed_width % 8 == 0)
         # 4: gate and up rows interleaved in tiles of 8
         ffn = block.ffn
         inner = ffn.spec.intermediate_size
@@ -95,14 +112,36 @@ class ParallelDecodeFusion:
         self.inner = inner
         self.position = attention.position
 
-    def supports(self, step, cache) -> bool:
+    def decode_supported(self, step, cache) -> bool:
         a = self.attention.spec
         rotary = self.position.rotary_dim if isinstance(self.position, Rope) else 0
         return (step.max_query_len == 1 and step.num_tokens <= MAX_ROWS and cache.owns_kv
                 and ops.mixer_decode_supported(a.num_heads, a.num_kv_heads, a.head_dim, cache.k_cache.shape[2],
                                                self.mamba.spec.state_size, step.max_seq_len, a.window, rotary))
 
-    def forward(self, residual: Residual, step, caches) -> None:
+    def forward(self, residual: Residual, step, caches) -> bool:
+        """Runs the layer and returns True, or returns False with nothing done (the block then
+        runs part by part)."""
+        if self.decode_supported(step, caches[self.attention_name]):
+            self.forward_decode(residual, step, caches)
+            return True
+        if self.general:
+            self.forward_general(residual, step, caches)
+            return True
+        return False
+
+    def forward_general(self, residual: Residual, step, caches) -> None:
+        block = self.block
+        normed = block.mixer_norm.forward(residual)
+        u = ops.linear(normed, self.w_in, self.b_in)
+        mixed = torch.empty((u.shape[0], self.mixed_width), dtype=u.dtype, device=u.device)
+        self.attention.mix(u[:, :self.qkv_width], step, caches[self.attention_name], mixed[:, :self.q_width])
+        self.mamba.mix(u[:, self.qkv_width:], step, caches[self.mamba_name], mixed[:, self.q_width:])
+        residual.pending = [ops.linear(mixed, self.w_out, self.b_out)]
+        normed = block.ffn_norm.forward(residual)
+        residual.pending = [block.ffn.forward(normed)]
+
+    def forward_decode(self, residual: Residual, step, caches) -> None:
         block, a, s = self.block, self.attention.spec, self.mamba.spec
         kv, state = caches[self.attention_name], caches[self.mamba_name]
         M = step.num_tokens

@@ -90,22 +90,28 @@ class Mamba2(Mixer):
         return step.derived[key]
 
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+        u = self.in_proj(x)                                               # [T, E + C + H]
+        gated = torch.empty((x.shape[0], self.spec.inner_size), dtype=u.dtype, device=u.device)
+        self.mix(u, step, cache, gated)
+        return self.out_proj(gated)
+
+    def mix(self, u: torch.Tensor, step, cache, gated: torch.Tensor) -> None:
+        """From the projected rows [z | x B C | dt] to the gated (and normed) scan output
+        ``gated`` [T, E]; both may be column views of wider matrices."""
         spec = self.spec
         E, C = spec.inner_size, spec.conv_width
-        T = x.shape[0]
+        T = u.shape[0]
         conv_state, ssm_state = cache.states["conv"], cache.states["ssm"]
-        u = self.in_proj(x)                                               # [T, E + C + H]
         xbc = torch.empty((T, C), dtype=u.dtype, device=u.device)
         ops.conv1d_silu(u, E, C, self.conv_weight, self.conv_bias, conv_state, step.lane_of_token,
                         step.cu_seqlens, step.slot_ids, xbc)
         ops.conv_state_update(u, E, C, spec.conv_kernel, conv_state, step.cu_seqlens, step.slot_ids)
-        gated = torch.empty((T, E), dtype=u.dtype, device=u.device)
         if self._chunked(u, step):
             arguments = (xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, self._chunk_table(step),
                          step.slot_ids, spec.num_groups)
-            if self.norm_weight is None and u.stride(0) % 4 == 0:
+            if self.norm_weight is None and u.stride(0) % 4 == 0 and gated.stride(0) % 4 == 0:
                 ops.ssd_prefill(*arguments, None, z=u[:, :E], gated=gated)      # the gate on the scan's way out
-                return self.out_proj(gated)
+                return
             y = torch.empty((T, E), dtype=torch.float32, device=u.device)
             ops.ssd_prefill(*arguments, y)
         else:
@@ -113,4 +119,3 @@ class Mamba2(Mixer):
             ops.ssm_scan(xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, step.cu_seqlens,
                          step.slot_ids, spec.num_groups, y)
         ops.gate_norm(y, u[:, :E], self.norm_weight, spec.num_groups, spec.norm_eps, gated)
-        return self.out_proj(gated)
