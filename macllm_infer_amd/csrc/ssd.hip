@@ -9,7 +9,7 @@
 // Every exponent is a difference of a non-increasing sequence taken forwards, so it is <= 0 and
 // nothing overflows.  The result does not depend on Q beyond rounding.  Five kernels:
 //     prepare     delta, L                                    (one workgroup per chunk and head)
-//     transpose   x and B of each chunk, token-contiguous and zero-padded to Q
+//     transpose   x and B of each chunk, token-contiguous and zero-padded to Q: [chunk, E + G*N, Q]
 //     chunk_state sum_s exp(L_end - L_s) delta_s x_s (outer) B_s  per chunk and head (matrix cores)
 //     state_pass  S_in of every chunk from the slot's state, serially over a lane's chunks; the
 //                 lane's final state goes back to the slot (float32 throughout)
@@ -108,13 +108,16 @@ ssd_transpose_kernel(const bf16_t* __restrict__ xbc, long ld, int channels, cons
 // chunk_state[chunk, h, p, n] = sum_s xT[h*P + p, s] * (BT[g*N + n, s] * exp(L_end - L_s) * delta_s)
 // computed as its transpose on the matrix cores: A = weighted BT rows (n), B = xT rows (p),
 // contraction over the Q tokens; a lane ends up with 4 consecutive n of one p.
-// chunk_decay[chunk, h] = exp(L_end).
+// chunk_decay[chunk, h] = exp(L_end).  TT is the transposed copy [chunk, E + G*N, Q]: x rows
+// first, B rows after.  QK = Q / 32 is a template parameter and a tile of rows that does not
+// exist is clamped, so that all fragments of a tile are asked for at once.
+template <int QK>
 __global__ void __launch_bounds__(256)
-ssd_chunk_state_kernel(const bf16_t* __restrict__ xT, int E, const bf16_t* __restrict__ BT, int GN,
-                       const float* __restrict__ delta, const float* __restrict__ cum,
-                       const int* __restrict__ chunks, int Q, int H, int P, int N, int G,
+ssd_chunk_state_kernel(const bf16_t* __restrict__ TT, int E, int GN, const float* __restrict__ delta,
+                       const float* __restrict__ cum, const int* __restrict__ chunks, int H, int P, int N, int G,
                        float* __restrict__ chunk_state, float* __restrict__ chunk_decay) {
-  __shared__ float weight[SSD_MAX_Q];
+  constexpr int Q = 32 * QK;
+  __shared__ float weight[Q];
   const int chunk = blockIdx.x;
   const int head = blockIdx.y;
   const int group = head / (H / G);
@@ -126,34 +129,44 @@ ssd_chunk_state_kernel(const bf16_t* __restrict__ xT, int E, const bf16_t* __res
   const int q = lane / 16;
   const int r = lane % 16;
   const float total = cum[(long)(t0 + length - 1) * H + head];
-  for (int s = tid; s < Q; s += 256)
-    weight[s] = s < length ? __expf(total - cum[(long)(t0 + s) * H + head]) * delta[(long)(t0 + s) * H + head] : 0.f;
+  for (int s = tid; s < Q; s += 256) {
+    const long at = (long)(t0 + min(s, length - 1)) * H + head;
+    const float value = __expf(total - cum[at]) * delta[at];
+    weight[s] = s < length ? value : 0.f;
+  }
   if (tid == 0) chunk_decay[(long)chunk * H + head] = __expf(total);
   __syncthreads();
-  const bf16_t* x_rows = xT + ((long)chunk * E + (long)head * P) * Q;
-  const bf16_t* b_rows = BT + ((long)chunk * GN + (long)group * N) * Q;
+  const bf16_t* x_rows = TT + ((long)chunk * (E + GN) + (long)head * P) * Q;
+  const bf16_t* b_rows = TT + ((long)chunk * (E + GN) + E + (long)group * N) * Q;
   float* out = chunk_state + ((long)chunk * H + head) * P * N;
+  const int p_tiles = P / 16;
   for (int nt = wave; nt < N / 16; nt += 4) {
-    for (int pt0 = 0; pt0 < P / 16; pt0 += 4) {            // up to four p-tiles share the weighted B fragments
+    for (int pt0 = 0; pt0 < p_tiles; pt0 += 4) {            // four p-tiles share the weighted B fragments
+      s_bf16x8 b_raw[QK], x[4][QK];
+#pragma unroll
+      for (int ks = 0; ks < QK; ++ks)
+        b_raw[ks] = *reinterpret_cast<const s_bf16x8*>(b_rows + (long)(nt * 16 + r) * Q + 32 * ks + 8 * q);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int pt = min(pt0 + i, p_tiles - 1);
+#pragma unroll
+        for (int ks = 0; ks < QK; ++ks)
+          x[i][ks] = *reinterpret_cast<const s_bf16x8*>(x_rows + (long)(pt * 16 + r) * Q + 32 * ks + 8 * q);
+      }
       s_floatx4 acc[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[i] = s_floatx4{0.f, 0.f, 0.f, 0.f};
-      for (int ks = 0; ks < Q / 32; ++ks) {
-        const s_bf16x8 b_raw = *reinterpret_cast<const s_bf16x8*>(b_rows + (long)(nt * 16 + r) * Q + 32 * ks + 8 * q);
+#pragma unroll
+      for (int ks = 0; ks < QK; ++ks) {
         s_bf16x8 a;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) a[j] = (bf16_t)((float)b_raw[j] * weight[32 * ks + 8 * q + j]);
+        for (int j = 0; j < 8; ++j) a[j] = (bf16_t)((float)b_raw[ks][j] * weight[32 * ks + 8 * q + j]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (pt0 + i < P / 16) {
-            const s_bf16x8 x = *reinterpret_cast<const s_bf16x8*>(x_rows + (long)((pt0 + i) * 16 + r) * Q + 32 * ks + 8 * q);
-            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, x, acc[i], 0, 0, 0);
-          }
-        }
+        for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, x[i][ks], acc[i], 0, 0, 0);
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (pt0 + i < P / 16)
+        if (pt0 + i < p_tiles)
           *reinterpret_cast<s_floatx4*>(out + (long)((pt0 + i) * 16 + r) * N + nt * 16 + 4 * q) = acc[i];
     }
   }
@@ -174,10 +187,21 @@ __global__ void ssd_state_pass_kernel(const float* __restrict__ chunk_state, con
   const int count = lane_chunks[2 * lane + 1];
   float* slot = ssm_state + ((long)slot_ids[lane] * H + head) * per_head + element;
   float running = *slot;
-  for (int c = first; c < first + count; ++c) {
-    const long at = ((long)c * H + head) * per_head + element;
-    state_in[at] = (bf16_t)running;
-    running = chunk_decay[(long)c * H + head] * running + chunk_state[at];
+  for (int c0 = first; c0 < first + count; c0 += 8) {       // eight chunks' loads at a time, then the recurrence
+    float added[8], decay[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int c = min(c0 + j, first + count - 1);
+      added[j] = chunk_state[((long)c * H + head) * per_head + element];
+      decay[j] = chunk_decay[(long)c * H + head];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (c0 + j < first + count) {
+        state_in[((long)(c0 + j) * H + head) * per_head + element] = (bf16_t)running;
+        running = decay[j] * running + added[j];
+      }
+    }
   }
   *slot = running;
 }
@@ -195,7 +219,7 @@ __global__ void ssd_state_pass_kernel(const float* __restrict__ chunk_state, con
 // order and a condition between them would make each wait for the one before.
 template <int HB, int NK>
 __global__ void __launch_bounds__(256)
-ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t* __restrict__ xT, int E,
+ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t* __restrict__ TT, int E,
                       const bf16_t* __restrict__ state_in, const float* __restrict__ delta,
                       const float* __restrict__ cum, const float* __restrict__ D, const int* __restrict__ chunks,
                       int Q, int H, int P, int G, float* __restrict__ y, long y_ld,
@@ -290,7 +314,7 @@ ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t*
 #pragma unroll
         for (int pi = 0; pi < PT; ++pi) {
           const int pt = min(pt0 + pi, p_tiles - 1);
-          const bf16_t* x_row = xT + ((long)chunk * E + (long)head * P + pt * 16 + n) * Q + s0 + 4 * q;
+          const bf16_t* x_row = TT + ((long)chunk * (E + G * N) + (long)head * P + pt * 16 + n) * Q + s0 + 4 * q;
           x_lo[hb][pi] = *reinterpret_cast<const s_bf16x4*>(x_row);
           x_hi[hb][pi] = *reinterpret_cast<const s_bf16x4*>(x_row + 16);
         }
@@ -365,7 +389,7 @@ extern "C" int mi_ssd_supported(int Q, int P, int N, int G, int E) {
 extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long dt_ld, const float* dt_bias,
                               const float* A, const float* D, float* ssm_state, const int* chunks, int n_chunks,
                               const int* lane_chunks, const int* slot_ids, int n_lanes, int Q, int H, int P, int N,
-                              int G, float* delta, float* cum, void* xT, void* BT, float* chunk_state,
+                              int G, float* delta, float* cum, void* TT, float* chunk_state,
                               float* chunk_decay, void* state_in, float* y, long y_ld, const void* z, long z_ld,
                               void* gated, long gated_ld, hipStream_t stream) {
   if (n_chunks <= 0 || n_lanes <= 0 || H <= 0 || G <= 0 || H % G != 0) return ERR_BAD_ARGUMENT;
@@ -383,17 +407,22 @@ extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long
     RETURN_IF_LAUNCH_FAILED();
   }
   {
-    const dim3 grid_x(n_chunks, (E + 63) / 64);
-    ssd_transpose_kernel<<<grid_x, 256, 0, stream>>>((const bf16_t*)xbc, xbc_ld, E, chunks, Q, (bf16_t*)xT);
-    RETURN_IF_LAUNCH_FAILED();
-    const dim3 grid_b(n_chunks, (GN + 63) / 64);
-    ssd_transpose_kernel<<<grid_b, 256, 0, stream>>>((const bf16_t*)xbc + E, xbc_ld, GN, chunks, Q, (bf16_t*)BT);
+    const dim3 grid_t(n_chunks, (E + GN + 63) / 64);         // x and B are neighbours in a row of xbc
+    ssd_transpose_kernel<<<grid_t, 256, 0, stream>>>((const bf16_t*)xbc, xbc_ld, E + GN, chunks, Q, (bf16_t*)TT);
     RETURN_IF_LAUNCH_FAILED();
   }
   {
     const dim3 grid(n_chunks, H);
-    ssd_chunk_state_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)xT, E, (const bf16_t*)BT, GN, delta, cum, chunks,
-                                                     Q, H, P, N, G, chunk_state, chunk_decay);
+#define STATE_CASE(QK_)                                                                                         \
+  case QK_:                                                                                                     \
+    ssd_chunk_state_kernel<QK_><<<grid, 256, 0, stream>>>((const bf16_t*)TT, E, GN, delta, cum, chunks, H, P, N, G, \
+                                                          chunk_state, chunk_decay);                          \
+    break;
+    switch (Q / 32) {
+      STATE_CASE(1) STATE_CASE(2) STATE_CASE(3) STATE_CASE(4) STATE_CASE(5) STATE_CASE(6) STATE_CASE(7) STATE_CASE(8)
+      default: return ERR_UNSUPPORTED_SIZE;
+    }
+#undef STATE_CASE
     RETURN_IF_LAUNCH_FAILED();
   }
   {
@@ -409,7 +438,7 @@ extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long
 #define SCAN_CASE(NK_)                                                                                            \
   case NK_:                                                                                                       \
     ssd_chunk_scan_kernel<SSD_HEADS_PER_BLOCK, NK_><<<grid, 256, 0, stream>>>(                                    \
-        (const bf16_t*)xbc, xbc_ld, (const bf16_t*)xT, E, (const bf16_t*)state_in, delta, cum, D, chunks, Q, H, P, \
+        (const bf16_t*)xbc, xbc_ld, (const bf16_t*)TT, E, (const bf16_t*)state_in, delta, cum, D, chunks, Q, H, P, \
         G, y, y_ld, (const bf16_t*)z, z_ld, (bf16_t*)gated, gated_ld);                                          \
     break;
     switch (N / 32) {

@@ -59,7 +59,7 @@ _SIGNATURES = {
     "ssd": {
         "mi_ssd_supported": [_c_int, _c_int, _c_int, _c_int, _c_int],
         "mi_ssd_prefill": [_c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr,
-                           _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                           _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
                            _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr],
     },
     "gemm": {
@@ -519,12 +519,11 @@ def ssd_prefill(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: t
     transposed = torch.empty((chunks * (E + GN) * Q,), dtype=torch.bfloat16, device=device)
     chunk_state = torch.empty((chunks * H * P * N + chunks * H,), dtype=torch.float32, device=device)
     state_in = torch.empty((chunks * H * P * N,), dtype=torch.bfloat16, device=device)
-    xT, BT = transposed[:chunks * E * Q], transposed[chunks * E * Q:]
     decay = chunk_state[chunks * H * P * N:]
     _check(_fn("ssd", "mi_ssd_prefill")(
         _p(xbc), xbc_ld, _p(dt), dt_ld, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(table.chunks), chunks,
         _p(table.lane_chunks), _p(slot_ids), table.num_lanes, Q, H, P, N, num_groups, _p(delta[0]), _p(delta[1]),
-        _p(xT), _p(BT), _p(chunk_state), _p(decay), _p(state_in), _p(y), y_ld, _p(z), z_ld, _p(gated), gated_ld,
+        _p(transposed), _p(chunk_state), _p(decay), _p(state_in), _p(y), y_ld, _p(z), z_ld, _p(gated), gated_ld,
         _stream()),
         "ssd_prefill", f"(Q={Q}, P={P}, N={N})")
 
