@@ -151,11 +151,12 @@ __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(float* __restrict__ logits, int V, int padded, const float* __restrict__ temperature,
               const int* __restrict__ top_k, const float* __restrict__ top_p,
               const unsigned long long* __restrict__ seeds, const int* __restrict__ draw_index,
-              unsigned long long* __restrict__ keys, int* __restrict__ out) {
+              unsigned long long* __restrict__ keys, int* __restrict__ out, const int* __restrict__ done) {
   __shared__ float scan_scratch[SAMPLE_THREADS];
   __shared__ unsigned long long key_scratch[SAMPLE_THREADS / WAVE];
   __shared__ int found;
   const int row = blockIdx.x;
+  if (done != nullptr && done[row] != 0) return;               // sample_select_kernel has drawn this row's token
   float* values = logits + (long)row * V;
   unsigned long long* sorted = keys + (long)row * padded;
   const float temp = temperature[row];
@@ -274,12 +275,276 @@ sample_kernel(float* __restrict__ logits, int V, int padded, const float* __rest
   if (threadIdx.x == 0) out[row] = found < V ? found : (int)(sorted[0] & 0xffffffffu);
 }
 
+// ---------------------------------------------------------------- the same without the full sort
+// What is kept after top-k and top-p is small; sorting the whole vocabulary to find it is not
+// needed.  With top-k (k <= SAMPLE_KMAX) the k smallest keys are found by a radix select over
+// the 64-bit keys (eight passes of a 256-bin histogram), gathered and sorted in LDS; without
+// top-k the SAMPLE_KMAX best candidates are taken the same way and the normalizer is summed over
+// the whole row; without top-k and top-p nothing is sorted at all.  The results are those of
+// sample_kernel up to the rounding of float32 sums.  A row this kernel does not cover (k above
+// SAMPLE_KMAX, or a nucleus that does not close within the candidates) is left with done[row] = 0
+// for sample_kernel, which skips the rows that are done.  The logits are not written.
+#define SAMPLE_KMAX 1024
+
+__device__ void lds_bitonic_sort(unsigned long long* keys, int padded) {
+  for (int size = 2; size <= padded; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      __syncthreads();
+      for (int i = threadIdx.x; i < padded / 2; i += blockDim.x) {
+        const int low = ((i / stride) * stride * 2) + (i % stride);
+        const int high = low + stride;
+        const bool ascending = ((low & size) == 0);
+        const unsigned long long a = keys[low];
+        const unsigned long long b = keys[high];
+        if ((a > b) == ascending) {
+          keys[low] = b;
+          keys[high] = a;
+        }
+      }
+    }
+  }
+  __syncthreads();
+}
+
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_select_kernel(const float* __restrict__ logits, int V, const float* __restrict__ temperature,
+                     const int* __restrict__ top_k, const float* __restrict__ top_p,
+                     const unsigned long long* __restrict__ seeds, const int* __restrict__ draw_index,
+                     int* __restrict__ out, int* __restrict__ done) {
+  __shared__ float scan_scratch[SAMPLE_THREADS];
+  __shared__ unsigned long long key_scratch[SAMPLE_THREADS / WAVE];
+  __shared__ unsigned long long candidates[SAMPLE_KMAX];
+  __shared__ unsigned long long by_index[SAMPLE_KMAX];
+  __shared__ unsigned int histogram[256];
+  __shared__ unsigned long long chosen_prefix;
+  __shared__ int remaining, found, gathered, bin_taken_whole;
+  const int row = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float* values = logits + (long)row * V;
+  const float temp = temperature[row];
+  if (tid == 0) done[row] = 0;
+
+  if (temp <= 0.f) {
+    unsigned long long best = ~0ull;
+    for (int v = tid; v < V; v += blockDim.x) {
+      const unsigned long long key = rank_key(values[v], v);
+      best = key < best ? key : best;
+    }
+    best = block_min_key(best, key_scratch);
+    if (tid == 0) {
+      out[row] = (int)(best & 0xffffffffu);
+      done[row] = 1;
+    }
+    return;
+  }
+  const int k = top_k[row];
+  const bool use_top_k = k > 0 && k < V;
+  const float p_limit = top_p[row];
+  const bool use_top_p = p_limit >= 0.f && p_limit < 1.f;
+  if (use_top_k && k > SAMPLE_KMAX) return;                    // sample_kernel's
+  const float u = draw_uniform(seeds[row], (unsigned long long)draw_index[row]);
+  const int vchunk = (V + blockDim.x - 1) / blockDim.x;
+  const int vbegin = min(V, tid * vchunk);
+  const int vend = min(V, vbegin + vchunk);
+
+  if (!use_top_k && !use_top_p) {
+    // every token is kept: maximum, normalizer, and the walk in index order
+    unsigned long long best = ~0ull;
+    for (int v = tid; v < V; v += blockDim.x) {
+      const unsigned long long key = rank_key(values[v] / temp, v);
+      best = key < best ? key : best;
+    }
+    best = block_min_key(best, key_scratch);
+    const float maximum = from_orderable(~(unsigned int)(best >> 32));
+    float local = 0.f;
+    for (int v = vbegin; v < vend; ++v) local += expf(values[v] / temp - maximum);
+    float normalizer;
+    block_exclusive_scan(local, scan_scratch, &normalizer);
+    float mass = 0.f;
+    for (int v = vbegin; v < vend; ++v) mass += expf(values[v] / temp - maximum) / normalizer;
+    float total;
+    const float start = block_exclusive_scan(mass, scan_scratch, &total);
+    const float target = u * total;
+    if (tid == 0) found = V;
+    __syncthreads();
+    float cumulative = start;
+    for (int v = vbegin; v < vend; ++v) {
+      const float p = expf(values[v] / temp - maximum) / normalizer;
+      if (p <= 0.f) continue;
+      cumulative += p;
+      if (target < cumulative) {
+        atomicMin(&found, v);
+        break;
+      }
+    }
+    __syncthreads();
+    if (tid == 0) {
+      out[row] = found < V ? found : (int)(best & 0xffffffffu);
+      done[row] = 1;
+    }
+    return;
+  }
+
+  // ---- the K smallest keys: radix select of the K-th, most significant byte first
+  const int K = use_top_k ? k : min(V, SAMPLE_KMAX);
+  if (tid == 0) {
+    chosen_prefix = 0ull;
+    remaining = K;
+  }
+  for (int pass = 7; pass >= 0; --pass) {
+    if (tid < 256) histogram[tid] = 0u;
+    __syncthreads();
+    const unsigned long long prefix = chosen_prefix;
+    const unsigned long long above = pass == 7 ? 0ull : (~0ull << (8 * (pass + 1)));
+    for (int v = tid; v < V; v += blockDim.x) {
+      const unsigned long long key = rank_key(values[v] / temp, v);
+      if ((key & above) == prefix) atomicAdd(&histogram[(unsigned int)(key >> (8 * pass)) & 255u], 1u);
+    }
+    __syncthreads();
+    // the bin in which the running count reaches what is still wanted: the first wave scans the
+    // 256 bins, four a lane
+    if (tid < WAVE) {
+      const int left = remaining;
+      unsigned int mine[4], sum = 0u;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        mine[j] = histogram[4 * tid + j];
+        sum += mine[j];
+      }
+      unsigned int inclusive = sum;
+#pragma unroll
+      for (int offset = 1; offset < WAVE; offset <<= 1) {
+        const unsigned int other = __shfl_up(inclusive, offset, WAVE);
+        if (tid >= offset) inclusive += other;
+      }
+      unsigned int before = inclusive - sum;
+      if ((int)before < left && (int)inclusive >= left) {          // exactly one lane
+        int bin = 4 * tid;
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+          if ((int)(before + mine[j]) < left) {
+            before += mine[j];
+            ++bin;
+          } else {
+            break;
+          }
+        }
+        remaining = left - (int)before;
+        chosen_prefix = prefix | ((unsigned long long)bin << (8 * pass));
+        // every key of the bin is wanted: the K-th is the bin's largest, whatever its lower bytes
+        bin_taken_whole = (int)histogram[bin] == left - (int)before ? 1 : 0;
+      }
+    }
+    __syncthreads();
+    if (bin_taken_whole) {
+      if (tid == 0 && pass > 0) chosen_prefix |= (~0ull >> (64 - 8 * pass));
+      __syncthreads();
+      break;
+    }
+  }
+  const unsigned long long kth = chosen_prefix;
+  int padded = 1;
+  while (padded < K) padded <<= 1;
+  for (int i = tid; i < padded; i += blockDim.x) candidates[i] = ~0ull;
+  if (tid == 0) gathered = 0;
+  __syncthreads();
+  for (int v = tid; v < V; v += blockDim.x) {
+    const unsigned long long key = rank_key(values[v] / temp, v);
+    if (key <= kth) {
+      const int slot = atomicAdd(&gathered, 1);
+      if (slot < SAMPLE_KMAX) candidates[slot] = key;
+    }
+  }
+  lds_bitonic_sort(candidates, padded);                        // descending values, ties by ascending index
+  const float maximum = from_orderable(~(unsigned int)(candidates[0] >> 32));
+
+  // ---- softmax normalizer: over the kept tokens (top-k), or over the whole row
+  float normalizer;
+  const int chunk = (K + blockDim.x - 1) / blockDim.x;
+  const int chunk_begin = min(K, tid * chunk);
+  const int chunk_end = min(K, chunk_begin + chunk);
+  float local = 0.f;
+  for (int i = chunk_begin; i < chunk_end; ++i)
+    local += expf(from_orderable(~(unsigned int)(candidates[i] >> 32)) - maximum);
+  float candidate_mass;
+  const float before = block_exclusive_scan(local, scan_scratch, &candidate_mass);
+  if (use_top_k) {
+    normalizer = candidate_mass;
+  } else {
+    float all = 0.f;
+    for (int v = vbegin; v < vend; ++v) all += expf(values[v] / temp - maximum);
+    block_exclusive_scan(all, scan_scratch, &normalizer);
+  }
+
+  // ---- top-p: the shortest prefix in sorted order whose mass reaches top_p
+  constexpr int OPEN = 0x7fffffff;
+  if (tid == 0) found = OPEN;
+  __syncthreads();
+  if (use_top_p) {
+    float cumulative = before / normalizer;
+    for (int i = chunk_begin; i < chunk_end; ++i) {
+      cumulative += expf(from_orderable(~(unsigned int)(candidates[i] >> 32)) - maximum) / normalizer;
+      if (cumulative >= p_limit) {
+        atomicMin(&found, i + 1);
+        break;
+      }
+    }
+  }
+  __syncthreads();
+  const int closed_at = found;
+  __syncthreads();
+  if (closed_at == OPEN && !use_top_k && K < V) return;        // the nucleus is wider than the candidates: sample_kernel's
+  const int nucleus = min(closed_at, K);
+
+  // ---- walk the nucleus in index order
+  int padded_nucleus = 1;
+  while (padded_nucleus < nucleus) padded_nucleus <<= 1;
+  for (int i = tid; i < padded_nucleus; i += blockDim.x)
+    by_index[i] = i < nucleus ? ((candidates[i] & 0xffffffffull) << 32) | (unsigned long long)i : ~0ull;
+  lds_bitonic_sort(by_index, padded_nucleus);
+  const int nchunk = (nucleus + blockDim.x - 1) / blockDim.x;
+  const int nbegin = min(nucleus, tid * nchunk);
+  const int nend = min(nucleus, nbegin + nchunk);
+  auto probability = [&](int position) {
+    const unsigned long long key = candidates[(int)(by_index[position] & 0xffffffffull)];
+    return expf(from_orderable(~(unsigned int)(key >> 32)) - maximum) / normalizer;
+  };
+  float mass = 0.f;
+  for (int i = nbegin; i < nend; ++i) mass += probability(i);
+  float total;
+  const float start = block_exclusive_scan(mass, scan_scratch, &total);
+  const float target = u * total;
+  if (tid == 0) found = nucleus;
+  __syncthreads();
+  float cumulative = start;
+  for (int i = nbegin; i < nend; ++i) {
+    const float p = probability(i);
+    if (p <= 0.f) continue;
+    cumulative += p;
+    if (target < cumulative) {
+      atomicMin(&found, i);
+      break;
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    out[row] = found < nucleus ? (int)(by_index[found] >> 32) : (int)(candidates[0] & 0xffffffffu);
+    done[row] = 1;
+  }
+}
+
 extern "C" int mi_sample(float* logits, int B, int V, int padded, const float* temperature, const int* top_k,
                          const float* top_p, const unsigned long long* seeds, const int* draw_index,
-                         unsigned long long* keys, int* out, hipStream_t stream) {
+                         unsigned long long* keys, int* out, int* done, hipStream_t stream) {
   if (B <= 0 || V <= 0 || padded < V || (padded & (padded - 1)) != 0) return ERR_BAD_ARGUMENT;
+  // done: int32 [B] work area, or null to sort every row (the reference path of the tests)
+  if (done != nullptr) {
+    sample_select_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, V, temperature, top_k, top_p, seeds, draw_index,
+                                                           out, done);
+    RETURN_IF_LAUNCH_FAILED();
+  }
   sample_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, V, padded, temperature, top_k, top_p, seeds,
-                                                  draw_index, keys, out);
+                                                  draw_index, keys, out, done);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

@@ -81,7 +81,7 @@ _SIGNATURES = {
                                _c_ptr, _c_ptr],
         "mi_argmax": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
         "mi_sample": [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                      _c_ptr],
+                      _c_ptr, _c_ptr],
     },
 }
 
@@ -689,8 +689,11 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     _check(_fn("sampling", "mi_argmax")(_p(logits), B, V, _p(out), _stream()), "argmax")
 
 
-def sample(logits, temperature, top_k, top_p, seeds, draw_index, keys, out) -> None:
-    """One token per row; overwrites ``logits``.  ``keys`` int64 [B, padded] work area."""
+def sample(logits, temperature, top_k, top_p, seeds, draw_index, keys, out, done=None) -> None:
+    """One token per row; may overwrite ``logits``.  ``keys`` int64 [B, padded] work area.  With
+    ``done`` (int32 [B] work area) the rows that need no full sort (top-k up to 1 024, or a
+    nucleus within the 1 024 best, or neither top-k nor top-p) are drawn by selection; without it
+    every row is sorted."""
     B, V = logits.shape
     _need(logits.dtype == torch.float32 and logits.is_contiguous() and logits.is_cuda, "sample: bad logits")
     padded = keys.shape[1]
@@ -700,5 +703,8 @@ def sample(logits, temperature, top_k, top_p, seeds, draw_index, keys, out) -> N
     _i32(top_k, "top_k")
     _i32(draw_index, "draw_index")
     _i32(out, "out")
+    if done is not None:
+        _i32(done, "done")
+        _need(done.numel() >= B, "sample: done must hold one flag per row")
     _check(_fn("sampling", "mi_sample")(_p(logits), B, V, padded, _p(temperature), _p(top_k), _p(top_p),
-                                        _p(seeds), _p(draw_index), _p(keys), _p(out), _stream()), "sample")
+                                        _p(seeds), _p(draw_index), _p(keys), _p(out), _p(done), _stream()), "sample")

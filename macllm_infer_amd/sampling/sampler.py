@@ -11,6 +11,7 @@ from __future__ import annotations
 
 from typing import List, Sequence
 
+import numpy as np
 import torch
 
 from ..kernels import build as kernel_build
@@ -59,9 +60,6 @@ class Sampler:
             raise ValueError(f"logits have shape {tuple(logits.shape)}, expected {(B, self.vocab_size)}")
         device = self.device
 
-        def upload(values, dtype):
-            return torch.tensor(values, dtype=dtype).to(device, non_blocking=True)
-
         if any(row.params.uses_penalties for row in rows):
             tokens: List[int] = []
             offsets = [0]
@@ -71,24 +69,33 @@ class Sampler:
                     tokens.extend(row.generated)
                 offsets.append(len(tokens))
             count_all, count_gen = self._count_areas(B)
+            # one upload: offsets (B+1) | prompt lengths | the three penalties (float bits) | the histories
+            head = 5 * B + 1
+            words = np.empty(head + max(len(tokens), 1), dtype=np.int32)
+            words[:B + 1] = offsets
+            words[B + 1:2 * B + 1] = [len(row.prompt) for row in rows]
+            words[2 * B + 1:3 * B + 1].view(np.float32)[:] = [row.params.repetition_penalty for row in rows]
+            words[3 * B + 1:4 * B + 1].view(np.float32)[:] = [row.params.presence_penalty for row in rows]
+            words[4 * B + 1:head].view(np.float32)[:] = [row.params.frequency_penalty for row in rows]
+            words[head:] = tokens or [0]
+            packed = torch.from_numpy(words).to(device, non_blocking=True)
             ops.apply_penalties(
-                logits, upload(tokens or [0], torch.int32), upload(offsets, torch.int32),
-                upload([len(row.prompt) for row in rows], torch.int32),
-                upload([row.params.repetition_penalty for row in rows], torch.float32),
-                upload([row.params.presence_penalty for row in rows], torch.float32),
-                upload([row.params.frequency_penalty for row in rows], torch.float32), count_all, count_gen)
+                logits, packed[head:], packed[:B + 1], packed[B + 1:2 * B + 1],
+                packed[2 * B + 1:3 * B + 1].view(torch.float32), packed[3 * B + 1:4 * B + 1].view(torch.float32),
+                packed[4 * B + 1:head].view(torch.float32), count_all, count_gen)
         out = torch.empty(B, dtype=torch.int32, device=device)
         if all(row.params.greedy for row in rows):
             ops.argmax(logits, out)
         else:
-            def as_signed(seed: int) -> int:
-                seed &= (1 << 64) - 1
-                return seed - (1 << 64) if seed >= (1 << 63) else seed
-            ops.sample(logits,
-                       upload([row.params.temperature for row in rows], torch.float32),
-                       upload([row.params.top_k for row in rows], torch.int32),
-                       upload([row.params.top_p for row in rows], torch.float32),
-                       upload([as_signed(row.params.seed) for row in rows], torch.int64),
-                       upload([len(row.generated) for row in rows], torch.int32),
-                       self._work(B), out)
+            # one upload for the five parameter arrays: seeds (int64) first, then 32-bit words
+            words = np.empty(6 * B, dtype=np.int32)
+            words[:2 * B].view(np.uint64)[:] = [row.params.seed & ((1 << 64) - 1) for row in rows]
+            words[2 * B:3 * B].view(np.float32)[:] = [row.params.temperature for row in rows]
+            words[3 * B:4 * B].view(np.float32)[:] = [row.params.top_p for row in rows]
+            words[4 * B:5 * B] = [row.params.top_k for row in rows]
+            words[5 * B:] = [len(row.generated) for row in rows]
+            packed = torch.from_numpy(words).to(device, non_blocking=True)
+            ops.sample(logits, packed[2 * B:3 * B].view(torch.float32), packed[4 * B:5 * B],
+                       packed[3 * B:4 * B].view(torch.float32), packed[:2 * B].view(torch.int64), packed[5 * B:],
+                       self._work(B), out, torch.empty(B, dtype=torch.int32, device=device))
         return out.cpu().tolist()

@@ -199,7 +199,7 @@ def apply_penalties(logits, tokens, offsets, prompt_lens, repetition, presence, 
                 logits[row, token] -= freq * generated.count(token) + pres
 
 
-def sample(logits, temperature, top_k, top_p, seeds, draw_index, keys, out):
+def sample(logits, temperature, top_k, top_p, seeds, draw_index, keys, out, done=None):
     import plain_impl
     for row in range(logits.shape[0]):
         out[row] = plain_impl.sample_token(

@@ -413,15 +413,22 @@ def test_argmax_and_ties(ops):
     assert out.cpu()[1] == 17 and out.cpu()[2] == 1002
 
 
+@pytest.mark.parametrize("select", [False, True], ids=["sorted", "selected"])
 @pytest.mark.parametrize("V", [320, 1003, 32784])
-def test_sampling_matches_the_plain_sampler(ops, V):
+def test_sampling_matches_the_plain_sampler(ops, V, select):
+    """Every row is sorted whole, or (``select``) rows are drawn by selection where that covers
+    them: top-k 1, 7, 20, 40 and 1 024; a nucleus that closes within the 1 024 best candidates
+    (rows with peaked logits) and one that does not (flat logits: handed on to the full sort);
+    top-k above 1 024 (handed on); neither top-k nor top-p; a greedy row."""
     import plain_impl
     settings = [(0.8, 0, 1.0), (1.0, 7, 1.0), (0.9, 0, 0.7), (1.2, 40, 0.85), (0.0, 0, 1.0), (0.7, 20, 0.8),
-                (1.0, V + 5, 0.999), (0.5, 1, 0.1)]
+                (1.0, V + 5, 0.999), (0.5, 1, 0.1), (1.0, 1024, 0.95), (1.1, 1500, 0.9), (0.6, 0, 0.9), (1.0, 0, 0.5)]
     B = len(settings)
     logits = rand(B, V, seed=81, scale=2.5)
-    seeds = [3, 99, 2 ** 63 + 5, 42, 0, 7, 11, 13]
-    draws = [0, 5, 17, 3, 0, 100, 1, 2]
+    logits[10] *= 4.0                                            # peaked: the nucleus is a handful of tokens
+    logits[11] *= 0.02                                           # flat: half the mass is half the vocabulary
+    seeds = [3, 99, 2 ** 63 + 5, 42, 0, 7, 11, 13, 17, 19, 23, 29]
+    draws = [0, 5, 17, 3, 0, 100, 1, 2, 8, 9, 10, 11]
     padded = 1
     while padded < V:
         padded <<= 1
@@ -432,7 +439,8 @@ def test_sampling_matches_the_plain_sampler(ops, V):
         ops.sample(work, torch.tensor([s[0] for s in settings]).to(DEV), i32([s[1] for s in settings]).to(DEV),
                    torch.tensor([s[2] for s in settings]).to(DEV), torch.tensor(signed, dtype=torch.int64).to(DEV),
                    i32([d + repeat for d in draws]).to(DEV),
-                   torch.empty(B, padded, dtype=torch.int64, device=DEV), out)
+                   torch.empty(B, padded, dtype=torch.int64, device=DEV), out,
+                   torch.full((B,), 7, dtype=torch.int32, device=DEV) if select else None)
         want = [plain_impl.sample_token(logits[row], temperature=settings[row][0], top_k=settings[row][1],
                                         top_p=settings[row][2], seed=seeds[row], draw_index=draws[row] + repeat)
                 for row in range(B)]
