@@ -26,7 +26,7 @@ typedef __bf16 s_bf16x4 __attribute__((ext_vector_type(4)));
 typedef float s_floatx4 __attribute__((ext_vector_type(4)));
 
 #define SSD_MAX_Q 256
-#define SSD_HEADS_PER_BLOCK 4
+#define SSD_HEADS_PER_BLOCK 1
 
 // chunk table: int32 [n_chunks, 4] = (lane, first token row, length, index of the chunk within its lane)
 
