@@ -378,6 +378,203 @@ ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t*
   }
 }
 
+// The same with the operands that the eight tiles of 128 tokens share staged in LDS: one
+// workgroup of eight waves per (chunk, head, 128 tokens), a tile of 16 tokens a wave.  S_in of
+// the head (64 rows at a time), then, 64 tokens s at a time, the rows of B and the columns of
+// x^T go through LDS once for all tiles instead of once per tile from the caches; only C, the
+// skip and the gate are read per tile.  Rows are padded by 16 bytes so that the 16 rows a
+// matrix-core operand reads fall in different banks.  Head sizes up to 128.
+#define SSD_SCAN_WAVES 8
+template <int NK, int PT>
+__global__ void __launch_bounds__(SSD_SCAN_WAVES * WAVE)
+ssd_chunk_scan_lds_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t* __restrict__ TT, int E,
+                          const bf16_t* __restrict__ state_in, const float* __restrict__ delta,
+                          const float* __restrict__ cum, const float* __restrict__ D,
+                          const int* __restrict__ chunks, int Q, int H, int G, float* __restrict__ y,
+                          long y_ld, const bf16_t* __restrict__ z, long z_ld, bf16_t* __restrict__ gated,
+                          long gated_ld) {
+  constexpr int N = 32 * NK;
+  constexpr int P = 16 * PT;
+  constexpr int LD1 = N + 8;                     // row stride of the S / B buffer
+  constexpr int LDX = 64 + 8;                    // row stride of the x^T buffer
+  constexpr int THREADS = SSD_SCAN_WAVES * WAVE;
+  extern __shared__ __align__(16) unsigned char scan_smem[];
+  bf16_t* buf1 = reinterpret_cast<bf16_t*>(scan_smem);                 // [64][LD1]: S_in rows, then B rows
+  bf16_t* buf_x = buf1 + 64 * LD1;                                     // [P][LDX]
+  float* L = reinterpret_cast<float*>(buf_x + (long)P * LDX);          // [Q]
+  float* step = L + Q;                                                 // [Q]
+  const int chunk = blockIdx.x;
+  const int head = blockIdx.y;
+  const int group = head / (H / G);
+  const int t0 = chunks[4 * chunk + 1];
+  const int length = chunks[4 * chunk + 2];
+  const int part = gridDim.z - 1 - blockIdx.z;                         // the later 128 tokens first: they have more before them
+  if (part * 128 >= length) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  const int q = lane / 16;
+  const int n = lane % 16;
+  const int tile = part * 8 + wave;
+  const int end_s = min(length, part * 128 + 128);
+  const int GN = G * N;
+  const int b_col = E + group * N;
+  const int c_col = E + GN + group * N;
+  const int last_row = t0 + length - 1;
+  const int t = tile * 16 + n;
+  const bool tile_live = tile * 16 < length;
+  const bool has_t = t < length;
+  const int t_safe = min(t, length - 1);
+  const long t_row = t0 + t_safe;
+
+  for (int s = tid; s < end_s; s += THREADS) {
+    L[s] = cum[(long)(t0 + s) * H + head];
+    step[s] = delta[(long)(t0 + s) * H + head];
+  }
+  // per tile: C of the column, the skip and the gate operands (asked for now, used at the end)
+  s_bf16x8 c_frag[NK];
+#pragma unroll
+  for (int kk = 0; kk < NK; ++kk)
+    c_frag[kk] = *reinterpret_cast<const s_bf16x8*>(xbc + t_row * xbc_ld + c_col + 32 * kk + 8 * q);
+  if (!has_t) {
+#pragma unroll
+    for (int kk = 0; kk < NK; ++kk)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) c_frag[kk][j] = (bf16_t)0.f;
+  }
+
+  s_floatx4 acc[PT];
+#pragma unroll
+  for (int pi = 0; pi < PT; ++pi) acc[pi] = s_floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // ---- inter-chunk term: S_in through LDS, 64 rows at a time
+  const bf16_t* s_head = state_in + ((long)chunk * H + head) * P * N;
+  for (int pb = 0; pb * 64 < P; ++pb) {
+    __syncthreads();
+    for (int index = tid; index < 64 * (N / 8); index += THREADS) {
+      const int row = index / (N / 8);
+      const int v = index % (N / 8);
+      const int p = min(pb * 64 + row, P - 1);
+      *reinterpret_cast<s_bf16x8*>(buf1 + row * LD1 + 8 * v) =
+          *reinterpret_cast<const s_bf16x8*>(s_head + (long)p * N + 8 * v);
+    }
+    __syncthreads();
+    if (tile_live) {
+#pragma unroll
+      for (int pi = 0; pi < PT; ++pi) {
+        if (pi / 4 == pb) {
+#pragma unroll
+          for (int kk = 0; kk < NK; ++kk) {
+            const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(buf1 + ((pi % 4) * 16 + n) * LD1 + 32 * kk + 8 * q);
+            acc[pi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], acc[pi], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  {
+    const float carry = __expf(L[min(t_safe, end_s - 1)]);
+#pragma unroll
+    for (int pi = 0; pi < PT; ++pi)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[pi][i] *= carry;
+  }
+
+  // ---- intra-chunk term: 64 tokens s at a time, B rows and x^T columns through LDS
+  const bf16_t* x_head = TT + ((long)chunk * (E + GN) + (long)head * P) * Q;
+  for (int sb = 0; sb * 64 < end_s; ++sb) {
+    __syncthreads();
+    for (int index = tid; index < 64 * (N / 8); index += THREADS) {
+      const int row = index / (N / 8);
+      const int v = index % (N / 8);
+      const long s_row = min((long)t0 + sb * 64 + row, (long)last_row);
+      *reinterpret_cast<s_bf16x8*>(buf1 + row * LD1 + 8 * v) =
+          *reinterpret_cast<const s_bf16x8*>(xbc + s_row * xbc_ld + b_col + 8 * v);
+    }
+    for (int index = tid; index < P * 8; index += THREADS) {
+      const int row = index / 8;
+      const int v = index % 8;
+      s_bf16x8 value;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) value[j] = (bf16_t)0.f;
+      if (sb * 64 + 8 * v < Q) value = *reinterpret_cast<const s_bf16x8*>(x_head + (long)row * Q + sb * 64 + 8 * v);
+      *reinterpret_cast<s_bf16x8*>(buf_x + row * LDX + 8 * v) = value;
+    }
+    __syncthreads();
+    if (!tile_live) continue;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int s0 = sb * 64 + 32 * j;
+      if (s0 > tile * 16 + 15 || s0 >= length) continue;
+      s_floatx4 w[2];
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        w[half] = s_floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) {
+          const s_bf16x8 a = *reinterpret_cast<const s_bf16x8*>(buf1 + (32 * j + 16 * half + n) * LD1 + 32 * kk + 8 * q);
+          w[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c_frag[kk], w[half], 0, 0, 0);
+        }
+      }
+      s_bf16x8 p_frag;
+      const float l_t = L[min(t_safe, end_s - 1)];
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int s = s0 + 16 * half + 4 * q + i;
+          const int s_safe = min(s, end_s - 1);
+          const bool visible = has_t && s <= t && s < length;
+          const float value = visible ? w[half][i] * __expf(l_t - L[s_safe]) * step[s_safe] : 0.f;
+          p_frag[4 * half + i] = (bf16_t)value;
+        }
+#pragma unroll
+      for (int pi = 0; pi < PT; ++pi) {
+        const bf16_t* x_row = buf_x + (pi * 16 + n) * LDX + 32 * j + 4 * q;
+        const s_bf16x4 lo = *reinterpret_cast<const s_bf16x4*>(x_row);
+        const s_bf16x4 hi = *reinterpret_cast<const s_bf16x4*>(x_row + 16);
+        s_bf16x8 a;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a[e] = lo[e];
+          a[4 + e] = hi[e];
+        }
+        acc[pi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p_frag, acc[pi], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- y[t, h*P + 16 pi + 4q + i] = acc + D x
+  if (!has_t) return;
+  const float skip = D[head];
+  s_bf16x4 x_skip[PT], gate[PT];
+#pragma unroll
+  for (int pi = 0; pi < PT; ++pi) {
+    const long column = (long)head * P + pi * 16 + 4 * q;
+    x_skip[pi] = *reinterpret_cast<const s_bf16x4*>(xbc + t_row * xbc_ld + column);
+    gate[pi] = *reinterpret_cast<const s_bf16x4*>((z != nullptr ? z + t_row * z_ld : xbc + t_row * xbc_ld) + column);
+  }
+#pragma unroll
+  for (int pi = 0; pi < PT; ++pi) {
+    const long column = (long)head * P + pi * 16 + 4 * q;
+    s_floatx4 out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = acc[pi][i] + skip * (float)x_skip[pi][i];
+    if (z != nullptr) {
+      s_bf16x4 packed;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(out[i] * silu_f((float)gate[pi][i]));
+      *reinterpret_cast<s_bf16x4*>(gated + t_row * gated_ld + column) = packed;
+    } else {
+      *reinterpret_cast<s_floatx4*>(y + t_row * y_ld + column) = out;
+    }
+  }
+}
+
+static size_t ssd_scan_lds_bytes(int Q, int P, int N) {
+  return (size_t)64 * (N + 8) * 2 + (size_t)P * (64 + 8) * 2 + (size_t)2 * Q * 4;
+}
+
 // Sizes: bfloat16; Q a multiple of 32 and at most 256; head_dim P a multiple of 16; state size N a
 // multiple of 32 and at most 256; row strides multiples of 8 elements.  Otherwise
 // ERR_UNSUPPORTED_SIZE (the caller uses mi_ssm_scan).
@@ -432,7 +629,23 @@ extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long
                                                     ssm_state, (bf16_t*)state_in);
     RETURN_IF_LAUNCH_FAILED();
   }
-  {
+  const bool staged = (P == 16 || P == 32 || P == 64 || P == 128) && (N == 32 || N == 64 || N == 128 || N == 256) &&
+                      ssd_scan_lds_bytes(Q, P, N) <= 64 * 1024;
+  if (staged) {
+    const dim3 grid(n_chunks, H, (Q + 127) / 128);
+    const size_t lds = ssd_scan_lds_bytes(Q, P, N);
+#define SCAN_LDS_CASE(NK_, PT_)                                                                                   \
+  if (N == 32 * NK_ && P == 16 * PT_)                                                                             \
+    ssd_chunk_scan_lds_kernel<NK_, PT_><<<grid, SSD_SCAN_WAVES * WAVE, lds, stream>>>(                            \
+        (const bf16_t*)xbc, xbc_ld, (const bf16_t*)TT, E, (const bf16_t*)state_in, delta, cum, D, chunks, Q, H, G, \
+        y, y_ld, (const bf16_t*)z, z_ld, (bf16_t*)gated, gated_ld);
+    SCAN_LDS_CASE(1, 1) SCAN_LDS_CASE(1, 2) SCAN_LDS_CASE(1, 4) SCAN_LDS_CASE(1, 8)
+    SCAN_LDS_CASE(2, 1) SCAN_LDS_CASE(2, 2) SCAN_LDS_CASE(2, 4) SCAN_LDS_CASE(2, 8)
+    SCAN_LDS_CASE(4, 1) SCAN_LDS_CASE(4, 2) SCAN_LDS_CASE(4, 4) SCAN_LDS_CASE(4, 8)
+    SCAN_LDS_CASE(8, 1) SCAN_LDS_CASE(8, 2) SCAN_LDS_CASE(8, 4) SCAN_LDS_CASE(8, 8)
+#undef SCAN_LDS_CASE
+    RETURN_IF_LAUNCH_FAILED();
+  } else {
     const int subsets = (H / G + SSD_HEADS_PER_BLOCK - 1) / SSD_HEADS_PER_BLOCK;
     const dim3 grid(n_chunks, G * subsets, (Q + 63) / 64);
 #define SCAN_CASE(NK_)                                                                                            \
