@@ -112,7 +112,7 @@ ssd_transpose_kernel(const bf16_t* __restrict__ xbc, long ld, int channels, cons
 // first, B rows after.  QK = Q / 32 is a template parameter and a tile of rows that does not
 // exist is clamped, so that all fragments of a tile are asked for at once.
 template <int QK>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 ssd_chunk_state_kernel(const bf16_t* __restrict__ TT, int E, int GN, const float* __restrict__ delta,
                        const float* __restrict__ cum, const int* __restrict__ chunks, int H, int P, int N, int G,
                        float* __restrict__ chunk_state, float* __restrict__ chunk_decay) {
@@ -129,7 +129,7 @@ ssd_chunk_state_kernel(const bf16_t* __restrict__ TT, int E, int GN, const float
   const int q = lane / 16;
   const int r = lane % 16;
   const float total = cum[(long)(t0 + length - 1) * H + head];
-  for (int s = tid; s < Q; s += 256) {
+  for (int s = tid; s < Q; s += 512) {
     const long at = (long)(t0 + min(s, length - 1)) * H + head;
     const float value = __expf(total - cum[at]) * delta[at];
     weight[s] = s < length ? value : 0.f;
@@ -140,7 +140,7 @@ ssd_chunk_state_kernel(const bf16_t* __restrict__ TT, int E, int GN, const float
   const bf16_t* b_rows = TT + ((long)chunk * (E + GN) + E + (long)group * N) * Q;
   float* out = chunk_state + ((long)chunk * H + head) * P * N;
   const int p_tiles = P / 16;
-  for (int nt = wave; nt < N / 16; nt += 4) {
+  for (int nt = wave; nt < N / 16; nt += 8) {
     for (int pt0 = 0; pt0 < p_tiles; pt0 += 4) {            // four p-tiles share the weighted B fragments
       s_bf16x8 b_raw[QK], x[4][QK];
 #pragma unroll
@@ -612,7 +612,7 @@ extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long
     const dim3 grid(n_chunks, H);
 #define STATE_CASE(QK_)                                                                                         \
   case QK_:                                                                                                     \
-    ssd_chunk_state_kernel<QK_><<<grid, 256, 0, stream>>>((const bf16_t*)TT, E, GN, delta, cum, chunks, H, P, N, G, \
+    ssd_chunk_state_kernel<QK_><<<grid, 512, 0, stream>>>((const bf16_t*)TT, E, GN, delta, cum, chunks, H, P, N, G, \
                                                           chunk_state, chunk_decay);                          \
     break;
     switch (Q / 32) {
