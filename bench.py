@@ -153,7 +153,8 @@ def main() -> int:
                    "heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
                    "head_dim": config.head_dim, "intermediate": config.intermediate_size,
                    "mamba_heads": config.mamba_n_heads, "mamba_head_dim": config.mamba_d_head,
-                   "mamba_state": config.mamba_d_state, "mamba_conv": config.mamba_d_conv, "vocab": vocab,
+                   "mamba_state": config.mamba_d_state, "mamba_groups": config.mamba_n_groups,
+                   "mamba_conv": config.mamba_d_conv, "mamba_chunk": config.mamba_chunk_size, "vocab": vocab,
                    "tied_embeddings": True, "global_batch": args.batch, "seq_len": CONTEXT,
                    "page_tokens": args.page_tokens, "parallelism": "single GPU"},
         "prefill": {"value": round(PREFILL_TOKENS / prefill_seconds, 1), "tokens": PREFILL_TOKENS,

@@ -138,14 +138,20 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
           score[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[st][t][kk], q_frag[s][kk], score[t], 0, 0, 0);
       }
       // scores in units of log2: s * scale * log2(e), so that the exponentials are bare v_exp
+      // visible keys of the column: first_visible .. min(position, last_key); relative to the step
+      // they are lo .. lo + span, so one unsigned compare per score decides (an empty range gets a
+      // lo that no offset reaches)
       const int position = col_pos[s];
-      const int first_visible = window > 0 ? position - window + 1 : 0;
+      const int first_visible = window > 0 ? max(position - window + 1, 0) : 0;
+      const int last_visible = min(position, last_key);
+      const bool any = last_visible >= first_visible;
+      const int lo = any ? first_visible - k0 : 0x40000000;
+      const unsigned span = any ? (unsigned)(last_visible - first_visible) : 0u;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int key = k0 + 16 * t + 4 * q + i;
-          const bool visible = key <= position && key >= first_visible && key <= last_key;
+          const bool visible = (unsigned)(16 * t + 4 * q + i - lo) <= span;
           score[t][i] = visible ? score[t][i] : -INFINITY;
         }
       float step_max = fmaxf(fmaxf(fmaxf(score[0][0], score[0][1]), fmaxf(score[0][2], score[0][3])),
