@@ -224,6 +224,8 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   // when the block has 16 x 16 outputs) is asked for now, behind the weights; no branch between
   // its loads either
   bf16_t tail_values[8];
+  float tap_values[9];
+  float tap_bias = 0.f;
   bool tail_ready = false;
   if (EPI == EPI_CONV) asm volatile("" : "+v"(tail_slot));      // keeps every use of the slot (and its wait) down here
   if (tail_wanted) {
@@ -231,6 +233,9 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
     const bf16_t* tail = p.conv_state + (long)tail_slot * (p.conv_k - 1) * channels + (tail_n - p.conv_lo);
 #pragma unroll
     for (int k = 0; k < 8; ++k) tail_values[k] = tail[(long)min(k, p.conv_k - 2) * channels];
+#pragma unroll
+    for (int k = 0; k < 9; ++k) tap_values[k] = p.conv_w[(long)(tail_n - p.conv_lo) * p.conv_k + min(k, p.conv_k - 1)];
+    if (p.conv_b) tap_bias = p.conv_b[tail_n - p.conv_lo];
     tail_ready = true;
   }
 
@@ -299,15 +304,31 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
       const int channel = n - p.conv_lo;
       const int channels = p.conv_hi - p.conv_lo;
       const int taps = p.conv_k;
-      bf16_t* tail = p.conv_state + (long)p.slot_ids[m] * (taps - 1) * channels + channel;
+      bf16_t* tail = p.conv_state + (long)(tail_ready ? tail_slot : p.slot_ids[m]) * (taps - 1) * channels + channel;
       const bf16_t sample = (bf16_t)v;
-      float sum = p.conv_b ? p.conv_b[channel] : 0.f;
-      for (int k = 0; k < taps - 1; ++k) {
-        const bf16_t old = tail_ready ? tail_values[k] : tail[(long)k * channels];
-        sum += p.conv_w[channel * taps + k] * (float)old;
-        if (k > 0) tail[(long)(k - 1) * channels] = old;       // roll the tail by one
+      float sum;
+      if (tail_ready) {                       // taps, bias and tail are in registers already
+        sum = tap_bias;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          if (k < taps - 1) {
+            sum += tap_values[k] * (float)tail_values[k];
+            if (k > 0) tail[(long)(k - 1) * channels] = tail_values[k];       // roll the tail by one
+          }
+        }
+        float last_tap = tap_values[0];
+#pragma unroll
+        for (int k = 1; k < 9; ++k) last_tap = k == taps - 1 ? tap_values[k] : last_tap;
+        sum += last_tap * (float)sample;
+      } else {
+        sum = p.conv_b ? p.conv_b[channel] : 0.f;
+        for (int k = 0; k < taps - 1; ++k) {
+          const bf16_t old = tail[(long)k * channels];
+          sum += p.conv_w[channel * taps + k] * (float)old;
+          if (k > 0) tail[(long)(k - 1) * channels] = old;       // roll the tail by one
+        }
+        sum += p.conv_w[channel * taps + taps - 1] * (float)sample;
       }
-      sum += p.conv_w[channel * taps + taps - 1] * (float)sample;
       if (taps > 1) tail[(long)(taps - 2) * channels] = sample;
       reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + n] = (bf16_t)silu_f(sum);
     } else if (p.out_f32) {
