@@ -634,6 +634,52 @@ def test_mixer_decode_against_the_separate_kernels(ops, Hq, Hkv, dh, H, P, N, G,
         close(torch.nan_to_num(got_pool.float()), torch.nan_to_num(want_pool.float()), dtype, 4.0)
 
 
+def test_mixer_decode_over_a_long_context(ops):
+    """Contexts of 5 000 and 9 000 tokens (10 and 18 runs of 512 keys: more than the merge takes
+    at once) beside a short one; one far key per long request is made to dominate, so a run that
+    is dropped or merged with the wrong weight shows."""
+    dtype = torch.bfloat16
+    Hq, Hkv, dh, H, P, N, G, page_size = 4, 2, 64, 2, 16, 32, 1, 16
+    lengths = [5000, 9000, 3]
+    M = len(lengths)
+    pool, table = paged_setup(lengths, page_size, Hkv, dh, dtype, seed=12)
+    E = H * P
+    q_col, k_col, v_col = 0, Hq * dh, (Hq + Hkv) * dh
+    z_col = (Hq + 2 * Hkv) * dh
+    x_col, dt_col = z_col + E, z_col + 2 * E + 2 * G * N
+    u = rand(M, -(-(dt_col + H) // 8) * 8, seed=420, dtype=dtype)
+    for lane, length in enumerate(lengths):
+        keys = rand(length, Hkv, dh, seed=430 + lane, dtype=dtype)
+        values = rand(length, Hkv, dh, seed=440 + lane, dtype=dtype)
+        if length > 1000:                                    # key 700 looks like the query of head 0 / 2
+            for kvh in range(Hkv):
+                keys[700, kvh] = u[lane, q_col + kvh * (Hq // Hkv) * dh:q_col + kvh * (Hq // Hkv) * dh + dh] * 3.0
+            values[700] = 5.0
+        fill_cache(pool, table, lane, keys, values, page_size)
+    positions = i32([length - 1 for length in lengths])
+    slot_mapping = i32([int(table[lane, (length - 1) // page_size]) * page_size + (length - 1) % page_size
+                        for lane, length in enumerate(lengths)])
+    slot_ids = i32([2, 0, 1])
+    state = rand(M + 1, H, P, N, seed=421, scale=0.5)
+    dt_bias, A, D = rand(H, seed=422) - 2.0, -(rand(H, seed=423).abs() + 0.1), rand(H, seed=424)
+    common = dict(num_heads=Hq, num_kv_heads=Hkv, head_dim=dh, q_col=q_col, k_col=k_col, v_col=v_col, inv_freq=None,
+                  rotary_dim=0, scale=0.125, window=None, max_seq_len=9216, ssm_heads=H, ssm_head_dim=P,
+                  state_size=N, num_groups=G, z_col=z_col, x_col=x_col, dt_col=dt_col)
+    want_pool, want_state = pool.clone(), state.clone()
+    want_out = torch.zeros(M, Hq * dh + E, dtype=dtype)
+    ref_ops.mixer_decode(u, k_cache=views(want_pool, page_size)[0], v_cache=views(want_pool, page_size)[1],
+                         block_tables=table, positions=positions, slot_mapping=slot_mapping, dt_bias=dt_bias, A=A, D=D,
+                         ssm_state=want_state, slot_ids=slot_ids, out=want_out, ssm_y=None, **common)
+    assert want_out[0, :dh].float().mean() > 3.0             # the far key does dominate head 0
+    got_pool, got_state = pool.clone().to(DEV), state.clone().to(DEV)
+    got_out = torch.zeros(M, Hq * dh + E, dtype=dtype, device=DEV)
+    ops.mixer_decode(u.to(DEV), k_cache=views(got_pool, page_size)[0], v_cache=views(got_pool, page_size)[1],
+                     block_tables=table.to(DEV), positions=positions.to(DEV), slot_mapping=slot_mapping.to(DEV),
+                     dt_bias=dt_bias.to(DEV), A=A.to(DEV), D=D.to(DEV), ssm_state=got_state,
+                     slot_ids=slot_ids.to(DEV), out=got_out, ssm_y=None, **common)
+    close(got_out, want_out, dtype, max(1.0, want_out.float().abs().max().item()))
+
+
 # ------------------------------------------------------------------ prefill attention on the matrix cores
 @pytest.mark.parametrize("Hq, Hkv, dh, page_size, window", [(8, 2, 64, 16, None), (4, 4, 128, 16, None),
                                                               (12, 2, 64, 4, None), (5, 1, 64, 64, None),
