@@ -164,45 +164,55 @@ extern "C" int mi_add_rmsnorm(float* h, const void* delta0, const void* delta1, 
 }
 
 // ---------------------------------------------------------------- SwiGLU
-// out[t, i] = SiLU(gu[t, i]) * gu[t, I + i]      (reference: src/decoder.rs:298-305)
+// out[t, i] = SiLU(g[t, i]) * u[t, i]      (reference: src/decoder.rs:298-305)
+// A row of the input holds [g | u] (tile = 0), or g and u interleaved in tiles:
+// [g[0:tile] | u[0:tile] | g[tile:2 tile] | ...], the layout the fused decode kernel wants its
+// weight rows in (tile = 8), so that one matrix serves both.
+__device__ __forceinline__ long swiglu_gate_at(int i, int I, int tile) {
+  return tile == 0 ? i : (long)(i / tile) * 2 * tile + i % tile;
+}
+
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, long ld, T* __restrict__ out, int I, long total) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, long ld, T* __restrict__ out, int I, int tile, long total) {
   const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (index >= total) return;
   const long t = index / I;
   const int i = (int)(index - t * I);
-  const float gate = to_float(gu[t * ld + i]);
-  const float up = to_float(gu[t * ld + I + i]);
+  const long at = swiglu_gate_at(i, I, tile);
+  const float gate = to_float(gu[t * ld + at]);
+  const float up = to_float(gu[t * ld + at + (tile == 0 ? I : tile)]);
   out[index] = from_float<T>(silu_f(gate) * up);
 }
 
-// bfloat16, eight elements a thread (I, ld and the addresses multiples of 8 elements)
+// bfloat16, eight elements a thread (I, ld and the addresses multiples of 8 elements; tile 0 or 8)
 typedef __bf16 common_bf16x8 __attribute__((ext_vector_type(8)));
 __global__ void __launch_bounds__(256)
-swiglu_vec_kernel(const bf16_t* __restrict__ gu, long ld, bf16_t* __restrict__ out, int I, long total) {
+swiglu_vec_kernel(const bf16_t* __restrict__ gu, long ld, bf16_t* __restrict__ out, int I, int tile, long total) {
   const long index = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (index >= total) return;
   const long t = index / I;
   const int i = (int)(index - t * I);
-  const common_bf16x8 gate = *reinterpret_cast<const common_bf16x8*>(gu + t * ld + i);
-  const common_bf16x8 up = *reinterpret_cast<const common_bf16x8*>(gu + t * ld + I + i);
+  const long at = tile == 0 ? i : 2L * i;
+  const common_bf16x8 gate = *reinterpret_cast<const common_bf16x8*>(gu + t * ld + at);
+  const common_bf16x8 up = *reinterpret_cast<const common_bf16x8*>(gu + t * ld + at + (tile == 0 ? I : 8));
   common_bf16x8 result;
 #pragma unroll
   for (int j = 0; j < 8; ++j) result[j] = (bf16_t)(silu_f((float)gate[j]) * (float)up[j]);
   *reinterpret_cast<common_bf16x8*>(out + index) = result;
 }
 
-extern "C" int mi_swiglu(const void* gu, int dtype, long ld, void* out, int T, int I, hipStream_t stream) {
-  if (T <= 0 || I <= 0 || ld < 2L * I) return ERR_BAD_ARGUMENT;
+extern "C" int mi_swiglu(const void* gu, int dtype, long ld, void* out, int T, int I, int tile, hipStream_t stream) {
+  if (T <= 0 || I <= 0 || ld < 2L * I || tile < 0 || (tile > 0 && I % tile != 0)) return ERR_BAD_ARGUMENT;
   const long total = (long)T * I;
   const int blocks = (int)((total + 255) / 256);
-  if (dtype == DT_BF16 && I % 8 == 0 && ld % 8 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+  if (dtype == DT_BF16 && I % 8 == 0 && ld % 8 == 0 && (tile == 0 || tile == 8) && ((uintptr_t)gu % 16) == 0 &&
+      ((uintptr_t)out % 16) == 0) {
     const int vec_blocks = (int)((total / 8 + 255) / 256);
-    swiglu_vec_kernel<<<vec_blocks, 256, 0, stream>>>((const bf16_t*)gu, ld, (bf16_t*)out, I, total);
+    swiglu_vec_kernel<<<vec_blocks, 256, 0, stream>>>((const bf16_t*)gu, ld, (bf16_t*)out, I, tile, total);
   } else if (dtype == DT_F32)
-    swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, ld, (float*)out, I, total);
+    swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, ld, (float*)out, I, tile, total);
   else if (dtype == DT_BF16)
-    swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, ld, (bf16_t*)out, I, total);
+    swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, ld, (bf16_t*)out, I, tile, total);
   else
     return ERR_BAD_ARGUMENT;
   RETURN_IF_LAUNCH_FAILED();

@@ -32,7 +32,7 @@ _SIGNATURES = {
         "mi_embed": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_int, _c_ptr],
         "mi_add_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int,
                            _c_int, _c_ptr],
-        "mi_swiglu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_ptr],
+        "mi_swiglu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
         "mi_scale_to_f32": [_c_ptr, _c_int, _c_float, _c_ptr, _c_long, _c_ptr],
     },
     "attention": {
@@ -190,13 +190,16 @@ def add_rmsnorm(h: torch.Tensor, deltas: Sequence[torch.Tensor], weight: torch.T
         "add_rmsnorm", f"(d={d})")
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, i] = SiLU(gate_up[t, i]) * gate_up[t, I + i]."""
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, tile: int = 0) -> None:
+    """out[t, i] = SiLU(g[t, i]) * u[t, i] with a row of ``gate_up`` holding [g | u] (``tile`` 0) or
+    g and u interleaved in tiles of ``tile`` columns: [g[0:tile] | u[0:tile] | g[tile:2 tile] | ...]."""
     ld = _row_major(gate_up, "gate_up")
     T, two_i = gate_up.shape
     _need(two_i % 2 == 0 and out.shape == (T, two_i // 2) and out.is_contiguous() and out.dtype == gate_up.dtype,
           "swiglu: out must be contiguous [T, I] of the input's dtype")
-    _check(_fn("common", "mi_swiglu")(_p(gate_up), _dt(gate_up), ld, _p(out), T, two_i // 2, _stream()), "swiglu")
+    _need(tile >= 0 and (tile == 0 or (two_i // 2) % tile == 0), "swiglu: the tile must divide the width")
+    _check(_fn("common", "mi_swiglu")(_p(gate_up), _dt(gate_up), ld, _p(out), T, two_i // 2, int(tile), _stream()),
+           "swiglu")
 
 
 def scale_to_f32(values: torch.Tensor, multiplier: float, out: torch.Tensor) -> None:

@@ -13,7 +13,9 @@ from .linear import Linear
 class SwiGLU(FeedForward):
     """down(SiLU(gate(x)) * up(x)); gate and up are one fused product
     (reference: src/decoder.rs:261-306).  ``gate_multiplier`` scales gate's output,
-    ``down_multiplier`` down's output; both are folded into the weights."""
+    ``down_multiplier`` down's output; both are folded into the weights.  When the width is a
+    multiple of 8 the rows of the fused matrix are stored in tiles of 8 gate rows and 8 up rows
+    (``tile``), the order the fused decode kernel wants, so that one matrix serves every path."""
     graph_safe = True
     kernel_modules = ("common", "gemm")
 
@@ -39,9 +41,15 @@ class SwiGLU(FeedForward):
                               weight_scale=scale, bias_scale=scale)
         self.down = Linear([get("down_proj.weight")], [get("down_proj.bias")], build,
                            weight_scale=spec.down_multiplier, bias_scale=spec.down_multiplier)
+        self.tile = 8 if inner % 8 == 0 else 0
+        if self.tile:
+            order = torch.arange(2 * inner).view(2, inner // 8, 8).permute(1, 0, 2).reshape(-1).to(build.device)
+            self.gate_up.weight = self.gate_up.weight[order].contiguous()
+            if self.gate_up.bias is not None:
+                self.gate_up.bias = self.gate_up.bias[order].contiguous()
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         gate_up = self.gate_up(x)
         activated = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=gate_up.dtype, device=x.device)
-        ops.swiglu(gate_up, activated)
+        ops.swiglu(gate_up, activated, self.tile)
         return self.down(activated)

@@ -63,7 +63,7 @@ class ParallelFusion:
         mixed_width = a.num_heads * a.head_dim + s.inner_size
         if a.head_dim not in (64, 128) or a.num_heads // a.num_kv_heads > 8 or s.state_size > 512:
             return None
-        if inner % 8 != 0 or hidden % 32 != 0 or mixed_width % 32 != 0 or inner % 32 != 0:
+        if block.ffn.tile != 8 or hidden % 32 != 0 or mixed_width % 32 != 0 or inner % 32 != 0:
             return None
         if not ops.fused_gemm_supported(True, 1, hidden):
             return None
@@ -103,12 +103,11 @@ class ParallelFusion:
         # the column views the mixers get must start at 16 bytes and rows must be multiples of 8 elements
         self.general = (self.in_width % 8 == 0 and self.qkv_width % 8 == 0 and q_width % 8 == 0
                         and self.mixed_width % 8 == 0)
-        # 4: gate and up rows interleaved in tiles of 8
+        # 4: gate and up rows interleaved in tiles of 8: the feed-forward part stores them so
         ffn = block.ffn
         inner = ffn.spec.intermediate_size
-        order = torch.arange(2 * inner, device=device).view(2, inner // 8, 8).permute(1, 0, 2).reshape(-1)
-        self.w_gate_up = ffn.gate_up.weight[order].contiguous()
-        self.b_gate_up = None if ffn.gate_up.bias is None else ffn.gate_up.bias[order].contiguous()
+        self.w_gate_up = ffn.gate_up.weight
+        self.b_gate_up = ffn.gate_up.bias
         self.inner = inner
         self.position = attention.position
 

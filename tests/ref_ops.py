@@ -37,9 +37,14 @@ def add_rmsnorm(h, deltas, weight, eps, out, rows=None):
         out.copy_(normed.to(out.dtype))
 
 
-def swiglu(gate_up, out):
+def swiglu(gate_up, out, tile=0):
     inner = gate_up.shape[1] // 2
-    out.copy_((F.silu(_f(gate_up[:, :inner])) * _f(gate_up[:, inner:])).to(out.dtype))
+    if tile:
+        tiles = gate_up.reshape(gate_up.shape[0], inner // tile, 2, tile)
+        gate, up = tiles[:, :, 0].reshape(-1, inner), tiles[:, :, 1].reshape(-1, inner)
+    else:
+        gate, up = gate_up[:, :inner], gate_up[:, inner:]
+    out.copy_((F.silu(_f(gate)) * _f(up)).to(out.dtype))
 
 
 def scale_to_f32(values, multiplier, out):

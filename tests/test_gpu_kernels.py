@@ -94,6 +94,15 @@ def test_swiglu_and_scale(ops, dtype):
     out = torch.empty(9, 77, dtype=dtype, device=DEV)
     ops.swiglu(gu.to(DEV), out)
     close(out, want, dtype, 4.0)
+    for width, tile in ((77, 7), (80, 8), (2048, 8)):          # gate and up interleaved in tiles
+        tiled = rand(9, 2 * width, seed=6, scale=2.0, dtype=dtype)
+        want = torch.empty(9, width, dtype=dtype)
+        ref_ops.swiglu(tiled, want, tile)
+        first = (torch.nn.functional.silu(tiled[:, :tile].float()) * tiled[:, tile:2 * tile].float()).to(dtype).float()
+        assert torch.allclose(want[:, :tile].float(), first, rtol=1e-2 if dtype == torch.bfloat16 else 1e-6, atol=1e-6)
+        out = torch.empty(9, width, dtype=dtype, device=DEV)
+        ops.swiglu(tiled.to(DEV), out, tile)
+        close(out, want, dtype, 4.0)
     logits = torch.empty(9, 154, device=DEV)
     ops.scale_to_f32(gu.to(DEV), 0.6, logits)
     close(logits, gu.float() * 0.6, torch.float32)
