@@ -25,6 +25,16 @@ SHAPE = dict(
     mamba_d_ssm=1536, mamba_d_state=128, mamba_n_groups=1, mamba_d_conv=4, mamba_chunk_size=128,
     mamba_conv_bias=True, mamba_proj_bias=False, mamba_rms_norm=False, attention_bias=False, mlp_bias=False,
     tie_word_embeddings=True)
+# further shapes of the family for measurements beside the headline one (--shape)
+SHAPES = {
+    "0.5b": SHAPE,
+    "7b": dict(SHAPE, hidden_size=3072, num_hidden_layers=44, num_attention_heads=12, num_key_value_heads=2,
+               head_dim=128, intermediate_size=12288, vocab_size=130049, mamba_n_heads=24, mamba_d_head=128,
+               mamba_d_ssm=3072, mamba_d_state=256, mamba_n_groups=1, tie_word_embeddings=False),
+    "34b": dict(SHAPE, hidden_size=5120, num_hidden_layers=72, num_attention_heads=20, num_key_value_heads=4,
+                head_dim=128, intermediate_size=21504, vocab_size=261120, mamba_n_heads=32, mamba_d_head=128,
+                mamba_d_ssm=4096, mamba_d_state=256, mamba_n_groups=2, tie_word_embeddings=False),
+}
 CONTEXT = 2048
 PREFILL_TOKENS = 2048
 
@@ -35,8 +45,10 @@ def main() -> int:
     parser.add_argument("--steps", type=int, default=64)
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
-    parser.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"],
-                        help="fewer layers than the configuration's 36 (both numbers are reported)")
+    parser.add_argument("--shape", default="0.5b", choices=sorted(SHAPES),
+                        help="layer sizes: the headline Falcon-H1-0.5B shape, or the 7B / 34B shapes")
+    parser.add_argument("--layers", type=int, default=None,
+                        help="fewer layers than the configuration has (both numbers are reported)")
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--page-tokens", type=int, default=16)
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
@@ -53,7 +65,8 @@ def main() -> int:
     from macllm_infer_amd.sampling import GREEDY, Sampler, SamplerRow
     from macllm_infer_amd.weights.random_init import random_tensors
 
-    raw = dict(SHAPE, num_hidden_layers=args.layers)
+    shape = SHAPES[args.shape]
+    raw = dict(shape, num_hidden_layers=args.layers or shape["num_hidden_layers"])
     config = FalconH1Config.from_dict(raw)
     storage = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     element = 2 if args.dtype == "bf16" else 4
@@ -148,14 +161,14 @@ def main() -> int:
         "value": round(headline["tokens_per_second"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(headline["ms"], 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
-        "config": {"model": "falcon-h1-0.5b-shaped, random weights", "layers": L,
-                   "layers_of_configuration": SHAPE["num_hidden_layers"], "hidden": d,
+        "config": {"model": f"falcon-h1-{args.shape}-shaped, random weights", "layers": L,
+                   "layers_of_configuration": shape["num_hidden_layers"], "hidden": d,
                    "heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
                    "head_dim": config.head_dim, "intermediate": config.intermediate_size,
                    "mamba_heads": config.mamba_n_heads, "mamba_head_dim": config.mamba_d_head,
                    "mamba_state": config.mamba_d_state, "mamba_groups": config.mamba_n_groups,
                    "mamba_conv": config.mamba_d_conv, "mamba_chunk": config.mamba_chunk_size, "vocab": vocab,
-                   "tied_embeddings": True, "global_batch": args.batch, "seq_len": CONTEXT,
+                   "tied_embeddings": config.tie_word_embeddings, "global_batch": args.batch, "seq_len": CONTEXT,
                    "page_tokens": args.page_tokens, "parallelism": "single GPU"},
         "prefill": {"value": round(PREFILL_TOKENS / prefill_seconds, 1), "tokens": PREFILL_TOKENS,
                     "ms": round(prefill_seconds * 1e3, 3),

@@ -65,7 +65,8 @@ class ParallelFusion:
             return None
         if block.ffn.tile != 8 or hidden % 32 != 0 or mixed_width % 32 != 0 or inner % 32 != 0:
             return None
-        if not ops.fused_gemm_supported(True, 1, hidden):
+        if not (ops.fused_gemm_supported(False, 1, hidden) and ops.fused_gemm_supported(False, 1, mixed_width)
+                and ops.fused_gemm_supported(False, 1, inner)):
             return None
         return ParallelFusion(block, attention, mamba, build)
 
@@ -110,6 +111,8 @@ class ParallelFusion:
         self.b_gate_up = ffn.gate_up.bias
         self.inner = inner
         self.position = attention.position
+        # a wide model's normed rows do not fit the norm prologue's LDS: its norms then run as kernels of their own
+        self.norm_fits = ops.fused_gemm_supported(True, 1, self.hidden)
 
     def decode_supported(self, step, cache) -> bool:
         a = self.attention.spec
@@ -149,7 +152,7 @@ class ParallelFusion:
 
         def norm_prologue(norm):
             """The input of a projection: the norm in the kernel's prologue, or its own kernel before."""
-            if M > MAX_NORM_ROWS:
+            if M > MAX_NORM_ROWS or not self.norm_fits:
                 return dict(x=norm.forward(residual)), None          # adds the pending deltas in place
             pending = residual.pending
             h_out = torch.empty_like(residual.h) if pending else None

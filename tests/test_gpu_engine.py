@@ -336,3 +336,43 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
             engine.finish(b)
     assert len(with_graphs.graphs._portion_graphs) == 1
     assert with_graphs.cache.stats() == eager.cache.stats()
+
+
+def test_a_wide_model_runs_through_the_fast_paths(tmp_path):
+    """Hidden size 2 112: the fused layer paths are built although the norm prologue does not fit;
+    prompt portions, a mixed step and graph-replayed decode steps against the plain model."""
+    from macllm_infer_amd import Engine, Lane
+    folder = tiny_configs.make_model_dir("D", tmp_path, torch.bfloat16)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=512,
+                    max_active_sequences=3)
+    fusion = engine.model.blocks[0].fusion
+    assert fusion is not None and not fusion.norm_fits and fusion.general
+    sequences = {key: tokens_for(cfg["vocab_size"], 70 + 9 * index, 900 + index) for index, key in enumerate("abc")}
+    got = {key: [] for key in sequences}
+    for key in sequences:
+        engine.add_request(key)
+
+    def step(spec):
+        lanes = [Lane(key, sequences[key][start:start + count], list(range(count))) for key, start, count in spec]
+        logits = engine.step(lanes).float().cpu()
+        row = 0
+        for key, start, count in spec:
+            got[key].append(logits[row:row + count])
+            row += count
+
+    step([("a", 0, 40), ("b", 0, 33)])
+    step([("a", 40, 1), ("b", 33, 30), ("c", 0, 70)])                  # a decoded token beside portions
+    cursor = {"a": 41, "b": 63, "c": 70}
+    while any(cursor[key] < len(sequences[key]) for key in sequences):
+        live = [key for key in sequences if cursor[key] < len(sequences[key])]
+        step([(key, cursor[key], 1) for key in live])
+        for key in live:
+            cursor[key] += 1
+    assert engine.graphs is not None and engine.graphs._graphs
+    for key, tokens in sequences.items():
+        want = plain_impl.falcon_h1_logits(cfg, tensors, tokens)
+        have = torch.cat(got[key])
+        scale = want.abs().max().item()
+        assert (have - want).abs().max().item() <= 6e-2 * scale
+        assert ((have - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()).item() <= 3e-2

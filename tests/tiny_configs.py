@@ -37,7 +37,17 @@ TINY_C = dict(
     attention_bias=False, mlp_bias=False, tie_word_embeddings=True,
     embedding_multiplier=1.2, lm_head_multiplier=0.8, key_multiplier=0.9, ssm_multipliers=[1.0, 1.2, 0.9, 1.1, 1.0])
 
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# One wide layer: the hidden size is beyond what the norm prologue of the fused decode kernels
+# holds in LDS (norms then run as kernels of their own), head_dim 128, 6 query heads on one kv head.
+TINY_D = dict(
+    architectures=["FalconH1ForCausalLM"], model_type="falcon_h1",
+    hidden_size=2112, num_hidden_layers=1, num_attention_heads=6, num_key_value_heads=1, head_dim=128,
+    intermediate_size=64, vocab_size=120, max_position_embeddings=640, rms_norm_eps=1e-5, rope_theta=1e5,
+    mamba_n_heads=8, mamba_d_head=16, mamba_d_ssm=128, mamba_d_state=64, mamba_n_groups=1, mamba_d_conv=4,
+    mamba_chunk_size=64, mamba_conv_bias=True, mamba_proj_bias=False, mamba_rms_norm=False,
+    attention_bias=False, mlp_bias=False, tie_word_embeddings=False)
+
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
 
 
 def config(name):
