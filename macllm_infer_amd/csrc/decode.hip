@@ -84,7 +84,9 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   const int per_wave = (chunks + FG_WAVES - 1) / FG_WAVES;
   const int first_chunk = wave * per_wave;
   const int iterations = max(0, min(per_wave, chunks - first_chunk));
-  constexpr int BATCH = 8;
+  // fragments of a wave in flight at once: few of them with 8 waves (long K, many workgroups a CU:
+  // the registers saved buy more waves, which hide more than deeper batches do)
+  constexpr int BATCH = FG_WAVES == 8 ? 4 : 8;
   bf16x8_t a[BATCH];
 
   // the slot of the row whose conv tail this thread will need: asked for before everything else,
