@@ -511,6 +511,8 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
   const int position = base_position + token;
   const int last_position = base_position + min(first_token + 15, lane_end - 1);
   const int first_position = base_position + first_token;
+  // every column of the wave holds a query (16 tokens, and the head sets divide the heads): the wave's bounds are known
+  const bool full_tile = first_token + 16 <= lane_end && (blockIdx.z + 1) * NSET <= G;
 
   mfma_bf16x8 q_frag[NSET][DH / 32];
   int col_pos[NSET];
@@ -553,7 +555,8 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
     wave_pages[wave][lane] = cache_pages[min(first_page + lane, max_pages - 1)];
     cache.pages = wave_pages[wave];
     cache.base_page = first_page;
-    attend_keys<DH, NSET, PREFILL_STEPS>(acc, q_frag, col_pos, window, scale, part_lo, part_hi, cache);
+    attend_keys<DH, NSET, PREFILL_STEPS>(acc, q_frag, col_pos, window, scale, part_lo, part_hi, cache,
+                                         full_tile ? first_position : -1, last_position);
     part_lo = part_hi;
   }
 

@@ -99,7 +99,10 @@ __device__ __forceinline__ void attn_load(AttnFragments<DH, STEPS>& f, int k00, 
 }
 
 // Scores, softmax step and values of the loaded steps, per set of columns.
-template <int DH, int NSET, int STEPS>
+// MASKED = false: the caller vouches that every key of the round is visible to every column
+// and lies inside the run (steps away from the diagonal, the window's edge and the run's end):
+// no masks are computed.
+template <int DH, int NSET, int STEPS, bool MASKED = true>
 __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, AttnFragments<DH, STEPS>& f,
                                              const mfma_bf16x8 (&q_frag)[NSET][DH / 32],
                                              const int (&col_pos)[NSET], int window, float scale, int k00,
@@ -114,17 +117,19 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
     if (k0 >= key_hi) break;
     // cells past the end of the run were never written: keep them out of the product (with bit
     // masks and without a branch, so that no wait for loads that are still under way is forced)
+    if (MASKED) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int valid = last_key - (k0 + 16 * t + 4 * q) + 1;            // cells of this lane's four that hold keys
-      const unsigned lo = valid >= 2 ? 0xffffffffu : (valid == 1 ? 0x0000ffffu : 0u);
-      const unsigned hi = valid >= 4 ? 0xffffffffu : (valid == 3 ? 0x0000ffffu : 0u);
+      for (int t = 0; t < 2; ++t) {
+        const int valid = last_key - (k0 + 16 * t + 4 * q) + 1;            // cells of this lane's four that hold keys
+        const unsigned lo = valid >= 2 ? 0xffffffffu : (valid == 1 ? 0x0000ffffu : 0u);
+        const unsigned hi = valid >= 4 ? 0xffffffffu : (valid == 3 ? 0x0000ffffu : 0u);
 #pragma unroll
-      for (int dt = 0; dt < DH / 16; ++dt) {
-        mfma_uintx4 bits = __builtin_bit_cast(mfma_uintx4, f.v[st][dt]);
-        bits[2 * t] &= lo;
-        bits[2 * t + 1] &= hi;
-        f.v[st][dt] = __builtin_bit_cast(mfma_bf16x8, bits);
+        for (int dt = 0; dt < DH / 16; ++dt) {
+          mfma_uintx4 bits = __builtin_bit_cast(mfma_uintx4, f.v[st][dt]);
+          bits[2 * t] &= lo;
+          bits[2 * t + 1] &= hi;
+          f.v[st][dt] = __builtin_bit_cast(mfma_bf16x8, bits);
+        }
       }
     }
 #pragma unroll
@@ -138,22 +143,24 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
           score[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[st][t][kk], q_frag[s][kk], score[t], 0, 0, 0);
       }
       // scores in units of log2: s * scale * log2(e), so that the exponentials are bare v_exp
-      // visible keys of the column: first_visible .. min(position, last_key); relative to the step
-      // they are lo .. lo + span, so one unsigned compare per score decides (an empty range gets a
-      // lo that no offset reaches)
-      const int position = col_pos[s];
-      const int first_visible = window > 0 ? max(position - window + 1, 0) : 0;
-      const int last_visible = min(position, last_key);
-      const bool any = last_visible >= first_visible;
-      const int lo = any ? first_visible - k0 : 0x40000000;
-      const unsigned span = any ? (unsigned)(last_visible - first_visible) : 0u;
+      if (MASKED) {
+        // visible keys of the column: first_visible .. min(position, last_key); relative to the step
+        // they are lo .. lo + span, so one unsigned compare per score decides (an empty range gets
+        // a lo that no offset reaches)
+        const int position = col_pos[s];
+        const int first_visible = window > 0 ? max(position - window + 1, 0) : 0;
+        const int last_visible = min(position, last_key);
+        const bool any = last_visible >= first_visible;
+        const int lo = any ? first_visible - k0 : 0x40000000;
+        const unsigned span = any ? (unsigned)(last_visible - first_visible) : 0u;
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const bool visible = (unsigned)(16 * t + 4 * q + i - lo) <= span;
-          score[t][i] = visible ? score[t][i] : -INFINITY;
-        }
+          for (int i = 0; i < 4; ++i) {
+            const bool visible = (unsigned)(16 * t + 4 * q + i - lo) <= span;
+            score[t][i] = visible ? score[t][i] : -INFINITY;
+          }
+      }
       float step_max = fmaxf(fmaxf(fmaxf(score[0][0], score[0][1]), fmaxf(score[0][2], score[0][3])),
                              fmaxf(fmaxf(score[1][0], score[1][1]), fmaxf(score[1][2], score[1][3])));
       step_max = fmaxf(step_max, __shfl_xor(step_max, 16, WAVE));
@@ -191,11 +198,13 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
 // requested before the first is used.  PIPELINED: the loads of the next STEPS steps are
 // requested before the current ones are worked on (twice the fragment registers), for callers
 // with long runs; a caller whose run is one round of STEPS steps gains nothing from it.
+// min_pos / max_pos: the smallest and largest position among the columns of the wave, when all
+// of them hold queries and the caller knows (the same value in every lane), else -1.
 template <int DH, int NSET, int STEPS, bool PIPELINED = false>
 __device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET>& acc,
                                             const mfma_bf16x8 (&q_frag)[NSET][DH / 32],
                                             const int (&col_pos)[NSET], int window, float scale, int key_lo,
-                                            int key_hi, const AttnCache& cache) {
+                                            int key_hi, const AttnCache& cache, int min_pos = -1, int max_pos = -1) {
   const int last_key = key_hi - 1;
   constexpr int ROUND = 32 * STEPS;
   if (PIPELINED) {
@@ -210,10 +219,20 @@ __device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET>& acc,
       if (k00 + ROUND < key_hi) attn_compute<DH, NSET, STEPS>(acc, odd, q_frag, col_pos, window, scale, k00 + ROUND, key_hi);
     }
   } else {
-    for (int k00 = key_lo; k00 < key_hi; k00 += ROUND) {
+    // rounds all of whose keys every column of the wave sees run without masks, in a loop of
+    // their own; the rest (the diagonal, a window's edge, the end of the run) with them
+    int open_hi = key_lo;
+    if (min_pos >= 0 && (window <= 0 || key_lo >= max_pos - window + 1))
+      open_hi = key_lo + max(0, (min(min_pos + 1, key_hi) - key_lo) / ROUND) * ROUND;
+    for (int k00 = key_lo; k00 < open_hi; k00 += ROUND) {
       AttnFragments<DH, STEPS> f;
       attn_load<DH, STEPS>(f, k00, last_key, cache);
-      attn_compute<DH, NSET, STEPS>(acc, f, q_frag, col_pos, window, scale, k00, key_hi);
+      attn_compute<DH, NSET, STEPS, false>(acc, f, q_frag, col_pos, window, scale, k00, key_hi);
+    }
+    for (int k00 = open_hi; k00 < key_hi; k00 += ROUND) {
+      AttnFragments<DH, STEPS> f;
+      attn_load<DH, STEPS>(f, k00, last_key, cache);
+      attn_compute<DH, NSET, STEPS, true>(acc, f, q_frag, col_pos, window, scale, k00, key_hi);
     }
   }
 }
