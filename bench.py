@@ -70,7 +70,8 @@ def main() -> int:
     config = FalconH1Config.from_dict(raw)
     storage = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     element = 2 if args.dtype == "bf16" else 4
-    tensors = random_tensors(config, 0, storage, "baseline")
+    # the 0.5B shape is drawn on the CPU like every test model; the large shapes on the GPU (minutes otherwise)
+    tensors = random_tensors(config, 0, storage, "baseline", device="cpu" if args.shape == "0.5b" else "cuda:0")
     batches = [args.batch] if args.skip_points else sorted({1, args.batch, 64})
     if args.prefill_only:
         batches = []

@@ -36,16 +36,16 @@ class Linear:
         rows = weight.shape[0]
         scale = _as_rows(weight_scale, rows)
         if scale is not None:
-            weight = weight * scale
+            weight = weight * scale.to(weight.device)
         self.weight = weight.to(keep).contiguous().to(build.device)
         self.bias = None
         if any(b is not None for b in biases):
-            parts = [torch.zeros(w.shape[0]) if b is None else b.to(torch.float32).reshape(-1)
+            parts = [torch.zeros(w.shape[0], device=w.device) if b is None else b.to(torch.float32).reshape(-1)
                      for w, b in zip(weights, biases)]
             bias = torch.cat(parts)
             scale = _as_rows(bias_scale, rows)
             if scale is not None:
-                bias = bias * scale.reshape(-1)
+                bias = bias * scale.reshape(-1).to(bias.device)
             self.bias = bias.contiguous().to(build.device)
         self.out_features, self.in_features = self.weight.shape
 

@@ -10,6 +10,8 @@ N(0, 1/sqrt(fan_in)), embeddings N(0, 1/sqrt(width)), conv taps N(0, 1/sqrt(K)),
 so that a fault in any part shows in the logits of a tiny model.
 Values are drawn in float32 on the CPU in declaration order, then rounded to the
 storage dtype; vectors of the state-space recurrence (A_log, D, dt_bias) stay float32.
+With ``device`` they are drawn on that device instead (another stream of numbers for the
+same seed): the way to get the billions of weights of a large shape in seconds.
 """
 from __future__ import annotations
 
@@ -27,17 +29,18 @@ _KEEP_F32 = ("A_log", "D", "dt_bias")
 
 
 def random_tensors(config, seed: int, storage_dtype: torch.dtype = torch.bfloat16,
-                   preset: str = "baseline") -> Dict[str, torch.Tensor]:
+                   preset: str = "baseline", device="cpu") -> Dict[str, torch.Tensor]:
     if preset not in ("baseline", "unit"):
         raise ValueError(f"unknown init preset {preset!r}")
-    generator = torch.Generator(device="cpu").manual_seed(int(seed))
+    device = torch.device(device)
+    generator = torch.Generator(device=device).manual_seed(int(seed))
     unit = preset == "unit"
 
     def normal(shape, std, mean=0.0):
-        return torch.randn(shape, generator=generator, dtype=torch.float32) * std + mean
+        return torch.randn(shape, generator=generator, dtype=torch.float32, device=device) * std + mean
 
     def uniform(shape, low, high):
-        return torch.rand(shape, generator=generator, dtype=torch.float32) * (high - low) + low
+        return torch.rand(shape, generator=generator, dtype=torch.float32, device=device) * (high - low) + low
 
     out: Dict[str, torch.Tensor] = {}
     for expect in DecoderModel.expected_tensors(config.to_model_spec()):
