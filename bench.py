@@ -92,7 +92,7 @@ def main() -> int:
 
     # ---------------------------------------------------------------- prefill: one 2,048-token prompt
     prefill_times = []
-    for repeat in range(3):
+    for repeat in range(6):
         prompt = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=generator).tolist()
         engine.add_request("prefill")
         synchronize()
@@ -101,7 +101,7 @@ def main() -> int:
         synchronize()
         prefill_times.append(time.perf_counter() - started)
         engine.finish("prefill")
-    prefill_seconds = min(prefill_times[1:])
+    prefill_seconds = min(prefill_times[3:])            # the step's graph is captured at its third sighting
 
     d, L = config.hidden_size, config.num_hidden_layers
     E = config.mamba_d_ssm

@@ -305,14 +305,14 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, requests):
 @pytest.mark.parametrize("name, dtype", [("B", "float32"), ("C", "bfloat16")])
 def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
     """Steps of one shape (two prompt portions of 70 and 40 tokens, some places wanted) come back:
-    from the second time on they are replayed from a captured graph.  Every step, through pages
+    from the third time on they are replayed from a captured graph.  Every step, through pages
     that are given back and used again and with a decode replay between, is compared with an
     engine without graphs."""
     from macllm_infer_amd import Engine, Lane
     folder = tiny_configs.make_model_dir(name, tmp_path, torch.float32 if dtype == "float32" else torch.bfloat16)
     cfg, _ = plain_impl.load_model_dir(folder)
     make = lambda graphs: Engine(folder, dtype=dtype, kv_cache_block_tokens=16, kv_cache_capacity_tokens=640,
-                                 max_active_sequences=4, decode_graphs=graphs)
+                                 max_active_sequences=5, decode_graphs=graphs)
     with_graphs, eager = make(True), make(False)
 
     def both(lanes):
@@ -328,7 +328,8 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
         for engine in (with_graphs, eager):
             engine.add_request(a)
             engine.add_request(b)
-        both([Lane(a, tokens_a[:70], [3, 69]), Lane(b, tokens_b[:40], [39])])
+        first = [Lane(a, tokens_a[:70], [3, 69]), Lane(b, tokens_b[:40], [39])]
+        both(first if round_index % 2 == 0 else first[::-1])      # the order of the lanes does not make another shape
         both([Lane(a, tokens_a[70:140], [3, 69]), Lane(b, tokens_b[40:80], [39])])      # same shape, later positions
         both([Lane(a, tokens_a[140:], [0]), Lane(b, tokens_b[80:], [0])])                 # a decode replay between
         for engine in (with_graphs, eager):
@@ -336,6 +337,26 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
             engine.finish(b)
     assert len(with_graphs.graphs._portion_graphs) == 1
     assert with_graphs.cache.stats() == eager.cache.stats()
+    # decoded tokens beside a portion: three, then four single-token lanes share one graph (padded to four)
+    for engine in (with_graphs, eager):
+        for key in "pqrst":
+            engine.add_request(key)
+    streams = {key: tokens_for(cfg["vocab_size"], 400, 950 + index) for index, key in enumerate("pqrst")}
+    cursor = {key: 0 for key in streams}
+
+    def lane(key, count, want):
+        tokens = streams[key][cursor[key]:cursor[key] + count]
+        cursor[key] += count
+        return Lane(key, tokens, want)
+
+    both([lane(key, 5, [4]) for key in "pqrs"])
+    replays = with_graphs.graphs.counts["portion_replays"]
+    for turn in range(6):
+        singles = "pqr" if turn < 3 else "pqrs"
+        lanes = [lane(key, 1, [0]) for key in singles] + [lane("t", 64, [63] if turn == 5 else [])]
+        both(lanes if turn % 2 == 0 else lanes[::-1])
+    assert len(with_graphs.graphs._portion_graphs) == 2
+    assert with_graphs.graphs.counts["portion_replays"] == replays + 3      # turns 2, 3 and 4
 
 
 def test_a_wide_model_runs_through_the_fast_paths(tmp_path):
