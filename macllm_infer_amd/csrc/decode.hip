@@ -266,17 +266,19 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
         }
       }
     }
+    // no branch around a product: under a condition the compiler moves the fragment's load into the
+    // branch and waits for it there, one at a time; a fragment past the end is read again (clamped
+    // above) and multiplied as zeros
 #pragma unroll
     for (int j = 0; j < BATCH; ++j) {
-      if (first + j < iterations) {
-        const int c = first_chunk + first + j;
+      const int c = first_chunk + min(first + j, iterations - 1);
+      const floatx4 weights = first + j < iterations ? *reinterpret_cast<const floatx4*>(&a[j]) : floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          bf16x8_t operand;
-          if (PRO == PRO_NORM) operand = *reinterpret_cast<const bf16x8_t*>(xs + (long)(mt * 16 + r) * ldx + c * 32 + 8 * q);
-          else operand = b[j][mt];
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], operand, acc[mt], 0, 0, 0);
-        }
+      for (int mt = 0; mt < MT; ++mt) {
+        bf16x8_t operand;
+        if (PRO == PRO_NORM) operand = *reinterpret_cast<const bf16x8_t*>(xs + (long)(mt * 16 + r) * ldx + c * 32 + 8 * q);
+        else operand = b[j][mt];
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8_t*>(&weights), operand, acc[mt], 0, 0, 0);
       }
     }
   }

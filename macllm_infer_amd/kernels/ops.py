@@ -51,6 +51,7 @@ _SIGNATURES = {
                            _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
         "mi_conv_state_update": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
                                  _c_ptr],
+        "mi_conv_step": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
         "mi_ssm_scan": [_c_ptr, _c_int, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_ptr],
         "mi_gate_norm": [_c_ptr, _c_long, _c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_float, _c_ptr, _c_long,
@@ -418,6 +419,26 @@ def conv_state_update(u: torch.Tensor, col_offset: int, width: int, kernel: int,
     _check(_fn("mamba2", "mi_conv_state_update")(
         _p(u), _dt(u), ld, col_offset, width, kernel, _p(conv_state), _p(cu_seqlens), _p(slot_ids), num_lanes,
         _stream()), "conv_state_update", f"(K={kernel})")
+
+
+def conv_step(u: torch.Tensor, col_offset: int, width: int, weight: torch.Tensor, bias: Optional[torch.Tensor],
+              conv_state: torch.Tensor, slot_ids: torch.Tensor) -> None:
+    """One conv step of single-token lanes, in place: row m of ``u`` is the new token of the request in
+    ``slot_ids[m]``; columns [col_offset, col_offset + width) become SiLU(conv over [tail ; sample]) and the
+    tail ``conv_state[slot]`` [K-1, width] is rolled by one and takes the sample."""
+    ld = _row_major(u, "u")
+    M = u.shape[0]
+    K = weight.shape[1]
+    _need(weight.shape == (width, K) and weight.dtype == torch.float32 and weight.is_contiguous(),
+          "conv_step: weight must be float32 [C, K]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == width), "conv_step: bad bias")
+    _need(conv_state.dim() == 3 and conv_state.shape[1:] == (max(K - 1, 0), width)
+          and conv_state.dtype == u.dtype and conv_state.is_contiguous(), "conv_step: bad conv_state")
+    _need(u.shape[1] >= col_offset + width, "conv_step: u is too narrow")
+    _i32(slot_ids, "slot_ids")
+    _need(slot_ids.numel() >= M, "conv_step: one slot per row")
+    _check(_fn("mamba2", "mi_conv_step")(_p(u), _dt(u), ld, col_offset, M, width, K, _p(weight), _p(bias),
+                                         _p(conv_state), _p(slot_ids), _stream()), "conv_step", f"(K={K})")
 
 
 def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, D: torch.Tensor,

@@ -16,13 +16,16 @@ Decode steps (every lane holds one token, at most 64 rows): five launches instea
     4. residual add + norm + gate/up projection + SiLU(g)*u                     (fused_gemm)
     5. down projection                                                          (fused_gemm)
 
+A large weight goes through the BLAS library instead where that is faster (``LIBRARY_MIN_WEIGHT``); the
+conv step and SiLU(g)*u then run as kernels of their own.
+
 The fusion belongs to the arrangement, which knows its parts; the parts stay as they are.  It
 is built only for bfloat16 weights and sizes the kernels cover; otherwise the block runs part
 by part.
 """
 from __future__ import annotations
 
-from typing import Optional
+from typing import Dict, Optional
 
 import torch
 
@@ -36,6 +39,74 @@ from .position import NoPosition, Rope
 
 MAX_ROWS = 64          # rows of a step the skinny kernels take
 MAX_NORM_ROWS = 16     # the norm prologue recomputes the normed rows in every workgroup: small batches only
+# A weight of this many elements or more is measured once, when the first layer of its shape is built, on
+# both ways: the skinny kernel, and the BLAS library with the conv step or SiLU(g)*u as a kernel of its own.
+# The skinny kernel reads the step's rows once per 16 weight rows and keeps all of K in one workgroup; the
+# library tiles the rows and splits a long K, but its choice of tile swings from shape to shape (a 5120 x
+# 21504 weight at 8 rows: 115 us against 69; a 3072 x 12288 one: 20 against 25), so the clock decides, per
+# shape and per step size (up to 16, 32, 64 rows).  Below the limit the skinny kernel wins everywhere.
+LIBRARY_MIN_WEIGHT = 8 << 20
+LIBRARY_MARGIN = 0.92          # the library has to be this much faster to be taken
+FORCE_LIBRARY: Optional[bool] = None      # tests: True or False instead of the clock
+TUNE_ROWS = (8, 32, 64)
+_library_wins: Dict[tuple, bool] = {}
+
+
+def _bucket(rows: int) -> int:
+    return 0 if rows <= MAX_NORM_ROWS else 1 if rows <= 32 else 2
+
+
+def _graph_microseconds(run) -> float:
+    """Time of one call of ``run`` on the GPU, replayed from a graph (no launch gaps)."""
+    device = torch.cuda.current_device()
+    side = torch.cuda.Stream(device=device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream(device).wait_stream(side)
+    torch.cuda.synchronize(device)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    graph.replay()
+    torch.cuda.synchronize(device)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(3):
+        graph.replay()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) * 1e3 / 3
+
+
+def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile: int, conv: Optional[dict]) -> bool:
+    """Whether the library way is faster for this weight at this many rows.  Copies of the weight are
+    cycled through so that the caches do not hold it, as in a model of many layers."""
+    N, K = weight.shape
+    device = weight.device
+    copies = max(2, min(8, (512 << 20) // (weight.numel() * 2)))
+    weights = [weight] + [weight.clone() for _ in range(copies - 1)]
+    x = torch.randn((rows, K), dtype=torch.bfloat16, device=device)
+    out = torch.empty((rows, N // 2 if epilogue == ops.EPI_SWIGLU else N), dtype=torch.bfloat16, device=device)
+    if conv is not None:
+        channels = conv["hi"] - conv["lo"]
+        conv = dict(conv, state=torch.zeros((rows, max(conv["taps"] - 1, 0), channels), dtype=torch.bfloat16, device=device),
+                    slot_ids=torch.arange(rows, dtype=torch.int32, device=device))
+
+    def skinny():
+        for w in weights:
+            ops.fused_gemm(w, bias, out, x=x, epilogue=epilogue, conv=conv)
+
+    def library():
+        for w in weights:
+            product = ops.linear(x, w, bias)
+            if epilogue == ops.EPI_SWIGLU:
+                ops.swiglu(product, out, tile)
+            elif epilogue == ops.EPI_CONV:
+                ops.conv_step(product, conv["lo"], conv["hi"] - conv["lo"], conv["weight"], conv["bias"], conv["state"],
+                              conv["slot_ids"])
+
+    return _graph_microseconds(library) < LIBRARY_MARGIN * _graph_microseconds(skinny)
 
 
 class ParallelFusion:
@@ -113,6 +184,12 @@ class ParallelFusion:
         self.position = attention.position
         # a wide model's normed rows do not fit the norm prologue's LDS: its norms then run as kernels of their own
         self.norm_fits = ops.fused_gemm_supported(True, 1, self.hidden)
+        # which projections go through the library, by step size
+        conv = dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=mamba.conv_weight, bias=mamba.conv_bias)
+        self.library_in = self._tune(self.w_in, self.b_in, ops.EPI_CONV, conv)
+        self.library_out = self._tune(self.w_out, self.b_out, ops.EPI_PLAIN)
+        self.library_gate_up = self._tune(self.w_gate_up, self.b_gate_up, ops.EPI_SWIGLU)
+        self.library_down = self._tune(ffn.down.weight, ffn.down.bias, ops.EPI_PLAIN)
 
     def decode_supported(self, step, cache) -> bool:
         a = self.attention.spec
@@ -143,10 +220,32 @@ class ParallelFusion:
         normed = block.ffn_norm.forward(residual)
         residual.pending = [block.ffn.forward(normed)]
 
+    def _tune(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict] = None) -> tuple:
+        """For step sizes of up to 16, 32 and 64 rows: whether this projection goes through the library.
+        (Where the norm runs in the skinny kernel's prologue, small steps stay with it.)"""
+        choices = self._tune_all(weight, bias, epilogue, conv)
+        if epilogue != ops.EPI_PLAIN and self.norm_fits:
+            choices = (False,) + choices[1:]
+        return choices
+
+    def _tune_all(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict]) -> tuple:
+        if not self.general or FORCE_LIBRARY is False or (FORCE_LIBRARY is None and weight.numel() < LIBRARY_MIN_WEIGHT):
+            return (False, False, False)
+        if FORCE_LIBRARY:
+            return (True, True, True)
+        choices = []
+        for bucket, rows in enumerate(TUNE_ROWS):
+            key = (tuple(weight.shape), epilogue, bias is None, bucket)
+            if key not in _library_wins:
+                _library_wins[key] = _measure_library(weight, bias, rows, epilogue, self.block.ffn.tile, conv)
+            choices.append(_library_wins[key])
+        return tuple(choices)
+
     def forward_decode(self, residual: Residual, step, caches) -> None:
         block, a, s = self.block, self.attention.spec, self.mamba.spec
         kv, state = caches[self.attention_name], caches[self.mamba_name]
         M = step.num_tokens
+        bucket = _bucket(M)
         device = residual.h.device
         bf16 = torch.bfloat16
 
@@ -160,14 +259,19 @@ class ParallelFusion:
             return arguments, h_out
 
         # 1
-        u = torch.empty((M, self.in_ld), dtype=bf16, device=device)
-        arguments, h_out = norm_prologue(block.mixer_norm)
-        ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=ops.EPI_CONV,
-                       conv=dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=self.mamba.conv_weight,
-                                 bias=self.mamba.conv_bias, state=state.states["conv"], slot_ids=step.slot_ids),
-                       **arguments)
-        if h_out is not None:
-            residual.h, residual.pending = h_out, []
+        if self.library_in[bucket]:
+            u = ops.linear(block.mixer_norm.forward(residual), self.w_in, self.b_in)
+            ops.conv_step(u, self.x_col, self.dt_col - self.x_col, self.mamba.conv_weight, self.mamba.conv_bias,
+                          state.states["conv"], step.slot_ids)
+        else:
+            u = torch.empty((M, self.in_ld), dtype=bf16, device=device)
+            arguments, h_out = norm_prologue(block.mixer_norm)
+            ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=ops.EPI_CONV,
+                           conv=dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=self.mamba.conv_weight,
+                                     bias=self.mamba.conv_bias, state=state.states["conv"], slot_ids=step.slot_ids),
+                           **arguments)
+            if h_out is not None:
+                residual.h, residual.pending = h_out, []
         # 2
         mixed = torch.empty((M, self.mixed_width), dtype=bf16, device=device)
         gated_norm = self.mamba.norm_weight is not None
@@ -187,19 +291,29 @@ class ParallelFusion:
             ops.gate_norm(y, u[:, self.z_col:self.z_col + s.inner_size], self.mamba.norm_weight, s.num_groups,
                           s.norm_eps, mixed[:, a.num_heads * a.head_dim:])
         # 3
-        delta = torch.empty((M, self.hidden), dtype=bf16, device=device)
-        ops.fused_gemm(self.w_out, self.b_out, delta, x=mixed)
+        if self.library_out[bucket]:
+            delta = ops.linear(mixed, self.w_out, self.b_out)
+        else:
+            delta = torch.empty((M, self.hidden), dtype=bf16, device=device)
+            ops.fused_gemm(self.w_out, self.b_out, delta, x=mixed)
         residual.pending = [delta]
         # 4
         activated = torch.empty((M, self.inner), dtype=bf16, device=device)
-        arguments, h_out = norm_prologue(block.ffn_norm)
-        ops.fused_gemm(self.w_gate_up, self.b_gate_up, activated, epilogue=ops.EPI_SWIGLU, **arguments)
-        if h_out is not None:
-            residual.h, residual.pending = h_out, []
+        if self.library_gate_up[bucket]:
+            ops.swiglu(ops.linear(block.ffn_norm.forward(residual), self.w_gate_up, self.b_gate_up), activated,
+                       block.ffn.tile)
+        else:
+            arguments, h_out = norm_prologue(block.ffn_norm)
+            ops.fused_gemm(self.w_gate_up, self.b_gate_up, activated, epilogue=ops.EPI_SWIGLU, **arguments)
+            if h_out is not None:
+                residual.h, residual.pending = h_out, []
         # 5
         down = block.ffn.down
-        delta = torch.empty((M, self.hidden), dtype=bf16, device=device)
-        ops.fused_gemm(down.weight, down.bias, delta, x=activated)
+        if self.library_down[bucket]:
+            delta = ops.linear(activated, down.weight, down.bias)
+        else:
+            delta = torch.empty((M, self.hidden), dtype=bf16, device=device)
+            ops.fused_gemm(down.weight, down.bias, delta, x=activated)
         residual.pending = [delta]
 
 

@@ -143,6 +143,15 @@ def conv_state_update(u, col_offset, width, kernel, conv_state, cu_seqlens, slot
         conv_state[slot] = window[-(kernel - 1):]
 
 
+def conv_step(u, col_offset, width, weight, bias, conv_state, slot_ids):
+    M = u.shape[0]
+    lanes = torch.arange(M + 1, dtype=torch.int32)
+    out = torch.empty((M, width), dtype=u.dtype)
+    conv1d_silu(u, col_offset, width, weight, bias, conv_state, lanes[:M], lanes, slot_ids[:M], out)
+    conv_state_update(u, col_offset, width, weight.shape[1], conv_state, lanes, slot_ids[:M])
+    u[:, col_offset:col_offset + width] = out
+
+
 def ssm_scan(xbc, dt, dt_bias, A, D, ssm_state, cu_seqlens, slot_ids, num_groups, y):
     _, H, P, N = ssm_state.shape
     E = H * P

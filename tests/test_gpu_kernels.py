@@ -318,6 +318,29 @@ def test_mamba2_kernels_over_ragged_lanes(ops, dtype, H, P, N, G, K):
         assert torch.equal(got[2][untouched].cpu(), ssm_state[untouched])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M, C, K, col_offset, ld", [(1, 40, 4, 0, 40), (7, 100, 3, 13, 131), (64, 1792, 4, 1536, 4120),
+                                                     (5, 33, 1, 2, 40), (9, 24, 9, 8, 32)])
+def test_conv_step_of_single_token_lanes(ops, dtype, M, C, K, col_offset, ld):
+    """The in-place conv step against conv1d_silu + conv_state_update of one-token lanes; the slots are a
+    permutation with unused ones between, whose tails must stay as they were; so must the other columns."""
+    u = rand(M, ld, seed=1, dtype=dtype)
+    weight, bias = rand(C, K, seed=2, scale=0.5), rand(C, seed=3)
+    slots = 2 * M + 1
+    state = rand(slots, max(K - 1, 0), C, seed=4, dtype=dtype)
+    slot_ids = i32(torch.randperm(slots, generator=torch.Generator().manual_seed(5))[:M].tolist())
+    for with_bias in (True, False):
+        want_u, want_state = u.clone(), state.clone()
+        ref_ops.conv_step(want_u, col_offset, C, weight, bias if with_bias else None, want_state, slot_ids)
+        got_u, got_state, w, b, ids = gpu(u.clone(), state.clone(), weight, bias if with_bias else None, slot_ids)
+        ops.conv_step(got_u, col_offset, C, w, b, got_state, ids)
+        close(got_u, want_u, dtype, 4.0)
+        assert torch.equal(got_state.cpu(), want_state)
+        untouched = torch.ones(ld, dtype=torch.bool)
+        untouched[col_offset:col_offset + C] = False
+        assert torch.equal(got_u.cpu()[:, untouched], u[:, untouched])
+
+
 @pytest.mark.parametrize("Q", [32, 64, 128, 256])
 @pytest.mark.parametrize("H, P, N, G", [(4, 16, 32, 1), (6, 32, 64, 2), (5, 64, 128, 1), (9, 16, 96, 3), (2, 48, 256, 2)])
 def test_chunked_scan_matches_the_token_by_token_scan(ops, Q, H, P, N, G):
