@@ -45,7 +45,7 @@ MAX_NORM_ROWS = 16     # the norm prologue recomputes the normed rows in every w
 # library tiles the rows and splits a long K, but its choice of tile swings from shape to shape (a 5120 x
 # 21504 weight at 8 rows: 115 us against 69; a 3072 x 12288 one: 20 against 25), so the clock decides, per
 # shape and per step size (up to 16, 32, 64 rows).  Below the limit the skinny kernel wins everywhere.
-LIBRARY_MIN_WEIGHT = 8 << 20
+LIBRARY_MIN_WEIGHT = 2 << 20
 LIBRARY_MARGIN = 0.92          # the library has to be this much faster to be taken
 FORCE_LIBRARY: Optional[bool] = None      # tests: True or False instead of the clock
 TUNE_ROWS = (8, 32, 64)
