@@ -450,6 +450,7 @@ extern "C" int mi_fused_gemm_supported(int pro, int M, int K) {
 #define MX_MAX_PAGES 80        // page ids of one run of keys (at most MX_SPLIT_KEYS / 8 + 2)
 #define MX_SPLIT_KEYS 512
 #define MX_SCAN_PER_THREAD 8
+#define MX_FEW_BLOCKS 512       // state-space workgroups of a step up to which each takes one row per thread group
 
 struct MixerParams {
   // the layer's projected row per token: [q | k | v | z | x B C (after conv) | dt], bfloat16
@@ -471,7 +472,7 @@ struct MixerParams {
   float scale;
   int window;
   // state space
-  int H, P, N, G, R, p_tiles, vector_scan, z_col, x_col, dt_col;
+  int H, P, N, G, R, p_tiles, vector_scan, rows_per_thread, z_col, x_col, dt_col;
   const float* dt_bias;
   const float* A;
   const float* D;
@@ -712,71 +713,92 @@ __global__ void mixer_merge_kernel(MixerParams p, int dh) {
 // One step of the selective scan for (token, head, tile of state rows); see ssm_scan_kernel.
 // A state row of N floats is shared by R lanes.  When N is 8*R (VECTOR) each lane owns 8
 // consecutive elements: two 16-byte state loads and one 16-byte load each of B and C.
-template <bool VECTOR>
+template <bool VECTOR, int RPT>
 __device__ void mixer_ssm_block(const MixerParams& p, int block) {
   const int tile = block % p.p_tiles;
   const int head = (block / p.p_tiles) % p.H;
   const long token = block / (p.p_tiles * p.H);
   const int R = p.R;
-  const int rows_per_block = MX_THREADS / R;
-  const int row_in_block = threadIdx.x / R;
-  const int r = threadIdx.x - row_in_block * R;
-  const int pi = tile * rows_per_block + row_in_block;
-  const bool active = pi < p.P;
+  const int rows_per_round = MX_THREADS / R;
+  const int row_in_round = threadIdx.x / R;
+  const int r = threadIdx.x - row_in_round * R;
   const int group = head / (p.H / p.G);
   const int N = p.N;
   const bf16_t* row = p.u + token * p.u_ld;
-  float* s_row = p.ssm_state + (((long)p.slot_ids[token] * p.H + head) * p.P + (active ? pi : 0)) * N;
   const bf16_t* b_row = row + p.x_col + p.H * p.P + group * N;
   const bf16_t* c_row = b_row + p.G * N;
-  const long column = (long)head * p.P + (active ? pi : 0);
-  // every load of the step is asked for before the first is used (the state first: it comes from
-  // furthest away), with no branch between them
-  floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+  // a thread owns 8 state elements of RPT rows (large batches: more bytes in flight per thread and
+  // fewer workgroups, each of which first waits for its slot id).  Every load of the step is asked for
+  // before the first is used (the state first: it comes from furthest away), with no branch between
+  // them; a row past P reads row 0 and is dropped
+  int pi[RPT];
+  bool active[RPT];
+  float* s_row[RPT];
+  const long slot_base = ((long)p.slot_ids[token] * p.H + head) * p.P;
+#pragma unroll
+  for (int j = 0; j < RPT; ++j) {
+    pi[j] = (tile * RPT + j) * rows_per_round + row_in_round;
+    active[j] = pi[j] < p.P;
+    s_row[j] = p.ssm_state + (slot_base + (active[j] ? pi[j] : 0)) * N;
+  }
+  floatx4 s0[RPT], s1[RPT];
   bf16x8_t b, c;
   if (VECTOR) {
-    s0 = *reinterpret_cast<const floatx4*>(s_row + r * 8);
-    s1 = *reinterpret_cast<const floatx4*>(s_row + r * 8 + 4);
+#pragma unroll
+    for (int j = 0; j < RPT; ++j) {
+      s0[j] = *reinterpret_cast<const floatx4*>(s_row[j] + r * 8);
+      s1[j] = *reinterpret_cast<const floatx4*>(s_row[j] + r * 8 + 4);
+    }
     b = *reinterpret_cast<const bf16x8_t*>(b_row + r * 8);
     c = *reinterpret_cast<const bf16x8_t*>(c_row + r * 8);
   }
   const bf16_t dt_bits = row[p.dt_col + head];
-  const bf16_t x_bits = row[p.x_col + column];
-  const bf16_t z_bits = row[p.z_col + column];
+  bf16_t x_bits[RPT], z_bits[RPT];
+#pragma unroll
+  for (int j = 0; j < RPT; ++j) {
+    const long column = (long)head * p.P + (active[j] ? pi[j] : 0);
+    x_bits[j] = row[p.x_col + column];
+    z_bits[j] = row[p.z_col + column];
+  }
   const float delta = softplus_f((float)dt_bits + p.dt_bias[head]);
   const float decay = expf(delta * p.A[head]);
-  const float x = active ? (float)x_bits : 0.f;
-  const float dx = delta * x;
-  float partial = 0.f;
-  if (VECTOR) {
-    if (active) {
+  const float skip = p.D[head];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        s0[i] = decay * s0[i] + dx * (float)b[i];
-        s1[i] = decay * s1[i] + dx * (float)b[4 + i];
-        partial += s0[i] * (float)c[i];
+  for (int j = 0; j < RPT; ++j) {
+    const long column = (long)head * p.P + (active[j] ? pi[j] : 0);
+    const float x = active[j] ? (float)x_bits[j] : 0.f;
+    const float dx = delta * x;
+    float partial = 0.f;
+    if (VECTOR) {
+      if (active[j]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          s0[j][i] = decay * s0[j][i] + dx * (float)b[i];
+          s1[j][i] = decay * s1[j][i] + dx * (float)b[4 + i];
+          partial += s0[j][i] * (float)c[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) partial += s1[j][i] * (float)c[4 + i];
+        *reinterpret_cast<floatx4*>(s_row[j] + r * 8) = s0[j];
+        *reinterpret_cast<floatx4*>(s_row[j] + r * 8 + 4) = s1[j];
       }
+    } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) partial += s1[i] * (float)c[4 + i];
-      *reinterpret_cast<floatx4*>(s_row + r * 8) = s0;
-      *reinterpret_cast<floatx4*>(s_row + r * 8 + 4) = s1;
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < MX_SCAN_PER_THREAD; ++i) {
-      const int n = r + i * R;
-      if (active && n < N) {
-        const float next = decay * s_row[n] + dx * (float)b_row[n];
-        s_row[n] = next;
-        partial += next * (float)c_row[n];
+      for (int i = 0; i < MX_SCAN_PER_THREAD; ++i) {
+        const int n = r + i * R;
+        if (active[j] && n < N) {
+          const float next = decay * s_row[j][n] + dx * (float)b_row[n];
+          s_row[j][n] = next;
+          partial += next * (float)c_row[n];
+        }
       }
     }
-  }
-  for (int offset = R / 2; offset > 0; offset >>= 1) partial += __shfl_xor(partial, offset, WAVE);
-  if (active && r == 0) {
-    const float y = partial + p.D[head] * x;
-    if (p.ssm_y) p.ssm_y[token * (long)(p.H * p.P) + column] = y;
-    else p.ssm_out[token * p.out_ld + column] = (bf16_t)(y * silu_f((float)z_bits));
+    for (int offset = R / 2; offset > 0; offset >>= 1) partial += __shfl_xor(partial, offset, WAVE);
+    if (active[j] && r == 0) {
+      const float y = partial + skip * x;
+      if (p.ssm_y) p.ssm_y[token * (long)(p.H * p.P) + column] = y;
+      else p.ssm_out[token * p.out_ld + column] = (bf16_t)(y * silu_f((float)z_bits[j]));
+    }
   }
 }
 
@@ -787,10 +809,16 @@ __global__ void __launch_bounds__(MX_THREADS) mixer_decode_kernel(MixerParams p)
   __shared__ float merge_lds[MX_WAVES * 8 * (DH + 2)];
   if ((int)blockIdx.x < p.attention_blocks)
     mixer_attention_block<DH>(p, blockIdx.x, pages_lds, cs, merge_lds);
-  else if (p.vector_scan)
-    mixer_ssm_block<true>(p, blockIdx.x - p.attention_blocks);
+  else if (!p.vector_scan)
+    mixer_ssm_block<false, 1>(p, blockIdx.x - p.attention_blocks);
+  else if (p.rows_per_thread == 1)
+    mixer_ssm_block<true, 1>(p, blockIdx.x - p.attention_blocks);
+  else if (p.rows_per_thread == 2)
+    mixer_ssm_block<true, 2>(p, blockIdx.x - p.attention_blocks);
+  else if (DH == 64 || p.rows_per_thread == 4)         // eight rows cost the 64-wide kernel a wave per SIMD
+    mixer_ssm_block<true, 4>(p, blockIdx.x - p.attention_blocks);
   else
-    mixer_ssm_block<false>(p, blockIdx.x - p.attention_blocks);
+    mixer_ssm_block<true, 8>(p, blockIdx.x - p.attention_blocks);
 }
 
 extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv, int dh, int q_col, int k_col,
@@ -847,7 +875,18 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
   }
   p.R = R;
   p.vector_scan = vector_scan ? 1 : 0;
-  const int rows_per_block = MX_THREADS / R;
+  // rows of a head per workgroup: one per thread group while the step has few workgroups (they hide each
+  // other's latency); more from then on.  The state-space workgroups run at the register count of the
+  // attention ones (two to four waves a SIMD), so what a large step needs is bytes in flight per thread;
+  // a launch of their own at full occupancy was measured slower than that.
+  int rows_per_block = MX_THREADS / R;
+  p.rows_per_thread = 1;
+  const int most_rows = dh == 128 ? 8 : 4;
+  while (vector_scan && p.rows_per_thread < most_rows && rows_per_block < P &&
+         (long)M * H * ((P + rows_per_block - 1) / rows_per_block) > MX_FEW_BLOCKS) {
+    p.rows_per_thread *= 2;
+    rows_per_block *= 2;
+  }
   p.p_tiles = (P + rows_per_block - 1) / rows_per_block;
   p.z_col = z_col;
   p.x_col = x_col;
