@@ -202,7 +202,7 @@ extern "C" int mi_conv_state_update(const void* u, int dtype, long ld, int col_o
 // [col_offset, col_offset + C): u = SiLU(bias + sum_k w[c, k] * window[k]) with window = [tail ; new
 // sample]; the tail is rolled by one and takes the sample (the same formula as conv1d_silu and
 // conv_state_update for a lane of length one).  One thread per (row, channel); all loads first.
-template <typename T>
+template <typename T, int MAXK>
 __global__ void conv_step_kernel(T* __restrict__ u, long ld, int col_offset, int C, int K, const float* __restrict__ weight,
                                  const float* __restrict__ bias, T* __restrict__ conv_state,
                                  const int* __restrict__ slot_ids, long total) {
@@ -213,16 +213,16 @@ __global__ void conv_step_kernel(T* __restrict__ u, long ld, int col_offset, int
   T* cell = u + (long)m * ld + col_offset + channel;
   T* tail = K > 1 ? conv_state + (long)slot_ids[m] * (K - 1) * C + channel : cell;      // no tail with one tap
   const T sample = *cell;
-  T window[CONV_MAX_K];
-  float taps[CONV_MAX_K];
+  T window[MAXK];
+  float taps[MAXK];
 #pragma unroll
-  for (int k = 0; k < CONV_MAX_K; ++k) {
+  for (int k = 0; k < MAXK; ++k) {
     window[k] = tail[(long)min(k, max(K - 2, 0)) * C];       // clamped: read, not used, past the tail
     taps[k] = weight[(long)channel * K + min(k, K - 1)];
   }
   float sum = bias ? bias[channel] : 0.f;
 #pragma unroll
-  for (int k = 0; k < CONV_MAX_K; ++k) {
+  for (int k = 0; k < MAXK; ++k) {
     if (k < K - 1) {
       sum += taps[k] * (float)window[k];
       if (k > 0) tail[(long)(k - 1) * C] = window[k];
@@ -239,14 +239,19 @@ extern "C" int mi_conv_step(void* u, int dtype, long ld, int col_offset, int M, 
   if (M <= 0 || C <= 0 || K <= 0 || K > CONV_MAX_K) return ERR_BAD_ARGUMENT;
   const long total = (long)M * C;
   const int blocks = (int)((total + 255) / 256);
-  if (dtype == DT_F32)
-    conv_step_kernel<float><<<blocks, 256, 0, stream>>>((float*)u, ld, col_offset, C, K, weight, bias, (float*)conv_state,
-                                                        slot_ids, total);
-  else if (dtype == DT_BF16)
-    conv_step_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)u, ld, col_offset, C, K, weight, bias,
-                                                         (bf16_t*)conv_state, slot_ids, total);
-  else
+#define CONV_STEP(T_, MAXK_)                                                                                  \
+  conv_step_kernel<T_, MAXK_><<<blocks, 256, 0, stream>>>((T_*)u, ld, col_offset, C, K, weight, bias, (T_*)conv_state, \
+                                                          slot_ids, total)
+  if (dtype == DT_F32) {
+    if (K <= 4) CONV_STEP(float, 4);
+    else CONV_STEP(float, CONV_MAX_K);
+  } else if (dtype == DT_BF16) {
+    if (K <= 4) CONV_STEP(bf16_t, 4);
+    else CONV_STEP(bf16_t, CONV_MAX_K);
+  } else {
     return ERR_BAD_ARGUMENT;
+  }
+#undef CONV_STEP
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

@@ -84,7 +84,7 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
     cycled through so that the caches do not hold it, as in a model of many layers."""
     N, K = weight.shape
     device = weight.device
-    copies = max(2, min(8, (512 << 20) // (weight.numel() * 2)))
+    copies = max(2, min(64, (512 << 20) // (weight.numel() * 2)))
     weights = [weight] + [weight.clone() for _ in range(copies - 1)]
     x = torch.randn((rows, K), dtype=torch.bfloat16, device=device)
     out = torch.empty((rows, N // 2 if epilogue == ops.EPI_SWIGLU else N), dtype=torch.bfloat16, device=device)
