@@ -50,6 +50,14 @@ LIBRARY_MARGIN = 0.92          # the library has to be this much faster to be ta
 FORCE_LIBRARY: Optional[bool] = None      # tests: True or False instead of the clock
 TUNE_ROWS = (8, 32, 64)
 _library_wins: Dict[tuple, bool] = {}
+# The library's tile for a prompt portion's input projection depends on the number of output features: 4 120
+# of them (0.5B-shaped) take 30.5 us at 2,048 rows, 4 352 (a multiple of 256) take 23.6.  Measured at build in
+# the same way; where padding pays, the prompt path multiplies with zero rows added and ignores their columns.
+PAD_FEATURES = 256
+PAD_ROWS = 2048
+PAD_MARGIN = 0.95
+FORCE_PADDING: Optional[bool] = None      # tests: True or False instead of the clock
+_padding_wins: Dict[tuple, bool] = {}
 
 
 def _bucket(rows: int) -> int:
@@ -77,6 +85,32 @@ def _graph_microseconds(run) -> float:
     end.record()
     end.synchronize()
     return start.elapsed_time(end) * 1e3 / 3
+
+
+def _padding_pays(weight: torch.Tensor) -> bool:
+    """Whether rows of zeros up to a multiple of PAD_FEATURES make the library's product of a prompt portion faster."""
+    N, K = weight.shape
+    if N % PAD_FEATURES == 0 or FORCE_PADDING is False:
+        return False
+    if FORCE_PADDING:
+        return True
+    if weight.numel() < LIBRARY_MIN_WEIGHT:
+        return False
+    key = (N, K)
+    if key not in _padding_wins:
+        x = torch.randn((PAD_ROWS, K), dtype=torch.bfloat16, device=weight.device)
+        padded = torch.cat([weight, weight.new_zeros((-N % PAD_FEATURES, K))])
+
+        def plain():
+            for _ in range(4):
+                torch.matmul(x, weight.t())
+
+        def wide():
+            for _ in range(4):
+                torch.matmul(x, padded.t())
+
+        _padding_wins[key] = _graph_microseconds(wide) < PAD_MARGIN * _graph_microseconds(plain)
+    return _padding_wins[key]
 
 
 def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile: int, conv: Optional[dict]) -> bool:
@@ -155,6 +189,14 @@ class ParallelFusion:
         # 1: [q | k | v | z | x B C | dt]
         self.w_in = torch.cat([attention.qkv.weight, mamba.in_proj.weight], dim=0).contiguous()
         self.b_in = _cat_bias([attention.qkv, mamba.in_proj], device)
+        # prompt portions may multiply with rows of zeros added (the decode kernels take the rows that count)
+        self.w_in_wide, self.b_in_wide = self.w_in, self.b_in
+        if _padding_pays(self.w_in):
+            extra = -self.w_in.shape[0] % PAD_FEATURES
+            self.w_in_wide = torch.cat([self.w_in, self.w_in.new_zeros((extra, self.w_in.shape[1]))])
+            self.w_in = self.w_in_wide[:self.w_in.shape[0]]
+            if self.b_in is not None:
+                self.b_in_wide = torch.cat([self.b_in, self.b_in.new_zeros(extra)])
         self.q_col, self.k_col, self.v_col = 0, q_width, q_width + kv_width
         self.z_col = q_width + 2 * kv_width
         self.x_col = self.z_col + E
@@ -212,10 +254,10 @@ class ParallelFusion:
     def forward_general(self, residual: Residual, step, caches) -> None:
         block = self.block
         normed = block.mixer_norm.forward(residual)
-        u = ops.linear(normed, self.w_in, self.b_in)
+        u = ops.linear(normed, self.w_in_wide, self.b_in_wide)
         mixed = torch.empty((u.shape[0], self.mixed_width), dtype=u.dtype, device=u.device)
         self.attention.mix(u[:, :self.qkv_width], step, caches[self.attention_name], mixed[:, :self.q_width])
-        self.mamba.mix(u[:, self.qkv_width:], step, caches[self.mamba_name], mixed[:, self.q_width:])
+        self.mamba.mix(u[:, self.qkv_width:self.in_width], step, caches[self.mamba_name], mixed[:, self.q_width:])
         residual.pending = [ops.linear(mixed, self.w_out, self.b_out)]
         normed = block.ffn_norm.forward(residual)
         residual.pending = [block.ffn.forward(normed)]

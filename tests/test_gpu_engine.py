@@ -367,16 +367,23 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
     assert with_graphs.graphs.counts["portion_replays"] == replays + 3      # turns 2, 3 and 4
 
 
-def test_a_wide_model_runs_through_the_fast_paths(tmp_path):
+@pytest.mark.parametrize("padding", [False, True])
+def test_a_wide_model_runs_through_the_fast_paths(tmp_path, monkeypatch, padding):
     """Hidden size 2 112: the fused layer paths are built although the norm prologue does not fit;
-    prompt portions, a mixed step and graph-replayed decode steps against the plain model."""
+    prompt portions, a mixed step and graph-replayed decode steps against the plain model.
+    ``padding``: the input projection of prompt portions multiplies with rows of zeros added up to
+    a multiple of 256 features (what a measurement at build decides for large weights)."""
     from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.parts import fused
+    monkeypatch.setattr(fused, "FORCE_PADDING", padding)
     folder = tiny_configs.make_model_dir("D", tmp_path, torch.bfloat16)
     cfg, tensors = plain_impl.load_model_dir(folder)
     engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=512,
                     max_active_sequences=3)
     fusion = engine.model.blocks[0].fusion
     assert fusion is not None and not fusion.norm_fits and fusion.general
+    assert (fusion.w_in_wide.shape[0] % 256 == 0) == padding and fusion.w_in.shape[0] == fusion.in_width
+    assert fusion.w_in.data_ptr() == fusion.w_in_wide.data_ptr()
     sequences = {key: tokens_for(cfg["vocab_size"], 70 + 9 * index, 900 + index) for index, key in enumerate("abc")}
     got = {key: [] for key in sequences}
     for key in sequences:
