@@ -32,12 +32,10 @@ typedef float s_floatx4 __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------- prepare
 // delta[t, h] = softplus(dt + bias); cum[t, h] = sum of delta*A over the chunk up to t (inclusive).
-__global__ void ssd_prepare_kernel(const bf16_t* __restrict__ dt, long dt_ld, const float* __restrict__ dt_bias,
-                                   const float* __restrict__ A, const int* __restrict__ chunks, int H,
-                                   float* __restrict__ delta, float* __restrict__ cum) {
-  __shared__ float wave_total[SSD_MAX_Q / WAVE];
-  const int chunk = blockIdx.x;
-  const int head = blockIdx.y;
+__device__ void ssd_prepare_block(const bf16_t* __restrict__ dt, long dt_ld, const float* __restrict__ dt_bias,
+                                  const float* __restrict__ A, const int* __restrict__ chunks, int H,
+                                  float* __restrict__ delta, float* __restrict__ cum, int chunk, int head,
+                                  float* wave_total) {
   const int t0 = chunks[4 * chunk + 1];
   const int length = chunks[4 * chunk + 2];
   const int s = threadIdx.x;
@@ -69,13 +67,9 @@ __global__ void ssd_prepare_kernel(const bf16_t* __restrict__ dt, long dt_ld, co
 // 64 channels of a chunk per workgroup: 16-byte loads along the channels, 2-byte stores into a
 // transposed LDS tile whose row stride (Q + 2 elements = an odd number of banks) keeps them
 // apart, 4-byte LDS reads and 16-byte stores along the tokens.
-__global__ void __launch_bounds__(256)
-ssd_transpose_kernel(const bf16_t* __restrict__ xbc, long ld, int channels, const int* __restrict__ chunks, int Q,
-                     bf16_t* __restrict__ out) {
-  __shared__ __align__(4) bf16_t tile[64 * (SSD_MAX_Q + 2)];
+__device__ void ssd_transpose_block(const bf16_t* __restrict__ xbc, long ld, int channels, const int* __restrict__ chunks,
+                                    int Q, bf16_t* __restrict__ out, int chunk, int c0, bf16_t* tile) {
   const int stride = Q + 2;
-  const int chunk = blockIdx.x;
-  const int c0 = blockIdx.y * 64;
   const int t0 = chunks[4 * chunk + 1];
   const int length = chunks[4 * chunk + 2];
   for (int index = threadIdx.x; index < Q * 8; index += 256) {
@@ -102,6 +96,144 @@ ssd_transpose_kernel(const bf16_t* __restrict__ xbc, long ld, int channels, cons
     v.w = words[3];
     *reinterpret_cast<uint4*>(out + ((long)chunk * channels + c0 + c) * Q + s) = v;
   }
+}
+
+// Both in one launch (they do not depend on each other and each is too small to fill the GPU): rows
+// 0 .. H-1 of the grid prepare a head, the rows after transpose 64 channels.
+__global__ void __launch_bounds__(256)
+ssd_prepare_transpose_kernel(const bf16_t* __restrict__ dt, long dt_ld, const float* __restrict__ dt_bias,
+                             const float* __restrict__ A, const int* __restrict__ chunks, int H, float* __restrict__ delta,
+                             float* __restrict__ cum, const bf16_t* __restrict__ xbc, long xbc_ld, int channels, int Q,
+                             bf16_t* __restrict__ TT) {
+  __shared__ __align__(4) bf16_t tile[64 * (SSD_MAX_Q + 2)];
+  __shared__ float wave_total[SSD_MAX_Q / WAVE];
+  if ((int)blockIdx.y < H)
+    ssd_prepare_block(dt, dt_ld, dt_bias, A, chunks, H, delta, cum, blockIdx.x, blockIdx.y, wave_total);
+  else
+    ssd_transpose_block(xbc, xbc_ld, channels, chunks, Q, TT, blockIdx.x, ((int)blockIdx.y - H) * 64, tile);
+}
+
+// ---------------------------------------------------------------- conv, fused with the transpose
+// The causal depthwise conv + SiLU of mamba2.hip (conv1d_silu) on a chunk's tokens and 64 channels, from the
+// raw projection rows: the result goes to xbc[t, channel] (row-major, what the chunk scan reads for C, B and
+// the skip) and, for the channels of x and B, into the transposed copy as well.  A thread takes 8 channels and
+// 4 consecutive tokens; the K-1 rows before a chunk are the lane's previous tokens, or the request's conv
+// tail when the chunk opens the lane.  All loads first, none under a condition (rows and channels that do
+// not exist are clamped and dropped).  The tail itself is updated later, by ssd_tail_block, once every
+// chunk has read it.
+template <int K>
+__device__ void ssd_conv_block(const bf16_t* __restrict__ u, long u_ld, int C, const float* __restrict__ conv_w,
+                               const float* __restrict__ conv_b, const bf16_t* __restrict__ conv_state,
+                               const int* __restrict__ chunks, const int* __restrict__ slot_ids, int Q,
+                               bf16_t* __restrict__ xbc, long xbc_ld, int tt_channels, bf16_t* __restrict__ TT,
+                               int chunk, int c0, bf16_t* tile) {
+  constexpr int ROWS = 4;
+  const int stride = Q + 2;
+  const int lane_id = chunks[4 * chunk];
+  const int t0 = chunks[4 * chunk + 1];
+  const int length = chunks[4 * chunk + 2];
+  const bool opens = chunks[4 * chunk + 3] == 0;
+  const bf16_t* tail = conv_state + (long)slot_ids[lane_id] * (K - 1) * C;
+  const long first_row = opens ? (long)t0 : (long)t0 - (K - 1);
+  const float* bias_or_taps = conv_b ? conv_b : conv_w;
+  for (int item = threadIdx.x; item < (Q / ROWS) * 8; item += 256) {
+    const int s0 = (item / 8) * ROWS;
+    const int c = (item % 8) * 8;
+    const bool real = c0 + c < C;
+    const int channel = real ? c0 + c : C - 8;
+    s_bf16x8 window[ROWS + K - 1], before[K - 1];
+#pragma unroll
+    for (int j = 0; j < ROWS + K - 1; ++j) {
+      const long row = min(max((long)t0 + s0 - (K - 1) + j, first_row), (long)t0 + length - 1);
+      window[j] = *reinterpret_cast<const s_bf16x8*>(u + row * u_ld + channel);
+    }
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j) before[j] = *reinterpret_cast<const s_bf16x8*>(tail + (long)j * C + channel);
+    s_floatx4 taps[2 * K];                          // conv_w[channel .. channel+8, 0 .. K): 8K contiguous floats
+#pragma unroll
+    for (int j = 0; j < 2 * K; ++j) taps[j] = *reinterpret_cast<const s_floatx4*>(conv_w + (long)channel * K + 4 * j);
+    const s_floatx4 b_lo = *reinterpret_cast<const s_floatx4*>(bias_or_taps + channel);
+    const s_floatx4 b_hi = *reinterpret_cast<const s_floatx4*>(bias_or_taps + channel + 4);
+    if (opens && s0 == 0) {
+#pragma unroll
+      for (int j = 0; j < K - 1; ++j) window[j] = before[j];
+    }
+    auto tap = [&](int cc, int k) { return taps[(cc * K + k) / 4][(cc * K + k) % 4]; };
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+      const int position = s0 + i;
+      float sum[8];
+#pragma unroll
+      for (int cc = 0; cc < 8; ++cc) sum[cc] = conv_b ? (cc < 4 ? b_lo[cc] : b_hi[cc - 4]) : 0.f;
+#pragma unroll
+      for (int k = 0; k < K; ++k)
+#pragma unroll
+        for (int cc = 0; cc < 8; ++cc) sum[cc] += tap(cc, k) * (float)window[i + k][cc];
+      s_bf16x8 result;
+      const bool live = real && position < length;
+#pragma unroll
+      for (int cc = 0; cc < 8; ++cc) result[cc] = live ? (bf16_t)silu_f(sum[cc]) : (bf16_t)0.f;
+      if (live) *reinterpret_cast<s_bf16x8*>(xbc + (long)(t0 + position) * xbc_ld + channel) = result;
+#pragma unroll
+      for (int cc = 0; cc < 8; ++cc) tile[(c + cc) * stride + position] = result[cc];
+    }
+  }
+  __syncthreads();
+  const int vectors = Q / 8;
+  for (int index = threadIdx.x; index < 64 * vectors; index += 256) {
+    const int c = index / vectors;
+    const int position = (index % vectors) * 8;
+    if (c0 + c >= tt_channels) continue;
+    const unsigned* words = reinterpret_cast<const unsigned*>(tile + c * stride + position);
+    uint4 v;
+    v.x = words[0];
+    v.y = words[1];
+    v.z = words[2];
+    v.w = words[3];
+    *reinterpret_cast<uint4*>(TT + ((long)chunk * tt_channels + c0 + c) * Q + position) = v;
+  }
+}
+
+// prepare (rows 0 .. H-1 of the grid) and the conv with the transpose (the rows after) in one launch
+template <int K>
+__global__ void __launch_bounds__(256)
+ssd_prepare_conv_kernel(const bf16_t* __restrict__ dt, long dt_ld, const float* __restrict__ dt_bias,
+                        const float* __restrict__ A, const int* __restrict__ chunks, int H, float* __restrict__ delta,
+                        float* __restrict__ cum, const bf16_t* __restrict__ u, long u_ld, int C,
+                        const float* __restrict__ conv_w, const float* __restrict__ conv_b,
+                        const bf16_t* __restrict__ conv_state, const int* __restrict__ slot_ids, int Q,
+                        bf16_t* __restrict__ xbc, long xbc_ld, int tt_channels, bf16_t* __restrict__ TT) {
+  __shared__ __align__(4) bf16_t tile[64 * (SSD_MAX_Q + 2)];
+  __shared__ float wave_total[SSD_MAX_Q / WAVE];
+  if ((int)blockIdx.y < H)
+    ssd_prepare_block(dt, dt_ld, dt_bias, A, chunks, H, delta, cum, blockIdx.x, blockIdx.y, wave_total);
+  else
+    ssd_conv_block<K>(u, u_ld, C, conv_w, conv_b, conv_state, chunks, slot_ids, Q, xbc, xbc_ld, tt_channels, TT,
+                      blockIdx.x, ((int)blockIdx.y - H) * 64, tile);
+}
+
+// The conv tail of a lane after its tokens: the last K-1 rows of [old tail ; the lane's raw rows]
+// (conv_state_update of mamba2.hip), one thread per channel; every old value is read before the first is written.
+__device__ void ssd_tail_block(const bf16_t* __restrict__ u, long u_ld, int C, int K, bf16_t* __restrict__ conv_state,
+                               const int* __restrict__ chunks, const int* __restrict__ lane_chunks,
+                               const int* __restrict__ slot_ids, int Q, int lane, int channel) {
+  if (channel >= C) return;
+  const int first = lane_chunks[2 * lane];
+  const int count = lane_chunks[2 * lane + 1];
+  const long start = chunks[4 * first + 1];
+  const long total = (long)(count - 1) * Q + chunks[4 * (first + count - 1) + 2];
+  bf16_t* tail = conv_state + (long)slot_ids[lane] * (K - 1) * C + channel;
+  bf16_t kept[3];
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    if (j < K - 1) {
+      const long source = total + j;                 // row of the (K-1 + total)-row window
+      kept[j] = source < K - 1 ? tail[source * C] : u[(start + source - (K - 1)) * u_ld + channel];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 3; ++j)
+    if (j < K - 1) tail[(long)j * C] = kept[j];
 }
 
 // ---------------------------------------------------------------- chunk state
@@ -178,8 +310,16 @@ ssd_chunk_state_kernel(const bf16_t* __restrict__ TT, int E, int GN, const float
 // starts from the request's slot and goes back to it, in float32.
 __global__ void ssd_state_pass_kernel(const float* __restrict__ chunk_state, const float* __restrict__ chunk_decay,
                                       const int* __restrict__ lane_chunks, const int* __restrict__ slot_ids, int H,
-                                      long per_head, float* __restrict__ ssm_state, bf16_t* __restrict__ state_in) {
+                                      long per_head, float* __restrict__ ssm_state, bf16_t* __restrict__ state_in,
+                                      const bf16_t* __restrict__ u, long u_ld, int C, int K,
+                                      bf16_t* __restrict__ conv_state, const int* __restrict__ chunks, int Q) {
   const int lane = blockIdx.z;
+  if ((int)blockIdx.y >= H) {                // rows past the heads (when the conv ran here): the lane's conv tail
+    if (blockIdx.x == 0)
+      ssd_tail_block(u, u_ld, C, K, conv_state, chunks, lane_chunks, slot_ids, Q, lane,
+                     ((int)blockIdx.y - H) * blockDim.x + threadIdx.x);
+    return;
+  }
   const int head = blockIdx.y;
   const long element = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (element >= per_head) return;
@@ -588,24 +728,38 @@ extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long
                               const int* lane_chunks, const int* slot_ids, int n_lanes, int Q, int H, int P, int N,
                               int G, float* delta, float* cum, void* TT, float* chunk_state,
                               float* chunk_decay, void* state_in, float* y, long y_ld, const void* z, long z_ld,
-                              void* gated, long gated_ld, hipStream_t stream) {
+                              void* gated, long gated_ld, const void* u, long u_ld, const float* conv_w,
+                              const float* conv_b, void* conv_state, int conv_k, hipStream_t stream) {
   if (n_chunks <= 0 || n_lanes <= 0 || H <= 0 || G <= 0 || H % G != 0) return ERR_BAD_ARGUMENT;
   const int E = H * P;
   const int GN = G * N;
+  const int C = E + 2 * GN;
+  const bool conv_here = u != nullptr;       // xbc is then written here, from the raw rows u [T, C] (+ u_ld)
+  if (conv_here && (!conv_w || !conv_state || conv_k < 2 || conv_k > 4 || u_ld % 8 != 0 || C % 8 != 0 ||
+                    ((uintptr_t)u % 16) != 0 || ((uintptr_t)conv_state % 16) != 0 || ((uintptr_t)conv_w % 16) != 0 ||
+                    ((uintptr_t)conv_b % 16) != 0 || H + (C + 63) / 64 > 65535 || H + (C + 255) / 256 > 65535))
+    return ERR_UNSUPPORTED_SIZE;
   if ((z == nullptr) != (gated == nullptr) || (z == nullptr && y == nullptr)) return ERR_BAD_ARGUMENT;
   if (!mi_ssd_supported(Q, P, N, G, E) || xbc_ld % 8 != 0 || y_ld % 4 != 0 || z_ld % 4 != 0 || gated_ld % 4 != 0 ||
       n_chunks > 65535 * 32 ||
-      H > 65535 || n_lanes > 65535)
+      H + (E + GN + 63) / 64 > 65535 || n_lanes > 65535)
     return ERR_UNSUPPORTED_SIZE;
-  {
-    const dim3 grid(n_chunks, H);
-    const int threads = ((Q + WAVE - 1) / WAVE) * WAVE;
-    ssd_prepare_kernel<<<grid, threads, 0, stream>>>((const bf16_t*)dt, dt_ld, dt_bias, A, chunks, H, delta, cum);
+  if (conv_here) {
+    const dim3 grid(n_chunks, H + (C + 63) / 64);
+#define CONV_CASE(K_)                                                                                              \
+  ssd_prepare_conv_kernel<K_><<<grid, 256, 0, stream>>>((const bf16_t*)dt, dt_ld, dt_bias, A, chunks, H, delta, cum,  \
+                                                        (const bf16_t*)u, u_ld, C, conv_w, conv_b,                  \
+                                                        (const bf16_t*)conv_state, slot_ids, Q, (bf16_t*)xbc,       \
+                                                        xbc_ld, E + GN, (bf16_t*)TT)
+    if (conv_k == 2) CONV_CASE(2);
+    else if (conv_k == 3) CONV_CASE(3);
+    else CONV_CASE(4);
+#undef CONV_CASE
     RETURN_IF_LAUNCH_FAILED();
-  }
-  {
-    const dim3 grid_t(n_chunks, (E + GN + 63) / 64);         // x and B are neighbours in a row of xbc
-    ssd_transpose_kernel<<<grid_t, 256, 0, stream>>>((const bf16_t*)xbc, xbc_ld, E + GN, chunks, Q, (bf16_t*)TT);
+  } else {
+    const dim3 grid(n_chunks, H + (E + GN + 63) / 64);       // x and B are neighbours in a row of xbc
+    ssd_prepare_transpose_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)dt, dt_ld, dt_bias, A, chunks, H, delta, cum,
+                                                           (const bf16_t*)xbc, xbc_ld, E + GN, Q, (bf16_t*)TT);
     RETURN_IF_LAUNCH_FAILED();
   }
   {
@@ -624,9 +778,10 @@ extern "C" int mi_ssd_prefill(const void* xbc, long xbc_ld, const void* dt, long
   }
   {
     const long per_head = (long)P * N;
-    const dim3 grid((unsigned)((per_head + 255) / 256), H, n_lanes);
+    const dim3 grid((unsigned)((per_head + 255) / 256), H + (conv_here ? (C + 255) / 256 : 0), n_lanes);
     ssd_state_pass_kernel<<<grid, 256, 0, stream>>>(chunk_state, chunk_decay, lane_chunks, slot_ids, H, per_head,
-                                                    ssm_state, (bf16_t*)state_in);
+                                                    ssm_state, (bf16_t*)state_in, (const bf16_t*)u, u_ld, C, conv_k,
+                                                    (bf16_t*)conv_state, chunks, Q);
     RETURN_IF_LAUNCH_FAILED();
   }
   const bool staged = (P == 16 || P == 32 || P == 64 || P == 128) && (N == 32 || N == 64 || N == 128 || N == 256) &&

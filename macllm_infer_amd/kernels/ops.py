@@ -61,7 +61,8 @@ _SIGNATURES = {
         "mi_ssd_supported": [_c_int, _c_int, _c_int, _c_int, _c_int],
         "mi_ssd_prefill": [_c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr,
                            _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
-                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr],
+                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_long,
+                           _c_ptr, _c_long, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
     },
     "gemm": {
         "mi_gemm_f32": [_c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr],
@@ -504,10 +505,13 @@ def ssd_supported(chunk_size: int, head_dim: int, state_size: int, num_groups: i
 def ssd_prefill(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
                 ssm_state: torch.Tensor, table: SsdChunks, slot_ids: torch.Tensor, num_groups: int,
                 y: Optional[torch.Tensor], z: Optional[torch.Tensor] = None,
-                gated: Optional[torch.Tensor] = None) -> None:
+                gated: Optional[torch.Tensor] = None, conv: Optional[dict] = None) -> None:
     """The selective scan of ``ssm_scan`` (same arguments and results beyond rounding) for bfloat16,
     in chunks on the matrix cores.  ``table`` cuts this step's lanes into chunks.  With ``z`` and
-    ``gated`` (bfloat16 [T, E], column views are fine) it writes gated = y * SiLU(z) and no y."""
+    ``gated`` (bfloat16 [T, E], column views are fine) it writes gated = y * SiLU(z) and no y.
+    With ``conv`` = {u, weight, bias, state} the conv runs here too: ``xbc`` is then written (what
+    ``conv1d_silu`` would put there from the raw rows ``u`` [T, C]) and the tails ``state`` updated
+    (as ``conv_state_update`` would); see ``ssd_conv_supported``."""
     xbc_ld = _row_major(xbc, "xbc")
     dt_ld = _row_major(dt, "dt")
     fused_gate = z is not None
@@ -544,12 +548,32 @@ def ssd_prefill(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: t
     chunk_state = torch.empty((chunks * H * P * N + chunks * H,), dtype=torch.float32, device=device)
     state_in = torch.empty((chunks * H * P * N,), dtype=torch.bfloat16, device=device)
     decay = chunk_state[chunks * H * P * N:]
+    raw = conv_w = conv_b = conv_state = None
+    raw_ld = taps = 0
+    if conv is not None:
+        raw, conv_w, conv_b, conv_state = conv["u"], conv["weight"], conv.get("bias"), conv["state"]
+        raw_ld = _row_major(raw, "conv u")
+        C = E + 2 * GN
+        taps = conv_w.shape[1]
+        _need(raw.dtype == torch.bfloat16 and raw.shape == (T, C), "ssd_prefill: conv u must be bfloat16 [T, C]")
+        _need(conv_w.dtype == torch.float32 and conv_w.shape == (C, taps) and conv_w.is_contiguous(),
+              "ssd_prefill: conv weight must be float32 [C, K]")
+        _need(conv_b is None or (conv_b.dtype == torch.float32 and conv_b.numel() == C), "ssd_prefill: bad conv bias")
+        _need(conv_state.dim() == 3 and conv_state.shape[1:] == (taps - 1, C) and conv_state.dtype == torch.bfloat16
+              and conv_state.is_contiguous(), "ssd_prefill: bad conv state")
+        _need(ssd_conv_supported(taps, C, raw), "ssd_prefill: the conv does not fit (see ssd_conv_supported)")
     _check(_fn("ssd", "mi_ssd_prefill")(
         _p(xbc), xbc_ld, _p(dt), dt_ld, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(table.chunks), chunks,
         _p(table.lane_chunks), _p(slot_ids), table.num_lanes, Q, H, P, N, num_groups, _p(delta[0]), _p(delta[1]),
         _p(transposed), _p(chunk_state), _p(decay), _p(state_in), _p(y), y_ld, _p(z), z_ld, _p(gated), gated_ld,
-        _stream()),
+        _p(raw), raw_ld, _p(conv_w), _p(conv_b), _p(conv_state), int(taps), _stream()),
         "ssd_prefill", f"(Q={Q}, P={P}, N={N})")
+
+
+def ssd_conv_supported(taps: int, channels: int, u: torch.Tensor) -> bool:
+    """Whether ``ssd_prefill`` can run the conv itself: 2 to 4 taps, channels in eights, 16-byte rows."""
+    return (2 <= taps <= 4 and channels % 8 == 0 and u.dim() == 2 and u.stride(1) == 1 and u.stride(0) % 8 == 0
+            and u.data_ptr() % 16 == 0)
 
 
 def gate_norm(y: torch.Tensor, z: torch.Tensor, weight: Optional[torch.Tensor], num_groups: int, eps: float,

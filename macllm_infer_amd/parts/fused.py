@@ -60,6 +60,17 @@ FORCE_PADDING: Optional[bool] = None      # tests: True or False instead of the 
 _padding_wins: Dict[tuple, bool] = {}
 
 
+OVERLAP_MIN_TOKENS = 256       # prompt portions from this size on run their two mixers on two streams
+_side_streams: Dict[int, "torch.cuda.Stream"] = {}
+
+
+def _side_stream(device: torch.device) -> "torch.cuda.Stream":
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _side_streams:
+        _side_streams[index] = torch.cuda.Stream(device=device)       # default priority
+    return _side_streams[index]
+
+
 def _bucket(rows: int) -> int:
     return 0 if rows <= MAX_NORM_ROWS else 1 if rows <= 32 else 2
 
@@ -98,7 +109,7 @@ def _padding_pays(weight: torch.Tensor) -> bool:
         return False
     key = (N, K)
     if key not in _padding_wins:
-        x = torch.randn((PAD_ROWS, K), dtype=torch.bfloat16, device=weight.device)
+        x = torch.full((PAD_ROWS, K), 0.01, dtype=torch.bfloat16, device=weight.device)
         padded = torch.cat([weight, weight.new_zeros((-N % PAD_FEATURES, K))])
 
         def plain():
@@ -120,7 +131,7 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
     device = weight.device
     copies = max(2, min(64, (512 << 20) // (weight.numel() * 2)))
     weights = [weight] + [weight.clone() for _ in range(copies - 1)]
-    x = torch.randn((rows, K), dtype=torch.bfloat16, device=device)
+    x = torch.full((rows, K), 0.01, dtype=torch.bfloat16, device=device)      # not drawn: the global generator stays as it is
     out = torch.empty((rows, N // 2 if epilogue == ops.EPI_SWIGLU else N), dtype=torch.bfloat16, device=device)
     if conv is not None:
         channels = conv["hi"] - conv["lo"]
@@ -256,8 +267,20 @@ class ParallelFusion:
         normed = block.mixer_norm.forward(residual)
         u = ops.linear(normed, self.w_in_wide, self.b_in_wide)
         mixed = torch.empty((u.shape[0], self.mixed_width), dtype=u.dtype, device=u.device)
-        self.attention.mix(u[:, :self.qkv_width], step, caches[self.attention_name], mixed[:, :self.q_width])
-        self.mamba.mix(u[:, self.qkv_width:self.in_width], step, caches[self.mamba_name], mixed[:, self.q_width:])
+        if u.shape[0] >= OVERLAP_MIN_TOKENS:
+            # the two mixers read the same rows and write different columns: attention runs on a second
+            # stream beside the state-space chain, whose kernels are many and small
+            main = torch.cuda.current_stream(u.device)
+            side = _side_stream(u.device)
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                self.attention.mix(u[:, :self.qkv_width], step, caches[self.attention_name], mixed[:, :self.q_width])
+
+            self.mamba.mix(u[:, self.qkv_width:self.in_width], step, caches[self.mamba_name], mixed[:, self.q_width:])
+            main.wait_stream(side)
+        else:
+            self.attention.mix(u[:, :self.qkv_width], step, caches[self.attention_name], mixed[:, :self.q_width])
+            self.mamba.mix(u[:, self.qkv_width:self.in_width], step, caches[self.mamba_name], mixed[:, self.q_width:])
         residual.pending = [ops.linear(mixed, self.w_out, self.b_out)]
         normed = block.ffn_norm.forward(residual)
         residual.pending = [block.ffn.forward(normed)]

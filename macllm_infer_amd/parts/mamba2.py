@@ -103,17 +103,24 @@ class Mamba2(Mixer):
         T = u.shape[0]
         conv_state, ssm_state = cache.states["conv"], cache.states["ssm"]
         xbc = torch.empty((T, C), dtype=u.dtype, device=u.device)
-        ops.conv1d_silu(u, E, C, self.conv_weight, self.conv_bias, conv_state, step.lane_of_token,
-                        step.cu_seqlens, step.slot_ids, xbc)
-        ops.conv_state_update(u, E, C, spec.conv_kernel, conv_state, step.cu_seqlens, step.slot_ids)
-        if self._chunked(u, step):
+        chunked = self._chunked(u, step)
+        raw = u[:, E:E + C]
+        conv = None
+        if chunked and ops.ssd_conv_supported(spec.conv_kernel, C, raw):
+            # the chunked scan runs the conv and the tail update in its own launches
+            conv = dict(u=raw, weight=self.conv_weight, bias=self.conv_bias, state=conv_state)
+        else:
+            ops.conv1d_silu(u, E, C, self.conv_weight, self.conv_bias, conv_state, step.lane_of_token,
+                            step.cu_seqlens, step.slot_ids, xbc)
+            ops.conv_state_update(u, E, C, spec.conv_kernel, conv_state, step.cu_seqlens, step.slot_ids)
+        if chunked:
             arguments = (xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, self._chunk_table(step),
                          step.slot_ids, spec.num_groups)
             if self.norm_weight is None and u.stride(0) % 4 == 0 and gated.stride(0) % 4 == 0:
-                ops.ssd_prefill(*arguments, None, z=u[:, :E], gated=gated)      # the gate on the scan's way out
+                ops.ssd_prefill(*arguments, None, z=u[:, :E], gated=gated, conv=conv)      # the gate on the scan's way out
                 return
             y = torch.empty((T, E), dtype=torch.float32, device=u.device)
-            ops.ssd_prefill(*arguments, y)
+            ops.ssd_prefill(*arguments, y, conv=conv)
         else:
             y = torch.empty((T, E), dtype=torch.float32, device=u.device)
             ops.ssm_scan(xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, step.cu_seqlens,

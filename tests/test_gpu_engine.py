@@ -367,6 +367,44 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
     assert with_graphs.graphs.counts["portion_replays"] == replays + 3      # turns 2, 3 and 4
 
 
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_long_portions_overlap_their_mixers(tmp_path, name):
+    """Portions of 256 tokens and more run attention on a second stream beside the state-space
+    chain (with the conv inside the chunked scan): a prompt of 300 tokens beside one of 259, eagerly
+    and, from the third step of that shape on, from a captured graph; then the same requests go on
+    with a portion and a decoded token.  Every wanted row against the plain model."""
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.parts import fused
+    folder = tiny_configs.make_model_dir(name, tmp_path, torch.bfloat16)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=4096,
+                    max_active_sequences=8)
+    assert engine.model.blocks[0].fusion is not None and fused.OVERLAP_MIN_TOKENS <= 259
+
+    def check(got, want):
+        scale = want.abs().max().item()
+        assert (got - want).abs().max().item() <= 6e-2 * scale
+        assert ((got - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()).item() <= 3e-2
+
+    for turn in range(4):
+        a, b = f"a{turn}", f"b{turn}"
+        tokens_a = tokens_for(cfg["vocab_size"], 340, 1000 + turn)
+        tokens_b = tokens_for(cfg["vocab_size"], 270, 1100 + turn)
+        engine.add_request(a)
+        engine.add_request(b)
+        logits = engine.step([Lane(a, tokens_a[:300], [0, 150, 299]), Lane(b, tokens_b[:259], [258])]).float().cpu()
+        want_a = plain_impl.falcon_h1_logits(cfg, tensors, tokens_a)
+        want_b = plain_impl.falcon_h1_logits(cfg, tensors, tokens_b)
+        check(logits[:3], want_a[[0, 150, 299]])
+        check(logits[3:], want_b[[258]])
+        logits = engine.step([Lane(a, tokens_a[300:], [39]), Lane(b, tokens_b[259:260], [0])]).float().cpu()
+        check(logits[:1], want_a[[339]])
+        check(logits[1:], want_b[[259]])
+        engine.finish(a)
+        engine.finish(b)
+    assert engine.graphs.counts["portion_replays"] >= 2
+
+
 @pytest.mark.parametrize("padding", [False, True])
 def test_a_wide_model_runs_through_the_fast_paths(tmp_path, monkeypatch, padding):
     """Hidden size 2 112: the fused layer paths are built although the norm prologue does not fit;

@@ -379,6 +379,54 @@ def test_chunked_scan_matches_the_token_by_token_scan(ops, Q, H, P, N, G):
     assert torch.equal(again, got_state)
 
 
+@pytest.mark.parametrize("K, Q, bias", [(4, 128, True), (3, 32, False), (2, 64, True), (4, 32, True)])
+def test_chunked_scan_with_the_conv_inside(ops, K, Q, bias):
+    """The conv and the tail update inside the chunked scan's launches against the separate kernels:
+    lanes of 1 and 2 tokens (shorter than the taps: part of the old tail stays), lanes that end on a
+    chunk's edge and one token after it, a lane of many chunks; shuffled slots; the raw rows are a
+    column view of a wider matrix; 192 conv channels = three blocks of 64, the last without x or B."""
+    H, P, N, G = 4, 16, 32, 2
+    E, GN = H * P, G * N
+    C = E + 2 * GN
+    counts = [1, 2, Q, Q + 1, 3 * Q + 7, 5]
+    T = sum(counts)
+    slots = len(counts) + 2
+    slot_ids = i32(torch.randperm(slots, generator=torch.Generator().manual_seed(9))[:len(counts)].tolist())
+    cu = i32([0] + torch.tensor(counts).cumsum(0).tolist())
+    lane_of_token = i32([lane for lane, count in enumerate(counts) for _ in range(count)])
+    wide = rand(T, 8 + C + H + 4, seed=90, dtype=torch.bfloat16).to(DEV)
+    raw, dt = wide[:, 8:8 + C], wide[:, 8 + C:8 + C + H]
+    weight, conv_bias = rand(C, K, seed=91, scale=0.5).to(DEV), (rand(C, seed=92).to(DEV) if bias else None)
+    tails = rand(slots, K - 1, C, seed=93, dtype=torch.bfloat16).to(DEV)
+    dt_bias, A, D = gpu(rand(H, seed=94) - 1.0, -torch.exp(torch.linspace(-3.0, 1.0, H)), rand(H, seed=95))
+    state = rand(slots, H, P, N, seed=96, scale=0.5).to(DEV)
+    table = ops.SsdChunks(counts, Q, DEV)
+    ids, cu, lane_of_token = gpu(slot_ids, cu, lane_of_token)
+    # the separate kernels
+    want_xbc, want_tails, want_state = torch.empty(T, C, dtype=torch.bfloat16, device=DEV), tails.clone(), state.clone()
+    ops.conv1d_silu(wide, 8, C, weight, conv_bias, want_tails, lane_of_token, cu, ids, want_xbc)
+    ops.conv_state_update(wide, 8, C, K, want_tails, cu, ids)
+    want_y = torch.empty(T, E, device=DEV)
+    ops.ssd_prefill(want_xbc, dt, dt_bias, A, D, want_state, table, ids, G, want_y)
+    # the conv inside
+    assert ops.ssd_conv_supported(K, C, raw)
+    got_xbc, got_tails, got_state = torch.full_like(want_xbc, float("nan")), tails.clone(), state.clone()
+    got_y = torch.empty(T, E, device=DEV)
+    ops.ssd_prefill(got_xbc, dt, dt_bias, A, D, got_state, table, ids, G, got_y,
+                    conv=dict(u=raw, weight=weight, bias=conv_bias, state=got_tails))
+    # the same sums in another order of fused multiply-adds: a last bit of bfloat16 may differ here and there
+    assert (got_xbc.float() - want_xbc.float()).abs().max().item() <= 2.0 ** -7 * want_xbc.float().abs().max().item()
+    assert (got_xbc != want_xbc).float().mean().item() < 1e-3
+    assert torch.equal(got_tails, want_tails)
+    close(got_y, want_y.cpu(), torch.bfloat16, max(1.0, want_y.abs().max().item()) * 0.1)
+    close(got_state, want_state.cpu(), torch.bfloat16, max(1.0, want_state.abs().max().item()) * 0.1)
+    # and both against the plain conv
+    plain_xbc, plain_tails = torch.empty(T, C, dtype=torch.bfloat16), tails.cpu().clone()
+    ref_ops.conv1d_silu(wide.cpu(), 8, C, weight.cpu(), None if conv_bias is None else conv_bias.cpu(), plain_tails,
+                        lane_of_token.cpu(), cu.cpu(), slot_ids, plain_xbc)
+    close(got_xbc, plain_xbc, torch.bfloat16, 4.0)
+
+
 def test_chunked_scan_carries_a_far_token_through_many_chunks(ops):
     """One token with a large x and a head that barely decays: 600 tokens later its state is what
     the output consists of; every chunk boundary between must pass it on."""
