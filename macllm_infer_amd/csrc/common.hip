@@ -67,7 +67,7 @@ template <typename T> struct Vec4;
 template <> struct Vec4<float> { typedef float type __attribute__((ext_vector_type(4))); };
 template <> struct Vec4<bf16_t> { typedef __bf16 type __attribute__((ext_vector_type(4))); };
 
-template <typename TD, typename TO>
+template <typename TD, typename TO, int ROUNDS>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta0, const TD* __restrict__ delta1,
                        const float* __restrict__ weight, float eps, TO* __restrict__ out,
@@ -79,53 +79,44 @@ add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta0, con
   const long out_row = blockIdx.x;
   const long row = rows ? (long)rows[out_row] : out_row;
   float* hr = h + row * d;
-  const int rounds = (d / 4 + 255) / 256;
-  f4 v[NORM_MAX_ROUNDS], w[NORM_MAX_ROUNDS];
-  d4 a[NORM_MAX_ROUNDS], b[NORM_MAX_ROUNDS];
-  int at[NORM_MAX_ROUNDS];
+  // every load first and none under a condition (a wait counts all loads before it): an absent delta
+  // reads the row itself and is dropped, a column past the end reads the last one
+  const TD* d0 = delta0 ? delta0 + row * d : reinterpret_cast<const TD*>(hr);
+  const TD* d1 = delta1 ? delta1 + row * d : reinterpret_cast<const TD*>(hr);
+  f4 v[ROUNDS], w[ROUNDS];
+  d4 a[ROUNDS], b[ROUNDS];
+  int at[ROUNDS];
 #pragma unroll
-  for (int r = 0; r < NORM_MAX_ROUNDS; ++r) at[r] = min(((int)threadIdx.x + r * 256) * 4, d - 4);
+  for (int r = 0; r < ROUNDS; ++r) at[r] = min(((int)threadIdx.x + r * 256) * 4, d - 4);
 #pragma unroll
-  for (int r = 0; r < NORM_MAX_ROUNDS; ++r)
-    if (r < rounds) v[r] = *reinterpret_cast<const f4*>(hr + at[r]);
-  if (delta0) {
+  for (int r = 0; r < ROUNDS; ++r) v[r] = *reinterpret_cast<const f4*>(hr + at[r]);
 #pragma unroll
-    for (int r = 0; r < NORM_MAX_ROUNDS; ++r)
-      if (r < rounds) a[r] = *reinterpret_cast<const d4*>(delta0 + row * d + at[r]);
-  }
-  if (delta1) {
+  for (int r = 0; r < ROUNDS; ++r) a[r] = *reinterpret_cast<const d4*>(d0 + at[r]);
 #pragma unroll
-    for (int r = 0; r < NORM_MAX_ROUNDS; ++r)
-      if (r < rounds) b[r] = *reinterpret_cast<const d4*>(delta1 + row * d + at[r]);
-  }
-  if (out) {
+  for (int r = 0; r < ROUNDS; ++r) b[r] = *reinterpret_cast<const d4*>(d1 + at[r]);
 #pragma unroll
-    for (int r = 0; r < NORM_MAX_ROUNDS; ++r)
-      if (r < rounds) w[r] = *reinterpret_cast<const f4*>(weight + at[r]);
-  }
+  for (int r = 0; r < ROUNDS; ++r) w[r] = *reinterpret_cast<const f4*>(weight + at[r]);
   float sum_squares = 0.f;
 #pragma unroll
-  for (int r = 0; r < NORM_MAX_ROUNDS; ++r) {
-    if (r < rounds) {
-      const bool mine = ((int)threadIdx.x + r * 256) * 4 < d;
+  for (int r = 0; r < ROUNDS; ++r) {
+    const bool mine = ((int)threadIdx.x + r * 256) * 4 < d;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float value = v[r][j];
-        if (delta0) value += (float)a[r][j];
-        if (delta1) value += (float)b[r][j];
-        v[r][j] = value;
-        if (mine) sum_squares += value * value;
-      }
-      if (mine && !rows && (delta0 || delta1)) *reinterpret_cast<f4*>(hr + at[r]) = v[r];
+    for (int j = 0; j < 4; ++j) {
+      float value = v[r][j];
+      if (delta0) value += (float)a[r][j];
+      if (delta1) value += (float)b[r][j];
+      v[r][j] = value;
+      if (mine) sum_squares += value * value;
     }
+    if (mine && !rows && (delta0 || delta1)) *reinterpret_cast<f4*>(hr + at[r]) = v[r];
   }
   const float total = block_sum(sum_squares, scratch);
   const float denominator = sqrtf(total / (float)d + eps);
   if (out) {
     TO* o = out + out_row * d;
 #pragma unroll
-    for (int r = 0; r < NORM_MAX_ROUNDS; ++r) {
-      if (r < rounds && ((int)threadIdx.x + r * 256) * 4 < d) {
+    for (int r = 0; r < ROUNDS; ++r) {
+      if (((int)threadIdx.x + r * 256) * 4 < d) {
         o4 packed;
 #pragma unroll
         for (int j = 0; j < 4; ++j) packed[j] = from_float<TO>(v[r][j] / denominator * w[r][j]);
@@ -146,9 +137,18 @@ extern "C" int mi_add_rmsnorm(float* h, const void* delta0, const void* delta1, 
   const size_t lds = (size_t)d * sizeof(float);
 #define LAUNCH(TD, TO)                                                                                      \
   do {                                                                                                      \
-    if (vectors)                                                                                            \
-      add_rmsnorm_vec_kernel<TD, TO><<<n_rows, 256, 0, stream>>>(h, (const TD*)delta0, (const TD*)delta1,   \
-                                                                 weight, eps, (TO*)out, rows, d);           \
+    if (vectors && d <= 1024)                                                                               \
+      add_rmsnorm_vec_kernel<TD, TO, 1><<<n_rows, 256, 0, stream>>>(h, (const TD*)delta0, (const TD*)delta1, \
+                                                                    weight, eps, (TO*)out, rows, d);        \
+    else if (vectors && d <= 2048)                                                                          \
+      add_rmsnorm_vec_kernel<TD, TO, 2><<<n_rows, 256, 0, stream>>>(h, (const TD*)delta0, (const TD*)delta1, \
+                                                                    weight, eps, (TO*)out, rows, d);        \
+    else if (vectors && d <= 4096)                                                                          \
+      add_rmsnorm_vec_kernel<TD, TO, 4><<<n_rows, 256, 0, stream>>>(h, (const TD*)delta0, (const TD*)delta1, \
+                                                                    weight, eps, (TO*)out, rows, d);        \
+    else if (vectors)                                                                                       \
+      add_rmsnorm_vec_kernel<TD, TO, NORM_MAX_ROUNDS><<<n_rows, 256, 0, stream>>>(                          \
+          h, (const TD*)delta0, (const TD*)delta1, weight, eps, (TO*)out, rows, d);                         \
     else                                                                                                    \
       add_rmsnorm_kernel<TD, TO><<<n_rows, 256, lds, stream>>>(h, (const TD*)delta0, (const TD*)delta1,     \
                                                                weight, eps, (TO*)out, rows, d);             \
