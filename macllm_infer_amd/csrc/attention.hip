@@ -615,7 +615,10 @@ extern "C" int mi_prefill_attention(const void* q, long q_ld, int Hq, int Hkv, i
   const int G = Hq / Hkv;
   if ((dh != 64 && dh != 128) || page_size % 4 != 0 || q_ld % 8 != 0 || out_ld % 4 != 0 || Hkv > 65535 || G > 64)
     return ERR_UNSUPPORTED_SIZE;
-  const int passes = (G + 3) / 4;
+  // up to four query heads share every K and V fragment; head size 128 holds twice the registers per head, and
+  // more than two heads would spill
+  const int most = dh == 128 ? 2 : 4;
+  const int passes = (G + most - 1) / most;
   const int nset = (G + passes - 1) / passes;
   if (n_tiles > (1 << 28)) return ERR_UNSUPPORTED_SIZE;
   const dim3 grid(4 * n_tiles, Hkv, passes);
