@@ -267,9 +267,10 @@ class ParallelFusion:
         normed = block.mixer_norm.forward(residual)
         u = ops.linear(normed, self.w_in_wide, self.b_in_wide)
         mixed = torch.empty((u.shape[0], self.mixed_width), dtype=u.dtype, device=u.device)
-        if u.shape[0] >= OVERLAP_MIN_TOKENS:
+        if u.shape[0] >= OVERLAP_MIN_TOKENS and torch.cuda.is_current_stream_capturing():
             # the two mixers read the same rows and write different columns: attention runs on a second
-            # stream beside the state-space chain, whose kernels are many and small
+            # stream beside the state-space chain, whose kernels are many and small (in a captured graph
+            # only: launched one by one the step waits for the host, which the second stream costs more)
             main = torch.cuda.current_stream(u.device)
             side = _side_stream(u.device)
             side.wait_stream(main)
