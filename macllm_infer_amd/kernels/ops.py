@@ -120,7 +120,13 @@ def _p(tensor: Optional[torch.Tensor]):
     return None if tensor is None else tensor.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)      # the handle without a Stream object around it
+
+
 def _stream():
+    """The current HIP stream of the current device, as the integer the launchers take."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
