@@ -2,12 +2,19 @@
 MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|f32] [--layers L]
+    python bench.py --workload serving [--shape 0.5b|7b|34b]
 
 One JSON line: ``value`` = decoded tokens a second at batch 8 with every request at a
 2,048-token context (a step = one decode step of the whole batch: model, greedy sampling,
 tokens fed back); ``prefill`` = one 2,048-token prompt in one step; ``roofline`` = the bytes
 the decode step has to read (every weight it uses once, and the cache and state of the live
 requests) over its time, against 8 TB/s; ``points`` = decode at batch 1 and 64.
+
+``--workload serving`` runs whole requests through the scheduler and the sampler instead
+(``LLM.generate``): for the 7B shape (and the 0.5B one) 64 requests with prompt lengths uniform in
+[128, 4096] and 256 greedy tokens each, prompts cut into portions of 2,048 tokens; for the 34B
+shape 8 prompts of 8,192 tokens and 128 greedy tokens each.  Its line reports prompt and generated
+tokens a second over the whole run and the spread of the rounds' times.
 """
 import argparse
 import json
@@ -37,6 +44,65 @@ SHAPES = {
 }
 CONTEXT = 2048
 PREFILL_TOKENS = 2048
+# whole-request workloads (--workload serving): requests, prompt lengths (lowest, highest), new tokens
+SERVING = {"0.5b": (64, 128, 4096, 256), "7b": (64, 128, 4096, 256), "34b": (8, 8192, 8192, 128)}
+SERVING_PORTION = 2048
+
+
+def serving(args, shape) -> int:
+    """Whole requests through the scheduler: admission, portions of prompts beside decoded tokens,
+    sampling, finishing."""
+    import torch
+    from macllm_infer_amd import LLM, Engine, EngineConfig, SamplingParams
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.weights.random_init import random_tensors
+
+    requests, shortest, longest, new_tokens = SERVING[args.shape]
+    layers = args.layers or shape["num_hidden_layers"]
+    raw = dict(shape, num_hidden_layers=layers, max_position_embeddings=longest + new_tokens)
+    config = FalconH1Config.from_dict(raw)
+    storage = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    tensors = random_tensors(config, 0, storage, "baseline", device="cpu" if args.shape == "0.5b" else "cuda:0")
+    generator = torch.Generator().manual_seed(0)
+    lengths = torch.randint(shortest, longest + 1, (requests,), generator=generator).tolist()
+    prompts = [torch.randint(0, config.vocab_size, (length,), generator=generator).tolist() for length in lengths]
+    capacity = sum(-(-(length + new_tokens) // 64) * 64 for length in lengths)
+    engine = Engine(config=config, tensors=tensors, dtype="bfloat16" if args.dtype == "bf16" else "float32",
+                    kv_cache_block_tokens=args.page_tokens, kv_cache_capacity_tokens=capacity,
+                    max_active_sequences=requests)
+    del tensors
+    llm = LLM(engine, engine_config=EngineConfig(max_active_sequences=requests, prefill_token_quantum=SERVING_PORTION,
+                                                 scheduler_token_budget=SERVING_PORTION + requests))
+    params = SamplingParams(max_new_tokens=new_tokens, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
+                            ignore_eos=True)
+    runs = []
+    for repeat in range(2):                      # the first run captures the graphs of the repeating shapes
+        round_times = []
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        results = llm.generate(prompts, params, on_round=round_times.append)
+        torch.cuda.synchronize()
+        runs.append((time.perf_counter() - started, results, sorted(round_times)))
+    seconds, results, round_times = runs[-1]
+    generated = sum(result.generated_tokens for result in results)
+    assert all(result.finish_reason == "length" for result in results), "a request did not run to its length"
+    first = sorted(result.time_to_first_token for result in results)
+    pick = lambda values, fraction: values[min(len(values) - 1, int(fraction * len(values)))]
+    print(json.dumps({
+        "metric": "generated tok/s over whole requests (scheduler, portions of prompts beside decoded tokens)",
+        "value": round(generated / seconds, 1), "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True,
+        "dtype": args.dtype, "data": "synthetic", "seconds": round(seconds, 3), "first_run_seconds": round(runs[0][0], 3),
+        "prompt_tokens": sum(lengths), "generated_tokens": generated,
+        "all_tokens_per_second": round((sum(lengths) + generated) / seconds, 1),
+        "rounds": len(round_times), "round_ms": {"mean": round(1e3 * sum(round_times) / len(round_times), 3),
+                                                 "p50": round(1e3 * pick(round_times, 0.5), 3),
+                                                 "p95": round(1e3 * pick(round_times, 0.95), 3)},
+        "first_token_s": {"p50": round(pick(first, 0.5), 3), "p95": round(pick(first, 0.95), 3)},
+        "config": {"model": f"falcon-h1-{args.shape}-shaped, random weights", "layers": layers,
+                   "layers_of_configuration": shape["num_hidden_layers"], "requests": requests,
+                   "prompt_tokens_lowest": shortest, "prompt_tokens_highest": longest, "new_tokens": new_tokens,
+                   "portion": SERVING_PORTION, "page_tokens": args.page_tokens, "sampling": "greedy"}}))
+    return 0
 
 
 def main() -> int:
@@ -54,10 +120,14 @@ def main() -> int:
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only the 2,048-token prefill (for profiles; the line then reports prefill tokens/s)")
+    parser.add_argument("--workload", default="steps", choices=["steps", "serving"],
+                        help="steps: the headline decode and prefill steps; serving: whole requests through the scheduler")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
         return 2
+    if args.workload == "serving":
+        return serving(args, SHAPES[args.shape])
 
     import torch
     from macllm_infer_amd import Engine, Lane

@@ -39,13 +39,22 @@ class GenerationResult:
 class LLM:
     """A loaded model with its cache, sampler and scheduler settings."""
 
-    def __init__(self, model: str, dtype: str = "bfloat16", device: str = "cuda:0",
+    def __init__(self, model: Union[str, Engine], dtype: str = "bfloat16", device: str = "cuda:0",
                  kv_cache_block_tokens: int = 16, kv_cache_capacity_tokens: Optional[int] = None,
                  engine_config: Optional[EngineConfig] = None):
+        """``model``: a folder with config.json and model.safetensors, or an ``Engine`` that is
+        already built (its own dtype and cache sizes then hold; it needs a state slot for each of
+        ``engine_config.max_active_sequences``)."""
         self.engine_config = engine_config or EngineConfig()
-        self.engine = Engine(model, dtype=dtype, device=device, kv_cache_block_tokens=kv_cache_block_tokens,
-                             kv_cache_capacity_tokens=kv_cache_capacity_tokens,
-                             max_active_sequences=self.engine_config.max_active_sequences)
+        if isinstance(model, Engine):
+            self.engine = model
+            if self.engine.cache.slots.total < self.engine_config.max_active_sequences:
+                raise ValueError(f"the engine has {self.engine.cache.slots.total} state slots, fewer than "
+                                 f"max_active_sequences = {self.engine_config.max_active_sequences}")
+        else:
+            self.engine = Engine(model, dtype=dtype, device=device, kv_cache_block_tokens=kv_cache_block_tokens,
+                                 kv_cache_capacity_tokens=kv_cache_capacity_tokens,
+                                 max_active_sequences=self.engine_config.max_active_sequences)
         self.sampler = Sampler(self.engine.vocab_size, self.engine.device)
         eos = getattr(self.engine.config, "eos_token_id", None)
         self.stop_token_ids = () if eos is None else (eos,)
@@ -53,10 +62,11 @@ class LLM:
 
     def generate(self, prompts: Sequence[Sequence[int]],
                  sampling_params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
-                 on_token=None) -> List[GenerationResult]:
+                 on_token=None, on_round=None) -> List[GenerationResult]:
         """``prompts``: token ids of each request.  One ``SamplingParams`` for all, or one per
         prompt; with a single one, request i samples with ``seed + i`` (the reference offsets
-        its seed per request the same way, src/main.rs:188-197)."""
+        its seed per request the same way, src/main.rs:188-197).  ``on_token(request, token)`` is
+        called for every emitted token, ``on_round(seconds)`` after every round of the scheduler."""
         if sampling_params is None:
             sampling_params = SamplingParams()
         if isinstance(sampling_params, SamplingParams):
@@ -74,7 +84,7 @@ class LLM:
             self._next_id += 1
             ids.append(request_id)
             scheduler.submit(request_id, prompt, params)
-        finished = scheduler.run()
+        finished = scheduler.run(on_round)
         results = []
         for request_id in ids:
             request: Request = finished[request_id]

@@ -195,8 +195,11 @@ class Scheduler:
         if len(request.generated) >= params.max_new_tokens:
             self._finish(request, "length")
 
-    def run(self) -> Dict[Hashable, Request]:
-        """Rounds until every submitted request has finished."""
+    def run(self, on_round: Optional[Callable] = None) -> Dict[Hashable, Request]:
+        """Rounds until every submitted request has finished; ``on_round(seconds)`` after each."""
         while self.has_work():
+            started = time.perf_counter()
             self.step()
+            if on_round is not None:
+                on_round(time.perf_counter() - started)
         return self.finished
