@@ -18,6 +18,11 @@ from .spec import (AttentionSpec, ConfigError, LayerSpec, Mamba2Spec, MixerSlot,
 
 _MISSING = object()
 
+# The names of the reference's table (src/architecture.rs:1595-1647) are the model's own; these
+# are the other spelling of the same tensors in checkpoints of the family.
+TENSOR_ALIASES = ((".input_layernorm.", ".attn_norm."), (".pre_ff_layernorm.", ".ffn_norm."),
+                  (".feed_forward.", ".mlp."), ("model.final_layernorm.", "model.norm."))
+
 
 @dataclass(frozen=True)
 class FalconH1Config:
@@ -232,6 +237,7 @@ class FalconH1Config:
             tied_embeddings=self.tie_word_embeddings,
             embedding_multiplier=self.embedding_multiplier,
             logit_multiplier=self.lm_head_multiplier,
+            tensor_aliases=TENSOR_ALIASES,
         )
 
     # ------------------------------------------------------------------ reports

@@ -203,6 +203,11 @@ class ModelSpec:
     embedding_name: str = "model.embed_tokens"
     final_norm_name: str = "model.norm"
     lm_head_name: str = "lm_head"
+    # other spellings under which checkpoints of this architecture store the same tensors:
+    # (piece of a stored name, the piece it stands for here)
+    tensor_aliases: Tuple[Tuple[str, str], ...] = ()
+    # a checkpoint none of whose names starts with this gets it in front of all but the output head's
+    root_namespace: str = "model."
 
     def validate(self) -> None:
         """Positivity, divisibility and bounds, field by field (src/architecture.rs:367-452)."""

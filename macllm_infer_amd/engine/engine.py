@@ -63,6 +63,7 @@ class Engine:
         self.spec.validate()
         if check_device:
             kernel_build.ensure_modules(DecoderModel.kernel_modules(self.spec))
+        source.apply_aliases(self.spec.tensor_aliases, root_prefix=self.spec.root_namespace)
         bound = bind(source, DecoderModel.expected_tensors(self.spec))
         source.close()
         build = BuildContext(hidden_size=self.spec.hidden_size, dtype=self.dtype, device=self.device,

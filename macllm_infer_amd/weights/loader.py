@@ -62,9 +62,35 @@ class WeightSource:
     def __init__(self, files: Sequence[SafetensorsFile]):
         self._files = list(files)
         self._where: Dict[str, SafetensorsFile] = {}
+        self._stored: Dict[str, str] = {}                 # name as asked for -> name in the file
+        self.clashes: List[Tuple[str, str]] = []          # (stored name, the stored name it doubles)
         for handle in self._files:
             for name in handle.names():
                 self._where[name] = handle
+                self._stored[name] = name
+
+    def apply_aliases(self, aliases: Sequence[Tuple[str, str]], root_prefix: str = "") -> None:
+        """Let tensors stored under another spelling answer to the model's names.  ``aliases``:
+        (other spelling, the model's spelling) of a piece of a name, e.g. (".feed_forward.",
+        ".mlp.") (the alias table idea of src/gguf.rs:1786-1813).  ``root_prefix``: if no stored
+        name starts with it, every stored name but the output head's gets it in front: a
+        checkpoint saved from the inner model has ``layers.0...`` for ``model.layers.0...``
+        (namespace choice of src/decoder.rs:2987-2995).  A tensor stored under two spellings is
+        reported by ``bind`` as unexpected."""
+        rooted = bool(root_prefix) and not any(name.startswith(root_prefix) for name in self._where)
+        renamed: Dict[str, str] = {}
+        for stored in sorted(self._where):
+            name = stored
+            if rooted and not name.startswith("lm_head"):
+                name = root_prefix + name
+            for other, ours in aliases:
+                if other in name:
+                    name = name.replace(other, ours)
+            if name in renamed:
+                self.clashes.append((stored, renamed[name]))
+            else:
+                renamed[name] = stored
+        self._stored = renamed
 
     @classmethod
     def from_dir(cls, model_dir: str) -> "WeightSource":
@@ -83,16 +109,22 @@ class WeightSource:
         return cls([_MemoryFile(tensors)])
 
     def names(self):
-        return self._where.keys()
+        return self._stored.keys()
+
+    def stored_name(self, name: str) -> str:
+        return self._stored[name]
 
     def shape(self, name: str):
-        return self._where[name].shape(name)
+        stored = self._stored[name]
+        return self._where[stored].shape(stored)
 
     def dtype(self, name: str):
-        return self._where[name].dtype(name)
+        stored = self._stored[name]
+        return self._where[stored].dtype(stored)
 
     def tensor(self, name: str) -> torch.Tensor:
-        return self._where[name].tensor(name)
+        stored = self._stored[name]
+        return self._where[stored].tensor(stored)
 
     def close(self) -> None:
         for handle in self._files:
@@ -127,7 +159,8 @@ def bind(source: WeightSource, expectations: Sequence[Expect]) -> Dict[str, torc
         wanted[expect.name] = expect                      # a name asked for twice (tied weights) is one tensor
     present = set(source.names())
     missing = sorted(name for name in wanted if name not in present)
-    unexpected = sorted(name for name in present if name not in wanted)
+    unexpected = sorted(source.stored_name(name) for name in present if name not in wanted)
+    unexpected += [f"{stored} (the same tensor as {other})" for stored, other in source.clashes]
     wrong_shape: List[Tuple[str, Tuple, Tuple]] = []
     wrong_dtype: List[Tuple[str, str]] = []
     for name, expect in wanted.items():

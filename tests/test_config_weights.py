@@ -166,3 +166,47 @@ def test_sharded_checkpoint(tmp_path):
     (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": weight_map}))
     bound = bind(WeightSource.from_dir(str(tmp_path)), DecoderModel.expected_tensors(config.to_model_spec()))
     assert all(torch.equal(bound[n], tensors[n]) for n in names)
+
+
+def _respell(tensors, pairs, strip=""):
+    out = {}
+    for name, tensor in tensors.items():
+        for ours, other in pairs:
+            name = name.replace(ours, other)
+        if strip and name.startswith(strip):
+            name = name[len(strip):]
+        out[name] = tensor
+    return out
+
+
+CHECKPOINT_SPELLING = ((".attn_norm.", ".input_layernorm."), (".ffn_norm.", ".pre_ff_layernorm."),
+                       (".mlp.", ".feed_forward."), ("model.norm.", "model.final_layernorm."))
+
+
+def test_the_other_spelling_of_the_tensor_names_binds_to_the_same_tensors():
+    config = tiny_configs.config("B")
+    spec = config.to_model_spec()
+    tensors = random_tensors(config, 3, torch.float32, "unit")
+    plain = bind(WeightSource.from_tensors(tensors), DecoderModel.expected_tensors(spec))
+    for strip in ("", "model."):                   # with the namespace, and saved from the inner model
+        source = WeightSource.from_tensors(_respell(tensors, CHECKPOINT_SPELLING, strip))
+        assert "model.layers.0.input_layernorm.weight"[len(strip):] in source.names()
+        source.apply_aliases(spec.tensor_aliases, root_prefix=spec.root_namespace)
+        bound = bind(source, DecoderModel.expected_tensors(spec))
+        assert bound.keys() == plain.keys()
+        assert all(torch.equal(bound[name], plain[name]) for name in plain)
+
+
+def test_a_tensor_under_both_spellings_and_a_stranger_are_reported_by_their_stored_names():
+    config = tiny_configs.config("A")
+    spec = config.to_model_spec()
+    tensors = _respell(random_tensors(config, 3, torch.float32, "unit"), CHECKPOINT_SPELLING)
+    tensors["model.layers.1.ffn_norm.weight"] = tensors["model.layers.1.pre_ff_layernorm.weight"]
+    tensors["model.layers.0.feed_forward.router.weight"] = torch.zeros(2, 2)
+    source = WeightSource.from_tensors(tensors)
+    source.apply_aliases(spec.tensor_aliases, root_prefix=spec.root_namespace)
+    with pytest.raises(WeightError) as caught:
+        bind(source, DecoderModel.expected_tensors(spec))
+    assert not caught.value.missing
+    assert "model.layers.0.feed_forward.router.weight" in caught.value.unexpected
+    assert any("pre_ff_layernorm" in name and "ffn_norm" in name for name in caught.value.unexpected)
