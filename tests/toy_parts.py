@@ -1,5 +1,6 @@
 """Toy parts for the tests of the framework's generality: a mixer with state of its own, a
-position encoding that is no rotation, and a toy architecture that uses them together with a
+position encoding that is no rotation, a feed-forward that routes each token to two of its
+experts, and a toy architecture that uses them together with a
 windowed attention layer, a layer that runs twice and a run that reads another run's cache.
 They are registered from here, without a change to the package, and never become a model."""
 from dataclasses import dataclass
@@ -29,10 +30,23 @@ class AlibiLikeSpec:
         pass
 
 
+@dataclass(frozen=True)
+class RoutedSpec:
+    """A toy feed-forward with routing: a float32 router picks each token's two best experts
+    (ties to the lower index), weighs them by the softmax of their two logits, and each expert
+    is down(relu(up(x)))."""
+    experts: int
+    inner: int
+    kind: str = "toy_routed"
+
+    def validate(self):
+        assert self.experts >= 2 and self.inner > 0
+
+
 @dataclass
 class ToyConfig:
     """A toy architecture: layer 0 = attention (toy position encoding) and the decay mixer in
-    parallel, layer 1 = windowed attention with partial RoPE.  ``raw["schedule"]`` lists
+    parallel, layer 1 = windowed attention with partial RoPE and the routed feed-forward.  ``raw["schedule"]`` lists
     (layer, entry whose cache is read or None) in running order."""
     raw: dict
     architecture_names = ("ToyForTests",)
@@ -57,7 +71,7 @@ class ToyConfig:
         ffn = SwiGLUSpec(intermediate_size=48)
         layers = (LayerSpec(prefix="model.layers.0", ffn=ffn, mixer_norm=norm, ffn_norm=norm,
                             mixers=(MixerSlot("self_attn", full), MixerSlot("decay", DecayMixerSpec(hidden, raw["decay"])))),
-                  LayerSpec(prefix="model.layers.1", ffn=ffn, mixer_norm=norm, ffn_norm=norm,
+                  LayerSpec(prefix="model.layers.1", ffn=RoutedSpec(raw["experts"], 24), mixer_norm=norm, ffn_norm=norm,
                             mixers=(MixerSlot("self_attn", windowed),)))
         schedule = tuple(ScheduleEntry(layer=layer, kv_from=source) for layer, source in raw["schedule"])
         return ModelSpec(architecture="ToyForTests", hidden_size=hidden, vocab_size=raw["vocab"], max_context=512,
@@ -67,7 +81,7 @@ class ToyConfig:
 def register_toys():
     from macllm_infer_amd.cache import StateNeed
     from macllm_infer_amd.config import register_architecture
-    from macllm_infer_amd.parts import Mixer, PositionEncoding, register_part
+    from macllm_infer_amd.parts import FeedForward, Mixer, PositionEncoding, register_part
     from macllm_infer_amd.weights import Expect
 
     @register_part("toy_decay")
@@ -111,7 +125,35 @@ def register_toys():
             width = (num_heads + num_kv_heads) * head_dim
             qkv[:, :width] = (qkv[:, :width].float() * factor).to(qkv.dtype)
 
+    @register_part("toy_routed")
+    class Routed(FeedForward):
+        @classmethod
+        def expected_tensors(cls, spec, prefix, hidden_size):
+            return [Expect(f"{prefix}.router.weight", ((spec.experts, hidden_size),)),
+                    Expect(f"{prefix}.up.weight", ((spec.experts, spec.inner, hidden_size),)),
+                    Expect(f"{prefix}.down.weight", ((spec.experts, hidden_size, spec.inner),))]
+
+        def __init__(self, spec, prefix, tensors, build):
+            self.router, self.up, self.down = (tensors[f"{prefix}.{name}.weight"].float().to(build.device)
+                                               for name in ("router", "up", "down"))
+
+        def forward(self, x):
+            return routed_feed_forward(x.float(), self.router, self.up, self.down).to(x.dtype)
+
     register_architecture(ToyConfig)
+
+
+def routed_feed_forward(x, router, up, down):
+    """Each token through its two best experts; a token's result depends on that token alone."""
+    logits = x @ router.T
+    best = torch.sort(logits, dim=-1, descending=True, stable=True).indices[:, :2]
+    weights = torch.softmax(torch.gather(logits, 1, best), dim=-1)
+    out = torch.zeros_like(x)
+    for rank in range(2):
+        chosen = best[:, rank]
+        hidden = torch.relu(torch.einsum("td,tid->ti", x, up[chosen]))
+        out += weights[:, rank:rank + 1] * torch.einsum("ti,tdi->td", hidden, down[chosen])
+    return out
 
 
 def toy_plain_logits(raw, tensors, tokens):
@@ -151,8 +193,22 @@ def toy_plain_logits(raw, tensors, tokens):
             mixed = mixed + torch.stack(rows)
         h = h + mixed
         f = plain_impl.rms_norm(h, tensors[p + "ffn_norm.weight"], 1e-5)
-        h = h + plain_impl.swiglu_mlp(f, {name[len(p + "mlp."):]: value for name, value in tensors.items()
-                                          if name.startswith(p + "mlp.")})
+        if layer == 0:
+            h = h + plain_impl.swiglu_mlp(f, {name[len(p + "mlp."):]: value for name, value in tensors.items()
+                                              if name.startswith(p + "mlp.")})
+        else:                                           # token by token, expert by expert
+            router, up, down = (tensors[p + f"mlp.{name}.weight"].float() for name in ("router", "up", "down"))
+            rows = []
+            for t in range(T):
+                logits = router @ f[t]
+                first = int(torch.argmax(logits))
+                rest = logits.clone()
+                rest[first] = float("-inf")
+                second = int(torch.argmax(rest))
+                gate = torch.softmax(torch.stack([logits[first], logits[second]]), dim=0)
+                rows.append(sum(gate[rank] * (down[expert] @ torch.relu(up[expert] @ f[t]))
+                                for rank, expert in enumerate((first, second))))
+            h = h + torch.stack(rows)
     h = plain_impl.rms_norm(h, tensors["model.norm.weight"], 1e-5)
     return h @ tensors["model.embed_tokens.weight"].float().T
 
@@ -175,10 +231,10 @@ def exercise(schedule, device, check_device):
     from macllm_infer_amd.weights.random_init import random_tensors
     register_toys()
     raw = {"architectures": ["ToyForTests"], "hidden": 32, "vocab": 90, "slope": 0.01, "decay": 0.9, "window": 13,
-           "schedule": schedule}
+           "experts": 5, "schedule": schedule}
     config = ToyConfig(raw)
     tensors = random_tensors(config, 5, torch.float32, "unit")
-    assert "model.layers.0.decay.w.weight" in tensors
+    assert "model.layers.0.decay.w.weight" in tensors and tensors["model.layers.1.mlp.up.weight"].shape == (5, 24, 32)
     engine = Engine(config=config, tensors=tensors, dtype="float32", device=device, kv_cache_block_tokens=4,
                     kv_cache_capacity_tokens=160, max_active_sequences=3, check_device=check_device)
     windows = sorted(str(group.need.window) for group in engine.cache.groups)
