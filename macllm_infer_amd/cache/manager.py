@@ -18,8 +18,10 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
+from . import native
 from .pages import BlockTable, CacheExhausted, PagePool, SlotPool
 
 
@@ -40,14 +42,38 @@ class StateNeed:
     dtype: str = "float32"
 
 
+class Core:
+    """The host-side core of one cache manager (``csrc/hostcore.cpp``): every group's page pool
+    and block tables, the slot pool and the requests' lengths."""
+
+    def __init__(self, page_sizes: Sequence[int], num_pages: Sequence[int], windows: Sequence[Optional[int]],
+                 max_requests: int):
+        self.lib = native.lib()
+        sizes, pages = native.as_ints(list(page_sizes)), native.as_ints(list(num_pages))
+        spans = native.as_ints([window or -1 for window in windows])
+        self.pointer = self.lib.hc_create(len(sizes), native.int_pointer(sizes), native.int_pointer(pages),
+                                          native.int_pointer(spans), max_requests)
+        if not self.pointer:
+            raise ValueError("page sizes, page counts and the number of requests must be positive")
+
+    def __del__(self):
+        if getattr(self, "pointer", None):
+            self.lib.hc_destroy(self.pointer)
+            self.pointer = None
+
+
 class PagedGroup:
+    """The layers with one ``KVNeed``: their storage, and a view of the group's pool and tables
+    in the core."""
+
     def __init__(self, need: KVNeed, page_size: int, num_pages: int):
         self.need = need
         self.page_size = page_size
-        self.pool = PagePool(num_pages)
+        self.num_pages = num_pages
         self.members: List[Hashable] = []
         self.tables: Dict[Hashable, BlockTable] = {}
         self.storage: Optional[torch.Tensor] = None
+        self.pool: Optional[PagePool] = None          # set once the core exists
 
     def add_member(self, key: Hashable) -> int:
         self.members.append(key)
@@ -56,12 +82,12 @@ class PagedGroup:
     def allocate(self, dtype: torch.dtype, device) -> None:
         need = self.need
         # one page more than the pool hands out: the scratch page padding lanes of a captured step write to
-        self.storage = torch.zeros((self.pool.total + 1, len(self.members), 2, need.num_kv_heads,
+        self.storage = torch.zeros((self.num_pages + 1, len(self.members), 2, need.num_kv_heads,
                                     self.page_size * need.head_dim), dtype=dtype, device=device)
 
     @property
     def scratch_page(self) -> int:
-        return self.pool.total
+        return self.num_pages
 
     def layer_views(self, layer: int):
         """One layer's K pages [pages, Hkv, page_size, dh] and V pages [pages, Hkv, dh, page_size]
@@ -74,47 +100,22 @@ class PagedGroup:
         need = self.need
         return 2 * len(self.members) * need.num_kv_heads * self.page_size * need.head_dim * element_size
 
-    # -- per request
-    def pages_missing(self, request: Hashable, new_length: int) -> int:
-        table = self.tables[request]
-        wanted = -(-new_length // self.page_size)
-        return max(0, wanted - len(table.pages))
-
-    def grow(self, request: Hashable, new_length: int) -> None:
-        table = self.tables[request]
-        table.pages.extend(self.pool.alloc(self.pages_missing(request, new_length)))
-
-    def release_passed(self, request: Hashable, length: int) -> None:
-        """Give back the pages every later query is past: with a window w the next query
-        (position ``length``) sees keys >= length - w + 1."""
-        window = self.need.window
-        if window is None:
-            return
-        table = self.tables[request]
-        first_needed_key = length - window + 1
-        if first_needed_key <= 0:
-            return
-        first_needed_page = min(first_needed_key // self.page_size, len(table.pages))
-        passed = [table.pages[index] for index in range(table.first_live, first_needed_page)]
-        if passed:
-            self.pool.free(passed)
-            for index in range(table.first_live, first_needed_page):
-                table.pages[index] = -1
-            table.first_live = first_needed_page
-
-    def release_all(self, request: Hashable) -> None:
-        table = self.tables.pop(request)
-        self.pool.free(table.live_pages())
-
     def check(self) -> None:
         held = [page for table in self.tables.values() for page in table.live_pages()]
         self.pool.check(held)
 
 
 class RequestCache:
-    def __init__(self, slot: int):
+    """A live request: its state slot (which is also its handle in the core) and its length."""
+
+    def __init__(self, core: Core, slot: int):
+        self._core = core
         self.slot = slot
-        self.length = 0          # tokens whose keys, values and state are in the cache
+
+    @property
+    def length(self) -> int:
+        """Tokens whose keys, values and state are in the cache."""
+        return self._core.lib.hc_length(self._core.pointer, self.slot)
 
 
 @dataclass
@@ -142,7 +143,7 @@ class CacheManager:
         num_pages = -(-capacity_tokens // page_size)
         self.groups: List[PagedGroup] = []
         self.entries: Dict[Hashable, EntryCache] = {}
-        self.slots = SlotPool(max_requests)
+        self.max_requests = max_requests
         self.requests: Dict[Hashable, RequestCache] = {}
         self._state_tensors: List[torch.Tensor] = []
         group_of: Dict[KVNeed, int] = {}
@@ -168,7 +169,11 @@ class CacheManager:
                 else:
                     raise TypeError(f"unknown cache need {need!r}")
             self.entries[key] = entry
-        for group in self.groups:
+        self.core = Core([group.page_size for group in self.groups], [group.num_pages for group in self.groups],
+                         [group.need.window for group in self.groups], max_requests)
+        self.slots = SlotPool.view(self.core.lib.hc_slot_pool(self.core.pointer), self.core)
+        for index, group in enumerate(self.groups):
+            group.pool = PagePool.view(self.core.lib.hc_group_pool(self.core.pointer, index), self.core)
             group.allocate(dtype, self.device)
         for key, entry in self.entries.items():
             source = shared_kv.get(key, key)
@@ -187,17 +192,19 @@ class CacheManager:
 
     @property
     def scratch_slot(self) -> int:
-        return self.slots.total
+        return self.max_requests
 
     # ------------------------------------------------------------------ requests
     def add_request(self, request: Hashable) -> RequestCache:
         if request in self.requests:
             raise KeyError(f"request {request!r} is already live")
-        slot = self.slots.alloc()
-        record = RequestCache(slot)
+        slot = self.core.lib.hc_add_request(self.core.pointer)
+        if slot < 0:
+            raise CacheExhausted("state slots", 1, 0, self.max_requests)
+        record = RequestCache(self.core, slot)
         self.requests[request] = record
-        for group in self.groups:
-            group.tables[request] = BlockTable()
+        for index, group in enumerate(self.groups):
+            group.tables[request] = BlockTable(self.core, index, slot)
         if self._state_tensors:                       # a fresh request starts from zeros
             torch._foreach_zero_([tensor[slot] for tensor in self._state_tensors])
         return record
@@ -205,35 +212,51 @@ class CacheManager:
     def can_ever_fit(self, total_tokens: int) -> bool:
         """Whether a request of ``total_tokens`` fits an empty cache
         (the admission check of src/engine.rs:2839-2863)."""
-        return all(-(-total_tokens // group.page_size) <= group.pool.total for group in self.groups)
+        return all(-(-total_tokens // group.page_size) <= group.num_pages for group in self.groups)
+
+    def slots_of(self, requests: Sequence[Hashable]) -> np.ndarray:
+        """The core's handles of live requests (KeyError for one that is not live)."""
+        records = self.requests
+        try:
+            return np.fromiter((records[request].slot for request in requests), dtype=np.int32, count=len(requests))
+        except KeyError as error:
+            raise KeyError(f"request {error.args[0]!r} is not live") from None
+
+    def lengths_of(self, slots: np.ndarray) -> np.ndarray:
+        out = np.empty(len(slots), dtype=np.int32)
+        self.core.lib.hc_lengths(self.core.pointer, len(slots), native.int_pointer(slots), native.int_pointer(out))
+        return out
 
     def reserve(self, growth: Sequence[Tuple[Hashable, int]]) -> None:
         """Pages for ``tokens`` more tokens of every listed request, all or nothing."""
-        for request, tokens in growth:
-            if request not in self.requests:
-                raise KeyError(f"request {request!r} is not live")
-            if tokens <= 0:
-                raise ValueError("a lane needs at least one token")
-        for group in self.groups:
-            missing = sum(group.pages_missing(request, self.requests[request].length + tokens)
-                          for request, tokens in growth)
-            if missing > group.pool.free_count:
-                raise CacheExhausted("pages", missing, group.pool.free_count, group.pool.total)
-        for group in self.groups:
-            for request, tokens in growth:
-                group.grow(request, self.requests[request].length + tokens)
+        self.reserve_slots(self.slots_of([request for request, _ in growth]),
+                           native.as_ints([tokens for _, tokens in growth]))
+
+    def reserve_slots(self, slots: np.ndarray, tokens: np.ndarray) -> None:
+        info = np.zeros(4, dtype=np.int32)
+        code = self.core.lib.hc_reserve(self.core.pointer, len(slots), native.int_pointer(slots),
+                                        native.int_pointer(tokens), native.int_pointer(info))
+        if code == 1:
+            raise CacheExhausted("pages", int(info[1]), int(info[2]), int(info[3]))
+        if code != 0:
+            raise ValueError(f"lane {int(info[0])} of the reservation: a request named twice, or no tokens")
 
     def commit(self, request: Hashable, tokens: int) -> None:
-        record = self.requests[request]
-        record.length += tokens
-        for group in self.groups:
-            group.release_passed(request, record.length)
+        self.commit_slots(self.slots_of([request]), native.as_ints([tokens]))
+
+    def commit_slots(self, slots: np.ndarray, tokens: np.ndarray) -> None:
+        """The step ran: lengths advance and window groups give back the pages all later queries
+        are past."""
+        if self.core.lib.hc_commit(self.core.pointer, len(slots), native.int_pointer(slots),
+                                   native.int_pointer(tokens)) != 0:
+            raise RuntimeError("commit of a request that is not live, or broken page accounting")
 
     def finish(self, request: Hashable) -> None:
         record = self.requests.pop(request)
         for group in self.groups:
-            group.release_all(request)
-        self.slots.free(record.slot)
+            del group.tables[request]
+        if self.core.lib.hc_finish(self.core.pointer, record.slot) != 0:
+            raise RuntimeError(f"request {request!r}: its slot or pages were not held")
 
     # ------------------------------------------------------------------ views and reports
     def entry(self, key: Hashable) -> EntryCache:
@@ -245,12 +268,16 @@ class CacheManager:
     def stats(self) -> dict:
         return {
             "groups": [{"window": group.need.window, "layers": len(group.members),
-                        "total_pages": group.pool.total, "free_pages": group.pool.free_count,
+                        "total_pages": group.num_pages, "free_pages": group.pool.free_count,
                         "used_pages": group.pool.used_count} for group in self.groups],
-            "total_slots": self.slots.total, "free_slots": self.slots.free_count,
+            "total_slots": self.max_requests, "free_slots": self.slots.free_count,
             "live_requests": len(self.requests),
         }
 
     def check(self) -> None:
+        """No page lost, held twice or held by a request that is gone."""
         for group in self.groups:
             group.check()
+        code = self.core.lib.hc_check(self.core.pointer)
+        if code != 0:
+            raise AssertionError(f"page accounting of group {code - 1} is broken")

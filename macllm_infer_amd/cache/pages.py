@@ -5,10 +5,17 @@ nothing of tensors.  The reference's pool tracks Free / Reserved / Live / Retire
 with typed, side-effect-free exhaustion (crates/macllm-kv/src/cache.rs:294-299,
 :649-658); with one stream every later kernel is ordered after the earlier ones, so a
 page is reusable as soon as it is freed and two states are enough.
+
+The pools and tables themselves live in the host-side core (``csrc/hostcore.cpp``); the
+classes here are views of them.
 """
 from __future__ import annotations
 
-from typing import Dict, List
+from typing import List
+
+import numpy as np
+
+from . import native
 
 
 class CacheExhausted(RuntimeError):
@@ -22,88 +29,97 @@ class CacheExhausted(RuntimeError):
 
 class PagePool:
     """``total`` page ids 0..total-1.  The most recently freed page is handed out first,
-    so a small pool reuses pages at once."""
+    so a small pool reuses pages at once.  ``PagePool(total)`` makes a pool of its own;
+    ``PagePool.view(pointer, owner)`` looks at one inside a cache core."""
+    what = "pages"
 
     def __init__(self, total: int):
         if total <= 0:
-            raise ValueError("a page pool needs at least one page")
-        self.total = total
-        self._free: List[int] = list(range(total - 1, -1, -1))
-        self._held = [False] * total
+            raise ValueError("a pool needs at least one id")
+        self._lib = native.lib()
+        self._pool = self._lib.hc_pool_create(total)
+        self._owner = None
+
+    @classmethod
+    def view(cls, pointer, owner):
+        pool = cls.__new__(cls)
+        pool._lib = native.lib()
+        pool._pool = pointer
+        pool._owner = owner                  # keeps the core alive
+        return pool
+
+    def __del__(self):
+        if getattr(self, "_owner", True) is None and getattr(self, "_pool", None):
+            self._lib.hc_pool_destroy(self._pool)
+            self._pool = None
+
+    @property
+    def total(self) -> int:
+        return self._lib.hc_pool_total(self._pool)
 
     @property
     def free_count(self) -> int:
-        return len(self._free)
+        return self._lib.hc_pool_free_count(self._pool)
 
     @property
     def used_count(self) -> int:
-        return self.total - len(self._free)
+        return self.total - self.free_count
 
     def alloc(self, count: int) -> List[int]:
         if count < 0:
-            raise ValueError("negative page count")
-        if count > len(self._free):
-            raise CacheExhausted("pages", count, len(self._free), self.total)
-        pages = [self._free.pop() for _ in range(count)]
-        for page in pages:
-            self._held[page] = True
-        return pages
+            raise ValueError("negative count")
+        out = np.empty(max(count, 1), dtype=np.int32)
+        if self._lib.hc_pool_take(self._pool, count, native.int_pointer(out)) != 0:
+            raise CacheExhausted(self.what, count, self.free_count, self.total)
+        return out[:count].tolist()
 
     def free(self, pages) -> None:
-        pages = list(pages)
-        for page in pages:
-            if not (0 <= page < self.total) or not self._held[page]:
-                raise RuntimeError(f"page {page} is freed but is not held")
-            self._held[page] = False
-        self._free.extend(pages)
+        ids = native.as_ints(list(pages))
+        if self._lib.hc_pool_give(self._pool, native.int_pointer(ids), len(ids)) != 0:
+            raise RuntimeError(f"one of the {self.what} {ids.tolist()} is freed but is not held")
 
     def check(self, held_elsewhere: List[int]) -> None:
-        """Every page is either free or in ``held_elsewhere``, exactly once
+        """Every id is either free or in ``held_elsewhere``, exactly once
         (the scan-based cross-check of crates/macllm-kv/src/cache.rs:3810-3841)."""
-        seen = sorted(self._free) + sorted(held_elsewhere)
-        if sorted(seen) != list(range(self.total)):
-            raise AssertionError("page accounting is broken: a page is lost or held twice")
-        for page in held_elsewhere:
-            if not self._held[page]:
-                raise AssertionError(f"page {page} is in a block table but marked free")
+        ids = native.as_ints(list(held_elsewhere))
+        code = self._lib.hc_pool_check(self._pool, native.int_pointer(ids), len(ids))
+        if code == 1:
+            raise AssertionError(f"accounting of {self.what} is broken: one is lost or held twice")
+        if code == 2:
+            raise AssertionError(f"one of the {self.what} is in a block table but marked free")
 
 
-class SlotPool:
+class SlotPool(PagePool):
     """Ids of the fixed-size per-request state slots."""
+    what = "state slots"
 
-    def __init__(self, total: int):
-        if total <= 0:
-            raise ValueError("a slot pool needs at least one slot")
-        self.total = total
-        self._free: List[int] = list(range(total - 1, -1, -1))
-        self._held = [False] * total
-
-    @property
-    def free_count(self) -> int:
-        return len(self._free)
-
-    def alloc(self) -> int:
-        if not self._free:
-            raise CacheExhausted("state slots", 1, 0, self.total)
-        slot = self._free.pop()
-        self._held[slot] = True
-        return slot
+    def alloc(self) -> int:                      # one slot at a time
+        return PagePool.alloc(self, 1)[0]
 
     def free(self, slot: int) -> None:
-        if not (0 <= slot < self.total) or not self._held[slot]:
-            raise RuntimeError(f"state slot {slot} is freed but is not held")
-        self._held[slot] = False
-        self._free.append(slot)
+        PagePool.free(self, [slot])
 
 
 class BlockTable:
     """One request's pages in one group: logical page index -> page id, or -1 once a
     window has passed the page and it was given back
-    (crates/macllm-kv/src/cache.rs:1434-1440)."""
+    (crates/macllm-kv/src/cache.rs:1434-1440).  A view of the core's table."""
 
-    def __init__(self):
-        self.pages: List[int] = []
-        self.first_live = 0          # logical pages before this one were given back
+    def __init__(self, core, group: int, slot: int):
+        self._core, self._group, self._slot = core, group, slot
+
+    @property
+    def pages(self) -> List[int]:
+        lib = native.lib()
+        count = lib.hc_table(self._core.pointer, self._group, self._slot, None, 0)
+        out = np.empty(max(count, 1), dtype=np.int32)
+        lib.hc_table(self._core.pointer, self._group, self._slot, native.int_pointer(out), count)
+        return out[:count].tolist()
+
+    @property
+    def first_live(self) -> int:
+        """Logical pages before this one were given back."""
+        return native.lib().hc_first_live(self._core.pointer, self._group, self._slot)
 
     def live_pages(self) -> List[int]:
         return [page for page in self.pages if page >= 0]

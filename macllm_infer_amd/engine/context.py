@@ -4,7 +4,8 @@ A step runs a list of lanes; a lane is a run of consecutive tokens of one reques
 starting at that request's current length: a portion of a prompt or one decoded
 token.  Lanes are packed without padding in submission order
 (reference: src/decoder.rs:4248-4260, lane struct paged_decode.metal:51-58).
-All index arrays are built on the host and uploaded in one copy.
+All index arrays are written by the host-side core (``csrc/hostcore.cpp``) into one buffer and
+uploaded in one copy.
 
 ``StaticStep`` keeps the arrays of a batch of single-token lanes at fixed addresses and
 fixed shapes, so that a captured HIP graph can be replayed on them; lanes beyond the
@@ -13,10 +14,13 @@ batch's real ones are padding that reads and writes the cache's scratch page and
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from itertools import chain
 from typing import Hashable, List, Optional, Sequence
 
 import numpy as np
 import torch
+
+from ..cache import native
 
 
 QUERY_TILE = 64        # tokens of one lane that one workgroup of the prefill attention kernel takes
@@ -51,49 +55,60 @@ class StepContext:
     derived: dict = field(default_factory=dict)   # tables parts derive from the step, shared by the layers
 
 
-def _pack(lanes: Sequence[Lane], cache, pad_lanes: int = 0, max_pages: Optional[int] = None,
-          pad_lengths: Sequence[int] = ()):
-    """Numpy sections of the step (in the order of ``_assemble``) and the block-table shapes.
-    ``pad_lanes`` single-token lanes on the scratch page and slot are appended (or lanes of
-    ``pad_lengths`` tokens, all of them on the scratch page)."""
-    pad_lengths = list(pad_lengths) if pad_lengths else [1] * pad_lanes
-    pad_lanes = len(pad_lengths)
-    lengths = [len(lane.tokens) for lane in lanes] + pad_lengths
-    starts = [cache.requests[lane.request].length for lane in lanes] + [0] * pad_lanes
-    Ln = len(lengths)
-    T = sum(lengths)
-    token_ids = np.concatenate([np.asarray(lane.tokens, dtype=np.int32) for lane in lanes]
-                               + [np.zeros(sum(pad_lengths), dtype=np.int32)])
-    positions = np.concatenate([np.arange(start, start + length, dtype=np.int32)
-                                for start, length in zip(starts, lengths)])
-    lane_of_token = np.repeat(np.arange(Ln, dtype=np.int32), lengths)
-    cu = np.zeros(Ln + 1, dtype=np.int32)
-    cu[1:] = np.cumsum(lengths)
-    start_pos = np.asarray(starts, dtype=np.int32)
-    seq_lens = start_pos + np.asarray(lengths, dtype=np.int32)
-    slot_ids = np.asarray([cache.requests[lane.request].slot for lane in lanes]
-                          + [cache.scratch_slot] * pad_lanes, dtype=np.int32)
-    want_rows = np.asarray([cu[index] + place for index, lane in enumerate(lanes) for place in lane.want],
-                           dtype=np.int32)
-    tiles = np.asarray([(index, row) for index in range(Ln) for row in range(cu[index], cu[index + 1], QUERY_TILE)],
-                       dtype=np.int32).reshape(-1)
-    sections = [token_ids, positions, lane_of_token, cu, start_pos, seq_lens, slot_ids, want_rows, tiles]
-    group_shapes = []
-    for group in cache.groups:
-        page_size = group.page_size
-        tables = ([group.tables[lane.request].pages for lane in lanes]
-                  + [[group.scratch_page] * -(-length // page_size) for length in pad_lengths])
-        width = max_pages if max_pages is not None else max(1, max(len(pages) for pages in tables))
-        table = np.zeros((Ln, width), dtype=np.int32)
-        mapping = np.empty(T, dtype=np.int32)
-        for row, pages in enumerate(tables):
-            pages = np.asarray(pages, dtype=np.int32)
-            table[row, :len(pages)] = np.maximum(pages, 0)
-            lane_positions = positions[cu[row]:cu[row + 1]]
-            mapping[cu[row]:cu[row + 1]] = pages[lane_positions // page_size] * page_size + lane_positions % page_size
-        sections += [mapping, table.reshape(-1)]
-        group_shapes.append((Ln, width))
-    return sections, group_shapes, lengths, starts
+@dataclass
+class LoweredLanes:
+    """A step's lanes as the arrays the host-side core reads."""
+    slots: np.ndarray            # [lanes] the requests' handles in the core (their state slots)
+    lengths: np.ndarray          # [lanes] tokens of each lane
+    tokens: np.ndarray           # [T] all lanes' tokens, lane after lane
+    want_counts: np.ndarray      # [lanes] wanted places of each lane
+    wants: np.ndarray            # [wanted] the places, lane after lane
+
+
+def lower_lanes(lanes: Sequence[Lane], cache) -> LoweredLanes:
+    """KeyError for a request that is not live, OverflowError / ValueError / TypeError for a token
+    or place that is no 32-bit integer."""
+    count = len(lanes)
+    slots = cache.slots_of([lane.request for lane in lanes])
+    lengths = np.fromiter((len(lane.tokens) for lane in lanes), dtype=np.int32, count=count)
+    want_counts = np.fromiter((len(lane.want) for lane in lanes), dtype=np.int32, count=count)
+    tokens = np.fromiter(chain.from_iterable(lane.tokens for lane in lanes), dtype=np.int64, count=int(lengths.sum()))
+    wants = np.fromiter(chain.from_iterable(lane.want for lane in lanes), dtype=np.int64, count=int(want_counts.sum()))
+    if tokens.size and (tokens.min() < -(1 << 31) or tokens.max() >= (1 << 31)):
+        raise OverflowError("a token id does not fit 32 bits")
+    if wants.size and (wants.min() < -(1 << 31) or wants.max() >= (1 << 31)):
+        raise OverflowError("a wanted place does not fit 32 bits")
+    return LoweredLanes(slots, lengths, tokens.astype(np.int32), want_counts, wants.astype(np.int32))
+
+
+_NO_LANES = LoweredLanes(*(np.zeros(0, dtype=np.int32) for _ in range(5)))
+
+
+def _pack(lowered: LoweredLanes, cache, out: Optional[np.ndarray], pad_lengths: Sequence[int] = (),
+          max_pages: Optional[int] = None, want_rows: Optional[np.ndarray] = None):
+    """The core writes the step's sections (in the order of ``_assemble``) into ``out``.  Returns
+    (words written or, negated, words needed when ``out`` is too small or None; section sizes;
+    block-table shapes; longest context after the step).  ``pad_lengths``: lanes appended on the
+    scratch page and slot.  ``want_rows`` replaces the lanes' own wanted rows."""
+    core = cache.core
+    pads = native.as_ints(list(pad_lengths))
+    groups = len(cache.groups)
+    meta = np.zeros(9 + 3 * groups + 1, dtype=np.int32)
+    fixed = native.as_ints(want_rows) if want_rows is not None else None
+    written = core.lib.hc_pack(
+        core.pointer, len(lowered.slots), native.int_pointer(lowered.slots), native.int_pointer(lowered.lengths),
+        native.int_pointer(lowered.tokens), native.int_pointer(lowered.want_counts), native.int_pointer(lowered.wants),
+        len(pads), native.int_pointer(pads), max_pages or 0, QUERY_TILE,
+        native.int_pointer(fixed) if fixed is not None else None, len(fixed) if fixed is not None else 0,
+        native.int_pointer(out) if out is not None else None, out.size if out is not None else 0,
+        native.int_pointer(meta))
+    if written == -1:
+        raise ValueError("the step cannot be packed: a request is not live, a wanted place lies outside its "
+                         "lane, or the step's pages were not reserved")
+    lanes = len(lowered.slots) + len(pads)
+    sizes = meta[:9 + 2 * groups].tolist()
+    shapes = [(lanes, int(width)) for width in meta[9 + 2 * groups:9 + 3 * groups]]
+    return int(written), sizes, shapes, int(meta[-1])
 
 
 def _assemble(views, group_shapes, lengths, starts, max_seq_len) -> StepContext:
@@ -108,23 +123,26 @@ def _assemble(views, group_shapes, lengths, starts, max_seq_len) -> StepContext:
     return context
 
 
-def _split(buffer: torch.Tensor, sections):
+def _split(buffer: torch.Tensor, sizes):
     views, offset = [], 0
-    for section in sections:
-        views.append(buffer[offset:offset + section.size])
-        offset += section.size
+    for size in sizes:
+        views.append(buffer[offset:offset + size])
+        offset += size
     return views
 
 
-def build_step_context(lanes: Sequence[Lane], cache, device) -> StepContext:
+def build_step_context(lanes: Sequence[Lane], cache, device, lowered: Optional[LoweredLanes] = None) -> StepContext:
     """``cache``: the CacheManager, after the step's pages were reserved."""
-    sections, group_shapes, lengths, starts = _pack(lanes, cache)
-    host = torch.from_numpy(np.concatenate(sections))
+    if lowered is None:
+        lowered = lower_lanes(lanes, cache)
+    needed, _, _, _ = _pack(lowered, cache, None)
+    host = torch.empty(-needed, dtype=torch.int32)
     if torch.device(device).type == "cuda":
         host = host.pin_memory()
+    _, sizes, shapes, longest = _pack(lowered, cache, host.numpy())
     packed = host.to(device, non_blocking=True)
-    context = _assemble(_split(packed, sections), group_shapes, lengths, starts,
-                        max(start + length for start, length in zip(starts, lengths)))
+    starts = cache.lengths_of(lowered.slots).tolist()
+    context = _assemble(_split(packed, sizes), shapes, lowered.lengths.tolist(), starts, longest)
     context._keepalive = host
     return context
 
@@ -138,22 +156,22 @@ class StaticStep:
                  want_rows: Sequence[int] = ()):
         self.cache = cache
         self.lanes = lanes
-        self.lengths = list(lengths)
+        self.lengths = list(lengths) if lengths else [1] * lanes
         self.max_pages = max(-(-max_seq_len // group.page_size) for group in cache.groups) if cache.groups else 1
-        self.want_rows = (np.asarray(want_rows, dtype=np.int32) if self.lengths
+        self.want_rows = (np.asarray(want_rows, dtype=np.int32) if lengths
                           else np.arange(lanes, dtype=np.int32))             # every lane's row is wanted
-        sections, group_shapes, lengths, starts = _pack([], cache, pad_lanes=lanes, max_pages=self.max_pages,
-                                                        pad_lengths=self.lengths)
-        sections[7] = self.want_rows
-        total = sum(section.size for section in sections)
-        self.host = torch.empty(total, dtype=torch.int32).pin_memory()
-        self.device_buffer = torch.empty(total, dtype=torch.int32, device=device)
-        self.host.copy_(torch.from_numpy(np.concatenate(sections)))
+        needed, sizes, shapes, _ = _pack(_NO_LANES, cache, None, self.lengths, self.max_pages, self.want_rows)
+        self.host = torch.empty(-needed, dtype=torch.int32)
+        if torch.device(device).type == "cuda":
+            self.host = self.host.pin_memory()
+        self.host_words = self.host.numpy()
+        self.device_buffer = torch.empty(-needed, dtype=torch.int32, device=device)
+        _pack(_NO_LANES, cache, self.host_words, self.lengths, self.max_pages, self.want_rows)
         self.device_buffer.copy_(self.host)
-        self.context = _assemble(_split(self.device_buffer, sections), group_shapes, lengths, starts, max_seq_len)
+        self.context = _assemble(_split(self.device_buffer, sizes), shapes, self.lengths, [0] * lanes, max_seq_len)
 
-    def fill(self, lanes: Sequence[Lane]) -> None:
-        sections, _, _, _ = _pack(lanes, self.cache, pad_lanes=self.lanes - len(lanes), max_pages=self.max_pages)
-        sections[7] = self.want_rows
-        self.host.copy_(torch.from_numpy(np.concatenate(sections)))
+    def fill(self, lowered: LoweredLanes) -> None:
+        """``lowered``: the real lanes, whose lengths are the first of this step's; the rest is padding."""
+        real = len(lowered.slots)
+        _pack(lowered, self.cache, self.host_words, self.lengths[real:], self.max_pages, self.want_rows)
         self.device_buffer.copy_(self.host, non_blocking=True)

@@ -12,6 +12,7 @@ from __future__ import annotations
 
 from typing import Dict, Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
@@ -21,7 +22,7 @@ from ..kernels import build as kernel_build
 from ..kernels import ops
 from ..parts.base import BuildContext
 from ..weights.loader import WeightSource, bind
-from .context import Lane, build_step_context
+from .context import Lane, LoweredLanes, build_step_context, lower_lanes
 from .model import DecoderModel
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
@@ -96,44 +97,58 @@ class Engine:
         return self.cache.requests[request].length
 
     # ------------------------------------------------------------------ the step function
-    def validate(self, lanes: Sequence[Lane]) -> None:
+    def validate(self, lanes: Sequence[Lane]) -> LoweredLanes:
+        """StepError for a step that cannot run; otherwise its lanes as arrays."""
         if not lanes:
             raise StepError("a step needs at least one lane")
-        seen = set()
-        for lane in lanes:
-            if lane.request not in self.cache.requests:
-                raise StepError(f"request {lane.request!r} is not live")
-            if lane.request in seen:
-                raise StepError(f"request {lane.request!r} appears twice in one step")
-            seen.add(lane.request)
-            count = len(lane.tokens)
-            if count == 0:
-                raise StepError(f"request {lane.request!r}: a lane cannot be empty")
-            for token in lane.tokens:
-                if not (0 <= int(token) < self.vocab_size):
-                    raise StepError(f"request {lane.request!r}: token {token} is outside the vocabulary "
-                                    f"of {self.vocab_size}")
-            if self.cache.requests[lane.request].length + count > self.max_context:
-                raise StepError(f"request {lane.request!r}: {self.cache.requests[lane.request].length} + {count} "
-                                f"tokens exceed the context limit {self.max_context}")
-            for place in lane.want:
-                if not (0 <= int(place) < count):
-                    raise StepError(f"request {lane.request!r}: wanted place {place} is outside its {count} tokens")
+        try:
+            lowered = lower_lanes(lanes, self.cache)
+        except KeyError as error:
+            raise StepError(str(error.args[0])) from None
+        except (OverflowError, TypeError, ValueError) as error:
+            raise StepError(f"tokens and wanted places must be integers: {error}") from None
+        names = [lane.request for lane in lanes]
+        if len(set(lowered.slots.tolist())) != len(lanes):
+            twice = next(name for index, name in enumerate(names) if name in names[:index])
+            raise StepError(f"request {twice!r} appears twice in one step")
+        lengths, tokens = lowered.lengths, lowered.tokens
+        if int(lengths.min()) == 0:
+            raise StepError(f"request {names[int(np.argmin(lengths))]!r}: a lane cannot be empty")
+        lane_of_token = np.repeat(np.arange(len(lanes)), lengths)
+        outside = (tokens < 0) | (tokens >= self.vocab_size)
+        if outside.any():
+            where = int(np.argmax(outside))
+            raise StepError(f"request {names[int(lane_of_token[where])]!r}: token {int(tokens[where])} is outside "
+                            f"the vocabulary of {self.vocab_size}")
+        starts = self.cache.lengths_of(lowered.slots)
+        beyond = starts.astype(np.int64) + lengths > self.max_context
+        if beyond.any():
+            where = int(np.argmax(beyond))
+            raise StepError(f"request {names[where]!r}: {int(starts[where])} + {int(lengths[where])} "
+                            f"tokens exceed the context limit {self.max_context}")
+        if lowered.wants.size:
+            lane_of_want = np.repeat(np.arange(len(lanes)), lowered.want_counts)
+            outside = (lowered.wants < 0) | (lowered.wants >= lengths[lane_of_want])
+            if outside.any():
+                where = int(np.argmax(outside))
+                lane = int(lane_of_want[where])
+                raise StepError(f"request {names[lane]!r}: wanted place {int(lowered.wants[where])} is outside "
+                                f"its {int(lengths[lane])} tokens")
+        return lowered
 
     def step(self, lanes: Sequence[Lane]) -> torch.Tensor:
         """Run one batch; returns float32 logits [wanted, vocab] in the order of the lanes and
         of each lane's ``want``.  Raises StepError or CacheExhausted with nothing changed."""
-        self.validate(lanes)
-        self.cache.reserve([(lane.request, len(lane.tokens)) for lane in lanes])
+        lowered = self.validate(lanes)
+        self.cache.reserve_slots(lowered.slots, lowered.lengths)
         logits = None
         if self.graphs is not None:
-            if all(len(lane.tokens) == 1 for lane in lanes):
-                logits = self.graphs.run(lanes)              # decode-only batch: a captured graph
+            if int(lowered.lengths.max()) == 1:
+                logits = self.graphs.run(lanes, lowered)              # decode-only batch: a captured graph
             else:
-                logits = self.graphs.run_portion(lanes)      # a shape of prompt portions seen before
+                logits = self.graphs.run_portion(lanes, lowered)      # a shape of prompt portions seen before
         if logits is None:
-            context = build_step_context(lanes, self.cache, self.device)
+            context = build_step_context(lanes, self.cache, self.device, lowered)
             logits = self.model.forward(context, self.cache)
-        for lane in lanes:
-            self.cache.commit(lane.request, len(lane.tokens))
+        self.cache.commit_slots(lowered.slots, lowered.lengths)
         return logits

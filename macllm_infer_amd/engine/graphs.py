@@ -19,7 +19,7 @@ from typing import Dict, Optional, Sequence
 
 import torch
 
-from .context import Lane, StaticStep
+from .context import Lane, LoweredLanes, StaticStep, lower_lanes
 
 
 def bucket_for(lanes: int) -> int:
@@ -45,7 +45,7 @@ class DecodeGraphs:
     PORTION_RECENT = 32            # steps with portions whose shapes are remembered
     PORTION_SIGHTINGS = 3          # sightings among them before a shape is captured
 
-    def run_portion(self, lanes: Sequence[Lane]) -> Optional[torch.Tensor]:
+    def run_portion(self, lanes: Sequence[Lane], lowered: LoweredLanes) -> Optional[torch.Tensor]:
         """Logits of a step with prompt portions from a captured graph of its shape, or None when
         the shape has no graph (yet): the caller then runs it launch by launch.
 
@@ -83,7 +83,7 @@ class DecodeGraphs:
         else:
             self._portion_graphs.move_to_end(key)
         static, graph, logits = entry
-        static.fill(ordered)
+        static.fill(lowered if order == list(range(len(lanes))) else lower_lanes(ordered, self.cache))
         graph.replay()
         self.counts["portion_replays"] += 1
         if padding == 0 and order == list(range(len(lanes))):
@@ -113,19 +113,19 @@ class DecodeGraphs:
             logits = self.model.forward(static.context, self.cache)
         return static, graph, logits
 
-    def run(self, lanes: Sequence[Lane]) -> torch.Tensor:
+    def run(self, lanes: Sequence[Lane], lowered: LoweredLanes) -> torch.Tensor:
         """Logits [wanted, vocab] of single-token lanes (a copy: the graph's own output tensor is
         overwritten by the next replay)."""
         bucket = bucket_for(len(lanes))
         if bucket not in self._graphs:
             self._graphs[bucket] = self._capture(bucket)
         static, graph, logits = self._graphs[bucket]
-        static.fill(lanes)
+        static.fill(lowered)
         graph.replay()
         self.counts["decode_replays"] += 1
-        rows = [index for index, lane in enumerate(lanes) if len(lane.want) > 0]
-        if len(rows) == len(lanes):
+        if int(lowered.want_counts.min()) > 0:
             return logits[:len(lanes)].clone()
+        rows = [index for index, lane in enumerate(lanes) if len(lane.want) > 0]
         if not rows:
             return logits[:0].clone()
         return logits[torch.tensor(rows, device=logits.device)]

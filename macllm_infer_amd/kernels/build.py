@@ -2,7 +2,8 @@
 
 Each ``csrc/<module>.hip`` becomes one shared library built with plain ``hipcc`` for
 gfx950 and loaded through ``ctypes``; entry points are ``extern "C"`` functions that
-take raw device pointers and a HIP stream.  A module is compiled the first time it
+take raw device pointers and a HIP stream.  ``csrc/<module>.cpp`` (the host-side core of the
+cache manager) is plain C++ built with the host compiler the same way.  A module is compiled the first time it
 is asked for (and again when its source or the flags change); the engine asks only
 for the modules its model's parts name.  Built libraries live in ``csrc/_build`` of
 the checkout, or in a per-user temporary folder if that is not writable.
@@ -26,7 +27,9 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-shared", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", "-Wno-pass-failed"]
-MODULES = ("common", "attention", "mamba2", "ssd", "gemm", "decode", "sampling")
+HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall"]
+HOST_MODULES = ("hostcore",)                      # plain C++, no GPU code
+MODULES = ("common", "attention", "mamba2", "ssd", "gemm", "decode", "sampling") + HOST_MODULES
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -44,17 +47,32 @@ def _hipcc() -> str:
                            "the HIP kernels cannot be built and there is no other code path")
 
 
+def _host_compiler() -> str:
+    for candidate in (os.environ.get("CXX"), "g++", "c++", "clang++", "/opt/rocm/llvm/bin/clang++"):
+        found = candidate and (candidate if os.path.isfile(candidate) else shutil.which(candidate))
+        if found:
+            return found
+    raise KernelBuildError("no C++ compiler was found (looked at $CXX, g++, c++, clang++); "
+                           "the host-side core cannot be built and there is no other code path")
+
+
+def _main_source(module: str) -> str:
+    return os.path.join(CSRC, f"{module}.cpp" if module in HOST_MODULES else f"{module}.hip")
+
+
 def _sources(module: str) -> List[str]:
-    main = os.path.join(CSRC, f"{module}.hip")
+    main = _main_source(module)
     if not os.path.isfile(main):
         raise KernelBuildError(f"no such kernel module: {main}")
+    if module in HOST_MODULES:
+        return [main]
     headers = sorted(os.path.join(CSRC, name) for name in os.listdir(CSRC) if name.endswith(".h"))
     return [main] + headers
 
 
 def _stamp(module: str) -> str:
     digest = hashlib.sha256()
-    digest.update(" ".join(FLAGS).encode())
+    digest.update(" ".join(HOST_FLAGS if module in HOST_MODULES else FLAGS).encode())
     for path in _sources(module):
         with open(path, "rb") as handle:
             digest.update(handle.read())
@@ -102,9 +120,14 @@ def compile_module(module: str, force: bool = False, quiet: bool = False) -> str
     folder = _writable_build_dir()
     library = os.path.join(folder, f"{module}.so")
     scratch = os.path.join(folder, f"{module}.{os.getpid()}.tmp.so")
-    command = [_hipcc()] + FLAGS + [os.path.join(CSRC, f"{module}.hip"), "-o", scratch]
+    if module in HOST_MODULES:
+        command = [_host_compiler()] + HOST_FLAGS + [_main_source(module), "-o", scratch]
+        what = f"host module '{module}'"
+    else:
+        command = [_hipcc()] + FLAGS + [_main_source(module), "-o", scratch]
+        what = f"HIP module '{module}' for {ARCH}"
     if not quiet:
-        print(f"[macllm_infer_amd] compiling HIP module '{module}' for {ARCH} ...", file=sys.stderr, flush=True)
+        print(f"[macllm_infer_amd] compiling {what} ...", file=sys.stderr, flush=True)
     started = time.time()
     environment = dict(os.environ)
     environment.setdefault("HOME", tempfile.gettempdir())
@@ -125,7 +148,7 @@ def compile_module(module: str, force: bool = False, quiet: bool = False) -> str
     if process.returncode != 0:
         if os.path.exists(scratch):
             os.remove(scratch)
-        raise KernelBuildError(f"hipcc failed for module '{module}':\n{''.join(output)}")
+        raise KernelBuildError(f"{command[0]} failed for module '{module}':\n{''.join(output)}")
     os.replace(scratch, library)
     with open(library + ".stamp", "w") as handle:
         handle.write(stamp)

@@ -180,3 +180,69 @@ def test_shared_kv_entries_read_the_owner():
     with pytest.raises(ValueError, match="differ"):
         CacheManager({(0, "attn"): [KVNeed(2, 4, None)], (1, "attn"): [KVNeed(1, 4, None)]},
                      {(1, "attn"): (0, "attn")}, 8, 32, 2, torch.float32, "cpu")
+
+
+def plain_packing(cache, lanes, pad_lengths, width):
+    """The step's index arrays, lane by lane, from the manager's tables: what the core's packer
+    has to write.  ``lanes``: (request, tokens, wanted places)."""
+    lengths = [len(tokens) for _, tokens, _ in lanes] + list(pad_lengths)
+    starts = [cache.requests[request].length for request, _, _ in lanes] + [0] * len(pad_lengths)
+    first = [sum(lengths[:index]) for index in range(len(lengths) + 1)]
+    out = {"token_ids": [token for _, tokens, _ in lanes for token in tokens] + [0] * sum(pad_lengths),
+           "positions": [start + t for start, length in zip(starts, lengths) for t in range(length)],
+           "lane_of_token": [index for index, length in enumerate(lengths) for _ in range(length)],
+           "cu_seqlens": first, "start_pos": starts,
+           "seq_lens": [start + length for start, length in zip(starts, lengths)],
+           "slot_ids": [cache.requests[request].slot for request, _, _ in lanes] + [cache.scratch_slot] * len(pad_lengths),
+           "want_rows": [first[index] + place for index, (_, _, want) in enumerate(lanes) for place in want],
+           "query_tiles": [[index, row] for index in range(len(lengths)) for row in range(first[index], first[index + 1], 64)],
+           "slot_mappings": [], "block_tables": []}
+    for number, group in enumerate(cache.groups):
+        size = group.page_size
+        tables = ([cache.table(number, request).pages for request, _, _ in lanes]
+                  + [[group.scratch_page] * -(-length // size) for length in pad_lengths])
+        columns = width or max(1, max(len(pages) for pages in tables))
+        out["block_tables"].append([[max(page, 0) for page in pages] + [0] * (columns - len(pages)) for pages in tables])
+        out["slot_mappings"].append([pages[(start + t) // size] * size + (start + t) % size
+                                     for pages, start, length in zip(tables, starts, lengths) for t in range(length)])
+    return out
+
+
+@pytest.mark.parametrize("decode_only", [False, True])
+@pytest.mark.parametrize("seed", range(5))
+def test_the_cores_packing_of_a_step_matches_a_plain_packing(seed, decode_only):
+    from macllm_infer_amd.engine.context import Lane, StaticStep, build_step_context, lower_lanes
+    rng = random.Random(seed)
+    cache = make(capacity=1200, page=rng.choice([4, 8, 16]), requests=5, window=rng.choice([None, 9, 40]))
+    names = ["a", "b", "c", "d"]
+    for name in names:
+        cache.add_request(name)
+        grown = rng.randrange(0, 150)
+        if grown:
+            cache.reserve([(name, grown)])
+            cache.commit(name, grown)                              # window groups have given pages back by now
+    picked = rng.sample(names, rng.randrange(1, 5))
+    lanes = []
+    for name in picked:
+        tokens = [rng.randrange(0, 1000) for _ in range(1 if decode_only else rng.choice([1, 1, 2, 7, 70, 130]))]
+        lanes.append((name, tokens, sorted(rng.sample(range(len(tokens)), rng.randrange(0, min(3, len(tokens)) + 1)))))
+    cache.reserve([(name, len(tokens)) for name, tokens, _ in lanes])
+    step_lanes = [Lane(*lane) for lane in lanes]
+
+    def compare(context, want):
+        for field, value in want.items():
+            got = getattr(context, field)
+            got = [item.tolist() for item in got] if isinstance(got, list) else got.tolist()
+            assert got == value, field
+
+    context = build_step_context(step_lanes, cache, "cpu")
+    compare(context, plain_packing(cache, lanes, [], None))
+    assert context.max_seq_len == max(cache.requests[name].length + len(tokens) for name, tokens, _ in lanes)
+    assert context.lane_starts == [cache.requests[name].length for name, _, _ in lanes]
+    if all(len(tokens) == 1 for _, tokens, _ in lanes):            # a captured decode step: padded, fixed width
+        static = StaticStep(cache, 4, 400, "cpu")
+        compare(static.context, dict(plain_packing(cache, [], [1] * 4, static.max_pages), want_rows=[0, 1, 2, 3]))
+        static.fill(lower_lanes(step_lanes, cache))
+        compare(static.context, dict(plain_packing(cache, lanes, [1] * (4 - len(lanes)), static.max_pages),
+                                     want_rows=[0, 1, 2, 3]))
+    cache.check()
