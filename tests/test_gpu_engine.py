@@ -5,6 +5,7 @@ reads another layer's cache, all registered from here without a change to the pa
 import math
 import subprocess
 import sys
+import numpy as np
 import pytest
 import torch
 
@@ -450,3 +451,58 @@ def test_a_wide_model_runs_through_the_fast_paths(tmp_path, monkeypatch, padding
         scale = want.abs().max().item()
         assert (have - want).abs().max().item() <= 6e-2 * scale
         assert ((have - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()).item() <= 3e-2
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_configurations_drawn_at_random_match_the_plain_model(seed):
+    """Every size and option at random (head sizes 16..128 in steps of 16, 1..12 heads, odd widths
+    and vocabularies, pages of 4..64 tokens): whole, and two requests cut at random beside each
+    other with their last tokens one by one, in float32 and in bfloat16."""
+    import random
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.weights.random_init import random_tensors
+    from test_gpu_replay import bfloat16_close
+    raw, page = tiny_configs.random_config(seed)
+    config = FalconH1Config.from_dict(raw)
+    rng = random.Random(seed)
+    generator = torch.Generator().manual_seed(seed)
+    first = torch.randint(0, raw["vocab_size"], (rng.choice([70, 131, 200]),), generator=generator).tolist()
+    second = torch.randint(0, raw["vocab_size"], (rng.choice([9, 40, 77]),), generator=generator).tolist()
+    for dtype in ("float32", "bfloat16"):
+        tensors = random_tensors(config, seed, torch.float32 if dtype == "float32" else torch.bfloat16, "unit")
+        plain = {name: tensor.float() for name, tensor in tensors.items()}
+        wanted = {"a": plain_impl.falcon_h1_logits(config.to_dict(), plain, first).numpy(),
+                  "b": plain_impl.falcon_h1_logits(config.to_dict(), plain, second).numpy()}
+
+        def close(got, want, what):
+            if dtype == "float32":
+                assert np.abs(got - want).max() <= 1e-4, f"seed {seed} {what}: {np.abs(got - want).max():.3e}"
+            else:
+                assert bfloat16_close(got, want), f"seed {seed} {what}: {np.abs(got - want).max():.3e} of {np.abs(want).max():.2f}"
+
+        engine = Engine(config=config, tensors=tensors, dtype=dtype, kv_cache_block_tokens=page,
+                        kv_cache_capacity_tokens=640, max_active_sequences=3)
+        engine.add_request("whole")
+        close(engine.step([Lane("whole", first, list(range(len(first))))]).cpu().numpy(), wanted["a"], "whole")
+        engine.finish("whole")
+        engine.add_request("a")
+        engine.add_request("b")
+        tokens, cursor, rows = {"a": first, "b": second}, {"a": 0, "b": 0}, {"a": [], "b": []}
+        while cursor["a"] < len(first) or cursor["b"] < len(second):
+            lanes = []
+            for name, tail, sizes in (("a", 12, [2, 5, 17, 64, 33]), ("b", 6, [2, 3, 11, 30])):
+                left = len(tokens[name]) - cursor[name]
+                if left > 0 and (name == "a" or rng.random() < 0.7):
+                    count = 1 if left <= tail else min(rng.choice(sizes), left - tail)
+                    lanes.append(Lane(name, tokens[name][cursor[name]:cursor[name] + count], list(range(count))))
+            if not lanes:
+                continue
+            out = engine.step(lanes).cpu().numpy()
+            for lane in lanes:
+                rows[lane.request].append(out[:len(lane.tokens)])
+                out = out[len(lane.tokens):]
+                cursor[lane.request] += len(lane.tokens)
+        for name in ("a", "b"):
+            close(np.concatenate(rows[name]), wanted[name], f"cut {name}")
+        engine.cache.check()
