@@ -506,3 +506,48 @@ def test_configurations_drawn_at_random_match_the_plain_model(seed):
         for name in ("a", "b"):
             close(np.concatenate(rows[name]), wanted[name], f"cut {name}")
         engine.cache.check()
+
+
+@pytest.mark.parametrize("shape, layers, vocab", [("0.5b", 2, None), ("7b", 1, 1003)])
+def test_layers_of_the_benchmark_shapes_match_the_plain_model(shape, layers, vocab):
+    """Layers with the sizes bench.py measures (0.5B shape: width 1024, 8 query heads on 2, 24
+    state-space heads of 64 x 128, chunk 128, a vocabulary of 32,784; 7B shape: width 3072, 12 query
+    heads of 128 on 2, state-space heads of 128 x 256, a small vocabulary), through the paths those
+    sizes take: a prompt in portions long enough for the chunked scan, the matrix-core attention and
+    the library's products, replayed from captured graphs, then decoding in a batch of three."""
+    import bench
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.weights.random_init import random_tensors
+    from test_gpu_replay import bfloat16_close
+    raw = dict(bench.SHAPES[shape], num_hidden_layers=layers)
+    config = FalconH1Config.from_dict(dict(raw, vocab_size=vocab or raw["vocab_size"]))
+    tensors = random_tensors(config, 7, torch.bfloat16, "unit")
+    plain = {name: tensor.float() for name, tensor in tensors.items()}
+    prompts = {name: tokens_for(config.vocab_size, length, seed)
+               for name, length, seed in (("long", 2 * 300 + 37 + 8, 1), ("short", 45 + 8, 2), ("third", 300 + 8, 3))}
+    engine = Engine(config=config, tensors=tensors, dtype="bfloat16", kv_cache_capacity_tokens=1536, max_active_sequences=3)
+    rows = {name: [] for name in prompts}
+    for name in prompts:
+        engine.add_request(name)
+    # the same shape (300 tokens, last place wanted) three times: launched, launched, captured and replayed
+    for name, first in (("long", 0), ("third", 0), ("long", 300)):
+        rows[name].append(engine.step([Lane(name, prompts[name][first:first + 300], [299])]).cpu())
+    assert engine.graphs.counts["portion_captures"] == 1 and engine.graphs.counts["portion_replays"] == 1
+    mixed = engine.step([Lane("long", prompts["long"][600:637], [36]), Lane("short", prompts["short"][:45], [0, 44])]).cpu()
+    rows["long"].append(mixed[:1])
+    rows["short"].append(mixed[1:])
+    rows["long"].append(engine.step([Lane("long", prompts["long"][637:638], [0])]).cpu())
+    for turn in range(7):
+        lanes = [Lane("long", [prompts["long"][638 + turn]], [0]), Lane("short", [prompts["short"][45 + turn]], [0]),
+                 Lane("third", [prompts["third"][300 + turn]], [0])]
+        out = engine.step(lanes).cpu()
+        for row, name in enumerate(("long", "short", "third")):
+            rows[name].append(out[row:row + 1])
+    places = {"long": [299, 599, 636] + list(range(637, 645)), "short": [0, 44] + list(range(45, 52)),
+              "third": [299] + list(range(300, 307))}
+    for name, tokens in prompts.items():
+        want = plain_impl.falcon_h1_logits(config.to_dict(), plain, tokens[:places[name][-1] + 1])[places[name]].numpy()
+        got = torch.cat(rows[name]).numpy()
+        assert got.shape == want.shape, name
+        assert bfloat16_close(got, want), f"{name}: {np.abs(got - want).max():.3e} of {np.abs(want).max():.2f}"
