@@ -89,14 +89,19 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   constexpr int BATCH = FG_WAVES == 8 ? 4 : 8;
   bf16x8_t a[BATCH];
 
-  // the slot of the row whose conv tail this thread will need: asked for before everything else,
-  // because the tail's address waits for it
-  int tail_slot = 0, tail_n = 0;
+  // The outputs this thread finishes in the epilogue: element tid + j * FG_THREADS of the block's
+  // MT x (16 rows x 16 features), all of one feature.  The slots of their rows are asked for before
+  // everything else, because the addresses of their conv tails wait for them.
+  constexpr int EPT = (MT * 256 + FG_THREADS - 1) / FG_THREADS;        // outputs a thread finishes
+  constexpr int TAILS = (MT == 1 && FG_THREADS == 256) ? 8 : 3;         // tail samples kept per output
+  const int tail_n = n0 + 4 * ((tid % 64) / 16) + (tid % 256) / 64;
+  int tail_slot[EPT] = {};
   bool tail_wanted = false;
-  if (EPI == EPI_CONV && MT == 1 && FG_THREADS == 256 && p.conv_k >= 2 && p.conv_k <= 9) {
-    tail_n = n0 + 4 * ((tid % 64) / 16) + (tid / 64);
-    tail_slot = p.slot_ids[min(tid % 16, p.M - 1)];
-    tail_wanted = tail_n >= p.conv_lo && tail_n < p.conv_hi && tid % 16 < p.M;
+  if (EPI == EPI_CONV && p.conv_k >= 2 && p.conv_k <= TAILS + 1) {
+    tail_wanted = tail_n >= p.conv_lo && tail_n < p.conv_hi;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j)
+      tail_slot[j] = p.slot_ids[min(((tid + j * FG_THREADS) / 256) * 16 + tid % 16, p.M - 1)];
   }
 
   // Loads come back in the order they were asked for, and a wait counts all of them.  The rows
@@ -222,21 +227,26 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
     __syncthreads();
   }
 
-  // the conv tail of the element this thread finishes in the epilogue (one element per thread
-  // when the block has 16 x 16 outputs) is asked for now, behind the weights; no branch between
-  // its loads either
-  bf16_t tail_values[8];
-  float tap_values[9];
+  // the conv tails of those outputs are asked for now, behind the weights; no branch between the
+  // loads either (a row past M reads the last row's tail and is not used)
+  bf16_t tail_values[EPT][TAILS];
+  float tap_values[TAILS + 1];
   float tap_bias = 0.f;
   bool tail_ready = false;
-  if (EPI == EPI_CONV) asm volatile("" : "+v"(tail_slot));      // keeps every use of the slot (and its wait) down here
+  if (EPI == EPI_CONV) {
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) asm volatile("" : "+v"(tail_slot[j]));   // keeps every use of the slots (and their wait) down here
+  }
   if (tail_wanted) {
     const int channels = p.conv_hi - p.conv_lo;
-    const bf16_t* tail = p.conv_state + (long)tail_slot * (p.conv_k - 1) * channels + (tail_n - p.conv_lo);
 #pragma unroll
-    for (int k = 0; k < 8; ++k) tail_values[k] = tail[(long)min(k, p.conv_k - 2) * channels];
+    for (int j = 0; j < EPT; ++j) {
+      const bf16_t* tail = p.conv_state + (long)tail_slot[j] * (p.conv_k - 1) * channels + (tail_n - p.conv_lo);
 #pragma unroll
-    for (int k = 0; k < 9; ++k) tap_values[k] = p.conv_w[(long)(tail_n - p.conv_lo) * p.conv_k + min(k, p.conv_k - 1)];
+      for (int k = 0; k < TAILS; ++k) tail_values[j][k] = tail[(long)min(k, p.conv_k - 2) * channels];
+    }
+#pragma unroll
+    for (int k = 0; k < TAILS + 1; ++k) tap_values[k] = p.conv_w[(long)(tail_n - p.conv_lo) * p.conv_k + min(k, p.conv_k - 1)];
     if (p.conv_b) tap_bias = p.conv_b[tail_n - p.conv_lo];
     tail_ready = true;
   }
@@ -288,7 +298,10 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
     for (int i = 0; i < 4; ++i) red[(wave * MT + mt) * 256 + i * 64 + lane] = acc[mt][i];
   __syncthreads();
 
-  for (int index = tid; index < MT * 256; index += FG_THREADS) {
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int index = tid + j * FG_THREADS;
+    if (index >= MT * 256) continue;
     float v = 0.f;
 #pragma unroll
     for (int w = 0; w < FG_WAVES; ++w) v += red[w * MT * 256 + index];
@@ -308,21 +321,21 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
       const int channel = n - p.conv_lo;
       const int channels = p.conv_hi - p.conv_lo;
       const int taps = p.conv_k;
-      bf16_t* tail = p.conv_state + (long)(tail_ready ? tail_slot : p.slot_ids[m]) * (taps - 1) * channels + channel;
+      bf16_t* tail = p.conv_state + (long)(tail_ready ? tail_slot[j] : p.slot_ids[m]) * (taps - 1) * channels + channel;
       const bf16_t sample = (bf16_t)v;
       float sum;
       if (tail_ready) {                       // taps, bias and tail are in registers already
         sum = tap_bias;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
+        for (int k = 0; k < TAILS; ++k) {
           if (k < taps - 1) {
-            sum += tap_values[k] * (float)tail_values[k];
-            if (k > 0) tail[(long)(k - 1) * channels] = tail_values[k];       // roll the tail by one
+            sum += tap_values[k] * (float)tail_values[j][k];
+            if (k > 0) tail[(long)(k - 1) * channels] = tail_values[j][k];       // roll the tail by one
           }
         }
         float last_tap = tap_values[0];
 #pragma unroll
-        for (int k = 1; k < 9; ++k) last_tap = k == taps - 1 ? tap_values[k] : last_tap;
+        for (int k = 1; k < TAILS + 1; ++k) last_tap = k == taps - 1 ? tap_values[k] : last_tap;
         sum += last_tap * (float)sample;
       } else {
         sum = p.conv_b ? p.conv_b[channel] : 0.f;

@@ -655,6 +655,31 @@ def test_fused_gemm_norm_prologue_and_epilogues(ops, M, N, K, deltas):
         assert torch.equal(got_state[unused].cpu(), state[unused])
 
 
+@pytest.mark.parametrize("M, N, K", [(24, 200, 1024), (64, 136, 1024), (7, 96, 2048), (64, 88, 3072), (40, 64, 64)])
+def test_fused_gemm_conv_step_of_wide_batches(ops, M, N, K):
+    """The conv epilogue behind the plain prologue: more than one tile of 16 rows, four and eight
+    waves (K beyond 1,024), taps the prefetched path holds (2..4) and more than it holds (6)."""
+    x = rand(M, K, seed=330, dtype=torch.bfloat16)
+    W, b = rand(N, K, seed=331, scale=0.1, dtype=torch.bfloat16), rand(N, seed=332)
+    lo, hi = 8, N - 24
+    for taps in (4, 2, 6):
+        C = hi - lo
+        state = rand(M + 3, taps - 1, C, seed=333, dtype=torch.bfloat16)
+        slot_ids = torch.randperm(M + 3, generator=torch.Generator().manual_seed(taps))[:M].to(torch.int32)
+        conv = dict(lo=lo, hi=hi, taps=taps, weight=rand(C, taps, seed=334, scale=0.5), bias=rand(C, seed=335, scale=0.1))
+        want_state, got_state = state.clone(), state.clone().to(DEV)
+        want = torch.empty(M, N, dtype=torch.bfloat16)
+        ref_ops.fused_gemm(W, b, want, x=x, epilogue=ref_ops.EPI_CONV, conv=dict(conv, state=want_state, slot_ids=slot_ids))
+        got = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        ops.fused_gemm(W.to(DEV), b.to(DEV), got, x=x.to(DEV), epilogue=ops.EPI_CONV,
+                       conv=dict(lo=lo, hi=hi, taps=taps, weight=conv["weight"].to(DEV), bias=conv["bias"].to(DEV),
+                                 state=got_state, slot_ids=slot_ids.to(DEV)))
+        close(got, want, torch.bfloat16, 8.0)
+        close(got_state, want_state, torch.bfloat16, 8.0)
+        unused = [slot for slot in range(M + 3) if slot not in slot_ids.tolist()]
+        assert torch.equal(got_state[unused].cpu(), state[unused])
+
+
 @pytest.mark.parametrize("Hq, Hkv, dh, H, P, N, G, page_size, window, rotary, gated", [
     (8, 2, 64, 24, 64, 128, 1, 16, None, 64, False), (12, 2, 128, 6, 40, 256, 2, 16, None, 128, True),
     (4, 4, 64, 3, 24, 40, 3, 8, 100, 32, False), (8, 1, 64, 5, 7, 9, 1, 32, None, 0, False)])
