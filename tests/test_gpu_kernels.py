@@ -739,6 +739,52 @@ def test_mixer_decode_against_the_separate_kernels(ops, Hq, Hkv, dh, H, P, N, G,
         close(torch.nan_to_num(got_pool.float()), torch.nan_to_num(want_pool.float()), dtype, 4.0)
 
 
+@pytest.mark.parametrize("M, Hq, Hkv, dh, H, P, N, G", [(40, 8, 2, 64, 24, 64, 128, 1), (48, 12, 2, 128, 24, 128, 256, 1),
+                                                      (64, 4, 2, 64, 12, 32, 64, 3), (30, 4, 2, 64, 20, 24, 128, 2)])
+def test_mixer_decode_of_wide_batches(ops, M, Hq, Hkv, dh, H, P, N, G):
+    """So many single-token lanes that a state-space workgroup takes several rows per thread group
+    (and rows of more than one head where a head has few): the state sizes of the benchmark shapes,
+    a head size that is no multiple of a workgroup's rows, groups of heads."""
+    dtype = torch.bfloat16
+    page_size = 16
+    lengths = [1 + (7 * lane) % 45 for lane in range(M)]
+    pool, table = paged_setup(lengths, page_size, Hkv, dh, dtype, seed=13)
+    for lane, length in enumerate(lengths):
+        fill_cache(pool, table, lane, rand(length, Hkv, dh, seed=600 + lane, dtype=dtype),
+                   rand(length, Hkv, dh, seed=700 + lane, dtype=dtype), page_size)
+    E, GN = H * P, G * N
+    q_col, k_col, v_col = 0, Hq * dh, (Hq + Hkv) * dh
+    z_col = (Hq + 2 * Hkv) * dh
+    x_col, dt_col = z_col + E, z_col + 2 * E + 2 * GN
+    u = rand(M, -(-(dt_col + H) // 8) * 8, seed=610, dtype=dtype)
+    positions = i32([length - 1 for length in lengths])
+    slot_mapping = i32([int(table[lane, (length - 1) // page_size]) * page_size + (length - 1) % page_size
+                        for lane, length in enumerate(lengths)])
+    inv_freq = torch.tensor([1.0 / (1e4 ** (i / dh)) for i in range(0, dh, 2)], dtype=torch.float64).float()
+    slot_ids = torch.randperm(M + 2, generator=torch.Generator().manual_seed(6))[:M].to(torch.int32)
+    state = rand(M + 2, H, P, N, seed=611, scale=0.5)
+    dt_bias, A, D = rand(H, seed=612) - 2.0, -(rand(H, seed=613).abs() + 0.1), rand(H, seed=614)
+    common = dict(num_heads=Hq, num_kv_heads=Hkv, head_dim=dh, q_col=q_col, k_col=k_col, v_col=v_col,
+                  rotary_dim=dh, scale=0.11, window=None, max_seq_len=64, ssm_heads=H, ssm_head_dim=P,
+                  state_size=N, num_groups=G, z_col=z_col, x_col=x_col, dt_col=dt_col)
+    want_pool, want_state = pool.clone(), state.clone()
+    want_out = torch.zeros(M, Hq * dh + E, dtype=dtype)
+    ref_ops.mixer_decode(u, inv_freq=inv_freq, k_cache=views(want_pool, page_size)[0], v_cache=views(want_pool, page_size)[1],
+                         block_tables=table, positions=positions, slot_mapping=slot_mapping, dt_bias=dt_bias, A=A, D=D,
+                         ssm_state=want_state, slot_ids=slot_ids, out=want_out, ssm_y=None, **common)
+    got_pool, got_state = pool.clone().to(DEV), state.clone().to(DEV)
+    got_out = torch.zeros(M, Hq * dh + E, dtype=dtype, device=DEV)
+    ops.mixer_decode(u.to(DEV), inv_freq=inv_freq.to(DEV), k_cache=views(got_pool, page_size)[0],
+                     v_cache=views(got_pool, page_size)[1], block_tables=table.to(DEV), positions=positions.to(DEV),
+                     slot_mapping=slot_mapping.to(DEV), dt_bias=dt_bias.to(DEV), A=A.to(DEV), D=D.to(DEV),
+                     ssm_state=got_state, slot_ids=slot_ids.to(DEV), out=got_out, ssm_y=None, **common)
+    close(got_out[:, :Hq * dh], want_out[:, :Hq * dh], dtype, 2.0)
+    close(got_state, want_state, torch.float32, max(1.0, want_state.abs().max().item()))
+    close(got_out[:, Hq * dh:], want_out[:, Hq * dh:], dtype, max(1.0, want_out.float().abs().max().item()))
+    unused = [slot for slot in range(M + 2) if slot not in slot_ids.tolist()]
+    assert torch.equal(got_state[unused].cpu(), state[unused])
+
+
 def test_mixer_decode_over_a_long_context(ops):
     """Contexts of 5 000 and 9 000 tokens (10 and 18 runs of 512 keys: more than the merge takes
     at once) beside a short one; one far key per long request is made to dominate, so a run that
