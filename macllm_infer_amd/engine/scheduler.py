@@ -10,9 +10,12 @@ Each round (reference: ``ServingScheduler::drive_once``, src/engine.rs:1938-1988
      dropped and the step retried (:2145-2149); if a single lane cannot fit, that request
      alone fails with ``resource_exhausted`` and gives back what it holds (:2150-2153,
      :2205-2231).  There is no preemption or swap;
-  4. sample for the lanes whose last prompt token or decoded token ran; a stop token ends
-     the request without being emitted, ``max_new_tokens`` ends it with the token emitted
-     (src/generation.rs:1221-1263);
+  4. sample for the lanes whose last prompt token or decoded token ran; a cancelled request ends
+     before its token is emitted, a stop token ends the request without being emitted, a
+     ``False`` from the caller's ``on_token`` ends it after the token, ``max_new_tokens`` ends
+     it with the token emitted (src/generation.rs:1217-1263).  A request cancelled while it
+     waits never starts; one cancelled between rounds gives back what it holds before the next
+     (src/engine.rs:1136-1143, 1668-1672, 1753-1765);
   5. finished requests give back pages and slot; visited ones go to the back of the line.
 """
 from __future__ import annotations
@@ -52,7 +55,8 @@ class Request:
     params: SamplingParams
     generated: List[int] = field(default_factory=list)
     cursor: int = 0                        # prompt tokens already in the cache
-    finish_reason: Optional[str] = None    # "stop", "length", "resource_exhausted", "rejected: ..."
+    finish_reason: Optional[str] = None    # "stop", "length", "cancelled", "resource_exhausted", "rejected: ..."
+    cancelled: bool = False
     submitted_at: float = 0.0
     first_token_at: Optional[float] = None
     finished_at: Optional[float] = None
@@ -65,6 +69,10 @@ class Request:
     def prefilling(self) -> bool:
         return self.cursor < len(self.prompt)
 
+    def cancel(self) -> None:
+        """Ask for the request to end; the scheduler honours it at its next decision about it."""
+        self.cancelled = True
+
 
 class QueueFull(RuntimeError):
     pass
@@ -74,7 +82,9 @@ class Scheduler:
     def __init__(self, engine, sampler, config: Optional[EngineConfig] = None,
                  stop_token_ids: Sequence[int] = (), on_token: Optional[Callable] = None):
         """``engine``: add_request / finish / step(lanes) / cache.can_ever_fit / vocab_size /
-        max_context.  ``sampler``: sample(logits, rows) -> tokens."""
+        max_context.  ``sampler``: sample(logits, rows) -> tokens.  ``on_token(request, token)`` is
+        called for every emitted token; returning ``False`` ends that request there (its own stop
+        condition), ``request.cancel()`` ends it before its next token."""
         self.engine = engine
         self.sampler = sampler
         self.config = config or EngineConfig()
@@ -97,6 +107,14 @@ class Scheduler:
     def has_work(self) -> bool:
         return bool(self.queue or self.active)
 
+    def cancel(self, request_id: Hashable) -> bool:
+        """Cancel a waiting or live request; False if there is no such request (any more)."""
+        for request in list(self.queue) + list(self.active):
+            if request.request_id == request_id:
+                request.cancel()
+                return True
+        return False
+
     # ------------------------------------------------------------------ one round
     def _reject(self, request: Request, why: str) -> None:
         request.finish_reason = f"rejected: {why}"
@@ -104,10 +122,16 @@ class Scheduler:
         self.finished[request.request_id] = request
 
     def _admit(self) -> None:
+        for request in [request for request in self.active if request.cancelled]:
+            self._finish(request, "cancelled")
         while self.queue and len(self.active) < self.config.max_active_sequences:
             request = self.queue.popleft()
             needed = len(request.prompt) + request.params.max_new_tokens - 1
-            if not request.prompt:
+            if request.cancelled:                      # never starts, holds nothing
+                request.finish_reason = "cancelled"
+                request.finished_at = time.perf_counter()
+                self.finished[request.request_id] = request
+            elif not request.prompt:
                 self._reject(request, "prompt must contain at least one token")
             elif any(not (0 <= token < self.engine.vocab_size) for token in request.prompt):
                 self._reject(request, "input contains a token ID outside the model vocabulary")
@@ -183,6 +207,9 @@ class Scheduler:
 
     def _complete(self, request: Request, token: int, now: float) -> None:
         params = request.params
+        if request.cancelled:                        # before the token becomes visible
+            self._finish(request, "cancelled")
+            return
         stops = self.stop_token_ids | set(params.stop_token_ids)
         if not params.ignore_eos and token in stops:
             self._finish(request, "stop")            # the stop token is not emitted
@@ -190,9 +217,9 @@ class Scheduler:
         if request.first_token_at is None:
             request.first_token_at = now
         request.generated.append(token)
-        if self.on_token is not None:
-            self.on_token(request, token)
-        if len(request.generated) >= params.max_new_tokens:
+        if self.on_token is not None and self.on_token(request, token) is False:
+            self._finish(request, "stop")            # the caller's own stop condition; the token stays emitted
+        elif len(request.generated) >= params.max_new_tokens:
             self._finish(request, "length")
 
     def run(self, on_round: Optional[Callable] = None) -> Dict[Hashable, Request]:

@@ -176,3 +176,47 @@ def test_scheduler_settings_are_checked():
     defaults = SamplingParams()                # the reference's defaults, src/sampling.rs:23-33
     assert (defaults.temperature, defaults.top_k, defaults.top_p, defaults.repetition_penalty, defaults.seed,
             defaults.max_new_tokens) == (0.7, 20, 0.8, 1.1, 42, 128)
+
+
+def test_cancelled_requests_never_start_or_stop_before_their_next_token():
+    """A request cancelled while it waits holds nothing and never runs; one cancelled while it
+    decodes ends before its next token is emitted and gives back what it holds; the others go on
+    (src/engine.rs:1668-1672, src/generation.rs:1217-1220)."""
+    engine = FakeEngine()
+    params = SamplingParams(max_new_tokens=6, temperature=0.0)
+
+    def on_token(request, token):
+        if request.request_id == 0 and len(request.generated) == 2:
+            request.cancel()
+
+    scheduler = Scheduler(engine, ArgmaxSampler(), EngineConfig(max_active_sequences=2), (), on_token)
+    for index, prompt in enumerate([[1, 2, 3], [10, 11], [20, 21]]):
+        scheduler.submit(index, prompt, params)
+    assert scheduler.cancel(2) and not scheduler.cancel("nobody")
+    finished = scheduler.run()
+    assert finished[2].finish_reason == "cancelled" and finished[2].generated == []
+    assert all(request != 2 for call in engine.calls for request, _, _, _ in call)
+    assert finished[0].finish_reason == "cancelled" and finished[0].generated == [4, 5]     # the third was not emitted
+    assert finished[1].finish_reason == "length" and finished[1].generated == [12, 13, 14, 15, 16, 17]
+    assert engine.lengths == {}
+
+
+def test_a_request_cancelled_between_rounds_is_finished_before_the_next():
+    engine = FakeEngine()
+    scheduler = Scheduler(engine, ArgmaxSampler(), EngineConfig(scheduler_token_budget=2, prefill_token_quantum=2))
+    scheduler.submit("a", [1, 2, 3, 4, 5, 6], SamplingParams(max_new_tokens=4, temperature=0.0))
+    scheduler.step()
+    assert engine.lengths == {"a": 2}
+    assert scheduler.cancel("a")
+    done = scheduler.step()
+    assert [request.finish_reason for request in done] == ["cancelled"] and engine.lengths == {} and len(engine.calls) == 1
+
+
+def test_the_callers_own_stop_condition_ends_a_request_after_the_token():
+    """``on_token`` returning False is the caller's stop sequence: the token stays emitted and the
+    reason is "stop" (src/generation.rs:1244-1254)."""
+    engine = FakeEngine()
+    scheduler = Scheduler(engine, ArgmaxSampler(), EngineConfig(), (), lambda request, token: token != 7)
+    scheduler.submit("a", [4], SamplingParams(max_new_tokens=10, temperature=0.0))
+    finished = scheduler.run()
+    assert finished["a"].generated == [5, 6, 7] and finished["a"].finish_reason == "stop"
