@@ -63,7 +63,7 @@ class Engine:
         self.spec = self.config.to_model_spec()
         self.spec.validate()
         if check_device:
-            kernel_build.ensure_modules(DecoderModel.kernel_modules(self.spec))
+            kernel_build.ensure_modules(DecoderModel.kernel_modules(self.spec) + list(kernel_build.HOST_MODULES))
         source.apply_aliases(self.spec.tensor_aliases, root_prefix=self.spec.root_namespace)
         bound = bind(source, DecoderModel.expected_tensors(self.spec))
         source.close()
