@@ -190,6 +190,32 @@ def test_greedy_generation_through_the_entry_point(tmp_path, name, dtype):
     assert llm.engine.cache.stats()["live_requests"] == 0
 
 
+def test_generation_when_pages_run_out(tmp_path):
+    """Seven requests on a cache of six pages, three live at a time: lanes are dropped from steps
+    and retried, pages and slots are used again, and a request that cannot grow while the others
+    hold their pages fails alone.  Whatever finishes says what the plain model says; whatever
+    fails said so up to there; nothing stays behind."""
+    from macllm_infer_amd import LLM, EngineConfig, SamplingParams
+    folder = tiny_configs.make_model_dir("A", tmp_path)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    prompts = [tokens_for(cfg["vocab_size"], length, 90 + length) for length in (20, 37, 9, 30, 41, 16, 200)]
+    llm = LLM(folder, dtype="float32", kv_cache_block_tokens=16, kv_cache_capacity_tokens=96,
+              engine_config=EngineConfig(max_active_sequences=3, scheduler_token_budget=40, prefill_token_quantum=13))
+    params = SamplingParams(max_new_tokens=10, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0)
+    results = llm.generate(prompts, params)
+    reasons = [result.finish_reason for result in results]
+    assert reasons[-1].startswith("rejected") and "cache capacity" in reasons[-1]      # could never fit
+    assert reasons.count("length") >= 3 and set(reasons[:-1]) <= {"length", "resource_exhausted"}
+    for prompt, result in zip(prompts[:-1], results[:-1]):
+        want = plain_impl.greedy_generate(cfg, tensors, prompt, 10)
+        assert result.token_ids == want[:len(result.token_ids)]
+        assert len(result.token_ids) == 10 or result.finish_reason == "resource_exhausted"
+    stats = llm.engine.cache.stats()
+    assert stats["live_requests"] == 0 and stats["free_slots"] == stats["total_slots"]
+    assert all(group["free_pages"] == group["total_pages"] for group in stats["groups"])
+    llm.engine.cache.check()
+
+
 def test_seeded_sampling_through_the_entry_point(tmp_path):
     """Config B's workload: five requests of 1/7/24/40/63 tokens, prompts cut into portions of
     11, temperature 0.8 with seeded draws, 20 decode steps, pages of 8."""
