@@ -93,7 +93,7 @@ class DecoderModel:
                            deltas=residual.pending, norm_weight=self.final_norm.weight, eps=self.final_norm.eps)
             return logits
         normed = self.final_norm.forward(residual, rows=step.want_rows)
-        raw = ops.linear(normed, self.lm_head, None)
+        raw = ops.linear(normed, self.lm_head, None, keep_float32=True)      # the sums as they are, not rounded to bfloat16
         ops.scale_to_f32(raw, spec.logit_multiplier, logits)
         return logits
 

@@ -218,8 +218,10 @@ def scale_to_f32(values: torch.Tensor, multiplier: float, out: torch.Tensor) -> 
 
 
 # --------------------------------------------------------------------------- matrix products
-def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
-    """x [M, K] . weight[N, K]^T (+ bias float32 [N]) -> [M, N] in x's dtype.
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], keep_float32: bool = False) -> torch.Tensor:
+    """x [M, K] . weight[N, K]^T (+ bias float32 [N]) -> [M, N] in x's dtype, or, with
+    ``keep_float32`` and no bias, in float32 whatever the operands are (the library writes its
+    float32 sums without rounding them to bfloat16: the logits).
 
     float32 operands: the hand-written float32 FMA kernel (true 32-bit).  bfloat16 operands:
     the BLAS library with float32 accumulation.  A float32 weight with bfloat16 activations
@@ -236,8 +238,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) 
             _need(bias.dtype == torch.float32 and bias.numel() == N, "linear: bias must be float32 [N]")
         _check(_fn("gemm", "mi_gemm_f32")(_p(xf), ldx, _p(weight), ldw, _p(bias), _p(out), N, M, N, K, _stream()),
                "gemm_f32", f"(M={M}, N={N}, K={K})")
-        return out if x.dtype == torch.float32 else out.to(x.dtype)
+        return out if x.dtype == torch.float32 or keep_float32 else out.to(x.dtype)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear: operands must share a dtype")
+    if keep_float32:
+        _need(bias is None, "linear: float32 results of bfloat16 operands come without a bias")
+        return torch.mm(x, weight.t(), out_dtype=torch.float32)
     if bias is None:
         return torch.matmul(x, weight.t())
     return torch.addmm(bias.to(torch.bfloat16), x, weight.t())

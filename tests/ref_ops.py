@@ -51,11 +51,11 @@ def scale_to_f32(values, multiplier, out):
     out.copy_(_f(values).reshape(out.shape) * multiplier)
 
 
-def linear(x, weight, bias):
+def linear(x, weight, bias, keep_float32=False):
     y = _f(x) @ _f(weight).T
     if bias is not None:
         y = y + bias
-    return y.to(x.dtype)
+    return y if keep_float32 else y.to(x.dtype)
 
 
 def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, rotary_dim, slot_mapping,
