@@ -210,3 +210,22 @@ def test_a_tensor_under_both_spellings_and_a_stranger_are_reported_by_their_stor
     assert not caught.value.missing
     assert "model.layers.0.feed_forward.router.weight" in caught.value.unexpected
     assert any("pre_ff_layernorm" in name and "ffn_norm" in name for name in caught.value.unexpected)
+
+
+def test_command_line_writes_and_inspects_a_random_model(tmp_path, capsys):
+    """``random-weights`` writes a model folder from a config.json and a seed (the same tensors as the
+    Python call with that seed); ``inspect`` prints the geometry the cache manager sizes itself by."""
+    from macllm_infer_amd import cli
+    (tmp_path / "config.json").write_text(json.dumps(tiny_configs.TINY_B))
+    folder = tmp_path / "model"
+    assert cli.main(["random-weights", "--config", str(tmp_path / "config.json"), "--seed", "3", "--out", str(folder),
+                     "--dtype", "f32"]) == 0
+    config = load_config(str(folder))
+    assert config == tiny_configs.config("B")
+    bound = bind(WeightSource.from_dir(str(folder)), DecoderModel.expected_tensors(config.to_model_spec()))
+    assert all(torch.equal(bound[name], tensor) for name, tensor in random_tensors(config, 3, torch.float32).items())
+    capsys.readouterr()
+    assert cli.main(["inspect", "-m", str(folder)]) == 0
+    report = json.loads(capsys.readouterr().out)
+    assert report["layers"] == 3 and report["kv_bytes_per_token_bf16"] == config.kv_bytes_per_token(2)
+    assert report["fixed_state_bytes_per_request_f32"] == config.fixed_state_bytes(4)
