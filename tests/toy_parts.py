@@ -1,6 +1,7 @@
 """Toy parts for the tests of the framework's generality: a mixer with state of its own, a
 position encoding that is no rotation, a feed-forward that routes each token to two of its
-experts, and a toy architecture that uses them together with a
+experts, a norm that centres its rows, an arrangement of a layer with a norm after the mixer, and a
+toy architecture that uses them together with a
 windowed attention layer, a layer that runs twice and a run that reads another run's cache.
 They are registered from here, without a change to the package, and never become a model."""
 from dataclasses import dataclass
@@ -43,10 +44,21 @@ class RoutedSpec:
         assert self.experts >= 2 and self.inner > 0
 
 
+@dataclass(frozen=True)
+class CentredNormSpec:
+    """A toy norm: y = (x - mean) / sqrt(var + eps) * w + b."""
+    eps: float
+    kind: str = "toy_centred_norm"
+
+    def validate(self):
+        assert self.eps > 0
+
+
 @dataclass
 class ToyConfig:
     """A toy architecture: layer 0 = attention (toy position encoding) and the decay mixer in
-    parallel, layer 1 = windowed attention with partial RoPE and the routed feed-forward.  ``raw["schedule"]`` lists
+    parallel, layer 1 = windowed attention with partial RoPE and the routed feed-forward, its norms
+    the centring toy norm, arranged with one more norm on the mixer's output (``toy_sandwich``).  ``raw["schedule"]`` lists
     (layer, entry whose cache is read or None) in running order."""
     raw: dict
     architecture_names = ("ToyForTests",)
@@ -71,7 +83,8 @@ class ToyConfig:
         ffn = SwiGLUSpec(intermediate_size=48)
         layers = (LayerSpec(prefix="model.layers.0", ffn=ffn, mixer_norm=norm, ffn_norm=norm,
                             mixers=(MixerSlot("self_attn", full), MixerSlot("decay", DecayMixerSpec(hidden, raw["decay"])))),
-                  LayerSpec(prefix="model.layers.1", ffn=RoutedSpec(raw["experts"], 24), mixer_norm=norm, ffn_norm=norm,
+                  LayerSpec(prefix="model.layers.1", ffn=RoutedSpec(raw["experts"], 24), mixer_norm=CentredNormSpec(1e-4),
+                            ffn_norm=CentredNormSpec(1e-4), arrangement="toy_sandwich",
                             mixers=(MixerSlot("self_attn", windowed),)))
         schedule = tuple(ScheduleEntry(layer=layer, kv_from=source) for layer, source in raw["schedule"])
         return ModelSpec(architecture="ToyForTests", hidden_size=hidden, vocab_size=raw["vocab"], max_context=512,
@@ -81,7 +94,8 @@ class ToyConfig:
 def register_toys():
     from macllm_infer_amd.cache import StateNeed
     from macllm_infer_amd.config import register_architecture
-    from macllm_infer_amd.parts import FeedForward, Mixer, PositionEncoding, register_part
+    from macllm_infer_amd.parts import (FeedForward, Mixer, Part, PositionEncoding, part_class, register_arrangement,
+                                        register_part)
     from macllm_infer_amd.weights import Expect
 
     @register_part("toy_decay")
@@ -140,7 +154,67 @@ def register_toys():
         def forward(self, x):
             return routed_feed_forward(x.float(), self.router, self.up, self.down).to(x.dtype)
 
+    @register_part("toy_centred_norm")
+    class CentredNorm(Part):
+        @classmethod
+        def expected_tensors(cls, spec, prefix, hidden_size):
+            return [Expect(f"{prefix}.weight", ((hidden_size,),), init="norm"),
+                    Expect(f"{prefix}.bias", ((hidden_size,),), init="bias")]
+
+        def __init__(self, spec, prefix, tensors, build):
+            self.eps, self.dtype = spec.eps, build.dtype
+            self.weight = tensors[f"{prefix}.weight"].float().to(build.device)
+            self.bias = tensors[f"{prefix}.bias"].float().to(build.device)
+
+        def forward(self, residual, rows=None):
+            for delta in residual.pending:                  # a norm folds the branch outputs into the stream
+                residual.h += delta.float()
+            residual.pending = []
+            x = residual.h if rows is None else residual.h[rows.long()]
+            return centred_norm(x, self.weight, self.bias, self.eps).to(self.dtype)
+
+    @register_arrangement("toy_sandwich")
+    class Sandwich:
+        """h += post(mixer(pre(h))); h += ffn(norm(h)): one mixer, and a norm of its own
+        (``<prefix>.post_norm``, of the kind of the layer's mixer norm) on the mixer's output."""
+
+        @classmethod
+        def parts(cls, layer):
+            norm = part_class(layer.mixer_norm)
+            slot = layer.mixers[0]
+            return [(norm, layer.mixer_norm, f"{layer.prefix}.{layer.mixer_norm_name}"),
+                    (part_class(slot.spec), slot.spec, f"{layer.prefix}.{slot.name}"),
+                    (norm, layer.mixer_norm, f"{layer.prefix}.post_norm"),
+                    (part_class(layer.ffn_norm), layer.ffn_norm, f"{layer.prefix}.{layer.ffn_norm_name}"),
+                    (part_class(layer.ffn), layer.ffn, f"{layer.prefix}.{layer.ffn_name}")]
+
+        @classmethod
+        def expected_tensors(cls, layer, hidden_size):
+            return [expect for kind, spec, prefix in cls.parts(layer)
+                    for expect in kind.expected_tensors(spec, prefix, hidden_size)]
+
+        @classmethod
+        def kernel_modules(cls, layer):
+            return [module for kind, _, _ in cls.parts(layer) for module in kind.kernel_modules]
+
+        def __init__(self, layer, tensors, build):
+            self.pre, self.mixer, self.post, self.ffn_norm, self.ffn = (
+                kind(spec, prefix, tensors, build) for kind, spec, prefix in self.parts(layer))
+            self.mixers = [(layer.mixers[0].name, self.mixer)]       # what the model asks caches for
+            self.graph_safe = False
+
+        def forward(self, residual, step, caches):
+            from macllm_infer_amd.parts.base import Residual
+            mixed = self.mixer.forward(self.pre.forward(residual), step, caches[self.mixers[0][0]])
+            residual.pending = [self.post.forward(Residual(mixed.float()))]
+            residual.pending = [self.ffn.forward(self.ffn_norm.forward(residual))]
+
     register_architecture(ToyConfig)
+
+
+def centred_norm(x, weight, bias, eps):
+    centred = x - x.mean(dim=-1, keepdim=True)
+    return centred / torch.sqrt(centred.pow(2).mean(dim=-1, keepdim=True) + eps) * weight + bias
 
 
 def routed_feed_forward(x, router, up, down):
@@ -164,7 +238,11 @@ def toy_plain_logits(raw, tensors, tokens):
     caches = {}
     for index, (layer, source) in enumerate(raw["schedule"]):
         p = f"model.layers.{layer}."
-        n = plain_impl.rms_norm(h, tensors[p + "attn_norm.weight"], 1e-5)
+        if layer == 0:
+            norm = lambda x, name: plain_impl.rms_norm(x, tensors[p + name + ".weight"], 1e-5)
+        else:
+            norm = lambda x, name: centred_norm(x, tensors[p + name + ".weight"].float(), tensors[p + name + ".bias"].float(), 1e-4)
+        n = norm(h, "attn_norm")
         w = {name[len(p + "self_attn."):]: value for name, value in tensors.items() if name.startswith(p + "self_attn.")}
         q = plain_impl.linear(n, w["q_proj.weight"], None).view(T, 4, 16)
         k = plain_impl.linear(n, w["k_proj.weight"], None).view(T, 2, 16)
@@ -191,8 +269,10 @@ def toy_plain_logits(raw, tensors, tokens):
                 s = raw["decay"] * s + projected[t]
                 rows.append(s)
             mixed = mixed + torch.stack(rows)
+        else:
+            mixed = norm(mixed, "post_norm")             # the sandwich: a norm on the mixer's output
         h = h + mixed
-        f = plain_impl.rms_norm(h, tensors[p + "ffn_norm.weight"], 1e-5)
+        f = norm(h, "ffn_norm")
         if layer == 0:
             h = h + plain_impl.swiglu_mlp(f, {name[len(p + "mlp."):]: value for name, value in tensors.items()
                                               if name.startswith(p + "mlp.")})
@@ -235,6 +315,7 @@ def exercise(schedule, device, check_device):
     config = ToyConfig(raw)
     tensors = random_tensors(config, 5, torch.float32, "unit")
     assert "model.layers.0.decay.w.weight" in tensors and tensors["model.layers.1.mlp.up.weight"].shape == (5, 24, 32)
+    assert "model.layers.1.post_norm.bias" in tensors and "model.layers.0.post_norm.weight" not in tensors
     engine = Engine(config=config, tensors=tensors, dtype="float32", device=device, kv_cache_block_tokens=4,
                     kv_cache_capacity_tokens=160, max_active_sequences=3, check_device=check_device)
     windows = sorted(str(group.need.window) for group in engine.cache.groups)
