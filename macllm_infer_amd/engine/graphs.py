@@ -3,7 +3,11 @@
 A step whose lanes all hold one token is launch-bound: hundreds of small kernels.  For
 each batch-size bucket the forward pass over a ``StaticStep`` is captured once and
 replayed; only the index arrays are rewritten between replays.  Buckets are powers of
-two; missing lanes are padding on the cache's scratch page and slot.
+two; missing lanes are padding on the cache's scratch page and slot.  A graph also fixes how
+long a context it can hold (the width of its block tables, the runs of keys its attention is
+launched for), so graphs come in buckets of context length as well, powers of two from 2,048
+tokens up to the longest the cache can hold: a model that allows 262,144 tokens does not pay
+for them while its requests are short.
 
 Prompt portions are launch-bound too once the kernels are fast (a portion of 2,048 tokens is
 some 700 launches).  A scheduler cuts long prompts into portions of one size, so the shape of
@@ -29,13 +33,16 @@ def bucket_for(lanes: int) -> int:
     return bucket
 
 
+CONTEXT_BUCKET_FROM = 2048
+
+
 class DecodeGraphs:
     def __init__(self, model, cache, device, max_seq_len: int):
         self.model = model
         self.cache = cache
         self.device = device
         self.max_seq_len = max_seq_len
-        self._graphs: Dict[int, tuple] = {}
+        self._graphs: Dict[tuple, tuple] = {}
         self._portion_graphs: "OrderedDict[tuple, tuple]" = OrderedDict()
         self._portion_recent: deque = deque(maxlen=self.PORTION_RECENT)
         self.counts = {"decode_replays": 0, "portion_replays": 0, "portion_captures": 0, "portion_eager": 0}
@@ -44,6 +51,14 @@ class DecodeGraphs:
     PORTION_GRAPHS = 8
     PORTION_RECENT = 32            # steps with portions whose shapes are remembered
     PORTION_SIGHTINGS = 3          # sightings among them before a shape is captured
+
+    def context_bucket(self, lowered: LoweredLanes) -> int:
+        """The smallest bucket of context length that holds every lane of the step after it ran."""
+        longest = int((self.cache.lengths_of(lowered.slots) + lowered.lengths).max())
+        bucket = CONTEXT_BUCKET_FROM
+        while bucket < longest:
+            bucket <<= 1
+        return min(bucket, self.max_seq_len)
 
     def run_portion(self, lanes: Sequence[Lane], lowered: LoweredLanes) -> Optional[torch.Tensor]:
         """Logits of a step with prompt portions from a captured graph of its shape, or None when
@@ -63,7 +78,8 @@ class DecodeGraphs:
         # padding lanes stand last, as single tokens whose logits are computed and dropped
         lengths = tuple(len(lane.tokens) for lane in ordered) + (1,) * padding
         wants = tuple(tuple(lane.want) for lane in ordered) + ((0,),) * padding
-        key = (lengths, wants)
+        context = self.context_bucket(lowered)
+        key = (lengths, wants, context)
         entry = self._portion_graphs.get(key)
         if entry is None:
             self._portion_recent.append(key)
@@ -74,7 +90,7 @@ class DecodeGraphs:
             for length, want in zip(lengths, wants):
                 rows += [first + place for place in want]
                 first += length
-            static = StaticStep(self.cache, len(lengths), self.max_seq_len, self.device, lengths=lengths, want_rows=rows)
+            static = StaticStep(self.cache, len(lengths), context, self.device, lengths=lengths, want_rows=rows)
             entry = self._capture(0, static, warm_runs=1)      # the libraries have seen these sizes already
             self.counts["portion_captures"] += 1
             while len(self._portion_graphs) >= self.PORTION_GRAPHS:
@@ -96,9 +112,9 @@ class DecodeGraphs:
         rows = [starts[index] + offset for index, lane in enumerate(lanes) for offset in range(len(lane.want))]
         return logits[torch.tensor(rows, dtype=torch.long, device=logits.device)] if rows else logits[:0].clone()
 
-    def _capture(self, bucket: int, static: Optional[StaticStep] = None, warm_runs: int = 2):
+    def _capture(self, bucket: int, static: Optional[StaticStep] = None, warm_runs: int = 2, context: int = 0):
         if static is None:
-            static = StaticStep(self.cache, bucket, self.max_seq_len, self.device)
+            static = StaticStep(self.cache, bucket, context or self.max_seq_len, self.device)
         # a first run outside the graph lets the libraries set themselves up; every lane is padding,
         # so only the scratch page and slot are touched
         side = torch.cuda.Stream(device=self.device)
@@ -116,10 +132,10 @@ class DecodeGraphs:
     def run(self, lanes: Sequence[Lane], lowered: LoweredLanes) -> torch.Tensor:
         """Logits [wanted, vocab] of single-token lanes (a copy: the graph's own output tensor is
         overwritten by the next replay)."""
-        bucket = bucket_for(len(lanes))
-        if bucket not in self._graphs:
-            self._graphs[bucket] = self._capture(bucket)
-        static, graph, logits = self._graphs[bucket]
+        key = (bucket_for(len(lanes)), self.context_bucket(lowered))
+        if key not in self._graphs:
+            self._graphs[key] = self._capture(key[0], context=key[1])
+        static, graph, logits = self._graphs[key]
         static.fill(lowered)
         graph.replay()
         self.counts["decode_replays"] += 1

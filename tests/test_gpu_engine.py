@@ -298,7 +298,7 @@ def test_decode_graphs_match_eager_steps(tmp_path, name, dtype):
         if turn % 7 == 6:
             live = live[:1]                                     # bucket 1
         both([(key, 1) for key in live])
-    assert set(with_graphs.graphs._graphs) == {1, 2, 4}
+    assert {lanes for lanes, _ in with_graphs.graphs._graphs} == {1, 2, 4}
     assert with_graphs.cache.stats() == eager.cache.stats()
 
 
@@ -328,13 +328,51 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
         logits = engine.step([Lane(index, [tokens[len(tokens) - 6 + turn]], [0]) for index, tokens in prompts.items()])
         for row, index in enumerate(prompts):
             got[index].append(logits[row].float().cpu())
-    assert set(engine.graphs._graphs) == {8 if requests <= 8 else 32 if requests <= 32 else 64}
+    assert {lanes for lanes, _ in engine.graphs._graphs} == {8 if requests <= 8 else 32 if requests <= 32 else 64}
     for index, tokens in prompts.items():
         want = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-6:]
         have = torch.stack(got[index])
         scale = want.abs().max().item()
         assert (have - want).abs().max().item() <= 6e-2 * scale
         assert ((have - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()).item() <= 3e-2
+
+
+def test_graphs_come_in_buckets_of_context_length():
+    """A model that allows long contexts: a short request decodes through a graph made for 2,048
+    tokens, a longer one through a graph made for 4,096 (wider block tables, more runs of keys),
+    beside each other through the wider one; all say what an engine without graphs says."""
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.weights.random_init import random_tensors
+    config = FalconH1Config.from_dict(dict(tiny_configs.TINY_C, max_position_embeddings=16384))
+    tensors = random_tensors(config, 4, torch.bfloat16, "unit")
+    make = lambda graphs: Engine(config=config, tensors=tensors, dtype="bfloat16", kv_cache_capacity_tokens=8192,
+                                 max_active_sequences=2, decode_graphs=graphs)
+    with_graphs, eager = make(True), make(False)
+    short, long = tokens_for(config.vocab_size, 40, 1), tokens_for(config.vocab_size, 2100, 2)
+
+    def both(lanes):
+        got, want = with_graphs.step(lanes).float().cpu(), eager.step(lanes).float().cpu()
+        assert got.shape == want.shape
+        if got.numel():
+            assert (got - want).abs().max() <= 3e-2 * max(1.0, want.abs().max().item())
+
+    for engine in (with_graphs, eager):
+        engine.add_request("short")
+        engine.add_request("long")
+    both([Lane("short", short[:30], [29])])
+    for token in short[30:35]:
+        both([Lane("short", [token], [0])])
+    assert set(with_graphs.graphs._graphs) == {(1, 2048)}
+    both([Lane("long", long[:2050], [2049])])
+    for token in long[2050:2055]:
+        both([Lane("long", [token], [0])])
+    assert set(with_graphs.graphs._graphs) == {(1, 2048), (1, 4096)}
+    for first, second in zip(short[35:40], long[2055:2060]):
+        both([Lane("short", [first], [0]), Lane("long", [second], [0])])
+    assert set(with_graphs.graphs._graphs) == {(1, 2048), (1, 4096), (2, 4096)}
+    both([Lane("short", [short[39]], [0])])                               # and back through the narrow one
+    assert with_graphs.graphs.counts["decode_replays"] == 16
 
 
 @pytest.mark.parametrize("name, dtype", [("B", "float32"), ("C", "bfloat16")])
