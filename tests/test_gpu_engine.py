@@ -615,3 +615,32 @@ def test_layers_of_the_benchmark_shapes_match_the_plain_model(shape, layers, voc
         got = torch.cat(rows[name]).numpy()
         assert got.shape == want.shape, name
         assert bfloat16_close(got, want), f"{name}: {np.abs(got - want).max():.3e} of {np.abs(want).max():.2f}"
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_float32_logits_are_the_same_bits_however_the_tokens_are_cut(tmp_path, name):
+    """Every float32 kernel sums in an order that the sizes alone fix, so a position's logits are
+    bit for bit the same whole, in portions, token by token and beside another request."""
+    from macllm_infer_amd import Engine, Lane
+    folder = tiny_configs.make_model_dir(name, tmp_path)
+    cfg, _ = plain_impl.load_model_dir(folder)
+    tokens, other = tokens_for(cfg["vocab_size"], 47, 31), tokens_for(cfg["vocab_size"], 29, 32)
+    engine = Engine(folder, dtype="float32", kv_cache_block_tokens=8, kv_cache_capacity_tokens=256, max_active_sequences=3)
+    engine.add_request("whole")
+    whole = engine.step([Lane("whole", tokens, list(range(47)))]).cpu()
+    engine.finish("whole")
+    for cuts in ([5] * 9 + [2], [1] * 47, [30, 16, 1]):
+        engine.add_request("cut")
+        engine.add_request("other")
+        rows, first, fed = [], 0, 0
+        for count in cuts:
+            lanes = [Lane("cut", tokens[first:first + count], list(range(count)))]
+            if fed < len(other):                                   # a neighbour whose lane changes from step to step
+                take = min(1 + first % 4, len(other) - fed)
+                lanes.insert(0, Lane("other", other[fed:fed + take], [take - 1]))
+                fed += take
+            rows.append(engine.step(lanes).cpu()[len(lanes) - 1:])
+            first += count
+        assert torch.equal(torch.cat(rows), whole), f"cuts {cuts[:3]}..."
+        engine.finish("cut")
+        engine.finish("other")
