@@ -460,8 +460,10 @@ extern "C" int mi_fused_gemm_supported(int pro, int M, int K) {
 // ---------------------------------------------------------------- mixer decode
 #define MX_THREADS 512
 #define MX_WAVES 8
-#define MX_MAX_PAGES 80        // page ids of one run of keys (at most MX_SPLIT_KEYS / 8 + 2)
-#define MX_SPLIT_KEYS 512
+#define MX_MAX_PAGES 132       // page ids of one run of keys (at most MX_SPLIT_MOST / 8 + 2)
+#define MX_SPLIT_LEAST 256     // keys of one attention workgroup: between these two, see mi_mixer_split_keys
+#define MX_SPLIT_MOST 1024
+#define MX_SPLIT_BLOCKS 128    // attention workgroups a step should at least have before its runs grow
 #define MX_SCAN_PER_THREAD 8
 #define MX_FEW_BLOCKS 512       // state-space workgroups of a step up to which each takes one row per thread group
 
@@ -834,6 +836,26 @@ __global__ void __launch_bounds__(MX_THREADS) mixer_decode_kernel(MixerParams p)
     mixer_ssm_block<true, 8>(p, blockIdx.x - p.attention_blocks);
 }
 
+// Keys of one attention workgroup (a run).  Long runs pay the start of a workgroup (position, page ids,
+// then keys: three round trips) and the merge of the runs less often; short runs give a small step more
+// workgroups.  Measured on one MI355X (mixer + merge of a layer, head size 64, 2 kv heads; runs of
+// 256 / 512 / 1,024 keys): 1 token at 2,048 keys 12.4 / 12.8 / 14.9 us, 8 tokens at 2,048 keys
+// 13.9 / 14.3 / 17.2, 8 tokens at 8,192 keys 23.6 / 20.6 / 18.7, 64 tokens at 2,048 keys 49.7 / 45.5 / 42.7,
+// 64 tokens at 8,192 keys 114 / 96 / 89.  So: the longest run that still leaves MX_SPLIT_BLOCKS
+// workgroups, and never more than 16 runs for a request.  `span`: the most keys a request can have.
+extern "C" int mi_mixer_split_keys(int M, int Hkv, int page_size, long span) {
+  if (M <= 0 || Hkv <= 0 || page_size <= 0 || span <= 0) return 0;
+  long split = MX_SPLIT_LEAST;
+  for (long candidate = MX_SPLIT_MOST; candidate > MX_SPLIT_LEAST; candidate /= 2)
+    if ((long)Hkv * M * ((span + candidate - 1) / candidate) >= MX_SPLIT_BLOCKS) {
+      split = candidate;
+      break;
+    }
+  while (split < MX_SPLIT_MOST && span > 16 * split) split *= 2;
+  if (split < page_size) split = page_size;
+  return (int)((split / page_size) * page_size);          // whole pages
+}
+
 extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv, int dh, int q_col, int k_col,
                                int v_col, const float* inv_freq, int rotary_dim, void* k_base, void* v_base,
                                long page_stride, int page_size, const int* block_tables, int max_pages,
@@ -846,7 +868,7 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
     return ERR_BAD_ARGUMENT;
   const int group = Hq / Hkv;
   const long span = window > 0 ? (long)window + page_size : (long)max_seq_len;
-  if ((dh != 64 && dh != 128) || group > 8 || page_size % 8 != 0 || page_size > MX_SPLIT_KEYS || max_seq_len <= 0 ||
+  if ((dh != 64 && dh != 128) || group > 8 || page_size % 8 != 0 || page_size > MX_SPLIT_LEAST * 2 || max_seq_len <= 0 ||
       N > WAVE * MX_SCAN_PER_THREAD ||
       u_ld % 8 != 0 || q_col % 8 != 0 || rotary_dim > dh || rotary_dim % 16 != 0)
     return ERR_UNSUPPORTED_SIZE;
@@ -913,7 +935,7 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
   p.ssm_out = (bf16_t*)ssm_out;
   p.ssm_y = ssm_y;
   p.out_ld = out_ld;
-  p.split_keys = (MX_SPLIT_KEYS / page_size) * page_size;          // whole pages
+  p.split_keys = mi_mixer_split_keys(M, Hkv, page_size, span);
   p.splits = (int)((span + p.split_keys - 1) / p.split_keys);
   if ((long)Hkv * M * p.splits > 0x3fffffffL || M > 65535 || Hq > 65535) return ERR_UNSUPPORTED_SIZE;
   if (!partial || partial_floats < (long)M * Hq * p.splits * (dh + 2)) return ERR_BAD_ARGUMENT;

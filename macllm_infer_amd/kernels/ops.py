@@ -72,6 +72,7 @@ _SIGNATURES = {
                           _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_int, _c_float, _c_int, _c_int, _c_int,
                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
         "mi_fused_gemm_supported": [_c_int, _c_int, _c_int],
+        "mi_mixer_split_keys": [_c_int, _c_int, _c_int, _c_long],
         "mi_mixer_decode": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int,
                             _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int,
                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -714,7 +715,8 @@ def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim
                  z_col + E, x_col + E + 2 * num_groups * state_size, dt_col + ssm_heads)
     _need(u.shape[1] >= widest, "mixer_decode: u is too narrow")
     span = max(1, int(max_seq_len)) if not window else window + page_size
-    split_keys = (512 // page_size) * page_size
+    split_keys = int(_fn("decode", "mi_mixer_split_keys")(M, num_kv_heads, page_size, span))      # the launcher's own rule
+    _need(split_keys > 0, "mixer_decode: no run length for these sizes")
     partial = torch.empty((M * num_heads * (-(-span // split_keys)) * (head_dim + 2),), dtype=torch.float32,
                           device=u.device)
     _check(_fn("decode", "mi_mixer_decode")(

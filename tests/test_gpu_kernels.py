@@ -786,7 +786,7 @@ def test_mixer_decode_of_wide_batches(ops, M, Hq, Hkv, dh, H, P, N, G):
 
 
 def test_mixer_decode_over_a_long_context(ops):
-    """Contexts of 5 000 and 9 000 tokens (10 and 18 runs of 512 keys: more than the merge takes
+    """Contexts of 5 000 and 9 000 tokens (more runs of keys than the merge takes
     at once) beside a short one; one far key per long request is made to dominate, so a run that
     is dropped or merged with the wrong weight shows."""
     dtype = torch.bfloat16
