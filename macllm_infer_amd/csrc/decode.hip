@@ -629,7 +629,7 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
 
   // ---- this wave's share of the run
   int span = (p.split_keys + MX_WAVES - 1) / MX_WAVES;
-  span = ((span + 63) / 64) * 64;
+  span = ((span + 31) / 32) * 32;
   const int wave_lo = run_lo + wave * span;
   const int wave_hi = min(wave_lo + span, run_hi);
   AttnAccumulator<DH, 1> acc;
@@ -838,15 +838,17 @@ __global__ void __launch_bounds__(MX_THREADS) mixer_decode_kernel(MixerParams p)
 
 // Keys of one attention workgroup (a run).  Long runs pay the start of a workgroup (position, page ids,
 // then keys: three round trips) and the merge of the runs less often; short runs give a small step more
-// workgroups.  Measured on one MI355X (mixer + merge of a layer, head size 64, 2 kv heads; runs of
-// 256 / 512 / 1,024 keys): 1 token at 2,048 keys 12.4 / 12.8 / 14.9 us, 8 tokens at 2,048 keys
-// 13.9 / 14.3 / 17.2, 8 tokens at 8,192 keys 23.6 / 20.6 / 18.7, 64 tokens at 2,048 keys 49.7 / 45.5 / 42.7,
-// 64 tokens at 8,192 keys 114 / 96 / 89.  So: the longest run that still leaves MX_SPLIT_BLOCKS
-// workgroups, and never more than 16 runs for a request.  `span`: the most keys a request can have.
+// workgroups, and a request whose context ends just behind a run's edge pays a whole workgroup for a few
+// keys.  Measured on one MI355X (mixer + merge of a layer, head size 64, 2 kv heads; runs of
+// 256 / 512 / 1,024 keys; contexts inside graphs made for 4,096 and 8,192 keys): 1 token at 2,100 keys
+// 11.3 / 12.0 / 15.0 us; 8 tokens at 2,100 keys 15.1 / 14.0 / 16.6, at 6,000 keys 20.3 / 17.2 / 17.8;
+// 64 tokens at 2,100 keys 61.0 / 56.0 / 52.0, at 6,000 keys 100 / 85 / 80.  So: the longest run that still
+// leaves MX_SPLIT_BLOCKS workgroups (up to 512 keys for steps of up to 16 tokens, 1,024 beyond), and never
+// more than 16 runs for a request.  `span`: the most keys a request of the step can have.
 extern "C" int mi_mixer_split_keys(int M, int Hkv, int page_size, long span) {
   if (M <= 0 || Hkv <= 0 || page_size <= 0 || span <= 0) return 0;
   long split = MX_SPLIT_LEAST;
-  for (long candidate = MX_SPLIT_MOST; candidate > MX_SPLIT_LEAST; candidate /= 2)
+  for (long candidate = M <= 16 ? MX_SPLIT_MOST / 2 : MX_SPLIT_MOST; candidate > MX_SPLIT_LEAST; candidate /= 2)
     if ((long)Hkv * M * ((span + candidate - 1) / candidate) >= MX_SPLIT_BLOCKS) {
       split = candidate;
       break;
