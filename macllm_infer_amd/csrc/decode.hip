@@ -463,6 +463,7 @@ extern "C" int mi_fused_gemm_supported(int pro, int M, int K) {
 #define MX_MAX_PAGES 132       // page ids of one run of keys (at most MX_SPLIT_MOST / 8 + 2)
 #define MX_SPLIT_LEAST 256     // keys of one attention workgroup: between these two, see mi_mixer_split_keys
 #define MX_SPLIT_MOST 1024
+#define MX_WALK_BLOCKS 256      // attention workgroups from which on a workgroup walks over several runs
 #define MX_SPLIT_BLOCKS 128    // attention workgroups a step should at least have before its runs grow
 #define MX_SCAN_PER_THREAD 8
 #define MX_FEW_BLOCKS 512       // state-space workgroups of a step up to which each takes one row per thread group
@@ -570,15 +571,20 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
   int first_key = 0;
   if (p.window > 0 && pos - p.window + 1 > 0) first_key = pos - p.window + 1;
   const int base_key = (first_key / p.page_size) * p.page_size;       // a page edge
-  const int run_lo = base_key + split * p.split_keys;
-  if (run_lo > pos) return;                                            // nothing of this request here
-  const int run_hi = min(run_lo + p.split_keys, pos + 1);
-  const bool writer = run_hi == pos + 1;                               // the run that holds the new token
-  const int base_page = run_lo / p.page_size;
-  {
-    const int last_page = (run_hi - 1) / p.page_size;
-    for (int t = tid; t <= last_page - base_page; t += MX_THREADS) pages_lds[t] = table[base_page + t];
-  }
+  // the request's keys are cut into runs of split_keys; this workgroup takes the runs split, split + splits,
+  // split + 2 splits, ... (a large step has fewer workgroups than runs: a workgroup that finds no keys costs
+  // some 30 ns of a step's time, and a graph made for long contexts would launch hundreds of them)
+  const int runs = (pos - base_key) / p.split_keys + 1;
+  if (split >= runs) return;                                           // nothing of this request here
+  const bool writer = (runs - 1) % p.splits == split;                  // the workgroup that holds the new token
+  auto stage_pages = [&](int run) {
+    const int lo = base_key + run * p.split_keys;
+    const int hi = min(lo + p.split_keys, pos + 1);
+    const int first_page = lo / p.page_size;
+    const int last_page = (hi - 1) / p.page_size;
+    for (int t = tid; t <= last_page - first_page; t += MX_THREADS) pages_lds[t] = table[first_page + t];
+  };
+  stage_pages(split);
   const float k_raw = (float)k_raw_bits, k_raw_pair = (float)k_pair_bits, v_raw = (float)v_raw_bits;
   if (rotate) {
     const float position = (float)pos;
@@ -627,24 +633,33 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
   __threadfence_block();
   __syncthreads();
 
-  // ---- this wave's share of the run
+  // ---- this wave's share of each run
   int span = (p.split_keys + MX_WAVES - 1) / MX_WAVES;
   span = ((span + 31) / 32) * 32;
-  const int wave_lo = run_lo + wave * span;
-  const int wave_hi = min(wave_lo + span, run_hi);
   AttnAccumulator<DH, 1> acc;
   acc.clear();
-  if (wave_lo < run_hi) {
-    AttnCache cache;
-    cache.k_base = p.k_base;
-    cache.v_base = p.v_base;
-    cache.page_stride = p.page_stride;
-    cache.page_size = p.page_size;
-    cache.kvh = kvh;
-    cache.pages = pages_lds;
-    cache.base_page = base_page;
-    const int col_pos[1] = {has_head ? pos : -1};
-    attend_keys<DH, 1, 2>(acc, q_frag, col_pos, p.window, p.scale, wave_lo, wave_hi, cache);
+  for (int run = split; run < runs; run += p.splits) {
+    if (run != split) {
+      __syncthreads();                                                 // the page ids of the run before are read
+      stage_pages(run);
+      __syncthreads();
+    }
+    const int run_lo = base_key + run * p.split_keys;
+    const int run_hi = min(run_lo + p.split_keys, pos + 1);
+    const int wave_lo = run_lo + wave * span;
+    const int wave_hi = min(wave_lo + span, run_hi);
+    if (wave_lo < run_hi) {
+      AttnCache cache;
+      cache.k_base = p.k_base;
+      cache.v_base = p.v_base;
+      cache.page_stride = p.page_stride;
+      cache.page_size = p.page_size;
+      cache.kvh = kvh;
+      cache.pages = pages_lds;
+      cache.base_page = run_lo / p.page_size;
+      const int col_pos[1] = {has_head ? pos : -1};
+      attend_keys<DH, 1, 2>(acc, q_frag, col_pos, p.window, p.scale, wave_lo, wave_hi, cache);
+    }
   }
 
   // ---- merge the waves: merge_lds[wave][head] = {m, l, o[DH]}
@@ -939,6 +954,9 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
   p.out_ld = out_ld;
   p.split_keys = mi_mixer_split_keys(M, Hkv, page_size, span);
   p.splits = (int)((span + p.split_keys - 1) / p.split_keys);
+  // workgroups per (token, kv head): one per run while the step is small, fewer (each walks over several
+  // runs) once the step has MX_WALK_BLOCKS of them anyway
+  p.splits = (int)min((long)p.splits, max(1L, (MX_WALK_BLOCKS + (long)Hkv * M - 1) / ((long)Hkv * M)));
   if ((long)Hkv * M * p.splits > 0x3fffffffL || M > 65535 || Hq > 65535) return ERR_UNSUPPORTED_SIZE;
   if (!partial || partial_floats < (long)M * Hq * p.splits * (dh + 2)) return ERR_BAD_ARGUMENT;
   p.partial = partial;
