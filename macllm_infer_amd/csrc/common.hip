@@ -126,6 +126,74 @@ add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta0, con
   }
 }
 
+// ---------------------------------------------------------------- residual add of partial sums + RMSNorm
+// The same as add_rmsnorm for a branch that arrives as S float32 slabs [S, T, d] (a product split
+// over K): h[row] += sum over the slabs (in slab order), out = h / sqrt(mean(h^2) + eps) * w.
+// One workgroup per row; a thread takes four columns at a time and asks for all its slabs at once.
+#define PARTIALS_MOST 16
+template <typename TO>
+__global__ void __launch_bounds__(256)
+add_partials_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ partial, int S, long slab,
+                            const float* __restrict__ weight, float eps, TO* __restrict__ out,
+                            const int* __restrict__ rows, int d) {
+  typedef typename Vec4<float>::type f4;
+  typedef typename Vec4<TO>::type o4;
+  __shared__ float scratch[16];
+  const long out_row = blockIdx.x;
+  const long row = rows ? (long)rows[out_row] : out_row;
+  float* hr = h + row * d;
+  const float* pr = partial + row * d;
+  float sum_squares = 0.f;
+  for (int column = (int)threadIdx.x * 4; column < d; column += 256 * 4) {
+    f4 value = *reinterpret_cast<const f4*>(hr + column);
+    f4 parts[PARTIALS_MOST];
+#pragma unroll
+    for (int s = 0; s < PARTIALS_MOST; ++s) parts[s] = *reinterpret_cast<const f4*>(pr + (long)min(s, S - 1) * slab + column);
+#pragma unroll
+    for (int s = 0; s < PARTIALS_MOST; ++s)
+      if (s < S) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) value[j] += parts[s][j];
+      }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sum_squares += value[j] * value[j];
+    *reinterpret_cast<f4*>(hr + column) = value;       // with `rows` the caller passes a copy's row: see the launcher
+  }
+  const float total = block_sum(sum_squares, scratch);
+  const float denominator = sqrtf(total / (float)d + eps);
+  if (out) {
+    TO* o = out + out_row * d;
+    for (int column = (int)threadIdx.x * 4; column < d; column += 256 * 4) {
+      const f4 value = *reinterpret_cast<const f4*>(hr + column);
+      const f4 w = *reinterpret_cast<const f4*>(weight + column);
+      o4 packed;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) packed[j] = from_float<TO>(value[j] / denominator * w[j]);
+      *reinterpret_cast<o4*>(o + column) = packed;
+    }
+  }
+}
+
+// With `rows` (a gather: only those rows are normed) the stream itself must stay as it is, and a row may be
+// asked for twice; the kernel above writes the sums back, so gathers are refused here and the caller adds
+// the partial sums to the stream first (rows == nullptr, out == nullptr) and gathers with mi_add_rmsnorm.
+extern "C" int mi_add_partials_rmsnorm(float* h, const float* partial, int S, const float* weight, float eps,
+                                       void* out, int out_dtype, const int* rows, int n_rows, int T, int d,
+                                       hipStream_t stream) {
+  if (!h || !partial || !weight || S < 1 || n_rows <= 0 || T <= 0 || d <= 0) return ERR_BAD_ARGUMENT;
+  if (rows) return ERR_BAD_ARGUMENT;
+  if (S > PARTIALS_MOST || d % 4 != 0) return ERR_UNSUPPORTED_SIZE;
+  const long slab = (long)T * d;
+  if (out_dtype == DT_BF16)
+    add_partials_rmsnorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(h, partial, S, slab, weight, eps, (bf16_t*)out, rows, d);
+  else if (out_dtype == DT_F32)
+    add_partials_rmsnorm_kernel<float><<<n_rows, 256, 0, stream>>>(h, partial, S, slab, weight, eps, (float*)out, rows, d);
+  else
+    return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
 extern "C" int mi_add_rmsnorm(float* h, const void* delta0, const void* delta1, int delta_dtype,
                               const float* weight, float eps, void* out, int out_dtype, const int* rows,
                               int n_rows, int d, hipStream_t stream) {

@@ -80,10 +80,15 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   const int n_row = min(n0 + r, p.N - 1);
   const bf16_t* w_row = p.W + (long)n_row * K + 8 * q;
   // wave w takes a contiguous run of k-chunks (of 32), so that its loads cover whole cache lines
+  // (a grid with several rows splits K among them: row y takes a run of chunks and writes its partial
+  // sums, float32, into slab y of the output; whoever reads them adds the slabs up)
   const int chunks = K / 32;
-  const int per_wave = (chunks + FG_WAVES - 1) / FG_WAVES;
-  const int first_chunk = wave * per_wave;
-  const int iterations = max(0, min(per_wave, chunks - first_chunk));
+  const int per_split = (chunks + (int)gridDim.y - 1) / (int)gridDim.y;
+  const int split_first = (int)blockIdx.y * per_split;
+  const int split_end = min(split_first + per_split, chunks);
+  const int per_wave = (max(split_end - split_first, 0) + FG_WAVES - 1) / FG_WAVES;
+  const int first_chunk = split_first + wave * per_wave;
+  const int iterations = max(0, min(per_wave, split_end - first_chunk));
   // fragments of a wave in flight at once: few of them with 8 waves (long K, many workgroups a CU:
   // the registers saved buy more waves, which hide more than deeper batches do)
   constexpr int BATCH = FG_WAVES == 8 ? 4 : 8;
@@ -311,7 +316,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
     const int n_local = 4 * (l / 16) + i;
     const int n = n0 + n_local;
     const int m = mt * 16 + (l % 16);
-    if (p.bias && n < p.N) v += p.bias[n];
+    if (p.bias && n < p.N && blockIdx.y == 0) v += p.bias[n];
     if (EPI == EPI_SWIGLU) {
       tile[n_local * (MT * 16) + m] = v;
       continue;
@@ -349,7 +354,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
       if (taps > 1) tail[(long)(taps - 2) * channels] = sample;
       reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + n] = (bf16_t)silu_f(sum);
     } else if (p.out_f32) {
-      reinterpret_cast<float*>(p.out)[(long)m * p.out_ld + n] = v * p.out_scale;
+      reinterpret_cast<float*>(p.out)[((long)blockIdx.y * p.M + m) * p.out_ld + n] = v * p.out_scale;
     } else {
       reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + n] = (bf16_t)(v * p.out_scale);
     }
@@ -378,10 +383,10 @@ static size_t fused_gemm_lds(int MT, int pro, int K) {
 }
 
 template <int MT>
-static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStream_t stream) {
-  const int blocks = (p.N + 15) / 16;
+static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStream_t stream, int k_splits = 1) {
+  const dim3 blocks((p.N + 15) / 16, k_splits);
   const size_t lds = fused_gemm_lds(MT, pro, p.K);
-  const int waves = fused_gemm_waves(p.K);
+  const int waves = fused_gemm_waves(p.K / k_splits);
 #define FG_LAUNCH(PRO_, EPI_)                                                                   \
   do {                                                                                          \
     if (waves == 8) fused_gemm_kernel<MT, PRO_, EPI_, 8><<<blocks, 8 * WAVE, lds, stream>>>(p); \
@@ -446,6 +451,38 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
   else if (MT == 2) code = launch_fused_gemm<2>(p, pro, epi, stream);
   else if (MT == 3) code = launch_fused_gemm<3>(p, pro, epi, stream);
   else code = launch_fused_gemm<4>(p, pro, epi, stream);
+  if (code != 0) return code;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// The same product split over K for steps of many rows and few output features (a long K over 64
+// workgroups leaves most of the GPU idle): `splits` rows of workgroups each take a run of K and write
+// float32 partial sums into slab s of `partial` [splits, M, N] (the bias goes into slab 0).  The slabs
+// are added up by whoever reads them: the residual add of the next norm.
+extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, const float* bias, int M, int N, int K,
+                                   float* partial, int splits, hipStream_t stream) {
+  if (M <= 0 || N <= 0 || K <= 0 || !W || !x || !partial || x_ld < K || x_ld % 8 != 0) return ERR_BAD_ARGUMENT;
+  if (M > 64 || K % 32 != 0 || splits < 1 || splits > 64 || K / 32 < splits) return ERR_UNSUPPORTED_SIZE;
+  const int MT = (M + 15) / 16;
+  if (fused_gemm_lds(MT, PRO_PLAIN, K) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  FusedGemmParams p = {};
+  p.x = (const bf16_t*)x;
+  p.x_ld = x_ld;
+  p.W = (const bf16_t*)W;
+  p.bias = bias;
+  p.M = M;
+  p.N = N;
+  p.K = K;
+  p.out = partial;
+  p.out_ld = N;
+  p.out_f32 = 1;
+  p.out_scale = 1.0f;
+  int code;
+  if (MT == 1) code = launch_fused_gemm<1>(p, PRO_PLAIN, EPI_PLAIN, stream, splits);
+  else if (MT == 2) code = launch_fused_gemm<2>(p, PRO_PLAIN, EPI_PLAIN, stream, splits);
+  else if (MT == 3) code = launch_fused_gemm<3>(p, PRO_PLAIN, EPI_PLAIN, stream, splits);
+  else code = launch_fused_gemm<4>(p, PRO_PLAIN, EPI_PLAIN, stream, splits);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;

@@ -32,6 +32,8 @@ _SIGNATURES = {
         "mi_embed": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_int, _c_ptr],
         "mi_add_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int,
                            _c_int, _c_ptr],
+        "mi_add_partials_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int,
+                                    _c_int, _c_ptr],
         "mi_swiglu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
         "mi_scale_to_f32": [_c_ptr, _c_int, _c_float, _c_ptr, _c_long, _c_ptr],
     },
@@ -72,6 +74,7 @@ _SIGNATURES = {
                           _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_int, _c_float, _c_int, _c_int, _c_int,
                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
         "mi_fused_gemm_supported": [_c_int, _c_int, _c_int],
+        "mi_fused_gemm_split": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_ptr],
         "mi_mixer_split_keys": [_c_int, _c_int, _c_int, _c_long],
         "mi_mixer_decode": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int,
                             _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int,
@@ -197,6 +200,23 @@ def add_rmsnorm(h: torch.Tensor, deltas: Sequence[torch.Tensor], weight: torch.T
         _p(h), _p(deltas[0]) if len(deltas) > 0 else None, _p(deltas[1]) if len(deltas) > 1 else None,
         delta_dtype, _p(weight), float(eps), _p(out), out_dtype, _p(rows), n_rows, d, _stream()),
         "add_rmsnorm", f"(d={d})")
+
+
+def add_partials_rmsnorm(h: torch.Tensor, partial: torch.Tensor, weight: torch.Tensor, eps: float,
+                         out: Optional[torch.Tensor]) -> None:
+    """``add_rmsnorm`` for a branch that arrives as float32 partial sums ``partial`` [S, T, d] (the
+    slabs of ``fused_gemm_split``): h += sum of the slabs (in slab order), and, with ``out``,
+    out = RMSNorm(h) * weight."""
+    T, d = h.shape
+    _need(h.dtype == torch.float32 and h.is_contiguous() and h.is_cuda, "add_partials_rmsnorm: h must be contiguous float32")
+    _need(partial.dtype == torch.float32 and partial.dim() == 3 and partial.shape[1:] == (T, d)
+          and partial.is_contiguous(), "add_partials_rmsnorm: partial must be contiguous float32 [S, T, d]")
+    _need(weight.dtype == torch.float32 and weight.numel() == d and weight.is_contiguous(),
+          "add_partials_rmsnorm: weight must be float32 [d]")
+    _need(out is None or (out.shape == (T, d) and out.is_contiguous()), "add_partials_rmsnorm: bad out")
+    _check(_fn("common", "mi_add_partials_rmsnorm")(
+        _p(h), _p(partial), partial.shape[0], _p(weight), float(eps), _p(out), _dt(out) if out is not None else DT_F32,
+        None, T, T, d, _stream()), "add_partials_rmsnorm", f"(d={d}, S={partial.shape[0]})")
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor, tile: int = 0) -> None:
@@ -611,6 +631,26 @@ EPI_PLAIN, EPI_SWIGLU, EPI_CONV = 0, 1, 2
 def fused_gemm_supported(normed: bool, rows: int, in_features: int) -> bool:
     """Whether ``fused_gemm`` covers a batch of ``rows`` rows of ``in_features`` inputs."""
     return bool(_fn("decode", "mi_fused_gemm_supported")(PRO_NORM if normed else PRO_PLAIN, rows, in_features))
+
+
+def fused_gemm_split(weight: torch.Tensor, bias: Optional[torch.Tensor], x: torch.Tensor, partial: torch.Tensor) -> None:
+    """x [M, K] . weight[N, K]^T (+ bias) for a small batch in bfloat16, split over K: slab s of
+    ``partial`` (float32 [S, M, N], contiguous) receives the sums over the s-th run of K, the bias
+    in slab 0.  The product is the sum of the slabs (``add_partials_rmsnorm`` adds them to the
+    residual stream): many rows, a long K and few output features fill the GPU this way."""
+    _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
+          "fused_gemm_split: weight must be contiguous bfloat16 [N, K]")
+    N, K = weight.shape
+    x_ld = _row_major(x, "x")
+    M = x.shape[0]
+    _need(x.dtype == torch.bfloat16 and x.shape == (M, K) and x.data_ptr() % 16 == 0, "fused_gemm_split: bad x")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()),
+          "fused_gemm_split: bias must be float32 [N]")
+    _need(partial.dtype == torch.float32 and partial.dim() == 3 and partial.shape[1:] == (M, N)
+          and partial.is_contiguous() and partial.is_cuda, "fused_gemm_split: partial must be contiguous float32 [S, M, N]")
+    _check(_fn("decode", "mi_fused_gemm_split")(_p(x), x_ld, _p(weight), _p(bias), M, N, K, _p(partial),
+                                                partial.shape[0], _stream()),
+           "fused_gemm_split", f"(M={M}, N={N}, K={K}, S={partial.shape[0]})")
 
 
 def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, *, out_scale: float = 1.0,

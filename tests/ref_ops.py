@@ -51,6 +51,25 @@ def scale_to_f32(values, multiplier, out):
     out.copy_(_f(values).reshape(out.shape) * multiplier)
 
 
+def fused_gemm_split(weight, bias, x, partial):
+    """Slab s: the sums over the s-th run of K (in chunks of 32), the bias in slab 0."""
+    S = partial.shape[0]
+    chunks = weight.shape[1] // 32
+    per_split = -(-chunks // S)
+    for s in range(S):
+        lo, hi = min(s * per_split, chunks) * 32, min((s + 1) * per_split, chunks) * 32
+        partial[s] = _f(x[:, lo:hi]) @ _f(weight[:, lo:hi]).T
+    if bias is not None:
+        partial[0] += bias
+
+
+def add_partials_rmsnorm(h, partial, weight, eps, out):
+    for s in range(partial.shape[0]):
+        h += partial[s]
+    if out is not None:
+        out.copy_((h / torch.sqrt(h.pow(2).mean(dim=-1, keepdim=True) + eps) * weight).to(out.dtype))
+
+
 def linear(x, weight, bias, keep_float32=False):
     y = _f(x) @ _f(weight).T
     if bias is not None:
@@ -188,7 +207,7 @@ def argmax(logits, out):
     out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
 
 
-NAMES = ["prefill_attention_supported", "decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "linear", "rope_kv_store", "paged_attention",
+NAMES = ["fused_gemm_split", "add_partials_rmsnorm", "prefill_attention_supported", "decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "linear", "rope_kv_store", "paged_attention",
          "conv1d_silu", "conv_state_update", "ssm_scan", "gate_norm", "argmax"]
 
 

@@ -655,6 +655,33 @@ def test_fused_gemm_norm_prologue_and_epilogues(ops, M, N, K, deltas):
         assert torch.equal(got_state[unused].cpu(), state[unused])
 
 
+@pytest.mark.parametrize("M, N, K, S", [(64, 1024, 2048, 8), (33, 100, 2048, 16), (17, 48, 96, 3), (64, 136, 3072, 5),
+                                        (5, 64, 64, 1)])
+def test_fused_gemm_split_over_k_and_the_norm_that_adds_its_slabs(ops, M, N, K, S):
+    """Partial sums over runs of K in float32 slabs (the bias in the first), then the residual add
+    of all slabs with the norm, against the plain product and norm."""
+    x = rand(M, K + 16, seed=340, dtype=torch.bfloat16)[:, :K]
+    W, b = rand(N, K, seed=341, scale=0.1, dtype=torch.bfloat16), rand(N, seed=342)
+    want = torch.zeros(S, M, N)
+    ref_ops.fused_gemm_split(W, b, x, want)
+    got = torch.full((S, M, N), float("nan"), device=DEV)
+    ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), got)
+    close(got, want, torch.float32, 50.0)
+    whole = x.float() @ W.float().T + b
+    close(got.sum(0), whole, torch.float32, 200.0)
+    if N % 4 == 0:
+        h, weight = rand(M, N, seed=343), rand(N, seed=344, scale=0.1) + 1.0
+        want_h, want_out = h.clone(), torch.empty(M, N, dtype=torch.bfloat16)
+        ref_ops.add_partials_rmsnorm(want_h, want, weight, 3e-6, want_out)
+        got_h, got_out = h.clone().to(DEV), torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        ops.add_partials_rmsnorm(got_h, got, weight.to(DEV), 3e-6, got_out)
+        close(got_h, want_h, torch.float32, 50.0)
+        close(got_out, want_out, torch.bfloat16, 4.0)
+        again = h.clone().to(DEV)
+        ops.add_partials_rmsnorm(again, got, weight.to(DEV), 3e-6, None)           # the sum alone
+        assert torch.equal(again, got_h)
+
+
 @pytest.mark.parametrize("M, N, K", [(24, 200, 1024), (64, 136, 1024), (7, 96, 2048), (64, 88, 3072), (40, 64, 64)])
 def test_fused_gemm_conv_step_of_wide_batches(ops, M, N, K):
     """The conv epilogue behind the plain prologue: more than one tile of 16 rows, four and eight
