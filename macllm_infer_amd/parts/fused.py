@@ -50,6 +50,14 @@ LIBRARY_MARGIN = 0.92          # the library has to be this much faster to be ta
 FORCE_LIBRARY: Optional[bool] = None      # tests: True or False instead of the clock
 TUNE_ROWS = (8, 32, 64)
 _library_wins: Dict[tuple, bool] = {}
+# An output or down projection at 32 to 64 rows has a long K and few output features: 64 workgroups of the
+# skinny kernel, or whatever tile the library picks (10.7 us for 1,024 x 2,048 at 64 rows).  Split over K into
+# float32 slabs that the next norm adds up, the skinny kernel fills the GPU (7.5 us with 2 slabs; at 32 rows 5.2 us against the library's 9.6).  Measured
+# at build like the library; the split has to win by SPLIT_MARGIN, for the norm reads the slabs.
+SPLIT_CHOICES = (2, 4, 8)
+SPLIT_MARGIN = 0.85
+FORCE_SPLIT: Optional[int] = None         # tests: a number of slabs (0 = never) instead of the clock
+_split_wins: Dict[tuple, int] = {}
 # The library's tile for a prompt portion's input projection depends on the number of output features: 4 120
 # of them (0.5B-shaped) take 30.5 us at 2,048 rows, 4 352 (a multiple of 256) take 23.6.  Measured at build in
 # the same way; where padding pays, the prompt path multiplies with zero rows added and ignores their columns.
@@ -122,6 +130,39 @@ def _padding_pays(weight: torch.Tensor) -> bool:
 
         _padding_wins[key] = _graph_microseconds(wide) < PAD_MARGIN * _graph_microseconds(plain)
     return _padding_wins[key]
+
+
+def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool) -> int:
+    """The number of float32 slabs over K with which the skinny kernel beats the way this projection would
+    go otherwise (the library, or the skinny kernel unsplit) at this many rows, or 0."""
+    N, K = weight.shape
+    device = weight.device
+    copies = max(2, min(64, (512 << 20) // (weight.numel() * 2)))
+    weights = [weight] + [weight.clone() for _ in range(copies - 1)]
+    x = torch.full((rows, K), 0.01, dtype=torch.bfloat16, device=device)
+    out = torch.empty((rows, N), dtype=torch.bfloat16, device=device)
+
+    def whole():
+        for w in weights:
+            if library:
+                ops.linear(x, w, bias)
+            else:
+                ops.fused_gemm(w, bias, out, x=x)
+
+    best, best_time = 0, SPLIT_MARGIN * _graph_microseconds(whole)
+    for slabs in SPLIT_CHOICES:
+        if K // 32 < slabs:
+            continue
+        partial = torch.empty((slabs, rows, N), dtype=torch.float32, device=device)
+
+        def split():
+            for w in weights:
+                ops.fused_gemm_split(w, bias, x, partial)
+
+        time = _graph_microseconds(split)
+        if time < best_time:
+            best, best_time = slabs, time
+    return best
 
 
 def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile: int, conv: Optional[dict]) -> bool:
@@ -243,6 +284,9 @@ class ParallelFusion:
         self.library_out = self._tune(self.w_out, self.b_out, ops.EPI_PLAIN)
         self.library_gate_up = self._tune(self.w_gate_up, self.b_gate_up, ops.EPI_SWIGLU)
         self.library_down = self._tune(ffn.down.weight, ffn.down.bias, ops.EPI_PLAIN)
+        # and which of the two that feed the residual stream are split over K instead (steps of more than 16 rows)
+        self.split_out = self._tune_split(self.w_out, self.b_out, self.library_out)
+        self.split_down = self._tune_split(ffn.down.weight, ffn.down.bias, self.library_down)
 
     def decode_supported(self, step, cache) -> bool:
         a = self.attention.spec
@@ -293,6 +337,24 @@ class ParallelFusion:
         if epilogue != ops.EPI_PLAIN and self.norm_fits:
             choices = (False,) + choices[1:]
         return choices
+
+    def _tune_split(self, weight: torch.Tensor, bias, library: tuple) -> tuple:
+        """For step sizes of up to 16, 32 and 64 rows: the number of slabs over K, or 0 for the whole product.
+        Steps of up to 16 rows feed the next kernel's norm prologue, which takes whole rows."""
+        if self.hidden % 4 != 0 or FORCE_SPLIT == 0:
+            return (0, 0, 0)
+        if FORCE_SPLIT:
+            slabs = FORCE_SPLIT if weight.shape[1] // 32 >= FORCE_SPLIT else 0
+            return (0, slabs, slabs)
+        if weight.numel() < LIBRARY_MIN_WEIGHT:
+            return (0, 0, 0)
+        choices = [0]
+        for bucket in (1, 2):
+            key = (tuple(weight.shape), bias is None, bucket, library[bucket])
+            if key not in _split_wins:
+                _split_wins[key] = _measure_split(weight, bias, TUNE_ROWS[bucket], library[bucket])
+            choices.append(_split_wins[key])
+        return tuple(choices)
 
     def _tune_all(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict]) -> tuple:
         if not self.general or FORCE_LIBRARY is False or (FORCE_LIBRARY is None and weight.numel() < LIBRARY_MIN_WEIGHT):
@@ -357,12 +419,8 @@ class ParallelFusion:
             ops.gate_norm(y, u[:, self.z_col:self.z_col + s.inner_size], self.mamba.norm_weight, s.num_groups,
                           s.norm_eps, mixed[:, a.num_heads * a.head_dim:])
         # 3
-        if self.library_out[bucket]:
-            delta = ops.linear(mixed, self.w_out, self.b_out)
-        else:
-            delta = torch.empty((M, self.hidden), dtype=bf16, device=device)
-            ops.fused_gemm(self.w_out, self.b_out, delta, x=mixed)
-        residual.pending = [delta]
+        residual.pending = self._to_the_stream(mixed, self.w_out, self.b_out, self.library_out[bucket],
+                                               self.split_out[bucket])
         # 4
         activated = torch.empty((M, self.inner), dtype=bf16, device=device)
         if self.library_gate_up[bucket]:
@@ -375,12 +433,22 @@ class ParallelFusion:
                 residual.h, residual.pending = h_out, []
         # 5
         down = block.ffn.down
-        if self.library_down[bucket]:
-            delta = ops.linear(activated, down.weight, down.bias)
-        else:
-            delta = torch.empty((M, self.hidden), dtype=bf16, device=device)
-            ops.fused_gemm(down.weight, down.bias, delta, x=activated)
-        residual.pending = [delta]
+        residual.pending = self._to_the_stream(activated, down.weight, down.bias, self.library_down[bucket],
+                                               self.split_down[bucket])
+
+    def _to_the_stream(self, x: torch.Tensor, weight: torch.Tensor, bias, library: bool, slabs: int) -> list:
+        """A projection whose result is added to the residual stream: what the next norm will add, as one
+        bfloat16 branch or as float32 partial sums over runs of K (views of one tensor, in order)."""
+        M = x.shape[0]
+        if slabs:
+            partial = torch.empty((slabs, M, self.hidden), dtype=torch.float32, device=x.device)
+            ops.fused_gemm_split(weight, bias, x, partial)
+            return list(partial.unbind(0))
+        if library:
+            return [ops.linear(x, weight, bias)]
+        delta = torch.empty((M, self.hidden), dtype=torch.bfloat16, device=x.device)
+        ops.fused_gemm(weight, bias, delta, x=x)
+        return [delta]
 
 
 def _cat_bias(linears, device):

@@ -10,6 +10,21 @@ from ..weights.loader import Expect
 from .base import BuildContext, Part, Residual, register_part
 
 
+def partial_slab(pending) -> Optional[torch.Tensor]:
+    """The float32 [S, T, d] tensor whose slabs, in order, ``pending`` lists (a branch that arrives as
+    partial sums of a product split over K), or None."""
+    if len(pending) < 2:
+        return None
+    base = pending[0]._base
+    if (base is None or base.dim() != 3 or base.dtype != torch.float32 or base.shape[0] != len(pending)
+            or not base.is_contiguous()):
+        return None
+    for index, slab in enumerate(pending):
+        if slab._base is not base or slab.shape != base.shape[1:] or slab.data_ptr() != base[index].data_ptr():
+            return None
+    return base
+
+
 @register_part("rmsnorm")
 class RmsNorm(Part):
     """y = x / sqrt(mean(x^2) + eps) * w, statistics in float32
@@ -30,6 +45,17 @@ class RmsNorm(Part):
         """Add the pending branch outputs to the residual stream and return its normed rows
         (all of them, or only ``rows``; with ``rows`` the stream itself is left unchanged)."""
         pending = residual.pending
+        slab = partial_slab(pending)
+        if slab is not None and slab.shape[0] <= 16 and residual.h.shape[1] % 4 == 0:
+            # partial sums of one branch: added and normed in one launch (with a gather: added here,
+            # the gather below then norms the rows of the stream itself)
+            out = None
+            if rows is None:
+                out = torch.empty(residual.h.shape, dtype=self.build.dtype, device=residual.h.device)
+            ops.add_partials_rmsnorm(residual.h, slab, self.weight, self.eps, out)
+            residual.pending = pending = []
+            if rows is None:
+                return out
         while len(pending) > 2:                    # more than two branches: add the extra ones first
             ops.add_rmsnorm(residual.h, pending[:2], self.weight, self.eps, None)
             pending = pending[2:]
