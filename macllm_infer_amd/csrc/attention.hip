@@ -476,11 +476,13 @@ extern "C" int mi_decode_attention(const void* q, long q_ld, int T, int Hq, int 
 // one to the workgroup's last position, are split in eight runs of whole 32-key steps, one per
 // wave, read straight from the cache pages (the portion's own keys were written by rope_kv_store
 // before), four steps in flight at a time; the eight partial results are merged through LDS,
-// set by set.  Workgroups with the longest contexts (the last tiles) are launched first.
+// set by set.  Workgroups with the longest contexts (the last tiles) are launched first, in every
+// other head pass last.
 #include "attn_mfma.h"
 
 #define PREFILL_STEPS 4
 #define PREFILL_WAVES 8
+#define PREFILL_FILL_BLOCKS 512   // two workgroups for each of the 256 compute units
 
 template <int DH, int NSET>
 __global__ void __launch_bounds__(PREFILL_WAVES * WAVE)
@@ -492,7 +494,9 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
   constexpr int ITEMS = 2 + 4 * (DH / 16);                    // m, l and the accumulator of one set
   __shared__ float part[PREFILL_WAVES][ITEMS][WAVE];
   __shared__ int wave_pages[PREFILL_WAVES][WAVE];
-  const int block = gridDim.x - 1 - blockIdx.x;               // heavy ones first
+  // heavy ones first; every other head pass the other way round, so that workgroups of two passes that
+  // run side by side bring about the same work together
+  const int block = (blockIdx.z & 1) ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
   const int tile = block / 4;
   const int kvh = blockIdx.y;
   const int G = Hq / Hkv;
@@ -616,8 +620,11 @@ extern "C" int mi_prefill_attention(const void* q, long q_ld, int Hq, int Hkv, i
   if ((dh != 64 && dh != 128) || page_size % 4 != 0 || q_ld % 8 != 0 || out_ld % 4 != 0 || Hkv > 65535 || G > 64)
     return ERR_UNSUPPORTED_SIZE;
   // up to four query heads share every K and V fragment; head size 128 holds twice the registers per head, and
-  // more than two heads would spill
-  const int most = dh == 128 ? 2 : 4;
+  // more than two heads would spill.  A grid that would leave compute units with fewer than two workgroups is
+  // bound by the softmax arithmetic of its longest tiles: it takes sets of two heads, so that twice the
+  // workgroups, every other pass from the light end, spread that work
+  int most = dh == 128 ? 2 : 4;
+  if (most > 2 && 4L * n_tiles * Hkv * ((G + most - 1) / most) < PREFILL_FILL_BLOCKS) most = 2;
   const int passes = (G + most - 1) / most;
   const int nset = (G + passes - 1) / passes;
   if (n_tiles > (1 << 28)) return ERR_UNSUPPORTED_SIZE;

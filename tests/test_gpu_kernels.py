@@ -890,6 +890,34 @@ def test_prefill_attention_on_the_matrix_cores(ops, Hq, Hkv, dh, page_size, wind
     close(got, want, dtype, 2.0)
 
 
+@pytest.mark.parametrize("Hq, Hkv, dh", [(8, 2, 64), (12, 2, 64), (3, 1, 64), (4, 2, 128)])
+def test_prefill_attention_many_short_portions(ops, Hq, Hkv, dh):
+    """130 requests with portions of one to three tokens after prefixes of different lengths: a grid large
+    enough for the widest sets of query heads that share a key fragment (few tiles take narrower sets)."""
+    dtype, page_size = torch.bfloat16, 16
+    generator = torch.Generator().manual_seed(77)
+    counts = torch.randint(1, 4, (130,), generator=generator).tolist()
+    starts = torch.randint(0, 90, (130,), generator=generator).tolist()
+    lengths = [s + c for s, c in zip(starts, counts)]
+    pool, table = paged_setup(lengths, page_size, Hkv, dh, dtype, seed=22)
+    for lane, length in enumerate(lengths):
+        fill_cache(pool, table, lane, rand(length, Hkv, dh, seed=800 + lane, dtype=dtype),
+                   rand(length, Hkv, dh, seed=1000 + lane, dtype=dtype), page_size)
+    T = sum(counts)
+    q = rand(T, Hq * dh, seed=611, dtype=dtype)
+    positions = torch.cat([torch.arange(s, s + c) for s, c in zip(starts, counts)]).to(torch.int32)
+    lane_of_token = torch.repeat_interleave(torch.arange(len(counts)), torch.tensor(counts)).to(torch.int32)
+    cu = torch.zeros(len(counts) + 1, dtype=torch.int32)
+    cu[1:] = torch.cumsum(torch.tensor(counts), 0)
+    tiles = i32([(lane, int(cu[lane])) for lane in range(len(counts))])
+    want = torch.empty(T, Hq * dh, dtype=dtype)
+    ref_ops.paged_attention(q, Hq, Hkv, dh, *views(pool, page_size), table, lane_of_token, positions, 0.17, None, want)
+    got = torch.full((T, Hq * dh), float("nan"), dtype=dtype, device=DEV)
+    ops.prefill_attention(q.to(DEV), Hq, Hkv, dh, *views(pool.to(DEV), page_size), table.to(DEV), tiles.to(DEV),
+                          cu.to(DEV), i32(starts).to(DEV), 0.17, None, got)
+    close(got, want, dtype, 2.0)
+
+
 def test_prefill_attention_finds_far_keys_and_edges(ops):
     """Queries at the end of a 700-token prompt; one chosen key takes all the weight."""
     Hq, Hkv, dh, length, page_size = 4, 2, 64, 700, 16
