@@ -314,14 +314,15 @@ class ParallelFusion:
         if u.shape[0] >= OVERLAP_MIN_TOKENS and torch.cuda.is_current_stream_capturing():
             # the two mixers read the same rows and write different columns: attention runs on a second
             # stream beside the state-space chain, whose kernels are many and small (in a captured graph
-            # only: launched one by one the step waits for the host, which the second stream costs more)
+            # only: launched one by one the step waits for the host, which the second stream costs more).
+            # The chain is recorded first: the graph keeps the branch it meets first on the queue of the
+            # projections before and after it, and the other branch pays the hops between queues
             main = torch.cuda.current_stream(u.device)
             side = _side_stream(u.device)
             side.wait_stream(main)
+            self.mamba.mix(u[:, self.qkv_width:self.in_width], step, caches[self.mamba_name], mixed[:, self.q_width:])
             with torch.cuda.stream(side):
                 self.attention.mix(u[:, :self.qkv_width], step, caches[self.attention_name], mixed[:, :self.q_width])
-
-            self.mamba.mix(u[:, self.qkv_width:self.in_width], step, caches[self.mamba_name], mixed[:, self.q_width:])
             main.wait_stream(side)
         else:
             self.attention.mix(u[:, :self.qkv_width], step, caches[self.attention_name], mixed[:, :self.q_width])
