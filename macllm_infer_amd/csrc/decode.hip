@@ -11,9 +11,10 @@
 //                 CONV  : rows in [conv_lo, conv_hi) are channels of a causal depthwise conv
 //                         with K taps: the new sample joins the request's tail, the tail is
 //                         rolled, SiLU(conv) is stored; other rows are stored as they are
-//     Each block owns 16 output rows; its 4 waves split K and feed the matrix cores
-//     (v_mfma_f32_16x16x32_bf16: A = 16 weight rows x 32 k, B = 16 batch rows x 32 k, both
-//     contiguous in k), then sum their partial tiles through LDS.
+//     Each block owns 16 output rows (or 2 or 4 tiles of 16 behind the plain prologue, for steps of
+//     many rows: the rows of x then cross the caches once per block and not once per 16 features); its
+//     waves split K and feed the matrix cores (v_mfma_f32_16x16x32_bf16: A = 16 weight rows x 32 k,
+//     B = 16 batch rows x 32 k, both contiguous in k), then sum their partial tiles through LDS.
 //
 //   mixer_decode : one launch with two kinds of blocks
 //       attention blocks: one per (token, kv head): rotation of q and of the new key, the write
@@ -61,8 +62,9 @@ struct FusedGemmParams {
 
 __device__ __forceinline__ float round_bf16(float v) { return (float)(bf16_t)v; }
 
-template <int MT, int PRO, int EPI, int FG_WAVES>
+template <int MT, int PRO, int EPI, int FG_WAVES, int NT>
 __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmParams p) {
+  static_assert(NT == 1 || PRO == PRO_PLAIN, "several feature tiles a workgroup: plain prologue only");
   constexpr int FG_THREADS = FG_WAVES * WAVE;
   extern __shared__ __align__(16) unsigned char smem[];
   const int K = p.K;
@@ -74,11 +76,12 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
 
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * NT;
   const int q = lane / 16;
   const int r = lane % 16;
-  const int n_row = min(n0 + r, p.N - 1);
-  const bf16_t* w_row = p.W + (long)n_row * K + 8 * q;
+  const bf16_t* w_row[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) w_row[nt] = p.W + (long)min(n0 + 16 * nt + r, p.N - 1) * K + 8 * q;
   // wave w takes a contiguous run of k-chunks (of 32), so that its loads cover whole cache lines
   // (a grid with several rows splits K among them: row y takes a run of chunks and writes its partial
   // sums, float32, into slab y of the output; whoever reads them adds the slabs up)
@@ -91,8 +94,8 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   const int iterations = max(0, min(per_wave, split_end - first_chunk));
   // fragments of a wave in flight at once: few of them with 8 waves (long K, many workgroups a CU:
   // the registers saved buy more waves, which hide more than deeper batches do)
-  constexpr int BATCH = FG_WAVES == 8 ? 4 : 8;
-  bf16x8_t a[BATCH];
+  constexpr int BATCH = (FG_WAVES == 8 || NT > 1) ? 4 : 8;
+  bf16x8_t a[BATCH][NT];
 
   // The outputs this thread finishes in the epilogue: element tid + j * FG_THREADS of the block's
   // MT x (16 rows x 16 features), all of one feature.  The slots of their rows are asked for before
@@ -102,7 +105,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   const int tail_n = n0 + 4 * ((tid % 64) / 16) + (tid % 256) / 64;
   int tail_slot[EPT] = {};
   bool tail_wanted = false;
-  if (EPI == EPI_CONV && p.conv_k >= 2 && p.conv_k <= TAILS + 1) {
+  if (EPI == EPI_CONV && NT == 1 && p.conv_k >= 2 && p.conv_k <= TAILS + 1) {
     tail_wanted = tail_n >= p.conv_lo && tail_n < p.conv_hi;
 #pragma unroll
     for (int j = 0; j < EPT; ++j)
@@ -152,7 +155,9 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   }
 #pragma unroll
   for (int j = 0; j < BATCH; ++j)      // no condition around these loads: a wave without chunks reads the last one
-    a[j] = *reinterpret_cast<const bf16x8_t*>(w_row + min(first_chunk + min(j, max(iterations, 1) - 1), chunks - 1) * 32);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      a[j][nt] = *reinterpret_cast<const bf16x8_t*>(w_row[nt] + min(first_chunk + min(j, max(iterations, 1) - 1), chunks - 1) * 32);
   if (PRO == PRO_NORM) {
     // one wave per row, two rows at a time: the rows are read once into registers (K <= 2048),
     // their sums of squares reduced in float32, and the normalized rows written in bfloat16
@@ -258,15 +263,18 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 
   // the product: eight weight fragments are requested before the first is used, so that a
   // wave keeps eight 1 KiB loads in flight
-  floatx4 acc[MT];
+  floatx4 acc[NT][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
   for (int first = 0; first < iterations; first += BATCH) {
     if (first > 0) {
 #pragma unroll
       for (int j = 0; j < BATCH; ++j) {
         const int c = first_chunk + min(first + j, iterations - 1);
-        a[j] = *reinterpret_cast<const bf16x8_t*>(w_row + c * 32);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) a[j][nt] = *reinterpret_cast<const bf16x8_t*>(w_row[nt] + c * 32);
       }
     }
     bf16x8_t b[BATCH][MT];
@@ -287,89 +295,98 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 #pragma unroll
     for (int j = 0; j < BATCH; ++j) {
       const int c = first_chunk + min(first + j, iterations - 1);
-      const floatx4 weights = first + j < iterations ? *reinterpret_cast<const floatx4*>(&a[j]) : floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        bf16x8_t operand;
-        if (PRO == PRO_NORM) operand = *reinterpret_cast<const bf16x8_t*>(xs + (long)(mt * 16 + r) * ldx + c * 32 + 8 * q);
-        else operand = b[j][mt];
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8_t*>(&weights), operand, acc[mt], 0, 0, 0);
+      for (int nt = 0; nt < NT; ++nt) {
+        const floatx4 weights = first + j < iterations ? *reinterpret_cast<const floatx4*>(&a[j][nt]) : floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          bf16x8_t operand;
+          if (PRO == PRO_NORM) operand = *reinterpret_cast<const bf16x8_t*>(xs + (long)(mt * 16 + r) * ldx + c * 32 + 8 * q);
+          else operand = b[j][mt];
+          acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8_t*>(&weights), operand, acc[nt][mt], 0, 0, 0);
+        }
       }
     }
   }
+  // the waves' partial tiles are summed through LDS and finished, one tile of 16 features after the other
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int nt = 0; nt < NT; ++nt) {
+    const int tile_n0 = n0 + 16 * nt;
+    if (nt > 0) __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[(wave * MT + mt) * 256 + i * 64 + lane] = acc[mt][i];
-  __syncthreads();
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[(wave * MT + mt) * 256 + i * 64 + lane] = acc[nt][mt][i];
+    __syncthreads();
 
 #pragma unroll
-  for (int j = 0; j < EPT; ++j) {
-    const int index = tid + j * FG_THREADS;
-    if (index >= MT * 256) continue;
-    float v = 0.f;
+    for (int j = 0; j < EPT; ++j) {
+      const int index = tid + j * FG_THREADS;
+      if (index >= MT * 256) continue;
+      float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < FG_WAVES; ++w) v += red[w * MT * 256 + index];
-    const int mt = index / 256;
-    const int i = (index % 256) / 64;
-    const int l = index % 64;
-    const int n_local = 4 * (l / 16) + i;
-    const int n = n0 + n_local;
-    const int m = mt * 16 + (l % 16);
-    if (p.bias && n < p.N && blockIdx.y == 0) v += p.bias[n];
-    if (EPI == EPI_SWIGLU) {
-      tile[n_local * (MT * 16) + m] = v;
-      continue;
-    }
-    if (n >= p.N || m >= p.M) continue;
-    if (EPI == EPI_CONV && n >= p.conv_lo && n < p.conv_hi) {
-      const int channel = n - p.conv_lo;
-      const int channels = p.conv_hi - p.conv_lo;
-      const int taps = p.conv_k;
-      bf16_t* tail = p.conv_state + (long)(tail_ready ? tail_slot[j] : p.slot_ids[m]) * (taps - 1) * channels + channel;
-      const bf16_t sample = (bf16_t)v;
-      float sum;
-      if (tail_ready) {                       // taps, bias and tail are in registers already
-        sum = tap_bias;
-#pragma unroll
-        for (int k = 0; k < TAILS; ++k) {
-          if (k < taps - 1) {
-            sum += tap_values[k] * (float)tail_values[j][k];
-            if (k > 0) tail[(long)(k - 1) * channels] = tail_values[j][k];       // roll the tail by one
-          }
-        }
-        float last_tap = tap_values[0];
-#pragma unroll
-        for (int k = 1; k < TAILS + 1; ++k) last_tap = k == taps - 1 ? tap_values[k] : last_tap;
-        sum += last_tap * (float)sample;
-      } else {
-        sum = p.conv_b ? p.conv_b[channel] : 0.f;
-        for (int k = 0; k < taps - 1; ++k) {
-          const bf16_t old = tail[(long)k * channels];
-          sum += p.conv_w[channel * taps + k] * (float)old;
-          if (k > 0) tail[(long)(k - 1) * channels] = old;       // roll the tail by one
-        }
-        sum += p.conv_w[channel * taps + taps - 1] * (float)sample;
+      for (int w = 0; w < FG_WAVES; ++w) v += red[w * MT * 256 + index];
+      const int mt = index / 256;
+      const int i = (index % 256) / 64;
+      const int l = index % 64;
+      const int n_local = 4 * (l / 16) + i;
+      const int n = tile_n0 + n_local;
+      const int m = mt * 16 + (l % 16);
+      if (p.bias && n < p.N && blockIdx.y == 0) v += p.bias[n];
+      if (EPI == EPI_SWIGLU) {
+        tile[n_local * (MT * 16) + m] = v;
+        continue;
       }
-      if (taps > 1) tail[(long)(taps - 2) * channels] = sample;
-      reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + n] = (bf16_t)silu_f(sum);
-    } else if (p.out_f32) {
-      reinterpret_cast<float*>(p.out)[((long)blockIdx.y * p.M + m) * p.out_ld + n] = v * p.out_scale;
-    } else {
-      reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + n] = (bf16_t)(v * p.out_scale);
+      if (n >= p.N || m >= p.M) continue;
+      if (EPI == EPI_CONV && n >= p.conv_lo && n < p.conv_hi) {
+        const int channel = n - p.conv_lo;
+        const int channels = p.conv_hi - p.conv_lo;
+        const int taps = p.conv_k;
+        bf16_t* tail = p.conv_state + (long)(tail_ready ? tail_slot[j] : p.slot_ids[m]) * (taps - 1) * channels + channel;
+        const bf16_t sample = (bf16_t)v;
+        float sum;
+        if (tail_ready) {                       // taps, bias and tail are in registers already
+          sum = tap_bias;
+#pragma unroll
+          for (int k = 0; k < TAILS; ++k) {
+            if (k < taps - 1) {
+              sum += tap_values[k] * (float)tail_values[j][k];
+              if (k > 0) tail[(long)(k - 1) * channels] = tail_values[j][k];       // roll the tail by one
+            }
+          }
+          float last_tap = tap_values[0];
+#pragma unroll
+          for (int k = 1; k < TAILS + 1; ++k) last_tap = k == taps - 1 ? tap_values[k] : last_tap;
+          sum += last_tap * (float)sample;
+        } else {
+          sum = p.conv_b ? p.conv_b[channel] : 0.f;
+          for (int k = 0; k < taps - 1; ++k) {
+            const bf16_t old = tail[(long)k * channels];
+            sum += p.conv_w[channel * taps + k] * (float)old;
+            if (k > 0) tail[(long)(k - 1) * channels] = old;       // roll the tail by one
+          }
+          sum += p.conv_w[channel * taps + taps - 1] * (float)sample;
+        }
+        if (taps > 1) tail[(long)(taps - 2) * channels] = sample;
+        reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + n] = (bf16_t)silu_f(sum);
+      } else if (p.out_f32) {
+        reinterpret_cast<float*>(p.out)[((long)blockIdx.y * p.M + m) * p.out_ld + n] = v * p.out_scale;
+      } else {
+        reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + n] = (bf16_t)(v * p.out_scale);
+      }
     }
-  }
-  if (EPI == EPI_SWIGLU) {
-    __syncthreads();
-    const int half_rows = p.N / 2;
-    for (int index = tid; index < 8 * MT * 16; index += FG_THREADS) {
-      const int i = index / (MT * 16);
-      const int m = index % (MT * 16);
-      const int column = blockIdx.x * 8 + i;
-      if (m >= p.M || column >= half_rows) continue;
-      const float gate = round_bf16(tile[i * (MT * 16) + m]);
-      const float up = round_bf16(tile[(8 + i) * (MT * 16) + m]);
-      reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + column] = (bf16_t)(silu_f(gate) * up);
+    if (EPI == EPI_SWIGLU) {
+      __syncthreads();
+      const int half_rows = p.N / 2;
+      for (int index = tid; index < 8 * MT * 16; index += FG_THREADS) {
+        const int i = index / (MT * 16);
+        const int m = index % (MT * 16);
+        const int column = (blockIdx.x * NT + nt) * 8 + i;
+        if (m >= p.M || column >= half_rows) continue;
+        const float gate = round_bf16(tile[i * (MT * 16) + m]);
+        const float up = round_bf16(tile[(8 + i) * (MT * 16) + m]);
+        reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + column] = (bf16_t)(silu_f(gate) * up);
+      }
     }
   }
 }
@@ -382,15 +399,34 @@ static size_t fused_gemm_lds(int MT, int pro, int K) {
   return bytes;
 }
 
+// feature_tiles: how many tiles of 16 output features a workgroup owns (1, 2 or 4).  With one, the rows of x
+// cross the caches once per 16 features, which is what bounds a step of many rows; with more, fewer
+// workgroups (of four waves) each keep more weight fragments in flight.  Plain prologue only.
 template <int MT>
-static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStream_t stream, int k_splits = 1) {
-  const dim3 blocks((p.N + 15) / 16, k_splits);
+static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStream_t stream, int k_splits = 1,
+                             int feature_tiles = 1) {
   const size_t lds = fused_gemm_lds(MT, pro, p.K);
+  if (feature_tiles > 1) {
+    if (pro != PRO_PLAIN || (feature_tiles != 2 && feature_tiles != 4)) return ERR_BAD_ARGUMENT;
+    const dim3 blocks((p.N + 16 * feature_tiles - 1) / (16 * feature_tiles), k_splits);
+#define FG_WIDE(EPI_)                                                                                  \
+  do {                                                                                                 \
+    if (feature_tiles == 2) fused_gemm_kernel<MT, PRO_PLAIN, EPI_, 4, 2><<<blocks, 4 * WAVE, lds, stream>>>(p); \
+    else fused_gemm_kernel<MT, PRO_PLAIN, EPI_, 4, 4><<<blocks, 4 * WAVE, lds, stream>>>(p);           \
+  } while (0)
+    if (epi == EPI_PLAIN) FG_WIDE(EPI_PLAIN);
+    else if (epi == EPI_SWIGLU) FG_WIDE(EPI_SWIGLU);
+    else if (epi == EPI_CONV) FG_WIDE(EPI_CONV);
+    else return ERR_BAD_ARGUMENT;
+#undef FG_WIDE
+    return 0;
+  }
+  const dim3 blocks((p.N + 15) / 16, k_splits);
   const int waves = fused_gemm_waves(p.K / k_splits);
-#define FG_LAUNCH(PRO_, EPI_)                                                                   \
-  do {                                                                                          \
-    if (waves == 8) fused_gemm_kernel<MT, PRO_, EPI_, 8><<<blocks, 8 * WAVE, lds, stream>>>(p); \
-    else fused_gemm_kernel<MT, PRO_, EPI_, 4><<<blocks, 4 * WAVE, lds, stream>>>(p);            \
+#define FG_LAUNCH(PRO_, EPI_)                                                                      \
+  do {                                                                                             \
+    if (waves == 8) fused_gemm_kernel<MT, PRO_, EPI_, 8, 1><<<blocks, 8 * WAVE, lds, stream>>>(p); \
+    else fused_gemm_kernel<MT, PRO_, EPI_, 4, 1><<<blocks, 4 * WAVE, lds, stream>>>(p);            \
   } while (0)
   if (pro == PRO_NORM && epi == EPI_PLAIN) FG_LAUNCH(PRO_NORM, EPI_PLAIN);
   else if (pro == PRO_NORM && epi == EPI_SWIGLU) FG_LAUNCH(PRO_NORM, EPI_SWIGLU);
@@ -410,8 +446,9 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
                              const void* W, const float* bias, int M, int N, int K, void* out, long out_ld,
                              int out_f32, float out_scale, int conv_lo, int conv_hi, int conv_k,
                              const float* conv_w, const float* conv_b, void* conv_state, const int* slot_ids,
-                             hipStream_t stream) {
+                             int feature_tiles, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !out) return ERR_BAD_ARGUMENT;
+  if (feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0) return ERR_UNSUPPORTED_SIZE;
   if (pro == PRO_NORM && (!h_in || !norm_w || h_out == h_in)) return ERR_BAD_ARGUMENT;
   if (pro == PRO_PLAIN && (!x || x_ld < K || x_ld % 8 != 0)) return ERR_BAD_ARGUMENT;
@@ -447,10 +484,10 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
   p.conv_state = (bf16_t*)conv_state;
   p.slot_ids = slot_ids;
   int code;
-  if (MT == 1) code = launch_fused_gemm<1>(p, pro, epi, stream);
-  else if (MT == 2) code = launch_fused_gemm<2>(p, pro, epi, stream);
-  else if (MT == 3) code = launch_fused_gemm<3>(p, pro, epi, stream);
-  else code = launch_fused_gemm<4>(p, pro, epi, stream);
+  if (MT == 1) code = launch_fused_gemm<1>(p, pro, epi, stream, 1, feature_tiles);
+  else if (MT == 2) code = launch_fused_gemm<2>(p, pro, epi, stream, 1, feature_tiles);
+  else if (MT == 3) code = launch_fused_gemm<3>(p, pro, epi, stream, 1, feature_tiles);
+  else code = launch_fused_gemm<4>(p, pro, epi, stream, 1, feature_tiles);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;
@@ -461,8 +498,9 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
 // float32 partial sums into slab s of `partial` [splits, M, N] (the bias goes into slab 0).  The slabs
 // are added up by whoever reads them: the residual add of the next norm.
 extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, const float* bias, int M, int N, int K,
-                                   float* partial, int splits, hipStream_t stream) {
+                                   float* partial, int splits, int feature_tiles, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !x || !partial || x_ld < K || x_ld % 8 != 0) return ERR_BAD_ARGUMENT;
+  if (feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0 || splits < 1 || splits > 64 || K / 32 < splits) return ERR_UNSUPPORTED_SIZE;
   const int MT = (M + 15) / 16;
   if (fused_gemm_lds(MT, PRO_PLAIN, K) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
@@ -479,10 +517,10 @@ extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, cons
   p.out_f32 = 1;
   p.out_scale = 1.0f;
   int code;
-  if (MT == 1) code = launch_fused_gemm<1>(p, PRO_PLAIN, EPI_PLAIN, stream, splits);
-  else if (MT == 2) code = launch_fused_gemm<2>(p, PRO_PLAIN, EPI_PLAIN, stream, splits);
-  else if (MT == 3) code = launch_fused_gemm<3>(p, PRO_PLAIN, EPI_PLAIN, stream, splits);
-  else code = launch_fused_gemm<4>(p, PRO_PLAIN, EPI_PLAIN, stream, splits);
+  if (MT == 1) code = launch_fused_gemm<1>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
+  else if (MT == 2) code = launch_fused_gemm<2>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
+  else if (MT == 3) code = launch_fused_gemm<3>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
+  else code = launch_fused_gemm<4>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;

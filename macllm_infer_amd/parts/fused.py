@@ -49,7 +49,7 @@ LIBRARY_MIN_WEIGHT = 2 << 20
 LIBRARY_MARGIN = 0.92          # the library has to be this much faster to be taken
 FORCE_LIBRARY: Optional[bool] = None      # tests: True or False instead of the clock
 TUNE_ROWS = (8, 32, 64)
-_library_wins: Dict[tuple, bool] = {}
+_library_wins: Dict[tuple, tuple] = {}
 # An output or down projection at 32 to 64 rows has a long K and few output features: 64 workgroups of the
 # skinny kernel, or whatever tile the library picks (10.7 us for 1,024 x 2,048 at 64 rows).  Split over K into
 # float32 slabs that the next norm adds up, the skinny kernel fills the GPU (7.5 us with 2 slabs; at 32 rows 5.2 us against the library's 9.6).  Measured
@@ -57,7 +57,13 @@ _library_wins: Dict[tuple, bool] = {}
 SPLIT_CHOICES = (2, 4, 8)
 SPLIT_MARGIN = 0.85
 FORCE_SPLIT: Optional[int] = None         # tests: a number of slabs (0 = never) instead of the clock
-_split_wins: Dict[tuple, int] = {}
+_split_wins: Dict[tuple, tuple] = {}
+# Beyond 16 rows the skinny kernel's workgroup may own 2 or 4 tiles of 16 output features instead of one: the
+# step's rows then cross the caches half or a quarter as often, and fewer workgroups each keep more weight
+# fragments in flight (a 5120 x 21504 weight at 32 rows: 135 us with one tile, 86 with two, the library 125).
+# Measured with the rest, per shape and step size.
+TILE_CHOICES = (1, 2, 4)
+FORCE_TILES: Optional[int] = None         # tests: this many tiles for steps of more than 16 rows instead of the clock
 # The library's tile for a prompt portion's input projection depends on the number of output features: 4 120
 # of them (0.5B-shaped) take 30.5 us at 2,048 rows, 4 352 (a multiple of 256) take 23.6.  Measured at build in
 # the same way; where padding pays, the prompt path multiplies with zero rows added and ignores their columns.
@@ -132,9 +138,9 @@ def _padding_pays(weight: torch.Tensor) -> bool:
     return _padding_wins[key]
 
 
-def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool) -> int:
-    """The number of float32 slabs over K with which the skinny kernel beats the way this projection would
-    go otherwise (the library, or the skinny kernel unsplit) at this many rows, or 0."""
+def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool, tiles: int) -> tuple:
+    """(slabs, feature tiles): the number of float32 slabs over K with which the skinny kernel beats the way this
+    projection would go otherwise (the library, or the skinny kernel unsplit) at this many rows, or 0."""
     N, K = weight.shape
     device = weight.device
     copies = max(2, min(64, (512 << 20) // (weight.numel() * 2)))
@@ -147,27 +153,29 @@ def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool) -> int:
             if library:
                 ops.linear(x, w, bias)
             else:
-                ops.fused_gemm(w, bias, out, x=x)
+                ops.fused_gemm(w, bias, out, x=x, feature_tiles=tiles)
 
-    best, best_time = 0, SPLIT_MARGIN * _graph_microseconds(whole)
+    best, best_time = (0, tiles), SPLIT_MARGIN * _graph_microseconds(whole)
     for slabs in SPLIT_CHOICES:
         if K // 32 < slabs:
             continue
         partial = torch.empty((slabs, rows, N), dtype=torch.float32, device=device)
+        for split_tiles in TILE_CHOICES[:2]:
 
-        def split():
-            for w in weights:
-                ops.fused_gemm_split(w, bias, x, partial)
+            def split():
+                for w in weights:
+                    ops.fused_gemm_split(w, bias, x, partial, feature_tiles=split_tiles)
 
-        time = _graph_microseconds(split)
-        if time < best_time:
-            best, best_time = slabs, time
+            time = _graph_microseconds(split)
+            if time < best_time:
+                best, best_time = (slabs, split_tiles), time
     return best
 
 
-def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile: int, conv: Optional[dict]) -> bool:
-    """Whether the library way is faster for this weight at this many rows.  Copies of the weight are
-    cycled through so that the caches do not hold it, as in a model of many layers."""
+def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile: int, conv: Optional[dict]) -> tuple:
+    """(whether the library way is faster for this weight at this many rows, the skinny kernel's best number
+    of feature tiles).  Copies of the weight are cycled through so that the caches do not hold it, as in a
+    model of many layers."""
     N, K = weight.shape
     device = weight.device
     copies = max(2, min(64, (512 << 20) // (weight.numel() * 2)))
@@ -179,9 +187,11 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
         conv = dict(conv, state=torch.zeros((rows, max(conv["taps"] - 1, 0), channels), dtype=torch.bfloat16, device=device),
                     slot_ids=torch.arange(rows, dtype=torch.int32, device=device))
 
-    def skinny():
-        for w in weights:
-            ops.fused_gemm(w, bias, out, x=x, epilogue=epilogue, conv=conv)
+    def skinny(tiles):
+        def run():
+            for w in weights:
+                ops.fused_gemm(w, bias, out, x=x, epilogue=epilogue, conv=conv, feature_tiles=tiles)
+        return run
 
     def library():
         for w in weights:
@@ -192,7 +202,9 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
                 ops.conv_step(product, conv["lo"], conv["hi"] - conv["lo"], conv["weight"], conv["bias"], conv["state"],
                               conv["slot_ids"])
 
-    return _graph_microseconds(library) < LIBRARY_MARGIN * _graph_microseconds(skinny)
+    times = {tiles: _graph_microseconds(skinny(tiles)) for tiles in (TILE_CHOICES if rows > MAX_NORM_ROWS else (1,))}
+    tiles = min(times, key=times.get)
+    return _graph_microseconds(library) < LIBRARY_MARGIN * times[tiles], tiles
 
 
 class ParallelFusion:
@@ -280,13 +292,15 @@ class ParallelFusion:
         self.norm_fits = ops.fused_gemm_supported(True, 1, self.hidden)
         # which projections go through the library, by step size
         conv = dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=mamba.conv_weight, bias=mamba.conv_bias)
-        self.library_in = self._tune(self.w_in, self.b_in, ops.EPI_CONV, conv)
-        self.library_out = self._tune(self.w_out, self.b_out, ops.EPI_PLAIN)
-        self.library_gate_up = self._tune(self.w_gate_up, self.b_gate_up, ops.EPI_SWIGLU)
-        self.library_down = self._tune(ffn.down.weight, ffn.down.bias, ops.EPI_PLAIN)
+        # (and how many tiles of 16 output features a workgroup of the skinny kernel owns where it is taken)
+        self.library_in, self.tiles_in = self._tune(self.w_in, self.b_in, ops.EPI_CONV, conv)
+        self.library_out, self.tiles_out = self._tune(self.w_out, self.b_out, ops.EPI_PLAIN)
+        self.library_gate_up, self.tiles_gate_up = self._tune(self.w_gate_up, self.b_gate_up, ops.EPI_SWIGLU)
+        self.library_down, self.tiles_down = self._tune(ffn.down.weight, ffn.down.bias, ops.EPI_PLAIN)
         # and which of the two that feed the residual stream are split over K instead (steps of more than 16 rows)
-        self.split_out = self._tune_split(self.w_out, self.b_out, self.library_out)
-        self.split_down = self._tune_split(ffn.down.weight, ffn.down.bias, self.library_down)
+        self.split_out, self.tiles_out = self._tune_split(self.w_out, self.b_out, self.library_out, self.tiles_out)
+        self.split_down, self.tiles_down = self._tune_split(ffn.down.weight, ffn.down.bias, self.library_down,
+                                                            self.tiles_down)
 
     def decode_supported(self, step, cache) -> bool:
         a = self.attention.spec
@@ -332,43 +346,49 @@ class ParallelFusion:
         residual.pending = [block.ffn.forward(normed)]
 
     def _tune(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict] = None) -> tuple:
-        """For step sizes of up to 16, 32 and 64 rows: whether this projection goes through the library.
-        (Where the norm runs in the skinny kernel's prologue, small steps stay with it.)"""
-        choices = self._tune_all(weight, bias, epilogue, conv)
+        """For step sizes of up to 16, 32 and 64 rows: whether this projection goes through the library, and
+        the feature tiles of the skinny kernel.  (Where the norm runs in the skinny kernel's prologue, small
+        steps stay with it.)"""
+        choices, tiles = self._tune_all(weight, bias, epilogue, conv)
         if epilogue != ops.EPI_PLAIN and self.norm_fits:
             choices = (False,) + choices[1:]
-        return choices
+        return choices, tiles
 
-    def _tune_split(self, weight: torch.Tensor, bias, library: tuple) -> tuple:
-        """For step sizes of up to 16, 32 and 64 rows: the number of slabs over K, or 0 for the whole product.
-        Steps of up to 16 rows feed the next kernel's norm prologue, which takes whole rows."""
+    def _tune_split(self, weight: torch.Tensor, bias, library: tuple, tiles: tuple) -> tuple:
+        """For step sizes of up to 16, 32 and 64 rows: the number of slabs over K, or 0 for the whole product,
+        and the feature tiles that go with it.  Steps of up to 16 rows feed the next kernel's norm prologue,
+        which takes whole rows."""
         if self.hidden % 4 != 0 or FORCE_SPLIT == 0:
-            return (0, 0, 0)
+            return (0, 0, 0), tiles
         if FORCE_SPLIT:
             slabs = FORCE_SPLIT if weight.shape[1] // 32 >= FORCE_SPLIT else 0
-            return (0, slabs, slabs)
+            return (0, slabs, slabs), tiles
         if weight.numel() < LIBRARY_MIN_WEIGHT:
-            return (0, 0, 0)
-        choices = [0]
+            return (0, 0, 0), tiles
+        slabs, split_tiles = [0], [tiles[0]]
         for bucket in (1, 2):
-            key = (tuple(weight.shape), bias is None, bucket, library[bucket])
+            key = (tuple(weight.shape), bias is None, bucket, library[bucket], tiles[bucket])
             if key not in _split_wins:
-                _split_wins[key] = _measure_split(weight, bias, TUNE_ROWS[bucket], library[bucket])
-            choices.append(_split_wins[key])
-        return tuple(choices)
+                _split_wins[key] = _measure_split(weight, bias, TUNE_ROWS[bucket], library[bucket], tiles[bucket])
+            slabs.append(_split_wins[key][0])
+            split_tiles.append(_split_wins[key][1])
+        return tuple(slabs), tuple(split_tiles)
 
     def _tune_all(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict]) -> tuple:
+        forced = 1 if FORCE_TILES is None else FORCE_TILES
+        fixed_tiles = (1, forced, forced)
         if not self.general or FORCE_LIBRARY is False or (FORCE_LIBRARY is None and weight.numel() < LIBRARY_MIN_WEIGHT):
-            return (False, False, False)
+            return (False, False, False), fixed_tiles
         if FORCE_LIBRARY:
-            return (True, True, True)
-        choices = []
+            return (True, True, True), fixed_tiles
+        choices, tiles = [], []
         for bucket, rows in enumerate(TUNE_ROWS):
             key = (tuple(weight.shape), epilogue, bias is None, bucket)
             if key not in _library_wins:
                 _library_wins[key] = _measure_library(weight, bias, rows, epilogue, self.block.ffn.tile, conv)
-            choices.append(_library_wins[key])
-        return tuple(choices)
+            choices.append(_library_wins[key][0])
+            tiles.append(_library_wins[key][1] if FORCE_TILES is None or bucket == 0 else FORCE_TILES)
+        return tuple(choices), tuple(tiles)
 
     def forward_decode(self, residual: Residual, step, caches) -> None:
         block, a, s = self.block, self.attention.spec, self.mamba.spec
@@ -398,7 +418,7 @@ class ParallelFusion:
             ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=ops.EPI_CONV,
                            conv=dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=self.mamba.conv_weight,
                                      bias=self.mamba.conv_bias, state=state.states["conv"], slot_ids=step.slot_ids),
-                           **arguments)
+                           feature_tiles=self.tiles_in[bucket] if "x" in arguments else 1, **arguments)
             if h_out is not None:
                 residual.h, residual.pending = h_out, []
         # 2
@@ -421,7 +441,7 @@ class ParallelFusion:
                           s.norm_eps, mixed[:, a.num_heads * a.head_dim:])
         # 3
         residual.pending = self._to_the_stream(mixed, self.w_out, self.b_out, self.library_out[bucket],
-                                               self.split_out[bucket])
+                                               self.split_out[bucket], self.tiles_out[bucket])
         # 4
         activated = torch.empty((M, self.inner), dtype=bf16, device=device)
         if self.library_gate_up[bucket]:
@@ -429,26 +449,27 @@ class ParallelFusion:
                        block.ffn.tile)
         else:
             arguments, h_out = norm_prologue(block.ffn_norm)
-            ops.fused_gemm(self.w_gate_up, self.b_gate_up, activated, epilogue=ops.EPI_SWIGLU, **arguments)
+            ops.fused_gemm(self.w_gate_up, self.b_gate_up, activated, epilogue=ops.EPI_SWIGLU,
+                           feature_tiles=self.tiles_gate_up[bucket] if "x" in arguments else 1, **arguments)
             if h_out is not None:
                 residual.h, residual.pending = h_out, []
         # 5
         down = block.ffn.down
         residual.pending = self._to_the_stream(activated, down.weight, down.bias, self.library_down[bucket],
-                                               self.split_down[bucket])
+                                               self.split_down[bucket], self.tiles_down[bucket])
 
-    def _to_the_stream(self, x: torch.Tensor, weight: torch.Tensor, bias, library: bool, slabs: int) -> list:
+    def _to_the_stream(self, x: torch.Tensor, weight: torch.Tensor, bias, library: bool, slabs: int, tiles: int) -> list:
         """A projection whose result is added to the residual stream: what the next norm will add, as one
         bfloat16 branch or as float32 partial sums over runs of K (views of one tensor, in order)."""
         M = x.shape[0]
         if slabs:
             partial = torch.empty((slabs, M, self.hidden), dtype=torch.float32, device=x.device)
-            ops.fused_gemm_split(weight, bias, x, partial)
+            ops.fused_gemm_split(weight, bias, x, partial, feature_tiles=tiles)
             return list(partial.unbind(0))
         if library:
             return [ops.linear(x, weight, bias)]
         delta = torch.empty((M, self.hidden), dtype=torch.bfloat16, device=x.device)
-        ops.fused_gemm(weight, bias, delta, x=x)
+        ops.fused_gemm(weight, bias, delta, x=x, feature_tiles=tiles)
         return [delta]
 
 

@@ -303,20 +303,24 @@ def test_decode_graphs_match_eager_steps(tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("requests, library", [(24, False), (40, False), (5, True), (24, True), (40, "clock"),
-                                               (24, "split"), (40, "split")])
+                                               (24, "split"), (40, "split"), (24, "tiles"), (40, "tiles")])
 def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, requests, library):
     """More single-token lanes than the norm-fused kernels take (16): the block's fast path with
     norms of their own, through graphs of buckets 32 and 64, against the plain model.  ``library``:
     the projections go through the BLAS library (with the conv step and SwiGLU as kernels of their
     own), as large weights do where that is measured to be faster; "clock": the measurement itself
     runs on this model's small weights and either outcome must be right; "split": the projections
-    that feed the residual stream are split over K into float32 slabs that the next norm adds up."""
+    that feed the residual stream are split over K into float32 slabs that the next norm adds up; "tiles": a
+    workgroup of the skinny kernel owns four tiles of 16 output features, split projections included."""
     from macllm_infer_amd import Engine, Lane
     from macllm_infer_amd.parts import fused
     if library == "clock":
         monkeypatch.setattr(fused, "LIBRARY_MIN_WEIGHT", 0)
     elif library == "split":
         monkeypatch.setattr(fused, "FORCE_SPLIT", 3)
+    elif library == "tiles":
+        monkeypatch.setattr(fused, "FORCE_TILES", 4)
+        monkeypatch.setattr(fused, "FORCE_SPLIT", 2 if requests == 40 else 0)
     elif library:
         monkeypatch.setattr(fused, "FORCE_LIBRARY", True)
     folder = tiny_configs.make_model_dir("C", tmp_path, torch.bfloat16)
@@ -326,6 +330,10 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
     if library == "split":
         fusion = engine.model.blocks[0].fusion
         assert fusion.split_out == (0, 3, 3) and fusion.split_down == (0, 3, 3)
+    if library == "tiles":
+        fusion = engine.model.blocks[0].fusion
+        assert fusion.tiles_in == fusion.tiles_gate_up == fusion.tiles_out == fusion.tiles_down == (1, 4, 4)
+        assert fusion.library_in == fusion.library_down == (False, False, False)
     prompts = {index: tokens_for(cfg["vocab_size"], 3 + index % 7 + 6, 500 + index) for index in range(requests)}
     for index, tokens in prompts.items():
         engine.add_request(index)

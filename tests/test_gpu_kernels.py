@@ -596,16 +596,26 @@ def test_decode_attention_finds_one_far_key(ops):
 
 # ------------------------------------------------------------------ fused decode kernels
 @pytest.mark.parametrize("M, N, K", [(1, 48, 64), (8, 4120, 1024), (5, 100, 96), (16, 250, 1024), (33, 64, 256),
-                                     (64, 130, 2048)])
+                                     (64, 130, 2048), (48, 4128, 1024), (20, 80, 3072)])
 def test_fused_gemm_plain_prologue(ops, M, N, K):
+    """Plain and SwiGLU epilogues behind rows given in bfloat16, with one, two and four tiles of 16 output
+    features a workgroup (a last workgroup with tiles past the end included)."""
     x = rand(M, K + 8, seed=300, dtype=torch.bfloat16)[:, :K]            # a row stride
     W, b = rand(N, K, seed=301, scale=0.1, dtype=torch.bfloat16), rand(N, seed=302)
-    for out_dtype, scale, bias in ((torch.bfloat16, 1.0, b), (torch.float32, 0.6, None)):
-        want = torch.empty(M, N, dtype=out_dtype)
-        ref_ops.fused_gemm(W, bias, want, x=x, out_scale=scale)
-        got = torch.empty(M, N, dtype=out_dtype, device=DEV)
-        ops.fused_gemm(W.to(DEV), None if bias is None else bias.to(DEV), got, x=x.to(DEV), out_scale=scale)
-        close(got, want, out_dtype, 6.0 if out_dtype == torch.bfloat16 else 200.0)
+    for feature_tiles in (1, 2, 4):
+        for out_dtype, scale, bias in ((torch.bfloat16, 1.0, b), (torch.float32, 0.6, None)):
+            want = torch.empty(M, N, dtype=out_dtype)
+            ref_ops.fused_gemm(W, bias, want, x=x, out_scale=scale)
+            got = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+            ops.fused_gemm(W.to(DEV), None if bias is None else bias.to(DEV), got, x=x.to(DEV), out_scale=scale,
+                           feature_tiles=feature_tiles)
+            close(got, want, out_dtype, 6.0 if out_dtype == torch.bfloat16 else 200.0)
+        if N % 16 == 0:
+            want = torch.empty(M, N // 2, dtype=torch.bfloat16)
+            ref_ops.fused_gemm(W, b, want, x=x, epilogue=ref_ops.EPI_SWIGLU)
+            got = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+            ops.fused_gemm(W.to(DEV), b.to(DEV), got, x=x.to(DEV), epilogue=ops.EPI_SWIGLU, feature_tiles=feature_tiles)
+            close(got, want, torch.bfloat16, 16.0)
     assert ops.fused_gemm_supported(False, M, K) and not ops.fused_gemm_supported(False, 65, K)
     assert not ops.fused_gemm_supported(False, M, K + 8)
 
@@ -664,9 +674,10 @@ def test_fused_gemm_split_over_k_and_the_norm_that_adds_its_slabs(ops, M, N, K, 
     W, b = rand(N, K, seed=341, scale=0.1, dtype=torch.bfloat16), rand(N, seed=342)
     want = torch.zeros(S, M, N)
     ref_ops.fused_gemm_split(W, b, x, want)
-    got = torch.full((S, M, N), float("nan"), device=DEV)
-    ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), got)
-    close(got, want, torch.float32, 50.0)
+    for feature_tiles in (4, 2, 1):
+        got = torch.full((S, M, N), float("nan"), device=DEV)
+        ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), got, feature_tiles=feature_tiles)
+        close(got, want, torch.float32, 50.0)
     whole = x.float() @ W.float().T + b
     close(got.sum(0), whole, torch.float32, 200.0)
     if N % 4 == 0:
@@ -689,7 +700,7 @@ def test_fused_gemm_conv_step_of_wide_batches(ops, M, N, K):
     x = rand(M, K, seed=330, dtype=torch.bfloat16)
     W, b = rand(N, K, seed=331, scale=0.1, dtype=torch.bfloat16), rand(N, seed=332)
     lo, hi = 8, N - 24
-    for taps in (4, 2, 6):
+    for taps, feature_tiles in ((4, 1), (2, 1), (6, 1), (4, 2), (3, 4), (6, 4)):
         C = hi - lo
         state = rand(M + 3, taps - 1, C, seed=333, dtype=torch.bfloat16)
         slot_ids = torch.randperm(M + 3, generator=torch.Generator().manual_seed(taps))[:M].to(torch.int32)
@@ -698,7 +709,7 @@ def test_fused_gemm_conv_step_of_wide_batches(ops, M, N, K):
         want = torch.empty(M, N, dtype=torch.bfloat16)
         ref_ops.fused_gemm(W, b, want, x=x, epilogue=ref_ops.EPI_CONV, conv=dict(conv, state=want_state, slot_ids=slot_ids))
         got = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
-        ops.fused_gemm(W.to(DEV), b.to(DEV), got, x=x.to(DEV), epilogue=ops.EPI_CONV,
+        ops.fused_gemm(W.to(DEV), b.to(DEV), got, x=x.to(DEV), epilogue=ops.EPI_CONV, feature_tiles=feature_tiles,
                        conv=dict(lo=lo, hi=hi, taps=taps, weight=conv["weight"].to(DEV), bias=conv["bias"].to(DEV),
                                  state=got_state, slot_ids=slot_ids.to(DEV)))
         close(got, want, torch.bfloat16, 8.0)
