@@ -103,13 +103,16 @@ def _graph_microseconds(run) -> float:
         run()
     graph.replay()
     torch.cuda.synchronize(device)
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(3):
-        graph.replay()
-    end.record()
-    end.synchronize()
-    return start.elapsed_time(end) * 1e3 / 3
+    best = float("inf")
+    for _ in range(3):                     # the least of three rounds: a round that something else disturbed is left out
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(3):
+            graph.replay()
+        end.record()
+        end.synchronize()
+        best = min(best, start.elapsed_time(end) * 1e3 / 3)
+    return best
 
 
 def _padding_pays(weight: torch.Tensor) -> bool:
