@@ -102,11 +102,12 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   // everything else, because the addresses of their conv tails wait for them.
   constexpr int EPT = (MT * 256 + FG_THREADS - 1) / FG_THREADS;        // outputs a thread finishes
   constexpr int TAILS = (MT == 1 && FG_THREADS == 256) ? 8 : 3;         // tail samples kept per output
-  const int tail_n = n0 + 4 * ((tid % 64) / 16) + (tid % 256) / 64;
+  const int tail_n = n0 + 4 * ((tid % 64) / 16) + (tid % 256) / 64;      // in the first tile; 16 more per tile
   int tail_slot[EPT] = {};
-  bool tail_wanted = false;
-  if (EPI == EPI_CONV && NT == 1 && p.conv_k >= 2 && p.conv_k <= TAILS + 1) {
-    tail_wanted = tail_n >= p.conv_lo && tail_n < p.conv_hi;
+  bool tail_wanted[NT] = {};
+  if (EPI == EPI_CONV && p.conv_k >= 2 && p.conv_k <= TAILS + 1) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) tail_wanted[nt] = tail_n + 16 * nt >= p.conv_lo && tail_n + 16 * nt < p.conv_hi;
 #pragma unroll
     for (int j = 0; j < EPT; ++j)
       tail_slot[j] = p.slot_ids[min(((tid + j * FG_THREADS) / 256) * 16 + tid % 16, p.M - 1)];
@@ -239,26 +240,29 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 
   // the conv tails of those outputs are asked for now, behind the weights; no branch between the
   // loads either (a row past M reads the last row's tail and is not used)
-  bf16_t tail_values[EPT][TAILS];
-  float tap_values[TAILS + 1];
-  float tap_bias = 0.f;
-  bool tail_ready = false;
+  bf16_t tail_values[NT][EPT][TAILS];
+  float tap_values[NT][TAILS + 1];
+  float tap_bias[NT] = {};
+  bool tail_ready[NT] = {};
   if (EPI == EPI_CONV) {
 #pragma unroll
     for (int j = 0; j < EPT; ++j) asm volatile("" : "+v"(tail_slot[j]));   // keeps every use of the slots (and their wait) down here
   }
-  if (tail_wanted) {
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    if (!tail_wanted[nt]) continue;
     const int channels = p.conv_hi - p.conv_lo;
+    const int channel = tail_n + 16 * nt - p.conv_lo;
 #pragma unroll
     for (int j = 0; j < EPT; ++j) {
-      const bf16_t* tail = p.conv_state + (long)tail_slot[j] * (p.conv_k - 1) * channels + (tail_n - p.conv_lo);
+      const bf16_t* tail = p.conv_state + (long)tail_slot[j] * (p.conv_k - 1) * channels + channel;
 #pragma unroll
-      for (int k = 0; k < TAILS; ++k) tail_values[j][k] = tail[(long)min(k, p.conv_k - 2) * channels];
+      for (int k = 0; k < TAILS; ++k) tail_values[nt][j][k] = tail[(long)min(k, p.conv_k - 2) * channels];
     }
 #pragma unroll
-    for (int k = 0; k < TAILS + 1; ++k) tap_values[k] = p.conv_w[(long)(tail_n - p.conv_lo) * p.conv_k + min(k, p.conv_k - 1)];
-    if (p.conv_b) tap_bias = p.conv_b[tail_n - p.conv_lo];
-    tail_ready = true;
+    for (int k = 0; k < TAILS + 1; ++k) tap_values[nt][k] = p.conv_w[(long)channel * p.conv_k + min(k, p.conv_k - 1)];
+    if (p.conv_b) tap_bias[nt] = p.conv_b[channel];
+    tail_ready[nt] = true;
   }
 
   // the product: eight weight fragments are requested before the first is used, so that a
@@ -342,21 +346,21 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
         const int channel = n - p.conv_lo;
         const int channels = p.conv_hi - p.conv_lo;
         const int taps = p.conv_k;
-        bf16_t* tail = p.conv_state + (long)(tail_ready ? tail_slot[j] : p.slot_ids[m]) * (taps - 1) * channels + channel;
+        bf16_t* tail = p.conv_state + (long)(tail_ready[nt] ? tail_slot[j] : p.slot_ids[m]) * (taps - 1) * channels + channel;
         const bf16_t sample = (bf16_t)v;
         float sum;
-        if (tail_ready) {                       // taps, bias and tail are in registers already
-          sum = tap_bias;
+        if (tail_ready[nt]) {                   // taps, bias and tail are in registers already
+          sum = tap_bias[nt];
 #pragma unroll
           for (int k = 0; k < TAILS; ++k) {
             if (k < taps - 1) {
-              sum += tap_values[k] * (float)tail_values[j][k];
-              if (k > 0) tail[(long)(k - 1) * channels] = tail_values[j][k];       // roll the tail by one
+              sum += tap_values[nt][k] * (float)tail_values[nt][j][k];
+              if (k > 0) tail[(long)(k - 1) * channels] = tail_values[nt][j][k];   // roll the tail by one
             }
           }
-          float last_tap = tap_values[0];
+          float last_tap = tap_values[nt][0];
 #pragma unroll
-          for (int k = 1; k < TAILS + 1; ++k) last_tap = k == taps - 1 ? tap_values[k] : last_tap;
+          for (int k = 1; k < TAILS + 1; ++k) last_tap = k == taps - 1 ? tap_values[nt][k] : last_tap;
           sum += last_tap * (float)sample;
         } else {
           sum = p.conv_b ? p.conv_b[channel] : 0.f;
