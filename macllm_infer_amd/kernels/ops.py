@@ -265,7 +265,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
         _need(bias is None, "linear: float32 results of bfloat16 operands come without a bias")
         return torch.mm(x, weight.t(), out_dtype=torch.float32)
     if bias is None:
-        return torch.matmul(x, weight.t())
+        return torch.mm(x, weight.t())
     return torch.addmm(bias.to(torch.bfloat16), x, weight.t())
 
 
