@@ -58,6 +58,7 @@ struct FusedGemmParams {
   const float* conv_b;
   bf16_t* conv_state;
   const int* slot_ids;
+  int w_tiled;
 };
 
 __device__ __forceinline__ float round_bf16(float v) { return (float)(bf16_t)v; }
@@ -79,9 +80,14 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   const int n0 = blockIdx.x * 16 * NT;
   const int q = lane / 16;
   const int r = lane % 16;
+  // W is row-major [N, K], or (w_tiled) in the order of the matrix-core fragments: [N / 16, K / 32, 64 lanes, 8],
+  // lane (q, r) of tile (n, c) holding W[16 n + r, 32 c + 8 q ..]: a wave's load then is one run of 1 KiB
   const bf16_t* w_row[NT];
+  const long w_step = p.w_tiled ? 512 : 32;
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) w_row[nt] = p.W + (long)min(n0 + 16 * nt + r, p.N - 1) * K + 8 * q;
+  for (int nt = 0; nt < NT; ++nt)
+    w_row[nt] = p.w_tiled ? p.W + (long)min((int)blockIdx.x * NT + nt, (p.N + 15) / 16 - 1) * (K / 32) * 512 + lane * 8
+                          : p.W + (long)min(n0 + 16 * nt + r, p.N - 1) * K + 8 * q;
   // wave w takes a contiguous run of k-chunks (of 32), so that its loads cover whole cache lines
   // (a grid with several rows splits K among them: row y takes a run of chunks and writes its partial
   // sums, float32, into slab y of the output; whoever reads them adds the slabs up)
@@ -158,7 +164,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   for (int j = 0; j < BATCH; ++j)      // no condition around these loads: a wave without chunks reads the last one
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
-      a[j][nt] = *reinterpret_cast<const bf16x8_t*>(w_row[nt] + min(first_chunk + min(j, max(iterations, 1) - 1), chunks - 1) * 32);
+      a[j][nt] = *reinterpret_cast<const bf16x8_t*>(w_row[nt] + min(first_chunk + min(j, max(iterations, 1) - 1), chunks - 1) * w_step);
   if (PRO == PRO_NORM) {
     // one wave per row, two rows at a time: the rows are read once into registers (K <= 2048),
     // their sums of squares reduced in float32, and the normalized rows written in bfloat16
@@ -278,7 +284,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
       for (int j = 0; j < BATCH; ++j) {
         const int c = first_chunk + min(first + j, iterations - 1);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) a[j][nt] = *reinterpret_cast<const bf16x8_t*>(w_row[nt] + c * 32);
+        for (int nt = 0; nt < NT; ++nt) a[j][nt] = *reinterpret_cast<const bf16x8_t*>(w_row[nt] + c * w_step);
       }
     }
     bf16x8_t b[BATCH][MT];
@@ -445,12 +451,16 @@ static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStre
 
 // Sizes: 1 <= M <= 64, K a multiple of 32; with the NORM prologue the normalized rows must fit
 // 64 KiB of LDS beside the reduction area.  EPI_SWIGLU wants N a multiple of 16.
+// w_fragments: W is not row-major [N, K] but a copy in the order of the matrix-core fragments,
+// [ceil(N / 16), K / 32, 4, 16, 8] with element [n, c, q, r, j] = W[16 n + r, 32 c + 8 q + j] (rows past N zero):
+// what a wave asks for at once is then one run of 1 KiB instead of 64 bytes of each of 16 rows, which
+// streams 15 to 25 % faster.
 extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* delta0, const void* delta1,
                              float* h_out, const float* norm_w, float eps, const void* x, long x_ld,
                              const void* W, const float* bias, int M, int N, int K, void* out, long out_ld,
                              int out_f32, float out_scale, int conv_lo, int conv_hi, int conv_k,
                              const float* conv_w, const float* conv_b, void* conv_state, const int* slot_ids,
-                             int feature_tiles, hipStream_t stream) {
+                             int feature_tiles, int w_fragments, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !out) return ERR_BAD_ARGUMENT;
   if (feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0) return ERR_UNSUPPORTED_SIZE;
@@ -487,6 +497,7 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
   p.conv_b = conv_b;
   p.conv_state = (bf16_t*)conv_state;
   p.slot_ids = slot_ids;
+  p.w_tiled = w_fragments ? 1 : 0;
   int code;
   if (MT == 1) code = launch_fused_gemm<1>(p, pro, epi, stream, 1, feature_tiles);
   else if (MT == 2) code = launch_fused_gemm<2>(p, pro, epi, stream, 1, feature_tiles);
@@ -502,7 +513,8 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
 // float32 partial sums into slab s of `partial` [splits, M, N] (the bias goes into slab 0).  The slabs
 // are added up by whoever reads them: the residual add of the next norm.
 extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, const float* bias, int M, int N, int K,
-                                   float* partial, int splits, int feature_tiles, hipStream_t stream) {
+                                   float* partial, int splits, int feature_tiles, int w_fragments,
+                                   hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !x || !partial || x_ld < K || x_ld % 8 != 0) return ERR_BAD_ARGUMENT;
   if (feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0 || splits < 1 || splits > 64 || K / 32 < splits) return ERR_UNSUPPORTED_SIZE;
@@ -520,6 +532,7 @@ extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, cons
   p.out_ld = N;
   p.out_f32 = 1;
   p.out_scale = 1.0f;
+  p.w_tiled = w_fragments ? 1 : 0;
   int code;
   if (MT == 1) code = launch_fused_gemm<1>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
   else if (MT == 2) code = launch_fused_gemm<2>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);

@@ -67,6 +67,10 @@ class DecoderModel:
             if build.dtype == torch.float32:
                 head = head.to(torch.float32)
             self.lm_head = head.contiguous().to(build.device)
+        # the copy of the head that the skinny kernel streams fastest, for decode steps that want every row
+        fused_head = (build.device.type == "cuda" and build.dtype == torch.bfloat16 and self.lm_head.dtype == torch.bfloat16
+                      and spec.hidden_size % 32 == 0 and ops.fused_gemm_supported(True, 1, spec.hidden_size))
+        self._head_fragments = ops.fragment_order(self.lm_head) if fused_head else None
 
     @property
     def graph_safe(self) -> bool:
@@ -90,7 +94,8 @@ class DecoderModel:
         if self._fused_head(step, wanted):
             # a decode step whose every row is wanted: residual add, norm, projection and scaling in one launch
             ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, h_in=residual.h,
-                           deltas=residual.pending, norm_weight=self.final_norm.weight, eps=self.final_norm.eps)
+                           deltas=residual.pending, norm_weight=self.final_norm.weight, eps=self.final_norm.eps,
+                           fragments=self._head_fragments)
             return logits
         normed = self.final_norm.forward(residual, rows=step.want_rows)
         raw = ops.linear(normed, self.lm_head, None, keep_float32=True)      # the sums as they are, not rounded to bfloat16

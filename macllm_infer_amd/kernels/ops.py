@@ -72,9 +72,10 @@ _SIGNATURES = {
     "decode": {
         "mi_fused_gemm": [_c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_long, _c_ptr,
                           _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_int, _c_float, _c_int, _c_int, _c_int,
-                          _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
+                          _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
         "mi_fused_gemm_supported": [_c_int, _c_int, _c_int],
-        "mi_fused_gemm_split": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
+        "mi_fused_gemm_split": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int,
+                                _c_ptr],
         "mi_mixer_split_keys": [_c_int, _c_int, _c_int, _c_long],
         "mi_mixer_decode": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int,
                             _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int,
@@ -633,8 +634,28 @@ def fused_gemm_supported(normed: bool, rows: int, in_features: int) -> bool:
     return bool(_fn("decode", "mi_fused_gemm_supported")(PRO_NORM if normed else PRO_PLAIN, rows, in_features))
 
 
+def fragment_order(weight: torch.Tensor) -> torch.Tensor:
+    """A copy of weight [N, K] (K a multiple of 32) in the order in which the skinny kernels' waves read it:
+    [ceil(N / 16), K / 32, 4, 16, 8] with element [n, c, q, r, j] = weight[16 n + r, 32 c + 8 q + j], rows past N
+    zero.  A wave's load of a fragment is then one run of 1 KiB."""
+    _need(weight.dim() == 2 and weight.shape[1] % 32 == 0, "fragment_order: weight must be [N, K] with K a multiple of 32")
+    N, K = weight.shape
+    if N % 16:
+        weight = torch.cat([weight, weight.new_zeros((-N % 16, K))])
+    return weight.view(-1, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
+
+
+def _weight_operand(weight: torch.Tensor, fragments: Optional[torch.Tensor], name: str) -> torch.Tensor:
+    if fragments is None:
+        return weight
+    N, K = weight.shape
+    _need(fragments.dtype == torch.bfloat16 and fragments.is_contiguous() and fragments.is_cuda
+          and fragments.shape == (-(-N // 16), K // 32, 4, 16, 8), f"{name}: fragments do not fit the weight")
+    return fragments
+
+
 def fused_gemm_split(weight: torch.Tensor, bias: Optional[torch.Tensor], x: torch.Tensor, partial: torch.Tensor,
-                     feature_tiles: int = 1) -> None:
+                     feature_tiles: int = 1, fragments: Optional[torch.Tensor] = None) -> None:
     """x [M, K] . weight[N, K]^T (+ bias) for a small batch in bfloat16, split over K: slab s of
     ``partial`` (float32 [S, M, N], contiguous) receives the sums over the s-th run of K, the bias
     in slab 0.  The product is the sum of the slabs (``add_partials_rmsnorm`` adds them to the
@@ -649,8 +670,10 @@ def fused_gemm_split(weight: torch.Tensor, bias: Optional[torch.Tensor], x: torc
           "fused_gemm_split: bias must be float32 [N]")
     _need(partial.dtype == torch.float32 and partial.dim() == 3 and partial.shape[1:] == (M, N)
           and partial.is_contiguous() and partial.is_cuda, "fused_gemm_split: partial must be contiguous float32 [S, M, N]")
-    _check(_fn("decode", "mi_fused_gemm_split")(_p(x), x_ld, _p(weight), _p(bias), M, N, K, _p(partial),
-                                                partial.shape[0], int(feature_tiles), _stream()),
+    operand = _weight_operand(weight, fragments, "fused_gemm_split")
+    _check(_fn("decode", "mi_fused_gemm_split")(_p(x), x_ld, _p(operand), _p(bias), M, N, K, _p(partial),
+                                                partial.shape[0], int(feature_tiles), int(fragments is not None),
+                                                _stream()),
            "fused_gemm_split", f"(M={M}, N={N}, K={K}, S={partial.shape[0]})")
 
 
@@ -658,7 +681,7 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
                x: Optional[torch.Tensor] = None, h_in: Optional[torch.Tensor] = None,
                deltas: Sequence[torch.Tensor] = (), h_out: Optional[torch.Tensor] = None,
                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, epilogue: int = EPI_PLAIN,
-               conv: Optional[dict] = None, feature_tiles: int = 1) -> None:
+               conv: Optional[dict] = None, feature_tiles: int = 1, fragments: Optional[torch.Tensor] = None) -> None:
     """out[M, N'] = epilogue(prologue . weight[N, K]^T + bias) for a small batch in bfloat16.
 
     Prologue: ``x`` [M, K] bfloat16, or ``h_in`` float32 [M, K] with up to two bfloat16 ``deltas``:
@@ -669,7 +692,7 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
     rows lo..hi-1 go through the causal depthwise conv step of their channel with the request's
     tail (which is rolled) and SiLU.  ``feature_tiles`` (1, 2 or 4; more than one with ``x`` only): how many
     tiles of 16 output features a workgroup owns; the rows of x cross the caches once per workgroup, so
-    steps of many rows gain from more."""
+    steps of many rows gain from more.  ``fragments``: ``fragment_order(weight)``, read instead of the weight."""
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm: weight must be contiguous bfloat16 [N, K]")
     _need(feature_tiles in (1, 2, 4) and (feature_tiles == 1 or x is not None),
@@ -711,9 +734,10 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
         _need(slot_ids.numel() >= M, "fused_gemm: one slot per row")
     _check(_fn("decode", "mi_fused_gemm")(
         pro, epilogue, _p(h_in), _p(deltas[0]) if len(deltas) > 0 else None, _p(deltas[1]) if len(deltas) > 1 else None,
-        _p(h_out), _p(norm_weight), float(eps), _p(x), x_ld, _p(weight), _p(bias), M, N, K, _p(out), out_ld,
+        _p(h_out), _p(norm_weight), float(eps), _p(x), x_ld, _p(_weight_operand(weight, fragments, "fused_gemm")),
+        _p(bias), M, N, K, _p(out), out_ld,
         1 if out.dtype == torch.float32 else 0, float(out_scale), lo, hi, taps, _p(conv_w), _p(conv_b), _p(conv_state),
-        _p(slot_ids), int(feature_tiles), _stream()), "fused_gemm", f"(M={M}, N={N}, K={K})")
+        _p(slot_ids), int(feature_tiles), int(fragments is not None), _stream()), "fused_gemm", f"(M={M}, N={N}, K={K})")
 
 
 def mixer_decode_supported(num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, state_size: int,

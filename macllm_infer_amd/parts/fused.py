@@ -148,15 +148,16 @@ def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool, tiles: 
     device = weight.device
     copies = max(2, min(64, (512 << 20) // (weight.numel() * 2)))
     weights = [weight] + [weight.clone() for _ in range(copies - 1)]
+    fragments = [ops.fragment_order(w) for w in weights]
     x = torch.full((rows, K), 0.01, dtype=torch.bfloat16, device=device)
     out = torch.empty((rows, N), dtype=torch.bfloat16, device=device)
 
     def whole():
-        for w in weights:
+        for w, f in zip(weights, fragments):
             if library:
                 ops.linear(x, w, bias)
             else:
-                ops.fused_gemm(w, bias, out, x=x, feature_tiles=tiles)
+                ops.fused_gemm(w, bias, out, x=x, feature_tiles=tiles, fragments=f)
 
     best, best_time = (0, tiles), SPLIT_MARGIN * _graph_microseconds(whole)
     for slabs in SPLIT_CHOICES:
@@ -166,8 +167,8 @@ def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool, tiles: 
         for split_tiles in TILE_CHOICES[:2]:
 
             def split():
-                for w in weights:
-                    ops.fused_gemm_split(w, bias, x, partial, feature_tiles=split_tiles)
+                for w, f in zip(weights, fragments):
+                    ops.fused_gemm_split(w, bias, x, partial, feature_tiles=split_tiles, fragments=f)
 
             time = _graph_microseconds(split)
             if time < best_time:
@@ -190,10 +191,12 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
         conv = dict(conv, state=torch.zeros((rows, max(conv["taps"] - 1, 0), channels), dtype=torch.bfloat16, device=device),
                     slot_ids=torch.arange(rows, dtype=torch.int32, device=device))
 
+    fragments = [ops.fragment_order(w) for w in weights]
+
     def skinny(tiles):
         def run():
-            for w in weights:
-                ops.fused_gemm(w, bias, out, x=x, epilogue=epilogue, conv=conv, feature_tiles=tiles)
+            for w, f in zip(weights, fragments):
+                ops.fused_gemm(w, bias, out, x=x, epilogue=epilogue, conv=conv, feature_tiles=tiles, fragments=f)
         return run
 
     def library():
@@ -304,6 +307,17 @@ class ParallelFusion:
         self.split_out, self.tiles_out = self._tune_split(self.w_out, self.b_out, self.library_out, self.tiles_out)
         self.split_down, self.tiles_down = self._tune_split(ffn.down.weight, ffn.down.bias, self.library_down,
                                                             self.tiles_down)
+        # what the skinny kernel reads: a second copy of each matrix in the order of its waves' fragments (one run
+        # of 1 KiB a load instead of 64 bytes of each of 16 rows: 15 to 25 % faster); the row-major ones stay for
+        # the library and for prompt portions.  A projection that always goes through the library has none.
+
+        def fragments(weight, library, split):
+            return None if all(library) and not any(split) else ops.fragment_order(weight)
+
+        self.f_in = fragments(self.w_in, self.library_in, ())
+        self.f_out = fragments(self.w_out, self.library_out, self.split_out)
+        self.f_gate_up = fragments(self.w_gate_up, self.library_gate_up, ())
+        self.f_down = fragments(ffn.down.weight, self.library_down, self.split_down)
 
     def decode_supported(self, step, cache) -> bool:
         a = self.attention.spec
@@ -421,7 +435,8 @@ class ParallelFusion:
             ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=ops.EPI_CONV,
                            conv=dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=self.mamba.conv_weight,
                                      bias=self.mamba.conv_bias, state=state.states["conv"], slot_ids=step.slot_ids),
-                           feature_tiles=self.tiles_in[bucket] if "x" in arguments else 1, **arguments)
+                           feature_tiles=self.tiles_in[bucket] if "x" in arguments else 1, fragments=self.f_in,
+                           **arguments)
             if h_out is not None:
                 residual.h, residual.pending = h_out, []
         # 2
@@ -444,7 +459,7 @@ class ParallelFusion:
                           s.norm_eps, mixed[:, a.num_heads * a.head_dim:])
         # 3
         residual.pending = self._to_the_stream(mixed, self.w_out, self.b_out, self.library_out[bucket],
-                                               self.split_out[bucket], self.tiles_out[bucket])
+                                               self.split_out[bucket], self.tiles_out[bucket], self.f_out)
         # 4
         activated = torch.empty((M, self.inner), dtype=bf16, device=device)
         if self.library_gate_up[bucket]:
@@ -453,26 +468,28 @@ class ParallelFusion:
         else:
             arguments, h_out = norm_prologue(block.ffn_norm)
             ops.fused_gemm(self.w_gate_up, self.b_gate_up, activated, epilogue=ops.EPI_SWIGLU,
-                           feature_tiles=self.tiles_gate_up[bucket] if "x" in arguments else 1, **arguments)
+                           feature_tiles=self.tiles_gate_up[bucket] if "x" in arguments else 1,
+                           fragments=self.f_gate_up, **arguments)
             if h_out is not None:
                 residual.h, residual.pending = h_out, []
         # 5
         down = block.ffn.down
         residual.pending = self._to_the_stream(activated, down.weight, down.bias, self.library_down[bucket],
-                                               self.split_down[bucket], self.tiles_down[bucket])
+                                               self.split_down[bucket], self.tiles_down[bucket], self.f_down)
 
-    def _to_the_stream(self, x: torch.Tensor, weight: torch.Tensor, bias, library: bool, slabs: int, tiles: int) -> list:
+    def _to_the_stream(self, x: torch.Tensor, weight: torch.Tensor, bias, library: bool, slabs: int, tiles: int,
+                       fragments) -> list:
         """A projection whose result is added to the residual stream: what the next norm will add, as one
         bfloat16 branch or as float32 partial sums over runs of K (views of one tensor, in order)."""
         M = x.shape[0]
         if slabs:
             partial = torch.empty((slabs, M, self.hidden), dtype=torch.float32, device=x.device)
-            ops.fused_gemm_split(weight, bias, x, partial, feature_tiles=tiles)
+            ops.fused_gemm_split(weight, bias, x, partial, feature_tiles=tiles, fragments=fragments)
             return list(partial.unbind(0))
         if library:
             return [ops.linear(x, weight, bias)]
         delta = torch.empty((M, self.hidden), dtype=torch.bfloat16, device=x.device)
-        ops.fused_gemm(weight, bias, delta, x=x, feature_tiles=tiles)
+        ops.fused_gemm(weight, bias, delta, x=x, feature_tiles=tiles, fragments=fragments)
         return [delta]
 
 

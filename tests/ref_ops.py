@@ -51,7 +51,7 @@ def scale_to_f32(values, multiplier, out):
     out.copy_(_f(values).reshape(out.shape) * multiplier)
 
 
-def fused_gemm_split(weight, bias, x, partial, feature_tiles=1):
+def fused_gemm_split(weight, bias, x, partial, feature_tiles=1, fragments=None):
     """Slab s: the sums over the s-th run of K (in chunks of 32), the bias in slab 0."""
     S = partial.shape[0]
     chunks = weight.shape[1] // 32
@@ -258,7 +258,7 @@ def mixer_decode_supported(num_heads, num_kv_heads, head_dim, page_size, state_s
 
 
 def fused_gemm(weight, bias, out, *, out_scale=1.0, x=None, h_in=None, deltas=(), h_out=None, norm_weight=None,
-               eps=0.0, epilogue=EPI_PLAIN, conv=None, feature_tiles=1):
+               eps=0.0, epilogue=EPI_PLAIN, conv=None, feature_tiles=1, fragments=None):
     if x is None:
         total = h_in.clone()
         for delta in deltas:

@@ -610,6 +610,10 @@ def test_fused_gemm_plain_prologue(ops, M, N, K):
             ops.fused_gemm(W.to(DEV), None if bias is None else bias.to(DEV), got, x=x.to(DEV), out_scale=scale,
                            feature_tiles=feature_tiles)
             close(got, want, out_dtype, 6.0 if out_dtype == torch.bfloat16 else 200.0)
+            again = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)        # the weight in fragment order
+            ops.fused_gemm(W.to(DEV), None if bias is None else bias.to(DEV), again, x=x.to(DEV), out_scale=scale,
+                           feature_tiles=feature_tiles, fragments=ops.fragment_order(W.to(DEV)))
+            assert torch.equal(again, got)
         if N % 16 == 0:
             want = torch.empty(M, N // 2, dtype=torch.bfloat16)
             ref_ops.fused_gemm(W, b, want, x=x, epilogue=ref_ops.EPI_SWIGLU)
@@ -635,6 +639,10 @@ def test_fused_gemm_norm_prologue_and_epilogues(ops, M, N, K, deltas):
                    eps=3e-6)
     close(got, want, torch.bfloat16, 8.0)
     close(got_h, want_h, torch.float32)
+    again = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)           # the weight in fragment order
+    ops.fused_gemm(W.to(DEV), b.to(DEV), again, h_in=h.to(DEV), deltas=gpu(*ds), norm_weight=norm_w.to(DEV), eps=3e-6,
+                   fragments=ops.fragment_order(W.to(DEV)))
+    assert torch.equal(again, got)
     # swiglu (tiles of 8 gate rows + 8 up rows)
     if N % 16 == 0:
         want = torch.empty(M, N // 2, dtype=torch.bfloat16)
@@ -678,6 +686,10 @@ def test_fused_gemm_split_over_k_and_the_norm_that_adds_its_slabs(ops, M, N, K, 
         got = torch.full((S, M, N), float("nan"), device=DEV)
         ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), got, feature_tiles=feature_tiles)
         close(got, want, torch.float32, 50.0)
+        again = torch.full((S, M, N), float("nan"), device=DEV)
+        ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), again, feature_tiles=feature_tiles,
+                             fragments=ops.fragment_order(W.to(DEV)))
+        assert torch.equal(again, got)
     whole = x.float() @ W.float().T + b
     close(got.sum(0), whole, torch.float32, 200.0)
     if N % 4 == 0:
