@@ -161,17 +161,35 @@ class StaticStep:
         self.want_rows = (np.asarray(want_rows, dtype=np.int32) if lengths
                           else np.arange(lanes, dtype=np.int32))             # every lane's row is wanted
         needed, sizes, shapes, _ = _pack(_NO_LANES, cache, None, self.lengths, self.max_pages, self.want_rows)
-        self.host = torch.empty(-needed, dtype=torch.int32)
-        if torch.device(device).type == "cuda":
-            self.host = self.host.pin_memory()
-        self.host_words = self.host.numpy()
+        # The host packs a step into pinned memory and queues its copy to the fixed device addresses; the
+        # copy runs when the stream gets there, so the memory it reads must stay as it is until then.  A few
+        # host buffers are filled in turn, each guarded by an event recorded behind its copy: the host may
+        # run that many steps ahead of the GPU and no further.
+        on_gpu = torch.device(device).type == "cuda"
+        self._hosts = []
+        for _ in range(self.HOST_BUFFERS):
+            host = torch.empty(-needed, dtype=torch.int32)
+            self._hosts.append(host.pin_memory() if on_gpu else host)
+        self._copied = [torch.cuda.Event() if on_gpu else None for _ in self._hosts]
+        self._pending = [False] * len(self._hosts)
+        self._turn = 0
         self.device_buffer = torch.empty(-needed, dtype=torch.int32, device=device)
-        _pack(_NO_LANES, cache, self.host_words, self.lengths, self.max_pages, self.want_rows)
-        self.device_buffer.copy_(self.host)
+        _pack(_NO_LANES, cache, self._hosts[0].numpy(), self.lengths, self.max_pages, self.want_rows)
+        self.device_buffer.copy_(self._hosts[0])
         self.context = _assemble(_split(self.device_buffer, sizes), shapes, self.lengths, [0] * lanes, max_seq_len)
+
+    HOST_BUFFERS = 2
 
     def fill(self, lowered: LoweredLanes) -> None:
         """``lowered``: the real lanes, whose lengths are the first of this step's; the rest is padding."""
         real = len(lowered.slots)
-        _pack(lowered, self.cache, self.host_words, self.lengths[real:], self.max_pages, self.want_rows)
-        self.device_buffer.copy_(self.host, non_blocking=True)
+        turn = self._turn
+        self._turn = (turn + 1) % len(self._hosts)
+        if self._pending[turn]:
+            self._copied[turn].synchronize()          # the copy that last read this buffer has run
+        host = self._hosts[turn]
+        _pack(lowered, self.cache, host.numpy(), self.lengths[real:], self.max_pages, self.want_rows)
+        self.device_buffer.copy_(host, non_blocking=True)
+        if self._copied[turn] is not None:
+            self._copied[turn].record()
+            self._pending[turn] = True

@@ -21,6 +21,7 @@ src/decoder.rs:2129, 2336), and the muP multipliers are applied at run time
 """
 from __future__ import annotations
 
+import contextlib
 import json
 import math
 import os
@@ -28,6 +29,40 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 import torch.nn.functional as F
+
+
+# --------------------------------------------------------------------------- rounding of activations
+# The model below is exact float32 by default.  Inside ``activations_rounded_to(torch.bfloat16)`` every
+# activation that a 16-bit engine keeps in 16 bits between two kernels (normed rows, projected rows, rotated
+# queries and keys, attended rows, the conv's output, the gated scan output, the feed-forward's activations
+# and each branch's output) is rounded to that dtype and widened again; sums, softmax, norm statistics, the
+# recurrence and the residual stream stay float32.  The distance of that model from the exact one is what 16-bit
+# activations cost on a given set of weights: a measure of the model's conditioning, not of any kernel.
+# With ``dither`` (a torch.Generator) every value is first moved by a random fraction of its last kept bit, so
+# that several runs give several samples of the rounding noise (an engine that sums in another order, or folds
+# a multiplier into a weight, is one more sample of the same noise).
+_ROUND_TO: Optional[torch.dtype] = None
+_DITHER: Optional[torch.Generator] = None
+
+
+@contextlib.contextmanager
+def activations_rounded_to(dtype: Optional[torch.dtype], dither: Optional[torch.Generator] = None):
+    global _ROUND_TO, _DITHER
+    before = (_ROUND_TO, _DITHER)
+    _ROUND_TO, _DITHER = dtype, dither
+    try:
+        yield
+    finally:
+        _ROUND_TO, _DITHER = before
+
+
+def _r(x: torch.Tensor) -> torch.Tensor:
+    if _ROUND_TO is None:
+        return x
+    if _DITHER is not None:
+        bits = 8 if _ROUND_TO == torch.bfloat16 else 11 if _ROUND_TO == torch.float16 else 24
+        x = x * (1.0 + (torch.rand(x.shape, generator=_DITHER) - 0.5) * 2.0 ** -bits)
+    return x.to(_ROUND_TO).float()
 
 
 # --------------------------------------------------------------------------- parts
@@ -198,15 +233,15 @@ def attention_mixer(n: torch.Tensor, w: Dict[str, torch.Tensor], *, num_heads: i
     T = n.shape[0]
     positions = torch.arange(T) if positions is None else positions
     n = n.float() * in_multiplier
-    q = linear(n, w["q_proj.weight"], w.get("q_proj.bias")).view(T, num_heads, head_dim)
+    q = _r(linear(n, w["q_proj.weight"], w.get("q_proj.bias"))).view(T, num_heads, head_dim)
     k = linear(n, w["k_proj.weight"], w.get("k_proj.bias")).view(T, num_kv_heads, head_dim)
-    k = k * key_multiplier
-    v = linear(n, w["v_proj.weight"], w.get("v_proj.bias")).view(T, num_kv_heads, head_dim)
+    k = _r(k * key_multiplier)
+    v = _r(linear(n, w["v_proj.weight"], w.get("v_proj.bias"))).view(T, num_kv_heads, head_dim)
     if use_rope:
-        q = rope_half_split(q, positions, theta)
-        k = rope_half_split(k, positions, theta)
-    o = gqa_causal_attention(q, k, v, 1.0 / math.sqrt(head_dim), window)
-    return linear(o.reshape(T, num_heads * head_dim), w["o_proj.weight"], w.get("o_proj.bias")) * out_multiplier
+        q = _r(rope_half_split(q, positions, theta))
+        k = _r(rope_half_split(k, positions, theta))
+    o = _r(gqa_causal_attention(q, k, v, 1.0 / math.sqrt(head_dim), window))
+    return _r(linear(o.reshape(T, num_heads * head_dim), w["o_proj.weight"], w.get("o_proj.bias")) * out_multiplier)
 
 
 def mamba2_mixer(n: torch.Tensor, w: Dict[str, torch.Tensor], *, num_heads: int, head_dim: int,
@@ -230,21 +265,21 @@ def mamba2_mixer(n: torch.Tensor, w: Dict[str, torch.Tensor], *, num_heads: int,
         u = projected.float()
     T = u.shape[0]
     z, x, B, C, dt = torch.split(u, [E, E, GN, GN, num_heads], dim=-1)
-    z, x, B, C, dt = (z * multipliers[0], x * multipliers[1], B * multipliers[2],
-                      C * multipliers[3], dt * multipliers[4])
+    z, x, B, C, dt = (_r(z * multipliers[0]), _r(x * multipliers[1]), _r(B * multipliers[2]),
+                      _r(C * multipliers[3]), _r(dt * multipliers[4]))
     xbc = torch.cat([x, B, C], dim=-1)
     conv_weight = w["conv1d.weight"]
     if conv_weight.dim() == 3:                      # [C, 1, K] accepted, src/decoder.rs:2089-2095
         conv_weight = conv_weight.squeeze(1)
-    conv = F.silu(causal_depthwise_conv(xbc, conv_weight, w.get("conv1d.bias")))
+    conv = _r(F.silu(causal_depthwise_conv(xbc, conv_weight, w.get("conv1d.bias"))))
     xc, Bc, Cc = torch.split(conv, [E, GN, GN], dim=-1)
     A = -torch.exp(w["A_log"].float().reshape(num_heads))
     y, state = selective_scan(
         xc.view(T, num_heads, head_dim), Bc.view(T, num_groups, state_size),
         Cc.view(T, num_groups, state_size), dt, w["dt_bias"].float(), A,
         w["D"].float().reshape(num_heads))
-    y = gate_and_group_norm(y.reshape(T, E), z, w.get("norm.weight"), num_groups, eps)
-    out = linear(y, w["out_proj.weight"], w.get("out_proj.bias")) * out_multiplier
+    y = _r(gate_and_group_norm(y.reshape(T, E), z, w.get("norm.weight"), num_groups, eps))
+    out = _r(linear(y, w["out_proj.weight"], w.get("out_proj.bias")) * out_multiplier)
     if return_state:
         return out, state, xbc[-(conv_kernel - 1):] if conv_kernel > 1 else None
     return out
@@ -253,9 +288,9 @@ def mamba2_mixer(n: torch.Tensor, w: Dict[str, torch.Tensor], *, num_heads: int,
 def swiglu_mlp(f: torch.Tensor, w: Dict[str, torch.Tensor], gate_multiplier: float = 1.0,
                down_multiplier: float = 1.0) -> torch.Tensor:
     """down(SiLU(gate(f)) * up(f)) (src/decoder.rs:276-304)."""
-    gate = linear(f, w["gate_proj.weight"], w.get("gate_proj.bias")) * gate_multiplier
-    up = linear(f, w["up_proj.weight"], w.get("up_proj.bias"))
-    return linear(swiglu(gate, up), w["down_proj.weight"], w.get("down_proj.bias")) * down_multiplier
+    gate = _r(linear(f, w["gate_proj.weight"], w.get("gate_proj.bias")) * gate_multiplier)
+    up = _r(linear(f, w["up_proj.weight"], w.get("up_proj.bias")))
+    return _r(linear(_r(swiglu(gate, up)), w["down_proj.weight"], w.get("down_proj.bias")) * down_multiplier)
 
 
 # --------------------------------------------------------------------------- the model
@@ -273,7 +308,7 @@ def falcon_h1_layer(h: torch.Tensor, tensors: Dict[str, torch.Tensor], layer: in
     """
     prefix = f"model.layers.{layer}."
     eps = cfg.get("rms_norm_eps", 1e-5)
-    n = rms_norm(h, tensors[prefix + "attn_norm.weight"], eps)
+    n = _r(rms_norm(h, tensors[prefix + "attn_norm.weight"], eps))
     mixed = torch.zeros_like(h)
     if "attention" not in ablate:
         mixed = mixed + attention_mixer(
@@ -298,7 +333,7 @@ def falcon_h1_layer(h: torch.Tensor, tensors: Dict[str, torch.Tensor], layer: in
     h1 = h + mixed
     if "mlp" in ablate:
         return h1
-    f = rms_norm(h1, tensors[prefix + "ffn_norm.weight"], eps)
+    f = _r(rms_norm(h1, tensors[prefix + "ffn_norm.weight"], eps))
     mlp_multipliers = cfg.get("mlp_multipliers", [1.0, 1.0])
     return h1 + swiglu_mlp(f, _sub(tensors, prefix + "mlp."), mlp_multipliers[0], mlp_multipliers[1])
 
@@ -315,7 +350,7 @@ def falcon_h1_logits(cfg: dict, tensors: Dict[str, torch.Tensor], tokens: Sequen
     h = embedding[token_ids] * cfg.get("embedding_multiplier", 1.0)
     for layer in range(cfg["num_hidden_layers"]):
         h = falcon_h1_layer(h, tensors, layer, cfg, ablate)
-    h = rms_norm(h, tensors["model.norm.weight"], cfg.get("rms_norm_eps", 1e-5))
+    h = _r(rms_norm(h, tensors["model.norm.weight"], cfg.get("rms_norm_eps", 1e-5)))
     head = embedding if cfg.get("tie_word_embeddings", False) else tensors["lm_head.weight"].float()
     return (h @ head.T) * cfg.get("lm_head_multiplier", 1.0)
 

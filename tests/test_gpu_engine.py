@@ -390,6 +390,57 @@ def test_graphs_come_in_buckets_of_context_length():
     assert with_graphs.graphs.counts["decode_replays"] == 16
 
 
+def test_replays_that_follow_one_another_without_a_wait_keep_their_own_arrays(tmp_path):
+    """Steps of one captured shape whose logits nobody wants (portions of prompts, decoded tokens of a
+    replay that asks for nothing) are queued one behind the other while the GPU is still busy with earlier
+    work: each replay must run with the positions, cells and block tables that were packed for it, not with
+    those of a step packed later.  The host is made to run ahead by a second of matrix products queued
+    first; the engine beside it launches the same steps kernel by kernel."""
+    from macllm_infer_amd import Engine, Lane
+    folder = tiny_configs.make_model_dir("C", tmp_path, torch.bfloat16)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    plain = {key: tensor.float() for key, tensor in tensors.items()}
+    make = lambda graphs: Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=2048,
+                                 max_active_sequences=6, decode_graphs=graphs)
+    with_graphs, eager = make(True), make(False)
+    names = "abcde"
+    streams = {key: tokens_for(cfg["vocab_size"], 64 * 3 + 12, 40 + index) for index, key in enumerate(names)}
+    for engine in (with_graphs, eager):
+        for key in names:
+            engine.add_request(key)
+    # the shape (one lane of 64 tokens, nothing wanted) comes three times and is captured
+    plan = [("a", 0), ("b", 0), ("c", 0)]
+    busy = [("a", 64), ("b", 64), ("c", 64), ("d", 0), ("e", 0), ("a", 128), ("d", 64), ("e", 64)]
+    for key, first in plan:
+        for engine in (with_graphs, eager):
+            assert engine.step([Lane(key, streams[key][first:first + 64], [])]).shape[0] == 0
+    assert with_graphs.graphs.counts["portion_captures"] == 1
+    ballast = torch.randn(4096, 4096, device=DEV, dtype=torch.bfloat16)
+    for engine in (with_graphs, eager):
+        torch.cuda.synchronize()
+        for _ in range(200):                           # some hundred milliseconds of work the steps queue behind
+            ballast @ ballast
+        for key, first in busy:
+            engine.step([Lane(key, streams[key][first:first + 64], [])])
+    assert with_graphs.graphs.counts["portion_replays"] == 1 + len(busy)
+    # decoded tokens, every request in a step of its own with nothing wanted, then all at once with their logits
+    cursor = {"a": 192, "b": 128, "c": 128, "d": 128, "e": 128}
+    for engine in (with_graphs, eager):
+        for _ in range(100):
+            ballast @ ballast
+        for turn in range(4):
+            for key in names:
+                engine.step([Lane(key, [streams[key][cursor[key] + turn]], [])])
+    lanes = [Lane(key, [streams[key][cursor[key] + 4]], [0]) for key in names]
+    got, want = with_graphs.step(lanes).float().cpu(), eager.step(lanes).float().cpu()
+    assert with_graphs.graphs.counts["decode_replays"] == 21
+    assert (got - want).abs().max() <= 3e-2 * max(1.0, want.abs().max().item())
+    for key in names:                                  # and against the plain model
+        exact = plain_impl.falcon_h1_logits(cfg, plain, streams[key][:cursor[key] + 5])[-1]
+        row = got[names.index(key)]
+        assert (row - exact).abs().max() <= 6e-2 * exact.abs().max(), key
+
+
 @pytest.mark.parametrize("name, dtype", [("B", "float32"), ("C", "bfloat16")])
 def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
     """Steps of one shape (two prompt portions of 70 and 40 tokens, some places wanted) come back:
@@ -532,59 +583,73 @@ def test_a_wide_model_runs_through_the_fast_paths(tmp_path, monkeypatch, padding
         assert ((have - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()).item() <= 3e-2
 
 
-@pytest.mark.parametrize("seed", range(12))
-def test_configurations_drawn_at_random_match_the_plain_model(seed):
-    """Every size and option at random (head sizes 16..128 in steps of 16, 1..12 heads, odd widths
-    and vocabularies, pages of 4..64 tokens): whole, and two requests cut at random beside each
-    other with their last tokens one by one, in float32 and in bfloat16."""
-    import random
+# Seeds 0 to 7 of both draws, and the cases of earlier sweeps (100 and 60 seeds) whose bfloat16 logits left the
+# plain gate.  Every one of them is the model's conditioning, not a kernel: the plain model with its
+# activations rounded to bfloat16 departs from the exact one as far at the same positions (3038: a width of 40
+# over one state-space head of 64 x 64 with the gated norm, off by the whole scale at position 52, where the
+# float32 engine is off by 3e-4 instead of 3e-6; 3024: 0.27 of the scale at position 195; 3022, 3040, 3041 and
+# the odd draw's 1, 3, 12, 22, 23, 28, 34, 57: 0.06 to 0.18).  ``gates.conditioned_close`` states the gate in
+# those terms.
+RANDOM_CASES = ([(seed, False) for seed in range(8)] + [(seed, True) for seed in range(8)]
+                + [(seed, False) for seed in (3022, 3024, 3038, 3040, 3041)]
+                + [(seed, True) for seed in (12, 22, 23, 28, 34, 57)])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed, odd", RANDOM_CASES)
+def test_configurations_drawn_at_random_match_the_plain_model(seed, odd, dtype):
+    """Every size and option at random (head sizes 16..128 in steps of 16, 1..12 heads, widths and
+    vocabularies that are multiples of nothing, multipliers 0.5..2, pages of 4..64 tokens; ``odd``: sizes no
+    matrix-core kernel takes): whole, and two requests cut at random beside each other with their last tokens
+    one by one."""
+    import gates
     from macllm_infer_amd import Engine, Lane
     from macllm_infer_amd.config import FalconH1Config
     from macllm_infer_amd.weights.random_init import random_tensors
-    from test_gpu_replay import bfloat16_close
-    raw, page = tiny_configs.random_config(seed)
+    raw, page, rng = tiny_configs.random_config(seed, odd)
     config = FalconH1Config.from_dict(raw)
-    rng = random.Random(seed)
+    cfg = config.to_dict()
+    tensors = random_tensors(config, seed, torch.float32 if dtype == "float32" else torch.bfloat16, "unit")
+    plain = {name: tensor.float() for name, tensor in tensors.items()}
     generator = torch.Generator().manual_seed(seed)
-    first = torch.randint(0, raw["vocab_size"], (rng.choice([70, 131, 200]),), generator=generator).tolist()
-    second = torch.randint(0, raw["vocab_size"], (rng.choice([9, 40, 77]),), generator=generator).tolist()
-    for dtype in ("float32", "bfloat16"):
-        tensors = random_tensors(config, seed, torch.float32 if dtype == "float32" else torch.bfloat16, "unit")
-        plain = {name: tensor.float() for name, tensor in tensors.items()}
-        wanted = {"a": plain_impl.falcon_h1_logits(config.to_dict(), plain, first).numpy(),
-                  "b": plain_impl.falcon_h1_logits(config.to_dict(), plain, second).numpy()}
+    tokens = {"a": torch.randint(0, raw["vocab_size"], (rng.choice([70, 131, 200]),), generator=generator).tolist()}
+    tokens["b"] = torch.randint(0, raw["vocab_size"], (rng.choice([9, 40, 77]),), generator=generator).tolist()
+    wanted = {name: plain_impl.falcon_h1_logits(cfg, plain, tokens[name]).numpy() for name in tokens}
 
-        def close(got, want, what):
-            if dtype == "float32":
-                assert np.abs(got - want).max() <= 1e-4, f"seed {seed} {what}: {np.abs(got - want).max():.3e}"
-            else:
-                assert bfloat16_close(got, want), f"seed {seed} {what}: {np.abs(got - want).max():.3e} of {np.abs(want).max():.2f}"
+    def close(got, name, what):
+        want = wanted[name]
+        if dtype == "float32":
+            error = np.abs(got - want).max()
+            assert error <= gates.FLOAT32_TOLERANCE * max(1.0, np.abs(want).max()), f"seed {seed} {what}: {error:.3e}"
+        else:
+            ok, text = gates.conditioned_close(got, want, cfg, plain, tokens[name])
+            assert ok, f"seed {seed} {what}: {text}"
 
-        engine = Engine(config=config, tensors=tensors, dtype=dtype, kv_cache_block_tokens=page,
-                        kv_cache_capacity_tokens=640, max_active_sequences=3)
-        engine.add_request("whole")
-        close(engine.step([Lane("whole", first, list(range(len(first))))]).cpu().numpy(), wanted["a"], "whole")
-        engine.finish("whole")
-        engine.add_request("a")
-        engine.add_request("b")
-        tokens, cursor, rows = {"a": first, "b": second}, {"a": 0, "b": 0}, {"a": [], "b": []}
-        while cursor["a"] < len(first) or cursor["b"] < len(second):
-            lanes = []
-            for name, tail, sizes in (("a", 12, [2, 5, 17, 64, 33]), ("b", 6, [2, 3, 11, 30])):
-                left = len(tokens[name]) - cursor[name]
-                if left > 0 and (name == "a" or rng.random() < 0.7):
-                    count = 1 if left <= tail else min(rng.choice(sizes), left - tail)
-                    lanes.append(Lane(name, tokens[name][cursor[name]:cursor[name] + count], list(range(count))))
-            if not lanes:
-                continue
-            out = engine.step(lanes).cpu().numpy()
-            for lane in lanes:
-                rows[lane.request].append(out[:len(lane.tokens)])
-                out = out[len(lane.tokens):]
-                cursor[lane.request] += len(lane.tokens)
-        for name in ("a", "b"):
-            close(np.concatenate(rows[name]), wanted[name], f"cut {name}")
-        engine.cache.check()
+    engine = Engine(config=config, tensors=tensors, dtype=dtype, kv_cache_block_tokens=page,
+                    kv_cache_capacity_tokens=640, max_active_sequences=3)
+    engine.add_request("whole")
+    close(engine.step([Lane("whole", tokens["a"], list(range(len(tokens["a"]))))]).cpu().numpy(), "a", "whole")
+    engine.finish("whole")
+    engine.add_request("a")
+    engine.add_request("b")
+    cursor, rows = {"a": 0, "b": 0}, {"a": [], "b": []}
+    while cursor["a"] < len(tokens["a"]) or cursor["b"] < len(tokens["b"]):
+        lanes = []
+        for name, tail, sizes in (("a", 12, [2, 5, 17, 64, 33]), ("b", 6, [2, 3, 11, 30])):
+            left = len(tokens[name]) - cursor[name]
+            if left > 0 and (name == "a" or rng.random() < 0.7):
+                count = 1 if left <= tail else min(rng.choice(sizes), left - tail)
+                lanes.append(Lane(name, tokens[name][cursor[name]:cursor[name] + count], list(range(count))))
+        if not lanes:
+            continue
+        out = engine.step(lanes).cpu().numpy()
+        for lane in lanes:
+            rows[lane.request].append(out[:len(lane.tokens)])
+            out = out[len(lane.tokens):]
+            cursor[lane.request] += len(lane.tokens)
+    for name in ("a", "b"):
+        close(np.concatenate(rows[name]), name, f"cut {name}")
+    engine.cache.check()
 
 
 @pytest.mark.parametrize("shape, layers, vocab", [("0.5b", 2, None), ("7b", 1, 1003)])
@@ -598,7 +663,7 @@ def test_layers_of_the_benchmark_shapes_match_the_plain_model(shape, layers, voc
     from macllm_infer_amd import Engine, Lane
     from macllm_infer_amd.config import FalconH1Config
     from macllm_infer_amd.weights.random_init import random_tensors
-    from test_gpu_replay import bfloat16_close
+    from gates import bfloat16_close
     raw = dict(bench.SHAPES[shape], num_hidden_layers=layers)
     config = FalconH1Config.from_dict(dict(raw, vocab_size=vocab or raw["vocab_size"]))
     tensors = random_tensors(config, 7, torch.bfloat16, "unit")

@@ -10,18 +10,9 @@ import torch
 import plain_impl
 import tiny_configs
 import traces
+from gates import FLOAT32_TOLERANCE, bfloat16_close
 
 pytestmark = pytest.mark.gpu
-
-FLOAT32_TOLERANCE = 1e-4           # max-abs on logits, every split
-
-
-def bfloat16_close(got, want):
-    """bfloat16 rounds to 8 bits (2^-8 = 0.4 %) at some thirty places between tokens and
-    logits; errors add up as a random walk to a few per cent of the logits' scale."""
-    scale = np.abs(want).max()
-    relative_rms = np.sqrt(((got - want) ** 2).mean() / (want ** 2).mean())
-    return np.abs(got - want).max() <= 0.06 * scale and relative_rms <= 0.03
 
 
 def requests_for(cfg, lengths, seed):
@@ -111,3 +102,33 @@ def test_nothing_wanted_writes_no_file_and_larger_pages(model, tmp_path):
     rows = np.fromfile(tmp_path / "1.f32", dtype="<f4").reshape(2, cfg["vocab_size"])
     want = plain_impl.falcon_h1_logits(cfg, tensors, tokens).numpy()[[40, 69]]
     assert np.abs(rows - want).max() <= FLOAT32_TOLERANCE if dtype == "float32" else bfloat16_close(rows, want)
+
+
+def test_decoded_tokens_whose_logits_nobody_wants(model, tmp_path):
+    """Three requests decode in turn, one request a step, and ask for no logits for forty steps in a row:
+    the replay program answers each step without waiting for the GPU, so steps of one shape queue one
+    behind the other.  The logits of the tokens after that must be those of the whole sequences."""
+    name, dtype, folder, cfg, tensors = model
+    requests = requests_for(cfg, [80, 75, 70], seed=6)
+    steps = []
+    for key, tokens in requests.items():
+        steps.append({"entries": [{"id": key, "tokens": tokens[:20], "want": []}], "end": []})
+    for turn in range(40):
+        for key, tokens in requests.items():
+            steps.append({"entries": [{"id": key, "tokens": [tokens[20 + turn]], "want": []}], "end": []})
+    wanted = {}
+    for key, tokens in requests.items():
+        for position in range(60, len(tokens)):
+            steps.append({"entries": [{"id": key, "tokens": [tokens[position]], "want": [0]}],
+                          "end": [key] if position == len(tokens) - 1 else []})
+    traces.number(steps)
+    traces.replay(folder, dtype, steps, max_tokens=256, out_dir=tmp_path)
+    got = traces.collect(steps, tmp_path, cfg["vocab_size"], {key: len(tokens) for key, tokens in requests.items()})
+    for key, tokens in requests.items():
+        want = plain_impl.falcon_h1_logits(cfg, tensors, tokens).numpy()[60:]
+        rows = got[key][60:]
+        assert not np.isnan(rows).any() and np.isnan(got[key][:60]).all()
+        if dtype == "float32":
+            assert np.abs(rows - want).max() <= FLOAT32_TOLERANCE, key
+        else:
+            assert bfloat16_close(rows, want), key

@@ -365,3 +365,43 @@ def test_every_branch_matters_in_the_tiny_models():
         # and the past matters: changing the first token changes the last logits
         other = [tokens[0] + 1] + tokens[1:]
         assert (P.falcon_h1_logits(raw, tensors, other)[-1] - full[-1]).abs().max() > 1e-3
+
+
+def test_rounding_activations_shows_a_models_conditioning_without_any_kernel():
+    """The plain model with its activations rounded to bfloat16 stays within a few per cent of the exact
+    one on the tiny configurations; on a randomly drawn model that amplifies rounding noise (a width of 40
+    over one state-space head of 64 x 64 with the gated norm, seed 3038 of the random draw) it leaves by a
+    large part of the logits' scale at the same position 52 at which a 16-bit engine does, and the rest
+    of the sequence stays close: the departure is the model's, and the gate says so."""
+    import gates
+    import tiny_configs
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.weights.random_init import random_tensors
+    for name in ("A", "B", "C"):
+        raw, seed = tiny_configs.CONFIGS[name]
+        tensors = {key: value.float() for key, value in
+                   random_tensors(FalconH1Config.from_dict(raw), seed, torch.bfloat16, "unit").items()}
+        tokens = torch.randint(0, raw["vocab_size"], (90,), generator=torch.Generator().manual_seed(5)).tolist()
+        exact = P.falcon_h1_logits(raw, tensors, tokens).numpy()
+        with P.activations_rounded_to(torch.bfloat16):
+            rounded = P.falcon_h1_logits(raw, tensors, tokens).numpy()
+        assert gates.bfloat16_close(rounded, exact), name
+        assert abs(rounded - exact).max() > 1e-4          # and the rounding is there
+        assert (P.falcon_h1_logits(raw, tensors, tokens).numpy() == exact).all()      # and gone again
+    raw, _, rng = tiny_configs.random_config(3038)
+    tensors = {key: value.float() for key, value in
+               random_tensors(FalconH1Config.from_dict(raw), 3038, torch.bfloat16, "unit").items()}
+    tokens = torch.randint(0, raw["vocab_size"], (rng.choice([70, 131, 200]),),
+                           generator=torch.Generator().manual_seed(3038)).tolist()
+    exact = P.falcon_h1_logits(raw, tensors, tokens).numpy()
+    with P.activations_rounded_to(torch.bfloat16):
+        rounded = P.falcon_h1_logits(raw, tensors, tokens).numpy()
+    error = abs(rounded - exact).max(axis=1)
+    scale = abs(exact).max()
+    assert error.argmax() == 52 and error[52] > 0.2 * scale and not gates.bfloat16_close(rounded, exact)
+    assert sorted(error)[len(error) // 2] < 0.03 * scale
+    ok, text = gates.conditioned_close(rounded, exact, raw, tensors, tokens)
+    assert ok, text
+    # a fault is not excused: the logits of the neighbouring position fail the same gate
+    ok, text = gates.conditioned_close(np.roll(exact, 1, axis=0), exact, raw, tensors, tokens)
+    assert not ok, text

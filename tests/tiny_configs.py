@@ -59,30 +59,35 @@ def make_model_dir(name, folder, dtype=torch.float32, preset="unit"):
     return write_random_model(FalconH1Config.from_dict(raw), seed, str(folder), dtype, preset)
 
 
-def random_config(seed):
-    """A tiny configuration with every size and option drawn at random: head sizes in steps of 16,
-    head counts and groups that are no powers of two, odd widths and vocabularies."""
+def random_config(seed, odd=False):
+    """(configuration, page size, the generator that drew them) with every size and option drawn at random:
+    head sizes in steps of 16, head counts and groups that are no powers of two, widths and vocabularies that
+    are no multiples of anything, multipliers between 0.5 and 2.  ``odd``: widths, state sizes and chunks
+    that no matrix-core kernel takes (the scalar paths of every part)."""
     import random
     rng = random.Random(seed)
     divisors = lambda n: [d for d in range(1, n + 1) if n % d == 0]
     heads = rng.choice([1, 2, 3, 4, 6, 8, 12])
     mamba_heads = rng.choice([1, 2, 3, 4, 6, 8])
-    head = rng.choice([8, 16, 24, 32, 64])
-    factor = lambda: rng.uniform(0.7, 1.4)
+    head = rng.choice([4, 12, 20, 36] if odd else [8, 16, 24, 32, 64])
+    factor = lambda: rng.uniform(0.5, 2)
     raw = dict(
         architectures=["FalconH1ForCausalLM"], model_type="falcon_h1",
-        hidden_size=rng.choice([40, 72, 100, 128, 136, 256, 520]), num_hidden_layers=rng.choice([1, 2]),
+        hidden_size=rng.choice([30, 50, 66, 90, 34] if odd else [40, 72, 100, 128, 136, 256, 520]),
+        num_hidden_layers=rng.choice([1, 2]),
         num_attention_heads=heads, num_key_value_heads=rng.choice(divisors(heads)),
-        head_dim=rng.choice([16, 32, 48, 64, 80, 128]), intermediate_size=rng.choice([24, 100, 136, 256]),
-        vocab_size=rng.choice([97, 320, 1003]), max_position_embeddings=512,
+        head_dim=rng.choice([16, 32, 48, 64, 80, 128]),
+        intermediate_size=rng.choice([10, 30, 50, 7] if odd else [24, 100, 136, 256]),
+        vocab_size=rng.choice([33, 50, 129] if odd else [97, 320, 1003]), max_position_embeddings=512,
         rms_norm_eps=rng.choice([1e-5, 1e-6, 3e-4]), rope_theta=rng.choice([1e4, 1e6, 1e11]),
         mamba_n_heads=mamba_heads, mamba_d_head=head, mamba_d_ssm=mamba_heads * head,
-        mamba_d_state=rng.choice([8, 16, 32, 40, 64, 128]), mamba_n_groups=rng.choice(divisors(mamba_heads)),
-        mamba_d_conv=rng.choice([2, 3, 4]), mamba_chunk_size=rng.choice([8, 32, 64, 128]),
+        mamba_d_state=rng.choice([4, 12, 24, 20] if odd else [8, 16, 32, 40, 64, 128]),
+        mamba_n_groups=rng.choice(divisors(mamba_heads)),
+        mamba_d_conv=rng.choice([2, 3, 4]), mamba_chunk_size=rng.choice([5, 16, 48, 100] if odd else [8, 32, 64, 128]),
         mamba_conv_bias=rng.random() < 0.5, mamba_proj_bias=rng.random() < 0.5, mamba_rms_norm=rng.random() < 0.5,
         attention_bias=rng.random() < 0.5, mlp_bias=rng.random() < 0.5, tie_word_embeddings=rng.random() < 0.5,
         embedding_multiplier=factor(), lm_head_multiplier=factor(), key_multiplier=factor(),
         attention_in_multiplier=factor(), attention_out_multiplier=factor(), ssm_in_multiplier=factor(),
         ssm_out_multiplier=factor(), ssm_multipliers=[factor() for _ in range(5)],
         mlp_multipliers=[factor() for _ in range(2)])
-    return raw, rng.choice([4, 8, 16, 64])
+    return raw, rng.choice([4, 8, 16, 64]), rng
