@@ -132,8 +132,8 @@ def collect(steps, out_dir, vocab, lengths):
         path = os.path.join(str(out_dir), f"{step['step']}.f32")
         if wanted == 0:
             assert not os.path.exists(path)
-            continue
-        rows = np.fromfile(path, dtype="<f4").reshape(wanted, vocab)
+        else:
+            rows = np.fromfile(path, dtype="<f4").reshape(wanted, vocab)
         row = 0
         for entry in step["entries"]:
             for place in entry["want"]:
