@@ -469,6 +469,59 @@ extern "C" int mi_decode_attention(const void* q, long q_ld, int T, int Hq, int 
   return 0;
 }
 
+// ---------------------------------------------------------------- decode attention without a workspace argument
+// The partial results live in an array of the library's device image (see static_scratch.h).  In host code
+// the array's name is a stand-in, not a device address: its address on each GPU is asked for once per
+// device, with that device current, and kept.
+#include "static_scratch.h"
+#include <mutex>
+
+static __device__ __align__(256) float scratch[MI_STATIC_SCRATCH_BYTES / sizeof(float)];
+
+#define STATIC_MAX_DEVICES 64
+static float* scratch_of_device[STATIC_MAX_DEVICES];
+static std::mutex scratch_lock;
+
+// The address of this GPU's copy of `scratch`, or null with *error set.
+static float* static_scratch(hipError_t* error) {
+  int device = -1;
+  *error = hipGetDevice(&device);
+  if (*error != hipSuccess) return nullptr;
+  if (device < 0 || device >= STATIC_MAX_DEVICES) {
+    *error = hipErrorInvalidDevice;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (scratch_of_device[device] == nullptr) {
+    float* address = nullptr;
+    *error = hipGetSymbolAddress((void**)&address, HIP_SYMBOL(scratch));
+    if (*error != hipSuccess) return nullptr;
+    scratch_of_device[device] = address;
+  }
+  return scratch_of_device[device];
+}
+
+extern "C" long mi_static_scratch_bytes(void) { return (long)MI_STATIC_SCRATCH_BYTES; }
+
+extern "C" int mi_decode_attention_static(const void* q, long q_ld, int T, int Hq, int Hkv, int dh,
+                                          const void* k_base, const void* v_base, long page_stride, int page_size,
+                                          const int* block_tables, int max_pages, const int* lane_of_token,
+                                          const int* positions, float scale, int window, int split_keys,
+                                          int splits, void* out, long out_ld, hipStream_t stream) {
+  if (T <= 0 || Hq <= 0 || dh <= 0 || splits <= 0) return ERR_BAD_ARGUMENT;
+  // partial outputs first, their (max, sum) behind them, each part in whole runs of 256 bytes
+  const unsigned long long rows = (unsigned long long)T * (unsigned long long)Hq * (unsigned long long)splits;
+  const unsigned long long o_floats = (rows * (unsigned long long)dh + 63ull) & ~63ull;
+  const unsigned long long ml_floats = (rows * 2ull + 63ull) & ~63ull;
+  if (o_floats + ml_floats > MI_STATIC_SCRATCH_BYTES / sizeof(float)) return ERR_UNSUPPORTED_SIZE;
+  hipError_t error = hipSuccess;
+  float* base = static_scratch(&error);
+  if (base == nullptr) return (int)error;
+  return mi_decode_attention(q, q_ld, T, Hq, Hkv, dh, k_base, v_base, page_stride, page_size, block_tables,
+                             max_pages, lane_of_token, positions, scale, window, split_keys, splits, base,
+                             base + o_floats, out, out_ld, stream);
+}
+
 // ---------------------------------------------------------------- prefill attention on the matrix cores
 // bfloat16, head_dim 64 or 128.  grid = (4 x query tiles, kv heads, head passes): a tile is up to 64
 // consecutive tokens of one lane and a workgroup takes 16 of them with the query heads of one kv
