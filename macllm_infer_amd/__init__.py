@@ -4,12 +4,13 @@ manager with state slots, one step function over mixed batches, a continuous-bat
 scheduler, GPU sampling, and hand-written HIP kernels with a true float32 path."""
 from .cache import CacheExhausted
 from .config import ConfigError, FalconH1Config, load_config, register_architecture
-from .engine import LLM, Engine, EngineConfig, GenerationResult, Lane, Scheduler, StepError, generate
+from .engine import (LLM, Engine, EngineConfig, GenerationResult, Lane, Scheduler, StepError, StepFailed,
+                     generate)
 from .sampling import GREEDY, Sampler, SamplingParams
 from .weights import WeightError
 
 __version__ = "0.1.0"
 
 __all__ = ["CacheExhausted", "ConfigError", "Engine", "EngineConfig", "FalconH1Config", "GREEDY",
-           "GenerationResult", "LLM", "Lane", "Sampler", "SamplingParams", "Scheduler", "StepError",
+           "GenerationResult", "LLM", "Lane", "Sampler", "SamplingParams", "Scheduler", "StepError", "StepFailed",
            "WeightError", "generate", "load_config", "register_architecture"]

@@ -24,6 +24,13 @@ TENSOR_ALIASES = ((".input_layernorm.", ".attn_norm."), (".pre_ff_layernorm.", "
                   (".feed_forward.", ".mlp."), ("model.final_layernorm.", "model.norm."))
 
 
+# the config.json keys behind the fields of the parts' specs, for messages about sizes the kernels refuse
+FIELD_NAMES = (("attention.head_dim", "head_dim"), ("attention.num_heads", "num_attention_heads"),
+               ("mamba2.conv_kernel", "mamba_d_conv"), ("mamba2.state_size", "mamba_d_state"),
+               ("mamba2.num_heads", "mamba_n_heads"), ("mamba2.num_groups", "mamba_n_groups"),
+               ("rmsnorm.hidden_size", "hidden_size"))
+
+
 @dataclass(frozen=True)
 class FalconH1Config:
     hidden_size: int
@@ -103,9 +110,36 @@ class FalconH1Config:
             raise ConfigError("config.json: 'sliding_window' is not supported for Falcon-H1")
         if raw.get("hidden_act", "silu") != "silu":
             raise ConfigError(f"config.json: 'hidden_act' must be 'silu', got {raw.get('hidden_act')!r}")
-        if raw.get("mamba_norm_before_gate", False):
-            raise ConfigError("config.json: 'mamba_norm_before_gate' = true is not supported "
-                              "(the gated norm runs after the gate)")
+        # the gated norm runs after the gate; the flag says nothing when there is no such norm
+        if raw.get("mamba_norm_before_gate", False) and raw.get("mamba_rms_norm", False):
+            raise ConfigError("config.json: 'mamba_norm_before_gate' = true together with 'mamba_rms_norm' is not "
+                              "supported (the gated norm runs after the gate)")
+        # the step size is softplus(dt + bias) as it comes (src/decoder.rs:2321-2324 has no clamp)
+        limit = raw.get("time_step_limit")
+        if limit is not None:
+            if (not isinstance(limit, (list, tuple)) or len(limit) != 2
+                    or any(isinstance(v, bool) or not isinstance(v, (int, float)) for v in limit)):
+                raise ConfigError(f"config.json: 'time_step_limit' must be a pair of numbers, got {limit!r}")
+            if float(limit[0]) > 0.0 or float(limit[1]) != float("inf"):
+                raise ConfigError(f"config.json: 'time_step_limit' {list(limit)!r} is not supported: the step size "
+                                  "is not clamped (only [0, inf])")
+        # newer writers keep the rope settings in one table: {"rope_theta": ..., "rope_type": "default"}
+        rope = raw.get("rope_parameters")
+        rope_theta_default = 1e11
+        if rope is not None:
+            if not isinstance(rope, dict):
+                raise ConfigError(f"config.json: 'rope_parameters' must be a table, got {rope!r}")
+            if rope.get("rope_type", rope.get("type", "default")) != "default":
+                raise ConfigError(f"config.json: 'rope_parameters.rope_type' "
+                                  f"{rope.get('rope_type', rope.get('type'))!r} is not supported (only 'default')")
+            if rope.get("rope_theta") is not None:
+                inner = rope["rope_theta"]
+                if isinstance(inner, bool) or not isinstance(inner, (int, float)):
+                    raise ConfigError(f"config.json: 'rope_parameters.rope_theta' must be a number, got {inner!r}")
+                if raw.get("rope_theta") is not None and float(raw["rope_theta"]) != float(inner):
+                    raise ConfigError(f"config.json: 'rope_theta' {raw['rope_theta']!r} and "
+                                      f"'rope_parameters.rope_theta' {inner!r} disagree")
+                rope_theta_default = float(inner)
 
         hidden = integer("hidden_size")
         heads = integer("num_attention_heads")
@@ -149,7 +183,7 @@ class FalconH1Config:
             attention_bias=flag("attention_bias", False),
             mlp_bias=flag("mlp_bias", False),
             rms_norm_eps=number("rms_norm_eps", 1e-5),
-            rope_theta=number("rope_theta", 1e11),
+            rope_theta=number("rope_theta", rope_theta_default),
             tie_word_embeddings=flag("tie_word_embeddings", False),
             embedding_multiplier=number("embedding_multiplier", 1.0),
             lm_head_multiplier=number("lm_head_multiplier", 1.0),
@@ -238,6 +272,7 @@ class FalconH1Config:
             embedding_multiplier=self.embedding_multiplier,
             logit_multiplier=self.lm_head_multiplier,
             tensor_aliases=TENSOR_ALIASES,
+            field_names=FIELD_NAMES,
         )
 
     # ------------------------------------------------------------------ reports

@@ -208,6 +208,8 @@ class ModelSpec:
     tensor_aliases: Tuple[Tuple[str, str], ...] = ()
     # a checkpoint none of whose names starts with this gets it in front of all but the output head's
     root_namespace: str = "model."
+    # ("part kind.spec field", the configuration file's key for it): for messages that name a field
+    field_names: Tuple[Tuple[str, str], ...] = ()
 
     def validate(self) -> None:
         """Positivity, divisibility and bounds, field by field (src/architecture.rs:367-452)."""

@@ -4,9 +4,15 @@
 wanted): portions of prompts beside single decoded tokens, cut anywhere.  It runs only
 the tokens it is given, as one batch, from the cache earlier steps left, and returns the
 logits at the wanted places.  Everything is validated and all pages are reserved before
-anything is launched, so a refused step changes nothing
+anything is launched, so a refused step (``StepError``, ``CacheExhausted``) changes nothing.
+Sizes that a kernel would refuse are found when the engine is built, before a weight is
+read (``ConfigError``).  A step that fails after its reservation, in a launch or anywhere
+else, leaves nothing half done behind: the kernels write keys, values and state in place, so
+the requests of that step cannot go on; they are ended, their pages and slots given back,
+and ``StepFailed`` names them
 (reference: src/architecture.rs:1187-1227 contract, src/decoder.rs:3878-3968 checks,
-:4125-4201 transactional execute).
+:4125-4201 transactional execute, which restores a checkpoint where this ends the requests;
+src/architecture.rs:367-667 validation before load).
 """
 from __future__ import annotations
 
@@ -18,6 +24,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.pages import CacheExhausted
 from ..config.registry import config_from_dict, load_config
+from ..config.spec import ConfigError
 from ..kernels import build as kernel_build
 from ..kernels import ops
 from ..parts.base import BuildContext
@@ -31,6 +38,17 @@ _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.
 
 class StepError(ValueError):
     """A step was refused before anything ran; the engine's state is unchanged."""
+
+
+class StepFailed(RuntimeError):
+    """A step failed after its pages were reserved.  ``requests``: the requests of its lanes, which have
+    been ended (their pages and state slots are free again, their tokens so far are lost); every other
+    request is as it was.  ``__cause__`` is the error that stopped the step."""
+
+    def __init__(self, requests, cause: BaseException):
+        self.requests = list(requests)
+        super().__init__(f"the step failed and its requests {self.requests!r} were ended: "
+                         f"{type(cause).__name__}: {cause}")
 
 
 def resolve_dtype(dtype) -> torch.dtype:
@@ -56,16 +74,18 @@ class Engine:
         self.device = ops.require_gpu(device) if check_device else torch.device(device)
         if model_dir is not None:
             self.config = load_config(model_dir)
-            source = WeightSource.from_dir(model_dir)
         else:
             self.config = config_from_dict(config) if isinstance(config, dict) else config
-            source = WeightSource.from_tensors(tensors)
         self.spec = self.config.to_model_spec()
         self.spec.validate()
+        beyond = DecoderModel.limits(self.spec)
+        if beyond:                                  # before any weight is read
+            raise ConfigError("config.json: " + "; ".join(limit.text(self.spec.field_names) for limit in beyond))
+        source = WeightSource.from_dir(model_dir) if model_dir is not None else WeightSource.from_tensors(tensors)
         if check_device:
             kernel_build.ensure_modules(DecoderModel.kernel_modules(self.spec) + list(kernel_build.HOST_MODULES))
         source.apply_aliases(self.spec.tensor_aliases, root_prefix=self.spec.root_namespace)
-        bound = bind(source, DecoderModel.expected_tensors(self.spec))
+        bound = bind(source, DecoderModel.expected_tensors(self.spec), DecoderModel.tensor_copies(self.spec))
         source.close()
         build = BuildContext(hidden_size=self.spec.hidden_size, dtype=self.dtype, device=self.device,
                              max_context=self.spec.max_context)
@@ -138,17 +158,25 @@ class Engine:
 
     def step(self, lanes: Sequence[Lane]) -> torch.Tensor:
         """Run one batch; returns float32 logits [wanted, vocab] in the order of the lanes and
-        of each lane's ``want``.  Raises StepError or CacheExhausted with nothing changed."""
+        of each lane's ``want``.  Raises StepError or CacheExhausted with nothing changed, or
+        StepFailed with the lanes' requests ended and everything they held given back."""
         lowered = self.validate(lanes)
         self.cache.reserve_slots(lowered.slots, lowered.lengths)
-        logits = None
-        if self.graphs is not None:
-            if int(lowered.lengths.max()) == 1:
-                logits = self.graphs.run(lanes, lowered)              # decode-only batch: a captured graph
-            else:
-                logits = self.graphs.run_portion(lanes, lowered)      # a shape of prompt portions seen before
-        if logits is None:
-            context = build_step_context(lanes, self.cache, self.device, lowered)
-            logits = self.model.forward(context, self.cache)
+        try:
+            logits = None
+            if self.graphs is not None:
+                if int(lowered.lengths.max()) == 1:
+                    logits = self.graphs.run(lanes, lowered)              # decode-only batch: a captured graph
+                else:
+                    logits = self.graphs.run_portion(lanes, lowered)      # a shape of prompt portions seen before
+            if logits is None:
+                context = build_step_context(lanes, self.cache, self.device, lowered)
+                logits = self.model.forward(context, self.cache)
+        except Exception as error:
+            # earlier layers have written keys, values and state in place: these requests cannot go on
+            names = [lane.request for lane in lanes]
+            for name in names:
+                self.cache.finish(name)
+            raise StepFailed(names, error) from error
         self.cache.commit_slots(lowered.slots, lowered.lengths)
         return logits

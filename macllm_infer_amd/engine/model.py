@@ -29,6 +29,24 @@ class DecoderModel:
         return out
 
     @staticmethod
+    def tensor_copies(spec: ModelSpec) -> Dict[str, str]:
+        """Tensors a checkpoint may hold although the model binds another one in their place, if both are
+        equal: a tied model saved with its output head written out beside the embedding."""
+        if spec.tied_embeddings:
+            return {f"{spec.lm_head_name}.weight": f"{spec.embedding_name}.weight"}
+        return {}
+
+    @staticmethod
+    def limits(spec: ModelSpec) -> list:
+        """Every size of the model that some part's kernels refuse, each once (``kernels.limits.Limit``)."""
+        found = list(part_class(spec.final_norm).limits(spec.final_norm, spec.hidden_size))
+        for layer in spec.layers:
+            arrangement = arrangement_class(layer.arrangement)
+            if hasattr(arrangement, "limits"):
+                found += arrangement.limits(layer, spec.hidden_size)
+        return list(dict.fromkeys(found))
+
+    @staticmethod
     def kernel_modules(spec: ModelSpec) -> List[str]:
         modules = ["common", "gemm"]
         for layer in spec.layers:

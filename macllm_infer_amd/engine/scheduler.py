@@ -9,7 +9,8 @@ Each round (reference: ``ServingScheduler::drive_once``, src/engine.rs:1938-1988
   3. run all chosen lanes as one step.  If the pages do not suffice the last lane is
      dropped and the step retried (:2145-2149); if a single lane cannot fit, that request
      alone fails with ``resource_exhausted`` and gives back what it holds (:2150-2153,
-     :2205-2231).  There is no preemption or swap;
+     :2205-2231).  There is no preemption or swap.  A step that fails once launched ends the
+     requests of its lanes (``failed: ...``), whose pages and slots the engine has taken back;
   4. sample for the lanes whose last prompt token or decoded token ran; a cancelled request ends
      before its token is emitted, a stop token ends the request without being emitted, a
      ``False`` from the caller's ``on_token`` ends it after the token, ``max_new_tokens`` ends
@@ -29,6 +30,7 @@ from ..cache.pages import CacheExhausted
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import SamplerRow
 from .context import Lane
+from .engine import StepFailed
 
 
 @dataclass
@@ -161,10 +163,11 @@ class Scheduler:
             visits.append((request, tokens, samples))
         return visits
 
-    def _finish(self, request: Request, reason: str) -> None:
+    def _finish(self, request: Request, reason: str, release: bool = True) -> None:
         request.finish_reason = reason
         request.finished_at = time.perf_counter()
-        self.engine.finish(request.request_id)
+        if release:
+            self.engine.finish(request.request_id)
         self.active.remove(request)
         self.finished[request.request_id] = request
 
@@ -188,6 +191,11 @@ class Scheduler:
                 else:
                     self._finish(visits[0][0], "resource_exhausted")
                     visits = self._collect()
+            except StepFailed as failure:
+                # the engine has ended the step's requests and taken back what they held; the others go on
+                for request, _, _ in visits:
+                    self._finish(request, f"failed: {failure.__cause__}", release=False)
+                visits = []
         if visits:
             sampled = [(request, tokens) for request, tokens, samples in visits if samples]
             for request, tokens, samples in visits:

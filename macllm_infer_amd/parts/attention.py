@@ -5,6 +5,7 @@ import torch
 
 from ..cache.manager import KVNeed
 from ..kernels import ops
+from ..kernels.limits import ATTENTION_MAX_HEAD_DIM, GRID_MOST, beyond
 from ..weights.loader import Expect
 from .base import BuildContext, Mixer, part_class, register_part
 from .linear import Linear
@@ -39,6 +40,13 @@ class Attention(Mixer):
         if spec.out_bias:
             out.append(Expect(f"{prefix}.o_proj.bias", ((hidden_size,),), init="bias"))
         return out
+
+    @classmethod
+    def limits(cls, spec, hidden_size: int):
+        return (beyond("attention", "head_dim", spec.head_dim, ATTENTION_MAX_HEAD_DIM,
+                       "a query row and its sums are kept in LDS and registers")
+                + beyond("attention", "num_heads", spec.num_heads, GRID_MOST, "heads index a dimension of the launch")
+                + part_class(spec.position).limits(spec.position, spec.head_dim))
 
     @classmethod
     def cache_needs(cls, spec):

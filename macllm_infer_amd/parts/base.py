@@ -16,7 +16,8 @@ mixer           ``cache_needs(spec) -> [KVNeed | StateNeed]`` (classmethod);
 feed-forward    ``forward(x [T, d]) -> [T, d]``
 norm            ``forward(residual, rows=None) -> normed activations``
 position        ``rotate_and_store(qkv, heads, kv_heads, head_dim, step, cache)``
-every part      ``graph_safe = True`` if its forward may be captured in a HIP graph
+every part      ``graph_safe = True`` if its forward may be captured in a HIP graph;
+                ``limits(spec, hidden_size) -> [Limit]`` (classmethod): sizes its kernels refuse
 """
 from __future__ import annotations
 
@@ -69,6 +70,12 @@ class Part:
 
     @classmethod
     def expected_tensors(cls, spec, prefix: str, hidden_size: int):
+        return []
+
+    @classmethod
+    def limits(cls, spec, hidden_size: int):
+        """The sizes of ``spec`` that no kernel of this part takes, as ``kernels.limits.Limit``s: asked when a
+        model is built, before its weights are read.  A part whose kernels take every size reports none."""
         return []
 
 

@@ -41,6 +41,14 @@ class ParallelPreNormBlock:
         return out
 
     @classmethod
+    def limits(cls, layer, hidden_size: int):
+        """What the kernels of this layer's parts refuse (see ``Part.limits``)."""
+        out = []
+        for spec in [layer.mixer_norm, layer.ffn_norm, layer.ffn] + [slot.spec for slot in layer.mixers]:
+            out += part_class(spec).limits(spec, hidden_size)
+        return out
+
+    @classmethod
     def kernel_modules(cls, layer):
         modules = []
         for spec in [layer.mixer_norm, layer.ffn_norm, layer.ffn] + [slot.spec for slot in layer.mixers]:

@@ -5,6 +5,7 @@ import torch
 
 from ..cache.manager import StateNeed
 from ..kernels import ops
+from ..kernels.limits import CONV_MAX_TAPS, GRID_MOST, SCAN_MAX_STATE, beyond
 from ..weights.loader import Expect
 from .base import BuildContext, Mixer, register_part
 from .linear import Linear
@@ -44,6 +45,13 @@ class Mamba2(Mixer):
                               ((spec.num_groups, spec.inner_size // spec.num_groups), (spec.inner_size,)),
                               init="norm"))
         return out
+
+    @classmethod
+    def limits(cls, spec, hidden_size: int):
+        return (beyond("mamba2", "conv_kernel", spec.conv_kernel, CONV_MAX_TAPS, "the taps of a channel are kept in registers")
+                + beyond("mamba2", "state_size", spec.state_size, SCAN_MAX_STATE, "a state row is spread over one wave")
+                + beyond("mamba2", "num_heads", spec.num_heads, GRID_MOST, "heads index a dimension of the launch")
+                + beyond("mamba2", "num_groups", spec.num_groups, GRID_MOST, "groups index a dimension of the launch"))
 
     @classmethod
     def cache_needs(cls, spec):

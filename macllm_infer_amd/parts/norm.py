@@ -6,6 +6,7 @@ from typing import Optional
 import torch
 
 from ..kernels import ops
+from ..kernels.limits import NORM_MAX_WIDTH, beyond
 from ..weights.loader import Expect
 from .base import BuildContext, Part, Residual, register_part
 
@@ -35,6 +36,10 @@ class RmsNorm(Part):
     @classmethod
     def expected_tensors(cls, spec, prefix: str, hidden_size: int):
         return [Expect(f"{prefix}.weight", ((hidden_size,),), init="norm")]
+
+    @classmethod
+    def limits(cls, spec, hidden_size: int):
+        return beyond("rmsnorm", "hidden_size", hidden_size, NORM_MAX_WIDTH, "the norm stages a float32 row in 64 KiB of LDS")
 
     def __init__(self, spec, prefix: str, tensors, build: BuildContext):
         self.eps = spec.eps

@@ -151,15 +151,28 @@ class _MemoryFile:
         return None
 
 
-def bind(source: WeightSource, expectations: Sequence[Expect]) -> Dict[str, torch.Tensor]:
+def bind(source: WeightSource, expectations: Sequence[Expect],
+         copies: Optional[Dict[str, str]] = None) -> Dict[str, torch.Tensor]:
     """Check the whole checkpoint against ``expectations`` and return name -> CPU tensor
-    (canonical shape, stored dtype; integer tables as int32)."""
+    (canonical shape, stored dtype; integer tables as int32).  ``copies``: name of a tensor the model
+    does not bind -> the bound tensor it may repeat (a tied output head saved beside the embedding);
+    it is accepted when both hold the same values and reported as unexpected otherwise."""
     wanted = {}
     for expect in expectations:
         wanted[expect.name] = expect                      # a name asked for twice (tied weights) is one tensor
     present = set(source.names())
     missing = sorted(name for name in wanted if name not in present)
-    unexpected = sorted(source.stored_name(name) for name in present if name not in wanted)
+    unexpected = []
+    for name in sorted(present - set(wanted)):
+        original = (copies or {}).get(name)
+        if original in wanted and original in present:
+            if (tuple(source.shape(name)) == tuple(source.shape(original))
+                    and torch.equal(source.tensor(name), source.tensor(original))):
+                continue
+            unexpected.append(f"{source.stored_name(name)} (the model shares {original}, and this tensor differs from it)")
+        else:
+            unexpected.append(source.stored_name(name))
+    unexpected.sort()
     unexpected += [f"{stored} (the same tensor as {other})" for stored, other in source.clashes]
     wrong_shape: List[Tuple[str, Tuple, Tuple]] = []
     wrong_dtype: List[Tuple[str, str]] = []

@@ -54,7 +54,13 @@ def test_state_and_cache_sizes_match_the_reference_gate():
     ({"rope_scaling": {"type": "linear", "factor": 2}}, "rope_scaling"),
     ({"sliding_window": 128}, "sliding_window"),
     ({"hidden_act": "gelu"}, "hidden_act"),
-    ({"mamba_norm_before_gate": True}, "mamba_norm_before_gate"),
+    ({"mamba_norm_before_gate": True, "mamba_rms_norm": True}, "mamba_norm_before_gate"),
+    ({"time_step_limit": [0.001, 0.1]}, "time_step_limit"),
+    ({"time_step_limit": [0.0, 100.0]}, "time_step_limit"),
+    ({"time_step_limit": "none"}, "time_step_limit"),
+    ({"rope_parameters": {"rope_type": "yarn", "rope_theta": 1e6, "factor": 4.0}}, "rope_type"),
+    ({"rope_parameters": {"rope_theta": 1e6}, "rope_theta": 1e4}, "disagree"),
+    ({"rope_parameters": [1e6]}, "rope_parameters"),
     ({"vocab_size": "many"}, "vocab_size"),
     ({"max_position_embeddings": 1 << 21}, "max_position_embeddings"),
 ])
@@ -78,6 +84,30 @@ def test_registry_maps_names_and_lists_them_for_an_unknown_one(tmp_path):
         config_from_dict({"hidden_size": 8})
     with pytest.raises(ConfigError, match="does not exist"):
         load_config(str(tmp_path))
+
+
+def test_config_as_the_family_tooling_writes_it():
+    """What checkpoints of the family carry in config.json beyond this engine's own keys: the rope base inside
+    a ``rope_parameters`` table, ``mamba_norm_before_gate`` (which says nothing when there is no gated norm),
+    an unclamped ``time_step_limit``, and keys that do not change the computation.  The result is the same
+    typed configuration, and so the same model, as the engine's own spelling gives."""
+    own = dict(tiny_configs.TINY_A, rope_theta=5e5)
+    theirs = {key: value for key, value in own.items() if key != "rope_theta"}
+    theirs.update(rope_parameters={"rope_theta": 5e5, "rope_type": "default"}, mamba_norm_before_gate=True,
+                  time_step_limit=[0.0, float("inf")], time_step_min=0.001, time_step_max=0.1, time_step_floor=1e-4,
+                  mamba_expand=2, mamba_use_mlp=True, projectors_bias=False, rope_scaling=None, sliding_window=None,
+                  num_logits_to_keep=1, bos_token_id=1, pad_token_id=0, use_cache=True, initializer_range=0.02,
+                  attention_dropout=0.0, transformers_version="5.0.0", dtype="bfloat16")
+    config = FalconH1Config.from_dict(json.loads(json.dumps(theirs)))         # through text, Infinity included
+    assert config == FalconH1Config.from_dict(own) and config.rope_theta == 5e5
+    assert config.to_model_spec() == FalconH1Config.from_dict(own).to_model_spec()
+    both = dict(own, rope_parameters={"rope_theta": 5e5})
+    assert FalconH1Config.from_dict(both).rope_theta == 5e5
+    # the flag matters only beside the gated norm
+    gated = dict(tiny_configs.TINY_B, mamba_norm_before_gate=False)
+    assert FalconH1Config.from_dict(gated) == FalconH1Config.from_dict(tiny_configs.TINY_B)
+    # and the engine's own spelling round-trips through its own writer
+    assert FalconH1Config.from_dict(config.to_dict()) == config
 
 
 def test_unknown_keys_are_ignored():
@@ -140,6 +170,27 @@ def test_weight_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     text = str(error)
     for word in ("model.layers.1.mamba.D", "lm_head.weight", "expected [32, 64], got [16, 64]"):
         assert word in text
+
+
+def test_a_tied_model_saved_with_its_output_head_binds_if_the_head_is_the_embedding():
+    config = tiny_configs.config("A")
+    spec = config.to_model_spec()
+    assert spec.tied_embeddings
+    tensors = random_tensors(config, 0, torch.float32)
+    expectations, copies = DecoderModel.expected_tensors(spec), DecoderModel.tensor_copies(spec)
+    tensors["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    bound = bind(WeightSource.from_tensors(tensors), expectations, copies)
+    assert "lm_head.weight" not in bound and len(bound) == len(tensors) - 1
+    tensors["lm_head.weight"][3, 5] += 1.0
+    with pytest.raises(WeightError, match="differs") as caught:
+        bind(WeightSource.from_tensors(tensors), expectations, copies)
+    assert len(caught.value.unexpected) == 1 and not caught.value.missing
+    tensors["lm_head.weight"] = torch.zeros(7, 64)
+    with pytest.raises(WeightError, match="differs"):
+        bind(WeightSource.from_tensors(tensors), expectations, copies)
+    # an untied model binds its head and allows no copy
+    untied = tiny_configs.config("B").to_model_spec()
+    assert DecoderModel.tensor_copies(untied) == {}
 
 
 def test_alternative_shapes_and_widening(tmp_path):

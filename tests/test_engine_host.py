@@ -145,3 +145,112 @@ def test_toy_parts_register_build_and_step_on_the_host(host_ops, schedule):
     cache, registered from the tests and stepped through the engine."""
     import toy_parts
     toy_parts.exercise(schedule, "cpu", check_device=False)
+
+
+def test_a_step_that_fails_once_launched_ends_its_requests_and_leaves_the_others_alone(host_ops, tmp_path, monkeypatch):
+    """A kernel refuses in the second layer, after the first has written keys, values and state in place:
+    the requests of that step are ended and give back pages and slots (the reference restores a checkpoint
+    instead, src/decoder.rs:4146-4190); a request that was not in the step goes on and still matches."""
+    from macllm_infer_amd import StepFailed
+    from macllm_infer_amd.kernels import ops
+    engine, cfg, tensors = engine_for("B", tmp_path, capacity=96, page=8, requests=3)
+    bystander, first, second = tokens_for(cfg, 30, 1), tokens_for(cfg, 20, 2), tokens_for(cfg, 9, 3)
+    for name in ("bystander", "first", "second"):
+        engine.add_request(name)
+    engine.step([Lane("bystander", bystander[:17], []), Lane("first", first[:12], [11])])
+    free_before = engine.cache.stats()["groups"][0]["free_pages"]
+    held = {name: len(engine.cache.table(0, name).live_pages()) for name in ("first", "bystander")}
+    real, calls = ops.gate_norm, {"count": 0}
+
+    def refuses_in_the_second_layer(*arguments, **named):
+        calls["count"] += 1
+        if calls["count"] == 2:
+            raise ops.KernelError("gate_norm: size not supported by this kernel")
+        return real(*arguments, **named)
+
+    monkeypatch.setattr(ops, "gate_norm", refuses_in_the_second_layer)
+    with pytest.raises(StepFailed) as caught:
+        engine.step([Lane("first", first[12:], [7]), Lane("second", second, [8])])
+    assert caught.value.requests == ["first", "second"] and isinstance(caught.value.__cause__, ops.KernelError)
+    assert not engine.has_request("first") and not engine.has_request("second") and engine.has_request("bystander")
+    stats = engine.cache.stats()
+    assert stats["groups"][0]["free_pages"] == free_before + held["first"] and stats["free_slots"] == 2
+    engine.cache.check()
+    monkeypatch.setattr(ops, "gate_norm", real)
+    want = plain_impl.falcon_h1_logits(cfg, tensors, bystander)
+    got = engine.step([Lane("bystander", bystander[17:], list(range(13)))])
+    assert (got - want[17:]).abs().max() < 1e-4
+    # the names are free again: the same request can start over in the slot and pages it gave back
+    engine.add_request("first")
+    got = engine.step([Lane("first", first, [19])])
+    assert (got - plain_impl.falcon_h1_logits(cfg, tensors, first)[[19]]).abs().max() < 1e-4
+
+
+def test_the_scheduler_fails_the_requests_of_a_failed_step_and_serves_the_rest(host_ops, tmp_path, monkeypatch):
+    from macllm_infer_amd.kernels import ops
+    engine, cfg, tensors = engine_for("A", tmp_path, capacity=160, page=8, requests=3)
+    sampler = Sampler(engine.vocab_size, "cpu", check_device=False)
+    scheduler = Scheduler(engine, sampler, EngineConfig(max_active_sequences=1, scheduler_token_budget=64,
+                                                        prefill_token_quantum=64))
+    prompts = [tokens_for(cfg, length, 70 + length) for length in (9, 14)]
+    params = SamplingParams(max_new_tokens=4, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0)
+    for index, prompt in enumerate(prompts):
+        scheduler.submit(index, prompt, params)
+    real, calls = ops.swiglu, {"count": 0}
+
+    def refuses_once(*arguments, **named):
+        calls["count"] += 1
+        if calls["count"] == 4:                  # the second decode step of request 0 (two layers a step)
+            raise ops.KernelError("swiglu: bad argument")
+        return real(*arguments, **named)
+
+    monkeypatch.setattr(ops, "swiglu", refuses_once)
+    finished = scheduler.run()
+    assert finished[0].finish_reason.startswith("failed: swiglu") and len(finished[0].generated) == 1
+    assert finished[1].finish_reason == "length"
+    assert finished[1].generated == plain_impl.greedy_generate(cfg, tensors, prompts[1], 4)
+    stats = engine.cache.stats()
+    assert stats["live_requests"] == 0 and stats["free_slots"] == 3
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("change, word", [
+    ({"mamba_d_conv": 17}, "'mamba_d_conv' = 17"),
+    ({"mamba_d_state": 520}, "'mamba_d_state' = 520"),
+    ({"head_dim": 258}, "'head_dim' = 258"),
+    ({"hidden_size": 16416, "num_attention_heads": 6}, "'hidden_size' = 16416"),
+    ({"mamba_d_conv": 20, "head_dim": 300}, "'head_dim' = 300.*'mamba_d_conv' = 20"),
+])
+def test_sizes_no_kernel_takes_are_refused_before_a_weight_is_read(change, word):
+    """The limits are the kernels' own (a test below reads them in the sources); the error names the
+    config.json key; ``tensors=None`` shows that no weight was asked for."""
+    from macllm_infer_amd.config import ConfigError
+    raw = dict(tiny_configs.TINY_B)
+    raw.update(change)
+    with pytest.raises(ConfigError, match=word):
+        Engine(config=raw, tensors=None, dtype="float32", device="cpu", check_device=False)
+    for dtype in ("float32", "bfloat16"):
+        with pytest.raises(ConfigError, match="more than the kernels take"):
+            Engine(config=raw, tensors=None, dtype=dtype, device="cpu", check_device=False)
+
+
+def test_the_limits_are_the_ones_in_the_kernel_sources():
+    import os
+    import re
+    from macllm_infer_amd.kernels import build, limits
+
+    def define(module, name):
+        with open(os.path.join(build.CSRC, f"{module}.hip")) as handle:
+            return int(re.search(rf"#define {name} (\d+)", handle.read()).group(1))
+
+    assert limits.ATTENTION_MAX_HEAD_DIM == define("attention", "ATT_MAX_DH")
+    assert limits.CONV_MAX_TAPS == define("mamba2", "CONV_MAX_K")
+    assert limits.SCAN_MAX_STATE == 64 * define("mamba2", "SCAN_MAX_PER_THREAD")
+    with open(os.path.join(build.CSRC, "common.hip")) as handle:
+        assert "(size_t)d * sizeof(float) > 64 * 1024" in handle.read()
+    assert limits.NORM_MAX_WIDTH * 4 == 64 * 1024
+    # and the sizes at the limits are accepted
+    raw = dict(tiny_configs.TINY_B, mamba_d_conv=16, mamba_d_state=512, head_dim=256)
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.engine.model import DecoderModel
+    assert DecoderModel.limits(FalconH1Config.from_dict(raw).to_model_spec()) == []
