@@ -27,19 +27,37 @@ from .pages import BlockTable, CacheExhausted, PagePool, SlotPool
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Token-proportional cache: K and V of ``num_kv_heads`` x ``head_dim`` per token;
-    ``window`` = how many of the most recent tokens must stay (None = all)."""
+    """Token-proportional cache: per token, keys of ``num_kv_heads`` x ``head_dim`` and values of
+    ``num_kv_heads`` x ``value_dim`` (None: the keys' width); ``window`` = how many of the most recent
+    tokens must stay (None = all)."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
+    token_proportional = True             # what tells this need from one of fixed size, whatever its class
+
+    @property
+    def value_width(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)
 class StateNeed:
-    """Fixed-size per-request state ``name`` of ``shape``; dtype "activation" or "float32"."""
+    """Fixed-size per-request state ``name`` of ``shape``; dtype "activation" (the engine's 16- or 32-bit
+    dtype), "float32", or any ``torch.dtype``."""
     name: str
     shape: Tuple[int, ...]
-    dtype: str = "float32"
+    dtype: object = "float32"
+    token_proportional = False
+
+    def storage_dtype(self, activation: torch.dtype) -> torch.dtype:
+        if isinstance(self.dtype, torch.dtype):
+            return self.dtype
+        if self.dtype == "activation":
+            return activation
+        if self.dtype == "float32":
+            return torch.float32
+        raise ValueError(f"state {self.name!r}: dtype {self.dtype!r} is neither 'activation', 'float32' nor a torch.dtype")
 
 
 class Core:
@@ -81,24 +99,28 @@ class PagedGroup:
 
     def allocate(self, dtype: torch.dtype, device) -> None:
         need = self.need
-        # one page more than the pool hands out: the scratch page padding lanes of a captured step write to
-        self.storage = torch.zeros((self.num_pages + 1, len(self.members), 2, need.num_kv_heads,
-                                    self.page_size * need.head_dim), dtype=dtype, device=device)
+        # one page more than the pool hands out: the scratch page padding lanes of a captured step write to.
+        # A layer's share of a page: its keys [kv head, token, key dim], then its values [kv head, value dim, token]
+        self.storage = torch.zeros((self.num_pages + 1, len(self.members),
+                                    need.num_kv_heads * self.page_size * (need.head_dim + need.value_width)),
+                                   dtype=dtype, device=device)
 
     @property
     def scratch_page(self) -> int:
         return self.num_pages
 
     def layer_views(self, layer: int):
-        """One layer's K pages [pages, Hkv, page_size, dh] and V pages [pages, Hkv, dh, page_size]
+        """One layer's K pages [pages, Hkv, page_size, key dim] and V pages [pages, Hkv, value dim, page_size]
         (V is kept transposed: its product contracts over tokens)."""
         need = self.need
-        return (self.storage[:, layer, 0].unflatten(-1, (self.page_size, need.head_dim)),
-                self.storage[:, layer, 1].unflatten(-1, (need.head_dim, self.page_size)))
+        keys = need.num_kv_heads * self.page_size * need.head_dim
+        return (self.storage[:, layer, :keys].unflatten(-1, (need.num_kv_heads, self.page_size, need.head_dim)),
+                self.storage[:, layer, keys:].unflatten(-1, (need.num_kv_heads, need.value_width, self.page_size)))
 
     def bytes_per_page(self, element_size: int) -> int:
         need = self.need
-        return 2 * len(self.members) * need.num_kv_heads * self.page_size * need.head_dim * element_size
+        return (len(self.members) * need.num_kv_heads * self.page_size * (need.head_dim + need.value_width)
+                * element_size)
 
     def check(self) -> None:
         held = [page for table in self.tables.values() for page in table.live_pages()]
@@ -151,7 +173,7 @@ class CacheManager:
         for key, key_needs in needs.items():
             entry = EntryCache(states={})
             for need in key_needs:
-                if isinstance(need, KVNeed):
+                if getattr(need, "token_proportional", False):
                     if key in shared_kv:
                         continue
                     if need not in group_of:
@@ -160,7 +182,7 @@ class CacheManager:
                     group = group_of[need]
                     layer_of[key] = (group, self.groups[group].add_member(key))
                 elif isinstance(need, StateNeed):
-                    state_dtype = dtype if need.dtype == "activation" else torch.float32
+                    state_dtype = need.storage_dtype(dtype)
                     # one slot more than the pool hands out: the scratch slot of padding lanes
                     tensor = torch.zeros((max_requests + 1,) + tuple(need.shape), dtype=state_dtype,
                                          device=self.device)
@@ -179,7 +201,7 @@ class CacheManager:
             source = shared_kv.get(key, key)
             if source in layer_of:
                 if key in shared_kv:
-                    own = [need for need in needs[key] if isinstance(need, KVNeed)]
+                    own = [need for need in needs[key] if getattr(need, "token_proportional", False)]
                     theirs = self.groups[layer_of[source][0]].need
                     if not own or own[0] != theirs:
                         raise ValueError(f"{key} cannot read the cache of {source}: their needs differ")

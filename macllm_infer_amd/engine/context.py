@@ -23,7 +23,7 @@ import torch
 from ..cache import native
 
 
-QUERY_TILE = 64        # tokens of one lane that one workgroup of the prefill attention kernel takes
+NO_TILES = 1 << 30     # the table of runs then has one run per lane: no mixer of the model reads it
 
 
 @dataclass
@@ -45,7 +45,7 @@ class StepContext:
     seq_lens: torch.Tensor           # [lanes] request length after the step
     slot_ids: torch.Tensor           # [lanes] state slot of each lane's request
     want_rows: torch.Tensor          # [wanted] token rows whose logits are returned
-    query_tiles: torch.Tensor        # [tiles, 2] (lane, first token row) of runs of up to 64 tokens of one lane
+    query_tiles: torch.Tensor        # [tiles, 2] (lane, first token row) of runs of up to ``query_tile`` tokens of one lane
     block_tables: List[torch.Tensor] = field(default_factory=list)   # per group [lanes, max_pages]
     slot_mappings: List[torch.Tensor] = field(default_factory=list)  # per group [T] page*page_size+offset
     lane_lengths: List[int] = field(default_factory=list)            # host copies
@@ -85,11 +85,12 @@ _NO_LANES = LoweredLanes(*(np.zeros(0, dtype=np.int32) for _ in range(5)))
 
 
 def _pack(lowered: LoweredLanes, cache, out: Optional[np.ndarray], pad_lengths: Sequence[int] = (),
-          max_pages: Optional[int] = None, want_rows: Optional[np.ndarray] = None):
+          max_pages: Optional[int] = None, want_rows: Optional[np.ndarray] = None, query_tile: int = 0):
     """The core writes the step's sections (in the order of ``_assemble``) into ``out``.  Returns
     (words written or, negated, words needed when ``out`` is too small or None; section sizes;
     block-table shapes; longest context after the step).  ``pad_lengths``: lanes appended on the
-    scratch page and slot.  ``want_rows`` replaces the lanes' own wanted rows."""
+    scratch page and slot.  ``want_rows`` replaces the lanes' own wanted rows.  ``query_tile``: the
+    longest run of one lane's tokens in the table of runs (what the model's mixers ask for; 0: none does)."""
     core = cache.core
     pads = native.as_ints(list(pad_lengths))
     groups = len(cache.groups)
@@ -98,7 +99,7 @@ def _pack(lowered: LoweredLanes, cache, out: Optional[np.ndarray], pad_lengths: 
     written = core.lib.hc_pack(
         core.pointer, len(lowered.slots), native.int_pointer(lowered.slots), native.int_pointer(lowered.lengths),
         native.int_pointer(lowered.tokens), native.int_pointer(lowered.want_counts), native.int_pointer(lowered.wants),
-        len(pads), native.int_pointer(pads), max_pages or 0, QUERY_TILE,
+        len(pads), native.int_pointer(pads), max_pages or 0, query_tile or NO_TILES,
         native.int_pointer(fixed) if fixed is not None else None, len(fixed) if fixed is not None else 0,
         native.int_pointer(out) if out is not None else None, out.size if out is not None else 0,
         native.int_pointer(meta))
@@ -131,15 +132,17 @@ def _split(buffer: torch.Tensor, sizes):
     return views
 
 
-def build_step_context(lanes: Sequence[Lane], cache, device, lowered: Optional[LoweredLanes] = None) -> StepContext:
-    """``cache``: the CacheManager, after the step's pages were reserved."""
+def build_step_context(lanes: Sequence[Lane], cache, device, lowered: Optional[LoweredLanes] = None,
+                       query_tile: int = 0) -> StepContext:
+    """``cache``: the CacheManager, after the step's pages were reserved.  ``query_tile``: see ``_pack``
+    (``DecoderModel.query_tile`` for a whole model)."""
     if lowered is None:
         lowered = lower_lanes(lanes, cache)
-    needed, _, _, _ = _pack(lowered, cache, None)
+    needed, _, _, _ = _pack(lowered, cache, None, query_tile=query_tile)
     host = torch.empty(-needed, dtype=torch.int32)
     if torch.device(device).type == "cuda":
         host = host.pin_memory()
-    _, sizes, shapes, longest = _pack(lowered, cache, host.numpy())
+    _, sizes, shapes, longest = _pack(lowered, cache, host.numpy(), query_tile=query_tile)
     packed = host.to(device, non_blocking=True)
     starts = cache.lengths_of(lowered.slots).tolist()
     context = _assemble(_split(packed, sizes), shapes, lowered.lengths.tolist(), starts, longest)
@@ -153,14 +156,16 @@ class StaticStep:
     ``fill`` rewrites them for the real lanes of a step of that shape."""
 
     def __init__(self, cache, lanes: int, max_seq_len: int, device, lengths: Sequence[int] = (),
-                 want_rows: Sequence[int] = ()):
+                 want_rows: Sequence[int] = (), query_tile: int = 0):
         self.cache = cache
+        self.query_tile = query_tile
         self.lanes = lanes
         self.lengths = list(lengths) if lengths else [1] * lanes
         self.max_pages = max(-(-max_seq_len // group.page_size) for group in cache.groups) if cache.groups else 1
         self.want_rows = (np.asarray(want_rows, dtype=np.int32) if lengths
                           else np.arange(lanes, dtype=np.int32))             # every lane's row is wanted
-        needed, sizes, shapes, _ = _pack(_NO_LANES, cache, None, self.lengths, self.max_pages, self.want_rows)
+        needed, sizes, shapes, _ = _pack(_NO_LANES, cache, None, self.lengths, self.max_pages, self.want_rows,
+                                         query_tile)
         # The host packs a step into pinned memory and queues its copy to the fixed device addresses; the
         # copy runs when the stream gets there, so the memory it reads must stay as it is until then.  A few
         # host buffers are filled in turn, each guarded by an event recorded behind its copy: the host may
@@ -174,7 +179,7 @@ class StaticStep:
         self._pending = [False] * len(self._hosts)
         self._turn = 0
         self.device_buffer = torch.empty(-needed, dtype=torch.int32, device=device)
-        _pack(_NO_LANES, cache, self._hosts[0].numpy(), self.lengths, self.max_pages, self.want_rows)
+        _pack(_NO_LANES, cache, self._hosts[0].numpy(), self.lengths, self.max_pages, self.want_rows, query_tile)
         self.device_buffer.copy_(self._hosts[0])
         self.context = _assemble(_split(self.device_buffer, sizes), shapes, self.lengths, [0] * lanes, max_seq_len)
 
@@ -188,7 +193,8 @@ class StaticStep:
         if self._pending[turn]:
             self._copied[turn].synchronize()          # the copy that last read this buffer has run
         host = self._hosts[turn]
-        _pack(lowered, self.cache, host.numpy(), self.lengths[real:], self.max_pages, self.want_rows)
+        _pack(lowered, self.cache, host.numpy(), self.lengths[real:], self.max_pages, self.want_rows,
+              self.query_tile)
         self.device_buffer.copy_(host, non_blocking=True)
         if self._copied[turn] is not None:
             self._copied[turn].record()

@@ -170,7 +170,7 @@ class Engine:
                 else:
                     logits = self.graphs.run_portion(lanes, lowered)      # a shape of prompt portions seen before
             if logits is None:
-                context = build_step_context(lanes, self.cache, self.device, lowered)
+                context = build_step_context(lanes, self.cache, self.device, lowered, self.model.query_tile)
                 logits = self.model.forward(context, self.cache)
         except Exception as error:
             # earlier layers have written keys, values and state in place: these requests cannot go on

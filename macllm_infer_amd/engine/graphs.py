@@ -90,7 +90,8 @@ class DecodeGraphs:
             for length, want in zip(lengths, wants):
                 rows += [first + place for place in want]
                 first += length
-            static = StaticStep(self.cache, len(lengths), context, self.device, lengths=lengths, want_rows=rows)
+            static = StaticStep(self.cache, len(lengths), context, self.device, lengths=lengths, want_rows=rows,
+                                query_tile=self.model.query_tile)
             entry = self._capture(0, static, warm_runs=1)      # the libraries have seen these sizes already
             self.counts["portion_captures"] += 1
             while len(self._portion_graphs) >= self.PORTION_GRAPHS:
@@ -114,7 +115,8 @@ class DecodeGraphs:
 
     def _capture(self, bucket: int, static: Optional[StaticStep] = None, warm_runs: int = 2, context: int = 0):
         if static is None:
-            static = StaticStep(self.cache, bucket, context or self.max_seq_len, self.device)
+            static = StaticStep(self.cache, bucket, context or self.max_seq_len, self.device,
+                                query_tile=self.model.query_tile)
         # a first run outside the graph lets the libraries set themselves up; every lane is padding,
         # so only the scratch page and slot are touched
         side = torch.cuda.Stream(device=self.device)

@@ -64,7 +64,7 @@ class DecoderModel:
             for slot in layer.mixers:
                 key = (index, slot.name)
                 needs[key] = list(part_class(slot.spec).cache_needs(slot.spec))
-                if entry.kv_from is not None and any(type(need).__name__ == "KVNeed" for need in needs[key]):
+                if entry.kv_from is not None and any(getattr(need, "token_proportional", False) for need in needs[key]):
                     shared[key] = (entry.kv_from, slot.name)
         return needs, shared
 
@@ -89,6 +89,12 @@ class DecoderModel:
         fused_head = (build.device.type == "cuda" and build.dtype == torch.bfloat16 and self.lm_head.dtype == torch.bfloat16
                       and spec.hidden_size % 32 == 0 and ops.fused_gemm_supported(True, 1, spec.hidden_size))
         self._head_fragments = ops.fragment_order(self.lm_head) if fused_head else None
+        # the final norm as the skinny kernel's prologue, if it is that kind of norm
+        prologue = getattr(self.final_norm, "rms_prologue", None)
+        self._final_rms = prologue() if prologue is not None else None
+        # the step's table of runs of one lane's tokens is cut for the mixer with the largest tile
+        self.query_tile = max((getattr(mixer, "query_tile", 0) for block in self.blocks for _, mixer in block.mixers),
+                              default=0)
 
     @property
     def graph_safe(self) -> bool:
@@ -112,7 +118,7 @@ class DecoderModel:
         if self._fused_head(step, wanted):
             # a decode step whose every row is wanted: residual add, norm, projection and scaling in one launch
             ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, h_in=residual.h,
-                           deltas=residual.pending, norm_weight=self.final_norm.weight, eps=self.final_norm.eps,
+                           deltas=residual.pending, norm_weight=self._final_rms[0], eps=self._final_rms[1],
                            fragments=self._head_fragments)
             return logits
         normed = self.final_norm.forward(residual, rows=step.want_rows)
@@ -121,9 +127,8 @@ class DecoderModel:
         return logits
 
     def _fused_head(self, step, wanted: int) -> bool:
-        from ..parts.norm import RmsNorm
         return (step.max_query_len == 1 and wanted == step.num_tokens and wanted <= 16
                 and self.build.dtype == torch.bfloat16 and self.lm_head.dtype == torch.bfloat16
-                and type(self.final_norm) is RmsNorm and len(step.lane_lengths) == wanted
+                and self._final_rms is not None and len(step.lane_lengths) == wanted
                 and self.build.device.type == "cuda" and self.spec.hidden_size % 32 == 0
                 and ops.fused_gemm_supported(True, wanted, self.spec.hidden_size))

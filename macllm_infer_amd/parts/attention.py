@@ -24,6 +24,7 @@ class Attention(Mixer):
     the output projection's output."""
     graph_safe = True
     kernel_modules = ("common", "attention", "gemm")
+    query_tile = 64          # tokens of one lane that a workgroup of the prompt attention kernels takes
 
     @classmethod
     def expected_tensors(cls, spec, prefix: str, hidden_size: int):
@@ -70,6 +71,9 @@ class Attention(Mixer):
                           weight_scale=spec.out_multiplier, bias_scale=spec.out_multiplier)
         self.position = part_class(spec.position)(spec.position, spec.head_dim, build)
         self.graph_safe = bool(getattr(self.position, "graph_safe", False))
+
+    def projections(self):
+        return self.qkv, self.out, self.spec.num_heads * self.spec.head_dim
 
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         spec = self.spec

@@ -12,9 +12,12 @@ every part      ``expected_tensors(spec, prefix, hidden_size) -> [Expect]`` (cla
                 ``kernel_modules`` (names of the HIP modules it launches),
                 ``__init__(spec, prefix, tensors, build)``
 mixer           ``cache_needs(spec) -> [KVNeed | StateNeed]`` (classmethod);
-                ``forward(x [T, d], step, cache: EntryCache) -> [T, d]``
-feed-forward    ``forward(x [T, d]) -> [T, d]``
-norm            ``forward(residual, rows=None) -> normed activations``
+                ``forward(x [T, d], step, cache: EntryCache) -> [T, d]``;
+                optional ``projections()`` + ``mix(...)``: see ``Mixer.projections``
+feed-forward    ``forward(x [T, d]) -> [T, d]``; optional ``gated_projections()``
+norm            ``forward(residual, rows=None) -> normed activations``; optional ``rms_prologue() ->
+                (weight, eps)``: the norm is y = x / sqrt(mean(x^2) + eps) * weight, which the skinny
+                kernels compute in their prologue
 position        ``rotate_and_store(qkv, heads, kv_heads, head_dim, step, cache)``
 every part      ``graph_safe = True`` if its forward may be captured in a HIP graph;
                 ``limits(spec, hidden_size) -> [Limit]`` (classmethod): sizes its kernels refuse
@@ -80,6 +83,10 @@ class Part:
 
 
 class Mixer(Part):
+    # rows of one lane that one workgroup of the mixer's prompt kernel takes: the step's table of such runs
+    # is cut to the largest tile any mixer of the model names (0: the mixer reads no such table)
+    query_tile = 0
+
     @classmethod
     def cache_needs(cls, spec):
         return []
@@ -87,7 +94,22 @@ class Mixer(Part):
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         raise NotImplementedError
 
+    def projections(self):
+        """A mixer that is "input projection of the normed rows, something in between, output projection"
+        may hand out the three pieces: ``(in Linear, out Linear, width of what lies between)``, with
+        ``mix(projected [T, in.out_features], step, cache, out [T, width])`` doing the part in between on
+        column views of wider matrices.  A layer can then run the projections of all its mixers as one
+        product each (and, for steps of single tokens, through the skinny kernels).  None: the mixer is
+        only ever run through ``forward``."""
+        return None
+
 
 class FeedForward(Part):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
+
+    def gated_projections(self):
+        """A feed-forward that is down(SiLU(gate(x)) * up(x)) may hand out ``(gate_up Linear, down Linear,
+        tile)``: gate and up rows of the first interleaved in tiles of ``tile`` rows.  None: it is only
+        ever run through ``forward``."""
+        return None

@@ -6,6 +6,17 @@ from typing import Dict
 from .base import BuildContext, Residual, part_class
 
 _ARRANGEMENTS: Dict[str, type] = {}
+_FUSIONS: Dict[str, object] = {}
+
+
+def register_fusion(arrangement: str):
+    """Register ``factory(block, build) -> fusion or None`` for layers of ``arrangement``: a fusion runs the
+    whole layer through fewer launches where its parts and sizes allow
+    (``forward(residual, step, caches) -> bool``: True when it ran the layer)."""
+    def decorate(factory):
+        _FUSIONS[arrangement] = factory
+        return factory
+    return decorate
 
 
 def register_arrangement(name: str):
@@ -64,8 +75,8 @@ class ParallelPreNormBlock:
         self.ffn_norm = part_class(layer.ffn_norm)(
             layer.ffn_norm, f"{layer.prefix}.{layer.ffn_norm_name}", tensors, build)
         self.ffn = part_class(layer.ffn)(layer.ffn, f"{layer.prefix}.{layer.ffn_name}", tensors, build)
-        from .fused import ParallelFusion
-        self.fusion = ParallelFusion.build(self, build)      # None when the parts or sizes do not fit
+        factory = _FUSIONS.get(layer.arrangement)
+        self.fusion = factory(self, build) if factory is not None else None      # None when parts or sizes do not fit
 
     @property
     def graph_safe(self) -> bool:

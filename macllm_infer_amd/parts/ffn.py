@@ -48,6 +48,9 @@ class SwiGLU(FeedForward):
             if self.gate_up.bias is not None:
                 self.gate_up.bias = self.gate_up.bias[order].contiguous()
 
+    def gated_projections(self):
+        return self.gate_up, self.down, self.tile
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         gate_up = self.gate_up(x)
         activated = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=gate_up.dtype, device=x.device)

@@ -1,27 +1,35 @@
-"""The fast paths of a layer made of RMSNorm, attention, Mamba2 and SwiGLU.  The two mixers read
-the same normed rows and their outputs are added, so their input projections are one matrix
-[q|k|v|z|x B C|dt] and their output projections one matrix [Wo | W_out] along the inputs; the
-parts' own matrices are views of these.
+"""The fast paths of a layer whose mixers read the same normed rows and add their outputs (the
+``parallel_prenorm`` arrangement, with one mixer or several).  A mixer that hands out its pieces
+(``Mixer.projections``: input projection, what lies between, output projection) lets the layer run the
+input projections of all its mixers as one matrix [mixer 0 | mixer 1 | ...] and their output projections
+as one matrix along the inputs; the parts' own matrices are views of these.  Nothing here names a model:
+any registered mixer that offers ``projections`` and ``mix`` takes part, and so does a feed-forward that
+offers ``gated_projections`` and a norm that offers ``rms_prologue``; parts that do not run through their
+own ``forward``.
 
-Any step in bfloat16 (prompt portions, mixed batches): norm, one input GEMM, the two mixers on
-column views of its output, one output GEMM, norm, feed-forward: two library GEMMs fewer than
-part by part.
+Any step in bfloat16 (prompt portions, mixed batches): norm, one input GEMM, the mixers on column views
+of its output, one output GEMM, norm, feed-forward: for two mixers, two library GEMMs fewer than part by
+part.
 
-Decode steps (every lane holds one token, at most 64 rows): five launches instead of fifteen
-(seven for batches of more than 16 rows, whose two norms run as kernels of their own)
+Decode steps (every lane holds one token, at most 64 rows) go through the skinny kernels:
 
-    1. residual add + norm + [q|k|v|z|x B C|dt] projection + conv step        (fused_gemm)
-    2. attention (rotation, cache write, split context) and SSM step           (mixer_decode)
-    3. [attention | ssm] . [Wo | W_out]^T                                       (fused_gemm)
+    1. residual add + norm + input projection of every mixer                    (fused_gemm)
+    2. the mixers, each through its ``mix``, or all of them in one launch where a kernel for that
+       set of mixers is registered (``register_mixer_kernel``)
+    3. [mixer outputs] . [output projections]^T                                 (fused_gemm)
     4. residual add + norm + gate/up projection + SiLU(g)*u                     (fused_gemm)
     5. down projection                                                          (fused_gemm)
+
+For attention beside Mamba2 such a kernel is registered below: the conv step runs in the epilogue of
+launch 1 and both mixers in one launch 2 (``mixer_decode``), five launches a layer instead of fifteen
+(seven for batches of more than 16 rows, whose two norms run as kernels of their own).
 
 A large weight goes through the BLAS library instead where that is faster (``LIBRARY_MIN_WEIGHT``); the
 conv step and SiLU(g)*u then run as kernels of their own.
 
-The fusion belongs to the arrangement, which knows its parts; the parts stay as they are.  It
-is built only for bfloat16 weights and sizes the kernels cover; otherwise the block runs part
-by part.
+The fusion belongs to the arrangement (``register_fusion``), which knows its parts; the parts stay as they
+are.  It is built only for bfloat16 weights and sizes the kernels cover; otherwise the block runs part by
+part.
 """
 from __future__ import annotations
 
@@ -30,11 +38,8 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .attention import Attention
 from .base import Residual
-from .ffn import SwiGLU
-from .mamba2 import Mamba2
-from .norm import RmsNorm
+from .block import register_fusion
 from .position import NoPosition, Rope
 
 MAX_ROWS = 64          # rows of a step the skinny kernels take
@@ -213,52 +218,57 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
     return _graph_microseconds(library) < LIBRARY_MARGIN * times[tiles], tiles
 
 
-class ParallelFusion:
+_MIXER_KERNELS: Dict[tuple, object] = {}
+
+
+def register_mixer_kernel(*kinds: str):
+    """Register ``factory(fusion) -> kernel or None`` for layers whose mixers are of exactly these kinds, in
+    this order: a kernel that runs all of them in one launch in steps of single tokens.  The kernel object
+    offers ``conv`` (None, or the columns of the input projection that go through a conv step in that
+    product's epilogue: {lo, hi, taps, weight, bias}), ``supported(step, caches)``,
+    ``conv_state(caches)`` and ``run(u, step, caches, mixed)``."""
+    def decorate(factory):
+        _MIXER_KERNELS[tuple(kinds)] = factory
+        return factory
+    return decorate
+
+
+@register_fusion("parallel_prenorm")
+def build_layer_fusion(block, build) -> Optional["LayerFusion"]:
+    return LayerFusion.build(block, build)
+
+
+class LayerFusion:
     @staticmethod
-    def build(block, build) -> Optional["ParallelFusion"]:
+    def build(block, build) -> Optional["LayerFusion"]:
         if build.dtype != torch.bfloat16 or build.device.type != "cuda":
             return None
-        mixers = dict(block.mixers)
-        if len(mixers) != 2:
+        pieces = [mixer.projections() if hasattr(mixer, "projections") else None for _, mixer in block.mixers]
+        if not pieces or any(piece is None for piece in pieces):
             return None
-        attention = next((m for m in mixers.values() if type(m) is Attention), None)
-        mamba = next((m for m in mixers.values() if type(m) is Mamba2), None)
-        if attention is None or mamba is None or type(block.ffn) is not SwiGLU:
-            return None
-        if type(block.mixer_norm) is not RmsNorm or type(block.ffn_norm) is not RmsNorm:
-            return None
-        if type(attention.position) not in (Rope, NoPosition):
-            return None
-        linears = [attention.qkv, attention.out, mamba.in_proj, mamba.out_proj, block.ffn.gate_up, block.ffn.down]
+        linears = [linear for piece in pieces for linear in piece[:2]]
         if any(linear.weight.dtype != torch.bfloat16 for linear in linears):
             return None
-        a, s = attention.spec, mamba.spec
-        hidden = build.hidden_size
-        inner = block.ffn.spec.intermediate_size
-        mixed_width = a.num_heads * a.head_dim + s.inner_size
-        if a.head_dim not in (64, 128) or a.num_heads // a.num_kv_heads > 8 or s.state_size > 512:
-            return None
-        if block.ffn.tile != 8 or hidden % 32 != 0 or mixed_width % 32 != 0 or inner % 32 != 0:
-            return None
-        if not (ops.fused_gemm_supported(False, 1, hidden) and ops.fused_gemm_supported(False, 1, mixed_width)
-                and ops.fused_gemm_supported(False, 1, inner)):
-            return None
-        return ParallelFusion(block, attention, mamba, build)
+        fusion = LayerFusion(block, pieces, build)
+        return fusion if fusion.general or fusion.decode_ok else None
 
-    def __init__(self, block, attention: Attention, mamba: Mamba2, build):
+    def __init__(self, block, pieces, build):
         self.block = block
-        self.attention = attention
-        self.mamba = mamba
-        self.attention_name = next(name for name, mixer in block.mixers if mixer is attention)
-        self.mamba_name = next(name for name, mixer in block.mixers if mixer is mamba)
         device = build.device
-        a, s = attention.spec, mamba.spec
         self.hidden = build.hidden_size
-        q_width, kv_width = a.num_heads * a.head_dim, a.num_kv_heads * a.head_dim
-        E, C = s.inner_size, s.conv_width
-        # 1: [q | k | v | z | x B C | dt]
-        self.w_in = torch.cat([attention.qkv.weight, mamba.in_proj.weight], dim=0).contiguous()
-        self.b_in = _cat_bias([attention.qkv, mamba.in_proj], device)
+        self.names = [name for name, _ in block.mixers]
+        self.mixers = [mixer for _, mixer in block.mixers]
+        in_linears, out_linears = [piece[0] for piece in pieces], [piece[1] for piece in pieces]
+        # columns of each mixer in the input projection's output and in the rows the output projection reads
+        self.in_cols, self.mixed_cols, first_in, first_mixed = [], [], 0, 0
+        for in_linear, _, width in pieces:
+            self.in_cols.append((first_in, first_in + in_linear.out_features))
+            self.mixed_cols.append((first_mixed, first_mixed + width))
+            first_in += in_linear.out_features
+            first_mixed += width
+        # 1: [mixer 0 | mixer 1 | ...]
+        self.w_in = torch.cat([linear.weight for linear in in_linears], dim=0).contiguous()
+        self.b_in = _cat_bias(in_linears, device)
         # prompt portions may multiply with rows of zeros added (the decode kernels take the rows that count)
         self.w_in_wide, self.b_in_wide = self.w_in, self.b_in
         if _padding_pays(self.w_in):
@@ -267,69 +277,81 @@ class ParallelFusion:
             self.w_in = self.w_in_wide[:self.w_in.shape[0]]
             if self.b_in is not None:
                 self.b_in_wide = torch.cat([self.b_in, self.b_in.new_zeros(extra)])
-        self.q_col, self.k_col, self.v_col = 0, q_width, q_width + kv_width
-        self.z_col = q_width + 2 * kv_width
-        self.x_col = self.z_col + E
-        self.dt_col = self.x_col + C
         self.in_width = self.w_in.shape[0]
         self.in_ld = -(-self.in_width // 8) * 8
-        self.qkv_width = q_width + 2 * kv_width
-        attention.qkv.weight = self.w_in[:self.qkv_width]             # the parts' matrices: views of the fused ones
-        mamba.in_proj.weight = self.w_in[self.qkv_width:]
-        # 3: [attention | ssm] . [Wo | W_out]^T
-        self.w_out = torch.cat([attention.out.weight, mamba.out_proj.weight], dim=1).contiguous()
-        biases = [linear.bias for linear in (attention.out, mamba.out_proj) if linear.bias is not None]
+        # 3: [mixer outputs] . [output projections]^T
+        self.w_out = torch.cat([linear.weight for linear in out_linears], dim=1).contiguous()
+        biases = [linear.bias for linear in out_linears if linear.bias is not None]
         self.b_out = sum(biases[1:], biases[0]).contiguous() if biases else None
-        self.mixed_width = q_width + E
-        self.q_width = q_width
-        attention.out.weight = self.w_out[:, :q_width]
-        mamba.out_proj.weight = self.w_out[:, q_width:]
+        self.mixed_width = first_mixed
+        for in_linear, out_linear, (lo, hi), (mixed_lo, mixed_hi) in zip(in_linears, out_linears, self.in_cols,
+                                                                         self.mixed_cols):
+            in_linear.weight = self.w_in[lo:hi]                       # the parts' matrices: views of the fused ones
+            out_linear.weight = self.w_out[:, mixed_lo:mixed_hi]
         # the column views the mixers get must start at 16 bytes and rows must be multiples of 8 elements
-        self.general = (self.in_width % 8 == 0 and self.qkv_width % 8 == 0 and q_width % 8 == 0
-                        and self.mixed_width % 8 == 0)
-        # 4: gate and up rows interleaved in tiles of 8: the feed-forward part stores them so
-        ffn = block.ffn
-        inner = ffn.spec.intermediate_size
-        self.w_gate_up = ffn.gate_up.weight
-        self.b_gate_up = ffn.gate_up.bias
-        self.inner = inner
-        self.position = attention.position
-        # a wide model's normed rows do not fit the norm prologue's LDS: its norms then run as kernels of their own
-        self.norm_fits = ops.fused_gemm_supported(True, 1, self.hidden)
+        self.aligned = self.mixed_width % 8 == 0 and all(lo % 8 == 0 for lo, _ in self.in_cols + self.mixed_cols)
+        self.general = self.aligned and self.in_width % 8 == 0
+        # 4 and 5: a gated feed-forward whose gate and up rows are interleaved in tiles of 8 (the part stores them
+        # so) runs through the skinny kernels as well; any other runs through its own forward
+        gated = block.ffn.gated_projections() if hasattr(block.ffn, "gated_projections") else None
+        self.gate_up, self.down, self.inner = None, None, 0
+        if gated is not None and gated[2] == 8 and gated[0].weight.dtype == torch.bfloat16 \
+                and gated[1].weight.dtype == torch.bfloat16 and gated[1].in_features % 32 == 0:
+            self.gate_up, self.down, _ = gated
+            self.inner = self.down.in_features
+        # the skinny kernels take K in chunks of 32
+        self.decode_ok = (self.hidden % 32 == 0 and self.mixed_width % 32 == 0
+                          and ops.fused_gemm_supported(False, 1, self.hidden)
+                          and ops.fused_gemm_supported(False, 1, self.mixed_width)
+                          and (self.gate_up is None or ops.fused_gemm_supported(False, 1, self.inner)))
+        # norms that the skinny kernel computes in its prologue (a wide model's rows do not fit its LDS, and another
+        # kind of norm is not what it computes: those run as kernels of their own)
+        fits = self.decode_ok and ops.fused_gemm_supported(True, 1, self.hidden)
+        self.mixer_rms = _rms_prologue(block.mixer_norm) if fits else None
+        self.ffn_rms = _rms_prologue(block.ffn_norm) if fits else None
+        self.norm_fits = self.mixer_rms is not None and self.ffn_rms is not None
+        # a kernel for this set of mixers, if one is registered and takes these sizes
+        factory = _MIXER_KERNELS.get(tuple(getattr(mixer, "kind", None) for mixer in self.mixers))
+        self.kernel = factory(self) if factory is not None and self.decode_ok else None
+        if self.kernel is None and not self.aligned:          # no view of its columns for a mixer's own ``mix``
+            self.decode_ok = False
+        conv = self.kernel.conv if self.kernel is not None else None
         # which projections go through the library, by step size
-        conv = dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=mamba.conv_weight, bias=mamba.conv_bias)
         # (and how many tiles of 16 output features a workgroup of the skinny kernel owns where it is taken)
-        self.library_in, self.tiles_in = self._tune(self.w_in, self.b_in, ops.EPI_CONV, conv)
+        self.library_in, self.tiles_in = self._tune(self.w_in, self.b_in, ops.EPI_CONV if conv else ops.EPI_PLAIN, conv,
+                                                    self.mixer_rms is not None)
         self.library_out, self.tiles_out = self._tune(self.w_out, self.b_out, ops.EPI_PLAIN)
-        self.library_gate_up, self.tiles_gate_up = self._tune(self.w_gate_up, self.b_gate_up, ops.EPI_SWIGLU)
-        self.library_down, self.tiles_down = self._tune(ffn.down.weight, ffn.down.bias, ops.EPI_PLAIN)
         # and which of the two that feed the residual stream are split over K instead (steps of more than 16 rows)
         self.split_out, self.tiles_out = self._tune_split(self.w_out, self.b_out, self.library_out, self.tiles_out)
-        self.split_down, self.tiles_down = self._tune_split(ffn.down.weight, ffn.down.bias, self.library_down,
-                                                            self.tiles_down)
         # what the skinny kernel reads: a second copy of each matrix in the order of its waves' fragments (one run
         # of 1 KiB a load instead of 64 bytes of each of 16 rows: 15 to 25 % faster); the row-major ones stay for
         # the library and for prompt portions.  A projection that always goes through the library has none.
 
         def fragments(weight, library, split):
-            return None if all(library) and not any(split) else ops.fragment_order(weight)
+            if not self.decode_ok or (all(library) and not any(split)):
+                return None
+            return ops.fragment_order(weight)
 
         self.f_in = fragments(self.w_in, self.library_in, ())
         self.f_out = fragments(self.w_out, self.library_out, self.split_out)
-        self.f_gate_up = fragments(self.w_gate_up, self.library_gate_up, ())
-        self.f_down = fragments(ffn.down.weight, self.library_down, self.split_down)
+        if self.gate_up is not None:
+            self.library_gate_up, self.tiles_gate_up = self._tune(self.gate_up.weight, self.gate_up.bias, ops.EPI_SWIGLU,
+                                                                  None, self.ffn_rms is not None)
+            self.library_down, self.tiles_down = self._tune(self.down.weight, self.down.bias, ops.EPI_PLAIN)
+            self.split_down, self.tiles_down = self._tune_split(self.down.weight, self.down.bias, self.library_down,
+                                                                self.tiles_down)
+            self.f_gate_up = fragments(self.gate_up.weight, self.library_gate_up, ())
+            self.f_down = fragments(self.down.weight, self.library_down, self.split_down)
 
-    def decode_supported(self, step, cache) -> bool:
-        a = self.attention.spec
-        rotary = self.position.rotary_dim if isinstance(self.position, Rope) else 0
-        return (step.max_query_len == 1 and step.num_tokens <= MAX_ROWS and cache.owns_kv
-                and ops.mixer_decode_supported(a.num_heads, a.num_kv_heads, a.head_dim, cache.k_cache.shape[2],
-                                               self.mamba.spec.state_size, step.max_seq_len, a.window, rotary))
+    def decode_supported(self, step, caches) -> bool:
+        if step.max_query_len != 1 or step.num_tokens > MAX_ROWS or not self.decode_ok:
+            return False
+        return self.aligned or self.kernel.supported(step, caches)
 
     def forward(self, residual: Residual, step, caches) -> bool:
         """Runs the layer and returns True, or returns False with nothing done (the block then
         runs part by part)."""
-        if self.decode_supported(step, caches[self.attention_name]):
+        if self.decode_supported(step, caches):
             self.forward_decode(residual, step, caches)
             return True
         if self.general:
@@ -337,37 +359,46 @@ class ParallelFusion:
             return True
         return False
 
+    def _mix_each(self, u: torch.Tensor, step, caches, mixed: torch.Tensor, order=None) -> None:
+        for index in (range(len(self.mixers)) if order is None else order):
+            (lo, hi), (mixed_lo, mixed_hi) = self.in_cols[index], self.mixed_cols[index]
+            self.mixers[index].mix(u[:, lo:hi], step, caches[self.names[index]], mixed[:, mixed_lo:mixed_hi])
+
     def forward_general(self, residual: Residual, step, caches) -> None:
         block = self.block
         normed = block.mixer_norm.forward(residual)
         u = ops.linear(normed, self.w_in_wide, self.b_in_wide)
         mixed = torch.empty((u.shape[0], self.mixed_width), dtype=u.dtype, device=u.device)
-        if u.shape[0] >= OVERLAP_MIN_TOKENS and torch.cuda.is_current_stream_capturing():
-            # the two mixers read the same rows and write different columns: attention runs on a second
-            # stream beside the state-space chain, whose kernels are many and small (in a captured graph
-            # only: launched one by one the step waits for the host, which the second stream costs more).
-            # The chain is recorded first: the graph keeps the branch it meets first on the queue of the
-            # projections before and after it, and the other branch pays the hops between queues
+        if (len(self.mixers) == 2 and u.shape[0] >= OVERLAP_MIN_TOKENS and torch.cuda.is_current_stream_capturing()
+                and all(getattr(mixer, "graph_safe", False) for mixer in self.mixers)):
+            # two mixers read the same rows and write different columns: the first runs on a second stream
+            # beside the second (in a captured graph only: launched one by one the step waits for the host,
+            # which the second stream costs more).  The mixer on the main stream is recorded first: the graph
+            # keeps the branch it meets first on the queue of the projections before and after it, and the
+            # other branch pays the hops between queues.  (Attention beside a state-space mixer, whose kernels
+            # are many and small: the state-space chain is the longer one and stays on the main queue.)
             main = torch.cuda.current_stream(u.device)
             side = _side_stream(u.device)
             side.wait_stream(main)
-            self.mamba.mix(u[:, self.qkv_width:self.in_width], step, caches[self.mamba_name], mixed[:, self.q_width:])
+            self._mix_each(u, step, caches, mixed, order=(1,))
             with torch.cuda.stream(side):
-                self.attention.mix(u[:, :self.qkv_width], step, caches[self.attention_name], mixed[:, :self.q_width])
+                self._mix_each(u, step, caches, mixed, order=(0,))
             main.wait_stream(side)
         else:
-            self.attention.mix(u[:, :self.qkv_width], step, caches[self.attention_name], mixed[:, :self.q_width])
-            self.mamba.mix(u[:, self.qkv_width:self.in_width], step, caches[self.mamba_name], mixed[:, self.q_width:])
+            self._mix_each(u, step, caches, mixed)
         residual.pending = [ops.linear(mixed, self.w_out, self.b_out)]
         normed = block.ffn_norm.forward(residual)
         residual.pending = [block.ffn.forward(normed)]
 
-    def _tune(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict] = None) -> tuple:
+    def _tune(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict] = None,
+              normed: bool = False) -> tuple:
         """For step sizes of up to 16, 32 and 64 rows: whether this projection goes through the library, and
-        the feature tiles of the skinny kernel.  (Where the norm runs in the skinny kernel's prologue, small
-        steps stay with it.)"""
+        the feature tiles of the skinny kernel.  (``normed``: the norm before it runs in the skinny kernel's
+        prologue; small steps then stay with it.)"""
+        if not self.decode_ok:
+            return (True, True, True), (1, 1, 1)
         choices, tiles = self._tune_all(weight, bias, epilogue, conv)
-        if epilogue != ops.EPI_PLAIN and self.norm_fits:
+        if normed:
             choices = (False,) + choices[1:]
         return choices, tiles
 
@@ -402,79 +433,73 @@ class ParallelFusion:
         for bucket, rows in enumerate(TUNE_ROWS):
             key = (tuple(weight.shape), epilogue, bias is None, bucket)
             if key not in _library_wins:
-                _library_wins[key] = _measure_library(weight, bias, rows, epilogue, self.block.ffn.tile, conv)
+                _library_wins[key] = _measure_library(weight, bias, rows, epilogue, 8, conv)
             choices.append(_library_wins[key][0])
             tiles.append(_library_wins[key][1] if FORCE_TILES is None or bucket == 0 else FORCE_TILES)
         return tuple(choices), tuple(tiles)
 
     def forward_decode(self, residual: Residual, step, caches) -> None:
-        block, a, s = self.block, self.attention.spec, self.mamba.spec
-        kv, state = caches[self.attention_name], caches[self.mamba_name]
+        block = self.block
         M = step.num_tokens
         bucket = _bucket(M)
         device = residual.h.device
         bf16 = torch.bfloat16
+        kernel = self.kernel if self.kernel is not None and self.kernel.supported(step, caches) else None
 
-        def norm_prologue(norm):
+        def norm_prologue(norm, rms):
             """The input of a projection: the norm in the kernel's prologue, or its own kernel before."""
-            if M > MAX_NORM_ROWS or not self.norm_fits:
+            if M > MAX_NORM_ROWS or rms is None:
                 return dict(x=norm.forward(residual)), None          # adds the pending deltas in place
             pending = residual.pending
+            if len(pending) > 2 or any(delta.dtype != bf16 for delta in pending):
+                return dict(x=norm.forward(residual)), None
             h_out = torch.empty_like(residual.h) if pending else None
-            arguments = dict(h_in=residual.h, deltas=pending, h_out=h_out, norm_weight=norm.weight, eps=norm.eps)
+            arguments = dict(h_in=residual.h, deltas=pending, h_out=h_out, norm_weight=rms[0], eps=rms[1])
             return arguments, h_out
 
         # 1
+        conv = None
+        if kernel is not None and kernel.conv is not None:
+            conv = dict(kernel.conv, state=kernel.conv_state(caches), slot_ids=step.slot_ids)
         if self.library_in[bucket]:
             u = ops.linear(block.mixer_norm.forward(residual), self.w_in, self.b_in)
-            ops.conv_step(u, self.x_col, self.dt_col - self.x_col, self.mamba.conv_weight, self.mamba.conv_bias,
-                          state.states["conv"], step.slot_ids)
+            if conv is not None:
+                ops.conv_step(u, conv["lo"], conv["hi"] - conv["lo"], conv["weight"], conv["bias"], conv["state"],
+                              conv["slot_ids"])
         else:
             u = torch.empty((M, self.in_ld), dtype=bf16, device=device)
-            arguments, h_out = norm_prologue(block.mixer_norm)
-            ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=ops.EPI_CONV,
-                           conv=dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=self.mamba.conv_weight,
-                                     bias=self.mamba.conv_bias, state=state.states["conv"], slot_ids=step.slot_ids),
+            arguments, h_out = norm_prologue(block.mixer_norm, self.mixer_rms)
+            ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width],
+                           epilogue=ops.EPI_CONV if conv is not None else ops.EPI_PLAIN, conv=conv,
                            feature_tiles=self.tiles_in[bucket] if "x" in arguments else 1, fragments=self.f_in,
                            **arguments)
             if h_out is not None:
                 residual.h, residual.pending = h_out, []
         # 2
         mixed = torch.empty((M, self.mixed_width), dtype=bf16, device=device)
-        gated_norm = self.mamba.norm_weight is not None
-        y = torch.empty((M, s.inner_size), dtype=torch.float32, device=device) if gated_norm else None
-        rope = isinstance(self.position, Rope)
-        ops.mixer_decode(
-            u, num_heads=a.num_heads, num_kv_heads=a.num_kv_heads, head_dim=a.head_dim, q_col=self.q_col,
-            k_col=self.k_col, v_col=self.v_col, inv_freq=self.position.inv_freq if rope else None,
-            rotary_dim=self.position.rotary_dim if rope else 0, k_cache=kv.k_cache, v_cache=kv.v_cache,
-            block_tables=step.block_tables[kv.group], positions=step.positions,
-            slot_mapping=step.slot_mappings[kv.group], scale=a.scale, window=a.window, max_seq_len=step.max_seq_len,
-            ssm_heads=s.num_heads, ssm_head_dim=s.head_dim, state_size=s.state_size,
-            num_groups=s.num_groups, z_col=self.z_col, x_col=self.x_col, dt_col=self.dt_col,
-            dt_bias=self.mamba.dt_bias, A=self.mamba.A, D=self.mamba.D, ssm_state=state.states["ssm"],
-            slot_ids=step.slot_ids, out=mixed, ssm_y=y)
-        if gated_norm:
-            ops.gate_norm(y, u[:, self.z_col:self.z_col + s.inner_size], self.mamba.norm_weight, s.num_groups,
-                          s.norm_eps, mixed[:, a.num_heads * a.head_dim:])
+        if kernel is not None:
+            kernel.run(u, step, caches, mixed)
+        else:
+            self._mix_each(u, step, caches, mixed)
         # 3
         residual.pending = self._to_the_stream(mixed, self.w_out, self.b_out, self.library_out[bucket],
                                                self.split_out[bucket], self.tiles_out[bucket], self.f_out)
         # 4
+        if self.gate_up is None:
+            residual.pending = [block.ffn.forward(block.ffn_norm.forward(residual))]
+            return
         activated = torch.empty((M, self.inner), dtype=bf16, device=device)
         if self.library_gate_up[bucket]:
-            ops.swiglu(ops.linear(block.ffn_norm.forward(residual), self.w_gate_up, self.b_gate_up), activated,
-                       block.ffn.tile)
+            ops.swiglu(ops.linear(block.ffn_norm.forward(residual), self.gate_up.weight, self.gate_up.bias), activated, 8)
         else:
-            arguments, h_out = norm_prologue(block.ffn_norm)
-            ops.fused_gemm(self.w_gate_up, self.b_gate_up, activated, epilogue=ops.EPI_SWIGLU,
+            arguments, h_out = norm_prologue(block.ffn_norm, self.ffn_rms)
+            ops.fused_gemm(self.gate_up.weight, self.gate_up.bias, activated, epilogue=ops.EPI_SWIGLU,
                            feature_tiles=self.tiles_gate_up[bucket] if "x" in arguments else 1,
                            fragments=self.f_gate_up, **arguments)
             if h_out is not None:
                 residual.h, residual.pending = h_out, []
         # 5
-        down = block.ffn.down
-        residual.pending = self._to_the_stream(activated, down.weight, down.bias, self.library_down[bucket],
+        residual.pending = self._to_the_stream(activated, self.down.weight, self.down.bias, self.library_down[bucket],
                                                self.split_down[bucket], self.tiles_down[bucket], self.f_down)
 
     def _to_the_stream(self, x: torch.Tensor, weight: torch.Tensor, bias, library: bool, slabs: int, tiles: int,
@@ -491,6 +516,75 @@ class ParallelFusion:
         delta = torch.empty((M, self.hidden), dtype=torch.bfloat16, device=x.device)
         ops.fused_gemm(weight, bias, delta, x=x, feature_tiles=tiles, fragments=fragments)
         return [delta]
+
+
+def _rms_prologue(norm):
+    prologue = getattr(norm, "rms_prologue", None)
+    return prologue() if prologue is not None else None
+
+
+@register_mixer_kernel("attention", "mamba2")
+def attention_mamba2_step(fusion: "LayerFusion") -> Optional["AttentionMamba2Step"]:
+    attention, mamba = fusion.mixers
+    a, s = attention.spec, mamba.spec
+    if type(attention.position) not in (Rope, NoPosition):
+        return None
+    if a.head_dim not in (64, 128) or a.num_heads // a.num_kv_heads > 8 or s.state_size > 512:
+        return None
+    return AttentionMamba2Step(fusion)
+
+
+class AttentionMamba2Step:
+    """Attention beside Mamba2 in steps of single tokens: the conv step of the state-space columns runs in the
+    epilogue of the input product, and one launch (``mixer_decode``) rotates q and the new key, writes the new
+    key and value into their cache cell, attends over the request's pages in runs that a small kernel merges,
+    and advances the state-space state by one step with the gate on the way out."""
+
+    def __init__(self, fusion: "LayerFusion"):
+        self.attention, self.mamba = fusion.mixers
+        self.attention_name, self.mamba_name = fusion.names
+        a, s = self.attention.spec, self.mamba.spec
+        q_width, kv_width = a.num_heads * a.head_dim, a.num_kv_heads * a.head_dim
+        first, second = fusion.in_cols[0][0], fusion.in_cols[1][0]
+        self.q_col, self.k_col, self.v_col = first, first + q_width, first + q_width + kv_width
+        self.z_col = second
+        self.x_col = second + s.inner_size
+        self.dt_col = self.x_col + s.conv_width
+        self.attended_width = q_width
+        self.position = self.attention.position
+        self.conv = dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=self.mamba.conv_weight,
+                         bias=self.mamba.conv_bias)
+
+    def conv_state(self, caches) -> torch.Tensor:
+        return caches[self.mamba_name].states["conv"]
+
+    def supported(self, step, caches) -> bool:
+        a = self.attention.spec
+        cache = caches[self.attention_name]
+        rotary = self.position.rotary_dim if isinstance(self.position, Rope) else 0
+        return (cache.owns_kv
+                and ops.mixer_decode_supported(a.num_heads, a.num_kv_heads, a.head_dim, cache.k_cache.shape[2],
+                                               self.mamba.spec.state_size, step.max_seq_len, a.window, rotary))
+
+    def run(self, u: torch.Tensor, step, caches, mixed: torch.Tensor) -> None:
+        a, s = self.attention.spec, self.mamba.spec
+        kv, state = caches[self.attention_name], caches[self.mamba_name]
+        gated_norm = self.mamba.norm_weight is not None
+        y = torch.empty((u.shape[0], s.inner_size), dtype=torch.float32, device=u.device) if gated_norm else None
+        rope = isinstance(self.position, Rope)
+        ops.mixer_decode(
+            u, num_heads=a.num_heads, num_kv_heads=a.num_kv_heads, head_dim=a.head_dim, q_col=self.q_col,
+            k_col=self.k_col, v_col=self.v_col, inv_freq=self.position.inv_freq if rope else None,
+            rotary_dim=self.position.rotary_dim if rope else 0, k_cache=kv.k_cache, v_cache=kv.v_cache,
+            block_tables=step.block_tables[kv.group], positions=step.positions,
+            slot_mapping=step.slot_mappings[kv.group], scale=a.scale, window=a.window, max_seq_len=step.max_seq_len,
+            ssm_heads=s.num_heads, ssm_head_dim=s.head_dim, state_size=s.state_size,
+            num_groups=s.num_groups, z_col=self.z_col, x_col=self.x_col, dt_col=self.dt_col,
+            dt_bias=self.mamba.dt_bias, A=self.mamba.A, D=self.mamba.D, ssm_state=state.states["ssm"],
+            slot_ids=step.slot_ids, out=mixed, ssm_y=y)
+        if gated_norm:
+            ops.gate_norm(y, u[:, self.z_col:self.z_col + s.inner_size], self.mamba.norm_weight, s.num_groups,
+                          s.norm_eps, mixed[:, self.attended_width:])
 
 
 def _cat_bias(linears, device):

@@ -97,6 +97,9 @@ class Mamba2(Mixer):
             step.derived[key] = ops.SsdChunks(step.lane_lengths, self.spec.chunk_size, step.token_ids.device)
         return step.derived[key]
 
+    def projections(self):
+        return self.in_proj, self.out_proj, self.spec.inner_size
+
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         u = self.in_proj(x)                                               # [T, E + C + H]
         gated = torch.empty((x.shape[0], self.spec.inner_size), dtype=u.dtype, device=u.device)

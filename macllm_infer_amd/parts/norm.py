@@ -46,6 +46,9 @@ class RmsNorm(Part):
         self.build = build
         self.weight = tensors[f"{prefix}.weight"].to(torch.float32).contiguous().to(build.device)
 
+    def rms_prologue(self):
+        return self.weight, self.eps
+
     def forward(self, residual: Residual, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Add the pending branch outputs to the residual stream and return its normed rows
         (all of them, or only ``rows``; with ``rows`` the stream itself is left unchanged)."""

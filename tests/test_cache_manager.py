@@ -42,13 +42,41 @@ def test_page_pool_invariants():
 def test_groups_share_a_table_per_geometry_and_windows_get_their_own():
     cache = make(window=10)
     assert len(cache.groups) == 2
-    assert cache.groups[0].storage.shape == (9, 2, 2, 2, 32)      # [page (+1 scratch), layer, K|V, kv head, token x dim]
+    assert cache.groups[0].storage.shape == (9, 2, 128)           # [page (+1 scratch), layer, K then V of 2 heads x 8 x 4]
     assert first_views(cache) == ((9, 2, 8, 4), (9, 2, 4, 8))     # V pages are transposed
+    keys, values = cache.entry((0, "attn")).k_cache, cache.entry((0, "attn")).v_cache
+    assert keys.stride() == (256, 32, 4, 1) and values.stride() == (256, 32, 8, 1)
+    assert values.data_ptr() - keys.data_ptr() == 64 * 4          # a layer's values follow its keys inside the page
     assert cache.groups[1].need.window == 10 and len(cache.groups[1].members) == 1
     first, second = cache.entry((0, "attn")), cache.entry((1, "attn"))
     assert first.group == second.group == 0 and first.k_cache.data_ptr() != second.k_cache.data_ptr()
     assert cache.entry((1, "rec")).states["s"].shape == (4, 3, 2)      # 3 slots + the scratch slot
     assert cache.entry((1, "rec")).states["c"].dtype == torch.float32
+
+
+def test_keys_and_values_of_different_widths_and_states_of_any_dtype():
+    """A mixer whose values are wider than its keys (or narrower) gets pages that hold both, and views of the
+    right shapes; it shares a group only with layers of the same two widths.  A state can ask for any dtype."""
+    needs = {(0, "wide"): [KVNeed(2, 4, None, value_dim=12)], (1, "wide"): [KVNeed(2, 4, None, value_dim=12)],
+             (2, "plain"): [KVNeed(2, 4, None), StateNeed("count", (3,), torch.int32),
+                            StateNeed("half", (2, 2), torch.float16)]}
+    cache = CacheManager(needs, {}, 8, 64, 2, torch.bfloat16, "cpu")
+    assert len(cache.groups) == 2 and cache.groups[0].need.value_width == 12 and cache.groups[1].need.value_width == 4
+    assert cache.groups[0].storage.shape == (9, 2, 2 * 8 * 16) and cache.groups[1].storage.shape == (9, 1, 2 * 8 * 8)
+    entry = cache.entry((1, "wide"))
+    assert tuple(entry.k_cache.shape) == (9, 2, 8, 4) and tuple(entry.v_cache.shape) == (9, 2, 12, 8)
+    assert cache.groups[0].bytes_per_page(2) == 2 * 2 * 8 * 16 * 2
+    # the views of the two layers and of keys and values tile a page without overlap
+    marks = torch.zeros_like(cache.groups[0].storage)
+    for layer in range(2):
+        for view in cache.groups[0].layer_views(layer):
+            view += 1
+    marks = cache.groups[0].storage
+    assert bool((marks == 1).all())
+    states = cache.entry((2, "plain")).states
+    assert states["count"].dtype == torch.int32 and states["half"].dtype == torch.float16
+    with pytest.raises(ValueError, match="dtype"):
+        CacheManager({(0, "x"): [StateNeed("s", (1,), "int7")]}, {}, 8, 64, 2, torch.bfloat16, "cpu")
 
 
 def test_reservation_is_all_or_nothing():
@@ -182,6 +210,9 @@ def test_shared_kv_entries_read_the_owner():
                      {(1, "attn"): (0, "attn")}, 8, 32, 2, torch.float32, "cpu")
 
 
+TILE = 64
+
+
 def plain_packing(cache, lanes, pad_lengths, width):
     """The step's index arrays, lane by lane, from the manager's tables: what the core's packer
     has to write.  ``lanes``: (request, tokens, wanted places)."""
@@ -195,7 +226,7 @@ def plain_packing(cache, lanes, pad_lengths, width):
            "seq_lens": [start + length for start, length in zip(starts, lengths)],
            "slot_ids": [cache.requests[request].slot for request, _, _ in lanes] + [cache.scratch_slot] * len(pad_lengths),
            "want_rows": [first[index] + place for index, (_, _, want) in enumerate(lanes) for place in want],
-           "query_tiles": [[index, row] for index in range(len(lengths)) for row in range(first[index], first[index + 1], 64)],
+           "query_tiles": [[index, row] for index in range(len(lengths)) for row in range(first[index], first[index + 1], TILE)],
            "slot_mappings": [], "block_tables": []}
     for number, group in enumerate(cache.groups):
         size = group.page_size
@@ -235,12 +266,12 @@ def test_the_cores_packing_of_a_step_matches_a_plain_packing(seed, decode_only):
             got = [item.tolist() for item in got] if isinstance(got, list) else got.tolist()
             assert got == value, field
 
-    context = build_step_context(step_lanes, cache, "cpu")
+    context = build_step_context(step_lanes, cache, "cpu", query_tile=TILE)
     compare(context, plain_packing(cache, lanes, [], None))
     assert context.max_seq_len == max(cache.requests[name].length + len(tokens) for name, tokens, _ in lanes)
     assert context.lane_starts == [cache.requests[name].length for name, _, _ in lanes]
     if all(len(tokens) == 1 for _, tokens, _ in lanes):            # a captured decode step: padded, fixed width
-        static = StaticStep(cache, 4, 400, "cpu")
+        static = StaticStep(cache, 4, 400, "cpu", query_tile=TILE)
         compare(static.context, dict(plain_packing(cache, [], [1] * 4, static.max_pages), want_rows=[0, 1, 2, 3]))
         static.fill(lower_lanes(step_lanes, cache))
         compare(static.context, dict(plain_packing(cache, lanes, [1] * (4 - len(lanes)), static.max_pages),

@@ -55,7 +55,8 @@ class PartHarness:
             if request not in self.cache.requests:
                 self.cache.add_request(request)
         self.cache.reserve([(request, x.shape[0]) for request, x in lanes])
-        step = build_step_context([Lane(request, [0] * x.shape[0]) for request, x in lanes], self.cache, DEV)
+        step = build_step_context([Lane(request, [0] * x.shape[0]) for request, x in lanes], self.cache, DEV,
+                                  query_tile=getattr(self.part, "query_tile", 0))
         x = torch.cat([x for _, x in lanes]).to(self.build.dtype).to(DEV)
         out = self.part.forward(x, step, self.cache.entry((0, "p"))).float().cpu()
         pieces, cursor = [], 0
@@ -388,6 +389,57 @@ def test_graphs_come_in_buckets_of_context_length():
     assert set(with_graphs.graphs._graphs) == {(1, 2048), (1, 4096), (2, 4096)}
     both([Lane("short", [short[39]], [0])])                               # and back through the narrow one
     assert with_graphs.graphs.counts["decode_replays"] == 16
+
+
+def test_layers_of_one_mixer_and_a_mixer_from_outside_take_the_fast_paths(monkeypatch):
+    """The fast paths of a layer belong to no model: a layer with attention alone decodes through the skinny
+    kernels (norm in the prologue, SiLU(g)*u in the epilogue), and so do the projections of a toy mixer with
+    state of its own that is registered from the tests and hands out its pieces, between toy norms and before
+    a routed toy feed-forward, which run through their own ``forward``.  Nothing in the package is edited."""
+    import gates
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.kernels import ops
+    from macllm_infer_amd.weights.random_init import random_tensors
+    toy_parts.register_toys()
+    raw = {"architectures": ["ToyFastForTests"], "hidden": 64, "vocab": 150, "width": 96, "decay": 0.8}
+    config = toy_parts.ToyFastConfig(raw)
+    tensors = random_tensors(config, 9, torch.bfloat16, "unit")
+    engine = Engine(config=config, tensors=tensors, dtype="bfloat16", kv_cache_block_tokens=16,
+                    kv_cache_capacity_tokens=512, max_active_sequences=3)
+    first, second = engine.model.blocks[0].fusion, engine.model.blocks[1].fusion
+    assert first is not None and first.decode_ok and first.norm_fits and first.gate_up is not None and first.kernel is None
+    assert second is not None and second.decode_ok and second.mixer_rms is None and second.gate_up is None
+    assert second.in_width == 192 and second.mixed_width == 96
+    calls = {"skinny": 0, "library": 0}
+    real_skinny, real_library = ops.fused_gemm, ops.linear
+
+    def skinny(*arguments, **named):
+        calls["skinny"] += 1
+        return real_skinny(*arguments, **named)
+
+    def library(*arguments, **named):
+        calls["library"] += 1
+        return real_library(*arguments, **named)
+
+    monkeypatch.setattr(ops, "fused_gemm", skinny)
+    monkeypatch.setattr(ops, "linear", library)
+    sequences = {"a": tokens_for(150, 60, 21), "b": tokens_for(150, 45, 22)}
+    rows = {"a": [], "b": []}
+    for name in sequences:
+        engine.add_request(name)
+    out = engine.step([Lane("a", sequences["a"][:40], list(range(40))), Lane("b", sequences["b"][:30], list(range(30)))])
+    rows["a"].append(out[:40].cpu()), rows["b"].append(out[40:].cpu())
+    assert calls["skinny"] == 0 and calls["library"] > 0          # a prompt portion: the fused matrices, library products
+    calls.update(skinny=0, library=0)
+    for position in range(15):
+        out = engine.step([Lane("a", [sequences["a"][40 + position]], [0]), Lane("b", [sequences["b"][30 + position]], [0])])
+        rows["a"].append(out[:1].cpu()), rows["b"].append(out[1:].cpu())
+    # a decode step: input and output projections of both layers, gate/up and down of the first, and the head
+    assert calls["skinny"] == 15 * 7 and calls["library"] == 0
+    for name, tokens in sequences.items():
+        want = toy_parts.toy_fast_plain_logits(raw, tensors, tokens[:len(torch.cat(rows[name]))]).numpy()
+        assert gates.bfloat16_close(torch.cat(rows[name]).numpy(), want), name
+    engine.cache.check()
 
 
 def test_replays_that_follow_one_another_without_a_wait_keep_their_own_arrays(tmp_path):

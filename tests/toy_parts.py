@@ -54,6 +54,50 @@ class CentredNormSpec:
         assert self.eps > 0
 
 
+@dataclass(frozen=True)
+class GatedDecaySpec:
+    """A toy mixer with state of its own that hands out its pieces: [a | b] = x W_in; s_t = decay * s_{t-1} + a_t;
+    y_t = s_t * sigmoid(b_t); out = y W_out."""
+    width: int
+    decay: float
+    kind: str = "toy_gated_decay"
+
+    def validate(self):
+        assert 0 < self.decay < 1 and self.width > 0
+
+
+@dataclass
+class ToyFastConfig:
+    """A toy architecture of two one-mixer layers for the fast paths of a layer: layer 0 = attention alone
+    with the package's own norm and feed-forward; layer 1 = the gated decay mixer alone, between the centring
+    toy norms, with the routed toy feed-forward."""
+    raw: dict
+    architecture_names = ("ToyFastForTests",)
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw)
+
+    def to_dict(self):
+        return dict(self.raw)
+
+    def to_model_spec(self):
+        from macllm_infer_amd.config import (AttentionSpec, LayerSpec, MixerSlot, ModelSpec, RmsNormSpec, RopeSpec,
+                                             ScheduleEntry, SwiGLUSpec)
+        raw = self.raw
+        norm = RmsNormSpec(eps=1e-5)
+        attention = AttentionSpec(num_heads=2, num_kv_heads=1, head_dim=64, scale=0.125,
+                                  position=RopeSpec(theta=1e4, rotary_dim=64))
+        layers = (LayerSpec(prefix="model.layers.0", ffn=SwiGLUSpec(intermediate_size=64), mixer_norm=norm, ffn_norm=norm,
+                            mixers=(MixerSlot("self_attn", attention),)),
+                  LayerSpec(prefix="model.layers.1", ffn=RoutedSpec(3, 24), mixer_norm=CentredNormSpec(1e-4),
+                            ffn_norm=CentredNormSpec(1e-4),
+                            mixers=(MixerSlot("decay", GatedDecaySpec(raw["width"], raw["decay"])),)))
+        return ModelSpec(architecture="ToyFastForTests", hidden_size=raw["hidden"], vocab_size=raw["vocab"],
+                         max_context=512, layers=layers, schedule=(ScheduleEntry(0), ScheduleEntry(1)),
+                         final_norm=norm, tied_embeddings=True)
+
+
 @dataclass
 class ToyConfig:
     """A toy architecture: layer 0 = attention (toy position encoding) and the decay mixer in
@@ -128,6 +172,46 @@ def register_toys():
                 state[slot] = s
                 cursor += length
             return out.to(x.dtype)
+
+    @register_part("toy_gated_decay")
+    class GatedDecay(Mixer):
+        kernel_modules = ("gemm",)
+
+        @classmethod
+        def expected_tensors(cls, spec, prefix, hidden_size):
+            return [Expect(f"{prefix}.in_proj.weight", ((2 * spec.width, hidden_size),)),
+                    Expect(f"{prefix}.out_proj.weight", ((hidden_size, spec.width),))]
+
+        @classmethod
+        def cache_needs(cls, spec):
+            return [StateNeed("s", (spec.width,), "float32")]
+
+        def __init__(self, spec, prefix, tensors, build):
+            from macllm_infer_amd.parts import Linear
+            self.spec = spec
+            self.in_proj = Linear([tensors[f"{prefix}.in_proj.weight"]], [None], build)
+            self.out_proj = Linear([tensors[f"{prefix}.out_proj.weight"]], [None], build)
+
+        def projections(self):
+            return self.in_proj, self.out_proj, self.spec.width
+
+        def forward(self, x, step, cache):
+            mixed = torch.empty((x.shape[0], self.spec.width), dtype=x.dtype, device=x.device)
+            self.mix(self.in_proj(x), step, cache, mixed)
+            return self.out_proj(mixed)
+
+        def mix(self, projected, step, cache, out):
+            width, state = self.spec.width, cache.states["s"]
+            a, b = projected[:, :width].float(), projected[:, width:2 * width].float()
+            cursor = 0
+            for lane, length in enumerate(step.lane_lengths):          # a toy: token-serial on the host
+                slot = int(step.slot_ids[lane])
+                s = state[slot].clone()
+                for t in range(cursor, cursor + length):
+                    s = self.spec.decay * s + a[t]
+                    out[t] = (s * torch.sigmoid(b[t])).to(out.dtype)
+                state[slot] = s
+                cursor += length
 
     @register_part("toy_scale_position")
     class ScalePosition(PositionEncoding):
@@ -210,6 +294,7 @@ def register_toys():
             residual.pending = [self.ffn.forward(self.ffn_norm.forward(residual))]
 
     register_architecture(ToyConfig)
+    register_architecture(ToyFastConfig)
 
 
 def centred_norm(x, weight, bias, eps):
@@ -347,3 +432,29 @@ def exercise(schedule, device, check_device):
     window_group = [group for group in engine.cache.groups if group.need.window][0]
     assert len(window_group.tables["a"].live_pages()) <= 5 < len(window_group.tables["a"].pages)   # passed pages went back
     engine.cache.check()
+
+
+def toy_fast_plain_logits(raw, tensors, tokens):
+    """The two one-mixer layers of ``ToyFastConfig``, whole sequence, from the plain parts."""
+    T = len(tokens)
+    t = {name: value.float() for name, value in tensors.items()}
+    h = t["model.embed_tokens.weight"][torch.tensor(tokens)]
+    sub = lambda prefix: {name[len(prefix):]: value for name, value in t.items() if name.startswith(prefix)}
+    n = plain_impl.rms_norm(h, t["model.layers.0.attn_norm.weight"], 1e-5)
+    h = h + plain_impl.attention_mixer(n, sub("model.layers.0.self_attn."), num_heads=2, num_kv_heads=1, head_dim=64,
+                                       theta=1e4)
+    h = h + plain_impl.swiglu_mlp(plain_impl.rms_norm(h, t["model.layers.0.ffn_norm.weight"], 1e-5),
+                                  sub("model.layers.0.mlp."))
+    p = "model.layers.1."
+    n = centred_norm(h, t[p + "attn_norm.weight"], t[p + "attn_norm.bias"], 1e-4)
+    projected = n @ t[p + "decay.in_proj.weight"].T
+    width = raw["width"]
+    s, rows = torch.zeros(width), []
+    for position in range(T):
+        s = raw["decay"] * s + projected[position, :width]
+        rows.append(s * torch.sigmoid(projected[position, width:]))
+    h = h + torch.stack(rows) @ t[p + "decay.out_proj.weight"].T
+    f = centred_norm(h, t[p + "ffn_norm.weight"], t[p + "ffn_norm.bias"], 1e-4)
+    h = h + routed_feed_forward(f, t[p + "mlp.router.weight"], t[p + "mlp.up.weight"], t[p + "mlp.down.weight"])
+    h = plain_impl.rms_norm(h, t["model.norm.weight"], 1e-5)
+    return h @ t["model.embed_tokens.weight"].T
