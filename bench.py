@@ -3,12 +3,22 @@ MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|f32] [--layers L]
     python bench.py --workload serving [--shape 0.5b|7b|34b]
+    python bench.py --microbench
 
 One JSON line: ``value`` = decoded tokens a second at batch 8 with every request at a
 2,048-token context (a step = one decode step of the whole batch: model, greedy sampling,
-tokens fed back); ``prefill`` = one 2,048-token prompt in one step; ``roofline`` = the bytes
-the decode step has to read (every weight it uses once, and the cache and state of the live
-requests) over its time, against 8 TB/s; ``points`` = decode at batch 1 and 64.
+tokens fed back); ``prefill`` = one 2,048-token prompt in one step (replayed from its captured
+graph; ``prefill_uncaptured_ms`` = the same step launched kernel by kernel, as a shape is when it
+comes for the first time); ``roofline`` = the bytes the decode step has to read (every weight it
+uses once, and the cache and state of the live requests; ``bytes`` gives them and what the step
+writes) over its time, against 8 TB/s; ``points`` = decode at batch 1 and 64; ``step_ms`` = mean,
+median and 95th percentile of the timed steps (the reference reports the same three:
+src/benchmark/stats.rs:10-16); ``choices`` = what the build-time measurements chose for each
+projection of a layer at up to 16 / 32 / 64 rows (L = library, S = skinny kernel, a digit = slabs
+over K; then the skinny kernel's tiles of 16 features).
+
+``--microbench`` prints what this GPU's memory delivers to a plain streaming read and a plain
+read-modify-write (the ceilings that the decode kernels can be held against).
 
 ``--workload serving`` runs whole requests through the scheduler and the sampler instead
 (``LLM.generate``): for the 7B shape (and the 0.5B one) 64 requests with prompt lengths uniform in
@@ -21,8 +31,9 @@ import json
 import sys
 import time
 
-PEAK_HBM_GBS = 8000.0
-PEAK_FLOPS = {"bf16": 2.5e15, "f32": 157.3e12}
+from macllm_infer_amd.utils.costs import PEAK_FLOPS, PEAK_HBM_BYTES, decode_step_costs, prefill_costs, total
+
+PEAK_HBM_GBS = PEAK_HBM_BYTES / 1e9
 
 # Falcon-H1-0.5B-shaped: the layer sizes of the benchmark configuration
 SHAPE = dict(
@@ -105,6 +116,58 @@ def serving(args, shape) -> int:
     return 0
 
 
+def microbench() -> int:
+    """Streaming read and read-modify-write bandwidth of this GPU, with this package's own kernels."""
+    import torch
+    from macllm_infer_amd.kernels import ops
+    ops.require_gpu("cuda:0")
+    results = {}
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda:0")
+    for name, megabytes in (("read", 4096), ("rmw", 2048)):
+        data = torch.ones(megabytes * (1 << 20) // 4, dtype=torch.float32, device="cuda:0")
+        best = 0.0
+        for blocks in (1024, 2048, 4096, 8192, 16384):
+            run = (lambda: ops.stream_read(data, sink, blocks)) if name == "read" else (lambda: ops.stream_rmw(data, 1.0, blocks))
+            for _ in range(2):
+                run()
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(5):
+                run()
+            end.record()
+            end.synchronize()
+            seconds = start.elapsed_time(end) * 1e-3 / 5
+            moved = data.numel() * 4 * (1 if name == "read" else 2)
+            best = max(best, moved / seconds / 1e9)
+        results[name] = best
+        del data
+    print(json.dumps({"metric": "streaming memory bandwidth of this GPU (16 bytes a lane a load, float32)",
+                      "read_gbs": round(results["read"], 1), "read_modify_write_gbs": round(results["rmw"], 1),
+                      "unit": "GB/s", "published_peak_gbs": PEAK_HBM_GBS,
+                      "read_frac": round(results["read"] / PEAK_HBM_GBS, 4),
+                      "read_modify_write_frac": round(results["rmw"] / PEAK_HBM_GBS, 4)}))
+    return 0
+
+
+def choices_of(engine) -> dict:
+    """What the first layer's fast path chose, as short strings (empty when the layer has none)."""
+    fusion = getattr(engine.model.blocks[0], "fusion", None)
+    if fusion is None or not getattr(fusion, "decode_ok", False):
+        return {}
+
+    def way(library, split=(0, 0, 0)):
+        return "/".join(str(slabs) if slabs else ("L" if lib else "S") for lib, slabs in zip(library, split))
+
+    out = {"in": way(fusion.library_in), "out": way(fusion.library_out, fusion.split_out),
+           "tiles_in": "/".join(map(str, fusion.tiles_in)), "tiles_out": "/".join(map(str, fusion.tiles_out)),
+           "padded_in": bool(fusion.w_in_wide.shape[0] != fusion.in_width)}
+    if fusion.gate_up is not None:
+        out.update({"gate_up": way(fusion.library_gate_up), "down": way(fusion.library_down, fusion.split_down),
+                    "tiles_gate_up": "/".join(map(str, fusion.tiles_gate_up)),
+                    "tiles_down": "/".join(map(str, fusion.tiles_down))})
+    return out
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -122,10 +185,14 @@ def main() -> int:
                         help="only the 2,048-token prefill (for profiles; the line then reports prefill tokens/s)")
     parser.add_argument("--workload", default="steps", choices=["steps", "serving"],
                         help="steps: the headline decode and prefill steps; serving: whole requests through the scheduler")
+    parser.add_argument("--microbench", action="store_true",
+                        help="only this GPU's streaming read and read-modify-write bandwidth")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
         return 2
+    if args.microbench:
+        return microbench()
     if args.workload == "serving":
         return serving(args, SHAPES[args.shape])
 
@@ -172,24 +239,12 @@ def main() -> int:
         prefill_times.append(time.perf_counter() - started)
         engine.finish("prefill")
     prefill_seconds = sorted(prefill_times[3:])[1]      # the median of three; the step's graph is captured at its third sighting
+    uncaptured_seconds = min(prefill_times[1:2])        # the second sighting: launched kernel by kernel, the libraries warm
 
     d, L = config.hidden_size, config.num_hidden_layers
-    E = config.mamba_d_ssm
-    conv_width = E + 2 * config.mamba_n_groups * config.mamba_d_state
-    q_width = config.num_attention_heads * config.head_dim
-    kv_width = config.num_key_value_heads * config.head_dim
-    layer_matrix = (d * (q_width + 2 * kv_width) + q_width * d + d * (E + conv_width + config.mamba_n_heads)
-                    + E * d + 3 * d * config.intermediate_size)
-    T = PREFILL_TOKENS
-    prefill_flops = (2.0 * T * layer_matrix * L + 2.0 * vocab * d
-                     + L * 2.0 * config.num_attention_heads * config.head_dim * T * T
-                     + L * 6.0 * config.mamba_n_heads * config.mamba_d_head * config.mamba_d_state * T)
+    prefill_flops = total(prefill_costs(engine.spec, PREFILL_TOKENS, element)).flops
 
     # ---------------------------------------------------------------- decode at each batch size
-    weight_bytes = (layer_matrix * L + vocab * d) * element
-    state_bytes_per_request = L * (2 * config.mamba_n_heads * config.mamba_d_head * config.mamba_d_state * 4
-                                   + 2 * (config.mamba_d_conv - 1) * conv_width * element)
-    kv_bytes_per_token = config.kv_bytes_per_token(element)
     results = {}
     for batch in batches:
         names = [f"b{batch}_{index}" for index in range(batch)]
@@ -207,18 +262,25 @@ def main() -> int:
         for _ in range(args.warmup):
             tokens = decode_step(tokens)
         synchronize()
+        step_times = []
         started = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(args.steps):                   # a step ends with its tokens on the host: each can be timed
+            before = time.perf_counter()
             tokens = decode_step(tokens)
+            step_times.append(time.perf_counter() - before)
         synchronize()
         seconds = time.perf_counter() - started
         for name in names:
             engine.finish(name)
         step_seconds = seconds / args.steps
         context = CONTEXT + args.warmup + args.steps / 2.0
-        bytes_moved = weight_bytes + batch * (state_bytes_per_request + kv_bytes_per_token * context)
+        moved = total(decode_step_costs(engine.spec, batch, context, element))
+        step_times.sort()
+        pick = lambda fraction: step_times[min(len(step_times) - 1, int(fraction * len(step_times)))]
         results[batch] = dict(tokens_per_second=batch / step_seconds, ms=step_seconds * 1e3,
-                              gbs=bytes_moved / step_seconds / 1e9)
+                              gbs=moved.read / step_seconds / 1e9, read_mb=moved.read / 1e6, written_mb=moved.written / 1e6,
+                              step_ms={"mean": round(1e3 * sum(step_times) / len(step_times), 4),
+                                       "p50": round(1e3 * pick(0.5), 4), "p95": round(1e3 * pick(0.95), 4)})
 
     if args.prefill_only:
         print(json.dumps({"metric": "prefill tok/s at 2,048 tokens", "value": round(PREFILL_TOKENS / prefill_seconds, 1),
@@ -248,6 +310,10 @@ def main() -> int:
                      "frac": round(headline["gbs"] / PEAK_HBM_GBS, 5)},
         "points": {f"decode_b{batch}": round(result["tokens_per_second"], 1) for batch, result in results.items()
                    if batch != args.batch},
+        "step_ms": headline["step_ms"],
+        "bytes": {"read_mb": round(headline["read_mb"], 1), "written_mb": round(headline["written_mb"], 1)},
+        "prefill_uncaptured_ms": round(uncaptured_seconds * 1e3, 3),
+        "choices": choices_of(engine),
     }
     print(json.dumps(record))
     return 0

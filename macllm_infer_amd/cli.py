@@ -56,11 +56,14 @@ def _run(args) -> int:
     results = llm.generate(prompts, params)
     for index, result in enumerate(results):
         print(" ".join(str(token) for token in result.token_ids))
-        rate = result.decode_tokens_per_second
-        print(f"[request {index}] prompt_tokens={result.prompt_tokens} output_tokens={result.generated_tokens} "
+        # the reference's metrics line (src/main.rs:1396-1410), without its prefix-cache figures
+        number = lambda value, form: "-" if value is None else format(value, form)
+        print(f"[request {index}] prompt={result.prompt_tokens} output={result.generated_tokens} "
               f"finish={result.finish_reason} "
-              f"ttft_ms={'-' if result.time_to_first_token is None else f'{result.time_to_first_token * 1e3:.2f}'} "
-              f"decode_tok_s={'-' if rate is None else f'{rate:.1f}'} total_ms={result.total_time * 1e3:.2f}",
+              f"TTFT={number(None if result.time_to_first_token is None else result.time_to_first_token * 1e3, '.1f')}ms "
+              f"prefill={number(result.prefill_tokens_per_second, '.1f')} tok/s "
+              f"model-decode={number(result.decode_tokens_per_second, '.1f')} tok/s "
+              f"e2e-output={number(result.output_tokens_per_second, '.1f')} tok/s total={result.total_time * 1e3:.1f}ms",
               file=sys.stderr)
     return 0
 

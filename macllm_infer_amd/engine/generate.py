@@ -23,10 +23,23 @@ class GenerationResult:
     prompt_tokens: int
     time_to_first_token: Optional[float]
     total_time: float
+    prefill_time: Optional[float] = None       # from the request's admission to its first token
 
     @property
     def generated_tokens(self) -> int:
         return len(self.token_ids)
+
+    @property
+    def prefill_tokens_per_second(self) -> Optional[float]:
+        """Prompt tokens over the time from admission to the first token (src/generation.rs:76-79)."""
+        if not self.prefill_time or self.prefill_time <= 0:
+            return None
+        return self.prompt_tokens / self.prefill_time
+
+    @property
+    def output_tokens_per_second(self) -> Optional[float]:
+        """Emitted tokens over the whole time of the request (src/generation.rs:93-98)."""
+        return len(self.token_ids) / self.total_time if self.total_time > 0 else None
 
     @property
     def decode_tokens_per_second(self) -> Optional[float]:
@@ -89,8 +102,11 @@ class LLM:
         for request_id in ids:
             request: Request = finished[request_id]
             ttft = None if request.first_token_at is None else request.first_token_at - request.submitted_at
+            prefill = None
+            if request.first_token_at is not None and request.started_at is not None:
+                prefill = request.first_token_at - request.started_at
             results.append(GenerationResult(list(request.generated), request.finish_reason, len(request.prompt),
-                                            ttft, request.finished_at - request.submitted_at))
+                                            ttft, request.finished_at - request.submitted_at, prefill))
         return results
 
 

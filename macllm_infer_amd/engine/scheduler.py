@@ -60,6 +60,7 @@ class Request:
     finish_reason: Optional[str] = None    # "stop", "length", "cancelled", "resource_exhausted", "rejected: ..."
     cancelled: bool = False
     submitted_at: float = 0.0
+    started_at: Optional[float] = None     # admission: the request got its slot
     first_token_at: Optional[float] = None
     finished_at: Optional[float] = None
 
@@ -143,6 +144,7 @@ class Scheduler:
                 self._reject(request, "prompt plus requested output exceeds the cache capacity")
             else:
                 self.engine.add_request(request.request_id)
+                request.started_at = time.perf_counter()
                 self.active.append(request)
 
     def _collect(self) -> List[tuple]:

@@ -29,7 +29,7 @@ FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-shared", "-fPIC",
          "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", "-Wno-pass-failed"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall"]
 HOST_MODULES = ("hostcore",)                      # plain C++, no GPU code
-MODULES = ("common", "attention", "mamba2", "ssd", "gemm", "decode", "sampling") + HOST_MODULES
+MODULES = ("common", "attention", "mamba2", "ssd", "gemm", "decode", "sampling", "microbench") + HOST_MODULES
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

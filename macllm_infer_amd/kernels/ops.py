@@ -83,6 +83,10 @@ _SIGNATURES = {
                             _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr, _c_long,
                             _c_ptr],
     },
+    "microbench": {
+        "mi_stream_read": [_c_ptr, _c_long, _c_ptr, _c_int, _c_ptr],
+        "mi_stream_rmw": [_c_ptr, _c_long, _c_float, _c_int, _c_ptr],
+    },
     "sampling": {
         "mi_apply_penalties": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                _c_ptr, _c_ptr],
@@ -795,6 +799,24 @@ def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim
         num_groups, z_col, x_col, dt_col, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(slot_ids), _p(out),
         out.data_ptr() + 2 * num_heads * head_dim,
         _p(ssm_y), out_ld, _p(partial), partial.numel(), _stream()), "mixer_decode")
+
+
+# --------------------------------------------------------------------------- memory microbenchmarks
+def stream_read(data: torch.Tensor, sink: torch.Tensor, blocks: int = 4096) -> None:
+    """Read ``data`` (contiguous, a multiple of 16 bytes) once; ``sink``: an int32 GPU tensor."""
+    _need(data.is_cuda and data.is_contiguous() and (data.numel() * data.element_size()) % 16 == 0,
+          "stream_read: data must be a contiguous GPU tensor of a multiple of 16 bytes")
+    _i32(sink, "sink")
+    _check(_fn("microbench", "mi_stream_read")(_p(data), data.numel() * data.element_size(), _p(sink), int(blocks),
+                                               _stream()), "stream_read")
+
+
+def stream_rmw(data: torch.Tensor, scale: float = 1.0, blocks: int = 4096) -> None:
+    """data *= scale in place, float32, read once and written once."""
+    _need(data.is_cuda and data.is_contiguous() and data.dtype == torch.float32 and data.numel() % 4 == 0,
+          "stream_rmw: data must be a contiguous float32 GPU tensor of a multiple of 4 elements")
+    _check(_fn("microbench", "mi_stream_rmw")(_p(data), data.numel() * 4, float(scale), int(blocks), _stream()),
+           "stream_rmw")
 
 
 # --------------------------------------------------------------------------- sampling

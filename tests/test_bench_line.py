@@ -55,5 +55,40 @@ def test_line_of_a_short_run():
     assert roofline["bound"] == "hbm" and roofline["unit"] == "GB/s" and roofline["peak"] == 8000.0
     assert roofline["frac"] == pytest.approx(roofline["achieved"] / roofline["peak"], abs=1e-4)
     assert 0.0 < roofline["frac"] < 1.0
+    # the bytes are those the step has to read (every weight once, the cache and state of its requests)
+    assert roofline["achieved"] == pytest.approx(record["bytes"]["read_mb"] / record["ms_per_step"], rel=2e-3)
+    assert 0 < record["bytes"]["written_mb"] < record["bytes"]["read_mb"]
+    times = record["step_ms"]
+    assert set(times) == {"mean", "p50", "p95"} and 0 < times["p50"] <= times["p95"]
+    assert times["mean"] == pytest.approx(record["ms_per_step"], rel=0.05)
+    assert record["prefill_uncaptured_ms"] >= 0.9 * prefill["ms"]
+    assert {"in", "out", "gate_up", "down"} <= set(record["choices"])
     assert set(record["points"]) == {"decode_b1", "decode_b64"}
     assert record["points"]["decode_b1"] < record["value"] < record["points"]["decode_b64"]
+
+
+@pytest.mark.gpu
+def test_microbench_line():
+    code, printed = run_bench(["--microbench"])
+    assert code == 0
+    record = json.loads([line for line in printed.splitlines() if line.startswith("{")][0])
+    assert 1000.0 < record["read_modify_write_gbs"] < 8000.0 and 1000.0 < record["read_gbs"] < 8000.0
+    assert record["read_frac"] == pytest.approx(record["read_gbs"] / 8000.0, abs=1e-3)
+
+
+def test_costs_of_the_headline_step_are_the_ones_worked_out_by_hand():
+    """Falcon-H1-0.5B shape: 974.8 MB of weights; at 2,048 tokens a request reads 37.7 MB of keys and values,
+    28.3 MB of state and 0.4 MB of conv tails; a 2,048-token prompt is 2.10 TFLOP."""
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.utils import costs
+    spec = FalconH1Config.from_dict(bench.SHAPE).to_model_spec()
+    step = costs.decode_step_costs(spec, 8, 2048.0)
+    weights = sum(step[name].read for name in step if name != "mixers")
+    assert weights == pytest.approx(974.8e6, rel=1e-3)
+    assert step["mixers"].read / 8 == pytest.approx(37.75e6 + 28.31e6 + 0.39e6, rel=2e-3)
+    assert step["mixers"].written / 8 == pytest.approx(28.31e6 + 0.39e6 + 36 * 2 * 2 * 64 * 2, rel=2e-3)
+    assert costs.total(costs.prefill_costs(spec, 2048)).flops == pytest.approx(2.10e12, rel=2e-3)
+    assert costs.group_of("void fused_gemm_kernel<1, 0, 2, 4, 1>(FusedGemmParams)", costs.DECODE_GROUPS) == "input projections"
+    assert costs.group_of("void fused_gemm_kernel<1, 1, 0, 8, 1>(FusedGemmParams)", costs.DECODE_GROUPS) \
+        == "output projections + down projections"
+    assert costs.merged(step, "output projections + down projections").read == pytest.approx(302.0e6, rel=1e-3)

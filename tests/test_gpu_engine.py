@@ -247,7 +247,8 @@ def test_command_line_run(tmp_path):
                           cwd=ROOT, capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stderr
     assert [int(t) for t in done.stdout.split()] == plain_impl.greedy_generate(cfg, tensors, prompt, 5)
-    assert "finish=length" in done.stderr and "decode_tok_s" in done.stderr
+    assert "finish=length" in done.stderr and "prefill=" in done.stderr and "model-decode=" in done.stderr
+    assert "tok/s" in done.stderr and "TTFT=" in done.stderr
 
 
 # ------------------------------------------------------------------ generality, shown with toy parts
