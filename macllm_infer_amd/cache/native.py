@@ -36,8 +36,8 @@ def lib() -> ctypes.CDLL:
             "hc_finish": (i, [p, i]), "hc_length": (i, [p, i]), "hc_lengths": (None, [p, i, _INT_P, _INT_P]),
             "hc_reserve": (i, [p, i, _INT_P, _INT_P, _INT_P]), "hc_commit": (i, [p, i, _INT_P, _INT_P]),
             "hc_table": (i, [p, i, i, _INT_P, i]), "hc_first_live": (i, [p, i, i]), "hc_check": (i, [p]),
-            "hc_pack": (l, [p, i, _INT_P, _INT_P, _INT_P, _INT_P, _INT_P, i, _INT_P, i, i, _INT_P, i, _INT_P, l,
-                            _INT_P]),
+            "hc_pack": (l, [p, i, _INT_P, _INT_P, _INT_P, _INT_P, _INT_P, i, _INT_P, i, i, _INT_P, i, i, i, i, _INT_P,
+                            _INT_P, _INT_P, l, _INT_P]),
         }
         for name, (result, arguments) in signatures.items():
             function = getattr(core, name)

@@ -555,6 +555,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
   const int G = Hq / Hkv;
   const int head0 = kvh * G + blockIdx.z * NSET;             // first head of this pass
   const int request = tiles[2 * tile];
+  if (request < 0) return;                                    // a row of the table past the step's own runs
   const int lane = threadIdx.x & (WAVE - 1);
   const int wave = threadIdx.x / WAVE;
   const int qd = lane / 16;

@@ -263,22 +263,36 @@ int hc_check(void* handle) {
 //   token ids [T] | positions [T] | lane of token [T] | first token of each lane [L+1] |
 //   start positions [L] | lengths after the step [L] | slot ids [L] | wanted rows [W] |
 //   query tiles [tiles, 2] = (lane, first row) of runs of up to `query_tile` rows of one lane |
-//   per group: cache cell of each token [T] | block table [L, width]
+//   per group: cache cell of each token [T] | block table [L, width] |
+//   per chunk size Q: chunks [n, 4] = (lane, first row, rows, index within the lane) of every lane cut from its
+//                     first token into runs of Q rows | lane chunks [L, 2] = (first chunk, chunks) of every lane
 // for `n` lanes of live slots (their pages already reserved) followed by `pad_lanes` padding lanes
 // of `pad_lengths[i]` tokens (token id 0, position from 0) on the scratch slot and the scratch page
 // of every group (ids one past the pools').  `max_pages` > 0 fixes every table's width; otherwise
 // it is the longest table of the step.  `want_rows_fixed`, if given, replaces the wanted rows
-// (`fixed_count` of them).  meta receives: the 9 + 2*groups section sizes, then each group's
-// width, then the longest context after the step.  Returns the words written, -1 when a slot is
-// not live or a wanted place is outside its lane, or -(words needed) when `capacity` is too small.
+// (`fixed_count` of them).
+//
+// A step of fixed capacity (one whose arrays a captured graph reads at fixed addresses, whatever lanes it
+// holds) fixes the sizes of the sections that depend on how the tokens fall into lanes: `tiles_cap` > 0 makes
+// the tile table that long (entries past the step's own hold lane -1: nothing to do), `wants_cap` > 0 the
+// wanted rows (entries past the step's own name row 0: computed and dropped), `chunks_cap[c]` > 0 the chunk
+// table of chunk size c (entries past the step's own hold lane -1 and no rows).
+//
+// meta receives: the 9 + 2*groups + 2*chunk_sizes section sizes, then each group's width, then the longest
+// context after the step, then the step's own number of chunks for each chunk size.  Returns the words
+// written, -1 when a slot is not live, a wanted place is outside its lane or the step's pages were not
+// reserved, -2 when the step does not fit a fixed capacity, or -(words needed) - 2 when `capacity` is too small.
 long hc_pack(void* handle, int n, const int* slots, const int* lengths, const int* tokens, const int* want_counts,
              const int* wants, int pad_lanes, const int* pad_lengths, int max_pages, int query_tile,
-             const int* want_rows_fixed, int fixed_count, int* out, long capacity, int* meta) {
+             const int* want_rows_fixed, int fixed_count, int tiles_cap, int wants_cap, int n_chunk_sizes,
+             const int* chunk_sizes, const int* chunks_cap, int* out, long capacity, int* meta) {
   Core* core = (Core*)handle;
   const int L = n + pad_lanes;
   const int G = (int)core->groups.size();
+  const int C = n_chunk_sizes;
   long T = 0, W = 0, tiles = 0;
   int longest = 0;
+  std::vector<long> chunk_count(C, 0);
   for (int i = 0; i < L; ++i) {
     const int length = i < n ? lengths[i] : pad_lengths[i - n];
     if (length <= 0 || query_tile <= 0) return -1;
@@ -291,8 +305,29 @@ long hc_pack(void* handle, int n, const int* slots, const int* lengths, const in
     }
     T += length;
     tiles += (length + query_tile - 1) / query_tile;
+    for (int c = 0; c < C; ++c) {
+      if (chunk_sizes[c] <= 0) return -1;
+      chunk_count[c] += (length + chunk_sizes[c] - 1) / chunk_sizes[c];
+    }
   }
   if (want_rows_fixed) W = fixed_count;
+  const long own_tiles = tiles, own_wants = W;
+  if (tiles_cap > 0) {
+    if (tiles > tiles_cap) return -2;
+    tiles = tiles_cap;
+  }
+  if (wants_cap > 0) {
+    if (W > wants_cap) return -2;
+    W = wants_cap;
+  }
+  std::vector<long> chunk_rows(C);
+  for (int c = 0; c < C; ++c) {
+    chunk_rows[c] = chunk_count[c];
+    if (chunks_cap && chunks_cap[c] > 0) {
+      if (chunk_count[c] > chunks_cap[c]) return -2;
+      chunk_rows[c] = chunks_cap[c];
+    }
+  }
   std::vector<int> width(G, 1);
   for (int g = 0; g < G; ++g) {
     const Group& group = core->groups[g];
@@ -306,13 +341,16 @@ long hc_pack(void* handle, int n, const int* slots, const int* lengths, const in
   }
   long total = 3 * T + (L + 1) + 3L * L + W + 2 * tiles;
   for (int g = 0; g < G; ++g) total += T + (long)L * width[g];
+  for (int c = 0; c < C; ++c) total += 4 * chunk_rows[c] + 2L * L;
   int* m = meta;
   *m++ = (int)T; *m++ = (int)T; *m++ = (int)T; *m++ = L + 1; *m++ = L; *m++ = L; *m++ = L; *m++ = (int)W;
   *m++ = (int)(2 * tiles);
   for (int g = 0; g < G; ++g) { *m++ = (int)T; *m++ = L * width[g]; }
+  for (int c = 0; c < C; ++c) { *m++ = (int)(4 * chunk_rows[c]); *m++ = 2 * L; }
   for (int g = 0; g < G; ++g) *m++ = width[g];
   *m++ = longest;
-  if (total > capacity) return -total;
+  for (int c = 0; c < C; ++c) *m++ = (int)chunk_count[c];
+  if (total > capacity) return -total - 2;
 
   int* token_ids = out;
   int* positions = token_ids + T;
@@ -326,6 +364,7 @@ long hc_pack(void* handle, int n, const int* slots, const int* lengths, const in
   int* cursor = tile_words + 2 * tiles;
 
   long row = 0, want_at = 0, want_out = 0;
+  int* tile_at = tile_words;
   for (int i = 0; i < L; ++i) {
     const bool real = i < n;
     const int length = real ? lengths[i] : pad_lengths[i - n];
@@ -351,13 +390,18 @@ long hc_pack(void* handle, int n, const int* slots, const int* lengths, const in
       lane_of_token[row + t] = i;
     }
     for (int first = 0; first < length; first += query_tile) {
-      *tile_words++ = i;
-      *tile_words++ = (int)row + first;
+      *tile_at++ = i;
+      *tile_at++ = (int)row + first;
     }
     row += length;
   }
   first_token[L] = (int)row;
   if (want_rows_fixed) std::memcpy(want_rows, want_rows_fixed, sizeof(int) * fixed_count);
+  for (long w = own_wants; w < W; ++w) want_rows[w] = 0;
+  for (long t = own_tiles; t < tiles; ++t) {
+    *tile_at++ = -1;
+    *tile_at++ = 0;
+  }
 
   for (int g = 0; g < G; ++g) {
     const Group& group = core->groups[g];
@@ -391,6 +435,35 @@ long hc_pack(void* handle, int n, const int* slots, const int* lengths, const in
       }
       for (int p = count; p < width[g]; ++p) table_row[p] = 0;
       row += length;
+    }
+  }
+
+  for (int c = 0; c < C; ++c) {
+    const int Q = chunk_sizes[c];
+    int* chunk_out = cursor;
+    int* lane_out = chunk_out + 4 * chunk_rows[c];
+    cursor = lane_out + 2L * L;
+    long at = 0;
+    row = 0;
+    for (int i = 0; i < L; ++i) {
+      const int length = i < n ? lengths[i] : pad_lengths[i - n];
+      const int count = (length + Q - 1) / Q;
+      lane_out[2 * i] = (int)at;
+      lane_out[2 * i + 1] = count;
+      for (int index = 0; index < count; ++index) {
+        chunk_out[4 * at] = i;
+        chunk_out[4 * at + 1] = (int)row + index * Q;
+        chunk_out[4 * at + 2] = std::min(Q, length - index * Q);
+        chunk_out[4 * at + 3] = index;
+        ++at;
+      }
+      row += length;
+    }
+    for (; at < chunk_rows[c]; ++at) {
+      chunk_out[4 * at] = -1;
+      chunk_out[4 * at + 1] = 0;
+      chunk_out[4 * at + 2] = 0;
+      chunk_out[4 * at + 3] = 1;                         // not the first chunk of anything
     }
   }
   return total;

@@ -38,6 +38,7 @@ __device__ void ssd_prepare_block(const bf16_t* __restrict__ dt, long dt_ld, con
                                   float* wave_total) {
   const int t0 = chunks[4 * chunk + 1];
   const int length = chunks[4 * chunk + 2];
+  if (length <= 0) return;                    // a row of the table past the step's own chunks: the whole workgroup leaves
   const int s = threadIdx.x;
   const int lane = s & (WAVE - 1);
   const int wave = s / WAVE;
@@ -72,6 +73,7 @@ __device__ void ssd_transpose_block(const bf16_t* __restrict__ xbc, long ld, int
   const int stride = Q + 2;
   const int t0 = chunks[4 * chunk + 1];
   const int length = chunks[4 * chunk + 2];
+  if (length <= 0) return;                    // a row of the table past the step's own chunks: the whole workgroup leaves
   for (int index = threadIdx.x; index < Q * 8; index += 256) {
     const int s = index / 8;
     const int c = (index % 8) * 8;
@@ -132,6 +134,7 @@ __device__ void ssd_conv_block(const bf16_t* __restrict__ u, long u_ld, int C, c
   const int lane_id = chunks[4 * chunk];
   const int t0 = chunks[4 * chunk + 1];
   const int length = chunks[4 * chunk + 2];
+  if (length <= 0) return;                    // a row of the table past the step's own chunks: the whole workgroup leaves
   const bool opens = chunks[4 * chunk + 3] == 0;
   const bf16_t* tail = conv_state + (long)slot_ids[lane_id] * (K - 1) * C;
   const long first_row = opens ? (long)t0 : (long)t0 - (K - 1);
@@ -255,6 +258,7 @@ ssd_chunk_state_kernel(const bf16_t* __restrict__ TT, int E, int GN, const float
   const int group = head / (H / G);
   const int t0 = chunks[4 * chunk + 1];
   const int length = chunks[4 * chunk + 2];
+  if (length <= 0) return;                    // a row of the table past the step's own chunks: the whole workgroup leaves
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
@@ -376,6 +380,7 @@ ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t*
   const int heads = min(HB, group * heads_per_group + heads_per_group - head0);
   const int t0 = chunks[4 * chunk + 1];
   const int length = chunks[4 * chunk + 2];
+  if (length <= 0) return;                    // a row of the table past the step's own chunks: the whole workgroup leaves
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
@@ -548,6 +553,7 @@ ssd_chunk_scan_lds_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf1
   const int group = head / (H / G);
   const int t0 = chunks[4 * chunk + 1];
   const int length = chunks[4 * chunk + 2];
+  if (length <= 0) return;                    // a row of the table past the step's own chunks: the whole workgroup leaves
   const int part = gridDim.z - 1 - blockIdx.z;                         // the later 128 tokens first: they have more before them
   if (part * 128 >= length) return;
   const int tid = threadIdx.x;

@@ -48,11 +48,12 @@ class StepContext:
     query_tiles: torch.Tensor        # [tiles, 2] (lane, first token row) of runs of up to ``query_tile`` tokens of one lane
     block_tables: List[torch.Tensor] = field(default_factory=list)   # per group [lanes, max_pages]
     slot_mappings: List[torch.Tensor] = field(default_factory=list)  # per group [T] page*page_size+offset
-    lane_lengths: List[int] = field(default_factory=list)            # host copies
-    lane_starts: List[int] = field(default_factory=list)
-    max_query_len: int = 0
+    lane_lengths: Optional[List[int]] = field(default_factory=list)   # host copies; None in a step of fixed capacity
+    lane_starts: Optional[List[int]] = field(default_factory=list)
+    max_query_len: int = 0           # the longest lane (its upper bound in a step of fixed capacity)
     max_seq_len: int = 0             # an upper bound of the longest context in the batch
     derived: dict = field(default_factory=dict)   # tables parts derive from the step, shared by the layers
+    chunk_tables: dict = field(default_factory=dict)   # chunk size -> ChunkTable, for the sizes the model's mixers name
 
 
 @dataclass
@@ -84,43 +85,81 @@ def lower_lanes(lanes: Sequence[Lane], cache) -> LoweredLanes:
 _NO_LANES = LoweredLanes(*(np.zeros(0, dtype=np.int32) for _ in range(5)))
 
 
+@dataclass
+class ChunkTable:
+    """Every lane of a step cut from its first token into chunks of ``chunk_size`` tokens (the last one of a
+    lane may be short).  ``chunks`` int32 [num_chunks, 4] = (lane, first token row, tokens, index within the
+    lane); ``lane_chunks`` int32 [lanes, 2] = (first chunk, number of chunks).  In a step of fixed capacity
+    ``num_chunks`` is the table's capacity: rows past the step's own chunks hold lane -1 and no tokens."""
+    chunk_size: int
+    num_tokens: int
+    num_lanes: int
+    num_chunks: int
+    chunks: torch.Tensor
+    lane_chunks: torch.Tensor
+
+
 def _pack(lowered: LoweredLanes, cache, out: Optional[np.ndarray], pad_lengths: Sequence[int] = (),
-          max_pages: Optional[int] = None, want_rows: Optional[np.ndarray] = None, query_tile: int = 0):
+          max_pages: Optional[int] = None, want_rows: Optional[np.ndarray] = None, query_tile: int = 0,
+          chunk_sizes: Sequence[int] = (), tiles_cap: int = 0, wants_cap: int = 0, chunks_cap: Sequence[int] = ()):
     """The core writes the step's sections (in the order of ``_assemble``) into ``out``.  Returns
     (words written or, negated, words needed when ``out`` is too small or None; section sizes;
-    block-table shapes; longest context after the step).  ``pad_lengths``: lanes appended on the
-    scratch page and slot.  ``want_rows`` replaces the lanes' own wanted rows.  ``query_tile``: the
-    longest run of one lane's tokens in the table of runs (what the model's mixers ask for; 0: none does)."""
+    block-table shapes; longest context after the step; the step's own chunks per chunk size).
+    ``pad_lengths``: lanes appended on the scratch page and slot.  ``want_rows`` replaces the lanes' own
+    wanted rows.  ``query_tile``: the longest run of one lane's tokens in the table of runs (what the
+    model's mixers ask for; 0: none does).  ``chunk_sizes``: the chunk tables the model's mixers ask for.
+    ``tiles_cap``, ``wants_cap``, ``chunks_cap``: fixed sizes of the sections that depend on how the tokens
+    fall into lanes (a step of fixed capacity); ValueError when the step does not fit them."""
     core = cache.core
     pads = native.as_ints(list(pad_lengths))
     groups = len(cache.groups)
-    meta = np.zeros(9 + 3 * groups + 1, dtype=np.int32)
+    kinds = len(chunk_sizes)
+    meta = np.zeros(9 + 3 * groups + 3 * kinds + 1, dtype=np.int32)
     fixed = native.as_ints(want_rows) if want_rows is not None else None
+    sizes_in = native.as_ints(list(chunk_sizes))
+    caps_in = native.as_ints(list(chunks_cap) if len(chunks_cap) else [0] * kinds)
     written = core.lib.hc_pack(
         core.pointer, len(lowered.slots), native.int_pointer(lowered.slots), native.int_pointer(lowered.lengths),
         native.int_pointer(lowered.tokens), native.int_pointer(lowered.want_counts), native.int_pointer(lowered.wants),
         len(pads), native.int_pointer(pads), max_pages or 0, query_tile or NO_TILES,
         native.int_pointer(fixed) if fixed is not None else None, len(fixed) if fixed is not None else 0,
+        int(tiles_cap), int(wants_cap), kinds, native.int_pointer(sizes_in), native.int_pointer(caps_in),
         native.int_pointer(out) if out is not None else None, out.size if out is not None else 0,
         native.int_pointer(meta))
     if written == -1:
         raise ValueError("the step cannot be packed: a request is not live, a wanted place lies outside its "
                          "lane, or the step's pages were not reserved")
+    if written == -2:
+        raise ValueError("the step does not fit the fixed capacity it is packed for")
+    if written < 0:
+        written += 2                                     # -(words needed) - 2
     lanes = len(lowered.slots) + len(pads)
-    sizes = meta[:9 + 2 * groups].tolist()
-    shapes = [(lanes, int(width)) for width in meta[9 + 2 * groups:9 + 3 * groups]]
-    return int(written), sizes, shapes, int(meta[-1])
+    count = 9 + 2 * groups + 2 * kinds
+    sizes = meta[:count].tolist()
+    shapes = [(lanes, int(width)) for width in meta[count:count + groups]]
+    return int(written), sizes, shapes, int(meta[count + groups]), meta[count + groups + 1:count + groups + 1 + kinds].tolist()
 
 
-def _assemble(views, group_shapes, lengths, starts, max_seq_len) -> StepContext:
+def _assemble(views, group_shapes, lengths, starts, max_seq_len, chunk_sizes=(), num_tokens=None, num_lanes=None,
+              max_query_len=None) -> StepContext:
+    """``lengths`` / ``starts``: the lanes' host copies, or None for a step of fixed capacity, whose lanes
+    differ from fill to fill (``num_tokens``, ``num_lanes`` and ``max_query_len`` are then its capacities)."""
+    tokens = sum(lengths) if lengths is not None else num_tokens
+    lanes = len(lengths) if lengths is not None else num_lanes
     context = StepContext(
-        num_tokens=sum(lengths), num_lanes=len(lengths), token_ids=views[0], positions=views[1],
+        num_tokens=tokens, num_lanes=lanes, token_ids=views[0], positions=views[1],
         lane_of_token=views[2], cu_seqlens=views[3], start_pos=views[4], seq_lens=views[5], slot_ids=views[6],
-        want_rows=views[7], query_tiles=views[8].view(-1, 2), lane_lengths=list(lengths), lane_starts=list(starts), max_query_len=max(lengths),
-        max_seq_len=max_seq_len)
+        want_rows=views[7], query_tiles=views[8].view(-1, 2),
+        lane_lengths=list(lengths) if lengths is not None else None,
+        lane_starts=list(starts) if starts is not None else None,
+        max_query_len=max(lengths) if lengths is not None else max_query_len, max_seq_len=max_seq_len)
+    groups = len(group_shapes)
     for index, shape in enumerate(group_shapes):
         context.slot_mappings.append(views[9 + 2 * index])
         context.block_tables.append(views[10 + 2 * index].view(shape))
+    for index, chunk_size in enumerate(chunk_sizes):
+        chunks, lane_chunks = views[9 + 2 * groups + 2 * index], views[10 + 2 * groups + 2 * index]
+        context.chunk_tables[chunk_size] = ChunkTable(chunk_size, tokens, lanes, chunks.numel() // 4, chunks, lane_chunks)
     return context
 
 
@@ -133,39 +172,64 @@ def _split(buffer: torch.Tensor, sizes):
 
 
 def build_step_context(lanes: Sequence[Lane], cache, device, lowered: Optional[LoweredLanes] = None,
-                       query_tile: int = 0) -> StepContext:
-    """``cache``: the CacheManager, after the step's pages were reserved.  ``query_tile``: see ``_pack``
-    (``DecoderModel.query_tile`` for a whole model)."""
+                       query_tile: int = 0, chunk_sizes: Sequence[int] = ()) -> StepContext:
+    """``cache``: the CacheManager, after the step's pages were reserved.  ``query_tile``, ``chunk_sizes``:
+    see ``_pack`` (``DecoderModel.query_tile`` and ``.chunk_sizes`` for a whole model)."""
     if lowered is None:
         lowered = lower_lanes(lanes, cache)
-    needed, _, _, _ = _pack(lowered, cache, None, query_tile=query_tile)
+    needed, _, _, _, _ = _pack(lowered, cache, None, query_tile=query_tile, chunk_sizes=chunk_sizes)
     host = torch.empty(-needed, dtype=torch.int32)
     if torch.device(device).type == "cuda":
         host = host.pin_memory()
-    _, sizes, shapes, longest = _pack(lowered, cache, host.numpy(), query_tile=query_tile)
+    _, sizes, shapes, longest, _ = _pack(lowered, cache, host.numpy(), query_tile=query_tile, chunk_sizes=chunk_sizes)
     packed = host.to(device, non_blocking=True)
     starts = cache.lengths_of(lowered.slots).tolist()
-    context = _assemble(_split(packed, sizes), shapes, lowered.lengths.tolist(), starts, longest)
+    context = _assemble(_split(packed, sizes), shapes, lowered.lengths.tolist(), starts, longest, chunk_sizes)
     context._keepalive = host
     return context
 
 
 class StaticStep:
-    """The arrays of a step of fixed shape at fixed device addresses: ``lanes`` single-token lanes
-    whose logits are all wanted, or lanes of ``lengths`` tokens with the wanted rows ``want_rows``.
-    ``fill`` rewrites them for the real lanes of a step of that shape."""
+    """The arrays of a step at fixed device addresses and of fixed sizes, which a captured graph reads:
+
+    * ``lanes`` single-token lanes whose logits are all wanted (a decode step), or lanes of ``lengths`` tokens
+      with the wanted rows ``want_rows``; or
+    * with ``tokens``: a step of fixed *capacity*: up to ``lanes`` lanes that hold ``tokens`` tokens together,
+      whatever their lengths, and up to ``wants`` wanted rows.  The tables that depend on how the tokens fall
+      into lanes (runs of a lane's tokens, chunks) have the size of the worst case and are rewritten with the
+      rest; what the step's own lanes leave of the capacity is padding lanes on the cache's scratch page and
+      slot, the first ones of one token and the last one with the remainder.
+
+    ``fill`` rewrites the arrays for the real lanes of a step."""
 
     def __init__(self, cache, lanes: int, max_seq_len: int, device, lengths: Sequence[int] = (),
-                 want_rows: Sequence[int] = (), query_tile: int = 0):
+                 want_rows: Sequence[int] = (), query_tile: int = 0, chunk_sizes: Sequence[int] = (),
+                 tokens: int = 0, wants: int = 0):
         self.cache = cache
         self.query_tile = query_tile
+        self.chunk_sizes = tuple(chunk_sizes)
         self.lanes = lanes
-        self.lengths = list(lengths) if lengths else [1] * lanes
+        self.tokens = tokens
         self.max_pages = max(-(-max_seq_len // group.page_size) for group in cache.groups) if cache.groups else 1
-        self.want_rows = (np.asarray(want_rows, dtype=np.int32) if lengths
-                          else np.arange(lanes, dtype=np.int32))             # every lane's row is wanted
-        needed, sizes, shapes, _ = _pack(_NO_LANES, cache, None, self.lengths, self.max_pages, self.want_rows,
-                                         query_tile)
+        self.capacity = tokens > 0
+        if self.capacity:
+            if tokens < lanes or wants <= 0:
+                raise ValueError("a step of fixed capacity holds at least one token a lane and wants a row")
+            self.lengths = None
+            self.want_rows = None
+            tile = query_tile or NO_TILES
+            self.caps = dict(tiles_cap=-(-tokens // tile) + lanes, wants_cap=wants,
+                             chunks_cap=[-(-tokens // size) + lanes for size in self.chunk_sizes])
+            first_pads = self._pads(0, 0)
+        else:
+            self.lengths = list(lengths) if lengths else [1] * lanes
+            self.want_rows = (np.asarray(want_rows, dtype=np.int32) if lengths
+                              else np.arange(lanes, dtype=np.int32))             # every lane's row is wanted
+            self.caps = {}
+            first_pads = self.lengths
+        pack = dict(max_pages=self.max_pages, want_rows=self.want_rows, query_tile=query_tile,
+                    chunk_sizes=self.chunk_sizes, **self.caps)
+        needed, sizes, shapes, _, _ = _pack(_NO_LANES, cache, None, first_pads, **pack)
         # The host packs a step into pinned memory and queues its copy to the fixed device addresses; the
         # copy runs when the stream gets there, so the memory it reads must stay as it is until then.  A few
         # host buffers are filled in turn, each guarded by an event recorded behind its copy: the host may
@@ -179,22 +243,46 @@ class StaticStep:
         self._pending = [False] * len(self._hosts)
         self._turn = 0
         self.device_buffer = torch.empty(-needed, dtype=torch.int32, device=device)
-        _pack(_NO_LANES, cache, self._hosts[0].numpy(), self.lengths, self.max_pages, self.want_rows, query_tile)
+        _pack(_NO_LANES, cache, self._hosts[0].numpy(), first_pads, **pack)
         self.device_buffer.copy_(self._hosts[0])
-        self.context = _assemble(_split(self.device_buffer, sizes), shapes, self.lengths, [0] * lanes, max_seq_len)
+        if self.capacity:
+            self.context = _assemble(_split(self.device_buffer, sizes), shapes, None, None, max_seq_len,
+                                     self.chunk_sizes, num_tokens=tokens, num_lanes=lanes, max_query_len=tokens)
+        else:
+            self.context = _assemble(_split(self.device_buffer, sizes), shapes, self.lengths, [0] * lanes, max_seq_len,
+                                     self.chunk_sizes)
 
     HOST_BUFFERS = 2
 
+    def _pads(self, real_lanes: int, real_tokens: int) -> List[int]:
+        """The padding lanes of a step of fixed capacity beside ``real_lanes`` lanes of ``real_tokens`` tokens."""
+        pads, rest = self.lanes - real_lanes, self.tokens - real_tokens
+        if pads < 0 or rest < pads or (pads == 0 and rest != 0):
+            raise ValueError(f"{real_lanes} lanes of {real_tokens} tokens do not fit a step of {self.lanes} lanes and "
+                             f"{self.tokens} tokens")
+        return [1] * (pads - 1) + [rest - (pads - 1)] if pads else []
+
+    @staticmethod
+    def fits(lanes_cap: int, tokens_cap: int, lanes: int, tokens: int) -> bool:
+        """Whether a step of ``lanes`` lanes and ``tokens`` tokens can be padded to the capacity."""
+        pads, rest = lanes_cap - lanes, tokens_cap - tokens
+        return pads >= 0 and ((pads == 0 and rest == 0) or (pads > 0 and rest >= pads))
+
     def fill(self, lowered: LoweredLanes) -> None:
-        """``lowered``: the real lanes, whose lengths are the first of this step's; the rest is padding."""
+        """``lowered``: the real lanes (a step of fixed lanes: their lengths are the first of this step's; the
+        rest is padding)."""
         real = len(lowered.slots)
+        if self.capacity:
+            pads = self._pads(real, int(lowered.lengths.sum()))
+        else:
+            pads = self.lengths[real:]
         turn = self._turn
         self._turn = (turn + 1) % len(self._hosts)
         if self._pending[turn]:
             self._copied[turn].synchronize()          # the copy that last read this buffer has run
         host = self._hosts[turn]
-        _pack(lowered, self.cache, host.numpy(), self.lengths[real:], self.max_pages, self.want_rows,
-              self.query_tile)
+        _pack(lowered, self.cache, host.numpy(), pads, max_pages=self.max_pages, want_rows=self.want_rows,
+              query_tile=self.query_tile, chunk_sizes=self.chunk_sizes, **self.caps)
         self.device_buffer.copy_(host, non_blocking=True)
         if self._copied[turn] is not None:
             self._copied[turn].record()

@@ -101,6 +101,12 @@ class Engine:
             from .graphs import DecodeGraphs
             self.graphs = DecodeGraphs(self.model, self.cache, self.device, min(self.max_context, capacity))
 
+    def warm_up(self, steps, context: int = 2048) -> list:
+        """Capture the graphs of steps of (lanes, tokens) before the first request comes (a serving process
+        does this once: no step of such a size is then ever launched kernel by kernel).  ``context``: the
+        longest context the steps' requests will hold.  Returns what was captured; nothing without graphs."""
+        return self.graphs.warm_up(steps, context) if self.graphs is not None else []
+
     # ------------------------------------------------------------------ requests
     def add_request(self, request: Hashable) -> None:
         """Make ``request`` live: a zeroed state slot and empty block tables."""
@@ -168,9 +174,10 @@ class Engine:
                 if int(lowered.lengths.max()) == 1:
                     logits = self.graphs.run(lanes, lowered)              # decode-only batch: a captured graph
                 else:
-                    logits = self.graphs.run_portion(lanes, lowered)      # a shape of prompt portions seen before
+                    logits = self.graphs.run_bucket(lanes, lowered)       # prompt portions: a graph of their capacity
             if logits is None:
-                context = build_step_context(lanes, self.cache, self.device, lowered, self.model.query_tile)
+                context = build_step_context(lanes, self.cache, self.device, lowered, self.model.query_tile,
+                                             self.model.chunk_sizes)
                 logits = self.model.forward(context, self.cache)
         except Exception as error:
             # earlier layers have written keys, values and state in place: these requests cannot go on

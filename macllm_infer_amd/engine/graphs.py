@@ -9,21 +9,25 @@ launched for), so graphs come in buckets of context length as well, powers of tw
 tokens up to the longest the cache can hold: a model that allows 262,144 tokens does not pay
 for them while its requests are short.
 
-Prompt portions are launch-bound too once the kernels are fast (a portion of 2,048 tokens is
-some 700 launches).  A scheduler cuts long prompts into portions of one size, so the shape of
-a step (the lengths of its lanes and the places wanted) repeats.  A capture costs as much as some
-ten steps' launches, and the last portion of every prompt has a length of its own, so a shape is
-captured only at its third sighting among the last 32 steps with portions, and replayed from then
-on; a few shapes are kept, the least recently used one goes.
+Steps with prompt portions are launch-bound too once the kernels are fast (a portion of 2,048 tokens is
+some 470 launches: launched one by one, the host needs 5 ms for them whatever their length).  Their
+graphs are made for a *capacity*, not for a shape: so many tokens in so many lanes with so many wanted
+rows, whatever the lanes' lengths.  Every kernel reads where a lane begins and ends from the step's
+arrays on the device, and the tables that depend on it (runs of a lane's tokens for the attention
+kernel, chunks for the scan) have the size of the worst case; what a step leaves of the capacity is
+padding lanes on the scratch page and slot.  A handful of capacities (token counts in steps of a quarter
+to a third, lane counts in powers of two) therefore serves every step a scheduler can make, a capacity is
+captured when it comes the second time (a single prompt is not worth a capture, which costs two passes of
+launches), and ``warm_up`` captures a list of them before the first request.
 """
 from __future__ import annotations
 
-from collections import OrderedDict, deque
-from typing import Dict, Optional, Sequence
+from collections import OrderedDict
+from typing import Dict, Iterable, List, Optional, Sequence, Tuple
 
 import torch
 
-from .context import Lane, LoweredLanes, StaticStep, lower_lanes
+from .context import Lane, LoweredLanes, StaticStep
 
 
 def bucket_for(lanes: int) -> int:
@@ -36,6 +40,20 @@ def bucket_for(lanes: int) -> int:
 CONTEXT_BUCKET_FROM = 2048
 
 
+def token_capacities(most: int) -> List[int]:
+    """The token counts that steps with prompt portions are padded to: 16, 32, 48, 64, then steps of a
+    quarter of the power of two below (80, 96, 112, 128, 160, ...) and, from 1,024 on, of an eighth (1,152,
+    1,280, ...: a scheduler's portion of 2,048 tokens beside a few decoded ones pads to 2,304), up to the first
+    one that holds ``most``."""
+    out, value = [], 16
+    while True:
+        out.append(value)
+        if value >= most:
+            return out
+        power = 1 << (value.bit_length() - 1)
+        value += max(16, power // (8 if value >= 1024 else 4))
+
+
 class DecodeGraphs:
     def __init__(self, model, cache, device, max_seq_len: int):
         self.model = model
@@ -43,80 +61,103 @@ class DecodeGraphs:
         self.device = device
         self.max_seq_len = max_seq_len
         self._graphs: Dict[tuple, tuple] = {}
-        self._portion_graphs: "OrderedDict[tuple, tuple]" = OrderedDict()
-        self._portion_recent: deque = deque(maxlen=self.PORTION_RECENT)
-        self.counts = {"decode_replays": 0, "portion_replays": 0, "portion_captures": 0, "portion_eager": 0}
+        self._bucket_graphs: "OrderedDict[tuple, tuple]" = OrderedDict()
+        self._seen: "OrderedDict[tuple, int]" = OrderedDict()
+        self._pool = None
+        self.counts = {"decode_replays": 0, "bucket_replays": 0, "bucket_captures": 0, "bucket_eager": 0}
 
-    PORTION_MIN_TOKENS = 64        # shorter steps are cheap to launch one by one
-    PORTION_GRAPHS = 8
-    PORTION_RECENT = 32            # steps with portions whose shapes are remembered
-    PORTION_SIGHTINGS = 3          # sightings among them before a shape is captured
+    BUCKET_GRAPHS = 24             # captured capacities kept; the least recently used one goes
+    BUCKET_SIGHTINGS = 2           # sightings of a capacity before it is captured
+    BUCKET_MOST_TOKENS = 16384     # steps beyond this many tokens are launched kernel by kernel
 
-    def context_bucket(self, lowered: LoweredLanes) -> int:
+    def context_bucket(self, lowered: LoweredLanes, at_least: int = 0) -> int:
         """The smallest bucket of context length that holds every lane of the step after it ran."""
-        longest = int((self.cache.lengths_of(lowered.slots) + lowered.lengths).max())
+        longest = max(int((self.cache.lengths_of(lowered.slots) + lowered.lengths).max()), at_least)
         bucket = CONTEXT_BUCKET_FROM
         while bucket < longest:
             bucket <<= 1
         return min(bucket, self.max_seq_len)
 
-    def run_portion(self, lanes: Sequence[Lane], lowered: LoweredLanes) -> Optional[torch.Tensor]:
-        """Logits of a step with prompt portions from a captured graph of its shape, or None when
-        the shape has no graph (yet): the caller then runs it launch by launch.
-
-        Lanes do not depend on each other, so the shape is taken in a canonical order (longest
-        first, then by the places wanted) and the single-token lanes are padded to a power of two:
-        a scheduler that rotates its requests, or whose decoding set grows by one, meets the same
-        graph again.  The logits come back in the caller's order."""
-        if sum(len(lane.tokens) for lane in lanes) < self.PORTION_MIN_TOKENS:
-            self.counts["portion_eager"] += 1
+    def capacity_for(self, lanes: int, tokens: int, wants: int) -> Optional[Tuple[int, int, int]]:
+        """(lanes, tokens, wanted rows) of the smallest capacity that holds such a step, or None."""
+        if tokens > self.BUCKET_MOST_TOKENS:
             return None
-        order = sorted(range(len(lanes)), key=lambda index: (-len(lanes[index].tokens), tuple(lanes[index].want), index))
-        ordered = [lanes[index] for index in order]
-        singles = sum(1 for lane in ordered if len(lane.tokens) == 1)
-        padding = bucket_for(singles) - singles if singles else 0
-        # padding lanes stand last, as single tokens whose logits are computed and dropped
-        lengths = tuple(len(lane.tokens) for lane in ordered) + (1,) * padding
-        wants = tuple(tuple(lane.want) for lane in ordered) + ((0,),) * padding
-        context = self.context_bucket(lowered)
-        key = (lengths, wants, context)
-        entry = self._portion_graphs.get(key)
+        lane_cap = bucket_for(lanes)
+        for _ in range(2):                                   # the lanes' own bucket, or the next one (room for padding lanes)
+            for token_cap in token_capacities(self.BUCKET_MOST_TOKENS):
+                if token_cap >= tokens and StaticStep.fits(lane_cap, token_cap, lanes, tokens):
+                    return lane_cap, token_cap, lane_cap if wants <= lane_cap else token_cap
+            lane_cap <<= 1
+        return None
+
+    def run_bucket(self, lanes: Sequence[Lane], lowered: LoweredLanes) -> Optional[torch.Tensor]:
+        """Logits of a step with prompt portions from the captured graph of its capacity, or None when that
+        capacity has no graph (yet): the caller then launches the step kernel by kernel."""
+        capacity = self.capacity_for(len(lanes), int(lowered.lengths.sum()), int(lowered.want_counts.sum()))
+        if capacity is None:
+            self.counts["bucket_eager"] += 1
+            return None
+        context = self.context_bucket(lowered, at_least=capacity[1])
+        if context < capacity[1]:                           # the cache cannot hold a padding lane of that many tokens
+            self.counts["bucket_eager"] += 1
+            return None
+        key = capacity + (context,)
+        entry = self._bucket_graphs.get(key)
         if entry is None:
-            self._portion_recent.append(key)
-            if sum(1 for recent in self._portion_recent if recent == key) < self.PORTION_SIGHTINGS:
-                self.counts["portion_eager"] += 1
+            self._seen[key] = self._seen.get(key, 0) + 1
+            self._seen.move_to_end(key)
+            while len(self._seen) > 4 * self.BUCKET_GRAPHS:
+                self._seen.popitem(last=False)
+            if self._seen[key] < self.BUCKET_SIGHTINGS:
+                self.counts["bucket_eager"] += 1
                 return None
-            first, rows = 0, []
-            for length, want in zip(lengths, wants):
-                rows += [first + place for place in want]
-                first += length
-            static = StaticStep(self.cache, len(lengths), context, self.device, lengths=lengths, want_rows=rows,
-                                query_tile=self.model.query_tile)
-            entry = self._capture(0, static, warm_runs=1)      # the libraries have seen these sizes already
-            self.counts["portion_captures"] += 1
-            while len(self._portion_graphs) >= self.PORTION_GRAPHS:
-                self._portion_graphs.popitem(last=False)
-            self._portion_graphs[key] = entry
+            entry = self._capture_bucket(key)
         else:
-            self._portion_graphs.move_to_end(key)
+            self._bucket_graphs.move_to_end(key)
         static, graph, logits = entry
-        static.fill(lowered if order == list(range(len(lanes))) else lower_lanes(ordered, self.cache))
+        static.fill(lowered)
         graph.replay()
-        self.counts["portion_replays"] += 1
-        if padding == 0 and order == list(range(len(lanes))):
-            return logits.clone()
-        # rows of the canonical order -> the caller's order
-        first_row, starts = 0, {}
-        for index, lane in zip(order, ordered):
-            starts[index] = first_row
-            first_row += len(lane.want)
-        rows = [starts[index] + offset for index, lane in enumerate(lanes) for offset in range(len(lane.want))]
-        return logits[torch.tensor(rows, dtype=torch.long, device=logits.device)] if rows else logits[:0].clone()
+        self.counts["bucket_replays"] += 1
+        return logits[:int(lowered.want_counts.sum())].clone()
+
+    def _capture_bucket(self, key: tuple):
+        lane_cap, token_cap, want_cap, context = key
+        static = StaticStep(self.cache, lane_cap, context, self.device, query_tile=self.model.query_tile,
+                            chunk_sizes=self.model.chunk_sizes, tokens=token_cap, wants=want_cap)
+        entry = self._capture(0, static, warm_runs=1)
+        self.counts["bucket_captures"] += 1
+        while len(self._bucket_graphs) >= self.BUCKET_GRAPHS:
+            self._bucket_graphs.popitem(last=False)
+        self._bucket_graphs[key] = entry
+        return entry
+
+    def warm_up(self, steps: Iterable[Tuple[int, int]], context: int = CONTEXT_BUCKET_FROM) -> List[tuple]:
+        """Capture, before the first request, the graphs of steps of (lanes, tokens) with one wanted row a
+        lane (steps of single tokens: their decode graphs); returns the keys of what was captured."""
+        done = []
+        for lanes, tokens in steps:
+            if tokens == lanes:
+                key = (bucket_for(lanes), min(max(context, CONTEXT_BUCKET_FROM), self.max_seq_len))
+                if key not in self._graphs:
+                    self._graphs[key] = self._capture(key[0], context=key[1])
+                    done.append(key)
+                continue
+            capacity = self.capacity_for(lanes, tokens, lanes)
+            if capacity is None:
+                continue
+            bucket = CONTEXT_BUCKET_FROM
+            while bucket < max(context, capacity[1]):
+                bucket <<= 1
+            key = capacity + (min(bucket, self.max_seq_len),)
+            if key[3] >= capacity[1] and key not in self._bucket_graphs:
+                self._capture_bucket(key)
+                done.append(key)
+        return done
 
     def _capture(self, bucket: int, static: Optional[StaticStep] = None, warm_runs: int = 2, context: int = 0):
         if static is None:
             static = StaticStep(self.cache, bucket, context or self.max_seq_len, self.device,
-                                query_tile=self.model.query_tile)
+                                query_tile=self.model.query_tile, chunk_sizes=self.model.chunk_sizes)
         # a first run outside the graph lets the libraries set themselves up; every lane is padding,
         # so only the scratch page and slot are touched
         side = torch.cuda.Stream(device=self.device)
@@ -127,7 +168,10 @@ class DecodeGraphs:
         torch.cuda.current_stream(self.device).wait_stream(side)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        # one pool for every graph: replays never overlap, so their intermediate buffers may share memory
+        if self._pool is None:
+            self._pool = torch.cuda.graph_pool_handle()
+        with torch.cuda.graph(graph, pool=self._pool):
             logits = self.model.forward(static.context, self.cache)
         return static, graph, logits
 

@@ -93,8 +93,10 @@ class DecoderModel:
         prologue = getattr(self.final_norm, "rms_prologue", None)
         self._final_rms = prologue() if prologue is not None else None
         # the step's table of runs of one lane's tokens is cut for the mixer with the largest tile
-        self.query_tile = max((getattr(mixer, "query_tile", 0) for block in self.blocks for _, mixer in block.mixers),
-                              default=0)
+        mixers = [mixer for block in self.blocks for _, mixer in block.mixers]
+        self.query_tile = max((getattr(mixer, "query_tile", 0) for mixer in mixers), default=0)
+        # and its tables of chunks for the chunk sizes the mixers name
+        self.chunk_sizes = tuple(sorted({getattr(mixer, "chunk_tokens", 0) for mixer in mixers} - {0}))
 
     @property
     def graph_safe(self) -> bool:

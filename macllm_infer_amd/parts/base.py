@@ -86,6 +86,9 @@ class Mixer(Part):
     # rows of one lane that one workgroup of the mixer's prompt kernel takes: the step's table of such runs
     # is cut to the largest tile any mixer of the model names (0: the mixer reads no such table)
     query_tile = 0
+    # tokens of a chunk: the step then carries every lane cut from its first token into chunks of that many
+    # (``step.chunk_tables[chunk_tokens]``); 0: the mixer reads no such table
+    chunk_tokens = 0
 
     @classmethod
     def cache_needs(cls, spec):

@@ -79,6 +79,7 @@ class Mamba2(Mixer):
         self.D = f32(get("D").reshape(H))
         self.norm_weight = f32(get("norm.weight").reshape(E)) if spec.gated_norm else None
         self._chunks_supported = None
+        self.chunk_tokens = spec.chunk_size          # the step's chunk table that the chunked scan reads
 
     def _chunked(self, u: torch.Tensor, step) -> bool:
         """Prompt portions in bfloat16 scan in chunks on the matrix cores; single tokens, float32
@@ -92,6 +93,10 @@ class Mamba2(Mixer):
         return self._chunks_supported
 
     def _chunk_table(self, step):
+        """The step's own table of chunks, or (a step that was packed without one) one made from its lanes."""
+        table = step.chunk_tables.get(self.spec.chunk_size)
+        if table is not None:
+            return table
         key = ("ssd_chunks", self.spec.chunk_size)
         if key not in step.derived:
             step.derived[key] = ops.SsdChunks(step.lane_lengths, self.spec.chunk_size, step.token_ids.device)

@@ -239,6 +239,89 @@ def plain_packing(cache, lanes, pad_lengths, width):
     return out
 
 
+def plain_chunks(lengths, size):
+    chunks, lane_chunks, first = [], [], 0
+    for lane, length in enumerate(lengths):
+        count = -(-length // size)
+        lane_chunks.append([len(chunks), count])
+        chunks += [[lane, first + index * size, min(size, length - index * size), index] for index in range(count)]
+        first += length
+    return chunks, lane_chunks
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_a_step_of_fixed_capacity_holds_any_lanes_that_fit_it(seed):
+    """The arrays of a captured step made for a capacity (so many tokens in so many lanes, so many wanted rows):
+    filled with lanes of any lengths they are the plain packing of those lanes followed by padding lanes on the
+    scratch page and slot (single tokens, then one lane with the remainder), with the tables of runs and of
+    chunks filled up to their fixed sizes by rows that say "nothing here"."""
+    from macllm_infer_amd.engine.context import Lane, StaticStep, lower_lanes
+    rng = random.Random(100 + seed)
+    cache = make(capacity=2400, page=rng.choice([4, 8, 16]), requests=6, window=rng.choice([None, 40]))
+    lane_cap, token_cap = rng.choice([(4, 96), (8, 200), (2, 64), (4, 33)])
+    want_cap = rng.choice([lane_cap, token_cap])
+    static = StaticStep(cache, lane_cap, 512, "cpu", query_tile=16, chunk_sizes=(8, 32), tokens=token_cap, wants=want_cap)
+    assert static.context.lane_lengths is None and static.context.num_tokens == token_cap
+    assert static.context.num_lanes == lane_cap and static.context.max_query_len == token_cap
+    addresses = [static.context.token_ids.data_ptr(), static.context.query_tiles.data_ptr(),
+                 static.context.chunk_tables[8].chunks.data_ptr(), static.context.block_tables[0].data_ptr()]
+    names = ["a", "b", "c", "d", "e"]
+    for name in names:
+        cache.add_request(name)
+        grown = rng.randrange(0, 90)
+        if grown:
+            cache.reserve([(name, grown)])
+            cache.commit(name, grown)
+    for fill in range(6):
+        count = rng.randrange(1, lane_cap + 1)
+        picked = rng.sample(names, min(count, len(names)))
+        room = token_cap - (lane_cap - len(picked))                   # every padding lane holds a token at least
+        lanes = []
+        for index, name in enumerate(picked):
+            most = room - sum(len(tokens) for _, tokens, _ in lanes) - (len(picked) - index - 1)
+            length = rng.randrange(1, max(2, min(most, 70) + 1)) if most > 1 else 1
+            if len(picked) == lane_cap and index == len(picked) - 1:
+                length = token_cap - sum(len(tokens) for _, tokens, _ in lanes)    # no padding lane: the capacity is met exactly
+            tokens = [rng.randrange(0, 1000) for _ in range(length)]
+            wanted = sorted(rng.sample(range(length), 1)) if index < want_cap else []
+            lanes.append((name, tokens, wanted))
+        if len(picked) == lane_cap and lanes[-1][1] == []:
+            continue
+        total = sum(len(tokens) for _, tokens, _ in lanes)
+        if not StaticStep.fits(lane_cap, token_cap, len(lanes), total) or any(len(tokens) < 1 for _, tokens, _ in lanes):
+            continue
+        cache.reserve([(name, len(tokens)) for name, tokens, _ in lanes])
+        static.fill(lower_lanes([Lane(*lane) for lane in lanes], cache))
+        pads = lane_cap - len(lanes)
+        pad_lengths = [1] * (pads - 1) + [token_cap - total - (pads - 1)] if pads else []
+        want = plain_packing(cache, lanes, pad_lengths, static.max_pages)
+        lengths = [len(tokens) for _, tokens, _ in lanes] + pad_lengths
+        first = [sum(lengths[:index]) for index in range(len(lengths) + 1)]
+        tiles = [[index, row] for index in range(len(lengths)) for row in range(first[index], first[index + 1], 16)]
+        tile_cap = -(-token_cap // 16) + lane_cap
+        want["query_tiles"] = tiles + [[-1, 0]] * (tile_cap - len(tiles))
+        want["want_rows"] = want["want_rows"] + [0] * (want_cap - len(want["want_rows"]))
+        for field, value in want.items():
+            got = getattr(static.context, field)
+            got = [item.tolist() for item in got] if isinstance(got, list) else got.tolist()
+            assert got == value, field
+        for size in (8, 32):
+            table = static.context.chunk_tables[size]
+            chunks, lane_chunks = plain_chunks(lengths, size)
+            cap = -(-token_cap // size) + lane_cap
+            assert table.num_chunks == cap and table.lane_chunks.view(-1, 2).tolist() == lane_chunks
+            assert table.chunks.view(-1, 4).tolist() == chunks + [[-1, 0, 0, 1]] * (cap - len(chunks))
+        assert addresses == [static.context.token_ids.data_ptr(), static.context.query_tiles.data_ptr(),
+                             static.context.chunk_tables[8].chunks.data_ptr(), static.context.block_tables[0].data_ptr()]
+        for name, tokens, _ in lanes:
+            cache.commit(name, len(tokens))
+    with pytest.raises(ValueError, match="do not fit"):
+        cache.reserve([("a", token_cap + 1)])
+        static.fill(lower_lanes([Lane("a", [1] * (token_cap + 1), [])], cache))
+    assert StaticStep.fits(4, 96, 4, 96) and StaticStep.fits(4, 96, 2, 94) and not StaticStep.fits(4, 96, 2, 95)
+    assert not StaticStep.fits(4, 96, 4, 95) and not StaticStep.fits(4, 96, 5, 96)
+
+
 @pytest.mark.parametrize("decode_only", [False, True])
 @pytest.mark.parametrize("seed", range(5))
 def test_the_cores_packing_of_a_step_matches_a_plain_packing(seed, decode_only):
@@ -266,8 +349,13 @@ def test_the_cores_packing_of_a_step_matches_a_plain_packing(seed, decode_only):
             got = [item.tolist() for item in got] if isinstance(got, list) else got.tolist()
             assert got == value, field
 
-    context = build_step_context(step_lanes, cache, "cpu", query_tile=TILE)
+    context = build_step_context(step_lanes, cache, "cpu", query_tile=TILE, chunk_sizes=(8, 48))
     compare(context, plain_packing(cache, lanes, [], None))
+    for size in (8, 48):                                            # every lane cut into chunks from its first token
+        table = context.chunk_tables[size]
+        chunks, lane_chunks = plain_chunks([len(tokens) for _, tokens, _ in lanes], size)
+        assert table.chunks.view(-1, 4).tolist() == chunks and table.lane_chunks.view(-1, 2).tolist() == lane_chunks
+        assert (table.num_chunks, table.num_lanes, table.num_tokens) == (len(chunks), len(lanes), context.num_tokens)
     assert context.max_seq_len == max(cache.requests[name].length + len(tokens) for name, tokens, _ in lanes)
     assert context.lane_starts == [cache.requests[name].length for name, _, _ in lanes]
     if all(len(tokens) == 1 for _, tokens, _ in lanes):            # a captured decode step: padded, fixed width

@@ -470,13 +470,13 @@ def test_replays_that_follow_one_another_without_a_wait_keep_their_own_arrays(tm
     for engine in (with_graphs, eager):
         for key in names:
             engine.add_request(key)
-    # the shape (one lane of 64 tokens, nothing wanted) comes three times and is captured
+    # a step of this size (one lane of 64 tokens) comes again and its capacity is captured
     plan = [("a", 0), ("b", 0), ("c", 0)]
     busy = [("a", 64), ("b", 64), ("c", 64), ("d", 0), ("e", 0), ("a", 128), ("d", 64), ("e", 64)]
     for key, first in plan:
         for engine in (with_graphs, eager):
             assert engine.step([Lane(key, streams[key][first:first + 64], [])]).shape[0] == 0
-    assert with_graphs.graphs.counts["portion_captures"] == 1
+    assert with_graphs.graphs.counts["bucket_captures"] == 1 and with_graphs.graphs.counts["bucket_replays"] == 2
     ballast = torch.randn(4096, 4096, device=DEV, dtype=torch.bfloat16)
     for engine in (with_graphs, eager):
         torch.cuda.synchronize()
@@ -484,7 +484,7 @@ def test_replays_that_follow_one_another_without_a_wait_keep_their_own_arrays(tm
             ballast @ ballast
         for key, first in busy:
             engine.step([Lane(key, streams[key][first:first + 64], [])])
-    assert with_graphs.graphs.counts["portion_replays"] == 1 + len(busy)
+    assert with_graphs.graphs.counts["bucket_replays"] == 2 + len(busy)
     # decoded tokens, every request in a step of its own with nothing wanted, then all at once with their logits
     cursor = {"a": 192, "b": 128, "c": 128, "d": 128, "e": 128}
     for engine in (with_graphs, eager):
@@ -505,10 +505,10 @@ def test_replays_that_follow_one_another_without_a_wait_keep_their_own_arrays(tm
 
 @pytest.mark.parametrize("name, dtype", [("B", "float32"), ("C", "bfloat16")])
 def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
-    """Steps of one shape (two prompt portions of 70 and 40 tokens, some places wanted) come back:
-    from the third time on they are replayed from a captured graph.  Every step, through pages
-    that are given back and used again and with a decode replay between, is compared with an
-    engine without graphs."""
+    """Steps with prompt portions run from graphs captured for a capacity (so many tokens in so many lanes):
+    portions of 70 and 40 tokens and of 60 and 40 meet the graph of 112 tokens in 4 lanes from their second
+    sighting on, a portion of 10 tokens the one of 16 tokens in 2 lanes, portions beside decoded tokens one more.  Every step, through pages that are given back and
+    used again and with decode replays between, is compared with an engine without graphs."""
     from macllm_infer_amd import Engine, Lane
     folder = tiny_configs.make_model_dir(name, tmp_path, torch.float32 if dtype == "float32" else torch.bfloat16)
     cfg, _ = plain_impl.load_model_dir(folder)
@@ -530,13 +530,15 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
             engine.add_request(a)
             engine.add_request(b)
         first = [Lane(a, tokens_a[:70], [3, 69]), Lane(b, tokens_b[:40], [39])]
-        both(first if round_index % 2 == 0 else first[::-1])      # the order of the lanes does not make another shape
-        both([Lane(a, tokens_a[70:140], [3, 69]), Lane(b, tokens_b[40:80], [39])])      # same shape, later positions
+        both(first if round_index % 2 == 0 else first[::-1])
+        both([Lane(a, tokens_a[70:130], [3, 59]), Lane(b, tokens_b[40:80], [39])])      # other lengths, the same capacity
+        both([Lane(a, tokens_a[130:140], [9])])                                           # a capacity of its own (16 tokens)
         both([Lane(a, tokens_a[140:], [0]), Lane(b, tokens_b[80:], [0])])                 # a decode replay between
         for engine in (with_graphs, eager):
             engine.finish(a)
             engine.finish(b)
-    assert len(with_graphs.graphs._portion_graphs) == 1
+    assert sorted(key[:2] for key in with_graphs.graphs._bucket_graphs) == [(2, 16), (4, 112)]
+    assert with_graphs.graphs.counts["bucket_eager"] == 2 and with_graphs.graphs.counts["bucket_replays"] == 10
     assert with_graphs.cache.stats() == eager.cache.stats()
     # decoded tokens beside a portion: three, then four single-token lanes share one graph (padded to four)
     for engine in (with_graphs, eager):
@@ -551,20 +553,21 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
         return Lane(key, tokens, want)
 
     both([lane(key, 5, [4]) for key in "pqrs"])
-    replays = with_graphs.graphs.counts["portion_replays"]
+    replays = with_graphs.graphs.counts["bucket_replays"]
     for turn in range(6):
         singles = "pqr" if turn < 3 else "pqrs"
         lanes = [lane(key, 1, [0]) for key in singles] + [lane("t", 64, [63] if turn == 5 else [])]
         both(lanes if turn % 2 == 0 else lanes[::-1])
-    assert len(with_graphs.graphs._portion_graphs) == 2
-    assert with_graphs.graphs.counts["portion_replays"] == replays + 3      # turns 2, 3 and 4
+    # three or four decoded tokens beside a portion of 64: 80 tokens in 8 lanes, whatever their order
+    assert (8, 80) in [key[:2] for key in with_graphs.graphs._bucket_graphs]
+    assert with_graphs.graphs.counts["bucket_replays"] == replays + 5
 
 
 @pytest.mark.parametrize("name", ["C", "D"])
 def test_long_portions_overlap_their_mixers(tmp_path, name):
     """Portions of 256 tokens and more run attention on a second stream beside the state-space
-    chain (with the conv inside the chunked scan): a prompt of 300 tokens beside one of 259, eagerly
-    and, from the third step of that shape on, from a captured graph; then the same requests go on
+    chain (with the conv inside the chunked scan): a prompt of 300 tokens beside one of 259, launched kernel
+    by kernel and, from the second step of that size on, from a captured graph; then the same requests go on
     with a portion and a decoded token.  Every wanted row against the plain model."""
     from macllm_infer_amd import Engine, Lane
     from macllm_infer_amd.parts import fused
@@ -595,7 +598,7 @@ def test_long_portions_overlap_their_mixers(tmp_path, name):
         check(logits[1:], want_b[[259]])
         engine.finish(a)
         engine.finish(b)
-    assert engine.graphs.counts["portion_replays"] >= 2
+    assert engine.graphs.counts["bucket_replays"] >= 5
 
 
 @pytest.mark.parametrize("padding", [False, True])
@@ -736,10 +739,10 @@ def test_layers_of_the_benchmark_shapes_match_the_plain_model(shape, layers, voc
     rows = {name: [] for name in prompts}
     for name in prompts:
         engine.add_request(name)
-    # the same shape (300 tokens, last place wanted) three times: launched, launched, captured and replayed
+    # steps of one size (300 tokens, last place wanted) three times: launched, captured and replayed, replayed
     for name, first in (("long", 0), ("third", 0), ("long", 300)):
         rows[name].append(engine.step([Lane(name, prompts[name][first:first + 300], [299])]).cpu())
-    assert engine.graphs.counts["portion_captures"] == 1 and engine.graphs.counts["portion_replays"] == 1
+    assert engine.graphs.counts["bucket_captures"] == 1 and engine.graphs.counts["bucket_replays"] == 2
     mixed = engine.step([Lane("long", prompts["long"][600:637], [36]), Lane("short", prompts["short"][:45], [0, 44])]).cpu()
     rows["long"].append(mixed[:1])
     rows["short"].append(mixed[1:])
