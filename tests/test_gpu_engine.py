@@ -563,6 +563,66 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
     assert with_graphs.graphs.counts["bucket_replays"] == replays + 5
 
 
+@pytest.mark.parametrize("name, dtype, seed", [("B", "float32", 0), ("C", "bfloat16", 1), ("A", "bfloat16", 2)])
+def test_steps_of_any_shape_through_graphs_of_a_capacity_match_eager_steps(tmp_path, name, dtype, seed):
+    """Sixty steps drawn at random (one to five lanes, portions of 2 to 90 tokens beside decoded tokens, wanted
+    places anywhere or nowhere, requests that end and begin) through an engine with graphs, some of them
+    captured before the first request, beside an engine that launches every step kernel by kernel: the same
+    logits and the same cache accounting, whichever way a step went (a capacity's first sighting is launched,
+    later ones replay its graph), and a step whose capacity was warmed up replays at once."""
+    import random
+    from macllm_infer_amd import Engine, Lane
+    folder = tiny_configs.make_model_dir(name, tmp_path, torch.float32 if dtype == "float32" else torch.bfloat16)
+    cfg, _ = plain_impl.load_model_dir(folder)
+    make = lambda graphs: Engine(folder, dtype=dtype, kv_cache_block_tokens=8, kv_cache_capacity_tokens=3000,
+                                 max_active_sequences=6, decode_graphs=graphs)
+    with_graphs, eager = make(True), make(False)
+    captured = with_graphs.warm_up([(1, 1), (4, 4), (1, 40), (2, 100), (3, 130), (5, 200)])
+    assert len(captured) == 6 and with_graphs.graphs.counts["bucket_replays"] == 0
+    first = tokens_for(cfg["vocab_size"], 100, 2999)
+    for engine in (with_graphs, eager):
+        engine.add_request("warm")
+        engine.add_request("warmer")
+    lanes = [Lane("warm", first[:63], [62]), Lane("warmer", first[63:], [0])]
+    got, want = with_graphs.step(lanes).float().cpu(), eager.step(lanes).float().cpu()
+    assert with_graphs.graphs.counts["bucket_replays"] == 1 and with_graphs.graphs.counts["bucket_eager"] == 0
+    assert (got - want).abs().max() <= (1e-5 if dtype == "float32" else 3e-2) * max(1.0, want.abs().max().item())
+    for engine in (with_graphs, eager):
+        engine.finish("warm")
+        engine.finish("warmer")
+    rng = random.Random(seed)
+    live, serial = {}, 0
+    for step in range(60):
+        while len(live) < 5 and (len(live) < 2 or rng.random() < 0.3):
+            live[f"r{serial}"] = [tokens_for(cfg["vocab_size"], rng.randrange(20, 260), 3000 + serial), 0]
+            serial += 1
+            for engine in (with_graphs, eager):
+                engine.add_request(f"r{serial - 1}")
+        picked = rng.sample(sorted(live), rng.randrange(1, len(live) + 1))
+        lanes = []
+        for key in picked:
+            tokens, cursor = live[key]
+            count = min(len(tokens) - cursor, 1 if rng.random() < 0.4 else rng.randrange(2, 91))
+            want = sorted(rng.sample(range(count), rng.randrange(0, min(count, 3) + 1)))
+            lanes.append(Lane(key, tokens[cursor:cursor + count], want))
+            live[key][1] += count
+        got, want = with_graphs.step(lanes).float().cpu(), eager.step(lanes).float().cpu()
+        assert got.shape == want.shape
+        if want.numel():
+            scale = max(1.0, want.abs().max().item())
+            assert (got - want).abs().max() <= (1e-5 if dtype == "float32" else 3e-2) * scale, f"step {step}"
+        for key in picked:
+            if live[key][1] == len(live[key][0]):
+                del live[key]
+                for engine in (with_graphs, eager):
+                    engine.finish(key)
+        assert with_graphs.cache.stats() == eager.cache.stats()
+    counts = with_graphs.graphs.counts
+    assert counts["bucket_eager"] + counts["bucket_replays"] + counts["decode_replays"] == 61
+    assert counts["bucket_replays"] >= 12 and counts["bucket_captures"] >= 8
+    with_graphs.cache.check()
+
+
 @pytest.mark.parametrize("name", ["C", "D"])
 def test_long_portions_overlap_their_mixers(tmp_path, name):
     """Portions of 256 tokens and more run attention on a second stream beside the state-space
