@@ -107,6 +107,12 @@ class Engine:
         longest context the steps' requests will hold.  Returns what was captured; nothing without graphs."""
         return self.graphs.warm_up(steps, context) if self.graphs is not None else []
 
+    def step_token_target(self, lanes: int, tokens: int) -> int:
+        """How many tokens (at most ``tokens``) a step of ``lanes`` lanes should hold if whoever makes it is free
+        to cut a prompt portion shorter: the size at which the step fills the capacity of a captured graph
+        instead of padding the next larger one."""
+        return self.graphs.token_target(lanes, tokens) if self.graphs is not None else tokens
+
     # ------------------------------------------------------------------ requests
     def add_request(self, request: Hashable) -> None:
         """Make ``request`` live: a zeroed state slot and empty block tables."""

@@ -90,6 +90,22 @@ class DecodeGraphs:
             lane_cap <<= 1
         return None
 
+    def token_target(self, lanes: int, tokens: int) -> int:
+        """For a scheduler that is free to cut a prompt portion shorter: the largest number of tokens, at most
+        ``tokens``, with which a step of ``lanes`` lanes fills a capacity but for one token in each padding
+        lane (``tokens`` itself when nothing within an eighth below it does)."""
+        if lanes >= tokens or tokens > self.BUCKET_MOST_TOKENS:
+            return tokens
+        lane_cap = bucket_for(lanes)
+        best = 0
+        for cap in (lane_cap, lane_cap << 1):
+            pads = cap - lanes
+            for token_cap in token_capacities(tokens + cap):
+                fill = token_cap - pads
+                if lanes < fill <= tokens and (pads > 0 or fill == token_cap):
+                    best = max(best, fill)
+        return best if best >= tokens - tokens // 8 else tokens
+
     def run_bucket(self, lanes: Sequence[Lane], lowered: LoweredLanes) -> Optional[torch.Tensor]:
         """Logits of a step with prompt portions from the captured graph of its capacity, or None when that
         capacity has no graph (yet): the caller then launches the step kernel by kernel."""

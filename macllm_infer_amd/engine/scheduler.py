@@ -163,6 +163,22 @@ class Scheduler:
                 samples = True
             budget -= len(tokens)
             visits.append((request, tokens, samples))
+        return self._trim(visits)
+
+    def _trim(self, visits: List[tuple]) -> List[tuple]:
+        """An engine that runs steps of certain sizes best says so (``step_token_target``): a portion that does
+        not end its prompt anyway is cut shorter by the few tokens that make the step such a size."""
+        target = getattr(self.engine, "step_token_target", None)
+        if target is None or not visits:
+            return visits
+        total = sum(len(tokens) for _, tokens, _ in visits)
+        for index in range(len(visits) - 1, -1, -1):
+            request, tokens, samples = visits[index]
+            if request.prefilling and not samples and len(tokens) > 1:
+                spare = total - int(target(len(visits), total))
+                if 0 < spare < len(tokens):
+                    visits[index] = (request, tokens[:len(tokens) - spare], False)
+                break
         return visits
 
     def _finish(self, request: Request, reason: str, release: bool = True) -> None:

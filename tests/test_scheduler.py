@@ -220,3 +220,30 @@ def test_the_callers_own_stop_condition_ends_a_request_after_the_token():
     scheduler.submit("a", [4], SamplingParams(max_new_tokens=10, temperature=0.0))
     finished = scheduler.run()
     assert finished["a"].generated == [5, 6, 7] and finished["a"].finish_reason == "stop"
+
+
+def test_a_portion_that_does_not_end_its_prompt_is_cut_to_the_size_the_engine_prefers():
+    """An engine whose steps run best at certain sizes says so; the scheduler then cuts a portion that would be
+    cut anyway a few tokens shorter, never one that ends its prompt, never below one token, and the tokens it
+    left come with the next portion."""
+    class Sized(FakeEngine):
+        max_context = 400
+
+        def step_token_target(self, lanes, tokens):
+            return tokens - tokens % 16 if tokens - tokens % 16 > lanes else tokens      # multiples of 16
+
+    engine = Sized()
+    prompt = [index % 50 for index in range(100)]
+    params = SamplingParams(max_new_tokens=3, temperature=0.0)
+    config = EngineConfig(max_active_sequences=2, scheduler_token_budget=45, prefill_token_quantum=40)
+    engine, scheduler, finished = run([[7, 8, 9], prompt], params, config, engine)
+    steps = [[(request, len(tokens)) for request, tokens, _, _ in call] for call in engine.calls]
+    # round 1: the short prompt whole (it ends: untouched) beside 40 of the long one: 43 tokens -> 32
+    assert steps[0] == [(0, 3), (1, 29)]
+    # round 2: a decoded token beside a portion of 40: 41 -> 32
+    assert steps[1] == [(0, 1), (1, 31)]
+    # round 3: the last 40 tokens end the prompt: not cut, although 41 is no preferred size
+    assert steps[2] == [(0, 1), (1, 40)] and engine.calls[2][1][3] == [39]
+    assert sum(count for step in steps[:3] for request, count in step if request == 1) == 100
+    assert finished[1].generated == [(prompt[-1] + 1) % 50, (prompt[-1] + 2) % 50, (prompt[-1] + 3) % 50]
+    assert finished[0].generated == [10, 11, 12]
