@@ -113,112 +113,191 @@ extern "C" int mi_rope_kv_store(void* qkv, int dtype, long ld, int T, int Hq, in
 }
 
 // ---------------------------------------------------------------- paged attention, any size
-// One wavefront per (token, query head).  Keys are taken 64 at a time: lane i scores key i
-// (full dot product over dh from its own cache row), the wave keeps the running maximum
-// and normalizer in float32 (online softmax), and for the value product lane i owns output
-// dims i, i+64, ...  Works for any head_dim <= 256, any page size, any group size.
+// Works for any head_dim <= 256, any page size, any group size, float32 and bfloat16; the float32 path of
+// the whole model uses it for prompts and for decoding alike.
 //   s = q.k * scale;  visible keys: position <= query position, and
 //   query - key < window when window > 0 (reference: src/decoder.rs:4515-4532);
 //   softmax in float32 (reference: src/decoder.rs:4665-4667).
+// The keys are cut into runs of PA_RUN by their absolute position.  One workgroup per (token, query head,
+// run): each of its four waves takes 64 keys of the run (lane i scores key i with a full dot product over
+// dh from its own cache row; for the value product lane i owns output dims i, i + 64, ...), keeps
+// (maximum, normalizer, sums) in float32, the waves are merged through LDS in their order and the workgroup
+// leaves one partial result; a second kernel merges the runs in ascending order (the (maximum, normalizer,
+// accumulator) merge the reference does across simdgroups, crates/macllm-kernels/src/metal/paged_decode.metal:145-183).
+// Which keys meet in a wave, and the order of every sum, depend on the query's position alone: a token's
+// result is bit for bit the same whatever else the step holds and however long the longest context is.
 #define ATT_MAX_DH 256
+#define PA_RUN 256
+#define PA_WAVES (PA_RUN / WAVE)
 
 template <typename T, bool FAST_EXP>
-__global__ void __launch_bounds__(WAVE)
+__global__ void __launch_bounds__(PA_RUN)
 paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int dh,
                        const T* __restrict__ k_base, const T* __restrict__ v_base, long page_stride,
                        int page_size, const int* __restrict__ block_tables, int max_pages,
                        const int* __restrict__ lane_of_token, const int* __restrict__ positions, float scale,
-                       int window, T* __restrict__ out, long out_ld) {
-  __shared__ float q_shared[ATT_MAX_DH];
-  __shared__ float p_shared[WAVE];
-  __shared__ long row_shared[WAVE];      // base of the key's (page, kv head) block
-  __shared__ int offset_shared[WAVE];    // the key's place inside its page
+                       int window, int runs, float* __restrict__ partial) {
+  typedef T vec4 __attribute__((ext_vector_type(4)));
+  __shared__ __align__(16) float q_shared[ATT_MAX_DH];
+  __shared__ float p_shared[PA_WAVES][WAVE];
+  __shared__ long row_shared[PA_WAVES][WAVE];     // base of the key's (page, kv head) block
+  __shared__ int offset_shared[PA_WAVES][WAVE];   // the key's place inside its page
+  __shared__ float wave_ml[PA_WAVES][2];
+  __shared__ float wave_o[PA_WAVES][ATT_MAX_DH];
   const long token = blockIdx.x;
   const int head = blockIdx.y;
-  const int kvh = head / (Hq / Hkv);
-  const int lane = threadIdx.x;
-  const int request = lane_of_token[token];
+  const int run = blockIdx.z;
   const int query_position = positions[token];
-  const int* table = block_tables + (long)request * max_pages;
-  const T* q_row = q + token * q_ld + (long)head * dh;
-  for (int i = lane; i < dh; i += WAVE) q_shared[i] = to_float(q_row[i]);
-  __syncthreads();
-
   int first_key = 0;
   if (window > 0 && query_position - window + 1 > 0) first_key = query_position - window + 1;
-  const int last_key = query_position;     // inclusive
+  if ((run + 1) * PA_RUN <= first_key || run * PA_RUN > query_position) return;   // no key of this run is visible
+  const int kvh = head / (Hq / Hkv);
+  const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  const int* table = block_tables + (long)lane_of_token[token] * max_pages;
+  const T* q_row = q + token * q_ld + (long)head * dh;
+  for (int i = tid; i < dh; i += PA_RUN) q_shared[i] = to_float(q_row[i]);
+  __syncthreads();
 
-  float running_max = -INFINITY;
-  float running_sum = 0.f;
-  float acc[ATT_MAX_DH / WAVE];
+  const int key = run * PA_RUN + wave * WAVE + lane;
+  const bool visible = key >= first_key && key <= query_position;
+  float score = -INFINITY;
+  long row_offset = 0;
+  int offset = 0;
+  if (visible) {
+    const int page = table[key / page_size];
+    offset = key % page_size;
+    row_offset = (long)page * page_stride + (long)kvh * page_size * dh;
+    const T* k_row = k_base + row_offset + (long)offset * dh;
+    float dot = 0.f;
+    if (dh % 4 == 0 && page_stride % 4 == 0 && ((unsigned long long)k_base % (4 * sizeof(T))) == 0) {
+      for (int i = 0; i < dh; i += 4) {
+        const vec4 piece = *reinterpret_cast<const vec4*>(k_row + i);
 #pragma unroll
-  for (int i = 0; i < ATT_MAX_DH / WAVE; ++i) acc[i] = 0.f;
-
-  for (int base = first_key; base <= last_key; base += WAVE) {
-    const int key = base + lane;
-    float score = -INFINITY;
-    long row_offset = 0;
-    int offset = 0;
-    if (key <= last_key) {
-      const int page = table[key / page_size];
-      offset = key % page_size;
-      row_offset = (long)page * page_stride + (long)kvh * page_size * dh;
-      const T* k_row = k_base + row_offset + (long)offset * dh;
-      float dot = 0.f;
-      for (int i = 0; i < dh; ++i) dot += q_shared[i] * to_float(k_row[i]);
-      score = dot * scale;
-    }
-    const float block_max = wave_max(score);
-    const float new_max = fmaxf(running_max, block_max);
-    const float correction = FAST_EXP ? __expf(running_max - new_max) : expf(running_max - new_max);
-    const float p = (key <= last_key) ? (FAST_EXP ? __expf(score - new_max) : expf(score - new_max)) : 0.f;
-    running_sum = running_sum * correction + wave_sum(p);
-    running_max = new_max;
-    __syncthreads();
-    p_shared[lane] = p;
-    row_shared[lane] = row_offset;
-    offset_shared[lane] = offset;
-    __syncthreads();
-    const int valid = min(WAVE, last_key - base + 1);
-#pragma unroll
-    for (int i = 0; i < ATT_MAX_DH / WAVE; ++i) {
-      const int dim = lane + i * WAVE;
-      if (dim < dh) {
-        float sum = acc[i] * correction;
-        for (int j = 0; j < valid; ++j)
-          sum += p_shared[j] * to_float(v_base[row_shared[j] + (long)dim * page_size + offset_shared[j]]);
-        acc[i] = sum;
+        for (int j = 0; j < 4; ++j) dot += q_shared[i + j] * to_float<T>(piece[j]);
       }
+    } else {
+      for (int i = 0; i < dh; ++i) dot += q_shared[i] * to_float(k_row[i]);
     }
+    score = dot * scale;
   }
-  T* o = out + token * out_ld + (long)head * dh;
+  const float maximum = wave_max(score);                    // -inf for a wave without visible keys
+  const float p = visible ? (FAST_EXP ? __expf(score - maximum) : expf(score - maximum)) : 0.f;
+  const float normalizer = wave_sum(p);
+  p_shared[wave][lane] = p;
+  row_shared[wave][lane] = row_offset;
+  offset_shared[wave][lane] = offset;
+  if (lane == 0) {
+    wave_ml[wave][0] = maximum;
+    wave_ml[wave][1] = normalizer;
+  }
+  __syncthreads();
+  const int wave_first = run * PA_RUN + wave * WAVE;
+  const int from = min(WAVE, max(0, first_key - wave_first));
+  const int to = min(WAVE, max(0, query_position - wave_first + 1));
 #pragma unroll
   for (int i = 0; i < ATT_MAX_DH / WAVE; ++i) {
     const int dim = lane + i * WAVE;
-    if (dim < dh) o[dim] = from_float<T>(acc[i] / running_sum);
+    if (dim < dh) {
+      float sum = 0.f;
+      for (int j = from; j < to; ++j)
+        sum += p_shared[wave][j] * to_float(v_base[row_shared[wave][j] + (long)dim * page_size + offset_shared[wave][j]]);
+      wave_o[wave][dim] = sum;
+    }
   }
+  __syncthreads();
+  // the waves in their order; a wave without keys has the weight exp(-inf) = 0
+  float best = wave_ml[0][0];
+#pragma unroll
+  for (int w = 1; w < PA_WAVES; ++w) best = fmaxf(best, wave_ml[w][0]);
+  float* mine = partial + ((token * Hq + head) * runs + run) * (long)(dh + 2);
+  float weight[PA_WAVES];
+  float denominator = 0.f;
+#pragma unroll
+  for (int w = 0; w < PA_WAVES; ++w) {
+    weight[w] = FAST_EXP ? __expf(wave_ml[w][0] - best) : expf(wave_ml[w][0] - best);
+    denominator += weight[w] * wave_ml[w][1];
+  }
+  if (tid == 0) {
+    mine[0] = best;
+    mine[1] = denominator;
+  }
+  for (int dim = tid; dim < dh; dim += PA_RUN) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < PA_WAVES; ++w) sum += weight[w] * wave_o[w][dim];
+    mine[2 + dim] = sum;
+  }
+}
+
+template <typename T, bool FAST_EXP>
+__global__ void paged_attention_merge_kernel(const float* __restrict__ partial, int Hq, int dh, int runs,
+                                             const int* __restrict__ positions, int window,
+                                             T* __restrict__ out, long out_ld) {
+  const long token = blockIdx.x;
+  const int head = blockIdx.y;
+  const int query_position = positions[token];
+  int first_key = 0;
+  if (window > 0 && query_position - window + 1 > 0) first_key = query_position - window + 1;
+  const int first_run = first_key / PA_RUN;
+  const int last_run = query_position / PA_RUN;
+  const float* theirs = partial + ((token * Hq + head) * runs) * (long)(dh + 2);
+  for (int dim = threadIdx.x; dim < dh; dim += blockDim.x) {
+    float maximum = -INFINITY, denominator = 0.f, sum = 0.f;
+    for (int run = first_run; run <= last_run; ++run) {
+      const float* one = theirs + (long)run * (dh + 2);
+      const float larger = fmaxf(maximum, one[0]);
+      const float keep = FAST_EXP ? __expf(maximum - larger) : expf(maximum - larger);     // 0 the first time
+      const float weight = FAST_EXP ? __expf(one[0] - larger) : expf(one[0] - larger);
+      denominator = denominator * keep + weight * one[1];
+      sum = sum * keep + weight * one[2 + dim];
+      maximum = larger;
+    }
+    out[token * out_ld + (long)head * dh + dim] = from_float<T>(sum / denominator);
+  }
+}
+
+// partial: work area of at least T * Hq * runs * (dh + 2) floats, runs = ceil(max_seq_len / PA_RUN), where
+// max_seq_len bounds the number of keys (position + 1) of every token of the step.
+extern "C" long mi_paged_attention_workspace(int T, int Hq, int dh, int max_seq_len) {
+  if (T <= 0 || Hq <= 0 || dh <= 0 || max_seq_len <= 0) return 0;
+  return (long)T * Hq * ((max_seq_len + PA_RUN - 1) / PA_RUN) * (dh + 2);
 }
 
 extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, int Hq, int Hkv, int dh,
                                   const void* k_base, const void* v_base, long page_stride, int page_size,
                                   const int* block_tables, int max_pages, const int* lane_of_token,
-                                  const int* positions, float scale, int window, void* out, long out_ld,
+                                  const int* positions, float scale, int window, int max_seq_len,
+                                  float* partial, long partial_floats, void* out, long out_ld,
                                   hipStream_t stream) {
-  if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || dh <= 0 || page_size <= 0 || max_pages <= 0)
+  if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || dh <= 0 || page_size <= 0 || max_pages <= 0 ||
+      max_seq_len <= 0 || !partial)
     return ERR_BAD_ARGUMENT;
   if (dh > ATT_MAX_DH) return ERR_UNSUPPORTED_SIZE;
-  if (Hq > 65535) return ERR_UNSUPPORTED_SIZE;
-  const dim3 grid(T, Hq);
-  if (dtype == DT_F32)
-    paged_attention_kernel<float, false><<<grid, WAVE, 0, stream>>>(
+  const int runs = (max_seq_len + PA_RUN - 1) / PA_RUN;
+  if (Hq > 65535 || runs > 65535) return ERR_UNSUPPORTED_SIZE;
+  if (partial_floats < mi_paged_attention_workspace(T, Hq, dh, max_seq_len)) return ERR_BAD_ARGUMENT;
+  const dim3 grid(T, Hq, runs);
+  const dim3 merge_grid(T, Hq);
+  const int merge_threads = dh <= WAVE ? WAVE : dh <= 2 * WAVE ? 2 * WAVE : 4 * WAVE;
+  if (dtype == DT_F32) {
+    paged_attention_kernel<float, false><<<grid, PA_RUN, 0, stream>>>(
         (const float*)q, q_ld, Hq, Hkv, dh, (const float*)k_base, (const float*)v_base, page_stride, page_size,
-        block_tables, max_pages, lane_of_token, positions, scale, window, (float*)out, out_ld);
-  else if (dtype == DT_BF16)
-    paged_attention_kernel<bf16_t, true><<<grid, WAVE, 0, stream>>>(
+        block_tables, max_pages, lane_of_token, positions, scale, window, runs, partial);
+    RETURN_IF_LAUNCH_FAILED();
+    paged_attention_merge_kernel<float, false><<<merge_grid, merge_threads, 0, stream>>>(
+        partial, Hq, dh, runs, positions, window, (float*)out, out_ld);
+  } else if (dtype == DT_BF16) {
+    paged_attention_kernel<bf16_t, true><<<grid, PA_RUN, 0, stream>>>(
         (const bf16_t*)q, q_ld, Hq, Hkv, dh, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride,
-        page_size, block_tables, max_pages, lane_of_token, positions, scale, window, (bf16_t*)out, out_ld);
-  else
+        page_size, block_tables, max_pages, lane_of_token, positions, scale, window, runs, partial);
+    RETURN_IF_LAUNCH_FAILED();
+    paged_attention_merge_kernel<bf16_t, true><<<merge_grid, merge_threads, 0, stream>>>(
+        partial, Hq, dh, runs, positions, window, (bf16_t*)out, out_ld);
+  } else {
     return ERR_BAD_ARGUMENT;
+  }
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

@@ -98,14 +98,37 @@ __device__ unsigned long long block_min_key(unsigned long long key, unsigned lon
   return best;
 }
 
+// One workgroup a row.  The row is read in 16-byte pieces, eight of them asked for before the first is
+// used (a row of 130,049 logits is 32 such pieces a thread); the elements before the first aligned piece
+// and behind the last are read one by one (a row starts where the row before it ends, so at any alignment).
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 argmax_kernel(const float* __restrict__ logits, int V, int* __restrict__ out) {
   __shared__ unsigned long long scratch[SAMPLE_THREADS / WAVE];
+  typedef float float4_t __attribute__((ext_vector_type(4)));
   const float* values = logits + (long)blockIdx.x * V;
+  const int head = min(V, (int)((4 - (((unsigned long long)values / sizeof(float)) & 3)) & 3));
+  const int pieces = (V - head) / 4;
   unsigned long long best = ~0ull;
-  for (int v = threadIdx.x; v < V; v += blockDim.x) {
-    const unsigned long long key = rank_key(values[v], v);
+  auto take = [&](float value, int index) {
+    const unsigned long long key = rank_key(value, index);
     best = key < best ? key : best;
+  };
+  if ((int)threadIdx.x < head) take(values[threadIdx.x], threadIdx.x);
+  for (int v = head + 4 * pieces + threadIdx.x; v < V; v += blockDim.x) take(values[v], v);
+  const float4_t* aligned = reinterpret_cast<const float4_t*>(values + head);
+  constexpr int BATCH = 8;
+  for (int first = threadIdx.x; first < pieces; first += BATCH * SAMPLE_THREADS) {
+    float4_t piece[BATCH];
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) piece[j] = aligned[min(first + j * SAMPLE_THREADS, pieces - 1)];
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) {
+      const int at = first + j * SAMPLE_THREADS;
+      if (at < pieces) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) take(piece[j][i], head + 4 * at + i);
+      }
+    }
   }
   best = block_min_key(best, scratch);
   if (threadIdx.x == 0) out[blockIdx.x] = (int)(best & 0xffffffffu);

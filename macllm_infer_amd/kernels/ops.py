@@ -41,7 +41,9 @@ _SIGNATURES = {
         "mi_rope_kv_store": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int,
                              _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr],
         "mi_paged_attention": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
-                               _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_long, _c_ptr],
+                               _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_long,
+                               _c_ptr, _c_long, _c_ptr],
+        "mi_paged_attention_workspace": [_c_int, _c_int, _c_int, _c_int],
         "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
                                  _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_long, _c_ptr],
         "mi_decode_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int,
@@ -99,13 +101,13 @@ _SIGNATURES = {
 _functions = {}
 
 
-def _fn(module: str, name: str):
+def _fn(module: str, name: str, restype=_c_int):
     key = (module, name)
     if key not in _functions:
         library = build.load_module(module)
         function = getattr(library, name)
         function.argtypes = _SIGNATURES[module][name]
-        function.restype = _c_int
+        function.restype = restype
         _functions[key] = function
     return _functions[key]
 
@@ -323,12 +325,14 @@ def _cache_view(k_cache, v_cache, num_kv_heads, head_dim, dtype):
 def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                     k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     lane_of_token: torch.Tensor, positions: torch.Tensor, scale: float,
-                    window: Optional[int], out: torch.Tensor) -> None:
+                    window: Optional[int], out: torch.Tensor, max_seq_len: Optional[int] = None) -> None:
     """Causal attention of every token over its request's cached keys (its own included).
 
     ``q`` [T, >= Hq*dh] (rotated); ``block_tables`` [lanes, max_pages] page ids by logical
     page; a key at position p is visible to a query at position s when p <= s and, with a
-    window w, s - p < w.  ``out`` [T, Hq*dh]."""
+    window w, s - p < w.  ``out`` [T, Hq*dh].  ``max_seq_len``: an upper bound of position + 1 over
+    the step's tokens (what the block tables can hold if it is not given); it sizes the launch and
+    the work area, never the result."""
     q_ld = _row_major(q, "q")
     out_ld = _row_major(out, "out")
     T = q.shape[0]
@@ -340,10 +344,15 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     _i32(positions, "positions")
     _need(block_tables.dim() == 2 and lane_of_token.numel() == T and positions.numel() == T,
           "paged_attention: metadata shapes do not match")
+    holds = block_tables.shape[1] * page_size
+    span = holds if max_seq_len is None else max(1, min(int(max_seq_len), holds))
+    floats = _fn("attention", "mi_paged_attention_workspace", _c_long)(T, num_heads, head_dim, span)
+    partial = torch.empty((max(int(floats), 1),), dtype=torch.float32, device=q.device)
     _check(_fn("attention", "mi_paged_attention")(
         _p(q), _dt(q), q_ld, T, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride,
         page_size, _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale),
-        int(window or 0), _p(out), out_ld, _stream()), "paged_attention", f"(head_dim={head_dim})")
+        int(window or 0), span, _p(partial), partial.numel(), _p(out), out_ld, _stream()), "paged_attention",
+        f"(head_dim={head_dim})")
 
 
 def prefill_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> bool:

@@ -97,4 +97,5 @@ class Attention(Mixer):
                                   attended)
         else:
             ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
-                                step.lane_of_token, step.positions, spec.scale, spec.window, attended)
+                                step.lane_of_token, step.positions, spec.scale, spec.window, attended,
+                                step.max_seq_len)

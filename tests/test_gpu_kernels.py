@@ -108,16 +108,20 @@ def test_swiglu_and_scale(ops, dtype):
     close(logits, gu.float() * 0.6, torch.float32)
 
 
-@pytest.mark.parametrize("shape", [(1, 64, 32), (5, 130, 97), (67, 100, 260), (130, 33, 1000)])
+@pytest.mark.parametrize("shape", [(1, 64, 32), (5, 130, 97), (67, 100, 260), (130, 33, 1000), (40, 70, 3), (200, 257, 708)])
 def test_float32_product_is_true_float32(ops, shape):
     M, N, K = shape
     x, w, b = rand(M, K, seed=6), rand(N, K, seed=7), rand(N, seed=8)
     want = (x.double() @ w.double().T + b.double()).float()
     got = ops.linear(x.to(DEV), w.to(DEV), b.to(DEV))
     assert (got.cpu() - want).abs().max() < 2e-5 * math.sqrt(K)       # float32 rounding only
-    # a row's result does not depend on the rows beside it
-    alone = ops.linear(x[:1].to(DEV), w.to(DEV), b.to(DEV))
-    assert torch.equal(alone[0], got[0])
+    # a row's result does not depend on the rows beside it, nor on the tiling that the number of rows selects
+    for rows in (1, 9, 17, 33, 65):
+        if rows <= M:
+            fewer = ops.linear(x[:rows].to(DEV), w.to(DEV), b.to(DEV))
+            assert torch.equal(fewer, got[:rows]), rows
+    last = ops.linear(x[M - 1:].to(DEV), w.to(DEV), b.to(DEV))
+    assert torch.equal(last[0], got[M - 1])
     # a strided input (a column block of a wider matrix)
     wide = rand(M, K + 24, seed=9)
     got = ops.linear(wide.to(DEV)[:, 8:8 + K], w.to(DEV), None)
@@ -219,7 +223,7 @@ def test_one_far_key_among_hundreds_is_found(ops, dtype, page_size):
     base_keys = rand(length, Hkv, dh, seed=51, scale=0.1, dtype=dtype)
     direction = torch.zeros(dh)
     direction[5] = 1.0
-    for chosen in (0, 1, page_size - 1, page_size, 63, 64, 65, 511, 512, length - 2, length - 1):
+    for chosen in (0, 1, page_size - 1, page_size, 63, 64, 65, 255, 256, 257, 511, 512, length - 2, length - 1):
         keys = base_keys.clone()
         keys[chosen] = (direction * 30.0).to(dtype)
         fill_cache(pool, table, 0, keys, values, page_size)
@@ -256,6 +260,59 @@ def test_window_edge(ops, dtype):
         ref_ops.paged_attention(q.cpu(), Hq, Hkv, dh, *views(pool, page_size), table, i32([0]),
                                 i32([length - 1]), 1.0 / math.sqrt(dh), window, want)
         close(out, want, dtype, 3.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_window_across_the_edge_of_a_run_of_keys(ops, dtype):
+    """The general kernel cuts the keys into runs of 256 by position: a window of 60 at position 299 holds
+    keys 240..299, on both sides of that edge; and one at position 600 of window 300 spans two edges."""
+    Hq, Hkv, dh, page_size = 3, 1, 48, 16
+    for length, window, cases in ((300, 60, ((240, True), (239, False), (255, True), (256, True))),
+                                  (601, 300, ((301, True), (300, False), (511, True), (512, True), (600, True)))):
+        pool, table = paged_setup([length], page_size, Hkv, dh, dtype, seed=14)
+        values = rand(length, Hkv, dh, seed=54, dtype=dtype)
+        direction = torch.zeros(dh)
+        direction[3] = 1.0
+        q = (direction * 30.0).repeat(Hq)[None].to(dtype).to(DEV)
+        for chosen, visible in cases:
+            keys = rand(length, Hkv, dh, seed=55, scale=0.1, dtype=dtype)
+            keys[chosen] = (direction * 30.0).to(dtype)
+            fill_cache(pool, table, 0, keys, values, page_size)
+            dev_pool = pool.to(DEV)
+            out = torch.empty(1, Hq * dh, dtype=dtype, device=DEV)
+            ops.paged_attention(q, Hq, Hkv, dh, *views(dev_pool, page_size), table.to(DEV), i32([0]).to(DEV),
+                                i32([length - 1]).to(DEV), 1.0 / math.sqrt(dh), window, out)
+            hit = (out.float().cpu()[0, :dh] - values[chosen, 0].float()).abs().max() < 1e-2
+            assert hit == visible, f"key {chosen} should be {'visible' if visible else 'masked'}"
+            want = torch.empty(1, Hq * dh, dtype=dtype)
+            ref_ops.paged_attention(q.cpu(), Hq, Hkv, dh, *views(pool, page_size), table, i32([0]),
+                                    i32([length - 1]), 1.0 / math.sqrt(dh), window, want)
+            close(out, want, dtype, 3.0)
+
+
+def test_general_attention_does_not_depend_on_the_step_around_a_token(ops):
+    """float32: a token's attended row is bit for bit the same alone, among the tokens of a prompt portion,
+    beside another request, and whatever bound of the longest context sizes the launch."""
+    Hq, Hkv, dh, page_size = 4, 2, 40, 16
+    lengths = [700, 90]
+    pool, table = paged_setup(lengths, page_size, Hkv, dh, torch.float32, seed=15)
+    for lane, length in enumerate(lengths):
+        fill_cache(pool, table, lane, rand(length, Hkv, dh, seed=56 + lane), rand(length, Hkv, dh, seed=58 + lane), page_size)
+    dev_pool, dev_table = pool.to(DEV), table.to(DEV)
+    positions = i32(list(range(500, 700)) + list(range(60, 90)))
+    lane_of_token = i32([0] * 200 + [1] * 30)
+    q = rand(230, Hq * dh, seed=60).to(DEV)
+    whole = torch.empty(230, Hq * dh, device=DEV)
+    ops.paged_attention(q, Hq, Hkv, dh, *views(dev_pool, page_size), dev_table, lane_of_token.to(DEV),
+                        positions.to(DEV), 0.2, None, whole)
+    want = torch.empty(230, Hq * dh)
+    ref_ops.paged_attention(q.cpu(), Hq, Hkv, dh, *views(pool, page_size), table, lane_of_token, positions, 0.2, None, want)
+    close(whole, want, torch.float32, 3.0)
+    for row, bound in ((0, None), (199, 700), (199, 704), (200, 90), (229, None), (12, 513)):
+        alone = torch.empty(1, Hq * dh, device=DEV)
+        ops.paged_attention(q[row:row + 1], Hq, Hkv, dh, *views(dev_pool, page_size), dev_table,
+                            lane_of_token[row:row + 1].to(DEV), positions[row:row + 1].to(DEV), 0.2, None, alone, bound)
+        assert torch.equal(alone[0], whole[row]), (row, bound)
 
 
 def test_attention_refuses_a_head_size_beyond_its_limit(ops):
@@ -491,6 +548,21 @@ def test_argmax_and_ties(ops):
     ops.argmax(logits.to(DEV), out)
     assert out.cpu().tolist() == torch.argmax(logits, -1).tolist()
     assert out.cpu()[1] == 17 and out.cpu()[2] == 1002
+
+
+@pytest.mark.parametrize("V", [3, 130049, 32784, 8191])
+def test_argmax_of_rows_at_every_alignment(ops, V):
+    """Rows of an odd width start at every alignment of the 16-byte pieces the kernel reads: the best element
+    is put, row by row, at the row's first and last elements, around the first aligned piece and far inside;
+    a tie between two pieces goes to the lower index."""
+    places = sorted({0, 1, 2, 3, 4, 5, V // 2, V - 5, V - 4, V - 3, V - 2, V - 1} & set(range(V)))
+    logits = rand(len(places) + 1, V, seed=81)
+    for row, place in enumerate(places):
+        logits[row, place] = 50.0
+    logits[-1, V - 1] = logits[-1, V // 3] = 60.0
+    out = torch.empty(len(places) + 1, dtype=torch.int32, device=DEV)
+    ops.argmax(logits.to(DEV), out)
+    assert out.cpu().tolist() == places + [min(V // 3, V - 1)]
 
 
 @pytest.mark.parametrize("select", [False, True], ids=["sorted", "selected"])
