@@ -6,6 +6,9 @@
 //       prologue  NORM : x = (h + delta0 + delta1) / sqrt(mean(.^2) + eps) * w   (residual add
 //                        and RMSNorm; block 0 also writes the summed residual to h_out)
 //                 PLAIN: x given in bfloat16
+//                 MERGE: x given in bfloat16, but for its first columns, the attended heads, which are
+//                        merged here from the partial results that mixer_decode's runs of keys left
+//                        (what mixer_merge_kernel does in a launch of its own, sum for sum)
 //       epilogue  PLAIN : bfloat16 or float32 (x scale) store
 //                 SWIGLU: rows come in tiles of 8 gate rows + 8 up rows; stores SiLU(g)*u
 //                 CONV  : rows in [conv_lo, conv_hi) are channels of a causal depthwise conv
@@ -34,7 +37,8 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 #define FG_PAD 8
 
-enum { PRO_NORM = 0, PRO_PLAIN = 1 };
+enum { PRO_NORM = 0, PRO_PLAIN = 1, PRO_MERGE = 2 };
+#define MERGE_AT_ONCE 8      // runs of keys asked for at once by a merge (mixer_merge_kernel and the MERGE prologue)
 enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_CONV = 2 };
 
 struct FusedGemmParams {
@@ -59,6 +63,10 @@ struct FusedGemmParams {
   bf16_t* conv_state;
   const int* slot_ids;
   int w_tiled;
+  // MERGE prologue: partial [M, heads, runs, head_dim + 2] = (maximum, normalizer, sums) per run of keys
+  const float* partial;
+  const int* positions;
+  int merge_heads, merge_dh, merge_runs, merge_run_keys, merge_page, merge_window;
 };
 
 __device__ __forceinline__ float round_bf16(float v) { return (float)(bf16_t)v; }
@@ -66,12 +74,14 @@ __device__ __forceinline__ float round_bf16(float v) { return (float)(bf16_t)v; 
 template <int MT, int PRO, int EPI, int FG_WAVES, int NT>
 __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmParams p) {
   static_assert(NT == 1 || PRO == PRO_PLAIN, "several feature tiles a workgroup: plain prologue only");
+  static_assert(PRO != PRO_MERGE || EPI == EPI_PLAIN, "the merge prologue comes with the plain epilogue");
   constexpr int FG_THREADS = FG_WAVES * WAVE;
   extern __shared__ __align__(16) unsigned char smem[];
   const int K = p.K;
-  const int ldx = K + FG_PAD;
+  const int staged = PRO == PRO_NORM ? K : PRO == PRO_MERGE ? p.merge_heads * p.merge_dh : 0;   // columns of x kept in LDS
+  const int ldx = staged + FG_PAD;
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem);
-  float* red = reinterpret_cast<float*>(smem + (PRO == PRO_NORM ? (size_t)MT * 16 * ldx * sizeof(bf16_t) : 0));
+  float* red = reinterpret_cast<float*>(smem + (staged ? (size_t)MT * 16 * ldx * sizeof(bf16_t) : 0));
   float* tile = red + FG_WAVES * MT * 256;
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
@@ -154,6 +164,30 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
         for (int i = 0; i < MAXV; ++i) d1v[tt][i] = *reinterpret_cast<const bf16x4_t*>(p.delta1 + at[tt][i]);
     }
   };
+  // MERGE: an item is 8 dims of one head of one token; its runs' (maximum, normalizer, 8 sums) are asked for
+  // before the weights, MERGE_AT_ONCE runs at once and before it is known how many of them hold keys (the
+  // position is on its way too; what a run without keys left in its place is read and not used)
+  const int merge_items = PRO == PRO_MERGE ? p.M * (staged / 8) : 0;
+  float run_max[MERGE_AT_ONCE], run_norm[MERGE_AT_ONCE];
+  float2 run_sums[MERGE_AT_ONCE][4];
+  int merge_position = 0;
+  auto merge_ask = [&](int item, int first_run) {
+    item = min(item, merge_items - 1);
+    const int token = item / (staged / 8);
+    const int column = (item - token * (staged / 8)) * 8;             // head * dh + dim
+    const int head = column / p.merge_dh;
+    const float* runs = p.partial + ((long)token * p.merge_heads + head) * p.merge_runs * (long)(p.merge_dh + 2);
+    if (first_run == 0) merge_position = p.positions[token];
+#pragma unroll
+    for (int j = 0; j < MERGE_AT_ONCE; ++j) {
+      const float* run = runs + (long)min(first_run + j, p.merge_runs - 1) * (p.merge_dh + 2);
+      run_max[j] = run[0];
+      run_norm[j] = run[1];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) run_sums[j][i] = *reinterpret_cast<const float2*>(run + 2 + (column - head * p.merge_dh) + 2 * i);
+    }
+  };
+  if (PRO == PRO_MERGE) merge_ask(tid, 0);
   if (in_registers) {
     load_pair(0, 0);
 #pragma unroll
@@ -243,6 +277,43 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
     }
     __syncthreads();
   }
+  if (PRO == PRO_MERGE) {
+    // out[token, head, :] = sum_s exp(m_s - m) o_s / sum_s exp(m_s - m) l_s over the runs that hold keys,
+    // in the order and with the roundings of mixer_merge_kernel
+    for (int item = tid; item < merge_items; item += FG_THREADS) {
+      if (item != tid) merge_ask(item, 0);
+      int first_key = 0;
+      if (p.merge_window > 0 && merge_position - p.merge_window + 1 > 0) first_key = merge_position - p.merge_window + 1;
+      const int base_key = (first_key / p.merge_page) * p.merge_page;
+      const int used = min(p.merge_runs, (merge_position - base_key) / p.merge_run_keys + 1);
+      float maximum = -INFINITY, denominator = 0.f, sums[8] = {};
+      for (int s0 = 0; s0 < used; s0 += MERGE_AT_ONCE) {
+        if (s0 > 0) merge_ask(item, s0);
+#pragma unroll
+        for (int j = 0; j < MERGE_AT_ONCE; ++j) {
+          if (s0 + j < used) {
+            const float larger = fmaxf(maximum, run_max[j]);
+            const float keep = __builtin_amdgcn_exp2f(maximum - larger);          // 0 the first time; units of log2
+            const float weight = __builtin_amdgcn_exp2f(run_max[j] - larger);
+            denominator = denominator * keep + weight * run_norm[j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              sums[2 * i] = sums[2 * i] * keep + weight * run_sums[j][i].x;
+              sums[2 * i + 1] = sums[2 * i + 1] * keep + weight * run_sums[j][i].y;
+            }
+            maximum = larger;
+          }
+        }
+      }
+      const int token = item / (staged / 8);
+      const int column = (item - token * (staged / 8)) * 8;
+      bf16x8_t packed;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) packed[i] = (bf16_t)(sums[i] / denominator);
+      *reinterpret_cast<bf16x8_t*>(xs + (long)token * ldx + column) = packed;
+    }
+    __syncthreads();
+  }
 
   // the conv tails of those outputs are asked for now, behind the weights; no branch between the
   // loads either (a row past M reads the last row's tail and is not used)
@@ -288,14 +359,15 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
       }
     }
     bf16x8_t b[BATCH][MT];
-    if (PRO == PRO_PLAIN) {
+    if (PRO == PRO_PLAIN || PRO == PRO_MERGE) {
 #pragma unroll
       for (int j = 0; j < BATCH; ++j) {
         const int c = first_chunk + min(first + j, iterations - 1);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const int m = min(mt * 16 + r, p.M - 1);
-          b[j][mt] = *reinterpret_cast<const bf16x8_t*>(p.x + (long)m * p.x_ld + c * 32 + 8 * q);
+          if (PRO == PRO_MERGE && c * 32 < staged) b[j][mt] = *reinterpret_cast<const bf16x8_t*>(xs + (long)m * ldx + c * 32 + 8 * q);
+          else b[j][mt] = *reinterpret_cast<const bf16x8_t*>(p.x + (long)m * p.x_ld + c * 32 + 8 * q);
         }
       }
     }
@@ -403,9 +475,11 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 
 static int fused_gemm_waves(int K) { return K / 32 > 32 ? 8 : 4; }   // 8 waves split a long K
 
-static size_t fused_gemm_lds(int MT, int pro, int K) {
+// staged: the columns of x the prologue keeps in LDS (all of K behind the norm, the merged heads behind the merge)
+static size_t fused_gemm_lds(int MT, int pro, int K, int staged = 0) {
   size_t bytes = (size_t)fused_gemm_waves(K) * MT * 256 * sizeof(float) + (size_t)16 * MT * 16 * sizeof(float);
-  if (pro == PRO_NORM) bytes += (size_t)MT * 16 * (K + FG_PAD) * sizeof(bf16_t);
+  if (pro == PRO_NORM) staged = K;
+  if (pro != PRO_PLAIN) bytes += (size_t)MT * 16 * (staged + FG_PAD) * sizeof(bf16_t);
   return bytes;
 }
 
@@ -415,7 +489,7 @@ static size_t fused_gemm_lds(int MT, int pro, int K) {
 template <int MT>
 static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStream_t stream, int k_splits = 1,
                              int feature_tiles = 1) {
-  const size_t lds = fused_gemm_lds(MT, pro, p.K);
+  const size_t lds = fused_gemm_lds(MT, pro, p.K, pro == PRO_MERGE ? p.merge_heads * p.merge_dh : 0);
   if (feature_tiles > 1) {
     if (pro != PRO_PLAIN || (feature_tiles != 2 && feature_tiles != 4)) return ERR_BAD_ARGUMENT;
     const dim3 blocks((p.N + 16 * feature_tiles - 1) / (16 * feature_tiles), k_splits);
@@ -438,7 +512,8 @@ static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStre
     if (waves == 8) fused_gemm_kernel<MT, PRO_, EPI_, 8, 1><<<blocks, 8 * WAVE, lds, stream>>>(p); \
     else fused_gemm_kernel<MT, PRO_, EPI_, 4, 1><<<blocks, 4 * WAVE, lds, stream>>>(p);            \
   } while (0)
-  if (pro == PRO_NORM && epi == EPI_PLAIN) FG_LAUNCH(PRO_NORM, EPI_PLAIN);
+  if (pro == PRO_MERGE && epi == EPI_PLAIN) FG_LAUNCH(PRO_MERGE, EPI_PLAIN);
+  else if (pro == PRO_NORM && epi == EPI_PLAIN) FG_LAUNCH(PRO_NORM, EPI_PLAIN);
   else if (pro == PRO_NORM && epi == EPI_SWIGLU) FG_LAUNCH(PRO_NORM, EPI_SWIGLU);
   else if (pro == PRO_NORM && epi == EPI_CONV) FG_LAUNCH(PRO_NORM, EPI_CONV);
   else if (pro == PRO_PLAIN && epi == EPI_PLAIN) FG_LAUNCH(PRO_PLAIN, EPI_PLAIN);
@@ -471,8 +546,9 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
                           (conv_k > 1 && (!conv_state || !slot_ids)) || out_f32))
     return ERR_BAD_ARGUMENT;
   const int MT = (M + 15) / 16;
+  if (pro != PRO_NORM && pro != PRO_PLAIN) return ERR_BAD_ARGUMENT;
   if (fused_gemm_lds(MT, pro, K) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
-  FusedGemmParams p;
+  FusedGemmParams p = {};
   p.h_in = h_in;
   p.delta0 = (const bf16_t*)delta0;
   p.delta1 = (const bf16_t*)delta1;
@@ -538,6 +614,47 @@ extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, cons
   else if (MT == 2) code = launch_fused_gemm<2>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
   else if (MT == 3) code = launch_fused_gemm<3>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
   else code = launch_fused_gemm<4>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
+  if (code != 0) return code;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// out[M, N] (bfloat16) = x[M, K] . W[N, K]^T + bias, where the first heads * head_dim columns of x are not read
+// from x but merged from `partial`, the (maximum, normalizer, sums) that mi_mixer_decode (merge = 0) left per
+// run of keys: [M, heads, runs, head_dim + 2], with the same runs, run_keys, page_size and window.  Every
+// workgroup merges all of them again (a few hundred KB from the caches), which is cheaper than a launch of
+// mixer_merge_kernel while the step is small.  M <= 16; the merged columns must fit LDS beside the sums.
+extern "C" int mi_fused_gemm_merge(const float* partial, const int* positions, int heads, int head_dim, int runs,
+                                   int run_keys, int page_size, int window, const void* x, long x_ld, const void* W,
+                                   const float* bias, int M, int N, int K, void* out, long out_ld, int w_fragments,
+                                   hipStream_t stream) {
+  if (M <= 0 || N <= 0 || K <= 0 || !W || !out || !x || !partial || !positions || x_ld < K || x_ld % 8 != 0)
+    return ERR_BAD_ARGUMENT;
+  if (heads <= 0 || head_dim <= 0 || runs <= 0 || run_keys <= 0 || page_size <= 0 || window < 0) return ERR_BAD_ARGUMENT;
+  const long merged = (long)heads * head_dim;
+  if (M > 16 || K % 32 != 0 || head_dim % 8 != 0 || merged % 32 != 0 || merged > K) return ERR_UNSUPPORTED_SIZE;
+  if (fused_gemm_lds(1, PRO_MERGE, K, (int)merged) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  FusedGemmParams p = {};
+  p.x = (const bf16_t*)x;
+  p.x_ld = x_ld;
+  p.W = (const bf16_t*)W;
+  p.bias = bias;
+  p.M = M;
+  p.N = N;
+  p.K = K;
+  p.out = out;
+  p.out_ld = out_ld;
+  p.out_scale = 1.0f;
+  p.w_tiled = w_fragments ? 1 : 0;
+  p.partial = partial;
+  p.positions = positions;
+  p.merge_heads = heads;
+  p.merge_dh = head_dim;
+  p.merge_runs = runs;
+  p.merge_run_keys = run_keys;
+  p.merge_page = page_size;
+  p.merge_window = window;
+  const int code = launch_fused_gemm<1>(p, PRO_MERGE, EPI_PLAIN, stream);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;
@@ -802,10 +919,10 @@ __global__ void mixer_merge_kernel(MixerParams p, int dh) {
   const int pos = p.positions[token];
   float maximum = -INFINITY, denominator = 0.f, sum = 0.f;
   int used = p.splits;
-  for (int s0 = 0; s0 < used; s0 += 8) {
-    float m_s[8], l_s[8], o_s[8];
+  for (int s0 = 0; s0 < used; s0 += MERGE_AT_ONCE) {
+    float m_s[MERGE_AT_ONCE], l_s[MERGE_AT_ONCE], o_s[MERGE_AT_ONCE];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < MERGE_AT_ONCE; ++j) {
       const float* run = runs + (long)min(s0 + j, p.splits - 1) * (dh + 2);
       m_s[j] = run[0];
       l_s[j] = run[1];
@@ -818,7 +935,7 @@ __global__ void mixer_merge_kernel(MixerParams p, int dh) {
       used = min(p.splits, (pos - base_key) / p.split_keys + 1);
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < MERGE_AT_ONCE; ++j) {
       if (s0 + j < used) {
         const float larger = fmaxf(maximum, m_s[j]);
         const float keep = __builtin_amdgcn_exp2f(maximum - larger);        // 0 the first time (maximum = -inf); units of log2
@@ -965,6 +1082,19 @@ extern "C" int mi_mixer_split_keys(int M, int Hkv, int page_size, long span) {
   return (int)((split / page_size) * page_size);          // whole pages
 }
 
+// The runs of keys of a step, as mi_mixer_decode cuts them: keys of a run and workgroups (partial results) per
+// (token, kv head): one per run while the step is small, fewer (each walks over several runs) once the step has
+// MX_WALK_BLOCKS of them anyway.  `span`: the most keys a request of the step can have.
+extern "C" int mi_mixer_runs(int M, int Hkv, int page_size, long span, int* run_keys, int* runs) {
+  const int keys = mi_mixer_split_keys(M, Hkv, page_size, span);
+  if (keys <= 0 || !run_keys || !runs) return ERR_BAD_ARGUMENT;
+  const long whole = (span + keys - 1) / keys;
+  *run_keys = keys;
+  *runs = (int)min(whole, max(1L, (MX_WALK_BLOCKS + (long)Hkv * M - 1) / ((long)Hkv * M)));
+  return 0;
+}
+
+// merge = 0: the attended heads are not written; `partial` is left for mi_fused_gemm_merge.
 extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv, int dh, int q_col, int k_col,
                                int v_col, const float* inv_freq, int rotary_dim, void* k_base, void* v_base,
                                long page_stride, int page_size, const int* block_tables, int max_pages,
@@ -972,7 +1102,7 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
                                int max_seq_len, int H, int P, int N, int G, int z_col, int x_col, int dt_col, const float* dt_bias,
                                const float* A, const float* D, float* ssm_state, const int* slot_ids,
                                void* attn_out, void* ssm_out, float* ssm_y, long out_ld, float* partial,
-                               long partial_floats, hipStream_t stream) {
+                               long partial_floats, int merge, hipStream_t stream) {
   if (M <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || H <= 0 || P <= 0 || N <= 0 || G <= 0 || H % G != 0)
     return ERR_BAD_ARGUMENT;
   const int group = Hq / Hkv;
@@ -1044,11 +1174,7 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
   p.ssm_out = (bf16_t*)ssm_out;
   p.ssm_y = ssm_y;
   p.out_ld = out_ld;
-  p.split_keys = mi_mixer_split_keys(M, Hkv, page_size, span);
-  p.splits = (int)((span + p.split_keys - 1) / p.split_keys);
-  // workgroups per (token, kv head): one per run while the step is small, fewer (each walks over several
-  // runs) once the step has MX_WALK_BLOCKS of them anyway
-  p.splits = (int)min((long)p.splits, max(1L, (MX_WALK_BLOCKS + (long)Hkv * M - 1) / ((long)Hkv * M)));
+  if (mi_mixer_runs(M, Hkv, page_size, span, &p.split_keys, &p.splits) != 0) return ERR_UNSUPPORTED_SIZE;
   if ((long)Hkv * M * p.splits > 0x3fffffffL || M > 65535 || Hq > 65535) return ERR_UNSUPPORTED_SIZE;
   if (!partial || partial_floats < (long)M * Hq * p.splits * (dh + 2)) return ERR_BAD_ARGUMENT;
   p.partial = partial;
@@ -1058,6 +1184,7 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
   if (dh == 64) mixer_decode_kernel<64><<<(unsigned)total, MX_THREADS, 0, stream>>>(p);
   else mixer_decode_kernel<128><<<(unsigned)total, MX_THREADS, 0, stream>>>(p);
   RETURN_IF_LAUNCH_FAILED();
+  if (!merge) return 0;
   const dim3 merge_grid(M, Hq);
   mixer_merge_kernel<<<merge_grid, dh, 0, stream>>>(p, dh);
   RETURN_IF_LAUNCH_FAILED();

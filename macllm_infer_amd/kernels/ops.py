@@ -9,6 +9,7 @@ without a GPU and the built modules these functions fail.
 from __future__ import annotations
 
 import ctypes
+from dataclasses import dataclass
 from typing import Optional, Sequence
 
 import torch
@@ -79,11 +80,14 @@ _SIGNATURES = {
         "mi_fused_gemm_split": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int,
                                 _c_ptr],
         "mi_mixer_split_keys": [_c_int, _c_int, _c_int, _c_long],
+        "mi_mixer_runs": [_c_int, _c_int, _c_int, _c_long, _c_ptr, _c_ptr],
+        "mi_fused_gemm_merge": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_ptr,
+                                _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_int, _c_ptr],
         "mi_mixer_decode": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int,
                             _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int,
                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                             _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr, _c_long,
-                            _c_ptr],
+                            _c_int, _c_ptr],
     },
     "microbench": {
         "mi_stream_read": [_c_ptr, _c_long, _c_ptr, _c_int, _c_ptr],
@@ -667,6 +671,55 @@ def _weight_operand(weight: torch.Tensor, fragments: Optional[torch.Tensor], nam
     return fragments
 
 
+@dataclass(frozen=True)
+class AttentionRuns:
+    """What ``mixer_decode(merge=False)`` leaves of the attended heads: ``partial`` float32
+    [M, heads, runs, head_dim + 2], (maximum, normalizer, sums) per run of ``run_keys`` keys."""
+    partial: torch.Tensor
+    positions: torch.Tensor
+    heads: int
+    head_dim: int
+    runs: int
+    run_keys: int
+    page_size: int
+    window: int
+
+
+def fused_gemm_merge_supported(M: int, K: int, heads: int, head_dim: int) -> bool:
+    """Whether ``fused_gemm_merge`` takes a step of M rows (the merged heads sit in LDS beside the waves' sums)."""
+    merged = heads * head_dim
+    waves = 8 if K // 32 > 32 else 4
+    return (M <= 16 and K % 32 == 0 and merged % 32 == 0 and merged <= K
+            and waves * 1024 + 1024 + 16 * (merged + 8) * 2 <= 64 * 1024)
+
+
+def fused_gemm_merge(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, x: torch.Tensor,
+                     attended: AttentionRuns, fragments: Optional[torch.Tensor] = None) -> None:
+    """out[M, N] = x [M, K] . weight[N, K]^T (+ bias) in bfloat16 for a step of up to 16 rows, where the first
+    heads * head_dim columns of x are not read but merged from the runs of keys that ``mixer_decode(merge=False)``
+    left: the merge of the runs and the product in one launch."""
+    _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
+          "fused_gemm_merge: weight must be contiguous bfloat16 [N, K]")
+    N, K = weight.shape
+    x_ld = _row_major(x, "x")
+    M = x.shape[0]
+    _need(x.dtype == torch.bfloat16 and x.shape == (M, K) and x.data_ptr() % 16 == 0, "fused_gemm_merge: bad x")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()),
+          "fused_gemm_merge: bias must be float32 [N]")
+    _need(out.dtype == torch.bfloat16 and out.shape == (M, N), "fused_gemm_merge: out must be bfloat16 [M, N]")
+    out_ld = _row_major(out, "out")
+    _need(attended.partial.dtype == torch.float32 and attended.partial.is_contiguous()
+          and attended.partial.numel() >= M * attended.heads * attended.runs * (attended.head_dim + 2),
+          "fused_gemm_merge: the partial results do not cover the step")
+    _i32(attended.positions, "positions")
+    _need(attended.positions.numel() == M, "fused_gemm_merge: one position per row")
+    operand = _weight_operand(weight, fragments, "fused_gemm_merge")
+    _check(_fn("decode", "mi_fused_gemm_merge")(
+        _p(attended.partial), _p(attended.positions), attended.heads, attended.head_dim, attended.runs,
+        attended.run_keys, attended.page_size, attended.window, _p(x), x_ld, _p(operand), _p(bias), M, N, K, _p(out),
+        out_ld, int(fragments is not None), _stream()), "fused_gemm_merge", f"(M={M}, N={N}, K={K})")
+
+
 def fused_gemm_split(weight: torch.Tensor, bias: Optional[torch.Tensor], x: torch.Tensor, partial: torch.Tensor,
                      feature_tiles: int = 1, fragments: Optional[torch.Tensor] = None) -> None:
     """x [M, K] . weight[N, K]^T (+ bias) for a small batch in bfloat16, split over K: slab s of
@@ -759,6 +812,18 @@ def mixer_decode_supported(num_heads: int, num_kv_heads: int, head_dim: int, pag
             and state_size <= 512 and rotary_dim % 16 == 0)
 
 
+MERGE_AT_ONCE = 8          # runs of keys a merge asks for at once (decode.hip)
+
+
+def mixer_runs(M: int, num_kv_heads: int, page_size: int, span: int):
+    """(keys of a run, runs per token and kv head) as ``mixer_decode`` cuts the contexts of a step of M tokens
+    whose requests hold up to ``span`` keys."""
+    run_keys, runs = ctypes.c_int(0), ctypes.c_int(0)
+    _check(_fn("decode", "mi_mixer_runs")(M, num_kv_heads, page_size, span, ctypes.addressof(run_keys),
+                                          ctypes.addressof(runs)), "mixer_decode", "(no run length for these sizes)")
+    return run_keys.value, runs.value
+
+
 def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int, q_col: int, k_col: int,
                  v_col: int, inv_freq: Optional[torch.Tensor], rotary_dim: int, k_cache: torch.Tensor,
                  v_cache: torch.Tensor, block_tables: torch.Tensor, positions: torch.Tensor,
@@ -766,13 +831,14 @@ def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim
                  ssm_heads: int, ssm_head_dim: int, state_size: int, num_groups: int,
                  z_col: int, x_col: int, dt_col: int, dt_bias: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
                  ssm_state: torch.Tensor, slot_ids: torch.Tensor, out: torch.Tensor,
-                 ssm_y: Optional[torch.Tensor]) -> None:
+                 ssm_y: Optional[torch.Tensor], merge: bool = True) -> Optional[AttentionRuns]:
     """Both mixers of a decode step in one launch.  ``u`` [M, >=cols] holds each token's projected
     row (q, k, v unrotated; x, B, C after the conv).  Attention: rotates q and the new key, writes
     the new K/V into the cache cell ``slot_mapping``, attends over the request's pages, writes
     ``out[:, :Hq*dh]``.  State space: one scan step from and into ``ssm_state[slot_ids]``, writes
     ``y * SiLU(z)`` to ``out[:, Hq*dh:]``, or float32 ``y`` to ``ssm_y`` when a grouped norm
-    follows.  ``max_seq_len``: an upper bound of the longest context in the batch."""
+    follows.  ``max_seq_len``: an upper bound of the longest context in the batch.  With ``merge=False``
+    ``out[:, :Hq*dh]`` is not written: the runs of keys are returned unmerged, for ``fused_gemm_merge``."""
     u_ld = _row_major(u, "u")
     out_ld = _row_major(out, "out")
     M = u.shape[0]
@@ -797,17 +863,18 @@ def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim
                  z_col + E, x_col + E + 2 * num_groups * state_size, dt_col + ssm_heads)
     _need(u.shape[1] >= widest, "mixer_decode: u is too narrow")
     span = max(1, int(max_seq_len)) if not window else window + page_size
-    split_keys = int(_fn("decode", "mi_mixer_split_keys")(M, num_kv_heads, page_size, span))      # the launcher's own rule
-    _need(split_keys > 0, "mixer_decode: no run length for these sizes")
-    partial = torch.empty((M * num_heads * (-(-span // split_keys)) * (head_dim + 2),), dtype=torch.float32,
-                          device=u.device)
+    run_keys, runs = mixer_runs(M, num_kv_heads, page_size, span)        # the launcher's own rule
+    partial = torch.empty((M * num_heads * runs * (head_dim + 2),), dtype=torch.float32, device=u.device)
     _check(_fn("decode", "mi_mixer_decode")(
         _p(u), u_ld, M, num_heads, num_kv_heads, head_dim, q_col, k_col, v_col, _p(inv_freq), rotary_dim,
         _p(k_cache), _p(v_cache), page_stride, page_size, _p(block_tables), block_tables.shape[1], _p(positions),
         _p(slot_mapping), float(scale), int(window or 0), int(max_seq_len), ssm_heads, ssm_head_dim, state_size,
         num_groups, z_col, x_col, dt_col, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(slot_ids), _p(out),
         out.data_ptr() + 2 * num_heads * head_dim,
-        _p(ssm_y), out_ld, _p(partial), partial.numel(), _stream()), "mixer_decode")
+        _p(ssm_y), out_ld, _p(partial), partial.numel(), int(merge), _stream()), "mixer_decode")
+    if merge:
+        return None
+    return AttentionRuns(partial, positions, num_heads, head_dim, runs, run_keys, page_size, int(window or 0))
 
 
 # --------------------------------------------------------------------------- memory microbenchmarks

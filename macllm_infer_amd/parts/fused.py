@@ -72,6 +72,14 @@ FORCE_TILES: Optional[int] = None         # tests: this many tiles for steps of 
 # The library's tile for a prompt portion's input projection depends on the number of output features: 4 120
 # of them (0.5B-shaped) take 30.5 us at 2,048 rows, 4 352 (a multiple of 256) take 23.6.  Measured at build in
 # the same way; where padding pays, the prompt path multiplies with zero rows added and ignores their columns.
+# The attended heads of a decode step come in runs of keys that a small kernel merges; the output projection
+# can merge them in its prologue instead, every workgroup of it again: one launch less, but the projection then
+# starts behind a read of the runs.  It pays while a workgroup reads few of them (0.5B-shaped at 2,048-token
+# contexts: 1.33 -> 1.26 ms a step at 1 row, 1.39 -> 1.37 at 4, even at 6 to 8, slower from 16; 7B-shaped: faster
+# at 1 and 2 rows, slower at 4): up to MERGE_LATER_BYTES of runs a workgroup.
+MERGE_LATER_ROWS = 16
+MERGE_LATER_BYTES = 96 << 10
+FORCE_MERGE_LATER: Optional[bool] = None  # tests: True or False instead of the rule
 PAD_FEATURES = 256
 PAD_ROWS = 2048
 PAD_MARGIN = 0.95
@@ -226,7 +234,9 @@ def register_mixer_kernel(*kinds: str):
     this order: a kernel that runs all of them in one launch in steps of single tokens.  The kernel object
     offers ``conv`` (None, or the columns of the input projection that go through a conv step in that
     product's epilogue: {lo, hi, taps, weight, bias}), ``supported(step, caches)``,
-    ``conv_state(caches)`` and ``run(u, step, caches, mixed)``."""
+    ``conv_state(caches)`` and ``run(u, step, caches, mixed, merge=True)``; a kernel with ``merge_later_bytes(step,
+    caches)`` returns, when called with ``merge=False``, the runs of keys of its attended heads (the first columns of
+    ``mixed``) unmerged, as ``ops.AttentionRuns``, for the output projection to merge."""
     def decorate(factory):
         _MIXER_KERNELS[tuple(kinds)] = factory
         return factory
@@ -477,13 +487,16 @@ class LayerFusion:
                 residual.h, residual.pending = h_out, []
         # 2
         mixed = torch.empty((M, self.mixed_width), dtype=bf16, device=device)
+        attended = None
         if kernel is not None:
-            kernel.run(u, step, caches, mixed)
+            later = (not self.library_out[bucket] and not self.split_out[bucket]
+                     and self._merges_later(kernel, step, caches))
+            attended = kernel.run(u, step, caches, mixed, merge=not later)
         else:
             self._mix_each(u, step, caches, mixed)
         # 3
         residual.pending = self._to_the_stream(mixed, self.w_out, self.b_out, self.library_out[bucket],
-                                               self.split_out[bucket], self.tiles_out[bucket], self.f_out)
+                                               self.split_out[bucket], self.tiles_out[bucket], self.f_out, attended)
         # 4
         if self.gate_up is None:
             residual.pending = [block.ffn.forward(block.ffn_norm.forward(residual))]
@@ -502,11 +515,29 @@ class LayerFusion:
         residual.pending = self._to_the_stream(activated, self.down.weight, self.down.bias, self.library_down[bucket],
                                                self.split_down[bucket], self.tiles_down[bucket], self.f_down)
 
+    def _merges_later(self, kernel, step, caches) -> bool:
+        """Whether the output projection merges the runs of keys of this step's attended heads itself."""
+        estimate = getattr(kernel, "merge_later_bytes", None)
+        rows = step.num_tokens
+        if estimate is None or rows > MERGE_LATER_ROWS or FORCE_MERGE_LATER is False:
+            return False
+        merged = estimate(step, caches)                  # (merged columns, bytes of runs one workgroup reads)
+        if merged is None or not ops.fused_gemm_merge_supported(rows, self.w_out.shape[1], 1, merged[0]):
+            return False
+        if FORCE_MERGE_LATER:
+            return True
+        return merged[1] <= MERGE_LATER_BYTES
+
     def _to_the_stream(self, x: torch.Tensor, weight: torch.Tensor, bias, library: bool, slabs: int, tiles: int,
-                       fragments) -> list:
+                       fragments, attended=None) -> list:
         """A projection whose result is added to the residual stream: what the next norm will add, as one
-        bfloat16 branch or as float32 partial sums over runs of K (views of one tensor, in order)."""
+        bfloat16 branch or as float32 partial sums over runs of K (views of one tensor, in order).
+        ``attended``: the first columns of x are to be merged from these runs of keys."""
         M = x.shape[0]
+        if attended is not None:
+            delta = torch.empty((M, self.hidden), dtype=torch.bfloat16, device=x.device)
+            ops.fused_gemm_merge(weight, bias, delta, x, attended, fragments)
+            return [delta]
         if slabs:
             partial = torch.empty((slabs, M, self.hidden), dtype=torch.float32, device=x.device)
             ops.fused_gemm_split(weight, bias, x, partial, feature_tiles=tiles, fragments=fragments)
@@ -566,13 +597,21 @@ class AttentionMamba2Step:
                 and ops.mixer_decode_supported(a.num_heads, a.num_kv_heads, a.head_dim, cache.k_cache.shape[2],
                                                self.mamba.spec.state_size, step.max_seq_len, a.window, rotary))
 
-    def run(self, u: torch.Tensor, step, caches, mixed: torch.Tensor) -> None:
+    def merge_later_bytes(self, step, caches):
+        """(columns of the attended heads, bytes of runs of keys a workgroup reads to merge them), or None."""
+        a = self.attention.spec
+        rows, page_size = step.num_tokens, caches[self.attention_name].k_cache.shape[2]
+        span = max(1, int(step.max_seq_len)) if not a.window else a.window + page_size
+        runs = ops.mixer_runs(rows, a.num_kv_heads, page_size, span)[1]
+        return a.num_heads * a.head_dim, rows * a.num_heads * min(runs, ops.MERGE_AT_ONCE) * (a.head_dim + 2) * 4
+
+    def run(self, u: torch.Tensor, step, caches, mixed: torch.Tensor, merge: bool = True):
         a, s = self.attention.spec, self.mamba.spec
         kv, state = caches[self.attention_name], caches[self.mamba_name]
         gated_norm = self.mamba.norm_weight is not None
         y = torch.empty((u.shape[0], s.inner_size), dtype=torch.float32, device=u.device) if gated_norm else None
         rope = isinstance(self.position, Rope)
-        ops.mixer_decode(
+        attended = ops.mixer_decode(
             u, num_heads=a.num_heads, num_kv_heads=a.num_kv_heads, head_dim=a.head_dim, q_col=self.q_col,
             k_col=self.k_col, v_col=self.v_col, inv_freq=self.position.inv_freq if rope else None,
             rotary_dim=self.position.rotary_dim if rope else 0, k_cache=kv.k_cache, v_cache=kv.v_cache,
@@ -581,10 +620,11 @@ class AttentionMamba2Step:
             ssm_heads=s.num_heads, ssm_head_dim=s.head_dim, state_size=s.state_size,
             num_groups=s.num_groups, z_col=self.z_col, x_col=self.x_col, dt_col=self.dt_col,
             dt_bias=self.mamba.dt_bias, A=self.mamba.A, D=self.mamba.D, ssm_state=state.states["ssm"],
-            slot_ids=step.slot_ids, out=mixed, ssm_y=y)
+            slot_ids=step.slot_ids, out=mixed, ssm_y=y, merge=merge)
         if gated_norm:
             ops.gate_norm(y, u[:, self.z_col:self.z_col + s.inner_size], self.mamba.norm_weight, s.num_groups,
                           s.norm_eps, mixed[:, self.attended_width:])
+        return attended
 
 
 def _cat_bias(linears, device):

@@ -2,7 +2,7 @@
 model's sizes, what each group of kernels has to move and compute against the time it took.
 
     python -m macllm_infer_amd.utils.kernel_trace RESULTS.db [--first KERNEL] [--last KERNEL] [--top N]
-        [--config CONFIG.json (--batch B --context C | --prefill T) [--dtype bf16|f32]]
+        [--config CONFIG.json (--batch B --context C | --prefill T) [--dtype bf16|f32]] [--timeline FROM:TO]
 
 A step starts at the last launch of the kernel whose name contains ``--first`` (default: the
 embedding kernel, the first launch of every forward pass) and runs to the end of the trace or,
@@ -11,6 +11,9 @@ durations), span (first start to last end) and the kernels by total time.  With 
 config.json of the model that ran) and the step's shape it adds, per group of kernels: the bytes
 the group has to read and write, its flops, the rates these make with the group's busy time, and
 their fractions of the published peaks (8 TB/s; 2.5 PFLOP/s bf16, 157.3 TFLOP/s float32).
+``--timeline FROM:TO`` lists launches FROM to TO of the step one by one (start after the first of them,
+duration, the time since the latest end of everything before it): which kernels of a layer run side
+by side on two streams, and where the GPU waits.
 """
 from __future__ import annotations
 
@@ -79,6 +82,7 @@ def main() -> None:
     parser.add_argument("--context", type=float, default=0, help="tokens each request of the decode step holds")
     parser.add_argument("--prefill", type=int, default=0, help="tokens of the prompt step (instead of --batch/--context)")
     parser.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
+    parser.add_argument("--timeline", default=None, help="FROM:TO, launches of the step to list one by one")
     args = parser.parse_args()
     step = last_step(args.database, args.first, args.last)
     busy = sum(end - start for _, start, end in step)
@@ -91,6 +95,16 @@ def main() -> None:
     print(f"{'kernel':72s} {'calls':>5s} {'total us':>10s} {'avg us':>8s} {'share':>6s}")
     for name, (calls, total) in sorted(totals.items(), key=lambda item: -item[1][1])[:args.top]:
         print(f"{name[:72]:72s} {calls:5d} {total / 1e3:10.1f} {total / calls / 1e3:8.2f} {100.0 * total / busy:5.1f}%")
+    if args.timeline:
+        low, high = (int(value) for value in args.timeline.split(":"))
+        stretch = step[low:high]
+        print()
+        print(f"{'launch':>6s} {'start us':>9s} {'us':>8s} {'idle before':>11s}  kernel")
+        latest = None
+        for index, (name, start, end) in enumerate(stretch, low):
+            idle = "" if latest is None else f"{(start - latest) / 1e3:11.2f}"
+            print(f"{index:6d} {(start - stretch[0][1]) / 1e3:9.2f} {(end - start) / 1e3:8.2f} {idle:>11s}  {name[:60]}")
+            latest = end if latest is None else max(latest, end)
     if args.config:
         from ..config.registry import config_from_dict
         with open(args.config) as handle:

@@ -104,7 +104,8 @@ def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, r
 
 
 def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token,
-                    positions, scale, window, out):
+                    positions, scale, window, out, max_seq_len=None):
+    """``max_seq_len`` sizes the kernel's launch and nothing else: not used here."""
     T = q.shape[0]
     page_size = k_cache.shape[2]
     group = num_heads // num_kv_heads

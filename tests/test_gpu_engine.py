@@ -363,6 +363,37 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
         assert ((have - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()).item() <= 3e-2
 
 
+def test_the_output_projection_may_merge_the_runs_of_keys(monkeypatch):
+    """Steps of up to 16 single tokens: whether the runs of keys of the attended heads are merged by a kernel of
+    their own or in the prologue of the output projection, the logits are the same bit for bit, with contexts
+    of one run of keys and of several, through graphs and without."""
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.parts import fused
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.weights.random_init import random_tensors
+    config = FalconH1Config.from_dict(dict(tiny_configs.TINY_C, max_position_embeddings=4096))
+    tensors = random_tensors(config, 5, torch.bfloat16, "unit")
+    prompts = {index: tokens_for(config.vocab_size, length, 700 + index) for index, length in enumerate([700, 3, 260, 41, 1030])}
+    results = {}
+    for later in (False, True):
+        monkeypatch.setattr(fused, "FORCE_MERGE_LATER", later)
+        for graphs in (False, True):
+            engine = Engine(config=config, tensors=tensors, dtype="bfloat16", kv_cache_block_tokens=16,
+                            kv_cache_capacity_tokens=4096, max_active_sequences=8, decode_graphs=graphs)
+            fusion = engine.model.blocks[0].fusion
+            assert fusion.kernel is not None and not fusion.library_out[0] and not fusion.split_out[0]
+            for index, tokens in prompts.items():
+                engine.add_request(index)
+                engine.step([Lane(index, tokens[:-1], [])])
+            rows = []
+            for turn in range(4):
+                lanes = [Lane(index, [tokens[-1] if turn == 0 else 5 + turn], [0]) for index, tokens in prompts.items()]
+                rows.append(engine.step(lanes[:1 + turn] if turn < 2 else lanes).float().cpu())
+            results[later, graphs] = torch.cat(rows)
+    for key, rows in results.items():
+        assert torch.equal(rows, results[False, False]), key
+
+
 def test_graphs_come_in_buckets_of_context_length():
     """A model that allows long contexts: a short request decodes through a graph made for 2,048
     tokens, a longer one through a graph made for 4,096 (wider block tables, more runs of keys),

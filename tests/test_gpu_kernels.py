@@ -907,6 +907,64 @@ def test_mixer_decode_of_wide_batches(ops, M, Hq, Hkv, dh, H, P, N, G):
     assert torch.equal(got_state[unused].cpu(), state[unused])
 
 
+@pytest.mark.parametrize("Hq, Hkv, dh, E, N_out, window, lengths", [
+    (8, 2, 64, 1536, 1024, None, [1, 17, 64, 65, 300, 1500, 2, 2060]),
+    (4, 2, 64, 96, 200, 40, [1, 17, 64, 65, 300, 1500, 2]),
+    (12, 2, 128, 512, 320, None, [700, 3]),
+    (4, 4, 64, 64, 48, None, [5000, 9000, 3] + [40 + lane for lane in range(13)]),
+])
+def test_output_projection_that_merges_the_runs_of_keys(ops, Hq, Hkv, dh, E, N_out, window, lengths):
+    """``mixer_decode(merge=False)`` followed by ``fused_gemm_merge`` gives bit for bit what ``mixer_decode``,
+    its merge kernel and ``fused_gemm`` give: contexts of one run and of more runs than a merge asks for at
+    once, a window, 16 rows, a K beyond 1 024.  The attended columns of x hold NaN where nobody may read them."""
+    dtype = torch.bfloat16
+    H, P, N, G, page_size = E // 32, 32, 32, 1, 16
+    M = len(lengths)
+    pool, table = paged_setup(lengths, page_size, Hkv, dh, dtype, seed=21)
+    for lane, length in enumerate(lengths):
+        fill_cache(pool, table, lane, rand(length, Hkv, dh, seed=800 + lane, dtype=dtype),
+                   rand(length, Hkv, dh, seed=900 + lane, dtype=dtype), page_size)
+    q_col, k_col, v_col = 0, Hq * dh, (Hq + Hkv) * dh
+    z_col = (Hq + 2 * Hkv) * dh
+    x_col, dt_col = z_col + E, z_col + 2 * E + 2 * G * N
+    u = rand(M, -(-(dt_col + H) // 8) * 8, seed=810, dtype=dtype).to(DEV)
+    positions = i32([length - 1 for length in lengths]).to(DEV)
+    slot_mapping = i32([int(table[lane, (length - 1) // page_size]) * page_size + (length - 1) % page_size
+                        for lane, length in enumerate(lengths)]).to(DEV)
+    inv_freq = torch.tensor([1.0 / (1e4 ** (i / dh)) for i in range(0, dh, 2)], dtype=torch.float64).float().to(DEV)
+    state = rand(M, H, P, N, seed=811, scale=0.5)
+    vectors = [rand(H, seed=812) - 2.0, -(rand(H, seed=813).abs() + 0.1), rand(H, seed=814)]
+    K = Hq * dh + E
+    weight, bias = rand(N_out, K, seed=815, scale=0.05, dtype=dtype).to(DEV), rand(N_out, seed=816).to(DEV)
+
+    def run(merge):
+        dev_pool = pool.clone().to(DEV)
+        mixed = torch.full((M, K), float("nan"), dtype=dtype, device=DEV)
+        runs = ops.mixer_decode(u, num_heads=Hq, num_kv_heads=Hkv, head_dim=dh, q_col=q_col, k_col=k_col, v_col=v_col,
+                                inv_freq=inv_freq, rotary_dim=dh, k_cache=views(dev_pool, page_size)[0],
+                                v_cache=views(dev_pool, page_size)[1], block_tables=table.to(DEV), positions=positions,
+                                slot_mapping=slot_mapping, scale=0.13, window=window, max_seq_len=max(lengths) + 5,
+                                ssm_heads=H, ssm_head_dim=P, state_size=N, num_groups=G, z_col=z_col, x_col=x_col,
+                                dt_col=dt_col, dt_bias=vectors[0].to(DEV), A=vectors[1].to(DEV), D=vectors[2].to(DEV),
+                                ssm_state=state.clone().to(DEV), slot_ids=i32(list(range(M))).to(DEV), out=mixed,
+                                ssm_y=None, merge=merge)
+        return mixed, runs
+
+    mixed, nothing = run(True)
+    assert nothing is None and not torch.isnan(mixed.float()).any()
+    want = torch.empty(M, N_out, dtype=dtype, device=DEV)
+    ops.fused_gemm(weight, bias, want, x=mixed)
+    unmerged, runs = run(False)
+    assert torch.isnan(unmerged[:, :Hq * dh].float()).all() and torch.equal(unmerged[:, Hq * dh:], mixed[:, Hq * dh:])
+    assert ops.fused_gemm_merge_supported(M, K, Hq, dh)
+    for fragments in (None, ops.fragment_order(weight)):
+        got = torch.empty(M, N_out, dtype=dtype, device=DEV)
+        ops.fused_gemm_merge(weight, bias, got, unmerged, runs, fragments)
+        assert torch.equal(got, want)
+    product = mixed.float().cpu() @ weight.float().cpu().T + bias.cpu()
+    close(want, product, dtype, max(1.0, product.abs().max().item()))
+
+
 def test_mixer_decode_over_a_long_context(ops):
     """Contexts of 5 000 and 9 000 tokens (more runs of keys than the merge takes
     at once) beside a short one; one far key per long request is made to dominate, so a run that
