@@ -187,12 +187,20 @@ def main() -> int:
                         help="steps: the headline decode and prefill steps; serving: whole requests through the scheduler")
     parser.add_argument("--microbench", action="store_true",
                         help="only this GPU's streaming read and read-modify-write bandwidth")
+    parser.add_argument("--write-config", default=None, metavar="PATH",
+                        help="write the config.json of --shape / --layers there and exit (what "
+                             "utils.kernel_trace --config reads)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
         return 2
     if args.microbench:
         return microbench()
+    if args.write_config:
+        shape = SHAPES[args.shape]
+        with open(args.write_config, "w") as handle:
+            json.dump(dict(shape, num_hidden_layers=args.layers or shape["num_hidden_layers"]), handle)
+        return 0
     if args.workload == "serving":
         return serving(args, SHAPES[args.shape])
 
