@@ -118,6 +118,8 @@ extern "C" int mi_rope_kv_store(void* qkv, int dtype, long ld, int T, int Hq, in
 //   s = q.k * scale;  visible keys: position <= query position, and
 //   query - key < window when window > 0 (reference: src/decoder.rs:4515-4532);
 //   softmax in float32 (reference: src/decoder.rs:4665-4667).
+// `slopes` (optional, float32 per query head): a position encoding that is a bias on the scores,
+//   s -= slopes[head] * (query position - key position)   (no counterpart in the reference).
 // The keys are cut into runs of PA_RUN by their absolute position.  One workgroup per (token, query head,
 // run): each of its four waves takes 64 keys of the run (lane i scores key i with a full dot product over
 // dh from its own cache row; for the value product lane i owns output dims i, i + 64, ...), keeps
@@ -136,7 +138,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
                        const T* __restrict__ k_base, const T* __restrict__ v_base, long page_stride,
                        int page_size, const int* __restrict__ block_tables, int max_pages,
                        const int* __restrict__ lane_of_token, const int* __restrict__ positions, float scale,
-                       int window, int runs, float* __restrict__ partial) {
+                       int window, const float* __restrict__ slopes, int runs, float* __restrict__ partial) {
   typedef T vec4 __attribute__((ext_vector_type(4)));
   __shared__ __align__(16) float q_shared[ATT_MAX_DH];
   __shared__ float p_shared[PA_WAVES][WAVE];
@@ -181,6 +183,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
       for (int i = 0; i < dh; ++i) dot += q_shared[i] * to_float(k_row[i]);
     }
     score = dot * scale;
+    if (slopes) score -= slopes[head] * (float)(query_position - key);
   }
   const float maximum = wave_max(score);                    // -inf for a wave without visible keys
   const float p = visible ? (FAST_EXP ? __expf(score - maximum) : expf(score - maximum)) : 0.f;
@@ -268,8 +271,8 @@ extern "C" long mi_paged_attention_workspace(int T, int Hq, int dh, int max_seq_
 extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, int Hq, int Hkv, int dh,
                                   const void* k_base, const void* v_base, long page_stride, int page_size,
                                   const int* block_tables, int max_pages, const int* lane_of_token,
-                                  const int* positions, float scale, int window, int max_seq_len,
-                                  float* partial, long partial_floats, void* out, long out_ld,
+                                  const int* positions, float scale, int window, const float* slopes,
+                                  int max_seq_len, float* partial, long partial_floats, void* out, long out_ld,
                                   hipStream_t stream) {
   if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || dh <= 0 || page_size <= 0 || max_pages <= 0 ||
       max_seq_len <= 0 || !partial)
@@ -284,14 +287,14 @@ extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, in
   if (dtype == DT_F32) {
     paged_attention_kernel<float, false><<<grid, PA_RUN, 0, stream>>>(
         (const float*)q, q_ld, Hq, Hkv, dh, (const float*)k_base, (const float*)v_base, page_stride, page_size,
-        block_tables, max_pages, lane_of_token, positions, scale, window, runs, partial);
+        block_tables, max_pages, lane_of_token, positions, scale, window, slopes, runs, partial);
     RETURN_IF_LAUNCH_FAILED();
     paged_attention_merge_kernel<float, false><<<merge_grid, merge_threads, 0, stream>>>(
         partial, Hq, dh, runs, positions, window, (float*)out, out_ld);
   } else if (dtype == DT_BF16) {
     paged_attention_kernel<bf16_t, true><<<grid, PA_RUN, 0, stream>>>(
         (const bf16_t*)q, q_ld, Hq, Hkv, dh, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride,
-        page_size, block_tables, max_pages, lane_of_token, positions, scale, window, runs, partial);
+        page_size, block_tables, max_pages, lane_of_token, positions, scale, window, slopes, runs, partial);
     RETURN_IF_LAUNCH_FAILED();
     paged_attention_merge_kernel<bf16_t, true><<<merge_grid, merge_threads, 0, stream>>>(
         partial, Hq, dh, runs, positions, window, (bf16_t*)out, out_ld);

@@ -42,7 +42,7 @@ _SIGNATURES = {
         "mi_rope_kv_store": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int,
                              _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr],
         "mi_paged_attention": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
-                               _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_long,
+                               _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_int, _c_ptr, _c_long,
                                _c_ptr, _c_long, _c_ptr],
         "mi_paged_attention_workspace": [_c_int, _c_int, _c_int, _c_int],
         "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
@@ -329,14 +329,16 @@ def _cache_view(k_cache, v_cache, num_kv_heads, head_dim, dtype):
 def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                     k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     lane_of_token: torch.Tensor, positions: torch.Tensor, scale: float,
-                    window: Optional[int], out: torch.Tensor, max_seq_len: Optional[int] = None) -> None:
+                    window: Optional[int], out: torch.Tensor, max_seq_len: Optional[int] = None,
+                    slopes: Optional[torch.Tensor] = None) -> None:
     """Causal attention of every token over its request's cached keys (its own included).
 
     ``q`` [T, >= Hq*dh] (rotated); ``block_tables`` [lanes, max_pages] page ids by logical
     page; a key at position p is visible to a query at position s when p <= s and, with a
     window w, s - p < w.  ``out`` [T, Hq*dh].  ``max_seq_len``: an upper bound of position + 1 over
     the step's tokens (what the block tables can hold if it is not given); it sizes the launch and
-    the work area, never the result."""
+    the work area, never the result.  ``slopes`` (float32 [Hq]): a bias on the scores by distance,
+    ``score -= slopes[head] * (s - p)``."""
     q_ld = _row_major(q, "q")
     out_ld = _row_major(out, "out")
     T = q.shape[0]
@@ -348,6 +350,8 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     _i32(positions, "positions")
     _need(block_tables.dim() == 2 and lane_of_token.numel() == T and positions.numel() == T,
           "paged_attention: metadata shapes do not match")
+    _need(slopes is None or (slopes.dtype == torch.float32 and slopes.numel() == num_heads and slopes.is_contiguous()
+                             and slopes.is_cuda), "paged_attention: slopes must be float32 [Hq] on the GPU")
     holds = block_tables.shape[1] * page_size
     span = holds if max_seq_len is None else max(1, min(int(max_seq_len), holds))
     floats = _fn("attention", "mi_paged_attention_workspace", _c_long)(T, num_heads, head_dim, span)
@@ -355,7 +359,7 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     _check(_fn("attention", "mi_paged_attention")(
         _p(q), _dt(q), q_ld, T, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride,
         page_size, _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale),
-        int(window or 0), span, _p(partial), partial.numel(), _p(out), out_ld, _stream()), "paged_attention",
+        int(window or 0), _p(slopes), span, _p(partial), partial.numel(), _p(out), out_ld, _stream()), "paged_attention",
         f"(head_dim={head_dim})")
 
 

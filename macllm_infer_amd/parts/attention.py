@@ -87,7 +87,12 @@ class Attention(Mixer):
         spec = self.spec
         self.position.rotate_and_store(qkv, spec.num_heads, spec.num_kv_heads, spec.head_dim, step, cache)
         geometry = (spec.num_heads, spec.num_kv_heads, spec.head_dim)
-        if step.max_query_len == 1 and ops.decode_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2]):
+        slopes = self.position.score_slopes
+        if slopes is not None:                           # a bias on the scores: the general kernel knows it
+            ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                step.lane_of_token, step.positions, spec.scale, spec.window, attended,
+                                step.max_seq_len, slopes)
+        elif step.max_query_len == 1 and ops.decode_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2]):
             ops.decode_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                  step.lane_of_token, step.positions, spec.scale, spec.window, step.max_seq_len,
                                  attended)

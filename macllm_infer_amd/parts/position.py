@@ -1,4 +1,4 @@
-"""Position encodings applied to q and k before the cache write."""
+"""Position encodings: transforms of q and k before the cache write, and biases on the attention scores."""
 from __future__ import annotations
 
 import torch
@@ -12,8 +12,13 @@ class PositionEncoding(Part):
     the q and k heads of ``qkv`` (q in place) and, if ``cache.owns_kv``, writes the encoded
     k and the raw v of every token into the cache cell ``step.slot_mappings[cache.group]``.
     A subclass may implement only ``rotate`` (in place on ``qkv``); the store is then done
-    by the cache-write kernel without rotation."""
+    by the cache-write kernel without rotation.
+
+    An encoding that (also) biases the scores by distance sets ``score_slopes``: a float32 tensor [query heads]
+    on the device, with score(head, query at s, key at p) -= score_slopes[head] * (s - p).  The attention part
+    then takes its general kernel, which knows the term; the matrix-core and fused decode kernels do not."""
     kernel_modules = ("attention",)
+    score_slopes = None
 
     def rotate(self, qkv, num_heads, num_kv_heads, head_dim, step) -> None:
         return None

@@ -104,8 +104,9 @@ def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, r
 
 
 def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token,
-                    positions, scale, window, out, max_seq_len=None):
-    """``max_seq_len`` sizes the kernel's launch and nothing else: not used here."""
+                    positions, scale, window, out, max_seq_len=None, slopes=None):
+    """``max_seq_len`` sizes the kernel's launch and nothing else: not used here.  ``slopes``: a bias on the
+    scores, ``-slopes[head] * (query position - key position)``."""
     T = q.shape[0]
     page_size = k_cache.shape[2]
     group = num_heads // num_kv_heads
@@ -121,6 +122,8 @@ def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, bloc
         for head in range(num_heads):
             query = _f(q[token, head * head_dim:(head + 1) * head_dim])
             scores = (k[:, head // group, :] @ query) * scale
+            if slopes is not None:
+                scores = scores - slopes[head] * (position - keys).float()
             weights = torch.softmax(scores, dim=0)
             out[token, head * head_dim:(head + 1) * head_dim] = (weights @ v[:, head // group, :]).to(out.dtype)
 

@@ -201,14 +201,21 @@ def test_rope_store_and_attention_over_pages(ops, dtype, Hq, Hkv, dh, page_size,
     assert torch.equal(torch.isnan(got_pool.float().cpu()), ~written)          # exactly the same cells
     close(torch.nan_to_num(got_pool.float()), torch.nan_to_num(want_pool.float()), dtype, 4.0)
     assert torch.isnan(got_pool[:, 0].float()).all()                           # the other layer is untouched
-    for window in (None, 9):
+    slopes = torch.tensor([0.4 / (head + 1) for head in range(Hq)])
+    for window, bias in ((None, None), (9, None), (None, slopes), (9, slopes)):     # bias: a slope per head times the distance
         want = torch.empty(T, Hq * dh, dtype=dtype)
         ref_ops.paged_attention(want_qkv, Hq, Hkv, dh, *views(want_pool, page_size), table,
-                                lane_of_token, positions, 0.37, window, want)
+                                lane_of_token, positions, 0.37, window, want, slopes=bias)
         got = torch.empty(T, Hq * dh, dtype=dtype, device=DEV)
         ops.paged_attention(got_qkv, Hq, Hkv, dh, *views(got_pool, page_size), table.to(DEV),
-                            lane_of_token.to(DEV), positions.to(DEV), 0.37, window, got)
+                            lane_of_token.to(DEV), positions.to(DEV), 0.37, window, got,
+                            slopes=None if bias is None else bias.to(DEV))
         close(got, want, dtype, 3.0)
+        if bias is not None and window is None:
+            plain = torch.empty(T, Hq * dh, dtype=dtype)
+            ref_ops.paged_attention(want_qkv, Hq, Hkv, dh, *views(want_pool, page_size), table,
+                                    lane_of_token, positions, 0.37, window, plain)
+            assert (plain.float() - want.float()).abs().max() > 0.05          # the bias changes the result
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -23,8 +23,11 @@ class DecayMixerSpec:
 
 @dataclass(frozen=True)
 class AlibiLikeSpec:
-    """A toy position encoding: scales q and k of head h by (1 + position * slope_h)."""
+    """A toy position encoding with both hooks: it scales q and k by (1 + position * slope) before the cache
+    write, and it biases the scores by distance: score(head h, query s, key p) -= bias / (h + 1) * (s - p)."""
     slope: float
+    bias: float = 0.0
+    heads: int = 4
     kind: str = "toy_scale_position"
 
     def validate(self, head_dim):
@@ -121,7 +124,7 @@ class ToyConfig:
         hidden = raw["hidden"]
         norm = RmsNormSpec(eps=1e-5)
         full = AttentionSpec(num_heads=4, num_kv_heads=2, head_dim=16, scale=0.25,
-                             position=AlibiLikeSpec(slope=raw["slope"]))
+                             position=AlibiLikeSpec(slope=raw["slope"], bias=raw.get("bias", 0.0)))
         windowed = AttentionSpec(num_heads=4, num_kv_heads=2, head_dim=16, scale=0.25,
                                  position=RopeSpec(theta=100.0, rotary_dim=8), window=raw["window"])
         ffn = SwiGLUSpec(intermediate_size=48)
@@ -217,6 +220,9 @@ def register_toys():
     class ScalePosition(PositionEncoding):
         def __init__(self, spec, head_dim, build):
             self.slope = spec.slope
+            if spec.bias:
+                self.score_slopes = torch.tensor([spec.bias / (head + 1) for head in range(spec.heads)],
+                                                 dtype=torch.float32, device=build.device)
 
         def rotate(self, qkv, num_heads, num_kv_heads, head_dim, step):
             factor = (1.0 + step.positions.float() * self.slope)[:, None]
@@ -302,6 +308,19 @@ def centred_norm(x, weight, bias, eps):
     return centred / torch.sqrt(centred.pow(2).mean(dim=-1, keepdim=True) + eps) * weight + bias
 
 
+def distance_biased_attention(q, k, v, scale, slopes):
+    """Causal attention, head by head, with score(s, p) = q_s . k_p * scale - slope_head * (s - p)."""
+    T, heads, _ = q.shape
+    group = heads // k.shape[1]
+    distance = (torch.arange(T)[:, None] - torch.arange(T)[None, :]).float()
+    out = torch.empty_like(q)
+    for head in range(heads):
+        scores = q[:, head] @ k[:, head // group].T * scale - slopes[head] * distance
+        scores = scores.masked_fill(distance < 0, float("-inf"))
+        out[:, head] = torch.softmax(scores, dim=-1) @ v[:, head // group]
+    return out
+
+
 def routed_feed_forward(x, router, up, down):
     """Each token through its two best experts; a token's result depends on that token alone."""
     logits = x @ router.T
@@ -344,8 +363,11 @@ def toy_plain_logits(raw, tensors, tokens):
             caches[index] = (k, v)
         else:
             k, v = caches[source]                       # reads the other run's keys and values
-        mixed = plain_impl.linear(plain_impl.gqa_causal_attention(q, k, v, 0.25, window).reshape(T, 64),
-                                  w["o_proj.weight"], None)
+        if layer == 0 and raw.get("bias"):
+            attended = distance_biased_attention(q, k, v, 0.25, [raw["bias"] / (head + 1) for head in range(4)])
+        else:
+            attended = plain_impl.gqa_causal_attention(q, k, v, 0.25, window)
+        mixed = plain_impl.linear(attended.reshape(T, 64), w["o_proj.weight"], None)
         if layer == 0:
             projected = n @ tensors[p + "decay.w.weight"].float().T
             s = torch.zeros(raw["hidden"])
@@ -395,8 +417,8 @@ def exercise(schedule, device, check_device):
     from macllm_infer_amd.engine.model import DecoderModel
     from macllm_infer_amd.weights.random_init import random_tensors
     register_toys()
-    raw = {"architectures": ["ToyForTests"], "hidden": 32, "vocab": 90, "slope": 0.01, "decay": 0.9, "window": 13,
-           "experts": 5, "schedule": schedule}
+    raw = {"architectures": ["ToyForTests"], "hidden": 32, "vocab": 90, "slope": 0.01, "bias": 0.3, "decay": 0.9,
+           "window": 13, "experts": 5, "schedule": schedule}
     config = ToyConfig(raw)
     tensors = random_tensors(config, 5, torch.float32, "unit")
     assert "model.layers.0.decay.w.weight" in tensors and tensors["model.layers.1.mlp.up.weight"].shape == (5, 24, 32)
