@@ -150,12 +150,14 @@ def microbench() -> int:
 
 
 def choices_of(engine) -> dict:
-    """What the first layer's fast path chose, as short strings (empty when the layer has none)."""
+    """What the first layer's fast path chose for steps of up to 8 / 16 / 32 / 48 / 64 rows, as short strings
+    (S: the skinny kernel, L: the library, a number: that many slabs over K; empty when the layer has none)."""
     fusion = getattr(engine.model.blocks[0], "fusion", None)
     if fusion is None or not getattr(fusion, "decode_ok", False):
         return {}
 
-    def way(library, split=(0, 0, 0)):
+    def way(library, split=None):
+        split = split or (0,) * len(library)
         return "/".join(str(slabs) if slabs else ("L" if lib else "S") for lib, slabs in zip(library, split))
 
     out = {"in": way(fusion.library_in), "out": way(fusion.library_out, fusion.split_out),

@@ -49,11 +49,12 @@ MAX_NORM_ROWS = 16     # the norm prologue recomputes the normed rows in every w
 # The skinny kernel reads the step's rows once per 16 weight rows and keeps all of K in one workgroup; the
 # library tiles the rows and splits a long K, but its choice of tile swings from shape to shape (a 5120 x
 # 21504 weight at 8 rows: 115 us against 69; a 3072 x 12288 one: 20 against 25), so the clock decides, per
-# shape and per step size (up to 16, 32, 64 rows).  Below the limit the skinny kernel wins everywhere.
+# shape and per step size (TUNE_ROWS: up to 8, 16, 32, 48 and 64 rows, each measured at its upper edge).  Below
+# the limit the skinny kernel wins everywhere.
 LIBRARY_MIN_WEIGHT = 2 << 20
 LIBRARY_MARGIN = 0.92          # the library has to be this much faster to be taken
 FORCE_LIBRARY: Optional[bool] = None      # tests: True or False instead of the clock
-TUNE_ROWS = (8, 32, 64)
+TUNE_ROWS = (8, 16, 32, 48, 64)
 _library_wins: Dict[tuple, tuple] = {}
 # An output or down projection at 32 to 64 rows has a long K and few output features: 64 workgroups of the
 # skinny kernel, or whatever tile the library picks (10.7 us for 1,024 x 2,048 at 64 rows).  Split over K into
@@ -68,6 +69,7 @@ _split_wins: Dict[tuple, tuple] = {}
 # fragments in flight (a 5120 x 21504 weight at 32 rows: 135 us with one tile, 86 with two, the library 125).
 # Measured with the rest, per shape and step size.
 TILE_CHOICES = (1, 2, 4)
+TILE_MARGIN = 0.95             # a wider tile has to be this much faster than one tile to be taken
 FORCE_TILES: Optional[int] = None         # tests: this many tiles for steps of more than 16 rows instead of the clock
 # The library's tile for a prompt portion's input projection depends on the number of output features: 4 120
 # of them (0.5B-shaped) take 30.5 us at 2,048 rows, 4 352 (a multiple of 256) take 23.6.  Measured at build in
@@ -99,7 +101,19 @@ def _side_stream(device: torch.device) -> "torch.cuda.Stream":
 
 
 def _bucket(rows: int) -> int:
-    return 0 if rows <= MAX_NORM_ROWS else 1 if rows <= 32 else 2
+    """The step size a step of ``rows`` rows was measured as: the first of TUNE_ROWS that holds it."""
+    for bucket, most in enumerate(TUNE_ROWS):
+        if rows <= most:
+            return bucket
+    return len(TUNE_ROWS) - 1
+
+
+BUCKETS = len(TUNE_ROWS)
+WIDE_BUCKETS = tuple(bucket for bucket, rows in enumerate(TUNE_ROWS) if rows > MAX_NORM_ROWS)   # no norm prologue there
+
+
+def _each(value) -> tuple:
+    return (value,) * BUCKETS
 
 
 def _graph_microseconds(run) -> float:
@@ -189,10 +203,11 @@ def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool, tiles: 
     return best
 
 
-def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile: int, conv: Optional[dict]) -> tuple:
+def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile: int, conv: Optional[dict],
+                     wide: bool) -> tuple:
     """(whether the library way is faster for this weight at this many rows, the skinny kernel's best number
-    of feature tiles).  Copies of the weight are cycled through so that the caches do not hold it, as in a
-    model of many layers."""
+    of feature tiles; ``wide``: more than one tile may be taken, i.e. the prologue is the plain one).  Copies
+    of the weight are cycled through so that the caches do not hold it, as in a model of many layers."""
     N, K = weight.shape
     device = weight.device
     copies = max(2, min(64, (512 << 20) // (weight.numel() * 2)))
@@ -221,8 +236,8 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
                 ops.conv_step(product, conv["lo"], conv["hi"] - conv["lo"], conv["weight"], conv["bias"], conv["state"],
                               conv["slot_ids"])
 
-    times = {tiles: _graph_microseconds(skinny(tiles)) for tiles in (TILE_CHOICES if rows > MAX_NORM_ROWS else (1,))}
-    tiles = min(times, key=times.get)
+    times = {tiles: _graph_microseconds(skinny(tiles)) for tiles in (TILE_CHOICES if wide else (1,))}
+    tiles = min(times, key=lambda count: times[count] * (1.0 if count == 1 else 1.0 / TILE_MARGIN))
     return _graph_microseconds(library) < LIBRARY_MARGIN * times[tiles], tiles
 
 
@@ -331,7 +346,7 @@ class LayerFusion:
         self.library_in, self.tiles_in = self._tune(self.w_in, self.b_in, ops.EPI_CONV if conv else ops.EPI_PLAIN, conv,
                                                     self.mixer_rms is not None)
         self.library_out, self.tiles_out = self._tune(self.w_out, self.b_out, ops.EPI_PLAIN)
-        # and which of the two that feed the residual stream are split over K instead (steps of more than 16 rows)
+        # and which of the two that feed the residual stream are split over K instead (steps of more than MAX_NORM_ROWS rows)
         self.split_out, self.tiles_out = self._tune_split(self.w_out, self.b_out, self.library_out, self.tiles_out)
         # what the skinny kernel reads: a second copy of each matrix in the order of its waves' fragments (one run
         # of 1 KiB a load instead of 64 bytes of each of 16 rows: 15 to 25 % faster); the row-major ones stay for
@@ -402,29 +417,33 @@ class LayerFusion:
 
     def _tune(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict] = None,
               normed: bool = False) -> tuple:
-        """For step sizes of up to 16, 32 and 64 rows: whether this projection goes through the library, and
-        the feature tiles of the skinny kernel.  (``normed``: the norm before it runs in the skinny kernel's
-        prologue; small steps then stay with it.)"""
+        """For every step size of TUNE_ROWS: whether this projection goes through the library, and the feature
+        tiles of the skinny kernel.  (``normed``: the norm before it runs in the skinny kernel's prologue in steps
+        of up to MAX_NORM_ROWS rows; those stay with the skinny kernel and one tile.)"""
         if not self.decode_ok:
-            return (True, True, True), (1, 1, 1)
-        choices, tiles = self._tune_all(weight, bias, epilogue, conv)
+            return _each(True), _each(1)
+        choices, tiles = self._tune_all(weight, bias, epilogue, conv, normed)
         if normed:
-            choices = (False,) + choices[1:]
+            choices = tuple(choice and bucket in WIDE_BUCKETS for bucket, choice in enumerate(choices))
         return choices, tiles
 
     def _tune_split(self, weight: torch.Tensor, bias, library: tuple, tiles: tuple) -> tuple:
-        """For step sizes of up to 16, 32 and 64 rows: the number of slabs over K, or 0 for the whole product,
-        and the feature tiles that go with it.  Steps of up to 16 rows feed the next kernel's norm prologue,
+        """For every step size of TUNE_ROWS: the number of slabs over K, or 0 for the whole product, and the
+        feature tiles that go with it.  Steps of up to MAX_NORM_ROWS rows feed the next kernel's norm prologue,
         which takes whole rows."""
         if self.hidden % 4 != 0 or FORCE_SPLIT == 0:
-            return (0, 0, 0), tiles
+            return _each(0), tiles
         if FORCE_SPLIT:
             slabs = FORCE_SPLIT if weight.shape[1] // 32 >= FORCE_SPLIT else 0
-            return (0, slabs, slabs), tiles
+            return tuple(slabs if bucket in WIDE_BUCKETS else 0 for bucket in range(BUCKETS)), tiles
         if weight.numel() < LIBRARY_MIN_WEIGHT:
-            return (0, 0, 0), tiles
-        slabs, split_tiles = [0], [tiles[0]]
-        for bucket in (1, 2):
+            return _each(0), tiles
+        slabs, split_tiles = [], []
+        for bucket in range(BUCKETS):
+            if bucket not in WIDE_BUCKETS:
+                slabs.append(0)
+                split_tiles.append(tiles[bucket])
+                continue
             key = (tuple(weight.shape), bias is None, bucket, library[bucket], tiles[bucket])
             if key not in _split_wins:
                 _split_wins[key] = _measure_split(weight, bias, TUNE_ROWS[bucket], library[bucket], tiles[bucket])
@@ -432,20 +451,21 @@ class LayerFusion:
             split_tiles.append(_split_wins[key][1])
         return tuple(slabs), tuple(split_tiles)
 
-    def _tune_all(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict]) -> tuple:
+    def _tune_all(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict], normed: bool) -> tuple:
         forced = 1 if FORCE_TILES is None else FORCE_TILES
-        fixed_tiles = (1, forced, forced)
+        fixed_tiles = tuple(forced if bucket in WIDE_BUCKETS else 1 for bucket in range(BUCKETS))
         if not self.general or FORCE_LIBRARY is False or (FORCE_LIBRARY is None and weight.numel() < LIBRARY_MIN_WEIGHT):
-            return (False, False, False), fixed_tiles
+            return _each(False), fixed_tiles
         if FORCE_LIBRARY:
-            return (True, True, True), fixed_tiles
+            return _each(True), fixed_tiles
         choices, tiles = [], []
         for bucket, rows in enumerate(TUNE_ROWS):
-            key = (tuple(weight.shape), epilogue, bias is None, bucket)
+            wide = bucket in WIDE_BUCKETS or not normed          # the plain prologue: a workgroup may own several tiles
+            key = (tuple(weight.shape), epilogue, bias is None, bucket, wide)
             if key not in _library_wins:
-                _library_wins[key] = _measure_library(weight, bias, rows, epilogue, 8, conv)
+                _library_wins[key] = _measure_library(weight, bias, rows, epilogue, 8, conv, wide)
             choices.append(_library_wins[key][0])
-            tiles.append(_library_wins[key][1] if FORCE_TILES is None or bucket == 0 else FORCE_TILES)
+            tiles.append(_library_wins[key][1] if FORCE_TILES is None or bucket not in WIDE_BUCKETS else FORCE_TILES)
         return tuple(choices), tuple(tiles)
 
     def forward_decode(self, residual: Residual, step, caches) -> None:

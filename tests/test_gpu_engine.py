@@ -340,11 +340,11 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
                     max_active_sequences=requests)
     if library == "split":
         fusion = engine.model.blocks[0].fusion
-        assert fusion.split_out == (0, 3, 3) and fusion.split_down == (0, 3, 3)
+        assert fusion.split_out == (0, 0, 3, 3, 3) and fusion.split_down == (0, 0, 3, 3, 3)
     if library == "tiles":
         fusion = engine.model.blocks[0].fusion
-        assert fusion.tiles_in == fusion.tiles_gate_up == fusion.tiles_out == fusion.tiles_down == (1, 4, 4)
-        assert fusion.library_in == fusion.library_down == (False, False, False)
+        assert fusion.tiles_in == fusion.tiles_gate_up == fusion.tiles_out == fusion.tiles_down == (1, 1, 4, 4, 4)
+        assert fusion.library_in == fusion.library_down == (False,) * 5
     prompts = {index: tokens_for(cfg["vocab_size"], 3 + index % 7 + 6, 500 + index) for index in range(requests)}
     for index, tokens in prompts.items():
         engine.add_request(index)
