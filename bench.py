@@ -162,7 +162,7 @@ def choices_of(engine) -> dict:
 
     out = {"in": way(fusion.library_in), "out": way(fusion.library_out, fusion.split_out),
            "tiles_in": "/".join(map(str, fusion.tiles_in)), "tiles_out": "/".join(map(str, fusion.tiles_out)),
-           "padded_in": bool(fusion.w_in_wide.shape[0] != fusion.in_width)}
+           "padded_in": "/".join("P" if pays else "-" for pays in fusion.padding_pays)}
     if fusion.gate_up is not None:
         out.update({"gate_up": way(fusion.library_gate_up), "down": way(fusion.library_down, fusion.split_down),
                     "tiles_gate_up": "/".join(map(str, fusion.tiles_gate_up)),

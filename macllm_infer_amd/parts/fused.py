@@ -73,7 +73,12 @@ TILE_MARGIN = 0.95             # a wider tile has to be this much faster than on
 FORCE_TILES: Optional[int] = None         # tests: this many tiles for steps of more than 16 rows instead of the clock
 # The library's tile for a prompt portion's input projection depends on the number of output features: 4 120
 # of them (0.5B-shaped) take 30.5 us at 2,048 rows, 4 352 (a multiple of 256) take 23.6.  Measured at build in
-# the same way; where padding pays, the prompt path multiplies with zero rows added and ignores their columns.
+# the same way, for portions of up to 256, 512, 1,024 and 2,048 tokens and beyond (each at its upper edge, the
+# last at 4,096); where padding pays, the prompt path multiplies with zero rows added and ignores their columns.
+PAD_FEATURES = 256
+PAD_ROWS = (256, 512, 1024, 2048, 4096)
+PAD_MARGIN = 0.95
+FORCE_PADDING: Optional[bool] = None      # tests: True or False instead of the clock
 # The attended heads of a decode step come in runs of keys that a small kernel merges; the output projection
 # can merge them in its prologue instead, every workgroup of it again: one launch less, but the projection then
 # starts behind a read of the runs.  It pays while a workgroup reads few of them (0.5B-shaped at 2,048-token
@@ -82,11 +87,7 @@ FORCE_TILES: Optional[int] = None         # tests: this many tiles for steps of 
 MERGE_LATER_ROWS = 16
 MERGE_LATER_BYTES = 96 << 10
 FORCE_MERGE_LATER: Optional[bool] = None  # tests: True or False instead of the rule
-PAD_FEATURES = 256
-PAD_ROWS = 2048
-PAD_MARGIN = 0.95
-FORCE_PADDING: Optional[bool] = None      # tests: True or False instead of the clock
-_padding_wins: Dict[tuple, bool] = {}
+_padding_wins: Dict[tuple, tuple] = {}
 
 
 OVERLAP_MIN_TOKENS = 256       # prompt portions from this size on run their two mixers on two streams
@@ -142,30 +143,41 @@ def _graph_microseconds(run) -> float:
     return best
 
 
-def _padding_pays(weight: torch.Tensor) -> bool:
-    """Whether rows of zeros up to a multiple of PAD_FEATURES make the library's product of a prompt portion faster."""
+def _padding_pays(weight: torch.Tensor) -> tuple:
+    """For every portion size of PAD_ROWS: whether rows of zeros up to a multiple of PAD_FEATURES make the
+    library's product of a prompt portion faster."""
     N, K = weight.shape
     if N % PAD_FEATURES == 0 or FORCE_PADDING is False:
-        return False
+        return (False,) * len(PAD_ROWS)
     if FORCE_PADDING:
-        return True
+        return (True,) * len(PAD_ROWS)
     if weight.numel() < LIBRARY_MIN_WEIGHT:
-        return False
+        return (False,) * len(PAD_ROWS)
     key = (N, K)
     if key not in _padding_wins:
-        x = torch.full((PAD_ROWS, K), 0.01, dtype=torch.bfloat16, device=weight.device)
         padded = torch.cat([weight, weight.new_zeros((-N % PAD_FEATURES, K))])
+        wins = []
+        for rows in PAD_ROWS:
+            x = torch.full((rows, K), 0.01, dtype=torch.bfloat16, device=weight.device)
 
-        def plain():
-            for _ in range(4):
-                torch.matmul(x, weight.t())
+            def plain():
+                for _ in range(4):
+                    torch.matmul(x, weight.t())
 
-        def wide():
-            for _ in range(4):
-                torch.matmul(x, padded.t())
+            def wide():
+                for _ in range(4):
+                    torch.matmul(x, padded.t())
 
-        _padding_wins[key] = _graph_microseconds(wide) < PAD_MARGIN * _graph_microseconds(plain)
+            wins.append(_graph_microseconds(wide) < PAD_MARGIN * _graph_microseconds(plain))
+        _padding_wins[key] = tuple(wins)
     return _padding_wins[key]
+
+
+def _portion_bucket(rows: int) -> int:
+    for bucket, most in enumerate(PAD_ROWS):
+        if rows <= most:
+            return bucket
+    return len(PAD_ROWS) - 1
 
 
 def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool, tiles: int) -> tuple:
@@ -296,7 +308,8 @@ class LayerFusion:
         self.b_in = _cat_bias(in_linears, device)
         # prompt portions may multiply with rows of zeros added (the decode kernels take the rows that count)
         self.w_in_wide, self.b_in_wide = self.w_in, self.b_in
-        if _padding_pays(self.w_in):
+        self.padding_pays = _padding_pays(self.w_in)          # by portion size
+        if any(self.padding_pays):
             extra = -self.w_in.shape[0] % PAD_FEATURES
             self.w_in_wide = torch.cat([self.w_in, self.w_in.new_zeros((extra, self.w_in.shape[1]))])
             self.w_in = self.w_in_wide[:self.w_in.shape[0]]
@@ -392,7 +405,10 @@ class LayerFusion:
     def forward_general(self, residual: Residual, step, caches) -> None:
         block = self.block
         normed = block.mixer_norm.forward(residual)
-        u = ops.linear(normed, self.w_in_wide, self.b_in_wide)
+        if self.padding_pays[_portion_bucket(normed.shape[0])]:
+            u = ops.linear(normed, self.w_in_wide, self.b_in_wide)
+        else:
+            u = ops.linear(normed, self.w_in, self.b_in)
         mixed = torch.empty((u.shape[0], self.mixed_width), dtype=u.dtype, device=u.device)
         if (len(self.mixers) == 2 and u.shape[0] >= OVERLAP_MIN_TOKENS and torch.cuda.is_current_stream_capturing()
                 and all(getattr(mixer, "graph_safe", False) for mixer in self.mixers)):
