@@ -152,22 +152,7 @@ def microbench() -> int:
 def choices_of(engine) -> dict:
     """What the first layer's fast path chose for steps of up to 8 / 16 / 32 / 48 / 64 rows, as short strings
     (S: the skinny kernel, L: the library, a number: that many slabs over K; empty when the layer has none)."""
-    fusion = getattr(engine.model.blocks[0], "fusion", None)
-    if fusion is None or not getattr(fusion, "decode_ok", False):
-        return {}
-
-    def way(library, split=None):
-        split = split or (0,) * len(library)
-        return "/".join(str(slabs) if slabs else ("L" if lib else "S") for lib, slabs in zip(library, split))
-
-    out = {"in": way(fusion.library_in), "out": way(fusion.library_out, fusion.split_out),
-           "tiles_in": "/".join(map(str, fusion.tiles_in)), "tiles_out": "/".join(map(str, fusion.tiles_out)),
-           "padded_in": "/".join("P" if pays else "-" for pays in fusion.padding_pays)}
-    if fusion.gate_up is not None:
-        out.update({"gate_up": way(fusion.library_gate_up), "down": way(fusion.library_down, fusion.split_down),
-                    "tiles_gate_up": "/".join(map(str, fusion.tiles_gate_up)),
-                    "tiles_down": "/".join(map(str, fusion.tiles_down))})
-    return out
+    return engine.path_choices()
 
 
 def main() -> int:

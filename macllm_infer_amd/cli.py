@@ -27,6 +27,9 @@ def _runtime_arguments(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--device", default="hip", choices=["hip"], help="backend (one MI355X)")
     parser.add_argument("--dtype", default="bf16", choices=["f32", "bf16", "float32", "bfloat16"],
                         help="activation dtype; f32 runs every product in true 32-bit")
+    parser.add_argument("--fixed-paths", action="store_true",
+                        help="no timing of alternative kernels when the model is built: the same kernels, and the "
+                             "same bits in bfloat16, in every process (slower on large models)")
     parser.add_argument("--kv-cache-block-tokens", type=int, default=16, help="tokens per cache page")
     parser.add_argument("--kv-cache-capacity-tokens", type=int, default=None,
                         help="token capacity of the cache shared by all requests (default: one model context)")
@@ -46,7 +49,7 @@ def _run(args) -> int:
     budget = max(args.scheduler_token_budget, 1)
     quantum = min(args.prefill_token_quantum or budget, budget)
     llm = LLM(args.model, dtype=args.dtype, kv_cache_block_tokens=args.kv_cache_block_tokens,
-              kv_cache_capacity_tokens=args.kv_cache_capacity_tokens,
+              kv_cache_capacity_tokens=args.kv_cache_capacity_tokens, measured_paths=not args.fixed_paths,
               engine_config=EngineConfig(max_active_sequences=args.max_active_sequences,
                                          scheduler_token_budget=budget, prefill_token_quantum=quantum))
     params = SamplingParams(max_new_tokens=args.max_new_tokens, temperature=args.temperature, top_k=args.top_k,

@@ -65,11 +65,14 @@ class Engine:
     def __init__(self, model_dir: Optional[str] = None, *, config=None, tensors=None, dtype="bfloat16",
                  device="cuda:0", kv_cache_block_tokens: int = 16,
                  kv_cache_capacity_tokens: Optional[int] = None, max_active_sequences: int = 8,
-                 check_device: bool = True, decode_graphs: bool = True):
+                 check_device: bool = True, decode_graphs: bool = True, measured_paths: bool = True):
         """Load from ``model_dir`` (config.json + safetensors), or from a config object (or raw
         dict) plus a name -> tensor mapping.  ``kv_cache_capacity_tokens`` defaults to one
         model context shared by all requests (reference: src/runtime.rs:175-201).  With
-        ``decode_graphs`` steps made of single tokens run as captured HIP graphs."""
+        ``decode_graphs`` steps run as captured HIP graphs.  ``measured_paths``: where two kernels can
+        serve a projection, the layers time both when the model is built and take the faster
+        (``path_choices()`` says which); False: fixed rules only, so that the same kernels run in every
+        process and bfloat16 results are the same bits from run to run."""
         self.dtype = resolve_dtype(dtype)
         self.device = ops.require_gpu(device) if check_device else torch.device(device)
         if model_dir is not None:
@@ -88,7 +91,7 @@ class Engine:
         bound = bind(source, DecoderModel.expected_tensors(self.spec), DecoderModel.tensor_copies(self.spec))
         source.close()
         build = BuildContext(hidden_size=self.spec.hidden_size, dtype=self.dtype, device=self.device,
-                             max_context=self.spec.max_context)
+                             max_context=self.spec.max_context, measure_paths=measured_paths)
         self.model = DecoderModel(self.spec, bound, build)
         needs, shared = DecoderModel.cache_layout(self.spec)
         capacity = kv_cache_capacity_tokens or self.spec.max_context
@@ -100,6 +103,13 @@ class Engine:
         if decode_graphs and check_device and self.model.graph_safe:
             from .graphs import DecodeGraphs
             self.graphs = DecodeGraphs(self.model, self.cache, self.device, min(self.max_context, capacity))
+
+    def path_choices(self) -> dict:
+        """What the first layer's fast path chose at build (empty when the layer has none): to be recorded
+        beside a result, since a close call of the clock can fall either way from one process to the next."""
+        fusion = getattr(self.model.blocks[0], "fusion", None) if self.model.blocks else None
+        choices = getattr(fusion, "path_choices", None)
+        return choices() if choices is not None else {}
 
     def warm_up(self, steps, context: int = 2048) -> list:
         """Capture the graphs of steps of (lanes, tokens) before the first request comes (a serving process

@@ -54,10 +54,10 @@ class LLM:
 
     def __init__(self, model: Union[str, Engine], dtype: str = "bfloat16", device: str = "cuda:0",
                  kv_cache_block_tokens: int = 16, kv_cache_capacity_tokens: Optional[int] = None,
-                 engine_config: Optional[EngineConfig] = None):
+                 engine_config: Optional[EngineConfig] = None, measured_paths: bool = True):
         """``model``: a folder with config.json and model.safetensors, or an ``Engine`` that is
         already built (its own dtype and cache sizes then hold; it needs a state slot for each of
-        ``engine_config.max_active_sequences``)."""
+        ``engine_config.max_active_sequences``).  ``measured_paths``: as for ``Engine``."""
         self.engine_config = engine_config or EngineConfig()
         if isinstance(model, Engine):
             self.engine = model
@@ -67,7 +67,8 @@ class LLM:
         else:
             self.engine = Engine(model, dtype=dtype, device=device, kv_cache_block_tokens=kv_cache_block_tokens,
                                  kv_cache_capacity_tokens=kv_cache_capacity_tokens,
-                                 max_active_sequences=self.engine_config.max_active_sequences)
+                                 max_active_sequences=self.engine_config.max_active_sequences,
+                                 measured_paths=measured_paths)
         self.sampler = Sampler(self.engine.vocab_size, self.engine.device)
         eos = getattr(self.engine.config, "eos_token_id", None)
         self.stop_token_ids = () if eos is None else (eos,)

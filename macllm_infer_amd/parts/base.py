@@ -53,6 +53,10 @@ class BuildContext:
     dtype: torch.dtype            # activation dtype: torch.float32 or torch.bfloat16
     device: torch.device
     max_context: int
+    # Where two kernels can serve a product, a fast path may time both when the model is built and take the
+    # faster one; False: fixed rules only, so that which kernel runs (and with it the last bits of bfloat16
+    # results) is the same in every process.
+    measure_paths: bool = True
 
 
 class Residual:

@@ -143,11 +143,11 @@ def _graph_microseconds(run) -> float:
     return best
 
 
-def _padding_pays(weight: torch.Tensor) -> tuple:
+def _padding_pays(weight: torch.Tensor, measure: bool = True) -> tuple:
     """For every portion size of PAD_ROWS: whether rows of zeros up to a multiple of PAD_FEATURES make the
     library's product of a prompt portion faster."""
     N, K = weight.shape
-    if N % PAD_FEATURES == 0 or FORCE_PADDING is False:
+    if N % PAD_FEATURES == 0 or FORCE_PADDING is False or (FORCE_PADDING is None and not measure):
         return (False,) * len(PAD_ROWS)
     if FORCE_PADDING:
         return (True,) * len(PAD_ROWS)
@@ -293,6 +293,7 @@ class LayerFusion:
         self.block = block
         device = build.device
         self.hidden = build.hidden_size
+        self.measure = bool(getattr(build, "measure_paths", True))
         self.names = [name for name, _ in block.mixers]
         self.mixers = [mixer for _, mixer in block.mixers]
         in_linears, out_linears = [piece[0] for piece in pieces], [piece[1] for piece in pieces]
@@ -308,7 +309,7 @@ class LayerFusion:
         self.b_in = _cat_bias(in_linears, device)
         # prompt portions may multiply with rows of zeros added (the decode kernels take the rows that count)
         self.w_in_wide, self.b_in_wide = self.w_in, self.b_in
-        self.padding_pays = _padding_pays(self.w_in)          # by portion size
+        self.padding_pays = _padding_pays(self.w_in, self.measure)          # by portion size
         if any(self.padding_pays):
             extra = -self.w_in.shape[0] % PAD_FEATURES
             self.w_in_wide = torch.cat([self.w_in, self.w_in.new_zeros((extra, self.w_in.shape[1]))])
@@ -381,6 +382,26 @@ class LayerFusion:
             self.f_gate_up = fragments(self.gate_up.weight, self.library_gate_up, ())
             self.f_down = fragments(self.down.weight, self.library_down, self.split_down)
 
+    def path_choices(self) -> dict:
+        """Which way each projection goes for steps of up to TUNE_ROWS rows, as short strings (S: the skinny
+        kernel, L: the library, a number: that many slabs over K), the feature tiles of the skinny kernel, and
+        for portions of up to PAD_ROWS tokens whether the input projection is padded (P)."""
+        if not self.decode_ok:
+            return {}
+
+        def way(library, split=None):
+            split = split or (0,) * len(library)
+            return "/".join(str(slabs) if slabs else ("L" if lib else "S") for lib, slabs in zip(library, split))
+
+        out = {"in": way(self.library_in), "out": way(self.library_out, self.split_out),
+               "tiles_in": "/".join(map(str, self.tiles_in)), "tiles_out": "/".join(map(str, self.tiles_out)),
+               "padded_in": "/".join("P" if pays else "-" for pays in self.padding_pays)}
+        if self.gate_up is not None:
+            out.update({"gate_up": way(self.library_gate_up), "down": way(self.library_down, self.split_down),
+                        "tiles_gate_up": "/".join(map(str, self.tiles_gate_up)),
+                        "tiles_down": "/".join(map(str, self.tiles_down))})
+        return out
+
     def decode_supported(self, step, caches) -> bool:
         if step.max_query_len != 1 or step.num_tokens > MAX_ROWS or not self.decode_ok:
             return False
@@ -452,7 +473,7 @@ class LayerFusion:
         if FORCE_SPLIT:
             slabs = FORCE_SPLIT if weight.shape[1] // 32 >= FORCE_SPLIT else 0
             return tuple(slabs if bucket in WIDE_BUCKETS else 0 for bucket in range(BUCKETS)), tiles
-        if weight.numel() < LIBRARY_MIN_WEIGHT:
+        if weight.numel() < LIBRARY_MIN_WEIGHT or not self.measure:
             return _each(0), tiles
         slabs, split_tiles = [], []
         for bucket in range(BUCKETS):
@@ -470,7 +491,8 @@ class LayerFusion:
     def _tune_all(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict], normed: bool) -> tuple:
         forced = 1 if FORCE_TILES is None else FORCE_TILES
         fixed_tiles = tuple(forced if bucket in WIDE_BUCKETS else 1 for bucket in range(BUCKETS))
-        if not self.general or FORCE_LIBRARY is False or (FORCE_LIBRARY is None and weight.numel() < LIBRARY_MIN_WEIGHT):
+        if (not self.general or FORCE_LIBRARY is False
+                or (FORCE_LIBRARY is None and (weight.numel() < LIBRARY_MIN_WEIGHT or not self.measure))):
             return _each(False), fixed_tiles
         if FORCE_LIBRARY:
             return _each(True), fixed_tiles

@@ -363,6 +363,36 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
         assert ((have - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()).item() <= 3e-2
 
 
+def test_fixed_paths_take_no_measurement(tmp_path, monkeypatch):
+    """``measured_paths=False``: even where every weight would be timed (the limit lowered to 0), the layers take
+    the fixed rules, the same in every process, and say so; the engine that measures reports a choice for each
+    of the five step sizes.  Both decode 24 lanes like the plain model."""
+    import gates
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.parts import fused
+    monkeypatch.setattr(fused, "LIBRARY_MIN_WEIGHT", 0)
+    folder = tiny_configs.make_model_dir("C", tmp_path, torch.bfloat16)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    prompts = {index: tokens_for(cfg["vocab_size"], 5 + index % 4, 900 + index) for index in range(24)}
+    for measured in (False, True):
+        engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * 24,
+                        max_active_sequences=24, measured_paths=measured)
+        choices = engine.path_choices()
+        assert set(choices) == {"in", "out", "gate_up", "down", "tiles_in", "tiles_out", "tiles_gate_up", "tiles_down",
+                                "padded_in"}
+        assert all(len(value.split("/")) == 5 for value in choices.values())
+        if not measured:
+            assert choices["in"] == choices["out"] == choices["gate_up"] == choices["down"] == "S/S/S/S/S"
+            assert choices["tiles_in"] == choices["tiles_down"] == "1/1/1/1/1" and choices["padded_in"] == "-/-/-/-/-"
+        for index in prompts:
+            engine.add_request(index)
+        engine.step([Lane(index, tokens[:-1], []) for index, tokens in prompts.items()])
+        logits = engine.step([Lane(index, tokens[-1:], [0]) for index, tokens in prompts.items()]).float().cpu()
+        for row, tokens in enumerate(prompts.values()):
+            want = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-1]
+            assert gates.bfloat16_close(logits[row].numpy(), want.numpy()), (measured, row)
+
+
 def test_the_output_projection_may_merge_the_runs_of_keys(monkeypatch):
     """Steps of up to 16 single tokens: whether the runs of keys of the attended heads are merged by a kernel of
     their own or in the prologue of the output projection, the logits are the same bit for bit, with contexts
