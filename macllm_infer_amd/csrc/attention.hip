@@ -748,19 +748,22 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
 extern "C" int mi_prefill_attention(const void* q, long q_ld, int Hq, int Hkv, int dh, const void* k_base,
                                     const void* v_base, long page_stride, int page_size, const int* block_tables,
                                     int max_pages, const int* tiles, int n_tiles, const int* cu_seqlens,
-                                    const int* start_pos, float scale, int window, void* out, long out_ld,
-                                    hipStream_t stream) {
+                                    const int* start_pos, float scale, int window, int max_seq_len, void* out,
+                                    long out_ld, hipStream_t stream) {
   if (n_tiles <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || page_size <= 0 || max_pages <= 0)
     return ERR_BAD_ARGUMENT;
   const int G = Hq / Hkv;
   if ((dh != 64 && dh != 128) || page_size % 4 != 0 || q_ld % 8 != 0 || out_ld % 4 != 0 || Hkv > 65535 || G > 64)
     return ERR_UNSUPPORTED_SIZE;
   // up to four query heads share every K and V fragment; head size 128 holds twice the registers per head, and
-  // more than two heads would spill.  A grid that would leave compute units with fewer than two workgroups is
+  // more than two heads would spill.  A grid that would leave compute units with fewer than two workgroups, over
+  // contexts of up to 2,048 keys (max_seq_len: an upper bound of the step's longest context, 0 = not known), is
   // bound by the softmax arithmetic of its longest tiles: it takes sets of two heads, so that twice the
-  // workgroups, every other pass from the light end, spread that work
+  // workgroups, every other pass from the light end, spread that work.  Over longer contexts the keys and
+  // values that four heads share count for more (a 2,048-token portion of the 0.5B shape behind 2,048 tokens
+  // of context: 7.29 ms with two heads a set, 6.85 with four; behind 30,000 tokens 19.0 and 16.4).
   int most = dh == 128 ? 2 : 4;
-  if (most > 2 && 4L * n_tiles * Hkv * ((G + most - 1) / most) < PREFILL_FILL_BLOCKS) most = 2;
+  if (most > 2 && max_seq_len <= 2048 && 4L * n_tiles * Hkv * ((G + most - 1) / most) < PREFILL_FILL_BLOCKS) most = 2;
   const int passes = (G + most - 1) / most;
   const int nset = (G + passes - 1) / passes;
   if (n_tiles > (1 << 28)) return ERR_UNSUPPORTED_SIZE;

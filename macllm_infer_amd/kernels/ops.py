@@ -46,7 +46,8 @@ _SIGNATURES = {
                                _c_ptr, _c_long, _c_ptr],
         "mi_paged_attention_workspace": [_c_int, _c_int, _c_int, _c_int],
         "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
-                                 _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_long, _c_ptr],
+                                 _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_long,
+                                 _c_ptr],
         "mi_decode_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int,
                                 _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
                                 _c_ptr, _c_long, _c_ptr],
@@ -372,10 +373,12 @@ def prefill_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_d
 def prefill_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, block_tables: torch.Tensor, query_tiles: torch.Tensor,
                       cu_seqlens: torch.Tensor, start_pos: torch.Tensor, scale: float, window: Optional[int],
-                      out: torch.Tensor) -> None:
+                      out: torch.Tensor, max_seq_len: int = 0) -> None:
     """``paged_attention`` on the matrix cores for bfloat16 (flash-style, online softmax in
     float32).  ``query_tiles`` [tiles, 2]: (lane, first token row) of runs of up to 64 tokens of
-    one lane; the keys and values of the step's own tokens must be in the cache already."""
+    one lane; the keys and values of the step's own tokens must be in the cache already.
+    ``max_seq_len``: an upper bound of the step's longest context if known (it picks how many heads share
+    a key fragment, never the result)."""
     q_ld = _row_major(q, "q")
     out_ld = _row_major(out, "out")
     T = q.shape[0]
@@ -394,7 +397,8 @@ def prefill_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     _check(_fn("attention", "mi_prefill_attention")(
         _p(q), q_ld, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride, page_size,
         _p(block_tables), block_tables.shape[1], _p(query_tiles), query_tiles.shape[0], _p(cu_seqlens),
-        _p(start_pos), float(scale), int(window or 0), _p(out), out_ld, _stream()), "prefill_attention")
+        _p(start_pos), float(scale), int(window or 0), int(max_seq_len or 0), _p(out), out_ld, _stream()),
+        "prefill_attention")
 
 
 def decode_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> bool:

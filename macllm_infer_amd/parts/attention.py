@@ -99,7 +99,7 @@ class Attention(Mixer):
         elif ops.prefill_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2]):
             ops.prefill_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                   step.query_tiles, step.cu_seqlens, step.start_pos, spec.scale, spec.window,
-                                  attended)
+                                  attended, step.max_seq_len)
         else:
             ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                 step.lane_of_token, step.positions, spec.scale, spec.window, attended,
