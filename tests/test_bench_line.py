@@ -29,6 +29,19 @@ def test_more_than_one_gpu_is_refused_in_one_line():
     assert len(printed.strip().splitlines()) == 1 and "--gpus 2" in printed
 
 
+def test_the_shape_is_written_as_a_config_json(tmp_path):
+    """What the kernel-trace summary reads as --config: the shape's keys with the number of layers asked for,
+    and the configuration class reads it back."""
+    from macllm_infer_amd.config.registry import config_from_dict
+    path = tmp_path / "config.json"
+    code, printed = run_bench(["--shape", "7b", "--layers", "12", "--write-config", str(path)])
+    assert code == 0 and printed == ""
+    raw = json.loads(path.read_text())
+    assert raw == dict(bench.SHAPES["7b"], num_hidden_layers=12)
+    spec = config_from_dict(raw).to_model_spec()
+    assert len(spec.layers) == 12 and spec.hidden_size == 3072
+
+
 @pytest.mark.gpu
 def test_line_of_a_short_run():
     code, printed = run_bench(["--layers", "2", "--steps", "3", "--warmup", "2"])
@@ -92,3 +105,44 @@ def test_costs_of_the_headline_step_are_the_ones_worked_out_by_hand():
     assert costs.group_of("void fused_gemm_kernel<1, 1, 0, 8, 1>(FusedGemmParams)", costs.DECODE_GROUPS) \
         == "output projections + down projections"
     assert costs.merged(step, "output projections + down projections").read == pytest.approx(302.0e6, rel=1e-3)
+
+
+def test_kernel_trace_summary_of_a_made_up_trace(tmp_path, capsys):
+    """``utils.kernel_trace`` on a small made-up trace database: the last step from its first kernel to its last,
+    launches, busy time and span, the kernels by total time, the roofline table from a model's sizes, and the
+    launches one by one with the idle time before each."""
+    import sqlite3
+    from macllm_infer_amd.utils import kernel_trace
+    database = tmp_path / "trace.db"
+    connection = sqlite3.connect(database)
+    connection.execute("create table kernels (name text, start integer, end integer)")
+    rows = []
+    for step in range(2):                                     # two steps; the second one is summarized
+        base = 1_000_000 * step
+        rows += [("embed_kernel", base, base + 4_000),
+                 ("void fused_gemm_kernel<1, 0, 2, 4, 1>(FusedGemmParams)", base + 4_000, base + 12_000),
+                 ("void mixer_decode_kernel<64>(MixerParams)", base + 12_000, base + 24_000),
+                 ("side_kernel", base + 13_000, base + 15_000),                 # beside the mixer, on another queue
+                 ("void fused_gemm_kernel<1, 0, 2, 4, 1>(FusedGemmParams)", base + 30_000, base + 38_000),
+                 ("argmax_kernel(float const*, int, int*)", base + 38_000, base + 45_000)]
+    connection.executemany("insert into kernels values (?, ?, ?)", rows)
+    connection.commit()
+    connection.close()
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(dict(bench.SHAPES["0.5b"], num_hidden_layers=1)))
+    saved = sys.argv
+    sys.argv = ["kernel_trace", str(database), "--first", "embed_kernel", "--last", "argmax", "--config", str(config),
+                "--batch", "8", "--context", "2060", "--timeline", "0:6"]
+    try:
+        kernel_trace.main()
+    finally:
+        sys.argv = saved
+    printed = capsys.readouterr().out
+    assert "launches 6   busy 41.0 us   span 45.0 us" in printed
+    lines = printed.splitlines()
+    first = next(line for line in lines if line.startswith("void fused_gemm_kernel"))
+    assert first.split()[-4:] == ["2", "16.0", "8.00", "39.0%"]                   # calls, total, average, share
+    assert any(line.startswith("input projections") for line in lines) and any("the step (all kernels" in line for line in lines)
+    timeline = [line.split() for line in lines if line.strip() and line.split()[0].isdigit()]
+    assert [row[0] for row in timeline] == ["0", "1", "2", "3", "4", "5"]
+    assert timeline[3][3] == "-11.00" and timeline[4][3] == "6.00"              # beside the mixer; a gap of 6 us before the next
