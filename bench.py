@@ -254,19 +254,29 @@ def main() -> int:
         tokens = torch.randint(0, vocab, (batch,), generator=generator).tolist()
         rows = [SamplerRow(GREEDY, (), ()) for _ in names]
 
-        def decode_step(tokens):
-            logits = engine.step([Lane(name, [token], [0]) for name, token in zip(names, tokens)])
-            return sampler.sample(logits, rows)
+        # a step is queued before the host has read the tokens of the step before it (they are fed on the
+        # device), as the scheduler does it; the host reads them while the GPU works
+        def decode_step(before):
+            if before is None:
+                lanes = [Lane(name, [token], [0]) for name, token in zip(names, tokens)]
+            else:
+                lanes = [Lane(name, [0], [0], feed=(before.device, row)) for row, name in enumerate(names)]
+            return sampler.sample_async(engine.step(lanes), rows)
 
+        on_their_way = decode_step(None)
         for _ in range(args.warmup):
-            tokens = decode_step(tokens)
+            newer = decode_step(on_their_way)
+            on_their_way.wait()
+            on_their_way = newer
         synchronize()
         step_times = []
         started = time.perf_counter()
-        for _ in range(args.steps):                   # a step ends with its tokens on the host: each can be timed
-            before = time.perf_counter()
-            tokens = decode_step(tokens)
-            step_times.append(time.perf_counter() - before)
+        for _ in range(args.steps):                   # a step's time: from one step's tokens on the host to the next's
+            tick = time.perf_counter()
+            newer = decode_step(on_their_way)
+            on_their_way.wait()
+            on_their_way = newer
+            step_times.append(time.perf_counter() - tick)
         synchronize()
         seconds = time.perf_counter() - started
         for name in names:

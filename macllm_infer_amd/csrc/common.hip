@@ -26,6 +26,41 @@ extern "C" int mi_embed(const int* ids, const void* table, int table_dtype, floa
   return 0;
 }
 
+// ---------------------------------------------------------------- tokens fed from the device
+// token_ids[dst[i]] = source[src[i]]: the tokens that the sampler left on the device for the step before go
+// into this step's token ids without a round trip through the host (the host learns them one step late).
+// The pairs travel in the launch's arguments, 64 a launch: no memory of their own.
+#define FEED_PAIRS 64
+struct FeedPairs {
+  int dst[FEED_PAIRS];
+  int src[FEED_PAIRS];
+};
+
+__global__ void feed_tokens_kernel(int* __restrict__ token_ids, const int* __restrict__ source, int count, FeedPairs pairs) {
+  const int i = threadIdx.x;
+  if (i < count) token_ids[pairs.dst[i]] = source[pairs.src[i]];
+}
+
+// dst, src: host arrays of `count` indices; every dst below tokens, every src below sources (checked here).
+extern "C" int mi_feed_tokens(int* token_ids, int tokens, const int* source, int sources, const int* dst,
+                              const int* src, int count, hipStream_t stream) {
+  if (count < 0 || tokens <= 0 || sources <= 0 || !token_ids || !source || (count > 0 && (!dst || !src)))
+    return ERR_BAD_ARGUMENT;
+  for (int i = 0; i < count; ++i)
+    if (dst[i] < 0 || dst[i] >= tokens || src[i] < 0 || src[i] >= sources) return ERR_BAD_ARGUMENT;
+  for (int first = 0; first < count; first += FEED_PAIRS) {
+    FeedPairs pairs = {};
+    const int n = count - first < FEED_PAIRS ? count - first : FEED_PAIRS;
+    for (int i = 0; i < n; ++i) {
+      pairs.dst[i] = dst[first + i];
+      pairs.src[i] = src[first + i];
+    }
+    feed_tokens_kernel<<<1, FEED_PAIRS, 0, stream>>>(token_ids, source, n, pairs);
+    RETURN_IF_LAUNCH_FAILED();
+  }
+  return 0;
+}
+
 // ---------------------------------------------------------------- add + rmsnorm
 // For each processed row r:  v = h[r] (+ delta0[r]) (+ delta1[r]);  if update: h[r] = v;
 // out[i] = v / sqrt(mean(v^2) + eps) * weight.

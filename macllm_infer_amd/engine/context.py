@@ -31,6 +31,9 @@ class Lane:
     request: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = ()         # places among ``tokens`` whose logits are asked for
+    # (int32 tensor on the device, row): the lane's one token is not known to the host yet; it is that element
+    # of the tensor (what a sampler left there for the step before) and ``tokens`` holds any valid id in its place
+    feed: Optional[tuple] = None
 
 
 @dataclass
@@ -64,6 +67,7 @@ class LoweredLanes:
     tokens: np.ndarray           # [T] all lanes' tokens, lane after lane
     want_counts: np.ndarray      # [lanes] wanted places of each lane
     wants: np.ndarray            # [wanted] the places, lane after lane
+    feeds: tuple = ()            # (token row, int32 tensor on the device, its row) of tokens the host does not know yet
 
 
 def lower_lanes(lanes: Sequence[Lane], cache) -> LoweredLanes:
@@ -80,6 +84,21 @@ def lower_lanes(lanes: Sequence[Lane], cache) -> LoweredLanes:
     if wants.size and (wants.min() < -(1 << 31) or wants.max() >= (1 << 31)):
         raise OverflowError("a wanted place does not fit 32 bits")
     return LoweredLanes(slots, lengths, tokens.astype(np.int32), want_counts, wants.astype(np.int32))
+
+
+def apply_feeds(token_ids: torch.Tensor, feeds) -> None:
+    """Write the tokens that are still on the device into the step's token ids (after their upload, before the
+    forward pass or the graph's replay, on the same stream)."""
+    if not feeds:
+        return
+    from ..kernels import ops
+    by_source = {}
+    for row, source, index in feeds:
+        by_source.setdefault(id(source), (source, [], []))
+        by_source[id(source)][1].append(row)
+        by_source[id(source)][2].append(index)
+    for source, rows, indices in by_source.values():
+        ops.feed_tokens(token_ids, source, rows, indices)
 
 
 _NO_LANES = LoweredLanes(*(np.zeros(0, dtype=np.int32) for _ in range(5)))

@@ -29,7 +29,7 @@ from ..kernels import build as kernel_build
 from ..kernels import ops
 from ..parts.base import BuildContext
 from ..weights.loader import WeightSource, bind
-from .context import Lane, LoweredLanes, build_step_context, lower_lanes
+from .context import Lane, LoweredLanes, apply_feeds, build_step_context, lower_lanes
 from .model import DecoderModel
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
@@ -168,6 +168,20 @@ class Engine:
             where = int(np.argmax(beyond))
             raise StepError(f"request {names[where]!r}: {int(starts[where])} + {int(lengths[where])} "
                             f"tokens exceed the context limit {self.max_context}")
+        if any(lane.feed is not None for lane in lanes):
+            first_rows = np.concatenate(([0], np.cumsum(lengths)[:-1]))
+            feeds = []
+            for index, lane in enumerate(lanes):
+                if lane.feed is None:
+                    continue
+                source, row = lane.feed
+                if int(lengths[index]) != 1:
+                    raise StepError(f"request {names[index]!r}: a lane fed from the device holds one token")
+                if not (isinstance(source, torch.Tensor) and source.dtype == torch.int32 and source.dim() == 1
+                        and 0 <= int(row) < source.numel()):
+                    raise StepError(f"request {names[index]!r}: the feed must be (an int32 vector, a row of it)")
+                feeds.append((int(first_rows[index]), source, int(row)))
+            lowered.feeds = tuple(feeds)
         if lowered.wants.size:
             lane_of_want = np.repeat(np.arange(len(lanes)), lowered.want_counts)
             outside = (lowered.wants < 0) | (lowered.wants >= lengths[lane_of_want])
@@ -178,10 +192,14 @@ class Engine:
                                 f"its {int(lengths[lane])} tokens")
         return lowered
 
+    feeds_tokens = True          # a lane's token may come from the device (``Lane.feed``)
+
     def step(self, lanes: Sequence[Lane]) -> torch.Tensor:
         """Run one batch; returns float32 logits [wanted, vocab] in the order of the lanes and
         of each lane's ``want``.  Raises StepError or CacheExhausted with nothing changed, or
-        StepFailed with the lanes' requests ended and everything they held given back."""
+        StepFailed with the lanes' requests ended and everything they held given back.  The work is
+        queued on the GPU; nothing here waits for it (a lane with ``feed`` takes its token from the device,
+        so a caller may queue the next step before it has read this one's tokens)."""
         lowered = self.validate(lanes)
         self.cache.reserve_slots(lowered.slots, lowered.lengths)
         try:
@@ -194,6 +212,7 @@ class Engine:
             if logits is None:
                 context = build_step_context(lanes, self.cache, self.device, lowered, self.model.query_tile,
                                              self.model.chunk_sizes)
+                apply_feeds(context.token_ids, lowered.feeds)
                 logits = self.model.forward(context, self.cache)
         except Exception as error:
             # earlier layers have written keys, values and state in place: these requests cannot go on

@@ -27,7 +27,7 @@ from typing import Dict, Iterable, List, Optional, Sequence, Tuple
 
 import torch
 
-from .context import Lane, LoweredLanes, StaticStep
+from .context import Lane, LoweredLanes, StaticStep, apply_feeds
 
 
 def bucket_for(lanes: int) -> int:
@@ -132,6 +132,7 @@ class DecodeGraphs:
             self._bucket_graphs.move_to_end(key)
         static, graph, logits = entry
         static.fill(lowered)
+        apply_feeds(static.context.token_ids, lowered.feeds)
         graph.replay()
         self.counts["bucket_replays"] += 1
         return logits[:int(lowered.want_counts.sum())].clone()
@@ -199,6 +200,7 @@ class DecodeGraphs:
             self._graphs[key] = self._capture(key[0], context=key[1])
         static, graph, logits = self._graphs[key]
         static.fill(lowered)
+        apply_feeds(static.context.token_ids, lowered.feeds)
         graph.replay()
         self.counts["decode_replays"] += 1
         if int(lowered.want_counts.min()) > 0:

@@ -18,6 +18,16 @@ Each round (reference: ``ServingScheduler::drive_once``, src/engine.rs:1938-1988
      waits never starts; one cancelled between rounds gives back what it holds before the next
      (src/engine.rs:1136-1143, 1668-1672, 1753-1765);
   5. finished requests give back pages and slot; visited ones go to the back of the line.
+
+One round ahead.  With a sampler that can leave its tokens on the device (``sample_async``) and an engine that
+can take a lane's token from there (``feeds_tokens``), a round is queued on the GPU before the tokens of the
+round before it have reached the host: a decoding request's lane is fed from the device, and the host reads
+the earlier round's tokens (emits them, applies the stop conditions) while the GPU works.  A request that
+turns out to have ended in the earlier round (a stop token, the caller's ``on_token``, a cancellation) has
+then run one token too far: that token is dropped and what the request held is given back as usual; a request
+that ends by ``max_new_tokens`` is known beforehand and is not queued again.  A request whose sampling needs
+its history on the host (penalties) waits for its tokens first, as do all rounds with a sampler or an engine
+that cannot do this (the reference reads every token before the next step, src/engine.rs:1938-1988).
 """
 from __future__ import annotations
 
@@ -63,6 +73,7 @@ class Request:
     started_at: Optional[float] = None     # admission: the request got its slot
     first_token_at: Optional[float] = None
     finished_at: Optional[float] = None
+    in_flight: Optional[tuple] = None      # (tokens still on the device, this request's row among them)
 
     @property
     def finished(self) -> bool:
@@ -98,6 +109,9 @@ class Scheduler:
         self.finished: Dict[Hashable, Request] = {}
         self.rounds = 0
         self.last_lanes: List[Lane] = []        # what the last round ran (for tests and metrics)
+        self.ahead = (getattr(sampler, "sample_async", None) is not None
+                      and bool(getattr(engine, "feeds_tokens", False)))
+        self._pending: Optional[tuple] = None   # (tokens on their way to the host, the requests they are for)
 
     # ------------------------------------------------------------------ submission
     def submit(self, request_id: Hashable, prompt: Sequence[int], params: SamplingParams) -> Request:
@@ -108,7 +122,7 @@ class Scheduler:
         return request
 
     def has_work(self) -> bool:
-        return bool(self.queue or self.active)
+        return bool(self.queue or self.active or self._pending)
 
     def cancel(self, request_id: Hashable) -> bool:
         """Cancel a waiting or live request; False if there is no such request (any more)."""
@@ -158,6 +172,11 @@ class Scheduler:
                 count = min(self.config.prefill_token_quantum, len(request.prompt) - request.cursor, budget)
                 tokens = request.prompt[request.cursor:request.cursor + count]
                 samples = request.cursor + count == len(request.prompt)
+            elif request.in_flight is not None:
+                if len(request.generated) + 1 >= request.params.max_new_tokens:
+                    continue                              # the token on its way is its last one
+                tokens = [0]                              # stands for the token that is still on the device
+                samples = True
             else:
                 tokens = [request.generated[-1]]
                 samples = True
@@ -189,15 +208,41 @@ class Scheduler:
         self.active.remove(request)
         self.finished[request.request_id] = request
 
+    def _resolve(self, pending: Optional[tuple] = None) -> None:
+        """Wait for a round's tokens and do with them what step 4 says."""
+        if pending is None:
+            pending, self._pending = self._pending, None
+        if pending is None:
+            return
+        handle, requests = pending
+        tokens_out = handle.wait()
+        now = time.perf_counter()
+        for request, token in zip(requests, tokens_out):
+            if request.in_flight is not None and request.in_flight[0] is handle:
+                request.in_flight = None
+            if not request.finished:                 # else it ended a round earlier: one token too far, dropped
+                self._complete(request, int(token), now)
+
+    def _needs_tokens_first(self) -> bool:
+        """Whether the round before has to be read before the next can be made up."""
+        if self._pending is None:
+            return False
+        return not self.ahead or any(request.params.uses_penalties and not request.finished
+                                     for request in self._pending[1])
+
     def step(self) -> List[Request]:
         """One round; returns the requests that finished in it."""
         self.rounds += 1
         done_before = set(self.finished)
+        if self._needs_tokens_first():
+            self._resolve()
         self._admit()
         visits = self._collect()
         logits = None
         while visits:
-            lanes = [Lane(request.request_id, tokens, [len(tokens) - 1] if samples else [])
+            lanes = [Lane(request.request_id, tokens, [len(tokens) - 1] if samples else [],
+                          feed=(request.in_flight[0].device, request.in_flight[1])
+                          if request.in_flight is not None and not request.prefilling else None)
                      for request, tokens, samples in visits]
             try:
                 logits = self.engine.step(lanes)
@@ -207,24 +252,39 @@ class Scheduler:
                 if len(visits) > 1:
                     visits.pop()                 # the last lane waits for a later round
                 else:
+                    self._resolve()              # whatever is on its way belongs to requests that still count
                     self._finish(visits[0][0], "resource_exhausted")
                     visits = self._collect()
             except StepFailed as failure:
                 # the engine has ended the step's requests and taken back what they held; the others go on
+                self._resolve()
                 for request, _, _ in visits:
-                    self._finish(request, f"failed: {failure.__cause__}", release=False)
+                    if not request.finished:
+                        self._finish(request, f"failed: {failure.__cause__}", release=False)
                 visits = []
+        before, self._pending = self._pending, None
         if visits:
             sampled = [(request, tokens) for request, tokens, samples in visits if samples]
             for request, tokens, samples in visits:
                 if request.prefilling:
                     request.cursor += len(tokens)
             if sampled:
-                rows = [SamplerRow(request.params, request.prompt, request.generated) for request, _ in sampled]
-                tokens_out = self.sampler.sample(logits, rows)
-                now = time.perf_counter()
-                for (request, _), token in zip(sampled, tokens_out):
-                    self._complete(request, int(token), now)
+                rows = [SamplerRow(request.params, request.prompt, request.generated,
+                                   1 if request.in_flight is not None else 0) for request, _ in sampled]
+                if self.ahead:
+                    handle = self.sampler.sample_async(logits, rows)
+                    self._pending = (handle, [request for request, _ in sampled])
+                else:
+                    tokens_out = self.sampler.sample(logits, rows)
+                    now = time.perf_counter()
+                    for (request, _), token in zip(sampled, tokens_out):
+                        self._complete(request, int(token), now)
+        if before is not None:
+            self._resolve(before)                # the GPU works on this round meanwhile
+        if self._pending is not None:
+            for row, request in enumerate(self._pending[1]):
+                request.in_flight = (self._pending[0], row)
+        if visits:
             for request, _, _ in visits:         # visited requests go to the back of the line
                 if not request.finished:
                     self.active.remove(request)

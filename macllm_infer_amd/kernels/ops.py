@@ -31,6 +31,7 @@ class KernelError(RuntimeError):
 _SIGNATURES = {
     "common": {
         "mi_embed": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_int, _c_ptr],
+        "mi_feed_tokens": [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
         "mi_add_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int,
                            _c_int, _c_ptr],
         "mi_add_partials_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int,
@@ -183,6 +184,22 @@ def embed(token_ids: torch.Tensor, table: torch.Tensor, multiplier: float, out: 
     _need(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous float32")
     _check(_fn("common", "mi_embed")(_p(token_ids), _p(table), _dt(table), float(multiplier), _p(out), T, d,
                                      _stream()), "embed")
+
+
+def feed_tokens(token_ids: torch.Tensor, source: torch.Tensor, dst: Sequence[int], src: Sequence[int]) -> None:
+    """token_ids[dst[i]] = source[src[i]] on the device (both int32): tokens that a sampler left on the
+    device go into a step's token ids without passing through the host."""
+    _i32(token_ids, "token_ids")
+    _i32(source, "source")
+    count = len(dst)
+    _need(len(src) == count, "feed_tokens: as many sources as places")
+    if count == 0:
+        return
+    places = (ctypes.c_int * count)(*[int(value) for value in dst])
+    sources = (ctypes.c_int * count)(*[int(value) for value in src])
+    _check(_fn("common", "mi_feed_tokens")(_p(token_ids), token_ids.numel(), _p(source), source.numel(),
+                                           ctypes.addressof(places), ctypes.addressof(sources), count, _stream()),
+           "feed_tokens")
 
 
 def add_rmsnorm(h: torch.Tensor, deltas: Sequence[torch.Tensor], weight: torch.Tensor, eps: float,

@@ -20,11 +20,26 @@ from .params import SamplingParams
 
 
 class SamplerRow:
-    """What the sampler needs to know of one request."""
-    __slots__ = ("params", "prompt", "generated")
+    """What the sampler needs to know of one request.  ``pending``: tokens already drawn for the request that
+    ``generated`` does not hold yet (they are still on the device); they count for the draw's index.  A row
+    with penalties needs all its tokens in ``generated``."""
+    __slots__ = ("params", "prompt", "generated", "pending")
 
-    def __init__(self, params: SamplingParams, prompt: Sequence[int], generated: Sequence[int]):
-        self.params, self.prompt, self.generated = params, prompt, generated
+    def __init__(self, params: SamplingParams, prompt: Sequence[int], generated: Sequence[int], pending: int = 0):
+        self.params, self.prompt, self.generated, self.pending = params, prompt, generated, pending
+
+
+class PendingTokens:
+    """The tokens of one ``sample_async`` call: on the device at once (``device``, int32 [B], what a next
+    step may be fed from), on the host after ``wait()``."""
+
+    def __init__(self, device: torch.Tensor, host: torch.Tensor, event):
+        self.device, self._host, self._event = device, host, event
+
+    def wait(self) -> List[int]:
+        if self._event is not None:
+            self._event.synchronize()
+        return self._host[:self.device.numel()].tolist()
 
 
 class Sampler:
@@ -41,6 +56,8 @@ class Sampler:
             kernel_build.ensure_modules(self.kernel_modules)
         self._keys = None
         self._counts = None
+        self._host_tokens: List[torch.Tensor] = []      # pinned, used in turn by the calls in flight
+        self._turn = 0
 
     def _work(self, rows: int):
         if self._keys is None or self._keys.shape[0] < rows:
@@ -53,14 +70,23 @@ class Sampler:
                             torch.zeros(rows * self.vocab_size, dtype=torch.int32, device=self.device))
         return self._counts
 
+    HOST_BUFFERS = 3               # calls whose tokens nobody has waited for yet, at most
+
     def sample(self, logits: torch.Tensor, rows: Sequence[SamplerRow]) -> List[int]:
         """One token for each row of ``logits`` [B, V] (float32; overwritten)."""
+        return self.sample_async(logits, rows).wait()
+
+    def sample_async(self, logits: torch.Tensor, rows: Sequence[SamplerRow]) -> PendingTokens:
+        """The same, without waiting: the kernels and the copy of the tokens to the host are queued, and the
+        caller waits for them when it needs them (at most HOST_BUFFERS - 1 calls later)."""
         B = len(rows)
         if logits.shape != (B, self.vocab_size):
             raise ValueError(f"logits have shape {tuple(logits.shape)}, expected {(B, self.vocab_size)}")
         device = self.device
 
         if any(row.params.uses_penalties for row in rows):
+            if any(row.pending and row.params.uses_penalties for row in rows):
+                raise ValueError("a row with penalties needs all its tokens on the host")
             tokens: List[int] = []
             offsets = [0]
             for row in rows:
@@ -93,9 +119,22 @@ class Sampler:
             words[2 * B:3 * B].view(np.float32)[:] = [row.params.temperature for row in rows]
             words[3 * B:4 * B].view(np.float32)[:] = [row.params.top_p for row in rows]
             words[4 * B:5 * B] = [row.params.top_k for row in rows]
-            words[5 * B:] = [len(row.generated) for row in rows]
+            words[5 * B:] = [len(row.generated) + row.pending for row in rows]
             packed = torch.from_numpy(words).to(device, non_blocking=True)
             ops.sample(logits, packed[2 * B:3 * B].view(torch.float32), packed[4 * B:5 * B],
                        packed[3 * B:4 * B].view(torch.float32), packed[:2 * B].view(torch.int64), packed[5 * B:],
                        self._work(B), out, torch.empty(B, dtype=torch.int32, device=device))
-        return out.cpu().tolist()
+        if self.device.type != "cuda":                 # host-side tests: nothing is in flight
+            return PendingTokens(out, out, None)
+        if len(self._host_tokens) < self.HOST_BUFFERS:
+            self._host_tokens.append(torch.empty(max(B, 64), dtype=torch.int32, pin_memory=True))
+            turn = len(self._host_tokens) - 1
+        else:
+            turn = self._turn = (self._turn + 1) % self.HOST_BUFFERS
+        if self._host_tokens[turn].numel() < B:
+            self._host_tokens[turn] = torch.empty(B, dtype=torch.int32, pin_memory=True)
+        host = self._host_tokens[turn]
+        host[:B].copy_(out, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return PendingTokens(out, host, event)

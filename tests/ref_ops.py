@@ -22,6 +22,11 @@ def embed(token_ids, table, multiplier, out):
     out.copy_(_f(table)[token_ids.long()] * multiplier)
 
 
+def feed_tokens(token_ids, source, dst, src):
+    for place, row in zip(dst, src):
+        token_ids[int(place)] = source[int(row)]
+
+
 def add_rmsnorm(h, deltas, weight, eps, out, rows=None):
     total = h.clone()
     for delta in deltas:
@@ -212,7 +217,7 @@ def argmax(logits, out):
 
 
 NAMES = ["fused_gemm_split", "add_partials_rmsnorm", "prefill_attention_supported", "decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "linear", "rope_kv_store", "paged_attention",
-         "conv1d_silu", "conv_state_update", "ssm_scan", "gate_norm", "argmax"]
+         "conv1d_silu", "conv_state_update", "ssm_scan", "gate_norm", "argmax", "feed_tokens"]
 
 
 def install(monkeypatch):

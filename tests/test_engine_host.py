@@ -254,3 +254,52 @@ def test_the_limits_are_the_ones_in_the_kernel_sources():
     from macllm_infer_amd.config import FalconH1Config
     from macllm_infer_amd.engine.model import DecoderModel
     assert DecoderModel.limits(FalconH1Config.from_dict(raw).to_model_spec()) == []
+
+
+def test_a_round_ahead_of_its_tokens_ends_requests_like_a_round_that_waits(host_ops, tmp_path):
+    """The scheduler that queues a round before it has read the tokens of the round before (tokens fed on the
+    device) and the one that reads every token first: the same tokens, finish reasons and callbacks for
+    requests that end by a stop token, by the caller's ``on_token``, by a cancellation, by their length, for a
+    request with penalties (it waits for its tokens) and under a budget that leaves requests out of rounds.
+    A request that ended one round earlier than the host knew has run one token too far: nothing of it shows,
+    and every page and slot comes back."""
+    engine, cfg, tensors = engine_for("B", tmp_path, capacity=512, page=8, requests=5)
+    prompts = [tokens_for(cfg, length, 70 + length) for length in (3, 9, 20, 5, 14, 6)]
+    greedy = dict(temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0)
+    free = [plain_impl.greedy_generate(cfg, tensors, prompt, 9) for prompt in prompts]
+    params = [SamplingParams(max_new_tokens=9, stop_token_ids=(free[0][3],), **greedy),          # a stop token on the way
+              SamplingParams(max_new_tokens=9, **greedy),                                       # the caller stops it
+              SamplingParams(max_new_tokens=9, **greedy),                                       # cancelled on the way
+              SamplingParams(max_new_tokens=4, **greedy),                                       # its length
+              SamplingParams(max_new_tokens=7, temperature=0.9, top_k=10, top_p=0.8, repetition_penalty=1.2,
+                             presence_penalty=0.3, seed=11),                                    # penalties
+              SamplingParams(max_new_tokens=8, temperature=0.8, top_k=0, top_p=1.0, repetition_penalty=1.0, seed=5)]
+    outcomes = {}
+    for ahead in (False, True):
+        sampler = Sampler(engine.vocab_size, "cpu", check_device=False)
+        emitted = []
+
+        def on_token(request, token):
+            emitted.append((request.request_id, token))
+            if request.request_id == 2 and len(request.generated) == 2:
+                request.cancel()
+            return not (request.request_id == 1 and len(request.generated) == 5)
+
+        scheduler = Scheduler(engine, sampler, EngineConfig(max_active_sequences=5, scheduler_token_budget=12,
+                                                            prefill_token_quantum=7), on_token=on_token)
+        assert scheduler.ahead
+        scheduler.ahead = ahead
+        for index, prompt in enumerate(prompts):
+            scheduler.submit(index, prompt, params[index])
+        finished = scheduler.run()
+        outcomes[ahead] = ({index: (request.generated, request.finish_reason) for index, request in finished.items()},
+                           sorted(emitted), scheduler.rounds)
+        stats = engine.cache.stats()
+        assert stats["live_requests"] == 0 and stats["free_slots"] == 5
+        assert all(group["free_pages"] == group["total_pages"] for group in stats["groups"])
+        engine.cache.check()
+    assert outcomes[True][0] == outcomes[False][0] and outcomes[True][1] == outcomes[False][1]
+    results = outcomes[True][0]
+    assert results[0] == (free[0][:3], "stop") and results[1] == (free[1][:5], "stop")
+    assert results[2] == (free[2][:2], "cancelled") and results[3] == (free[3][:4], "length")
+    assert results[4][1] == results[5][1] == "length" and len(results[4][0]) == 7 and len(results[5][0]) == 8

@@ -363,6 +363,54 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
         assert ((have - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()).item() <= 3e-2
 
 
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
+def test_lanes_fed_from_the_device_say_what_lanes_fed_by_the_host_say(tmp_path, graphs):
+    """Two engines decode the same three requests greedily, one with every token read by the host before the
+    next step, one with each step queued before the tokens of the step before were read (``Lane.feed`` from
+    the sampler's tokens on the device), beside a prompt portion of a fourth request in some steps: the same
+    logits bit for bit and the same tokens, and the tokens the plain model prefers."""
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.sampling import GREEDY, Sampler, SamplerRow
+    folder = tiny_configs.make_model_dir("C", tmp_path, torch.bfloat16)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    prompts = {name: tokens_for(cfg["vocab_size"], length, 60 + length) for name, length in (("a", 9), ("b", 33), ("c", 70))}
+    late = tokens_for(cfg["vocab_size"], 40, 99)
+    results = {}
+    for fed in (False, True):
+        engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=1024,
+                        max_active_sequences=4, decode_graphs=graphs)
+        sampler = Sampler(engine.vocab_size, engine.device)
+        rows = [SamplerRow(GREEDY, (), ()) for _ in prompts]
+        for name, tokens in prompts.items():
+            engine.add_request(name)
+        logits = engine.step([Lane(name, tokens, [len(tokens) - 1]) for name, tokens in prompts.items()])
+        handle = sampler.sample_async(logits.clone(), rows)
+        seen, emitted = [logits.float().cpu()], []
+        engine.add_request("late")
+        for turn in range(10):
+            if fed:
+                lanes = [Lane(name, [0], [0], feed=(handle.device, row)) for row, name in enumerate(prompts)]
+            else:
+                lanes = [Lane(name, [token], [0]) for name, token in zip(prompts, handle.wait())]
+            if turn in (2, 3, 5):                                   # a portion of another prompt beside them
+                portion = late[(turn - 2) * 10:(turn - 1) * 10] if turn < 5 else late[20:]
+                lanes.insert(1, Lane("late", portion, []))
+            logits = engine.step(lanes)
+            newer = sampler.sample_async(logits.clone(), rows)
+            emitted.append(handle.wait())
+            handle = newer
+            seen.append(logits.float().cpu())
+        emitted.append(handle.wait())
+        results[fed] = (torch.cat(seen), emitted)
+    assert torch.equal(results[True][0], results[False][0]) and results[True][1] == results[False][1]
+    for row, (name, tokens) in enumerate(prompts.items()):
+        mine = [step[row] for step in results[True][1]]
+        want = plain_impl.falcon_h1_logits(cfg, tensors, tokens + mine[:-1])[len(tokens) - 1:]
+        for place, token in enumerate(mine):                          # each token is the plain model's choice, or as good
+            best = want[place].max().item()
+            assert want[place][token].item() >= best - 0.06 * want[place].abs().max().item(), (name, place)
+
+
 def test_fixed_paths_take_no_measurement(tmp_path, monkeypatch):
     """``measured_paths=False``: even where every weight would be timed (the limit lowered to 0), the layers take
     the fixed rules, the same in every process, and say so; the engine that measures reports a choice for each

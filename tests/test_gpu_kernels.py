@@ -546,6 +546,27 @@ def test_softplus_is_stable_in_the_scan(ops):
     close(dev_state, want_state, torch.float32, 30.0)
 
 
+def test_tokens_fed_on_the_device(ops):
+    """token_ids[dst] = source[src] for 1, 64 and 150 pairs (more than a launch carries); places not named keep
+    their values; an index outside either vector is refused before anything is launched."""
+    generator = torch.Generator().manual_seed(5)
+    for count in (1, 64, 150):
+        token_ids = torch.arange(1000, 1000 + 400, dtype=torch.int32)
+        source = torch.randint(0, 30000, (200,), generator=generator, dtype=torch.int32)
+        dst = torch.randperm(400, generator=generator)[:count].tolist()
+        src = torch.randint(0, 200, (count,), generator=generator).tolist()
+        want = token_ids.clone()
+        ref_ops.feed_tokens(want, source, dst, src)
+        got = token_ids.to(DEV)
+        ops.feed_tokens(got, source.to(DEV), dst, src)
+        assert torch.equal(got.cpu(), want)
+    with pytest.raises(ops.KernelError):
+        ops.feed_tokens(got, source.to(DEV), [400], [0])
+    with pytest.raises(ops.KernelError):
+        ops.feed_tokens(got, source.to(DEV), [0], [200])
+    assert torch.equal(got.cpu(), want)
+
+
 # ------------------------------------------------------------------ sampling
 def test_argmax_and_ties(ops):
     logits = rand(5, 1003, seed=80)
