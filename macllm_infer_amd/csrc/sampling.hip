@@ -27,12 +27,14 @@ __device__ __forceinline__ float from_orderable(unsigned int key) {
 // ---------------------------------------------------------------- penalties
 // tokens[offsets[b] .. offsets[b+1]) is row b's history (prompt then generated);
 // the first prompt_lens[b] of them are the prompt.  count_all / count_gen are [B, V]
-// int32 work areas that hold zeros on entry and on exit.
+// int32 work areas that hold zeros on entry and on exit.  A row's newest generated token may still be
+// on the device only: extra_rows[b] >= 0 names its place in extra_source, and it counts like the others.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 penalties_kernel(float* __restrict__ logits, int V, const int* __restrict__ tokens,
                  const int* __restrict__ offsets, const int* __restrict__ prompt_lens,
                  const float* __restrict__ repetition, const float* __restrict__ presence,
-                 const float* __restrict__ frequency, int* __restrict__ count_all, int* __restrict__ count_gen) {
+                 const float* __restrict__ frequency, int* __restrict__ count_all, int* __restrict__ count_gen,
+                 const int* __restrict__ extra_source, const int* __restrict__ extra_rows) {
   const int row = blockIdx.x;
   float* values = logits + (long)row * V;
   int* all = count_all + (long)row * V;
@@ -45,6 +47,13 @@ penalties_kernel(float* __restrict__ logits, int V, const int* __restrict__ toke
     if (token < 0 || token >= V) continue;
     atomicAdd(&all[token], 1);
     if (i - begin >= prompt) atomicAdd(&gen[token], 1);
+  }
+  if (threadIdx.x == 0 && extra_source && extra_rows && extra_rows[row] >= 0) {
+    const int token = extra_source[extra_rows[row]];
+    if (token >= 0 && token < V) {
+      atomicAdd(&all[token], 1);
+      atomicAdd(&gen[token], 1);
+    }
   }
   __threadfence();
   __syncthreads();
@@ -68,10 +77,12 @@ penalties_kernel(float* __restrict__ logits, int V, const int* __restrict__ toke
 
 extern "C" int mi_apply_penalties(float* logits, int B, int V, const int* tokens, const int* offsets,
                                   const int* prompt_lens, const float* repetition, const float* presence,
-                                  const float* frequency, int* count_all, int* count_gen, hipStream_t stream) {
-  if (B <= 0 || V <= 0) return ERR_BAD_ARGUMENT;
+                                  const float* frequency, int* count_all, int* count_gen, const int* extra_source,
+                                  const int* extra_rows, hipStream_t stream) {
+  if (B <= 0 || V <= 0 || (extra_source == nullptr) != (extra_rows == nullptr)) return ERR_BAD_ARGUMENT;
   penalties_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, V, tokens, offsets, prompt_lens, repetition,
-                                                     presence, frequency, count_all, count_gen);
+                                                     presence, frequency, count_all, count_gen, extra_source,
+                                                     extra_rows);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

@@ -25,9 +25,9 @@ round before it have reached the host: a decoding request's lane is fed from the
 the earlier round's tokens (emits them, applies the stop conditions) while the GPU works.  A request that
 turns out to have ended in the earlier round (a stop token, the caller's ``on_token``, a cancellation) has
 then run one token too far: that token is dropped and what the request held is given back as usual; a request
-that ends by ``max_new_tokens`` is known beforehand and is not queued again.  A request whose sampling needs
-its history on the host (penalties) waits for its tokens first, as do all rounds with a sampler or an engine
-that cannot do this (the reference reads every token before the next step, src/engine.rs:1938-1988).
+that ends by ``max_new_tokens`` is known beforehand and is not queued again.  Penalties count the token that
+is still on the device there.  With a sampler or an engine that cannot do this every round waits for its
+tokens (as the reference does, src/engine.rs:1938-1988).
 """
 from __future__ import annotations
 
@@ -227,8 +227,7 @@ class Scheduler:
         """Whether the round before has to be read before the next can be made up."""
         if self._pending is None:
             return False
-        return not self.ahead or any(request.params.uses_penalties and not request.finished
-                                     for request in self._pending[1])
+        return not self.ahead
 
     def step(self) -> List[Request]:
         """One round; returns the requests that finished in it."""
@@ -270,7 +269,8 @@ class Scheduler:
                     request.cursor += len(tokens)
             if sampled:
                 rows = [SamplerRow(request.params, request.prompt, request.generated,
-                                   1 if request.in_flight is not None else 0) for request, _ in sampled]
+                                   None if request.in_flight is None else (request.in_flight[0].device, request.in_flight[1]))
+                        for request, _ in sampled]
                 if self.ahead:
                     handle = self.sampler.sample_async(logits, rows)
                     self._pending = (handle, [request for request, _ in sampled])

@@ -97,7 +97,7 @@ _SIGNATURES = {
     },
     "sampling": {
         "mi_apply_penalties": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                               _c_ptr, _c_ptr],
+                               _c_ptr, _c_ptr, _c_ptr, _c_ptr],
         "mi_argmax": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
         "mi_sample": [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                       _c_ptr, _c_ptr],
@@ -921,7 +921,11 @@ def stream_rmw(data: torch.Tensor, scale: float = 1.0, blocks: int = 4096) -> No
 
 
 # --------------------------------------------------------------------------- sampling
-def apply_penalties(logits, tokens, offsets, prompt_lens, repetition, presence, frequency, count_all, count_gen):
+def apply_penalties(logits, tokens, offsets, prompt_lens, repetition, presence, frequency, count_all, count_gen,
+                    extra_source=None, extra_rows=None):
+    """Repetition, presence and frequency penalties over each row's history ``tokens[offsets[b]:offsets[b + 1]]``
+    (its first ``prompt_lens[b]`` tokens are the prompt).  A row's newest generated token may be on the device
+    only: ``extra_rows[b]`` (int32, -1 = none) is then its place in ``extra_source`` (int32)."""
     B, V = logits.shape
     _need(logits.dtype == torch.float32 and logits.is_contiguous() and logits.is_cuda, "penalties: bad logits")
     for name, tensor in (("tokens", tokens), ("offsets", offsets), ("prompt_lens", prompt_lens),
@@ -929,9 +933,14 @@ def apply_penalties(logits, tokens, offsets, prompt_lens, repetition, presence, 
         _i32(tensor, name)
     _need(count_all.numel() >= B * V and count_gen.numel() >= B * V, "penalties: work areas are too small")
     _need(offsets.numel() == B + 1 and prompt_lens.numel() == B, "penalties: bad history layout")
+    _need((extra_source is None) == (extra_rows is None), "penalties: extra tokens need their source and their rows")
+    if extra_source is not None:
+        _i32(extra_source, "extra_source")
+        _i32(extra_rows, "extra_rows")
+        _need(extra_rows.numel() == B, "penalties: one extra row index per row")
     _check(_fn("sampling", "mi_apply_penalties")(
         _p(logits), B, V, _p(tokens), _p(offsets), _p(prompt_lens), _p(repetition), _p(presence), _p(frequency),
-        _p(count_all), _p(count_gen), _stream()), "apply_penalties")
+        _p(count_all), _p(count_gen), _p(extra_source), _p(extra_rows), _stream()), "apply_penalties")
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:

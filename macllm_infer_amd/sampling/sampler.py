@@ -9,7 +9,7 @@ request's tokens do not depend on what else is in the batch.
 """
 from __future__ import annotations
 
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -20,13 +20,18 @@ from .params import SamplingParams
 
 
 class SamplerRow:
-    """What the sampler needs to know of one request.  ``pending``: tokens already drawn for the request that
-    ``generated`` does not hold yet (they are still on the device); they count for the draw's index.  A row
-    with penalties needs all its tokens in ``generated``."""
-    __slots__ = ("params", "prompt", "generated", "pending")
+    """What the sampler needs to know of one request.  ``newest``: (int32 tensor on the device, row) of a token
+    already drawn for the request that ``generated`` does not hold yet; it counts for the draw's index and,
+    read on the device, for the penalties."""
+    __slots__ = ("params", "prompt", "generated", "newest")
 
-    def __init__(self, params: SamplingParams, prompt: Sequence[int], generated: Sequence[int], pending: int = 0):
-        self.params, self.prompt, self.generated, self.pending = params, prompt, generated, pending
+    def __init__(self, params: SamplingParams, prompt: Sequence[int], generated: Sequence[int],
+                 newest: Optional[tuple] = None):
+        self.params, self.prompt, self.generated, self.newest = params, prompt, generated, newest
+
+    @property
+    def pending(self) -> int:
+        return 0 if self.newest is None else 1
 
 
 class PendingTokens:
@@ -85,8 +90,9 @@ class Sampler:
         device = self.device
 
         if any(row.params.uses_penalties for row in rows):
-            if any(row.pending and row.params.uses_penalties for row in rows):
-                raise ValueError("a row with penalties needs all its tokens on the host")
+            newest = [row for row in rows if row.newest is not None and row.params.uses_penalties]
+            if any(row.newest[0] is not newest[0].newest[0] for row in newest):
+                raise ValueError("the newest tokens of a call's rows must lie in one tensor")
             tokens: List[int] = []
             offsets = [0]
             for row in rows:
@@ -95,20 +101,24 @@ class Sampler:
                     tokens.extend(row.generated)
                 offsets.append(len(tokens))
             count_all, count_gen = self._count_areas(B)
-            # one upload: offsets (B+1) | prompt lengths | the three penalties (float bits) | the histories
-            head = 5 * B + 1
+            # one upload: offsets (B+1) | prompt lengths | the three penalties (float bits) | rows of the newest
+            # tokens on the device | the histories
+            head = 6 * B + 1
             words = np.empty(head + max(len(tokens), 1), dtype=np.int32)
             words[:B + 1] = offsets
             words[B + 1:2 * B + 1] = [len(row.prompt) for row in rows]
             words[2 * B + 1:3 * B + 1].view(np.float32)[:] = [row.params.repetition_penalty for row in rows]
             words[3 * B + 1:4 * B + 1].view(np.float32)[:] = [row.params.presence_penalty for row in rows]
-            words[4 * B + 1:head].view(np.float32)[:] = [row.params.frequency_penalty for row in rows]
+            words[4 * B + 1:5 * B + 1].view(np.float32)[:] = [row.params.frequency_penalty for row in rows]
+            words[5 * B + 1:head] = [row.newest[1] if row.newest is not None and row.params.uses_penalties else -1
+                                     for row in rows]
             words[head:] = tokens or [0]
             packed = torch.from_numpy(words).to(device, non_blocking=True)
             ops.apply_penalties(
                 logits, packed[head:], packed[:B + 1], packed[B + 1:2 * B + 1],
                 packed[2 * B + 1:3 * B + 1].view(torch.float32), packed[3 * B + 1:4 * B + 1].view(torch.float32),
-                packed[4 * B + 1:head].view(torch.float32), count_all, count_gen)
+                packed[4 * B + 1:5 * B + 1].view(torch.float32), count_all, count_gen,
+                newest[0].newest[0] if newest else None, packed[5 * B + 1:head] if newest else None)
         out = torch.empty(B, dtype=torch.int32, device=device)
         if all(row.params.greedy for row in rows):
             ops.argmax(logits, out)

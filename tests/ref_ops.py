@@ -227,9 +227,12 @@ def install(monkeypatch):
         monkeypatch.setattr(ops, name, globals()[name])
 
 
-def apply_penalties(logits, tokens, offsets, prompt_lens, repetition, presence, frequency, count_all, count_gen):
+def apply_penalties(logits, tokens, offsets, prompt_lens, repetition, presence, frequency, count_all, count_gen,
+                    extra_source=None, extra_rows=None):
     for row in range(logits.shape[0]):
         history = tokens[int(offsets[row]):int(offsets[row + 1])].tolist()
+        if extra_rows is not None and int(extra_rows[row]) >= 0:
+            history.append(int(extra_source[int(extra_rows[row])]))          # the newest token, still on the device
         generated = history[int(prompt_lens[row]):]
         rep, pres, freq = float(repetition[row]), float(presence[row]), float(frequency[row])
         if rep > 0 and abs(rep - 1.0) >= 1.1920929e-07:

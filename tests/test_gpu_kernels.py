@@ -644,6 +644,22 @@ def test_penalties_match_the_plain_rule(ops):
                         torch.tensor(rep).to(DEV), torch.tensor(pres).to(DEV), torch.tensor(freq).to(DEV), *counts)
     close(got, want, torch.float32)
     assert not torch.equal(want, logits) and int(counts[0].sum()) == 0 and int(counts[1].sum()) == 0
+    # a row's newest token still on the device: it counts as if it closed the row's history
+    source, extra_rows = i32([9, 77, 400, 3]), i32([2, -1, 1])
+    longer = [histories[0] + [400], histories[1], histories[2] + [77]]
+    want = logits.clone()
+    ref_ops.apply_penalties(want, i32([token for history in longer for token in history]), i32([0, 7, 7, 12]),
+                            i32(prompt_lens), torch.tensor(rep), torch.tensor(pres), torch.tensor(freq), None, None)
+    fed = logits.clone()
+    ref_ops.apply_penalties(fed, i32(flat), i32(offsets), i32(prompt_lens), torch.tensor(rep), torch.tensor(pres),
+                            torch.tensor(freq), None, None, source, extra_rows)
+    assert torch.equal(fed, want)
+    got = logits.clone().to(DEV)
+    ops.apply_penalties(got, i32(flat).to(DEV), i32(offsets).to(DEV), i32(prompt_lens).to(DEV),
+                        torch.tensor(rep).to(DEV), torch.tensor(pres).to(DEV), torch.tensor(freq).to(DEV), *counts,
+                        source.to(DEV), extra_rows.to(DEV))
+    close(got, want, torch.float32)
+    assert int(counts[0].sum()) == 0 and int(counts[1].sum()) == 0
 
 
 # ------------------------------------------------------------------ decode attention (split over the context)
