@@ -899,6 +899,10 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
       denominator += weight * theirs[1];
       sum += weight * theirs[2 + dim];
     }
+    if (p.splits == 1) {             // the only workgroup of this token and kv head: nothing is left to merge
+      p.attn_out[token * p.out_ld + (long)(kvh * G + g) * DH + dim] = (bf16_t)(sum / denominator);
+      continue;
+    }
     float* mine = p.partial + ((token * p.Hq + kvh * G + g) * p.splits + split) * (long)(DH + 2);
     if (dim == 0) {
       mine[0] = maximum;
@@ -1094,7 +1098,9 @@ extern "C" int mi_mixer_runs(int M, int Hkv, int page_size, long span, int* run_
   return 0;
 }
 
-// merge = 0: the attended heads are not written; `partial` is left for mi_fused_gemm_merge.
+// merge = 0: the attended heads are not written; `partial` is left for mi_fused_gemm_merge.  (When a token and
+// kv head have one workgroup, mi_mixer_runs says runs = 1, there is nothing to merge: that workgroup writes the
+// attended heads itself, whatever `merge` says, and no merge kernel is launched.)
 extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv, int dh, int q_col, int k_col,
                                int v_col, const float* inv_freq, int rotary_dim, void* k_base, void* v_base,
                                long page_stride, int page_size, const int* block_tables, int max_pages,
@@ -1184,7 +1190,7 @@ extern "C" int mi_mixer_decode(const void* u, long u_ld, int M, int Hq, int Hkv,
   if (dh == 64) mixer_decode_kernel<64><<<(unsigned)total, MX_THREADS, 0, stream>>>(p);
   else mixer_decode_kernel<128><<<(unsigned)total, MX_THREADS, 0, stream>>>(p);
   RETURN_IF_LAUNCH_FAILED();
-  if (!merge) return 0;
+  if (!merge || p.splits == 1) return 0;
   const dim3 merge_grid(M, Hq);
   mixer_merge_kernel<<<merge_grid, dh, 0, stream>>>(p, dh);
   RETURN_IF_LAUNCH_FAILED();

@@ -897,7 +897,7 @@ def mixer_decode(u: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim
         num_groups, z_col, x_col, dt_col, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(slot_ids), _p(out),
         out.data_ptr() + 2 * num_heads * head_dim,
         _p(ssm_y), out_ld, _p(partial), partial.numel(), int(merge), _stream()), "mixer_decode")
-    if merge:
+    if merge or runs == 1:                  # one workgroup per token and kv head has written the heads itself
         return None
     return AttentionRuns(partial, positions, num_heads, head_dim, runs, run_keys, page_size, int(window or 0))
 

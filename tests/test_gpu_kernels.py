@@ -960,7 +960,8 @@ def test_mixer_decode_of_wide_batches(ops, M, Hq, Hkv, dh, H, P, N, G):
 def test_output_projection_that_merges_the_runs_of_keys(ops, Hq, Hkv, dh, E, N_out, window, lengths):
     """``mixer_decode(merge=False)`` followed by ``fused_gemm_merge`` gives bit for bit what ``mixer_decode``,
     its merge kernel and ``fused_gemm`` give: contexts of one run and of more runs than a merge asks for at
-    once, a window, 16 rows, a K beyond 1 024.  The attended columns of x hold NaN where nobody may read them."""
+    once, 16 rows, a K beyond 1 024; with a window of one run there is nothing to merge and ``mixer_decode``
+    writes the heads itself.  The attended columns of x hold NaN where nobody may read them."""
     dtype = torch.bfloat16
     H, P, N, G, page_size = E // 32, 32, 32, 1, 16
     M = len(lengths)
@@ -999,6 +1000,9 @@ def test_output_projection_that_merges_the_runs_of_keys(ops, Hq, Hkv, dh, E, N_o
     want = torch.empty(M, N_out, dtype=dtype, device=DEV)
     ops.fused_gemm(weight, bias, want, x=mixed)
     unmerged, runs = run(False)
+    if window is not None:           # a window of 40 keys is one run: its workgroup writes the heads itself, nothing is left over
+        assert runs is None and torch.equal(unmerged, mixed)
+        return
     assert torch.isnan(unmerged[:, :Hq * dh].float()).all() and torch.equal(unmerged[:, Hq * dh:], mixed[:, Hq * dh:])
     assert ops.fused_gemm_merge_supported(M, K, Hq, dh)
     for fragments in (None, ops.fragment_order(weight)):
