@@ -79,9 +79,10 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   extern __shared__ __align__(16) unsigned char smem[];
   const int K = p.K;
   const int staged = PRO == PRO_NORM ? K : PRO == PRO_MERGE ? p.merge_heads * p.merge_dh : 0;   // columns of x kept in LDS
+  const int staged_rows = min(p.M, MT * 16);          // and its rows: the step's own (a tile's rows past M read row M - 1)
   const int ldx = staged + FG_PAD;
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem);
-  float* red = reinterpret_cast<float*>(smem + (staged ? (size_t)MT * 16 * ldx * sizeof(bf16_t) : 0));
+  float* red = reinterpret_cast<float*>(smem + (staged ? (size_t)staged_rows * ldx * sizeof(bf16_t) : 0));
   float* tile = red + FG_WAVES * MT * 256;
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
@@ -209,15 +210,8 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt) {
           const int m = m0 + wave + (2 * pair + tt) * FG_WAVES;
-          if (m >= MT * 16) continue;
+          if (m >= staged_rows) continue;
           bf16_t* x_row = xs + (long)m * ldx;
-          if (m >= p.M) {
-            for (int k = lane * 4; k < K; k += WAVE * 4) {
-              const bf16x4_t zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
-              *reinterpret_cast<bf16x4_t*>(x_row + k) = zero;
-            }
-            continue;
-          }
           const float* h_row = p.h_in + (long)m * K;
           auto row_value = [&](int k) {
             floatx4 value = *reinterpret_cast<const floatx4*>(h_row + k);
@@ -383,7 +377,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           bf16x8_t operand;
-          if (PRO == PRO_NORM) operand = *reinterpret_cast<const bf16x8_t*>(xs + (long)(mt * 16 + r) * ldx + c * 32 + 8 * q);
+          if (PRO == PRO_NORM) operand = *reinterpret_cast<const bf16x8_t*>(xs + (long)min(mt * 16 + r, p.M - 1) * ldx + c * 32 + 8 * q);
           else operand = b[j][mt];
           acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8_t*>(&weights), operand, acc[nt][mt], 0, 0, 0);
         }
@@ -475,11 +469,12 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 
 static int fused_gemm_waves(int K) { return K / 32 > 32 ? 8 : 4; }   // 8 waves split a long K
 
-// staged: the columns of x the prologue keeps in LDS (all of K behind the norm, the merged heads behind the merge)
-static size_t fused_gemm_lds(int MT, int pro, int K, int staged = 0) {
+// staged: the columns of x the prologue keeps in LDS (all of K behind the norm, the merged heads behind the
+// merge), for the M rows of the step
+static size_t fused_gemm_lds(int MT, int pro, int K, int M, int staged = 0) {
   size_t bytes = (size_t)fused_gemm_waves(K) * MT * 256 * sizeof(float) + (size_t)16 * MT * 16 * sizeof(float);
   if (pro == PRO_NORM) staged = K;
-  if (pro != PRO_PLAIN) bytes += (size_t)MT * 16 * (staged + FG_PAD) * sizeof(bf16_t);
+  if (pro != PRO_PLAIN) bytes += (size_t)(M < MT * 16 ? M : MT * 16) * (staged + FG_PAD) * sizeof(bf16_t);
   return bytes;
 }
 
@@ -489,7 +484,7 @@ static size_t fused_gemm_lds(int MT, int pro, int K, int staged = 0) {
 template <int MT>
 static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStream_t stream, int k_splits = 1,
                              int feature_tiles = 1) {
-  const size_t lds = fused_gemm_lds(MT, pro, p.K, pro == PRO_MERGE ? p.merge_heads * p.merge_dh : 0);
+  const size_t lds = fused_gemm_lds(MT, pro, p.K, p.M, pro == PRO_MERGE ? p.merge_heads * p.merge_dh : 0);
   if (feature_tiles > 1) {
     if (pro != PRO_PLAIN || (feature_tiles != 2 && feature_tiles != 4)) return ERR_BAD_ARGUMENT;
     const dim3 blocks((p.N + 16 * feature_tiles - 1) / (16 * feature_tiles), k_splits);
@@ -524,8 +519,8 @@ static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStre
   return 0;
 }
 
-// Sizes: 1 <= M <= 64, K a multiple of 32; with the NORM prologue the normalized rows must fit
-// 64 KiB of LDS beside the reduction area.  EPI_SWIGLU wants N a multiple of 16.
+// Sizes: 1 <= M <= 64, K a multiple of 32; with the NORM prologue the step's M normalized rows must fit
+// 64 KiB of LDS beside the reduction area (16 rows of 1,024, 8 of 3,072).  EPI_SWIGLU wants N a multiple of 16.
 // w_fragments: W is not row-major [N, K] but a copy in the order of the matrix-core fragments,
 // [ceil(N / 16), K / 32, 4, 16, 8] with element [n, c, q, r, j] = W[16 n + r, 32 c + 8 q + j] (rows past N zero):
 // what a wave asks for at once is then one run of 1 KiB instead of 64 bytes of each of 16 rows, which
@@ -547,7 +542,7 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
     return ERR_BAD_ARGUMENT;
   const int MT = (M + 15) / 16;
   if (pro != PRO_NORM && pro != PRO_PLAIN) return ERR_BAD_ARGUMENT;
-  if (fused_gemm_lds(MT, pro, K) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  if (fused_gemm_lds(MT, pro, K, M) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   FusedGemmParams p = {};
   p.h_in = h_in;
   p.delta0 = (const bf16_t*)delta0;
@@ -595,7 +590,7 @@ extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, cons
   if (feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0 || splits < 1 || splits > 64 || K / 32 < splits) return ERR_UNSUPPORTED_SIZE;
   const int MT = (M + 15) / 16;
-  if (fused_gemm_lds(MT, PRO_PLAIN, K) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  if (fused_gemm_lds(MT, PRO_PLAIN, K, M) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   FusedGemmParams p = {};
   p.x = (const bf16_t*)x;
   p.x_ld = x_ld;
@@ -633,7 +628,7 @@ extern "C" int mi_fused_gemm_merge(const float* partial, const int* positions, i
   if (heads <= 0 || head_dim <= 0 || runs <= 0 || run_keys <= 0 || page_size <= 0 || window < 0) return ERR_BAD_ARGUMENT;
   const long merged = (long)heads * head_dim;
   if (M > 16 || K % 32 != 0 || head_dim % 8 != 0 || merged % 32 != 0 || merged > K) return ERR_UNSUPPORTED_SIZE;
-  if (fused_gemm_lds(1, PRO_MERGE, K, (int)merged) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  if (fused_gemm_lds(1, PRO_MERGE, K, M, (int)merged) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   FusedGemmParams p = {};
   p.x = (const bf16_t*)x;
   p.x_ld = x_ld;
@@ -663,7 +658,7 @@ extern "C" int mi_fused_gemm_merge(const float* partial, const int* positions, i
 // Whether mi_fused_gemm covers a shape (the host asks before it builds a fused path).
 extern "C" int mi_fused_gemm_supported(int pro, int M, int K) {
   if (M <= 0 || M > 64 || K % 32 != 0) return 0;
-  return fused_gemm_lds((M + 15) / 16, pro, K) <= 64 * 1024 ? 1 : 0;
+  return fused_gemm_lds((M + 15) / 16, pro, K, M) <= 64 * 1024 ? 1 : 0;
 }
 
 // ---------------------------------------------------------------- mixer decode

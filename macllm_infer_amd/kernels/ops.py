@@ -715,7 +715,7 @@ def fused_gemm_merge_supported(M: int, K: int, heads: int, head_dim: int) -> boo
     merged = heads * head_dim
     waves = 8 if K // 32 > 32 else 4
     return (M <= 16 and K % 32 == 0 and merged % 32 == 0 and merged <= K
-            and waves * 1024 + 1024 + 16 * (merged + 8) * 2 <= 64 * 1024)
+            and waves * 1024 + 1024 + M * (merged + 8) * 2 <= 64 * 1024)
 
 
 def fused_gemm_merge(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, x: torch.Tensor,

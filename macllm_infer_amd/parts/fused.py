@@ -44,6 +44,10 @@ from .position import NoPosition, Rope
 
 MAX_ROWS = 64          # rows of a step the skinny kernels take
 MAX_NORM_ROWS = 16     # the norm prologue recomputes the normed rows in every workgroup: small batches only
+# (and only as many rows as fit LDS at the layer's width, see LayerFusion.norm_rows), and narrow layers only: up to
+# MAX_NORM_WIDTH a wave holds a row in registers; beyond, every workgroup reads its rows twice and its LDS fills
+# a compute unit (a 3,072-wide layer at 8 rows: 7.84 ms a step with the prologue, 4.96 with the norms as kernels)
+MAX_NORM_WIDTH = 2048
 # A weight of this many elements or more is measured once, when the first layer of its shape is built, on
 # both ways: the skinny kernel, and the BLAS library with the conv step or SiLU(g)*u as a kernel of its own.
 # The skinny kernel reads the step's rows once per 16 weight rows and keeps all of K in one workgroup; the
@@ -110,7 +114,6 @@ def _bucket(rows: int) -> int:
 
 
 BUCKETS = len(TUNE_ROWS)
-WIDE_BUCKETS = tuple(bucket for bucket, rows in enumerate(TUNE_ROWS) if rows > MAX_NORM_ROWS)   # no norm prologue there
 
 
 def _each(value) -> tuple:
@@ -345,9 +348,14 @@ class LayerFusion:
                           and (self.gate_up is None or ops.fused_gemm_supported(False, 1, self.inner)))
         # norms that the skinny kernel computes in its prologue (a wide model's rows do not fit its LDS, and another
         # kind of norm is not what it computes: those run as kernels of their own)
-        fits = self.decode_ok and ops.fused_gemm_supported(True, 1, self.hidden)
-        self.mixer_rms = _rms_prologue(block.mixer_norm) if fits else None
-        self.ffn_rms = _rms_prologue(block.ffn_norm) if fits else None
+        # (the largest step size of TUNE_ROWS, up to MAX_NORM_ROWS, whose rows fit LDS at this width; steps of more
+        # rows, the "wide" step sizes, run their norms as kernels of their own)
+        self.norm_rows = max([rows for rows in TUNE_ROWS if rows <= MAX_NORM_ROWS and self.decode_ok
+                              and self.hidden <= MAX_NORM_WIDTH and ops.fused_gemm_supported(True, rows, self.hidden)],
+                             default=0)
+        self.wide_buckets = tuple(bucket for bucket, rows in enumerate(TUNE_ROWS) if rows > self.norm_rows)
+        self.mixer_rms = _rms_prologue(block.mixer_norm) if self.norm_rows else None
+        self.ffn_rms = _rms_prologue(block.ffn_norm) if self.norm_rows else None
         self.norm_fits = self.mixer_rms is not None and self.ffn_rms is not None
         # a kernel for this set of mixers, if one is registered and takes these sizes
         factory = _MIXER_KERNELS.get(tuple(getattr(mixer, "kind", None) for mixer in self.mixers))
@@ -360,7 +368,7 @@ class LayerFusion:
         self.library_in, self.tiles_in = self._tune(self.w_in, self.b_in, ops.EPI_CONV if conv else ops.EPI_PLAIN, conv,
                                                     self.mixer_rms is not None)
         self.library_out, self.tiles_out = self._tune(self.w_out, self.b_out, ops.EPI_PLAIN)
-        # and which of the two that feed the residual stream are split over K instead (steps of more than MAX_NORM_ROWS rows)
+        # and which of the two that feed the residual stream are split over K instead (steps of more than norm_rows rows)
         self.split_out, self.tiles_out = self._tune_split(self.w_out, self.b_out, self.library_out, self.tiles_out)
         # what the skinny kernel reads: a second copy of each matrix in the order of its waves' fragments (one run
         # of 1 KiB a load instead of 64 bytes of each of 16 rows: 15 to 25 % faster); the row-major ones stay for
@@ -456,28 +464,28 @@ class LayerFusion:
               normed: bool = False) -> tuple:
         """For every step size of TUNE_ROWS: whether this projection goes through the library, and the feature
         tiles of the skinny kernel.  (``normed``: the norm before it runs in the skinny kernel's prologue in steps
-        of up to MAX_NORM_ROWS rows; those stay with the skinny kernel and one tile.)"""
+        of up to ``norm_rows`` rows; those stay with the skinny kernel and one tile.)"""
         if not self.decode_ok:
             return _each(True), _each(1)
         choices, tiles = self._tune_all(weight, bias, epilogue, conv, normed)
         if normed:
-            choices = tuple(choice and bucket in WIDE_BUCKETS for bucket, choice in enumerate(choices))
+            choices = tuple(choice and bucket in self.wide_buckets for bucket, choice in enumerate(choices))
         return choices, tiles
 
     def _tune_split(self, weight: torch.Tensor, bias, library: tuple, tiles: tuple) -> tuple:
         """For every step size of TUNE_ROWS: the number of slabs over K, or 0 for the whole product, and the
-        feature tiles that go with it.  Steps of up to MAX_NORM_ROWS rows feed the next kernel's norm prologue,
+        feature tiles that go with it.  Steps of up to ``norm_rows`` rows feed the next kernel's norm prologue,
         which takes whole rows."""
         if self.hidden % 4 != 0 or FORCE_SPLIT == 0:
             return _each(0), tiles
         if FORCE_SPLIT:
             slabs = FORCE_SPLIT if weight.shape[1] // 32 >= FORCE_SPLIT else 0
-            return tuple(slabs if bucket in WIDE_BUCKETS else 0 for bucket in range(BUCKETS)), tiles
+            return tuple(slabs if bucket in self.wide_buckets else 0 for bucket in range(BUCKETS)), tiles
         if weight.numel() < LIBRARY_MIN_WEIGHT or not self.measure:
             return _each(0), tiles
         slabs, split_tiles = [], []
         for bucket in range(BUCKETS):
-            if bucket not in WIDE_BUCKETS:
+            if bucket not in self.wide_buckets:
                 slabs.append(0)
                 split_tiles.append(tiles[bucket])
                 continue
@@ -490,7 +498,7 @@ class LayerFusion:
 
     def _tune_all(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict], normed: bool) -> tuple:
         forced = 1 if FORCE_TILES is None else FORCE_TILES
-        fixed_tiles = tuple(forced if bucket in WIDE_BUCKETS else 1 for bucket in range(BUCKETS))
+        fixed_tiles = tuple(forced if bucket in self.wide_buckets else 1 for bucket in range(BUCKETS))
         if (not self.general or FORCE_LIBRARY is False
                 or (FORCE_LIBRARY is None and (weight.numel() < LIBRARY_MIN_WEIGHT or not self.measure))):
             return _each(False), fixed_tiles
@@ -498,12 +506,12 @@ class LayerFusion:
             return _each(True), fixed_tiles
         choices, tiles = [], []
         for bucket, rows in enumerate(TUNE_ROWS):
-            wide = bucket in WIDE_BUCKETS or not normed          # the plain prologue: a workgroup may own several tiles
+            wide = bucket in self.wide_buckets or not normed          # the plain prologue: a workgroup may own several tiles
             key = (tuple(weight.shape), epilogue, bias is None, bucket, wide)
             if key not in _library_wins:
                 _library_wins[key] = _measure_library(weight, bias, rows, epilogue, 8, conv, wide)
             choices.append(_library_wins[key][0])
-            tiles.append(_library_wins[key][1] if FORCE_TILES is None or bucket not in WIDE_BUCKETS else FORCE_TILES)
+            tiles.append(_library_wins[key][1] if FORCE_TILES is None or bucket not in self.wide_buckets else FORCE_TILES)
         return tuple(choices), tuple(tiles)
 
     def forward_decode(self, residual: Residual, step, caches) -> None:
@@ -516,7 +524,7 @@ class LayerFusion:
 
         def norm_prologue(norm, rms):
             """The input of a projection: the norm in the kernel's prologue, or its own kernel before."""
-            if M > MAX_NORM_ROWS or rms is None:
+            if M > self.norm_rows or rms is None:
                 return dict(x=norm.forward(residual)), None          # adds the pending deltas in place
             pending = residual.pending
             if len(pending) > 2 or any(delta.dtype != bf16 for delta in pending):

@@ -740,8 +740,10 @@ def test_fused_gemm_plain_prologue(ops, M, N, K):
     assert not ops.fused_gemm_supported(False, M, K + 8)
 
 
-@pytest.mark.parametrize("M, N, K, deltas", [(1, 64, 64, 0), (8, 160, 1024, 2), (13, 48, 96, 1), (16, 4120, 1024, 2)])
+@pytest.mark.parametrize("M, N, K, deltas", [(1, 64, 64, 0), (8, 160, 1024, 2), (13, 48, 96, 1), (16, 4120, 1024, 2),
+                                             (8, 272, 3072, 2), (3, 80, 5120, 1), (5, 64, 3072, 0)])
 def test_fused_gemm_norm_prologue_and_epilogues(ops, M, N, K, deltas):
+    """Only the step's own rows are staged in LDS: 8 rows of 3,072 and 3 of 5,120 fit where 16 would not."""
     h = rand(M, K, seed=310)
     ds = [rand(M, K, seed=311 + i, dtype=torch.bfloat16) for i in range(deltas)]
     norm_w = rand(K, seed=314, scale=0.1) + 1.0
