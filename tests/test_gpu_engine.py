@@ -200,6 +200,55 @@ def test_greedy_generation_through_the_entry_point(tmp_path, name, dtype):
     assert llm.engine.cache.stats()["live_requests"] == 0
 
 
+def test_sampled_generation_a_round_ahead_equals_generation_that_waits(tmp_path):
+    """float32 on the GPU, where a token does not depend on what shares its step: twenty requests with seeded
+    sampling (penalties for most), stop tokens that are hit, callers' stops and a tight budget, once with every
+    round queued ahead of the tokens of the round before and once with every token read first.  The same tokens
+    and finish reasons, token for token what the plain sampler draws from the plain model for three of them."""
+    from macllm_infer_amd import Engine, EngineConfig, SamplingParams
+    from macllm_infer_amd.engine.scheduler import Scheduler
+    from macllm_infer_amd.sampling import Sampler
+    folder = tiny_configs.make_model_dir("B", tmp_path, torch.float32)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    generator = torch.Generator().manual_seed(7)
+    prompts = [tokens_for(cfg["vocab_size"], int(torch.randint(1, 40, (1,), generator=generator)), 300 + index)
+               for index in range(20)]
+    params = [SamplingParams(max_new_tokens=4 + index % 9, temperature=0.0 if index % 5 == 0 else 0.7 + 0.05 * (index % 4),
+                             top_k=0 if index % 3 == 0 else 12, top_p=1.0 if index % 2 else 0.85,
+                             repetition_penalty=1.0 if index % 4 == 0 else 1.15, presence_penalty=0.2 * (index % 3),
+                             frequency_penalty=0.1 * (index % 2), seed=50 + index,
+                             stop_token_ids=tuple(range(0, cfg["vocab_size"], 9)) if index % 6 == 1 else ())
+              for index in range(20)]
+    outcomes = []
+    for ahead in (True, False):
+        engine = Engine(folder, dtype="float32", kv_cache_block_tokens=8, kv_cache_capacity_tokens=512,
+                        max_active_sequences=6)
+        scheduler = Scheduler(engine, Sampler(engine.vocab_size, engine.device),
+                              EngineConfig(max_active_sequences=6, scheduler_token_budget=20, prefill_token_quantum=9),
+                              on_token=lambda request, token: not (request.request_id % 7 == 3 and len(request.generated) == 3))
+        assert scheduler.ahead
+        scheduler.ahead = ahead
+        for index, prompt in enumerate(prompts):
+            scheduler.submit(index, prompt, params[index])
+        finished = scheduler.run()
+        outcomes.append({index: (request.generated, request.finish_reason) for index, request in finished.items()})
+        assert engine.cache.stats()["live_requests"] == 0
+        engine.cache.check()
+    assert outcomes[0] == outcomes[1]
+    assert {reason for _, reason in outcomes[0].values()} == {"length", "stop"}
+    for index in (2, 5, 11):
+        p, tokens, generated = params[index], list(prompts[index]), []
+        for draw in range(len(outcomes[0][index][0])):
+            logits = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-1]
+            token = plain_impl.sample_token(
+                logits, temperature=p.temperature, top_k=p.top_k, top_p=p.top_p, repetition_penalty=p.repetition_penalty,
+                presence_penalty=p.presence_penalty, frequency_penalty=p.frequency_penalty, history=tokens,
+                generated=generated, seed=p.seed, draw_index=draw)
+            tokens.append(token)
+            generated.append(token)
+        assert generated == outcomes[0][index][0], index
+
+
 def test_generation_when_pages_run_out(tmp_path):
     """Seven requests on a cache of six pages, three live at a time: lanes are dropped from steps
     and retried, pages and slots are used again, and a request that cannot grow while the others
