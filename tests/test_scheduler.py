@@ -238,11 +238,11 @@ def test_a_portion_that_does_not_end_its_prompt_is_cut_to_the_size_the_engine_pr
     config = EngineConfig(max_active_sequences=2, scheduler_token_budget=45, prefill_token_quantum=40)
     engine, scheduler, finished = run([[7, 8, 9], prompt], params, config, engine)
     steps = [[(request, len(tokens)) for request, tokens, _, _ in call] for call in engine.calls]
-    # round 1: the short prompt whole (it ends: untouched) beside 40 of the long one: 43 tokens -> 32
+    # the first round: the short prompt whole (it ends: untouched) beside 40 of the long one: 43 tokens -> 32
     assert steps[0] == [(0, 3), (1, 29)]
-    # round 2: a decoded token beside a portion of 40: 41 -> 32
+    # the second round: a decoded token beside a portion of 40: 41 -> 32
     assert steps[1] == [(0, 1), (1, 31)]
-    # round 3: the last 40 tokens end the prompt: not cut, although 41 is no preferred size
+    # the third round: the last 40 tokens end the prompt: not cut, although 41 is no preferred size
     assert steps[2] == [(0, 1), (1, 40)] and engine.calls[2][1][3] == [39]
     assert sum(count for step in steps[:3] for request, count in step if request == 1) == 100
     assert finished[1].generated == [(prompt[-1] + 1) % 50, (prompt[-1] + 2) % 50, (prompt[-1] + 3) % 50]
