@@ -21,6 +21,7 @@ import numpy as np
 import torch
 
 from ..cache import native
+from ..kernels import ops
 
 
 NO_TILES = 1 << 30     # the table of runs then has one run per lane: no mixer of the model reads it
@@ -91,7 +92,6 @@ def apply_feeds(token_ids: torch.Tensor, feeds) -> None:
     forward pass or the graph's replay, on the same stream)."""
     if not feeds:
         return
-    from ..kernels import ops
     by_source = {}
     for row, source, index in feeds:
         by_source.setdefault(id(source), (source, [], []))
