@@ -411,8 +411,13 @@ class LayerFusion:
         return out
 
     def decode_supported(self, step, caches) -> bool:
-        if step.max_query_len != 1 or step.num_tokens > MAX_ROWS or not self.decode_ok:
+        """Whether the step's rows go through the skinny products: steps of up to MAX_ROWS single tokens, and
+        steps of as few tokens in portions of prompts (a short prompt, the tail of a long one, beside decoded
+        tokens), whose mixers then run their own kernels between the skinny products."""
+        if step.num_tokens > MAX_ROWS or not self.decode_ok:
             return False
+        if step.max_query_len != 1:
+            return self.aligned
         return self.aligned or self.kernel.supported(step, caches)
 
     def forward(self, residual: Residual, step, caches) -> bool:
@@ -520,7 +525,8 @@ class LayerFusion:
         bucket = _bucket(M)
         device = residual.h.device
         bf16 = torch.bfloat16
-        kernel = self.kernel if self.kernel is not None and self.kernel.supported(step, caches) else None
+        kernel = self.kernel if (self.kernel is not None and step.max_query_len == 1
+                                 and self.kernel.supported(step, caches)) else None
 
         def norm_prologue(norm, rms):
             """The input of a projection: the norm in the kernel's prologue, or its own kernel before."""
