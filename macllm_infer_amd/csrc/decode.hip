@@ -9,7 +9,15 @@
 //                 MERGE: x given in bfloat16, but for its first columns, the attended heads, which are
 //                        merged here from the partial results that mixer_decode's runs of keys left
 //                        (what mixer_merge_kernel does in a launch of its own, sum for sum)
+//                 A row scale may follow any prologue that gives x as it is (PLAIN, MERGE): x is then a row of the
+//                 residual stream times a norm's weight, rounded to bfloat16 but not yet divided by its root mean
+//                 square, and the sums of a row are multiplied by 1 / sqrt(sum of squares / width + eps), from the
+//                 partial sums of squares that the RESIDUAL epilogue of the product before left (the norm without
+//                 a pass of its own: its statistics in float32, its division applied to float32 sums)
 //       epilogue  PLAIN : bfloat16 or float32 (x scale) store
+//                 RESIDUAL: the result is added to the float32 residual stream in place, h += result; the new rows
+//                        times the next norm's weight go out in bfloat16, and the sums of their squares over the
+//                        workgroup's 16 features go to ssq[workgroup][row]
 //                 SWIGLU: rows come in tiles of 8 gate rows + 8 up rows; stores SiLU(g)*u
 //                 CONV  : rows in [conv_lo, conv_hi) are channels of a causal depthwise conv
 //                         with K taps: the new sample joins the request's tail, the tail is
@@ -39,7 +47,9 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 enum { PRO_NORM = 0, PRO_PLAIN = 1, PRO_MERGE = 2 };
 #define MERGE_AT_ONCE 8      // runs of keys asked for at once by a merge (mixer_merge_kernel and the MERGE prologue)
-enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_CONV = 2 };
+enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_CONV = 2, EPI_RESIDUAL = 3 };
+#define SSQ_PARTS 16         // threads that share the sum of a row's partial sums of squares
+#define SSQ_EARLY 12         // partial sums a thread asks for before the products (rows of up to 3,072 at 16 rows)
 
 struct FusedGemmParams {
   const float* h_in;
@@ -67,6 +77,16 @@ struct FusedGemmParams {
   const float* partial;
   const int* positions;
   int merge_heads, merge_dh, merge_runs, merge_run_keys, merge_page, merge_window;
+  // RESIDUAL epilogue: h [M, N] float32 (in place), hb [M, hb_ld] bfloat16 = h * next_w[n], ssq_out [workgroups, 16 MT]
+  float* res_h;
+  bf16_t* res_hb;
+  long res_hb_ld;
+  const float* res_w;
+  float* ssq_out;
+  // row scale: ssq_in [ssq_blocks, 16 MT] partial sums of squares of rows of ssq_width elements
+  const float* ssq_in;
+  int ssq_blocks, ssq_width;
+  float ssq_eps;
 };
 
 __device__ __forceinline__ float round_bf16(float v) { return (float)(bf16_t)v; }
@@ -74,7 +94,8 @@ __device__ __forceinline__ float round_bf16(float v) { return (float)(bf16_t)v; 
 template <int MT, int PRO, int EPI, int FG_WAVES, int NT>
 __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmParams p) {
   static_assert(NT == 1 || PRO == PRO_PLAIN, "several feature tiles a workgroup: plain prologue only");
-  static_assert(PRO != PRO_MERGE || EPI == EPI_PLAIN, "the merge prologue comes with the plain epilogue");
+  static_assert(PRO != PRO_MERGE || EPI == EPI_PLAIN || EPI == EPI_RESIDUAL, "the merge prologue comes with the plain or the residual epilogue");
+  static_assert(EPI != EPI_RESIDUAL || (NT == 1 && PRO != PRO_NORM), "the residual epilogue: one tile of features, rows given as they are");
   constexpr int FG_THREADS = FG_WAVES * WAVE;
   extern __shared__ __align__(16) unsigned char smem[];
   const int K = p.K;
@@ -84,6 +105,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem);
   float* red = reinterpret_cast<float*>(smem + (staged ? (size_t)staged_rows * ldx * sizeof(bf16_t) : 0));
   float* tile = red + FG_WAVES * MT * 256;
+  float* ssq_parts = tile + 16 * MT * 16;            // [SSQ_PARTS][16 MT]
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
@@ -128,6 +150,30 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 #pragma unroll
     for (int j = 0; j < EPT; ++j)
       tail_slot[j] = p.slot_ids[min(((tid + j * FG_THREADS) / 256) * 16 + tid % 16, p.M - 1)];
+  }
+
+  // the partial sums of squares of the rows (row scale), 16 MT rows by SSQ_PARTS threads each, and the elements of
+  // the residual stream that this thread will add to (RESIDUAL) are asked for up here as well
+  constexpr int PARTS = SSQ_PARTS / MT;               // PARTS * 16 MT threads: within the 256 of four waves
+  // asked for without a branch (under one, the wave waits for them before it asks for its weights) and not added
+  // up before the products are done; without a row scale, and past the last workgroup's sums, a valid address
+  float ssq_early[SSQ_EARLY];
+  {
+    const float* sums = p.ssq_in ? p.ssq_in : reinterpret_cast<const float*>(p.W);
+    const int last = p.ssq_in ? p.ssq_blocks - 1 : 0;
+    const int row = p.ssq_in ? tid % (16 * MT) : 0;
+#pragma unroll
+    for (int i = 0; i < SSQ_EARLY; ++i)
+      ssq_early[i] = sums[(long)min(tid / (16 * MT) + i * PARTS, last) * (16 * MT) + row];
+  }
+  float res_old[EPT] = {};
+  float res_weight = 0.f;
+  if (EPI == EPI_RESIDUAL) {
+    const int n_mine = min(n0 + 4 * ((tid % 64) / 16) + (tid % 256) / 64, p.N - 1);
+    res_weight = p.res_w[n_mine];
+#pragma unroll
+    for (int j = 0; j < EPT; ++j)
+      res_old[j] = p.res_h[(long)min(((tid + j * FG_THREADS) / 256) * 16 + tid % 16, p.M - 1) * p.N + n_mine];
   }
 
   // Loads come back in the order they were asked for, and a wait counts all of them.  The rows
@@ -384,6 +430,15 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
       }
     }
   }
+  if (p.ssq_in && tid < PARTS * 16 * MT) {          // read behind the barrier below
+    const int part = tid / (16 * MT);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < SSQ_EARLY; ++i) sum += part + i * PARTS < p.ssq_blocks ? ssq_early[i] : 0.f;
+    // rows wider than SSQ_EARLY sums a thread: the rest now
+    for (int b = part + SSQ_EARLY * PARTS; b < p.ssq_blocks; b += PARTS) sum += p.ssq_in[(long)b * (16 * MT) + tid % (16 * MT)];
+    ssq_parts[tid] = sum;
+  }
   // the waves' partial tiles are summed through LDS and finished, one tile of 16 features after the other
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
@@ -408,9 +463,26 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
       const int n_local = 4 * (l / 16) + i;
       const int n = tile_n0 + n_local;
       const int m = mt * 16 + (l % 16);
+      if (p.ssq_in) {                          // the norm's division, on the float32 sums
+        float squares = 0.f;
+#pragma unroll
+        for (int part = 0; part < PARTS; ++part) squares += ssq_parts[part * (16 * MT) + m];
+        v *= 1.0f / sqrtf(squares / (float)p.ssq_width + p.ssq_eps);
+      }
       if (p.bias && n < p.N && blockIdx.y == 0) v += p.bias[n];
       if (EPI == EPI_SWIGLU) {
         tile[n_local * (MT * 16) + m] = v;
+        continue;
+      }
+      if (EPI == EPI_RESIDUAL) {
+        float square = 0.f;
+        if (n < p.N && m < p.M) {
+          const float updated = res_old[j] + v * p.out_scale;
+          p.res_h[(long)m * p.N + n] = updated;
+          p.res_hb[(long)m * p.res_hb_ld + n] = (bf16_t)(updated * res_weight);
+          square = updated * updated;
+        }
+        tile[n_local * (MT * 16) + m] = square;
         continue;
       }
       if (n >= p.N || m >= p.M) continue;
@@ -451,6 +523,15 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
         reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + n] = (bf16_t)(v * p.out_scale);
       }
     }
+    if (EPI == EPI_RESIDUAL) {
+      __syncthreads();
+      if (tid < MT * 16) {
+        float squares = 0.f;
+#pragma unroll
+        for (int f = 0; f < 16; ++f) squares += tile[f * (MT * 16) + tid];
+        p.ssq_out[(long)blockIdx.x * (MT * 16) + tid] = squares;
+      }
+    }
     if (EPI == EPI_SWIGLU) {
       __syncthreads();
       const int half_rows = p.N / 2;
@@ -472,7 +553,8 @@ static int fused_gemm_waves(int K) { return K / 32 > 32 ? 8 : 4; }   // 8 waves 
 // staged: the columns of x the prologue keeps in LDS (all of K behind the norm, the merged heads behind the
 // merge), for the M rows of the step
 static size_t fused_gemm_lds(int MT, int pro, int K, int M, int staged = 0) {
-  size_t bytes = (size_t)fused_gemm_waves(K) * MT * 256 * sizeof(float) + (size_t)16 * MT * 16 * sizeof(float);
+  size_t bytes = (size_t)fused_gemm_waves(K) * MT * 256 * sizeof(float) + (size_t)16 * MT * 16 * sizeof(float) +
+                 (size_t)SSQ_PARTS * 16 * MT * sizeof(float);
   if (pro == PRO_NORM) staged = K;
   if (pro != PRO_PLAIN) bytes += (size_t)(M < MT * 16 ? M : MT * 16) * (staged + FG_PAD) * sizeof(bf16_t);
   return bytes;
@@ -508,6 +590,8 @@ static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStre
     else fused_gemm_kernel<MT, PRO_, EPI_, 4, 1><<<blocks, 4 * WAVE, lds, stream>>>(p);            \
   } while (0)
   if (pro == PRO_MERGE && epi == EPI_PLAIN) FG_LAUNCH(PRO_MERGE, EPI_PLAIN);
+  else if (pro == PRO_MERGE && epi == EPI_RESIDUAL) FG_LAUNCH(PRO_MERGE, EPI_RESIDUAL);
+  else if (pro == PRO_PLAIN && epi == EPI_RESIDUAL) FG_LAUNCH(PRO_PLAIN, EPI_RESIDUAL);
   else if (pro == PRO_NORM && epi == EPI_PLAIN) FG_LAUNCH(PRO_NORM, EPI_PLAIN);
   else if (pro == PRO_NORM && epi == EPI_SWIGLU) FG_LAUNCH(PRO_NORM, EPI_SWIGLU);
   else if (pro == PRO_NORM && epi == EPI_CONV) FG_LAUNCH(PRO_NORM, EPI_CONV);
@@ -530,8 +614,10 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
                              const void* W, const float* bias, int M, int N, int K, void* out, long out_ld,
                              int out_f32, float out_scale, int conv_lo, int conv_hi, int conv_k,
                              const float* conv_w, const float* conv_b, void* conv_state, const int* slot_ids,
-                             int feature_tiles, int w_fragments, hipStream_t stream) {
+                             int feature_tiles, int w_fragments, const float* ssq_in, int ssq_blocks, int ssq_width,
+                             float ssq_eps, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !out) return ERR_BAD_ARGUMENT;
+  if (ssq_in && (pro != PRO_PLAIN || ssq_blocks <= 0 || ssq_width <= 0)) return ERR_BAD_ARGUMENT;
   if (feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0) return ERR_UNSUPPORTED_SIZE;
   if (pro == PRO_NORM && (!h_in || !norm_w || h_out == h_in)) return ERR_BAD_ARGUMENT;
@@ -569,6 +655,10 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
   p.conv_state = (bf16_t*)conv_state;
   p.slot_ids = slot_ids;
   p.w_tiled = w_fragments ? 1 : 0;
+  p.ssq_in = ssq_in;
+  p.ssq_blocks = ssq_blocks;
+  p.ssq_width = ssq_width;
+  p.ssq_eps = ssq_eps;
   int code;
   if (MT == 1) code = launch_fused_gemm<1>(p, pro, epi, stream, 1, feature_tiles);
   else if (MT == 2) code = launch_fused_gemm<2>(p, pro, epi, stream, 1, feature_tiles);
@@ -619,12 +709,16 @@ extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, cons
 // run of keys: [M, heads, runs, head_dim + 2], with the same runs, run_keys, page_size and window.  Every
 // workgroup merges all of them again (a few hundred KB from the caches), which is cheaper than a launch of
 // mixer_merge_kernel while the step is small.  M <= 16; the merged columns must fit LDS beside the sums.
+// With res_h the result is not stored in `out` but added to the residual stream (the RESIDUAL epilogue, as in
+// mi_fused_gemm_residual).
 extern "C" int mi_fused_gemm_merge(const float* partial, const int* positions, int heads, int head_dim, int runs,
                                    int run_keys, int page_size, int window, const void* x, long x_ld, const void* W,
                                    const float* bias, int M, int N, int K, void* out, long out_ld, int w_fragments,
+                                   float* res_h, void* res_hb, long res_hb_ld, const float* res_w, float* ssq_out,
                                    hipStream_t stream) {
-  if (M <= 0 || N <= 0 || K <= 0 || !W || !out || !x || !partial || !positions || x_ld < K || x_ld % 8 != 0)
+  if (M <= 0 || N <= 0 || K <= 0 || !W || !x || !partial || !positions || x_ld < K || x_ld % 8 != 0)
     return ERR_BAD_ARGUMENT;
+  if (res_h ? (!res_hb || !res_w || !ssq_out || res_hb_ld < N) : !out) return ERR_BAD_ARGUMENT;
   if (heads <= 0 || head_dim <= 0 || runs <= 0 || run_keys <= 0 || page_size <= 0 || window < 0) return ERR_BAD_ARGUMENT;
   const long merged = (long)heads * head_dim;
   if (M > 16 || K % 32 != 0 || head_dim % 8 != 0 || merged % 32 != 0 || merged > K) return ERR_UNSUPPORTED_SIZE;
@@ -649,7 +743,50 @@ extern "C" int mi_fused_gemm_merge(const float* partial, const int* positions, i
   p.merge_run_keys = run_keys;
   p.merge_page = page_size;
   p.merge_window = window;
-  const int code = launch_fused_gemm<1>(p, PRO_MERGE, EPI_PLAIN, stream);
+  p.res_h = res_h;
+  p.res_hb = (bf16_t*)res_hb;
+  p.res_hb_ld = res_hb_ld;
+  p.res_w = res_w;
+  p.ssq_out = ssq_out;
+  const int code = launch_fused_gemm<1>(p, PRO_MERGE, res_h ? EPI_RESIDUAL : EPI_PLAIN, stream);
+  if (code != 0) return code;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// h[M, N] += x[M, K] . W[N, K]^T + bias in float32, in place: a projection whose result joins the residual stream.
+// Beside it, what the next norm's product needs without a pass of its own: hb[M, hb_ld] = bfloat16(h * next_w[n]),
+// the new rows times that norm's weight, and ssq_out[ceil(N / 16), 16 ceil(M / 16)], the sums of squares of each
+// new row over each workgroup's 16 features (mi_fused_gemm takes them as its row scale).  M <= 64.
+extern "C" int mi_fused_gemm_residual(const void* x, long x_ld, const void* W, const float* bias, int M, int N, int K,
+                                      float* res_h, void* res_hb, long res_hb_ld, const float* res_w, float* ssq_out,
+                                      int w_fragments, hipStream_t stream) {
+  if (M <= 0 || N <= 0 || K <= 0 || !W || !x || x_ld < K || x_ld % 8 != 0 || !res_h || !res_hb || !res_w || !ssq_out ||
+      res_hb_ld < N)
+    return ERR_BAD_ARGUMENT;
+  if (M > 64 || K % 32 != 0) return ERR_UNSUPPORTED_SIZE;
+  const int MT = (M + 15) / 16;
+  if (fused_gemm_lds(MT, PRO_PLAIN, K, M) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  FusedGemmParams p = {};
+  p.x = (const bf16_t*)x;
+  p.x_ld = x_ld;
+  p.W = (const bf16_t*)W;
+  p.bias = bias;
+  p.M = M;
+  p.N = N;
+  p.K = K;
+  p.out_scale = 1.0f;
+  p.w_tiled = w_fragments ? 1 : 0;
+  p.res_h = res_h;
+  p.res_hb = (bf16_t*)res_hb;
+  p.res_hb_ld = res_hb_ld;
+  p.res_w = res_w;
+  p.ssq_out = ssq_out;
+  int code;
+  if (MT == 1) code = launch_fused_gemm<1>(p, PRO_PLAIN, EPI_RESIDUAL, stream);
+  else if (MT == 2) code = launch_fused_gemm<2>(p, PRO_PLAIN, EPI_RESIDUAL, stream);
+  else if (MT == 3) code = launch_fused_gemm<3>(p, PRO_PLAIN, EPI_RESIDUAL, stream);
+  else code = launch_fused_gemm<4>(p, PRO_PLAIN, EPI_RESIDUAL, stream);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;

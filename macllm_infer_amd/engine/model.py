@@ -92,6 +92,14 @@ class DecoderModel:
         # the final norm as the skinny kernel's prologue, if it is that kind of norm
         prologue = getattr(self.final_norm, "rms_prologue", None)
         self._final_rms = prologue() if prologue is not None else None
+        # for every scheduled layer the (weight, eps) of the norm that follows it, where that is a root-mean-square
+        # norm: a layer may then hand the stream over prepared for it
+        def rms_of(norm):
+            prologue = getattr(norm, "rms_prologue", None)
+            return prologue() if prologue is not None else None
+
+        firsts = [rms_of(getattr(self.blocks[entry.layer], "first_norm", None)) for entry in spec.schedule]
+        self._next_norms = firsts[1:] + [self._final_rms]
         # the step's table of runs of one lane's tokens is cut for the mixer with the largest tile
         mixers = [mixer for block in self.blocks for _, mixer in block.mixers]
         self.query_tile = max((getattr(mixer, "query_tile", 0) for mixer in mixers), default=0)
@@ -112,6 +120,7 @@ class DecoderModel:
         for index, entry in enumerate(spec.schedule):
             block = self.blocks[entry.layer]
             caches = {name: cache.entry((index, name)) for name, _ in block.mixers}
+            residual.next_norm = self._next_norms[index]
             block.forward(residual, step, caches)
         wanted = step.want_rows.numel()
         if wanted == 0:
@@ -119,6 +128,13 @@ class DecoderModel:
         logits = torch.empty((wanted, spec.vocab_size), dtype=torch.float32, device=self.build.device)
         if self._fused_head(step, wanted):
             # a decode step whose every row is wanted: residual add, norm, projection and scaling in one launch
+            scaled = residual.scaled
+            if scaled is not None and scaled.weight is self._final_rms[0]:
+                # the last layer left the rows times the norm's weight and their sums of squares
+                ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, x=scaled.rows,
+                               row_scale=ops.RowScale(scaled.ssq, spec.hidden_size, self._final_rms[1]),
+                               fragments=self._head_fragments)
+                return logits
             ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, h_in=residual.h,
                            deltas=residual.pending, norm_weight=self._final_rms[0], eps=self._final_rms[1],
                            fragments=self._head_fragments)

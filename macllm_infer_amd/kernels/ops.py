@@ -77,14 +77,17 @@ _SIGNATURES = {
     "decode": {
         "mi_fused_gemm": [_c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_long, _c_ptr,
                           _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_int, _c_float, _c_int, _c_int, _c_int,
-                          _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+                          _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_float, _c_ptr],
+        "mi_fused_gemm_residual": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
+                                   _c_ptr, _c_ptr, _c_int, _c_ptr],
         "mi_fused_gemm_supported": [_c_int, _c_int, _c_int],
         "mi_fused_gemm_split": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int,
                                 _c_ptr],
         "mi_mixer_split_keys": [_c_int, _c_int, _c_int, _c_long],
         "mi_mixer_runs": [_c_int, _c_int, _c_int, _c_long, _c_ptr, _c_ptr],
         "mi_fused_gemm_merge": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_ptr,
-                                _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_int, _c_ptr],
+                                _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_int, _c_ptr, _c_ptr, _c_long, _c_ptr,
+                                _c_ptr, _c_ptr],
         "mi_mixer_decode": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int,
                             _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int,
                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -718,11 +721,13 @@ def fused_gemm_merge_supported(M: int, K: int, heads: int, head_dim: int) -> boo
             and waves * 1024 + 1024 + M * (merged + 8) * 2 <= 64 * 1024)
 
 
-def fused_gemm_merge(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, x: torch.Tensor,
-                     attended: AttentionRuns, fragments: Optional[torch.Tensor] = None) -> None:
+def fused_gemm_merge(weight: torch.Tensor, bias: Optional[torch.Tensor], out: Optional[torch.Tensor], x: torch.Tensor,
+                     attended: AttentionRuns, fragments: Optional[torch.Tensor] = None,
+                     residual: Optional[tuple] = None) -> None:
     """out[M, N] = x [M, K] . weight[N, K]^T (+ bias) in bfloat16 for a step of up to 16 rows, where the first
     heads * head_dim columns of x are not read but merged from the runs of keys that ``mixer_decode(merge=False)``
-    left: the merge of the runs and the product in one launch."""
+    left: the merge of the runs and the product in one launch.  With ``residual`` = (h, hb, next norm's weight,
+    ssq) the result is added to the residual stream as ``fused_gemm_residual`` does it, and ``out`` is None."""
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm_merge: weight must be contiguous bfloat16 [N, K]")
     N, K = weight.shape
@@ -731,8 +736,14 @@ def fused_gemm_merge(weight: torch.Tensor, bias: Optional[torch.Tensor], out: to
     _need(x.dtype == torch.bfloat16 and x.shape == (M, K) and x.data_ptr() % 16 == 0, "fused_gemm_merge: bad x")
     _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()),
           "fused_gemm_merge: bias must be float32 [N]")
-    _need(out.dtype == torch.bfloat16 and out.shape == (M, N), "fused_gemm_merge: out must be bfloat16 [M, N]")
-    out_ld = _row_major(out, "out")
+    h = hb = next_weight = ssq = None
+    hb_ld = out_ld = 0
+    if residual is not None:
+        h, hb, next_weight, ssq = residual
+        hb_ld = _residual_arguments(h, hb, next_weight, ssq, M, N, "fused_gemm_merge")
+    else:
+        _need(out.dtype == torch.bfloat16 and out.shape == (M, N), "fused_gemm_merge: out must be bfloat16 [M, N]")
+        out_ld = _row_major(out, "out")
     _need(attended.partial.dtype == torch.float32 and attended.partial.is_contiguous()
           and attended.partial.numel() >= M * attended.heads * attended.runs * (attended.head_dim + 2),
           "fused_gemm_merge: the partial results do not cover the step")
@@ -742,7 +753,8 @@ def fused_gemm_merge(weight: torch.Tensor, bias: Optional[torch.Tensor], out: to
     _check(_fn("decode", "mi_fused_gemm_merge")(
         _p(attended.partial), _p(attended.positions), attended.heads, attended.head_dim, attended.runs,
         attended.run_keys, attended.page_size, attended.window, _p(x), x_ld, _p(operand), _p(bias), M, N, K, _p(out),
-        out_ld, int(fragments is not None), _stream()), "fused_gemm_merge", f"(M={M}, N={N}, K={K})")
+        out_ld, int(fragments is not None), _p(h), _p(hb), hb_ld, _p(next_weight), _p(ssq), _stream()),
+        "fused_gemm_merge", f"(M={M}, N={N}, K={K})")
 
 
 def fused_gemm_split(weight: torch.Tensor, bias: Optional[torch.Tensor], x: torch.Tensor, partial: torch.Tensor,
@@ -772,7 +784,8 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
                x: Optional[torch.Tensor] = None, h_in: Optional[torch.Tensor] = None,
                deltas: Sequence[torch.Tensor] = (), h_out: Optional[torch.Tensor] = None,
                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, epilogue: int = EPI_PLAIN,
-               conv: Optional[dict] = None, feature_tiles: int = 1, fragments: Optional[torch.Tensor] = None) -> None:
+               conv: Optional[dict] = None, feature_tiles: int = 1, fragments: Optional[torch.Tensor] = None,
+               row_scale: Optional["RowScale"] = None) -> None:
     """out[M, N'] = epilogue(prologue . weight[N, K]^T + bias) for a small batch in bfloat16.
 
     Prologue: ``x`` [M, K] bfloat16, or ``h_in`` float32 [M, K] with up to two bfloat16 ``deltas``:
@@ -783,9 +796,16 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
     rows lo..hi-1 go through the causal depthwise conv step of their channel with the request's
     tail (which is rolled) and SiLU.  ``feature_tiles`` (1, 2 or 4; more than one with ``x`` only): how many
     tiles of 16 output features a workgroup owns; the rows of x cross the caches once per workgroup, so
-    steps of many rows gain from more.  ``fragments``: ``fragment_order(weight)``, read instead of the weight."""
+    steps of many rows gain from more.  ``fragments``: ``fragment_order(weight)``, read instead of the weight.
+    ``row_scale`` (with ``x``): x holds rows times a norm's weight that are not divided by their root mean
+    square yet; the sums of row m are multiplied by 1 / sqrt(sum of squares of the row / width + eps) before the
+    bias, from the partial sums of squares that ``fused_gemm_residual`` left."""
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm: weight must be contiguous bfloat16 [N, K]")
+    _need(row_scale is None or x is not None, "fused_gemm: a row scale needs x")
+    if row_scale is not None:
+        _need(row_scale.ssq.dtype == torch.float32 and row_scale.ssq.is_contiguous() and row_scale.ssq.dim() == 2
+              and row_scale.ssq.shape[1] == 16 * (-(-out.shape[0] // 16)), "fused_gemm: the partial sums of squares do not fit the step")
     _need(feature_tiles in (1, 2, 4) and (feature_tiles == 1 or x is not None),
           "fused_gemm: feature_tiles is 1, 2 or 4, and more than 1 needs x")
     N, K = weight.shape
@@ -828,7 +848,56 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
         _p(h_out), _p(norm_weight), float(eps), _p(x), x_ld, _p(_weight_operand(weight, fragments, "fused_gemm")),
         _p(bias), M, N, K, _p(out), out_ld,
         1 if out.dtype == torch.float32 else 0, float(out_scale), lo, hi, taps, _p(conv_w), _p(conv_b), _p(conv_state),
-        _p(slot_ids), int(feature_tiles), int(fragments is not None), _stream()), "fused_gemm", f"(M={M}, N={N}, K={K})")
+        _p(slot_ids), int(feature_tiles), int(fragments is not None),
+        _p(row_scale.ssq) if row_scale is not None else None, row_scale.ssq.shape[0] if row_scale is not None else 0,
+        int(row_scale.width) if row_scale is not None else 0, float(row_scale.eps) if row_scale is not None else 0.0,
+        _stream()), "fused_gemm", f"(M={M}, N={N}, K={K})")
+
+
+@dataclass(frozen=True)
+class RowScale:
+    """Partial sums of squares ``ssq`` float32 [workgroups, 16 ceil(M / 16)] of rows of ``width`` elements, and the
+    ``eps`` of the norm they belong to: what ``fused_gemm_residual`` leaves for the product behind the norm."""
+    ssq: torch.Tensor
+    width: int
+    eps: float
+
+
+def residual_workspace(M: int, N: int, device) -> torch.Tensor:
+    """The partial sums of squares of a step of M rows of N elements, for ``fused_gemm_residual`` to fill."""
+    return torch.empty((-(-N // 16), 16 * (-(-M // 16))), dtype=torch.float32, device=device)
+
+
+def _residual_arguments(h, hb, next_weight, ssq, M, N, name):
+    _need(h.dtype == torch.float32 and h.shape == (M, N) and h.is_contiguous(), f"{name}: h must be contiguous float32 [M, N]")
+    _need(hb.dtype == torch.bfloat16 and hb.shape == (M, N), f"{name}: hb must be bfloat16 [M, N]")
+    _need(next_weight.dtype == torch.float32 and next_weight.numel() == N and next_weight.is_contiguous(),
+          f"{name}: the next norm's weight must be float32 [N]")
+    _need(ssq.dtype == torch.float32 and ssq.is_contiguous() and ssq.shape == (-(-N // 16), 16 * (-(-M // 16))),
+          f"{name}: ssq must be float32 [ceil(N / 16), 16 ceil(M / 16)]")
+    return _row_major(hb, "hb")
+
+
+def fused_gemm_residual(weight: torch.Tensor, bias: Optional[torch.Tensor], x: torch.Tensor, h: torch.Tensor,
+                        hb: torch.Tensor, next_weight: torch.Tensor, ssq: torch.Tensor,
+                        fragments: Optional[torch.Tensor] = None) -> None:
+    """h += x [M, K] . weight[N, K]^T (+ bias), float32 in place: a projection whose result joins the residual
+    stream.  Beside it ``hb`` = bfloat16(h * next_weight), the new rows times the next norm's weight, and ``ssq``
+    (``residual_workspace``), the sums of squares of the new rows over every 16 features: what ``fused_gemm`` with
+    ``row_scale`` needs to be the product behind that norm, without a pass for the norm."""
+    _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
+          "fused_gemm_residual: weight must be contiguous bfloat16 [N, K]")
+    N, K = weight.shape
+    x_ld = _row_major(x, "x")
+    M = x.shape[0]
+    _need(x.dtype == torch.bfloat16 and x.shape == (M, K) and x.data_ptr() % 16 == 0, "fused_gemm_residual: bad x")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()),
+          "fused_gemm_residual: bias must be float32 [N]")
+    hb_ld = _residual_arguments(h, hb, next_weight, ssq, M, N, "fused_gemm_residual")
+    _check(_fn("decode", "mi_fused_gemm_residual")(
+        _p(x), x_ld, _p(_weight_operand(weight, fragments, "fused_gemm_residual")), _p(bias), M, N, K, _p(h), _p(hb),
+        hb_ld, _p(next_weight), _p(ssq), int(fragments is not None), _stream()), "fused_gemm_residual",
+        f"(M={M}, N={N}, K={K})")
 
 
 def mixer_decode_supported(num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, state_size: int,

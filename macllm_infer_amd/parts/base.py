@@ -59,13 +59,46 @@ class BuildContext:
     measure_paths: bool = True
 
 
+@dataclass
+class ScaledRows:
+    """The residual stream's rows as the product behind a norm wants them, but for the division by the root mean
+    square: ``rows`` bfloat16 [T, d] = h * weight, with the partial sums of squares of h (``ssq``, float32
+    [workgroups, rows rounded up to 16]) that give it.  ``weight`` is the norm's weight they were made for."""
+    rows: torch.Tensor
+    ssq: torch.Tensor
+    weight: torch.Tensor
+
+
 class Residual:
     """The float32 residual stream [T, d] plus the branch outputs not yet added to it.
-    The next norm adds them and normalizes in one kernel."""
+    The next norm adds them and normalizes in one kernel.
+
+    ``next_norm``: (weight, eps) of the norm that the layer after the one running starts with (the final norm
+    after the last), if that norm is a root-mean-square norm, set by whoever runs the layers; a layer whose last
+    projection adds to the stream itself may then leave ``scaled`` rows for it.  ``scaled`` is dropped whenever
+    ``h`` or ``pending`` is assigned: whoever changes the stream without knowing of it makes it stale."""
 
     def __init__(self, h: torch.Tensor):
-        self.h = h
-        self.pending: List[torch.Tensor] = []
+        self._h = h
+        self._pending: List[torch.Tensor] = []
+        self.scaled: Optional[ScaledRows] = None
+        self.next_norm: Optional[tuple] = None
+
+    @property
+    def h(self) -> torch.Tensor:
+        return self._h
+
+    @h.setter
+    def h(self, value: torch.Tensor) -> None:
+        self._h, self.scaled = value, None
+
+    @property
+    def pending(self) -> List[torch.Tensor]:
+        return self._pending
+
+    @pending.setter
+    def pending(self, value: List[torch.Tensor]) -> None:
+        self._pending, self.scaled = value, None
 
 
 class Part:

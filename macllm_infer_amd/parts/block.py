@@ -83,6 +83,11 @@ class ParallelPreNormBlock:
         parts = [self.mixer_norm, self.ffn_norm, self.ffn] + [mixer for _, mixer in self.mixers]
         return all(getattr(part, "graph_safe", False) for part in parts)
 
+    @property
+    def first_norm(self):
+        """The norm this arrangement starts with: what a layer before it may prepare the stream for."""
+        return self.mixer_norm
+
     def forward(self, residual: Residual, step, caches) -> None:
         """``caches``: mixer name -> EntryCache of this run of the layer."""
         fusion = self.fusion

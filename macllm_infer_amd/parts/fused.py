@@ -38,7 +38,7 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .base import Residual
+from .base import Residual, ScaledRows
 from .block import register_fusion
 from .position import NoPosition, Rope
 
@@ -92,6 +92,12 @@ MERGE_LATER_ROWS = 16
 MERGE_LATER_BYTES = 96 << 10
 FORCE_MERGE_LATER: Optional[bool] = None  # tests: True or False instead of the rule
 _padding_wins: Dict[tuple, tuple] = {}
+# A projection whose result joins the residual stream can add it there itself (float32, in place) and leave, beside
+# the stream, its rows times the next norm's weight in bfloat16 with the partial sums of their squares; the product
+# behind that norm then reads those rows and multiplies its float32 sums by 1 / sqrt(mean square + eps): the norm
+# costs no pass of its own and no prologue in every workgroup.  Taken for the step sizes at which a layer's four
+# projections all run through the skinny kernel unsplit, with one tile in the two that feed the stream.
+FORCE_DEFERRED_NORM: Optional[bool] = None  # tests: False = never
 
 
 OVERLAP_MIN_TOKENS = 256       # prompt portions from this size on run their two mixers on two streams
@@ -357,6 +363,9 @@ class LayerFusion:
         self.mixer_rms = _rms_prologue(block.mixer_norm) if self.norm_rows else None
         self.ffn_rms = _rms_prologue(block.ffn_norm) if self.norm_rows else None
         self.norm_fits = self.mixer_rms is not None and self.ffn_rms is not None
+        # the same two norms for the products that take them as a row scale (any width)
+        self.mixer_scale = _rms_prologue(block.mixer_norm) if self.decode_ok else None
+        self.ffn_scale = _rms_prologue(block.ffn_norm) if self.decode_ok else None
         # a kernel for this set of mixers, if one is registered and takes these sizes
         factory = _MIXER_KERNELS.get(tuple(getattr(mixer, "kind", None) for mixer in self.mixers))
         self.kernel = factory(self) if factory is not None and self.decode_ok else None
@@ -389,6 +398,16 @@ class LayerFusion:
                                                                 self.tiles_down)
             self.f_gate_up = fragments(self.gate_up.weight, self.library_gate_up, ())
             self.f_down = fragments(self.down.weight, self.library_down, self.split_down)
+        # step sizes at which the norms are left to the projections around them
+        self.deferred = tuple(self._defers(bucket) for bucket in range(BUCKETS))
+
+    def _defers(self, bucket: int) -> bool:
+        if (FORCE_DEFERRED_NORM is False or self.gate_up is None or not self.decode_ok or self.ffn_scale is None
+                or self.hidden % 16 != 0):
+            return False
+        return not (self.library_in[bucket] or self.library_out[bucket] or self.library_gate_up[bucket]
+                    or self.library_down[bucket] or self.split_out[bucket] or self.split_down[bucket]
+                    or self.tiles_out[bucket] != 1 or self.tiles_down[bucket] != 1)
 
     def path_choices(self) -> dict:
         """Which way each projection goes for steps of up to TUNE_ROWS rows, as short strings (S: the skinny
@@ -407,7 +426,8 @@ class LayerFusion:
         if self.gate_up is not None:
             out.update({"gate_up": way(self.library_gate_up), "down": way(self.library_down, self.split_down),
                         "tiles_gate_up": "/".join(map(str, self.tiles_gate_up)),
-                        "tiles_down": "/".join(map(str, self.tiles_down))})
+                        "tiles_down": "/".join(map(str, self.tiles_down)),
+                        "norms": "/".join("D" if deferred else "-" for deferred in self.deferred)})
         return out
 
     def decode_supported(self, step, caches) -> bool:
@@ -539,11 +559,35 @@ class LayerFusion:
             arguments = dict(h_in=residual.h, deltas=pending, h_out=h_out, norm_weight=rms[0], eps=rms[1])
             return arguments, h_out
 
+        deferred = self.deferred[bucket]
+        scaled = residual.scaled
+
+        def to_the_stream(x, weight, bias, fragments, next_weight, attended=None):
+            """h += the projection, with the rows the product behind the norm of ``next_weight`` reads."""
+            rows = torch.empty((M, self.hidden), dtype=bf16, device=device)
+            ssq = ops.residual_workspace(M, self.hidden, device)
+            if attended is not None:
+                ops.fused_gemm_merge(weight, bias, None, x, attended, fragments,
+                                     residual=(residual.h, rows, next_weight, ssq))
+            else:
+                ops.fused_gemm_residual(weight, bias, x, residual.h, rows, next_weight, ssq, fragments)
+            residual.scaled = ScaledRows(rows, ssq, next_weight)
+
+        def behind_the_norm(rms):
+            return dict(x=scaled.rows, row_scale=ops.RowScale(scaled.ssq, self.hidden, rms[1]))
+
         # 1
         conv = None
         if kernel is not None and kernel.conv is not None:
             conv = dict(kernel.conv, state=kernel.conv_state(caches), slot_ids=step.slot_ids)
-        if self.library_in[bucket]:
+        if (scaled is not None and not self.library_in[bucket] and self.mixer_scale is not None
+                and scaled.weight is self.mixer_scale[0] and not residual.pending):
+            # the layer before left the stream prepared for this norm
+            u = torch.empty((M, self.in_ld), dtype=bf16, device=device)
+            ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width],
+                           epilogue=ops.EPI_CONV if conv is not None else ops.EPI_PLAIN, conv=conv,
+                           feature_tiles=self.tiles_in[bucket], fragments=self.f_in, **behind_the_norm(self.mixer_scale))
+        elif self.library_in[bucket]:
             u = ops.linear(block.mixer_norm.forward(residual), self.w_in, self.b_in)
             if conv is not None:
                 ops.conv_step(u, conv["lo"], conv["hi"] - conv["lo"], conv["weight"], conv["bias"], conv["state"],
@@ -566,15 +610,25 @@ class LayerFusion:
             attended = kernel.run(u, step, caches, mixed, merge=not later)
         else:
             self._mix_each(u, step, caches, mixed)
-        # 3
-        residual.pending = self._to_the_stream(mixed, self.w_out, self.b_out, self.library_out[bucket],
-                                               self.split_out[bucket], self.tiles_out[bucket], self.f_out, attended)
+        # 3 (whatever ran in 1 has added what was pending to the stream)
+        if deferred and not residual.pending:
+            to_the_stream(mixed, self.w_out, self.b_out, self.f_out, self.ffn_scale[0], attended)
+        else:
+            residual.pending = self._to_the_stream(mixed, self.w_out, self.b_out, self.library_out[bucket],
+                                                   self.split_out[bucket], self.tiles_out[bucket], self.f_out, attended)
         # 4
         if self.gate_up is None:
             residual.pending = [block.ffn.forward(block.ffn_norm.forward(residual))]
             return
         activated = torch.empty((M, self.inner), dtype=bf16, device=device)
-        if self.library_gate_up[bucket]:
+        scaled = residual.scaled
+        if scaled is not None and (self.ffn_scale is None or scaled.weight is not self.ffn_scale[0]):
+            scaled = None
+        if scaled is not None:
+            ops.fused_gemm(self.gate_up.weight, self.gate_up.bias, activated, epilogue=ops.EPI_SWIGLU,
+                           feature_tiles=self.tiles_gate_up[bucket], fragments=self.f_gate_up,
+                           **behind_the_norm(self.ffn_scale))
+        elif self.library_gate_up[bucket]:
             ops.swiglu(ops.linear(block.ffn_norm.forward(residual), self.gate_up.weight, self.gate_up.bias), activated, 8)
         else:
             arguments, h_out = norm_prologue(block.ffn_norm, self.ffn_rms)
@@ -584,6 +638,9 @@ class LayerFusion:
             if h_out is not None:
                 residual.h, residual.pending = h_out, []
         # 5
+        if scaled is not None and residual.next_norm is not None:
+            to_the_stream(activated, self.down.weight, self.down.bias, self.f_down, residual.next_norm[0])
+            return
         residual.pending = self._to_the_stream(activated, self.down.weight, self.down.bias, self.library_down[bucket],
                                                self.split_down[bucket], self.tiles_down[bucket], self.f_down)
 

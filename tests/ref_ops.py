@@ -269,8 +269,22 @@ def mixer_decode_supported(num_heads, num_kv_heads, head_dim, page_size, state_s
     return False
 
 
+def fused_gemm_residual(weight, bias, x, h, hb, next_weight, ssq, fragments=None):
+    """h += x . W^T + bias; hb = bfloat16(h * next_weight); ssq[b, m] = the sum of h[m]^2 over features 16 b .. 16 b + 15."""
+    y = _f(x) @ _f(weight).T
+    if bias is not None:
+        y = y + bias
+    h += y
+    hb.copy_((h * next_weight).to(hb.dtype))
+    M, N = h.shape
+    squares = torch.zeros(M, ssq.shape[0] * 16)
+    squares[:, :N] = h.pow(2)
+    ssq.zero_()
+    ssq[:, :M] = squares.reshape(M, -1, 16).sum(-1).T
+
+
 def fused_gemm(weight, bias, out, *, out_scale=1.0, x=None, h_in=None, deltas=(), h_out=None, norm_weight=None,
-               eps=0.0, epilogue=EPI_PLAIN, conv=None, feature_tiles=1, fragments=None):
+               eps=0.0, epilogue=EPI_PLAIN, conv=None, feature_tiles=1, fragments=None, row_scale=None):
     if x is None:
         total = h_in.clone()
         for delta in deltas:
@@ -282,6 +296,9 @@ def fused_gemm(weight, bias, out, *, out_scale=1.0, x=None, h_in=None, deltas=()
     else:
         rows = _f(x)
     y = rows @ _f(weight).T
+    if row_scale is not None:                  # the norm's division, on the float32 sums
+        squares = row_scale.ssq[:, :y.shape[0]].sum(0)
+        y = y * (1.0 / torch.sqrt(squares / row_scale.width + row_scale.eps))[:, None]
     if bias is not None:
         y = y + bias
     M, N = y.shape

@@ -476,10 +476,11 @@ def test_fixed_paths_take_no_measurement(tmp_path, monkeypatch):
                         max_active_sequences=24, measured_paths=measured)
         choices = engine.path_choices()
         assert set(choices) == {"in", "out", "gate_up", "down", "tiles_in", "tiles_out", "tiles_gate_up", "tiles_down",
-                                "padded_in"}
+                                "padded_in", "norms"}
         assert all(len(value.split("/")) == 5 for value in choices.values())
         if not measured:
             assert choices["in"] == choices["out"] == choices["gate_up"] == choices["down"] == "S/S/S/S/S"
+            assert choices["norms"] == "D/D/D/D/D"
             assert choices["tiles_in"] == choices["tiles_down"] == "1/1/1/1/1" and choices["padded_in"] == "-/-/-/-/-"
         for index in prompts:
             engine.add_request(index)
@@ -488,6 +489,47 @@ def test_fixed_paths_take_no_measurement(tmp_path, monkeypatch):
         for row, tokens in enumerate(prompts.values()):
             want = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-1]
             assert gates.bfloat16_close(logits[row].numpy(), want.numpy()), (measured, row)
+
+
+def test_norms_left_to_the_projections_around_them(tmp_path, monkeypatch):
+    """A layer whose projections all run through the skinny kernels leaves its norms to them: the output and
+    down projections add to the float32 stream themselves and hand on the rows times the next norm's weight with
+    their sums of squares, up to the output head.  With that switched off the norms run in prologues or as
+    kernels of their own.  Both ways: steps of 1, 5 and 18 single tokens and a step of 20 and 3 prompt tokens
+    beside decoded ones (more than 16 rows: several row tiles), each close to the plain model."""
+    import gates
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.parts import fused
+    folder = tiny_configs.make_model_dir("C", tmp_path, torch.bfloat16)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    prompts = {index: tokens_for(cfg["vocab_size"], 6 + index % 5, 400 + index) for index in range(24)}
+    late = {"x": tokens_for(cfg["vocab_size"], 21, 450), "y": tokens_for(cfg["vocab_size"], 4, 451)}
+    for deferred in (False, None):
+        monkeypatch.setattr(fused, "FORCE_DEFERRED_NORM", deferred)
+        engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * 26,
+                        max_active_sequences=26)
+        assert engine.path_choices()["norms"] == ("-/-/-/-/-" if deferred is False else "D/D/D/D/D")
+        for index in list(prompts) + list(late):
+            engine.add_request(index)
+        engine.step([Lane(index, tokens[:-1], []) for index, tokens in prompts.items()])
+        checked = 0
+        for group in (range(0, 1), range(1, 6), range(6, 24)):             # steps of 1, 5 and 18 single tokens
+            logits = engine.step([Lane(index, prompts[index][-1:], [0]) for index in group]).float().cpu()
+            for row, index in enumerate(group):
+                want = plain_impl.falcon_h1_logits(cfg, tensors, prompts[index])[-1]
+                assert gates.bfloat16_close(logits[row].numpy(), want.numpy()), (deferred, index)
+                checked += 1
+        lanes = [Lane("x", late["x"][:20], [19]), Lane("y", late["y"][:3], [0, 2])]
+        lanes += [Lane(index, [7 + index], [0]) for index in range(3)]
+        logits = engine.step(lanes).float().cpu()
+        wants = [plain_impl.falcon_h1_logits(cfg, tensors, late["x"][:20])[19],
+                 plain_impl.falcon_h1_logits(cfg, tensors, late["y"][:3])[0],
+                 plain_impl.falcon_h1_logits(cfg, tensors, late["y"][:3])[2]]
+        wants += [plain_impl.falcon_h1_logits(cfg, tensors, prompts[index] + [7 + index])[-1] for index in range(3)]
+        for row, want in enumerate(wants):
+            assert gates.bfloat16_close(logits[row].numpy(), want.numpy()), (deferred, "mixed", row)
+        assert checked == 24
+        engine.cache.check()
 
 
 def test_the_output_projection_may_merge_the_runs_of_keys(monkeypatch):
@@ -589,7 +631,15 @@ def test_layers_of_one_mixer_and_a_mixer_from_outside_take_the_fast_paths(monkey
         calls["library"] += 1
         return real_library(*arguments, **named)
 
+    calls["to the stream"] = 0
+    real_residual = ops.fused_gemm_residual
+
+    def to_the_stream(*arguments, **named):
+        calls["to the stream"] += 1
+        return real_residual(*arguments, **named)
+
     monkeypatch.setattr(ops, "fused_gemm", skinny)
+    monkeypatch.setattr(ops, "fused_gemm_residual", to_the_stream)
     monkeypatch.setattr(ops, "linear", library)
     sequences = {"a": tokens_for(150, 60, 21), "b": tokens_for(150, 45, 22)}
     rows = {"a": [], "b": []}
@@ -602,8 +652,10 @@ def test_layers_of_one_mixer_and_a_mixer_from_outside_take_the_fast_paths(monkey
     for position in range(15):
         out = engine.step([Lane("a", [sequences["a"][40 + position]], [0]), Lane("b", [sequences["b"][30 + position]], [0])])
         rows["a"].append(out[:1].cpu()), rows["b"].append(out[1:].cpu())
-    # a decode step: input and output projections of both layers, gate/up and down of the first, and the head
-    assert calls["skinny"] == 15 * 7 and calls["library"] == 0
+    # a decode step: input and output projections of both layers, gate/up and down of the first, and the head; the
+    # first layer's output projection adds to the stream itself and leaves the norm to gate/up (its down projection
+    # does not: the toy norm that follows is none it could prepare for)
+    assert calls["skinny"] == 15 * 6 and calls["to the stream"] == 15 and calls["library"] == 0
     for name, tokens in sequences.items():
         want = toy_parts.toy_fast_plain_logits(raw, tensors, tokens[:len(torch.cat(rows[name]))]).numpy()
         assert gates.bfloat16_close(torch.cat(rows[name]).numpy(), want), name

@@ -791,6 +791,49 @@ def test_fused_gemm_norm_prologue_and_epilogues(ops, M, N, K, deltas):
         assert torch.equal(got_state[unused].cpu(), state[unused])
 
 
+@pytest.mark.parametrize("M, N, K, N2", [(8, 1024, 2048, 4120), (1, 72, 64, 48), (13, 1000, 96, 160), (16, 3072, 4608, 272),
+                                         (40, 200, 2048, 96), (40, 256, 2048, 96), (24, 96, 64, 80), (64, 1024, 2048, 272)])
+def test_a_product_that_joins_the_residual_stream_and_the_product_behind_the_next_norm(ops, M, N, K, N2):
+    """``fused_gemm_residual``: h += x . W^T + b in float32 in place, with the new rows times the next norm's
+    weight in bfloat16 and the partial sums of their squares; then ``fused_gemm`` with that row scale against the
+    norm written out (the division of the root mean square applied to the rows, then the product), plain, with
+    the SwiGLU epilogue and with the conv step; a width that is no multiple of 16, 1 to 40 rows."""
+    x = rand(M, K, seed=350, dtype=torch.bfloat16)
+    W, b = rand(N, K, seed=351, scale=0.1, dtype=torch.bfloat16), rand(N, seed=352)
+    h = rand(M, N, seed=353, scale=2.0)
+    next_w = rand(N, seed=354, scale=0.1) + 1.0
+    want_h, want_hb, want_ssq = h.clone(), torch.empty(M, N, dtype=torch.bfloat16), ops.residual_workspace(M, N, "cpu")
+    ref_ops.fused_gemm_residual(W, b, x, want_h, want_hb, next_w, want_ssq)
+    assert torch.allclose(want_h, h + x.float() @ W.float().T + b, atol=1e-4)
+    for fragments in (None, ops.fragment_order(W.to(DEV))):
+        got_h, got_hb = h.clone().to(DEV), torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        got_ssq = torch.full_like(ops.residual_workspace(M, N, DEV), float("nan"))
+        ops.fused_gemm_residual(W.to(DEV), b.to(DEV), x.to(DEV), got_h, got_hb, next_w.to(DEV), got_ssq, fragments)
+        close(got_h, want_h, torch.float32, max(1.0, want_h.abs().max().item()))
+        close(got_hb, want_hb, torch.bfloat16, max(1.0, want_hb.float().abs().max().item()))
+        assert torch.allclose(got_ssq[:, :M].cpu(), want_ssq[:, :M], rtol=1e-4, atol=1e-4)
+    # the product behind the norm: rows = h / rms(h) * w, rounded to bfloat16
+    eps = 3e-5
+    normed = (want_h / torch.sqrt(want_h.pow(2).mean(-1, keepdim=True) + eps) * next_w)
+    W2, b2 = rand(N2, N, seed=355, scale=0.1, dtype=torch.bfloat16), rand(N2, seed=356)
+    scale = ops.RowScale(got_ssq, N, eps)
+    if N % 32 == 0 and M <= 64:
+        want = normed @ W2.float().T + b2
+        got = torch.empty(M, N2, dtype=torch.bfloat16, device=DEV)
+        ops.fused_gemm(W2.to(DEV), b2.to(DEV), got, x=got_hb, row_scale=scale)
+        close(got, want, torch.bfloat16, 3.0 * max(1.0, want.abs().max().item()))
+        again = torch.empty(M, N2, dtype=torch.bfloat16)
+        ref_ops.fused_gemm(W2, b2, again, x=got_hb.cpu(), row_scale=ops.RowScale(got_ssq.cpu(), N, eps))
+        close(got, again, torch.bfloat16, max(1.0, want.abs().max().item()))
+        if N2 % 16 == 0:
+            want = torch.empty(M, N2 // 2, dtype=torch.bfloat16)
+            ref_ops.fused_gemm(W2, b2, want, x=got_hb.cpu(), row_scale=ops.RowScale(got_ssq.cpu(), N, eps), epilogue=ref_ops.EPI_SWIGLU)
+            got = torch.empty(M, N2 // 2, dtype=torch.bfloat16, device=DEV)
+            ops.fused_gemm(W2.to(DEV), b2.to(DEV), got, x=got_hb, row_scale=scale, epilogue=ops.EPI_SWIGLU,
+                           feature_tiles=2 if M > 16 else 1)
+            close(got, want, torch.bfloat16, 16.0)
+
+
 @pytest.mark.parametrize("M, N, K, S", [(64, 1024, 2048, 8), (33, 100, 2048, 16), (17, 48, 96, 3), (64, 136, 3072, 5),
                                         (5, 64, 64, 1)])
 def test_fused_gemm_split_over_k_and_the_norm_that_adds_its_slabs(ops, M, N, K, S):
@@ -1011,6 +1054,16 @@ def test_output_projection_that_merges_the_runs_of_keys(ops, Hq, Hkv, dh, E, N_o
         got = torch.empty(M, N_out, dtype=dtype, device=DEV)
         ops.fused_gemm_merge(weight, bias, got, unmerged, runs, fragments)
         assert torch.equal(got, want)
+    # and the same with the result added to the residual stream: what ``fused_gemm_residual`` gives on the merged rows
+    h, next_w = rand(M, N_out, seed=817, scale=2.0).to(DEV), (rand(N_out, seed=818, scale=0.1) + 1.0).to(DEV)
+    want_h, want_rows = h.clone(), torch.empty(M, N_out, dtype=dtype, device=DEV)
+    want_ssq = ops.residual_workspace(M, N_out, DEV)
+    ops.fused_gemm_residual(weight, bias, mixed, want_h, want_rows, next_w, want_ssq)
+    got_h, got_rows = h.clone(), torch.empty(M, N_out, dtype=dtype, device=DEV)
+    got_ssq = ops.residual_workspace(M, N_out, DEV)
+    ops.fused_gemm_merge(weight, bias, None, unmerged, runs, None, residual=(got_h, got_rows, next_w, got_ssq))
+    assert torch.equal(got_h, want_h) and torch.equal(got_rows, want_rows)
+    assert torch.equal(got_ssq[:, :M], want_ssq[:, :M])
     product = mixed.float().cpu() @ weight.float().cpu().T + bias.cpu()
     close(want, product, dtype, max(1.0, product.abs().max().item()))
 
