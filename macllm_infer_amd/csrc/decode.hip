@@ -157,14 +157,13 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   constexpr int PARTS = SSQ_PARTS / MT;               // PARTS * 16 MT threads: within the 256 of four waves
   // asked for without a branch (under one, the wave waits for them before it asks for its weights) and not added
   // up before the products are done; without a row scale, and past the last workgroup's sums, a valid address
-  float ssq_early[SSQ_EARLY];
-  {
-    const float* sums = p.ssq_in ? p.ssq_in : reinterpret_cast<const float*>(p.W);
-    const int last = p.ssq_in ? p.ssq_blocks - 1 : 0;
-    const int row = p.ssq_in ? tid % (16 * MT) : 0;
+  float ssq_early[SSQ_EARLY] = {};
+  if (p.ssq_in) {
+    const int last = p.ssq_blocks - 1;
+    const int row = tid % (16 * MT);
 #pragma unroll
     for (int i = 0; i < SSQ_EARLY; ++i)
-      ssq_early[i] = sums[(long)min(tid / (16 * MT) + i * PARTS, last) * (16 * MT) + row];
+      ssq_early[i] = p.ssq_in[(long)min(tid / (16 * MT) + i * PARTS, last) * (16 * MT) + row];
   }
   float res_old[EPT] = {};
   float res_weight = 0.f;

@@ -15,6 +15,14 @@ from ..parts.block import arrangement_class
 from ..weights.loader import Expect
 
 
+# Up to this many wanted rows the output head streams through the skinny kernel (the norm as a kernel of its own
+# before it), beyond through the library: a 130,049 x 3,072 head takes 138 / 144 / 159 / 203 us at 1 / 4 / 8 / 16 rows
+# against the library's 147 / 152 / 155 / 160, a 32,784 x 1,024 one 22 to 24 against 25 to 26.  (The norm in the skinny
+# kernel's prologue, every workgroup normalizing the rows again, took 305 to 370 us on the first and 23 to 39 on the
+# second, and 1,333 on a 261,120 x 5,120 head that streams in 450.)
+HEAD_SKINNY_ROWS = 8
+
+
 class DecoderModel:
     @staticmethod
     def expected_tensors(spec: ModelSpec) -> List[Expect]:
@@ -77,6 +85,10 @@ class DecoderModel:
             table = table.to(torch.float32)
         self.embedding = table.contiguous().to(build.device)
         self.blocks = [arrangement_class(layer.arrangement)(layer, tensors, build) for layer in spec.layers]
+        for block in self.blocks:                    # what a layer decides by timing itself among the others
+            tune = getattr(block, "tune", None)
+            if tune is not None:
+                tune(self.blocks)
         self.final_norm = part_class(spec.final_norm)(spec.final_norm, spec.final_norm_name, tensors, build)
         if spec.tied_embeddings:
             self.lm_head = self.embedding
@@ -85,11 +97,11 @@ class DecoderModel:
             if build.dtype == torch.float32:
                 head = head.to(torch.float32)
             self.lm_head = head.contiguous().to(build.device)
-        # the copy of the head that the skinny kernel streams fastest, for decode steps that want every row
+        # the copy of the head that the skinny kernel streams fastest, for steps that want few rows
         fused_head = (build.device.type == "cuda" and build.dtype == torch.bfloat16 and self.lm_head.dtype == torch.bfloat16
-                      and spec.hidden_size % 32 == 0 and ops.fused_gemm_supported(True, 1, spec.hidden_size))
+                      and spec.hidden_size % 32 == 0 and ops.fused_gemm_supported(False, 1, spec.hidden_size))
         self._head_fragments = ops.fragment_order(self.lm_head) if fused_head else None
-        # the final norm as the skinny kernel's prologue, if it is that kind of norm
+        # the final norm's (weight, eps), if it is a root-mean-square norm: the last layer may prepare the stream for it
         prologue = getattr(self.final_norm, "rms_prologue", None)
         self._final_rms = prologue() if prologue is not None else None
         # for every scheduled layer the (weight, eps) of the norm that follows it, where that is a root-mean-square
@@ -126,27 +138,26 @@ class DecoderModel:
         if wanted == 0:
             return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.build.device)
         logits = torch.empty((wanted, spec.vocab_size), dtype=torch.float32, device=self.build.device)
-        if self._fused_head(step, wanted):
-            # a decode step whose every row is wanted: residual add, norm, projection and scaling in one launch
-            scaled = residual.scaled
-            if scaled is not None and scaled.weight is self._final_rms[0]:
-                # the last layer left the rows times the norm's weight and their sums of squares
-                ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, x=scaled.rows,
-                               row_scale=ops.RowScale(scaled.ssq, spec.hidden_size, self._final_rms[1]),
-                               fragments=self._head_fragments)
-                return logits
-            ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, h_in=residual.h,
-                           deltas=residual.pending, norm_weight=self._final_rms[0], eps=self._final_rms[1],
+        scaled = residual.scaled
+        if (self._head_fragments is not None and scaled is not None and self._final_rms is not None
+                and scaled.weight is self._final_rms[0] and not residual.pending and self._every_row_wanted(step, wanted)):
+            # the last layer left the rows times the norm's weight and their sums of squares: projection, the
+            # norm's division and the scaling of the logits in one launch
+            ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, x=scaled.rows,
+                           row_scale=ops.RowScale(scaled.ssq, spec.hidden_size, self._final_rms[1]),
                            fragments=self._head_fragments)
             return logits
         normed = self.final_norm.forward(residual, rows=step.want_rows)
+        if self._head_fragments is not None and wanted <= HEAD_SKINNY_ROWS:
+            ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, x=normed,
+                           fragments=self._head_fragments)
+            return logits
         raw = ops.linear(normed, self.lm_head, None, keep_float32=True)      # the sums as they are, not rounded to bfloat16
         ops.scale_to_f32(raw, spec.logit_multiplier, logits)
         return logits
 
-    def _fused_head(self, step, wanted: int) -> bool:
-        return (step.max_query_len == 1 and wanted == step.num_tokens and wanted <= 16
-                and self.build.dtype == torch.bfloat16 and self.lm_head.dtype == torch.bfloat16
-                and self._final_rms is not None and len(step.lane_lengths) == wanted
-                and self.build.device.type == "cuda" and self.spec.hidden_size % 32 == 0
-                and ops.fused_gemm_supported(True, wanted, self.spec.hidden_size))
+    @staticmethod
+    def _every_row_wanted(step, wanted: int) -> bool:
+        """A step of single tokens that wants the logits of each: the wanted rows are the step's rows."""
+        return (step.max_query_len == 1 and wanted == step.num_tokens and wanted <= HEAD_SKINNY_ROWS
+                and len(step.lane_lengths) == wanted)

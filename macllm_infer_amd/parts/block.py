@@ -83,6 +83,13 @@ class ParallelPreNormBlock:
         parts = [self.mixer_norm, self.ffn_norm, self.ffn] + [mixer for _, mixer in self.mixers]
         return all(getattr(part, "graph_safe", False) for part in parts)
 
+    def tune(self, peers) -> None:
+        """Called once every layer of the model is built, with all of them: what a layer can only decide by
+        timing itself among the others."""
+        tune = getattr(self.fusion, "tune_chain", None)
+        if tune is not None:
+            tune([getattr(peer, "fusion", None) for peer in peers])
+
     @property
     def first_norm(self):
         """The norm this arrangement starts with: what a layer before it may prepare the stream for."""

@@ -53,12 +53,12 @@ MAX_NORM_WIDTH = 2048
 # The skinny kernel reads the step's rows once per 16 weight rows and keeps all of K in one workgroup; the
 # library tiles the rows and splits a long K, but its choice of tile swings from shape to shape (a 5120 x
 # 21504 weight at 8 rows: 115 us against 69; a 3072 x 12288 one: 20 against 25), so the clock decides, per
-# shape and per step size (TUNE_ROWS: up to 8, 16, 32, 48 and 64 rows, each measured at its upper edge).  Below
+# shape and per step size (TUNE_ROWS: up to 4, 8, 16, 32, 48 and 64 rows, each measured at its upper edge).  Below
 # the limit the skinny kernel wins everywhere.
 LIBRARY_MIN_WEIGHT = 2 << 20
 LIBRARY_MARGIN = 0.92          # the library has to be this much faster to be taken
 FORCE_LIBRARY: Optional[bool] = None      # tests: True or False instead of the clock
-TUNE_ROWS = (8, 16, 32, 48, 64)
+TUNE_ROWS = (4, 8, 16, 32, 48, 64)
 _library_wins: Dict[tuple, tuple] = {}
 # An output or down projection at 32 to 64 rows has a long K and few output features: 64 workgroups of the
 # skinny kernel, or whatever tile the library picks (10.7 us for 1,024 x 2,048 at 64 rows).  Split over K into
@@ -98,6 +98,19 @@ _padding_wins: Dict[tuple, tuple] = {}
 # costs no pass of its own and no prologue in every workgroup.  Taken for the step sizes at which a layer's four
 # projections all run through the skinny kernel unsplit, with one tile in the two that feed the stream.
 FORCE_DEFERRED_NORM: Optional[bool] = None  # tests: False = never
+# What is fastest for one projection alone need not be fastest for the layer: a down projection that wins by a
+# microsecond with two tiles or in slabs keeps the norms as kernels of their own.  So once a model's layers are
+# built, a chain of up to CHAIN_LAYERS layers of one shape (their projections and norms, without the mixers) is
+# timed per step size with the projections' own choices, with the norms left to them where those choices allow
+# it, and with all four through the skinny kernel and the norms left to them; the alternatives have to win by
+# CHAIN_MARGIN.  (8 layers of the 34B shape at 1 to 4 rows: 2.95 -> 2.03 ms a step; at 8 rows the projections'
+# own choices stay.)
+CHAIN_LAYERS = 8
+CHAIN_MARGIN = 0.97
+PLAN_FIELDS = ("library_in", "library_out", "library_gate_up", "library_down", "split_out", "split_down",
+               "tiles_in", "tiles_out", "tiles_gate_up", "tiles_down", "deferred")
+_chain_wins: Dict[tuple, tuple] = {}
+_chain_times: list = []     # (rows, microseconds a layer of each candidate, the one taken): what was measured, for whoever asks
 
 
 OVERLAP_MIN_TOKENS = 256       # prompt portions from this size on run their two mixers on two streams
@@ -284,6 +297,45 @@ def build_layer_fusion(block, build) -> Optional["LayerFusion"]:
     return LayerFusion.build(block, build)
 
 
+def _run_chain(chain, rows: int, bucket: int, h: torch.Tensor, mixed: torch.Tensor) -> None:
+    """The projections and norms of the layers of ``chain`` one after the other, as a decode step of ``rows``
+    rows runs them (the mixers left out: the same rows stand for what they would write)."""
+    residual = Residual(h)
+    for index, fusion in enumerate(chain):
+        residual.next_norm = chain[(index + 1) % len(chain)].mixer_scale
+        fusion._project_in(residual, rows, bucket, None)
+        fusion._after_the_mixers(residual, mixed, None, rows, bucket)
+
+
+def _measure_chain(chain, bucket: int) -> dict:
+    """The fastest plan (a value for each of PLAN_FIELDS) for steps of TUNE_ROWS[bucket] rows through the layers
+    of ``chain``, which are of one shape; the layers are left as they were."""
+    first = chain[0]
+    rows = TUNE_ROWS[bucket]
+    current = first._plan(bucket)
+    candidates = [dict(current, deferred=False)]
+    if first._may_defer(current):
+        candidates.append(dict(current, deferred=True))
+    skinny = dict(current, library_in=False, library_out=False, library_gate_up=False, library_down=False,
+                  split_out=0, split_down=0, tiles_out=1, tiles_down=1, deferred=True)
+    if (skinny not in candidates and first._may_defer(skinny)
+            and all(f is not None for fusion in chain for f in (fusion.f_in, fusion.f_out, fusion.f_gate_up, fusion.f_down))):
+        candidates.append(skinny)
+    device = first.w_in.device
+    h = torch.full((rows, first.hidden), 0.01, dtype=torch.float32, device=device)
+    mixed = torch.full((rows, first.mixed_width), 0.01, dtype=torch.bfloat16, device=device)
+    times = []
+    for plan in candidates:
+        for fusion in chain:
+            fusion._apply(bucket, plan)
+        times.append(_graph_microseconds(lambda: _run_chain(chain, rows, bucket, h, mixed)))
+    for fusion in chain:
+        fusion._apply(bucket, current)
+    best = min(range(len(candidates)), key=lambda index: times[index] / (1.0 if index == 0 else CHAIN_MARGIN))
+    _chain_times.append((rows, [round(time / len(chain), 2) for time in times], best))
+    return candidates[best]
+
+
 class LayerFusion:
     @staticmethod
     def build(block, build) -> Optional["LayerFusion"]:
@@ -399,15 +451,50 @@ class LayerFusion:
             self.f_gate_up = fragments(self.gate_up.weight, self.library_gate_up, ())
             self.f_down = fragments(self.down.weight, self.library_down, self.split_down)
         # step sizes at which the norms are left to the projections around them
-        self.deferred = tuple(self._defers(bucket) for bucket in range(BUCKETS))
+        self.deferred = _each(False)
+        self.deferred = tuple(self._may_defer(self._plan(bucket)) for bucket in range(BUCKETS))
 
-    def _defers(self, bucket: int) -> bool:
+    def _plan(self, bucket: int) -> dict:
+        """How steps of TUNE_ROWS[bucket] rows go through the layer's projections."""
+        if self.gate_up is None:
+            return {}
+        return {name: getattr(self, name)[bucket] for name in PLAN_FIELDS}
+
+    def _apply(self, bucket: int, plan: dict) -> None:
+        for name, value in plan.items():
+            values = list(getattr(self, name))
+            values[bucket] = value
+            setattr(self, name, tuple(values))
+
+    def _may_defer(self, plan: dict) -> bool:
+        """Whether the norms can be left to the projections under ``plan``: all four through the skinny kernel,
+        the two that feed the stream whole and with one tile."""
         if (FORCE_DEFERRED_NORM is False or self.gate_up is None or not self.decode_ok or self.ffn_scale is None
                 or self.hidden % 16 != 0):
             return False
-        return not (self.library_in[bucket] or self.library_out[bucket] or self.library_gate_up[bucket]
-                    or self.library_down[bucket] or self.split_out[bucket] or self.split_down[bucket]
-                    or self.tiles_out[bucket] != 1 or self.tiles_down[bucket] != 1)
+        return not (plan["library_in"] or plan["library_out"] or plan["library_gate_up"] or plan["library_down"]
+                    or plan["split_out"] or plan["split_down"] or plan["tiles_out"] != 1 or plan["tiles_down"] != 1)
+
+    def _shape_key(self) -> tuple:
+        return (tuple(self.w_in.shape), tuple(self.w_out.shape), self.inner, self.b_in is None, self.b_out is None,
+                self.gate_up is not None and self.gate_up.bias is None, self.down is not None and self.down.bias is None,
+                self.norm_rows, self.mixer_scale is None, self.ffn_scale is None)
+
+    def tune_chain(self, peers) -> None:
+        """Called once the model's layers are built, with the fusions of all of them: the plan of each step size
+        by the clock over a chain of layers of this one's shape (measured once per shape)."""
+        if (not self.measure or not self.decode_ok or self.gate_up is None or self.ffn_scale is None
+                or self.mixer_scale is None
+                or any(force is not None for force in (FORCE_DEFERRED_NORM, FORCE_LIBRARY, FORCE_SPLIT, FORCE_TILES))
+                or self.w_in.numel() + self.w_out.numel() + self.gate_up.weight.numel() + self.down.weight.numel()
+                < LIBRARY_MIN_WEIGHT):
+            return
+        key = self._shape_key()
+        if key not in _chain_wins:
+            chain = [peer for peer in peers if isinstance(peer, LayerFusion) and peer._shape_key() == key][:CHAIN_LAYERS]
+            _chain_wins[key] = tuple(_measure_chain(chain, bucket) for bucket in range(BUCKETS))
+        for bucket, plan in enumerate(_chain_wins[key]):
+            self._apply(bucket, plan)
 
     def path_choices(self) -> dict:
         """Which way each projection goes for steps of up to TUNE_ROWS rows, as short strings (S: the skinny
@@ -540,69 +627,15 @@ class LayerFusion:
         return tuple(choices), tuple(tiles)
 
     def forward_decode(self, residual: Residual, step, caches) -> None:
-        block = self.block
         M = step.num_tokens
         bucket = _bucket(M)
-        device = residual.h.device
-        bf16 = torch.bfloat16
         kernel = self.kernel if (self.kernel is not None and step.max_query_len == 1
                                  and self.kernel.supported(step, caches)) else None
-
-        def norm_prologue(norm, rms):
-            """The input of a projection: the norm in the kernel's prologue, or its own kernel before."""
-            if M > self.norm_rows or rms is None:
-                return dict(x=norm.forward(residual)), None          # adds the pending deltas in place
-            pending = residual.pending
-            if len(pending) > 2 or any(delta.dtype != bf16 for delta in pending):
-                return dict(x=norm.forward(residual)), None
-            h_out = torch.empty_like(residual.h) if pending else None
-            arguments = dict(h_in=residual.h, deltas=pending, h_out=h_out, norm_weight=rms[0], eps=rms[1])
-            return arguments, h_out
-
-        deferred = self.deferred[bucket]
-        scaled = residual.scaled
-
-        def to_the_stream(x, weight, bias, fragments, next_weight, attended=None):
-            """h += the projection, with the rows the product behind the norm of ``next_weight`` reads."""
-            rows = torch.empty((M, self.hidden), dtype=bf16, device=device)
-            ssq = ops.residual_workspace(M, self.hidden, device)
-            if attended is not None:
-                ops.fused_gemm_merge(weight, bias, None, x, attended, fragments,
-                                     residual=(residual.h, rows, next_weight, ssq))
-            else:
-                ops.fused_gemm_residual(weight, bias, x, residual.h, rows, next_weight, ssq, fragments)
-            residual.scaled = ScaledRows(rows, ssq, next_weight)
-
-        def behind_the_norm(rms):
-            return dict(x=scaled.rows, row_scale=ops.RowScale(scaled.ssq, self.hidden, rms[1]))
-
-        # 1
         conv = None
         if kernel is not None and kernel.conv is not None:
             conv = dict(kernel.conv, state=kernel.conv_state(caches), slot_ids=step.slot_ids)
-        if (scaled is not None and not self.library_in[bucket] and self.mixer_scale is not None
-                and scaled.weight is self.mixer_scale[0] and not residual.pending):
-            # the layer before left the stream prepared for this norm
-            u = torch.empty((M, self.in_ld), dtype=bf16, device=device)
-            ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width],
-                           epilogue=ops.EPI_CONV if conv is not None else ops.EPI_PLAIN, conv=conv,
-                           feature_tiles=self.tiles_in[bucket], fragments=self.f_in, **behind_the_norm(self.mixer_scale))
-        elif self.library_in[bucket]:
-            u = ops.linear(block.mixer_norm.forward(residual), self.w_in, self.b_in)
-            if conv is not None:
-                ops.conv_step(u, conv["lo"], conv["hi"] - conv["lo"], conv["weight"], conv["bias"], conv["state"],
-                              conv["slot_ids"])
-        else:
-            u = torch.empty((M, self.in_ld), dtype=bf16, device=device)
-            arguments, h_out = norm_prologue(block.mixer_norm, self.mixer_rms)
-            ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width],
-                           epilogue=ops.EPI_CONV if conv is not None else ops.EPI_PLAIN, conv=conv,
-                           feature_tiles=self.tiles_in[bucket] if "x" in arguments else 1, fragments=self.f_in,
-                           **arguments)
-            if h_out is not None:
-                residual.h, residual.pending = h_out, []
-        # 2
-        mixed = torch.empty((M, self.mixed_width), dtype=bf16, device=device)
+        u = self._project_in(residual, M, bucket, conv)
+        mixed = torch.empty((M, self.mixed_width), dtype=torch.bfloat16, device=u.device)
         attended = None
         if kernel is not None:
             later = (not self.library_out[bucket] and not self.split_out[bucket]
@@ -610,9 +643,68 @@ class LayerFusion:
             attended = kernel.run(u, step, caches, mixed, merge=not later)
         else:
             self._mix_each(u, step, caches, mixed)
-        # 3 (whatever ran in 1 has added what was pending to the stream)
-        if deferred and not residual.pending:
-            to_the_stream(mixed, self.w_out, self.b_out, self.f_out, self.ffn_scale[0], attended)
+        self._after_the_mixers(residual, mixed, attended, M, bucket)
+
+    def _norm_prologue(self, residual: Residual, M: int, norm, rms):
+        """The input of a projection: the norm in the kernel's prologue, or its own kernel before."""
+        if M > self.norm_rows or rms is None:
+            return dict(x=norm.forward(residual)), None          # adds the pending deltas in place
+        pending = residual.pending
+        if len(pending) > 2 or any(delta.dtype != torch.bfloat16 for delta in pending):
+            return dict(x=norm.forward(residual)), None
+        h_out = torch.empty_like(residual.h) if pending else None
+        arguments = dict(h_in=residual.h, deltas=pending, h_out=h_out, norm_weight=rms[0], eps=rms[1])
+        return arguments, h_out
+
+    def _add_to_the_stream(self, residual: Residual, x, weight, bias, fragments, next_weight, attended=None) -> None:
+        """h += the projection, with the rows that the product behind the norm of ``next_weight`` reads."""
+        M, device = x.shape[0], x.device
+        rows = torch.empty((M, self.hidden), dtype=torch.bfloat16, device=device)
+        ssq = ops.residual_workspace(M, self.hidden, device)
+        if attended is not None:
+            ops.fused_gemm_merge(weight, bias, None, x, attended, fragments, residual=(residual.h, rows, next_weight, ssq))
+        else:
+            ops.fused_gemm_residual(weight, bias, x, residual.h, rows, next_weight, ssq, fragments)
+        residual.scaled = ScaledRows(rows, ssq, next_weight)
+
+    def _behind_the_norm(self, scaled: ScaledRows, rms) -> dict:
+        return dict(x=scaled.rows, row_scale=ops.RowScale(scaled.ssq, self.hidden, rms[1]))
+
+    def _project_in(self, residual: Residual, M: int, bucket: int, conv: Optional[dict]) -> torch.Tensor:
+        """1: the mixers' input projection of the normed rows (with the conv step of ``conv``'s columns)."""
+        block = self.block
+        device = residual.h.device
+        epilogue = ops.EPI_CONV if conv is not None else ops.EPI_PLAIN
+        scaled = residual.scaled
+        if (scaled is not None and not self.library_in[bucket] and self.mixer_scale is not None
+                and scaled.weight is self.mixer_scale[0] and not residual.pending):
+            # the layer before left the stream prepared for this norm
+            u = torch.empty((M, self.in_ld), dtype=torch.bfloat16, device=device)
+            ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=epilogue, conv=conv,
+                           feature_tiles=self.tiles_in[bucket], fragments=self.f_in,
+                           **self._behind_the_norm(scaled, self.mixer_scale))
+        elif self.library_in[bucket]:
+            u = ops.linear(block.mixer_norm.forward(residual), self.w_in, self.b_in)
+            if conv is not None:
+                ops.conv_step(u, conv["lo"], conv["hi"] - conv["lo"], conv["weight"], conv["bias"], conv["state"],
+                              conv["slot_ids"])
+        else:
+            u = torch.empty((M, self.in_ld), dtype=torch.bfloat16, device=device)
+            arguments, h_out = self._norm_prologue(residual, M, block.mixer_norm, self.mixer_rms)
+            ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=epilogue, conv=conv,
+                           feature_tiles=self.tiles_in[bucket] if "x" in arguments else 1, fragments=self.f_in,
+                           **arguments)
+            if h_out is not None:
+                residual.h, residual.pending = h_out, []
+        return u
+
+    def _after_the_mixers(self, residual: Residual, mixed: torch.Tensor, attended, M: int, bucket: int) -> None:
+        """3 to 5: the output projection, the norm, the feed-forward.  (Whatever ran in 1 has added what was
+        pending to the stream.)"""
+        block = self.block
+        # 3
+        if self.deferred[bucket] and not residual.pending:
+            self._add_to_the_stream(residual, mixed, self.w_out, self.b_out, self.f_out, self.ffn_scale[0], attended)
         else:
             residual.pending = self._to_the_stream(mixed, self.w_out, self.b_out, self.library_out[bucket],
                                                    self.split_out[bucket], self.tiles_out[bucket], self.f_out, attended)
@@ -620,18 +712,18 @@ class LayerFusion:
         if self.gate_up is None:
             residual.pending = [block.ffn.forward(block.ffn_norm.forward(residual))]
             return
-        activated = torch.empty((M, self.inner), dtype=bf16, device=device)
+        activated = torch.empty((M, self.inner), dtype=torch.bfloat16, device=mixed.device)
         scaled = residual.scaled
         if scaled is not None and (self.ffn_scale is None or scaled.weight is not self.ffn_scale[0]):
             scaled = None
         if scaled is not None:
             ops.fused_gemm(self.gate_up.weight, self.gate_up.bias, activated, epilogue=ops.EPI_SWIGLU,
                            feature_tiles=self.tiles_gate_up[bucket], fragments=self.f_gate_up,
-                           **behind_the_norm(self.ffn_scale))
+                           **self._behind_the_norm(scaled, self.ffn_scale))
         elif self.library_gate_up[bucket]:
             ops.swiglu(ops.linear(block.ffn_norm.forward(residual), self.gate_up.weight, self.gate_up.bias), activated, 8)
         else:
-            arguments, h_out = norm_prologue(block.ffn_norm, self.ffn_rms)
+            arguments, h_out = self._norm_prologue(residual, M, block.ffn_norm, self.ffn_rms)
             ops.fused_gemm(self.gate_up.weight, self.gate_up.bias, activated, epilogue=ops.EPI_SWIGLU,
                            feature_tiles=self.tiles_gate_up[bucket] if "x" in arguments else 1,
                            fragments=self.f_gate_up, **arguments)
@@ -639,7 +731,8 @@ class LayerFusion:
                 residual.h, residual.pending = h_out, []
         # 5
         if scaled is not None and residual.next_norm is not None:
-            to_the_stream(activated, self.down.weight, self.down.bias, self.f_down, residual.next_norm[0])
+            self._add_to_the_stream(residual, activated, self.down.weight, self.down.bias, self.f_down,
+                                    residual.next_norm[0])
             return
         residual.pending = self._to_the_stream(activated, self.down.weight, self.down.bias, self.library_down[bucket],
                                                self.split_down[bucket], self.tiles_down[bucket], self.f_down)

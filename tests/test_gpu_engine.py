@@ -389,11 +389,11 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
                     max_active_sequences=requests)
     if library == "split":
         fusion = engine.model.blocks[0].fusion
-        assert fusion.split_out == (0, 0, 3, 3, 3) and fusion.split_down == (0, 0, 3, 3, 3)
+        assert fusion.split_out == (0, 0, 0, 3, 3, 3) and fusion.split_down == (0, 0, 0, 3, 3, 3)
     if library == "tiles":
         fusion = engine.model.blocks[0].fusion
-        assert fusion.tiles_in == fusion.tiles_gate_up == fusion.tiles_out == fusion.tiles_down == (1, 1, 4, 4, 4)
-        assert fusion.library_in == fusion.library_down == (False,) * 5
+        assert fusion.tiles_in == fusion.tiles_gate_up == fusion.tiles_out == fusion.tiles_down == (1, 1, 1, 4, 4, 4)
+        assert fusion.library_in == fusion.library_down == (False,) * 6
     prompts = {index: tokens_for(cfg["vocab_size"], 3 + index % 7 + 6, 500 + index) for index in range(requests)}
     for index, tokens in prompts.items():
         engine.add_request(index)
@@ -463,11 +463,12 @@ def test_lanes_fed_from_the_device_say_what_lanes_fed_by_the_host_say(tmp_path, 
 def test_fixed_paths_take_no_measurement(tmp_path, monkeypatch):
     """``measured_paths=False``: even where every weight would be timed (the limit lowered to 0), the layers take
     the fixed rules, the same in every process, and say so; the engine that measures reports a choice for each
-    of the five step sizes.  Both decode 24 lanes like the plain model."""
+    of the six step sizes.  Both decode 24 lanes like the plain model."""
     import gates
     from macllm_infer_amd import Engine, Lane
     from macllm_infer_amd.parts import fused
     monkeypatch.setattr(fused, "LIBRARY_MIN_WEIGHT", 0)
+    monkeypatch.setattr(fused, "_chain_wins", {})
     folder = tiny_configs.make_model_dir("C", tmp_path, torch.bfloat16)
     cfg, tensors = plain_impl.load_model_dir(folder)
     prompts = {index: tokens_for(cfg["vocab_size"], 5 + index % 4, 900 + index) for index in range(24)}
@@ -477,11 +478,12 @@ def test_fixed_paths_take_no_measurement(tmp_path, monkeypatch):
         choices = engine.path_choices()
         assert set(choices) == {"in", "out", "gate_up", "down", "tiles_in", "tiles_out", "tiles_gate_up", "tiles_down",
                                 "padded_in", "norms"}
-        assert all(len(value.split("/")) == 5 for value in choices.values())
+        assert all(len(value.split("/")) == (5 if name == "padded_in" else 6) for name, value in choices.items())
+        assert bool(fused._chain_wins) == measured          # the layers' chain was timed too, once for the shape
         if not measured:
-            assert choices["in"] == choices["out"] == choices["gate_up"] == choices["down"] == "S/S/S/S/S"
-            assert choices["norms"] == "D/D/D/D/D"
-            assert choices["tiles_in"] == choices["tiles_down"] == "1/1/1/1/1" and choices["padded_in"] == "-/-/-/-/-"
+            assert choices["in"] == choices["out"] == choices["gate_up"] == choices["down"] == "S/S/S/S/S/S"
+            assert choices["norms"] == "D/D/D/D/D/D"
+            assert choices["tiles_in"] == choices["tiles_down"] == "1/1/1/1/1/1" and choices["padded_in"] == "-/-/-/-/-"
         for index in prompts:
             engine.add_request(index)
         engine.step([Lane(index, tokens[:-1], []) for index, tokens in prompts.items()])
@@ -508,7 +510,7 @@ def test_norms_left_to_the_projections_around_them(tmp_path, monkeypatch):
         monkeypatch.setattr(fused, "FORCE_DEFERRED_NORM", deferred)
         engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * 26,
                         max_active_sequences=26)
-        assert engine.path_choices()["norms"] == ("-/-/-/-/-" if deferred is False else "D/D/D/D/D")
+        assert engine.path_choices()["norms"] == ("-/-/-/-/-/-" if deferred is False else "D/D/D/D/D/D")
         for index in list(prompts) + list(late):
             engine.add_request(index)
         engine.step([Lane(index, tokens[:-1], []) for index, tokens in prompts.items()])
