@@ -314,11 +314,132 @@ sample_kernel(float* __restrict__ logits, int V, int padded, const float* __rest
 // needed.  With top-k (k <= SAMPLE_KMAX) the k smallest keys are found by a radix select over
 // the 64-bit keys (eight passes of a 256-bin histogram), gathered and sorted in LDS; without
 // top-k the SAMPLE_KMAX best candidates are taken the same way and the normalizer is summed over
-// the whole row; without top-k and top-p nothing is sorted at all.  The results are those of
-// sample_kernel up to the rounding of float32 sums.  A row this kernel does not cover (k above
-// SAMPLE_KMAX, or a nucleus that does not close within the candidates) is left with done[row] = 0
-// for sample_kernel, which skips the rows that are done.  The logits are not written.
+// the whole row, and a nucleus that does not close within them (flat logits) gets its last token from a
+// second radix select that counts mass instead of tokens; without top-k and top-p nothing is sorted at
+// all.  The results are those of sample_kernel up to the rounding of float32 sums.  A row this kernel
+// does not cover (k above SAMPLE_KMAX) is left with done[row] = 0 for sample_kernel, which skips the
+// rows that are done.  The logits of a row that is drawn here are divided by its temperature in place.
 #define SAMPLE_KMAX 1024
+#define SAMPLE_LIST 2048             // keys that share their two upper bytes with the one looked for, listed in LDS
+#define SAMPLE_ROW_PASSES_FROM 6     // the passes over bytes 7 and 6 read the row; those below read the list
+
+// A row is read by one workgroup, which waits a microsecond for whatever it asks of memory: ROW_LOADS loads of a
+// thread are asked for before the first is used (a row of 261,120 logits: 16 rounds instead of 255).
+#define ROW_LOADS 16
+
+// f(key) for every token of the row.  The row holds logits divided by the temperature; the first pass over it
+// (SCALE) does the division and leaves the quotients in place: a division is a dozen instructions, and one
+// workgroup's passes over a row are bound by its instructions.
+template <bool SCALE, typename F>
+__device__ __forceinline__ void for_each_key(float* __restrict__ values, int V, float temp, F f) {
+  for (int base = threadIdx.x; base < V; base += ROW_LOADS * blockDim.x) {
+    float x[ROW_LOADS];
+#pragma unroll
+    for (int j = 0; j < ROW_LOADS; ++j) x[j] = values[min(base + j * (int)blockDim.x, V - 1)];
+#pragma unroll
+    for (int j = 0; j < ROW_LOADS; ++j) {
+      const int v = base + j * (int)blockDim.x;
+      if (v < V) {
+        if (SCALE) {
+          x[j] = x[j] / temp;
+          values[v] = x[j];
+        }
+        f(rank_key(x[j], v));
+      }
+    }
+  }
+}
+
+// The sum of a value a thread over the block, added in a fixed order (lanes by halves, then the waves in turn).
+__device__ float block_total(float value, float* scratch /* one float a wave */) {
+#pragma unroll
+  for (int offset = WAVE / 2; offset > 0; offset >>= 1) value += __shfl_xor(value, offset, WAVE);
+  __syncthreads();
+  if ((threadIdx.x & (WAVE - 1)) == 0) scratch[threadIdx.x / WAVE] = value;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < (int)blockDim.x / WAVE; ++w) total += scratch[w];
+  return total;
+}
+
+// The sum of f(value, v) over the row, consecutive lanes on consecutive tokens.
+template <typename F>
+__device__ float row_sum(const float* __restrict__ values, int V, float* scratch, F f) {
+  float local = 0.f;
+  for (int base = threadIdx.x; base < V; base += ROW_LOADS * blockDim.x) {
+    float x[ROW_LOADS];
+#pragma unroll
+    for (int j = 0; j < ROW_LOADS; ++j) x[j] = values[min(base + j * (int)blockDim.x, V - 1)];
+#pragma unroll
+    for (int j = 0; j < ROW_LOADS; ++j) {
+      const int v = base + j * (int)blockDim.x;
+      if (v < V) local += f(x[j], v);
+    }
+  }
+  return block_total(local, scratch);
+}
+
+// The first token, in index order, at which the running sum of mass(value, v) exceeds u times the sum
+// over the row (V if there is none: rounding, when u is close to 1).  Every wave owns a run of consecutive
+// tokens and sums it with consecutive lanes on consecutive tokens; the wave whose run holds the target then
+// walks it 64 tokens at a time with a running sum across its lanes.
+template <typename F>
+__device__ int walk_in_index_order(const float* __restrict__ values, int V, float u, float* scratch, int* found,
+                                   F mass) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wave = threadIdx.x / WAVE;
+  const int waves = blockDim.x / WAVE;
+  const int run = ((V + waves - 1) / waves + WAVE - 1) / WAVE * WAVE;
+  const int lo = min(V, wave * run);
+  const int hi = min(V, lo + run);
+  float local = 0.f;
+  for (int base = lo + lane; base < hi; base += ROW_LOADS * WAVE) {
+    float x[ROW_LOADS];
+#pragma unroll
+    for (int j = 0; j < ROW_LOADS; ++j) x[j] = values[min(base + j * WAVE, V - 1)];
+#pragma unroll
+    for (int j = 0; j < ROW_LOADS; ++j) {
+      const int v = base + j * WAVE;
+      if (v < hi) local += mass(x[j], v);
+    }
+  }
+#pragma unroll
+  for (int offset = WAVE / 2; offset > 0; offset >>= 1) local += __shfl_xor(local, offset, WAVE);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = local;
+  if (threadIdx.x == 0) *found = V;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < waves; ++w) total += scratch[w];
+  const float target = u * total;
+  float before = 0.f;
+  int holder = -1;
+  for (int w = 0; w < waves; ++w) {
+    if (holder < 0 && target < before + scratch[w]) holder = w;
+    if (holder < 0) before += scratch[w];
+  }
+  if (wave == holder) {
+    float running = before;
+    for (int base = lo; base < hi; base += WAVE) {
+      const int v = base + lane;
+      const float p = v < hi ? mass(values[min(v, V - 1)], v) : 0.f;
+      float inclusive = p;
+#pragma unroll
+      for (int offset = 1; offset < WAVE; offset <<= 1) {
+        const float other = __shfl_up(inclusive, offset, WAVE);
+        if (lane >= offset) inclusive += other;
+      }
+      const unsigned long long crossed = __ballot(p > 0.f && target < running + inclusive);
+      if (crossed != 0ull) {
+        if (lane == 0) *found = base + __ffsll((long long)crossed) - 1;
+        break;
+      }
+      running += __shfl(inclusive, WAVE - 1, WAVE);
+    }
+  }
+  __syncthreads();
+  return *found;
+}
 
 __device__ void lds_bitonic_sort(unsigned long long* keys, int padded) {
   for (int size = 2; size <= padded; size <<= 1) {
@@ -341,7 +462,7 @@ __device__ void lds_bitonic_sort(unsigned long long* keys, int padded) {
 }
 
 __global__ void __launch_bounds__(SAMPLE_THREADS)
-sample_select_kernel(const float* __restrict__ logits, int V, const float* __restrict__ temperature,
+sample_select_kernel(float* __restrict__ logits, int V, const float* __restrict__ temperature,
                      const int* __restrict__ top_k, const float* __restrict__ top_p,
                      const unsigned long long* __restrict__ seeds, const int* __restrict__ draw_index,
                      int* __restrict__ out, int* __restrict__ done) {
@@ -350,11 +471,14 @@ sample_select_kernel(const float* __restrict__ logits, int V, const float* __res
   __shared__ unsigned long long candidates[SAMPLE_KMAX];
   __shared__ unsigned long long by_index[SAMPLE_KMAX];
   __shared__ unsigned int histogram[256];
-  __shared__ unsigned long long chosen_prefix;
+  __shared__ unsigned long long mass_histogram[256];
+  __shared__ unsigned long long chosen_prefix, remaining_mass;
+  __shared__ unsigned long long list[SAMPLE_LIST];
+  __shared__ int listed;
   __shared__ int remaining, found, gathered, bin_taken_whole;
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
-  const float* values = logits + (long)row * V;
+  float* values = logits + (long)row * V;          // divided by the temperature in the first pass over them
   const float temp = temperature[row];
   if (tid == 0) done[row] = 0;
 
@@ -377,43 +501,18 @@ sample_select_kernel(const float* __restrict__ logits, int V, const float* __res
   const bool use_top_p = p_limit >= 0.f && p_limit < 1.f;
   if (use_top_k && k > SAMPLE_KMAX) return;                    // sample_kernel's
   const float u = draw_uniform(seeds[row], (unsigned long long)draw_index[row]);
-  const int vchunk = (V + blockDim.x - 1) / blockDim.x;
-  const int vbegin = min(V, tid * vchunk);
-  const int vend = min(V, vbegin + vchunk);
 
   if (!use_top_k && !use_top_p) {
     // every token is kept: maximum, normalizer, and the walk in index order
     unsigned long long best = ~0ull;
-    for (int v = tid; v < V; v += blockDim.x) {
-      const unsigned long long key = rank_key(values[v] / temp, v);
-      best = key < best ? key : best;
-    }
+    for_each_key<true>(values, V, temp, [&](unsigned long long key) { best = key < best ? key : best; });
     best = block_min_key(best, key_scratch);
     const float maximum = from_orderable(~(unsigned int)(best >> 32));
-    float local = 0.f;
-    for (int v = vbegin; v < vend; ++v) local += expf(values[v] / temp - maximum);
-    float normalizer;
-    block_exclusive_scan(local, scan_scratch, &normalizer);
-    float mass = 0.f;
-    for (int v = vbegin; v < vend; ++v) mass += expf(values[v] / temp - maximum) / normalizer;
-    float total;
-    const float start = block_exclusive_scan(mass, scan_scratch, &total);
-    const float target = u * total;
-    if (tid == 0) found = V;
-    __syncthreads();
-    float cumulative = start;
-    for (int v = vbegin; v < vend; ++v) {
-      const float p = expf(values[v] / temp - maximum) / normalizer;
-      if (p <= 0.f) continue;
-      cumulative += p;
-      if (target < cumulative) {
-        atomicMin(&found, v);
-        break;
-      }
-    }
-    __syncthreads();
+    const float normalizer = row_sum(values, V, scan_scratch, [&](float scaled, int) { return expf(scaled - maximum); });
+    const int token = walk_in_index_order(values, V, u, scan_scratch, &found,
+                                          [&](float scaled, int) { return expf(scaled - maximum) / normalizer; });
     if (tid == 0) {
-      out[row] = found < V ? found : (int)(best & 0xffffffffu);
+      out[row] = token < V ? token : (int)(best & 0xffffffffu);
       done[row] = 1;
     }
     return;
@@ -425,14 +524,32 @@ sample_select_kernel(const float* __restrict__ logits, int V, const float* __res
     chosen_prefix = 0ull;
     remaining = K;
   }
+  if (tid == 0) listed = 0;
   for (int pass = 7; pass >= 0; --pass) {
     if (tid < 256) histogram[tid] = 0u;
     __syncthreads();
     const unsigned long long prefix = chosen_prefix;
     const unsigned long long above = pass == 7 ? 0ull : (~0ull << (8 * (pass + 1)));
-    for (int v = tid; v < V; v += blockDim.x) {
-      const unsigned long long key = rank_key(values[v] / temp, v);
+    if (pass == SAMPLE_ROW_PASSES_FROM - 1) {
+      // two bytes of the keys are fixed: the keys that still match are few; they are listed, and the bytes below
+      // are found among them instead of in passes over the row (when they fit the list)
+      for_each_key<false>(values, V, temp, [&](unsigned long long key) {
+        if ((key & above) == prefix) {
+          const int slot = atomicAdd(&listed, 1);
+          if (slot < SAMPLE_LIST) list[slot] = key;
+        }
+      });
+      __syncthreads();
+    }
+    auto count = [&](unsigned long long key) {
       if ((key & above) == prefix) atomicAdd(&histogram[(unsigned int)(key >> (8 * pass)) & 255u], 1u);
+    };
+    if (pass < SAMPLE_ROW_PASSES_FROM && listed <= SAMPLE_LIST) {
+      for (int i = tid; i < listed; i += blockDim.x) count(list[i]);
+    } else if (pass == 7) {
+      for_each_key<true>(values, V, temp, count);
+    } else {
+      for_each_key<false>(values, V, temp, count);
     }
     __syncthreads();
     // the bin in which the running count reaches what is still wanted: the first wave scans the
@@ -482,13 +599,12 @@ sample_select_kernel(const float* __restrict__ logits, int V, const float* __res
   for (int i = tid; i < padded; i += blockDim.x) candidates[i] = ~0ull;
   if (tid == 0) gathered = 0;
   __syncthreads();
-  for (int v = tid; v < V; v += blockDim.x) {
-    const unsigned long long key = rank_key(values[v] / temp, v);
+  for_each_key<false>(values, V, temp, [&](unsigned long long key) {
     if (key <= kth) {
       const int slot = atomicAdd(&gathered, 1);
       if (slot < SAMPLE_KMAX) candidates[slot] = key;
     }
-  }
+  });
   lds_bitonic_sort(candidates, padded);                        // descending values, ties by ascending index
   const float maximum = from_orderable(~(unsigned int)(candidates[0] >> 32));
 
@@ -505,9 +621,7 @@ sample_select_kernel(const float* __restrict__ logits, int V, const float* __res
   if (use_top_k) {
     normalizer = candidate_mass;
   } else {
-    float all = 0.f;
-    for (int v = vbegin; v < vend; ++v) all += expf(values[v] / temp - maximum);
-    block_exclusive_scan(all, scan_scratch, &normalizer);
+    normalizer = row_sum(values, V, scan_scratch, [&](float scaled, int) { return expf(scaled - maximum); });
   }
 
   // ---- top-p: the shortest prefix in sorted order whose mass reaches top_p
@@ -527,7 +641,88 @@ sample_select_kernel(const float* __restrict__ logits, int V, const float* __res
   __syncthreads();
   const int closed_at = found;
   __syncthreads();
-  if (closed_at == OPEN && !use_top_k && K < V) return;        // the nucleus is wider than the candidates: sample_kernel's
+  if (closed_at == OPEN && !use_top_k && K < V) {
+    // ---- the nucleus is wider than the candidates (flat logits): its last token by a radix select over the
+    // keys again, this time counting mass instead of tokens.  Masses are fixed-point (probability * 2^40,
+    // 64-bit sums: exact, so every pass sees the same totals whatever the order of the additions): the bin in
+    // which the running mass reaches what is still wanted is taken, byte by byte, down to one key.
+    const float fixed_one = 1099511627776.f;
+    if (tid == 0) {
+      chosen_prefix = 0ull;
+      remaining_mass = (unsigned long long)(p_limit * fixed_one);
+    }
+    for (int pass = 7; pass >= 0; --pass) {
+      if (tid < 256) mass_histogram[tid] = 0ull;
+      __syncthreads();
+      const unsigned long long prefix = chosen_prefix;
+      const unsigned long long above = pass == 7 ? 0ull : (~0ull << (8 * (pass + 1)));
+      auto add_mass = [&](unsigned long long key) {
+        if ((key & above) == prefix)
+          atomicAdd(&mass_histogram[(unsigned int)(key >> (8 * pass)) & 255u],
+                    (unsigned long long)(expf(from_orderable(~(unsigned int)(key >> 32)) - maximum) / normalizer * fixed_one));
+      };
+      if (pass == SAMPLE_ROW_PASSES_FROM - 1) {
+        if (tid == 0) listed = 0;
+        __syncthreads();
+        for_each_key<false>(values, V, temp, [&](unsigned long long key) {
+          if ((key & above) == prefix) {
+            const int slot = atomicAdd(&listed, 1);
+            if (slot < SAMPLE_LIST) list[slot] = key;
+          }
+        });
+        __syncthreads();
+      }
+      if (pass < SAMPLE_ROW_PASSES_FROM && listed <= SAMPLE_LIST) {
+        for (int i = tid; i < listed; i += blockDim.x) add_mass(list[i]);
+      } else {
+        for_each_key<false>(values, V, temp, add_mass);
+      }
+      __syncthreads();
+      if (tid < WAVE) {
+        unsigned long long mine[4], sum = 0ull;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          mine[j] = mass_histogram[4 * tid + j];
+          sum += mine[j];
+        }
+        unsigned long long inclusive = sum;
+#pragma unroll
+        for (int offset = 1; offset < WAVE; offset <<= 1) {
+          const unsigned long long other = __shfl_up(inclusive, offset, WAVE);
+          if (tid >= offset) inclusive += other;
+        }
+        const unsigned long long all = __shfl(inclusive, WAVE - 1, WAVE);
+        // what is wanted is at most what there is (the top pass; below it the bin taken holds it by construction)
+        const unsigned long long wanted = remaining_mass < all ? remaining_mass : all;
+        unsigned long long before = inclusive - sum;
+        if (sum > 0ull && before < wanted && inclusive >= wanted) {      // exactly one lane (none if wanted is 0)
+          int bin = 4 * tid;
+#pragma unroll
+          for (int j = 0; j < 3; ++j) {
+            if (before + mine[j] < wanted) {
+              before += mine[j];
+              ++bin;
+            } else {
+              break;
+            }
+          }
+          remaining_mass = wanted - before;
+          chosen_prefix = prefix | ((unsigned long long)bin << (8 * pass));
+        }
+      }
+      __syncthreads();
+    }
+    const unsigned long long last_kept = remaining_mass > 0ull ? chosen_prefix : candidates[0];
+    // ---- walk the kept tokens in index order
+    const int token = walk_in_index_order(values, V, u, scan_scratch, &found, [&](float scaled, int v) {
+      return rank_key(scaled, v) <= last_kept ? expf(scaled - maximum) / normalizer : 0.f;
+    });
+    if (tid == 0) {
+      out[row] = token < V ? token : (int)(candidates[0] & 0xffffffffu);
+      done[row] = 1;
+    }
+    return;
+  }
   const int nucleus = min(closed_at, K);
 
   // ---- walk the nucleus in index order

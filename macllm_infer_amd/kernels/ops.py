@@ -1022,9 +1022,8 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
 
 def sample(logits, temperature, top_k, top_p, seeds, draw_index, keys, out, done=None) -> None:
     """One token per row; may overwrite ``logits``.  ``keys`` int64 [B, padded] work area.  With
-    ``done`` (int32 [B] work area) the rows that need no full sort (top-k up to 1 024, or a
-    nucleus within the 1 024 best, or neither top-k nor top-p) are drawn by selection; without it
-    every row is sorted."""
+    ``done`` (int32 [B] work area) the rows that need no full sort (all but a top-k above 1 024) are
+    drawn by selection; without it every row is sorted."""
     B, V = logits.shape
     _need(logits.dtype == torch.float32 and logits.is_contiguous() and logits.is_cuda, "sample: bad logits")
     padded = keys.shape[1]

@@ -598,8 +598,8 @@ def test_argmax_of_rows_at_every_alignment(ops, V):
 def test_sampling_matches_the_plain_sampler(ops, V, select):
     """Every row is sorted whole, or (``select``) rows are drawn by selection where that covers
     them: top-k 1, 7, 20, 40 and 1 024; a nucleus that closes within the 1 024 best candidates
-    (rows with peaked logits) and one that does not (flat logits: handed on to the full sort);
-    top-k above 1 024 (handed on); neither top-k nor top-p; a greedy row."""
+    (rows with peaked logits) and one that does not (flat logits: its last token by a select over mass);
+    top-k above 1 024 (handed on to the full sort); neither top-k nor top-p; a greedy row."""
     import plain_impl
     settings = [(0.8, 0, 1.0), (1.0, 7, 1.0), (0.9, 0, 0.7), (1.2, 40, 0.85), (0.0, 0, 1.0), (0.7, 20, 0.8),
                 (1.0, V + 5, 0.999), (0.5, 1, 0.1), (1.0, 1024, 0.95), (1.1, 1500, 0.9), (0.6, 0, 0.9), (1.0, 0, 0.5)]
@@ -625,6 +625,63 @@ def test_sampling_matches_the_plain_sampler(ops, V, select):
                                         top_p=settings[row][2], seed=seeds[row], draw_index=draws[row] + repeat)
                 for row in range(B)]
         assert out.cpu().tolist() == want
+
+
+@pytest.mark.parametrize("V", [5000, 40001])
+def test_a_nucleus_wider_than_the_candidates(ops, V):
+    """Top-p without top-k over flat rows, where the nucleus is thousands of tokens (more than the 1 024
+    candidates that are sorted): nearly equal logits, logits that are all equal (the nucleus is cut among
+    ties, by index; more ties than the list of the select holds), two values half and half, an ordinary
+    row at a high temperature; several draws each.
+
+    Over thousands of nearly equal masses the order in which float32 sums are taken moves a running sum by
+    more than one token's mass (the plain sampler adds one by one, a GPU adds in blocks), so tokens are not
+    compared one to one here: the drawn token must be a valid draw of the rule computed in float64: it lies in
+    the nucleus (the shortest descending prefix, ties by index, whose mass reaches top_p; one token of slack at
+    its end), and u times the kept mass falls into the token's own interval of the running sum in index order,
+    give or take V float32 roundings of the total."""
+    import numpy as np
+    import plain_impl
+    settings = [(1.0, 0.5), (1.0, 0.9), (0.7, 0.999), (1.0, 0.25), (1.3, 0.6), (5.0, 0.95), (1.0, 0.0)]
+    B = len(settings)
+    logits = rand(B, V, seed=83, scale=0.02)
+    logits[1] = 0.25                                             # all equal
+    logits[3, :V // 2] = 1.0                                     # two values
+    logits[3, V // 2:] = 0.0
+    logits[5] = rand(V, seed=84, scale=3.0)
+    logits[6] = rand(V, seed=85, scale=3.0)                      # top_p 0: the best token alone
+    padded = 1
+    while padded < V:
+        padded <<= 1
+    drawn = set()
+    for repeat in range(4):
+        work = logits.clone().to(DEV)
+        out = torch.empty(B, dtype=torch.int32, device=DEV)
+        ops.sample(work, torch.tensor([s[0] for s in settings]).to(DEV), i32([0] * B).to(DEV),
+                   torch.tensor([s[1] for s in settings]).to(DEV), torch.tensor([31 + row for row in range(B)], dtype=torch.int64).to(DEV),
+                   i32([repeat * 7 + row for row in range(B)]).to(DEV),
+                   torch.empty(B, padded, dtype=torch.int64, device=DEV), out,
+                   torch.full((B,), 7, dtype=torch.int32, device=DEV))
+        tokens = out.cpu().tolist()
+        for row, (temperature, top_p) in enumerate(settings):
+            scaled = (logits[row].numpy() / np.float32(temperature)).astype(np.float64)
+            mass = np.exp(scaled - scaled.max())
+            mass /= mass.sum()
+            order = sorted(range(V), key=lambda index: (-mass[index], index))
+            running = np.cumsum(mass[order])
+            keep = int(np.searchsorted(running, top_p, side="left")) + 1          # the first prefix that reaches top_p
+            token = tokens[row]
+            place = order.index(token)
+            assert place < min(V, keep + 1), (row, repeat, token, place, keep)
+            kept = np.zeros(V)
+            kept[order[:keep]] = mass[order[:keep]]
+            upto = np.cumsum(kept)
+            target = plain_impl.draw_uniform(31 + row, repeat * 7 + row) * upto[-1]
+            slack = V * 2.0 ** -23 * upto[-1] + mass[order[min(keep, V - 1)]]
+            assert upto[token] - kept[token] - slack <= target <= upto[token] + slack, (row, repeat, token)
+            drawn.add((row, token))
+    assert tokens[6] == int(torch.argmax(logits[6]))
+    assert len(drawn) > 3 * B                                    # the draws differ from one another
 
 
 def test_penalties_match_the_plain_rule(ops):
