@@ -133,6 +133,7 @@ def _bucket(rows: int) -> int:
 
 
 BUCKETS = len(TUNE_ROWS)
+BEYOND = BUCKETS       # the place, behind the measured step sizes, of the plan for steps of more than MAX_ROWS single tokens
 
 
 def _each(value) -> tuple:
@@ -453,6 +454,13 @@ class LayerFusion:
         # step sizes at which the norms are left to the projections around them
         self.deferred = _each(False)
         self.deferred = tuple(self._may_defer(self._plan(bucket)) for bucket in range(BUCKETS))
+        # and behind the measured step sizes the plan of steps of more than MAX_ROWS single tokens: every projection
+        # through the library, with the mixers' decode kernel between them
+        beyond = dict(library_in=True, library_out=True, library_gate_up=True, library_down=True, split_out=0,
+                      split_down=0, tiles_in=1, tiles_out=1, tiles_gate_up=1, tiles_down=1, deferred=False)
+        for name, value in beyond.items():
+            if hasattr(self, name):
+                setattr(self, name, getattr(self, name) + (value,))
 
     def _plan(self, bucket: int) -> dict:
         """How steps of TUNE_ROWS[bucket] rows go through the layer's projections."""
@@ -504,25 +512,32 @@ class LayerFusion:
             return {}
 
         def way(library, split=None):
+            library = library[:BUCKETS]
             split = split or (0,) * len(library)
             return "/".join(str(slabs) if slabs else ("L" if lib else "S") for lib, slabs in zip(library, split))
 
         out = {"in": way(self.library_in), "out": way(self.library_out, self.split_out),
-               "tiles_in": "/".join(map(str, self.tiles_in)), "tiles_out": "/".join(map(str, self.tiles_out)),
+               "tiles_in": "/".join(map(str, self.tiles_in[:BUCKETS])), "tiles_out": "/".join(map(str, self.tiles_out[:BUCKETS])),
                "padded_in": "/".join("P" if pays else "-" for pays in self.padding_pays)}
         if self.gate_up is not None:
             out.update({"gate_up": way(self.library_gate_up), "down": way(self.library_down, self.split_down),
-                        "tiles_gate_up": "/".join(map(str, self.tiles_gate_up)),
-                        "tiles_down": "/".join(map(str, self.tiles_down)),
-                        "norms": "/".join("D" if deferred else "-" for deferred in self.deferred)})
+                        "tiles_gate_up": "/".join(map(str, self.tiles_gate_up[:BUCKETS])),
+                        "tiles_down": "/".join(map(str, self.tiles_down[:BUCKETS])),
+                        "norms": "/".join("D" if deferred else "-" for deferred in self.deferred[:BUCKETS])})
         return out
 
     def decode_supported(self, step, caches) -> bool:
-        """Whether the step's rows go through the skinny products: steps of up to MAX_ROWS single tokens, and
-        steps of as few tokens in portions of prompts (a short prompt, the tail of a long one, beside decoded
-        tokens), whose mixers then run their own kernels between the skinny products."""
-        if step.num_tokens > MAX_ROWS or not self.decode_ok:
+        """Whether the step's rows go through the decode path: steps of up to MAX_ROWS single tokens through the
+        skinny products (or the library, as measured) around the mixers' decode kernel; steps of as few tokens in
+        portions of prompts (a short prompt, the tail of a long one, beside decoded tokens), whose mixers then
+        run their own kernels between those products; and steps of more single tokens than that, whose products
+        all go through the library, when there is a decode kernel for the mixers (the prompt kernels would take a
+        step of 96 single tokens as 96 prompts of one token: 9.1 ms on the 0.5B shape against 3.3 for 64)."""
+        if not self.decode_ok:
             return False
+        if step.num_tokens > MAX_ROWS:
+            return (self.general and step.max_query_len == 1 and self.kernel is not None
+                    and self.kernel.supported(step, caches))
         if step.max_query_len != 1:
             return self.aligned
         return self.aligned or self.kernel.supported(step, caches)
@@ -628,7 +643,7 @@ class LayerFusion:
 
     def forward_decode(self, residual: Residual, step, caches) -> None:
         M = step.num_tokens
-        bucket = _bucket(M)
+        bucket = _bucket(M) if M <= MAX_ROWS else BEYOND
         kernel = self.kernel if (self.kernel is not None and step.max_query_len == 1
                                  and self.kernel.supported(step, caches)) else None
         conv = None

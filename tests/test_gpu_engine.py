@@ -363,7 +363,7 @@ def test_decode_graphs_match_eager_steps(tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("requests, library", [(24, False), (40, False), (5, True), (24, True), (40, "clock"),
-                                               (24, "split"), (40, "split"), (24, "tiles"), (40, "tiles")])
+                                               (24, "split"), (40, "split"), (24, "tiles"), (40, "tiles"), (80, False)])
 def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, requests, library):
     """More single-token lanes than the norm-fused kernels take (16): the block's fast path with
     norms of their own, through graphs of buckets 32 and 64, against the plain model.  ``library``:
@@ -371,7 +371,9 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
     own), as large weights do where that is measured to be faster; "clock": the measurement itself
     runs on this model's small weights and either outcome must be right; "split": the projections
     that feed the residual stream are split over K into float32 slabs that the next norm adds up; "tiles": a
-    workgroup of the skinny kernel owns four tiles of 16 output features, split projections included."""
+    workgroup of the skinny kernel owns four tiles of 16 output features, split projections included.  80
+    requests: more rows than the skinny kernels take; every product through the library, around the mixers'
+    decode kernel (not the prompt kernels, which would take them as 80 prompts of one token)."""
     from macllm_infer_amd import Engine, Lane
     from macllm_infer_amd.parts import fused
     if library == "clock":
@@ -383,17 +385,21 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
         monkeypatch.setattr(fused, "FORCE_SPLIT", 2 if requests == 40 else 0)
     elif library:
         monkeypatch.setattr(fused, "FORCE_LIBRARY", True)
-    folder = tiny_configs.make_model_dir("C", tmp_path, torch.bfloat16)
+    # (the library takes rows whose width is a multiple of 8 elements: configuration D's; C's are not)
+    folder = tiny_configs.make_model_dir("D" if library is True or requests > 64 else "C", tmp_path, torch.bfloat16)
     cfg, tensors = plain_impl.load_model_dir(folder)
     engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * requests,
                     max_active_sequences=requests)
+    if library is True:
+        fusion = engine.model.blocks[0].fusion
+        assert fusion.general and all(fusion.library_in) and all(fusion.library_out) and all(fusion.library_down)
     if library == "split":
         fusion = engine.model.blocks[0].fusion
-        assert fusion.split_out == (0, 0, 0, 3, 3, 3) and fusion.split_down == (0, 0, 0, 3, 3, 3)
+        assert fusion.split_out[:6] == (0, 0, 0, 3, 3, 3) and fusion.split_down[:6] == (0, 0, 0, 3, 3, 3)
     if library == "tiles":
         fusion = engine.model.blocks[0].fusion
-        assert fusion.tiles_in == fusion.tiles_gate_up == fusion.tiles_out == fusion.tiles_down == (1, 1, 1, 4, 4, 4)
-        assert fusion.library_in == fusion.library_down == (False,) * 6
+        assert fusion.tiles_in[:6] == fusion.tiles_gate_up[:6] == fusion.tiles_out[:6] == fusion.tiles_down[:6] == (1, 1, 1, 4, 4, 4)
+        assert fusion.library_in[:6] == fusion.library_down[:6] == (False,) * 6
     prompts = {index: tokens_for(cfg["vocab_size"], 3 + index % 7 + 6, 500 + index) for index in range(requests)}
     for index, tokens in prompts.items():
         engine.add_request(index)
@@ -403,7 +409,10 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
         logits = engine.step([Lane(index, [tokens[len(tokens) - 6 + turn]], [0]) for index, tokens in prompts.items()])
         for row, index in enumerate(prompts):
             got[index].append(logits[row].float().cpu())
-    assert {lanes for lanes, _ in engine.graphs._graphs} == {8 if requests <= 8 else 32 if requests <= 32 else 64}
+    assert {lanes for lanes, _ in engine.graphs._graphs} == {8 if requests <= 8 else 32 if requests <= 32 else 64 if requests <= 64 else 128}
+    if requests > 64:
+        fusion = engine.model.blocks[0].fusion
+        assert fusion.general and fusion.library_in[fused.BEYOND] and fusion.library_down[fused.BEYOND]
     for index, tokens in prompts.items():
         want = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-6:]
         have = torch.stack(got[index])
