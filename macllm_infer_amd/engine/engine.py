@@ -61,6 +61,12 @@ def resolve_dtype(dtype) -> torch.dtype:
     return _DTYPES[dtype]
 
 
+# A step with portions of prompts beside at least this many single decoded tokens runs as two batches (see
+# ``Engine._run_in_two``): beside 2,048 prompt tokens, 8 decoded tokens cost 2.7 ms as part of the batch and 1.3 ms
+# as a batch of their own.
+SPLIT_FROM_LANES = 4
+
+
 class Engine:
     def __init__(self, model_dir: Optional[str] = None, *, config=None, tensors=None, dtype="bfloat16",
                  device="cuda:0", kv_cache_block_tokens: int = 16,
@@ -193,6 +199,7 @@ class Engine:
         return lowered
 
     feeds_tokens = True          # a lane's token may come from the device (``Lane.feed``)
+    split_from_lanes = SPLIT_FROM_LANES      # single tokens beside portions from which on they are a batch of their own
 
     def step(self, lanes: Sequence[Lane]) -> torch.Tensor:
         """Run one batch; returns float32 logits [wanted, vocab] in the order of the lanes and
@@ -203,17 +210,11 @@ class Engine:
         lowered = self.validate(lanes)
         self.cache.reserve_slots(lowered.slots, lowered.lengths)
         try:
-            logits = None
-            if self.graphs is not None:
-                if int(lowered.lengths.max()) == 1:
-                    logits = self.graphs.run(lanes, lowered)              # decode-only batch: a captured graph
-                else:
-                    logits = self.graphs.run_bucket(lanes, lowered)       # prompt portions: a graph of their capacity
-            if logits is None:
-                context = build_step_context(lanes, self.cache, self.device, lowered, self.model.query_tile,
-                                             self.model.chunk_sizes)
-                apply_feeds(context.token_ids, lowered.feeds)
-                logits = self.model.forward(context, self.cache)
+            single = lowered.lengths == 1
+            if self.split_from_lanes <= int(single.sum()) < len(lanes):
+                logits = self._run_in_two(lanes, lowered, single)
+            else:
+                logits = self._run(lanes, lowered)
         except Exception as error:
             # earlier layers have written keys, values and state in place: these requests cannot go on
             names = [lane.request for lane in lanes]
@@ -222,3 +223,38 @@ class Engine:
             raise StepFailed(names, error) from error
         self.cache.commit_slots(lowered.slots, lowered.lengths)
         return logits
+
+    def _run(self, lanes: Sequence[Lane], lowered: LoweredLanes) -> torch.Tensor:
+        """Queue the lanes' tokens as one batch: a captured graph where one fits, else launch by launch."""
+        logits = None
+        if self.graphs is not None:
+            if int(lowered.lengths.max()) == 1:
+                logits = self.graphs.run(lanes, lowered)              # decode-only batch: a captured graph
+            else:
+                logits = self.graphs.run_bucket(lanes, lowered)       # prompt portions: a graph of their capacity
+        if logits is None:
+            context = build_step_context(lanes, self.cache, self.device, lowered, self.model.query_tile,
+                                         self.model.chunk_sizes)
+            apply_feeds(context.token_ids, lowered.feeds)
+            logits = self.model.forward(context, self.cache)
+        return logits
+
+    def _run_in_two(self, lanes: Sequence[Lane], lowered: LoweredLanes, single: np.ndarray) -> torch.Tensor:
+        """A step that holds portions of prompts beside several single decoded tokens, as two batches one after
+        the other: the portions through the prompt kernels, the single tokens through the decode kernels.  (As
+        one batch the prompt kernels take every single token as a prompt of its own, a tile of the attention
+        kernel and a chunk of the scan each: 2,048 prompt tokens beside 63 decoded ones took 19.4 ms on the
+        0.5B shape, where the two batches take 6.3 and 3.1.)  The logits come back in the order of the lanes."""
+        parts, rows = [], []
+        first_rows = np.concatenate(([0], np.cumsum(lowered.want_counts)[:-1]))
+        for chosen in (~single, single):
+            members = [lane for lane, mine in zip(lanes, chosen) if mine]
+            parts.append(self._run(members, self.validate(members)))
+            for index in np.nonzero(chosen)[0]:
+                rows.extend(range(int(first_rows[index]), int(first_rows[index]) + int(lowered.want_counts[index])))
+        logits = torch.cat(parts) if parts[0].numel() and parts[1].numel() else (parts[0] if parts[0].numel() else parts[1])
+        if rows == list(range(len(rows))):
+            return logits
+        order = np.empty(len(rows), dtype=np.int64)
+        order[np.asarray(rows, dtype=np.int64)] = np.arange(len(rows))
+        return logits[torch.from_numpy(order).to(logits.device)]

@@ -191,10 +191,16 @@ class Scheduler:
         if target is None or not visits:
             return visits
         total = sum(len(tokens) for _, tokens, _ in visits)
+        lanes = len(visits)
+        # an engine that runs the single tokens of a step as a batch of their own sizes the portions without them
+        singles = sum(1 for _, tokens, _ in visits if len(tokens) == 1)
+        split_from = getattr(self.engine, "split_from_lanes", None)
+        if split_from is not None and split_from <= singles < lanes:
+            lanes, total = lanes - singles, total - singles
         for index in range(len(visits) - 1, -1, -1):
             request, tokens, samples = visits[index]
             if request.prefilling and not samples and len(tokens) > 1:
-                spare = total - int(target(len(visits), total))
+                spare = total - int(target(lanes, total))
                 if 0 < spare < len(tokens):
                     visits[index] = (request, tokens[:len(tokens) - spare], False)
                 break

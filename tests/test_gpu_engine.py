@@ -728,7 +728,8 @@ def test_replays_that_follow_one_another_without_a_wait_keep_their_own_arrays(tm
 def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
     """Steps with prompt portions run from graphs captured for a capacity (so many tokens in so many lanes):
     portions of 70 and 40 tokens and of 60 and 40 meet the graph of 112 tokens in 4 lanes from their second
-    sighting on, a portion of 10 tokens the one of 16 tokens in 2 lanes, portions beside decoded tokens one more.  Every step, through pages that are given back and
+    sighting on, a portion of 10 tokens the one of 16 tokens in 2 lanes, portions beside three decoded tokens
+    one more; four decoded tokens beside a portion run as a batch of their own.  Every step, through pages that are given back and
     used again and with decode replays between, is compared with an engine without graphs."""
     from macllm_infer_amd import Engine, Lane
     folder = tiny_configs.make_model_dir(name, tmp_path, torch.float32 if dtype == "float32" else torch.bfloat16)
@@ -776,12 +777,20 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
     both([lane(key, 5, [4]) for key in "pqrs"])
     replays = with_graphs.graphs.counts["bucket_replays"]
     for turn in range(6):
-        singles = "pqr" if turn < 3 else "pqrs"
-        lanes = [lane(key, 1, [0]) for key in singles] + [lane("t", 64, [63] if turn == 5 else [])]
+        lanes = [lane(key, 1, [0]) for key in "pqr"] + [lane("t", 32, [31] if turn == 5 else [])]
         both(lanes if turn % 2 == 0 else lanes[::-1])
-    # three or four decoded tokens beside a portion of 64: 80 tokens in 8 lanes, whatever their order
-    assert (8, 80) in [key[:2] for key in with_graphs.graphs._bucket_graphs]
+    # three decoded tokens beside a portion of 32: 48 tokens in 8 lanes (four cannot be padded), whatever their order
+    assert (8, 48) in [key[:2] for key in with_graphs.graphs._bucket_graphs]
     assert with_graphs.graphs.counts["bucket_replays"] == replays + 5
+    # four decoded tokens beside a portion are a batch of their own: the portion goes through the graph of its
+    # capacity, the four through a decode graph, and the logits come back in the order of the lanes
+    replays, decodes = with_graphs.graphs.counts["bucket_replays"], with_graphs.graphs.counts["decode_replays"]
+    for turn in range(4):
+        lanes = [lane(key, 1, [0]) for key in "pq"] + [lane("t", 20, [0, 19] if turn != 1 else [])]
+        lanes += [lane(key, 1, [0]) for key in "rs"]
+        both(lanes if turn % 2 == 0 else lanes[::-1])
+    assert with_graphs.graphs.counts["decode_replays"] == decodes + 4
+    assert with_graphs.graphs.counts["bucket_replays"] == replays + 3
 
 
 @pytest.mark.parametrize("name, dtype, seed", [("B", "float32", 0), ("C", "bfloat16", 1), ("A", "bfloat16", 2)])
