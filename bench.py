@@ -150,7 +150,7 @@ def microbench() -> int:
 
 
 def choices_of(engine) -> dict:
-    """What the first layer's fast path chose for steps of up to 8 / 16 / 32 / 48 / 64 rows, as short strings
+    """What the first layer's fast path chose for steps of up to 4 / 8 / 16 / 32 / 48 / 64 rows, as short strings
     (S: the skinny kernel, L: the library, a number: that many slabs over K; empty when the layer has none)."""
     return engine.path_choices()
 

@@ -17,7 +17,7 @@ mixer           ``cache_needs(spec) -> [KVNeed | StateNeed]`` (classmethod);
 feed-forward    ``forward(x [T, d]) -> [T, d]``; optional ``gated_projections()``
 norm            ``forward(residual, rows=None) -> normed activations``; optional ``rms_prologue() ->
                 (weight, eps)``: the norm is y = x / sqrt(mean(x^2) + eps) * weight, which the skinny
-                kernels compute in their prologue
+                kernels compute in their prologue, or take over altogether (``Residual.scaled``)
 position        ``rotate_and_store(qkv, heads, kv_heads, head_dim, step, cache)``
 every part      ``graph_safe = True`` if its forward may be captured in a HIP graph;
                 ``limits(spec, hidden_size) -> [Limit]`` (classmethod): sizes its kernels refuse

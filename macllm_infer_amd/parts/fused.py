@@ -22,10 +22,16 @@ Decode steps (every lane holds one token, at most 64 rows) go through the skinny
 
 For attention beside Mamba2 such a kernel is registered below: the conv step runs in the epilogue of
 launch 1 and both mixers in one launch 2 (``mixer_decode``), five launches a layer instead of fifteen
-(seven for batches of more than 16 rows, whose two norms run as kernels of their own).
+(seven for batches of more than 16 rows, whose two norms run as kernels of their own).  Where all four
+products run through the skinny kernel, 3 and 5 may add to the residual stream themselves and leave the rows
+that 4 and the next layer's 1 read, so that no launch and no prologue computes a norm (``FORCE_DEFERRED_NORM``
+has the story).
 
 A large weight goes through the BLAS library instead where that is faster (``LIBRARY_MIN_WEIGHT``); the
-conv step and SiLU(g)*u then run as kernels of their own.
+conv step and SiLU(g)*u then run as kernels of their own.  Which way each product goes is measured per step
+size when the layer is built, and the layer's whole plan once more over a chain of layers when the model is
+(``CHAIN_LAYERS``).  Steps of more single tokens than the skinny kernels take rows run every product through
+the library around the same ``mixer_decode``.
 
 The fusion belongs to the arrangement (``register_fusion``), which knows its parts; the parts stay as they
 are.  It is built only for bfloat16 weights and sizes the kernels cover; otherwise the block runs part by
