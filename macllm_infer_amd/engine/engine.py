@@ -61,10 +61,25 @@ def resolve_dtype(dtype) -> torch.dtype:
     return _DTYPES[dtype]
 
 
-# A step with portions of prompts beside at least this many single decoded tokens runs as two batches (see
-# ``Engine._run_in_two``): beside 2,048 prompt tokens, 8 decoded tokens cost 2.7 ms as part of the batch and 1.3 ms
-# as a batch of their own.
-SPLIT_FROM_LANES = 4
+# A step with portions of prompts beside several single decoded tokens runs as two batches (see
+# ``Engine._run_in_two``) when the single tokens cost more as part of the portions' batch than as a batch of their
+# own.  As part of it every one of them is a prompt of one token to the prompt kernels, some SPLIT_LANE_SECONDS a
+# layer (beside 2,048 prompt tokens of the 0.5B shape, 8 decoded tokens cost 2.7 ms and 63 cost 13); a batch of
+# their own reads every weight once more (at some SPLIT_READ_RATE bytes a second) and pays its dependent kernels,
+# SPLIT_LAYER_SECONDS a layer.  That makes 5 single tokens for the 0.5B shape, 17 for the 7B shape and 39 for the 34B
+# shape, whose 68 GB of weights are better read once for both.
+SPLIT_LANE_SECONDS = 6e-6
+SPLIT_LAYER_SECONDS = 24e-6
+SPLIT_READ_RATE = 4.5e12
+SPLIT_FROM_LANES = 4                 # and never fewer than this
+
+
+def split_from_lanes(weight_bytes: int, layers: int) -> int:
+    """From how many single decoded tokens beside portions of prompts on a step runs as two batches."""
+    if layers <= 0:
+        return SPLIT_FROM_LANES
+    own_batch = weight_bytes / SPLIT_READ_RATE + layers * SPLIT_LAYER_SECONDS
+    return max(SPLIT_FROM_LANES, int(own_batch / (layers * SPLIT_LANE_SECONDS) + 0.5))
 
 
 class Engine:
@@ -99,6 +114,9 @@ class Engine:
         build = BuildContext(hidden_size=self.spec.hidden_size, dtype=self.dtype, device=self.device,
                              max_context=self.spec.max_context, measure_paths=measured_paths)
         self.model = DecoderModel(self.spec, bound, build)
+        weight_bytes = sum(tensor.numel() * tensor.element_size() for tensor in bound.values()
+                           if isinstance(tensor, torch.Tensor))
+        self.split_from_lanes = split_from_lanes(weight_bytes, len(self.spec.schedule))
         needs, shared = DecoderModel.cache_layout(self.spec)
         capacity = kv_cache_capacity_tokens or self.spec.max_context
         self.cache = CacheManager(needs, shared, kv_cache_block_tokens, capacity, max_active_sequences,
@@ -199,7 +217,6 @@ class Engine:
         return lowered
 
     feeds_tokens = True          # a lane's token may come from the device (``Lane.feed``)
-    split_from_lanes = SPLIT_FROM_LANES      # single tokens beside portions from which on they are a batch of their own
 
     def step(self, lanes: Sequence[Lane]) -> torch.Tensor:
         """Run one batch; returns float32 logits [wanted, vocab] in the order of the lanes and
