@@ -55,6 +55,48 @@ def test_whole_chunked_and_mixed_match_the_plain_model(host_ops, tmp_path, name)
     engine.cache.check()
 
 
+def test_portions_beside_several_decoded_tokens_run_as_two_batches_in_the_callers_order(host_ops, tmp_path, monkeypatch):
+    """A step that holds portions of prompts beside four or more single tokens is queued as two batches (the
+    portions, then the single tokens); the logits come back in the order of the lanes and of their wanted
+    places, whatever that order is, and are the plain model's.  A step that is refused is refused whole."""
+    engine, cfg, tensors = engine_for("A", tmp_path, capacity=400, page=8, requests=7)
+    assert engine.split_from_lanes == 4
+    batches = []
+    real = engine._run
+    monkeypatch.setattr(engine, "_run", lambda lanes, lowered: (batches.append([lane.request for lane in lanes]), real(lanes, lowered))[1])
+    streams = {key: tokens_for(cfg, 40, 30 + index) for index, key in enumerate("abcdefg")}
+    wants = {key: plain_impl.falcon_h1_logits(cfg, tensors, tokens) for key, tokens in streams.items()}
+    for key in streams:
+        engine.add_request(key)
+    engine.step([Lane(key, streams[key][:10], []) for key in "abcde"])                  # five requests that decode
+    assert batches == [list("abcde")]
+    batches.clear()
+    # portions of f and g between the single tokens of a..e; f wants two places, g none, d none
+    lanes = [Lane("a", streams["a"][10:11], [0]), Lane("f", streams["f"][:12], [3, 11]), Lane("b", streams["b"][10:11], [0]),
+             Lane("c", streams["c"][10:11], [0]), Lane("g", streams["g"][:7], []), Lane("d", streams["d"][10:11], []),
+             Lane("e", streams["e"][10:11], [0])]
+    got = engine.step(lanes)
+    assert batches == [["f", "g"], ["a", "b", "c", "d", "e"]]
+    expected = [wants["a"][10], wants["f"][3], wants["f"][11], wants["b"][10], wants["c"][10], wants["e"][10]]
+    assert got.shape[0] == len(expected)
+    for row, want in enumerate(expected):
+        assert (got[row] - want).abs().max() < 1e-4, row
+    # three single tokens beside a portion stay one batch
+    batches.clear()
+    got = engine.step([Lane("a", streams["a"][11:12], [0]), Lane("g", streams["g"][7:20], [12]), Lane("b", streams["b"][11:12], [0]),
+                       Lane("c", streams["c"][11:12], [0])])
+    assert batches == [["a", "g", "b", "c"]]
+    for row, want in enumerate([wants["a"][11], wants["g"][19], wants["b"][11], wants["c"][11]]):
+        assert (got[row] - want).abs().max() < 1e-4, row
+    # a token outside the vocabulary in the portion: nothing runs, nothing changes
+    batches.clear()
+    before = engine.cache.stats()
+    with pytest.raises(StepError):
+        engine.step([Lane(key, streams[key][12:13], [0]) for key in "abcd"] + [Lane("f", [cfg["vocab_size"]] * 3, [])])
+    assert batches == [] and engine.cache.stats() == before
+    engine.cache.check()
+
+
 def test_refused_steps_change_nothing(host_ops, tmp_path):
     engine, cfg, tensors = engine_for("A", tmp_path, capacity=32, page=8, requests=2)
     engine.add_request("a")
