@@ -66,7 +66,12 @@ class DecodeGraphs:
         self._pool = None
         self.counts = {"decode_replays": 0, "bucket_replays": 0, "bucket_captures": 0, "bucket_eager": 0}
 
-    BUCKET_GRAPHS = 24             # captured capacities kept; the least recently used one goes
+    # captured capacities kept; the least recently used one goes.  A capture costs about as much as thirty replays
+    # save, so the graphs of a workload must all fit: 150 requests of 16 to 1,200 prompt tokens through the
+    # scheduler meet 31 capacities (portions that end a prompt have any length), and with room for 24 every run
+    # of them captured a dozen again (1.06 s a run instead of 0.78).  The graphs share one memory pool: more of them
+    # cost their index arrays and nodes, not activations.
+    BUCKET_GRAPHS = 96
     BUCKET_SIGHTINGS = 2           # sightings of a capacity before it is captured
     BUCKET_MOST_TOKENS = 16384     # steps beyond this many tokens are launched kernel by kernel
 
