@@ -249,6 +249,39 @@ def test_sampled_generation_a_round_ahead_equals_generation_that_waits(tmp_path)
         assert generated == outcomes[0][index][0], index
 
 
+def test_generation_with_more_live_requests_than_the_skinny_kernels_take_rows(tmp_path):
+    """Seventy-two requests live at once through the scheduler (bfloat16, configuration D): prompts of 3 to 40
+    tokens in portions of 24 beside the decoded tokens of the others (so steps run as two batches), then rounds of
+    up to 72 single tokens (the decode kernel between library products).  Every request runs to its length, no
+    page or slot is left held, and for five of the requests every token is the plain model's choice or as good
+    as it (the plain model's logit of the token within a few per cent of its best: bfloat16 may swap near ties)."""
+    from macllm_infer_amd import LLM, EngineConfig, SamplingParams
+    folder = tiny_configs.make_model_dir("D", tmp_path, torch.bfloat16)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    count = 72
+    prompts = [tokens_for(cfg["vocab_size"], 3 + (7 * index) % 38, 500 + index) for index in range(count)]
+    llm = LLM(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * count,
+              engine_config=EngineConfig(max_active_sequences=count, scheduler_token_budget=24 + count,
+                                         prefill_token_quantum=24))
+    runs = []
+    real = llm.engine._run
+    llm.engine._run = lambda lanes, lowered: (runs.append((len(lanes), int(lowered.lengths.max()))), real(lanes, lowered))[1]
+    params = SamplingParams(max_new_tokens=7, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0, ignore_eos=True)
+    results = llm.generate(prompts, params)
+    assert [result.finish_reason for result in results] == ["length"] * count
+    assert all(len(result.token_ids) == 7 for result in results)
+    assert any(lanes > 64 and longest == 1 for lanes, longest in runs)            # rounds of more than 64 single tokens
+    assert any(longest > 1 for _, longest in runs) and any(lanes >= 4 and longest == 1 for lanes, longest in runs)
+    assert llm.engine.cache.stats()["live_requests"] == 0
+    llm.engine.cache.check()
+    for index in (0, 17, 40, 63, 71):
+        tokens = list(prompts[index])
+        for token in results[index].token_ids:
+            logits = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-1]
+            assert logits[token].item() >= logits.max().item() - 0.06 * logits.abs().max().item(), (index, len(tokens))
+            tokens.append(token)
+
+
 def test_generation_when_pages_run_out(tmp_path):
     """Seven requests on a cache of six pages, three live at a time: lanes are dropped from steps
     and retried, pages and slots are used again, and a request that cannot grow while the others
