@@ -320,6 +320,7 @@ sample_kernel(float* __restrict__ logits, int V, int padded, const float* __rest
 // does not cover (k above SAMPLE_KMAX) is left with done[row] = 0 for sample_kernel, which skips the
 // rows that are done.  The logits of a row that is drawn here are divided by its temperature in place.
 #define SAMPLE_KMAX 1024
+#define HISTOGRAM_COPIES 16
 #define SAMPLE_LIST 2048             // keys that share their two upper bytes with the one looked for, listed in LDS
 #define SAMPLE_ROW_PASSES_FROM 6     // the passes over bytes 7 and 6 read the row; those below read the list
 
@@ -471,6 +472,7 @@ sample_select_kernel(float* __restrict__ logits, int V, const float* __restrict_
   __shared__ unsigned long long candidates[SAMPLE_KMAX];
   __shared__ unsigned long long by_index[SAMPLE_KMAX];
   __shared__ unsigned int histogram[256];
+  __shared__ unsigned int histogram_copies[HISTOGRAM_COPIES][256];   // the passes over the row count into the copy of their lane
   __shared__ unsigned long long mass_histogram[256];
   __shared__ unsigned long long chosen_prefix, remaining_mass;
   __shared__ unsigned long long list[SAMPLE_LIST];
@@ -527,6 +529,7 @@ sample_select_kernel(float* __restrict__ logits, int V, const float* __restrict_
   if (tid == 0) listed = 0;
   for (int pass = 7; pass >= 0; --pass) {
     if (tid < 256) histogram[tid] = 0u;
+    for (int i = tid; i < HISTOGRAM_COPIES * 256; i += blockDim.x) (&histogram_copies[0][0])[i] = 0u;
     __syncthreads();
     const unsigned long long prefix = chosen_prefix;
     const unsigned long long above = pass == 7 ? 0ull : (~0ull << (8 * (pass + 1)));
@@ -544,12 +547,27 @@ sample_select_kernel(float* __restrict__ logits, int V, const float* __restrict_
     auto count = [&](unsigned long long key) {
       if ((key & above) == prefix) atomicAdd(&histogram[(unsigned int)(key >> (8 * pass)) & 255u], 1u);
     };
+    // over the row, nearly all keys of the top bytes fall into a few bins, and additions of one wave to one LDS
+    // address are done one after the other: every lane counts into one of HISTOGRAM_COPIES copies, added up after
+    auto count_row = [&](unsigned long long key) {
+      if ((key & above) == prefix)
+        atomicAdd(&histogram_copies[tid % HISTOGRAM_COPIES][(unsigned int)(key >> (8 * pass)) & 255u], 1u);
+    };
+    bool over_the_row = true;
     if (pass < SAMPLE_ROW_PASSES_FROM && listed <= SAMPLE_LIST) {
       for (int i = tid; i < listed; i += blockDim.x) count(list[i]);
+      over_the_row = false;
     } else if (pass == 7) {
-      for_each_key<true>(values, V, temp, count);
+      for_each_key<true>(values, V, temp, count_row);
     } else {
-      for_each_key<false>(values, V, temp, count);
+      for_each_key<false>(values, V, temp, count_row);
+    }
+    __syncthreads();
+    if (over_the_row && tid < 256) {
+      unsigned int sum = 0u;
+#pragma unroll
+      for (int copy = 0; copy < HISTOGRAM_COPIES; ++copy) sum += histogram_copies[copy][tid];
+      histogram[tid] = sum;
     }
     __syncthreads();
     // the bin in which the running count reaches what is still wanted: the first wave scans the
