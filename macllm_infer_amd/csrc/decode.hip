@@ -602,6 +602,150 @@ static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStre
   return 0;
 }
 
+// The product in float32 slabs over K for steps of many rows, with the rows shared.  In fused_gemm_kernel every
+// wave walks columns of its own, so every wave fetches its own part of the step's rows: at 48 to 64 rows four
+// times the bytes of the weights cross the caches (a 5,120 x 21,504 weight at 64 rows: 93 us where the weights
+// alone stream in 49).  Here the four waves of a workgroup own NT tiles of 16 features each and walk the same
+// columns: the rows of a stage (SR_CHUNKS * 32 columns) are fetched once a workgroup, laid in LDS (two stages,
+// one barrier a stage) and read from there by all four, while each wave asks for its next stage's weights before
+// it multiplies the current one's.
+constexpr int SR_CHUNKS = 4;
+constexpr int SR_LD = SR_CHUNKS * 32 + 8;        // a stage's row in LDS, padded against bank conflicts
+
+template <int MT, int NT>
+__global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p) {
+  __shared__ __align__(16) bf16_t stage[2][MT * 16 * SR_LD];
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE, q = lane / 16, r = lane % 16;
+  const int tiles = (p.N + 15) / 16;
+  const int chunks = p.K / 32;
+  const int per_split = (chunks + gridDim.y - 1) / gridDim.y;
+  const int first_chunk = blockIdx.y * per_split;
+  const int end_chunk = min(first_chunk + per_split, chunks);          // may lie before first_chunk: an empty slab
+  const int stages = max(0, end_chunk - first_chunk + SR_CHUNKS - 1) / SR_CHUNKS;
+  const int tile0 = (blockIdx.x * 4 + wave) * NT;
+
+  const int w_step = p.w_tiled ? 512 : 32;
+  const bf16_t* w_row[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int tile = min(tile0 + nt, tiles - 1);
+    w_row[nt] = p.w_tiled ? p.W + (long)tile * chunks * 512 + lane * 8
+                          : p.W + (long)min(tile * 16 + r, p.N - 1) * p.K + 8 * q;
+  }
+  // a thread's pieces of a stage's rows: 8 columns each, 16 pieces a row
+  const bf16_t* x_from[MT];
+  int x_to[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int piece = tid + j * 256;
+    x_from[j] = p.x + (long)min(piece / 16, p.M - 1) * p.x_ld + (piece % 16) * 8;
+    x_to[j] = (piece / 16) * SR_LD + (piece % 16) * 8;
+  }
+  // no condition around a load (a stage or chunk past the end reads the last one again and is multiplied as zeros)
+  auto ask_rows = [&](bf16x8_t (&rows)[MT], int s) {
+    const int c0 = min(first_chunk + s * SR_CHUNKS, chunks - SR_CHUNKS);
+#pragma unroll
+    for (int j = 0; j < MT; ++j) rows[j] = *reinterpret_cast<const bf16x8_t*>(x_from[j] + (long)max(c0, 0) * 32);
+  };
+  auto ask_weights = [&](bf16x8_t (&a)[SR_CHUNKS][NT], int s) {
+    const int c0 = max(min(first_chunk + s * SR_CHUNKS, chunks - SR_CHUNKS), 0);
+#pragma unroll
+    for (int j = 0; j < SR_CHUNKS; ++j)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        a[j][nt] = *reinterpret_cast<const bf16x8_t*>(w_row[nt] + (long)min(c0 + j, chunks - 1) * w_step);
+  };
+  auto lay_rows = [&](const bf16x8_t (&rows)[MT], int buffer) {
+#pragma unroll
+    for (int j = 0; j < MT; ++j) *reinterpret_cast<bf16x8_t*>(&stage[buffer][x_to[j]]) = rows[j];
+  };
+
+  floatx4 acc[NT][MT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // the stage that starts at chunk c0 (clamped as in the loads) holds the chunks c0 .. c0 + SR_CHUNKS - 1; those
+  // outside [from, end_chunk) count as zeros: before `from` where the clamp moved the stage back over chunks
+  // that an earlier stage has multiplied already
+  auto multiply = [&](const bf16x8_t (&a)[SR_CHUNKS][NT], int s, int buffer) {
+    const int wanted = first_chunk + s * SR_CHUNKS;
+    const int c0 = max(min(wanted, chunks - SR_CHUNKS), 0);
+#pragma unroll
+    for (int j = 0; j < SR_CHUNKS; ++j) {
+      const bool counts = c0 + j >= wanted && c0 + j < end_chunk;
+      bf16x8_t b[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        b[mt] = *reinterpret_cast<const bf16x8_t*>(&stage[buffer][(mt * 16 + r) * SR_LD + j * 32 + 8 * q]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const floatx4 weights = counts ? *reinterpret_cast<const floatx4*>(&a[j][nt]) : floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8_t*>(&weights), b[mt],
+                                                                acc[nt][mt], 0, 0, 0);
+      }
+    }
+  };
+
+  bf16x8_t rows[MT], a_even[SR_CHUNKS][NT], a_odd[SR_CHUNKS][NT];
+  ask_rows(rows, 0);
+  ask_weights(a_even, 0);
+  lay_rows(rows, 0);
+  __syncthreads();
+  for (int s = 0; s < stages; s += 2) {
+    ask_rows(rows, s + 1);
+    ask_weights(a_odd, s + 1);
+    multiply(a_even, s, 0);
+    lay_rows(rows, 1);
+    __syncthreads();
+    if (s + 1 >= stages) break;
+    ask_rows(rows, s + 2);
+    ask_weights(a_even, s + 2);
+    multiply(a_odd, s + 1, 1);
+    lay_rows(rows, 0);
+    __syncthreads();
+  }
+
+  // lane (q, r) holds features 4 q .. 4 q + 3 of row r of every tile: 16 bytes of a slab's row
+  float* slab = reinterpret_cast<float*>(p.out) + (long)blockIdx.y * p.M * p.out_ld;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n = (tile0 + nt) * 16 + 4 * q;
+    if (tile0 + nt >= tiles) continue;
+    floatx4 bias = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias && blockIdx.y == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bias[i] = p.bias[min(n + i, p.N - 1)];
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + r;
+      if (m >= p.M) continue;
+      const floatx4 v = acc[nt][mt] + bias;
+      float* to = slab + (long)m * p.out_ld + n;
+      if (p.out_ld % 4 == 0 && n + 3 < p.N) {
+        *reinterpret_cast<floatx4*>(to) = v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < p.N) to[i] = v[i];
+      }
+    }
+  }
+}
+
+template <int MT>
+static int launch_shared_rows(const FusedGemmParams& p, hipStream_t stream, int k_splits, int feature_tiles) {
+  const int tiles = (p.N + 15) / 16;
+  const dim3 blocks((tiles + 4 * feature_tiles - 1) / (4 * feature_tiles), k_splits);
+  if (feature_tiles == 1) shared_rows_gemm_kernel<MT, 1><<<blocks, 4 * WAVE, 0, stream>>>(p);
+  else if (feature_tiles == 2) shared_rows_gemm_kernel<MT, 2><<<blocks, 4 * WAVE, 0, stream>>>(p);
+  else return ERR_BAD_ARGUMENT;
+  return 0;
+}
+
 // Sizes: 1 <= M <= 64, K a multiple of 32; with the NORM prologue the step's M normalized rows must fit
 // 64 KiB of LDS beside the reduction area (16 rows of 1,024, 8 of 3,072).  EPI_SWIGLU wants N a multiple of 16.
 // w_fragments: W is not row-major [N, K] but a copy in the order of the matrix-core fragments,
@@ -698,6 +842,36 @@ extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, cons
   else if (MT == 2) code = launch_fused_gemm<2>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
   else if (MT == 3) code = launch_fused_gemm<3>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
   else code = launch_fused_gemm<4>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
+  if (code != 0) return code;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// The same slabs for steps of 17 to 64 rows through shared_rows_gemm_kernel: a workgroup's four waves own
+// feature_tiles (1 or 2) tiles of 16 features each and share the step's rows through LDS.  K >= 128.
+extern "C" int mi_shared_rows_gemm_split(const void* x, long x_ld, const void* W, const float* bias, int M, int N,
+                                         int K, float* partial, int splits, int feature_tiles, int w_fragments,
+                                         hipStream_t stream) {
+  if (M <= 0 || N <= 0 || K <= 0 || !W || !x || !partial || x_ld < K || x_ld % 8 != 0) return ERR_BAD_ARGUMENT;
+  if (feature_tiles != 1 && feature_tiles != 2) return ERR_BAD_ARGUMENT;
+  if (M <= 16 || M > 64 || K % 32 != 0 || K / 32 < SR_CHUNKS || splits < 1 || splits > 64 || K / 32 < splits)
+    return ERR_UNSUPPORTED_SIZE;
+  FusedGemmParams p = {};
+  p.x = (const bf16_t*)x;
+  p.x_ld = x_ld;
+  p.W = (const bf16_t*)W;
+  p.bias = bias;
+  p.M = M;
+  p.N = N;
+  p.K = K;
+  p.out = partial;
+  p.out_ld = N;
+  p.out_f32 = 1;
+  p.out_scale = 1.0f;
+  p.w_tiled = w_fragments ? 1 : 0;
+  const int code = M <= 32   ? launch_shared_rows<2>(p, stream, splits, feature_tiles)
+                   : M <= 48 ? launch_shared_rows<3>(p, stream, splits, feature_tiles)
+                             : launch_shared_rows<4>(p, stream, splits, feature_tiles);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;

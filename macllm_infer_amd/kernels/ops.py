@@ -83,6 +83,8 @@ _SIGNATURES = {
         "mi_fused_gemm_supported": [_c_int, _c_int, _c_int],
         "mi_fused_gemm_split": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int,
                                 _c_ptr],
+        "mi_shared_rows_gemm_split": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int,
+                                      _c_int, _c_ptr],
         "mi_mixer_split_keys": [_c_int, _c_int, _c_int, _c_long],
         "mi_mixer_runs": [_c_int, _c_int, _c_int, _c_long, _c_ptr, _c_ptr],
         "mi_fused_gemm_merge": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_ptr,
@@ -758,11 +760,14 @@ def fused_gemm_merge(weight: torch.Tensor, bias: Optional[torch.Tensor], out: Op
 
 
 def fused_gemm_split(weight: torch.Tensor, bias: Optional[torch.Tensor], x: torch.Tensor, partial: torch.Tensor,
-                     feature_tiles: int = 1, fragments: Optional[torch.Tensor] = None) -> None:
+                     feature_tiles: int = 1, fragments: Optional[torch.Tensor] = None,
+                     shared_rows: bool = False) -> None:
     """x [M, K] . weight[N, K]^T (+ bias) for a small batch in bfloat16, split over K: slab s of
     ``partial`` (float32 [S, M, N], contiguous) receives the sums over the s-th run of K, the bias
     in slab 0.  The product is the sum of the slabs (``add_partials_rmsnorm`` adds them to the
-    residual stream): many rows, a long K and few output features fill the GPU this way."""
+    residual stream): many rows, a long K and few output features fill the GPU this way.
+    ``shared_rows`` (17 to 64 rows, K >= 128, 1 or 2 feature tiles a wave): the kernel whose four waves
+    share the step's rows through LDS instead of fetching them each."""
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm_split: weight must be contiguous bfloat16 [N, K]")
     N, K = weight.shape
@@ -774,10 +779,10 @@ def fused_gemm_split(weight: torch.Tensor, bias: Optional[torch.Tensor], x: torc
     _need(partial.dtype == torch.float32 and partial.dim() == 3 and partial.shape[1:] == (M, N)
           and partial.is_contiguous() and partial.is_cuda, "fused_gemm_split: partial must be contiguous float32 [S, M, N]")
     operand = _weight_operand(weight, fragments, "fused_gemm_split")
-    _check(_fn("decode", "mi_fused_gemm_split")(_p(x), x_ld, _p(operand), _p(bias), M, N, K, _p(partial),
-                                                partial.shape[0], int(feature_tiles), int(fragments is not None),
-                                                _stream()),
-           "fused_gemm_split", f"(M={M}, N={N}, K={K}, S={partial.shape[0]})")
+    entry = "mi_shared_rows_gemm_split" if shared_rows else "mi_fused_gemm_split"
+    _check(_fn("decode", entry)(_p(x), x_ld, _p(operand), _p(bias), M, N, K, _p(partial), partial.shape[0],
+                                int(feature_tiles), int(fragments is not None), _stream()),
+           "fused_gemm_split", f"(M={M}, N={N}, K={K}, S={partial.shape[0]}, shared_rows={shared_rows})")
 
 
 def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, *, out_scale: float = 1.0,

@@ -72,6 +72,15 @@ _library_wins: Dict[tuple, tuple] = {}
 # at build like the library; the split has to win by SPLIT_MARGIN, for the norm reads the slabs.
 SPLIT_CHOICES = (2, 4, 8)
 SPLIT_MARGIN = 0.85
+# From 17 rows on the slabs can also come from the kernel whose four waves own feature tiles and share the step's
+# rows through LDS (in the skinny kernel every wave fetches rows of its own, four times the bytes of the weights
+# at 64 rows): a 5,120 x 21,504 weight at 64 rows in 52 us with 8 slabs, against 93 and the library's 133; a
+# 3,072 x 12,288 one in 21 against 34 and 35.  Written as a negative number of feature tiles (that many a wave).
+# A slab costs the norm behind it a read, counted at SLAB_READ_RATE bytes a microsecond.
+SHARED_ROWS_FROM = 17
+FORCE_SHARED_ROWS: Optional[int] = None   # tests, with FORCE_SPLIT: this many tiles a wave of that kernel
+SHARED_SPLIT_CHOICES = (4, 8, 16)
+SLAB_READ_RATE = 4.0e6
 FORCE_SPLIT: Optional[int] = None         # tests: a number of slabs (0 = never) instead of the clock
 _split_wins: Dict[tuple, tuple] = {}
 # Beyond 16 rows the skinny kernel's workgroup may own 2 or 4 tiles of 16 output features instead of one: the
@@ -228,17 +237,21 @@ def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool, tiles: 
                 ops.fused_gemm(w, bias, out, x=x, feature_tiles=tiles, fragments=f)
 
     best, best_time = (0, tiles), SPLIT_MARGIN * _graph_microseconds(whole)
-    for slabs in SPLIT_CHOICES:
+    shared_from = SHARED_ROWS_FROM if K // 32 >= 4 else rows + 1
+    for slabs in sorted(set(SPLIT_CHOICES) | (set(SHARED_SPLIT_CHOICES) if rows >= shared_from else set())):
         if K // 32 < slabs:
             continue
         partial = torch.empty((slabs, rows, N), dtype=torch.float32, device=device)
-        for split_tiles in TILE_CHOICES[:2]:
+        ways = [tile for tile in TILE_CHOICES[:2] if slabs in SPLIT_CHOICES]
+        ways += [-tile for tile in TILE_CHOICES[:2] if rows >= shared_from and slabs in SHARED_SPLIT_CHOICES]
+        for split_tiles in ways:
 
             def split():
                 for w, f in zip(weights, fragments):
-                    ops.fused_gemm_split(w, bias, x, partial, feature_tiles=split_tiles, fragments=f)
+                    ops.fused_gemm_split(w, bias, x, partial, feature_tiles=abs(split_tiles), fragments=f,
+                                         shared_rows=split_tiles < 0)
 
-            time = _graph_microseconds(split)
+            time = _graph_microseconds(split) + len(weights) * partial.numel() * 4 / SLAB_READ_RATE
             if time < best_time:
                 best, best_time = (slabs, split_tiles), time
     return best
@@ -499,7 +512,8 @@ class LayerFusion:
         by the clock over a chain of layers of this one's shape (measured once per shape)."""
         if (not self.measure or not self.decode_ok or self.gate_up is None or self.ffn_scale is None
                 or self.mixer_scale is None
-                or any(force is not None for force in (FORCE_DEFERRED_NORM, FORCE_LIBRARY, FORCE_SPLIT, FORCE_TILES))
+                or any(force is not None for force in (FORCE_DEFERRED_NORM, FORCE_LIBRARY, FORCE_SPLIT, FORCE_TILES,
+                                                      FORCE_SHARED_ROWS))
                 or self.w_in.numel() + self.w_out.numel() + self.gate_up.weight.numel() + self.down.weight.numel()
                 < LIBRARY_MIN_WEIGHT):
             return
@@ -512,8 +526,9 @@ class LayerFusion:
 
     def path_choices(self) -> dict:
         """Which way each projection goes for steps of up to TUNE_ROWS rows, as short strings (S: the skinny
-        kernel, L: the library, a number: that many slabs over K), the feature tiles of the skinny kernel, and
-        for portions of up to PAD_ROWS tokens whether the input projection is padded (P)."""
+        kernel, L: the library, a number: that many slabs over K), the feature tiles of the skinny kernel (with
+        an r: a wave's, of the kernel that shares the rows), and for portions of up to PAD_ROWS tokens whether
+        the input projection is padded (P)."""
         if not self.decode_ok:
             return {}
 
@@ -522,13 +537,15 @@ class LayerFusion:
             split = split or (0,) * len(library)
             return "/".join(str(slabs) if slabs else ("L" if lib else "S") for lib, slabs in zip(library, split))
 
+        def tiled(tiles):
+            return "/".join(str(tile) if tile > 0 else f"{-tile}r" for tile in tiles[:BUCKETS])
+
         out = {"in": way(self.library_in), "out": way(self.library_out, self.split_out),
-               "tiles_in": "/".join(map(str, self.tiles_in[:BUCKETS])), "tiles_out": "/".join(map(str, self.tiles_out[:BUCKETS])),
+               "tiles_in": tiled(self.tiles_in), "tiles_out": tiled(self.tiles_out),
                "padded_in": "/".join("P" if pays else "-" for pays in self.padding_pays)}
         if self.gate_up is not None:
             out.update({"gate_up": way(self.library_gate_up), "down": way(self.library_down, self.split_down),
-                        "tiles_gate_up": "/".join(map(str, self.tiles_gate_up[:BUCKETS])),
-                        "tiles_down": "/".join(map(str, self.tiles_down[:BUCKETS])),
+                        "tiles_gate_up": tiled(self.tiles_gate_up), "tiles_down": tiled(self.tiles_down),
                         "norms": "/".join("D" if deferred else "-" for deferred in self.deferred[:BUCKETS])})
         return out
 
@@ -613,6 +630,8 @@ class LayerFusion:
             return _each(0), tiles
         if FORCE_SPLIT:
             slabs = FORCE_SPLIT if weight.shape[1] // 32 >= FORCE_SPLIT else 0
+            if FORCE_SHARED_ROWS and slabs and weight.shape[1] // 32 >= 4:
+                tiles = tuple(-FORCE_SHARED_ROWS if bucket in self.wide_buckets else tile for bucket, tile in enumerate(tiles))
             return tuple(slabs if bucket in self.wide_buckets else 0 for bucket in range(BUCKETS)), tiles
         if weight.numel() < LIBRARY_MIN_WEIGHT or not self.measure:
             return _each(0), tiles
@@ -783,7 +802,9 @@ class LayerFusion:
             return [delta]
         if slabs:
             partial = torch.empty((slabs, M, self.hidden), dtype=torch.float32, device=x.device)
-            ops.fused_gemm_split(weight, bias, x, partial, feature_tiles=tiles, fragments=fragments)
+            shared = tiles < 0 and M >= SHARED_ROWS_FROM
+            ops.fused_gemm_split(weight, bias, x, partial, feature_tiles=abs(tiles), fragments=fragments,
+                                 shared_rows=shared)
             return list(partial.unbind(0))
         if library:
             return [ops.linear(x, weight, bias)]

@@ -396,7 +396,8 @@ def test_decode_graphs_match_eager_steps(tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("requests, library", [(24, False), (40, False), (5, True), (24, True), (40, "clock"),
-                                               (24, "split"), (40, "split"), (24, "tiles"), (40, "tiles"), (80, False)])
+                                               (24, "split"), (40, "split"), (24, "tiles"), (40, "tiles"), (80, False),
+                                               (24, "shared"), (40, "shared"), (57, "shared")])
 def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, requests, library):
     """More single-token lanes than the norm-fused kernels take (16): the block's fast path with
     norms of their own, through graphs of buckets 32 and 64, against the plain model.  ``library``:
@@ -404,7 +405,8 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
     own), as large weights do where that is measured to be faster; "clock": the measurement itself
     runs on this model's small weights and either outcome must be right; "split": the projections
     that feed the residual stream are split over K into float32 slabs that the next norm adds up; "tiles": a
-    workgroup of the skinny kernel owns four tiles of 16 output features, split projections included.  80
+    workgroup of the skinny kernel owns four tiles of 16 output features, split projections included; "shared":
+    the slabs come from the kernel whose waves own feature tiles and share the step's rows through LDS.  80
     requests: more rows than the skinny kernels take; every product through the library, around the mixers'
     decode kernel (not the prompt kernels, which would take them as 80 prompts of one token)."""
     from macllm_infer_amd import Engine, Lane
@@ -413,6 +415,9 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
         monkeypatch.setattr(fused, "LIBRARY_MIN_WEIGHT", 0)
     elif library == "split":
         monkeypatch.setattr(fused, "FORCE_SPLIT", 3)
+    elif library == "shared":
+        monkeypatch.setattr(fused, "FORCE_SPLIT", 2 if requests == 40 else 3)
+        monkeypatch.setattr(fused, "FORCE_SHARED_ROWS", 2 if requests == 24 else 1)
     elif library == "tiles":
         monkeypatch.setattr(fused, "FORCE_TILES", 4)
         monkeypatch.setattr(fused, "FORCE_SPLIT", 2 if requests == 40 else 0)
@@ -429,6 +434,12 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
     if library == "split":
         fusion = engine.model.blocks[0].fusion
         assert fusion.split_out[:6] == (0, 0, 0, 3, 3, 3) and fusion.split_down[:6] == (0, 0, 0, 3, 3, 3)
+    if library == "shared":
+        fusion = engine.model.blocks[0].fusion
+        slabs, tiles = (2 if requests == 40 else 3), (-2 if requests == 24 else -1)
+        assert fusion.split_out[:6] == fusion.split_down[:6] == (0, 0, 0, slabs, slabs, slabs)
+        assert fusion.tiles_out[:6] == (1, 1, 1, tiles, tiles, tiles)
+        assert fusion.tiles_down[:6] == (1,) * 6                  # a K of 96 is below that kernel's stage of 128 columns
     if library == "tiles":
         fusion = engine.model.blocks[0].fusion
         assert fusion.tiles_in[:6] == fusion.tiles_gate_up[:6] == fusion.tiles_out[:6] == fusion.tiles_down[:6] == (1, 1, 1, 4, 4, 4)

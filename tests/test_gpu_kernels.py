@@ -923,6 +923,43 @@ def test_fused_gemm_split_over_k_and_the_norm_that_adds_its_slabs(ops, M, N, K, 
         assert torch.equal(again, got_h)
 
 
+@pytest.mark.parametrize("M, N, K, S", [(64, 1024, 2048, 8), (33, 100, 2048, 16), (48, 138, 1056, 3), (49, 72, 3072, 5),
+                                        (64, 50, 128, 1), (40, 272, 288, 8), (57, 16, 4672, 64), (17, 40, 160, 2), (32, 264, 1024, 4)])
+def test_fused_gemm_split_with_the_rows_shared_by_a_workgroups_waves(ops, M, N, K, S):
+    """The slabs of the kernel whose waves own feature tiles and share the rows through LDS: widths with a last
+    tile of fewer than 16 features and rows that are no multiple of four floats, a K whose last stage is short or
+    is moved back over chunks already multiplied, more slabs than stages, slabs without chunks, row-major
+    weights and the fragment order, against the plain product per slab and the unshared kernel's slabs."""
+    x = rand(M, K + 24, seed=350, dtype=torch.bfloat16)[:, :K]
+    W, b = rand(N, K, seed=351, scale=0.1, dtype=torch.bfloat16), rand(N, seed=352)
+    want = torch.zeros(S, M, N)
+    ref_ops.fused_gemm_split(W, b, x, want)
+    other = torch.full((S, M, N), float("nan"), device=DEV)
+    ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), other)
+    for feature_tiles in (1, 2):
+        got = torch.full((S, M, N), float("nan"), device=DEV)
+        ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), got, feature_tiles=feature_tiles, shared_rows=True)
+        close(got, want, torch.float32, 50.0)
+        close(got, other.cpu(), torch.float32, 50.0)
+        again = torch.full((S, M, N), float("nan"), device=DEV)
+        ops.fused_gemm_split(W.to(DEV), None, x.to(DEV), again, feature_tiles=feature_tiles,
+                             fragments=ops.fragment_order(W.to(DEV)), shared_rows=True)
+        again[0] += b.to(DEV)
+        close(again, got.cpu(), torch.float32, 2.0)
+
+
+def test_fused_gemm_split_with_the_rows_shared_refuses_other_sizes(ops):
+    """16 rows or fewer and more than 64, a K below one stage of 128 columns, four tiles a wave: an error,
+    and nothing written."""
+    for rows, K, tiles in ((16, 256, 1), (65, 256, 1), (40, 96, 1), (40, 256, 4)):
+        W = torch.zeros(48, K, dtype=torch.bfloat16, device=DEV)
+        x = torch.zeros(rows, K, dtype=torch.bfloat16, device=DEV)
+        partial = torch.full((1, rows, 48), 7.0, device=DEV)
+        with pytest.raises((ValueError, RuntimeError)):
+            ops.fused_gemm_split(W, None, x, partial, feature_tiles=tiles, shared_rows=True)
+        assert bool((partial == 7.0).all())
+
+
 @pytest.mark.parametrize("M, N, K", [(24, 200, 1024), (64, 136, 1024), (7, 96, 2048), (64, 88, 3072), (40, 64, 64)])
 def test_fused_gemm_conv_step_of_wide_batches(ops, M, N, K):
     """The conv epilogue behind the plain prologue: more than one tile of 16 rows, four and eight
