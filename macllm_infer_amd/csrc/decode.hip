@@ -608,13 +608,16 @@ static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStre
 // alone stream in 49).  Here the four waves of a workgroup own NT tiles of 16 features each and walk the same
 // columns: the rows of a stage (SR_CHUNKS * 32 columns) are fetched once a workgroup, laid in LDS (two stages,
 // one barrier a stage) and read from there by all four, while each wave asks for its next stage's weights before
-// it multiplies the current one's.
+// it multiplies the current one's.  EPI_PLAIN: float32 slabs over K, one a row of workgroups.  EPI_SWIGLU: all of
+// K in one workgroup (a gate and up projection has features enough to fill the GPU), SiLU(gate) * up in
+// bfloat16 as in fused_gemm_kernel, with the row scale of a norm left to this product if there is one.
 constexpr int SR_CHUNKS = 4;
 constexpr int SR_LD = SR_CHUNKS * 32 + 8;        // a stage's row in LDS, padded against bank conflicts
 
-template <int MT, int NT>
+template <int MT, int NT, int EPI>
 __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p) {
   __shared__ __align__(16) bf16_t stage[2][MT * 16 * SR_LD];
+  __shared__ float squares[4][MT * 16];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE, q = lane / 16, r = lane % 16;
   const int tiles = (p.N + 15) / 16;
   const int chunks = p.K / 32;
@@ -692,6 +695,13 @@ __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p
   bf16x8_t rows[MT], a_even[SR_CHUNKS][NT], a_odd[SR_CHUNKS][NT];
   ask_rows(rows, 0);
   ask_weights(a_even, 0);
+  if (EPI == EPI_SWIGLU && p.ssq_in && tid < 4 * MT * 16) {
+    // the rows' sums of squares, which the workgroups of the product before left in parts: four threads a row
+    const int row = tid % (MT * 16);
+    float sum = 0.f;
+    for (int b = tid / (MT * 16); b < p.ssq_blocks; b += 4) sum += p.ssq_in[(long)b * (MT * 16) + row];
+    squares[tid / (MT * 16)][row] = sum;
+  }
   lay_rows(rows, 0);
   __syncthreads();
   for (int s = 0; s < stages; s += 2) {
@@ -708,7 +718,52 @@ __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p
     __syncthreads();
   }
 
-  // lane (q, r) holds features 4 q .. 4 q + 3 of row r of every tile: 16 bytes of a slab's row
+  // lane (q, r) holds features 4 q .. 4 q + 3 of row r of every tile
+  if (EPI == EPI_SWIGLU) {
+    // a tile is 8 gate features, then the 8 up features of the same columns: lanes q = 0, 1 take their up
+    // values from the lanes q + 2 and write 4 columns of bfloat16
+    float factor[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      factor[mt] = 1.0f;
+      if (p.ssq_in) {
+        const int m = mt * 16 + r;
+        const float sum = squares[0][m] + squares[1][m] + squares[2][m] + squares[3][m];
+        factor[mt] = 1.0f / sqrtf(sum / (float)p.ssq_width + p.ssq_eps);
+      }
+    }
+    bf16_t* out = reinterpret_cast<bf16_t*>(p.out);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int n = (tile0 + nt) * 16 + 4 * q;
+      floatx4 bias = {0.f, 0.f, 0.f, 0.f};
+      if (p.bias) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bias[i] = p.bias[min(n + i, p.N - 1)];
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const floatx4 v = acc[nt][mt] * factor[mt] + bias;
+        floatx4 up;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) up[i] = __shfl(v[i], (lane + 32) % WAVE);
+        const int m = mt * 16 + r;
+        const int column = (tile0 + nt) * 8 + 4 * q;
+        if (tile0 + nt >= tiles || q >= 2 || m >= p.M) continue;
+        bf16x4_t packed;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(silu_f(round_bf16(v[i])) * round_bf16(up[i]));
+        bf16_t* to = out + (long)m * p.out_ld + column;
+        if (p.out_ld % 4 == 0) {
+          *reinterpret_cast<bf16x4_t*>(to) = packed;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) to[i] = packed[i];
+        }
+      }
+    }
+    return;
+  }
   float* slab = reinterpret_cast<float*>(p.out) + (long)blockIdx.y * p.M * p.out_ld;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
@@ -736,12 +791,12 @@ __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p
   }
 }
 
-template <int MT>
+template <int MT, int EPI>
 static int launch_shared_rows(const FusedGemmParams& p, hipStream_t stream, int k_splits, int feature_tiles) {
   const int tiles = (p.N + 15) / 16;
   const dim3 blocks((tiles + 4 * feature_tiles - 1) / (4 * feature_tiles), k_splits);
-  if (feature_tiles == 1) shared_rows_gemm_kernel<MT, 1><<<blocks, 4 * WAVE, 0, stream>>>(p);
-  else if (feature_tiles == 2) shared_rows_gemm_kernel<MT, 2><<<blocks, 4 * WAVE, 0, stream>>>(p);
+  if (feature_tiles == 1) shared_rows_gemm_kernel<MT, 1, EPI><<<blocks, 4 * WAVE, 0, stream>>>(p);
+  else if (feature_tiles == 2) shared_rows_gemm_kernel<MT, 2, EPI><<<blocks, 4 * WAVE, 0, stream>>>(p);
   else return ERR_BAD_ARGUMENT;
   return 0;
 }
@@ -751,7 +806,8 @@ static int launch_shared_rows(const FusedGemmParams& p, hipStream_t stream, int 
 // w_fragments: W is not row-major [N, K] but a copy in the order of the matrix-core fragments,
 // [ceil(N / 16), K / 32, 4, 16, 8] with element [n, c, q, r, j] = W[16 n + r, 32 c + 8 q + j] (rows past N zero):
 // what a wave asks for at once is then one run of 1 KiB instead of 64 bytes of each of 16 rows, which
-// streams 15 to 25 % faster.
+// streams 15 to 25 % faster.  feature_tiles -1 or -2 (17 to 64 rows, K >= 128, plain prologue, EPI_SWIGLU): that
+// many tiles a wave of the kernel whose waves share the step's rows through LDS.
 extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* delta0, const void* delta1,
                              float* h_out, const float* norm_w, float eps, const void* x, long x_ld,
                              const void* W, const float* bias, int M, int N, int K, void* out, long out_ld,
@@ -761,8 +817,11 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
                              float ssq_eps, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !out) return ERR_BAD_ARGUMENT;
   if (ssq_in && (pro != PRO_PLAIN || ssq_blocks <= 0 || ssq_width <= 0)) return ERR_BAD_ARGUMENT;
-  if (feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
+  const bool shared_rows = feature_tiles < 0;       // -1, -2: that many tiles a wave of shared_rows_gemm_kernel
+  if (shared_rows && (feature_tiles < -2 || pro != PRO_PLAIN || epi != EPI_SWIGLU)) return ERR_BAD_ARGUMENT;
+  if (!shared_rows && feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0) return ERR_UNSUPPORTED_SIZE;
+  if (shared_rows && (M <= 16 || K / 32 < SR_CHUNKS)) return ERR_UNSUPPORTED_SIZE;
   if (pro == PRO_NORM && (!h_in || !norm_w || h_out == h_in)) return ERR_BAD_ARGUMENT;
   if (pro == PRO_PLAIN && (!x || x_ld < K || x_ld % 8 != 0)) return ERR_BAD_ARGUMENT;
   if (epi == EPI_SWIGLU && (N % 16 != 0 || out_f32)) return ERR_BAD_ARGUMENT;
@@ -803,7 +862,10 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
   p.ssq_width = ssq_width;
   p.ssq_eps = ssq_eps;
   int code;
-  if (MT == 1) code = launch_fused_gemm<1>(p, pro, epi, stream, 1, feature_tiles);
+  if (shared_rows && MT == 2) code = launch_shared_rows<2, EPI_SWIGLU>(p, stream, 1, -feature_tiles);
+  else if (shared_rows && MT == 3) code = launch_shared_rows<3, EPI_SWIGLU>(p, stream, 1, -feature_tiles);
+  else if (shared_rows) code = launch_shared_rows<4, EPI_SWIGLU>(p, stream, 1, -feature_tiles);
+  else if (MT == 1) code = launch_fused_gemm<1>(p, pro, epi, stream, 1, feature_tiles);
   else if (MT == 2) code = launch_fused_gemm<2>(p, pro, epi, stream, 1, feature_tiles);
   else if (MT == 3) code = launch_fused_gemm<3>(p, pro, epi, stream, 1, feature_tiles);
   else code = launch_fused_gemm<4>(p, pro, epi, stream, 1, feature_tiles);
@@ -869,9 +931,9 @@ extern "C" int mi_shared_rows_gemm_split(const void* x, long x_ld, const void* W
   p.out_f32 = 1;
   p.out_scale = 1.0f;
   p.w_tiled = w_fragments ? 1 : 0;
-  const int code = M <= 32   ? launch_shared_rows<2>(p, stream, splits, feature_tiles)
-                   : M <= 48 ? launch_shared_rows<3>(p, stream, splits, feature_tiles)
-                             : launch_shared_rows<4>(p, stream, splits, feature_tiles);
+  const int code = M <= 32   ? launch_shared_rows<2, EPI_PLAIN>(p, stream, splits, feature_tiles)
+                   : M <= 48 ? launch_shared_rows<3, EPI_PLAIN>(p, stream, splits, feature_tiles)
+                             : launch_shared_rows<4, EPI_PLAIN>(p, stream, splits, feature_tiles);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;

@@ -790,7 +790,7 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
                deltas: Sequence[torch.Tensor] = (), h_out: Optional[torch.Tensor] = None,
                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, epilogue: int = EPI_PLAIN,
                conv: Optional[dict] = None, feature_tiles: int = 1, fragments: Optional[torch.Tensor] = None,
-               row_scale: Optional["RowScale"] = None) -> None:
+               row_scale: Optional["RowScale"] = None, shared_rows: bool = False) -> None:
     """out[M, N'] = epilogue(prologue . weight[N, K]^T + bias) for a small batch in bfloat16.
 
     Prologue: ``x`` [M, K] bfloat16, or ``h_in`` float32 [M, K] with up to two bfloat16 ``deltas``:
@@ -804,7 +804,9 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
     steps of many rows gain from more.  ``fragments``: ``fragment_order(weight)``, read instead of the weight.
     ``row_scale`` (with ``x``): x holds rows times a norm's weight that are not divided by their root mean
     square yet; the sums of row m are multiplied by 1 / sqrt(sum of squares of the row / width + eps) before the
-    bias, from the partial sums of squares that ``fused_gemm_residual`` left."""
+    bias, from the partial sums of squares that ``fused_gemm_residual`` left.  ``shared_rows`` (17 to 64 rows of
+    ``x``, K >= 128, SWIGLU, 1 or 2 feature tiles a wave): the kernel whose four waves own feature tiles and share
+    the step's rows through LDS instead of fetching them each."""
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm: weight must be contiguous bfloat16 [N, K]")
     _need(row_scale is None or x is not None, "fused_gemm: a row scale needs x")
@@ -813,6 +815,8 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
               and row_scale.ssq.shape[1] == 16 * (-(-out.shape[0] // 16)), "fused_gemm: the partial sums of squares do not fit the step")
     _need(feature_tiles in (1, 2, 4) and (feature_tiles == 1 or x is not None),
           "fused_gemm: feature_tiles is 1, 2 or 4, and more than 1 needs x")
+    _need(not shared_rows or (x is not None and epilogue == EPI_SWIGLU and feature_tiles in (1, 2)),
+          "fused_gemm: shared_rows takes x, the SwiGLU epilogue and 1 or 2 feature tiles a wave")
     N, K = weight.shape
     M = out.shape[0]
     _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()),
@@ -853,7 +857,7 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
         _p(h_out), _p(norm_weight), float(eps), _p(x), x_ld, _p(_weight_operand(weight, fragments, "fused_gemm")),
         _p(bias), M, N, K, _p(out), out_ld,
         1 if out.dtype == torch.float32 else 0, float(out_scale), lo, hi, taps, _p(conv_w), _p(conv_b), _p(conv_state),
-        _p(slot_ids), int(feature_tiles), int(fragments is not None),
+        _p(slot_ids), -int(feature_tiles) if shared_rows else int(feature_tiles), int(fragments is not None),
         _p(row_scale.ssq) if row_scale is not None else None, row_scale.ssq.shape[0] if row_scale is not None else 0,
         int(row_scale.width) if row_scale is not None else 0, float(row_scale.eps) if row_scale is not None else 0.0,
         _stream()), "fused_gemm", f"(M={M}, N={N}, K={K})")

@@ -69,9 +69,9 @@ _library_wins: Dict[tuple, tuple] = {}
 # An output or down projection at 32 to 64 rows has a long K and few output features: 64 workgroups of the
 # skinny kernel, or whatever tile the library picks (10.7 us for 1,024 x 2,048 at 64 rows).  Split over K into
 # float32 slabs that the next norm adds up, the skinny kernel fills the GPU (7.5 us with 2 slabs; at 32 rows 5.2 us against the library's 9.6).  Measured
-# at build like the library; the split has to win by SPLIT_MARGIN, for the norm reads the slabs.
+# at build like the library; the split has to win by SPLIT_MARGIN.
 SPLIT_CHOICES = (2, 4, 8)
-SPLIT_MARGIN = 0.85
+SPLIT_MARGIN = 0.92
 # From 17 rows on the slabs can also come from the kernel whose four waves own feature tiles and share the step's
 # rows through LDS (in the skinny kernel every wave fetches rows of its own, four times the bytes of the weights
 # at 64 rows): a 5,120 x 21,504 weight at 64 rows in 52 us with 8 slabs, against 93 and the library's 133; a
@@ -129,14 +129,22 @@ _chain_times: list = []     # (rows, microseconds a layer of each candidate, the
 
 
 OVERLAP_MIN_TOKENS = 256       # prompt portions from this size on run their two mixers on two streams
-_side_streams: Dict[int, "torch.cuda.Stream"] = {}
+_side_streams: Dict[int, list] = {}
 
 
-def _side_stream(device: torch.device) -> "torch.cuda.Stream":
+def _side_stream(device: torch.device, beside: "torch.cuda.Stream") -> "torch.cuda.Stream":
+    """A second stream of the device (default priority) that is not ``beside``.  Streams come from a pool of a
+    few dozen that hands them out in turn, so the one drawn may be the very stream a graph is being captured on:
+    work recorded "beside" it would queue behind (a 2,048-token prompt of the 0.5B shape: 7.2 ms instead of 6.3)."""
     index = device.index if device.index is not None else torch.cuda.current_device()
-    if index not in _side_streams:
-        _side_streams[index] = torch.cuda.Stream(device=device)       # default priority
-    return _side_streams[index]
+    streams = _side_streams.setdefault(index, [])
+    for stream in streams:
+        if stream != beside:
+            return stream
+    while True:
+        streams.append(torch.cuda.Stream(device=device))
+        if streams[-1] != beside:
+            return streams[-1]
 
 
 def _bucket(rows: int) -> int:
@@ -260,7 +268,8 @@ def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool, tiles: 
 def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile: int, conv: Optional[dict],
                      wide: bool) -> tuple:
     """(whether the library way is faster for this weight at this many rows, the skinny kernel's best number
-    of feature tiles; ``wide``: more than one tile may be taken, i.e. the prologue is the plain one).  Copies
+    of feature tiles; ``wide``: more than one tile may be taken, i.e. the prologue is the plain one; negative:
+    that many a wave of the kernel that shares the rows, which SiLU(gate) * up can come from).  Copies
     of the weight are cycled through so that the caches do not hold it, as in a model of many layers."""
     N, K = weight.shape
     device = weight.device
@@ -290,7 +299,15 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
                 ops.conv_step(product, conv["lo"], conv["hi"] - conv["lo"], conv["weight"], conv["bias"], conv["state"],
                               conv["slot_ids"])
 
+    def shared_rows(tiles):
+        def run():
+            for w, f in zip(weights, fragments):
+                ops.fused_gemm(w, bias, out, x=x, epilogue=epilogue, feature_tiles=tiles, fragments=f, shared_rows=True)
+        return run
+
     times = {tiles: _graph_microseconds(skinny(tiles)) for tiles in (TILE_CHOICES if wide else (1,))}
+    if wide and epilogue == ops.EPI_SWIGLU and rows >= SHARED_ROWS_FROM and K // 32 >= 4:
+        times.update({-tiles: _graph_microseconds(shared_rows(tiles)) for tiles in TILE_CHOICES[:2]})
     tiles = min(times, key=lambda count: times[count] * (1.0 if count == 1 else 1.0 / TILE_MARGIN))
     return _graph_microseconds(library) < LIBRARY_MARGIN * times[tiles], tiles
 
@@ -598,7 +615,7 @@ class LayerFusion:
             # other branch pays the hops between queues.  (Attention beside a state-space mixer, whose kernels
             # are many and small: the state-space chain is the longer one and stays on the main queue.)
             main = torch.cuda.current_stream(u.device)
-            side = _side_stream(u.device)
+            side = _side_stream(u.device, main)
             side.wait_stream(main)
             self._mix_each(u, step, caches, mixed, order=(1,))
             with torch.cuda.stream(side):
@@ -650,6 +667,8 @@ class LayerFusion:
 
     def _tune_all(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict], normed: bool) -> tuple:
         forced = 1 if FORCE_TILES is None else FORCE_TILES
+        if FORCE_SHARED_ROWS and epilogue == ops.EPI_SWIGLU and weight.shape[1] // 32 >= 4:
+            forced = -FORCE_SHARED_ROWS
         fixed_tiles = tuple(forced if bucket in self.wide_buckets else 1 for bucket in range(BUCKETS))
         if (not self.general or FORCE_LIBRARY is False
                 or (FORCE_LIBRARY is None and (weight.numel() < LIBRARY_MIN_WEIGHT or not self.measure))):
@@ -758,15 +777,15 @@ class LayerFusion:
             scaled = None
         if scaled is not None:
             ops.fused_gemm(self.gate_up.weight, self.gate_up.bias, activated, epilogue=ops.EPI_SWIGLU,
-                           feature_tiles=self.tiles_gate_up[bucket], fragments=self.f_gate_up,
+                           fragments=self.f_gate_up, **_tiles(self.tiles_gate_up[bucket], M),
                            **self._behind_the_norm(scaled, self.ffn_scale))
         elif self.library_gate_up[bucket]:
             ops.swiglu(ops.linear(block.ffn_norm.forward(residual), self.gate_up.weight, self.gate_up.bias), activated, 8)
         else:
             arguments, h_out = self._norm_prologue(residual, M, block.ffn_norm, self.ffn_rms)
             ops.fused_gemm(self.gate_up.weight, self.gate_up.bias, activated, epilogue=ops.EPI_SWIGLU,
-                           feature_tiles=self.tiles_gate_up[bucket] if "x" in arguments else 1,
-                           fragments=self.f_gate_up, **arguments)
+                           fragments=self.f_gate_up, **(_tiles(self.tiles_gate_up[bucket], M) if "x" in arguments else {}),
+                           **arguments)
             if h_out is not None:
                 residual.h, residual.pending = h_out, []
         # 5
@@ -802,15 +821,19 @@ class LayerFusion:
             return [delta]
         if slabs:
             partial = torch.empty((slabs, M, self.hidden), dtype=torch.float32, device=x.device)
-            shared = tiles < 0 and M >= SHARED_ROWS_FROM
-            ops.fused_gemm_split(weight, bias, x, partial, feature_tiles=abs(tiles), fragments=fragments,
-                                 shared_rows=shared)
+            ops.fused_gemm_split(weight, bias, x, partial, fragments=fragments, **_tiles(tiles, M))
             return list(partial.unbind(0))
         if library:
             return [ops.linear(x, weight, bias)]
         delta = torch.empty((M, self.hidden), dtype=torch.bfloat16, device=x.device)
-        ops.fused_gemm(weight, bias, delta, x=x, feature_tiles=tiles, fragments=fragments)
+        ops.fused_gemm(weight, bias, delta, x=x, feature_tiles=abs(tiles), fragments=fragments)
         return [delta]
+
+
+def _tiles(tiles: int, rows: int) -> dict:
+    """A plan's number of feature tiles as the products' arguments: negative, that many a wave of the kernel that
+    shares the rows (steps of fewer rows than it takes: as many a workgroup of the skinny kernel)."""
+    return dict(feature_tiles=abs(tiles), shared_rows=tiles < 0 and rows >= SHARED_ROWS_FROM)
 
 
 def _rms_prologue(norm):

@@ -440,6 +440,7 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
         assert fusion.split_out[:6] == fusion.split_down[:6] == (0, 0, 0, slabs, slabs, slabs)
         assert fusion.tiles_out[:6] == (1, 1, 1, tiles, tiles, tiles)
         assert fusion.tiles_down[:6] == (1,) * 6                  # a K of 96 is below that kernel's stage of 128 columns
+        assert fusion.tiles_gate_up[:6] == (1, 1, 1, tiles, tiles, tiles) and fusion.library_gate_up[:6] == (False,) * 6
     if library == "tiles":
         fusion = engine.model.blocks[0].fusion
         assert fusion.tiles_in[:6] == fusion.tiles_gate_up[:6] == fusion.tiles_out[:6] == fusion.tiles_down[:6] == (1, 1, 1, 4, 4, 4)
@@ -933,6 +934,20 @@ def test_long_portions_overlap_their_mixers(tmp_path, name):
         engine.finish(a)
         engine.finish(b)
     assert engine.graphs.counts["bucket_replays"] >= 5
+
+
+def test_the_second_stream_is_never_the_stream_it_runs_beside(monkeypatch):
+    """Streams come from a pool that hands them out in turn; whichever of them a graph is captured on, the
+    stream that the first mixer of a long portion runs on is another one (on the same one the two mixers
+    would run one after the other), and two streams are all that is ever drawn for it."""
+    from macllm_infer_amd.parts import fused
+    monkeypatch.setattr(fused, "_side_streams", {})
+    device = torch.device(DEV)
+    pool = [torch.cuda.Stream(device=device) for _ in range(70)]           # every stream of the pool, twice over
+    for main in pool + [torch.cuda.current_stream(device)]:
+        side = fused._side_stream(device, main)
+        assert side != main and side.device == main.device
+    assert len(fused._side_streams[device.index]) <= 2
 
 
 @pytest.mark.parametrize("padding", [False, True])

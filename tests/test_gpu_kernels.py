@@ -948,6 +948,39 @@ def test_fused_gemm_split_with_the_rows_shared_by_a_workgroups_waves(ops, M, N, 
         close(again, got.cpu(), torch.float32, 2.0)
 
 
+@pytest.mark.parametrize("M, N, K, scaled", [(64, 1024, 2048, False), (33, 112, 1056, True), (48, 272, 128, True),
+                                             (17, 48, 288, False), (57, 4112, 160, True), (32, 16, 4672, True)])
+def test_fused_gemm_swiglu_with_the_rows_shared_by_a_workgroups_waves(ops, M, N, K, scaled):
+    """SiLU(gate) * up from the kernel whose waves own feature tiles and share the rows through LDS, with and
+    without the row scale of a norm left to it, one and two tiles a wave, row-major weights and the fragment
+    order, a last workgroup with waves that own no tile, an output whose rows are no multiple of four columns
+    apart: against the plain product and the skinny kernel's result."""
+    x = rand(M, K + 8, seed=360, dtype=torch.bfloat16)[:, :K]
+    W, b = rand(N, K, seed=361, scale=0.1, dtype=torch.bfloat16), rand(N, seed=362)
+    width, eps = 520, 2e-5
+    ssq = rand(width // 16 + 1, 16 * (-(-M // 16)), seed=363).abs() * 3.0 if scaled else None
+    want = torch.empty(M, N // 2, dtype=torch.bfloat16)
+    ref_ops.fused_gemm(W, b, want, x=x, epilogue=ref_ops.EPI_SWIGLU, row_scale=ops.RowScale(ssq, width, eps) if scaled else None)
+    scale = ops.RowScale(ssq.to(DEV), width, eps) if scaled else None
+    skinny = torch.empty(M, N // 2, dtype=torch.bfloat16, device=DEV)
+    ops.fused_gemm(W.to(DEV), b.to(DEV), skinny, x=x.to(DEV), epilogue=ops.EPI_SWIGLU, row_scale=scale)
+    for feature_tiles in (1, 2):
+        for fragments in (None, ops.fragment_order(W.to(DEV))):
+            for pad in (0, 3):
+                got = torch.full((M, N // 2 + pad), float("nan"), dtype=torch.bfloat16, device=DEV)[:, :N // 2]
+                ops.fused_gemm(W.to(DEV), b.to(DEV), got, x=x.to(DEV), epilogue=ops.EPI_SWIGLU, row_scale=scale,
+                               feature_tiles=feature_tiles, fragments=fragments, shared_rows=True)
+                close(got, want, torch.bfloat16, 16.0)
+                close(got, skinny.cpu(), torch.bfloat16, max(2.0, want.float().abs().max().item() / 4))   # an ulp of the largest, between two orders of summation
+    for rows, k, tiles, epilogue in ((16, 256, 1, ops.EPI_SWIGLU), (40, 96, 1, ops.EPI_SWIGLU), (40, 256, 4, ops.EPI_SWIGLU),
+                                     (40, 256, 1, ops.EPI_PLAIN)):
+        weight = torch.zeros(32, k, dtype=torch.bfloat16, device=DEV)
+        out = torch.zeros(rows, 16 if epilogue == ops.EPI_SWIGLU else 32, dtype=torch.bfloat16, device=DEV)
+        with pytest.raises((ValueError, RuntimeError)):
+            ops.fused_gemm(weight, None, out, x=torch.zeros(rows, k, dtype=torch.bfloat16, device=DEV), epilogue=epilogue,
+                           feature_tiles=tiles, shared_rows=True)
+
+
 def test_fused_gemm_split_with_the_rows_shared_refuses_other_sizes(ops):
     """16 rows or fewer and more than 64, a K below one stage of 128 columns, four tiles a wave: an error,
     and nothing written."""
