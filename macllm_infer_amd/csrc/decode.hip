@@ -608,9 +608,11 @@ static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStre
 // alone stream in 49).  Here the four waves of a workgroup own NT tiles of 16 features each and walk the same
 // columns: the rows of a stage (SR_CHUNKS * 32 columns) are fetched once a workgroup, laid in LDS (two stages,
 // one barrier a stage) and read from there by all four, while each wave asks for its next stage's weights before
-// it multiplies the current one's.  EPI_PLAIN: float32 slabs over K, one a row of workgroups.  EPI_SWIGLU: all of
-// K in one workgroup (a gate and up projection has features enough to fill the GPU), SiLU(gate) * up in
-// bfloat16 as in fused_gemm_kernel, with the row scale of a norm left to this product if there is one.
+// it multiplies the current one's.  EPI_PLAIN: float32 slabs over K, one a row of workgroups.  EPI_SWIGLU and
+// EPI_CONV: all of K in one workgroup (a gate and up projection or a layer's input projection has features
+// enough to fill the GPU); SiLU(gate) * up, or rows in bfloat16 with the conv step of the columns that have
+// one (none: plain rows), as in fused_gemm_kernel, with the row scale of a norm left to this product if
+// there is one.
 constexpr int SR_CHUNKS = 4;
 constexpr int SR_LD = SR_CHUNKS * 32 + 8;        // a stage's row in LDS, padded against bank conflicts
 
@@ -695,7 +697,10 @@ __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p
   bf16x8_t rows[MT], a_even[SR_CHUNKS][NT], a_odd[SR_CHUNKS][NT];
   ask_rows(rows, 0);
   ask_weights(a_even, 0);
-  if (EPI == EPI_SWIGLU && p.ssq_in && tid < 4 * MT * 16) {
+  int slot[MT];                                     // CONV: the rows' conv tails, asked for with the first loads
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) slot[mt] = EPI == EPI_CONV && p.slot_ids ? p.slot_ids[min(mt * 16 + r, p.M - 1)] : 0;
+  if (EPI != EPI_PLAIN && p.ssq_in && tid < 4 * MT * 16) {
     // the rows' sums of squares, which the workgroups of the product before left in parts: four threads a row
     const int row = tid % (MT * 16);
     float sum = 0.f;
@@ -719,19 +724,63 @@ __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p
   }
 
   // lane (q, r) holds features 4 q .. 4 q + 3 of row r of every tile
+  float factor[MT];                                 // the norm's division, on the float32 sums
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    factor[mt] = 1.0f;
+    if (EPI != EPI_PLAIN && p.ssq_in) {
+      const int m = mt * 16 + r;
+      const float sum = squares[0][m] + squares[1][m] + squares[2][m] + squares[3][m];
+      factor[mt] = 1.0f / sqrtf(sum / (float)p.ssq_width + p.ssq_eps);
+    }
+  }
+  if (EPI == EPI_CONV) {
+    // bfloat16 rows; the columns conv_lo .. conv_hi - 1 through the conv step of their channel with the row's
+    // tail, which is rolled by one, and SiLU, as in fused_gemm_kernel (no channel is anyone else's)
+    bf16_t* out = reinterpret_cast<bf16_t*>(p.out);
+    const int channels = p.conv_hi - p.conv_lo;
+    const int taps = p.conv_k;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int n = (tile0 + nt) * 16 + 4 * q;
+      if (tile0 + nt >= tiles) continue;
+      floatx4 bias = {0.f, 0.f, 0.f, 0.f};
+      if (p.bias) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bias[i] = p.bias[min(n + i, p.N - 1)];
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + r;
+        if (m >= p.M) continue;
+        const floatx4 v = acc[nt][mt] * factor[mt] + bias;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (n + i >= p.N) continue;
+          if (n + i < p.conv_lo || n + i >= p.conv_hi) {
+            out[(long)m * p.out_ld + n + i] = (bf16_t)(v[i] * p.out_scale);
+            continue;
+          }
+          const int channel = n + i - p.conv_lo;
+          bf16_t* tail = p.conv_state + (long)slot[mt] * (taps - 1) * channels + channel;
+          const bf16_t sample = (bf16_t)v[i];
+          float sum = p.conv_b ? p.conv_b[channel] : 0.f;
+          for (int k = 0; k < taps - 1; ++k) {
+            const bf16_t old = tail[(long)k * channels];
+            sum += p.conv_w[channel * taps + k] * (float)old;
+            if (k > 0) tail[(long)(k - 1) * channels] = old;       // roll the tail by one
+          }
+          sum += p.conv_w[channel * taps + taps - 1] * (float)sample;
+          if (taps > 1) tail[(long)(taps - 2) * channels] = sample;
+          out[(long)m * p.out_ld + n + i] = (bf16_t)silu_f(sum);
+        }
+      }
+    }
+    return;
+  }
   if (EPI == EPI_SWIGLU) {
     // a tile is 8 gate features, then the 8 up features of the same columns: lanes q = 0, 1 take their up
     // values from the lanes q + 2 and write 4 columns of bfloat16
-    float factor[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      factor[mt] = 1.0f;
-      if (p.ssq_in) {
-        const int m = mt * 16 + r;
-        const float sum = squares[0][m] + squares[1][m] + squares[2][m] + squares[3][m];
-        factor[mt] = 1.0f / sqrtf(sum / (float)p.ssq_width + p.ssq_eps);
-      }
-    }
     bf16_t* out = reinterpret_cast<bf16_t*>(p.out);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -806,7 +855,7 @@ static int launch_shared_rows(const FusedGemmParams& p, hipStream_t stream, int 
 // w_fragments: W is not row-major [N, K] but a copy in the order of the matrix-core fragments,
 // [ceil(N / 16), K / 32, 4, 16, 8] with element [n, c, q, r, j] = W[16 n + r, 32 c + 8 q + j] (rows past N zero):
 // what a wave asks for at once is then one run of 1 KiB instead of 64 bytes of each of 16 rows, which
-// streams 15 to 25 % faster.  feature_tiles -1 or -2 (17 to 64 rows, K >= 128, plain prologue, EPI_SWIGLU): that
+// streams 15 to 25 % faster.  feature_tiles -1 or -2 (17 to 64 rows, K >= 128, plain prologue, bfloat16 out): that
 // many tiles a wave of the kernel whose waves share the step's rows through LDS.
 extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* delta0, const void* delta1,
                              float* h_out, const float* norm_w, float eps, const void* x, long x_ld,
@@ -818,7 +867,7 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
   if (M <= 0 || N <= 0 || K <= 0 || !W || !out) return ERR_BAD_ARGUMENT;
   if (ssq_in && (pro != PRO_PLAIN || ssq_blocks <= 0 || ssq_width <= 0)) return ERR_BAD_ARGUMENT;
   const bool shared_rows = feature_tiles < 0;       // -1, -2: that many tiles a wave of shared_rows_gemm_kernel
-  if (shared_rows && (feature_tiles < -2 || pro != PRO_PLAIN || epi != EPI_SWIGLU)) return ERR_BAD_ARGUMENT;
+  if (shared_rows && (feature_tiles < -2 || pro != PRO_PLAIN || out_f32)) return ERR_BAD_ARGUMENT;
   if (!shared_rows && feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0) return ERR_UNSUPPORTED_SIZE;
   if (shared_rows && (M <= 16 || K / 32 < SR_CHUNKS)) return ERR_UNSUPPORTED_SIZE;
@@ -862,7 +911,15 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
   p.ssq_width = ssq_width;
   p.ssq_eps = ssq_eps;
   int code;
-  if (shared_rows && MT == 2) code = launch_shared_rows<2, EPI_SWIGLU>(p, stream, 1, -feature_tiles);
+  if (shared_rows && epi != EPI_SWIGLU) {           // plain rows in bfloat16: the conv epilogue without a conv column
+    if (epi == EPI_PLAIN) {
+      p.conv_lo = p.conv_hi = 0;
+      p.conv_k = 1;
+    }
+    code = MT == 2   ? launch_shared_rows<2, EPI_CONV>(p, stream, 1, -feature_tiles)
+           : MT == 3 ? launch_shared_rows<3, EPI_CONV>(p, stream, 1, -feature_tiles)
+                     : launch_shared_rows<4, EPI_CONV>(p, stream, 1, -feature_tiles);
+  } else if (shared_rows && MT == 2) code = launch_shared_rows<2, EPI_SWIGLU>(p, stream, 1, -feature_tiles);
   else if (shared_rows && MT == 3) code = launch_shared_rows<3, EPI_SWIGLU>(p, stream, 1, -feature_tiles);
   else if (shared_rows) code = launch_shared_rows<4, EPI_SWIGLU>(p, stream, 1, -feature_tiles);
   else if (MT == 1) code = launch_fused_gemm<1>(p, pro, epi, stream, 1, feature_tiles);

@@ -805,8 +805,8 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
     ``row_scale`` (with ``x``): x holds rows times a norm's weight that are not divided by their root mean
     square yet; the sums of row m are multiplied by 1 / sqrt(sum of squares of the row / width + eps) before the
     bias, from the partial sums of squares that ``fused_gemm_residual`` left.  ``shared_rows`` (17 to 64 rows of
-    ``x``, K >= 128, SWIGLU, 1 or 2 feature tiles a wave): the kernel whose four waves own feature tiles and share
-    the step's rows through LDS instead of fetching them each."""
+    ``x``, K >= 128, bfloat16 ``out``, 1 or 2 feature tiles a wave): the kernel whose four waves own feature tiles
+    and share the step's rows through LDS instead of fetching them each."""
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm: weight must be contiguous bfloat16 [N, K]")
     _need(row_scale is None or x is not None, "fused_gemm: a row scale needs x")
@@ -815,8 +815,8 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
               and row_scale.ssq.shape[1] == 16 * (-(-out.shape[0] // 16)), "fused_gemm: the partial sums of squares do not fit the step")
     _need(feature_tiles in (1, 2, 4) and (feature_tiles == 1 or x is not None),
           "fused_gemm: feature_tiles is 1, 2 or 4, and more than 1 needs x")
-    _need(not shared_rows or (x is not None and epilogue == EPI_SWIGLU and feature_tiles in (1, 2)),
-          "fused_gemm: shared_rows takes x, the SwiGLU epilogue and 1 or 2 feature tiles a wave")
+    _need(not shared_rows or (x is not None and out.dtype == torch.bfloat16 and feature_tiles in (1, 2)),
+          "fused_gemm: shared_rows takes x, writes bfloat16 and has 1 or 2 feature tiles a wave")
     N, K = weight.shape
     M = out.shape[0]
     _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()),

@@ -269,7 +269,8 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
                      wide: bool) -> tuple:
     """(whether the library way is faster for this weight at this many rows, the skinny kernel's best number
     of feature tiles; ``wide``: more than one tile may be taken, i.e. the prologue is the plain one; negative:
-    that many a wave of the kernel that shares the rows, which SiLU(gate) * up can come from).  Copies
+    that many a wave of the kernel that shares the rows, which SiLU(gate) * up and the conv step can come from;
+    the two that feed the residual stream take its slabs or none).  Copies
     of the weight are cycled through so that the caches do not hold it, as in a model of many layers."""
     N, K = weight.shape
     device = weight.device
@@ -302,11 +303,12 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
     def shared_rows(tiles):
         def run():
             for w, f in zip(weights, fragments):
-                ops.fused_gemm(w, bias, out, x=x, epilogue=epilogue, feature_tiles=tiles, fragments=f, shared_rows=True)
+                ops.fused_gemm(w, bias, out, x=x, epilogue=epilogue, conv=conv, feature_tiles=tiles, fragments=f,
+                               shared_rows=True)
         return run
 
     times = {tiles: _graph_microseconds(skinny(tiles)) for tiles in (TILE_CHOICES if wide else (1,))}
-    if wide and epilogue == ops.EPI_SWIGLU and rows >= SHARED_ROWS_FROM and K // 32 >= 4:
+    if wide and epilogue != ops.EPI_PLAIN and rows >= SHARED_ROWS_FROM and K // 32 >= 4:
         times.update({-tiles: _graph_microseconds(shared_rows(tiles)) for tiles in TILE_CHOICES[:2]})
     tiles = min(times, key=lambda count: times[count] * (1.0 if count == 1 else 1.0 / TILE_MARGIN))
     return _graph_microseconds(library) < LIBRARY_MARGIN * times[tiles], tiles
@@ -667,7 +669,7 @@ class LayerFusion:
 
     def _tune_all(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict], normed: bool) -> tuple:
         forced = 1 if FORCE_TILES is None else FORCE_TILES
-        if FORCE_SHARED_ROWS and epilogue == ops.EPI_SWIGLU and weight.shape[1] // 32 >= 4:
+        if FORCE_SHARED_ROWS and epilogue != ops.EPI_PLAIN and weight.shape[1] // 32 >= 4:
             forced = -FORCE_SHARED_ROWS
         fixed_tiles = tuple(forced if bucket in self.wide_buckets else 1 for bucket in range(BUCKETS))
         if (not self.general or FORCE_LIBRARY is False
@@ -740,7 +742,7 @@ class LayerFusion:
             # the layer before left the stream prepared for this norm
             u = torch.empty((M, self.in_ld), dtype=torch.bfloat16, device=device)
             ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=epilogue, conv=conv,
-                           feature_tiles=self.tiles_in[bucket], fragments=self.f_in,
+                           fragments=self.f_in, **_tiles(self.tiles_in[bucket], M),
                            **self._behind_the_norm(scaled, self.mixer_scale))
         elif self.library_in[bucket]:
             u = ops.linear(block.mixer_norm.forward(residual), self.w_in, self.b_in)
@@ -751,7 +753,7 @@ class LayerFusion:
             u = torch.empty((M, self.in_ld), dtype=torch.bfloat16, device=device)
             arguments, h_out = self._norm_prologue(residual, M, block.mixer_norm, self.mixer_rms)
             ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=epilogue, conv=conv,
-                           feature_tiles=self.tiles_in[bucket] if "x" in arguments else 1, fragments=self.f_in,
+                           fragments=self.f_in, **(_tiles(self.tiles_in[bucket], M) if "x" in arguments else {}),
                            **arguments)
             if h_out is not None:
                 residual.h, residual.pending = h_out, []

@@ -441,6 +441,7 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
         assert fusion.tiles_out[:6] == (1, 1, 1, tiles, tiles, tiles)
         assert fusion.tiles_down[:6] == (1,) * 6                  # a K of 96 is below that kernel's stage of 128 columns
         assert fusion.tiles_gate_up[:6] == (1, 1, 1, tiles, tiles, tiles) and fusion.library_gate_up[:6] == (False,) * 6
+        assert fusion.tiles_in[:6] == (1, 1, 1, tiles, tiles, tiles) and fusion.library_in[:6] == (False,) * 6
     if library == "tiles":
         fusion = engine.model.blocks[0].fusion
         assert fusion.tiles_in[:6] == fusion.tiles_gate_up[:6] == fusion.tiles_out[:6] == fusion.tiles_down[:6] == (1, 1, 1, 4, 4, 4)

@@ -972,13 +972,12 @@ def test_fused_gemm_swiglu_with_the_rows_shared_by_a_workgroups_waves(ops, M, N,
                                feature_tiles=feature_tiles, fragments=fragments, shared_rows=True)
                 close(got, want, torch.bfloat16, 16.0)
                 close(got, skinny.cpu(), torch.bfloat16, max(2.0, want.float().abs().max().item() / 4))   # an ulp of the largest, between two orders of summation
-    for rows, k, tiles, epilogue in ((16, 256, 1, ops.EPI_SWIGLU), (40, 96, 1, ops.EPI_SWIGLU), (40, 256, 4, ops.EPI_SWIGLU),
-                                     (40, 256, 1, ops.EPI_PLAIN)):
+    for rows, k, tiles in ((16, 256, 1), (40, 96, 1), (40, 256, 4)):
         weight = torch.zeros(32, k, dtype=torch.bfloat16, device=DEV)
-        out = torch.zeros(rows, 16 if epilogue == ops.EPI_SWIGLU else 32, dtype=torch.bfloat16, device=DEV)
+        out = torch.zeros(rows, 16, dtype=torch.bfloat16, device=DEV)
         with pytest.raises((ValueError, RuntimeError)):
-            ops.fused_gemm(weight, None, out, x=torch.zeros(rows, k, dtype=torch.bfloat16, device=DEV), epilogue=epilogue,
-                           feature_tiles=tiles, shared_rows=True)
+            ops.fused_gemm(weight, None, out, x=torch.zeros(rows, k, dtype=torch.bfloat16, device=DEV),
+                           epilogue=ops.EPI_SWIGLU, feature_tiles=tiles, shared_rows=True)
 
 
 def test_fused_gemm_split_with_the_rows_shared_refuses_other_sizes(ops):
@@ -1016,6 +1015,46 @@ def test_fused_gemm_conv_step_of_wide_batches(ops, M, N, K):
         close(got_state, want_state, torch.bfloat16, 8.0)
         unused = [slot for slot in range(M + 3) if slot not in slot_ids.tolist()]
         assert torch.equal(got_state[unused].cpu(), state[unused])
+
+
+@pytest.mark.parametrize("M, N, K", [(24, 200, 1024), (64, 136, 1056), (17, 96, 128), (49, 90, 3072), (40, 1048, 160)])
+def test_fused_gemm_conv_step_with_the_rows_shared_by_a_workgroups_waves(ops, M, N, K):
+    """The conv epilogue of the kernel whose waves own feature tiles and share the rows through LDS: taps 1 to 6,
+    a width that is no multiple of 16 or 4, conv columns that start and end inside a lane's four, with the row
+    scale of a norm left to the product and without, padded output rows; and plain rows in bfloat16 (no conv
+    column) times a scale.  Against the plain reference, rolled tails included."""
+    x = rand(M, K + 8, seed=370, dtype=torch.bfloat16)[:, :K]
+    W, b = rand(N, K, seed=371, scale=0.1, dtype=torch.bfloat16), rand(N, seed=372)
+    lo, hi = 6, N - 21
+    C = hi - lo
+    width, eps = 264, 3e-5
+    ssq = rand(width // 16, 16 * (-(-M // 16)), seed=373).abs() * 2.0
+    for taps, feature_tiles, scaled in ((4, 1, False), (2, 2, True), (6, 1, True), (1, 2, False), (3, 1, True)):
+        state = rand(M + 3, taps - 1, C, seed=374, dtype=torch.bfloat16)
+        slot_ids = torch.randperm(M + 3, generator=torch.Generator().manual_seed(taps))[:M].to(torch.int32)
+        conv = dict(lo=lo, hi=hi, taps=taps, weight=rand(C, taps, seed=375, scale=0.5), bias=rand(C, seed=376, scale=0.1))
+        want_state, got_state = state.clone(), state.clone().to(DEV)
+        want = torch.empty(M, N, dtype=torch.bfloat16)
+        ref_ops.fused_gemm(W, b, want, x=x, epilogue=ref_ops.EPI_CONV, conv=dict(conv, state=want_state, slot_ids=slot_ids),
+                           row_scale=ops.RowScale(ssq, width, eps) if scaled else None)
+        got = torch.full((M, N + 5), float("nan"), dtype=torch.bfloat16, device=DEV)[:, :N]
+        ops.fused_gemm(W.to(DEV), b.to(DEV), got, x=x.to(DEV), epilogue=ops.EPI_CONV, feature_tiles=feature_tiles,
+                       shared_rows=True, fragments=ops.fragment_order(W.to(DEV)) if taps % 2 else None,
+                       row_scale=ops.RowScale(ssq.to(DEV), width, eps) if scaled else None,
+                       conv=dict(lo=lo, hi=hi, taps=taps, weight=conv["weight"].to(DEV), bias=conv["bias"].to(DEV),
+                                 state=got_state, slot_ids=slot_ids.to(DEV)))
+        close(got, want, torch.bfloat16, 8.0)
+        close(got_state, want_state, torch.bfloat16, 8.0)
+        unused = [slot for slot in range(M + 3) if slot not in slot_ids.tolist()]
+        assert torch.equal(got_state[unused].cpu(), state[unused])
+    want = torch.empty(M, N, dtype=torch.bfloat16)
+    ref_ops.fused_gemm(W, b, want, x=x, out_scale=0.7)
+    for feature_tiles in (1, 2):
+        got = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.fused_gemm(W.to(DEV), b.to(DEV), got, x=x.to(DEV), out_scale=0.7, feature_tiles=feature_tiles, shared_rows=True)
+        close(got, want, torch.bfloat16, 8.0)
+    with pytest.raises((ValueError, RuntimeError)):                     # float32 rows are the slabs' entry's
+        ops.fused_gemm(W.to(DEV), None, torch.empty(M, N, device=DEV), x=x.to(DEV), shared_rows=True)
 
 
 @pytest.mark.parametrize("Hq, Hkv, dh, H, P, N, G, page_size, window, rotary, gated", [
