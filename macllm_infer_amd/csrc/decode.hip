@@ -619,7 +619,8 @@ constexpr int SR_LD = SR_CHUNKS * 32 + 8;        // a stage's row in LDS, padded
 template <int MT, int NT, int EPI>
 __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p) {
   __shared__ __align__(16) bf16_t stage[2][MT * 16 * SR_LD];
-  __shared__ float squares[4][MT * 16];
+  constexpr int SQUARE_PARTS = MT <= 4 ? 4 : 2;      // threads that add up a row's sums of squares
+  __shared__ float squares[SQUARE_PARTS][MT * 16];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE, q = lane / 16, r = lane % 16;
   const int tiles = (p.N + 15) / 16;
   const int chunks = p.K / 32;
@@ -700,11 +701,11 @@ __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p
   int slot[MT];                                     // CONV: the rows' conv tails, asked for with the first loads
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) slot[mt] = EPI == EPI_CONV && p.slot_ids ? p.slot_ids[min(mt * 16 + r, p.M - 1)] : 0;
-  if (EPI != EPI_PLAIN && p.ssq_in && tid < 4 * MT * 16) {
-    // the rows' sums of squares, which the workgroups of the product before left in parts: four threads a row
+  if (EPI != EPI_PLAIN && p.ssq_in && tid < SQUARE_PARTS * MT * 16) {
+    // the rows' sums of squares, which the workgroups of the product before left in parts: a few threads a row
     const int row = tid % (MT * 16);
     float sum = 0.f;
-    for (int b = tid / (MT * 16); b < p.ssq_blocks; b += 4) sum += p.ssq_in[(long)b * (MT * 16) + row];
+    for (int b = tid / (MT * 16); b < p.ssq_blocks; b += SQUARE_PARTS) sum += p.ssq_in[(long)b * (MT * 16) + row];
     squares[tid / (MT * 16)][row] = sum;
   }
   lay_rows(rows, 0);
@@ -730,7 +731,9 @@ __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p
     factor[mt] = 1.0f;
     if (EPI != EPI_PLAIN && p.ssq_in) {
       const int m = mt * 16 + r;
-      const float sum = squares[0][m] + squares[1][m] + squares[2][m] + squares[3][m];
+      float sum = 0.f;
+#pragma unroll
+      for (int part = 0; part < SQUARE_PARTS; ++part) sum += squares[part][m];
       factor[mt] = 1.0f / sqrtf(sum / (float)p.ssq_width + p.ssq_eps);
     }
   }
@@ -850,6 +853,23 @@ static int launch_shared_rows(const FusedGemmParams& p, hipStream_t stream, int 
   return 0;
 }
 
+// 17 to 64 rows in tiles of 16; 65 to 128 rows (the slabs only) in 6 or 8 tiles with one tile of features a wave
+template <int EPI>
+static int launch_shared_rows_for(int M, const FusedGemmParams& p, hipStream_t stream, int k_splits, int feature_tiles) {
+  if (M <= 32) return launch_shared_rows<2, EPI>(p, stream, k_splits, feature_tiles);
+  if (M <= 48) return launch_shared_rows<3, EPI>(p, stream, k_splits, feature_tiles);
+  if (M <= 64) return launch_shared_rows<4, EPI>(p, stream, k_splits, feature_tiles);
+  if constexpr (EPI == EPI_PLAIN) {
+    if (feature_tiles != 1) return ERR_UNSUPPORTED_SIZE;
+    const int tiles = (p.N + 15) / 16;
+    const dim3 blocks((tiles + 3) / 4, k_splits);
+    if (M <= 96) shared_rows_gemm_kernel<6, 1, EPI><<<blocks, 4 * WAVE, 0, stream>>>(p);
+    else shared_rows_gemm_kernel<8, 1, EPI><<<blocks, 4 * WAVE, 0, stream>>>(p);
+    return 0;
+  }
+  return ERR_UNSUPPORTED_SIZE;
+}
+
 // Sizes: 1 <= M <= 64, K a multiple of 32; with the NORM prologue the step's M normalized rows must fit
 // 64 KiB of LDS beside the reduction area (16 rows of 1,024, 8 of 3,072).  EPI_SWIGLU wants N a multiple of 16.
 // w_fragments: W is not row-major [N, K] but a copy in the order of the matrix-core fragments,
@@ -879,7 +899,7 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
     return ERR_BAD_ARGUMENT;
   const int MT = (M + 15) / 16;
   if (pro != PRO_NORM && pro != PRO_PLAIN) return ERR_BAD_ARGUMENT;
-  if (fused_gemm_lds(MT, pro, K, M) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  if (!shared_rows && fused_gemm_lds(MT, pro, K, M) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   FusedGemmParams p = {};
   p.h_in = h_in;
   p.delta0 = (const bf16_t*)delta0;
@@ -916,12 +936,8 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
       p.conv_lo = p.conv_hi = 0;
       p.conv_k = 1;
     }
-    code = MT == 2   ? launch_shared_rows<2, EPI_CONV>(p, stream, 1, -feature_tiles)
-           : MT == 3 ? launch_shared_rows<3, EPI_CONV>(p, stream, 1, -feature_tiles)
-                     : launch_shared_rows<4, EPI_CONV>(p, stream, 1, -feature_tiles);
-  } else if (shared_rows && MT == 2) code = launch_shared_rows<2, EPI_SWIGLU>(p, stream, 1, -feature_tiles);
-  else if (shared_rows && MT == 3) code = launch_shared_rows<3, EPI_SWIGLU>(p, stream, 1, -feature_tiles);
-  else if (shared_rows) code = launch_shared_rows<4, EPI_SWIGLU>(p, stream, 1, -feature_tiles);
+    code = launch_shared_rows_for<EPI_CONV>(M, p, stream, 1, -feature_tiles);
+  } else if (shared_rows) code = launch_shared_rows_for<EPI_SWIGLU>(M, p, stream, 1, -feature_tiles);
   else if (MT == 1) code = launch_fused_gemm<1>(p, pro, epi, stream, 1, feature_tiles);
   else if (MT == 2) code = launch_fused_gemm<2>(p, pro, epi, stream, 1, feature_tiles);
   else if (MT == 3) code = launch_fused_gemm<3>(p, pro, epi, stream, 1, feature_tiles);
@@ -966,14 +982,15 @@ extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, cons
   return 0;
 }
 
-// The same slabs for steps of 17 to 64 rows through shared_rows_gemm_kernel: a workgroup's four waves own
-// feature_tiles (1 or 2) tiles of 16 features each and share the step's rows through LDS.  K >= 128.
+// The same slabs for steps of 17 to 128 rows through shared_rows_gemm_kernel: a workgroup's four waves own
+// feature_tiles (1 or 2; 1 beyond 64 rows) tiles of 16 features each and share the step's rows through LDS.
+// K >= 128.
 extern "C" int mi_shared_rows_gemm_split(const void* x, long x_ld, const void* W, const float* bias, int M, int N,
                                          int K, float* partial, int splits, int feature_tiles, int w_fragments,
                                          hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !x || !partial || x_ld < K || x_ld % 8 != 0) return ERR_BAD_ARGUMENT;
   if (feature_tiles != 1 && feature_tiles != 2) return ERR_BAD_ARGUMENT;
-  if (M <= 16 || M > 64 || K % 32 != 0 || K / 32 < SR_CHUNKS || splits < 1 || splits > 64 || K / 32 < splits)
+  if (M <= 16 || M > 128 || K % 32 != 0 || K / 32 < SR_CHUNKS || splits < 1 || splits > 64 || K / 32 < splits)
     return ERR_UNSUPPORTED_SIZE;
   FusedGemmParams p = {};
   p.x = (const bf16_t*)x;
@@ -988,9 +1005,7 @@ extern "C" int mi_shared_rows_gemm_split(const void* x, long x_ld, const void* W
   p.out_f32 = 1;
   p.out_scale = 1.0f;
   p.w_tiled = w_fragments ? 1 : 0;
-  const int code = M <= 32   ? launch_shared_rows<2, EPI_PLAIN>(p, stream, splits, feature_tiles)
-                   : M <= 48 ? launch_shared_rows<3, EPI_PLAIN>(p, stream, splits, feature_tiles)
-                             : launch_shared_rows<4, EPI_PLAIN>(p, stream, splits, feature_tiles);
+  const int code = launch_shared_rows_for<EPI_PLAIN>(M, p, stream, splits, feature_tiles);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;

@@ -78,6 +78,12 @@ SPLIT_MARGIN = 0.92
 # 3,072 x 12,288 one in 21 against 34 and 35.  Written as a negative number of feature tiles (that many a wave).
 # A slab costs the norm behind it a read, counted at SLAB_READ_RATE bytes a microsecond.
 SHARED_ROWS_FROM = 17
+# That kernel takes up to 128 rows (6 or 8 tiles of 16 rows a workgroup), the only one of this engine's products
+# that does: steps of 65 to 128 single tokens, whose products otherwise all go through the library, take its slabs
+# for the output and down projections where a measurement at 128 rows says so (3,072 x 12,288 at 96 / 128 rows: 25
+# and 30 us against the library's 54 and 65; 5,120 x 21,504: 62 and 79 against 144 and 153; SiLU(gate) * up from
+# it is slower than the library's product there and is not offered).
+SHARED_ROWS_MOST = 128
 FORCE_SHARED_ROWS: Optional[int] = None   # tests, with FORCE_SPLIT: this many tiles a wave of that kernel
 SHARED_SPLIT_CHOICES = (4, 8, 16)
 SLAB_READ_RATE = 4.0e6
@@ -227,8 +233,9 @@ def _portion_bucket(rows: int) -> int:
 
 
 def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool, tiles: int) -> tuple:
-    """(slabs, feature tiles): the number of float32 slabs over K with which the skinny kernel beats the way this
-    projection would go otherwise (the library, or the skinny kernel unsplit) at this many rows, or 0."""
+    """(slabs, feature tiles): the number of float32 slabs over K with which the skinny kernel, or the kernel that
+    shares the rows (negative tiles; the only one beyond MAX_ROWS rows), beats the way this projection would go
+    otherwise (the library, or the skinny kernel unsplit) at this many rows, or 0."""
     N, K = weight.shape
     device = weight.device
     copies = max(2, min(64, (512 << 20) // (weight.numel() * 2)))
@@ -250,8 +257,9 @@ def _measure_split(weight: torch.Tensor, bias, rows: int, library: bool, tiles: 
         if K // 32 < slabs:
             continue
         partial = torch.empty((slabs, rows, N), dtype=torch.float32, device=device)
-        ways = [tile for tile in TILE_CHOICES[:2] if slabs in SPLIT_CHOICES]
-        ways += [-tile for tile in TILE_CHOICES[:2] if rows >= shared_from and slabs in SHARED_SPLIT_CHOICES]
+        ways = [tile for tile in TILE_CHOICES[:2] if slabs in SPLIT_CHOICES and rows <= MAX_ROWS]
+        ways += [-tile for tile in TILE_CHOICES[:1 if rows > MAX_ROWS else 2]
+                 if rows >= shared_from and slabs in SHARED_SPLIT_CHOICES]
         for split_tiles in ways:
 
             def split():
@@ -470,6 +478,7 @@ class LayerFusion:
         self.library_out, self.tiles_out = self._tune(self.w_out, self.b_out, ops.EPI_PLAIN)
         # and which of the two that feed the residual stream are split over K instead (steps of more than norm_rows rows)
         self.split_out, self.tiles_out = self._tune_split(self.w_out, self.b_out, self.library_out, self.tiles_out)
+        beyond_out, beyond_down = self._tune_split_beyond(self.w_out, self.b_out), (0, 1)
         # what the skinny kernel reads: a second copy of each matrix in the order of its waves' fragments (one run
         # of 1 KiB a load instead of 64 bytes of each of 16 rows: 15 to 25 % faster); the row-major ones stay for
         # the library and for prompt portions.  A projection that always goes through the library has none.
@@ -480,22 +489,25 @@ class LayerFusion:
             return ops.fragment_order(weight)
 
         self.f_in = fragments(self.w_in, self.library_in, ())
-        self.f_out = fragments(self.w_out, self.library_out, self.split_out)
+        self.f_out = fragments(self.w_out, self.library_out, self.split_out + beyond_out[:1])
         if self.gate_up is not None:
             self.library_gate_up, self.tiles_gate_up = self._tune(self.gate_up.weight, self.gate_up.bias, ops.EPI_SWIGLU,
                                                                   None, self.ffn_rms is not None)
             self.library_down, self.tiles_down = self._tune(self.down.weight, self.down.bias, ops.EPI_PLAIN)
             self.split_down, self.tiles_down = self._tune_split(self.down.weight, self.down.bias, self.library_down,
                                                                 self.tiles_down)
+            beyond_down = self._tune_split_beyond(self.down.weight, self.down.bias)
             self.f_gate_up = fragments(self.gate_up.weight, self.library_gate_up, ())
-            self.f_down = fragments(self.down.weight, self.library_down, self.split_down)
+            self.f_down = fragments(self.down.weight, self.library_down, self.split_down + beyond_down[:1])
         # step sizes at which the norms are left to the projections around them
         self.deferred = _each(False)
         self.deferred = tuple(self._may_defer(self._plan(bucket)) for bucket in range(BUCKETS))
         # and behind the measured step sizes the plan of steps of more than MAX_ROWS single tokens: every projection
-        # through the library, with the mixers' decode kernel between them
-        beyond = dict(library_in=True, library_out=True, library_gate_up=True, library_down=True, split_out=0,
-                      split_down=0, tiles_in=1, tiles_out=1, tiles_gate_up=1, tiles_down=1, deferred=False)
+        # through the library, with the mixers' decode kernel between them; for up to SHARED_ROWS_MOST of them the two
+        # that feed the stream in slabs from the kernel that shares the rows, where that is faster
+        beyond = dict(library_in=True, library_out=True, library_gate_up=True, library_down=True,
+                      split_out=beyond_out[0], split_down=beyond_down[0], tiles_in=1, tiles_out=beyond_out[1],
+                      tiles_gate_up=1, tiles_down=beyond_down[1], deferred=False)
         for name, value in beyond.items():
             if hasattr(self, name):
                 setattr(self, name, getattr(self, name) + (value,))
@@ -546,8 +558,9 @@ class LayerFusion:
     def path_choices(self) -> dict:
         """Which way each projection goes for steps of up to TUNE_ROWS rows, as short strings (S: the skinny
         kernel, L: the library, a number: that many slabs over K), the feature tiles of the skinny kernel (with
-        an r: a wave's, of the kernel that shares the rows), and for portions of up to PAD_ROWS tokens whether
-        the input projection is padded (P)."""
+        an r: a wave's, of the kernel that shares the rows), for portions of up to PAD_ROWS tokens whether
+        the input projection is padded (P), and how the output and down projections of steps of more than
+        MAX_ROWS single tokens go (up to SHARED_ROWS_MOST of them: slabs, or L)."""
         if not self.decode_ok:
             return {}
 
@@ -559,13 +572,17 @@ class LayerFusion:
         def tiled(tiles):
             return "/".join(str(tile) if tile > 0 else f"{-tile}r" for tile in tiles[:BUCKETS])
 
+        def beyond(split):
+            return str(split[BEYOND]) if split[BEYOND] else "L"
+
         out = {"in": way(self.library_in), "out": way(self.library_out, self.split_out),
                "tiles_in": tiled(self.tiles_in), "tiles_out": tiled(self.tiles_out),
                "padded_in": "/".join("P" if pays else "-" for pays in self.padding_pays)}
         if self.gate_up is not None:
             out.update({"gate_up": way(self.library_gate_up), "down": way(self.library_down, self.split_down),
                         "tiles_gate_up": tiled(self.tiles_gate_up), "tiles_down": tiled(self.tiles_down),
-                        "norms": "/".join("D" if deferred else "-" for deferred in self.deferred[:BUCKETS])})
+                        "norms": "/".join("D" if deferred else "-" for deferred in self.deferred[:BUCKETS]),
+                        "beyond_out_down": f"{beyond(self.split_out)}/{beyond(self.split_down)}"})
         return out
 
     def decode_supported(self, step, caches) -> bool:
@@ -666,6 +683,21 @@ class LayerFusion:
             slabs.append(_split_wins[key][0])
             split_tiles.append(_split_wins[key][1])
         return tuple(slabs), tuple(split_tiles)
+
+    def _tune_split_beyond(self, weight: torch.Tensor, bias) -> tuple:
+        """(slabs, feature tiles) for steps of more than MAX_ROWS and up to SHARED_ROWS_MOST single tokens: slabs
+        from the kernel that shares the rows (one tile a wave: -1), or (0, 1) for the library."""
+        chunks = weight.shape[1] // 32
+        if not self.decode_ok or self.hidden % 4 != 0 or FORCE_SPLIT == 0 or chunks < 4:
+            return 0, 1
+        if FORCE_SPLIT:
+            return (FORCE_SPLIT, -1) if FORCE_SHARED_ROWS and chunks >= FORCE_SPLIT else (0, 1)
+        if weight.numel() < LIBRARY_MIN_WEIGHT or not self.measure or FORCE_LIBRARY is not None:
+            return 0, 1
+        key = (tuple(weight.shape), bias is None, BEYOND, True, 1)
+        if key not in _split_wins:
+            _split_wins[key] = _measure_split(weight, bias, SHARED_ROWS_MOST, True, 1)
+        return _split_wins[key]
 
     def _tune_all(self, weight: torch.Tensor, bias, epilogue: int, conv: Optional[dict], normed: bool) -> tuple:
         forced = 1 if FORCE_TILES is None else FORCE_TILES
@@ -821,11 +853,11 @@ class LayerFusion:
             delta = torch.empty((M, self.hidden), dtype=torch.bfloat16, device=x.device)
             ops.fused_gemm_merge(weight, bias, delta, x, attended, fragments)
             return [delta]
-        if slabs:
+        if slabs and (M <= MAX_ROWS or (tiles < 0 and M <= SHARED_ROWS_MOST)):
             partial = torch.empty((slabs, M, self.hidden), dtype=torch.float32, device=x.device)
             ops.fused_gemm_split(weight, bias, x, partial, fragments=fragments, **_tiles(tiles, M))
             return list(partial.unbind(0))
-        if library:
+        if library or M > MAX_ROWS:
             return [ops.linear(x, weight, bias)]
         delta = torch.empty((M, self.hidden), dtype=torch.bfloat16, device=x.device)
         ops.fused_gemm(weight, bias, delta, x=x, feature_tiles=abs(tiles), fragments=fragments)

@@ -397,7 +397,7 @@ def test_decode_graphs_match_eager_steps(tmp_path, name, dtype):
 
 @pytest.mark.parametrize("requests, library", [(24, False), (40, False), (5, True), (24, True), (40, "clock"),
                                                (24, "split"), (40, "split"), (24, "tiles"), (40, "tiles"), (80, False),
-                                               (24, "shared"), (40, "shared"), (57, "shared")])
+                                               (24, "shared"), (40, "shared"), (57, "shared"), (80, "shared"), (128, "shared")])
 def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, requests, library):
     """More single-token lanes than the norm-fused kernels take (16): the block's fast path with
     norms of their own, through graphs of buckets 32 and 64, against the plain model.  ``library``:
@@ -406,7 +406,8 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
     runs on this model's small weights and either outcome must be right; "split": the projections
     that feed the residual stream are split over K into float32 slabs that the next norm adds up; "tiles": a
     workgroup of the skinny kernel owns four tiles of 16 output features, split projections included; "shared":
-    the slabs come from the kernel whose waves own feature tiles and share the step's rows through LDS.  80
+    the slabs come from the kernel whose waves own feature tiles and share the step's rows through LDS (the only
+    one of them that also takes 80 and 128 rows, the output projection of which then comes from it).  80
     requests: more rows than the skinny kernels take; every product through the library, around the mixers'
     decode kernel (not the prompt kernels, which would take them as 80 prompts of one token)."""
     from macllm_infer_amd import Engine, Lane
@@ -434,7 +435,11 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
     if library == "split":
         fusion = engine.model.blocks[0].fusion
         assert fusion.split_out[:6] == (0, 0, 0, 3, 3, 3) and fusion.split_down[:6] == (0, 0, 0, 3, 3, 3)
-    if library == "shared":
+    if library == "shared" and requests > 64:
+        fusion = engine.model.blocks[0].fusion
+        assert fusion.split_out[fused.BEYOND] == 3 and fusion.tiles_out[fused.BEYOND] == -1 and fusion.f_out is not None
+        assert fusion.split_down[fused.BEYOND] == 0               # a K of 64
+    elif library == "shared":
         fusion = engine.model.blocks[0].fusion
         slabs, tiles = (2 if requests == 40 else 3), (-2 if requests == 24 else -1)
         assert fusion.split_out[:6] == fusion.split_down[:6] == (0, 0, 0, slabs, slabs, slabs)
@@ -532,13 +537,15 @@ def test_fixed_paths_take_no_measurement(tmp_path, monkeypatch):
                         max_active_sequences=24, measured_paths=measured)
         choices = engine.path_choices()
         assert set(choices) == {"in", "out", "gate_up", "down", "tiles_in", "tiles_out", "tiles_gate_up", "tiles_down",
-                                "padded_in", "norms"}
-        assert all(len(value.split("/")) == (5 if name == "padded_in" else 6) for name, value in choices.items())
+                                "padded_in", "norms", "beyond_out_down"}
+        assert all(len(value.split("/")) == {"padded_in": 5, "beyond_out_down": 2}.get(name, 6)
+                   for name, value in choices.items())
         assert bool(fused._chain_wins) == measured          # the layers' chain was timed too, once for the shape
         if not measured:
             assert choices["in"] == choices["out"] == choices["gate_up"] == choices["down"] == "S/S/S/S/S/S"
             assert choices["norms"] == "D/D/D/D/D/D"
             assert choices["tiles_in"] == choices["tiles_down"] == "1/1/1/1/1/1" and choices["padded_in"] == "-/-/-/-/-"
+            assert choices["beyond_out_down"] == "L/L"
         for index in prompts:
             engine.add_request(index)
         engine.step([Lane(index, tokens[:-1], []) for index, tokens in prompts.items()])

@@ -924,19 +924,27 @@ def test_fused_gemm_split_over_k_and_the_norm_that_adds_its_slabs(ops, M, N, K, 
 
 
 @pytest.mark.parametrize("M, N, K, S", [(64, 1024, 2048, 8), (33, 100, 2048, 16), (48, 138, 1056, 3), (49, 72, 3072, 5),
-                                        (64, 50, 128, 1), (40, 272, 288, 8), (57, 16, 4672, 64), (17, 40, 160, 2), (32, 264, 1024, 4)])
+                                        (64, 50, 128, 1), (40, 272, 288, 8), (57, 16, 4672, 64), (17, 40, 160, 2), (32, 264, 1024, 4),
+                                        (65, 100, 160, 2), (96, 272, 1056, 4), (113, 48, 4672, 16), (128, 1024, 2048, 8)])
 def test_fused_gemm_split_with_the_rows_shared_by_a_workgroups_waves(ops, M, N, K, S):
     """The slabs of the kernel whose waves own feature tiles and share the rows through LDS: widths with a last
     tile of fewer than 16 features and rows that are no multiple of four floats, a K whose last stage is short or
     is moved back over chunks already multiplied, more slabs than stages, slabs without chunks, row-major
-    weights and the fragment order, against the plain product per slab and the unshared kernel's slabs."""
+    weights and the fragment order, against the plain product per slab and the unshared kernel's slabs; 65 to
+    128 rows (6 and 8 tiles of rows, one tile of features a wave), which only this kernel takes."""
     x = rand(M, K + 24, seed=350, dtype=torch.bfloat16)[:, :K]
     W, b = rand(N, K, seed=351, scale=0.1, dtype=torch.bfloat16), rand(N, seed=352)
     want = torch.zeros(S, M, N)
     ref_ops.fused_gemm_split(W, b, x, want)
     other = torch.full((S, M, N), float("nan"), device=DEV)
-    ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), other)
-    for feature_tiles in (1, 2):
+    if M <= 64:
+        ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), other)
+    else:
+        other = want.to(DEV)
+        with pytest.raises((ValueError, RuntimeError)):
+            ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), torch.empty((S, M, N), device=DEV), feature_tiles=2,
+                                 shared_rows=True)
+    for feature_tiles in (1, 2) if M <= 64 else (1,):
         got = torch.full((S, M, N), float("nan"), device=DEV)
         ops.fused_gemm_split(W.to(DEV), b.to(DEV), x.to(DEV), got, feature_tiles=feature_tiles, shared_rows=True)
         close(got, want, torch.float32, 50.0)
@@ -981,9 +989,9 @@ def test_fused_gemm_swiglu_with_the_rows_shared_by_a_workgroups_waves(ops, M, N,
 
 
 def test_fused_gemm_split_with_the_rows_shared_refuses_other_sizes(ops):
-    """16 rows or fewer and more than 64, a K below one stage of 128 columns, four tiles a wave: an error,
+    """16 rows or fewer and more than 128, a K below one stage of 128 columns, four tiles a wave: an error,
     and nothing written."""
-    for rows, K, tiles in ((16, 256, 1), (65, 256, 1), (40, 96, 1), (40, 256, 4)):
+    for rows, K, tiles in ((16, 256, 1), (129, 256, 1), (40, 96, 1), (40, 256, 4)):
         W = torch.zeros(48, K, dtype=torch.bfloat16, device=DEV)
         x = torch.zeros(rows, K, dtype=torch.bfloat16, device=DEV)
         partial = torch.full((1, rows, 48), 7.0, device=DEV)
