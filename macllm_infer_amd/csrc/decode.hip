@@ -1,6 +1,6 @@
 // Fused kernels for decode steps in bfloat16: every lane of the batch holds one token, the
 // batch is small (M <= 64 rows), and a step is bound by weight reads and by the latency of
-// each dependent kernel.  Two kernels cover a layer's hot path:
+// each dependent kernel.  Three kernels cover a layer's hot path:
 //
 //   fused_gemm : out[M, N] = epilogue( prologue(x)[M, K] . W[N, K]^T + bias )
 //       prologue  NORM : x = (h + delta0 + delta1) / sqrt(mean(.^2) + eps) * w   (residual add
@@ -26,6 +26,11 @@
 //     many rows: the rows of x then cross the caches once per block and not once per 16 features); its
 //     waves split K and feed the matrix cores (v_mfma_f32_16x16x32_bf16: A = 16 weight rows x 32 k,
 //     B = 16 batch rows x 32 k, both contiguous in k), then sum their partial tiles through LDS.
+//
+//   shared_rows_gemm : the same product behind the plain prologue for steps of 17 rows and more, where the
+//     rows of x, fetched by every wave, cross the caches several times as often as the weights: a workgroup's
+//     four waves own tiles of 16 features each and walk the same columns, which go through LDS once a
+//     workgroup.  Epilogues: float32 slabs over K (to 128 rows), SWIGLU, CONV or plain bfloat16 rows.
 //
 //   mixer_decode : one launch with two kinds of blocks
 //       attention blocks: one per (token, kv head): rotation of q and of the new key, the write

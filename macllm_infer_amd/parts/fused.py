@@ -30,8 +30,10 @@ has the story).
 A large weight goes through the BLAS library instead where that is faster (``LIBRARY_MIN_WEIGHT``); the
 conv step and SiLU(g)*u then run as kernels of their own.  Which way each product goes is measured per step
 size when the layer is built, and the layer's whole plan once more over a chain of layers when the model is
-(``CHAIN_LAYERS``).  Steps of more single tokens than the skinny kernels take rows run every product through
-the library around the same ``mixer_decode``.
+(``CHAIN_LAYERS``).  From 17 rows on a second kernel of this engine's own is measured with them, whose waves
+share the step's rows (``SHARED_ROWS_FROM``).  Steps of more single tokens than the skinny kernels take rows run
+their products through the library around the same ``mixer_decode``, but for 3 and 5 in steps of up to 128 rows
+where that second kernel's slabs are faster (``SHARED_ROWS_MOST``).
 
 The fusion belongs to the arrangement (``register_fusion``), which knows its parts; the parts stay as they
 are.  It is built only for bfloat16 weights and sizes the kernels cover; otherwise the block runs part by
