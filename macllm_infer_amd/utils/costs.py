@@ -101,15 +101,20 @@ def total(costs: Dict[str, Cost]) -> Cost:
 
 
 # Which kernels do the work of which group (name patterns of this package's kernels and of the BLAS library's).
-# fused_gemm_kernel<row tiles, prologue (0 norm, 1 plain), epilogue (0 plain, 1 SiLU(g)*u, 2 conv), ...>
+# fused_gemm_kernel<row tiles, prologue (0 norm, 1 plain, 2 merge of the attention runs), epilogue (0 plain,
+# 1 SiLU(g)*u, 2 conv, 3 add to the residual stream), ...>; shared_rows_gemm_kernel<row tiles, feature tiles a
+# wave, epilogue (0 float32 slabs, 1 SiLU(g)*u, 2 conv or plain rows)>.  A product with the plain epilogue that is
+# launched once a step is the output head; launched more often, an output or down projection (the library's
+# products carry no such mark and stay with the other kernels).
 DECODE_GROUPS: List[Tuple[str, str]] = [
     (r"mixer_decode_kernel|mixer_merge_kernel|decode_attention_kernel|decode_merge_kernel|ssm_scan_kernel|conv_step_kernel|"
      r"gate_norm_kernel|rope_kv_store_kernel|paged_attention_kernel", "mixers"),
-    (r"fused_gemm_kernel<\d+, \d+, 2", "input projections"),
-    (r"fused_gemm_kernel<\d+, \d+, 1", "gate and up projections"),
-    (r"fused_gemm_kernel<\d+, 1, 0|fused_gemm_split_kernel", "output projections + down projections"),
-    (r"fused_gemm_kernel<\d+, 0, 0", "output head"),
+    (r"fused_gemm_kernel<\d+, \d+, 2|shared_rows_gemm_kernel<\d+, \d+, 2", "input projections"),
+    (r"fused_gemm_kernel<\d+, \d+, 1|shared_rows_gemm_kernel<\d+, \d+, 1", "gate and up projections"),
+    (r"fused_gemm_kernel<\d+, \d+, 3|fused_gemm_kernel<\d+, 2, 0|shared_rows_gemm_kernel<\d+, \d+, 0|fused_gemm_split_kernel",
+     "output projections + down projections"),
 ]
+PLAIN_PRODUCT = r"fused_gemm_kernel<\d+, [01], 0"
 PREFILL_GROUPS: List[Tuple[str, str]] = [
     (r"^Cijk_|gemm_f32_kernel", "matrix products"),
     (r"prefill_attention|paged_attention_kernel|rope_kv_store_kernel", "attention"),
@@ -117,10 +122,14 @@ PREFILL_GROUPS: List[Tuple[str, str]] = [
 ]
 
 
-def group_of(kernel: str, groups: List[Tuple[str, str]]) -> Optional[str]:
+def group_of(kernel: str, groups: List[Tuple[str, str]], calls: int = 2) -> Optional[str]:
+    """The group of a kernel by its name and, for the products that carry no other mark, by how often a step
+    launches it (``calls``)."""
     for pattern, name in groups:
         if re.search(pattern, kernel):
             return name
+    if groups is DECODE_GROUPS and re.search(PLAIN_PRODUCT, kernel):
+        return "output head" if calls == 1 else "output projections + down projections"
     return None
 
 

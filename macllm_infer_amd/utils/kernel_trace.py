@@ -50,8 +50,11 @@ def roofline_table(step, spec, batch, context, prefill, dtype: str) -> None:
     else:
         model, groups = costs.decode_step_costs(spec, batch, context, element), costs.DECODE_GROUPS
     busy = defaultdict(float)
+    calls = defaultdict(int)
+    for name, _, _ in step:
+        calls[name] += 1
     for name, start, end in step:
-        busy[costs.group_of(name, groups) or "(other kernels)"] += (end - start) * 1e-9
+        busy[costs.group_of(name, groups, calls[name]) or "(other kernels)"] += (end - start) * 1e-9
     print()
     print(f"{'group of kernels':44s} {'busy us':>9s} {'read MB':>9s} {'write MB':>9s} {'GB/s':>8s} {'of 8 TB/s':>9s} "
           f"{'GFLOP':>9s} {'TFLOP/s':>8s} {'of peak':>8s}")

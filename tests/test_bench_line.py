@@ -106,6 +106,13 @@ def test_costs_of_the_headline_step_are_the_ones_worked_out_by_hand():
     assert costs.group_of("void fused_gemm_kernel<1, 0, 2, 4, 1>(FusedGemmParams)", costs.DECODE_GROUPS) == "input projections"
     assert costs.group_of("void fused_gemm_kernel<1, 1, 0, 8, 1>(FusedGemmParams)", costs.DECODE_GROUPS) \
         == "output projections + down projections"
+    assert costs.group_of("void fused_gemm_kernel<1, 1, 0, 8, 1>(FusedGemmParams)", costs.DECODE_GROUPS, calls=1) == "output head"
+    for kernel in ("void fused_gemm_kernel<4, 1, 3, 8, 1>(FusedGemmParams)", "void fused_gemm_kernel<1, 2, 0, 8, 1>(FusedGemmParams)",
+                   "void shared_rows_gemm_kernel<4, 1, 0>(FusedGemmParams)"):
+        assert costs.group_of(kernel, costs.DECODE_GROUPS, calls=1) == "output projections + down projections"
+    assert costs.group_of("void shared_rows_gemm_kernel<3, 2, 1>(FusedGemmParams)", costs.DECODE_GROUPS) == "gate and up projections"
+    assert costs.group_of("void shared_rows_gemm_kernel<3, 2, 2>(FusedGemmParams)", costs.DECODE_GROUPS) == "input projections"
+    assert costs.group_of("Cijk_Alik_Bljk_BBS_BH", costs.DECODE_GROUPS) is None
     assert costs.merged(step, "output projections + down projections").read == pytest.approx(302.0e6, rel=1e-3)
 
 
