@@ -27,8 +27,8 @@
 //     waves split K and feed the matrix cores (v_mfma_f32_16x16x32_bf16: A = 16 weight rows x 32 k,
 //     B = 16 batch rows x 32 k, both contiguous in k), then sum their partial tiles through LDS.
 //
-//   shared_rows_gemm : the same product behind the plain prologue for steps of 17 rows and more, where the
-//     rows of x, fetched by every wave, cross the caches several times as often as the weights: a workgroup's
+//   shared_rows_gemm : the same product behind the plain prologue where the rows of x, fetched by every wave
+//     of fused_gemm, cross the caches as often as the weights (16 rows) or several times as often: a workgroup's
 //     four waves own tiles of 16 features each and walk the same columns, which go through LDS once a
 //     workgroup.  Epilogues: float32 slabs over K (to 128 rows), SWIGLU, CONV or plain bfloat16 rows.
 //
@@ -858,9 +858,10 @@ static int launch_shared_rows(const FusedGemmParams& p, hipStream_t stream, int 
   return 0;
 }
 
-// 17 to 64 rows in tiles of 16; 65 to 128 rows (the slabs only) in 6 or 8 tiles with one tile of features a wave
+// up to 64 rows in tiles of 16; 65 to 128 rows (the slabs only) in 6 or 8 tiles with one tile of features a wave
 template <int EPI>
 static int launch_shared_rows_for(int M, const FusedGemmParams& p, hipStream_t stream, int k_splits, int feature_tiles) {
+  if (M <= 16) return launch_shared_rows<1, EPI>(p, stream, k_splits, feature_tiles);
   if (M <= 32) return launch_shared_rows<2, EPI>(p, stream, k_splits, feature_tiles);
   if (M <= 48) return launch_shared_rows<3, EPI>(p, stream, k_splits, feature_tiles);
   if (M <= 64) return launch_shared_rows<4, EPI>(p, stream, k_splits, feature_tiles);
@@ -880,7 +881,7 @@ static int launch_shared_rows_for(int M, const FusedGemmParams& p, hipStream_t s
 // w_fragments: W is not row-major [N, K] but a copy in the order of the matrix-core fragments,
 // [ceil(N / 16), K / 32, 4, 16, 8] with element [n, c, q, r, j] = W[16 n + r, 32 c + 8 q + j] (rows past N zero):
 // what a wave asks for at once is then one run of 1 KiB instead of 64 bytes of each of 16 rows, which
-// streams 15 to 25 % faster.  feature_tiles -1 or -2 (17 to 64 rows, K >= 128, plain prologue, bfloat16 out): that
+// streams 15 to 25 % faster.  feature_tiles -1 or -2 (K >= 128, plain prologue, bfloat16 out): that
 // many tiles a wave of the kernel whose waves share the step's rows through LDS.
 extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* delta0, const void* delta1,
                              float* h_out, const float* norm_w, float eps, const void* x, long x_ld,
@@ -895,7 +896,7 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
   if (shared_rows && (feature_tiles < -2 || pro != PRO_PLAIN || out_f32)) return ERR_BAD_ARGUMENT;
   if (!shared_rows && feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0) return ERR_UNSUPPORTED_SIZE;
-  if (shared_rows && (M <= 16 || K / 32 < SR_CHUNKS)) return ERR_UNSUPPORTED_SIZE;
+  if (shared_rows && K / 32 < SR_CHUNKS) return ERR_UNSUPPORTED_SIZE;
   if (pro == PRO_NORM && (!h_in || !norm_w || h_out == h_in)) return ERR_BAD_ARGUMENT;
   if (pro == PRO_PLAIN && (!x || x_ld < K || x_ld % 8 != 0)) return ERR_BAD_ARGUMENT;
   if (epi == EPI_SWIGLU && (N % 16 != 0 || out_f32)) return ERR_BAD_ARGUMENT;
@@ -987,7 +988,7 @@ extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, cons
   return 0;
 }
 
-// The same slabs for steps of 17 to 128 rows through shared_rows_gemm_kernel: a workgroup's four waves own
+// The same slabs for steps of up to 128 rows through shared_rows_gemm_kernel: a workgroup's four waves own
 // feature_tiles (1 or 2; 1 beyond 64 rows) tiles of 16 features each and share the step's rows through LDS.
 // K >= 128.
 extern "C" int mi_shared_rows_gemm_split(const void* x, long x_ld, const void* W, const float* bias, int M, int N,
@@ -995,7 +996,7 @@ extern "C" int mi_shared_rows_gemm_split(const void* x, long x_ld, const void* W
                                          hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !x || !partial || x_ld < K || x_ld % 8 != 0) return ERR_BAD_ARGUMENT;
   if (feature_tiles != 1 && feature_tiles != 2) return ERR_BAD_ARGUMENT;
-  if (M <= 16 || M > 128 || K % 32 != 0 || K / 32 < SR_CHUNKS || splits < 1 || splits > 64 || K / 32 < splits)
+  if (M > 128 || K % 32 != 0 || K / 32 < SR_CHUNKS || splits < 1 || splits > 64 || K / 32 < splits)
     return ERR_UNSUPPORTED_SIZE;
   FusedGemmParams p = {};
   p.x = (const bf16_t*)x;

@@ -766,7 +766,7 @@ def fused_gemm_split(weight: torch.Tensor, bias: Optional[torch.Tensor], x: torc
     ``partial`` (float32 [S, M, N], contiguous) receives the sums over the s-th run of K, the bias
     in slab 0.  The product is the sum of the slabs (``add_partials_rmsnorm`` adds them to the
     residual stream): many rows, a long K and few output features fill the GPU this way.
-    ``shared_rows`` (17 to 64 rows, K >= 128, 1 or 2 feature tiles a wave): the kernel whose four waves
+    ``shared_rows`` (up to 128 rows, one feature tile a wave beyond 64; K >= 128): the kernel whose four waves
     share the step's rows through LDS instead of fetching them each."""
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm_split: weight must be contiguous bfloat16 [N, K]")
@@ -804,8 +804,8 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
     steps of many rows gain from more.  ``fragments``: ``fragment_order(weight)``, read instead of the weight.
     ``row_scale`` (with ``x``): x holds rows times a norm's weight that are not divided by their root mean
     square yet; the sums of row m are multiplied by 1 / sqrt(sum of squares of the row / width + eps) before the
-    bias, from the partial sums of squares that ``fused_gemm_residual`` left.  ``shared_rows`` (17 to 64 rows of
-    ``x``, K >= 128, bfloat16 ``out``, 1 or 2 feature tiles a wave): the kernel whose four waves own feature tiles
+    bias, from the partial sums of squares that ``fused_gemm_residual`` left.  ``shared_rows`` (``x``, K >= 128,
+    bfloat16 ``out``, 1 or 2 feature tiles a wave): the kernel whose four waves own feature tiles
     and share the step's rows through LDS instead of fetching them each."""
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm: weight must be contiguous bfloat16 [N, K]")

@@ -30,8 +30,8 @@ has the story).
 A large weight goes through the BLAS library instead where that is faster (``LIBRARY_MIN_WEIGHT``); the
 conv step and SiLU(g)*u then run as kernels of their own.  Which way each product goes is measured per step
 size when the layer is built, and the layer's whole plan once more over a chain of layers when the model is
-(``CHAIN_LAYERS``).  From 17 rows on a second kernel of this engine's own is measured with them, whose waves
-share the step's rows (``SHARED_ROWS_FROM``).  Steps of more single tokens than the skinny kernels take rows run
+(``CHAIN_LAYERS``).  A second kernel of this engine's own is measured with them, whose waves share the step's
+rows (``SHARED_ROWS_FROM``).  Steps of more single tokens than the skinny kernels take rows run
 their products through the library around the same ``mixer_decode``, but for 3 and 5 in steps of up to 128 rows
 where that second kernel's slabs are faster (``SHARED_ROWS_MOST``).
 
@@ -74,11 +74,16 @@ _library_wins: Dict[tuple, tuple] = {}
 # at build like the library; the split has to win by SPLIT_MARGIN.
 SPLIT_CHOICES = (2, 4, 8)
 SPLIT_MARGIN = 0.92
-# From 17 rows on the slabs can also come from the kernel whose four waves own feature tiles and share the step's
-# rows through LDS (in the skinny kernel every wave fetches rows of its own, four times the bytes of the weights
-# at 64 rows): a 5,120 x 21,504 weight at 64 rows in 52 us with 8 slabs, against 93 and the library's 133; a
-# 3,072 x 12,288 one in 21 against 34 and 35.  Written as a negative number of feature tiles (that many a wave).
-# A slab costs the norm behind it a read, counted at SLAB_READ_RATE bytes a microsecond.
+# The slabs can also come from the kernel whose four waves own feature tiles and share the step's rows through
+# LDS (in the skinny kernel every wave fetches rows of its own: as many bytes as the weights at 16 rows, four
+# times as many at 64): a 5,120 x 21,504 weight at 64 rows in 52 us with 8 slabs, against 93 and the library's 133,
+# at 8 rows in 43 against 50; a 3,072 x 12,288 one at 64 rows in 21 against 34 and 35.  Written as a negative
+# number of feature tiles (that many a wave).  A slab costs the norm behind it a read, counted at SLAB_READ_RATE
+# bytes a microsecond.  The kernel takes any number of rows, but is offered to the measurements from
+# SHARED_ROWS_FROM rows on: below, what it gains on a product alone (the second weight above at 16 rows: 16 us in 8
+# slabs against 22) a whole step loses again, with the norms as kernels of their own behind the slabs (the 7B shape
+# at 8 / 16 rows: 5.01 / 6.46 ms a step with it, 4.96 / 6.25 without; the 34B shape at 8 rows 6.27 against 6.08 for
+# 24 layers).
 SHARED_ROWS_FROM = 17
 # That kernel takes up to 128 rows (6 or 8 tiles of 16 rows a workgroup), the only one of this engine's products
 # that does: steps of 65 to 128 single tokens, whose products otherwise all go through the library, take its slabs
@@ -776,7 +781,7 @@ class LayerFusion:
             # the layer before left the stream prepared for this norm
             u = torch.empty((M, self.in_ld), dtype=torch.bfloat16, device=device)
             ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=epilogue, conv=conv,
-                           fragments=self.f_in, **_tiles(self.tiles_in[bucket], M),
+                           fragments=self.f_in, **_tiles(self.tiles_in[bucket]),
                            **self._behind_the_norm(scaled, self.mixer_scale))
         elif self.library_in[bucket]:
             u = ops.linear(block.mixer_norm.forward(residual), self.w_in, self.b_in)
@@ -787,7 +792,7 @@ class LayerFusion:
             u = torch.empty((M, self.in_ld), dtype=torch.bfloat16, device=device)
             arguments, h_out = self._norm_prologue(residual, M, block.mixer_norm, self.mixer_rms)
             ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=epilogue, conv=conv,
-                           fragments=self.f_in, **(_tiles(self.tiles_in[bucket], M) if "x" in arguments else {}),
+                           fragments=self.f_in, **(_tiles(self.tiles_in[bucket]) if "x" in arguments else {}),
                            **arguments)
             if h_out is not None:
                 residual.h, residual.pending = h_out, []
@@ -813,14 +818,14 @@ class LayerFusion:
             scaled = None
         if scaled is not None:
             ops.fused_gemm(self.gate_up.weight, self.gate_up.bias, activated, epilogue=ops.EPI_SWIGLU,
-                           fragments=self.f_gate_up, **_tiles(self.tiles_gate_up[bucket], M),
+                           fragments=self.f_gate_up, **_tiles(self.tiles_gate_up[bucket]),
                            **self._behind_the_norm(scaled, self.ffn_scale))
         elif self.library_gate_up[bucket]:
             ops.swiglu(ops.linear(block.ffn_norm.forward(residual), self.gate_up.weight, self.gate_up.bias), activated, 8)
         else:
             arguments, h_out = self._norm_prologue(residual, M, block.ffn_norm, self.ffn_rms)
             ops.fused_gemm(self.gate_up.weight, self.gate_up.bias, activated, epilogue=ops.EPI_SWIGLU,
-                           fragments=self.f_gate_up, **(_tiles(self.tiles_gate_up[bucket], M) if "x" in arguments else {}),
+                           fragments=self.f_gate_up, **(_tiles(self.tiles_gate_up[bucket]) if "x" in arguments else {}),
                            **arguments)
             if h_out is not None:
                 residual.h, residual.pending = h_out, []
@@ -857,7 +862,7 @@ class LayerFusion:
             return [delta]
         if slabs and (M <= MAX_ROWS or (tiles < 0 and M <= SHARED_ROWS_MOST)):
             partial = torch.empty((slabs, M, self.hidden), dtype=torch.float32, device=x.device)
-            ops.fused_gemm_split(weight, bias, x, partial, fragments=fragments, **_tiles(tiles, M))
+            ops.fused_gemm_split(weight, bias, x, partial, fragments=fragments, **_tiles(tiles))
             return list(partial.unbind(0))
         if library or M > MAX_ROWS:
             return [ops.linear(x, weight, bias)]
@@ -866,10 +871,10 @@ class LayerFusion:
         return [delta]
 
 
-def _tiles(tiles: int, rows: int) -> dict:
+def _tiles(tiles: int) -> dict:
     """A plan's number of feature tiles as the products' arguments: negative, that many a wave of the kernel that
-    shares the rows (steps of fewer rows than it takes: as many a workgroup of the skinny kernel)."""
-    return dict(feature_tiles=abs(tiles), shared_rows=tiles < 0 and rows >= SHARED_ROWS_FROM)
+    shares the rows."""
+    return dict(feature_tiles=abs(tiles), shared_rows=tiles < 0)
 
 
 def _rms_prologue(norm):

@@ -397,7 +397,8 @@ def test_decode_graphs_match_eager_steps(tmp_path, name, dtype):
 
 @pytest.mark.parametrize("requests, library", [(24, False), (40, False), (5, True), (24, True), (40, "clock"),
                                                (24, "split"), (40, "split"), (24, "tiles"), (40, "tiles"), (80, False),
-                                               (24, "shared"), (40, "shared"), (57, "shared"), (80, "shared"), (128, "shared")])
+                                               (24, "shared"), (40, "shared"), (57, "shared"), (80, "shared"), (128, "shared"),
+                                               (5, "shared"), (14, "shared")])
 def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, requests, library):
     """More single-token lanes than the norm-fused kernels take (16): the block's fast path with
     norms of their own, through graphs of buckets 32 and 64, against the plain model.  ``library``:
@@ -425,7 +426,9 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
     elif library:
         monkeypatch.setattr(fused, "FORCE_LIBRARY", True)
     # (the library takes rows whose width is a multiple of 8 elements: configuration D's; C's are not)
-    folder = tiny_configs.make_model_dir("D" if library is True or requests > 64 else "C", tmp_path, torch.bfloat16)
+    # (and every step size of D runs its norms as kernels, so that the forced ways apply to steps of 5 and 14 rows too)
+    wide = library is True or requests > 64 or (library == "shared" and requests < 16)
+    folder = tiny_configs.make_model_dir("D" if wide else "C", tmp_path, torch.bfloat16)
     cfg, tensors = plain_impl.load_model_dir(folder)
     engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * (requests + 1),
                     max_active_sequences=requests + 1)
@@ -435,10 +438,11 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
     if library == "split":
         fusion = engine.model.blocks[0].fusion
         assert fusion.split_out[:6] == (0, 0, 0, 3, 3, 3) and fusion.split_down[:6] == (0, 0, 0, 3, 3, 3)
-    if library == "shared" and requests > 64:
+    if library == "shared" and wide:
         fusion = engine.model.blocks[0].fusion
         assert fusion.split_out[fused.BEYOND] == 3 and fusion.tiles_out[fused.BEYOND] == -1 and fusion.f_out is not None
         assert fusion.split_down[fused.BEYOND] == 0               # a K of 64
+        assert fusion.split_out[:6] == (3,) * 6 and fusion.tiles_out[:6] == fusion.tiles_gate_up[:6] == (-1,) * 6
     elif library == "shared":
         fusion = engine.model.blocks[0].fusion
         slabs, tiles = (2 if requests == 40 else 3), (-2 if requests == 24 else -1)
@@ -460,7 +464,7 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
         logits = engine.step([Lane(index, [tokens[len(tokens) - 6 + turn]], [0]) for index, tokens in prompts.items()])
         for row, index in enumerate(prompts):
             got[index].append(logits[row].float().cpu())
-    assert {lanes for lanes, _ in engine.graphs._graphs} == {8 if requests <= 8 else 32 if requests <= 32 else 64 if requests <= 64 else 128}
+    assert {lanes for lanes, _ in engine.graphs._graphs} == {8 if requests <= 8 else 16 if requests <= 16 else 32 if requests <= 32 else 64 if requests <= 64 else 128}
     if requests > 64:
         fusion = engine.model.blocks[0].fusion
         assert fusion.general and fusion.library_in[fused.BEYOND] and fusion.library_down[fused.BEYOND]

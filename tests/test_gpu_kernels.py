@@ -925,7 +925,8 @@ def test_fused_gemm_split_over_k_and_the_norm_that_adds_its_slabs(ops, M, N, K, 
 
 @pytest.mark.parametrize("M, N, K, S", [(64, 1024, 2048, 8), (33, 100, 2048, 16), (48, 138, 1056, 3), (49, 72, 3072, 5),
                                         (64, 50, 128, 1), (40, 272, 288, 8), (57, 16, 4672, 64), (17, 40, 160, 2), (32, 264, 1024, 4),
-                                        (65, 100, 160, 2), (96, 272, 1056, 4), (113, 48, 4672, 16), (128, 1024, 2048, 8)])
+                                        (65, 100, 160, 2), (96, 272, 1056, 4), (113, 48, 4672, 16), (128, 1024, 2048, 8),
+                                        (1, 72, 160, 3), (8, 1024, 2048, 8), (16, 100, 1056, 4), (5, 40, 128, 1)])
 def test_fused_gemm_split_with_the_rows_shared_by_a_workgroups_waves(ops, M, N, K, S):
     """The slabs of the kernel whose waves own feature tiles and share the rows through LDS: widths with a last
     tile of fewer than 16 features and rows that are no multiple of four floats, a K whose last stage is short or
@@ -957,7 +958,8 @@ def test_fused_gemm_split_with_the_rows_shared_by_a_workgroups_waves(ops, M, N, 
 
 
 @pytest.mark.parametrize("M, N, K, scaled", [(64, 1024, 2048, False), (33, 112, 1056, True), (48, 272, 128, True),
-                                             (17, 48, 288, False), (57, 4112, 160, True), (32, 16, 4672, True)])
+                                             (17, 48, 288, False), (57, 4112, 160, True), (32, 16, 4672, True),
+                                             (1, 112, 160, True), (8, 1024, 2048, False), (16, 272, 1056, True)])
 def test_fused_gemm_swiglu_with_the_rows_shared_by_a_workgroups_waves(ops, M, N, K, scaled):
     """SiLU(gate) * up from the kernel whose waves own feature tiles and share the rows through LDS, with and
     without the row scale of a norm left to it, one and two tiles a wave, row-major weights and the fragment
@@ -980,7 +982,7 @@ def test_fused_gemm_swiglu_with_the_rows_shared_by_a_workgroups_waves(ops, M, N,
                                feature_tiles=feature_tiles, fragments=fragments, shared_rows=True)
                 close(got, want, torch.bfloat16, 16.0)
                 close(got, skinny.cpu(), torch.bfloat16, max(2.0, want.float().abs().max().item() / 4))   # an ulp of the largest, between two orders of summation
-    for rows, k, tiles in ((16, 256, 1), (40, 96, 1), (40, 256, 4)):
+    for rows, k, tiles in ((65, 256, 1), (40, 96, 1), (40, 256, 4)):
         weight = torch.zeros(32, k, dtype=torch.bfloat16, device=DEV)
         out = torch.zeros(rows, 16, dtype=torch.bfloat16, device=DEV)
         with pytest.raises((ValueError, RuntimeError)):
@@ -989,9 +991,9 @@ def test_fused_gemm_swiglu_with_the_rows_shared_by_a_workgroups_waves(ops, M, N,
 
 
 def test_fused_gemm_split_with_the_rows_shared_refuses_other_sizes(ops):
-    """16 rows or fewer and more than 128, a K below one stage of 128 columns, four tiles a wave: an error,
-    and nothing written."""
-    for rows, K, tiles in ((16, 256, 1), (129, 256, 1), (40, 96, 1), (40, 256, 4)):
+    """More than 128 rows, a K below one stage of 128 columns, four tiles a wave: an error, and nothing
+    written."""
+    for rows, K, tiles in ((129, 256, 1), (40, 96, 1), (40, 256, 4)):
         W = torch.zeros(48, K, dtype=torch.bfloat16, device=DEV)
         x = torch.zeros(rows, K, dtype=torch.bfloat16, device=DEV)
         partial = torch.full((1, rows, 48), 7.0, device=DEV)
@@ -1025,7 +1027,8 @@ def test_fused_gemm_conv_step_of_wide_batches(ops, M, N, K):
         assert torch.equal(got_state[unused].cpu(), state[unused])
 
 
-@pytest.mark.parametrize("M, N, K", [(24, 200, 1024), (64, 136, 1056), (17, 96, 128), (49, 90, 3072), (40, 1048, 160)])
+@pytest.mark.parametrize("M, N, K", [(24, 200, 1024), (64, 136, 1056), (17, 96, 128), (49, 90, 3072), (40, 1048, 160),
+                                     (1, 96, 160), (7, 200, 1024), (16, 136, 288)])
 def test_fused_gemm_conv_step_with_the_rows_shared_by_a_workgroups_waves(ops, M, N, K):
     """The conv epilogue of the kernel whose waves own feature tiles and share the rows through LDS: taps 1 to 6,
     a width that is no multiple of 16 or 4, conv columns that start and end inside a lane's four, with the row
