@@ -16,13 +16,12 @@ src/architecture.rs:367-667 validation before load).
 """
 from __future__ import annotations
 
-from typing import Dict, Hashable, List, Optional, Sequence
+from typing import Hashable, Optional, Sequence
 
 import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
-from ..cache.pages import CacheExhausted
 from ..config.registry import config_from_dict, load_config
 from ..config.spec import ConfigError
 from ..kernels import build as kernel_build

@@ -5,9 +5,8 @@ src/generation.rs:1412-1533) is the scheduler run with one or many requests.
 """
 from __future__ import annotations
 
-import time
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence, Union
+from typing import List, Optional, Sequence, Union
 
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler

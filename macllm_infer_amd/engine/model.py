@@ -4,7 +4,7 @@ and output projection, put together from registered parts according to a ``Model
 """
 from __future__ import annotations
 
-from typing import Dict, Hashable, List, Tuple
+from typing import Dict, Hashable, List
 
 import torch
 

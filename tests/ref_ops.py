@@ -8,8 +8,6 @@ doubles only: the package itself has no CPU path.
 """
 from __future__ import annotations
 
-import math
-
 import torch
 import torch.nn.functional as F
 

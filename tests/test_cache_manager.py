@@ -6,7 +6,7 @@ import random
 import pytest
 import torch
 
-from macllm_infer_amd.cache import CacheExhausted, CacheManager, KVNeed, PagePool, SlotPool, StateNeed
+from macllm_infer_amd.cache import CacheExhausted, CacheManager, KVNeed, PagePool, StateNeed
 
 
 def make(capacity=64, page=8, requests=3, window=None):

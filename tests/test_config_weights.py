@@ -10,7 +10,7 @@ from macllm_infer_amd.config import (ConfigError, FalconH1Config, config_from_di
                                      registered_architectures)
 from macllm_infer_amd.engine.model import DecoderModel
 from macllm_infer_amd.weights import WeightError, WeightSource, bind, write_safetensors
-from macllm_infer_amd.weights.random_init import random_tensors, write_random_model
+from macllm_infer_amd.weights.random_init import random_tensors
 
 
 def test_config_reads_its_own_keys_and_defaults():

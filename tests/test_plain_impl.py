@@ -5,7 +5,6 @@ convolution, a norm in the wrong place) fails it."""
 import math
 
 import numpy as np
-import pytest
 import torch
 import torch.nn.functional as F
 

@@ -5,7 +5,7 @@ multipliers, rope base, norm eps and vocabulary."""
 import torch
 
 from macllm_infer_amd.config import FalconH1Config
-from macllm_infer_amd.weights.random_init import random_tensors, write_random_model
+from macllm_infer_amd.weights.random_init import write_random_model
 
 TINY_A = dict(
     architectures=["FalconH1ForCausalLM"], model_type="falcon_h1",

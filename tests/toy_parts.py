@@ -414,7 +414,6 @@ def exercise(schedule, device, check_device):
     """Register the toys, build the toy model through the engine and compare whole, cut and
     mixed steps with ``toy_plain_logits``."""
     from macllm_infer_amd import Engine, Lane
-    from macllm_infer_amd.engine.model import DecoderModel
     from macllm_infer_amd.weights.random_init import random_tensors
     register_toys()
     raw = {"architectures": ["ToyForTests"], "hidden": 32, "vocab": 90, "slope": 0.01, "bias": 0.3, "decay": 0.9,
