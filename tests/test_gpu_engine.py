@@ -860,20 +860,32 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
     assert with_graphs.graphs.counts["bucket_replays"] == replays + 3
 
 
-@pytest.mark.parametrize("name, dtype, seed", [("B", "float32", 0), ("C", "bfloat16", 1), ("A", "bfloat16", 2)])
-def test_steps_of_any_shape_through_graphs_of_a_capacity_match_eager_steps(tmp_path, name, dtype, seed):
+@pytest.mark.parametrize("name, dtype, seed, shared", [("B", "float32", 0, False), ("C", "bfloat16", 1, False),
+                                                      ("A", "bfloat16", 2, False), ("C", "bfloat16", 3, True)])
+def test_steps_of_any_shape_through_graphs_of_a_capacity_match_eager_steps(tmp_path, monkeypatch, name, dtype, seed, shared):
     """Sixty steps drawn at random (one to five lanes, portions of 2 to 90 tokens beside decoded tokens, wanted
     places anywhere or nowhere, requests that end and begin) through an engine with graphs, some of them
     captured before the first request, beside an engine that launches every step kernel by kernel: the same
     logits and the same cache accounting, whichever way a step went (a capacity's first sighting is launched,
-    later ones replay its graph), and a step whose capacity was warmed up replays at once."""
+    later ones replay its graph), and a step whose capacity was warmed up replays at once.  ``shared``: the engine
+    with graphs takes the kernel that shares the rows wherever a product of a step of 17 to 64 tokens has it
+    (in slabs where it feeds the stream), the other engine none of it."""
     import random
     from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.parts import fused
     folder = tiny_configs.make_model_dir(name, tmp_path, torch.float32 if dtype == "float32" else torch.bfloat16)
     cfg, _ = plain_impl.load_model_dir(folder)
     make = lambda graphs: Engine(folder, dtype=dtype, kv_cache_block_tokens=8, kv_cache_capacity_tokens=3000,
                                  max_active_sequences=6, decode_graphs=graphs)
-    with_graphs, eager = make(True), make(False)
+    if shared:
+        monkeypatch.setattr(fused, "FORCE_SPLIT", 2)
+        monkeypatch.setattr(fused, "FORCE_SHARED_ROWS", 1)
+    with_graphs = make(True)
+    if shared:
+        assert with_graphs.model.blocks[0].fusion.tiles_out[3:6] == with_graphs.model.blocks[0].fusion.tiles_in[3:6] == (-1,) * 3
+        monkeypatch.setattr(fused, "FORCE_SPLIT", None)
+        monkeypatch.setattr(fused, "FORCE_SHARED_ROWS", None)
+    eager = make(False)
     captured = with_graphs.warm_up([(1, 1), (4, 4), (1, 40), (2, 100), (3, 130), (5, 200)])
     assert len(captured) == 6 and with_graphs.graphs.counts["bucket_replays"] == 0
     first = tokens_for(cfg["vocab_size"], 100, 2999)
