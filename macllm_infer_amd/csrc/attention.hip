@@ -244,7 +244,9 @@ __global__ void paged_attention_merge_kernel(const float* __restrict__ partial, 
   int first_key = 0;
   if (window > 0 && query_position - window + 1 > 0) first_key = query_position - window + 1;
   const int first_run = first_key / PA_RUN;
-  const int last_run = query_position / PA_RUN;
+  // a caller's bound on the contexts sizes the work area: a token beyond that bound merges the runs that
+  // were launched for it and never reads outside the area
+  const int last_run = min(query_position / PA_RUN, runs - 1);
   const float* theirs = partial + ((token * Hq + head) * runs) * (long)(dh + 2);
   for (int dim = threadIdx.x; dim < dh; dim += blockDim.x) {
     float maximum = -INFINITY, denominator = 0.f, sum = 0.f;

@@ -343,3 +343,20 @@ extern "C" int mi_scale_to_f32(const void* in, int dtype, float multiplier, floa
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
+
+// ---------------------------------------------------------------- bias behind a library product
+// out[m, n] = bf16(sums[m, n] + bias[n]): the float32 sums of a bfloat16 product get their float32 bias and are
+// rounded once (reference: src/model_weights.rs:530-545 adds the bias to the product's result).
+__global__ void add_bias_round_kernel(const float* __restrict__ sums, const float* __restrict__ bias,
+                                      bf16_t* __restrict__ out, int N, long total) {
+  const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (index < total) out[index] = (bf16_t)(sums[index] + bias[index % N]);
+}
+
+extern "C" int mi_add_bias_round(const float* sums, const float* bias, void* out, int M, int N, hipStream_t stream) {
+  if (M <= 0 || N <= 0 || !sums || !bias || !out) return ERR_BAD_ARGUMENT;
+  const long total = (long)M * N;
+  add_bias_round_kernel<<<(int)((total + 255) / 256), 256, 0, stream>>>(sums, bias, (bf16_t*)out, N, total);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}

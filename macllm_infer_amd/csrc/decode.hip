@@ -620,12 +620,18 @@ static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStre
 // there is one.
 constexpr int SR_CHUNKS = 4;
 constexpr int SR_LD = SR_CHUNKS * 32 + 8;        // a stage's row in LDS, padded against bank conflicts
+// gfx950 gives a workgroup up to 160 KiB of LDS (earlier targets: 64 KiB).  The kernels of this file that size
+// their LDS at run time stay within 64 KiB; the two stages of 96 or 128 rows below are static and exceed it,
+// which is stated here rather than left to the target.
+constexpr int GFX950_LDS_PER_WORKGROUP = 160 * 1024;
 
 template <int MT, int NT, int EPI>
 __global__ __launch_bounds__(256) void shared_rows_gemm_kernel(FusedGemmParams p) {
   __shared__ __align__(16) bf16_t stage[2][MT * 16 * SR_LD];
   constexpr int SQUARE_PARTS = MT <= 4 ? 4 : 2;      // threads that add up a row's sums of squares
   __shared__ float squares[SQUARE_PARTS][MT * 16];
+  static_assert(sizeof(bf16_t) * 2 * MT * 16 * SR_LD + sizeof(float) * SQUARE_PARTS * MT * 16 <= GFX950_LDS_PER_WORKGROUP,
+                "the two stages of the step's rows do not fit a gfx950 workgroup's LDS");
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE, q = lane / 16, r = lane % 16;
   const int tiles = (p.N + 15) / 16;
   const int chunks = p.K / 32;

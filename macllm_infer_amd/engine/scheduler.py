@@ -256,8 +256,12 @@ class Scheduler:
             except CacheExhausted:
                 if len(visits) > 1:
                     visits.pop()                 # the last lane waits for a later round
+                elif self._pending is not None:
+                    # a round is still on its way: its tokens may end requests (this one too) and give pages
+                    # back, so they are read first and the round is made up again from what is then live
+                    self._resolve()
+                    visits = self._collect()
                 else:
-                    self._resolve()              # whatever is on its way belongs to requests that still count
                     self._finish(visits[0][0], "resource_exhausted")
                     visits = self._collect()
             except StepFailed as failure:

@@ -38,6 +38,7 @@ _SIGNATURES = {
                                     _c_int, _c_ptr],
         "mi_swiglu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
         "mi_scale_to_f32": [_c_ptr, _c_int, _c_float, _c_ptr, _c_long, _c_ptr],
+        "mi_add_bias_round": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     },
     "attention": {
         "mi_rope_kv_store": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int,
@@ -300,7 +301,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
         return torch.mm(x, weight.t(), out_dtype=torch.float32)
     if bias is None:
         return torch.mm(x, weight.t())
-    return torch.addmm(bias.to(torch.bfloat16), x, weight.t())
+    # the bias stays float32: it is added to the product's float32 sums, and the result is rounded once
+    _need(bias.dtype == torch.float32 and bias.numel() == weight.shape[0] and bias.is_contiguous(),
+          "linear: bias must be float32 [N]")
+    sums = torch.mm(x, weight.t(), out_dtype=torch.float32)
+    out = torch.empty(sums.shape, dtype=torch.bfloat16, device=x.device)
+    _check(_fn("common", "mi_add_bias_round")(_p(sums), _p(bias), _p(out), sums.shape[0], sums.shape[1], _stream()),
+           "add_bias_round")
+    return out
 
 
 # --------------------------------------------------------------------------- attention

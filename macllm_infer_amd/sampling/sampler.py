@@ -136,11 +136,12 @@ class Sampler:
                        self._work(B), out, torch.empty(B, dtype=torch.int32, device=device))
         if self.device.type != "cuda":                 # host-side tests: nothing is in flight
             return PendingTokens(out, out, None)
-        if len(self._host_tokens) < self.HOST_BUFFERS:
+        # the buffers are used strictly in turn: call n writes buffer n % HOST_BUFFERS, so a call's tokens stay
+        # readable until HOST_BUFFERS - 1 further calls have been made
+        turn = self._turn
+        self._turn = (turn + 1) % self.HOST_BUFFERS
+        if len(self._host_tokens) <= turn:
             self._host_tokens.append(torch.empty(max(B, 64), dtype=torch.int32, pin_memory=True))
-            turn = len(self._host_tokens) - 1
-        else:
-            turn = self._turn = (self._turn + 1) % self.HOST_BUFFERS
         if self._host_tokens[turn].numel() < B:
             self._host_tokens[turn] = torch.empty(B, dtype=torch.int32, pin_memory=True)
         host = self._host_tokens[turn]

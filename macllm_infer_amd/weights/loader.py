@@ -15,12 +15,17 @@ from __future__ import annotations
 
 import json
 import os
+import warnings
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
 from .safetensors_io import SafetensorsFile
+
+
+class Float16Narrowed(UserWarning):
+    """Tensors stored in float16 were kept in bfloat16, which drops 3 bits of their mantissas."""
 
 
 class WeightError(ValueError):
@@ -186,6 +191,7 @@ def bind(source: WeightSource, expectations: Sequence[Expect],
     if missing or unexpected or wrong_shape or wrong_dtype:
         raise WeightError(missing, unexpected, sorted(wrong_shape), sorted(wrong_dtype))
     out: Dict[str, torch.Tensor] = {}
+    narrowed: List[str] = []
     for name, expect in wanted.items():
         tensor = source.tensor(name).reshape(expect.shapes[0])
         if expect.integer:
@@ -194,5 +200,11 @@ def bind(source: WeightSource, expectations: Sequence[Expect],
             tensor = tensor.to(torch.float32)
         elif tensor.dtype == torch.float16:
             tensor = tensor.to(torch.bfloat16)            # the 16-bit serving dtype is bfloat16
+            narrowed.append(name)
         out[name] = tensor
+    if narrowed:
+        warnings.warn(f"{len(narrowed)} tensors stored in float16 (the first: {narrowed[0]}) are kept in bfloat16: "
+                      "3 of their 10 mantissa bits are dropped and values beyond bfloat16's 8 bits are rounded; "
+                      "store the checkpoint in bfloat16 or float32 to choose the rounding yourself",
+                      Float16Narrowed, stacklevel=2)
     return out

@@ -43,6 +43,21 @@ import torch.nn.functional as F
 # a multiplier into a weight, is one more sample of the same noise).
 _ROUND_TO: Optional[torch.dtype] = None
 _DITHER: Optional[torch.Generator] = None
+# The precision everything is computed in.  float32 is the model; inside ``computed_in(torch.float64)`` the same
+# functions run in float64 on the same weights and tokens, which tells how far float32 rounding alone moves this
+# model's logits (the inverse frequencies of the rotation stay rounded to float32: they are part of the model).
+_EXACT: torch.dtype = torch.float32
+
+
+@contextlib.contextmanager
+def computed_in(dtype: torch.dtype):
+    global _EXACT
+    before = _EXACT
+    _EXACT = dtype
+    try:
+        yield
+    finally:
+        _EXACT = before
 
 
 @contextlib.contextmanager
@@ -61,8 +76,8 @@ def _r(x: torch.Tensor) -> torch.Tensor:
         return x
     if _DITHER is not None:
         bits = 8 if _ROUND_TO == torch.bfloat16 else 11 if _ROUND_TO == torch.float16 else 24
-        x = x * (1.0 + (torch.rand(x.shape, generator=_DITHER) - 0.5) * 2.0 ** -bits)
-    return x.to(_ROUND_TO).float()
+        x = x * (1.0 + (torch.rand(x.shape, generator=_DITHER).to(_EXACT) - 0.5) * 2.0 ** -bits)
+    return x.to(_ROUND_TO).to(_EXACT)
 
 
 # --------------------------------------------------------------------------- parts
@@ -73,8 +88,8 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     Closed form confirmed by the golden of src/decoder.rs:10331-10334; built at
     src/model_weights.rs:563-565.
     """
-    x = x.float()
-    return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    x = x.to(_EXACT)
+    return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight.to(_EXACT)
 
 
 def rope_inverse_frequencies(theta: float, rotary_dim: int) -> torch.Tensor:
@@ -95,12 +110,12 @@ def rope_half_split(x: torch.Tensor, positions: torch.Tensor, theta: float,
     out[j+half] = x[j+half] cos + x[j] sin (layout doc src/architecture.rs:44-48);
     dims past rotary_dim pass through (src/decoder.rs:226-251).
     """
-    x = x.float()
+    x = x.to(_EXACT)
     dh = x.shape[-1]
     rotary_dim = dh if rotary_dim is None else rotary_dim
     half = rotary_dim // 2
     freq = rope_inverse_frequencies(theta, rotary_dim)
-    angle = positions.to(torch.float32)[:, None] * freq[None, :]      # [T, half]
+    angle = positions.to(_EXACT)[:, None] * freq.to(_EXACT)[None, :]      # [T, half]
     cos = angle.cos()[:, None, :]
     sin = angle.sin()[:, None, :]
     first, second = x[..., :half], x[..., half:rotary_dim]
@@ -117,11 +132,11 @@ def gqa_causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scal
     is after the query's, or when query - key >= window (src/decoder.rs:4515-4532);
     softmax in float32 (src/decoder.rs:4665-4667); o = p @ v.  Returns [T, Hq, dh].
     """
-    q, k, v = q.float(), k.float(), v.float()
+    q, k, v = q.to(_EXACT), k.to(_EXACT), v.to(_EXACT)
     T, Hq, dh = q.shape
     Hkv = k.shape[1]
     group = Hq // Hkv
-    out = torch.empty(T, Hq, v.shape[-1])
+    out = torch.empty(T, Hq, v.shape[-1], dtype=_EXACT)
     position = torch.arange(T)
     masked = position[None, :] > position[:, None]
     if window is not None:
@@ -143,15 +158,15 @@ def causal_depthwise_conv(x: torch.Tensor, weight: torch.Tensor,
     x [T, C]; weight [C, K].  src/decoder.rs:2211-2252 (window = history ++ x,
     tap k reads window[t + k]); orientation comment :5948-5950.
     """
-    x = x.float()
+    x = x.to(_EXACT)
     T, C = x.shape
     K = weight.shape[1]
-    window = torch.cat([torch.zeros(K - 1, C), x], dim=0)
-    out = torch.zeros(T, C)
+    window = torch.cat([torch.zeros(K - 1, C, dtype=_EXACT), x], dim=0)
+    out = torch.zeros(T, C, dtype=_EXACT)
     for tap in range(K):
-        out = out + window[tap:tap + T, :] * weight[:, tap].float()[None, :]
+        out = out + window[tap:tap + T, :] * weight[:, tap].to(_EXACT)[None, :]
     if bias is not None:
-        out = out + bias.float()[None, :]
+        out = out + bias.to(_EXACT)[None, :]
     return out
 
 
@@ -172,20 +187,20 @@ def selective_scan(x: torch.Tensor, B: torch.Tensor, C: torch.Tensor, dt_raw: to
     crates/macllm-kernels/src/mamba2.rs:259-288; src/decoder.rs:2321-2346.
     Returns (y [T, H, P], final state).
     """
-    x, B, C, dt_raw = x.float(), B.float(), C.float(), dt_raw.float()
+    x, B, C, dt_raw = x.to(_EXACT), B.to(_EXACT), C.to(_EXACT), dt_raw.to(_EXACT)
     T, H, P = x.shape
     G, N = B.shape[1], B.shape[2]
     heads_per_group = H // G
-    state = torch.zeros(H, P, N) if initial_state is None else initial_state.clone().float()
-    delta = softplus(dt_raw + dt_bias.float()[None, :])              # [T, H]
-    y = torch.empty(T, H, P)
+    state = torch.zeros(H, P, N, dtype=_EXACT) if initial_state is None else initial_state.clone().to(_EXACT)
+    delta = softplus(dt_raw + dt_bias.to(_EXACT)[None, :])              # [T, H]
+    y = torch.empty(T, H, P, dtype=_EXACT)
     group_of_head = torch.arange(H) // heads_per_group
     for t in range(T):
-        decay = torch.exp(delta[t] * A.float())                       # [H]
+        decay = torch.exp(delta[t] * A.to(_EXACT))                       # [H]
         Bt = B[t][group_of_head]                                      # [H, N]
         Ct = C[t][group_of_head]
         state = state * decay[:, None, None] + (delta[t][:, None, None] * x[t][:, :, None]) * Bt[:, None, :]
-        y[t] = (state * Ct[:, None, :]).sum(-1) + D.float()[:, None] * x[t]
+        y[t] = (state * Ct[:, None, :]).sum(-1) + D.to(_EXACT)[:, None] * x[t]
     return y, state
 
 
@@ -195,24 +210,24 @@ def gate_and_group_norm(y: torch.Tensor, z: torch.Tensor, norm_weight: Optional[
 
     y, z [T, E].  Gate first, norm after (src/decoder.rs:2350-2367).
     """
-    y = y.float() * F.silu(z.float())
+    y = y.to(_EXACT) * F.silu(z.to(_EXACT))
     if norm_weight is None:
         return y
     T, E = y.shape
     grouped = y.view(T, groups, E // groups)
     grouped = grouped / torch.sqrt(grouped.pow(2).mean(-1, keepdim=True) + eps)
-    return (grouped * norm_weight.float().reshape(groups, E // groups)[None]).reshape(T, E)
+    return (grouped * norm_weight.to(_EXACT).reshape(groups, E // groups)[None]).reshape(T, E)
 
 
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """SiLU(gate) * up (src/decoder.rs:298-305)."""
-    return F.silu(gate.float()) * up.float()
+    return F.silu(gate.to(_EXACT)) * up.to(_EXACT)
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
     """x @ W.T (+ b) (src/model_weights.rs:530-545)."""
-    y = x.float() @ weight.float().T
-    return y if bias is None else y + bias.float()
+    y = x.to(_EXACT) @ weight.to(_EXACT).T
+    return y if bias is None else y + bias.to(_EXACT)
 
 
 # --------------------------------------------------------------------------- mixers
@@ -232,7 +247,7 @@ def attention_mixer(n: torch.Tensor, w: Dict[str, torch.Tensor], *, num_heads: i
     """
     T = n.shape[0]
     positions = torch.arange(T) if positions is None else positions
-    n = n.float() * in_multiplier
+    n = n.to(_EXACT) * in_multiplier
     q = _r(linear(n, w["q_proj.weight"], w.get("q_proj.bias"))).view(T, num_heads, head_dim)
     k = linear(n, w["k_proj.weight"], w.get("k_proj.bias")).view(T, num_kv_heads, head_dim)
     k = _r(k * key_multiplier)
@@ -260,9 +275,9 @@ def mamba2_mixer(n: torch.Tensor, w: Dict[str, torch.Tensor], *, num_heads: int,
     E = num_heads * head_dim
     GN = num_groups * state_size
     if projected is None:
-        u = linear(n.float() * in_multiplier, w["in_proj.weight"], w.get("in_proj.bias"))
+        u = linear(n.to(_EXACT) * in_multiplier, w["in_proj.weight"], w.get("in_proj.bias"))
     else:
-        u = projected.float()
+        u = projected.to(_EXACT)
     T = u.shape[0]
     z, x, B, C, dt = torch.split(u, [E, E, GN, GN, num_heads], dim=-1)
     z, x, B, C, dt = (_r(z * multipliers[0]), _r(x * multipliers[1]), _r(B * multipliers[2]),
@@ -273,11 +288,11 @@ def mamba2_mixer(n: torch.Tensor, w: Dict[str, torch.Tensor], *, num_heads: int,
         conv_weight = conv_weight.squeeze(1)
     conv = _r(F.silu(causal_depthwise_conv(xbc, conv_weight, w.get("conv1d.bias"))))
     xc, Bc, Cc = torch.split(conv, [E, GN, GN], dim=-1)
-    A = -torch.exp(w["A_log"].float().reshape(num_heads))
+    A = -torch.exp(w["A_log"].to(_EXACT).reshape(num_heads))
     y, state = selective_scan(
         xc.view(T, num_heads, head_dim), Bc.view(T, num_groups, state_size),
-        Cc.view(T, num_groups, state_size), dt, w["dt_bias"].float(), A,
-        w["D"].float().reshape(num_heads))
+        Cc.view(T, num_groups, state_size), dt, w["dt_bias"].to(_EXACT), A,
+        w["D"].to(_EXACT).reshape(num_heads))
     y = _r(gate_and_group_norm(y.reshape(T, E), z, w.get("norm.weight"), num_groups, eps))
     out = _r(linear(y, w["out_proj.weight"], w.get("out_proj.bias")) * out_multiplier)
     if return_state:
@@ -346,12 +361,12 @@ def falcon_h1_logits(cfg: dict, tensors: Dict[str, torch.Tensor], tokens: Sequen
     the embedding matrix, src/decoder.rs:3045-3053) * multiplier (src/decoder.rs:3349-3357).
     """
     token_ids = torch.tensor(list(tokens), dtype=torch.long)
-    embedding = tensors["model.embed_tokens.weight"].float()
+    embedding = tensors["model.embed_tokens.weight"].to(_EXACT)
     h = embedding[token_ids] * cfg.get("embedding_multiplier", 1.0)
     for layer in range(cfg["num_hidden_layers"]):
         h = falcon_h1_layer(h, tensors, layer, cfg, ablate)
     h = _r(rms_norm(h, tensors["model.norm.weight"], cfg.get("rms_norm_eps", 1e-5)))
-    head = embedding if cfg.get("tie_word_embeddings", False) else tensors["lm_head.weight"].float()
+    head = embedding if cfg.get("tie_word_embeddings", False) else tensors["lm_head.weight"].to(_EXACT)
     return (h @ head.T) * cfg.get("lm_head_multiplier", 1.0)
 
 

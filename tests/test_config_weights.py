@@ -199,7 +199,9 @@ def test_alternative_shapes_and_widening(tmp_path):
     tensors["model.layers.0.mamba.conv1d.weight"] = tensors["model.layers.0.mamba.conv1d.weight"].reshape(96, 1, 4)
     tensors["model.layers.0.mamba.A_log"] = tensors["model.layers.0.mamba.A_log"].reshape(8, 1).double()
     tensors["model.layers.0.mamba.D"] = tensors["model.layers.0.mamba.D"].half()
-    bound = bind(WeightSource.from_tensors(tensors), DecoderModel.expected_tensors(config.to_model_spec()))
+    from macllm_infer_amd.weights import Float16Narrowed
+    with pytest.warns(Float16Narrowed, match="1 tensors stored in float16.*model.layers.0.mamba.D"):   # not silently
+        bound = bind(WeightSource.from_tensors(tensors), DecoderModel.expected_tensors(config.to_model_spec()))
     assert bound["model.layers.0.mamba.conv1d.weight"].shape == (96, 4)
     assert bound["model.layers.0.mamba.A_log"].shape == (8,) and bound["model.layers.0.mamba.A_log"].dtype == torch.float32
     assert bound["model.layers.0.mamba.D"].dtype == torch.bfloat16

@@ -679,6 +679,110 @@ def test_graphs_come_in_buckets_of_context_length():
     assert with_graphs.graphs.counts["decode_replays"] == 16
 
 
+def sharpened(tensors, factor=8.0):
+    """Random weights give every key nearly the same score, and a fault in one far page is then one part in
+    thousands of an attended row.  With the query and key projections scaled up the scores spread over several
+    units and a few keys anywhere in the context carry a row: a wrong page, run of keys or rotation shows."""
+    out = dict(tensors)
+    for name, tensor in tensors.items():
+        if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
+            out[name] = (tensor.float() * factor).to(tensor.dtype)
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_contexts_beyond_2048_tokens_match_the_plain_model(dtype):
+    """What the benchmark's contexts go through, against the plain model: a prompt of 2,100 tokens in portions of
+    512 (the second portion captures the graph of its capacity, the later ones replay it, the last ones through
+    the wider bucket of contexts), then eight decode steps of three requests at 2,100, 700 and 40 tokens in one
+    batch (several runs of keys for one request beside a single short one).  Every row is wanted and compared.
+    The attention scores are sharpened so that far keys count (``sharpened``)."""
+    import gates
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.weights.random_init import random_tensors
+    config = FalconH1Config.from_dict(dict(tiny_configs.TINY_C, max_position_embeddings=16384))
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    tensors = sharpened(random_tensors(config, 4, storage, "unit"))
+    plain = {name: tensor.float() for name, tensor in tensors.items()}
+    cfg = config.to_dict()
+    lengths = {"long": 2100, "mid": 700, "short": 40}
+    tokens = {name: tokens_for(config.vocab_size, count + 8, 70 + index) for index, (name, count) in enumerate(lengths.items())}
+    engine = Engine(config=config, tensors=tensors, dtype=dtype, kv_cache_capacity_tokens=4096, max_active_sequences=3)
+    rows = {name: [] for name in tokens}
+    for name in tokens:
+        engine.add_request(name)
+    for first in range(0, 2100, 512):
+        count = min(512, 2100 - first)
+        rows["long"].append(engine.step([Lane("long", tokens["long"][first:first + count], list(range(count)))]).cpu())
+    if engine.graphs is not None:
+        assert engine.graphs.counts["bucket_captures"] >= 1 and engine.graphs.counts["bucket_replays"] >= 3
+    mixed = engine.step([Lane("mid", tokens["mid"][:700], list(range(700))),
+                         Lane("short", tokens["short"][:40], list(range(40)))]).cpu()
+    rows["mid"].append(mixed[:700])
+    rows["short"].append(mixed[700:])
+    for turn in range(8):
+        out = engine.step([Lane(name, [tokens[name][lengths[name] + turn]], [0]) for name in tokens]).cpu()
+        for row, name in enumerate(tokens):
+            rows[name].append(out[row:row + 1])
+    for name in tokens:
+        want = plain_impl.falcon_h1_logits(cfg, plain, tokens[name]).numpy()
+        got = torch.cat(rows[name]).numpy()
+        assert got.shape == want.shape
+        if dtype == "float32":
+            ok, text = gates.conditioned_close_f32(got, want, cfg, plain, tokens[name])
+        else:
+            ok, text = gates.conditioned_close(got, want, cfg, plain, tokens[name])
+        assert ok, f"{name}: {text}"
+        # the far keys do count: the same rows with the first 256 positions' keys and values out of reach
+        # (the sequence without its first 256 tokens) are somewhere else
+    shifted = plain_impl.falcon_h1_logits(cfg, plain, tokens["long"][256:]).numpy()
+    whole = plain_impl.falcon_h1_logits(cfg, plain, tokens["long"]).numpy()
+    assert np.abs(shifted[-8:] - whole[-8:]).max() > 0.05 * np.abs(whole).max()
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("name, dtype", [("C", "bfloat16"), ("B", "float32")])
+def test_capacity_graphs_with_four_lanes_and_padding_match_the_plain_model(tmp_path, name, dtype):
+    """Steps of four lanes (portions of changing sizes beside single tokens) whose tokens do not fill a capacity:
+    the graph of eight lanes is captured at the second step and replayed for the rest, with three padding lanes of
+    one token and one that holds the remainder; every row against the plain model, not against another path of
+    the engine."""
+    import gates
+    from macllm_infer_amd import Engine, Lane
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = tiny_configs.make_model_dir(name, tmp_path, storage)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    plain = {key: value.float() for key, value in tensors.items()}
+    engine = Engine(folder, dtype=dtype, kv_cache_block_tokens=8, kv_cache_capacity_tokens=768, max_active_sequences=4)
+    engine.split_from_lanes = 1 << 30                       # one batch a step, whatever it holds
+    sequences = {key: tokens_for(cfg["vocab_size"], 150, 40 + index) for index, key in enumerate("abcd")}
+    cursor = {key: 0 for key in sequences}
+    rows = {key: [] for key in sequences}
+    for key in sequences:
+        engine.add_request(key)
+    shapes = [(20, 1, 15, 2), (1, 19, 3, 13), (9, 9, 9, 9), (2, 1, 30, 1), (17, 16, 2, 2), (1, 1, 1, 34), (5, 21, 1, 11),
+              (12, 3, 12, 12)]
+    for shape in shapes:                                                     # 33 to 48 tokens each: one capacity
+        assert 32 < sum(shape) <= 44
+        lanes = [Lane(key, sequences[key][cursor[key]:cursor[key] + count], list(range(count)))
+                 for key, count in zip(sequences, shape)]
+        out = engine.step(lanes).cpu()
+        for key, count in zip(sequences, shape):
+            rows[key].append(out[:count])
+            out = out[count:]
+            cursor[key] += count
+    counts = engine.graphs.counts
+    assert counts["bucket_captures"] == 1 and counts["bucket_replays"] == len(shapes) - 1 and counts["bucket_eager"] == 1
+    assert [key[:2] for key in engine.graphs._bucket_graphs] == [(8, 48)]
+    for key, sequence in sequences.items():
+        want = plain_impl.falcon_h1_logits(cfg, plain, sequence[:cursor[key]]).numpy()
+        got = torch.cat(rows[key]).numpy()
+        ok = gates.float32_close(got, want) if dtype == "float32" else gates.bfloat16_close(got, want)
+        assert ok, f"{key}: {np.abs(got - want).max():.3e} of {np.abs(want).max():.2f}"
+    engine.cache.check()
+
+
 def test_layers_of_one_mixer_and_a_mixer_from_outside_take_the_fast_paths(monkeypatch):
     """The fast paths of a layer belong to no model: a layer with attention alone decodes through the skinny
     kernels (norm in the prologue, SiLU(g)*u in the epilogue), and so do the projections of a toy mixer with
@@ -1038,9 +1142,15 @@ def test_a_wide_model_runs_through_the_fast_paths(tmp_path, monkeypatch, padding
 # float32 engine is off by 3e-4 instead of 3e-6; 3024: 0.27 of the scale at position 195; 3022, 3040, 3041 and
 # the odd draw's 1, 3, 12, 22, 23, 28, 34, 57: 0.06 to 0.18).  ``gates.conditioned_close`` states the gate in
 # those terms.
+# A further sweep (seeds 7000 to 7059 of the even draw, 8000 to 8039 of the odd one) left the fixed gates at 7019
+# in float32 (one position, where the plain model in float32 is itself 7.7e-4 from the plain model in float64:
+# ``gates.conditioned_close_f32``) and in bfloat16 at 7019, 7027, 7039, 7047, 7054 and the odd draw's 8002, 8009,
+# 8011; those run here in both dtypes, under the gates that state the model's own rounding noise.
 RANDOM_CASES = ([(seed, False) for seed in range(8)] + [(seed, True) for seed in range(8)]
                 + [(seed, False) for seed in (3022, 3024, 3038, 3040, 3041)]
-                + [(seed, True) for seed in (12, 22, 23, 28, 34, 57)])
+                + [(seed, True) for seed in (12, 22, 23, 28, 34, 57)]
+                + [(seed, False) for seed in (7019, 7027, 7039, 7047, 7054)]
+                + [(seed, True) for seed in (8002, 8009, 8011)])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -1067,11 +1177,10 @@ def test_configurations_drawn_at_random_match_the_plain_model(seed, odd, dtype):
     def close(got, name, what):
         want = wanted[name]
         if dtype == "float32":
-            error = np.abs(got - want).max()
-            assert error <= gates.FLOAT32_TOLERANCE * max(1.0, np.abs(want).max()), f"seed {seed} {what}: {error:.3e}"
+            ok, text = gates.conditioned_close_f32(got, want, cfg, plain, tokens[name])
         else:
             ok, text = gates.conditioned_close(got, want, cfg, plain, tokens[name])
-            assert ok, f"seed {seed} {what}: {text}"
+        assert ok, f"seed {seed} {what}: {text}"
 
     engine = Engine(config=config, tensors=tensors, dtype=dtype, kv_cache_block_tokens=page,
                     kv_cache_capacity_tokens=640, max_active_sequences=3)

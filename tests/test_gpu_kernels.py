@@ -137,6 +137,18 @@ def test_mixed_product_keeps_a_32bit_weight(ops):
     close(both, x.float() @ w.to(torch.bfloat16).float().T + rand(50, seed=12), torch.bfloat16, 10.0)
 
 
+def test_bfloat16_product_adds_its_bias_in_float32(ops):
+    """A bias that 16 bits cannot hold: 1 + 2^-8 rounds to 1 in bfloat16, and a product of 2^-8 added to that
+    rounds to 1 again; added to the float32 sum it gives 1 + 2^-7, which bfloat16 holds."""
+    x = torch.zeros(3, 32, dtype=torch.bfloat16)
+    x[:, 0] = 2.0 ** -8
+    w = torch.zeros(5, 32, dtype=torch.bfloat16)
+    w[:, 0] = 1.0
+    bias = torch.full((5,), 1.0 + 2.0 ** -8)
+    got = ops.linear(x.to(DEV), w.to(DEV), bias.to(DEV))
+    assert got.dtype == torch.bfloat16 and bool((got.float().cpu() == 1.0 + 2.0 ** -7).all())
+
+
 # ------------------------------------------------------------------ attention
 def paged_setup(lengths, page_size, Hkv, dh, dtype, layers=2, seed=0):
     """A pool of shuffled pages [page, layer, K|V, Hkv, page_size*dh] and a block table per lane."""

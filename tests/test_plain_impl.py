@@ -404,3 +404,47 @@ def test_rounding_activations_shows_a_models_conditioning_without_any_kernel():
     # a fault is not excused: the logits of the neighbouring position fail the same gate
     ok, text = gates.conditioned_close(np.roll(exact, 1, axis=0), exact, raw, tensors, tokens)
     assert not ok, text
+
+
+def test_float64_runs_of_the_plain_model_and_the_float32_gate_in_terms_of_float32_rounding():
+    """The plain model computed in float64 agrees with its float32 self to float32 rounding on the tiny
+    configurations.  On seed 7019 of the random draw (one state-space head of 24 whose gated norm divides by a mean
+    square of 0.2 at position 123, where the median is 82) float32 rounding alone moves the plain model's logits at
+    that position by more than the fixed float32 gate allows an engine, and nowhere else: the gate stated in terms
+    of that rounding accepts another float32 evaluation of the model and still refuses a neighbour's logits."""
+    import gates
+    import tiny_configs
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.weights.random_init import random_tensors
+    for name in ("A", "B"):
+        raw, seed = tiny_configs.CONFIGS[name]
+        tensors = random_tensors(FalconH1Config.from_dict(raw), seed, torch.float32, "unit")
+        tokens = torch.randint(0, raw["vocab_size"], (60,), generator=torch.Generator().manual_seed(6)).tolist()
+        single = P.falcon_h1_logits(raw, tensors, tokens)
+        with P.computed_in(torch.float64):
+            double = P.falcon_h1_logits(raw, {key: value.double() for key, value in tensors.items()}, tokens)
+        assert single.dtype == torch.float32 and double.dtype == torch.float64
+        assert 0 < (single.double() - double).abs().max() < 2e-5, name
+        assert torch.equal(P.falcon_h1_logits(raw, tensors, tokens), single)          # and float32 again afterwards
+    raw, _, rng = tiny_configs.random_config(7019)
+    tensors = random_tensors(FalconH1Config.from_dict(raw), 7019, torch.float32, "unit")
+    tokens = torch.randint(0, raw["vocab_size"], (rng.choice([70, 131, 200]),),
+                           generator=torch.Generator().manual_seed(7019)).tolist()
+    want = P.falcon_h1_logits(raw, tensors, tokens).numpy()
+    noise = gates.float32_noise(raw, tensors, tokens, want)
+    tolerance = gates.FLOAT32_TOLERANCE * max(1.0, float(abs(want).max()))
+    assert noise.argmax() == 123 and noise[123] > tolerance
+    assert np.median(noise) < 0.1 * tolerance
+    # another float32 evaluation: the weights moved by half an ulp (a draw the gate's own samples do not hold)
+    generator = torch.Generator().manual_seed(99)
+    moved = {key: value * (1.0 + 6e-8 * torch.randn(value.shape, generator=generator)) for key, value in tensors.items()}
+    other = P.falcon_h1_logits(raw, moved, tokens).numpy()
+    ok, text = gates.conditioned_close_f32(other, want, raw, tensors, tokens)
+    assert ok, text
+    ok, text = gates.conditioned_close_f32(np.roll(want, 1, axis=0), want, raw, tensors, tokens)
+    assert not ok, text
+    # a fault at the ill-conditioned position alone is not excused either when it is large
+    broken = want.copy()
+    broken[123] += 50 * noise[123]
+    ok, text = gates.conditioned_close_f32(broken, want, raw, tensors, tokens)
+    assert not ok, text

@@ -247,3 +247,65 @@ def test_a_portion_that_does_not_end_its_prompt_is_cut_to_the_size_the_engine_pr
     assert sum(count for step in steps[:3] for request, count in step if request == 1) == 100
     assert finished[1].generated == [(prompt[-1] + 1) % 50, (prompt[-1] + 2) % 50, (prompt[-1] + 3) % 50]
     assert finished[0].generated == [10, 11, 12]
+
+
+class AheadEngine(FakeEngine):
+    """A fake engine whose lanes may take their token from the device (``Lane.feed``)."""
+    feeds_tokens = True
+
+    def step(self, lanes):
+        for lane in lanes:
+            if lane.feed is not None:
+                source, row = lane.feed
+                lane.tokens = [int(source[row])]
+        return super().step(lanes)
+
+
+class AsyncArgmaxSampler(ArgmaxSampler):
+    """Leaves its tokens "on the device": the scheduler then queues a round before it has read the one before."""
+    class Handle:
+        def __init__(self, tokens):
+            self.device = tokens
+
+        def wait(self):
+            return self.device.tolist()
+
+    def sample_async(self, logits, rows):
+        assert logits.shape[0] == len(rows)
+        return self.Handle(torch.argmax(logits, dim=-1).to(torch.int32))
+
+
+@pytest.mark.parametrize("prompts, stopper", [([[1, 2, 3], [11, 12, 13]], 0), ([[11, 12, 13], [1, 2, 3]], 1)])
+@pytest.mark.parametrize("ahead", [True, False])
+def test_a_stop_token_on_its_way_while_a_single_lane_finds_no_pages(prompts, stopper, ahead):
+    """Two pages of four tokens, two requests of three prompt tokens: the round in which both want a second page
+    shrinks to the first request's lane, which alone does not fit either.  The round before is then still on its way,
+    and its token for the request that counts 4, 5 is that request's stop token.  Whether the lane without pages
+    belongs to the request that stops (it must end once, with "stop") or to the other one (which fits as soon as the
+    stopped request's page is back, and must not fail with resource_exhausted), the outcome is the one of a scheduler
+    that waits for every round's tokens."""
+    engine = AheadEngine(capacity=8, page=4)
+    scheduler = Scheduler(engine, AsyncArgmaxSampler(), EngineConfig(), (5,))
+    assert scheduler.ahead
+    scheduler.ahead = ahead
+    params = SamplingParams(max_new_tokens=6, temperature=0.0)
+    for index, prompt in enumerate(prompts):
+        scheduler.submit(index, prompt, params)
+    finished = scheduler.run()
+    other = 1 - stopper
+    assert finished[stopper].finish_reason == "stop" and finished[stopper].generated == [4]
+    assert finished[other].finish_reason == "length" and finished[other].generated == [14, 15, 16, 17, 18, 19]
+    assert engine.lengths == {} and not scheduler.active
+
+
+def test_a_single_lane_without_pages_and_nothing_on_its_way_fails_alone_a_round_ahead():
+    """The same pressure with no stop token anywhere: nothing that is on its way can free a page, so the request
+    whose lane cannot grow fails with resource_exhausted, once, and the other runs to its length."""
+    engine = AheadEngine(capacity=8, page=4)
+    scheduler = Scheduler(engine, AsyncArgmaxSampler(), EngineConfig())
+    params = SamplingParams(max_new_tokens=6, temperature=0.0)
+    for index, prompt in enumerate([[1, 2, 3], [11, 12, 13]]):
+        scheduler.submit(index, prompt, params)
+    finished = scheduler.run()
+    assert sorted(request.finish_reason for request in finished.values()) == ["length", "resource_exhausted"]
+    assert engine.lengths == {} and not scheduler.active

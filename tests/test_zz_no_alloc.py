@@ -47,7 +47,7 @@ def test_decode_attention_from_the_static_array_matches_the_one_with_a_workspace
     k_cache, v_cache = views(dev_pool, page_size)
     stream = torch.cuda.current_stream().cuda_stream
 
-    def both(subset):
+    def both(subset, first_call=False):
         T = len(subset)
         queries, lanes, places = q[subset].to(DEV), i32(subset).to(DEV), positions[subset].to(DEV)
         longest = max(lengths[index] for index in subset)
@@ -56,16 +56,20 @@ def test_decode_attention_from_the_static_array_matches_the_one_with_a_workspace
         got = torch.full((T, Hq * dh), float("nan"), dtype=dtype, device=DEV)
         split_keys, splits = _splits(T, Hkv, page_size, longest)
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
+        # the device's own count of free bytes (torch's counters see only torch's allocator: a hipMalloc inside
+        # the library would pass them); the first call on a device may load the code object and resolve the symbol
+        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
         code = static(queries.data_ptr(), queries.stride(0), T, Hq, Hkv, dh, k_cache.data_ptr(), v_cache.data_ptr(),
                       k_cache.stride(0), page_size, dev_table.data_ptr(), dev_table.shape[1], lanes.data_ptr(),
                       places.data_ptr(), 0.11, 0, split_keys, splits, got.data_ptr(), got.stride(0), stream)
         assert code == 0, f"mi_decode_attention_static returned {code}"
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == before
+        if not first_call:
+            assert torch.cuda.mem_get_info()[0] == free_before, "the device's free memory changed across the call"
         assert torch.equal(got, want), f"subset {subset}: {(got.float() - want.float()).abs().max().item()}"
 
-    both(list(range(len(lengths))))          # the first call on this device asks for the array's address
+    both(list(range(len(lengths))), first_call=True)     # the first call on this device asks for the array's address
     both([6, 2])                             # a smaller step right behind it, in the same array
     both([0])
     both(list(range(len(lengths))))
