@@ -11,7 +11,9 @@ tokens fed back); ``prefill`` = one 2,048-token prompt in one step (replayed fro
 graph; ``prefill_uncaptured_ms`` = the same step launched kernel by kernel, as a shape is when it
 comes for the first time); ``roofline`` = the bytes the decode step has to read (every weight it
 uses once, and the cache and state of the live requests; ``bytes`` gives them and what the step
-writes) over its time, against 8 TB/s; ``points`` = decode at batch 1 and 64; ``step_ms`` = mean,
+writes) over its time, against 8 TB/s; ``points`` = decode at batch 1 and 64, and at longer contexts (batch 8
+at 8,192 and 32,768 tokens, batch 64 at 8,192, from an engine of the same layers that allows such contexts;
+``points_frac`` = their fractions of 8 TB/s on the bytes they have to read); ``step_ms`` = mean,
 median and 95th percentile of the timed steps (the reference reports the same three:
 src/benchmark/stats.rs:10-16); ``choices`` = what the build-time measurements chose for each
 projection of a layer at up to 16 / 32 / 64 rows (L = library, S = skinny kernel, a digit = slabs
@@ -55,6 +57,7 @@ SHAPES = {
 }
 CONTEXT = 2048
 PREFILL_TOKENS = 2048
+LONG_POINTS = ((8, 8192), (8, 32768), (64, 8192))      # (batch, context) of the decode points beyond the headline context
 # whole-request workloads (--workload serving): requests, prompt lengths (lowest, highest), new tokens
 SERVING = {"0.5b": (64, 128, 4096, 256), "7b": (64, 128, 4096, 256), "34b": (8, 8192, 8192, 128)}
 SERVING_PORTION = 2048
@@ -168,6 +171,7 @@ def main() -> int:
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--page-tokens", type=int, default=16)
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
+    parser.add_argument("--skip-long-points", action="store_true", help="no decode points at longer contexts")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only the 2,048-token prefill (for profiles; the line then reports prefill tokens/s)")
     parser.add_argument("--workload", default="steps", choices=["steps", "serving"],
@@ -214,7 +218,6 @@ def main() -> int:
                     kv_cache_block_tokens=args.page_tokens,
                     kv_cache_capacity_tokens=per_request * largest + PREFILL_TOKENS + 64,
                     max_active_sequences=largest + 1)
-    del tensors
     sampler = Sampler(engine.vocab_size, engine.device)
     generator = torch.Generator().manual_seed(0)
     vocab = config.vocab_size
@@ -244,13 +247,13 @@ def main() -> int:
     prefill_flops = total(prefill_costs(engine.spec, PREFILL_TOKENS, element)).flops
 
     # ---------------------------------------------------------------- decode at each batch size
-    results = {}
-    for batch in batches:
+    def decode_point(engine, sampler, batch, context_tokens):
         names = [f"b{batch}_{index}" for index in range(batch)]
         for name in names:
             engine.add_request(name)
-            prompt = torch.randint(0, vocab, (CONTEXT,), generator=generator).tolist()
-            engine.step([Lane(name, prompt, [])])
+            prompt = torch.randint(0, vocab, (context_tokens,), generator=generator).tolist()
+            for first in range(0, context_tokens, PREFILL_TOKENS):          # long contexts in portions
+                engine.step([Lane(name, prompt[first:first + PREFILL_TOKENS], [])])
         tokens = torch.randint(0, vocab, (batch,), generator=generator).tolist()
         rows = [SamplerRow(GREEDY, (), ()) for _ in names]
 
@@ -282,14 +285,35 @@ def main() -> int:
         for name in names:
             engine.finish(name)
         step_seconds = seconds / args.steps
-        context = CONTEXT + args.warmup + args.steps / 2.0
+        context = context_tokens + args.warmup + args.steps / 2.0
         moved = total(decode_step_costs(engine.spec, batch, context, element))
         step_times.sort()
         pick = lambda fraction: step_times[min(len(step_times) - 1, int(fraction * len(step_times)))]
-        results[batch] = dict(tokens_per_second=batch / step_seconds, ms=step_seconds * 1e3,
-                              gbs=moved.read / step_seconds / 1e9, read_mb=moved.read / 1e6, written_mb=moved.written / 1e6,
-                              step_ms={"mean": round(1e3 * sum(step_times) / len(step_times), 4),
-                                       "p50": round(1e3 * pick(0.5), 4), "p95": round(1e3 * pick(0.95), 4)})
+        return dict(tokens_per_second=batch / step_seconds, ms=step_seconds * 1e3,
+                    gbs=moved.read / step_seconds / 1e9, read_mb=moved.read / 1e6, written_mb=moved.written / 1e6,
+                    step_ms={"mean": round(1e3 * sum(step_times) / len(step_times), 4),
+                             "p50": round(1e3 * pick(0.5), 4), "p95": round(1e3 * pick(0.95), 4)})
+
+    results = {batch: decode_point(engine, sampler, batch, CONTEXT) for batch in batches}
+
+    # ---------------------------------------------------------------- the same at longer contexts
+    long_points = {}
+    if not (args.skip_points or args.skip_long_points or args.prefill_only):
+        choices = choices_of(engine)
+        del engine, sampler, graphs
+        torch.cuda.empty_cache()
+        most = max(context for _, context in LONG_POINTS)
+        long_config = FalconH1Config.from_dict(dict(raw, max_position_embeddings=most + 2 * per_request))
+        room = max(batch * (-(-(context + total_steps + 1) // 64) * 64) for batch, context in LONG_POINTS)
+        long_engine = Engine(config=long_config, tensors=tensors, dtype="bfloat16" if args.dtype == "bf16" else "float32",
+                             kv_cache_block_tokens=args.page_tokens, kv_cache_capacity_tokens=room + 64,
+                             max_active_sequences=max(batch for batch, _ in LONG_POINTS) + 1)
+        long_sampler = Sampler(long_engine.vocab_size, long_engine.device)
+        for batch, context in LONG_POINTS:
+            long_points[(batch, context)] = decode_point(long_engine, long_sampler, batch, context)
+    else:
+        choices = choices_of(engine)
+    del tensors
 
     if args.prefill_only:
         print(json.dumps({"metric": "prefill tok/s at 2,048 tokens", "value": round(PREFILL_TOKENS / prefill_seconds, 1),
@@ -317,12 +341,18 @@ def main() -> int:
                     "frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS[args.dtype], 5)},
         "roofline": {"bound": "hbm", "achieved": round(headline["gbs"], 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(headline["gbs"] / PEAK_HBM_GBS, 5)},
-        "points": {f"decode_b{batch}": round(result["tokens_per_second"], 1) for batch, result in results.items()
-                   if batch != args.batch},
+        "points": dict({f"decode_b{batch}": round(result["tokens_per_second"], 1) for batch, result in results.items()
+                        if batch != args.batch},
+                       **{f"decode_b{batch}_ctx{context}": round(result["tokens_per_second"], 1)
+                          for (batch, context), result in long_points.items()}),
+        "points_frac": dict({f"decode_b{batch}": round(result["gbs"] / PEAK_HBM_GBS, 5) for batch, result in results.items()
+                             if batch != args.batch},
+                            **{f"decode_b{batch}_ctx{context}": round(result["gbs"] / PEAK_HBM_GBS, 5)
+                               for (batch, context), result in long_points.items()}),
         "step_ms": headline["step_ms"],
         "bytes": {"read_mb": round(headline["read_mb"], 1), "written_mb": round(headline["written_mb"], 1)},
         "prefill_uncaptured_ms": round(uncaptured_seconds * 1e3, 3),
-        "choices": choices_of(engine),
+        "choices": choices,
     }
     print(json.dumps(record))
     return 0

@@ -11,6 +11,7 @@
 // (The reference pages its cache the same way, K and V both token-major:
 // crates/macllm-kv/src/cache.rs:558-566, crates/macllm-kernels/src/metal/paged_decode.metal:109-113.)
 #include "common.h"
+#include <type_traits>
 
 // ---------------------------------------------------------------- rope + cache write
 // For token t at absolute position p:
@@ -177,35 +178,38 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
       for (int i = 0; i < dh; i += 4) {
         const vec4 piece = *reinterpret_cast<const vec4*>(k_row + i);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) dot += q_shared[i + j] * to_float<T>(piece[j]);
+        for (int j = 0; j < 4; ++j) dot = fmaf(q_shared[i + j], to_float<T>(piece[j]), dot);
       }
     } else {
-      for (int i = 0; i < dh; ++i) dot += q_shared[i] * to_float(k_row[i]);
+      for (int i = 0; i < dh; ++i) dot = fmaf(q_shared[i], to_float(k_row[i]), dot);
     }
     score = dot * scale;
-    if (slopes) score -= slopes[head] * (float)(query_position - key);
+    if (slopes) score = fmaf(-slopes[head], (float)(query_position - key), score);
   }
   const float maximum = wave_max(score);                    // -inf for a wave without visible keys
   const float p = visible ? (FAST_EXP ? __expf(score - maximum) : expf(score - maximum)) : 0.f;
-  const float normalizer = wave_sum(p);
   p_shared[wave][lane] = p;
   row_shared[wave][lane] = row_offset;
   offset_shared[wave][lane] = offset;
-  if (lane == 0) {
-    wave_ml[wave][0] = maximum;
-    wave_ml[wave][1] = normalizer;
-  }
   __syncthreads();
   const int wave_first = run * PA_RUN + wave * WAVE;
   const int from = min(WAVE, max(0, first_key - wave_first));
   const int to = min(WAVE, max(0, query_position - wave_first + 1));
+  if (lane == 0) {
+    // the normalizer: the probabilities added up in the order of their keys (a sum whose order the keys fix,
+    // not the lanes: the tiled kernel below forms the same sum without a pass over the wave)
+    float normalizer = 0.f;
+    for (int j = from; j < to; ++j) normalizer += p_shared[wave][j];
+    wave_ml[wave][0] = maximum;
+    wave_ml[wave][1] = normalizer;
+  }
 #pragma unroll
   for (int i = 0; i < ATT_MAX_DH / WAVE; ++i) {
     const int dim = lane + i * WAVE;
     if (dim < dh) {
       float sum = 0.f;
       for (int j = from; j < to; ++j)
-        sum += p_shared[wave][j] * to_float(v_base[row_shared[wave][j] + (long)dim * page_size + offset_shared[wave][j]]);
+        sum = fmaf(p_shared[wave][j], to_float(v_base[row_shared[wave][j] + (long)dim * page_size + offset_shared[wave][j]]), sum);
       wave_o[wave][dim] = sum;
     }
   }
@@ -220,7 +224,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
 #pragma unroll
   for (int w = 0; w < PA_WAVES; ++w) {
     weight[w] = FAST_EXP ? __expf(wave_ml[w][0] - best) : expf(wave_ml[w][0] - best);
-    denominator += weight[w] * wave_ml[w][1];
+    denominator = fmaf(weight[w], wave_ml[w][1], denominator);
   }
   if (tid == 0) {
     mine[0] = best;
@@ -229,8 +233,247 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
   for (int dim = tid; dim < dh; dim += PA_RUN) {
     float sum = 0.f;
 #pragma unroll
-    for (int w = 0; w < PA_WAVES; ++w) sum += weight[w] * wave_o[w][dim];
+    for (int w = 0; w < PA_WAVES; ++w) sum = fmaf(weight[w], wave_o[w][dim], sum);
     mine[2 + dim] = sum;
+  }
+}
+
+// The same partial results for steps whose lanes hold several tokens, from a workgroup that takes PT_QUERIES
+// consecutive tokens of one lane, one query head and one run of PA_RUN keys: the run's keys and values go through
+// LDS once for all of its queries, 64 keys at a time (the per-token kernel above fetches them once a token: a
+// prompt of 2,048 tokens reads every key a thousand times).  A query's scores, softmax and sums are the per-token
+// kernel's, operation for operation: 64 keys a wave-sized group in the order of their positions, lane i scoring
+// key i with a dot product in ascending dims, the group's maximum and normalizer over the wave, lane d summing
+// dim d in ascending keys, the four groups of a run weighted and added in their order.  So a position's result is
+// the same bits from either kernel: whole prompts, portions and single tokens agree.
+// Wave w takes the queries w, w + 4, ... of the tile.
+// The largest value of a wave, in every lane: shifts within the rows of 16 lanes, then the last lane of a row
+// to the row behind it, then the last lane of the lower half to the upper half (the data-parallel primitives of
+// this GPU family; a maximum does not depend on the order it is taken in, so this is wave_max without six trips
+// through the LDS crossbar).
+template <int CONTROL, int ROW_MASK>
+__device__ __forceinline__ float dpp_or_minus_infinity(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, -INFINITY), __builtin_bit_cast(int, x),
+                                                               CONTROL, ROW_MASK, 0xf, false));
+}
+
+__device__ __forceinline__ float wave_max_dpp(float v) {
+  v = fmaxf(v, dpp_or_minus_infinity<0x111, 0xf>(v));      // row_shr:1
+  v = fmaxf(v, dpp_or_minus_infinity<0x112, 0xf>(v));      // row_shr:2
+  v = fmaxf(v, dpp_or_minus_infinity<0x114, 0xf>(v));      // row_shr:4
+  v = fmaxf(v, dpp_or_minus_infinity<0x118, 0xf>(v));      // row_shr:8: lane 15 of each row holds the row's maximum
+  v = fmaxf(v, dpp_or_minus_infinity<0x142, 0xa>(v));      // row_bcast:15 into rows 1 and 3
+  v = fmaxf(v, dpp_or_minus_infinity<0x143, 0xc>(v));      // row_bcast:31 into rows 2 and 3: lane 63 holds the wave's maximum
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+#define PT_QUERIES 16
+#define PT_PER_WAVE (PT_QUERIES / PA_WAVES)
+#define PT_PAD 4
+
+// DIMS: dims of a head a lane sums (1, 2 or 4: the head size in units of 64, rounded up)
+template <typename T, bool FAST_EXP, int DIMS>
+__global__ void __launch_bounds__(PA_RUN)
+paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int dh,
+                            const T* __restrict__ k_base, const T* __restrict__ v_base, long page_stride,
+                            int page_size, const int* __restrict__ block_tables, int max_pages,
+                            const int* __restrict__ query_tiles, int tile_tokens, const int* __restrict__ cu_seqlens,
+                            const int* __restrict__ positions, float scale, int window,
+                            const float* __restrict__ slopes, int runs, float* __restrict__ partial) {
+  typedef T vec4 __attribute__((ext_vector_type(4)));
+  extern __shared__ __align__(16) float tile_lds[];
+  const int k_ld = dh + PT_PAD;                      // a key's row in LDS
+  const int v_ld = WAVE + PT_PAD;                    // a dim's row of values in LDS
+  float* q_lds = tile_lds;                           // [PT_QUERIES][dh]
+  float* k_lds = q_lds + PT_QUERIES * dh;            // [64][k_ld]
+  float* v_lds = k_lds + WAVE * k_ld;                // [dh][v_ld]
+  float* p_lds = v_lds + dh * v_ld;                  // [PA_WAVES][64]
+  const int subtiles = tile_tokens / PT_QUERIES;
+  const int tile = blockIdx.x / subtiles;
+  const int head = blockIdx.y;
+  const int run = blockIdx.z;
+  const int lane_of_tile = query_tiles[2 * tile];
+  if (lane_of_tile < 0) return;                      // a row of the table that holds nothing (a step of fixed capacity)
+  const int first_row = query_tiles[2 * tile + 1] + (blockIdx.x - tile * subtiles) * PT_QUERIES;
+  const int lane_end = cu_seqlens[lane_of_tile + 1];
+  const int tile_end = min(query_tiles[2 * tile + 1] + tile_tokens, lane_end);
+  const int count = min(PT_QUERIES, tile_end - first_row);          // queries of this workgroup
+  if (count <= 0) return;
+  const int last_position = positions[first_row + count - 1];      // positions ascend within a lane
+  const int first_position = positions[first_row];
+  int tile_first_key = 0;                                           // the oldest key any query of the tile sees
+  if (window > 0 && first_position - window + 1 > 0) tile_first_key = first_position - window + 1;
+  if (run * PA_RUN > last_position || (run + 1) * PA_RUN <= tile_first_key) return;
+  const int kvh = head / (Hq / Hkv);
+  const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  const int* table = block_tables + (long)lane_of_tile * max_pages;
+  for (int index = tid; index < count * dh; index += PA_RUN) {
+    const int query = index / dh;
+    q_lds[index] = to_float(q[(long)(first_row + query) * q_ld + (long)head * dh + (index - query * dh)]);
+  }
+  // what a wave keeps of its queries' groups: (maximum, normalizer, sums of lane's dims), group by group
+  float group_max[PT_PER_WAVE][PA_WAVES], group_norm[PT_PER_WAVE][PA_WAVES], group_o[PT_PER_WAVE][PA_WAVES][DIMS];
+#pragma unroll
+  for (int i = 0; i < PT_PER_WAVE; ++i)
+#pragma unroll
+    for (int g = 0; g < PA_WAVES; ++g) {
+      group_max[i][g] = -INFINITY;
+      group_norm[i][g] = 0.f;
+#pragma unroll
+      for (int d = 0; d < DIMS; ++d) group_o[i][g][d] = 0.f;
+    }
+  int query_position[PT_PER_WAVE];
+#pragma unroll
+  for (int i = 0; i < PT_PER_WAVE; ++i) {
+    const int query = wave + i * PA_WAVES;
+    query_position[i] = query < count ? positions[first_row + query] : -1;
+  }
+
+  // one group of 64 keys; called with a constant group so that what a wave keeps of it stays in registers
+  auto take_group = [&](auto group_constant) {
+    constexpr int g = decltype(group_constant)::value;
+    const int group_first = run * PA_RUN + g * WAVE;
+    if (group_first > last_position || group_first + WAVE <= tile_first_key) return;       // the same for every thread
+    __syncthreads();                                    // the group before is read (and the queries are laid down)
+    // keys group_first .. group_first + 63 that some query of the tile sees; the others (cells never written,
+    // pages the request does not hold) are not fetched and lie in LDS as zeros that nobody multiplies
+    const int keys = min(WAVE, last_position - group_first + 1);
+    const int skipped = max(0, tile_first_key - group_first);      // keys before every query's window: their pages may be gone
+    {
+      // keys: four threads a key, each a quarter of its dims, 4 dims a load
+      const int key_in = tid >> 2;
+      const int quarter = dh >> 2;
+      const int dim0 = (tid & 3) * quarter;
+      float* to = k_lds + key_in * k_ld + dim0;
+      if (key_in < keys && key_in >= skipped) {
+        const int key = group_first + key_in;
+        const int page = table[key / page_size];
+        const T* from = k_base + (long)page * page_stride + ((long)kvh * page_size + key % page_size) * dh + dim0;
+        for (int d = 0; d < quarter; d += 4) {
+          const vec4 piece = *reinterpret_cast<const vec4*>(from + d);
+          *reinterpret_cast<float4*>(to + d) = make_float4(to_float<T>(piece[0]), to_float<T>(piece[1]),
+                                                           to_float<T>(piece[2]), to_float<T>(piece[3]));
+        }
+      } else {
+        for (int d = 0; d < quarter; d += 4) *reinterpret_cast<float4*>(to + d) = make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
+    {
+      // values: a thread a key (the lanes of a wave walk along a page's tokens), the waves take every fourth dim
+      const int key_in = lane;
+      if (key_in < keys && key_in >= skipped) {
+        const int key = group_first + key_in;
+        const int page = table[key / page_size];
+        const T* from = v_base + (long)page * page_stride + (long)kvh * dh * page_size + key % page_size;
+        for (int dim = wave; dim < dh; dim += PA_WAVES) v_lds[dim * v_ld + key_in] = to_float(from[(long)dim * page_size]);
+      } else {
+        for (int dim = wave; dim < dh; dim += PA_WAVES) v_lds[dim * v_ld + key_in] = 0.f;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < PT_PER_WAVE; ++i) {
+      const int position = query_position[i];
+      int first_key = 0;
+      if (window > 0 && position - window + 1 > 0) first_key = position - window + 1;
+      if (position >= group_first && group_first + WAVE > first_key) {           // else: no key of this group for the query
+      const int key = group_first + lane;
+      const bool visible = key >= first_key && key <= position;
+      float score = -INFINITY;
+      if (visible) {
+        const float* q_row = q_lds + (wave + i * PA_WAVES) * dh;
+        const float* k_row = k_lds + lane * k_ld;
+        float dot = 0.f;
+        for (int d = 0; d < dh; d += 4) {
+          const float4 qv = *reinterpret_cast<const float4*>(q_row + d);
+          const float4 kv = *reinterpret_cast<const float4*>(k_row + d);
+          dot = fmaf(qv.x, kv.x, dot);
+          dot = fmaf(qv.y, kv.y, dot);
+          dot = fmaf(qv.z, kv.z, dot);
+          dot = fmaf(qv.w, kv.w, dot);
+        }
+        score = dot * scale;
+        if (slopes) score = fmaf(-slopes[head], (float)(position - key), score);
+      }
+      const float maximum = wave_max_dpp(score);
+      const float p = visible ? (FAST_EXP ? __expf(score - maximum) : expf(score - maximum)) : 0.f;
+      p_lds[wave * WAVE + lane] = p;                  // read by this wave only: no barrier, the wave runs in step
+      __builtin_amdgcn_wave_barrier();
+      // sums over all 64 keys of the group: a key the query does not see has the probability 0 and a finite
+      // value (a key some query of the tile sees, or a zero laid down above), so it adds an exact zero and the
+      // sums are those of the keys from `from` to `to` in their order, which is what the per-token kernel adds
+      const float* p_row = p_lds + wave * WAVE;
+      float normalizer = 0.f;
+      float sums[DIMS] = {};
+      const float* v_row[DIMS];
+#pragma unroll
+      for (int d = 0; d < DIMS; ++d) v_row[d] = v_lds + min(lane + d * WAVE, dh - 1) * v_ld;
+#pragma unroll
+      for (int j = 0; j < WAVE; j += 4) {
+        const float4 pj = *reinterpret_cast<const float4*>(p_row + j);
+        normalizer += pj.x;
+        normalizer += pj.y;
+        normalizer += pj.z;
+        normalizer += pj.w;
+#pragma unroll
+        for (int d = 0; d < DIMS; ++d) {
+          if (d * WAVE < dh) {                          // the same for every lane
+            const float4 vj = *reinterpret_cast<const float4*>(v_row[d] + j);
+            sums[d] = fmaf(pj.x, vj.x, sums[d]);
+            sums[d] = fmaf(pj.y, vj.y, sums[d]);
+            sums[d] = fmaf(pj.z, vj.z, sums[d]);
+            sums[d] = fmaf(pj.w, vj.w, sums[d]);
+          }
+        }
+      }
+      group_max[i][g] = maximum;
+      group_norm[i][g] = normalizer;
+#pragma unroll
+      for (int d = 0; d < DIMS; ++d) group_o[i][g][d] = sums[d];
+      __builtin_amdgcn_wave_barrier();
+      }
+    }
+  };
+  take_group(std::integral_constant<int, 0>{});
+  take_group(std::integral_constant<int, 1>{});
+  take_group(std::integral_constant<int, 2>{});
+  take_group(std::integral_constant<int, 3>{});
+  static_assert(PA_WAVES == 4, "a run of keys is four groups of 64");
+  // the groups of the run in their order, as the per-token kernel merges its waves
+#pragma unroll
+  for (int i = 0; i < PT_PER_WAVE; ++i) {
+    const int position = query_position[i];
+    int first_key = 0;
+    if (window > 0 && position - window + 1 > 0) first_key = position - window + 1;
+    if (position < 0 || (run + 1) * PA_RUN <= first_key || run * PA_RUN > position) continue;    // the per-token kernel writes nothing either
+    float best = group_max[i][0];
+#pragma unroll
+    for (int g = 1; g < PA_WAVES; ++g) best = fmaxf(best, group_max[i][g]);
+    float weight[PA_WAVES];
+    float denominator = 0.f;
+#pragma unroll
+    for (int g = 0; g < PA_WAVES; ++g) {
+      weight[g] = FAST_EXP ? __expf(group_max[i][g] - best) : expf(group_max[i][g] - best);
+      denominator = fmaf(weight[g], group_norm[i][g], denominator);
+    }
+    const long token = first_row + wave + i * PA_WAVES;
+    float* mine = partial + ((token * Hq + head) * runs + run) * (long)(dh + 2);
+    if (lane == 0) {
+      mine[0] = best;
+      mine[1] = denominator;
+    }
+#pragma unroll
+    for (int d = 0; d < DIMS; ++d) {
+      const int dim = lane + d * WAVE;
+      if (dim < dh) {
+        float sum = 0.f;
+#pragma unroll
+        for (int g = 0; g < PA_WAVES; ++g) sum = fmaf(weight[g], group_o[i][g][d], sum);
+        mine[2 + dim] = sum;
+      }
+    }
   }
 }
 
@@ -270,11 +513,36 @@ extern "C" long mi_paged_attention_workspace(int T, int Hq, int dh, int max_seq_
   return (long)T * Hq * ((max_seq_len + PA_RUN - 1) / PA_RUN) * (dh + 2);
 }
 
+// LDS of a workgroup of the tiled kernel: the tile's queries, 64 keys, their values, a wave's probabilities
+static size_t paged_attention_tile_lds(int dh) {
+  return ((size_t)PT_QUERIES * dh + (size_t)WAVE * (dh + PT_PAD) + (size_t)dh * (WAVE + PT_PAD) + PA_RUN) * sizeof(float);
+}
+
+template <typename T, bool FAST_EXP, int DIMS>
+static int raise_tile_lds(size_t bytes) {
+  // beyond 64 KiB a kernel has to be told once per device that it may have that much (gfx950 has 160 KiB)
+  static bool raised[64] = {};          // per instantiation of this function
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return ERR_BAD_ARGUMENT;
+  if (raised[device]) return 0;
+  if (hipFuncSetAttribute((const void*)paged_attention_tile_kernel<T, FAST_EXP, DIMS>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return ERR_UNSUPPORTED_SIZE;
+  }
+  raised[device] = true;
+  return 0;
+}
+
+// query_tiles (optional) [num_tiles, 2] = (lane or -1, first token row) of runs of up to tile_tokens tokens of one
+// lane (tile_tokens a multiple of 16), with cu_seqlens [lanes + 1]: the step's lanes hold several tokens, and the
+// partial results come from the kernel that shares a run's keys among the queries of a tile (the same bits).
 extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, int Hq, int Hkv, int dh,
                                   const void* k_base, const void* v_base, long page_stride, int page_size,
                                   const int* block_tables, int max_pages, const int* lane_of_token,
                                   const int* positions, float scale, int window, const float* slopes,
                                   int max_seq_len, float* partial, long partial_floats, void* out, long out_ld,
+                                  const int* query_tiles, int num_tiles, int tile_tokens, const int* cu_seqlens,
                                   hipStream_t stream) {
   if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || dh <= 0 || page_size <= 0 || max_pages <= 0 ||
       max_seq_len <= 0 || !partial)
@@ -283,26 +551,53 @@ extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, in
   const int runs = (max_seq_len + PA_RUN - 1) / PA_RUN;
   if (Hq > 65535 || runs > 65535) return ERR_UNSUPPORTED_SIZE;
   if (partial_floats < mi_paged_attention_workspace(T, Hq, dh, max_seq_len)) return ERR_BAD_ARGUMENT;
+  const int element = dtype == DT_F32 ? 4 : 2;
+  // the tiled kernel: head sizes in steps of 16, 4 elements a load from the cache
+  bool tiled = query_tiles != nullptr && num_tiles > 0 && cu_seqlens != nullptr && tile_tokens > 0 &&
+               tile_tokens % PT_QUERIES == 0 && dh % 16 == 0 && page_stride % 4 == 0 &&
+               ((uintptr_t)k_base % (4 * element)) == 0 && (long)num_tiles * (tile_tokens / PT_QUERIES) <= 0x7fffffffL;
+  const size_t tile_lds = paged_attention_tile_lds(dh);
+  const int dims = dh <= WAVE ? 1 : dh <= 2 * WAVE ? 2 : 4;
+  if (tiled && tile_lds > 64 * 1024) {
+    int code;
+    if (dtype == DT_F32) code = dims == 2 ? raise_tile_lds<float, false, 2>(tile_lds) : raise_tile_lds<float, false, 4>(tile_lds);
+    else code = dims == 2 ? raise_tile_lds<bf16_t, true, 2>(tile_lds) : raise_tile_lds<bf16_t, true, 4>(tile_lds);
+    if (code != 0) tiled = false;                      // the per-token kernel takes any size
+  }
   const dim3 grid(T, Hq, runs);
+  const dim3 tile_grid(tiled ? num_tiles * (tile_tokens / PT_QUERIES) : 1, Hq, runs);
   const dim3 merge_grid(T, Hq);
   const int merge_threads = dh <= WAVE ? WAVE : dh <= 2 * WAVE ? 2 * WAVE : 4 * WAVE;
   if (dtype == DT_F32) {
-    paged_attention_kernel<float, false><<<grid, PA_RUN, 0, stream>>>(
-        (const float*)q, q_ld, Hq, Hkv, dh, (const float*)k_base, (const float*)v_base, page_stride, page_size,
-        block_tables, max_pages, lane_of_token, positions, scale, window, slopes, runs, partial);
+#define TILE_LAUNCH(T_, FAST_, DIMS_)                                                                                 \
+  paged_attention_tile_kernel<T_, FAST_, DIMS_><<<tile_grid, PA_RUN, tile_lds, stream>>>(                              \
+      (const T_*)q, q_ld, Hq, Hkv, dh, (const T_*)k_base, (const T_*)v_base, page_stride, page_size, block_tables,     \
+      max_pages, query_tiles, tile_tokens, cu_seqlens, positions, scale, window, slopes, runs, partial)
+    if (tiled && dims == 1) TILE_LAUNCH(float, false, 1);
+    else if (tiled && dims == 2) TILE_LAUNCH(float, false, 2);
+    else if (tiled) TILE_LAUNCH(float, false, 4);
+    else
+      paged_attention_kernel<float, false><<<grid, PA_RUN, 0, stream>>>(
+          (const float*)q, q_ld, Hq, Hkv, dh, (const float*)k_base, (const float*)v_base, page_stride, page_size,
+          block_tables, max_pages, lane_of_token, positions, scale, window, slopes, runs, partial);
     RETURN_IF_LAUNCH_FAILED();
     paged_attention_merge_kernel<float, false><<<merge_grid, merge_threads, 0, stream>>>(
         partial, Hq, dh, runs, positions, window, (float*)out, out_ld);
   } else if (dtype == DT_BF16) {
-    paged_attention_kernel<bf16_t, true><<<grid, PA_RUN, 0, stream>>>(
-        (const bf16_t*)q, q_ld, Hq, Hkv, dh, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride,
-        page_size, block_tables, max_pages, lane_of_token, positions, scale, window, slopes, runs, partial);
+    if (tiled && dims == 1) TILE_LAUNCH(bf16_t, true, 1);
+    else if (tiled && dims == 2) TILE_LAUNCH(bf16_t, true, 2);
+    else if (tiled) TILE_LAUNCH(bf16_t, true, 4);
+    else
+      paged_attention_kernel<bf16_t, true><<<grid, PA_RUN, 0, stream>>>(
+          (const bf16_t*)q, q_ld, Hq, Hkv, dh, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride,
+          page_size, block_tables, max_pages, lane_of_token, positions, scale, window, slopes, runs, partial);
     RETURN_IF_LAUNCH_FAILED();
     paged_attention_merge_kernel<bf16_t, true><<<merge_grid, merge_threads, 0, stream>>>(
         partial, Hq, dh, runs, positions, window, (bf16_t*)out, out_ld);
   } else {
     return ERR_BAD_ARGUMENT;
   }
+#undef TILE_LAUNCH
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

@@ -261,70 +261,316 @@ extern "C" int mi_conv_step(void* u, int dtype, long ld, int col_offset, int M, 
 //   delta = softplus(dt + dt_bias[h]);  s = exp(delta*A[h]) * s + delta * x[p] * B[g, :];
 //   y[p] = s . C[g, :] + D[h] * x[p]
 // (reference: crates/macllm-kernels/src/mamba2.rs:259-288, metal/mamba2_scan.metal:45-77).
-// A state row is spread over R lanes of a wavefront (R = power of two <= 64), each holding
-// up to SCAN_MAX_PER_THREAD strided elements; 256/R rows per block.
+// A state row is spread over R lanes of a wavefront (R = power of two <= 64), each holding PER neighbouring
+// elements (1, 2, 4 or 8: the smallest number that covers N; one load where alignment allows); 256/R rows per block.
+//
+// The recurrence is serial in the tokens, so what a token costs is what its step waits for.  The tokens of a
+// lane come in blocks of 16 / PER (8 at most): a block's B, C, x and dt are asked for four blocks ahead, each element
+// once a workgroup, laid in LDS one block ahead, and read from there into the registers of the threads that use them
+// before the block's first token; softplus and the exponential are taken once a token, not once a thread; what the lanes of a row add up for a
+// token's output goes to LDS and is added up for the whole block at its end, in the order of the lanes (a pass
+// over the wave for every token costs more than the token's own arithmetic).  Every token goes through the same
+// operations in the same order whatever block it falls into, and in the kernel for steps of single tokens
+// (SINGLE: nothing staged, few registers, many workgroups a compute unit): a step of one token and a prompt of
+// thousands give a position the same bits.
 #define SCAN_MAX_PER_THREAD 8
+#define SCAN_BLOCK_ELEMENTS 16      // tokens of a block times PER
+#define SCAN_STAGE_PIECES (SCAN_BLOCK_ELEMENTS / 2)   // loads of four elements of B|C a lane of the wave whose turn it is sends for
 
-template <typename T>
-__global__ void __launch_bounds__(256)
+// The shares of a row's R lanes as one sum: four quarters of the row (two halves of two lanes, one lane), each
+// added up in the order of its lanes, then ((q0 + q1) + q2) + q3.  scan_part_sum is one quarter; scan_row_sum all
+// of it in one thread; four threads that take a quarter each and then add the four in that order get the same bits.
+__device__ __forceinline__ float scan_part_sum(const float* shares, int R, int part) {
+  const int width = R >= 4 ? R / 4 : 1;
+  const float* mine = shares + part * width;
+  float sum = 0.f;
+#pragma unroll 16
+  for (int index = 0; index < width; ++index) sum += mine[index];
+  return sum;
+}
+
+__device__ __forceinline__ float scan_join_parts(float q0, float q1, float q2, float q3, int R) {
+  float sum = q0;
+  if (R >= 2) sum += q1;
+  if (R >= 4) sum = (sum + q2) + q3;
+  return sum;
+}
+
+__device__ __forceinline__ float scan_row_sum(const float* shares, int R) {
+  return scan_join_parts(scan_part_sum(shares, R, 0), R >= 2 ? scan_part_sum(shares, R, 1) : 0.f,
+                         R >= 4 ? scan_part_sum(shares, R, 2) : 0.f, R >= 4 ? scan_part_sum(shares, R, 3) : 0.f, R);
+}
+
+// A barrier of the workgroup for what went through LDS, and nothing else.  __syncthreads() also waits for every load
+// from memory that is under way (its fences order all memory), and the loads for the blocks ahead are meant to stay
+// under way across the barriers of the block that is being scanned.
+__device__ __forceinline__ void scan_lds_barrier() {
+  __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): this wave's LDS reads and writes are done; vmcnt, expcnt: any
+  __builtin_amdgcn_s_barrier();
+}
+
+// lane `which` of every group of four lanes, in all four (the data-parallel quad permutation)
+template <int WHICH>
+__device__ __forceinline__ float scan_quad_lane(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), WHICH * 0x55, 0xf, 0xf, true));
+}
+
+// VECTORS (staged kernel only): B and C come four neighbouring elements a load (N, the row stride and the columns
+// of B are multiples of 4 and the rows 16-byte aligned); else element by element.
+template <typename T, int PER, bool SINGLE, bool VECTORS>
+__global__ void __launch_bounds__(256, 2)          // two workgroups a compute unit at least
 ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt, long dt_ld,
                 const float* __restrict__ dt_bias, const float* __restrict__ A, const float* __restrict__ D,
                 float* __restrict__ state, const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids,
-                int H, int P, int N, int G, int R, float* __restrict__ y, long y_ld) {
+                int H, int P, int N, int G, int R, int block_tokens, float* __restrict__ y, long y_ld) {
+  constexpr int TB = PER == 1 ? SCAN_BLOCK_ELEMENTS / 2 : SCAN_BLOCK_ELEMENTS / PER;    // tokens of a block at most (block_tokens <= TB: a block's x
+                                                       // values are one a thread)
+  extern __shared__ __align__(16) float shares_l[];    // [tokens of a block][rows_per_block][R shares, then the row's x]
+  __shared__ float decay_l[2][TB], delta_l[2][TB];
   const int lane = blockIdx.z;
   const int head = blockIdx.y;
-  const int rows_per_block = blockDim.x / R;
-  const int row_in_block = threadIdx.x / R;
-  const int r = threadIdx.x - row_in_block * R;
-  const int p = blockIdx.x * rows_per_block + row_in_block;
+  const int tid = threadIdx.x;
+  const int rows_per_block = 256 / R;
+  const int row_in_block = tid / R;
+  const int r = tid - row_in_block * R;
+  const int p0 = blockIdx.x * rows_per_block;
+  const int p = p0 + row_in_block;
   const bool active = p < P;
   const int group = head / (H / G);
   const int E = H * P;
   const long t_begin = cu_seqlens[lane];
   const long t_end = cu_seqlens[lane + 1];
+  if (t_end <= t_begin) return;                        // a lane without tokens (padding of a fixed capacity)
   float* s_row = state + (((long)slot_ids[lane] * H + head) * P + (active ? p : 0)) * N;
-  float s[SCAN_MAX_PER_THREAD];
+  float s[PER];
 #pragma unroll
-  for (int i = 0; i < SCAN_MAX_PER_THREAD; ++i) {
-    const int n = r + i * R;
+  for (int i = 0; i < PER; ++i) {
+    const int n = r * PER + i;
     s[i] = (active && n < N) ? s_row[n] : 0.f;
   }
   const float a = A[head];
   const float bias = dt_bias[head];
   const float skip = D[head];
-  for (long t = t_begin; t < t_end; ++t) {
-    const T* row = xbc + t * xbc_ld;
-    const float delta = softplus_f(to_float(dt[t * dt_ld + head]) + bias);
-    const float decay = expf(delta * a);
-    const float x = active ? to_float(row[(long)head * P + p]) : 0.f;
-    const T* b_row = row + E + (long)group * N;
-    const T* c_row = row + E + (long)G * N + (long)group * N;
-    const float dx = delta * x;
-    float partial = 0.f;
+  // the state is waited for here, once: left to the compiler, the wait lands inside the loop over the blocks, where
+  // it also waits for the loads of the blocks ahead, every time round
+  __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0)
+  const long b_col = E + (long)group * N;
+  const long c_col = E + (long)G * N + (long)group * N;
+  const long x_col = (long)head * P + (active ? p : 0);
+  const int share_ld = R + 1;
+  const int token_ld = rows_per_block * share_ld;
+
+  if (SINGLE) {
+    for (long t = t_begin; t < t_end; ++t) {
+      const T* row = xbc + t * xbc_ld;
+      const float delta = softplus_f(to_float(dt[t * dt_ld + head]) + bias);
+      const float decay = expf(delta * a);
+      const float x = active ? to_float(row[x_col]) : 0.f;
+      const float dx = delta * x;
+      float partial = 0.f;
 #pragma unroll
-    for (int i = 0; i < SCAN_MAX_PER_THREAD; ++i) {
-      const int n = r + i * R;
-      if (n < N) {
-        const float next = decay * s[i] + dx * to_float(b_row[n]);
-        s[i] = next;
-        partial += next * to_float(c_row[n]);
+      for (int i = 0; i < PER; ++i) {
+        const int n = r * PER + i;
+        if (n < N) {
+          const float next = fmaf(decay, s[i], dx * to_float(row[b_col + n]));
+          s[i] = next;
+          partial = fmaf(next, to_float(row[c_col + n]), partial);
+        }
+      }
+      shares_l[row_in_block * share_ld + r] = partial;
+      if (r == 0) shares_l[row_in_block * share_ld + R] = x;
+      __syncthreads();
+      if (tid < rows_per_block && p0 + tid < P) {
+        const float* shares = shares_l + tid * share_ld;
+        y[t * y_ld + (long)head * P + p0 + tid] = fmaf(skip, shares[R], scan_row_sum(shares, R));
+      }
+      __syncthreads();
+    }
+  } else {
+    // A block's B, C, x and dt are brought in by one of the workgroup's four waves, the waves taking turns: wave w
+    // asks for the blocks w, w + 4, ... into its registers, four blocks before their turn, and lays a block in LDS
+    // while the block before it is added up.  A wave's loads therefore have four blocks' time to arrive, and the
+    // wait for them (which a wave can only state for all of its loads at once) never meets a load that was asked
+    // for a moment ago.  Every element comes in once a workgroup: the rows of a head, and the heads of a group,
+    // read the same B and C.
+    float* b_l = shares_l + block_tokens * token_ld;            // [2][block_tokens][2 N]: B then C of a token
+    float* x_l = b_l + 2 * block_tokens * 2 * N;                // [2][block_tokens][rows_per_block]
+    typedef T pieces __attribute__((ext_vector_type(4)));
+    const int row_floats = 2 * N;
+    const int pieces_a_row = (row_floats + 3) / 4;
+    const bool whole_rows = N == R * PER && block_tokens == TB;          // no lane of a row is idle, blocks are of TB tokens
+    const int wave = tid / WAVE;
+    const int lane64 = tid % WAVE;
+    float staged_bc[SCAN_STAGE_PIECES][4], staged_x[4], staged_dt = 0.f;
+    // where this lane's pieces lie in a block (the same for every block: worked out once, a division each)
+    int piece_token[SCAN_STAGE_PIECES], piece_col[SCAN_STAGE_PIECES];
+#pragma unroll
+    for (int j = 0; j < SCAN_STAGE_PIECES; ++j) {
+      const int index = lane64 + j * WAVE;
+      piece_token[j] = index / pieces_a_row;
+      piece_col[j] = (index - piece_token[j] * pieces_a_row) * 4;
+    }
+    const int rows_shift = __ffs(rows_per_block) - 1;               // rows_per_block is a power of two
+    // block `block` of the lane into this wave's registers (nothing if the lane has no such block)
+    auto fetch = [&](int block) {
+      const long t0 = t_begin + (long)block * block_tokens;
+      const int count = (int)max(0L, min((long)block_tokens, t_end - t0));
+      if (count <= 0) return;
+#pragma unroll
+      for (int j = 0; j < SCAN_STAGE_PIECES; ++j) {
+        const int token = min(piece_token[j], count - 1);           // a piece past the block reads its last token, unused
+        const int col = piece_col[j];
+        if (VECTORS) {
+          // B and C of a group lie apart in a row: columns N .. 2 N of the staged row are C
+          const pieces four = *reinterpret_cast<const pieces*>(xbc + (t0 + token) * xbc_ld + (col < N ? b_col + col : c_col + (col - N)));
+#pragma unroll
+          for (int i = 0; i < 4; ++i) staged_bc[j][i] = to_float<T>(four[i]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {                         // element by element: a piece may straddle B and C
+            const int at = min(col + i, row_floats - 1);
+            staged_bc[j][i] = to_float(xbc[(t0 + token) * xbc_ld + (at < N ? b_col + at : c_col + (at - N))]);
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int index = min(lane64 + j * WAVE, count * rows_per_block - 1);
+        const int token = index >> rows_shift;
+        const int row = p0 + index - (token << rows_shift);
+        staged_x[j] = row < P ? to_float(xbc[(t0 + token) * xbc_ld + (long)head * P + row]) : 0.f;
+      }
+      staged_dt = to_float(dt[(t0 + min(lane64, count - 1)) * dt_ld + head]);
+    };
+    // this wave's registers (block `block`) into LDS: B, C and x as they are, dt as delta and decay
+    auto lay_down = [&](int block) {
+      const long t0 = t_begin + (long)block * block_tokens;
+      const int count = (int)max(0L, min((long)block_tokens, t_end - t0));
+      if (count <= 0) return;
+      const int phase = block & 1;
+      float* rows_l = b_l + phase * block_tokens * row_floats;
+#pragma unroll
+      for (int j = 0; j < SCAN_STAGE_PIECES; ++j) {
+        const int token = piece_token[j];
+        const int col = piece_col[j];
+        if (token < count) {
+          float* to = rows_l + token * row_floats + col;
+          if (VECTORS) {
+            *reinterpret_cast<float4*>(to) = make_float4(staged_bc[j][0], staged_bc[j][1], staged_bc[j][2], staged_bc[j][3]);
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (col + i < row_floats) to[i] = staged_bc[j][i];
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (lane64 + j * WAVE < count * rows_per_block) x_l[phase * block_tokens * rows_per_block + lane64 + j * WAVE] = staged_x[j];
+      if (lane64 < count) {
+        const float delta = softplus_f(staged_dt + bias);
+        delta_l[phase][lane64] = delta;
+        decay_l[phase][lane64] = expf(delta * a);
+      }
+    };
+    fetch(wave);                             // blocks 0 .. 3, one a wave
+    if (wave == 0) {
+      lay_down(0);
+      fetch(4);
+    }
+    const int blocks = (int)((t_end - t_begin + block_tokens - 1) / block_tokens);
+    for (int block = 0; block < blocks; ++block) {
+      const long t0 = t_begin + (long)block * block_tokens;
+      const int count = (int)min((long)block_tokens, t_end - t0);
+      const int phase = block & 1;
+      scan_lds_barrier();                   // this block's operands are laid down, and the block before has been
+                                            // added up: its shares may be overwritten
+      const float* rows_l = b_l + phase * block_tokens * row_floats;
+      const float* x_now = x_l + phase * block_tokens * rows_per_block + row_in_block;
+      const float* mine_l = rows_l + min(r * PER, N - PER > 0 ? N - PER : 0);    // this thread's columns of B (C: N further)
+      float* shares_mine = shares_l + row_in_block * share_ld + r;
+      // a whole block of a row whose lanes all hold PER elements runs without a condition: straight code whose
+      // LDS addresses are constants; the last block of a lane and rows with idle lanes take the guarded loop
+      if (count == TB && whole_rows) {
+        float b[TB][PER], c[TB][PER], decay[TB], dx[TB], x[TB];
+#pragma unroll
+        for (int token = 0; token < TB; ++token) {
+          decay[token] = decay_l[phase][token];
+          x[token] = x_now[token * rows_per_block];
+          dx[token] = delta_l[phase][token] * x[token];
+#pragma unroll
+          for (int i = 0; i < PER; ++i) {
+            b[token][i] = mine_l[token * row_floats + i];
+            c[token][i] = mine_l[token * row_floats + N + i];
+          }
+        }
+#pragma unroll
+        for (int token = 0; token < TB; ++token) {
+          float partial = 0.f;
+#pragma unroll
+          for (int i = 0; i < PER; ++i) {
+            const float next_s = fmaf(decay[token], s[i], dx[token] * b[token][i]);
+            s[i] = next_s;
+            partial = fmaf(next_s, c[token][i], partial);
+          }
+          shares_mine[token * token_ld] = partial;
+          if (r == 0) shares_mine[token * token_ld + R] = x[token];
+        }
+      } else {
+        for (int token = 0; token < count; ++token) {
+          const float decay = decay_l[phase][token];
+          const float x = x_now[token * rows_per_block];
+          const float dx = delta_l[phase][token] * x;
+          float partial = 0.f;
+#pragma unroll
+          for (int i = 0; i < PER; ++i) {
+            const int n = r * PER + i;
+            if (n < N) {
+              const float next_s = fmaf(decay, s[i], dx * rows_l[token * row_floats + n]);
+              s[i] = next_s;
+              partial = fmaf(next_s, rows_l[token * row_floats + N + n], partial);
+            }
+          }
+          shares_mine[token * token_ld] = partial;
+          if (r == 0) shares_mine[token * token_ld + R] = x;
+        }
+      }
+      scan_lds_barrier();
+      // the wave whose turn it is lays the next block down and asks for the block four after that one
+      if (wave == ((block + 1) & 3)) {
+        lay_down(block + 1);
+        fetch(block + 5);
+      }
+      // four threads an output, a quarter of the row's shares each
+      const int outputs = count * rows_per_block;
+      for (int first = 0; first < outputs; first += 64) {
+        const int index = min(first + tid / 4, outputs - 1);
+        const int token = index >> rows_shift;
+        const int row = index - (token << rows_shift);
+        const float* shares = shares_l + token * token_ld + row * share_ld;
+        const int part = tid & 3;
+        const float quarter = (part == 0 || R >= 4 || (part == 1 && R >= 2)) ? scan_part_sum(shares, R, part) : 0.f;
+        const float sum = scan_join_parts(scan_quad_lane<0>(quarter), scan_quad_lane<1>(quarter), scan_quad_lane<2>(quarter),
+                                          scan_quad_lane<3>(quarter), R);
+        if (part == 0 && first + tid / 4 < outputs && p0 + row < P)
+          y[(t0 + token) * y_ld + (long)head * P + p0 + row] = fmaf(skip, shares[R], sum);
       }
     }
-    for (int offset = R / 2; offset > 0; offset >>= 1) partial += __shfl_xor(partial, offset, WAVE);
-    if (active && r == 0) y[t * y_ld + (long)head * P + p] = partial + skip * x;
   }
   if (active) {
 #pragma unroll
-    for (int i = 0; i < SCAN_MAX_PER_THREAD; ++i) {
-      const int n = r + i * R;
+    for (int i = 0; i < PER; ++i) {
+      const int n = r * PER + i;
       if (n < N) s_row[n] = s[i];
     }
   }
 }
 
+// longest: an upper bound of the tokens of a lane (0: unknown); a step whose lanes all hold one token takes the
+// kernel without staging.
 extern "C" int mi_ssm_scan(const void* xbc, int dtype, long xbc_ld, const void* dt, long dt_ld,
                            const float* dt_bias, const float* A, const float* D, float* state,
-                           const int* cu_seqlens, const int* slot_ids, int num_lanes, int H, int P, int N,
+                           const int* cu_seqlens, const int* slot_ids, int num_lanes, int longest, int H, int P, int N,
                            int G, float* y, long y_ld, hipStream_t stream) {
   if (num_lanes <= 0 || H <= 0 || P <= 0 || N <= 0 || G <= 0 || H % G != 0) return ERR_BAD_ARGUMENT;
   if (N > WAVE * SCAN_MAX_PER_THREAD) return ERR_UNSUPPORTED_SIZE;
@@ -333,15 +579,43 @@ extern "C" int mi_ssm_scan(const void* xbc, int dtype, long xbc_ld, const void* 
   while (R < N && R < WAVE) R <<= 1;
   const int rows_per_block = 256 / R;
   const dim3 grid((P + rows_per_block - 1) / rows_per_block, H, num_lanes);
-  if (dtype == DT_F32)
-    ssm_scan_kernel<float><<<grid, 256, 0, stream>>>((const float*)xbc, xbc_ld, (const float*)dt, dt_ld, dt_bias,
-                                                      A, D, state, cu_seqlens, slot_ids, H, P, N, G, R, y, y_ld);
-  else if (dtype == DT_BF16)
-    ssm_scan_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)xbc, xbc_ld, (const bf16_t*)dt, dt_ld,
-                                                       dt_bias, A, D, state, cu_seqlens, slot_ids, H, P, N, G, R,
-                                                       y, y_ld);
-  else
-    return ERR_BAD_ARGUMENT;
+  const int per_needed = (N + R - 1) / R;
+  const int per = per_needed <= 1 ? 1 : per_needed <= 2 ? 2 : per_needed <= 4 ? 4 : 8;
+  const bool single = longest == 1;
+  // tokens of a block: 16 / PER (8 at most), no more than R (so that a block's x values, one a row and token, are at most 256), and
+  // B and C of a block are no more than the wave whose turn it is sends for
+  int block_tokens = per == 1 ? SCAN_BLOCK_ELEMENTS / 2 : SCAN_BLOCK_ELEMENTS / per;
+  if (block_tokens > R) block_tokens = R;
+  while (block_tokens > 1 && (long)block_tokens * 2 * N > (long)WAVE * 4 * SCAN_STAGE_PIECES) block_tokens /= 2;
+  if (single) block_tokens = 1;
+  const size_t bytes = ((size_t)block_tokens * rows_per_block * (R + 1) +
+                        (single ? 0 : 2 * (size_t)block_tokens * (2 * N + rows_per_block))) * sizeof(float);
+  // four elements a load: every head's and group's columns of B and C start at multiples of 4
+  const bool vectors = !single && N % 4 == 0 && xbc_ld % 4 == 0 && ((long)H * P) % 4 == 0 &&
+                       ((uintptr_t)xbc % (dtype == DT_F32 ? 16 : 8)) == 0;
+#define SCAN_LAUNCH(T_, PER_, SINGLE_, VECTORS_)                                                                     \
+  ssm_scan_kernel<T_, PER_, SINGLE_, VECTORS_><<<grid, 256, bytes, stream>>>(                                        \
+      (const T_*)xbc, xbc_ld, (const T_*)dt, dt_ld, dt_bias, A, D, state, cu_seqlens, slot_ids, H, P, N, G, R,       \
+      block_tokens, y, y_ld)
+#define SCAN_BY_PER(T_, SINGLE_, VECTORS_)                     \
+  do {                                                         \
+    if (per == 1) SCAN_LAUNCH(T_, 1, SINGLE_, VECTORS_);       \
+    else if (per == 2) SCAN_LAUNCH(T_, 2, SINGLE_, VECTORS_);  \
+    else if (per == 4) SCAN_LAUNCH(T_, 4, SINGLE_, VECTORS_);  \
+    else SCAN_LAUNCH(T_, 8, SINGLE_, VECTORS_);                \
+  } while (0)
+#define SCAN_BY_KIND(T_)                               \
+  do {                                                 \
+    if (single) SCAN_BY_PER(T_, true, false);          \
+    else if (vectors) SCAN_BY_PER(T_, false, true);    \
+    else SCAN_BY_PER(T_, false, false);                \
+  } while (0)
+  if (dtype == DT_F32) SCAN_BY_KIND(float);
+  else if (dtype == DT_BF16) SCAN_BY_KIND(bf16_t);
+  else return ERR_BAD_ARGUMENT;
+#undef SCAN_BY_KIND
+#undef SCAN_BY_PER
+#undef SCAN_LAUNCH
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

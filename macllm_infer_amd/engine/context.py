@@ -50,6 +50,7 @@ class StepContext:
     slot_ids: torch.Tensor           # [lanes] state slot of each lane's request
     want_rows: torch.Tensor          # [wanted] token rows whose logits are returned
     query_tiles: torch.Tensor        # [tiles, 2] (lane, first token row) of runs of up to ``query_tile`` tokens of one lane
+    query_tile: int = 0              # the longest run of that table (0: one run a lane, whatever its length)
     block_tables: List[torch.Tensor] = field(default_factory=list)   # per group [lanes, max_pages]
     slot_mappings: List[torch.Tensor] = field(default_factory=list)  # per group [T] page*page_size+offset
     lane_lengths: Optional[List[int]] = field(default_factory=list)   # host copies; None in a step of fixed capacity
@@ -160,7 +161,7 @@ def _pack(lowered: LoweredLanes, cache, out: Optional[np.ndarray], pad_lengths: 
 
 
 def _assemble(views, group_shapes, lengths, starts, max_seq_len, chunk_sizes=(), num_tokens=None, num_lanes=None,
-              max_query_len=None) -> StepContext:
+              max_query_len=None, query_tile: int = 0) -> StepContext:
     """``lengths`` / ``starts``: the lanes' host copies, or None for a step of fixed capacity, whose lanes
     differ from fill to fill (``num_tokens``, ``num_lanes`` and ``max_query_len`` are then its capacities)."""
     tokens = sum(lengths) if lengths is not None else num_tokens
@@ -168,7 +169,7 @@ def _assemble(views, group_shapes, lengths, starts, max_seq_len, chunk_sizes=(),
     context = StepContext(
         num_tokens=tokens, num_lanes=lanes, token_ids=views[0], positions=views[1],
         lane_of_token=views[2], cu_seqlens=views[3], start_pos=views[4], seq_lens=views[5], slot_ids=views[6],
-        want_rows=views[7], query_tiles=views[8].view(-1, 2),
+        want_rows=views[7], query_tiles=views[8].view(-1, 2), query_tile=int(query_tile or 0),
         lane_lengths=list(lengths) if lengths is not None else None,
         lane_starts=list(starts) if starts is not None else None,
         max_query_len=max(lengths) if lengths is not None else max_query_len, max_seq_len=max_seq_len)
@@ -203,7 +204,8 @@ def build_step_context(lanes: Sequence[Lane], cache, device, lowered: Optional[L
     _, sizes, shapes, longest, _ = _pack(lowered, cache, host.numpy(), query_tile=query_tile, chunk_sizes=chunk_sizes)
     packed = host.to(device, non_blocking=True)
     starts = cache.lengths_of(lowered.slots).tolist()
-    context = _assemble(_split(packed, sizes), shapes, lowered.lengths.tolist(), starts, longest, chunk_sizes)
+    context = _assemble(_split(packed, sizes), shapes, lowered.lengths.tolist(), starts, longest, chunk_sizes,
+                        query_tile=query_tile)
     context._keepalive = host
     return context
 
@@ -266,10 +268,11 @@ class StaticStep:
         self.device_buffer.copy_(self._hosts[0])
         if self.capacity:
             self.context = _assemble(_split(self.device_buffer, sizes), shapes, None, None, max_seq_len,
-                                     self.chunk_sizes, num_tokens=tokens, num_lanes=lanes, max_query_len=tokens)
+                                     self.chunk_sizes, num_tokens=tokens, num_lanes=lanes, max_query_len=tokens,
+                                     query_tile=query_tile)
         else:
             self.context = _assemble(_split(self.device_buffer, sizes), shapes, self.lengths, [0] * lanes, max_seq_len,
-                                     self.chunk_sizes)
+                                     self.chunk_sizes, query_tile=query_tile)
 
     HOST_BUFFERS = 2
 

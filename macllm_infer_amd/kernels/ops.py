@@ -45,7 +45,7 @@ _SIGNATURES = {
                              _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr],
         "mi_paged_attention": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
                                _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_int, _c_ptr, _c_long,
-                               _c_ptr, _c_long, _c_ptr],
+                               _c_ptr, _c_long, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
         "mi_paged_attention_workspace": [_c_int, _c_int, _c_int, _c_int],
         "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
                                  _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_long,
@@ -61,7 +61,7 @@ _SIGNATURES = {
                                  _c_ptr],
         "mi_conv_step": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
         "mi_ssm_scan": [_c_ptr, _c_int, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_ptr],
+                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_ptr],
         "mi_gate_norm": [_c_ptr, _c_long, _c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_float, _c_ptr, _c_long,
                          _c_int, _c_int, _c_ptr],
     },
@@ -361,7 +361,8 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
                     k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     lane_of_token: torch.Tensor, positions: torch.Tensor, scale: float,
                     window: Optional[int], out: torch.Tensor, max_seq_len: Optional[int] = None,
-                    slopes: Optional[torch.Tensor] = None) -> None:
+                    slopes: Optional[torch.Tensor] = None, query_tiles: Optional[torch.Tensor] = None,
+                    tile_tokens: int = 0, cu_seqlens: Optional[torch.Tensor] = None) -> None:
     """Causal attention of every token over its request's cached keys (its own included).
 
     ``q`` [T, >= Hq*dh] (rotated); ``block_tables`` [lanes, max_pages] page ids by logical
@@ -369,7 +370,9 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     window w, s - p < w.  ``out`` [T, Hq*dh].  ``max_seq_len``: an upper bound of position + 1 over
     the step's tokens (what the block tables can hold if it is not given); it sizes the launch and
     the work area, never the result.  ``slopes`` (float32 [Hq]): a bias on the scores by distance,
-    ``score -= slopes[head] * (s - p)``."""
+    ``score -= slopes[head] * (s - p)``.  ``query_tiles`` [tiles, 2] = (lane or -1, first token row) of runs of
+    up to ``tile_tokens`` tokens of one lane, with ``cu_seqlens`` [lanes + 1]: for steps whose lanes hold several
+    tokens, a kernel that fetches a run of keys once for sixteen queries (the same bits as without)."""
     q_ld = _row_major(q, "q")
     out_ld = _row_major(out, "out")
     T = q.shape[0]
@@ -387,11 +390,19 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     span = holds if max_seq_len is None else max(1, min(int(max_seq_len), holds))
     floats = _fn("attention", "mi_paged_attention_workspace", _c_long)(T, num_heads, head_dim, span)
     partial = torch.empty((max(int(floats), 1),), dtype=torch.float32, device=q.device)
+    tiles = 0
+    if query_tiles is not None and tile_tokens and tile_tokens % 16 == 0 and cu_seqlens is not None:
+        _i32(query_tiles, "query_tiles")
+        _i32(cu_seqlens, "cu_seqlens")
+        _need(query_tiles.dim() == 2 and query_tiles.shape[1] == 2 and cu_seqlens.numel() == block_tables.shape[0] + 1,
+              "paged_attention: the table of runs or the lanes' offsets do not fit the step")
+        tiles = query_tiles.shape[0]
     _check(_fn("attention", "mi_paged_attention")(
         _p(q), _dt(q), q_ld, T, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride,
         page_size, _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale),
-        int(window or 0), _p(slopes), span, _p(partial), partial.numel(), _p(out), out_ld, _stream()), "paged_attention",
-        f"(head_dim={head_dim})")
+        int(window or 0), _p(slopes), span, _p(partial), partial.numel(), _p(out), out_ld,
+        _p(query_tiles) if tiles else None, tiles, int(tile_tokens) if tiles else 0, _p(cu_seqlens) if tiles else None,
+        _stream()), "paged_attention", f"(head_dim={head_dim})")
 
 
 def prefill_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> bool:
@@ -532,11 +543,12 @@ def conv_step(u: torch.Tensor, col_offset: int, width: int, weight: torch.Tensor
 
 def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
              ssm_state: torch.Tensor, cu_seqlens: torch.Tensor, slot_ids: torch.Tensor, num_groups: int,
-             y: torch.Tensor) -> None:
+             y: torch.Tensor, longest: int = 0) -> None:
     """Selective scan of every lane from and into ``ssm_state[slot]`` [H, P, N] (float32).
 
     ``xbc`` [T, E + 2*G*N] = post-conv x | B | C; ``dt`` [T, H] raw (a column view is fine);
-    ``y`` float32 [T, E] gets s.C + D*x."""
+    ``y`` float32 [T, E] gets s.C + D*x.  ``longest``: an upper bound of the tokens of a lane if known (it
+    sizes the blocks of tokens a workgroup stages, never the result)."""
     xbc_ld = _row_major(xbc, "xbc")
     dt_ld = _row_major(dt, "dt")
     y_ld = _row_major(y, "y")
@@ -555,7 +567,8 @@ def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: torc
     _need(cu_seqlens.numel() == num_lanes + 1, "ssm_scan: cu_seqlens must have lanes+1 entries")
     _check(_fn("mamba2", "mi_ssm_scan")(
         _p(xbc), _dt(xbc), xbc_ld, _p(dt), dt_ld, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(cu_seqlens),
-        _p(slot_ids), num_lanes, H, P, N, num_groups, _p(y), y_ld, _stream()), "ssm_scan", f"(N={N})")
+        _p(slot_ids), num_lanes, min(int(longest), T) if longest and longest > 0 else T, H, P, N, num_groups, _p(y), y_ld,
+        _stream()), "ssm_scan", f"(N={N})")
 
 
 class SsdChunks:

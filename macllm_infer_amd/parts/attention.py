@@ -88,10 +88,15 @@ class Attention(Mixer):
         self.position.rotate_and_store(qkv, spec.num_heads, spec.num_kv_heads, spec.head_dim, step, cache)
         geometry = (spec.num_heads, spec.num_kv_heads, spec.head_dim)
         slopes = self.position.score_slopes
+        # lanes of several tokens: the general kernel shares a run of keys among the queries of a tile of the step's
+        # table of runs (when the step was packed with one)
+        tiles = {}
+        if step.max_query_len > 1 and 0 < getattr(step, "query_tile", 0) < (1 << 20):
+            tiles = dict(query_tiles=step.query_tiles, tile_tokens=step.query_tile, cu_seqlens=step.cu_seqlens)
         if slopes is not None:                           # a bias on the scores: the general kernel knows it
             ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                 step.lane_of_token, step.positions, spec.scale, spec.window, attended,
-                                step.max_seq_len, slopes)
+                                step.max_seq_len, slopes, **tiles)
         elif step.max_query_len == 1 and ops.decode_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2]):
             ops.decode_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                  step.lane_of_token, step.positions, spec.scale, spec.window, step.max_seq_len,
@@ -103,4 +108,4 @@ class Attention(Mixer):
         else:
             ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                 step.lane_of_token, step.positions, spec.scale, spec.window, attended,
-                                step.max_seq_len)
+                                step.max_seq_len, **tiles)

@@ -140,5 +140,5 @@ class Mamba2(Mixer):
         else:
             y = torch.empty((T, E), dtype=torch.float32, device=u.device)
             ops.ssm_scan(xbc, u[:, E + C:], self.dt_bias, self.A, self.D, ssm_state, step.cu_seqlens,
-                         step.slot_ids, spec.num_groups, y)
+                         step.slot_ids, spec.num_groups, y, step.max_query_len)
         ops.gate_norm(y, u[:, :E], self.norm_weight, spec.num_groups, spec.norm_eps, gated)

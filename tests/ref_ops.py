@@ -107,9 +107,11 @@ def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, r
 
 
 def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token,
-                    positions, scale, window, out, max_seq_len=None, slopes=None):
-    """``max_seq_len`` sizes the kernel's launch and nothing else: not used here.  ``slopes``: a bias on the
-    scores, ``-slopes[head] * (query position - key position)``."""
+                    positions, scale, window, out, max_seq_len=None, slopes=None, query_tiles=None, tile_tokens=0,
+                    cu_seqlens=None):
+    """``max_seq_len`` sizes the kernel's launch and nothing else: not used here, and neither is the table of
+    runs that picks the kernel for lanes of several tokens.  ``slopes``: a bias on the scores,
+    ``-slopes[head] * (query position - key position)``."""
     T = q.shape[0]
     page_size = k_cache.shape[2]
     group = num_heads // num_kv_heads
@@ -178,7 +180,7 @@ def conv_step(u, col_offset, width, weight, bias, conv_state, slot_ids):
     u[:, col_offset:col_offset + width] = out
 
 
-def ssm_scan(xbc, dt, dt_bias, A, D, ssm_state, cu_seqlens, slot_ids, num_groups, y):
+def ssm_scan(xbc, dt, dt_bias, A, D, ssm_state, cu_seqlens, slot_ids, num_groups, y, longest=0):
     _, H, P, N = ssm_state.shape
     E = H * P
     GN = num_groups * N

@@ -78,8 +78,13 @@ def test_line_of_a_short_run():
     assert 0.85 * record["ms_per_step"] <= times["mean"] <= 1.02 * record["ms_per_step"]
     assert record["prefill_uncaptured_ms"] >= 0.9 * prefill["ms"]
     assert {"in", "out", "gate_up", "down"} <= set(record["choices"])
-    assert set(record["points"]) == {"decode_b1", "decode_b64"}
+    long_points = {f"decode_b{batch}_ctx{context}" for batch, context in bench.LONG_POINTS}
+    assert set(record["points"]) == {"decode_b1", "decode_b64"} | long_points == set(record["points_frac"])
     assert record["points"]["decode_b1"] < record["value"] < record["points"]["decode_b64"]
+    # a longer context costs time and raises the fraction of the bandwidth (more bytes beside the same latencies;
+    # with the two layers of this run the points among themselves are within noise of each other)
+    assert record["points_frac"]["decode_b8_ctx32768"] > record["roofline"]["frac"]
+    assert all(0.0 < value < 1.0 for value in record["points_frac"].values())
 
 
 @pytest.mark.gpu

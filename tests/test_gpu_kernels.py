@@ -334,6 +334,51 @@ def test_general_attention_does_not_depend_on_the_step_around_a_token(ops):
         assert torch.equal(alone[0], whole[row]), (row, bound)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq, Hkv, dh, page_size, tile", [(4, 2, 64, 16, 64), (6, 2, 48, 8, 16), (3, 1, 128, 4, 32),
+                                                           (2, 2, 256, 64, 64), (5, 5, 16, 16, 48)])
+def test_tiled_general_attention_gives_the_per_token_kernels_bits(ops, dtype, Hq, Hkv, dh, page_size, tile):
+    """Lanes of several tokens go through the kernel that fetches a run of keys once for sixteen queries; a
+    position's attended row must be the per-token kernel's, bit for bit, in both dtypes, with a window, with a
+    bias by distance, for portions that cross the edges of pages, of 64-key groups and of 256-key runs, beside a
+    single token and a short fresh prompt, with rows of the table that hold nothing, and with NaN in every cache
+    cell that no request wrote."""
+    starts, counts = [300, 0, 519, 250, 0], [150, 70, 1, 9, 3]
+    lengths = [s + c for s, c in zip(starts, counts)]
+    pool, table = paged_setup(lengths, page_size, Hkv, dh, dtype, seed=31)
+    for lane, length in enumerate(lengths):
+        fill_cache(pool, table, lane, rand(length, Hkv, dh, seed=300 + lane, dtype=dtype),
+                   rand(length, Hkv, dh, seed=320 + lane, dtype=dtype), page_size)
+    T = sum(counts)
+    q = rand(T, Hq * dh + 16, seed=340, dtype=dtype).to(DEV)[:, :Hq * dh]            # a row stride
+    positions = torch.cat([torch.arange(s, s + c) for s, c in zip(starts, counts)]).to(torch.int32)
+    lane_of_token = torch.repeat_interleave(torch.arange(len(counts)), torch.tensor(counts)).to(torch.int32)
+    cu = [0]
+    for count in counts:
+        cu.append(cu[-1] + count)
+    tiles = [[-1, 0]]                                                       # a row that holds nothing, first
+    for lane, count in enumerate(counts):
+        tiles += [[lane, row] for row in range(cu[lane], cu[lane + 1], tile)]
+    tiles += [[-1, 0], [-1, 0]]
+    dev_pool = pool.to(DEV)
+    k_cache, v_cache = views(dev_pool, page_size)
+    slopes = torch.tensor([0.3 / (head + 1) for head in range(Hq)])
+    for window, bias, bound in ((None, None, None), (70, None, 520), (None, slopes, 700), (300, slopes, None)):
+        results = []
+        for with_tiles in (False, True):
+            out = torch.full((T, Hq * dh), float("nan"), dtype=dtype, device=DEV)
+            extra = dict(query_tiles=i32(tiles).to(DEV), tile_tokens=tile, cu_seqlens=i32(cu).to(DEV)) if with_tiles else {}
+            ops.paged_attention(q, Hq, Hkv, dh, k_cache, v_cache, table.to(DEV), lane_of_token.to(DEV), positions.to(DEV),
+                                0.31, window, out, bound, None if bias is None else bias.to(DEV), **extra)
+            results.append(out)
+        assert not torch.isnan(results[0].float()).any()
+        assert torch.equal(results[0], results[1]), (window, bias is not None, (results[0].float() - results[1].float()).abs().max().item())
+    want = torch.empty(T, Hq * dh, dtype=dtype)
+    ref_ops.paged_attention(q.cpu(), Hq, Hkv, dh, *views(pool, page_size), table, lane_of_token, positions, 0.31, 300,
+                            want, slopes=slopes)
+    close(results[1], want, dtype, 3.0)
+
+
 def test_attention_refuses_a_head_size_beyond_its_limit(ops):
     pool = torch.zeros(2, 1, 2, 1, 16 * 320, device=DEV)
     q = torch.zeros(1, 320, device=DEV)
