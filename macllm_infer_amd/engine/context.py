@@ -15,7 +15,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 from itertools import chain
-from typing import Hashable, List, Optional, Sequence
+from typing import Callable, Hashable, List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -59,6 +59,7 @@ class StepContext:
     max_seq_len: int = 0             # an upper bound of the longest context in the batch
     derived: dict = field(default_factory=dict)   # tables parts derive from the step, shared by the layers
     chunk_tables: dict = field(default_factory=dict)   # chunk size -> ChunkTable, for the sizes the model's mixers name
+    tables: dict = field(default_factory=dict)         # name -> int32 tensor, for the tables the model's mixers declare
 
 
 @dataclass
@@ -100,6 +101,62 @@ def apply_feeds(token_ids: torch.Tensor, feeds) -> None:
         by_source[id(source)][2].append(index)
     for source, rows, indices in by_source.values():
         ops.feed_tokens(token_ids, source, rows, indices)
+
+
+@dataclass(frozen=True)
+class StepTable:
+    """An int32 table of a step that a mixer declares (``Mixer.step_tables``) and finds, on the device, in
+    ``step.tables[name]``: written on the host with the step's other index arrays, uploaded in the same copy,
+    and at a fixed address and of a fixed size in a step that a captured graph reads.
+
+    ``words(lanes, tokens)``: the table's size for a step of that many lanes and tokens, and never smaller for
+    fewer of either: a step of fixed capacity holds the table of its capacity.
+    ``fill(out, packed)``: writes all of ``out`` (int32 [words], zeros before) from ``packed``, a
+    ``PackedLanes`` of every lane of the step, padding lanes included."""
+    name: str
+    words: Callable[[int, int], int]
+    fill: Callable[[np.ndarray, "PackedLanes"], None]
+
+
+@dataclass
+class PackedLanes:
+    """The lanes of a packed step as the host sees them (views of the buffer that is uploaded): what the fill
+    function of a ``StepTable`` reads.  Padding lanes of a captured step stand at the end, on ``scratch_slot``."""
+    num_lanes: int
+    num_tokens: int
+    positions: np.ndarray        # [T] absolute position of each token row
+    lane_of_token: np.ndarray    # [T]
+    first_token: np.ndarray      # [lanes + 1] first token row of each lane
+    start_pos: np.ndarray        # [lanes] request length before the step
+    seq_lens: np.ndarray         # [lanes] request length after the step
+    slot_ids: np.ndarray         # [lanes] state slot of each lane's request
+    scratch_slot: int            # the state slot that padding lanes read and write
+
+
+def _fill_tables(tables: Sequence[StepTable], host: np.ndarray, sizes, table_sizes, cache) -> None:
+    """Write the declared tables behind the core's sections of ``host`` (whose sizes are ``sizes``)."""
+    if not tables:
+        return
+    views = _split(host, sizes)
+    lanes = views[4].size
+    packed = PackedLanes(lanes, views[0].size, views[1], views[2], views[3], views[4], views[5], views[6],
+                         int(cache.scratch_slot))
+    offset = int(sum(sizes))
+    for table, size in zip(tables, table_sizes):
+        out = host[offset:offset + size]
+        out[:] = 0
+        table.fill(out, packed)
+        offset += size
+
+
+def _table_sizes(tables: Sequence[StepTable], lanes: int, tokens: int) -> List[int]:
+    sizes = []
+    for table in tables:
+        size = int(table.words(lanes, tokens))
+        if size < 0:
+            raise ValueError(f"the step table {table.name!r} declares a negative size")
+        sizes.append(size)
+    return sizes
 
 
 _NO_LANES = LoweredLanes(*(np.zeros(0, dtype=np.int32) for _ in range(5)))
@@ -161,7 +218,7 @@ def _pack(lowered: LoweredLanes, cache, out: Optional[np.ndarray], pad_lengths: 
 
 
 def _assemble(views, group_shapes, lengths, starts, max_seq_len, chunk_sizes=(), num_tokens=None, num_lanes=None,
-              max_query_len=None, query_tile: int = 0) -> StepContext:
+              max_query_len=None, query_tile: int = 0, tables: Sequence[StepTable] = ()) -> StepContext:
     """``lengths`` / ``starts``: the lanes' host copies, or None for a step of fixed capacity, whose lanes
     differ from fill to fill (``num_tokens``, ``num_lanes`` and ``max_query_len`` are then its capacities)."""
     tokens = sum(lengths) if lengths is not None else num_tokens
@@ -180,6 +237,9 @@ def _assemble(views, group_shapes, lengths, starts, max_seq_len, chunk_sizes=(),
     for index, chunk_size in enumerate(chunk_sizes):
         chunks, lane_chunks = views[9 + 2 * groups + 2 * index], views[10 + 2 * groups + 2 * index]
         context.chunk_tables[chunk_size] = ChunkTable(chunk_size, tokens, lanes, chunks.numel() // 4, chunks, lane_chunks)
+    first = 9 + 2 * groups + 2 * len(chunk_sizes)
+    for index, table in enumerate(tables):                 # the declared tables lie behind the core's sections
+        context.tables[table.name] = views[first + index]
     return context
 
 
@@ -192,20 +252,24 @@ def _split(buffer: torch.Tensor, sizes):
 
 
 def build_step_context(lanes: Sequence[Lane], cache, device, lowered: Optional[LoweredLanes] = None,
-                       query_tile: int = 0, chunk_sizes: Sequence[int] = ()) -> StepContext:
+                       query_tile: int = 0, chunk_sizes: Sequence[int] = (),
+                       tables: Sequence[StepTable] = ()) -> StepContext:
     """``cache``: the CacheManager, after the step's pages were reserved.  ``query_tile``, ``chunk_sizes``:
-    see ``_pack`` (``DecoderModel.query_tile`` and ``.chunk_sizes`` for a whole model)."""
+    see ``_pack``; ``tables``: the tables the model's mixers declare (``DecoderModel.step_layout`` holds all
+    three for a whole model)."""
     if lowered is None:
         lowered = lower_lanes(lanes, cache)
     needed, _, _, _, _ = _pack(lowered, cache, None, query_tile=query_tile, chunk_sizes=chunk_sizes)
-    host = torch.empty(-needed, dtype=torch.int32)
+    table_sizes = _table_sizes(tables, len(lowered.slots), int(lowered.lengths.sum()))
+    host = torch.empty(-needed + sum(table_sizes), dtype=torch.int32)
     if torch.device(device).type == "cuda":
         host = host.pin_memory()
     _, sizes, shapes, longest, _ = _pack(lowered, cache, host.numpy(), query_tile=query_tile, chunk_sizes=chunk_sizes)
+    _fill_tables(tables, host.numpy(), sizes, table_sizes, cache)
     packed = host.to(device, non_blocking=True)
     starts = cache.lengths_of(lowered.slots).tolist()
-    context = _assemble(_split(packed, sizes), shapes, lowered.lengths.tolist(), starts, longest, chunk_sizes,
-                        query_tile=query_tile)
+    context = _assemble(_split(packed, sizes + table_sizes), shapes, lowered.lengths.tolist(), starts, longest,
+                        chunk_sizes, query_tile=query_tile, tables=tables)
     context._keepalive = host
     return context
 
@@ -225,10 +289,11 @@ class StaticStep:
 
     def __init__(self, cache, lanes: int, max_seq_len: int, device, lengths: Sequence[int] = (),
                  want_rows: Sequence[int] = (), query_tile: int = 0, chunk_sizes: Sequence[int] = (),
-                 tokens: int = 0, wants: int = 0):
+                 tokens: int = 0, wants: int = 0, tables: Sequence[StepTable] = ()):
         self.cache = cache
         self.query_tile = query_tile
         self.chunk_sizes = tuple(chunk_sizes)
+        self.tables = tuple(tables)
         self.lanes = lanes
         self.tokens = tokens
         self.max_pages = max(-(-max_seq_len // group.page_size) for group in cache.groups) if cache.groups else 1
@@ -251,6 +316,11 @@ class StaticStep:
         pack = dict(max_pages=self.max_pages, want_rows=self.want_rows, query_tile=query_tile,
                     chunk_sizes=self.chunk_sizes, **self.caps)
         needed, sizes, shapes, _, _ = _pack(_NO_LANES, cache, None, first_pads, **pack)
+        # the declared tables, at the size of this step's capacity, behind the core's sections
+        self._core_sizes = sizes
+        self._table_sizes = _table_sizes(self.tables, lanes, tokens if self.capacity else sum(self.lengths))
+        needed -= sum(self._table_sizes)
+        sizes = sizes + self._table_sizes
         # The host packs a step into pinned memory and queues its copy to the fixed device addresses; the
         # copy runs when the stream gets there, so the memory it reads must stay as it is until then.  A few
         # host buffers are filled in turn, each guarded by an event recorded behind its copy: the host may
@@ -265,14 +335,15 @@ class StaticStep:
         self._turn = 0
         self.device_buffer = torch.empty(-needed, dtype=torch.int32, device=device)
         _pack(_NO_LANES, cache, self._hosts[0].numpy(), first_pads, **pack)
+        _fill_tables(self.tables, self._hosts[0].numpy(), self._core_sizes, self._table_sizes, cache)
         self.device_buffer.copy_(self._hosts[0])
         if self.capacity:
             self.context = _assemble(_split(self.device_buffer, sizes), shapes, None, None, max_seq_len,
                                      self.chunk_sizes, num_tokens=tokens, num_lanes=lanes, max_query_len=tokens,
-                                     query_tile=query_tile)
+                                     query_tile=query_tile, tables=self.tables)
         else:
             self.context = _assemble(_split(self.device_buffer, sizes), shapes, self.lengths, [0] * lanes, max_seq_len,
-                                     self.chunk_sizes, query_tile=query_tile)
+                                     self.chunk_sizes, query_tile=query_tile, tables=self.tables)
 
     HOST_BUFFERS = 2
 
@@ -305,6 +376,7 @@ class StaticStep:
         host = self._hosts[turn]
         _pack(lowered, self.cache, host.numpy(), pads, max_pages=self.max_pages, want_rows=self.want_rows,
               query_tile=self.query_tile, chunk_sizes=self.chunk_sizes, **self.caps)
+        _fill_tables(self.tables, host.numpy(), self._core_sizes, self._table_sizes, self.cache)
         self.device_buffer.copy_(host, non_blocking=True)
         if self._copied[turn] is not None:
             self._copied[turn].record()

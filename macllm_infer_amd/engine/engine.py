@@ -62,23 +62,26 @@ def resolve_dtype(dtype) -> torch.dtype:
 
 # A step with portions of prompts beside several single decoded tokens runs as two batches (see
 # ``Engine._run_in_two``) when the single tokens cost more as part of the portions' batch than as a batch of their
-# own.  As part of it every one of them is a prompt of one token to the prompt kernels, some SPLIT_LANE_SECONDS a
-# layer (beside 2,048 prompt tokens of the 0.5B shape, 8 decoded tokens cost 2.7 ms and 63 cost 13); a batch of
-# their own reads every weight once more (at some SPLIT_READ_RATE bytes a second) and pays its dependent kernels,
-# SPLIT_LAYER_SECONDS a layer.  That makes 5 single tokens for the 0.5B shape, 17 for the 7B shape and 39 for the 34B
-# shape, whose 68 GB of weights are better read once for both.
-SPLIT_LANE_SECONDS = 6e-6
-SPLIT_LAYER_SECONDS = 24e-6
-SPLIT_READ_RATE = 4.5e12
-SPLIT_FROM_LANES = 4                 # and never fewer than this
+# own.  As part of it every one of them is a prompt of one token to the prompt kernels (beside 2,048 prompt tokens
+# of the 0.5B shape, 8 decoded tokens cost 2.7 ms and 63 cost 13); a batch of their own reads every weight once
+# more and pays its dependent kernels.  Both depend on the model and on the GPU, so the clock decides when the
+# first step that could be split comes (``DecodeGraphs.measure_split``): from so many single tokens on that they
+# cost, beside the portions, what a batch of their own costs (the 0.5B shape: 17 beside a portion of 256 tokens, 9
+# beside one of 2,048; eight layers of the 7B shape: 20 and 7; a third of a second for the three graphs).  Without a clock (no graphs, or ``measured_paths=False``) a step
+# is split from SPLIT_FROM_LANES single tokens on, which is also the fewest the clock can say.
+SPLIT_FROM_LANES = 4
+SPLIT_NEVER = 1 << 30
 
 
-def split_from_lanes(weight_bytes: int, layers: int) -> int:
-    """From how many single decoded tokens beside portions of prompts on a step runs as two batches."""
-    if layers <= 0:
+def split_from_lanes(lane_share: Optional[float]) -> int:
+    """From how many single decoded tokens beside portions of prompts on a step runs as two batches.
+    ``lane_share``: what one of them costs beside the portions, as a share of what a batch of them costs alone
+    (None: not measured)."""
+    if lane_share is None:
         return SPLIT_FROM_LANES
-    own_batch = weight_bytes / SPLIT_READ_RATE + layers * SPLIT_LAYER_SECONDS
-    return max(SPLIT_FROM_LANES, int(own_batch / (layers * SPLIT_LANE_SECONDS) + 0.5))
+    if lane_share <= 0:
+        return SPLIT_NEVER
+    return max(SPLIT_FROM_LANES, int(1.0 / lane_share + 0.5))
 
 
 class Engine:
@@ -113,9 +116,9 @@ class Engine:
         build = BuildContext(hidden_size=self.spec.hidden_size, dtype=self.dtype, device=self.device,
                              max_context=self.spec.max_context, measure_paths=measured_paths)
         self.model = DecoderModel(self.spec, bound, build)
-        weight_bytes = sum(tensor.numel() * tensor.element_size() for tensor in bound.values()
-                           if isinstance(tensor, torch.Tensor))
-        self.split_from_lanes = split_from_lanes(weight_bytes, len(self.spec.schedule))
+        self.lane_share: Optional[float] = None
+        self._split_from_lanes: Optional[int] = None
+        self._measure_split = measured_paths
         needs, shared = DecoderModel.cache_layout(self.spec)
         capacity = kv_cache_capacity_tokens or self.spec.max_context
         self.cache = CacheManager(needs, shared, kv_cache_block_tokens, capacity, max_active_sequences,
@@ -126,6 +129,22 @@ class Engine:
         if decode_graphs and check_device and self.model.graph_safe:
             from .graphs import DecodeGraphs
             self.graphs = DecodeGraphs(self.model, self.cache, self.device, min(self.max_context, capacity))
+
+    @property
+    def split_from_lanes(self) -> int:
+        """From how many single decoded tokens beside portions of prompts on a step runs as two batches: asked of
+        the clock when it is first needed (or by ``warm_up``), where there is one."""
+        if self._split_from_lanes is None:
+            if self._measure_split and self.graphs is not None:
+                self.lane_share = self.graphs.measure_split()
+                self._split_from_lanes = split_from_lanes(self.lane_share) if self.lane_share is not None else SPLIT_NEVER
+            else:
+                self._split_from_lanes = split_from_lanes(None)
+        return self._split_from_lanes
+
+    @split_from_lanes.setter
+    def split_from_lanes(self, value: int) -> None:
+        self._split_from_lanes = int(value)
 
     def path_choices(self) -> dict:
         """What the first layer's fast path chose at build (empty when the layer has none): to be recorded
@@ -138,6 +157,7 @@ class Engine:
         """Capture the graphs of steps of (lanes, tokens) before the first request comes (a serving process
         does this once: no step of such a size is then ever launched kernel by kernel).  ``context``: the
         longest context the steps' requests will hold.  Returns what was captured; nothing without graphs."""
+        self.split_from_lanes                        # the clock's say on mixed steps, before the first of them
         return self.graphs.warm_up(steps, context) if self.graphs is not None else []
 
     def step_token_target(self, lanes: int, tokens: int) -> int:
@@ -224,10 +244,13 @@ class Engine:
         queued on the GPU; nothing here waits for it (a lane with ``feed`` takes its token from the device,
         so a caller may queue the next step before it has read this one's tokens)."""
         lowered = self.validate(lanes)
+        single = lowered.lengths == 1
+        singles = int(single.sum())
+        # (the clock is asked, once, only by a step that may need its answer, and before anything is reserved)
+        in_two = SPLIT_FROM_LANES <= singles < len(lanes) and self.split_from_lanes <= singles
         self.cache.reserve_slots(lowered.slots, lowered.lengths)
         try:
-            single = lowered.lengths == 1
-            if self.split_from_lanes <= int(single.sum()) < len(lanes):
+            if in_two:
                 logits = self._run_in_two(lanes, lowered, single)
             else:
                 logits = self._run(lanes, lowered)
@@ -249,8 +272,7 @@ class Engine:
             else:
                 logits = self.graphs.run_bucket(lanes, lowered)       # prompt portions: a graph of their capacity
         if logits is None:
-            context = build_step_context(lanes, self.cache, self.device, lowered, self.model.query_tile,
-                                         self.model.chunk_sizes)
+            context = build_step_context(lanes, self.cache, self.device, lowered, **self.model.step_layout)
             apply_feeds(context.token_ids, lowered.feeds)
             logits = self.model.forward(context, self.cache)
         return logits

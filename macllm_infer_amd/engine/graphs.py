@@ -144,8 +144,8 @@ class DecodeGraphs:
 
     def _capture_bucket(self, key: tuple):
         lane_cap, token_cap, want_cap, context = key
-        static = StaticStep(self.cache, lane_cap, context, self.device, query_tile=self.model.query_tile,
-                            chunk_sizes=self.model.chunk_sizes, tokens=token_cap, wants=want_cap)
+        static = StaticStep(self.cache, lane_cap, context, self.device, tokens=token_cap, wants=want_cap,
+                            **self.model.step_layout)
         entry = self._capture(0, static, warm_runs=1)
         self.counts["bucket_captures"] += 1
         while len(self._bucket_graphs) >= self.BUCKET_GRAPHS:
@@ -176,10 +176,44 @@ class DecodeGraphs:
                 done.append(key)
         return done
 
-    def _capture(self, bucket: int, static: Optional[StaticStep] = None, warm_runs: int = 2, context: int = 0):
+    def measure_split(self, prompt_tokens: int = 1024, singles: int = 16, replays: int = 5) -> Optional[float]:
+        """The clock's answer to what a single decoded token costs beside a portion of a prompt, in units of what
+        a batch of single tokens of its own costs: (time of ``prompt_tokens`` + ``singles`` single tokens as one
+        batch - time of the portion alone) / ``singles`` / time of the ``singles`` alone.  Each of the three is
+        a captured step whose lanes are all padding (nothing but the scratch page and slot is touched), replayed
+        ``replays`` times; the median counts.  None when the single tokens cost nothing measurable."""
+        prompt_tokens = min(prompt_tokens, self.max_seq_len)
+        if prompt_tokens < 2:
+            return None
+        times = []
+        for lengths in ([prompt_tokens], [prompt_tokens] + [1] * singles, [1] * singles):
+            ends, row = [], 0
+            for length in lengths:
+                row += length
+                ends.append(row - 1)
+            static = StaticStep(self.cache, len(lengths), max(prompt_tokens, 64), self.device, lengths=lengths,
+                                want_rows=ends, **self.model.step_layout)
+            # (a memory pool of its own: the graphs' shared pool ends with the last graph in it)
+            _, graph, _ = self._capture(0, static, warm_runs=1, pool=torch.cuda.graph_pool_handle())
+            marks = [torch.cuda.Event(enable_timing=True) for _ in range(replays + 1)]
+            graph.replay()
+            marks[0].record()
+            for mark in marks[1:]:
+                graph.replay()
+                mark.record()
+            torch.cuda.synchronize(self.device)
+            times.append(sorted(a.elapsed_time(b) for a, b in zip(marks, marks[1:]))[replays // 2])
+            del graph, static
+        portion, both, alone = times
+        if both <= portion or alone <= 0:
+            return None
+        return (both - portion) / singles / alone
+
+    def _capture(self, bucket: int, static: Optional[StaticStep] = None, warm_runs: int = 2, context: int = 0,
+                 pool=None):
         if static is None:
             static = StaticStep(self.cache, bucket, context or self.max_seq_len, self.device,
-                                query_tile=self.model.query_tile, chunk_sizes=self.model.chunk_sizes)
+                                **self.model.step_layout)
         # a first run outside the graph lets the libraries set themselves up; every lane is padding,
         # so only the scratch page and slot are touched
         side = torch.cuda.Stream(device=self.device)
@@ -191,9 +225,11 @@ class DecodeGraphs:
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
         # one pool for every graph: replays never overlap, so their intermediate buffers may share memory
-        if self._pool is None:
-            self._pool = torch.cuda.graph_pool_handle()
-        with torch.cuda.graph(graph, pool=self._pool):
+        if pool is None:
+            if self._pool is None:
+                self._pool = torch.cuda.graph_pool_handle()
+            pool = self._pool
+        with torch.cuda.graph(graph, pool=pool):
             logits = self.model.forward(static.context, self.cache)
         return static, graph, logits
 

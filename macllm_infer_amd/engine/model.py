@@ -117,6 +117,18 @@ class DecoderModel:
         self.query_tile = max((getattr(mixer, "query_tile", 0) for mixer in mixers), default=0)
         # and its tables of chunks for the chunk sizes the mixers name
         self.chunk_sizes = tuple(sorted({getattr(mixer, "chunk_tokens", 0) for mixer in mixers} - {0}))
+        # and the tables the mixers declare themselves; one name is one table, whichever layers read it
+        declared = {}
+        for mixer in mixers:
+            for table in (mixer.step_tables() if hasattr(mixer, "step_tables") else ()):
+                declared.setdefault(table.name, table)
+        self.step_tables = tuple(declared.values())
+
+    @property
+    def step_layout(self) -> dict:
+        """What the step's index arrays hold beyond the lanes themselves, as the arguments of
+        ``build_step_context`` and ``StaticStep``."""
+        return dict(query_tile=self.query_tile, chunk_sizes=self.chunk_sizes, tables=self.step_tables)
 
     @property
     def graph_safe(self) -> bool:

@@ -7,7 +7,8 @@ from .attention import Attention
 from .mamba2 import Mamba2
 from .ffn import SwiGLU
 from . import fused          # registers the fast paths of the layer arrangements
+from .fused import FastPathDeclined
 
-__all__ = ["Attention", "BuildContext", "FeedForward", "Linear", "Mamba2", "Mixer", "NoPosition", "Part",
+__all__ = ["Attention", "BuildContext", "FastPathDeclined", "FeedForward", "Linear", "Mamba2", "Mixer", "NoPosition", "Part",
            "ParallelPreNormBlock", "PositionEncoding", "Residual", "RmsNorm", "Rope", "SwiGLU",
            "arrangement_class", "part_class", "register_arrangement", "register_fusion", "register_part"]

@@ -13,12 +13,15 @@ every part      ``expected_tensors(spec, prefix, hidden_size) -> [Expect]`` (cla
                 ``__init__(spec, prefix, tensors, build)``
 mixer           ``cache_needs(spec) -> [KVNeed | StateNeed]`` (classmethod);
                 ``forward(x [T, d], step, cache: EntryCache) -> [T, d]``;
+                optional ``step_tables() -> [StepTable]``: index tables of its own in every step;
                 optional ``projections()`` + ``mix(...)``: see ``Mixer.projections``
 feed-forward    ``forward(x [T, d]) -> [T, d]``; optional ``gated_projections()``
 norm            ``forward(residual, rows=None) -> normed activations``; optional ``rms_prologue() ->
                 (weight, eps)``: the norm is y = x / sqrt(mean(x^2) + eps) * weight, which the skinny
                 kernels compute in their prologue, or take over altogether (``Residual.scaled``)
-position        ``rotate_and_store(qkv, heads, kv_heads, head_dim, step, cache)``
+position        ``rotate_and_store(qkv, heads, kv_heads, head_dim, step, cache)``; optional
+                ``fused_rotation() -> (inv_freq or None, rotary_dim) | None``: what the fused decode kernel
+                applies in its place
 every part      ``graph_safe = True`` if its forward may be captured in a HIP graph;
                 ``limits(spec, hidden_size) -> [Limit]`` (classmethod): sizes its kernels refuse
 """
@@ -130,6 +133,14 @@ class Mixer(Part):
     @classmethod
     def cache_needs(cls, spec):
         return []
+
+    def step_tables(self):
+        """Index tables of its own that the mixer wants in every step, as ``engine.context.StepTable``s: each is
+        written on the host from the step's lanes by the function the mixer gives, uploaded with the step's
+        other arrays, and found in ``step.tables[name]`` (int32, on the device); in a step that a captured graph
+        reads it has the size of the step's capacity and a fixed address.  Mixers that declare the same name
+        share one table."""
+        return ()
 
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         raise NotImplementedError

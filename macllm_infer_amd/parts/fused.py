@@ -41,6 +41,7 @@ part.
 """
 from __future__ import annotations
 
+import warnings
 from typing import Dict, Optional
 
 import torch
@@ -48,7 +49,6 @@ import torch
 from ..kernels import ops
 from .base import Residual, ScaledRows
 from .block import register_fusion
-from .position import NoPosition, Rope
 
 MAX_ROWS = 64          # rows of a step the skinny kernels take
 MAX_NORM_ROWS = 16     # the norm prologue recomputes the normed rows in every workgroup: small batches only
@@ -330,6 +330,15 @@ def _measure_library(weight: torch.Tensor, bias, rows: int, epilogue: int, tile:
 
 
 _MIXER_KERNELS: Dict[tuple, object] = {}
+
+
+class FastPathDeclined(UserWarning):
+    """A layer that could have run its steps of single tokens in one launch runs them through the general kernels
+    instead (correct, several times slower): the message says what the fast path misses."""
+
+
+def _decline(reason: str) -> None:
+    warnings.warn(f"no fused decode step for this layer: {reason}", FastPathDeclined, stacklevel=3)
 
 
 def register_mixer_kernel(*kinds: str):
@@ -886,9 +895,14 @@ def _rms_prologue(norm):
 def attention_mamba2_step(fusion: "LayerFusion") -> Optional["AttentionMamba2Step"]:
     attention, mamba = fusion.mixers
     a, s = attention.spec, mamba.spec
-    if type(attention.position) not in (Rope, NoPosition):
+    fused_rotation = getattr(attention.position, "fused_rotation", None)
+    if fused_rotation is None or fused_rotation() is None or attention.position.score_slopes is not None:
+        _decline(f"the position encoding {type(attention.position).__name__} declares no rotation the decode kernel "
+                 "applies (fused_rotation)")
         return None
     if a.head_dim not in (64, 128) or a.num_heads // a.num_kv_heads > 8 or s.state_size > 512:
+        _decline(f"the decode kernel takes heads of 64 or 128 dimensions in groups of up to 8 and states of up to 512 "
+                 f"columns, not {a.head_dim}, {a.num_heads // a.num_kv_heads} and {s.state_size}")
         return None
     return AttentionMamba2Step(fusion)
 
@@ -910,7 +924,7 @@ class AttentionMamba2Step:
         self.x_col = second + s.inner_size
         self.dt_col = self.x_col + s.conv_width
         self.attended_width = q_width
-        self.position = self.attention.position
+        self.inv_freq, self.rotary_dim = self.attention.position.fused_rotation()
         self.conv = dict(lo=self.x_col, hi=self.dt_col, taps=s.conv_kernel, weight=self.mamba.conv_weight,
                          bias=self.mamba.conv_bias)
 
@@ -920,10 +934,9 @@ class AttentionMamba2Step:
     def supported(self, step, caches) -> bool:
         a = self.attention.spec
         cache = caches[self.attention_name]
-        rotary = self.position.rotary_dim if isinstance(self.position, Rope) else 0
         return (cache.owns_kv
                 and ops.mixer_decode_supported(a.num_heads, a.num_kv_heads, a.head_dim, cache.k_cache.shape[2],
-                                               self.mamba.spec.state_size, step.max_seq_len, a.window, rotary))
+                                               self.mamba.spec.state_size, step.max_seq_len, a.window, self.rotary_dim))
 
     def merge_later_bytes(self, step, caches):
         """(columns of the attended heads, bytes of runs of keys a workgroup reads to merge them), or None."""
@@ -938,11 +951,10 @@ class AttentionMamba2Step:
         kv, state = caches[self.attention_name], caches[self.mamba_name]
         gated_norm = self.mamba.norm_weight is not None
         y = torch.empty((u.shape[0], s.inner_size), dtype=torch.float32, device=u.device) if gated_norm else None
-        rope = isinstance(self.position, Rope)
         attended = ops.mixer_decode(
             u, num_heads=a.num_heads, num_kv_heads=a.num_kv_heads, head_dim=a.head_dim, q_col=self.q_col,
-            k_col=self.k_col, v_col=self.v_col, inv_freq=self.position.inv_freq if rope else None,
-            rotary_dim=self.position.rotary_dim if rope else 0, k_cache=kv.k_cache, v_cache=kv.v_cache,
+            k_col=self.k_col, v_col=self.v_col, inv_freq=self.inv_freq,
+            rotary_dim=self.rotary_dim, k_cache=kv.k_cache, v_cache=kv.v_cache,
             block_tables=step.block_tables[kv.group], positions=step.positions,
             slot_mapping=step.slot_mappings[kv.group], scale=a.scale, window=a.window, max_seq_len=step.max_seq_len,
             ssm_heads=s.num_heads, ssm_head_dim=s.head_dim, state_size=s.state_size,

@@ -20,6 +20,13 @@ class PositionEncoding(Part):
     kernel_modules = ("attention",)
     score_slopes = None
 
+    def fused_rotation(self):
+        """What a kernel that rotates q and the new key itself has to apply in place of ``rotate_and_store``:
+        ``(inv_freq, rotary_dim)`` of a half-split rotation by position * inv_freq[j] of the first ``rotary_dim``
+        dimensions of every head (``(None, 0)``: nothing), or None when the encoding is no such rotation; the
+        layer then runs this part's own ``rotate_and_store`` and the general kernels."""
+        return None
+
     def rotate(self, qkv, num_heads, num_kv_heads, head_dim, step) -> None:
         return None
 
@@ -37,6 +44,9 @@ class NoPosition(PositionEncoding):
     def __init__(self, spec, head_dim: int, build: BuildContext):
         pass
 
+    def fused_rotation(self):
+        return None, 0
+
 
 @register_part("rope")
 class Rope(PositionEncoding):
@@ -49,6 +59,9 @@ class Rope(PositionEncoding):
         self.rotary_dim = spec.rotary_dim
         frequencies = [1.0 / (spec.theta ** (index / spec.rotary_dim)) for index in range(0, spec.rotary_dim, 2)]
         self.inv_freq = torch.tensor(frequencies, dtype=torch.float64).to(torch.float32).to(build.device)
+
+    def fused_rotation(self):
+        return self.inv_freq, self.rotary_dim
 
     def rotate_and_store(self, qkv, num_heads, num_kv_heads, head_dim, step, cache) -> None:
         owns = cache.owns_kv

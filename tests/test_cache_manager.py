@@ -255,12 +255,26 @@ def test_a_step_of_fixed_capacity_holds_any_lanes_that_fit_it(seed):
     filled with lanes of any lengths they are the plain packing of those lanes followed by padding lanes on the
     scratch page and slot (single tokens, then one lane with the remainder), with the tables of runs and of
     chunks filled up to their fixed sizes by rows that say "nothing here"."""
-    from macllm_infer_amd.engine.context import Lane, StaticStep, lower_lanes
+    from macllm_infer_amd.engine.context import Lane, StaticStep, StepTable, lower_lanes
     rng = random.Random(100 + seed)
     cache = make(capacity=2400, page=rng.choice([4, 8, 16]), requests=6, window=rng.choice([None, 40]))
     lane_cap, token_cap = rng.choice([(4, 96), (8, 200), (2, 64), (4, 33)])
     want_cap = rng.choice([lane_cap, token_cap])
-    static = StaticStep(cache, lane_cap, 512, "cpu", query_tile=16, chunk_sizes=(8, 32), tokens=token_cap, wants=want_cap)
+
+    def fill_ends(out, packed):                # a table that a mixer might declare: (slot, length after the step) of
+        assert not out.any()                   # every lane, then every token's position counted from its lane's end
+        out[0:2 * packed.num_lanes:2] = packed.slot_ids
+        out[1:2 * packed.num_lanes:2] = packed.seq_lens
+        out[2 * packed.num_lanes:] = packed.seq_lens[packed.lane_of_token] - 1 - packed.positions
+        assert (packed.slot_ids[packed.num_lanes - 1] == packed.scratch_slot) == (packed.first_token[-1] > 0 and pads_now[0] > 0)
+
+    pads_now = [lane_cap]
+    declared = [StepTable("ends", lambda lanes, tokens: 2 * lanes + tokens, fill_ends),
+                StepTable("nothing", lambda lanes, tokens: 0, lambda out, packed: None)]
+    static = StaticStep(cache, lane_cap, 512, "cpu", query_tile=16, chunk_sizes=(8, 32), tokens=token_cap, wants=want_cap,
+                        tables=declared)
+    assert static.context.tables["ends"].numel() == 2 * lane_cap + token_cap and static.context.tables["nothing"].numel() == 0
+    ends_at = static.context.tables["ends"].data_ptr()
     assert static.context.lane_lengths is None and static.context.num_tokens == token_cap
     assert static.context.num_lanes == lane_cap and static.context.max_query_len == token_cap
     addresses = [static.context.token_ids.data_ptr(), static.context.query_tiles.data_ptr(),
@@ -291,6 +305,7 @@ def test_a_step_of_fixed_capacity_holds_any_lanes_that_fit_it(seed):
         if not StaticStep.fits(lane_cap, token_cap, len(lanes), total) or any(len(tokens) < 1 for _, tokens, _ in lanes):
             continue
         cache.reserve([(name, len(tokens)) for name, tokens, _ in lanes])
+        pads_now[0] = lane_cap - len(lanes)
         static.fill(lower_lanes([Lane(*lane) for lane in lanes], cache))
         pads = lane_cap - len(lanes)
         pad_lengths = [1] * (pads - 1) + [token_cap - total - (pads - 1)] if pads else []
@@ -305,6 +320,9 @@ def test_a_step_of_fixed_capacity_holds_any_lanes_that_fit_it(seed):
             got = getattr(static.context, field)
             got = [item.tolist() for item in got] if isinstance(got, list) else got.tolist()
             assert got == value, field
+        ends = [value for pair in zip(want["slot_ids"], want["seq_lens"]) for value in pair]
+        ends += [want["seq_lens"][lane] - 1 - position for lane, position in zip(want["lane_of_token"], want["positions"])]
+        assert static.context.tables["ends"].tolist() == ends and static.context.tables["ends"].data_ptr() == ends_at
         for size in (8, 32):
             table = static.context.chunk_tables[size]
             chunks, lane_chunks = plain_chunks(lengths, size)

@@ -189,6 +189,16 @@ def test_toy_parts_register_build_and_step_on_the_host(host_ops, schedule):
     toy_parts.exercise(schedule, "cpu", check_device=False)
 
 
+def test_a_mixer_declares_a_step_table_of_its_own_on_the_host(host_ops):
+    """A toy mixer, registered from the tests, names an index table of its own; the step carries it, written by the
+    mixer's function from the step's lanes, and the model says what the plain one says."""
+    import toy_parts
+    del toy_parts.TABLE_FILLS[:]
+    engine = toy_parts.exercise_step_table("cpu", check_device=False, graphs=False)
+    assert (2, 14) in toy_parts.TABLE_FILLS and (3, 3) in toy_parts.TABLE_FILLS
+    assert engine.graphs is None
+
+
 def test_a_step_that_fails_once_launched_ends_its_requests_and_leaves_the_others_alone(host_ops, tmp_path, monkeypatch):
     """A kernel refuses in the second layer, after the first has written keys, values and state in place:
     the requests of that step are ended and give back pages and slots (the reference restores a checkpoint

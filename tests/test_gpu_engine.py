@@ -263,6 +263,7 @@ def test_generation_with_more_live_requests_than_the_skinny_kernels_take_rows(tm
     llm = LLM(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * count,
               engine_config=EngineConfig(max_active_sequences=count, scheduler_token_budget=24 + count,
                                          prefill_token_quantum=24))
+    llm.engine.split_from_lanes = 4             # two batches from four single tokens on, whatever the clock would say
     runs = []
     real = llm.engine._run
     llm.engine._run = lambda lanes, lowered: (runs.append((len(lanes), int(lowered.lengths.max()))), real(lanes, lowered))[1]
@@ -610,6 +611,87 @@ def test_norms_left_to_the_projections_around_them(tmp_path, monkeypatch):
         engine.cache.check()
 
 
+def test_the_clock_says_from_how_many_single_tokens_a_mixed_step_runs_as_two_batches(tmp_path):
+    """Nothing is measured until a step could need the answer (portions beside four single tokens or more); then the
+    engine times a portion alone, beside single tokens and the single tokens alone, once, on padding lanes, and
+    splits from the number the three times give.  Without the clock the fewest allowed stands."""
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.engine import engine as engine_module
+    folder = tiny_configs.make_model_dir("C", tmp_path, torch.bfloat16)
+    cfg, _ = plain_impl.load_model_dir(folder)
+    fixed = Engine(folder, dtype="bfloat16", kv_cache_capacity_tokens=1024, max_active_sequences=8, measured_paths=False)
+    assert fixed.split_from_lanes == engine_module.SPLIT_FROM_LANES and fixed.lane_share is None
+    engine = Engine(folder, dtype="bfloat16", kv_cache_capacity_tokens=1024, max_active_sequences=8)
+    for index in range(6):
+        engine.add_request(index)
+        engine.step([Lane(index, tokens_for(cfg["vocab_size"], 9, index), [])])
+    engine.step([Lane(0, [1, 2, 3], []), Lane(1, [4], [0]), Lane(2, [5], [0])])
+    assert engine._split_from_lanes is None                       # two single tokens: no question
+    got = engine.step([Lane(0, [1, 2, 3], [2])] + [Lane(index, [7], [0]) for index in range(1, 6)])
+    assert got.shape[0] == 6
+    print("lane share", engine.lane_share, "split from", engine.split_from_lanes)
+    assert engine._split_from_lanes is not None and engine.split_from_lanes >= engine_module.SPLIT_FROM_LANES
+    assert engine.lane_share is None or engine.lane_share > 0
+    if engine.lane_share is not None:
+        assert engine.split_from_lanes == max(engine_module.SPLIT_FROM_LANES, int(1.0 / engine.lane_share + 0.5))
+    engine.cache.check()
+
+
+def test_a_mixer_with_a_step_table_of_its_own_runs_under_captured_graphs():
+    """A toy mixer, registered from the tests, declares an index table of its own.  The step carries it at a fixed
+    address with the size of the step's capacity; the mixer's function rewrites it before every replay, and graphs
+    of single tokens and of prompt portions say what the plain model says, whatever the order of the lanes."""
+    del toy_parts.TABLE_FILLS[:]
+    engine = toy_parts.exercise_step_table(DEV, check_device=True, graphs=True)
+    counts = engine.graphs.counts
+    assert counts["bucket_captures"] == 1 and counts["bucket_replays"] >= 4 and counts["decode_replays"] >= 30
+    assert (4, 16) in toy_parts.TABLE_FILLS                 # the capacity that the portions were padded to
+    assert {fill for fill in toy_parts.TABLE_FILLS if fill[0] == fill[1]} >= {(1, 1), (2, 2), (4, 4)}   # decode buckets
+    eager = toy_parts.exercise_step_table(DEV, check_device=True, graphs=False)
+    assert eager.graphs is None
+
+
+def test_a_position_encoding_that_declares_its_rotation_gets_the_fused_decode_step():
+    """A toy rotation, registered from the tests: the class that says what it rotates by (``fused_rotation``) decodes
+    through the one-launch mixer kernel; the class that keeps it to itself is told so with a warning and decodes
+    through its own ``rotate_and_store`` and the general kernels.  Both say the same, and not what the package's own
+    rotation says."""
+    import gates
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.config import FalconH1Config
+    from macllm_infer_amd.parts import FastPathDeclined
+    from macllm_infer_amd.weights.random_init import random_tensors
+    toy_parts.register_toys()
+    base = dict(tiny_configs.TINY_C, rope_theta=50.0)
+    tensors = random_tensors(FalconH1Config.from_dict(base), 6, torch.bfloat16, "unit")
+    prompts = {index: tokens_for(base["vocab_size"], length, 40 + index) for index, length in enumerate([90, 33, 61])}
+
+    def decode(config, expect_kernel):
+        engine = Engine(config=config, tensors=tensors, dtype="bfloat16", kv_cache_block_tokens=16,
+                        kv_cache_capacity_tokens=1024, max_active_sequences=4, measured_paths=False)
+        fusion = engine.model.blocks[0].fusion
+        assert (fusion.kernel is not None) == expect_kernel
+        for index, tokens in prompts.items():
+            engine.add_request(index)
+            engine.step([Lane(index, tokens[:-6], [])])
+        rows = [engine.step([Lane(index, [tokens[turn - 6]], [0]) for index, tokens in prompts.items()]).float().cpu()
+                for turn in range(6)]
+        return torch.cat(rows)
+
+    stretched = lambda kind: toy_parts.ToyStretchedConfig({"architectures": ["ToyStretchedForTests"], "base": base,
+                                                          "stretch": 3.0, "position_kind": kind})
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("error", FastPathDeclined)
+        said = decode(stretched("toy_stretched_rope"), True)
+        own = decode(FalconH1Config.from_dict(base), True)
+    with pytest.warns(FastPathDeclined, match="StretchedRopeUnsaid declares no rotation"):
+        unsaid = decode(stretched("toy_stretched_rope_unsaid"), False)
+    for row in range(said.shape[0]):
+        assert gates.bfloat16_close(said[row].numpy(), unsaid[row].numpy()), row
+    assert not all(gates.bfloat16_close(said[row].numpy(), own[row].numpy()) for row in range(said.shape[0]))
+
+
 def test_the_output_projection_may_merge_the_runs_of_keys(monkeypatch):
     """Steps of up to 16 single tokens: whether the runs of keys of the attended heads are merged by a kernel of
     their own or in the prologue of the output projection, the logits are the same bit for bit, with contexts
@@ -953,8 +1035,10 @@ def test_portion_graphs_match_eager_steps(tmp_path, name, dtype):
     # three decoded tokens beside a portion of 32: 48 tokens in 8 lanes (four cannot be padded), whatever their order
     assert (8, 48) in [key[:2] for key in with_graphs.graphs._bucket_graphs]
     assert with_graphs.graphs.counts["bucket_replays"] == replays + 5
-    # four decoded tokens beside a portion are a batch of their own: the portion goes through the graph of its
-    # capacity, the four through a decode graph, and the logits come back in the order of the lanes
+    # four decoded tokens beside a portion are a batch of their own (where the clock, set aside here, says so): the
+    # portion goes through the graph of its capacity, the four through a decode graph, and the logits come back in
+    # the order of the lanes
+    with_graphs.split_from_lanes = eager.split_from_lanes = 4
     replays, decodes = with_graphs.graphs.counts["bucket_replays"], with_graphs.graphs.counts["decode_replays"]
     for turn in range(4):
         lanes = [lane(key, 1, [0]) for key in "pq"] + [lane("t", 20, [0, 19] if turn != 1 else [])]

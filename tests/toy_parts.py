@@ -138,6 +138,94 @@ class ToyConfig:
                          layers=layers, schedule=schedule, final_norm=norm, tied_embeddings=True)
 
 
+@dataclass(frozen=True)
+class TableDecaySpec:
+    """The decay mixer once more, s_t = decay * s_{t-1} + x_t W; y_t = s_t, without a look at the host: where a
+    token's lane begins and which state slot it reads and writes comes from an index table of the mixer's own in
+    every step (``step_tables``), so that its forward pass can be captured in a graph."""
+    width: int
+    decay: float
+    kind: str = "toy_table_decay"
+
+    def validate(self):
+        assert 0 < self.decay < 1 and self.width > 0
+
+
+@dataclass
+class ToyTableConfig:
+    """A toy architecture of one layer: attention beside the decay mixer that reads a step table of its own."""
+    raw: dict
+    architecture_names = ("ToyTableForTests",)
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw)
+
+    def to_dict(self):
+        return dict(self.raw)
+
+    def to_model_spec(self):
+        from macllm_infer_amd.config import (AttentionSpec, LayerSpec, MixerSlot, ModelSpec, RmsNormSpec, RopeSpec,
+                                             ScheduleEntry, SwiGLUSpec)
+        raw = self.raw
+        norm = RmsNormSpec(eps=1e-5)
+        attention = AttentionSpec(num_heads=2, num_kv_heads=1, head_dim=32, scale=32 ** -0.5,
+                                  position=RopeSpec(theta=1e3, rotary_dim=32))
+        layer = LayerSpec(prefix="model.layers.0", ffn=SwiGLUSpec(intermediate_size=48), mixer_norm=norm, ffn_norm=norm,
+                          mixers=(MixerSlot("self_attn", attention),
+                                  MixerSlot("decay", TableDecaySpec(raw["hidden"], raw["decay"]))))
+        return ModelSpec(architecture="ToyTableForTests", hidden_size=raw["hidden"], vocab_size=raw["vocab"],
+                         max_context=512, layers=(layer,), schedule=(ScheduleEntry(0), ScheduleEntry(0)),
+                         final_norm=norm, tied_embeddings=True)
+
+
+@dataclass(frozen=True)
+class StretchedRopeSpec:
+    """A toy position encoding: the half-split rotation with every angle divided by ``stretch``.  ``kind`` picks the
+    class that says so to the fused decode kernel (``fused_rotation``) or the one that keeps it to itself."""
+    theta: float
+    rotary_dim: int
+    stretch: float
+    kind: str = "toy_stretched_rope"
+
+    def validate(self, head_dim=None):
+        assert self.stretch > 0 and self.rotary_dim % 2 == 0
+
+
+@dataclass
+class ToyStretchedConfig:
+    """The package's own hybrid architecture with the toy rotation in place of its own in every layer:
+    ``raw["base"]`` is that architecture's config.json, ``raw["stretch"]`` and ``raw["position_kind"]`` the toy's."""
+    raw: dict
+    architecture_names = ("ToyStretchedForTests",)
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw)
+
+    def to_dict(self):
+        return dict(self.raw)
+
+    def to_model_spec(self):
+        from dataclasses import replace
+        from macllm_infer_amd.config import FalconH1Config
+        spec = FalconH1Config.from_dict(self.raw["base"]).to_model_spec()
+        layers = []
+        for layer in spec.layers:
+            mixers = []
+            for slot in layer.mixers:
+                position = getattr(slot.spec, "position", None)
+                if position is not None:
+                    toy = StretchedRopeSpec(position.theta, position.rotary_dim, self.raw["stretch"], self.raw["position_kind"])
+                    slot = replace(slot, spec=replace(slot.spec, position=toy))
+                mixers.append(slot)
+            layers.append(replace(layer, mixers=tuple(mixers)))
+        return replace(spec, architecture="ToyStretchedForTests", layers=tuple(layers))
+
+
+TABLE_FILLS = []          # (lanes, tokens) of every fill of the toy mixer's step table
+
+
 def register_toys():
     from macllm_infer_amd.cache import StateNeed
     from macllm_infer_amd.config import register_architecture
@@ -174,6 +262,56 @@ def register_toys():
                     out[t] = s
                 state[slot] = s
                 cursor += length
+            return out.to(x.dtype)
+
+    @register_part("toy_table_decay")
+    class TableDecay(Mixer):
+        kernel_modules = ()
+        graph_safe = True
+        TABLE = "toy_decay_rows"
+
+        @classmethod
+        def expected_tensors(cls, spec, prefix, hidden_size):
+            return [Expect(f"{prefix}.w.weight", ((spec.width, hidden_size),))]
+
+        @classmethod
+        def cache_needs(cls, spec):
+            return [StateNeed("s", (spec.width,), "float32")]
+
+        def __init__(self, spec, prefix, tensors, build):
+            self.spec = spec
+            self.weight = tensors[f"{prefix}.w.weight"].float().to(build.device)
+
+        def step_tables(self):
+            from macllm_infer_amd.engine import StepTable
+
+            def fill(out, packed):
+                # a row a token: (first row of its lane, state slot it reads, state slot its state is written to:
+                # the lane's own for the lane's last token, the spare one for every other)
+                TABLE_FILLS.append((packed.num_lanes, packed.num_tokens))
+                rows = out.reshape(-1, 3)
+                for lane in range(packed.num_lanes):
+                    first, end = int(packed.first_token[lane]), int(packed.first_token[lane + 1])
+                    rows[first:end, 0] = first
+                    rows[first:end, 1] = packed.slot_ids[lane]
+                    rows[first:end, 2] = packed.scratch_slot
+                    rows[end - 1, 2] = packed.slot_ids[lane]
+
+            return [StepTable(self.TABLE, lambda lanes, tokens: 3 * tokens, fill)]
+
+        def forward(self, x, step, cache):
+            state = cache.states["s"]
+            tokens = x.shape[0]
+            table = step.tables[self.TABLE].view(-1, 3)[:tokens].long()
+            first, read_from, write_to = table[:, 0], table[:, 1], table[:, 2]
+            projected = x.float() @ self.weight.T
+            rows = torch.arange(tokens, device=x.device)
+            distance = rows[:, None] - rows[None, :]
+            together = (first[:, None] == first[None, :]) & (distance >= 0)
+            powers = torch.where(together, torch.pow(self.spec.decay, distance.clamp(min=0).float()), 0.0)
+            carried = state[read_from] * torch.pow(self.spec.decay, (rows - first + 1).float())[:, None]
+            out = powers @ projected + carried
+            state.index_copy_(0, write_to, out)
             return out.to(x.dtype)
 
     @register_part("toy_gated_decay")
@@ -228,6 +366,29 @@ def register_toys():
             factor = (1.0 + step.positions.float() * self.slope)[:, None]
             width = (num_heads + num_kv_heads) * head_dim
             qkv[:, :width] = (qkv[:, :width].float() * factor).to(qkv.dtype)
+
+    @register_part("toy_stretched_rope_unsaid")
+    class StretchedRopeUnsaid(PositionEncoding):
+        graph_safe = True
+
+        def __init__(self, spec, head_dim, build):
+            from macllm_infer_amd.kernels import ops
+            self.ops = ops
+            self.rotary_dim = spec.rotary_dim
+            frequencies = [1.0 / (spec.theta ** (index / spec.rotary_dim)) / spec.stretch
+                           for index in range(0, spec.rotary_dim, 2)]
+            self.inv_freq = torch.tensor(frequencies, dtype=torch.float64).to(torch.float32).to(build.device)
+
+        def rotate_and_store(self, qkv, num_heads, num_kv_heads, head_dim, step, cache):
+            owns = cache.owns_kv
+            self.ops.rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, step.positions, self.inv_freq,
+                                   self.rotary_dim, step.slot_mappings[cache.group] if owns else None,
+                                   cache.k_cache if owns else None, cache.v_cache if owns else None)
+
+    @register_part("toy_stretched_rope")
+    class StretchedRope(StretchedRopeUnsaid):
+        def fused_rotation(self):
+            return self.inv_freq, self.rotary_dim
 
     @register_part("toy_routed")
     class Routed(FeedForward):
@@ -301,6 +462,8 @@ def register_toys():
 
     register_architecture(ToyConfig)
     register_architecture(ToyFastConfig)
+    register_architecture(ToyTableConfig)
+    register_architecture(ToyStretchedConfig)
 
 
 def centred_norm(x, weight, bias, eps):
@@ -479,3 +642,75 @@ def toy_fast_plain_logits(raw, tensors, tokens):
     h = h + routed_feed_forward(f, t[p + "mlp.router.weight"], t[p + "mlp.up.weight"], t[p + "mlp.down.weight"])
     h = plain_impl.rms_norm(h, t["model.norm.weight"], 1e-5)
     return h @ t["model.embed_tokens.weight"].T
+
+
+def toy_table_plain_logits(raw, tensors, tokens):
+    """The layer of ``ToyTableConfig``, run twice, whole sequence, from the plain parts."""
+    T = len(tokens)
+    t = {name: value.float() for name, value in tensors.items()}
+    h = t["model.embed_tokens.weight"][torch.tensor(tokens)]
+    sub = lambda prefix: {name[len(prefix):]: value for name, value in t.items() if name.startswith(prefix)}
+    p = "model.layers.0."
+    for _ in range(2):
+        n = plain_impl.rms_norm(h, t[p + "attn_norm.weight"], 1e-5)
+        attended = plain_impl.attention_mixer(n, sub(p + "self_attn."), num_heads=2, num_kv_heads=1, head_dim=32,
+                                              theta=1e3)
+        projected = n @ t[p + "decay.w.weight"].T
+        s, rows = torch.zeros(raw["hidden"]), []
+        for position in range(T):
+            s = raw["decay"] * s + projected[position]
+            rows.append(s)
+        h = h + attended + torch.stack(rows)
+        h = h + plain_impl.swiglu_mlp(plain_impl.rms_norm(h, t[p + "ffn_norm.weight"], 1e-5), sub(p + "mlp."))
+    h = plain_impl.rms_norm(h, t["model.norm.weight"], 1e-5)
+    return h @ t["model.embed_tokens.weight"].T
+
+
+def exercise_step_table(device, check_device, graphs):
+    """The toy mixer with a step table of its own: registered, built and stepped (whole, in portions beside decoded
+    tokens of others, lanes in changing order), against ``toy_table_plain_logits``.  Returns the engine."""
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.weights.random_init import random_tensors
+    register_toys()
+    raw = {"architectures": ["ToyTableForTests"], "hidden": 40, "vocab": 77, "decay": 0.8}
+    config = ToyTableConfig(raw)
+    tensors = random_tensors(config, 11, torch.float32, "unit")
+    engine = Engine(config=config, tensors=tensors, dtype="float32", device=device, kv_cache_block_tokens=8,
+                    kv_cache_capacity_tokens=512, max_active_sequences=4, check_device=check_device,
+                    decode_graphs=graphs)
+    assert [table.name for table in engine.model.step_tables] == ["toy_decay_rows"]      # two runs of the layer, one table
+    prompts = {name: tokens_for(77, length, seed) for seed, (name, length) in enumerate([("a", 61), ("b", 38), ("c", 50)])}
+    wants = {name: toy_table_plain_logits(raw, tensors, tokens) for name, tokens in prompts.items()}
+    got = {name: [] for name in prompts}
+    done = {name: 0 for name in prompts}
+
+    def run(portions):
+        lanes = []
+        for name, count in portions:
+            lanes.append(Lane(name, prompts[name][done[name]:done[name] + count], list(range(count))))
+        out = engine.step(lanes).cpu()
+        row = 0
+        for name, count in portions:
+            got[name].append(out[row:row + count])
+            done[name] += count
+            row += count
+
+    for name in prompts:
+        engine.add_request(name)
+    # portions of the same capacity several times over (a graph of that capacity is captured at the second), with
+    # the lanes in changing order and single tokens beside them; then single tokens alone, lanes coming and going
+    run([("a", 13), ("b", 1)])
+    run([("b", 1), ("a", 13)])
+    run([("c", 11), ("a", 2), ("b", 1)])
+    run([("b", 12), ("c", 2)])
+    run([("c", 1), ("b", 13)])
+    run([("a", 9), ("c", 5)])
+    while any(done[name] < len(prompts[name]) for name in prompts):
+        order = [name for name in ("c", "a", "b") if done[name] < len(prompts[name])]
+        if done["a"] % 2:
+            order.reverse()
+        run([(name, 1) for name in order])
+    for name in prompts:
+        assert (torch.cat(got[name]) - wants[name]).abs().max() < 1e-4, name
+    engine.cache.check()
+    return engine
