@@ -200,6 +200,8 @@ class ModelSpec:
     tied_embeddings: bool = False
     embedding_multiplier: float = 1.0
     logit_multiplier: float = 1.0
+    # logits <- cap * tanh(logits / cap) after their scaling (src/decoder.rs:3349-3355, 4791-4796); None: no cap
+    logit_softcap: Optional[float] = None
     embedding_name: str = "model.embed_tokens"
     final_norm_name: str = "model.norm"
     lm_head_name: str = "lm_head"
@@ -219,6 +221,8 @@ class ModelSpec:
                  f"max_position_embeddings {self.max_context} must be in 1..=2^20")
         _require(0 < len(self.layers) <= 4096, "num_hidden_layers must be in 1..=4096")
         _require(len(self.schedule) > 0, "the schedule of layers is empty")
+        _require(self.logit_softcap is None or (0 < self.logit_softcap < float("inf")),
+                 f"the cap on the logits must be finite and positive, got {self.logit_softcap}")
         self.final_norm.validate()
         for layer in self.layers:
             _require(len(layer.mixers) > 0, f"layer {layer.prefix} has no mixer")

@@ -344,6 +344,22 @@ extern "C" int mi_scale_to_f32(const void* in, int dtype, float multiplier, floa
   return 0;
 }
 
+// ---------------------------------------------------------------- a cap on the logits
+// x <- cap * tanh(x / cap), in place on float32 (reference: src/decoder.rs:4791-4796, after the scaling of the
+// logits, :3349-3355)
+__global__ void tanh_softcap_kernel(float* __restrict__ x, float cap, float inverse, long total) {
+  const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (index < total) x[index] = cap * tanhf(x[index] * inverse);
+}
+
+extern "C" int mi_tanh_softcap(float* x, float cap, long total, hipStream_t stream) {
+  if (total <= 0 || !x || !(cap > 0.f)) return ERR_BAD_ARGUMENT;
+  const int blocks = (int)((total + 255) / 256);
+  tanh_softcap_kernel<<<blocks, 256, 0, stream>>>(x, cap, 1.0f / cap, total);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
 // ---------------------------------------------------------------- bias behind a library product
 // out[m, n] = bf16(sums[m, n] + bias[n]): the float32 sums of a bfloat16 product get their float32 bias and are
 // rounded once (reference: src/model_weights.rs:530-545 adds the bias to the product's result).

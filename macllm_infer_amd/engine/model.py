@@ -158,14 +158,19 @@ class DecoderModel:
             ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, x=scaled.rows,
                            row_scale=ops.RowScale(scaled.ssq, spec.hidden_size, self._final_rms[1]),
                            fragments=self._head_fragments)
-            return logits
+            return self._capped(logits)
         normed = self.final_norm.forward(residual, rows=step.want_rows)
         if self._head_fragments is not None and wanted <= HEAD_SKINNY_ROWS:
             ops.fused_gemm(self.lm_head, None, logits, out_scale=spec.logit_multiplier, x=normed,
                            fragments=self._head_fragments)
-            return logits
+            return self._capped(logits)
         raw = ops.linear(normed, self.lm_head, None, keep_float32=True)      # the sums as they are, not rounded to bfloat16
         ops.scale_to_f32(raw, spec.logit_multiplier, logits)
+        return self._capped(logits)
+
+    def _capped(self, logits: torch.Tensor) -> torch.Tensor:
+        if self.spec.logit_softcap is not None:
+            ops.tanh_softcap(logits, self.spec.logit_softcap)
         return logits
 
     @staticmethod

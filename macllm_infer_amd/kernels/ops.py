@@ -38,6 +38,7 @@ _SIGNATURES = {
                                     _c_int, _c_ptr],
         "mi_swiglu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
         "mi_scale_to_f32": [_c_ptr, _c_int, _c_float, _c_ptr, _c_long, _c_ptr],
+        "mi_tanh_softcap": [_c_ptr, _c_float, _c_long, _c_ptr],
         "mi_add_bias_round": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     },
     "attention": {
@@ -271,6 +272,14 @@ def scale_to_f32(values: torch.Tensor, multiplier: float, out: torch.Tensor) -> 
           and out.numel() == values.numel() and values.is_cuda, "scale_to_f32: shapes do not match")
     _check(_fn("common", "mi_scale_to_f32")(_p(values), _dt(values), float(multiplier), _p(out), values.numel(),
                                             _stream()), "scale_to_f32")
+
+
+def tanh_softcap(logits: torch.Tensor, cap: float) -> None:
+    """logits <- cap * tanh(logits / cap), in place (float32)."""
+    _need(logits.is_contiguous() and logits.dtype == torch.float32 and logits.is_cuda and cap > 0,
+          "tanh_softcap: contiguous float32 logits on the GPU and a positive cap")
+    if logits.numel():
+        _check(_fn("common", "mi_tanh_softcap")(_p(logits), float(cap), logits.numel(), _stream()), "tanh_softcap")
 
 
 # --------------------------------------------------------------------------- matrix products

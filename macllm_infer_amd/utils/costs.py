@@ -108,7 +108,8 @@ def total(costs: Dict[str, Cost]) -> Cost:
 # products carry no such mark and stay with the other kernels).
 DECODE_GROUPS: List[Tuple[str, str]] = [
     (r"mixer_decode_kernel|mixer_merge_kernel|decode_attention_kernel|decode_merge_kernel|ssm_scan_kernel|conv_step_kernel|"
-     r"gate_norm_kernel|rope_kv_store_kernel|paged_attention_kernel", "mixers"),
+     r"gate_norm_kernel|rope_kv_store_kernel|paged_attention_kernel|paged_attention_tile_kernel|"
+     r"paged_attention_merge_kernel", "mixers"),
     (r"fused_gemm_kernel<\d+, \d+, 2|shared_rows_gemm_kernel<\d+, \d+, 2", "input projections"),
     (r"fused_gemm_kernel<\d+, \d+, 1|shared_rows_gemm_kernel<\d+, \d+, 1", "gate and up projections"),
     (r"fused_gemm_kernel<\d+, \d+, 3|fused_gemm_kernel<\d+, 2, 0|shared_rows_gemm_kernel<\d+, \d+, 0|fused_gemm_split_kernel",
@@ -117,7 +118,8 @@ DECODE_GROUPS: List[Tuple[str, str]] = [
 PLAIN_PRODUCT = r"fused_gemm_kernel<\d+, [01], 0"
 PREFILL_GROUPS: List[Tuple[str, str]] = [
     (r"^Cijk_|gemm_f32_kernel", "matrix products"),
-    (r"prefill_attention|paged_attention_kernel|rope_kv_store_kernel", "attention"),
+    (r"prefill_attention|paged_attention_kernel|paged_attention_tile_kernel|paged_attention_merge_kernel|"
+     r"rope_kv_store_kernel", "attention"),
     (r"ssd_|ssm_scan_kernel|conv1d_silu|conv_state_update|gate_norm_kernel", "state-space scan"),
 ]
 

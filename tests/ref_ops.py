@@ -54,6 +54,10 @@ def scale_to_f32(values, multiplier, out):
     out.copy_(_f(values).reshape(out.shape) * multiplier)
 
 
+def tanh_softcap(logits, cap):
+    logits.copy_(cap * torch.tanh(logits / cap))
+
+
 def fused_gemm_split(weight, bias, x, partial, feature_tiles=1, fragments=None):
     """Slab s: the sums over the s-th run of K (in chunks of 32), the bias in slab 0."""
     S = partial.shape[0]
@@ -216,7 +220,7 @@ def argmax(logits, out):
     out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
 
 
-NAMES = ["fused_gemm_split", "add_partials_rmsnorm", "prefill_attention_supported", "decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "linear", "rope_kv_store", "paged_attention",
+NAMES = ["fused_gemm_split", "add_partials_rmsnorm", "prefill_attention_supported", "decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "tanh_softcap", "linear", "rope_kv_store", "paged_attention",
          "conv1d_silu", "conv_state_update", "ssm_scan", "gate_norm", "argmax", "feed_tokens"]
 
 

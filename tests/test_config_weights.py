@@ -73,6 +73,17 @@ def test_config_errors_name_the_field(change, word):
         FalconH1Config.from_dict(raw)
 
 
+def test_the_model_spec_refuses_a_cap_on_the_logits_that_is_no_positive_number():
+    from dataclasses import replace
+    from macllm_infer_amd.config import ConfigError
+    spec = tiny_configs.config("A").to_model_spec()
+    assert spec.logit_softcap is None
+    replace(spec, logit_softcap=30.0).validate()
+    for cap in (0.0, -1.0, float("inf"), float("nan")):
+        with pytest.raises(ConfigError, match="cap on the logits"):
+            replace(spec, logit_softcap=cap).validate()
+
+
 def test_registry_maps_names_and_lists_them_for_an_unknown_one(tmp_path):
     assert "FalconH1ForCausalLM" in registered_architectures() and "falcon_h1" in registered_architectures()
     assert isinstance(config_from_dict(tiny_configs.TINY_A), FalconH1Config)

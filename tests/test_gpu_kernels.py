@@ -149,6 +149,20 @@ def test_bfloat16_product_adds_its_bias_in_float32(ops):
     assert got.dtype == torch.bfloat16 and bool((got.float().cpu() == 1.0 + 2.0 ** -7).all())
 
 
+def test_the_cap_on_the_logits_is_a_scaled_tanh(ops):
+    """cap * tanh(x / cap), in place, at a size that is no multiple of the workgroup; small logits pass nearly as
+    they are, large ones end at the cap, and the sign stays."""
+    x = torch.randn(3, 1031, generator=torch.Generator().manual_seed(4)) * 6.0
+    x[0, :4] = torch.tensor([0.0, 1e-3, -400.0, 400.0])
+    got = x.to(DEV)
+    ops.tanh_softcap(got, 2.5)
+    want = 2.5 * torch.tanh(x.double() / 2.5)
+    assert (got.cpu().double() - want).abs().max() < 1e-6
+    assert got[0, :4].cpu().tolist() == pytest.approx([0.0, 1e-3, -2.5, 2.5], abs=1e-7)
+    with pytest.raises(ops.KernelError):
+        ops.tanh_softcap(got, 0.0)
+
+
 # ------------------------------------------------------------------ attention
 def paged_setup(lengths, page_size, Hkv, dh, dtype, layers=2, seed=0):
     """A pool of shuffled pages [page, layer, K|V, Hkv, page_size*dh] and a block table per lane."""

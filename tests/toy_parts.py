@@ -176,7 +176,8 @@ class ToyTableConfig:
                                   MixerSlot("decay", TableDecaySpec(raw["hidden"], raw["decay"]))))
         return ModelSpec(architecture="ToyTableForTests", hidden_size=raw["hidden"], vocab_size=raw["vocab"],
                          max_context=512, layers=(layer,), schedule=(ScheduleEntry(0), ScheduleEntry(0)),
-                         final_norm=norm, tied_embeddings=True)
+                         final_norm=norm, tied_embeddings=True, logit_multiplier=raw["logit_scale"],
+                         logit_softcap=raw["logit_cap"])
 
 
 @dataclass(frozen=True)
@@ -663,7 +664,8 @@ def toy_table_plain_logits(raw, tensors, tokens):
         h = h + attended + torch.stack(rows)
         h = h + plain_impl.swiglu_mlp(plain_impl.rms_norm(h, t[p + "ffn_norm.weight"], 1e-5), sub(p + "mlp."))
     h = plain_impl.rms_norm(h, t["model.norm.weight"], 1e-5)
-    return h @ t["model.embed_tokens.weight"].T
+    logits = h @ t["model.embed_tokens.weight"].T * raw["logit_scale"]
+    return raw["logit_cap"] * torch.tanh(logits / raw["logit_cap"])       # src/decoder.rs:3349-3355, 4791-4796
 
 
 def exercise_step_table(device, check_device, graphs):
@@ -672,7 +674,8 @@ def exercise_step_table(device, check_device, graphs):
     from macllm_infer_amd import Engine, Lane
     from macllm_infer_amd.weights.random_init import random_tensors
     register_toys()
-    raw = {"architectures": ["ToyTableForTests"], "hidden": 40, "vocab": 77, "decay": 0.8}
+    raw = {"architectures": ["ToyTableForTests"], "hidden": 40, "vocab": 77, "decay": 0.8, "logit_scale": 1.75,
+           "logit_cap": 2.5}
     config = ToyTableConfig(raw)
     tensors = random_tensors(config, 11, torch.float32, "unit")
     engine = Engine(config=config, tensors=tensors, dtype="float32", device=device, kv_cache_block_tokens=8,
@@ -712,5 +715,6 @@ def exercise_step_table(device, check_device, graphs):
         run([(name, 1) for name in order])
     for name in prompts:
         assert (torch.cat(got[name]) - wants[name]).abs().max() < 1e-4, name
+        assert 2.0 < wants[name].abs().max() < 2.5                # the cap on the logits is felt
     engine.cache.check()
     return engine
