@@ -87,6 +87,37 @@ extern "C" int mi_apply_penalties(float* logits, int B, int V, const int* tokens
   return 0;
 }
 
+// ---------------------------------------------------------------- a constraint on the tokens
+// Rows with a list of allowed tokens (ids[offsets[b] .. offsets[b + 1]), not empty) keep the logits of those and
+// get -inf everywhere else; rows without one stay as they are.  After the penalties and before argmax or the draw
+// (reference: src/sampling.rs:119-130, a constraint masks the penalized row).  One workgroup a row: the row's
+// corner of `keep` (float32 [B, keep_ld]) is filled with -inf, takes the allowed logits, and is copied back.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+keep_allowed_kernel(float* __restrict__ logits, int V, const int* __restrict__ ids, const int* __restrict__ offsets,
+                    float* __restrict__ keep, long keep_ld) {
+  const int row = blockIdx.x;
+  const int lo = offsets[row], hi = offsets[row + 1];
+  if (lo >= hi) return;
+  float* mine = logits + (long)row * V;
+  float* kept = keep + (long)row * keep_ld;
+  for (int v = threadIdx.x; v < V; v += blockDim.x) kept[v] = -INFINITY;
+  __syncthreads();
+  for (int j = lo + threadIdx.x; j < hi; j += blockDim.x) {
+    const int id = ids[j];
+    if (id >= 0 && id < V) kept[id] = mine[id];
+  }
+  __syncthreads();
+  for (int v = threadIdx.x; v < V; v += blockDim.x) mine[v] = kept[v];
+}
+
+extern "C" int mi_keep_allowed(float* logits, int B, int V, const int* ids, const int* offsets, float* keep,
+                               long keep_ld, hipStream_t stream) {
+  if (B <= 0 || V <= 0 || !logits || !ids || !offsets || !keep || keep_ld < V) return ERR_BAD_ARGUMENT;
+  keep_allowed_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, V, ids, offsets, keep, keep_ld);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
 // ---------------------------------------------------------------- argmax
 // (value descending, index ascending) packed so that the smallest 64-bit key wins.
 __device__ __forceinline__ unsigned long long rank_key(float value, int index) {

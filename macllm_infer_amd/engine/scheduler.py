@@ -277,10 +277,29 @@ class Scheduler:
             for request, tokens, samples in visits:
                 if request.prefilling:
                     request.cursor += len(tokens)
+            if sampled and before is not None and any(request.params.constrained_by_history for request, _ in sampled):
+                # a constraint that reads what was generated: the round on its way is read first (the GPU works
+                # on this round's forward pass meanwhile); a request that it ended drops out of the sampling
+                self._resolve(before)
+                before = None
+                keep = [row for row, (request, _) in enumerate(sampled) if not request.finished]
+                if len(keep) < len(sampled):
+                    sampled = [sampled[row] for row in keep]
+                    logits = logits[keep] if keep else None
             if sampled:
-                rows = [SamplerRow(request.params, request.prompt, request.generated,
-                                   None if request.in_flight is None else (request.in_flight[0].device, request.in_flight[1]))
-                        for request, _ in sampled]
+                rows, kept = [], []
+                for row, (request, _) in enumerate(sampled):
+                    try:
+                        rows.append(SamplerRow(request.params, request.prompt, request.generated,
+                                               None if request.in_flight is None
+                                               else (request.in_flight[0].device, request.in_flight[1])))
+                        kept.append(row)
+                    except ValueError as error:          # its constraint allows no token: the request fails alone
+                        self._finish(request, f"failed: {error}")
+                if len(kept) < len(sampled):
+                    sampled = [sampled[row] for row in kept]
+                    logits = logits[kept] if kept else None
+            if sampled:
                 if self.ahead:
                     handle = self.sampler.sample_async(logits, rows)
                     self._pending = (handle, [request for request, _ in sampled])

@@ -106,6 +106,7 @@ _SIGNATURES = {
         "mi_apply_penalties": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                _c_ptr, _c_ptr, _c_ptr, _c_ptr],
         "mi_argmax": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
+        "mi_keep_allowed": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_ptr],
         "mi_sample": [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                       _c_ptr, _c_ptr],
     },
@@ -1049,6 +1050,23 @@ def apply_penalties(logits, tokens, offsets, prompt_lens, repetition, presence, 
     _check(_fn("sampling", "mi_apply_penalties")(
         _p(logits), B, V, _p(tokens), _p(offsets), _p(prompt_lens), _p(repetition), _p(presence), _p(frequency),
         _p(count_all), _p(count_gen), _p(extra_source), _p(extra_rows), _stream()), "apply_penalties")
+
+
+def keep_allowed(logits: torch.Tensor, ids: torch.Tensor, offsets: torch.Tensor, keep: torch.Tensor) -> None:
+    """Rows ``b`` with a list of allowed tokens ``ids[offsets[b]:offsets[b + 1]]`` keep those logits and get -inf
+    everywhere else; rows whose list is empty stay as they are.  ``keep``: a work area with a row of at least
+    ``V`` 32-bit words for each row of ``logits``."""
+    B, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.is_contiguous() and logits.is_cuda, "keep_allowed: bad logits")
+    _i32(ids, "ids")
+    _i32(offsets, "offsets")
+    _need(offsets.numel() == B + 1, "keep_allowed: one offset a row and one more")
+    _need(keep.is_cuda and keep.dim() == 2 and keep.stride(1) == 1 and keep.shape[0] >= B
+          and keep.element_size() in (4, 8), "keep_allowed: bad work area")
+    words = keep.element_size() // 4
+    _need(keep.shape[1] * words >= V, "keep_allowed: the work area's rows are too short")
+    _check(_fn("sampling", "mi_keep_allowed")(_p(logits), B, V, _p(ids), _p(offsets), _p(keep),
+                                              keep.stride(0) * words, _stream()), "keep_allowed")
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:

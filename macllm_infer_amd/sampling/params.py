@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import math
 from dataclasses import dataclass, field
-from typing import Tuple
+from typing import Callable, Optional, Sequence, Tuple, Union
 
 
 @dataclass(frozen=True)
@@ -19,6 +19,11 @@ class SamplingParams:
     seed: int = 42
     ignore_eos: bool = False          # fixed-length runs (the reference's bench mode, src/main.rs:1169)
     stop_token_ids: Tuple[int, ...] = field(default_factory=tuple)
+    # A constraint on what may be generated (the reference masks the penalized logits through a constraint object,
+    # src/sampling.rs:119-130): the token ids that may come next, every other logit counting as -inf; either a
+    # fixed list, or a function of the tokens generated so far that returns the list for the next one (None: any
+    # token).  A request with such a function has its tokens read before its next one is drawn.
+    allowed_token_ids: Optional[Union[Tuple[int, ...], Callable[[Sequence[int]], Optional[Sequence[int]]]]] = None
 
     def __post_init__(self):
         # the reference's checks: src/sampling.rs:43-55, :67-75
@@ -37,6 +42,27 @@ class SamplingParams:
         if self.max_new_tokens <= 0:
             raise ValueError("max_new_tokens must be positive")
         object.__setattr__(self, "stop_token_ids", tuple(int(token) for token in self.stop_token_ids))
+        if self.allowed_token_ids is not None and not callable(self.allowed_token_ids):
+            allowed = tuple(int(token) for token in self.allowed_token_ids)
+            if not allowed or min(allowed) < 0:
+                raise ValueError("allowed_token_ids must name at least one token, none of them negative")
+            object.__setattr__(self, "allowed_token_ids", allowed)
+
+    @property
+    def constrained_by_history(self) -> bool:
+        return callable(self.allowed_token_ids)
+
+    def allowed_after(self, generated: Sequence[int]) -> Optional[Tuple[int, ...]]:
+        """The tokens that may follow ``generated``, or None for any."""
+        if not callable(self.allowed_token_ids):
+            return self.allowed_token_ids
+        allowed = self.allowed_token_ids(generated)
+        if allowed is None:
+            return None
+        allowed = tuple(int(token) for token in allowed)
+        if not allowed or min(allowed) < 0:
+            raise ValueError("the constraint rejected every token")           # src/sampling.rs:131-134
+        return allowed
 
     @property
     def greedy(self) -> bool:

@@ -2,7 +2,8 @@
 
 Order of operations, as the reference's sampler (src/sampling.rs:95-161): repetition
 penalty over prompt and generated tokens, presence and frequency penalties over generated
-tokens, then argmax (lowest index on ties) or temperature -> top-k -> softmax -> top-p ->
+tokens, then the request's constraint if it has one (only the allowed tokens keep their logits), then
+argmax (lowest index on ties) or temperature -> top-k -> softmax -> top-p ->
 one uniform draw, walked in index order.  One draw per stochastic token; the uniform
 comes from a counter-based generator keyed by (seed, number of tokens drawn so far), so a
 request's tokens do not depend on what else is in the batch.
@@ -23,11 +24,14 @@ class SamplerRow:
     """What the sampler needs to know of one request.  ``newest``: (int32 tensor on the device, row) of a token
     already drawn for the request that ``generated`` does not hold yet; it counts for the draw's index and,
     read on the device, for the penalties."""
-    __slots__ = ("params", "prompt", "generated", "newest")
+    __slots__ = ("params", "prompt", "generated", "newest", "allowed")
 
     def __init__(self, params: SamplingParams, prompt: Sequence[int], generated: Sequence[int],
                  newest: Optional[tuple] = None):
         self.params, self.prompt, self.generated, self.newest = params, prompt, generated, newest
+        if newest is not None and params.constrained_by_history:
+            raise ValueError("a constraint that reads the generated tokens needs them all on the host")
+        self.allowed = params.allowed_after(generated)          # the tokens that may come now, or None for any
 
     @property
     def pending(self) -> int:
@@ -119,6 +123,19 @@ class Sampler:
                 packed[2 * B + 1:3 * B + 1].view(torch.float32), packed[3 * B + 1:4 * B + 1].view(torch.float32),
                 packed[4 * B + 1:5 * B + 1].view(torch.float32), count_all, count_gen,
                 newest[0].newest[0] if newest else None, packed[5 * B + 1:head] if newest else None)
+        if any(row.allowed is not None for row in rows):
+            # after the penalties, before the choice (src/sampling.rs:119-130): one upload, offsets then ids
+            offsets = [0]
+            ids: List[int] = []
+            for row in rows:
+                if row.allowed is not None:
+                    if max(row.allowed) >= self.vocab_size:
+                        raise ValueError(f"allowed token {max(row.allowed)} is outside the vocabulary of {self.vocab_size}")
+                    ids.extend(row.allowed)
+                offsets.append(len(ids))
+            words = np.asarray(offsets + ids, dtype=np.int32)
+            packed = torch.from_numpy(words).to(device, non_blocking=True)
+            ops.keep_allowed(logits, packed[B + 1:], packed[:B + 1], self._work(B))
         out = torch.empty(B, dtype=torch.int32, device=device)
         if all(row.params.greedy for row in rows):
             ops.argmax(logits, out)

@@ -399,7 +399,7 @@ def sample_token(logits: torch.Tensor, *, temperature: float = 0.0, top_k: int =
                  top_p: float = 1.0, repetition_penalty: float = 1.0,
                  presence_penalty: float = 0.0, frequency_penalty: float = 0.0,
                  history: Sequence[int] = (), generated: Sequence[int] = (),
-                 seed: int = 0, draw_index: int = 0) -> int:
+                 seed: int = 0, draw_index: int = 0, allowed: Optional[Sequence[int]] = None) -> int:
     """One token from one row of logits, in the reference's order of operations.
 
     Repetition penalty over prompt+generated (x<0 ? x*p : x/p, src/sampling.rs:407-423),
@@ -407,7 +407,8 @@ def sample_token(logits: torch.Tensor, *, temperature: float = 0.0, top_k: int =
     index on ties (:425-433) or: divide by temperature, keep the top-k (value
     descending, index ascending), softmax (max-subtracted, float32), keep the shortest
     descending prefix whose mass reaches top_p (:337-375), draw u*total and walk the
-    kept tokens in index order (:165-169, :378-390).
+    kept tokens in index order (:165-169, :378-390).  ``allowed``: a constraint's mask over the penalized
+    row, every other token at -inf (:119-130, before argmax or the stochastic path).
     """
     import numpy as np
     values = logits.detach().float().cpu().numpy().astype(np.float32).copy()
@@ -423,6 +424,11 @@ def sample_token(logits: torch.Tensor, *, temperature: float = 0.0, top_k: int =
         for token, count in counts.items():
             if 0 <= token < values.size:
                 values[token] -= np.float32(frequency_penalty) * np.float32(count) + np.float32(presence_penalty)
+    if allowed is not None:
+        masked = np.full_like(values, -np.inf)
+        for token in allowed:
+            masked[int(token)] = values[int(token)]
+        values = masked
     if temperature <= 0.0:
         return int(np.argmax(values))                      # first index of the maximum
     values = values / np.float32(temperature)

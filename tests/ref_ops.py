@@ -221,7 +221,7 @@ def argmax(logits, out):
 
 
 NAMES = ["fused_gemm_split", "add_partials_rmsnorm", "prefill_attention_supported", "decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "tanh_softcap", "linear", "rope_kv_store", "paged_attention",
-         "conv1d_silu", "conv_state_update", "ssm_scan", "gate_norm", "argmax", "feed_tokens"]
+         "conv1d_silu", "conv_state_update", "ssm_scan", "gate_norm", "argmax", "feed_tokens", "keep_allowed"]
 
 
 def install(monkeypatch):
@@ -246,6 +246,15 @@ def apply_penalties(logits, tokens, offsets, prompt_lens, repetition, presence, 
         if pres != 0.0 or freq != 0.0:
             for token in set(generated):
                 logits[row, token] -= freq * generated.count(token) + pres
+
+
+def keep_allowed(logits, ids, offsets, keep):
+    for row in range(logits.shape[0]):
+        allowed = ids[int(offsets[row]):int(offsets[row + 1])].long()
+        if allowed.numel():
+            kept = torch.full_like(logits[row], float("-inf"))
+            kept[allowed] = logits[row, allowed]
+            logits[row] = kept
 
 
 def sample(logits, temperature, top_k, top_p, seeds, draw_index, keys, out, done=None):

@@ -249,6 +249,61 @@ def test_sampled_generation_a_round_ahead_equals_generation_that_waits(tmp_path)
         assert generated == outcomes[0][index][0], index
 
 
+def test_generation_under_a_constraint_on_the_tokens(tmp_path):
+    """Requests with a fixed list of allowed tokens, with a list that follows what was generated (the next token
+    must be one of three that depend on the last: the scheduler reads the round on its way before it draws),
+    without any, and one whose constraint comes to allow nothing (it fails alone).  A round ahead and waiting give
+    the same tokens; every token is an allowed one, and the greedy ones are the plain model's best allowed token."""
+    from macllm_infer_amd import Engine, EngineConfig, SamplingParams
+    from macllm_infer_amd.engine.scheduler import Scheduler
+    from macllm_infer_amd.sampling import Sampler
+    folder = tiny_configs.make_model_dir("B", tmp_path, torch.float32)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    V = cfg["vocab_size"]
+    follows = lambda generated: [(generated[-1] * 7 + 3 + k) % V for k in range(3)] if generated else [11, 12, 13]
+    dead_end = lambda generated: [5, 6] if len(generated) < 2 else []
+    fixed = tuple(range(40, 60))
+    params = [SamplingParams(max_new_tokens=9, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0, allowed_token_ids=fixed),
+              SamplingParams(max_new_tokens=8, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.2, allowed_token_ids=follows),
+              SamplingParams(max_new_tokens=7, temperature=0.9, top_k=5, top_p=0.9, seed=3, allowed_token_ids=follows),
+              SamplingParams(max_new_tokens=6, temperature=0.8, top_k=0, top_p=1.0, seed=4, allowed_token_ids=(7, 300, 9)),
+              SamplingParams(max_new_tokens=6, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0),
+              SamplingParams(max_new_tokens=6, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0, allowed_token_ids=dead_end)]
+    prompts = [tokens_for(V, 5 + 3 * index, 600 + index) for index in range(len(params))]
+    outcomes = []
+    for ahead in (True, False):
+        engine = Engine(folder, dtype="float32", kv_cache_block_tokens=8, kv_cache_capacity_tokens=512, max_active_sequences=6)
+        scheduler = Scheduler(engine, Sampler(engine.vocab_size, engine.device),
+                              EngineConfig(max_active_sequences=6, scheduler_token_budget=24, prefill_token_quantum=7))
+        scheduler.ahead = ahead
+        for index, prompt in enumerate(prompts):
+            scheduler.submit(index, prompt, params[index])
+        finished = scheduler.run()
+        outcomes.append({index: (request.generated, request.finish_reason) for index, request in finished.items()})
+        assert engine.cache.stats()["live_requests"] == 0
+        engine.cache.check()
+    assert outcomes[0] == outcomes[1]
+    got = outcomes[0]
+    assert [got[index][1] for index in range(5)] == ["length"] * 5
+    assert got[5][1].startswith("failed") and "rejected every token" in got[5][1] and len(got[5][0]) == 2
+    assert set(got[5][0]) <= {5, 6} and set(got[0][0]) <= set(fixed) and set(got[3][0]) <= {7, 300, 9}
+    for index in (1, 2):
+        generated = got[index][0]
+        assert all(token in follows(generated[:place]) for place, token in enumerate(generated))
+    assert not set(got[4][0]) <= set(fixed)
+    for index in (0, 1):                                           # greedy: the plain model's best allowed token
+        p, tokens, generated = params[index], list(prompts[index]), []
+        for _ in got[index][0]:
+            logits = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-1]
+            allowed = list(p.allowed_after(generated))
+            token = plain_impl.sample_token(
+                logits, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=p.repetition_penalty, presence_penalty=0.0,
+                frequency_penalty=0.0, history=tokens, generated=generated, seed=p.seed, draw_index=0, allowed=allowed)
+            tokens.append(token)
+            generated.append(token)
+        assert generated == got[index][0], index
+
+
 def test_generation_with_more_live_requests_than_the_skinny_kernels_take_rows(tmp_path):
     """Seventy-two requests live at once through the scheduler (bfloat16, configuration D): prompts of 3 to 40
     tokens in portions of 24 beside the decoded tokens of the others (so steps run as two batches), then rounds of

@@ -790,6 +790,32 @@ def test_penalties_match_the_plain_rule(ops):
     assert int(counts[0].sum()) == 0 and int(counts[1].sum()) == 0
 
 
+def test_allowed_tokens_keep_their_logits_and_the_rest_is_minus_infinity(ops):
+    """Rows with a list keep exactly the listed logits (a list may name a token twice, and the last and the first of
+    a vocabulary that is no multiple of anything); a row without one is untouched; argmax then takes the best
+    allowed token, the lower index on ties."""
+    V = 1031
+    logits = rand(4, V, seed=91)
+    logits[2, 17] = logits[2, 800] = 50.0                       # a tie among the allowed ones
+    lists = [[0, 5, 1030, 5], [], [800, 17, 3], [1030]]
+    offsets, flat = [0], []
+    for allowed in lists:
+        flat += allowed
+        offsets.append(len(flat))
+    want = logits.clone()
+    ref_ops.keep_allowed(want, i32(flat), i32(offsets), None)
+    got = logits.clone().to(DEV)
+    keep = torch.full((4, 2048), 7, dtype=torch.int64, device=DEV)            # the sampler's work area, dirty
+    ops.keep_allowed(got, i32(flat).to(DEV), i32(offsets).to(DEV), keep)
+    assert torch.equal(got.cpu(), want)
+    assert torch.equal(want[1], logits[1]) and int(torch.isfinite(want[0]).sum()) == 3 and int(torch.isfinite(want[3]).sum()) == 1
+    out = torch.empty(4, dtype=torch.int32, device=DEV)
+    ops.argmax(got, out)
+    assert out.cpu().tolist() == [max((0, 5, 1030), key=lambda token: float(logits[0, token])), int(logits[1].argmax()), 17, 1030]
+    with pytest.raises(ops.KernelError):
+        ops.keep_allowed(got, i32(flat).to(DEV), i32(offsets).to(DEV), torch.empty((4, 500), dtype=torch.float32, device=DEV))
+
+
 # ------------------------------------------------------------------ decode attention (split over the context)
 @pytest.mark.parametrize("Hq, Hkv, dh, page_size, window", [(8, 2, 64, 16, None), (12, 2, 128, 16, None),
                                                               (5, 5, 64, 8, None), (8, 1, 128, 64, None),

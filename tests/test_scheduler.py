@@ -309,3 +309,65 @@ def test_a_single_lane_without_pages_and_nothing_on_its_way_fails_alone_a_round_
     finished = scheduler.run()
     assert sorted(request.finish_reason for request in finished.values()) == ["length", "resource_exhausted"]
     assert engine.lengths == {} and not scheduler.active
+
+
+class ConstrainedSampler(AsyncArgmaxSampler):
+    """The best allowed token of every row (what the sampler's mask and argmax make of a row)."""
+    def _masked(self, logits, rows):
+        logits = logits.clone()
+        for index, row in enumerate(rows):
+            if row.allowed is not None:
+                kept = torch.full_like(logits[index], float("-inf"))
+                kept[list(row.allowed)] = logits[index, list(row.allowed)]
+                logits[index] = kept
+        return logits
+
+    def sample(self, logits, rows):
+        return super().sample(self._masked(logits, rows), rows)
+
+    def sample_async(self, logits, rows):
+        return super().sample_async(self._masked(logits, rows), rows)
+
+
+@pytest.mark.parametrize("ahead", [True, False])
+def test_a_constraint_that_follows_the_generated_tokens_is_asked_with_all_of_them(ahead):
+    """The fake model wants last + 1; request 0 may only take last + 2 (of what it generated last, or 20 to begin
+    with), request 1 only tokens of a fixed list, request 2 anything, and request 3's constraint allows nothing
+    after two tokens.  A round ahead, the scheduler reads the round on its way before it asks request 0's
+    constraint; the outcome is that of the scheduler that waits, and request 3 fails alone."""
+    engine = AheadEngine()
+    scheduler = Scheduler(engine, ConstrainedSampler(), EngineConfig(), ())
+    scheduler.ahead = ahead
+    asked = []
+
+    def plus_two(generated):
+        asked.append(list(generated))
+        return [(generated[-1] + 2) % 50] if generated else [20]
+
+    common = dict(max_new_tokens=5, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0)
+    scheduler.submit(0, [1, 2, 3], SamplingParams(allowed_token_ids=plus_two, **common))
+    scheduler.submit(1, [7, 8], SamplingParams(allowed_token_ids=(30, 31, 40), **common))
+    scheduler.submit(2, [11, 12, 13, 14], SamplingParams(**common))
+    scheduler.submit(3, [5], SamplingParams(allowed_token_ids=lambda generated: [9] if len(generated) < 2 else [], **common))
+    finished = scheduler.run()
+    assert finished[0].generated == [20, 22, 24, 26, 28] and finished[0].finish_reason == "length"
+    assert asked == [[], [20], [20, 22], [20, 22, 24], [20, 22, 24, 26]]      # every call saw every token before it
+    assert set(finished[1].generated) <= {30, 31, 40} and len(finished[1].generated) == 5
+    assert finished[2].generated == [15, 16, 17, 18, 19]
+    assert finished[3].generated == [9, 9] and finished[3].finish_reason.startswith("failed")
+    assert "rejected every token" in finished[3].finish_reason
+    assert not engine.lengths                                                 # everything was given back
+    # the constrained request's lanes carried the tokens it generated, never one still on its way
+    lanes_of_0 = [tokens for call in engine.calls for request, tokens, _, _ in call if request == 0]
+    assert lanes_of_0 == [[1, 2, 3], [20], [22], [24], [26]]
+
+
+def test_allowed_token_ids_are_checked_where_they_are_given():
+    with pytest.raises(ValueError, match="at least one token"):
+        SamplingParams(allowed_token_ids=())
+    with pytest.raises(ValueError, match="at least one token"):
+        SamplingParams(allowed_token_ids=(3, -1))
+    params = SamplingParams(allowed_token_ids=[4, 2])
+    assert params.allowed_token_ids == (4, 2) and params.allowed_after([1, 2]) == (4, 2) and not params.constrained_by_history
+    follows = SamplingParams(allowed_token_ids=lambda generated: None if not generated else [generated[-1]])
+    assert follows.constrained_by_history and follows.allowed_after([]) is None and follows.allowed_after([3, 8]) == (8,)
