@@ -9,6 +9,7 @@
 // [slot, H, P, N] in float32 (reference: src/decoder.rs:2269-2294).  A fresh request's slot
 // holds zeros.
 #include "common.h"
+#include <cstdlib>
 
 #define CONV_MAX_K 16
 
@@ -265,40 +266,42 @@ extern "C" int mi_conv_step(void* u, int dtype, long ld, int col_offset, int M, 
 // elements (1, 2, 4 or 8: the smallest number that covers N; one load where alignment allows); 256/R rows per block.
 //
 // The recurrence is serial in the tokens, so what a token costs is what its step waits for.  The tokens of a
-// lane come in blocks of 16 / PER (8 at most): a block's B, C, x and dt are asked for four blocks ahead, each element
-// once a workgroup, laid in LDS one block ahead, and read from there into the registers of the threads that use them
-// before the block's first token; softplus and the exponential are taken once a token, not once a thread; what the lanes of a row add up for a
-// token's output goes to LDS and is added up for the whole block at its end, in the order of the lanes (a pass
-// over the wave for every token costs more than the token's own arithmetic).  Every token goes through the same
-// operations in the same order whatever block it falls into, and in the kernel for steps of single tokens
-// (SINGLE: nothing staged, few registers, many workgroups a compute unit): a step of one token and a prompt of
-// thousands give a position the same bits.
+// lane come in blocks of up to 16: a block's B, C, x, delta and decay are asked for two blocks ahead by all threads
+// of the workgroup, a few elements each and each element once a workgroup, laid in LDS one block ahead, and read
+// from there into the registers of the threads that use them, eight tokens (16 / PER) at a time before the first of
+// them; softplus and the exponential are taken once a token and head, by a small kernel ahead of the scan.  What
+// the R lanes of a row add up for a token's output is added in registers (scan_lanes_sum: a butterfly over the
+// lanes in which both partners of every step add the same two numbers), the outputs of a block wait in a register
+// of the lane with the token's number and leave with one store a block.  Every token goes through the same
+// operations in the same order whatever block it falls into, and in the kernel for steps of single tokens (SINGLE:
+// nothing staged, few registers, many workgroups a compute unit): a step of one token and a prompt of thousands
+// give a position the same bits.
 #define SCAN_MAX_PER_THREAD 8
-#define SCAN_BLOCK_ELEMENTS 16      // tokens of a block times PER
-#define SCAN_STAGE_PIECES (SCAN_BLOCK_ELEMENTS / 2)   // loads of four elements of B|C a lane of the wave whose turn it is sends for
+#define SCAN_BLOCK_ELEMENTS 16      // tokens of a run that goes without a condition, times PER
+#define SCAN_BLOCK_TOKENS 16        // tokens of a block that a workgroup stages, at most
+#define SCAN_THREAD_PIECES 4        // loads of four elements of B|C that a thread sends for, a block
 
-// The shares of a row's R lanes as one sum: four quarters of the row (two halves of two lanes, one lane), each
-// added up in the order of its lanes, then ((q0 + q1) + q2) + q3.  scan_part_sum is one quarter; scan_row_sum all
-// of it in one thread; four threads that take a quarter each and then add the four in that order get the same bits.
-__device__ __forceinline__ float scan_part_sum(const float* shares, int R, int part) {
-  const int width = R >= 4 ? R / 4 : 1;
-  const float* mine = shares + part * width;
-  float sum = 0.f;
-#pragma unroll 16
-  for (int index = 0; index < width; ++index) sum += mine[index];
-  return sum;
+template <int CONTROL, int ROW_MASK>
+__device__ __forceinline__ float scan_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CONTROL, ROW_MASK, 0xf, false));
 }
 
-__device__ __forceinline__ float scan_join_parts(float q0, float q1, float q2, float q3, int R) {
-  float sum = q0;
-  if (R >= 2) sum += q1;
-  if (R >= 4) sum = (sum + q2) + q3;
-  return sum;
-}
-
-__device__ __forceinline__ float scan_row_sum(const float* shares, int R) {
-  return scan_join_parts(scan_part_sum(shares, R, 0), R >= 2 ? scan_part_sum(shares, R, 1) : 0.f,
-                         R >= 4 ? scan_part_sum(shares, R, 2) : 0.f, R >= 4 ? scan_part_sum(shares, R, 3) : 0.f, R);
+// The sum of a value over the R lanes of a row (R a power of two, rows at multiples of R), in the last 16 lanes of
+// the row (in all of them if R <= 16), the same bits in each of those: within 16 lanes step k adds what the lane's
+// group of 2^k lanes holds to what its neighbour group holds, and the lanes of both groups add the same two numbers
+// (neighbours within a quad by quad permutation, then the mirrors of half a row and of a row of 16: after the steps
+// before, every lane of a group holds the group's sum, so any lane of the neighbour group will do); the sums of the
+// 16-lane rows then travel upwards, the last lane of a row to every lane of the next, and of the first two rows to
+// the last two: ((s3 + s2) + (s1 + s0)) in a row of 64.  All in the vector pipeline, nothing through LDS.
+template <int R>
+__device__ __forceinline__ float scan_lanes_sum(float v) {
+  if (R >= 2) v += scan_dpp<0xB1, 0xf>(v);            // quad_perm [1, 0, 3, 2]
+  if (R >= 4) v += scan_dpp<0x4E, 0xf>(v);            // quad_perm [2, 3, 0, 1]
+  if (R >= 8) v += scan_dpp<0x141, 0xf>(v);           // row_half_mirror
+  if (R >= 16) v += scan_dpp<0x140, 0xf>(v);          // row_mirror
+  if (R >= 32) v += scan_dpp<0x142, 0xa>(v);          // row_bcast15 into rows 1 and 3 (the others add 0)
+  if (R >= 64) v += scan_dpp<0x143, 0xc>(v);          // row_bcast31 into rows 2 and 3
+  return v;
 }
 
 // A barrier of the workgroup for what went through LDS, and nothing else.  __syncthreads() also waits for every load
@@ -309,31 +312,26 @@ __device__ __forceinline__ void scan_lds_barrier() {
   __builtin_amdgcn_s_barrier();
 }
 
-// lane `which` of every group of four lanes, in all four (the data-parallel quad permutation)
-template <int WHICH>
-__device__ __forceinline__ float scan_quad_lane(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), WHICH * 0x55, 0xf, 0xf, true));
-}
-
 // VECTORS (staged kernel only): B and C come four neighbouring elements a load (N, the row stride and the columns
 // of B are multiples of 4 and the rows 16-byte aligned); else element by element.
-template <typename T, int PER, bool SINGLE, bool VECTORS>
+template <typename T, int PER, int R, bool SINGLE, bool VECTORS>
 __global__ void __launch_bounds__(256, 2)          // two workgroups a compute unit at least
 ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt, long dt_ld,
                 const float* __restrict__ dt_bias, const float* __restrict__ A, const float* __restrict__ D,
                 float* __restrict__ state, const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids,
-                int H, int P, int N, int G, int R, int block_tokens, float* __restrict__ y, long y_ld) {
-  constexpr int TB = PER == 1 ? SCAN_BLOCK_ELEMENTS / 2 : SCAN_BLOCK_ELEMENTS / PER;    // tokens of a block at most (block_tokens <= TB: a block's x
-                                                       // values are one a thread)
-  extern __shared__ __align__(16) float shares_l[];    // [tokens of a block][rows_per_block][R shares, then the row's x]
-  __shared__ float decay_l[2][TB], delta_l[2][TB];
+                int H, int P, int N, int G, int block_tokens, const float* __restrict__ delta_decay,
+                float* __restrict__ y, long y_ld) {
+  constexpr int TB = PER == 1 ? SCAN_BLOCK_ELEMENTS / 2 : SCAN_BLOCK_ELEMENTS / PER;    // tokens of a run that goes without a condition
+  constexpr int ROWS = 256 / R;                        // rows of a workgroup
+  constexpr int SUM_LANES = R < 16 ? R : 16;           // the last lanes of a row, which hold its sums
+  constexpr int FIRST_SUM_LANE = R - SUM_LANES;
+  extern __shared__ __align__(16) float staged_l[];    // the staged kernel's two blocks of operands
   const int lane = blockIdx.z;
   const int head = blockIdx.y;
   const int tid = threadIdx.x;
-  const int rows_per_block = 256 / R;
   const int row_in_block = tid / R;
-  const int r = tid - row_in_block * R;
-  const int p0 = blockIdx.x * rows_per_block;
+  const int r = tid % R;
+  const int p0 = blockIdx.x * ROWS;
   const int p = p0 + row_in_block;
   const bool active = p < P;
   const int group = head / (H / G);
@@ -348,8 +346,6 @@ ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt
     const int n = r * PER + i;
     s[i] = (active && n < N) ? s_row[n] : 0.f;
   }
-  const float a = A[head];
-  const float bias = dt_bias[head];
   const float skip = D[head];
   // the state is waited for here, once: left to the compiler, the wait lands inside the loop over the blocks, where
   // it also waits for the loads of the blocks ahead, every time round
@@ -357,10 +353,11 @@ ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt
   const long b_col = E + (long)group * N;
   const long c_col = E + (long)G * N + (long)group * N;
   const long x_col = (long)head * P + (active ? p : 0);
-  const int share_ld = R + 1;
-  const int token_ld = rows_per_block * share_ld;
+  float* y_mine = y + (long)head * P + (active ? p : 0);
 
   if (SINGLE) {
+    const float a = A[head];
+    const float bias = dt_bias[head];
     for (long t = t_begin; t < t_end; ++t) {
       const T* row = xbc + t * xbc_ld;
       const float delta = softplus_f(to_float(dt[t * dt_ld + head]) + bias);
@@ -377,47 +374,40 @@ ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt
           partial = fmaf(next, to_float(row[c_col + n]), partial);
         }
       }
-      shares_l[row_in_block * share_ld + r] = partial;
-      if (r == 0) shares_l[row_in_block * share_ld + R] = x;
-      __syncthreads();
-      if (tid < rows_per_block && p0 + tid < P) {
-        const float* shares = shares_l + tid * share_ld;
-        y[t * y_ld + (long)head * P + p0 + tid] = fmaf(skip, shares[R], scan_row_sum(shares, R));
-      }
-      __syncthreads();
+      const float sum = scan_lanes_sum<R>(partial);
+      if (r == R - 1 && active) y_mine[t * y_ld] = fmaf(skip, x, sum);
     }
   } else {
-    // A block's B, C, x and dt are brought in by one of the workgroup's four waves, the waves taking turns: wave w
-    // asks for the blocks w, w + 4, ... into its registers, four blocks before their turn, and lays a block in LDS
-    // while the block before it is added up.  A wave's loads therefore have four blocks' time to arrive, and the
-    // wait for them (which a wave can only state for all of its loads at once) never meets a load that was asked
-    // for a moment ago.  Every element comes in once a workgroup: the rows of a head, and the heads of a group,
-    // read the same B and C.
-    float* b_l = shares_l + block_tokens * token_ld;            // [2][block_tokens][2 N]: B then C of a token
-    float* x_l = b_l + 2 * block_tokens * 2 * N;                // [2][block_tokens][rows_per_block]
-    typedef T pieces __attribute__((ext_vector_type(4)));
+    // A block's operands are brought in by all 256 threads: a thread lays its share of block b + 1 in LDS at the
+    // start of the round of block b, asks for its share of block b + 2 into the same registers, stores the outputs
+    // of block b - 1, and then works on block b.  Its loads so have a block's time to arrive, and the wait for
+    // them (which a wave can only state for all it has asked of memory at once, stores included) never meets a
+    // load or a store of a moment ago.  Every element comes in once a workgroup: the rows of a head, and the
+    // heads of a group, read the same B and C.
     const int row_floats = 2 * N;
+    float* b_l = staged_l;                                      // [2][block_tokens][2 N]: B then C of a token
+    float* x_l = b_l + 2 * block_tokens * row_floats;           // [2][block_tokens][ROWS]
+    float* dd_l = x_l + 2 * block_tokens * ROWS;                // [2][block_tokens][2]: delta, decay
+    typedef T pieces __attribute__((ext_vector_type(4)));
     const int pieces_a_row = (row_floats + 3) / 4;
-    const bool whole_rows = N == R * PER && block_tokens == TB;          // no lane of a row is idle, blocks are of TB tokens
-    const int wave = tid / WAVE;
-    const int lane64 = tid % WAVE;
-    float staged_bc[SCAN_STAGE_PIECES][4], staged_x[4], staged_dt = 0.f;
-    // where this lane's pieces lie in a block (the same for every block: worked out once, a division each)
-    int piece_token[SCAN_STAGE_PIECES], piece_col[SCAN_STAGE_PIECES];
+    const bool whole_rows = N == R * PER;                       // no lane of a row is idle
+    float staged_bc[SCAN_THREAD_PIECES][4], staged_x = 0.f, staged_dd = 0.f;
+    // where this thread's pieces lie in a block (the same for every block: worked out once, a division each)
+    int piece_token[SCAN_THREAD_PIECES], piece_col[SCAN_THREAD_PIECES];
 #pragma unroll
-    for (int j = 0; j < SCAN_STAGE_PIECES; ++j) {
-      const int index = lane64 + j * WAVE;
+    for (int j = 0; j < SCAN_THREAD_PIECES; ++j) {
+      const int index = tid + j * 256;
       piece_token[j] = index / pieces_a_row;
       piece_col[j] = (index - piece_token[j] * pieces_a_row) * 4;
     }
-    const int rows_shift = __ffs(rows_per_block) - 1;               // rows_per_block is a power of two
-    // block `block` of the lane into this wave's registers (nothing if the lane has no such block)
+    const int x_token = tid / ROWS, x_row = tid % ROWS;
+    // this thread's share of block `block` of the lane into its registers (nothing if the lane has no such block)
     auto fetch = [&](int block) {
       const long t0 = t_begin + (long)block * block_tokens;
       const int count = (int)max(0L, min((long)block_tokens, t_end - t0));
       if (count <= 0) return;
 #pragma unroll
-      for (int j = 0; j < SCAN_STAGE_PIECES; ++j) {
+      for (int j = 0; j < SCAN_THREAD_PIECES; ++j) {
         const int token = min(piece_token[j], count - 1);           // a piece past the block reads its last token, unused
         const int col = piece_col[j];
         if (VECTORS) {
@@ -433,16 +423,11 @@ ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt
           }
         }
       }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int index = min(lane64 + j * WAVE, count * rows_per_block - 1);
-        const int token = index >> rows_shift;
-        const int row = p0 + index - (token << rows_shift);
-        staged_x[j] = row < P ? to_float(xbc[(t0 + token) * xbc_ld + (long)head * P + row]) : 0.f;
-      }
-      staged_dt = to_float(dt[(t0 + min(lane64, count - 1)) * dt_ld + head]);
+      const int row = p0 + x_row;
+      staged_x = row < P ? to_float(xbc[(t0 + min(x_token, count - 1)) * xbc_ld + (long)head * P + row]) : 0.f;
+      staged_dd = delta_decay[((t0 + min(tid >> 1, count - 1)) * H + head) * 2 + (tid & 1)];
     };
-    // this wave's registers (block `block`) into LDS: B, C and x as they are, dt as delta and decay
+    // this thread's registers (block `block`) into LDS
     auto lay_down = [&](int block) {
       const long t0 = t_begin + (long)block * block_tokens;
       const int count = (int)max(0L, min((long)block_tokens, t_end - t0));
@@ -450,7 +435,7 @@ ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt
       const int phase = block & 1;
       float* rows_l = b_l + phase * block_tokens * row_floats;
 #pragma unroll
-      for (int j = 0; j < SCAN_STAGE_PIECES; ++j) {
+      for (int j = 0; j < SCAN_THREAD_PIECES; ++j) {
         const int token = piece_token[j];
         const int col = piece_col[j];
         if (token < count) {
@@ -464,98 +449,93 @@ ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt
           }
         }
       }
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (lane64 + j * WAVE < count * rows_per_block) x_l[phase * block_tokens * rows_per_block + lane64 + j * WAVE] = staged_x[j];
-      if (lane64 < count) {
-        const float delta = softplus_f(staged_dt + bias);
-        delta_l[phase][lane64] = delta;
-        decay_l[phase][lane64] = expf(delta * a);
-      }
+      if (x_token < count) x_l[phase * block_tokens * ROWS + tid] = staged_x;
+      if (tid < 2 * count) dd_l[phase * block_tokens * 2 + tid] = staged_dd;
     };
-    fetch(wave);                             // blocks 0 .. 3, one a wave
-    if (wave == 0) {
-      lay_down(0);
-      fetch(4);
-    }
+    // the outputs of the block before: token i of the block waits in the i-th of the row's lanes that hold sums
+    // (block_tokens <= SUM_LANES)
+    float kept = 0.f;
+    long kept_t0 = 0;
+    int kept_count = 0;
+    auto store_kept = [&]() {
+      if (r >= FIRST_SUM_LANE && r - FIRST_SUM_LANE < kept_count && active) y_mine[(kept_t0 + r - FIRST_SUM_LANE) * y_ld] = kept;
+    };
+    fetch(0);
+    lay_down(0);
+    fetch(1);
     const int blocks = (int)((t_end - t_begin + block_tokens - 1) / block_tokens);
     for (int block = 0; block < blocks; ++block) {
       const long t0 = t_begin + (long)block * block_tokens;
       const int count = (int)min((long)block_tokens, t_end - t0);
       const int phase = block & 1;
-      scan_lds_barrier();                   // this block's operands are laid down, and the block before has been
-                                            // added up: its shares may be overwritten
+      scan_lds_barrier();                   // this block's operands are laid down, and everybody has read the block
+                                            // before the last: its place may be written
+      if (block > 0) {
+        lay_down(block + 1);
+        fetch(block + 2);
+        store_kept();
+      }
       const float* rows_l = b_l + phase * block_tokens * row_floats;
-      const float* x_now = x_l + phase * block_tokens * rows_per_block + row_in_block;
+      const float* x_now = x_l + phase * block_tokens * ROWS + row_in_block;
+      const float* dd_now = dd_l + phase * block_tokens * 2;
       const float* mine_l = rows_l + min(r * PER, N - PER > 0 ? N - PER : 0);    // this thread's columns of B (C: N further)
-      float* shares_mine = shares_l + row_in_block * share_ld + r;
-      // a whole block of a row whose lanes all hold PER elements runs without a condition: straight code whose
-      // LDS addresses are constants; the last block of a lane and rows with idle lanes take the guarded loop
-      if (count == TB && whole_rows) {
-        float b[TB][PER], c[TB][PER], decay[TB], dx[TB], x[TB];
+      // runs of TB tokens of a row whose lanes all hold PER elements go without a condition: straight code that
+      // asks LDS for the run's operands at once; what is left of a block, and rows with idle lanes, take the
+      // guarded loop
+      int done = 0;
+      if (whole_rows) {
+        for (; done + TB <= count; done += TB) {
+          float b[TB][PER], c[TB][PER], decay[TB], dx[TB], x[TB];
 #pragma unroll
-        for (int token = 0; token < TB; ++token) {
-          decay[token] = decay_l[phase][token];
-          x[token] = x_now[token * rows_per_block];
-          dx[token] = delta_l[phase][token] * x[token];
+          for (int token = 0; token < TB; ++token) {
+            decay[token] = dd_now[(done + token) * 2 + 1];
+            x[token] = x_now[(done + token) * ROWS];
+            dx[token] = dd_now[(done + token) * 2] * x[token];
 #pragma unroll
-          for (int i = 0; i < PER; ++i) {
-            b[token][i] = mine_l[token * row_floats + i];
-            c[token][i] = mine_l[token * row_floats + N + i];
-          }
-        }
-#pragma unroll
-        for (int token = 0; token < TB; ++token) {
-          float partial = 0.f;
-#pragma unroll
-          for (int i = 0; i < PER; ++i) {
-            const float next_s = fmaf(decay[token], s[i], dx[token] * b[token][i]);
-            s[i] = next_s;
-            partial = fmaf(next_s, c[token][i], partial);
-          }
-          shares_mine[token * token_ld] = partial;
-          if (r == 0) shares_mine[token * token_ld + R] = x[token];
-        }
-      } else {
-        for (int token = 0; token < count; ++token) {
-          const float decay = decay_l[phase][token];
-          const float x = x_now[token * rows_per_block];
-          const float dx = delta_l[phase][token] * x;
-          float partial = 0.f;
-#pragma unroll
-          for (int i = 0; i < PER; ++i) {
-            const int n = r * PER + i;
-            if (n < N) {
-              const float next_s = fmaf(decay, s[i], dx * rows_l[token * row_floats + n]);
-              s[i] = next_s;
-              partial = fmaf(next_s, rows_l[token * row_floats + N + n], partial);
+            for (int i = 0; i < PER; ++i) {
+              b[token][i] = mine_l[(done + token) * row_floats + i];
+              c[token][i] = mine_l[(done + token) * row_floats + N + i];
             }
           }
-          shares_mine[token * token_ld] = partial;
-          if (r == 0) shares_mine[token * token_ld + R] = x;
+#pragma unroll
+          for (int token = 0; token < TB; ++token) {
+            float partial = 0.f;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+              const float next_s = fmaf(decay[token], s[i], dx[token] * b[token][i]);
+              s[i] = next_s;
+              partial = fmaf(next_s, c[token][i], partial);
+            }
+            const float out = fmaf(skip, x[token], scan_lanes_sum<R>(partial));
+            kept = r == FIRST_SUM_LANE + done + token ? out : kept;
+          }
         }
       }
-      scan_lds_barrier();
-      // the wave whose turn it is lays the next block down and asks for the block four after that one
-      if (wave == ((block + 1) & 3)) {
-        lay_down(block + 1);
-        fetch(block + 5);
+      for (int token = done; token < count; ++token) {
+        const float decay = dd_now[token * 2 + 1];
+        const float x = x_now[token * ROWS];
+        const float dx = dd_now[token * 2] * x;
+        float partial = 0.f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int n = r * PER + i;
+          if (n < N) {
+            const float next_s = fmaf(decay, s[i], dx * rows_l[token * row_floats + n]);
+            s[i] = next_s;
+            partial = fmaf(next_s, rows_l[token * row_floats + N + n], partial);
+          }
+        }
+        const float out = fmaf(skip, x, scan_lanes_sum<R>(partial));
+        kept = r == FIRST_SUM_LANE + token ? out : kept;
       }
-      // four threads an output, a quarter of the row's shares each
-      const int outputs = count * rows_per_block;
-      for (int first = 0; first < outputs; first += 64) {
-        const int index = min(first + tid / 4, outputs - 1);
-        const int token = index >> rows_shift;
-        const int row = index - (token << rows_shift);
-        const float* shares = shares_l + token * token_ld + row * share_ld;
-        const int part = tid & 3;
-        const float quarter = (part == 0 || R >= 4 || (part == 1 && R >= 2)) ? scan_part_sum(shares, R, part) : 0.f;
-        const float sum = scan_join_parts(scan_quad_lane<0>(quarter), scan_quad_lane<1>(quarter), scan_quad_lane<2>(quarter),
-                                          scan_quad_lane<3>(quarter), R);
-        if (part == 0 && first + tid / 4 < outputs && p0 + row < P)
-          y[(t0 + token) * y_ld + (long)head * P + p0 + row] = fmaf(skip, shares[R], sum);
+      kept_t0 = t0;
+      kept_count = count;
+      if (block == 0) {                     // the first round lays the second block down behind its own work
+        lay_down(1);
+        fetch(2);
       }
     }
+    store_kept();
   }
   if (active) {
 #pragma unroll
@@ -566,15 +546,45 @@ ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt
   }
 }
 
+// delta = softplus(dt + dt_bias[h]) and decay = exp(delta * A[h]) of every token and head, once, for the staged scan
+// (the kernel for steps of single tokens forms the same two values from the same operations itself).
+template <typename T>
+__global__ void scan_delta_decay_kernel(const T* __restrict__ dt, long dt_ld, const float* __restrict__ dt_bias,
+                                        const float* __restrict__ A, int H, long total, float* __restrict__ out) {
+  const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (index >= total) return;
+  const long token = index / H;
+  const int head = (int)(index - token * H);
+  const float delta = softplus_f(to_float(dt[token * dt_ld + head]) + dt_bias[head]);
+  out[2 * index] = delta;
+  out[2 * index + 1] = expf(delta * A[head]);
+}
+
+template <typename T, int PER, int R>
+static void launch_scan(dim3 grid, size_t bytes, hipStream_t stream, bool single, bool vectors, const void* xbc,
+                        long xbc_ld, const void* dt, long dt_ld, const float* dt_bias, const float* A, const float* D,
+                        float* state, const int* cu_seqlens, const int* slot_ids, int H, int P, int N, int G,
+                        int block_tokens, const float* delta_decay, float* y, long y_ld) {
+#define SCAN_ARGUMENTS                                                                                              \
+  (const T*)xbc, xbc_ld, (const T*)dt, dt_ld, dt_bias, A, D, state, cu_seqlens, slot_ids, H, P, N, G, block_tokens, \
+      delta_decay, y, y_ld
+  if (single) ssm_scan_kernel<T, PER, R, true, false><<<grid, 256, bytes, stream>>>(SCAN_ARGUMENTS);
+  else if (vectors) ssm_scan_kernel<T, PER, R, false, true><<<grid, 256, bytes, stream>>>(SCAN_ARGUMENTS);
+  else ssm_scan_kernel<T, PER, R, false, false><<<grid, 256, bytes, stream>>>(SCAN_ARGUMENTS);
+#undef SCAN_ARGUMENTS
+}
+
 // longest: an upper bound of the tokens of a lane (0: unknown); a step whose lanes all hold one token takes the
-// kernel without staging.
+// kernel without staging.  delta_decay: float32 [T, H, 2], a work area that the staged kernel needs (T: the tokens
+// of all lanes); it may be null when longest == 1.
 extern "C" int mi_ssm_scan(const void* xbc, int dtype, long xbc_ld, const void* dt, long dt_ld,
                            const float* dt_bias, const float* A, const float* D, float* state,
                            const int* cu_seqlens, const int* slot_ids, int num_lanes, int longest, int H, int P, int N,
-                           int G, float* y, long y_ld, hipStream_t stream) {
+                           int G, float* delta_decay, long tokens, float* y, long y_ld, hipStream_t stream) {
   if (num_lanes <= 0 || H <= 0 || P <= 0 || N <= 0 || G <= 0 || H % G != 0) return ERR_BAD_ARGUMENT;
   if (N > WAVE * SCAN_MAX_PER_THREAD) return ERR_UNSUPPORTED_SIZE;
   if (H > 65535 || num_lanes > 65535) return ERR_UNSUPPORTED_SIZE;
+  if (dtype != DT_F32 && dtype != DT_BF16) return ERR_BAD_ARGUMENT;
   int R = 1;
   while (R < N && R < WAVE) R <<= 1;
   const int rows_per_block = 256 / R;
@@ -582,40 +592,38 @@ extern "C" int mi_ssm_scan(const void* xbc, int dtype, long xbc_ld, const void* 
   const int per_needed = (N + R - 1) / R;
   const int per = per_needed <= 1 ? 1 : per_needed <= 2 ? 2 : per_needed <= 4 ? 4 : 8;
   const bool single = longest == 1;
-  // tokens of a block: 16 / PER (8 at most), no more than R (so that a block's x values, one a row and token, are at most 256), and
-  // B and C of a block are no more than the wave whose turn it is sends for
-  int block_tokens = per == 1 ? SCAN_BLOCK_ELEMENTS / 2 : SCAN_BLOCK_ELEMENTS / per;
+  if (!single && (!delta_decay || tokens <= 0)) return ERR_BAD_ARGUMENT;
+  // tokens of a block: no more than R (a block's x values, one a row and token, are one a thread, and its outputs
+  // wait one a lane of the row), and B and C of a block no more than SCAN_THREAD_PIECES loads of four elements a thread
+  int block_tokens = SCAN_BLOCK_TOKENS;
   if (block_tokens > R) block_tokens = R;
-  while (block_tokens > 1 && (long)block_tokens * 2 * N > (long)WAVE * 4 * SCAN_STAGE_PIECES) block_tokens /= 2;
-  if (single) block_tokens = 1;
-  const size_t bytes = ((size_t)block_tokens * rows_per_block * (R + 1) +
-                        (single ? 0 : 2 * (size_t)block_tokens * (2 * N + rows_per_block))) * sizeof(float);
+  while (block_tokens > 1 && (long)block_tokens * ((2 * N + 3) / 4) > 256L * SCAN_THREAD_PIECES) block_tokens /= 2;
+  const size_t bytes = single ? 0 : 2 * (size_t)block_tokens * (2 * N + rows_per_block + 2) * sizeof(float);
   // four elements a load: every head's and group's columns of B and C start at multiples of 4
   const bool vectors = !single && N % 4 == 0 && xbc_ld % 4 == 0 && ((long)H * P) % 4 == 0 &&
                        ((uintptr_t)xbc % (dtype == DT_F32 ? 16 : 8)) == 0;
-#define SCAN_LAUNCH(T_, PER_, SINGLE_, VECTORS_)                                                                     \
-  ssm_scan_kernel<T_, PER_, SINGLE_, VECTORS_><<<grid, 256, bytes, stream>>>(                                        \
-      (const T_*)xbc, xbc_ld, (const T_*)dt, dt_ld, dt_bias, A, D, state, cu_seqlens, slot_ids, H, P, N, G, R,       \
-      block_tokens, y, y_ld)
-#define SCAN_BY_PER(T_, SINGLE_, VECTORS_)                     \
-  do {                                                         \
-    if (per == 1) SCAN_LAUNCH(T_, 1, SINGLE_, VECTORS_);       \
-    else if (per == 2) SCAN_LAUNCH(T_, 2, SINGLE_, VECTORS_);  \
-    else if (per == 4) SCAN_LAUNCH(T_, 4, SINGLE_, VECTORS_);  \
-    else SCAN_LAUNCH(T_, 8, SINGLE_, VECTORS_);                \
-  } while (0)
-#define SCAN_BY_KIND(T_)                               \
-  do {                                                 \
-    if (single) SCAN_BY_PER(T_, true, false);          \
-    else if (vectors) SCAN_BY_PER(T_, false, true);    \
-    else SCAN_BY_PER(T_, false, false);                \
-  } while (0)
-  if (dtype == DT_F32) SCAN_BY_KIND(float);
-  else if (dtype == DT_BF16) SCAN_BY_KIND(bf16_t);
-  else return ERR_BAD_ARGUMENT;
-#undef SCAN_BY_KIND
-#undef SCAN_BY_PER
-#undef SCAN_LAUNCH
+  if (!single) {
+    const long total = tokens * H;
+    const int blocks = (int)((total + 255) / 256);
+    if (dtype == DT_F32)
+      scan_delta_decay_kernel<float><<<blocks, 256, 0, stream>>>((const float*)dt, dt_ld, dt_bias, A, H, total, delta_decay);
+    else
+      scan_delta_decay_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)dt, dt_ld, dt_bias, A, H, total, delta_decay);
+    RETURN_IF_LAUNCH_FAILED();
+  }
+#define SCAN_CASE(PER_, R_)                                                                                          \
+  if (per == PER_ && R == R_) {                                                                                      \
+    if (dtype == DT_F32)                                                                                             \
+      launch_scan<float, PER_, R_>(grid, bytes, stream, single, vectors, xbc, xbc_ld, dt, dt_ld, dt_bias, A, D,      \
+                                   state, cu_seqlens, slot_ids, H, P, N, G, block_tokens, delta_decay, y, y_ld);    \
+    else                                                                                                             \
+      launch_scan<bf16_t, PER_, R_>(grid, bytes, stream, single, vectors, xbc, xbc_ld, dt, dt_ld, dt_bias, A, D,     \
+                                    state, cu_seqlens, slot_ids, H, P, N, G, block_tokens, delta_decay, y, y_ld);   \
+  }
+  // a row narrower than a wave has one element a lane; a row of 64 lanes 1, 2, 4 or 8
+  SCAN_CASE(1, 1) SCAN_CASE(1, 2) SCAN_CASE(1, 4) SCAN_CASE(1, 8) SCAN_CASE(1, 16) SCAN_CASE(1, 32) SCAN_CASE(1, 64)
+  SCAN_CASE(2, 64) SCAN_CASE(4, 64) SCAN_CASE(8, 64)
+#undef SCAN_CASE
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

@@ -62,7 +62,7 @@ _SIGNATURES = {
                                  _c_ptr],
         "mi_conv_step": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
         "mi_ssm_scan": [_c_ptr, _c_int, _c_long, _c_ptr, _c_long, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_ptr],
+                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr],
         "mi_gate_norm": [_c_ptr, _c_long, _c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_float, _c_ptr, _c_long,
                          _c_int, _c_int, _c_ptr],
     },
@@ -575,9 +575,12 @@ def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A: torc
     _i32(slot_ids, "slot_ids")
     num_lanes = slot_ids.numel()
     _need(cu_seqlens.numel() == num_lanes + 1, "ssm_scan: cu_seqlens must have lanes+1 entries")
+    longest = min(int(longest), T) if longest and longest > 0 else T
+    # lanes of several tokens: every token's delta and decay are formed once, ahead of the scan, into a work area
+    delta_decay = None if longest == 1 else torch.empty((T, H, 2), dtype=torch.float32, device=xbc.device)
     _check(_fn("mamba2", "mi_ssm_scan")(
         _p(xbc), _dt(xbc), xbc_ld, _p(dt), dt_ld, _p(dt_bias), _p(A), _p(D), _p(ssm_state), _p(cu_seqlens),
-        _p(slot_ids), num_lanes, min(int(longest), T) if longest and longest > 0 else T, H, P, N, num_groups, _p(y), y_ld,
+        _p(slot_ids), num_lanes, longest, H, P, N, num_groups, _p(delta_decay), T, _p(y), y_ld,
         _stream()), "ssm_scan", f"(N={N})")
 
 
