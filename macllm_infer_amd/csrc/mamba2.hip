@@ -42,6 +42,50 @@ __global__ void conv1d_silu_kernel(const T* __restrict__ u, long ld, int col_off
   out[index] = from_float<T>(silu_f(sum));
 }
 
+// The same for float32 with four neighbouring channels a thread (16-byte loads of the rows, the taps of the four
+// channels in K loads): every channel's sum is formed from the same products in the same order as above.
+template <int K>
+__global__ void __launch_bounds__(256)
+conv1d_silu_f32x4_kernel(const float* __restrict__ u, long ld, int col_offset, int C,
+                         const float* __restrict__ weight, const float* __restrict__ bias,
+                         const float* __restrict__ conv_state, const int* __restrict__ lane_of_token,
+                         const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids,
+                         float* __restrict__ out, long total) {
+  const long index = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (index >= total) return;
+  const int vectors = C / 4;
+  const long token = index / vectors;
+  const int channel = (int)(index - token * vectors) * 4;
+  const int lane = lane_of_token[token];
+  const long lane_start = cu_seqlens[lane];
+  const float* tail = conv_state + (long)slot_ids[lane] * (K - 1) * C;
+  float4 window[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const long source = token - (K - 1) + k;
+    // one load, from the rows or from the tail: the address is chosen, not the load
+    const float* from = source >= lane_start ? u + source * ld + col_offset + channel
+                                             : tail + ((K - 1) + (source - lane_start)) * C + channel;
+    window[k] = *reinterpret_cast<const float4*>(from);
+  }
+  float taps[4 * K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    const float4 four = *reinterpret_cast<const float4*>(weight + (long)channel * K + 4 * j);
+    taps[4 * j] = four.x, taps[4 * j + 1] = four.y, taps[4 * j + 2] = four.z, taps[4 * j + 3] = four.w;
+  }
+  float4 result;
+  float* results = reinterpret_cast<float*>(&result);
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    float sum = bias ? bias[channel + c] : 0.f;
+#pragma unroll
+    for (int k = 0; k < K; ++k) sum += taps[c * K + k] * reinterpret_cast<const float*>(&window[k])[c];
+    results[c] = silu_f(sum);
+  }
+  *reinterpret_cast<float4*>(out + token * (long)C + channel) = result;
+}
+
 // The same for bfloat16 with 8 channels and 4 consecutive token rows per thread: the rows the four
 // windows share are loaded once, 16 bytes at a time, together with the taps (contiguous for 8
 // channels) and the lanes of the four tokens; no load stands under a condition.  The common case
@@ -137,6 +181,22 @@ extern "C" int mi_conv1d_silu(const void* u, int dtype, long ld, int col_offset,
     else if (K == 3) CONV_CASE(3);
     else CONV_CASE(4);
 #undef CONV_CASE
+    RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
+  const bool aligned4 = C % 4 == 0 && ld % 4 == 0 && col_offset % 4 == 0 && ((uintptr_t)u % 16) == 0 &&
+                        ((uintptr_t)out % 16) == 0 && ((uintptr_t)conv_state % 16) == 0 && ((uintptr_t)weight % 16) == 0;
+  if (dtype == DT_F32 && aligned4 && K >= 2 && K <= 4) {
+    const long threads = (long)T * (C / 4);
+    const int vec_blocks = (int)((threads + 255) / 256);
+#define CONV_F32_CASE(K_)                                                                                        \
+  conv1d_silu_f32x4_kernel<K_><<<vec_blocks, 256, 0, stream>>>((const float*)u, ld, col_offset, C, weight, bias, \
+                                                               (const float*)conv_state, lane_of_token,          \
+                                                               cu_seqlens, slot_ids, (float*)out, threads)
+    if (K == 2) CONV_F32_CASE(2);
+    else if (K == 3) CONV_F32_CASE(3);
+    else CONV_F32_CASE(4);
+#undef CONV_F32_CASE
     RETURN_IF_LAUNCH_FAILED();
     return 0;
   }
@@ -485,18 +545,22 @@ ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt
       int done = 0;
       if (whole_rows) {
         for (; done + TB <= count; done += TB) {
-          float b[TB][PER], c[TB][PER], decay[TB], dx[TB], x[TB];
+          float b[TB][PER], c[TB][PER], decay[TB], dx[TB];
 #pragma unroll
           for (int token = 0; token < TB; ++token) {
-            decay[token] = dd_now[(done + token) * 2 + 1];
-            x[token] = x_now[(done + token) * ROWS];
-            dx[token] = dd_now[(done + token) * 2] * x[token];
+            const float2 delta_and_decay = *reinterpret_cast<const float2*>(dd_now + (done + token) * 2);
+            decay[token] = delta_and_decay.y;
+            dx[token] = delta_and_decay.x * x_now[(done + token) * ROWS];
 #pragma unroll
             for (int i = 0; i < PER; ++i) {
               b[token][i] = mine_l[(done + token) * row_floats + i];
               c[token][i] = mine_l[(done + token) * row_floats + N + i];
             }
           }
+          // the x of the token whose output this lane keeps (any token of the run for the other lanes)
+          const int my_token = done + ((r - FIRST_SUM_LANE - done) & (TB - 1));
+          const float my_x = x_now[my_token * ROWS];
+          float my_sum = 0.f;
 #pragma unroll
           for (int token = 0; token < TB; ++token) {
             float partial = 0.f;
@@ -506,9 +570,10 @@ ssm_scan_kernel(const T* __restrict__ xbc, long xbc_ld, const T* __restrict__ dt
               s[i] = next_s;
               partial = fmaf(next_s, c[token][i], partial);
             }
-            const float out = fmaf(skip, x[token], scan_lanes_sum<R>(partial));
-            kept = r == FIRST_SUM_LANE + done + token ? out : kept;
+            const float sum = scan_lanes_sum<R>(partial);
+            my_sum = my_token == done + token ? sum : my_sum;
           }
+          kept = (r >= FIRST_SUM_LANE + done && r < FIRST_SUM_LANE + done + TB) ? fmaf(skip, my_x, my_sum) : kept;
         }
       }
       for (int token = done; token < count; ++token) {

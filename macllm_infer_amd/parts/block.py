@@ -3,10 +3,39 @@ from __future__ import annotations
 
 from typing import Dict
 
+import torch
+
 from .base import BuildContext, Residual, part_class
 
 _ARRANGEMENTS: Dict[str, type] = {}
 _FUSIONS: Dict[str, object] = {}
+
+OVERLAP_MIN_TOKENS = 256       # prompt portions from this size on run their two mixers on two streams
+_side_streams: Dict[int, list] = {}
+
+
+def side_stream(device: torch.device, beside: "torch.cuda.Stream") -> "torch.cuda.Stream":
+    """A second stream of the device (default priority) that is not ``beside``.  Streams come from a pool of a
+    few dozen that hands them out in turn, so the one drawn may be the very stream a graph is being captured on:
+    work recorded "beside" it would queue behind (a 2,048-token prompt of the 0.5B shape: 7.2 ms instead of 6.3)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    streams = _side_streams.setdefault(index, [])
+    for stream in streams:
+        if stream != beside:
+            return stream
+    while True:
+        streams.append(torch.cuda.Stream(device=device))
+        if streams[-1] != beside:
+            return streams[-1]
+
+
+def overlap_pays(mixers, rows: int, device: torch.device) -> bool:
+    """Whether two mixers of a layer that read the same rows should run beside each other on two streams: in a
+    captured graph only (launched one by one the step waits for the host, which the second stream costs more),
+    for portions long enough to be worth the hops between the queues, and if both only queue work."""
+    return (len(mixers) == 2 and rows >= OVERLAP_MIN_TOKENS and device.type == "cuda"
+            and torch.cuda.is_current_stream_capturing()
+            and all(getattr(mixer, "graph_safe", False) for mixer in mixers))
 
 
 def register_fusion(arrangement: str):
@@ -101,6 +130,19 @@ class ParallelPreNormBlock:
         if fusion is not None and fusion.forward(residual, step, caches):
             return
         normed = self.mixer_norm.forward(residual)
-        residual.pending = [mixer.forward(normed, step, caches[name]) for name, mixer in self.mixers]
+        if overlap_pays([mixer for _, mixer in self.mixers], normed.shape[0], normed.device):
+            # the second mixer is recorded first and stays on the queue of the kernels around it (see the fast
+            # path's ``forward_general``); what either allocates is its own stream's until the join
+            (first_name, first), (second_name, second) = self.mixers
+            main = torch.cuda.current_stream(normed.device)
+            side = side_stream(normed.device, main)
+            side.wait_stream(main)
+            second_out = second.forward(normed, step, caches[second_name])
+            with torch.cuda.stream(side):
+                first_out = first.forward(normed, step, caches[first_name])
+            main.wait_stream(side)
+            residual.pending = [first_out, second_out]
+        else:
+            residual.pending = [mixer.forward(normed, step, caches[name]) for name, mixer in self.mixers]
         normed = self.ffn_norm.forward(residual)
         residual.pending = [self.ffn.forward(normed)]

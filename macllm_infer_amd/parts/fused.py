@@ -48,7 +48,7 @@ import torch
 
 from ..kernels import ops
 from .base import Residual, ScaledRows
-from .block import register_fusion
+from .block import overlap_pays, register_fusion, side_stream
 
 MAX_ROWS = 64          # rows of a step the skinny kernels take
 MAX_NORM_ROWS = 16     # the norm prologue recomputes the normed rows in every workgroup: small batches only
@@ -139,25 +139,6 @@ PLAN_FIELDS = ("library_in", "library_out", "library_gate_up", "library_down", "
                "tiles_in", "tiles_out", "tiles_gate_up", "tiles_down", "deferred")
 _chain_wins: Dict[tuple, tuple] = {}
 _chain_times: list = []     # (rows, microseconds a layer of each candidate, the one taken): what was measured, for whoever asks
-
-
-OVERLAP_MIN_TOKENS = 256       # prompt portions from this size on run their two mixers on two streams
-_side_streams: Dict[int, list] = {}
-
-
-def _side_stream(device: torch.device, beside: "torch.cuda.Stream") -> "torch.cuda.Stream":
-    """A second stream of the device (default priority) that is not ``beside``.  Streams come from a pool of a
-    few dozen that hands them out in turn, so the one drawn may be the very stream a graph is being captured on:
-    work recorded "beside" it would queue behind (a 2,048-token prompt of the 0.5B shape: 7.2 ms instead of 6.3)."""
-    index = device.index if device.index is not None else torch.cuda.current_device()
-    streams = _side_streams.setdefault(index, [])
-    for stream in streams:
-        if stream != beside:
-            return stream
-    while True:
-        streams.append(torch.cuda.Stream(device=device))
-        if streams[-1] != beside:
-            return streams[-1]
 
 
 def _bucket(rows: int) -> int:
@@ -641,8 +622,7 @@ class LayerFusion:
         else:
             u = ops.linear(normed, self.w_in, self.b_in)
         mixed = torch.empty((u.shape[0], self.mixed_width), dtype=u.dtype, device=u.device)
-        if (len(self.mixers) == 2 and u.shape[0] >= OVERLAP_MIN_TOKENS and torch.cuda.is_current_stream_capturing()
-                and all(getattr(mixer, "graph_safe", False) for mixer in self.mixers)):
+        if overlap_pays(self.mixers, u.shape[0], u.device):
             # two mixers read the same rows and write different columns: the first runs on a second stream
             # beside the second (in a captured graph only: launched one by one the step waits for the host,
             # which the second stream costs more).  The mixer on the main stream is recorded first: the graph
@@ -650,7 +630,7 @@ class LayerFusion:
             # other branch pays the hops between queues.  (Attention beside a state-space mixer, whose kernels
             # are many and small: the state-space chain is the longer one and stays on the main queue.)
             main = torch.cuda.current_stream(u.device)
-            side = _side_stream(u.device, main)
+            side = side_stream(u.device, main)
             side.wait_stream(main)
             self._mix_each(u, step, caches, mixed, order=(1,))
             with torch.cuda.stream(side):

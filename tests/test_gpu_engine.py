@@ -1182,12 +1182,12 @@ def test_long_portions_overlap_their_mixers(tmp_path, name):
     by kernel and, from the second step of that size on, from a captured graph; then the same requests go on
     with a portion and a decoded token.  Every wanted row against the plain model."""
     from macllm_infer_amd import Engine, Lane
-    from macllm_infer_amd.parts import fused
+    from macllm_infer_amd.parts import block
     folder = tiny_configs.make_model_dir(name, tmp_path, torch.bfloat16)
     cfg, tensors = plain_impl.load_model_dir(folder)
     engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=4096,
                     max_active_sequences=8)
-    assert engine.model.blocks[0].fusion is not None and fused.OVERLAP_MIN_TOKENS <= 259
+    assert engine.model.blocks[0].fusion is not None and block.OVERLAP_MIN_TOKENS <= 259
 
     def check(got, want):
         scale = want.abs().max().item()
@@ -1217,14 +1217,53 @@ def test_the_second_stream_is_never_the_stream_it_runs_beside(monkeypatch):
     """Streams come from a pool that hands them out in turn; whichever of them a graph is captured on, the
     stream that the first mixer of a long portion runs on is another one (on the same one the two mixers
     would run one after the other), and two streams are all that is ever drawn for it."""
-    from macllm_infer_amd.parts import fused
-    monkeypatch.setattr(fused, "_side_streams", {})
+    from macllm_infer_amd.parts import block
+    monkeypatch.setattr(block, "_side_streams", {})
     device = torch.device(DEV)
     pool = [torch.cuda.Stream(device=device) for _ in range(70)]           # every stream of the pool, twice over
     for main in pool + [torch.cuda.current_stream(device)]:
-        side = fused._side_stream(device, main)
+        side = block.side_stream(device, main)
         assert side != main and side.device == main.device
-    assert len(fused._side_streams[device.index]) <= 2
+    assert len(block._side_streams[device.index]) <= 2
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_long_float32_portions_overlap_their_mixers_and_keep_their_bits(tmp_path, monkeypatch, name):
+    """The float32 path runs a layer part by part; in a captured graph the two mixers of a portion of 256 tokens
+    or more run beside each other on two streams there too.  Prompts of 300 and 259 tokens beside each other, the
+    same shape of step four times over (launched kernel by kernel first, from the graph of its capacity after):
+    every replay gives the bits of an engine without graphs, which never leaves one stream."""
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.parts import block
+    folder = tiny_configs.make_model_dir(name, tmp_path, torch.float32)
+    cfg, _ = plain_impl.load_model_dir(folder)
+    forks = []
+    real = block.side_stream
+    monkeypatch.setattr(block, "side_stream", lambda device, beside: (forks.append(1), real(device, beside))[1])
+    make = lambda graphs: Engine(folder, dtype="float32", kv_cache_block_tokens=16, kv_cache_capacity_tokens=4096,
+                                 max_active_sequences=8, decode_graphs=graphs)
+    with_graphs, eager = make(True), make(False)
+    assert with_graphs.model.blocks[0].fusion is None
+    for turn in range(4):
+        a, b = f"a{turn}", f"b{turn}"
+        tokens_a = tokens_for(cfg["vocab_size"], 340, 2000 + turn)
+        tokens_b = tokens_for(cfg["vocab_size"], 270, 2100 + turn)
+        rows = []
+        for engine in (with_graphs, eager):
+            engine.add_request(a)
+            engine.add_request(b)
+            first = engine.step([Lane(a, tokens_a[:300], [0, 150, 299]), Lane(b, tokens_b[:259], [258])]).cpu()
+            second = engine.step([Lane(a, tokens_a[300:], [39]), Lane(b, tokens_b[259:260], [0])]).cpu()
+            rows.append(torch.cat([first, second]))
+            engine.finish(a)
+            engine.finish(b)
+        assert torch.equal(rows[0], rows[1]), turn
+    assert with_graphs.graphs.counts["bucket_replays"] >= 2
+    assert len(forks) >= len(cfg_layers(cfg))                   # every layer of the captured step forked
+
+
+def cfg_layers(cfg):
+    return range(cfg["num_hidden_layers"])
 
 
 @pytest.mark.parametrize("padding", [False, True])
