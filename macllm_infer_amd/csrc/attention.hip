@@ -284,10 +284,11 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
   extern __shared__ __align__(16) float tile_lds[];
   const int k_ld = dh + PT_PAD;                      // a key's row in LDS
   const int v_ld = WAVE + PT_PAD;                    // a dim's row of values in LDS
+  const int p_ld = WAVE + PT_PAD;                    // a query's row of probabilities in LDS
   float* q_lds = tile_lds;                           // [PT_QUERIES][dh]
   float* k_lds = q_lds + PT_QUERIES * dh;            // [64][k_ld]
   float* v_lds = k_lds + WAVE * k_ld;                // [dh][v_ld]
-  float* p_lds = v_lds + dh * v_ld;                  // [PA_WAVES][64]
+  float* p_lds = v_lds + dh * v_ld;                  // [PA_WAVES][PT_PER_WAVE][p_ld]
   const int subtiles = tile_tokens / PT_QUERIES;
   const int tile = blockIdx.x / subtiles;
   const int head = blockIdx.y;
@@ -373,68 +374,93 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
       }
     }
     __syncthreads();
+    // the wave's four queries together: a key's dims and a key's values come out of LDS once for the four (LDS, not
+    // the arithmetic, is what this kernel waits for); every query's products and sums are the ones of the per-token
+    // kernel in their order.  A query that sees no key of the group ends with what its group started with
+    // (maximum -inf, zeros); a query slot past the tile's last is computed on whatever LDS holds and never stored.
+    float dot[PT_PER_WAVE];
+#pragma unroll
+    for (int i = 0; i < PT_PER_WAVE; ++i) dot[i] = 0.f;
+    {
+      const float* k_row = k_lds + lane * k_ld;
+      for (int d = 0; d < dh; d += 4) {
+        const float4 kv = *reinterpret_cast<const float4*>(k_row + d);
+#pragma unroll
+        for (int i = 0; i < PT_PER_WAVE; ++i) {
+          const float4 qv = *reinterpret_cast<const float4*>(q_lds + (wave + i * PA_WAVES) * dh + d);
+          dot[i] = fmaf(qv.x, kv.x, dot[i]);
+          dot[i] = fmaf(qv.y, kv.y, dot[i]);
+          dot[i] = fmaf(qv.z, kv.z, dot[i]);
+          dot[i] = fmaf(qv.w, kv.w, dot[i]);
+        }
+      }
+    }
+    float* p_rows = p_lds + wave * (PT_PER_WAVE * p_ld);          // this wave's four rows of probabilities: no barrier, the wave runs in step
 #pragma unroll
     for (int i = 0; i < PT_PER_WAVE; ++i) {
       const int position = query_position[i];
       int first_key = 0;
       if (window > 0 && position - window + 1 > 0) first_key = position - window + 1;
-      if (position >= group_first && group_first + WAVE > first_key) {           // else: no key of this group for the query
       const int key = group_first + lane;
       const bool visible = key >= first_key && key <= position;
       float score = -INFINITY;
       if (visible) {
-        const float* q_row = q_lds + (wave + i * PA_WAVES) * dh;
-        const float* k_row = k_lds + lane * k_ld;
-        float dot = 0.f;
-        for (int d = 0; d < dh; d += 4) {
-          const float4 qv = *reinterpret_cast<const float4*>(q_row + d);
-          const float4 kv = *reinterpret_cast<const float4*>(k_row + d);
-          dot = fmaf(qv.x, kv.x, dot);
-          dot = fmaf(qv.y, kv.y, dot);
-          dot = fmaf(qv.z, kv.z, dot);
-          dot = fmaf(qv.w, kv.w, dot);
-        }
-        score = dot * scale;
+        score = dot[i] * scale;
         if (slopes) score = fmaf(-slopes[head], (float)(position - key), score);
       }
       const float maximum = wave_max_dpp(score);
       const float p = visible ? (FAST_EXP ? __expf(score - maximum) : expf(score - maximum)) : 0.f;
-      p_lds[wave * WAVE + lane] = p;                  // read by this wave only: no barrier, the wave runs in step
-      __builtin_amdgcn_wave_barrier();
-      // sums over all 64 keys of the group: a key the query does not see has the probability 0 and a finite
-      // value (a key some query of the tile sees, or a zero laid down above), so it adds an exact zero and the
-      // sums are those of the keys from `from` to `to` in their order, which is what the per-token kernel adds
-      const float* p_row = p_lds + wave * WAVE;
-      float normalizer = 0.f;
-      float sums[DIMS] = {};
+      p_rows[i * p_ld + lane] = p;
+      group_max[i][g] = maximum;
+    }
+    __builtin_amdgcn_wave_barrier();
+    // sums over all 64 keys of the group: a key the query does not see has the probability 0 and a finite
+    // value (a key some query of the tile sees, or a zero laid down above), so it adds an exact zero and the
+    // sums are those of the keys from `from` to `to` in their order, which is what the per-token kernel adds
+    {
+      float sums[PT_PER_WAVE][DIMS];
+#pragma unroll
+      for (int i = 0; i < PT_PER_WAVE; ++i)
+#pragma unroll
+        for (int d = 0; d < DIMS; ++d) sums[i][d] = 0.f;
       const float* v_row[DIMS];
 #pragma unroll
       for (int d = 0; d < DIMS; ++d) v_row[d] = v_lds + min(lane + d * WAVE, dh - 1) * v_ld;
+      // the normalizers: lane i adds the probabilities of query i in the order of the keys
+      const float* p_mine = p_rows + (lane & (PT_PER_WAVE - 1)) * p_ld;
+      float normalizer = 0.f;
 #pragma unroll
       for (int j = 0; j < WAVE; j += 4) {
-        const float4 pj = *reinterpret_cast<const float4*>(p_row + j);
-        normalizer += pj.x;
-        normalizer += pj.y;
-        normalizer += pj.z;
-        normalizer += pj.w;
+        const float4 mine = *reinterpret_cast<const float4*>(p_mine + j);
+        normalizer += mine.x;
+        normalizer += mine.y;
+        normalizer += mine.z;
+        normalizer += mine.w;
+        float4 pj[PT_PER_WAVE];
+#pragma unroll
+        for (int i = 0; i < PT_PER_WAVE; ++i) pj[i] = *reinterpret_cast<const float4*>(p_rows + i * p_ld + j);
 #pragma unroll
         for (int d = 0; d < DIMS; ++d) {
           if (d * WAVE < dh) {                          // the same for every lane
             const float4 vj = *reinterpret_cast<const float4*>(v_row[d] + j);
-            sums[d] = fmaf(pj.x, vj.x, sums[d]);
-            sums[d] = fmaf(pj.y, vj.y, sums[d]);
-            sums[d] = fmaf(pj.z, vj.z, sums[d]);
-            sums[d] = fmaf(pj.w, vj.w, sums[d]);
+#pragma unroll
+            for (int i = 0; i < PT_PER_WAVE; ++i) {
+              sums[i][d] = fmaf(pj[i].x, vj.x, sums[i][d]);
+              sums[i][d] = fmaf(pj[i].y, vj.y, sums[i][d]);
+              sums[i][d] = fmaf(pj[i].z, vj.z, sums[i][d]);
+              sums[i][d] = fmaf(pj[i].w, vj.w, sums[i][d]);
+            }
           }
         }
       }
-      group_max[i][g] = maximum;
-      group_norm[i][g] = normalizer;
 #pragma unroll
-      for (int d = 0; d < DIMS; ++d) group_o[i][g][d] = sums[d];
-      __builtin_amdgcn_wave_barrier();
+      for (int i = 0; i < PT_PER_WAVE; ++i) {
+        group_norm[i][g] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, normalizer), i));
+#pragma unroll
+        for (int d = 0; d < DIMS; ++d) group_o[i][g][d] = sums[i][d];
       }
     }
+    __builtin_amdgcn_wave_barrier();
   };
   take_group(std::integral_constant<int, 0>{});
   take_group(std::integral_constant<int, 1>{});
@@ -515,7 +541,8 @@ extern "C" long mi_paged_attention_workspace(int T, int Hq, int dh, int max_seq_
 
 // LDS of a workgroup of the tiled kernel: the tile's queries, 64 keys, their values, a wave's probabilities
 static size_t paged_attention_tile_lds(int dh) {
-  return ((size_t)PT_QUERIES * dh + (size_t)WAVE * (dh + PT_PAD) + (size_t)dh * (WAVE + PT_PAD) + PA_RUN) * sizeof(float);
+  return ((size_t)PT_QUERIES * dh + (size_t)WAVE * (dh + PT_PAD) + (size_t)dh * (WAVE + PT_PAD) +
+          (size_t)PT_QUERIES * (WAVE + PT_PAD)) * sizeof(float);
 }
 
 template <typename T, bool FAST_EXP, int DIMS>
