@@ -404,7 +404,8 @@ def test_attention_refuses_a_head_size_beyond_its_limit(ops):
 # ------------------------------------------------------------------ mamba2
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H, P, N, G, K", [(8, 8, 16, 1, 4), (6, 16, 32, 2, 3), (3, 24, 40, 3, 2), (4, 64, 128, 1, 4),
-                                             (2, 40, 256, 2, 4), (5, 7, 9, 1, 1)])
+                                             (2, 40, 256, 2, 4), (5, 7, 9, 1, 1), (1, 8, 512, 1, 4), (2, 16, 64, 1, 4),
+                                             (3, 5, 4, 1, 2), (2, 3, 1, 1, 2), (2, 6, 72, 2, 4)])
 def test_mamba2_kernels_over_ragged_lanes(ops, dtype, H, P, N, G, K):
     """Lanes of 1, 2 (shorter than the conv tail), 19 and 45 tokens with non-zero conv tails
     and states in shuffled slots; the slot no lane uses must stay as it was."""
