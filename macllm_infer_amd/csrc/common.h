@@ -48,6 +48,9 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 }
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+// the same with the hardware's exponential and reciprocal (a few float32 ulps): for results that are rounded to
+// bfloat16 at once
+__device__ __forceinline__ float silu_bf16_f(float x) { return x * __frcp_rn(1.0f + __expf(-x)); }
 
 // max(x,0) + log1p(exp(-|x|)): finite for any finite x.
 __device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }

@@ -300,7 +300,7 @@ swiglu_vec_kernel(const bf16_t* __restrict__ gu, long ld, bf16_t* __restrict__ o
   const common_bf16x8 up = *reinterpret_cast<const common_bf16x8*>(gu + t * ld + at + (tile == 0 ? I : 8));
   common_bf16x8 result;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) result[j] = (bf16_t)(silu_f((float)gate[j]) * (float)up[j]);
+  for (int j = 0; j < 8; ++j) result[j] = (bf16_t)(silu_bf16_f((float)gate[j]) * (float)up[j]);
   *reinterpret_cast<common_bf16x8*>(out + index) = result;
 }
 

@@ -175,7 +175,7 @@ __device__ void ssd_conv_block(const bf16_t* __restrict__ u, long u_ld, int C, c
       s_bf16x8 result;
       const bool live = real && position < length;
 #pragma unroll
-      for (int cc = 0; cc < 8; ++cc) result[cc] = live ? (bf16_t)silu_f(sum[cc]) : (bf16_t)0.f;
+      for (int cc = 0; cc < 8; ++cc) result[cc] = live ? (bf16_t)silu_bf16_f(sum[cc]) : (bf16_t)0.f;
       if (live) *reinterpret_cast<s_bf16x8*>(xbc + (long)(t0 + position) * xbc_ld + channel) = result;
 #pragma unroll
       for (int cc = 0; cc < 8; ++cc) tile[(c + cc) * stride + position] = result[cc];
@@ -513,7 +513,7 @@ ssd_chunk_scan_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf16_t*
         if (z != nullptr) {
           s_bf16x4 packed;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(out[i] * silu_f((float)gate[hb][pi][i]));
+          for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(out[i] * silu_bf16_f((float)gate[hb][pi][i]));
           *reinterpret_cast<s_bf16x4*>(gated + t_row * gated_ld + column) = packed;
         } else {
           *reinterpret_cast<s_floatx4*>(y + t_row * y_ld + column) = out;
@@ -709,7 +709,7 @@ ssd_chunk_scan_lds_kernel(const bf16_t* __restrict__ xbc, long xbc_ld, const bf1
     if (z != nullptr) {
       s_bf16x4 packed;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(out[i] * silu_f((float)gate[pi][i]));
+      for (int i = 0; i < 4; ++i) packed[i] = (bf16_t)(out[i] * silu_bf16_f((float)gate[pi][i]));
       *reinterpret_cast<s_bf16x4*>(gated + t_row * gated_ld + column) = packed;
     } else {
       *reinterpret_cast<s_floatx4*>(y + t_row * y_ld + column) = out;
