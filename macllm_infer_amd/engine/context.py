@@ -5,7 +5,8 @@ starting at that request's current length: a portion of a prompt or one decoded
 token.  Lanes are packed without padding in submission order
 (reference: src/decoder.rs:4248-4260, lane struct paged_decode.metal:51-58).
 All index arrays are written by the host-side core (``csrc/hostcore.cpp``) into one buffer and
-uploaded in one copy.
+uploaded in one copy; tables that a mixer declares for itself (``StepTable``) are written behind them
+by the mixer's own function and travel in the same copy.
 
 ``StaticStep`` keeps the arrays of a batch of single-token lanes at fixed addresses and
 fixed shapes, so that a captured HIP graph can be replayed on them; lanes beyond the
