@@ -9,7 +9,6 @@
 // [slot, H, P, N] in float32 (reference: src/decoder.rs:2269-2294).  A fresh request's slot
 // holds zeros.
 #include "common.h"
-#include <cstdlib>
 
 #define CONV_MAX_K 16
 
