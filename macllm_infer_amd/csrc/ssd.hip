@@ -331,16 +331,17 @@ __global__ void ssd_state_pass_kernel(const float* __restrict__ chunk_state, con
   const int count = lane_chunks[2 * lane + 1];
   float* slot = ssm_state + ((long)slot_ids[lane] * H + head) * per_head + element;
   float running = *slot;
-  for (int c0 = first; c0 < first + count; c0 += 8) {       // eight chunks' loads at a time, then the recurrence
-    float added[8], decay[8];
+  constexpr int AT_ONCE = 16;                               // chunks whose loads are asked for at once, then the recurrence
+  for (int c0 = first; c0 < first + count; c0 += AT_ONCE) { // (a portion of 2,048 tokens in chunks of 128: one round)
+    float added[AT_ONCE], decay[AT_ONCE];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < AT_ONCE; ++j) {
       const int c = min(c0 + j, first + count - 1);
       added[j] = chunk_state[((long)c * H + head) * per_head + element];
       decay[j] = chunk_decay[(long)c * H + head];
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < AT_ONCE; ++j) {
       if (c0 + j < first + count) {
         state_in[((long)(c0 + j) * H + head) * per_head + element] = (bf16_t)running;
         running = decay[j] * running + added[j];
