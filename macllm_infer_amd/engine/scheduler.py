@@ -152,6 +152,9 @@ class Scheduler:
                 self._reject(request, "prompt must contain at least one token")
             elif any(not (0 <= token < self.engine.vocab_size) for token in request.prompt):
                 self._reject(request, "input contains a token ID outside the model vocabulary")
+            elif (isinstance(request.params.allowed_token_ids, tuple)
+                  and max(request.params.allowed_token_ids) >= self.engine.vocab_size):
+                self._reject(request, "allowed_token_ids names a token ID outside the model vocabulary")
             elif needed > self.engine.max_context:
                 self._reject(request, "prompt plus requested output exceeds model context limit")
             elif not self.engine.cache.can_ever_fit(needed):
@@ -290,9 +293,12 @@ class Scheduler:
                 rows, kept = [], []
                 for row, (request, _) in enumerate(sampled):
                     try:
-                        rows.append(SamplerRow(request.params, request.prompt, request.generated,
-                                               None if request.in_flight is None
-                                               else (request.in_flight[0].device, request.in_flight[1])))
+                        made = SamplerRow(request.params, request.prompt, request.generated,
+                                          None if request.in_flight is None
+                                          else (request.in_flight[0].device, request.in_flight[1]))
+                        if made.allowed is not None and max(made.allowed) >= self.engine.vocab_size:
+                            raise ValueError("the constraint names a token ID outside the model vocabulary")
+                        rows.append(made)
                         kept.append(row)
                     except ValueError as error:          # its constraint allows no token: the request fails alone
                         self._finish(request, f"failed: {error}")

@@ -362,6 +362,23 @@ def test_a_constraint_that_follows_the_generated_tokens_is_asked_with_all_of_the
     assert lanes_of_0 == [[1, 2, 3], [20], [22], [24], [26]]
 
 
+def test_a_constraint_beyond_the_vocabulary_ends_its_request_alone():
+    """A fixed list that names a token the model does not have is refused at admission; a list that comes to name one
+    later ends its request there; the request beside them runs to its length."""
+    engine = AheadEngine()
+    scheduler = Scheduler(engine, ConstrainedSampler(), EngineConfig(), ())
+    common = dict(max_new_tokens=4, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0)
+    scheduler.submit(0, [1, 2], SamplingParams(allowed_token_ids=(3, 50), **common))                  # the vocabulary is 0 .. 49
+    scheduler.submit(1, [4, 5], SamplingParams(allowed_token_ids=lambda generated: [7] if len(generated) < 2 else [77], **common))
+    scheduler.submit(2, [9], SamplingParams(**common))
+    finished = scheduler.run()
+    assert finished[0].finish_reason.startswith("rejected") and "allowed_token_ids" in finished[0].finish_reason
+    assert finished[0].generated == []
+    assert finished[1].generated == [7, 7] and "outside the model vocabulary" in finished[1].finish_reason
+    assert finished[2].generated == [10, 11, 12, 13] and finished[2].finish_reason == "length"
+    assert not engine.lengths
+
+
 def test_allowed_token_ids_are_checked_where_they_are_given():
     with pytest.raises(ValueError, match="at least one token"):
         SamplingParams(allowed_token_ids=())
