@@ -300,7 +300,7 @@ class Scheduler:
                             raise ValueError("the constraint names a token ID outside the model vocabulary")
                         rows.append(made)
                         kept.append(row)
-                    except ValueError as error:          # its constraint allows no token: the request fails alone
+                    except Exception as error:           # its constraint allows no token, or fails itself: the request fails alone
                         self._finish(request, f"failed: {error}")
                 if len(kept) < len(sampled):
                     sampled = [sampled[row] for row in kept]
