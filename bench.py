@@ -13,7 +13,9 @@ comes for the first time); ``roofline`` = the bytes the decode step has to read 
 uses once, and the cache and state of the live requests; ``bytes`` gives them and what the step
 writes) over its time, against 8 TB/s; ``points`` = decode at batch 1 and 64, and at longer contexts (batch 8
 at 8,192 and 32,768 tokens, batch 64 at 8,192, from an engine of the same layers that allows such contexts;
-``points_frac`` = their fractions of 8 TB/s on the bytes they have to read); ``step_ms`` = mean,
+``points_frac`` = their fractions of 8 TB/s on the bytes they have to read); ``prefill_f32`` = the same prompt
+step through the true 32-bit path (the headline shape only), against the float32 matrix cores' peak;
+``step_ms`` = mean,
 median and 95th percentile of the timed steps (the reference reports the same three:
 src/benchmark/stats.rs:10-16); ``choices`` = what the build-time measurements chose for each
 projection of a layer at up to 16 / 32 / 64 rows (L = library, S = skinny kernel, a digit = slabs
@@ -226,7 +228,7 @@ def main() -> int:
         torch.cuda.synchronize()
 
     # ---------------------------------------------------------------- prefill: one 2,048-token prompt
-    def prefill_step():
+    def prefill_step(engine=engine):
         prompt = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=generator).tolist()
         engine.add_request("prefill")
         synchronize()
@@ -313,6 +315,19 @@ def main() -> int:
             long_points[(batch, context)] = decode_point(long_engine, long_sampler, batch, context)
     else:
         choices = choices_of(engine)
+    # the same prefill through the true 32-bit path (the small shape only: the weights once more in float32)
+    prefill_f32 = None
+    if args.dtype == "bf16" and args.shape == "0.5b" and not (args.skip_points or args.skip_long_points or args.prefill_only):
+        wide = {name: tensor.to(torch.float32) for name, tensor in tensors.items()}
+        wide_engine = Engine(config=config, tensors=wide, dtype="float32", kv_cache_block_tokens=args.page_tokens,
+                             kv_cache_capacity_tokens=PREFILL_TOKENS + 64, max_active_sequences=1)
+        del wide
+        times = [prefill_step(wide_engine) for _ in range(6)]
+        seconds = sorted(times[3:])[1]
+        flops = total(prefill_costs(wide_engine.spec, PREFILL_TOKENS, 4)).flops
+        prefill_f32 = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS, "ms": round(seconds * 1e3, 3),
+                       "frac": round(flops / seconds / PEAK_FLOPS["f32"], 5)}
+        del wide_engine
     del tensors
 
     if args.prefill_only:
@@ -354,6 +369,8 @@ def main() -> int:
         "prefill_uncaptured_ms": round(uncaptured_seconds * 1e3, 3),
         "choices": choices,
     }
+    if prefill_f32 is not None:
+        record["prefill_f32"] = prefill_f32
     print(json.dumps(record))
     return 0
 

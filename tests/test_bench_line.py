@@ -77,6 +77,10 @@ def test_line_of_a_short_run():
     # tokens to the next's, and the last step's work ends after the last of these times: 1 part in 20 here
     assert 0.85 * record["ms_per_step"] <= times["mean"] <= 1.02 * record["ms_per_step"]
     assert record["prefill_uncaptured_ms"] >= 0.9 * prefill["ms"]
+    # the same prompt through the true 32-bit path: slower than bfloat16, against the float32 peak
+    wide = record["prefill_f32"]
+    assert set(wide) == {"value", "tokens", "ms", "frac"} and wide["tokens"] == bench.PREFILL_TOKENS
+    assert wide["ms"] > prefill["ms"] and 0.0 < wide["frac"] < 1.0
     assert {"in", "out", "gate_up", "down"} <= set(record["choices"])
     long_points = {f"decode_b{batch}_ctx{context}" for batch, context in bench.LONG_POINTS}
     assert set(record["points"]) == {"decode_b1", "decode_b64"} | long_points == set(record["points_frac"])
