@@ -1328,7 +1328,8 @@ RANDOM_CASES = ([(seed, False) for seed in range(8)] + [(seed, True) for seed in
                 + [(seed, False) for seed in (3022, 3024, 3038, 3040, 3041)]
                 + [(seed, True) for seed in (12, 22, 23, 28, 34, 57)]
                 + [(seed, False) for seed in (7019, 7027, 7039, 7047, 7054)]
-                + [(seed, True) for seed in (8002, 8009, 8011)])
+                + [(seed, True) for seed in (8002, 8009, 8011)]
+                + [(9109, False), (9305, True)])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
