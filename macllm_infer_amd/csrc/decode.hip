@@ -92,13 +92,48 @@ struct FusedGemmParams {
   const float* ssq_in;
   int ssq_blocks, ssq_width;
   float ssq_eps;
+  // both tables of partial sums of squares have rows of ssq_ld floats: one per row of the step, to a multiple of 16
+  int ssq_ld;
+  // the step's rows dealt out to row_tiles workgroups per tile of features (1: every workgroup takes them all)
+  int row_tiles;
 };
+
+// What is left of a step for a workgroup that takes `rows` of its rows from row0 on (plain prologue).
+__device__ __forceinline__ void take_rows(FusedGemmParams& p, int row0, int rows) {
+  if (p.x) p.x += (long)row0 * p.x_ld;
+  if (p.out) p.out = p.out_f32 ? (void*)(reinterpret_cast<float*>(p.out) + (long)row0 * p.out_ld)
+                               : (void*)(reinterpret_cast<bf16_t*>(p.out) + (long)row0 * p.out_ld);
+  if (p.slot_ids) p.slot_ids += row0;
+  if (p.res_h) {
+    p.res_h += (long)row0 * p.N;
+    p.res_hb += (long)row0 * p.res_hb_ld;
+    p.ssq_out += row0;
+  }
+  if (p.ssq_in) p.ssq_in += row0;
+  p.M = min(rows, p.M - row0);
+}
 
 __device__ __forceinline__ float round_bf16(float v) { return (float)(bf16_t)v; }
 
-template <int MT, int PRO, int EPI, int FG_WAVES, int NT>
-__global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmParams p) {
+template <int MT, int PRO, int EPI, int FG_WAVES, int NT, bool ROW_TILES = false>
+__global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmParams whole_step) {
   static_assert(NT == 1 || PRO == PRO_PLAIN, "several feature tiles a workgroup: plain prologue only");
+  // Row tiles: a workgroup takes MT tiles of 16 rows of the step and row_tiles workgroups share a tile of
+  // features.  Workgroups go to the eight dies in turn and each die has a cache of its own, so those that share
+  // weights are given numbers that are 8 apart and follow each other: the weights leave memory once.
+  FusedGemmParams p = whole_step;
+  const int slab_rows = p.M;
+  int block_x = blockIdx.x;
+  int ssq_rows = p.ssq_ld;              // rows of the tables of partial sums of squares from this workgroup's first row on
+  if (ROW_TILES) {
+    static_assert(!ROW_TILES || (PRO == PRO_PLAIN && NT == 1), "rows dealt out: plain prologue, one tile of features");
+    const int die = block_x % 8, turn = block_x / 8;
+    block_x = (turn / p.row_tiles) * 8 + die;
+    if (block_x * 16 * NT >= p.N) return;
+    const int row0 = (turn % p.row_tiles) * MT * 16;
+    ssq_rows -= row0;
+    take_rows(p, row0, MT * 16);
+  }
   static_assert(PRO != PRO_MERGE || EPI == EPI_PLAIN || EPI == EPI_RESIDUAL, "the merge prologue comes with the plain or the residual epilogue");
   static_assert(EPI != EPI_RESIDUAL || (NT == 1 && PRO != PRO_NORM), "the residual epilogue: one tile of features, rows given as they are");
   constexpr int FG_THREADS = FG_WAVES * WAVE;
@@ -115,7 +150,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
 
-  const int n0 = blockIdx.x * 16 * NT;
+  const int n0 = block_x * 16 * NT;
   const int q = lane / 16;
   const int r = lane % 16;
   // W is row-major [N, K], or (w_tiled) in the order of the matrix-core fragments: [N / 16, K / 32, 64 lanes, 8],
@@ -124,7 +159,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   const long w_step = p.w_tiled ? 512 : 32;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
-    w_row[nt] = p.w_tiled ? p.W + (long)min((int)blockIdx.x * NT + nt, (p.N + 15) / 16 - 1) * (K / 32) * 512 + lane * 8
+    w_row[nt] = p.w_tiled ? p.W + (long)min(block_x * NT + nt, (p.N + 15) / 16 - 1) * (K / 32) * 512 + lane * 8
                           : p.W + (long)min(n0 + 16 * nt + r, p.N - 1) * K + 8 * q;
   // wave w takes a contiguous run of k-chunks (of 32), so that its loads cover whole cache lines
   // (a grid with several rows splits K among them: row y takes a run of chunks and writes its partial
@@ -165,10 +200,10 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
   float ssq_early[SSQ_EARLY] = {};
   if (p.ssq_in) {
     const int last = p.ssq_blocks - 1;
-    const int row = tid % (16 * MT);
+    const int row = min(tid % (16 * MT), ssq_rows - 1);
 #pragma unroll
     for (int i = 0; i < SSQ_EARLY; ++i)
-      ssq_early[i] = p.ssq_in[(long)min(tid / (16 * MT) + i * PARTS, last) * (16 * MT) + row];
+      ssq_early[i] = p.ssq_in[(long)min(tid / (16 * MT) + i * PARTS, last) * p.ssq_ld + row];
   }
   float res_old[EPT] = {};
   float res_weight = 0.f;
@@ -300,7 +335,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
           sum_squares = wave_sum(sum_squares);
           const float inverse = 1.0f / sqrtf(sum_squares / (float)K + p.eps);
           auto finish = [&](int k, const floatx4& value, const floatx4& w) {
-            if (blockIdx.x == 0 && p.h_out) *reinterpret_cast<floatx4*>(p.h_out + (long)m * K + k) = value;
+            if (block_x == 0 && p.h_out) *reinterpret_cast<floatx4*>(p.h_out + (long)m * K + k) = value;
             bf16x4_t packed;
 #pragma unroll
             for (int j = 0; j < 4; ++j) packed[j] = (bf16_t)(value[j] * inverse * w[j]);
@@ -440,7 +475,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 #pragma unroll
     for (int i = 0; i < SSQ_EARLY; ++i) sum += part + i * PARTS < p.ssq_blocks ? ssq_early[i] : 0.f;
     // rows wider than SSQ_EARLY sums a thread: the rest now
-    for (int b = part + SSQ_EARLY * PARTS; b < p.ssq_blocks; b += PARTS) sum += p.ssq_in[(long)b * (16 * MT) + tid % (16 * MT)];
+    for (int b = part + SSQ_EARLY * PARTS; b < p.ssq_blocks; b += PARTS) sum += p.ssq_in[(long)b * p.ssq_ld + min(tid % (16 * MT), ssq_rows - 1)];
     ssq_parts[tid] = sum;
   }
   // the waves' partial tiles are summed through LDS and finished, one tile of 16 features after the other
@@ -522,18 +557,18 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
         if (taps > 1) tail[(long)(taps - 2) * channels] = sample;
         reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + n] = (bf16_t)silu_f(sum);
       } else if (p.out_f32) {
-        reinterpret_cast<float*>(p.out)[((long)blockIdx.y * p.M + m) * p.out_ld + n] = v * p.out_scale;
+        reinterpret_cast<float*>(p.out)[((long)blockIdx.y * slab_rows + m) * p.out_ld + n] = v * p.out_scale;
       } else {
         reinterpret_cast<bf16_t*>(p.out)[(long)m * p.out_ld + n] = (bf16_t)(v * p.out_scale);
       }
     }
     if (EPI == EPI_RESIDUAL) {
       __syncthreads();
-      if (tid < MT * 16) {
+      if (tid < min(MT * 16, ssq_rows)) {
         float squares = 0.f;
 #pragma unroll
         for (int f = 0; f < 16; ++f) squares += tile[f * (MT * 16) + tid];
-        p.ssq_out[(long)blockIdx.x * (MT * 16) + tid] = squares;
+        p.ssq_out[(long)block_x * p.ssq_ld + tid] = squares;
       }
     }
     if (EPI == EPI_SWIGLU) {
@@ -542,7 +577,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
       for (int index = tid; index < 8 * MT * 16; index += FG_THREADS) {
         const int i = index / (MT * 16);
         const int m = index % (MT * 16);
-        const int column = (blockIdx.x * NT + nt) * 8 + i;
+        const int column = (block_x * NT + nt) * 8 + i;
         if (m >= p.M || column >= half_rows) continue;
         const float gate = round_bf16(tile[i * (MT * 16) + m]);
         const float up = round_bf16(tile[(8 + i) * (MT * 16) + m]);
@@ -586,13 +621,32 @@ static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStre
 #undef FG_WIDE
     return 0;
   }
-  const dim3 blocks((p.N + 15) / 16, k_splits);
+  const int feature_blocks = (p.N + 15) / 16;
+  const dim3 blocks(p.row_tiles > 1 ? (feature_blocks + 7) / 8 * 8 * p.row_tiles : feature_blocks, k_splits);
   const int waves = fused_gemm_waves(p.K / k_splits);
 #define FG_LAUNCH(PRO_, EPI_)                                                                      \
   do {                                                                                             \
     if (waves == 8) fused_gemm_kernel<MT, PRO_, EPI_, 8, 1><<<blocks, 8 * WAVE, lds, stream>>>(p); \
     else fused_gemm_kernel<MT, PRO_, EPI_, 4, 1><<<blocks, 4 * WAVE, lds, stream>>>(p);            \
   } while (0)
+#define FG_LAUNCH_ROWS(EPI_)                                                                                  \
+  do {                                                                                                        \
+    if (waves == 8) fused_gemm_kernel<MT, PRO_PLAIN, EPI_, 8, 1, true><<<blocks, 8 * WAVE, lds, stream>>>(p); \
+    else fused_gemm_kernel<MT, PRO_PLAIN, EPI_, 4, 1, true><<<blocks, 4 * WAVE, lds, stream>>>(p);            \
+  } while (0)
+  if (p.row_tiles > 1) {           // MT of 1 or 2: the tiles of a step of up to 64 rows over two workgroups or more
+    if (pro != PRO_PLAIN) return ERR_BAD_ARGUMENT;
+    if constexpr (MT <= 2) {
+      if (epi == EPI_RESIDUAL) FG_LAUNCH_ROWS(EPI_RESIDUAL);
+      else if (epi == EPI_PLAIN) FG_LAUNCH_ROWS(EPI_PLAIN);
+      else if (epi == EPI_SWIGLU) FG_LAUNCH_ROWS(EPI_SWIGLU);
+      else if (epi == EPI_CONV) FG_LAUNCH_ROWS(EPI_CONV);
+      else return ERR_BAD_ARGUMENT;
+      return 0;
+    } else {
+      return ERR_BAD_ARGUMENT;
+    }
+  }
   if (pro == PRO_MERGE && epi == EPI_PLAIN) FG_LAUNCH(PRO_MERGE, EPI_PLAIN);
   else if (pro == PRO_MERGE && epi == EPI_RESIDUAL) FG_LAUNCH(PRO_MERGE, EPI_RESIDUAL);
   else if (pro == PRO_PLAIN && epi == EPI_RESIDUAL) FG_LAUNCH(PRO_PLAIN, EPI_RESIDUAL);
@@ -604,7 +658,30 @@ static int launch_fused_gemm(const FusedGemmParams& p, int pro, int epi, hipStre
   else if (pro == PRO_PLAIN && epi == EPI_CONV) FG_LAUNCH(PRO_PLAIN, EPI_CONV);
   else return ERR_BAD_ARGUMENT;
 #undef FG_LAUNCH
+#undef FG_LAUNCH_ROWS
   return 0;
+}
+
+// The same for a step of p.M rows (up to 64).  row_tiles > 1 (plain prologue, one tile of features a workgroup): the
+// tiles of 16 rows are dealt out to that many workgroups per tile of features (64 rows over 4: every workgroup
+// multiplies 16 rows), which fills the GPU where a projection has few output features without slabs over K, and
+// moves a quarter of the rows through each compute unit; the weights cross the caches row_tiles times.
+static int launch_fused_gemm_rows(FusedGemmParams& p, int pro, int epi, hipStream_t stream, int k_splits = 1,
+                                  int feature_tiles = 1, int row_tiles = 1) {
+  const int step_tiles = (p.M + 15) / 16;
+  int MT = step_tiles;
+  p.ssq_ld = 16 * step_tiles;
+  p.row_tiles = 1;
+  if (row_tiles > 1) {
+    if (pro != PRO_PLAIN || feature_tiles != 1) return ERR_BAD_ARGUMENT;
+    MT = (step_tiles + row_tiles - 1) / row_tiles;
+    p.row_tiles = (step_tiles + MT - 1) / MT;
+  }
+  if (MT == 1) return launch_fused_gemm<1>(p, pro, epi, stream, k_splits, feature_tiles);
+  if (MT == 2) return launch_fused_gemm<2>(p, pro, epi, stream, k_splits, feature_tiles);
+  if (MT == 3) return launch_fused_gemm<3>(p, pro, epi, stream, k_splits, feature_tiles);
+  if (MT == 4) return launch_fused_gemm<4>(p, pro, epi, stream, k_splits, feature_tiles);
+  return ERR_UNSUPPORTED_SIZE;
 }
 
 // The product in float32 slabs over K for steps of many rows, with the rows shared.  In fused_gemm_kernel every
@@ -895,11 +972,13 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
                              int out_f32, float out_scale, int conv_lo, int conv_hi, int conv_k,
                              const float* conv_w, const float* conv_b, void* conv_state, const int* slot_ids,
                              int feature_tiles, int w_fragments, const float* ssq_in, int ssq_blocks, int ssq_width,
-                             float ssq_eps, hipStream_t stream) {
+                             float ssq_eps, int row_tiles, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !out) return ERR_BAD_ARGUMENT;
   if (ssq_in && (pro != PRO_PLAIN || ssq_blocks <= 0 || ssq_width <= 0)) return ERR_BAD_ARGUMENT;
   const bool shared_rows = feature_tiles < 0;       // -1, -2: that many tiles a wave of shared_rows_gemm_kernel
   if (shared_rows && (feature_tiles < -2 || pro != PRO_PLAIN || out_f32)) return ERR_BAD_ARGUMENT;
+  if (row_tiles < 1 || row_tiles > 4 || (row_tiles > 1 && (shared_rows || pro != PRO_PLAIN || feature_tiles != 1)))
+    return ERR_BAD_ARGUMENT;
   if (!shared_rows && feature_tiles != 1 && feature_tiles != 2 && feature_tiles != 4) return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0) return ERR_UNSUPPORTED_SIZE;
   if (shared_rows && K / 32 < SR_CHUNKS) return ERR_UNSUPPORTED_SIZE;
@@ -950,10 +1029,7 @@ extern "C" int mi_fused_gemm(int pro, int epi, const float* h_in, const void* de
     }
     code = launch_shared_rows_for<EPI_CONV>(M, p, stream, 1, -feature_tiles);
   } else if (shared_rows) code = launch_shared_rows_for<EPI_SWIGLU>(M, p, stream, 1, -feature_tiles);
-  else if (MT == 1) code = launch_fused_gemm<1>(p, pro, epi, stream, 1, feature_tiles);
-  else if (MT == 2) code = launch_fused_gemm<2>(p, pro, epi, stream, 1, feature_tiles);
-  else if (MT == 3) code = launch_fused_gemm<3>(p, pro, epi, stream, 1, feature_tiles);
-  else code = launch_fused_gemm<4>(p, pro, epi, stream, 1, feature_tiles);
+  else code = launch_fused_gemm_rows(p, pro, epi, stream, 1, feature_tiles, row_tiles);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;
@@ -984,11 +1060,7 @@ extern "C" int mi_fused_gemm_split(const void* x, long x_ld, const void* W, cons
   p.out_f32 = 1;
   p.out_scale = 1.0f;
   p.w_tiled = w_fragments ? 1 : 0;
-  int code;
-  if (MT == 1) code = launch_fused_gemm<1>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
-  else if (MT == 2) code = launch_fused_gemm<2>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
-  else if (MT == 3) code = launch_fused_gemm<3>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
-  else code = launch_fused_gemm<4>(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
+  const int code = launch_fused_gemm_rows(p, PRO_PLAIN, EPI_PLAIN, stream, splits, feature_tiles);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;
@@ -1067,7 +1139,7 @@ extern "C" int mi_fused_gemm_merge(const float* partial, const int* positions, i
   p.res_hb_ld = res_hb_ld;
   p.res_w = res_w;
   p.ssq_out = ssq_out;
-  const int code = launch_fused_gemm<1>(p, PRO_MERGE, res_h ? EPI_RESIDUAL : EPI_PLAIN, stream);
+  const int code = launch_fused_gemm_rows(p, PRO_MERGE, res_h ? EPI_RESIDUAL : EPI_PLAIN, stream);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;
@@ -1079,11 +1151,12 @@ extern "C" int mi_fused_gemm_merge(const float* partial, const int* positions, i
 // new row over each workgroup's 16 features (mi_fused_gemm takes them as its row scale).  M <= 64.
 extern "C" int mi_fused_gemm_residual(const void* x, long x_ld, const void* W, const float* bias, int M, int N, int K,
                                       float* res_h, void* res_hb, long res_hb_ld, const float* res_w, float* ssq_out,
-                                      int w_fragments, hipStream_t stream) {
+                                      int w_fragments, int row_tiles, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || !W || !x || x_ld < K || x_ld % 8 != 0 || !res_h || !res_hb || !res_w || !ssq_out ||
       res_hb_ld < N)
     return ERR_BAD_ARGUMENT;
   if (M > 64 || K % 32 != 0) return ERR_UNSUPPORTED_SIZE;
+  if (row_tiles < 1 || row_tiles > 4) return ERR_BAD_ARGUMENT;
   const int MT = (M + 15) / 16;
   if (fused_gemm_lds(MT, PRO_PLAIN, K, M) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   FusedGemmParams p = {};
@@ -1101,11 +1174,7 @@ extern "C" int mi_fused_gemm_residual(const void* x, long x_ld, const void* W, c
   p.res_hb_ld = res_hb_ld;
   p.res_w = res_w;
   p.ssq_out = ssq_out;
-  int code;
-  if (MT == 1) code = launch_fused_gemm<1>(p, PRO_PLAIN, EPI_RESIDUAL, stream);
-  else if (MT == 2) code = launch_fused_gemm<2>(p, PRO_PLAIN, EPI_RESIDUAL, stream);
-  else if (MT == 3) code = launch_fused_gemm<3>(p, PRO_PLAIN, EPI_RESIDUAL, stream);
-  else code = launch_fused_gemm<4>(p, PRO_PLAIN, EPI_RESIDUAL, stream);
+  const int code = launch_fused_gemm_rows(p, PRO_PLAIN, EPI_RESIDUAL, stream, 1, 1, row_tiles);
   if (code != 0) return code;
   RETURN_IF_LAUNCH_FAILED();
   return 0;

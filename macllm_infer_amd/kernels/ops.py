@@ -79,9 +79,10 @@ _SIGNATURES = {
     "decode": {
         "mi_fused_gemm": [_c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_long, _c_ptr,
                           _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_long, _c_int, _c_float, _c_int, _c_int, _c_int,
-                          _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_float, _c_ptr],
+                          _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_float, _c_int,
+                          _c_ptr],
         "mi_fused_gemm_residual": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
-                                   _c_ptr, _c_ptr, _c_int, _c_ptr],
+                                   _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
         "mi_fused_gemm_supported": [_c_int, _c_int, _c_int],
         "mi_fused_gemm_split": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int,
                                 _c_ptr],
@@ -824,7 +825,7 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
                deltas: Sequence[torch.Tensor] = (), h_out: Optional[torch.Tensor] = None,
                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, epilogue: int = EPI_PLAIN,
                conv: Optional[dict] = None, feature_tiles: int = 1, fragments: Optional[torch.Tensor] = None,
-               row_scale: Optional["RowScale"] = None, shared_rows: bool = False) -> None:
+               row_scale: Optional["RowScale"] = None, shared_rows: bool = False, row_tiles: int = 1) -> None:
     """out[M, N'] = epilogue(prologue . weight[N, K]^T + bias) for a small batch in bfloat16.
 
     Prologue: ``x`` [M, K] bfloat16, or ``h_in`` float32 [M, K] with up to two bfloat16 ``deltas``:
@@ -840,10 +841,14 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
     square yet; the sums of row m are multiplied by 1 / sqrt(sum of squares of the row / width + eps) before the
     bias, from the partial sums of squares that ``fused_gemm_residual`` left.  ``shared_rows`` (``x``, K >= 128,
     bfloat16 ``out``, 1 or 2 feature tiles a wave): the kernel whose four waves own feature tiles
-    and share the step's rows through LDS instead of fetching them each."""
+    and share the step's rows through LDS instead of fetching them each.  ``row_tiles`` (1 to 4; more than one
+    with ``x``, one feature tile, not ``shared_rows``): the step's tiles of 16 rows are dealt out to that many
+    workgroups per tile of features, each of which fetches its own rows only."""
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm: weight must be contiguous bfloat16 [N, K]")
     _need(row_scale is None or x is not None, "fused_gemm: a row scale needs x")
+    _need(1 <= row_tiles <= 4 and (row_tiles == 1 or (x is not None and feature_tiles == 1 and not shared_rows)),
+          "fused_gemm: row_tiles is 1 to 4, and more than 1 needs x, one feature tile and the skinny kernel")
     if row_scale is not None:
         _need(row_scale.ssq.dtype == torch.float32 and row_scale.ssq.is_contiguous() and row_scale.ssq.dim() == 2
               and row_scale.ssq.shape[1] == 16 * (-(-out.shape[0] // 16)), "fused_gemm: the partial sums of squares do not fit the step")
@@ -894,7 +899,7 @@ def fused_gemm(weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Te
         _p(slot_ids), -int(feature_tiles) if shared_rows else int(feature_tiles), int(fragments is not None),
         _p(row_scale.ssq) if row_scale is not None else None, row_scale.ssq.shape[0] if row_scale is not None else 0,
         int(row_scale.width) if row_scale is not None else 0, float(row_scale.eps) if row_scale is not None else 0.0,
-        _stream()), "fused_gemm", f"(M={M}, N={N}, K={K})")
+        int(row_tiles), _stream()), "fused_gemm", f"(M={M}, N={N}, K={K})")
 
 
 @dataclass(frozen=True)
@@ -923,11 +928,14 @@ def _residual_arguments(h, hb, next_weight, ssq, M, N, name):
 
 def fused_gemm_residual(weight: torch.Tensor, bias: Optional[torch.Tensor], x: torch.Tensor, h: torch.Tensor,
                         hb: torch.Tensor, next_weight: torch.Tensor, ssq: torch.Tensor,
-                        fragments: Optional[torch.Tensor] = None) -> None:
+                        fragments: Optional[torch.Tensor] = None, row_tiles: int = 1) -> None:
     """h += x [M, K] . weight[N, K]^T (+ bias), float32 in place: a projection whose result joins the residual
     stream.  Beside it ``hb`` = bfloat16(h * next_weight), the new rows times the next norm's weight, and ``ssq``
     (``residual_workspace``), the sums of squares of the new rows over every 16 features: what ``fused_gemm`` with
-    ``row_scale`` needs to be the product behind that norm, without a pass for the norm."""
+    ``row_scale`` needs to be the product behind that norm, without a pass for the norm.  ``row_tiles`` (1 to 4):
+    the step's tiles of 16 rows dealt out to that many workgroups per tile of features (a projection into the
+    stream has few features: 64 workgroups for 1,024 of them, 256 with the 64 rows of a step over four)."""
+    _need(1 <= row_tiles <= 4, "fused_gemm_residual: row_tiles is 1 to 4")
     _need(weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.is_contiguous() and weight.is_cuda,
           "fused_gemm_residual: weight must be contiguous bfloat16 [N, K]")
     N, K = weight.shape
@@ -939,7 +947,7 @@ def fused_gemm_residual(weight: torch.Tensor, bias: Optional[torch.Tensor], x: t
     hb_ld = _residual_arguments(h, hb, next_weight, ssq, M, N, "fused_gemm_residual")
     _check(_fn("decode", "mi_fused_gemm_residual")(
         _p(x), x_ld, _p(_weight_operand(weight, fragments, "fused_gemm_residual")), _p(bias), M, N, K, _p(h), _p(hb),
-        hb_ld, _p(next_weight), _p(ssq), int(fragments is not None), _stream()), "fused_gemm_residual",
+        hb_ld, _p(next_weight), _p(ssq), int(fragments is not None), int(row_tiles), _stream()), "fused_gemm_residual",
         f"(M={M}, N={N}, K={K})")
 
 

@@ -135,8 +135,20 @@ FORCE_DEFERRED_NORM: Optional[bool] = None  # tests: False = never
 # own choices stay.)
 CHAIN_LAYERS = 8
 CHAIN_MARGIN = 0.97
+# Where the norms are left to the projections, a step of more than 16 rows can have its tiles of 16 rows dealt out
+# to several workgroups per tile of features instead of every workgroup taking them all.  The two projections that
+# feed the stream have few output features (1,024 of them: 64 workgroups, each of which fetches all of the step's
+# rows): with 64 rows over four workgroups 1,024 x 2,048 takes 5.9 us instead of 11.4, at 32 rows 5.7 instead of
+# 7.5, and the same bits come out, so this is a fixed rule up to ROW_TILES_FEATURES output features (3,072 x 7,680
+# gains at 64 rows only, 35 us against 41, and loses below).  The products behind the norms gain less (4,120 x 1,024
+# at 64 rows: 9.4 us against 11.8) and add their rows' partial sums of squares in another order, so for them, and
+# beyond the rule, the clock decides over the chain of layers.  A plan's number: 1 = every workgroup all rows,
+# 2 = over two workgroups, 4 = one tile of 16 rows each.
+ROW_TILES_FEATURES = 2048
+FORCE_ROW_TILES: Optional[int] = None     # tests: this number for all four projections instead of the rule and the clock
 PLAN_FIELDS = ("library_in", "library_out", "library_gate_up", "library_down", "split_out", "split_down",
-               "tiles_in", "tiles_out", "tiles_gate_up", "tiles_down", "deferred")
+               "tiles_in", "tiles_out", "tiles_gate_up", "tiles_down", "deferred",
+               "rows_in", "rows_out", "rows_gate_up", "rows_down")
 _chain_wins: Dict[tuple, tuple] = {}
 _chain_times: list = []     # (rows, microseconds a layer of each candidate, the one taken): what was measured, for whoever asks
 
@@ -365,6 +377,14 @@ def _measure_chain(chain, bucket: int) -> dict:
     if (skinny not in candidates and first._may_defer(skinny)
             and all(f is not None for fusion in chain for f in (fusion.f_in, fusion.f_out, fusion.f_gate_up, fusion.f_down))):
         candidates.append(skinny)
+    if rows > 16:                 # the same with the rows dealt out: (into the stream, behind the norms)
+        for base in [plan for plan in candidates if plan["deferred"]]:
+            for stream, behind in ((1, 1), (4, 1), (2, 1), (4, 4), (4, 2)):
+                variant = dict(base, rows_out=stream, rows_down=stream, rows_in=behind, rows_gate_up=behind)
+                if behind > 1:
+                    variant.update(tiles_in=1, tiles_gate_up=1)
+                if variant not in candidates:
+                    candidates.append(variant)
     device = first.w_in.device
     h = torch.full((rows, first.hidden), 0.01, dtype=torch.float32, device=device)
     mixed = torch.full((rows, first.mixed_width), 0.01, dtype=torch.bfloat16, device=device)
@@ -496,6 +516,10 @@ class LayerFusion:
             beyond_down = self._tune_split_beyond(self.down.weight, self.down.bias)
             self.f_gate_up = fragments(self.gate_up.weight, self.library_gate_up, ())
             self.f_down = fragments(self.down.weight, self.library_down, self.split_down + beyond_down[:1])
+        # how the rows of a step are dealt out where the norms are left to the projections
+        self.rows_in = self.rows_gate_up = _each(1 if FORCE_ROW_TILES is None else FORCE_ROW_TILES)
+        self.rows_out = self._row_tiles(self.w_out)
+        self.rows_down = self._row_tiles(self.down.weight) if self.down is not None else _each(1)
         # step sizes at which the norms are left to the projections around them
         self.deferred = _each(False)
         self.deferred = tuple(self._may_defer(self._plan(bucket)) for bucket in range(BUCKETS))
@@ -504,10 +528,18 @@ class LayerFusion:
         # that feed the stream in slabs from the kernel that shares the rows, where that is faster
         beyond = dict(library_in=True, library_out=True, library_gate_up=True, library_down=True,
                       split_out=beyond_out[0], split_down=beyond_down[0], tiles_in=1, tiles_out=beyond_out[1],
-                      tiles_gate_up=1, tiles_down=beyond_down[1], deferred=False)
+                      tiles_gate_up=1, tiles_down=beyond_down[1], deferred=False, rows_in=1, rows_out=1, rows_gate_up=1,
+                      rows_down=1)
         for name, value in beyond.items():
             if hasattr(self, name):
                 setattr(self, name, getattr(self, name) + (value,))
+
+    def _row_tiles(self, weight: torch.Tensor) -> tuple:
+        """The fixed rule for a projection into the stream: one tile of 16 rows a workgroup where it has few output
+        features and the step more than 16 rows."""
+        if FORCE_ROW_TILES is not None:
+            return _each(FORCE_ROW_TILES)
+        return tuple(4 if rows > 16 and weight.shape[0] <= ROW_TILES_FEATURES else 1 for rows in TUNE_ROWS)
 
     def _plan(self, bucket: int) -> dict:
         """How steps of TUNE_ROWS[bucket] rows go through the layer's projections."""
@@ -541,7 +573,7 @@ class LayerFusion:
         if (not self.measure or not self.decode_ok or self.gate_up is None or self.ffn_scale is None
                 or self.mixer_scale is None
                 or any(force is not None for force in (FORCE_DEFERRED_NORM, FORCE_LIBRARY, FORCE_SPLIT, FORCE_TILES,
-                                                      FORCE_SHARED_ROWS))
+                                                      FORCE_SHARED_ROWS, FORCE_ROW_TILES))
                 or self.w_in.numel() + self.w_out.numel() + self.gate_up.weight.numel() + self.down.weight.numel()
                 < LIBRARY_MIN_WEIGHT):
             return
@@ -579,6 +611,9 @@ class LayerFusion:
             out.update({"gate_up": way(self.library_gate_up), "down": way(self.library_down, self.split_down),
                         "tiles_gate_up": tiled(self.tiles_gate_up), "tiles_down": tiled(self.tiles_down),
                         "norms": "/".join("D" if deferred else "-" for deferred in self.deferred[:BUCKETS]),
+                        "rows": "/".join("".join(str(rows[bucket]) for rows in (self.rows_in, self.rows_out, self.rows_gate_up,
+                                                                                self.rows_down)) if self.deferred[bucket] else "-"
+                                         for bucket in range(BUCKETS)),
                         "beyond_out_down": f"{beyond(self.split_out)}/{beyond(self.split_down)}"})
         return out
 
@@ -745,7 +780,8 @@ class LayerFusion:
         arguments = dict(h_in=residual.h, deltas=pending, h_out=h_out, norm_weight=rms[0], eps=rms[1])
         return arguments, h_out
 
-    def _add_to_the_stream(self, residual: Residual, x, weight, bias, fragments, next_weight, attended=None) -> None:
+    def _add_to_the_stream(self, residual: Residual, x, weight, bias, fragments, next_weight, attended=None,
+                           row_tiles: int = 1) -> None:
         """h += the projection, with the rows that the product behind the norm of ``next_weight`` reads."""
         M, device = x.shape[0], x.device
         rows = torch.empty((M, self.hidden), dtype=torch.bfloat16, device=device)
@@ -753,7 +789,7 @@ class LayerFusion:
         if attended is not None:
             ops.fused_gemm_merge(weight, bias, None, x, attended, fragments, residual=(residual.h, rows, next_weight, ssq))
         else:
-            ops.fused_gemm_residual(weight, bias, x, residual.h, rows, next_weight, ssq, fragments)
+            ops.fused_gemm_residual(weight, bias, x, residual.h, rows, next_weight, ssq, fragments, row_tiles=row_tiles)
         residual.scaled = ScaledRows(rows, ssq, next_weight)
 
     def _behind_the_norm(self, scaled: ScaledRows, rms) -> dict:
@@ -770,7 +806,7 @@ class LayerFusion:
             # the layer before left the stream prepared for this norm
             u = torch.empty((M, self.in_ld), dtype=torch.bfloat16, device=device)
             ops.fused_gemm(self.w_in, self.b_in, u[:, :self.in_width], epilogue=epilogue, conv=conv,
-                           fragments=self.f_in, **_tiles(self.tiles_in[bucket]),
+                           fragments=self.f_in, **_tiles(self.tiles_in[bucket], self.rows_in[bucket]),
                            **self._behind_the_norm(scaled, self.mixer_scale))
         elif self.library_in[bucket]:
             u = ops.linear(block.mixer_norm.forward(residual), self.w_in, self.b_in)
@@ -793,7 +829,8 @@ class LayerFusion:
         block = self.block
         # 3
         if self.deferred[bucket] and not residual.pending:
-            self._add_to_the_stream(residual, mixed, self.w_out, self.b_out, self.f_out, self.ffn_scale[0], attended)
+            self._add_to_the_stream(residual, mixed, self.w_out, self.b_out, self.f_out, self.ffn_scale[0], attended,
+                                    self.rows_out[bucket])
         else:
             residual.pending = self._to_the_stream(mixed, self.w_out, self.b_out, self.library_out[bucket],
                                                    self.split_out[bucket], self.tiles_out[bucket], self.f_out, attended)
@@ -807,7 +844,7 @@ class LayerFusion:
             scaled = None
         if scaled is not None:
             ops.fused_gemm(self.gate_up.weight, self.gate_up.bias, activated, epilogue=ops.EPI_SWIGLU,
-                           fragments=self.f_gate_up, **_tiles(self.tiles_gate_up[bucket]),
+                           fragments=self.f_gate_up, **_tiles(self.tiles_gate_up[bucket], self.rows_gate_up[bucket]),
                            **self._behind_the_norm(scaled, self.ffn_scale))
         elif self.library_gate_up[bucket]:
             ops.swiglu(ops.linear(block.ffn_norm.forward(residual), self.gate_up.weight, self.gate_up.bias), activated, 8)
@@ -821,7 +858,7 @@ class LayerFusion:
         # 5
         if scaled is not None and residual.next_norm is not None:
             self._add_to_the_stream(residual, activated, self.down.weight, self.down.bias, self.f_down,
-                                    residual.next_norm[0])
+                                    residual.next_norm[0], row_tiles=self.rows_down[bucket])
             return
         residual.pending = self._to_the_stream(activated, self.down.weight, self.down.bias, self.library_down[bucket],
                                                self.split_down[bucket], self.tiles_down[bucket], self.f_down)
@@ -851,7 +888,8 @@ class LayerFusion:
             return [delta]
         if slabs and (M <= MAX_ROWS or (tiles < 0 and M <= SHARED_ROWS_MOST)):
             partial = torch.empty((slabs, M, self.hidden), dtype=torch.float32, device=x.device)
-            ops.fused_gemm_split(weight, bias, x, partial, fragments=fragments, **_tiles(tiles))
+            ops.fused_gemm_split(weight, bias, x, partial, fragments=fragments, feature_tiles=abs(tiles),
+                                 shared_rows=tiles < 0)
             return list(partial.unbind(0))
         if library or M > MAX_ROWS:
             return [ops.linear(x, weight, bias)]
@@ -860,10 +898,11 @@ class LayerFusion:
         return [delta]
 
 
-def _tiles(tiles: int) -> dict:
+def _tiles(tiles: int, rows: int = 1) -> dict:
     """A plan's number of feature tiles as the products' arguments: negative, that many a wave of the kernel that
-    shares the rows."""
-    return dict(feature_tiles=abs(tiles), shared_rows=tiles < 0)
+    shares the rows.  ``rows``: over how many workgroups the step's rows are dealt out (the skinny kernel with one
+    tile of features only)."""
+    return dict(feature_tiles=abs(tiles), shared_rows=tiles < 0, row_tiles=rows if tiles == 1 else 1)
 
 
 def _rms_prologue(norm):

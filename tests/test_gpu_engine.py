@@ -607,7 +607,7 @@ def test_fixed_paths_take_no_measurement(tmp_path, monkeypatch):
                         max_active_sequences=24, measured_paths=measured)
         choices = engine.path_choices()
         assert set(choices) == {"in", "out", "gate_up", "down", "tiles_in", "tiles_out", "tiles_gate_up", "tiles_down",
-                                "padded_in", "norms", "beyond_out_down"}
+                                "padded_in", "norms", "rows", "beyond_out_down"}
         assert all(len(value.split("/")) == {"padded_in": 5, "beyond_out_down": 2}.get(name, 6)
                    for name, value in choices.items())
         assert bool(fused._chain_wins) == measured          # the layers' chain was timed too, once for the shape
@@ -616,6 +616,7 @@ def test_fixed_paths_take_no_measurement(tmp_path, monkeypatch):
             assert choices["norms"] == "D/D/D/D/D/D"
             assert choices["tiles_in"] == choices["tiles_down"] == "1/1/1/1/1/1" and choices["padded_in"] == "-/-/-/-/-"
             assert choices["beyond_out_down"] == "L/L"
+            assert choices["rows"] == "1111/1111/1111/1414/1414/1414"       # few output features: one tile of rows a workgroup
         for index in prompts:
             engine.add_request(index)
         engine.step([Lane(index, tokens[:-1], []) for index, tokens in prompts.items()])
@@ -664,6 +665,39 @@ def test_norms_left_to_the_projections_around_them(tmp_path, monkeypatch):
             assert gates.bfloat16_close(logits[row].numpy(), want.numpy()), (deferred, "mixed", row)
         assert checked == 24
         engine.cache.check()
+
+
+@pytest.mark.parametrize("row_tiles", [2, 4])
+def test_the_rows_of_a_step_dealt_out_to_several_workgroups(tmp_path, monkeypatch, row_tiles):
+    """Where the norms are left to the projections, a step of more than 16 rows may have its tiles of 16 rows
+    dealt out to two or four workgroups per tile of features, in all four projections of a layer (the conv step of
+    each row's own slot included): steps of 40, 33 and 17 single tokens, each close to the plain model."""
+    import gates
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.parts import fused
+    monkeypatch.setattr(fused, "FORCE_ROW_TILES", row_tiles)
+    folder = tiny_configs.make_model_dir("C", tmp_path, torch.bfloat16)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    prompts = {index: tokens_for(cfg["vocab_size"], 5 + index % 6, 700 + index) for index in range(40)}
+    engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * 40,
+                    max_active_sequences=40)
+    choices = engine.path_choices()
+    assert choices["norms"] == "D/D/D/D/D/D" and choices["rows"] == "/".join([str(row_tiles) * 4] * 6)
+    for index in prompts:
+        engine.add_request(index)
+    for first in range(0, 40, 8):                                           # the prompts, eight at a time
+        engine.step([Lane(index, prompts[index], []) for index in range(first, first + 8)])
+    history = {index: list(tokens) for index, tokens in prompts.items()}
+    for group in (range(40), range(7, 40), range(3, 20)):
+        lanes = []
+        for index in group:
+            history[index].append((index * 7 + len(history[index])) % cfg["vocab_size"])
+            lanes.append(Lane(index, history[index][-1:], [0]))
+        logits = engine.step(lanes).float().cpu()
+        for row, index in enumerate(group):
+            want = plain_impl.falcon_h1_logits(cfg, tensors, history[index])[-1]
+            assert gates.bfloat16_close(logits[row].numpy(), want.numpy()), (row_tiles, len(group), index)
+    engine.cache.check()
 
 
 def test_the_clock_says_from_how_many_single_tokens_a_mixed_step_runs_as_two_batches(tmp_path):

@@ -947,12 +947,16 @@ def test_fused_gemm_norm_prologue_and_epilogues(ops, M, N, K, deltas):
 
 
 @pytest.mark.parametrize("M, N, K, N2", [(8, 1024, 2048, 4120), (1, 72, 64, 48), (13, 1000, 96, 160), (16, 3072, 4608, 272),
-                                         (40, 200, 2048, 96), (40, 256, 2048, 96), (24, 96, 64, 80), (64, 1024, 2048, 272)])
+                                         (40, 200, 2048, 96), (40, 256, 2048, 96), (24, 96, 64, 80), (64, 1024, 2048, 272),
+                                         (48, 1024, 2048, 136), (33, 136, 96, 4120)])
 def test_a_product_that_joins_the_residual_stream_and_the_product_behind_the_next_norm(ops, M, N, K, N2):
     """``fused_gemm_residual``: h += x . W^T + b in float32 in place, with the new rows times the next norm's
     weight in bfloat16 and the partial sums of their squares; then ``fused_gemm`` with that row scale against the
     norm written out (the division of the root mean square applied to the rows, then the product), plain, with
-    the SwiGLU epilogue and with the conv step; a width that is no multiple of 16, 1 to 40 rows."""
+    the SwiGLU epilogue and with the conv step; a width that is no multiple of 16, 1 to 64 rows.  Every workgroup
+    with all of the step's rows, and the rows dealt out to two and to four workgroups per tile of features (the
+    same bits into the stream; nothing written beside the table of partial sums, whose guard rows stay as
+    they were)."""
     x = rand(M, K, seed=350, dtype=torch.bfloat16)
     W, b = rand(N, K, seed=351, scale=0.1, dtype=torch.bfloat16), rand(N, seed=352)
     h = rand(M, N, seed=353, scale=2.0)
@@ -960,13 +964,24 @@ def test_a_product_that_joins_the_residual_stream_and_the_product_behind_the_nex
     want_h, want_hb, want_ssq = h.clone(), torch.empty(M, N, dtype=torch.bfloat16), ops.residual_workspace(M, N, "cpu")
     ref_ops.fused_gemm_residual(W, b, x, want_h, want_hb, next_w, want_ssq)
     assert torch.allclose(want_h, h + x.float() @ W.float().T + b, atol=1e-4)
+    blocks, columns = want_ssq.shape
+    first = None
     for fragments in (None, ops.fragment_order(W.to(DEV))):
-        got_h, got_hb = h.clone().to(DEV), torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
-        got_ssq = torch.full_like(ops.residual_workspace(M, N, DEV), float("nan"))
-        ops.fused_gemm_residual(W.to(DEV), b.to(DEV), x.to(DEV), got_h, got_hb, next_w.to(DEV), got_ssq, fragments)
-        close(got_h, want_h, torch.float32, max(1.0, want_h.abs().max().item()))
-        close(got_hb, want_hb, torch.bfloat16, max(1.0, want_hb.float().abs().max().item()))
-        assert torch.allclose(got_ssq[:, :M].cpu(), want_ssq[:, :M], rtol=1e-4, atol=1e-4)
+        for row_tiles in (1, 2, 4):
+            got_h, got_hb = h.clone().to(DEV), torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+            guarded = torch.full((blocks + 2, columns), float("nan"), device=DEV)       # a row of guards on either side
+            got_ssq = guarded[1:-1]
+            ops.fused_gemm_residual(W.to(DEV), b.to(DEV), x.to(DEV), got_h, got_hb, next_w.to(DEV), got_ssq, fragments,
+                                    row_tiles=row_tiles)
+            close(got_h, want_h, torch.float32, max(1.0, want_h.abs().max().item()))
+            close(got_hb, want_hb, torch.bfloat16, max(1.0, want_hb.float().abs().max().item()))
+            assert torch.allclose(got_ssq[:, :M].cpu(), want_ssq[:, :M], rtol=1e-4, atol=1e-4)
+            assert torch.isnan(guarded[0]).all() and torch.isnan(guarded[-1]).all()
+            if first is None:
+                first = (got_h.clone(), got_hb.clone(), got_ssq[:, :M].clone())
+            else:
+                assert all(torch.equal(a, b_) for a, b_ in zip(first, (got_h, got_hb, got_ssq[:, :M])))
+    got_ssq = got_ssq.contiguous()
     # the product behind the norm: rows = h / rms(h) * w, rounded to bfloat16
     eps = 3e-5
     normed = (want_h / torch.sqrt(want_h.pow(2).mean(-1, keepdim=True) + eps) * next_w)
@@ -974,12 +989,14 @@ def test_a_product_that_joins_the_residual_stream_and_the_product_behind_the_nex
     scale = ops.RowScale(got_ssq, N, eps)
     if N % 32 == 0 and M <= 64:
         want = normed @ W2.float().T + b2
-        got = torch.empty(M, N2, dtype=torch.bfloat16, device=DEV)
-        ops.fused_gemm(W2.to(DEV), b2.to(DEV), got, x=got_hb, row_scale=scale)
-        close(got, want, torch.bfloat16, 3.0 * max(1.0, want.abs().max().item()))
         again = torch.empty(M, N2, dtype=torch.bfloat16)
         ref_ops.fused_gemm(W2, b2, again, x=got_hb.cpu(), row_scale=ops.RowScale(got_ssq.cpu(), N, eps))
-        close(got, again, torch.bfloat16, max(1.0, want.abs().max().item()))
+        for row_tiles in (1, 2, 4):
+            got = torch.full((M + 1, N2), float("nan"), dtype=torch.bfloat16, device=DEV)
+            ops.fused_gemm(W2.to(DEV), b2.to(DEV), got[:M], x=got_hb, row_scale=scale, row_tiles=row_tiles)
+            assert torch.isnan(got[M].float()).all()
+            close(got[:M], want, torch.bfloat16, 3.0 * max(1.0, want.abs().max().item()))
+            close(got[:M], again, torch.bfloat16, max(1.0, want.abs().max().item()))
         if N2 % 16 == 0:
             want = torch.empty(M, N2 // 2, dtype=torch.bfloat16)
             ref_ops.fused_gemm(W2, b2, want, x=got_hb.cpu(), row_scale=ops.RowScale(got_ssq.cpu(), N, eps), epilogue=ref_ops.EPI_SWIGLU)
@@ -987,6 +1004,11 @@ def test_a_product_that_joins_the_residual_stream_and_the_product_behind_the_nex
             ops.fused_gemm(W2.to(DEV), b2.to(DEV), got, x=got_hb, row_scale=scale, epilogue=ops.EPI_SWIGLU,
                            feature_tiles=2 if M > 16 else 1)
             close(got, want, torch.bfloat16, 16.0)
+            for row_tiles in (2, 4):
+                got = torch.empty(M, N2 // 2, dtype=torch.bfloat16, device=DEV)
+                ops.fused_gemm(W2.to(DEV), b2.to(DEV), got, x=got_hb, row_scale=scale, epilogue=ops.EPI_SWIGLU,
+                               row_tiles=row_tiles)
+                close(got, want, torch.bfloat16, 16.0)
 
 
 @pytest.mark.parametrize("M, N, K, S", [(64, 1024, 2048, 8), (33, 100, 2048, 16), (17, 48, 96, 3), (64, 136, 3072, 5),
@@ -1103,11 +1125,14 @@ def test_fused_gemm_split_with_the_rows_shared_refuses_other_sizes(ops):
 @pytest.mark.parametrize("M, N, K", [(24, 200, 1024), (64, 136, 1024), (7, 96, 2048), (64, 88, 3072), (40, 64, 64)])
 def test_fused_gemm_conv_step_of_wide_batches(ops, M, N, K):
     """The conv epilogue behind the plain prologue: more than one tile of 16 rows, four and eight
-    waves (K beyond 1,024), taps the prefetched path holds (2..4) and more than it holds (6)."""
+    waves (K beyond 1,024), taps the prefetched path holds (2..4) and more than it holds (6); every workgroup
+    with all the rows, and the rows dealt out to two or four workgroups per tile of features (each rolls the
+    tails of its own rows' slots only)."""
     x = rand(M, K, seed=330, dtype=torch.bfloat16)
     W, b = rand(N, K, seed=331, scale=0.1, dtype=torch.bfloat16), rand(N, seed=332)
     lo, hi = 8, N - 24
-    for taps, feature_tiles in ((4, 1), (2, 1), (6, 1), (4, 2), (3, 4), (6, 4)):
+    for taps, feature_tiles, row_tiles in ((4, 1, 1), (2, 1, 1), (6, 1, 1), (4, 2, 1), (3, 4, 1), (6, 4, 1), (4, 1, 4), (3, 1, 2),
+                                           (6, 1, 4)):
         C = hi - lo
         state = rand(M + 3, taps - 1, C, seed=333, dtype=torch.bfloat16)
         slot_ids = torch.randperm(M + 3, generator=torch.Generator().manual_seed(taps))[:M].to(torch.int32)
@@ -1117,12 +1142,16 @@ def test_fused_gemm_conv_step_of_wide_batches(ops, M, N, K):
         ref_ops.fused_gemm(W, b, want, x=x, epilogue=ref_ops.EPI_CONV, conv=dict(conv, state=want_state, slot_ids=slot_ids))
         got = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
         ops.fused_gemm(W.to(DEV), b.to(DEV), got, x=x.to(DEV), epilogue=ops.EPI_CONV, feature_tiles=feature_tiles,
+                       row_tiles=row_tiles,
                        conv=dict(lo=lo, hi=hi, taps=taps, weight=conv["weight"].to(DEV), bias=conv["bias"].to(DEV),
                                  state=got_state, slot_ids=slot_ids.to(DEV)))
         close(got, want, torch.bfloat16, 8.0)
         close(got_state, want_state, torch.bfloat16, 8.0)
         unused = [slot for slot in range(M + 3) if slot not in slot_ids.tolist()]
         assert torch.equal(got_state[unused].cpu(), state[unused])
+    with pytest.raises((ValueError, RuntimeError)):            # rows dealt out: one tile of features a workgroup only
+        ops.fused_gemm(W.to(DEV), b.to(DEV), torch.empty(M, N, dtype=torch.bfloat16, device=DEV), x=x.to(DEV),
+                       feature_tiles=2, row_tiles=2)
 
 
 @pytest.mark.parametrize("M, N, K", [(24, 200, 1024), (64, 136, 1056), (17, 96, 128), (49, 90, 3072), (40, 1048, 160),
