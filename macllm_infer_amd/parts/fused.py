@@ -353,13 +353,17 @@ def build_layer_fusion(block, build) -> Optional["LayerFusion"]:
     return LayerFusion.build(block, build)
 
 
-def _run_chain(chain, rows: int, bucket: int, h: torch.Tensor, mixed: torch.Tensor) -> None:
+def _run_chain(chain, rows: int, bucket: int, h: torch.Tensor, mixed: torch.Tensor, tails=None) -> None:
     """The projections and norms of the layers of ``chain`` one after the other, as a decode step of ``rows``
-    rows runs them (the mixers left out: the same rows stand for what they would write)."""
+    rows runs them (the mixers left out: the same rows stand for what they would write).  ``tails``: (conv state
+    of ``rows`` slots, their ids), where the input projection runs a conv step in its epilogue."""
     residual = Residual(h)
     for index, fusion in enumerate(chain):
         residual.next_norm = chain[(index + 1) % len(chain)].mixer_scale
-        fusion._project_in(residual, rows, bucket, None)
+        conv = None
+        if tails is not None and fusion.kernel is not None and fusion.kernel.conv is not None:
+            conv = dict(fusion.kernel.conv, state=tails[0], slot_ids=tails[1])
+        fusion._project_in(residual, rows, bucket, conv)
         fusion._after_the_mixers(residual, mixed, None, rows, bucket)
 
 
@@ -388,11 +392,16 @@ def _measure_chain(chain, bucket: int) -> dict:
     device = first.w_in.device
     h = torch.full((rows, first.hidden), 0.01, dtype=torch.float32, device=device)
     mixed = torch.full((rows, first.mixed_width), 0.01, dtype=torch.bfloat16, device=device)
+    tails = None
+    conv = first.kernel.conv if first.kernel is not None else None
+    if conv is not None:            # the conv step is part of the input projection's time (4 of its 14 us at 64 rows of 4,120 features)
+        tails = (torch.zeros((rows, max(conv["taps"] - 1, 0), conv["hi"] - conv["lo"]), dtype=torch.bfloat16, device=device),
+                 torch.arange(rows, dtype=torch.int32, device=device))
     times = []
     for plan in candidates:
         for fusion in chain:
             fusion._apply(bucket, plan)
-        times.append(_graph_microseconds(lambda: _run_chain(chain, rows, bucket, h, mixed)))
+        times.append(_graph_microseconds(lambda: _run_chain(chain, rows, bucket, h, mixed, tails)))
     for fusion in chain:
         fusion._apply(bucket, current)
     best = min(range(len(candidates)), key=lambda index: times[index] / (1.0 if index == 0 else CHAIN_MARGIN))
