@@ -71,6 +71,17 @@ def resolve_dtype(dtype) -> torch.dtype:
 # is split from SPLIT_FROM_LANES single tokens on, which is also the fewest the clock can say.
 SPLIT_FROM_LANES = 4
 SPLIT_NEVER = 1 << 30
+# A step of more single decoded tokens than the skinny kernels take rows runs as two halves at once, each a
+# captured graph of its own on a stream of its own (``Engine._run_in_halves``): a half's products go through the
+# skinny kernels instead of the library, and while one half's mixer kernel streams states, keys and values the
+# other half's products, which wait on latency rather than on bandwidth, run beside it.  The 0.5B shape at
+# 2,048-token contexts: 96 single tokens in 3.97 ms instead of 4.53 as one graph, 128 in 4.41 instead of 5.03
+# (two halves of 32 gain nothing on one graph of 64: 3.14 ms against 3.04).  The halves read every weight twice: a
+# model whose steps wait for their weights loses (the 7B shape: 96 single tokens in 20.8 ms instead of 15.6), so the
+# clock decides when the first such step comes (``DecodeGraphs.measure_halves``; the halves have to win by
+# HALVES_MARGIN); without a clock such a step stays one graph.
+HALVES_FROM_LANES = 65
+HALVES_MARGIN = 0.95
 
 
 def split_from_lanes(lane_share: Optional[float]) -> int:
@@ -126,6 +137,10 @@ class Engine:
         self.vocab_size = self.spec.vocab_size
         self.max_context = self.spec.max_context
         self.graphs = None
+        self.graphs_beside = None                    # the graphs of the second half of a step that runs as two halves at once
+        self._beside = None                          # and the stream they are replayed on
+        self._in_halves: Optional[bool] = None
+        self.halves_share: Optional[float] = None
         if decode_graphs and check_device and self.model.graph_safe:
             from .graphs import DecodeGraphs
             self.graphs = DecodeGraphs(self.model, self.cache, self.device, min(self.max_context, capacity))
@@ -146,6 +161,21 @@ class Engine:
     def split_from_lanes(self, value: int) -> None:
         self._split_from_lanes = int(value)
 
+    @property
+    def in_halves(self) -> bool:
+        """Whether a step of HALVES_FROM_LANES single tokens or more runs as two halves at once: asked of the clock
+        when it is first needed (or by ``warm_up``), where there is one."""
+        if self._in_halves is None:
+            self._in_halves = False
+            if self._measure_split and self.graphs is not None:
+                self.halves_share = self.graphs.measure_halves()
+                self._in_halves = self.halves_share is not None and self.halves_share < HALVES_MARGIN
+        return self._in_halves
+
+    @in_halves.setter
+    def in_halves(self, value: bool) -> None:
+        self._in_halves = bool(value)
+
     def path_choices(self) -> dict:
         """What the first layer's fast path chose at build (empty when the layer has none): to be recorded
         beside a result, since a close call of the clock can fall either way from one process to the next."""
@@ -158,7 +188,22 @@ class Engine:
         does this once: no step of such a size is then ever launched kernel by kernel).  ``context``: the
         longest context the steps' requests will hold.  Returns what was captured; nothing without graphs."""
         self.split_from_lanes                        # the clock's say on mixed steps, before the first of them
-        return self.graphs.warm_up(steps, context) if self.graphs is not None else []
+        if self.graphs is None:
+            return []
+        whole, halves = [], []
+        for lanes, tokens in steps:
+            if tokens == lanes >= HALVES_FROM_LANES and self.in_halves:      # runs as two halves: a graph for each
+                halves.append(((lanes + 1) // 2, lanes - (lanes + 1) // 2))
+            else:
+                whole.append((lanes, tokens))
+        done = self.graphs.warm_up(whole + [(first, first) for first, _ in halves], context)
+        if halves:
+            from .graphs import DecodeGraphs
+            if self.graphs_beside is None:
+                self.graphs_beside = DecodeGraphs(self.model, self.cache, self.device, self.graphs.max_seq_len)
+                self._beside = torch.cuda.Stream(device=self.device)
+            done += self.graphs_beside.warm_up([(second, second) for _, second in halves], context)
+        return done
 
     def step_token_target(self, lanes: int, tokens: int) -> int:
         """How many tokens (at most ``tokens``) a step of ``lanes`` lanes should hold if whoever makes it is free
@@ -248,10 +293,13 @@ class Engine:
         singles = int(single.sum())
         # (the clock is asked, once, only by a step that may need its answer, and before anything is reserved)
         in_two = SPLIT_FROM_LANES <= singles < len(lanes) and self.split_from_lanes <= singles
+        in_halves = singles == len(lanes) >= HALVES_FROM_LANES and self.graphs is not None and self.in_halves
         self.cache.reserve_slots(lowered.slots, lowered.lengths)
         try:
             if in_two:
                 logits = self._run_in_two(lanes, lowered, single)
+            elif in_halves:
+                logits = self._run_in_halves(lanes)
             else:
                 logits = self._run(lanes, lowered)
         except Exception as error:
@@ -263,19 +311,42 @@ class Engine:
         self.cache.commit_slots(lowered.slots, lowered.lengths)
         return logits
 
-    def _run(self, lanes: Sequence[Lane], lowered: LoweredLanes) -> torch.Tensor:
+    def _run(self, lanes: Sequence[Lane], lowered: LoweredLanes, graphs=None) -> torch.Tensor:
         """Queue the lanes' tokens as one batch: a captured graph where one fits, else launch by launch."""
         logits = None
-        if self.graphs is not None:
+        graphs = graphs if graphs is not None else self.graphs
+        if graphs is not None:
             if int(lowered.lengths.max()) == 1:
-                logits = self.graphs.run(lanes, lowered)              # decode-only batch: a captured graph
+                logits = graphs.run(lanes, lowered)                   # decode-only batch: a captured graph
             else:
-                logits = self.graphs.run_bucket(lanes, lowered)       # prompt portions: a graph of their capacity
+                logits = graphs.run_bucket(lanes, lowered)            # prompt portions: a graph of their capacity
         if logits is None:
             context = build_step_context(lanes, self.cache, self.device, lowered, **self.model.step_layout)
             apply_feeds(context.token_ids, lowered.feeds)
             logits = self.model.forward(context, self.cache)
         return logits
+
+    def _run_in_halves(self, lanes: Sequence[Lane]) -> torch.Tensor:
+        """A step of many single decoded tokens as two halves at once: the second half's graph is replayed on a
+        stream of its own, which starts behind everything queued so far (the tokens that lanes are fed from
+        among it) and which the caller's stream waits for before it reads the rows.  The halves belong to
+        different requests, so they share no page and no slot but the scratch ones of their padding lanes, whose
+        contents nobody reads; their graphs have memory pools of their own."""
+        main = torch.cuda.current_stream(self.device)
+        if self.graphs_beside is None:
+            from .graphs import DecodeGraphs
+            self.graphs_beside = DecodeGraphs(self.model, self.cache, self.device, self.graphs.max_seq_len)
+            self._beside = torch.cuda.Stream(device=self.device)
+        half = (len(lanes) + 1) // 2
+        first, second = list(lanes[:half]), list(lanes[half:])
+        lowered_second = self.validate(second)
+        self._beside.wait_stream(main)
+        with torch.cuda.stream(self._beside):
+            rows_second = self._run(second, lowered_second, self.graphs_beside)
+        rows_first = self._run(first, self.validate(first))
+        main.wait_stream(self._beside)
+        rows_second.record_stream(main)
+        return torch.cat([rows_first, rows_second])
 
     def _run_in_two(self, lanes: Sequence[Lane], lowered: LoweredLanes, single: np.ndarray) -> torch.Tensor:
         """A step that holds portions of prompts beside several single decoded tokens, as two batches one after

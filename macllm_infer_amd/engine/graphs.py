@@ -209,6 +209,44 @@ class DecodeGraphs:
             return None
         return (both - portion) / singles / alone
 
+    def measure_halves(self, lanes: int = 128, replays: int = 5) -> Optional[float]:
+        """The clock's answer to whether a step of ``lanes`` single tokens is faster as two halves at once, each a
+        graph of its own on a stream of its own, than as one graph: the time of the two halves over the time of the
+        one.  The halves read every weight twice, which a model whose steps wait for its weights cannot afford
+        (the 7B shape: 20.8 ms for 96 single tokens in halves, 15.6 as one graph), while a small model's halves
+        go through the skinny kernels and fill each other's waits (the 0.5B shape: 3.9 ms against 4.4).  Every
+        lane of the three graphs is padding (nothing but the scratch page and slot is touched: the mixers' kernels
+        cost little here, the products what they cost in a step); the median of ``replays`` counts."""
+        context = min(CONTEXT_BUCKET_FROM, self.max_seq_len)
+        whole = self._capture(bucket_for(lanes), context=context, warm_runs=1, pool=torch.cuda.graph_pool_handle())
+        halves = [self._capture(bucket_for((lanes + 1) // 2), context=context, warm_runs=1,
+                                pool=torch.cuda.graph_pool_handle()) for _ in range(2)]
+        main = torch.cuda.current_stream(self.device)
+        beside = torch.cuda.Stream(device=self.device)
+
+        def as_one():
+            whole[1].replay()
+
+        def as_halves():
+            beside.wait_stream(main)
+            with torch.cuda.stream(beside):
+                halves[1][1].replay()
+            halves[0][1].replay()
+            main.wait_stream(beside)
+
+        times = []
+        for run in (as_one, as_halves):
+            marks = [torch.cuda.Event(enable_timing=True) for _ in range(replays + 1)]
+            run()
+            marks[0].record()
+            for mark in marks[1:]:
+                run()
+                mark.record()
+            torch.cuda.synchronize(self.device)
+            times.append(sorted(a.elapsed_time(b) for a, b in zip(marks, marks[1:]))[replays // 2])
+        del whole, halves
+        return times[1] / times[0] if times[0] > 0 else None
+
     def _capture(self, bucket: int, static: Optional[StaticStep] = None, warm_runs: int = 2, context: int = 0,
                  pool=None):
         if static is None:

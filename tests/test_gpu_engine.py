@@ -307,7 +307,7 @@ def test_generation_under_a_constraint_on_the_tokens(tmp_path):
 def test_generation_with_more_live_requests_than_the_skinny_kernels_take_rows(tmp_path):
     """Seventy-two requests live at once through the scheduler (bfloat16, configuration D): prompts of 3 to 40
     tokens in portions of 24 beside the decoded tokens of the others (so steps run as two batches), then rounds of
-    up to 72 single tokens (the decode kernel between library products).  Every request runs to its length, no
+    up to 72 single tokens (two halves at once, each a graph of its own on a stream of its own).  Every request runs to its length, no
     page or slot is left held, and for five of the requests every token is the plain model's choice or as good
     as it (the plain model's logit of the token within a few per cent of its best: bfloat16 may swap near ties)."""
     from macllm_infer_amd import LLM, EngineConfig, SamplingParams
@@ -319,14 +319,17 @@ def test_generation_with_more_live_requests_than_the_skinny_kernels_take_rows(tm
               engine_config=EngineConfig(max_active_sequences=count, scheduler_token_budget=24 + count,
                                          prefill_token_quantum=24))
     llm.engine.split_from_lanes = 4             # two batches from four single tokens on, whatever the clock would say
-    runs = []
-    real = llm.engine._run
-    llm.engine._run = lambda lanes, lowered: (runs.append((len(lanes), int(lowered.lengths.max()))), real(lanes, lowered))[1]
+    llm.engine.in_halves = True                 # and more than 64 single tokens as two halves at once
+    runs, halves = [], []
+    real, real_halves = llm.engine._run, llm.engine._run_in_halves
+    llm.engine._run = lambda lanes, lowered, graphs=None: (runs.append((len(lanes), int(lowered.lengths.max()))),
+                                                           real(lanes, lowered, graphs))[1]
+    llm.engine._run_in_halves = lambda lanes: (halves.append(len(lanes)), real_halves(lanes))[1]
     params = SamplingParams(max_new_tokens=7, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0, ignore_eos=True)
     results = llm.generate(prompts, params)
     assert [result.finish_reason for result in results] == ["length"] * count
     assert all(len(result.token_ids) == 7 for result in results)
-    assert any(lanes > 64 and longest == 1 for lanes, longest in runs)            # rounds of more than 64 single tokens
+    assert halves and max(halves) > 64 and llm.engine.graphs_beside.counts["decode_replays"] == len(halves)   # rounds of more than 64 single tokens: two halves at once
     assert any(longest > 1 for _, longest in runs) and any(lanes >= 4 and longest == 1 for lanes, longest in runs)
     assert llm.engine.cache.stats()["live_requests"] == 0
     llm.engine.cache.check()
@@ -336,6 +339,87 @@ def test_generation_with_more_live_requests_than_the_skinny_kernels_take_rows(tm
             logits = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-1]
             assert logits[token].item() >= logits.max().item() - 0.06 * logits.abs().max().item(), (index, len(tokens))
             tokens.append(token)
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_a_step_of_many_single_tokens_runs_as_two_halves_at_once(tmp_path, dtype):
+    """More single decoded tokens than the skinny kernels take rows (81 and 100 of them, uneven halves): the step
+    runs as two halves at once, each half a captured graph of its own on a stream of its own, the second half fed
+    from the device like the first.  Six steps in a row with nothing waiting in between; every row against the
+    plain model, in float32 the same bits as the same step through one graph, and nothing held afterwards."""
+    import gates
+    from macllm_infer_amd import Engine, Lane
+    folder = tiny_configs.make_model_dir("D", tmp_path, torch.bfloat16 if dtype == "bfloat16" else torch.float32)
+    cfg, tensors = plain_impl.load_model_dir(folder)
+    requests = 100
+    prompts = {index: tokens_for(cfg["vocab_size"], 4 + index % 9 + 6, 800 + index) for index in range(requests)}
+    outcomes = {}
+    for in_halves in (True, False):
+        engine = Engine(folder, dtype=dtype, kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * (requests + 1),
+                        max_active_sequences=requests + 1)
+        engine.in_halves = in_halves
+        if in_halves:
+            assert len(engine.warm_up([(100, 100), (81, 81)])) == 2          # 50 + 50 and 41 + 40: a graph of 64 lanes in each bank
+        for index in prompts:
+            engine.add_request(index)
+        for first in range(0, requests, 25):
+            engine.step([Lane(index, prompts[index][:-6], []) for index in range(first, first + 25)])
+        rows = {index: [] for index in prompts}
+        for turn in range(6):
+            live = range(requests) if turn % 2 == 0 else range(19, requests)                 # 100, then 81
+            logits = engine.step([Lane(index, [prompts[index][len(prompts[index]) - 6 + len(rows[index])]], [0])
+                                  for index in live])
+            for row, index in enumerate(live):
+                rows[index].append(logits[row])
+        torch.cuda.synchronize()
+        if in_halves:
+            assert engine.graphs_beside is not None and engine.graphs_beside.counts["decode_replays"] == 6
+            assert engine.graphs.counts["decode_replays"] == 6
+        else:
+            assert engine.graphs_beside is None
+        outcomes[in_halves] = {index: torch.stack(values).float().cpu() for index, values in rows.items()}
+        for index in prompts:
+            engine.finish(index)
+        engine.cache.check()
+        assert engine.cache.stats()["live_requests"] == 0
+    for index in (0, 18, 19, 49, 50, 59, 60, 99):
+        tokens = prompts[index]
+        want = plain_impl.falcon_h1_logits(cfg, tensors, tokens)[-6:]
+        have = outcomes[True][index]
+        assert have.shape[0] == (6 if index >= 19 else 3)
+        for place in range(have.shape[0]):
+            if dtype == "float32":
+                assert gates.float32_close(have[place].numpy(), want[place].numpy()), (index, place)
+            else:
+                assert gates.bfloat16_close(have[place].numpy(), want[place].numpy()), (index, place)
+    if dtype == "float32":
+        assert all(torch.equal(outcomes[True][index], outcomes[False][index]) for index in prompts)
+
+
+def test_the_clock_says_whether_many_single_tokens_run_as_two_halves(tmp_path):
+    """Nothing is measured until a step of 65 single tokens or more comes; then one graph of 128 padding lanes is
+    timed against two of 64 at once, once, and the halves are taken if they win by the margin.  Without a clock
+    such a step stays one graph."""
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.engine import engine as engine_module
+    folder = tiny_configs.make_model_dir("D", tmp_path, torch.bfloat16)
+    cfg, _ = plain_impl.load_model_dir(folder)
+    fixed = Engine(folder, dtype="bfloat16", kv_cache_capacity_tokens=70 * 32, max_active_sequences=70, measured_paths=False)
+    assert fixed.in_halves is False and fixed.halves_share is None
+    engine = Engine(folder, dtype="bfloat16", kv_cache_capacity_tokens=70 * 32, max_active_sequences=70)
+    for index in range(70):
+        engine.add_request(index)
+    for first in range(0, 70, 35):
+        engine.step([Lane(index, tokens_for(cfg["vocab_size"], 5, index), []) for index in range(first, first + 35)])
+    engine.step([Lane(index, [3], [0]) for index in range(64)])
+    assert engine._in_halves is None                                   # 64 single tokens: no question
+    got = engine.step([Lane(index, [4], [0]) for index in range(70)])
+    assert got.shape[0] == 70
+    print("two halves over one graph:", engine.halves_share, "in halves:", engine.in_halves)
+    assert engine.halves_share is not None and engine.halves_share > 0
+    assert engine.in_halves == (engine.halves_share < engine_module.HALVES_MARGIN)
+    assert (engine.graphs_beside is not None) == engine.in_halves
+    engine.cache.check()
 
 
 def test_generation_when_pages_run_out(tmp_path):
@@ -488,6 +572,7 @@ def test_wide_decode_batches_match_the_plain_model(tmp_path, monkeypatch, reques
     cfg, tensors = plain_impl.load_model_dir(folder)
     engine = Engine(folder, dtype="bfloat16", kv_cache_block_tokens=16, kv_cache_capacity_tokens=64 * (requests + 1),
                     max_active_sequences=requests + 1)
+    engine.in_halves = False                     # 80 and 128 single tokens as one graph (not as two halves at once)
     if library is True:
         fusion = engine.model.blocks[0].fusion
         assert fusion.general and all(fusion.library_in) and all(fusion.library_out) and all(fusion.library_down)
