@@ -81,6 +81,7 @@ SPLIT_NEVER = 1 << 30
 # clock decides when the first such step comes (``DecodeGraphs.measure_halves``; the halves have to win by
 # HALVES_MARGIN); without a clock such a step stays one graph.
 HALVES_FROM_LANES = 65
+HALVES_MOST_LANES = 128        # beyond, a half would leave the skinny kernels too: one graph, as measured for no such size
 HALVES_MARGIN = 0.95
 
 
@@ -192,7 +193,7 @@ class Engine:
             return []
         whole, halves = [], []
         for lanes, tokens in steps:
-            if tokens == lanes >= HALVES_FROM_LANES and self.in_halves:      # runs as two halves: a graph for each
+            if tokens == lanes and HALVES_FROM_LANES <= lanes <= HALVES_MOST_LANES and self.in_halves:      # runs as two halves: a graph for each
                 halves.append(((lanes + 1) // 2, lanes - (lanes + 1) // 2))
             else:
                 whole.append((lanes, tokens))
@@ -293,7 +294,8 @@ class Engine:
         singles = int(single.sum())
         # (the clock is asked, once, only by a step that may need its answer, and before anything is reserved)
         in_two = SPLIT_FROM_LANES <= singles < len(lanes) and self.split_from_lanes <= singles
-        in_halves = singles == len(lanes) >= HALVES_FROM_LANES and self.graphs is not None and self.in_halves
+        in_halves = (singles == len(lanes) and HALVES_FROM_LANES <= singles <= HALVES_MOST_LANES
+                     and self.graphs is not None and self.in_halves)
         self.cache.reserve_slots(lowered.slots, lowered.lengths)
         try:
             if in_two:
