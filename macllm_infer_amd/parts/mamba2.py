@@ -118,13 +118,18 @@ class Mamba2(Mixer):
         E, C = spec.inner_size, spec.conv_width
         T = u.shape[0]
         conv_state, ssm_state = cache.states["conv"], cache.states["ssm"]
-        xbc = torch.empty((T, C), dtype=u.dtype, device=u.device)
         chunked = self._chunked(u, step)
         raw = u[:, E:E + C]
+        xbc = raw if step.max_query_len == 1 and not chunked else torch.empty((T, C), dtype=u.dtype, device=u.device)
         conv = None
         if chunked and ops.ssd_conv_supported(spec.conv_kernel, C, raw):
             # the chunked scan runs the conv and the tail update in its own launches
             conv = dict(u=raw, weight=self.conv_weight, bias=self.conv_bias, state=conv_state)
+        elif step.max_query_len == 1:
+            # single tokens: the conv step in place and the tail rolled by one, in one launch (the same products in
+            # the same order as the two kernels below give for a lane of one token)
+            ops.conv_step(u, E, C, self.conv_weight, self.conv_bias, conv_state, step.slot_ids)
+            xbc = raw
         else:
             ops.conv1d_silu(u, E, C, self.conv_weight, self.conv_bias, conv_state, step.lane_of_token,
                             step.cu_seqlens, step.slot_ids, xbc)
