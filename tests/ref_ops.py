@@ -221,7 +221,7 @@ def argmax(logits, out):
 
 
 NAMES = ["fused_gemm_split", "add_partials_rmsnorm", "prefill_attention_supported", "decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "tanh_softcap", "linear", "rope_kv_store", "paged_attention",
-         "conv1d_silu", "conv_state_update", "ssm_scan", "gate_norm", "argmax", "feed_tokens", "keep_allowed"]
+         "conv1d_silu", "conv_state_update", "conv_step", "ssm_scan", "gate_norm", "argmax", "feed_tokens", "keep_allowed"]
 
 
 def install(monkeypatch):
