@@ -343,10 +343,14 @@ class Engine:
         first, second = list(lanes[:half]), list(lanes[half:])
         lowered_second = self.validate(second)
         self._beside.wait_stream(main)
-        with torch.cuda.stream(self._beside):
-            rows_second = self._run(second, lowered_second, self.graphs_beside)
-        rows_first = self._run(first, self.validate(first))
-        main.wait_stream(self._beside)
+        try:
+            with torch.cuda.stream(self._beside):
+                rows_second = self._run(second, lowered_second, self.graphs_beside)
+            rows_first = self._run(first, self.validate(first))
+        finally:
+            # whatever happens, nothing queued behind this step (pages given back and used again among it) may
+            # overtake what the second stream still has to do
+            main.wait_stream(self._beside)
         rows_second.record_stream(main)
         return torch.cat([rows_first, rows_second])
 
