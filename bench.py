@@ -157,7 +157,10 @@ def microbench() -> int:
 def choices_of(engine) -> dict:
     """What the first layer's fast path chose for steps of up to 4 / 8 / 16 / 32 / 48 / 64 rows, as short strings
     (S: the skinny kernel, L: the library, a number: that many slabs over K; empty when the layer has none)."""
-    return engine.path_choices()
+    choices = dict(engine.path_choices())
+    if getattr(engine, "halves_share", None) is not None:     # a step of more than 64 single tokens came: two halves at once over one graph
+        choices["halves_over_one_graph"] = round(engine.halves_share, 3)
+    return choices
 
 
 def main() -> int:
