@@ -77,6 +77,10 @@ gemm_f32_kernel(const float* __restrict__ x, long ldx, const float* __restrict__
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) b[j][mt] = load_k4<VEC>(x_row[mt], k, K);
     }
+    // a step of few rows waits for its weights: every load of the round is asked for before its first product (left
+    // to itself the scheduler moves each load down to the product that uses it and waits for it there, one round
+    // trip to memory after the other; the tiles of many rows, which wait for their products, are better left to it)
+    if (NT == 1) __builtin_amdgcn_sched_barrier(0);
     // no branch around the products either (under one the compiler waits for each load where it is used,
     // one at a time): a chunk past the end is multiplied as zeros
 #pragma unroll
