@@ -207,9 +207,23 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
   for (int i = 0; i < ATT_MAX_DH / WAVE; ++i) {
     const int dim = lane + i * WAVE;
     if (dim < dh) {
+      // sixteen values asked for at once, then added in the order of their keys (one at a time, each load would
+      // wait for the one before: 64 round trips a wave); a key past the last reads the last again and is not added
       float sum = 0.f;
-      for (int j = from; j < to; ++j)
-        sum = fmaf(p_shared[wave][j], to_float(v_base[row_shared[wave][j] + (long)dim * page_size + offset_shared[wave][j]]), sum);
+      for (int j0 = from; j0 < to; j0 += 16) {
+        float values[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int j = min(j0 + u, to - 1);
+          values[u] = to_float(v_base[row_shared[wave][j] + (long)dim * page_size + offset_shared[wave][j]]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const float added = fmaf(p_shared[wave][min(j0 + u, WAVE - 1)], values[u], sum);
+          sum = j0 + u < to ? added : sum;
+        }
+      }
       wave_o[wave][dim] = sum;
     }
   }
