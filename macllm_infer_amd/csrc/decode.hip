@@ -192,19 +192,9 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
       tail_slot[j] = p.slot_ids[min(((tid + j * FG_THREADS) / 256) * 16 + tid % 16, p.M - 1)];
   }
 
-  // the partial sums of squares of the rows (row scale), 16 MT rows by SSQ_PARTS threads each, and the elements of
-  // the residual stream that this thread will add to (RESIDUAL) are asked for up here as well
+  // the elements of the residual stream that this thread will add to (RESIDUAL) are asked for up here as well
   constexpr int PARTS = SSQ_PARTS / MT;               // PARTS * 16 MT threads: within the 256 of four waves
-  // asked for without a branch (under one, the wave waits for them before it asks for its weights) and not added
-  // up before the products are done; without a row scale, and past the last workgroup's sums, a valid address
-  float ssq_early[SSQ_EARLY] = {};
-  if (p.ssq_in) {
-    const int last = p.ssq_blocks - 1;
-    const int row = min(tid % (16 * MT), ssq_rows - 1);
-#pragma unroll
-    for (int i = 0; i < SSQ_EARLY; ++i)
-      ssq_early[i] = p.ssq_in[(long)min(tid / (16 * MT) + i * PARTS, last) * p.ssq_ld + row];
-  }
+
   float res_old[EPT] = {};
   float res_weight = 0.f;
   if (EPI == EPI_RESIDUAL) {
@@ -285,6 +275,18 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
       a[j][nt] = *reinterpret_cast<const bf16x8_t*>(w_row[nt] + min(first_chunk + min(j, max(iterations, 1) - 1), chunks - 1) * w_step);
+  // the partial sums of squares of the rows (row scale), 16 MT rows by SSQ_PARTS threads each: asked for right behind
+  // the weights (ahead of them, these dozen loads of what the kernel before has just written on other dies hold the
+  // weights back: a decode step of 8 rows took 1.383 ms so, 1.367 this way) and not added up before the products
+  // are done; without a row scale, and past the last workgroup's sums, a valid address
+  float ssq_early[SSQ_EARLY] = {};
+  if (p.ssq_in) {
+    const int last = p.ssq_blocks - 1;
+    const int row = min(tid % (16 * MT), ssq_rows - 1);
+#pragma unroll
+    for (int i = 0; i < SSQ_EARLY; ++i)
+      ssq_early[i] = p.ssq_in[(long)min(tid / (16 * MT) + i * PARTS, last) * p.ssq_ld + row];
+  }
   if (PRO == PRO_NORM) {
     // one wave per row, two rows at a time: the rows are read once into registers (K <= 2048),
     // their sums of squares reduced in float32, and the normalized rows written in bfloat16
