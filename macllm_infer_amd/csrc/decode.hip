@@ -275,18 +275,20 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
       a[j][nt] = *reinterpret_cast<const bf16x8_t*>(w_row[nt] + min(first_chunk + min(j, max(iterations, 1) - 1), chunks - 1) * w_step);
-  // the partial sums of squares of the rows (row scale), 16 MT rows by SSQ_PARTS threads each: asked for right behind
-  // the weights (ahead of them, these dozen loads of what the kernel before has just written on other dies hold the
-  // weights back: a decode step of 8 rows took 1.383 ms so, 1.367 this way) and not added up before the products
-  // are done; without a row scale, and past the last workgroup's sums, a valid address
+  // the partial sums of squares of the rows (row scale), 16 MT rows by SSQ_PARTS threads each: asked for behind the
+  // weights and behind the step's rows of the first round of products (ahead of them, these dozen loads of what the
+  // kernel before has just written on other dies hold back what the products wait for: a decode step of 8 rows took
+  // 1.383 ms with the sums first, 1.364 with them behind the weights, 1.355 behind the rows too) and not added up
+  // before the products are done; past the last workgroup's sums, a valid address
   float ssq_early[SSQ_EARLY] = {};
-  if (p.ssq_in) {
+  auto ask_ssq = [&]() {
     const int last = p.ssq_blocks - 1;
     const int row = min(tid % (16 * MT), ssq_rows - 1);
 #pragma unroll
     for (int i = 0; i < SSQ_EARLY; ++i)
       ssq_early[i] = p.ssq_in[(long)min(tid / (16 * MT) + i * PARTS, last) * p.ssq_ld + row];
-  }
+  };
+  if (p.ssq_in && iterations == 0) ask_ssq();          // a wave without a run of K has no round
   if (PRO == PRO_NORM) {
     // one wave per row, two rows at a time: the rows are read once into registers (K <= 2048),
     // their sums of squares reduced in float32, and the normalized rows written in bfloat16
@@ -452,6 +454,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
         }
       }
     }
+    if (first == 0 && p.ssq_in) ask_ssq();
     // no branch around a product: under a condition the compiler moves the fragment's load into the
     // branch and waits for it there, one at a time; a fragment past the end is read again (clamped
     // above) and multiplied as zeros
