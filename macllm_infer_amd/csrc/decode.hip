@@ -288,7 +288,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
     for (int i = 0; i < SSQ_EARLY; ++i)
       ssq_early[i] = p.ssq_in[(long)min(tid / (16 * MT) + i * PARTS, last) * p.ssq_ld + row];
   };
-  if (p.ssq_in && iterations == 0) ask_ssq();          // a wave without a run of K has no round
+  if (PRO == PRO_PLAIN && p.ssq_in && iterations == 0) ask_ssq();          // a wave without a run of K has no round
   if (PRO == PRO_NORM) {
     // one wave per row, two rows at a time: the rows are read once into registers (K <= 2048),
     // their sums of squares reduced in float32, and the normalized rows written in bfloat16
@@ -454,7 +454,7 @@ __global__ void __launch_bounds__(FG_WAVES * WAVE) fused_gemm_kernel(FusedGemmPa
         }
       }
     }
-    if (first == 0 && p.ssq_in) ask_ssq();
+    if (PRO == PRO_PLAIN && first == 0 && p.ssq_in) ask_ssq();         // (a row scale comes with the plain prologue only)
     // no branch around a product: under a condition the compiler moves the fragment's load into the
     // branch and waits for it there, one at a time; a fragment past the end is read again (clamped
     // above) and multiplied as zeros
