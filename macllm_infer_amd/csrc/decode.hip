@@ -1281,6 +1281,10 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
   // between the loads (an index that is not needed is clamped to one that is valid): the query
   // heads, the new key and value, the cache cell, the rotation frequencies
   const bool rotate = p.inv_freq != nullptr;
+  // (the position first: the page ids wait for it, the keys for them, and loads come back in the order they were
+  // asked for; behind the query's rows, which the kernel before has just written on other dies, it would wait for them)
+  const int pos = p.positions[token];
+  const long cell = p.slot_mapping[token];
   mfma_bf16x8 q_own[DH / 32], q_pair[DH / 32];
   const bool has_head = n < G;
   const bf16_t* q_head = row + p.q_col + (kvh * G + (has_head ? n : 0)) * DH;
@@ -1291,8 +1295,6 @@ __device__ void mixer_attention_block(const MixerParams& p, int block, int* page
     q_own[kk] = *reinterpret_cast<const mfma_bf16x8*>(q_head + own_dim);
     q_pair[kk] = *reinterpret_cast<const mfma_bf16x8*>(q_head + pair_dim);
   }
-  const int pos = p.positions[token];
-  const long cell = p.slot_mapping[token];
   const int k_dim = min(tid, DH - 1);
   const int k_pair_dim = k_dim < p.rotary_dim ? (k_dim < half ? k_dim + half : k_dim - half) : k_dim;
   const bf16_t* k_head = row + p.k_col + kvh * DH;
