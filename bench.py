@@ -85,7 +85,7 @@ def serving(args, shape) -> int:
     capacity = sum(-(-(length + new_tokens) // 64) * 64 for length in lengths)
     engine = Engine(config=config, tensors=tensors, dtype="bfloat16" if args.dtype == "bf16" else "float32",
                     kv_cache_block_tokens=args.page_tokens, kv_cache_capacity_tokens=capacity,
-                    max_active_sequences=requests)
+                    max_active_sequences=requests, measured_paths=not args.fixed_paths)
     del tensors
     llm = LLM(engine, engine_config=EngineConfig(max_active_sequences=requests, prefill_token_quantum=SERVING_PORTION,
                                                  scheduler_token_budget=SERVING_PORTION + requests))
@@ -175,6 +175,9 @@ def main() -> int:
                         help="fewer layers than the configuration has (both numbers are reported)")
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--page-tokens", type=int, default=16)
+    parser.add_argument("--fixed-paths", action="store_true",
+                        help="the layers' fixed rules instead of the build-time clock (as `run --fixed-paths`): the same "
+                             "kernels in every process, also under a profiler, whose overhead the clock would measure")
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
     parser.add_argument("--skip-long-points", action="store_true", help="no decode points at longer contexts")
     parser.add_argument("--prefill-only", action="store_true",
@@ -222,7 +225,7 @@ def main() -> int:
     engine = Engine(config=config, tensors=tensors, dtype="bfloat16" if args.dtype == "bf16" else "float32",
                     kv_cache_block_tokens=args.page_tokens,
                     kv_cache_capacity_tokens=per_request * largest + PREFILL_TOKENS + 64,
-                    max_active_sequences=largest + 1)
+                    max_active_sequences=largest + 1, measured_paths=not args.fixed_paths)
     sampler = Sampler(engine.vocab_size, engine.device)
     generator = torch.Generator().manual_seed(0)
     vocab = config.vocab_size
